@@ -1,0 +1,23 @@
+"""MI355X-native Mega/Mega2 sequence-mixing path: hand-written HIP kernels (libmega_hip.so,
+C ABI in include/mega_hip.h) behind the reference's operator and module surface."""
+from . import _lib, ops  # noqa: F401
+from .modules import (  # noqa: F401
+    AttentionSoftmax,
+    BaseMovingLayer,
+    EfficientAttention,
+    MultiHeadComplexEMA,
+    MultiHeadEMA,
+    SwiGLU,
+    TimestepNorm,
+)
+
+__all__ = [
+    "ops",
+    "AttentionSoftmax",
+    "BaseMovingLayer",
+    "EfficientAttention",
+    "MultiHeadComplexEMA",
+    "MultiHeadEMA",
+    "SwiGLU",
+    "TimestepNorm",
+]

@@ -1,0 +1,70 @@
+"""ctypes binding of libmega_hip.so (the C ABI declared in include/mega_hip.h).
+
+The library is the product: there is no CPU or PyTorch fallback.  If it has not been
+built, loading raises with the build command; if a call is rejected, the reason the
+library recorded is raised as RuntimeError (the reference raises RuntimeError from
+TORCH_CHECK in the same situations).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmega_hip.so")
+
+F32, BF16, F16 = 0, 1, 2
+
+_p = C.c_void_p
+_i64 = C.c_int64
+_int = C.c_int
+_sz = C.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/mega_hip.h
+SIGNATURES = {
+    "mega_last_error": (C.c_char_p, []),
+    "mega_abi_version": (_int, []),
+    "mega_ema_parameters_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _p, _p]),
+    "mega_ema_hidden_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "mega_ema_hidden_fwd": (_int, [_p, _int, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _p, _sz, _p]),
+    "mega_ema_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _int, _i64]),
+    "mega_ema_fwd": (_int, [_p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _int, _p, _p, _p, _p,
+                            _i64, _i64, _i64, _i64, _int, _i64, _int, _p, _sz, _p]),
+    "mega_ema_step": (_int, [_p, _p, _int, _p, _p, _p, _int, _p, _p, _p, _i64, _i64, _i64, _p]),
+    "mega_long_conv_fwd": (_int, [_p, _p, _int, _p, _i64, _i64, _i64, _i64, _int, _int, _p]),
+    "mega_timestep_norm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
+    "mega_group_timestep_norm_fwd": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, C.c_double,
+                                            _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mega_timestep_norm_fwd": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, C.c_double,
+                                      _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mega_attention_softmax_fwd": (_int, [_p, _p, _int, _i64, _i64, _i64, _int, _p]),
+    "mega_attention_fwd": (_int, [_p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_float, _int, _p]),
+    "mega_swiglu_fwd": (_int, [_p, _p, _p, _int, _i64, _p]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python fairseq-apollo_amd/build.py` "
+            "(hipcc --offload-arch=gfx950).  There is no fallback path."
+        )
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mega_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what}: {msg} (code {rc})")

@@ -1,0 +1,163 @@
+// Attention softmax (right-aligned causal mask, fully masked rows -> zeros) and the fused
+// attention op y = softmax_causal(scale q k^T) v.
+//
+// Semantics: fairseq/csrc/softmax.cuh:90-153 (row r of an [outer, inner] matrix keeps the
+// first inner - outer + r + 1 columns; a row whose maximum is -inf, or whose sum is zero,
+// becomes zeros) and fairseq/csrc/ops/attention_kernel.cu:40-131 (q, k: [B,L,Nh,H1],
+// v: [B,L,Nh,H2]).
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ float block_reduce(float v, float* red, bool is_max) {
+  for (int m = 32; m >= 1; m >>= 1) {
+    const float o = __shfl_xor(v, m);
+    v = is_max ? fmaxf(v, o) : v + o;
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < kBlock / 64; ++i) r = is_max ? fmaxf(r, red[i]) : r + red[i];
+  return r;
+}
+
+// one workgroup per row
+template <typename T>
+__global__ __launch_bounds__(kBlock) void softmax_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                         int64_t outer, int64_t inner, int causal) {
+  __shared__ float red[kBlock / 64];
+  const int64_t row = blockIdx.x;
+  const int64_t r = row % outer;
+  int64_t n = causal ? inner - outer + r + 1 : inner;
+  if (n < 0) n = 0;
+  const T* xp = x + row * inner;
+  T* yp = y + row * inner;
+  float m = -INFINITY;
+  for (int64_t j = threadIdx.x; j < n; j += kBlock) m = fmaxf(m, to_float(xp[j]));
+  m = block_reduce(m, red, true);
+  const bool dead = !(m > -INFINITY) || !(m < INFINITY);
+  float s = 0.f;
+  if (!dead)
+    for (int64_t j = threadIdx.x; j < n; j += kBlock) s += __expf(to_float(xp[j]) - m);
+  s = block_reduce(s, red, false);
+  const float c = (dead || s == 0.f) ? 0.f : 1.0f / s;
+  for (int64_t j = threadIdx.x; j < inner; j += kBlock) {
+    const float e = (j < n && !dead) ? __expf(to_float(xp[j]) - m) * c : 0.f;
+    yp[j] = from_float<T>(e);
+  }
+}
+
+// Plain attention: one workgroup per (b, head, query row); scores of the row live in LDS.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                               const T* __restrict__ v, T* __restrict__ y,
+                                                               T* __restrict__ w, int B, int L, int Nh, int H1,
+                                                               int H2, float scale, int causal) {
+  extern __shared__ float sc[];     // [L] scores, then [H1] the query row
+  __shared__ float red[kBlock / 64];
+  float* qs = sc + L;
+  const int l = blockIdx.x % L;
+  const int n = (blockIdx.x / L) % Nh;
+  const int b = blockIdx.x / (L * Nh);
+  const int nk = causal ? l + 1 : L;
+  const T* qp = q + (((size_t)b * L + l) * Nh + n) * H1;
+  for (int i = threadIdx.x; i < H1; i += kBlock) qs[i] = to_float(qp[i]);
+  __syncthreads();
+  float m = -INFINITY;
+  for (int j = threadIdx.x; j < nk; j += kBlock) {
+    const T* kp = k + (((size_t)b * L + j) * Nh + n) * H1;
+    float s = 0.f;
+    for (int i = 0; i < H1; ++i) s += qs[i] * to_float(kp[i]);
+    s *= scale;
+    sc[j] = s;
+    m = fmaxf(m, s);
+  }
+  m = block_reduce(m, red, true);
+  const bool dead = !(m > -INFINITY) || !(m < INFINITY);
+  float s = 0.f;
+  for (int j = threadIdx.x; j < nk; j += kBlock) {
+    const float e = dead ? 0.f : __expf(sc[j] - m);
+    sc[j] = e;
+    s += e;
+  }
+  s = block_reduce(s, red, false);
+  const float c = (dead || s == 0.f) ? 0.f : 1.0f / s;
+  __syncthreads();
+  if (w) {
+    T* wp = w + (((size_t)b * Nh + n) * L + l) * L;
+    for (int j = threadIdx.x; j < L; j += kBlock) wp[j] = from_float<T>(j < nk ? sc[j] * c : 0.f);
+  }
+  T* yp = y + (((size_t)b * L + l) * Nh + n) * H2;
+  for (int f = threadIdx.x; f < H2; f += kBlock) {
+    float acc = 0.f;
+    for (int j = 0; j < nk; ++j) acc += sc[j] * to_float(v[(((size_t)b * L + j) * Nh + n) * H2 + f]);
+    yp[f] = from_float<T>(acc * c);
+  }
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch, int64_t outer,
+                                          int64_t inner, int causal, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "attention_softmax_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(batch >= 0 && outer >= 0 && inner >= 0, MEGA_ERR_ARG, "attention_softmax_fwd: negative size");
+  const int64_t rows = batch * outer;
+  if (rows == 0 || inner == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && y, MEGA_ERR_ARG, "attention_softmax_fwd: null pointer argument");
+  MEGA_REQUIRE(rows < (int64_t)1 << 31, MEGA_ERR_UNSUPPORTED, "attention_softmax_fwd: too many rows");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)rows);
+  switch (dtype) {
+    case MEGA_F32:
+      hipLaunchKernelGGL(softmax_kernel<float>, grid, dim3(kBlock), 0, s, (const float*)x, (float*)y, outer, inner, causal);
+      break;
+    case MEGA_BF16:
+      hipLaunchKernelGGL(softmax_kernel<bf16_t>, grid, dim3(kBlock), 0, s, (const bf16_t*)x, (bf16_t*)y, outer, inner, causal);
+      break;
+    default:
+      hipLaunchKernelGGL(softmax_kernel<f16_t>, grid, dim3(kBlock), 0, s, (const f16_t*)x, (f16_t*)y, outer, inner, causal);
+      break;
+  }
+  MEGA_CHECK_LAUNCH("attention_softmax_fwd");
+  return MEGA_OK;
+}
+
+extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
+                                  int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
+                                  int causal, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "attention_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && L >= 0 && Nh > 0 && H1 > 0 && H2 > 0, MEGA_ERR_ARG, "attention_fwd: bad shape");
+  if (B == 0 || L == 0) return MEGA_OK;
+  MEGA_REQUIRE(q && k && v && y, MEGA_ERR_ARG, "attention_fwd: null pointer argument");
+  MEGA_REQUIRE(B * L * Nh < (int64_t)1 << 31, MEGA_ERR_UNSUPPORTED, "attention_fwd: too many rows");
+  const size_t smem = (size_t)(L + H1) * 4;
+  MEGA_REQUIRE(smem <= 150 * 1024, MEGA_ERR_UNSUPPORTED, "attention_fwd: L=%ld too long for one chunk", (long)L);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)(B * L * Nh));
+#define LAUNCH_ATT(T)                                                                                      \
+  do {                                                                                                     \
+    if (smem > 64 * 1024)                                                                                  \
+      hipFuncSetAttribute((const void*)attention_row_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                          (int)smem);                                                                      \
+    hipLaunchKernelGGL(attention_row_kernel<T>, grid, dim3(kBlock), smem, s, (const T*)q, (const T*)k,     \
+                       (const T*)v, (T*)y, (T*)w, (int)B, (int)L, (int)Nh, (int)H1, (int)H2, scale, causal); \
+  } while (0)
+  switch (dtype) {
+    case MEGA_F32: LAUNCH_ATT(float); break;
+    case MEGA_BF16: LAUNCH_ATT(bf16_t); break;
+    default: LAUNCH_ATT(f16_t); break;
+  }
+#undef LAUNCH_ATT
+  MEGA_CHECK_LAUNCH("attention_fwd");
+  return MEGA_OK;
+}

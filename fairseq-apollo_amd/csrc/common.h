@@ -1,0 +1,139 @@
+// Shared host/device helpers for libmega_hip (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/mega_hip.h"
+
+namespace mega {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+
+#define MEGA_REQUIRE(cond, code, ...)  \
+  do {                                 \
+    if (!(cond)) {                     \
+      ::mega::set_error(__VA_ARGS__);  \
+      return (code);                   \
+    }                                  \
+  } while (0)
+
+#define MEGA_CHECK_LAUNCH(what)                                           \
+  do {                                                                    \
+    hipError_t e__ = hipGetLastError();                                   \
+    if (e__ != hipSuccess) {                                              \
+      ::mega::set_error("%s: launch failed: %s", what, hipGetErrorString(e__)); \
+      return MEGA_ERR_LAUNCH;                                             \
+    }                                                                     \
+  } while (0)
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
+
+// ---------------------------------------------------------------- element types
+struct bf16_t { uint16_t u; };
+struct f16_t { _Float16 h; };
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((uint32_t)v.u) << 16); }
+__device__ __forceinline__ float to_float(f16_t v) { return (float)v.h; }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
+  // round to nearest even; NaN stays NaN
+  uint32_t u = __float_as_uint(v);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.u = (uint16_t)((u >> 16) | 0x0040u);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.u = (uint16_t)(u >> 16);
+  }
+  return r;
+}
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) {
+  f16_t r;
+  r.h = (_Float16)v;
+  return r;
+}
+
+// a naturally aligned vector of VEC elements, moved with one memory instruction
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) Vec {
+  T v[VEC];
+};
+
+// ---------------------------------------------------------------- complex
+struct cfloat {
+  float re, im;
+};
+__device__ __forceinline__ cfloat cmul(cfloat a, cfloat b) {
+  return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+__device__ __forceinline__ cfloat cadd(cfloat a, cfloat b) { return {a.re + b.re, a.im + b.im}; }
+
+// q^e for a non-negative integer e by binary exponentiation (double precision)
+__host__ __device__ inline void cpow_int(double qr, double qi, int64_t e, double* rr, double* ri) {
+  double ar = 1.0, ai = 0.0;
+  double br = qr, bi = qi;
+  while (e > 0) {
+    if (e & 1) {
+      const double t = ar * br - ai * bi;
+      ai = ar * bi + ai * br;
+      ar = t;
+    }
+    const double t = br * br - bi * bi;
+    bi = 2.0 * br * bi;
+    br = t;
+    e >>= 1;
+  }
+  *rr = ar;
+  *ri = ai;
+}
+
+// ---------------------------------------------------------------- Welford
+// state: n elements' worth of weight, their mean and their biased variance
+// (the combine operator of the streaming norm; equal weights merge exactly as
+// WelfordCombine does for counts).
+struct Moments {
+  float n, mean, var;
+};
+__device__ __forceinline__ Moments combine(Moments a, Moments b) {
+  const float n = a.n + b.n;
+  if (n == 0.f) return {0.f, 0.f, 0.f};
+  const float ca = a.n / n, cb = b.n / n;
+  const float d = b.mean - a.mean;
+  Moments r;
+  r.n = n;
+  r.mean = ca * a.mean + cb * b.mean;
+  r.var = ca * a.var + cb * b.var + (ca * d) * (cb * d);
+  return r;
+}
+
+// ---------------------------------------------------------------- cross-workgroup signalling
+// Values that one workgroup publishes for another travel through these (device scope)
+// atomics so that they are coherent across the per-XCD L2 caches.
+__device__ __forceinline__ void publish_f32(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float fetch_f32(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish_u32(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t fetch_u32(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void release_flag(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t acquire_flag(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace mega

@@ -1,0 +1,67 @@
+// SwiGLU gate y = silu(a) * b (elementwise, streamed with 16-byte accesses).
+#include "common.h"
+
+namespace mega {
+namespace {
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                     T* __restrict__ y, int64_t n) {
+  using V = Vec<T, VEC>;
+  const int64_t nv = n / VEC;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+    const V av = ((const V*)a)[i];
+    const V bv = ((const V*)b)[i];
+    V o;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float x = to_float(av.v[k]);
+      const float s = x / (1.0f + __expf(-x));
+      o.v[k] = from_float<T>(s * to_float(bv.v[k]));
+    }
+    ((V*)y)[i] = o;
+  }
+  // tail
+  const int64_t t = nv * VEC + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) {
+    const float x = to_float(a[t]);
+    y[t] = from_float<T>(x / (1.0f + __expf(-x)) * to_float(b[t]));
+  }
+}
+
+template <typename T>
+int launch_swiglu(const void* a, const void* b, void* y, int64_t n, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool aligned = (((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) % 16) == 0;
+  int64_t blocks = ceil_div(ceil_div(n, VEC), 256);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  if (aligned)
+    hipLaunchKernelGGL((swiglu_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)a, (const T*)b,
+                       (T*)y, n);
+  else
+    hipLaunchKernelGGL((swiglu_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)a, (const T*)b,
+                       (T*)y, n);
+  MEGA_CHECK_LAUNCH("swiglu_fwd");
+  return MEGA_OK;
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" int mega_swiglu_fwd(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "swiglu_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(n >= 0, MEGA_ERR_ARG, "swiglu_fwd: negative size");
+  if (n == 0) return MEGA_OK;
+  MEGA_REQUIRE(a && b && y, MEGA_ERR_ARG, "swiglu_fwd: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MEGA_F32: return launch_swiglu<float>(a, b, y, n, s);
+    case MEGA_BF16: return launch_swiglu<bf16_t>(a, b, y, n, s);
+    default: return launch_swiglu<f16_t>(a, b, y, n, s);
+  }
+}

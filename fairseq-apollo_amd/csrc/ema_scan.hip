@@ -1,0 +1,604 @@
+// Generic (any N <= 32, real or complex, any stride) EMA path on the vector ALUs:
+// the recurrence h' = q h + p x, y = Re sum_n gamma h, evaluated as a chunked scan.
+//
+//   pass A  chunk_state : S[c] = sum_{i in chunk c} q^{len-1-i} u_i        (zero start)
+//   pass B  chunk_scan  : H_in[c] = state at the start of chunk c (serial over the few
+//                         chunks), H_out = state after the last chunk
+//   pass C  chunk_apply : runs the recurrence inside every chunk from H_in[c] and writes y
+//
+// This is exactly the decomposition the reference uses for incremental evaluation
+// (kernel + carried-state bias + ema_hidden,
+// fairseq/modules/base_moving_average.py:144-160, fairseq/csrc/ops/ema_parameters.cc:54-77,
+// fairseq/csrc/ops/ema_hidden.cc:31-63), applied per chunk instead of per call; the
+// D x L convolution kernel is never formed.
+//
+// A "pass set" (A, B, C) evaluates one causal filter along one time direction.  The
+// layer is a sum of pass sets: forward direction; for bidirectional layers the reversed
+// direction with the second half of the coefficient rows
+// (fairseq/modules/fused_ops/fftconv.py:85-100); a kernel truncated to Lk taps is
+// "full filter minus the same filter delayed by Lk and scaled by q^Lk".
+//
+// Thread mapping: TPR = ceil(N/4) lanes share one (batch, channel) row, 4 complex
+// states each; rows are laid out channel-fastest so that [B,L,D] activations are read
+// coalesced.
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kNPT = 4;          // complex states per thread
+constexpr int kBlock = 256;
+
+// coefficient image of one pass set, padded to NP = TPR*4 states per row (zeros beyond N)
+struct PassCoef {
+  const float* q;   // [Drows, NP, 2]
+  const float* c;   // [Drows, NP, 2]  output coefficient (gamma, or -gamma q^Lk)
+  const float* p;   // [Drows, NP]     input coefficient
+};
+
+struct PassArgs {
+  const void* x;
+  int64_t sxb, sxd, sxl;
+  const uint8_t* mask;     // [B, L] or null
+  PassCoef coef;
+  const float* h_in;       // [B, D, N, 2] or null (true carried state)
+  float* h_out;            // [B, D, N, 2] or null
+  float* st;               // [B, nchunks, D, NP, 2] chunk states / chunk-start states
+  int B, D, N, L;
+  int NP, TPR;
+  int Tc, nchunks;
+  int reverse;             // logical time runs from the end of the sequence
+  int before;              // output uses the state before absorbing the current sample
+  int tshift;              // the filter input is delayed by tshift samples
+  // output stage
+  const float* acc_in;     // [B, L, D] fp32 partial sums from earlier pass sets, or null
+  float* acc_out;          // [B, L, D] fp32, or null when this pass set writes y
+  void* y;
+  int64_t syb, syd, syl;
+  const float* omega;      // [D]
+};
+
+template <typename T>
+__device__ __forceinline__ float load_u(const PassArgs& A, int b, int d, int tau) {
+  // logical sample tau of the (delayed, masked) filter input
+  const int ts = tau - A.tshift;
+  if (ts < 0) return 0.f;
+  const int t = A.reverse ? A.L - 1 - ts : ts;
+  if (A.mask && A.mask[(size_t)b * A.L + t]) return 0.f;
+  return to_float(((const T*)A.x)[b * A.sxb + d * A.sxd + t * A.sxl]);
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_state_kernel(const PassArgs A) {
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t total = (int64_t)A.B * A.nchunks * A.D * A.TPR;
+  if (gid >= total) return;
+  const int ns = (int)(gid % A.TPR);
+  const int d = (int)((gid / A.TPR) % A.D);
+  const int c = (int)((gid / ((int64_t)A.TPR * A.D)) % A.nchunks);
+  const int b = (int)(gid / ((int64_t)A.TPR * A.D * A.nchunks));
+  float qr[kNPT], qi[kNPT], hr[kNPT], hi[kNPT];
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    qr[k] = A.coef.q[o];
+    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    hr[k] = 0.f;
+    hi[k] = 0.f;
+  }
+  const int t0 = c * A.Tc;
+  const int t1 = min(t0 + A.Tc, A.L);
+  for (int tau = t0; tau < t1; ++tau) {
+    const float u = load_u<T>(A, b, d, tau);
+#pragma unroll
+    for (int k = 0; k < kNPT; ++k) {
+      if (CPLX) {
+        const float nr = qr[k] * hr[k] - qi[k] * hi[k] + u;
+        const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+        hr[k] = nr;
+        hi[k] = ni;
+      } else {
+        hr[k] = qr[k] * hr[k] + u;
+      }
+    }
+  }
+  float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + ns * kNPT) * 2;
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    sp[2 * k] = hr[k];
+    sp[2 * k + 1] = hi[k];
+  }
+}
+
+// one thread per (b, d, state): serial over the chunks
+template <bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A) {
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t total = (int64_t)A.B * A.D * A.NP;
+  if (gid >= total) return;
+  const int n = (int)(gid % A.NP);
+  const int d = (int)((gid / A.NP) % A.D);
+  const int b = (int)(gid / ((int64_t)A.NP * A.D));
+  const size_t oc = ((size_t)d * A.NP + n) * 2;
+  const double qr = A.coef.q[oc], qi = CPLX ? A.coef.q[oc + 1] : 0.0;
+  const float p = A.coef.p[(size_t)d * A.NP + n];
+  double Qr, Qi;
+  cpow_int(qr, qi, A.Tc, &Qr, &Qi);
+  float hr = 0.f, hi = 0.f;
+  if (A.h_in && n < A.N) {
+    const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
+    hr = A.h_in[oh];
+    hi = CPLX ? A.h_in[oh + 1] : 0.f;
+  }
+  const float fQr = (float)Qr, fQi = (float)Qi;
+  for (int c = 0; c < A.nchunks; ++c) {
+    float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + n) * 2;
+    const float sr = sp[0], si = sp[1];
+    sp[0] = hr;
+    sp[1] = hi;
+    float Ar = fQr, Ai = fQi;
+    if (c == A.nchunks - 1) {
+      // the last chunk may be shorter
+      double lr, li;
+      cpow_int(qr, qi, A.L - c * A.Tc, &lr, &li);
+      Ar = (float)lr;
+      Ai = (float)li;
+    }
+    const float nr = Ar * hr - Ai * hi + p * sr;
+    const float ni = Ar * hi + Ai * hr + p * si;
+    hr = nr;
+    hi = ni;
+  }
+  if (A.h_out && n < A.N) {
+    const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
+    A.h_out[oh] = hr;
+    A.h_out[oh + 1] = hi;
+  }
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t total = (int64_t)A.B * A.nchunks * A.D * A.TPR;
+  const bool live = gid < total;
+  const int64_t g2 = live ? gid : total - 1;     // keep whole lane groups converged for the shuffles
+  const int ns = (int)(g2 % A.TPR);
+  const int d = (int)((g2 / A.TPR) % A.D);
+  const int c = (int)((g2 / ((int64_t)A.TPR * A.D)) % A.nchunks);
+  const int b = (int)(g2 / ((int64_t)A.TPR * A.D * A.nchunks));
+  float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], pp[kNPT], hr[kNPT], hi[kNPT];
+  const float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + ns * kNPT) * 2;
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    qr[k] = A.coef.q[o];
+    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    cr[k] = A.coef.c[o];
+    ci[k] = CPLX ? A.coef.c[o + 1] : 0.f;
+    pp[k] = A.coef.p[o / 2];
+    hr[k] = sp[2 * k];
+    hi[k] = sp[2 * k + 1];
+  }
+  const float om = A.omega ? A.omega[d] : 0.f;
+  const int t0 = c * A.Tc;
+  const int t1 = min(t0 + A.Tc, A.L);
+  for (int tau = t0; tau < t1; ++tau) {
+    const float u = load_u<T>(A, b, d, tau);
+    float acc = 0.f;
+    if (A.before) {
+#pragma unroll
+      for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+    }
+#pragma unroll
+    for (int k = 0; k < kNPT; ++k) {
+      const float pu = pp[k] * u;
+      if (CPLX) {
+        const float nr = qr[k] * hr[k] - qi[k] * hi[k] + pu;
+        const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+        hr[k] = nr;
+        hi[k] = ni;
+      } else {
+        hr[k] = qr[k] * hr[k] + pu;
+      }
+    }
+    if (!A.before) {
+#pragma unroll
+      for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+    }
+    for (int m = 1; m < A.TPR; m <<= 1) acc += __shfl_xor(acc, m);
+    if (ns == 0 && live) {
+      const int t = A.reverse ? A.L - 1 - tau : tau;
+      const size_t oa = ((size_t)b * A.L + t) * A.D + d;
+      if (A.acc_in) acc += A.acc_in[oa];
+      if (A.acc_out) {
+        A.acc_out[oa] = acc;
+      } else {
+        float xr = 0.f;
+        if (A.omega) xr = to_float(((const T*)A.x)[b * A.sxb + d * A.sxd + t * A.sxl]);
+        ((T*)A.y)[b * A.syb + d * A.syd + t * A.syl] = from_float<T>(acc + om * xr);
+      }
+    }
+  }
+}
+
+// builds the padded coefficient images of up to 4 pass sets:
+//   set 0: forward rows [0,D)            set 1: forward tail  (c = -gamma q^Lk)
+//   set 2: backward rows [D,2D)          set 3: backward tail
+// `from_log`: q_or_logq holds log q (operator-level entry points) instead of q
+__global__ void coef_prep_kernel(const float* __restrict__ p, const float* __restrict__ q_or_logq,
+                                 const float* __restrict__ gamma, int from_log, int cplx, int D, int N,
+                                 int NP, int nsets_dir, int64_t Lk, float* out) {
+  // out layout per set: q [D,NP,2], c [D,NP,2], p [D,NP]
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t per = (int64_t)D * NP;
+  if (gid >= per * nsets_dir) return;
+  const int dir = (int)(gid / per);
+  const int d = (int)((gid % per) / NP);
+  const int n = (int)(gid % NP);
+  const size_t setsz = (size_t)per * 5;
+  float* o_full = out + (size_t)(2 * dir) * setsz;
+  float* o_tail = out + (size_t)(2 * dir + 1) * setsz;
+  const size_t oi = (size_t)d * NP + n;
+  double qr = 0, qi = 0, gr = 0, gi = 0, pv = 0;
+  if (n < N) {
+    const size_t src = ((size_t)(dir * D + d) * N + n);
+    const double a = q_or_logq[src * 2], bb = cplx ? q_or_logq[src * 2 + 1] : 0.0;
+    if (from_log) {
+      const double m = exp(a);
+      qr = m * cos(bb);
+      qi = m * sin(bb);
+    } else {
+      qr = a;
+      qi = bb;
+    }
+    gr = gamma[src * 2];
+    gi = cplx ? gamma[src * 2 + 1] : 0.0;
+    pv = p ? p[src] : 1.0;
+  }
+  o_full[oi * 2] = (float)qr;
+  o_full[oi * 2 + 1] = (float)qi;
+  o_full[per * 2 + oi * 2] = (float)gr;
+  o_full[per * 2 + oi * 2 + 1] = (float)gi;
+  o_full[per * 4 + oi] = (float)pv;
+  if (Lk > 0) {
+    double tr, ti;
+    cpow_int(qr, qi, Lk, &tr, &ti);
+    o_tail[oi * 2] = (float)qr;
+    o_tail[oi * 2 + 1] = (float)qi;
+    o_tail[per * 2 + oi * 2] = (float)(-(gr * tr - gi * ti));
+    o_tail[per * 2 + oi * 2 + 1] = (float)(-(gr * ti + gi * tr));
+    o_tail[per * 4 + oi] = (float)pv;
+  }
+}
+
+struct Plan {
+  int NP, TPR, Tc, nchunks;
+  size_t coef_bytes, st_bytes, acc_bytes, total;
+};
+
+Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_acc) {
+  Plan pl;
+  int tpr = 1;
+  while (tpr * kNPT < N) tpr <<= 1;
+  pl.TPR = tpr;
+  pl.NP = tpr * kNPT;
+  const int64_t rows = B * D * tpr;
+  int64_t want = ceil_div(262144, rows > 0 ? rows : 1);
+  int64_t maxc = ceil_div(L, 32);
+  int64_t nch = want < 1 ? 1 : want;
+  if (nch > maxc) nch = maxc;
+  if (nch < 1) nch = 1;
+  int64_t tc = ceil_div(L, nch);
+  tc = ceil_div(tc, 8) * 8;
+  if (tc < 1) tc = 1;
+  pl.Tc = (int)tc;
+  pl.nchunks = (int)ceil_div(L, tc);
+  if (pl.nchunks < 1) pl.nchunks = 1;
+  pl.coef_bytes = align_up((size_t)D * pl.NP * 5 * 4 * 4, 256);   // 4 sets
+  pl.st_bytes = align_up((size_t)B * pl.nchunks * D * pl.NP * 2 * 4, 256);
+  pl.acc_bytes = need_acc ? align_up((size_t)B * L * D * 4, 256) : 0;
+  (void)nsets;
+  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes;
+  return pl;
+}
+
+template <typename T>
+int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
+  const int64_t tA = (int64_t)A.B * A.nchunks * A.D * A.TPR;
+  const int64_t tB = (int64_t)A.B * A.D * A.NP;
+  if (cplx) {
+    hipLaunchKernelGGL((chunk_state_kernel<T, true>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
+    hipLaunchKernelGGL((chunk_scan_kernel<true>), dim3((unsigned)ceil_div(tB, kBlock)), dim3(kBlock), 0, s, A);
+    if (!state_only)
+      hipLaunchKernelGGL((chunk_apply_kernel<T, true>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
+  } else {
+    hipLaunchKernelGGL((chunk_state_kernel<T, false>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
+    hipLaunchKernelGGL((chunk_scan_kernel<false>), dim3((unsigned)ceil_div(tB, kBlock)), dim3(kBlock), 0, s, A);
+    if (!state_only)
+      hipLaunchKernelGGL((chunk_apply_kernel<T, false>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
+  }
+  MEGA_CHECK_LAUNCH("ema pass");
+  return MEGA_OK;
+}
+
+int run_pass_set_dtype(int dtype, PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
+  switch (dtype) {
+    case MEGA_F32: return run_pass_set<float>(A, cplx, state_only, s);
+    case MEGA_BF16: return run_pass_set<bf16_t>(A, cplx, state_only, s);
+    default: return run_pass_set<f16_t>(A, cplx, state_only, s);
+  }
+}
+
+PassCoef coef_of(float* base, int set, int64_t D, int NP) {
+  const size_t per = (size_t)D * NP;
+  float* o = base + (size_t)set * per * 5;
+  return PassCoef{o, o + per * 2, o + per * 4};
+}
+
+// ---------------------------------------------------------------- single decode step
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void ema_step_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                          const float* __restrict__ p,
+                                                          const float* __restrict__ q,
+                                                          const float* __restrict__ gamma,
+                                                          const float* __restrict__ omega,
+                                                          const float* h_in, float* h_out, int B, int D,
+                                                          int N) {
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (gid >= (int64_t)B * D) return;
+  const int d = (int)(gid % D);
+  const float xv = to_float(x[gid]);
+  float acc = 0.f;
+  const size_t ho = (size_t)gid * N * 2;
+  const size_t co = (size_t)d * N;
+  for (int n = 0; n < N; ++n) {
+    const float qr = q[(co + n) * 2], qi = CPLX ? q[(co + n) * 2 + 1] : 0.f;
+    const float gr = gamma[(co + n) * 2], gi = CPLX ? gamma[(co + n) * 2 + 1] : 0.f;
+    float hr = 0.f, hi = 0.f;
+    if (h_in) {
+      hr = h_in[ho + 2 * n];
+      hi = CPLX ? h_in[ho + 2 * n + 1] : 0.f;
+    }
+    const float nr = qr * hr - qi * hi + p[co + n] * xv;
+    const float ni = qr * hi + qi * hr;
+    h_out[ho + 2 * n] = nr;
+    h_out[ho + 2 * n + 1] = ni;
+    acc += gr * nr - gi * ni;
+  }
+  y[gid] = from_float<T>(acc + omega[d] * xv);
+}
+
+// ---------------------------------------------------------------- materialised kernel / bias
+// w[d,l] = Re sum_n p gamma exp(l log q); b[b,d,l] = Re sum_n gamma h exp((l+1) log q)
+// (fairseq/csrc/ops/ema_parameters.cc:37-77).  One thread per (row, block of 16 lags): the
+// block base power is taken from exp / sincos with the phase reduced in double, the 15
+// following powers by multiplication.
+constexpr int kLagBlock = 16;
+__global__ __launch_bounds__(kBlock) void ema_kernel_bias_kernel(const float* __restrict__ p,
+                                                                 const float* __restrict__ log_q,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* __restrict__ h, int B, int K,
+                                                                 int N, int L, float* w, float* bias) {
+  // rows: first K kernel rows, then B*K bias rows
+  const int nblk = (L + kLagBlock - 1) / kLagBlock;
+  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t rows = (int64_t)K + (h ? (int64_t)B * K : 0);
+  if (gid >= rows * nblk) return;
+  const int blk = (int)(gid % nblk);
+  const int64_t row = gid / nblk;
+  const bool is_bias = row >= K;
+  const int d = is_bias ? (int)((row - K) % K) : (int)row;
+  const int64_t bd = is_bias ? row - K : 0;
+  const int l0 = blk * kLagBlock;
+  const int e0 = is_bias ? l0 + 1 : l0;
+  float acc[kLagBlock];
+#pragma unroll
+  for (int i = 0; i < kLagBlock; ++i) acc[i] = 0.f;
+  for (int n = 0; n < N; ++n) {
+    const size_t o = ((size_t)d * N + n) * 2;
+    const double lr = log_q[o], li = log_q[o + 1];
+    double cr, ci;
+    if (is_bias) {
+      const size_t oh = ((size_t)bd * N + n) * 2;
+      const double gr = gamma[o], gi = gamma[o + 1], hr = h[oh], hi = h[oh + 1];
+      cr = gr * hr - gi * hi;
+      ci = gr * hi + gi * hr;
+    } else {
+      cr = (double)p[o / 2] * gamma[o];
+      ci = (double)p[o / 2] * gamma[o + 1];
+    }
+    const double mag = exp(lr * e0);
+    double ang = li * e0;
+    ang -= 6.283185307179586476925 * rint(ang * 0.15915494309189533577);
+    double sn, cs;
+    sincos(ang, &sn, &cs);
+    // v = c q^{e0}
+    float vr = (float)(mag * (cr * cs - ci * sn));
+    float vi = (float)(mag * (cr * sn + ci * cs));
+    const double m1 = exp(lr);
+    double s1, c1;
+    sincos(li, &s1, &c1);
+    const float qr = (float)(m1 * c1), qi = (float)(m1 * s1);
+#pragma unroll
+    for (int i = 0; i < kLagBlock; ++i) {
+      acc[i] += vr;
+      const float t = vr * qr - vi * qi;
+      vi = vr * qi + vi * qr;
+      vr = t;
+    }
+  }
+  float* out = is_bias ? bias + (size_t)bd * L : w + (size_t)d * L;
+#pragma unroll
+  for (int i = 0; i < kLagBlock; ++i)
+    if (l0 + i < L) out[l0 + i] = acc[i];
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" size_t mega_ema_fwd_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L,
+                                               int bidirectional, int64_t truncation) {
+  if (B <= 0 || D <= 0 || N <= 0 || L <= 0) return 256;
+  const bool trunc = truncation > 0 && truncation < L;
+  const bool need_acc = bidirectional || trunc;
+  return make_plan(B, D, N, L, 4, need_acc).total;
+}
+
+extern "C" size_t mega_ema_hidden_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L) {
+  if (B <= 0 || D <= 0 || N <= 0 || L <= 0) return 256;
+  return make_plan(B, D, N, L, 1, false).total;
+}
+
+static int check_common(const char* who, int dtype, int64_t B, int64_t D, int64_t N, int64_t L) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG, "%s: unknown dtype %d",
+               who, dtype);
+  MEGA_REQUIRE(B >= 0 && D > 0 && N > 0 && L >= 0, MEGA_ERR_ARG, "%s: bad shape B=%ld D=%ld N=%ld L=%ld", who,
+               (long)B, (long)D, (long)N, (long)L);
+  MEGA_REQUIRE(N <= 32, MEGA_ERR_UNSUPPORTED, "%s: ndim=%ld > 32 is not supported", who, (long)N);
+  MEGA_REQUIRE(B * D * 8 < (int64_t)1 << 31 && L < (int64_t)1 << 30, MEGA_ERR_UNSUPPORTED, "%s: shape too large",
+               who);
+  return MEGA_OK;
+}
+
+extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
+                            int64_t syb, int64_t syd, int64_t syl, const float* p, const float* q,
+                            const float* gamma, int is_complex, const float* omega, const uint8_t* mask,
+                            const float* h_in, float* h_out, int64_t B, int64_t D, int64_t N, int64_t L,
+                            int bidirectional, int64_t truncation, int shift, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+  int rc = check_common("ema_fwd", dtype, B, D, N, L);
+  if (rc) return rc;
+  MEGA_REQUIRE(!(bidirectional && (h_in || h_out)), MEGA_ERR_ARG,
+               "ema_fwd: bidirectional EMA does not support incremental state");
+  if (B == 0 || L == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && y && p && q && gamma && omega, MEGA_ERR_ARG, "ema_fwd: null pointer argument");
+  const int64_t Lk = (truncation > 0 && truncation < L) ? truncation : 0;
+  MEGA_REQUIRE(!(Lk > 0 && (h_in || h_out)), MEGA_ERR_UNSUPPORTED,
+               "ema_fwd: truncation together with incremental state is not supported");
+  const bool need_acc = bidirectional || Lk > 0;
+  const Plan pl = make_plan(B, D, N, L, 4, need_acc);
+  MEGA_REQUIRE(workspace && workspace_bytes >= pl.total, MEGA_ERR_WORKSPACE,
+               "ema_fwd: workspace of %zu bytes needed", pl.total);
+  hipStream_t s = (hipStream_t)stream;
+  char* w = (char*)workspace;
+  float* coef = (float*)w;
+  float* st = (float*)(w + pl.coef_bytes);
+  float* acc = need_acc ? (float*)(w + pl.coef_bytes + pl.st_bytes) : nullptr;
+  const int ndir = bidirectional ? 2 : 1;
+  {
+    const int64_t n = (int64_t)D * pl.NP * ndir;
+    hipLaunchKernelGGL(coef_prep_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, p, q, gamma, 0,
+                       is_complex ? 1 : 0, (int)D, (int)N, pl.NP, ndir, Lk, coef);
+    MEGA_CHECK_LAUNCH("ema_fwd coefficient prep");
+  }
+  // list of pass sets; the last one writes y
+  struct SetDesc { int set, reverse, before, tshift; };
+  SetDesc sets[4];
+  int ns = 0;
+  if (bidirectional) {
+    sets[ns++] = {2, 1, shift ? 1 : 0, 0};
+    if (Lk > 0) sets[ns++] = {3, 1, shift ? 1 : 0, (int)Lk};
+  }
+  if (Lk > 0) sets[ns++] = {1, 0, 0, (int)Lk};
+  sets[ns++] = {0, 0, 0, 0};
+  for (int i = 0; i < ns; ++i) {
+    PassArgs A;
+    A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
+    A.coef = coef_of(coef, sets[i].set, D, pl.NP);
+    const bool main_set = sets[i].set == 0;
+    A.h_in = main_set ? h_in : nullptr;
+    A.h_out = main_set ? h_out : nullptr;
+    A.st = st;
+    A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+    A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
+    A.reverse = sets[i].reverse; A.before = sets[i].before; A.tshift = sets[i].tshift;
+    A.acc_in = i > 0 ? acc : nullptr;
+    A.acc_out = i < ns - 1 ? acc : nullptr;
+    A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
+    A.omega = omega;
+    rc = run_pass_set_dtype(dtype, A, is_complex != 0, false, s);
+    if (rc) return rc;
+  }
+  return MEGA_OK;
+}
+
+extern "C" int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
+                                   const float* p, const float* log_q, const float* h, int64_t B, int64_t D,
+                                   int64_t N, int64_t L, float* h_out, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  int rc = check_common("ema_hidden_fwd", dtype, B, D, N, L);
+  if (rc) return rc;
+  if (B == 0) return MEGA_OK;
+  MEGA_REQUIRE(p && log_q && h_out && (L == 0 || x), MEGA_ERR_ARG, "ema_hidden_fwd: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  if (L == 0) {
+    if (h) hipMemcpyAsync(h_out, h, (size_t)B * D * N * 8, hipMemcpyDeviceToDevice, s);
+    else hipMemsetAsync(h_out, 0, (size_t)B * D * N * 8, s);
+    return MEGA_OK;
+  }
+  const Plan pl = make_plan(B, D, N, L, 1, false);
+  MEGA_REQUIRE(workspace && workspace_bytes >= pl.total, MEGA_ERR_WORKSPACE,
+               "ema_hidden_fwd: workspace of %zu bytes needed", pl.total);
+  char* w = (char*)workspace;
+  float* coef = (float*)w;
+  float* st = (float*)(w + pl.coef_bytes);
+  const int64_t n = (int64_t)D * pl.NP;
+  // gamma is not needed for the state; pass log_q as a stand-in that is never read as gamma
+  hipLaunchKernelGGL(coef_prep_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, p, log_q, log_q, 1, 1,
+                     (int)D, (int)N, pl.NP, 1, (int64_t)0, coef);
+  MEGA_CHECK_LAUNCH("ema_hidden_fwd coefficient prep");
+  PassArgs A;
+  A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = nullptr;
+  A.coef = coef_of(coef, 0, D, pl.NP);
+  A.h_in = h; A.h_out = h_out; A.st = st;
+  A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+  A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
+  A.reverse = 0; A.before = 0; A.tshift = 0;
+  A.acc_in = nullptr; A.acc_out = nullptr; A.y = nullptr; A.syb = A.syd = A.syl = 0; A.omega = nullptr;
+  return run_pass_set_dtype(dtype, A, true, true, s);
+}
+
+extern "C" int mega_ema_step(const void* x, void* y, int dtype, const float* p, const float* q,
+                             const float* gamma, int is_complex, const float* omega, const float* h_in,
+                             float* h_out, int64_t B, int64_t D, int64_t N, void* stream) {
+  int rc = check_common("ema_step", dtype, B, D, N, 1);
+  if (rc) return rc;
+  if (B == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && y && p && q && gamma && omega && h_out, MEGA_ERR_ARG, "ema_step: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)ceil_div(B * D, kBlock));
+#define LAUNCH_STEP(T, C)                                                                             \
+  hipLaunchKernelGGL((ema_step_kernel<T, C>), grid, dim3(kBlock), 0, s, (const T*)x, (T*)y, p, q, gamma, \
+                     omega, h_in, h_out, (int)B, (int)D, (int)N)
+  if (is_complex) {
+    if (dtype == MEGA_F32) LAUNCH_STEP(float, true);
+    else if (dtype == MEGA_BF16) LAUNCH_STEP(bf16_t, true);
+    else LAUNCH_STEP(f16_t, true);
+  } else {
+    if (dtype == MEGA_F32) LAUNCH_STEP(float, false);
+    else if (dtype == MEGA_BF16) LAUNCH_STEP(bf16_t, false);
+    else LAUNCH_STEP(f16_t, false);
+  }
+#undef LAUNCH_STEP
+  MEGA_CHECK_LAUNCH("ema_step");
+  return MEGA_OK;
+}
+
+extern "C" int mega_ema_parameters_fwd(const float* p, const float* log_q, const float* gamma, const float* h,
+                                       int64_t B, int64_t K, int64_t N, int64_t L, float* w, float* b,
+                                       void* stream) {
+  MEGA_REQUIRE(K > 0 && N > 0 && L >= 0 && B >= 0, MEGA_ERR_ARG, "ema_parameters_fwd: bad shape");
+  MEGA_REQUIRE(N <= 32, MEGA_ERR_UNSUPPORTED, "ema_parameters_fwd: ndim=%ld > 32 is not supported", (long)N);
+  MEGA_REQUIRE(p && log_q && gamma && w, MEGA_ERR_ARG, "ema_parameters_fwd: null pointer argument");
+  MEGA_REQUIRE(!h || b, MEGA_ERR_ARG, "ema_parameters_fwd: carried state given without a bias output");
+  if (L == 0) return MEGA_OK;
+  const int64_t rows = K + (h ? B * K : 0);
+  const int64_t nblk = ceil_div(L, kLagBlock);
+  MEGA_REQUIRE(rows * nblk < (int64_t)1 << 40, MEGA_ERR_UNSUPPORTED, "ema_parameters_fwd: shape too large");
+  hipLaunchKernelGGL(ema_kernel_bias_kernel, dim3((unsigned)ceil_div(rows * nblk, kBlock)), dim3(kBlock), 0,
+                     (hipStream_t)stream, p, log_q, gamma, h, (int)B, (int)K, (int)N, (int)L, w, b);
+  MEGA_CHECK_LAUNCH("ema_parameters_fwd");
+  return MEGA_OK;
+}

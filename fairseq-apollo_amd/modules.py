@@ -1,0 +1,390 @@
+"""Module surface: drop-in counterparts of the reference's PyTorch modules for the
+Mega/Mega2 sequence-mixing path, with the same constructor arguments, parameter names and
+shapes (so reference checkpoints load) and the same incremental-state keys.
+
+    MultiHeadEMA            fairseq/modules/exponential_moving_average.py:13-94
+    MultiHeadComplexEMA     fairseq/modules/complex_exponential_moving_average.py:15-113
+    (both on)  BaseMovingLayer  fairseq/modules/base_moving_average.py:18-197
+    TimestepNorm            fairseq/modules/norm_layer/timestep_norm.py:71-167
+    AttentionSoftmax        fairseq/modules/attention_softmax.py:44-56
+    EfficientAttention      fairseq/modules/efficient_attention.py:45-63
+    SwiGLU                  no counterpart in the reference (its FFN is
+                            fairseq/modules/normalized_feedforward_network.py:77-93)
+
+Forward / inference only: the HIP kernels have no backward pass yet, so a forward that
+would need gradients raises instead of silently detaching.
+"""
+from __future__ import annotations
+
+import math
+import uuid
+from collections import OrderedDict
+from typing import Dict, Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+from torch.nn.parameter import Parameter
+
+from . import ops
+
+
+class IncrementalState(object):
+    """Per-module namespacing of the shared incremental_state dict
+    (fairseq/incremental_decoding_utils.py:12-50)."""
+
+    def init_incremental_state(self):
+        self._incremental_state_id = str(uuid.uuid4())
+
+    def _get_full_incremental_state_key(self, key: str) -> str:
+        return "{}.{}".format(self._incremental_state_id, key)
+
+    def get_incremental_state(self, incremental_state, key: str):
+        full_key = self._get_full_incremental_state_key(key)
+        if incremental_state is None or full_key not in incremental_state:
+            return None
+        return incremental_state[full_key]
+
+    def set_incremental_state(self, incremental_state, key: str, value):
+        if incremental_state is not None:
+            incremental_state[self._get_full_incremental_state_key(key)] = value
+        return incremental_state
+
+
+def _no_grad_only(module: nn.Module, *tensors):
+    if torch.is_grad_enabled() and (
+        any(t is not None and t.requires_grad for t in tensors)
+        or any(p.requires_grad for p in module.parameters())
+    ):
+        raise RuntimeError(
+            f"{type(module).__name__}: the HIP path implements the forward pass only; "
+            "call it under torch.no_grad() (inference)"
+        )
+
+
+class BaseMovingLayer(nn.Module, IncrementalState):
+    """fairseq/modules/base_moving_average.py:18-197."""
+
+    def __init__(self, bidirectional=False, truncation=None, shift=True):
+        super().__init__()
+        self.init_incremental_state()
+        self._parameters_no_weight_decay = OrderedDict()
+        self.complex = False
+        self.bidirectional = bidirectional
+        self.truncation = truncation
+        self.shift = shift
+        self._coeffs = None
+        assert self.bidirectional or (self.truncation is None or self.truncation < 1), \
+            'one directional moving average should not have positive trunction: {}'.format(truncation)
+
+    def register_parameters_no_weight_decay(self, name, param):
+        self._parameters_no_weight_decay[name] = param
+
+    def parameters_no_weight_decay(self):
+        for name, param in self._parameters_no_weight_decay.items():
+            yield name, param
+
+    def _calc_coeffs(self):
+        raise NotImplementedError
+
+    def coeffs(self):
+        """(p, q, gamma); cached in eval mode like the reference (base_moving_average.py:52-58)."""
+        with torch.no_grad():           # forward only: coefficients never carry a graph
+            if self.training:
+                return self._calc_coeffs()
+            if self._coeffs is None:
+                self._coeffs = self._calc_coeffs()
+            return self._coeffs
+
+    def train(self, mode: bool = True):
+        self._coeffs = None
+        return super().train(mode)
+
+    def kernel(self, length: int, hx: Optional[Tensor] = None):
+        """(k[K, Lk], bias[B, K, L] or None) -- the materialised convolution kernel; the forward
+        pass does not use it (base_moving_average.py:60-62)."""
+        kernel_size = length if self.truncation is None or self.truncation < 1 else min(self.truncation, length)
+        p, q, gamma = self.coeffs()
+        w, b, _ = ops.ema_parameters_fwd(p.squeeze(-1), torch.log(q.squeeze(-1).to(torch.complex64)),
+                                         gamma.to(torch.complex64), hx, kernel_size)
+        return w, b
+
+    def one_step(self, x, hx=None):
+        """x: [B, D, 1] -> (out [B, D, 1] without the residual, h [B, D, N])
+        (base_moving_average.py:105-118)."""
+        p, q, gamma = self.coeffs()
+        zero = torch.zeros_like(self.omega.reshape(-1))
+        y, h = ops.ema_step(x.squeeze(-1), p.squeeze(-1), q.squeeze(-1), gamma, zero, hx)
+        return y.unsqueeze(-1), h
+
+    def forward(self, x, padding_mask: Optional[Tensor] = None,
+                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None) -> Tensor:
+        """x: [B, D, L]; padding_mask: [B, L] with 1 / True at padding; returns [B, D, L]."""
+        _no_grad_only(self, x)
+        bsz, embed_dim, seq_len = x.size()
+        assert embed_dim == self.embed_dim
+        assert not self.bidirectional or incremental_state is None, \
+            'Bidirectional EMA does not support incremental state'
+        p, q, gamma = self.coeffs()
+        p2, q2 = p.squeeze(-1), q.squeeze(-1)
+        omega = self.omega.reshape(-1)
+        if incremental_state is not None:
+            saved_state = self._get_input_buffer(incremental_state)
+            h = saved_state['prev_state'] if 'prev_state' in saved_state else None
+            out, h = ops.ema_forward(x, p2, q2, gamma, omega, padding_mask, h, want_state=True)
+            saved_state['prev_state'] = h
+            self._set_input_buffer(incremental_state, saved_state)
+        else:
+            out, _ = ops.ema_forward(x, p2, q2, gamma, omega, padding_mask, None, want_state=False,
+                                     bidirectional=self.bidirectional, truncation=self.truncation,
+                                     shift=self.shift)
+        return out
+
+    def _get_input_buffer(self, incremental_state):
+        result = self.get_incremental_state(incremental_state, "ema_state")
+        return result if result is not None else {}
+
+    def _set_input_buffer(self, incremental_state, buffer):
+        return self.set_incremental_state(incremental_state, "ema_state", buffer)
+
+    def reorder_incremental_state(self, incremental_state, new_order: Tensor):
+        """Reorder the carried state for beam search (base_moving_average.py:185-197)."""
+        input_buffer = self._get_input_buffer(incremental_state)
+        if input_buffer is not None:
+            for k in input_buffer.keys():
+                if input_buffer[k] is not None:
+                    input_buffer[k] = input_buffer[k].index_select(0, new_order)
+            incremental_state = self._set_input_buffer(incremental_state, input_buffer)
+        return incremental_state
+
+    def extra_repr(self) -> str:
+        return 'edim={}, ndim={}, bidirectional={}, trunction={}, shift={}'.format(
+            self.embed_dim, self.ndim, self.bidirectional, self.truncation, self.shift)
+
+
+class MultiHeadEMA(BaseMovingLayer):
+    """Real-valued multi-dimensional damped EMA
+    (fairseq/modules/exponential_moving_average.py:13-94).  The reference class is out of
+    step with its base class in this snapshot; this one implements the formulas it states
+    (q = 1 - s(alpha) s(delta), p = s(alpha) beta, gamma scaled by sqrt(1/N), omega per
+    channel) behind the same interface as the complex layer."""
+
+    def __init__(self, embed_dim, ndim=2, bidirectional=False, truncation=None, shift=True):
+        super().__init__(bidirectional, truncation, shift)
+        self.complex = False
+        self.embed_dim = embed_dim
+        self.ndim = ndim
+        self.scale = math.sqrt(1.0 / self.ndim)
+        kernel_dim = 2 * embed_dim if self.bidirectional else embed_dim
+        self.alpha = nn.Parameter(torch.Tensor(kernel_dim, ndim, 1))
+        self.delta = nn.Parameter(torch.Tensor(kernel_dim, ndim, 1))
+        self.beta = nn.Parameter(torch.Tensor(kernel_dim, ndim, 1))
+        self.gamma = nn.Parameter(torch.Tensor(kernel_dim, ndim))
+        self.omega = nn.Parameter(torch.Tensor(embed_dim))
+        self.register_parameters_no_weight_decay('alpha', self.alpha)
+        self.register_parameters_no_weight_decay('delta', self.delta)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        with torch.no_grad():
+            nn.init.normal_(self.alpha, mean=0.0, std=0.2)
+            nn.init.normal_(self.delta, mean=0.0, std=0.2)
+            # beta alternates +1 / -1 around a small normal perturbation
+            val = torch.ones(self.ndim, 1)
+            if self.ndim > 1:
+                val[1::2] = -1.0
+            self.beta.normal_(mean=0.0, std=0.02).add_(val)
+            nn.init.normal_(self.gamma, mean=0.0, std=1.0)
+            nn.init.normal_(self.omega, mean=0.0, std=1.0)
+
+    def _calc_coeffs(self):
+        self._coeffs = None
+        alpha = torch.sigmoid(self.alpha.float())
+        delta = torch.sigmoid(self.delta.float())
+        q = 1.0 - alpha * delta
+        p = alpha * self.beta.float()
+        gamma = self.gamma.float() * self.scale
+        return p, q, gamma
+
+
+class MultiHeadComplexEMA(BaseMovingLayer):
+    """Complex EMA of Mega2 (fairseq/modules/complex_exponential_moving_average.py:15-113)."""
+
+    def __init__(self, embed_dim, ndim=2, bidirectional=False, truncation=None, shift=True):
+        super().__init__(bidirectional, truncation, shift)
+        self.complex = True
+        self.embed_dim = embed_dim
+        self.ndim = ndim
+        self.scale = math.sqrt(1.0 / self.ndim)
+        kernel_dim = 2 * embed_dim if self.bidirectional else embed_dim
+        self.alpha = nn.Parameter(torch.Tensor(kernel_dim, ndim, 1))
+        self.delta = nn.Parameter(torch.Tensor(kernel_dim, ndim, 1))
+        self.theta = nn.Parameter(torch.Tensor(kernel_dim, 1, 1))
+        self.gamma = nn.Parameter(torch.Tensor(kernel_dim, ndim, 2))
+        self.omega = nn.Parameter(torch.Tensor(embed_dim, 1))
+        self.register_parameters_no_weight_decay('alpha', self.alpha)
+        self.register_parameters_no_weight_decay('delta', self.delta)
+        self.register_parameters_no_weight_decay('theta', self.theta)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        with torch.no_grad():
+            nn.init.normal_(self.alpha, mean=0.0, std=0.2)
+            nn.init.normal_(self.delta, mean=0.0, std=0.2)
+            # theta: logit of a random permutation of exp(-j ln(D) / D), j = 1..D
+            freqs = math.log(self.embed_dim) / self.embed_dim
+            freqs = torch.exp(torch.arange(1, self.embed_dim + 1) * -freqs)
+            freqs = freqs[torch.randperm(self.embed_dim)].to(self.theta).view(self.embed_dim, 1, 1)
+            if self.bidirectional:
+                freqs = freqs.repeat(2, 1, 1)
+            self.theta.copy_(torch.log(freqs / (1.0 - freqs)))
+            nn.init.normal_(self.gamma, mean=0.0, std=1.0)
+            self.gamma[:, :, 1] = 0.
+            nn.init.normal_(self.omega, mean=0.0, std=1.0)
+
+    def _calc_coeffs(self):
+        self._coeffs = None
+        theta = torch.sigmoid(self.theta.float()) * (2 * math.pi / self.ndim)
+        wavelets = torch.arange(1, self.ndim + 1, dtype=theta.dtype, device=theta.device).view(1, self.ndim)
+        theta = wavelets.unsqueeze(2) * theta
+        alpha = torch.sigmoid(self.alpha.float())
+        delta = torch.sigmoid(self.delta.float())
+        p = alpha
+        q = torch.polar(1.0 - alpha * delta, theta)
+        gamma = torch.view_as_complex(self.gamma.float().contiguous()) * self.scale
+        return p, q, gamma
+
+
+class TimestepNorm(nn.Module, IncrementalState):
+    """Streaming cumulative (group) normalisation with a carried (count, mean, var) state
+    (fairseq/modules/norm_layer/timestep_norm.py:71-167).  mean / var are carried in fp32."""
+
+    def __init__(self, num_features: int, num_groups: Optional[int] = None, prior_count: int = 0,
+                 eps: float = 1e-5) -> None:
+        super().__init__()
+        self.init_incremental_state()
+        self.num_features = num_features
+        self.num_groups = num_groups
+        self._prior_count = prior_count
+        if num_groups is None or num_groups == num_features:
+            num_groups = num_features
+            assert prior_count > 1
+        else:
+            assert self.num_features % num_groups == 0
+        self.register_buffer("prior_count", torch.tensor(prior_count, dtype=torch.int64))
+        if prior_count > 0:
+            self.register_parameter("prior_mean", Parameter(torch.zeros(num_groups), requires_grad=True))
+            self.register_parameter("prior_logv", Parameter(torch.zeros(num_groups), requires_grad=True))
+        else:
+            self.register_buffer("prior_mean", torch.zeros(num_groups))
+            self.register_buffer("prior_logv", torch.zeros(num_groups))
+        self.register_parameter("weight", Parameter(torch.zeros(num_features), requires_grad=True))
+        self.register_parameter("bias", Parameter(torch.zeros(num_features), requires_grad=True))
+        self.eps = eps
+
+    def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
+                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None) -> Tensor:
+        _no_grad_only(self, x)
+        batch_size = x.size(0)
+        prev_mean = prev_var = prev_count = None
+        saved_state = None
+        if incremental_state is not None:
+            saved_state = self._get_input_buffer(incremental_state)
+            if 'prev_mean' in saved_state:
+                prev_mean = saved_state['prev_mean']
+                assert 'prev_var' in saved_state and 'prev_count' in saved_state
+                prev_var = saved_state['prev_var']
+                prev_count = saved_state['prev_count']
+        if prev_count is None:
+            prev_count = self.prior_count.expand(batch_size).contiguous()
+        if prev_mean is None:
+            prev_mean = self.prior_mean.expand(batch_size, -1).contiguous()
+        if prev_var is None:
+            prev_var = torch.exp(self.prior_logv).expand(batch_size, -1).contiguous()
+        gamma = self.weight.float() + 1.0
+        if self.num_groups is None:
+            out, count, mean, var, _, _ = ops.timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, self.bias,
+                                                                padding_mask, self.eps, need_stats=False)
+        else:
+            out, count, mean, var, _, _, _ = ops.group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma,
+                                                                         self.bias, padding_mask, self.num_groups,
+                                                                         self.eps, need_stats=False)
+        if incremental_state is not None:
+            saved_state['prev_mean'] = mean
+            saved_state['prev_var'] = var
+            saved_state['prev_count'] = count
+            self._set_input_buffer(incremental_state, saved_state)
+        return out
+
+    def _get_input_buffer(self, incremental_state):
+        result = self.get_incremental_state(incremental_state, "norm_state")
+        return result if result is not None else {}
+
+    def _set_input_buffer(self, incremental_state, buffer):
+        return self.set_incremental_state(incremental_state, "norm_state", buffer)
+
+    def reorder_incremental_state(self, incremental_state, new_order: Tensor):
+        input_buffer = self._get_input_buffer(incremental_state)
+        if input_buffer is not None:
+            for k in input_buffer.keys():
+                if input_buffer[k] is not None:
+                    input_buffer[k] = input_buffer[k].index_select(0, new_order)
+            incremental_state = self._set_input_buffer(incremental_state, input_buffer)
+        return incremental_state
+
+    def extra_repr(self) -> str:
+        return 'num_features={num_features}, num_groups={num_groups}, prior_count={_prior_count}, eps={eps}'.format(
+            **self.__dict__)
+
+
+class AttentionSoftmax(nn.Module):
+    """fairseq/modules/attention_softmax.py:44-56."""
+
+    def __init__(self, dropout: float = 0.0, use_causal_mask: bool = False) -> None:
+        super().__init__()
+        self._dropout = dropout
+        self._causal = use_causal_mask
+
+    def forward(self, x: Tensor) -> Tensor:
+        _no_grad_only(self, x)
+        return ops.attention_softmax_fwd(x, self._dropout if self.training else 0.0, self._causal)
+
+    def extra_repr(self) -> str:
+        return 'causal={}, dropout={}'.format(self._causal, self._dropout)
+
+
+class EfficientAttention(nn.Module):
+    """fairseq/modules/efficient_attention.py:45-63: q, k: [B, L, H1], v: [B, L, H2]
+    (single head), or the 4-D [B, L, Nh, H] layout of the op itself."""
+
+    def __init__(self, scale: float = 1.0, dropout: float = 0.0, use_causal_mask: bool = True) -> None:
+        super().__init__()
+        self._scale = scale
+        self._dropout = dropout
+        self._causal = use_causal_mask
+
+    def forward(self, q: Tensor, k: Tensor, v: Tensor) -> Tensor:
+        _no_grad_only(self, q, k, v)
+        squeeze = q.dim() == 3
+        if squeeze:
+            q, k, v = q.unsqueeze(2), k.unsqueeze(2), v.unsqueeze(2)
+        out, _ = ops.attention_fwd(q, k, v, self._scale, self._dropout if self.training else 0.0, self._causal)
+        return out.squeeze(2) if squeeze else out
+
+    def extra_repr(self) -> str:
+        return 'causal={}, dropout={}'.format(self._causal, self._dropout)
+
+
+class SwiGLU(nn.Module):
+    """W2 (silu(W1 x) * W3 x) with the gate evaluated by the HIP kernel; the three
+    projections are library GEMMs."""
+
+    def __init__(self, embed_dim: int, hidden_dim: int, bias: bool = False) -> None:
+        super().__init__()
+        self.w1 = nn.Linear(embed_dim, hidden_dim, bias=bias)
+        self.w3 = nn.Linear(embed_dim, hidden_dim, bias=bias)
+        self.w2 = nn.Linear(hidden_dim, embed_dim, bias=bias)
+
+    def forward(self, x: Tensor) -> Tensor:
+        _no_grad_only(self, x)
+        return self.w2(ops.swiglu(self.w1(x), self.w3(x)))

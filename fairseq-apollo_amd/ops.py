@@ -1,0 +1,392 @@
+"""Operator surface: the functions fairseq model code reaches through
+`fairseq.mega2_extension.ops` (fairseq/csrc/mega2_extension.cc:14-24), with the same names,
+argument order and return tuples, plus the fused inference entry points the modules use.
+
+Every function takes torch tensors that live on a HIP device, allocates its outputs with
+torch (so they belong to the caller, as torch::empty_like does in the reference), and
+enqueues the HIP kernels of libmega_hip.so on torch's current stream.  CPU tensors are
+rejected: there is no fallback.  Forward only (inference); dropout must be 0.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import BF16, F16, F32
+
+_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported activation dtype {t.dtype} (float32, bfloat16, float16)") from None
+
+
+def _need_gpu(*ts) -> torch.device:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("mega HIP ops need tensors on a HIP device; there is no CPU path")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(dev: torch.device):
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _f32c(t: torch.Tensor) -> torch.Tensor:
+    return t.detach().to(torch.float32).contiguous()
+
+
+def _cplx_as_f32(t: torch.Tensor) -> torch.Tensor:
+    """complex [...] -> float32 [..., 2]; real [...] -> [..., 2] with a zero imaginary part."""
+    t = t.detach()
+    if t.is_complex():
+        return torch.view_as_real(t.to(torch.complex64).contiguous()).contiguous()
+    return torch.stack([t.to(torch.float32), torch.zeros_like(t, dtype=torch.float32)], dim=-1).contiguous()
+
+
+_tsn_ws = {}
+
+
+def _tsn_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Zero-filled once; the kernels leave it zero-filled, so it is reused per (device, stream)."""
+    key = (dev.index, _stream(dev))
+    ws = _tsn_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
+        _tsn_ws[key] = ws
+    return ws
+
+
+def timestep_norm_status(dev=None) -> int:
+    """Error word of the TimestepNorm workspaces of `dev` (non-zero: a tile gave up waiting for
+    an earlier tile).  Synchronises; meant for tests and debugging."""
+    bad = 0
+    for (idx, _), ws in _tsn_ws.items():
+        if dev is None or torch.device(dev).index in (None, idx):
+            bad |= int(ws[8:12].view(torch.int32).item())
+    return bad
+
+
+# --------------------------------------------------------------------------------------
+# ops with the reference's names
+# --------------------------------------------------------------------------------------
+
+
+def ema_parameters_fwd(p: torch.Tensor, log_q: torch.Tensor, gamma: torch.Tensor,
+                       h: Optional[torch.Tensor], L: int):
+    """-> (w[K,L], b[B,K,L] or None, None).  Reference: ema_parameters_fwd,
+    fairseq/csrc/ops/ema_parameters.cc:211-286.  The Vandermonde tensor the reference saves
+    for its backward pass is not produced (third value None)."""
+    dev = _need_gpu(p, log_q, gamma, h)
+    lib = _lib.load()
+    K, N = p.shape[0], p.shape[1]
+    pf = _f32c(p).reshape(K, N)
+    lq = _cplx_as_f32(log_q.reshape(K, N))
+    g = _cplx_as_f32(gamma.reshape(K, N))
+    w = torch.empty(K, L, dtype=torch.float32, device=dev)
+    hb = b = None
+    B = 0
+    if h is not None:
+        B = h.shape[0]
+        hb = _cplx_as_f32(h.reshape(B, K, N))
+        b = torch.empty(B, K, L, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mega_ema_parameters_fwd(_ptr(pf), _ptr(lq), _ptr(g), _ptr(hb), B, K, N, L, _ptr(w), _ptr(b),
+                                         _stream(dev))
+    _lib.check(rc, "ema_parameters_fwd")
+    return w, b, None
+
+
+def ema_hidden_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, h: Optional[torch.Tensor]):
+    """-> (h'[B,D,N] complex64, None).  Reference: ema_hidden_fwd,
+    fairseq/csrc/ops/ema_hidden.cc:163-194."""
+    dev = _need_gpu(x, p, log_q, h)
+    lib = _lib.load()
+    B, D, L = x.shape
+    N = p.shape[1]
+    pf = _f32c(p).reshape(D, N)
+    lq = _cplx_as_f32(log_q.reshape(D, N))
+    hb = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
+    out = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev)
+    nws = lib.mega_ema_hidden_workspace_bytes(B, D, N, L)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    xd = x.detach()
+    with torch.cuda.device(dev):
+        rc = lib.mega_ema_hidden_fwd(_ptr(xd), _dtype_code(xd), xd.stride(0), xd.stride(1), xd.stride(2), _ptr(pf),
+                                     _ptr(lq), _ptr(hb), B, D, N, L, _ptr(out), _ptr(ws), nws, _stream(dev))
+    _lib.check(rc, "ema_hidden_fwd")
+    return torch.view_as_complex(out), None
+
+
+def _norm_state(prev_count, prev_mean, prev_var, B, G, dev):
+    pc = prev_count.detach().to(device=dev, dtype=torch.int64).contiguous()
+    pm = _f32c(prev_mean).reshape(B, G)
+    pv = _f32c(prev_var).reshape(B, G)
+    return pc, pm, pv
+
+
+def _mask_u8(mask: Optional[torch.Tensor], B: int, L: int):
+    if mask is None:
+        return None
+    m = mask.detach()
+    if m.shape != (B, L):
+        raise RuntimeError(f"padding_mask must have shape ({B}, {L}), got {tuple(m.shape)}")
+    if m.dtype == torch.bool:
+        return m.contiguous().view(torch.uint8)
+    return (m != 0).contiguous().view(torch.uint8)
+
+
+def group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, num_groups: int,
+                            eps: float, need_stats: bool = True):
+    """-> (y, count[B] int64, mean[B,G], var[B,G], group_mean, cummean, cumrstd) with the last
+    three [B,L,G] fp32 (None when need_stats is False; they only serve a backward pass).
+    Reference: group_timestep_norm_fwd, fairseq/csrc/ops/timestep_norm.cc:568-636.
+    mean / var are carried in fp32 whatever the activation dtype."""
+    dev = _need_gpu(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask)
+    lib = _lib.load()
+    if x.dim() != 3:
+        raise RuntimeError("x must be [B, L, H]")
+    B, L, H = x.shape
+    G = int(num_groups)
+    if G <= 0 or H % G != 0:
+        raise RuntimeError(f"num_features={H} is not divisible by num_groups={G}")
+    xd = x.detach().contiguous()
+    dt = _dtype_code(xd)
+    y = torch.empty_like(xd)
+    pc, pm, pv = _norm_state(prev_count, prev_mean, prev_var, B, G, dev)
+    count = torch.empty(B, dtype=torch.int64, device=dev)
+    mean = torch.empty(B, G, dtype=torch.float32, device=dev)
+    var = torch.empty(B, G, dtype=torch.float32, device=dev)
+    gm = cm = cr = None
+    if need_stats:
+        gm = torch.empty(B, L, G, dtype=torch.float32, device=dev)
+        cm = torch.empty_like(gm)
+        cr = torch.empty_like(gm)
+    nws = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, G)
+    ws = _tsn_workspace(dev, nws)
+    m8 = _mask_u8(padding_mask, B, L)
+    gf, bf = _f32c(gamma), _f32c(beta)
+    with torch.cuda.device(dev):
+        rc = lib.mega_group_timestep_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf),
+                                              _ptr(m8), B, L, H, G, float(eps), _ptr(count), _ptr(mean), _ptr(var),
+                                              _ptr(gm), _ptr(cm), _ptr(cr), _ptr(ws), ws.numel(), _stream(dev))
+    _lib.check(rc, "group_timestep_norm_fwd")
+    return y, count, mean, var, gm, cm, cr
+
+
+def timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, eps: float,
+                      need_stats: bool = True):
+    """-> (y, count, mean[B,H], var[B,H], cummean, cumrstd).  Reference: timestep_norm_fwd,
+    fairseq/csrc/ops/timestep_norm.cc:452-510 (per-feature running statistics)."""
+    dev = _need_gpu(x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask)
+    lib = _lib.load()
+    B, L, H = x.shape
+    xd = x.detach().contiguous()
+    dt = _dtype_code(xd)
+    y = torch.empty_like(xd)
+    pc, pm, pv = _norm_state(prev_count, prev_mean, prev_var, B, H, dev)
+    count = torch.empty(B, dtype=torch.int64, device=dev)
+    mean = torch.empty(B, H, dtype=torch.float32, device=dev)
+    var = torch.empty(B, H, dtype=torch.float32, device=dev)
+    cm = cr = None
+    if need_stats:
+        cm = torch.empty(B, L, H, dtype=torch.float32, device=dev)
+        cr = torch.empty_like(cm)
+    m8 = _mask_u8(padding_mask, B, L)
+    gf, bf = _f32c(gamma), _f32c(beta)
+    with torch.cuda.device(dev):
+        rc = lib.mega_timestep_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf),
+                                        _ptr(m8), B, L, H, float(eps), _ptr(count), _ptr(mean), _ptr(var), _ptr(cm),
+                                        _ptr(cr), None, 0, _stream(dev))
+    _lib.check(rc, "timestep_norm_fwd")
+    return y, count, mean, var, cm, cr
+
+
+def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
+    """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18."""
+    if dropout != 0.0:
+        raise RuntimeError("attention_softmax_fwd: DropKey dropout (training) is not implemented; pass 0")
+    dev = _need_gpu(x)
+    lib = _lib.load()
+    if x.dim() < 2:
+        raise RuntimeError("x must have at least 2 dimensions")
+    xd = x.detach().contiguous()
+    outer, inner = xd.shape[-2], xd.shape[-1]
+    batch = xd.numel() // max(outer * inner, 1)
+    y = torch.empty_like(xd)
+    with torch.cuda.device(dev):
+        rc = lib.mega_attention_softmax_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), batch, outer, inner,
+                                            1 if use_causal_mask else 0, _stream(dev))
+    _lib.check(rc, "attention_softmax_fwd")
+    return y
+
+
+def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, need_weights: bool = False):
+    """-> (y[B,L,Nh,H2], w[B,Nh,L,L] or None).  Reference: attention_fwd,
+    fairseq/csrc/ops/attention_kernel.cu:40-131; the L x L weights are only written on request."""
+    if dropout != 0.0:
+        raise RuntimeError("attention_fwd: dropout (training) is not implemented; pass 0")
+    dev = _need_gpu(q, k, v)
+    lib = _lib.load()
+    if q.dim() != 4 or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise RuntimeError("attention_fwd: q, k must be [B,L,N,H1] and v [B,L,N,H2]")
+    qd, kd, vd = (t.detach().contiguous() for t in (q, k, v))
+    if not (qd.dtype == kd.dtype == vd.dtype):
+        raise RuntimeError("attention_fwd: q, k, v must share one dtype")
+    B, L, Nh, H1 = qd.shape
+    H2 = vd.shape[3]
+    y = torch.empty(B, L, Nh, H2, dtype=qd.dtype, device=dev)
+    w = torch.empty(B, Nh, L, L, dtype=qd.dtype, device=dev) if need_weights else None
+    with torch.cuda.device(dev):
+        rc = lib.mega_attention_fwd(_ptr(qd), _ptr(kd), _ptr(vd), _ptr(y), _ptr(w), _dtype_code(qd), B, L, Nh, H1, H2,
+                                    float(scale), 1 if use_causal_mask else 0, _stream(dev))
+    _lib.check(rc, "attention_fwd")
+    return y, w
+
+
+# --------------------------------------------------------------------------------------
+# fused inference entry points used by the modules
+# --------------------------------------------------------------------------------------
+
+
+def ema_forward(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, omega: torch.Tensor,
+                padding_mask: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
+                want_state: bool = False, bidirectional: bool = False, truncation: Optional[int] = None,
+                shift: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Whole moving-average layer in one call (BaseMovingLayer.forward,
+    fairseq/modules/base_moving_average.py:120-172).
+
+    x: [B, D, L] (any strides; a transposed view of a [B, L, D] tensor is read in place);
+    p: [K, N]; q, gamma: [K, N] real or complex; omega: [D]; h: [B, D, N] carried state.
+    Returns (y, h') with y shaped [B, D, L] in x's memory layout and h' complex64 (or None).
+    """
+    dev = _need_gpu(x, p, q, gamma, omega, padding_mask, h)
+    lib = _lib.load()
+    if x.dim() != 3:
+        raise RuntimeError("x must be [B, D, L]")
+    B, D, L = x.shape
+    K = 2 * D if bidirectional else D
+    N = p.shape[1]
+    if p.shape[0] != K:
+        raise RuntimeError(f"coefficient rows {p.shape[0]} do not match kernel_dim {K}")
+    is_complex = q.is_complex() or gamma.is_complex()
+    xd = x.detach()
+    dt = _dtype_code(xd)
+    if 0 in xd.stride() and xd.numel() > 0:
+        xd = xd.contiguous()
+    y = torch.empty_strided(xd.shape, xd.stride(), dtype=xd.dtype, device=dev) if _dense(xd) else torch.empty_like(
+        xd, memory_format=torch.contiguous_format)
+    pf = _f32c(p).reshape(K, N)
+    qf = _cplx_as_f32(q.reshape(K, N))
+    gf = _cplx_as_f32(gamma.reshape(K, N))
+    of = _f32c(omega).reshape(D)
+    m8 = _mask_u8(padding_mask, B, L)
+    hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
+    hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev) if (want_state or h is not None) else None
+    trunc = 0 if truncation is None or truncation < 1 else int(truncation)
+    nws = lib.mega_ema_fwd_workspace_bytes(B, D, N, L, 1 if bidirectional else 0, trunc)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mega_ema_fwd(_ptr(xd), _ptr(y), dt, xd.stride(0), xd.stride(1), xd.stride(2), y.stride(0),
+                              y.stride(1), y.stride(2), _ptr(pf), _ptr(qf), _ptr(gf), 1 if is_complex else 0,
+                              _ptr(of), _ptr(m8), _ptr(hin), _ptr(hout), B, D, N, L, 1 if bidirectional else 0,
+                              trunc, 1 if shift else 0, _ptr(ws), nws, _stream(dev))
+    _lib.check(rc, "ema_fwd")
+    hc = None
+    if hout is not None:
+        hc = torch.view_as_complex(hout) if is_complex else hout[..., 0]
+    return y, hc
+
+
+def _dense(t: torch.Tensor) -> bool:
+    """True when the tensor's strides describe a permutation of a contiguous block."""
+    if t.numel() == 0:
+        return False
+    pairs = sorted(((s, n) for s, n in zip(t.stride(), t.shape) if n > 1), reverse=True)
+    expect = 1
+    for s, n in reversed(pairs):
+        if s != expect:
+            return False
+        expect *= n
+    return True
+
+
+def ema_step(x_t: torch.Tensor, p, q, gamma, omega, h: Optional[torch.Tensor]):
+    """One decode step: x_t [B, D] -> (y_t [B, D], h' [B, D, N]).
+    BaseMovingLayer.one_step, fairseq/modules/base_moving_average.py:105-118, plus omega x."""
+    dev = _need_gpu(x_t, p, q, gamma, omega, h)
+    lib = _lib.load()
+    B, D = x_t.shape
+    N = p.shape[1]
+    is_complex = q.is_complex() or gamma.is_complex()
+    xd = x_t.detach().contiguous()
+    y = torch.empty_like(xd)
+    pf = _f32c(p).reshape(D, N)
+    qf = _cplx_as_f32(q.reshape(D, N))
+    gf = _cplx_as_f32(gamma.reshape(D, N))
+    of = _f32c(omega).reshape(D)
+    hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
+    hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.mega_ema_step(_ptr(xd), _ptr(y), _dtype_code(xd), _ptr(pf), _ptr(qf), _ptr(gf),
+                               1 if is_complex else 0, _ptr(of), _ptr(hin), _ptr(hout), B, D, N, _stream(dev))
+    _lib.check(rc, "ema_step")
+    return y, (torch.view_as_complex(hout) if is_complex else hout[..., 0])
+
+
+def fftconv(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    """Causal long convolution with an explicit kernel k[D, Lk] (fftconv,
+    fairseq/modules/fused_ops/fftconv.py:11-27); evaluated in the time domain."""
+    return _long_conv(x, k, False, True)
+
+
+def bidirectional_fftconv(x: torch.Tensor, k: torch.Tensor, shift: bool = True) -> torch.Tensor:
+    """bidirectional_fftconv, fairseq/modules/fused_ops/fftconv.py:85-100; k is [2D, Lk]."""
+    return _long_conv(x, k, True, shift)
+
+
+def _long_conv(x, k, bidirectional, shift):
+    dev = _need_gpu(x, k)
+    lib = _lib.load()
+    B, D, L = x.shape
+    xd = x.detach().contiguous()
+    kf = _f32c(k)
+    if kf.shape[0] != (2 * D if bidirectional else D):
+        raise RuntimeError("kernel rows do not match the channel count")
+    Lk = kf.shape[1]
+    y = torch.empty_like(xd)
+    with torch.cuda.device(dev):
+        rc = lib.mega_long_conv_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), _ptr(kf), B, D, L, Lk,
+                                    1 if bidirectional else 0, 1 if shift else 0, _stream(dev))
+    _lib.check(rc, "long_conv_fwd")
+    return y
+
+
+def swiglu(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """silu(a) * b, elementwise."""
+    dev = _need_gpu(a, b)
+    lib = _lib.load()
+    if a.shape != b.shape or a.dtype != b.dtype:
+        raise RuntimeError("swiglu: a and b must have the same shape and dtype")
+    ad, bd = a.detach().contiguous(), b.detach().contiguous()
+    y = torch.empty_like(ad)
+    with torch.cuda.device(dev):
+        rc = lib.mega_swiglu_fwd(_ptr(ad), _ptr(bd), _ptr(y), _dtype_code(ad), ad.numel(), _stream(dev))
+    _lib.check(rc, "swiglu_fwd")
+    return y

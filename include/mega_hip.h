@@ -1,0 +1,189 @@
+/* mega_hip.h -- C ABI of libmega_hip.so: the Mega/Mega2 sequence-mixing hot path
+ * (EMA kernel generation, long causal / bidirectional convolution, TimestepNorm,
+ * chunked attention softmax, SwiGLU gate) as hand-written HIP kernels for gfx950.
+ *
+ * Conventions (every entry point):
+ *  - plain pointers and sizes only; every data pointer is DEVICE memory of the
+ *    current HIP device unless the comment says "host";
+ *  - outputs are caller-allocated, inputs are never written;
+ *  - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *    default stream) and the call returns without synchronising;
+ *  - the library never allocates device memory: scratch comes in through
+ *    `workspace` (size from the matching *_workspace_bytes query).  A workspace
+ *    that is handed to mega_*_timestep_norm_fwd must be zero-filled once when it
+ *    is created; the kernels leave it zero-filled again, so it can be reused by
+ *    later calls on the same stream.  Calls that share one workspace must not
+ *    overlap in time;
+ *  - return value 0 = launched; a negative value = rejected before anything was
+ *    launched (MEGA_ERR_*), with a human-readable reason in mega_last_error()
+ *    (thread-local).  This mirrors the TORCH_CHECK -> RuntimeError behaviour of
+ *    the reference ops; the Python host raises RuntimeError from it.
+ *
+ * The reference has no C ABI: its boundary is C++ functions over torch::Tensor
+ * exported by pybind11 as fairseq.mega2_extension.ops
+ * (fairseq/csrc/mega2_extension.cc:14-24).  Each entry point below cites the
+ * reference function it stands in for.
+ */
+#ifndef MEGA_HIP_H_
+#define MEGA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of activations */
+enum { MEGA_F32 = 0, MEGA_BF16 = 1, MEGA_F16 = 2 };
+
+/* error codes */
+enum {
+  MEGA_OK = 0,
+  MEGA_ERR_ARG = -1,       /* bad shape / pointer / flag                     */
+  MEGA_ERR_UNSUPPORTED = -2, /* valid request outside the implemented envelope */
+  MEGA_ERR_WORKSPACE = -3, /* workspace missing or too small                 */
+  MEGA_ERR_LAUNCH = -4     /* hipLaunchKernel reported an error              */
+};
+
+/* reason for the last negative return on this thread (never NULL) */
+const char* mega_last_error(void);
+
+/* library version, bumped when a signature changes */
+int mega_abi_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* EMA coefficients -> convolution kernel and carried-state bias            */
+/* stands in for ema_parameters_fwd (fairseq/csrc/ops/ema_parameters.cc:211-286,
+ * CUDA side ops/ema_parameters_kernel.cu:446-525; Python caller
+ * fairseq/modules/fused_ops/ema_parameters.py:13-20).
+ *   p      [K,N]      real
+ *   log_q  [K,N,2]    complex (re,im) -- principal log of q, as the reference passes it
+ *   gamma  [K,N,2]    complex
+ *   h      [B,K,N,2]  complex carried state, or NULL
+ *   w      [K,L]      out: w[d,l] = Re sum_n p gamma exp(l log q)
+ *   b      [B,K,L]    out (only if h != NULL): Re sum_n gamma h exp((l+1) log q)
+ * N <= 32 (the limit of the reference, ema_parameters_kernel.cu:455).            */
+int mega_ema_parameters_fwd(const float* p, const float* log_q, const float* gamma,
+                            const float* h, int64_t B, int64_t K, int64_t N, int64_t L,
+                            float* w, float* b, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* EMA hidden state after a chunk                                            */
+/* stands in for ema_hidden_fwd (fairseq/csrc/ops/ema_hidden.cc:163-194, CUDA
+ * side ops/ema_hidden_kernel.cu:472-536; caller fused_ops/ema_hidden.py:13-17).
+ *   x      [B,D,L] activations of type `dtype`, element strides (sxb,sxd,sxl)
+ *   p      [D,N]; log_q [D,N,2]; h [B,D,N,2] or NULL
+ *   h_out  [B,D,N,2]: p sum_j q^{L-1-j} x_j + q^L h                              */
+size_t mega_ema_hidden_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L);
+int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
+                        const float* p, const float* log_q, const float* h, int64_t B,
+                        int64_t D, int64_t N, int64_t L, float* h_out, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Fused moving-average layer forward                                        */
+/* stands in for BaseMovingLayer.forward as a whole
+ * (fairseq/modules/base_moving_average.py:120-172): mask, kernel generation
+ * (ema_parameters), long convolution (fftconv / bidirectional_fftconv,
+ * fairseq/modules/fused_ops/fftconv.py:11-27, 85-100), carried-state bias,
+ * ema_hidden and the omega residual in one pass over x.  The D x L kernel is
+ * never materialised.
+ *   x, y    [B,D,L] of `dtype` with element strides (sxb,sxd,sxl) / (syb,syd,syl);
+ *           any of the two contiguous layouts [B,D,L] or [B,L,D] is streamed coalesced
+ *   p       [K,N] real, q [K,N,2] complex (q itself, not its log), gamma [K,N,2]
+ *           complex already scaled by sqrt(1/N); K = D, or 2D when bidirectional
+ *   is_complex   0: imaginary parts are ignored / assumed zero (real EMA)
+ *   omega   [D]
+ *   mask    [B,L] bytes, non-zero = padding, or NULL
+ *   h_in    [B,D,N,2] carried state or NULL; h_out [B,D,N,2] or NULL
+ *           (both must be NULL when bidirectional)
+ *   truncation  <= 0: kernel length L; otherwise min(truncation, L)
+ *   shift   bidirectional only: 1 = the backward half starts at lag 1            */
+size_t mega_ema_fwd_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L,
+                                    int bidirectional, int64_t truncation);
+int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
+                 int64_t syb, int64_t syd, int64_t syl, const float* p, const float* q,
+                 const float* gamma, int is_complex, const float* omega,
+                 const uint8_t* mask, const float* h_in, float* h_out, int64_t B,
+                 int64_t D, int64_t N, int64_t L, int bidirectional, int64_t truncation,
+                 int shift, void* workspace, size_t workspace_bytes, void* stream);
+
+/* One decode step of the same layer: h' = q h + p x, y = Re sum gamma h' + omega x
+ * (BaseMovingLayer.one_step, fairseq/modules/base_moving_average.py:105-118, and the
+ * L = 1 case of forward with incremental_state).
+ *   x, y [B,D] of `dtype` (contiguous); h_in may be NULL (zero state); h_out [B,D,N,2];
+ *   h_out may alias h_in.                                                         */
+int mega_ema_step(const void* x, void* y, int dtype, const float* p, const float* q,
+                  const float* gamma, int is_complex, const float* omega, const float* h_in,
+                  float* h_out, int64_t B, int64_t D, int64_t N, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Long convolution with an explicit time-domain kernel                      */
+/* stands in for fftconv(x, k) (fairseq/modules/fused_ops/fftconv.py:11-27, 45-61;
+ * fused CUDA op fftconv_fwd, ops/fftconv_kernel.cu:431-470) and
+ * bidirectional_fftconv (fused_ops/fftconv.py:85-100).
+ *   x, y [B,D,L] contiguous of `dtype`; k [K,Lk] fp32, K = D (causal) or 2D
+ *   (bidirectional), Lk <= L.                                                    */
+int mega_long_conv_fwd(const void* x, void* y, int dtype, const float* k, int64_t B,
+                       int64_t D, int64_t L, int64_t Lk, int bidirectional, int shift,
+                       void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* TimestepNorm                                                               */
+/* group variant: stands in for group_timestep_norm_fwd
+ * (fairseq/csrc/ops/timestep_norm.cc:568-636, CUDA side
+ * ops/timestep_norm_kernel.cu:712-784; caller norm_layer/timestep_norm.py:35).
+ *   x, y         [B,L,H] contiguous of `dtype`
+ *   prev_count   [B] int64; prev_mean, prev_var [B,G] fp32
+ *   gamma, beta  [H] fp32 (gamma is weight + 1, as the module passes it)
+ *   mask         [B,L] bytes, non-zero = padding, or NULL
+ *   count [B] int64, mean, var [B,G] fp32: state after the last token
+ *   group_mean, cummean, cumrstd: [B,L,G] fp32 each, or NULL to skip (they exist for
+ *   the backward pass only)
+ * per-feature variant (G == H): stands in for timestep_norm_fwd
+ * (timestep_norm.cc:452-510; timestep_norm_kernel.cu:602-654); here prev_mean,
+ * prev_var, mean, var, cummean, cumrstd have H in place of G and group_mean is unused. */
+size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G);
+int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* prev_count,
+                                 const float* prev_mean, const float* prev_var,
+                                 const float* gamma, const float* beta, const uint8_t* mask,
+                                 int64_t B, int64_t L, int64_t H, int64_t G, double eps,
+                                 int64_t* count, float* mean, float* var, float* group_mean,
+                                 float* cummean, float* cumrstd, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* prev_count,
+                           const float* prev_mean, const float* prev_var, const float* gamma,
+                           const float* beta, const uint8_t* mask, int64_t B, int64_t L,
+                           int64_t H, double eps, int64_t* count, float* mean, float* var,
+                           float* cummean, float* cumrstd, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* Attention softmax and the fused attention op                              */
+/* stands in for attention_softmax_fwd (fairseq/csrc/ops/attention_softmax.cc:6-18,
+ * ops/attention_softmax_kernel.cu:22-64, softmax.cuh:90-153), dropout = 0.
+ *   x, y [batch, outer, inner] contiguous of `dtype`; causal: row r keeps the first
+ *   inner - outer + r + 1 columns; a fully masked row becomes zeros.              */
+int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch, int64_t outer,
+                               int64_t inner, int causal, void* stream);
+
+/* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276),
+ * dropout = 0:  q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;
+ *   y[b,:,n,:] = softmax_causal(scale q k^T) v per (b, n).  The L x L weights are
+ *   not materialised unless w != NULL (w [B,Nh,L,L] of `dtype`).                  */
+int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
+                       int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
+                       int causal, void* stream);
+
+/* ------------------------------------------------------------------------ */
+/* SwiGLU gate: y = silu(a) * b, elementwise over n elements of `dtype`.
+ * No counterpart in the reference (its FFN is SiLU-MLP,
+ * fairseq/modules/normalized_feedforward_network.py:77-93); the activation itself is
+ * the reference's F.silu.                                                         */
+int mega_swiglu_fwd(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEGA_HIP_H_ */

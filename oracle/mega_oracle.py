@@ -1,0 +1,439 @@
+"""CPU oracle for the Mega/Mega2 sequence-mixing path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may
+import this module.  It is never on the product path: the product is the HIP
+library under fairseq-apollo_amd/csrc and fails loudly without it.
+
+Every function restates, in numpy (fp64 unless told otherwise), what the
+reference computes; the reference location it follows is cited per function
+(paths relative to the reference tree).  The reference ships no tests, golden
+vectors or fixtures for this path, so each function is pinned by
+tests/test_oracle_*.py against closed forms, brute force and library routines
+(and against oracle/_ref, the reference's own CPU translation units compiled in
+place, where that build exists).  Pin status per function:
+
+  ema_coeffs_real / ema_coeffs_complex   closed forms + invariants
+  ema_kernel / ema_bias / ema_hidden     brute-force powers, geometric series, oracle/_ref
+  causal_conv / bidirectional_conv       direct O(L^2) sums, numpy.convolve, impulse/shift
+  ema_forward / ema_one_step             chunk-split invariance, step-vs-parallel equality
+  timestep_norm (group / per feature)    numpy.mean/var on prefixes, oracle/_ref
+  attention_softmax / attention          explicit masked softmax, rows sum to 1
+  swiglu / silu_ffn / rotary / gated_attention_layer
+                                         closed forms only; SwiGLU and multi-head are not
+                                         in the reference: parity unpinned (spec only)
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+
+# --------------------------------------------------------------------------
+# helpers
+# --------------------------------------------------------------------------
+
+
+def _sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def _silu(x):
+    return x * _sigmoid(x)
+
+
+def pow2ceil(L: int) -> int:
+    """fused_ops/fftconv.py:47 -- N = L if L is a power of two else 1 << bit_length."""
+    return L if (L & (L - 1)) == 0 else (1 << int(L).bit_length())
+
+
+# --------------------------------------------------------------------------
+# A1/A2: coefficients
+# --------------------------------------------------------------------------
+
+
+def ema_coeffs_real(alpha, delta, beta, gamma, dtype=np.float64):
+    """Real EMA coefficients, modules/exponential_moving_average.py:71-80.
+
+    alpha, delta, beta: [K, N, 1] (or [K, N]); gamma: [K, N].
+    Returns p[K,N], q[K,N], gamma'[K,N] with q = 1 - s(alpha) s(delta),
+    p = s(alpha) beta, gamma' = gamma sqrt(1/N).
+    """
+    alpha = np.asarray(alpha, dtype).reshape(gamma.shape[0], -1)
+    delta = np.asarray(delta, dtype).reshape(gamma.shape[0], -1)
+    beta = np.asarray(beta, dtype).reshape(gamma.shape[0], -1)
+    gamma = np.asarray(gamma, dtype)
+    N = gamma.shape[1]
+    a = _sigmoid(alpha)
+    d = _sigmoid(delta)
+    q = 1.0 - a * d
+    p = a * beta
+    return p, q, gamma * math.sqrt(1.0 / N)
+
+
+def ema_coeffs_complex(alpha, delta, theta, gamma, dtype=np.float64):
+    """Complex EMA coefficients, modules/complex_exponential_moving_average.py:79-96.
+
+    alpha, delta: [K, N, 1]; theta: [K, 1, 1]; gamma: [K, N, 2] (re, im).
+    theta_{d,n} = (n+1) s(theta_d) 2pi/N; p = s(alpha);
+    q = (1 - s(alpha) s(delta)) e^{i theta}; gamma' = (g0 + i g1) sqrt(1/N).
+    """
+    gamma = np.asarray(gamma, dtype)
+    K, N = gamma.shape[0], gamma.shape[1]
+    alpha = np.asarray(alpha, dtype).reshape(K, N)
+    delta = np.asarray(delta, dtype).reshape(K, N)
+    theta = np.asarray(theta, dtype).reshape(K, 1)
+    ctype = np.complex128 if dtype == np.float64 else np.complex64
+    phi = _sigmoid(theta) * (2.0 * math.pi / N)
+    wav = np.arange(1, N + 1, dtype=dtype).reshape(1, N)
+    ang = wav * phi
+    a = _sigmoid(alpha)
+    d = _sigmoid(delta)
+    mag = 1.0 - a * d
+    q = (mag * np.cos(ang) + 1j * mag * np.sin(ang)).astype(ctype)
+    g = (gamma[..., 0] + 1j * gamma[..., 1]).astype(ctype) * math.sqrt(1.0 / N)
+    return a, q, g
+
+
+# --------------------------------------------------------------------------
+# A3: kernel / bias; A7: hidden state
+# --------------------------------------------------------------------------
+
+
+def ema_kernel(p, q, gamma, L: int):
+    """w[d,l] = Re sum_n p gamma exp(l log q), csrc/ops/ema_parameters.cc:37-52
+    (same as complex_exponential_moving_average.py:104-109 and
+    exponential_moving_average.py:82-90 for real q)."""
+    q = np.asarray(q)
+    logq = np.log(q.astype(np.complex128 if np.iscomplexobj(q) else q.dtype))
+    l = np.arange(L).reshape(1, 1, L)
+    vander = np.exp(l * logq[..., None])            # K x N x L
+    c = np.asarray(p)[..., None] * np.asarray(gamma)[..., None]
+    return np.real((c * vander).sum(axis=1))
+
+
+def ema_bias(q, gamma, h, L: int):
+    """b[b,d,l] = Re sum_n exp((l+1) log q) gamma h, csrc/ops/ema_parameters.cc:54-77
+    (equals base_moving_average.py:73-80).  h: [B, K, N]."""
+    q = np.asarray(q)
+    logq = np.log(q.astype(np.complex128 if np.iscomplexobj(q) else q.dtype))
+    l = np.arange(1, L + 1).reshape(1, 1, L)
+    vander = np.exp(l * logq[..., None]) * np.asarray(gamma)[..., None]   # K x N x L
+    return np.real(np.einsum('bdn,dnl->bdl', np.asarray(h), vander))
+
+
+def ema_hidden(x, p, q, h=None):
+    """h'[b,d,n] = p sum_j q^{L-1-j} x[b,d,j] + q^L h, csrc/ops/ema_hidden.cc:31-63.
+    x: [B, D, L] real.  Returns [B, D, N] (complex if q is)."""
+    x = np.asarray(x, np.float64)
+    q = np.asarray(q)
+    L = x.shape[-1]
+    logq = np.log(q.astype(np.complex128 if np.iscomplexobj(q) else q.dtype))
+    e = np.arange(L - 1, -1, -1).reshape(1, 1, L)
+    vander = np.exp(e * logq[..., None])            # D x N x L
+    out = np.einsum('bdl,dnl->bdn', x, vander) * np.asarray(p)[None]
+    if h is not None:
+        out = out + np.exp(L * logq)[None] * np.asarray(h)
+    return out
+
+
+# --------------------------------------------------------------------------
+# A4/A5: long convolution
+# --------------------------------------------------------------------------
+
+
+def causal_conv(x, k):
+    """y[...,t] = sum_{j<=t, j<Lk} k[d,j] x[...,t-j] through the zero-padded real FFT of
+    length 2*pow2ceil(L), exactly the order of operations of
+    fused_ops/fftconv.py:45-61 (_fftconv_fwd).  x: [B, D, L]; k: [D, Lk], Lk <= L."""
+    x = np.asarray(x, np.float64)
+    k = np.asarray(k, np.float64)
+    L = x.shape[-1]
+    n2 = 2 * pow2ceil(L)
+    x_f = np.fft.rfft(x, n=n2)
+    k_f = np.fft.rfft(k, n=n2) / n2                 # norm="forward" on the kernel
+    y = np.fft.irfft(x_f * k_f, n=n2) * n2          # norm="forward" on the inverse
+    return y[..., :L]
+
+
+def causal_conv_direct(x, k):
+    """The same convolution as an explicit double loop (small inputs only)."""
+    x = np.asarray(x, np.float64)
+    k = np.asarray(k, np.float64)
+    B, D, L = x.shape
+    Lk = k.shape[-1]
+    y = np.zeros_like(x)
+    for t in range(L):
+        for j in range(min(t + 1, Lk)):
+            y[:, :, t] += k[None, :, j] * x[:, :, t - j]
+    return y
+
+
+def bidirectional_conv(x, k, shift: bool = True):
+    """fused_ops/fftconv.py:85-100 (bidirectional_fftconv): k = [k1; k2] of shape
+    [2D, Lk]; circular real FFT of length L + Lk."""
+    x = np.asarray(x, np.float64)
+    k = np.asarray(k, np.float64)
+    B, D, L = x.shape
+    Lk = k.shape[1]
+    F = L + Lk
+    k1, k2 = k[:D], k[D:]
+    kk = np.zeros((D, F))
+    kk[:, :Lk] += k1
+    if shift:
+        kk[:, L:] += k2[:, ::-1]
+    else:
+        kk[:, 0] += k2[:, 0]
+        kk[:, L + 1:] += k2[:, 1:][:, ::-1]
+    k_f = np.fft.rfft(kk, n=F) / F
+    x_f = np.fft.rfft(x, n=F)
+    return (np.fft.irfft(x_f * k_f, n=F) * F)[..., :L]
+
+
+def bidirectional_conv_direct(x, k, shift: bool = True):
+    """The two explicit lag sums: forward lags j >= 0 with k1; backward lags m >= 1 with
+    k2[m-1] (shift) or k2[m] plus the lag-0 tap k2[0] (no shift)."""
+    x = np.asarray(x, np.float64)
+    k = np.asarray(k, np.float64)
+    B, D, L = x.shape
+    Lk = k.shape[1]
+    k1, k2 = k[:D], k[D:]
+    y = np.zeros_like(x)
+    for t in range(L):
+        for j in range(min(t + 1, Lk)):
+            y[:, :, t] += k1[None, :, j] * x[:, :, t - j]
+        if shift:
+            for m in range(1, Lk + 1):
+                if t + m < L:
+                    y[:, :, t] += k2[None, :, m - 1] * x[:, :, t + m]
+        else:
+            y[:, :, t] += k2[None, :, 0] * x[:, :, t]
+            for m in range(1, Lk):
+                if t + m < L:
+                    y[:, :, t] += k2[None, :, m] * x[:, :, t + m]
+    return y
+
+
+# --------------------------------------------------------------------------
+# A6: the moving-average layer
+# --------------------------------------------------------------------------
+
+
+def ema_forward(x, p, q, gamma, omega, padding_mask=None, h=None,
+                bidirectional: bool = False, truncation: Optional[int] = None,
+                shift: bool = True, incremental: bool = False):
+    """BaseMovingLayer.forward, modules/base_moving_average.py:120-172.
+
+    x: [B, D, L]; p, q, gamma: [K, N] with K = 2D when bidirectional; omega: [D];
+    padding_mask: [B, L] (True = pad); h: [B, D, N] carried state or None.
+    Returns (y[B,D,L], h' or None).  The carried-state bias is always added (the GPU
+    behaviour of the reference; its CPU branch drops it, see
+    complex_exponential_moving_average.py:98-109).
+    """
+    x = np.asarray(x, np.float64)
+    B, D, L = x.shape
+    residual = x * np.asarray(omega, np.float64).reshape(1, D, 1)
+    xm = x
+    if padding_mask is not None:
+        xm = x * (1.0 - np.asarray(padding_mask, np.float64)[:, None, :])
+    Lk = L if truncation is None or truncation < 1 else min(truncation, L)
+    k = ema_kernel(p, q, gamma, Lk)
+    h_new = None
+    if bidirectional:
+        assert h is None and not incremental
+        out = bidirectional_conv(xm, k, shift)
+    else:
+        out = causal_conv(xm, k)
+        if incremental or h is not None:
+            if h is not None:
+                out = out + ema_bias(q, gamma, h, L)
+            h_new = ema_hidden(xm, p, q, h)
+    return out + residual, h_new
+
+
+def ema_one_step(x_t, p, q, gamma, omega, h=None):
+    """BaseMovingLayer.one_step, modules/base_moving_average.py:105-118, plus the
+    residual the caller adds.  x_t: [B, D]; h: [B, D, N]."""
+    x_t = np.asarray(x_t, np.float64)
+    hh = np.asarray(p)[None] * x_t[..., None]
+    if h is not None:
+        hh = hh + np.asarray(q)[None] * np.asarray(h)
+    out = np.real(np.einsum('bdn,dn->bd', hh, np.asarray(gamma)))
+    return out + x_t * np.asarray(omega, np.float64).reshape(1, -1), hh
+
+
+# --------------------------------------------------------------------------
+# A8: TimestepNorm
+# --------------------------------------------------------------------------
+
+
+def _welford_update(m0, m1, m2, x):
+    """csrc/utils.h:55-64."""
+    m0 = m0 + 1
+    coef = 1.0 / m0
+    d1 = x - m1
+    m1 = m1 + coef * d1
+    d2 = d1 * (x - m1) - m2
+    m2 = m2 + coef * d2
+    return m0, m1, m2
+
+
+def _welford_combine(a0, a1, a2, b0, b1, b2):
+    """csrc/utils.h:66-76."""
+    m0 = a0 + b0
+    c1 = 0.0 if m0 == 0 else a0 / m0
+    c2 = 0.0 if m0 == 0 else b0 / m0
+    delta = b1 - a1
+    m1 = c1 * a1 + c2 * b1
+    m2 = c1 * a2 + c2 * b2 + (c1 * delta) * (c2 * delta)
+    return m0, m1, m2
+
+
+def timestep_norm(x, prev_count, prev_mean, prev_var, gamma, beta,
+                  padding_mask=None, num_groups: Optional[int] = None, eps: float = 1e-5,
+                  dtype=np.float64):
+    """Group variant: csrc/ops/timestep_norm.cc:218-316; per-feature variant
+    (num_groups None): csrc/ops/timestep_norm.cc:23-103.  Literal serial loop.
+
+    x: [B, L, H]; prev_count: [B] int; prev_mean, prev_var: [B, G]; gamma (= weight + 1),
+    beta: [H].  Returns (y, count[B] int64, mean[B,G], var[B,G]).
+    """
+    x = np.asarray(x, dtype)
+    B, L, H = x.shape
+    gamma = np.asarray(gamma, dtype)
+    beta = np.asarray(beta, dtype)
+    G = H if num_groups is None else num_groups
+    Dg = H // G
+    y = np.zeros_like(x)
+    count = np.array(prev_count, dtype=np.int64).copy()
+    mean = np.array(prev_mean, dtype=dtype).reshape(B, G).copy()
+    var = np.array(prev_var, dtype=dtype).reshape(B, G).copy()
+    if num_groups is not None:
+        xg = x.reshape(B, L, G, Dg)
+        gmean = xg.mean(axis=-1)
+        gvar = xg.var(axis=-1)                      # biased, as RowwiseMoments (utils.h:79-118)
+    for b in range(B):
+        m0 = int(count[b])
+        u = mean[b].copy()
+        v = var[b].copy()
+        for t in range(L):
+            masked = padding_mask is not None and bool(padding_mask[b][t])
+            if num_groups is None:
+                _, m1, m2 = _welford_update(m0, u, v, x[b, t])
+                rstd = 1.0 / np.sqrt(m2 + dtype(eps))
+                if not masked:
+                    y[b, t] = (x[b, t] - m1) * rstd * gamma + beta
+                    u, v = m1, m2
+            else:
+                _, m1, m2 = _welford_combine(m0, u, v, 1, gmean[b, t], gvar[b, t])
+                rstd = 1.0 / np.sqrt(m2 + dtype(eps))
+                if not masked:
+                    y[b, t] = ((xg[b, t] - m1[:, None]) * rstd[:, None]).reshape(H) * gamma + beta
+                    u, v = m1, m2
+            if not masked:
+                m0 += 1
+        count[b] = m0
+        mean[b] = u
+        var[b] = v
+    return y, count, mean, var
+
+
+def timestep_norm_closed_form(x, padding_mask=None, num_groups: Optional[int] = None,
+                              eps: float = 1e-5, gamma=None, beta=None):
+    """Textbook statement for zero prior count: after step t the state is the mean and the
+    biased variance of every unmasked element x[b, <=t, group].  Independent of the
+    recurrences above (cumulative sums in fp64)."""
+    x = np.asarray(x, np.float64)
+    B, L, H = x.shape
+    G = H if num_groups is None else num_groups
+    Dg = H // G
+    xg = x.reshape(B, L, G, Dg)
+    keep = np.ones((B, L)) if padding_mask is None else 1.0 - np.asarray(padding_mask, np.float64)
+    s1 = np.cumsum(xg.sum(-1) * keep[..., None], axis=1)
+    s2 = np.cumsum((xg ** 2).sum(-1) * keep[..., None], axis=1)
+    n = np.cumsum(keep, axis=1)[..., None] * Dg
+    with np.errstate(divide='ignore', invalid='ignore'):
+        mu = np.where(n > 0, s1 / n, 0.0)
+        var = np.where(n > 0, s2 / n - mu ** 2, 0.0)
+    y = (xg - mu[..., None]) / np.sqrt(var[..., None] + eps)
+    y = y.reshape(B, L, H)
+    if gamma is not None:
+        y = y * np.asarray(gamma, np.float64)
+    if beta is not None:
+        y = y + np.asarray(beta, np.float64)
+    y = y * keep[..., None]
+    return y, mu, var
+
+
+# --------------------------------------------------------------------------
+# A9/A10: attention softmax and the fused attention op
+# --------------------------------------------------------------------------
+
+
+def attention_softmax(x, causal: bool = False):
+    """csrc/softmax.cuh:90-153: softmax over the last axis of x[..., R, C]; causal keeps
+    columns [0, C - R + r] of row r; a row whose maximum is -inf (or whose sum is 0)
+    becomes zeros."""
+    x = np.asarray(x, np.float64)
+    R, C = x.shape[-2], x.shape[-1]
+    if causal:
+        r = np.arange(R)[:, None]
+        c = np.arange(C)[None, :]
+        x = np.where(c <= C - R + r, x, -np.inf)
+    m = x.max(axis=-1, keepdims=True)
+    dead = ~np.isfinite(m)
+    e = np.exp(x - np.where(dead, 0.0, m))
+    e = np.where(dead, 0.0, e)
+    s = e.sum(axis=-1, keepdims=True)
+    return np.where(s > 0, e / np.where(s > 0, s, 1.0), 0.0)
+
+
+def attention(q, k, v, scale: float = 1.0, causal: bool = True):
+    """csrc/ops/attention_kernel.cu:40-131: q, k: [B, L, Nh, H1]; v: [B, L, Nh, H2];
+    w[b,n] = softmax_causal(scale q k^T); y[b,:,n,:] = w v.  Returns (y, w)."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    s = np.einsum('blnh,bmnh->bnlm', q, k) * scale
+    w = attention_softmax(s, causal)
+    y = np.einsum('bnlm,bmnh->blnh', w, v)
+    return y, w
+
+
+# --------------------------------------------------------------------------
+# A11/A12: layer glue (spec-level restatement)
+# --------------------------------------------------------------------------
+
+
+def swiglu(a, b):
+    """silu(a) * b -- the gate of the north-star SwiGLU FFN; not present in the
+    reference (its FFN is normalized_feedforward_network.py:77-93): parity unpinned."""
+    a = np.asarray(a, np.float64)
+    return _silu(a) * np.asarray(b, np.float64)
+
+
+def swiglu_ffn(x, w1, w3, w2):
+    """W2 (silu(W1 x) * W3 x); weights are [out, in]."""
+    x = np.asarray(x, np.float64)
+    return swiglu(x @ np.asarray(w1, np.float64).T, x @ np.asarray(w3, np.float64).T) @ np.asarray(w2, np.float64).T
+
+
+def silu_ffn(x, w1, b1, w2, b2):
+    """normalized_feedforward_network.py:77-93 without the norm: x + fc2(silu(fc1(x)))."""
+    x = np.asarray(x, np.float64)
+    return x + _silu(x @ np.asarray(w1, np.float64).T + b1) @ np.asarray(w2, np.float64).T + b2
+
+
+def rotary(x, base: float = 10000.0):
+    """modules/relative_positional_bias.py:57-88 (RotaryRelativePositionalBias):
+    x: [..., L, S]; features (2i, 2i+1) form one complex number that is multiplied by
+    exp(i t base^{-2i/S}) for position t (positions start at 0)."""
+    x = np.asarray(x, np.float64)
+    L, S = x.shape[-2], x.shape[-1]
+    freq = 1.0 / (base ** (np.arange(0, S, 2) / S))
+    ang = np.arange(L)[:, None] * freq[None, :]
+    z = (x[..., 0::2] + 1j * x[..., 1::2]) * np.exp(1j * ang)
+    out = np.empty_like(x)
+    out[..., 0::2] = z.real
+    out[..., 1::2] = z.imag
+    return out

@@ -1,0 +1,51 @@
+"""The C-ABI library loads and exports every symbol include/mega_hip.h declares, the ctypes
+table covers the same set, and argument checks answer without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+import fairseq_apollo_amd as M
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mega_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mega_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared()
+    assert len(names) >= 15
+    lib = ctypes.CDLL(M._lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mega_hip.h but not exported"
+    assert sorted(M._lib.SIGNATURES) == names
+
+
+def test_argument_checks_need_no_gpu():
+    lib = M._lib.load()
+    assert lib.mega_abi_version() == 1
+    # bad dtype is rejected before anything touches a device
+    rc = lib.mega_swiglu_fwd(None, None, None, 7, 16, None)
+    assert rc == -1 and b"dtype" in lib.mega_last_error()
+    rc = lib.mega_group_timestep_norm_fwd(None, None, 1, None, None, None, None, None, None, 2, 8, 30, 4, 1e-5,
+                                          None, None, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"multiple" in lib.mega_last_error()
+    rc = lib.mega_ema_fwd(None, None, 1, 0, 0, 0, 0, 0, 0, None, None, None, 1, None, None, None, None, 2, 8, 64, 16,
+                          0, 0, 1, None, 0, None)
+    assert rc == -2 and b"ndim" in lib.mega_last_error()
+    assert lib.mega_timestep_norm_workspace_bytes(1, 4, 4096, 1024, 16) > 0
+    assert lib.mega_ema_fwd_workspace_bytes(4, 1024, 16, 4096, 0, 0) > 0
+
+
+def test_ops_reject_cpu_tensors():
+    import torch
+    x = torch.zeros(1, 4, 8)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        M.ops.swiglu(x, x)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        M.ops.attention_softmax_fwd(x, 0.0, True)

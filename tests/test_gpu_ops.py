@@ -1,0 +1,96 @@
+"""The remaining operator entry points on the GPU against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import mega_init_complex, rel_err
+from gpu_util import DEV, TOL, dev, host, rounded
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_ema_parameters_and_hidden_ops():
+    rng = np.random.default_rng(21)
+    K, N, L, B = 40, 16, 300, 3
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
+    h = rng.normal(size=(B, K, N)) + 1j * rng.normal(size=(B, K, N))
+    tq = dev(q)
+    w, b, _ = M.ops.ema_parameters_fwd(dev(p), tq.log(), dev(g), dev(h), L)
+    assert rel_err(host(w), O.ema_kernel(p, q, g, L)) < 1e-4
+    assert rel_err(host(b), O.ema_bias(q, g, h, L)) < 1e-4
+    w0, b0, _ = M.ops.ema_parameters_fwd(dev(p), tq.log(), dev(g), None, 1)
+    assert b0 is None and rel_err(host(w0), O.ema_kernel(p, q, g, 1)) < 1e-5
+    x, x64 = rounded(rng.normal(size=(B, K, L)), torch.bfloat16)
+    hh, _ = M.ops.ema_hidden_fwd(x, dev(p), tq.log(), dev(h))
+    ref = O.ema_hidden(x64, p, q, h)
+    assert rel_err(np.real(host(hh)), ref.real) < 1e-4 and rel_err(np.imag(host(hh)), ref.imag) < 1e-4
+
+
+def test_long_kernel_phase_accuracy():
+    """|q| close to 1 and 16k lags: the phase l*theta must not drift in fp32."""
+    K, N, L = 4, 16, 16384
+    rng = np.random.default_rng(22)
+    mag = 1 - 10 ** rng.uniform(-5, -3, size=(K, N))
+    q = mag * np.exp(1j * rng.uniform(0, np.pi, size=(K, N)))
+    p = rng.random((K, N)); g = rng.normal(size=(K, N)) + 0j
+    w, _, _ = M.ops.ema_parameters_fwd(dev(p), dev(q).log(), dev(g), None, L)
+    q32 = q.astype(np.complex64).astype(np.complex128)
+    logq = np.log(q32).astype(np.complex64).astype(np.complex128)      # what the op is handed
+    ref = np.real((p[..., None] * g[..., None] * np.exp(np.arange(L) * logq[..., None])).sum(1))
+    assert rel_err(host(w), ref) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Lk", [700, 1, 33])
+def test_long_conv(dtype, Lk):
+    rng = np.random.default_rng(23)
+    B, D, L = 2, 6, 700
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    k = (rng.normal(size=(2 * D, Lk)) * 0.2).astype(np.float32)
+    y = M.ops.fftconv(x, dev(k[:D]))
+    assert rel_err(host(y), O.causal_conv(x64, np.pad(k[:D].astype(np.float64), ((0, 0), (0, L - Lk))))) < TOL[dtype]
+    for shift in (True, False):
+        y = M.ops.bidirectional_fftconv(x, dev(k), shift)
+        assert rel_err(host(y), O.bidirectional_conv(x64, k.astype(np.float64), shift)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 5, 40, 40), (2, 17, 300), (2, 64, 2048), (1, 6, 3)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_softmax(dtype, shape, causal):
+    rng = np.random.default_rng(24)
+    a = rng.normal(size=shape) * 3
+    a[..., 0, :] = -np.inf
+    x, x64 = rounded(a, dtype)
+    y = M.AttentionSoftmax(use_causal_mask=causal).eval()(x)
+    yo = O.attention_softmax(x64, causal)
+    assert np.abs(host(y) - yo).max() < (1e-5 if dtype == torch.float32 else 4e-3)
+    assert torch.all(y[..., 0, :] == 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,Nh,H1,H2", [(2, 50, 1, 16, 24), (1, 130, 4, 32, 64), (2, 7, 2, 5, 3)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention(dtype, B, L, Nh, H1, H2, causal):
+    rng = np.random.default_rng(25)
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    y, w = M.ops.attention_fwd(q, k, v, 0.8, 0.0, causal, need_weights=True)
+    yo, wo = O.attention(q64, k64, v64, 0.8, causal)
+    assert rel_err(host(y), yo) < TOL[dtype]
+    assert np.abs(host(w) - wo).max() < (1e-5 if dtype == torch.float32 else 4e-3)
+    if Nh == 1:
+        ym = M.EfficientAttention(scale=0.8, use_causal_mask=causal).eval()(q[:, :, 0], k[:, :, 0], v[:, :, 0])
+        assert torch.equal(ym, y[:, :, 0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_swiglu(dtype, n):
+    rng = np.random.default_rng(26)
+    a, a64 = rounded(rng.normal(size=n) * 3, dtype)
+    b, b64 = rounded(rng.normal(size=n), dtype)
+    assert rel_err(host(M.ops.swiglu(a, b)), O.swiglu(a64, b64)) < TOL[dtype]

@@ -1,0 +1,107 @@
+"""HIP TimestepNorm against the fp64 oracle (group and per-feature variants)."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import rel_err
+from gpu_util import DEV, TOL, dev, host, rounded
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, B, L, H, G, dtype, masked, prior):
+    rng = np.random.default_rng(seed)
+    x, x64 = rounded(rng.normal(size=(B, L, H)) * 1.5 + 0.3, dtype)
+    Gs = H if G is None else G
+    mask = (rng.random((B, L)) < 0.25) if masked else None
+    if prior:
+        pc = rng.integers(2, 9, size=B).astype(np.int64)
+        pm = rng.normal(size=(B, Gs)).astype(np.float32) * 0.3
+        pv = (rng.random((B, Gs)) + 0.5).astype(np.float32)
+    else:
+        pc = np.zeros(B, np.int64); pm = np.zeros((B, Gs), np.float32); pv = np.ones((B, Gs), np.float32)
+    gamma = (rng.normal(size=H) * 0.2 + 1).astype(np.float32)
+    beta = (rng.normal(size=H) * 0.2).astype(np.float32)
+    return x, x64, mask, pc, pm, pv, gamma, beta
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H,G", [(2, 37, 64, 4), (3, 300, 256, 16), (1, 1, 128, 8), (2, 129, 96, 2),
+                                     (1, 70, 2048, 16), (2, 50, 48, 12)])
+@pytest.mark.parametrize("masked,prior", [(False, False), (True, True)])
+def test_group_matches_oracle(dtype, B, L, H, G, masked, prior):
+    print(f"case dtype={dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior}", flush=True)
+    x, x64, mask, pc, pm, pv, gamma, beta = _case(1, B, L, H, G, dtype, masked, prior)
+    out = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma), dev(beta),
+                                        None if mask is None else dev(mask, torch.bool), G, 1e-5)
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    y, c, mu, v = O.timestep_norm(x64, pc, pm, pv, gamma, beta, mask, G, 1e-5)
+    assert rel_err(host(out[0]), y) < TOL[dtype]
+    assert np.array_equal(host(out[1]), c)
+    assert rel_err(host(out[2]), mu) < 1e-4 and rel_err(host(out[3]), v) < 1e-4
+    if mask is not None:
+        assert torch.all(out[0][dev(mask, torch.bool)] == 0)
+    # statistics saved for a backward pass: running mean / rstd after each unmasked step
+    _, muc, varc = O.timestep_norm_closed_form(x64, mask, G) if not prior else (None, None, None)
+    if muc is not None and mask is None:
+        assert rel_err(host(out[5]), muc) < 1e-4
+        assert rel_err(host(out[6]), 1 / np.sqrt(varc + 1e-5)) < 1e-4
+        assert rel_err(host(out[4]), x64.reshape(B, L, G, -1).mean(-1)) < 1e-4
+
+
+def test_chunked_streaming_equals_one_shot():
+    rng = np.random.default_rng(5)
+    B, L, H, G = 2, 256, 128, 8
+    tn = M.TimestepNorm(H, G).to(DEV).eval()
+    with torch.no_grad():
+        tn.weight.copy_(dev(rng.normal(size=H) * 0.1)); tn.bias.copy_(dev(rng.normal(size=H) * 0.1))
+        x, x64 = rounded(rng.normal(size=(B, L, H)), torch.float32)
+        full = tn(x)
+        state = {}
+        parts = [tn(x[:, a:b], None, state) for a, b in ((0, 100), (100, 101), (101, 256))]
+    assert rel_err(host(torch.cat(parts, 1)), host(full)) < 1e-5
+    saved = tn._get_input_buffer(state)
+    assert saved["prev_count"].tolist() == [L, L]
+    y, _, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)),
+                                  host(tn.weight) + 1, host(tn.bias), None, G, 1e-5)
+    assert rel_err(host(full), y) < 1e-4 and rel_err(host(saved["prev_mean"]), mu) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feature_variant_matches_oracle(dtype):
+    x, x64, mask, pc, pm, pv, gamma, beta = _case(7, 2, 90, 40, None, dtype, True, True)
+    out = M.ops.timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma), dev(beta),
+                                  dev(mask, torch.bool), 1e-5)
+    y, c, mu, v = O.timestep_norm(x64, pc, pm, pv, gamma, beta, mask, None, 1e-5)
+    assert rel_err(host(out[0]), y) < TOL[dtype] and np.array_equal(host(out[1]), c)
+    assert rel_err(host(out[2]), mu) < 1e-4 and rel_err(host(out[3]), v) < 1e-4
+
+
+def test_headline_shape_against_closed_form():
+    """B4 x L4096 x D1024, 16 groups, bf16: the textbook cumulative statistics in fp64."""
+    rng = np.random.default_rng(1236)
+    B, L, H, G = 4, 4096, 1024, 16
+    x, x64 = rounded(rng.normal(size=(B, L, H)), torch.bfloat16)
+    tn = M.TimestepNorm(H, G).to(DEV).eval()
+    with torch.no_grad():
+        y = tn(x)
+        y2 = tn(x)
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    assert torch.equal(y, y2)                   # deterministic, workspace left clean
+    yc, _, _ = O.timestep_norm_closed_form(x64, None, G)
+    assert rel_err(host(y), yc) < TOL[torch.bfloat16]
+    # the bf16 rounding of y is the only error source that matters: compare before rounding
+    err = np.abs(host(y) - yc)
+    assert np.median(err) < 4e-3
+
+
+def test_errors():
+    x = torch.zeros(1, 4, 30, device=DEV)
+    z = torch.zeros(1, 4, device=DEV)
+    with pytest.raises(RuntimeError, match="divisible"):
+        M.ops.group_timestep_norm_fwd(x, torch.zeros(1, dtype=torch.int64, device=DEV), z, z,
+                                      torch.ones(30, device=DEV), torch.zeros(30, device=DEV), None, 4, 1e-5)

@@ -1,0 +1,71 @@
+"""Host-side mirror of the reference modules: parameter names / shapes (checkpoint
+compatibility), coefficient formulas against the oracle, incremental-state bookkeeping."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from oracle import mega_oracle as O
+
+
+def test_parameter_names_and_shapes():
+    ema = M.MultiHeadEMA(8, ndim=4, bidirectional=True)
+    sd = {k: tuple(v.shape) for k, v in ema.state_dict().items()}
+    assert sd == {"alpha": (16, 4, 1), "delta": (16, 4, 1), "beta": (16, 4, 1), "gamma": (16, 4), "omega": (8,)}
+    cema = M.MultiHeadComplexEMA(8, ndim=4)
+    sd = {k: tuple(v.shape) for k, v in cema.state_dict().items()}
+    assert sd == {"alpha": (8, 4, 1), "delta": (8, 4, 1), "theta": (8, 1, 1), "gamma": (8, 4, 2), "omega": (8, 1)}
+    assert [n for n, _ in cema.parameters_no_weight_decay()] == ["alpha", "delta", "theta"]
+    tn = M.TimestepNorm(32, 4)
+    sd = {k: tuple(v.shape) for k, v in tn.state_dict().items()}
+    assert sd == {"weight": (32,), "bias": (32,), "prior_count": (), "prior_mean": (4,), "prior_logv": (4,)}
+    assert len(list(tn.parameters())) == 2
+    tn2 = M.TimestepNorm(32, 4, prior_count=3)
+    assert len(list(tn2.parameters())) == 4
+    with pytest.raises(AssertionError):
+        M.TimestepNorm(32)                      # per-feature variant needs prior_count > 1
+    with pytest.raises(AssertionError):
+        M.MultiHeadEMA(8, truncation=4)         # truncation only with bidirectional
+
+
+def test_coefficients_match_oracle_and_init_statistics():
+    torch.manual_seed(0)
+    cema = M.MultiHeadComplexEMA(64, ndim=16).eval()
+    p, q, g = cema.coeffs()
+    po, qo, go = O.ema_coeffs_complex(cema.alpha.detach().numpy(), cema.delta.detach().numpy(),
+                                      cema.theta.detach().numpy(), cema.gamma.detach().numpy())
+    assert np.allclose(p.squeeze(-1).numpy(), po, atol=1e-6)
+    assert np.allclose(q.squeeze(-1).numpy(), qo, atol=1e-6)
+    assert np.allclose(g.numpy(), go, atol=1e-6)
+    assert torch.all(cema.gamma[..., 1] == 0)
+    assert cema.coeffs() is cema.coeffs()       # cached in eval mode
+    cema.train()
+    assert cema._coeffs is None
+    ema = M.MultiHeadEMA(64, ndim=16).eval()
+    p, q, g = ema.coeffs()
+    po, qo, go = O.ema_coeffs_real(ema.alpha.detach().numpy(), ema.delta.detach().numpy(),
+                                   ema.beta.detach().numpy(), ema.gamma.detach().numpy())
+    assert np.allclose(p.squeeze(-1).numpy(), po, atol=1e-6) and np.allclose(q.squeeze(-1).numpy(), qo, atol=1e-6)
+    b = ema.beta.detach().squeeze(-1)
+    assert torch.all(b[:, 0::2] > 0.8) and torch.all(b[:, 1::2] < -0.8)
+
+
+def test_incremental_state_keys_are_per_module():
+    a, b = M.TimestepNorm(8, 2), M.TimestepNorm(8, 2)
+    state = {}
+    a.set_incremental_state(state, "norm_state", {"prev_count": 1})
+    assert a.get_incremental_state(state, "norm_state") == {"prev_count": 1}
+    assert b.get_incremental_state(state, "norm_state") is None
+    key, = state.keys()
+    assert key.endswith(".norm_state")
+    e = M.MultiHeadComplexEMA(4, ndim=2)
+    inc = {}
+    e._set_input_buffer(inc, {"prev_state": torch.arange(6.).reshape(3, 2)})
+    e.reorder_incremental_state(inc, torch.tensor([2, 0]))
+    assert torch.equal(e._get_input_buffer(inc)["prev_state"], torch.tensor([[4., 5.], [0., 1.]]))
+
+
+def test_forward_needs_no_grad():
+    e = M.MultiHeadComplexEMA(4, ndim=2)
+    with pytest.raises(RuntimeError, match="forward pass only"):
+        e(torch.zeros(1, 4, 8))
