@@ -35,9 +35,9 @@ def test_long_kernel_phase_accuracy():
     mag = 1 - 10 ** rng.uniform(-5, -3, size=(K, N))
     q = mag * np.exp(1j * rng.uniform(0, np.pi, size=(K, N)))
     p = rng.random((K, N)); g = rng.normal(size=(K, N)) + 0j
-    w, _, _ = M.ops.ema_parameters_fwd(dev(p), dev(q).log(), dev(g), None, L)
-    q32 = q.astype(np.complex64).astype(np.complex128)
-    logq = np.log(q32).astype(np.complex64).astype(np.complex128)      # what the op is handed
+    lq = dev(q).log()
+    w, _, _ = M.ops.ema_parameters_fwd(dev(p), lq, dev(g), None, L)
+    logq = host(lq)                                # exactly the complex64 values the op is handed
     ref = np.real((p[..., None] * g[..., None] * np.exp(np.arange(L) * logq[..., None])).sum(1))
     assert rel_err(host(w), ref) < 1e-4
 
