@@ -1,0 +1,214 @@
+"""Headline benchmark: TimestepNorm -> complex EMA block (Mega2), B=4, L=4096, D=1024, N=16,
+bf16 activations, fp32 parameters and accumulation, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step = one forward of the block over one batch of synthetic input that already sits in
+HBM: xn = TimestepNorm(x) ([B, L, D], 16 groups), y = CEMA(xn^T) read and written in the same
+[B, L, D] memory layout.  Inputs rotate over several buffers so that a step never finds its
+input in the 256 MB last-level cache.  Prints one JSON line (tokens/s of the whole job), with
+the HBM roofline of the dominant kernel and the CPU oracle timed on the host cores beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+B, L, D, N, G = 4, 4096, 1024, 16, 16
+HBM_PEAK_GBS = 8000.0
+NBUF = 8
+
+
+def make_params(rng):
+    import numpy as np
+
+    alpha = rng.normal(0, 0.2, (D, N, 1))
+    delta = rng.normal(0, 0.2, (D, N, 1))
+    th = rng.uniform(0.0, np.pi, (D, 1, 1)).clip(1e-3, np.pi - 1e-3)
+    frac = th / (2 * np.pi)
+    theta = np.log(frac / (1 - frac))
+    gamma = np.zeros((D, N, 2))
+    gamma[..., 0] = rng.normal(0, 1.0, (D, N))
+    omega = rng.normal(0, 1.0, (D, 1))
+    return alpha, delta, theta, gamma, omega
+
+
+def cpu_baseline(params, x_bf16_as_f32, threads):
+    """The oracle timed on the host cores: the reference's CPU algorithm for the same block
+    (two-stage Welford TimestepNorm loops in C, kernel generation by exp(l log q) in C, the
+    zero-padded real-FFT convolution of fused_ops/fftconv.py:45-61 through scipy's pocketfft)."""
+    import numpy as np
+    import scipy.fft as sfft
+
+    import oracle_c_api as OC
+    from oracle import mega_oracle as O
+
+    alpha, delta, theta, gamma, omega = params
+    p, q, g = O.ema_coeffs_complex(alpha, delta, theta, gamma, dtype=np.float32)
+    x = x_bf16_as_f32
+    ones, zeros = np.ones(D, np.float32), np.zeros(D, np.float32)
+
+    def run():
+        xn, _, _, _ = OC.timestep_norm(x, np.zeros(B, np.int64), np.zeros((B, G), np.float32),
+                                       np.ones((B, G), np.float32), ones, zeros, None, G, 1e-5, np.float32)
+        k = OC.ema_kernel(p, q, g, L, np.float32)
+        xt = np.ascontiguousarray(xn.transpose(0, 2, 1))
+        n2 = 2 * O.pow2ceil(L)
+        x_f = sfft.rfft(xt, n=n2, workers=threads)
+        k_f = sfft.rfft(k, n=n2, workers=threads) / n2
+        y = sfft.irfft(x_f * k_f, n=n2, workers=threads)[..., :L] * n2
+        y = y + omega.reshape(1, D, 1).astype(np.float32) * xt
+        return y
+
+    run()
+    times = []
+    t_end = time.time() + 20.0
+    while len(times) < 3 or (time.time() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    return {"value": B * L / t, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"the full B{B}xL{L}xD{D} block, median of {len(times)} runs ({t * 1e3:.0f} ms each)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    rng = np.random.default_rng(1236)
+    params = make_params(rng)
+    alpha, delta, theta, gamma, omega = params
+
+    norm = M.TimestepNorm(D, G).to(dev).eval()
+    ema = M.MultiHeadComplexEMA(D, ndim=N).to(dev).eval()
+    with torch.no_grad():
+        for name, val in (("alpha", alpha), ("delta", delta), ("theta", theta), ("gamma", gamma), ("omega", omega)):
+            getattr(ema, name).copy_(torch.from_numpy(val.astype(np.float32)))
+    ema._coeffs = None
+    ema._prepared = None
+
+    gen = torch.Generator().manual_seed(1236)
+    xs = [torch.randn(B, L, D, generator=gen, dtype=torch.float32).to(torch.bfloat16).to(dev) for _ in range(NBUF)]
+
+    def step(i):
+        x = xs[i % NBUF]
+        xn = norm(x)
+        y = ema(xn.transpose(1, 2))
+        return xn, y
+
+    with torch.no_grad():
+        for i in range(args.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            step(i)
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        gpu_ms = e0.elapsed_time(e1)
+        ms_per_step = max(wall * 1e3, gpu_ms) / args.steps
+
+        # per-operator device time (events on the launch stream around each call)
+        def timed(fn, reps):
+            evs = []
+            for i in range(reps):
+                a = torch.cuda.Event(enable_timing=True)
+                b = torch.cuda.Event(enable_timing=True)
+                arg = fn.prep(i)
+                a.record()
+                fn(arg)
+                b.record()
+                evs.append((a, b))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) for a, b in evs)
+            return sum(ts) / len(ts), ts[len(ts) // 2]
+
+        class NormCall:
+            @staticmethod
+            def prep(i):
+                return xs[i % NBUF]
+
+            def __call__(self, x):
+                return norm(x)
+
+        xns = [norm(x) for x in xs]
+
+        class EmaCall:
+            @staticmethod
+            def prep(i):
+                return xns[i % NBUF].transpose(1, 2)
+
+            def __call__(self, x):
+                return ema(x)
+
+        reps = max(20, min(args.steps, 200))
+        norm_avg, norm_med = timed(NormCall(), reps)
+        ema_avg, ema_med = timed(EmaCall(), reps)
+    status = M.ops.timestep_norm_status()
+
+    tokens = B * L
+    alg_bytes_block = 4 * B * L * D * 2          # norm: read x, write xn; EMA: read xn, write y
+    alg_bytes_ema = 2 * B * L * D * 2
+    alg_bytes_norm = 2 * B * L * D * 2
+    ema_gbs = alg_bytes_ema / (ema_avg * 1e-3) / 1e9
+    norm_gbs = alg_bytes_norm / (norm_avg * 1e-3) / 1e9
+    out = {
+        "metric": "EMA+norm block tokens/sec @B4xL4096xD1024; achieved HBM GB/s vs peak",
+        "value": tokens / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: TimestepNorm(16 groups) -> complex EMA (N=16), B=4 L=4096 D=1024, "
+                               "bf16 activations, fp32 parameters/accumulation, forward",
+                   "input_buffers_rotated": NBUF},
+        "block_hbm_gbs": alg_bytes_block / (ms_per_step * 1e-3) / 1e9,
+        "block_hbm_frac": alg_bytes_block / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "ema_fwd (every launch of one call)", "achieved": ema_gbs,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg, "median_ms": ema_med},
+        "roofline_timestep_norm": {"bound": "hbm", "kernel": "group_tsn_kernel", "achieved": norm_gbs,
+                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": norm_gbs / HBM_PEAK_GBS,
+                                   "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg,
+                                   "median_ms": norm_med},
+        "timestep_norm_status": status,
+    }
+    if not args.no_cpu:
+        threads = min(os.cpu_count() or 1, 16)
+        x_host = xs[0].float().cpu().numpy()
+        out["cpu_baseline"] = cpu_baseline(params, x_host, threads)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -74,6 +74,7 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         self.truncation = truncation
         self.shift = shift
         self._coeffs = None
+        self._prepared = None
         assert self.bidirectional or (self.truncation is None or self.truncation < 1), \
             'one directional moving average should not have positive trunction: {}'.format(truncation)
 
@@ -98,7 +99,14 @@ class BaseMovingLayer(nn.Module, IncrementalState):
 
     def train(self, mode: bool = True):
         self._coeffs = None
+        self._prepared = None
         return super().train(mode)
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() / .half(): cached coefficients would stay on the old device
+        self._coeffs = None
+        self._prepared = None
+        return super()._apply(fn, *args, **kwargs)
 
     def kernel(self, length: int, hx: Optional[Tensor] = None):
         """(k[K, Lk], bias[B, K, L] or None) -- the materialised convolution kernel; the forward
@@ -125,20 +133,26 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         assert embed_dim == self.embed_dim
         assert not self.bidirectional or incremental_state is None, \
             'Bidirectional EMA does not support incremental state'
-        p, q, gamma = self.coeffs()
-        p2, q2 = p.squeeze(-1), q.squeeze(-1)
-        omega = self.omega.reshape(-1)
+        layer = self._prepared_layer()
         if incremental_state is not None:
             saved_state = self._get_input_buffer(incremental_state)
             h = saved_state['prev_state'] if 'prev_state' in saved_state else None
-            out, h = ops.ema_forward(x, p2, q2, gamma, omega, padding_mask, h, want_state=True)
+            out, h = layer(x, padding_mask, h, want_state=True)
             saved_state['prev_state'] = h
             self._set_input_buffer(incremental_state, saved_state)
         else:
-            out, _ = ops.ema_forward(x, p2, q2, gamma, omega, padding_mask, None, want_state=False,
-                                     bidirectional=self.bidirectional, truncation=self.truncation,
-                                     shift=self.shift)
+            out, _ = layer(x, padding_mask, None, want_state=False)
         return out
+
+    def _prepared_layer(self) -> "ops.PreparedEMA":
+        """Coefficients in the library's layout; kept while the eval-mode coefficient cache lives."""
+        if not self.training and self._prepared is not None and self._coeffs is not None:
+            return self._prepared
+        p, q, gamma = self.coeffs()
+        layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, self.omega.reshape(-1), self.bidirectional,
+                                self.truncation, self.shift)
+        self._prepared = None if self.training else layer
+        return layer
 
     def _get_input_buffer(self, incremental_state):
         result = self.get_incremental_state(incremental_state, "ema_state")
@@ -266,6 +280,8 @@ class TimestepNorm(nn.Module, IncrementalState):
         self.num_features = num_features
         self.num_groups = num_groups
         self._prior_count = prior_count
+        self._prior_cache = {}
+        self._affine_cache = None
         if num_groups is None or num_groups == num_features:
             num_groups = num_features
             assert prior_count > 1
@@ -295,19 +311,18 @@ class TimestepNorm(nn.Module, IncrementalState):
                 assert 'prev_var' in saved_state and 'prev_count' in saved_state
                 prev_var = saved_state['prev_var']
                 prev_count = saved_state['prev_count']
-        if prev_count is None:
-            prev_count = self.prior_count.expand(batch_size).contiguous()
-        if prev_mean is None:
-            prev_mean = self.prior_mean.expand(batch_size, -1).contiguous()
-        if prev_var is None:
-            prev_var = torch.exp(self.prior_logv).expand(batch_size, -1).contiguous()
-        gamma = self.weight.float() + 1.0
+        if prev_count is None or prev_mean is None or prev_var is None:
+            d_count, d_mean, d_var = self._prior_state(batch_size)
+            prev_count = d_count if prev_count is None else prev_count
+            prev_mean = d_mean if prev_mean is None else prev_mean
+            prev_var = d_var if prev_var is None else prev_var
+        gamma, beta = self._affine()
         if self.num_groups is None:
-            out, count, mean, var, _, _ = ops.timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, self.bias,
+            out, count, mean, var, _, _ = ops.timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta,
                                                                 padding_mask, self.eps, need_stats=False)
         else:
             out, count, mean, var, _, _, _ = ops.group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma,
-                                                                         self.bias, padding_mask, self.num_groups,
+                                                                         beta, padding_mask, self.num_groups,
                                                                          self.eps, need_stats=False)
         if incremental_state is not None:
             saved_state['prev_mean'] = mean
@@ -315,6 +330,38 @@ class TimestepNorm(nn.Module, IncrementalState):
             saved_state['prev_count'] = count
             self._set_input_buffer(incremental_state, saved_state)
         return out
+
+    def _prior_state(self, batch_size: int):
+        """(count[B], mean[B,G], var[B,G]) of the prior (timestep_norm.py:122-127); cached in eval mode."""
+        key = batch_size
+        if not self.training and key in self._prior_cache:
+            return self._prior_cache[key]
+        with torch.no_grad():
+            st = (self.prior_count.expand(batch_size).contiguous(),
+                  self.prior_mean.float().expand(batch_size, -1).contiguous(),
+                  torch.exp(self.prior_logv.float()).expand(batch_size, -1).contiguous())
+        if not self.training:
+            self._prior_cache[key] = st
+        return st
+
+    def _affine(self):
+        """(weight + 1, bias) in fp32, as the reference passes them (timestep_norm.py:129-131)."""
+        if not self.training and self._affine_cache is not None:
+            return self._affine_cache
+        with torch.no_grad():
+            ab = (self.weight.float() + 1.0, self.bias.float().contiguous())
+        self._affine_cache = None if self.training else ab
+        return ab
+
+    def train(self, mode: bool = True):
+        self._prior_cache = {}
+        self._affine_cache = None
+        return super().train(mode)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._prior_cache = {}
+        self._affine_cache = None
+        return super()._apply(fn, *args, **kwargs)
 
     def _get_input_buffer(self, incremental_state):
         result = self.get_incremental_state(incremental_state, "norm_state")

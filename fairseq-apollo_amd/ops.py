@@ -73,6 +73,20 @@ def _tsn_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+_scratch = {}
+
+
+def _scratch_buffer(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Grow-only scratch per (device, stream): calls on one stream are ordered, so they can
+    share it; its contents never need to survive a call."""
+    key = (dev.index, _stream(dev))
+    ws = _scratch.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
+        _scratch[key] = ws
+    return ws
+
+
 def timestep_norm_status(dev=None) -> int:
     """Error word of the TimestepNorm workspaces of `dev` (non-zero: a tile gave up waiting for
     an earlier tile).  Synchronises; meant for tests and debugging."""
@@ -265,6 +279,69 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
 # --------------------------------------------------------------------------------------
 
 
+class PreparedEMA:
+    """Coefficients of one moving-average layer converted once to the layout the library
+    takes (fp32, complex as (re, im) pairs); calling it runs the fused layer forward.
+    Modules in eval mode keep one of these next to their cached coefficients."""
+
+    def __init__(self, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, omega: torch.Tensor,
+                 bidirectional: bool = False, truncation: Optional[int] = None, shift: bool = True):
+        self.dev = _need_gpu(p, q, gamma, omega)
+        self.K, self.N = p.shape[0], p.shape[1]
+        self.D = self.K // 2 if bidirectional else self.K
+        if omega.numel() != self.D:
+            raise RuntimeError(f"coefficient rows {self.K} do not match kernel_dim for embed_dim {omega.numel()}")
+        self.is_complex = bool(q.is_complex() or gamma.is_complex())
+        self.p = _f32c(p).reshape(self.K, self.N)
+        self.q = _cplx_as_f32(q.reshape(self.K, self.N))
+        self.gamma = _cplx_as_f32(gamma.reshape(self.K, self.N))
+        self.omega = _f32c(omega).reshape(self.D)
+        self.bidirectional = bool(bidirectional)
+        self.trunc = 0 if truncation is None or truncation < 1 else int(truncation)
+        self.shift = bool(shift)
+
+    def __call__(self, x: torch.Tensor, padding_mask: Optional[torch.Tensor] = None,
+                 h: Optional[torch.Tensor] = None, want_state: bool = False,
+                 out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        dev = self.dev
+        _need_gpu(x, padding_mask, h)
+        lib = _lib.load()
+        if x.dim() != 3:
+            raise RuntimeError("x must be [B, D, L]")
+        B, D, L = x.shape
+        if D != self.D:
+            raise RuntimeError(f"coefficient rows {self.K} do not match kernel_dim {2 * D if self.bidirectional else D}")
+        xd = x.detach()
+        dt = _dtype_code(xd)
+        if 0 in xd.stride() and xd.numel() > 0:
+            xd = xd.contiguous()
+        if out is not None:
+            y = out
+            if y.shape != xd.shape or y.dtype != xd.dtype:
+                raise RuntimeError("out must match x in shape and dtype")
+        elif _dense(xd):
+            y = torch.empty_strided(xd.shape, xd.stride(), dtype=xd.dtype, device=dev)
+        else:
+            y = torch.empty_like(xd, memory_format=torch.contiguous_format)
+        m8 = _mask_u8(padding_mask, B, L)
+        N = self.N
+        hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
+        hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev) if (want_state or h is not None) else None
+        nws = lib.mega_ema_fwd_workspace_bytes(B, D, N, L, 1 if self.bidirectional else 0, self.trunc)
+        ws = _scratch_buffer(dev, nws)
+        with torch.cuda.device(dev):
+            rc = lib.mega_ema_fwd(_ptr(xd), _ptr(y), dt, xd.stride(0), xd.stride(1), xd.stride(2), y.stride(0),
+                                  y.stride(1), y.stride(2), _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
+                                  1 if self.is_complex else 0, _ptr(self.omega), _ptr(m8), _ptr(hin), _ptr(hout),
+                                  B, D, N, L, 1 if self.bidirectional else 0, self.trunc, 1 if self.shift else 0,
+                                  _ptr(ws), ws.numel(), _stream(dev))
+        _lib.check(rc, "ema_fwd")
+        hc = None
+        if hout is not None:
+            hc = torch.view_as_complex(hout) if self.is_complex else hout[..., 0]
+        return y, hc
+
+
 def ema_forward(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, omega: torch.Tensor,
                 padding_mask: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
                 want_state: bool = False, bidirectional: bool = False, truncation: Optional[int] = None,
@@ -276,42 +353,8 @@ def ema_forward(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.
     p: [K, N]; q, gamma: [K, N] real or complex; omega: [D]; h: [B, D, N] carried state.
     Returns (y, h') with y shaped [B, D, L] in x's memory layout and h' complex64 (or None).
     """
-    dev = _need_gpu(x, p, q, gamma, omega, padding_mask, h)
-    lib = _lib.load()
-    if x.dim() != 3:
-        raise RuntimeError("x must be [B, D, L]")
-    B, D, L = x.shape
-    K = 2 * D if bidirectional else D
-    N = p.shape[1]
-    if p.shape[0] != K:
-        raise RuntimeError(f"coefficient rows {p.shape[0]} do not match kernel_dim {K}")
-    is_complex = q.is_complex() or gamma.is_complex()
-    xd = x.detach()
-    dt = _dtype_code(xd)
-    if 0 in xd.stride() and xd.numel() > 0:
-        xd = xd.contiguous()
-    y = torch.empty_strided(xd.shape, xd.stride(), dtype=xd.dtype, device=dev) if _dense(xd) else torch.empty_like(
-        xd, memory_format=torch.contiguous_format)
-    pf = _f32c(p).reshape(K, N)
-    qf = _cplx_as_f32(q.reshape(K, N))
-    gf = _cplx_as_f32(gamma.reshape(K, N))
-    of = _f32c(omega).reshape(D)
-    m8 = _mask_u8(padding_mask, B, L)
-    hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
-    hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev) if (want_state or h is not None) else None
-    trunc = 0 if truncation is None or truncation < 1 else int(truncation)
-    nws = lib.mega_ema_fwd_workspace_bytes(B, D, N, L, 1 if bidirectional else 0, trunc)
-    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
-        rc = lib.mega_ema_fwd(_ptr(xd), _ptr(y), dt, xd.stride(0), xd.stride(1), xd.stride(2), y.stride(0),
-                              y.stride(1), y.stride(2), _ptr(pf), _ptr(qf), _ptr(gf), 1 if is_complex else 0,
-                              _ptr(of), _ptr(m8), _ptr(hin), _ptr(hout), B, D, N, L, 1 if bidirectional else 0,
-                              trunc, 1 if shift else 0, _ptr(ws), nws, _stream(dev))
-    _lib.check(rc, "ema_fwd")
-    hc = None
-    if hout is not None:
-        hc = torch.view_as_complex(hout) if is_complex else hout[..., 0]
-    return y, hc
+    _need_gpu(x)
+    return PreparedEMA(p, q, gamma, omega, bidirectional, truncation, shift)(x, padding_mask, h, want_state)
 
 
 def _dense(t: torch.Tensor) -> bool:
