@@ -17,6 +17,7 @@ SOURCES = [
     "capi.hip",
     "timestep_norm.hip",
     "ema_scan.hip",
+    "ema_mfma.hip",
     "elementwise.hip",
     "attention.hip",
     "long_conv.hip",

@@ -1,0 +1,632 @@
+// Moving-average layer forward on the matrix cores (gfx950 MFMA), ndim <= 16, bf16 activations.
+//
+// For one channel the layer is y = k * x + omega x with k[l] = Re sum_n p gamma q^l
+// (fairseq/modules/complex_exponential_moving_average.py:98-109,
+// fairseq/modules/base_moving_average.py:120-172).  Time is cut into tiles of 32 tokens.
+// With h the carried state (h' = q h + p x, fairseq/csrc/ops/ema_hidden.cc:31-63) a tile is
+//
+//     y_tile = K x_tile + C h_start        K[i][i'] = k[i - i'] (lower-triangular Toeplitz)
+//     h_end  = Q h_start + P x_tile        C[i][n]  = gamma_n q_n^{i+1},  P[n][i] = p_n q_n^{31-i}
+//
+// which is the reference's own incremental decomposition (kernel + carried-state bias,
+// fairseq/csrc/ops/ema_parameters.cc:37-77) applied per tile.  K, P, C are 32x32 matrices that
+// depend on the channel only, so they are generated once per wave from a q-power table in LDS
+// (kernel generation fused in) and kept in registers as MFMA A-operands; the B-operands are 16
+// columns of 32 tokens each, i.e. all three products are v_mfma_f32_16x16x32_bf16.
+//
+// One wave owns one (batch, channel) row for the whole sequence; a workgroup is 16 waves = 16
+// adjacent channels, so a [B, L, D] activation tensor is streamed as 32-byte pieces per token
+// that the workgroup transposes through LDS (the four workgroups that share a 128-byte line are
+// placed on the same XCD), and a [B, D, L] tensor as contiguous rows.
+//
+// A super-chunk of 16 segments x SEGT tiles is resident in LDS.  The 16 MFMA columns are the 16
+// segments, so the tile-to-tile recurrence of the state stays inside a lane:
+//   sweep 1: segment end states from a zero start            (P products only)
+//   scan   : 16-step serial scan over the segments per state (through LDS, lanes 0..15)
+//   sweep 2: K, P, C products with the true start states; y overwrites x in LDS
+#include "common.h"
+
+namespace mega {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kWaves = 16;               // channels per workgroup
+constexpr int kThreadsM = kWaves * 64;
+constexpr int kNS = 16;                  // complex states per channel (zero padded)
+
+struct MfmaArgs {
+  const void* x;
+  void* y;
+  int64_t sxb, sxd, sxl, syb, syd, syl;
+  const float* p;        // [K, N]
+  const float* q;        // [K, N, 2]
+  const float* gamma;    // [K, N, 2]
+  const float* omega;    // [D] or null (null: no residual in this pass)
+  const uint8_t* mask;   // [B, L] or null
+  const float* h_in;     // [B, D, N, 2] or null
+  float* h_tile;         // [B, D, 16, 2]: state after the last whole 32-token tile, or null
+  const float* acc_in;   // fp32, strides (sab, sad, sal), or null
+  float* acc_out;        // fp32, same strides; when set y is not written
+  int64_t sab, sad, sal;
+  int B, D, N, L;
+  int koff;              // first coefficient row of this direction
+  int reverse;           // logical time runs backwards
+  int lag;               // 1: the output at t excludes x[t] (backward half with shift)
+  int is_complex;
+  int xcd_map;           // 1: sibling channel blocks share an XCD
+};
+
+__device__ __forceinline__ float bf_hi(float v, __bf16* h) {
+  *h = (__bf16)v;
+  return v - (float)(*h);
+}
+
+template <int SEGT>
+struct Geo {
+  static constexpr int SEG = SEGT * 32;            // tokens per segment
+  static constexpr int SC = SEG * 16;              // tokens per super-chunk
+  static constexpr int SEGB = SEG * 2 + 16;        // bytes per segment in an LDS row (padded)
+  static constexpr int ROWB = SEGB * 16;           // bytes per channel row
+  static constexpr int XBUF = ROWB * kWaves;
+  static constexpr int POWB = 33 * kNS * 8;        // q-power table per channel (setup only, aliases xbuf)
+  static constexpr int SCANB = 16 * kNS * 8;       // segment states per channel
+  static constexpr int AUXB = 64 * 4 + kNS * 4 + kNS * 8;   // k table (64), p (16), gamma (16 x 2)
+  static constexpr int TOTAL = XBUF + kWaves * (SCANB + AUXB);
+  static_assert(POWB * kWaves <= XBUF, "power table must fit in the staging buffer");
+  __device__ static __forceinline__ int pos(int t) { return (t / SEG) * SEGB + (t % SEG) * 2; }
+};
+
+// LAYOUT 0: [B, D, L] rows contiguous in time; LAYOUT 1: [B, L, D] channels contiguous.
+template <int SEGT, int NW, int LAYOUT>
+__global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
+  using G = Geo<SEGT>;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int j = lane & 15, r = lane >> 4;          // MFMA column / row block
+
+  // ---- which (batch, channel block)
+  const int ncb = (A.D + kWaves - 1) / kWaves;
+  int b, cb;
+  {
+    int g = blockIdx.x;
+    if (A.xcd_map) {
+      const int xcd = g & 7, slot = g >> 3;
+      const int s = slot & 3, gi = (slot >> 2) * 8 + xcd;
+      const int per = ncb >> 2;
+      b = gi / per;
+      cb = (gi - b * per) * 4 + s;
+    } else {
+      b = g / ncb;
+      cb = g - b * ncb;
+    }
+  }
+  const int ch = cb * kWaves + wave;
+  const bool ch_ok = ch < A.D;
+  const int chc = ch_ok ? ch : A.D - 1;            // clamp: idle waves compute on a valid row, never store
+  const int kr = A.koff + chc;
+
+  char* xrow = smem + wave * G::ROWB;
+  char* powt = smem + wave * G::POWB;              // aliases the staging buffer during setup
+  char* scan = smem + G::XBUF + wave * G::SCANB;
+  char* aux = smem + G::XBUF + kWaves * G::SCANB + wave * G::AUXB;
+  float* kkt = (float*)aux;                        // [64]: k[idx] at kkt[32 + idx], zeros below
+  float* pbuf = kkt + 64;                          // [16]
+  float2* gbuf = (float2*)(pbuf + kNS);            // [16]
+
+  // ================= setup: q powers -> LDS, then K / P / C operands in registers
+  {
+    const int n = lane & 15, blk = lane >> 4;
+    float qr = 0.f, qi = 0.f, pv = 0.f, gr = 0.f, gi = 0.f;
+    if (n < A.N) {
+      const size_t o = ((size_t)kr * A.N + n);
+      qr = A.q[o * 2];
+      qi = A.is_complex ? A.q[o * 2 + 1] : 0.f;
+      pv = A.p[o];
+      gr = A.gamma[o * 2];
+      gi = A.is_complex ? A.gamma[o * 2 + 1] : 0.f;
+    }
+    // q^2, q^4, q^8, q^16, q^24
+    cfloat q1 = {qr, qi};
+    cfloat q2 = cmul(q1, q1), q4 = cmul(q2, q2), q8 = cmul(q4, q4), q16 = cmul(q8, q8), q24 = cmul(q16, q8);
+    cfloat base = blk == 0 ? cfloat{1.f, 0.f} : blk == 1 ? q8 : blk == 2 ? q16 : q24;
+    float2* pw = (float2*)powt;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      pw[(8 * blk + t) * kNS + n] = make_float2(base.re, base.im);
+      base = cmul(base, q1);
+    }
+    if (blk == 3) pw[32 * kNS + n] = make_float2(base.re, base.im);
+    if (blk == 0) {
+      pbuf[n] = pv;
+      gbuf[n] = make_float2(gr, gi);
+    }
+  }
+  __syncthreads();
+  bf16x8 Kw[NW][2], Pw[NW][2], Cw[NW][2];
+  float Qr[4], Qi[4];       // q^32 of this lane's four states
+  float Rr = 0.f, Ri = 0.f; // q^(32*SEGT) of state `lane` (lanes 0..15, segment scan)
+  float Hcr = 0.f, Hci = 0.f;
+  {
+    const float2* pw = (const float2*)powt;
+    // k table: lane e (< 32) sums over the states
+    {
+      const int e = lane & 31;
+      float s = 0.f;
+#pragma unroll
+      for (int n = 0; n < kNS; ++n) {
+        const float2 w = pw[e * kNS + n];
+        const float2 g = gbuf[n];
+        const float pn = pbuf[n];
+        s += pn * (g.x * w.x - g.y * w.y);
+      }
+      // lag 1 shifts the kernel by one tap; omega joins tap 0 of the pass that carries the residual
+      const int idx = e + A.lag;
+      if (lane < 32) {
+        if (idx < 32) kkt[32 + idx] = s;
+        kkt[lane] = 0.f;
+      }
+    }
+    __syncthreads();
+    if (lane == 0) {
+      if (A.lag) kkt[32] = 0.f;
+      if (A.omega) kkt[32] += A.omega[chc];
+    }
+    __syncthreads();
+    const int m = lane & 15, g = lane >> 4;
+    int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float2 w = pw[32 * kNS + nn[u]];
+      Qr[u] = w.x;
+      Qi[u] = w.y;
+    }
+    if (lane < 16) {
+      cfloat R = {1.f, 0.f};
+      const float2 w = pw[32 * kNS + lane];
+      for (int t = 0; t < SEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
+      Rr = R.re;
+      Ri = R.im;
+      if (A.h_in && lane < A.N && ch_ok) {
+        const size_t o = (((size_t)b * A.D + ch) * A.N + lane) * 2;
+        Hcr = A.h_in[o];
+        Hci = A.is_complex ? A.h_in[o + 1] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      float kv[8], pvv[8], cv[8];
+      const int row = 16 * mb + m;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int k = 8 * g + t;
+        // K: Toeplitz, rows = output time, k = input time
+        kv[t] = kkt[32 + row - k];
+        // P: rows = (state, part), k = input time i: p q^{31-i}
+        {
+          const int n = row >> 1, part = row & 1;
+          const float2 w = pw[(31 - k) * kNS + n];
+          pvv[t] = pbuf[n] * (part ? w.y : w.x);
+        }
+        // C: rows = output time i, k-slot t of block g <-> state nn[t/2 (+2)] part t&1;
+        // gamma q^{i+1-lag}: real part multiplies Re h, minus imaginary part multiplies Im h
+        {
+          const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
+          const int part = t & 1;
+          const int e = row + 1 - A.lag;
+          const float2 w = pw[e * kNS + n];
+          const float2 gm = gbuf[n];
+          const float re = gm.x * w.x - gm.y * w.y;
+          const float im = gm.x * w.y + gm.y * w.x;
+          cv[t] = part ? -im : re;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        __bf16 h;
+        float rem = bf_hi(kv[t], &h);
+        Kw[0][mb][t] = h;
+        if (NW > 1) Kw[NW - 1][mb][t] = (__bf16)rem;
+        rem = bf_hi(pvv[t], &h);
+        Pw[0][mb][t] = h;
+        if (NW > 1) Pw[NW - 1][mb][t] = (__bf16)rem;
+        rem = bf_hi(cv[t], &h);
+        Cw[0][mb][t] = h;
+        if (NW > 1) Cw[NW - 1][mb][t] = (__bf16)rem;
+      }
+    }
+  }
+  __syncthreads();      // the power table (aliasing the staging buffer) is dead from here on
+
+  // ================= streaming over super-chunks
+  const int nsc = (A.L + G::SC - 1) / G::SC;
+  const int last_tile = A.L / 32 - 1;             // global index of the last whole tile
+  constexpr int NLD = G::SC * 2 * kWaves / (kThreadsM * 16);   // 16-byte loads per thread per super-chunk
+  uint4 pre[NLD];
+  const bf16_t* xg = (const bf16_t*)A.x;
+
+  auto issue_loads = [&](int sc) {
+    const int t0 = sc * G::SC;
+#pragma unroll
+    for (int k = 0; k < NLD; ++k) {
+      pre[k] = make_uint4(0, 0, 0, 0);
+      if (LAYOUT == 1) {
+        // thread -> (token, half of the 16 channels)
+        const int tk = k * (kThreadsM / 2) + (tid >> 1);
+        const int half = tid & 1;
+        const int tau = t0 + tk;
+        const int c0 = cb * kWaves + half * 8;
+        if (tau < A.L && c0 < A.D) {
+          const int t = A.reverse ? A.L - 1 - tau : tau;
+          if (!(A.mask && A.mask[(size_t)b * A.L + t]))
+            pre[k] = *(const uint4*)(xg + b * A.sxb + (int64_t)t * A.sxl + c0);
+        }
+      } else {
+        // wave -> its own row; lane -> 8 consecutive tokens
+        const int tk = k * 512 + lane * 8;
+        const int tau = t0 + tk;
+        if (tau < A.L) {
+          const int t = A.reverse ? A.L - 8 - tau : tau;
+          uint4 v = *(const uint4*)(xg + b * A.sxb + (int64_t)chc * A.sxd + t);
+          if (A.reverse) {
+            // reverse the 8 elements
+            uint4 w;
+            w.x = (v.w >> 16) | (v.w << 16);
+            w.y = (v.z >> 16) | (v.z << 16);
+            w.z = (v.y >> 16) | (v.y << 16);
+            w.w = (v.x >> 16) | (v.x << 16);
+            v = w;
+          }
+          if (A.mask) {
+            const uint2 mk = *(const uint2*)(A.mask + (size_t)b * A.L + t);
+            uint32_t mm[2] = {mk.x, mk.y};
+            uint32_t* vv = (uint32_t*)&v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int src = A.reverse ? 7 - e : e;           // mask byte of logical element e
+              const bool pad = ((mm[src >> 2] >> ((src & 3) * 8)) & 0xffu) != 0;
+              if (pad) vv[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+            }
+          }
+          pre[k] = v;
+        }
+      }
+    }
+  };
+
+  issue_loads(0);
+  for (int sc = 0; sc < nsc; ++sc) {
+    const int t0 = sc * G::SC;
+    // ---- stage the prefetched super-chunk into LDS
+#pragma unroll
+    for (int k = 0; k < NLD; ++k) {
+      if (LAYOUT == 1) {
+        const int tk = k * (kThreadsM / 2) + (tid >> 1);
+        const int half = tid & 1;
+        const uint32_t* vv = (const uint32_t*)&pre[k];
+        char* base = smem + (half * 8) * G::ROWB + G::pos(tk);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const uint16_t el = (uint16_t)(vv[e >> 1] >> ((e & 1) * 16));
+          *(uint16_t*)(base + e * G::ROWB) = el;
+        }
+      } else {
+        const int tk = k * 512 + lane * 8;
+        *(uint4*)(xrow + G::pos(tk)) = pre[k];
+      }
+    }
+    __syncthreads();
+    if (sc + 1 < nsc) issue_loads(sc + 1);
+
+    // ---- sweep 1: segment end states from a zero start
+    float Er[4] = {0.f, 0.f, 0.f, 0.f}, Ei[4] = {0.f, 0.f, 0.f, 0.f};
+    const char* xcol = xrow + j * G::SEGB + r * 16;
+#pragma unroll
+    for (int i = 0; i < SEGT; ++i) {
+      const bf16x8 X = *(const bf16x8*)(xcol + i * 64);
+      f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][0], X, S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][1], X, S1, 0, 0, 0);
+      }
+      const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
+      const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float nr = Qr[u] * Er[u] - Qi[u] * Ei[u] + sr[u];
+        const float ni = Qr[u] * Ei[u] + Qi[u] * Er[u] + si[u];
+        Er[u] = nr;
+        Ei[u] = ni;
+      }
+    }
+    // ---- scan over the 16 segments (per state), carried across super-chunks
+    {
+      float4* sb = (float4*)scan;     // [16 segments][8 float4]: states (2r, 2r+1) at [j][r], (8+2r, 9+2r) at [j][4+r]
+      sb[j * 8 + r] = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
+      sb[j * 8 + 4 + r] = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+      if (lane < 16) {
+        float2* s2 = (float2*)scan;   // [16][16] complex, state n of segment jj at s2[jj*16 + slot(n)]
+        const int slot = lane < 8 ? lane : lane;      // states are stored in order 0..15
+        float hr = Hcr, hi = Hci;
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) {
+          const float2 e = s2[jj * 16 + slot];
+          s2[jj * 16 + slot] = make_float2(hr, hi);
+          const float nr = Rr * hr - Ri * hi + e.x;
+          const float ni = Rr * hi + Ri * hr + e.y;
+          hr = nr;
+          hi = ni;
+        }
+        Hcr = hr;
+        Hci = hi;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_wave_barrier();
+    }
+    float Hr[4], Hi[4];
+    {
+      const float4* sb = (const float4*)scan;
+      const float4 a = sb[j * 8 + r], c = sb[j * 8 + 4 + r];
+      Hr[0] = a.x; Hi[0] = a.y; Hr[1] = a.z; Hi[1] = a.w;
+      Hr[2] = c.x; Hi[2] = c.y; Hr[3] = c.z; Hi[3] = c.w;
+    }
+    // ---- sweep 2: outputs
+    char* ycol = xrow + j * G::SEGB;
+#pragma unroll
+    for (int i = 0; i < SEGT; ++i) {
+      const bf16x8 X = *(const bf16x8*)(xcol + i * 64);
+      f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
+      f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
+      bf16x8 Hop[NW];
+      {
+        const float hv[8] = {Hr[0], Hi[0], Hr[1], Hi[1], Hr[2], Hi[2], Hr[3], Hi[3]};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          __bf16 h;
+          const float rem = bf_hi(hv[t], &h);
+          Hop[0][t] = h;
+          if (NW > 1) Hop[NW - 1][t] = (__bf16)rem;
+        }
+      }
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][0], X, S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][1], X, S1, 0, 0, 0);
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][0], X, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][1], X, Y1, 0, 0, 0);
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop[0], Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop[0], Y1, 0, 0, 0);
+      }
+      if (NW > 1) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[0][0], Hop[NW - 1], Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[0][1], Hop[NW - 1], Y1, 0, 0, 0);
+      }
+      const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
+      const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float nr = Qr[u] * Hr[u] - Qi[u] * Hi[u] + sr[u];
+        const float ni = Qr[u] * Hi[u] + Qi[u] * Hr[u] + si[u];
+        Hr[u] = nr;
+        Hi[u] = ni;
+      }
+      if (A.h_tile && ch_ok) {
+        const int gt = (t0 + j * G::SEG + i * 32) >> 5;
+        if (gt == last_tile) {
+          float* ho = A.h_tile + (((size_t)b * A.D + ch) * kNS) * 2;
+          const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            ho[nn[u] * 2] = Hr[u];
+            ho[nn[u] * 2 + 1] = Hi[u];
+          }
+        }
+      }
+      // y (bf16) overwrites x in place: tokens 32 i + 16 mb + 4 r + {0..3} of segment j
+      {
+        bf16_t o0[4], o1[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          o0[u] = from_float<bf16_t>(Y0[u]);
+          o1[u] = from_float<bf16_t>(Y1[u]);
+        }
+        *(uint2*)(ycol + i * 64 + r * 8) = *(const uint2*)o0;
+        *(uint2*)(ycol + i * 64 + 32 + r * 8) = *(const uint2*)o1;
+      }
+    }
+    __syncthreads();
+    // ---- store the super-chunk
+    bf16_t* yg = (bf16_t*)A.y;
+#pragma unroll
+    for (int k = 0; k < NLD; ++k) {
+      if (LAYOUT == 1) {
+        const int tk = k * (kThreadsM / 2) + (tid >> 1);
+        const int half = tid & 1;
+        const int tau = t0 + tk;
+        const int c0 = cb * kWaves + half * 8;
+        if (tau < A.L && c0 < A.D) {
+          const int t = A.reverse ? A.L - 1 - tau : tau;
+          const char* base = smem + (half * 8) * G::ROWB + G::pos(tk);
+          float v[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            bf16_t el;
+            el.u = *(const uint16_t*)(base + e * G::ROWB);
+            v[e] = to_float(el);
+          }
+          const bool direct = !A.acc_in && !A.acc_out && !(A.mask && A.omega);
+          if (direct) {
+            uint4 o;
+            uint32_t* oo = (uint32_t*)&o;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+              oo[e >> 1] = (uint32_t)(*(const uint16_t*)(base + e * G::ROWB)) |
+                           ((uint32_t)(*(const uint16_t*)(base + (e + 1) * G::ROWB)) << 16);
+            *(uint4*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = o;
+          } else {
+            if (A.acc_in) {
+              const float* ai = A.acc_in + b * A.sab + (int64_t)t * A.sal + c0;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] += ai[e];
+            }
+            if (A.mask && A.omega && A.mask[(size_t)b * A.L + t]) {
+              // the residual uses the unmasked input (base_moving_average.py:138)
+              const bf16_t* xo = xg + b * A.sxb + (int64_t)t * A.sxl + c0;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] += A.omega[c0 + e] * to_float(xo[e]);
+            }
+            if (A.acc_out) {
+              float* ao = A.acc_out + b * A.sab + (int64_t)t * A.sal + c0;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) ao[e] = v[e];
+            } else {
+              Vec<bf16_t, 8> o;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16_t>(v[e]);
+              *(Vec<bf16_t, 8>*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = o;
+            }
+          }
+        }
+      } else {
+        const int tk = k * 512 + lane * 8;
+        const int tau = t0 + tk;
+        if (tau < A.L && ch_ok) {
+          const int t = A.reverse ? A.L - 8 - tau : tau;       // first physical token of the 8
+          Vec<bf16_t, 8> in = *(const Vec<bf16_t, 8>*)(xrow + G::pos(tk));
+          float v[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = to_float(in.v[A.reverse ? 7 - e : e]);   // physical order
+          if (A.acc_in) {
+            const float* ai = A.acc_in + b * A.sab + (int64_t)ch * A.sad + t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += ai[e];
+          }
+          if (A.mask && A.omega) {
+            const uint8_t* mk = A.mask + (size_t)b * A.L + t;
+            const bf16_t* xo = xg + b * A.sxb + (int64_t)ch * A.sxd + t;
+            const float om = A.omega[ch];
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (mk[e]) v[e] += om * to_float(xo[e]);
+          }
+          if (A.acc_out) {
+            float* ao = A.acc_out + b * A.sab + (int64_t)ch * A.sad + t;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ao[e] = v[e];
+          } else {
+            Vec<bf16_t, 8> o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16_t>(v[e]);
+            *(Vec<bf16_t, 8>*)(yg + b * A.syb + (int64_t)ch * A.syd + t) = o;
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Finishes the carried state: from the state after the last whole tile (time Lb = 32 floor(L/32))
+// to time L: h = q^r h_tile + sum_{i<r} p q^{r-1-i} x[Lb + i], r = L - Lb < 32.
+template <typename T>
+__global__ void ema_state_tail_kernel(const T* __restrict__ x, int64_t sxb, int64_t sxd, int64_t sxl,
+                                      const uint8_t* __restrict__ mask, const float* __restrict__ p,
+                                      const float* __restrict__ q, const float* __restrict__ h_tile,
+                                      float* __restrict__ h_out, int B, int D, int N, int L, int is_complex) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= (int64_t)B * D * N) return;
+  const int n = (int)(gid % N);
+  const int d = (int)((gid / N) % D);
+  const int b = (int)(gid / ((int64_t)N * D));
+  const float qr = q[((size_t)d * N + n) * 2], qi = is_complex ? q[((size_t)d * N + n) * 2 + 1] : 0.f;
+  const float pv = p[(size_t)d * N + n];
+  const float* ht = h_tile + (((size_t)b * D + d) * kNS + n) * 2;
+  float hr = ht[0], hi = ht[1];
+  const int Lb = (L / 32) * 32;
+  for (int t = Lb; t < L; ++t) {
+    float u = 0.f;
+    if (!(mask && mask[(size_t)b * L + t])) u = to_float(x[b * sxb + d * sxd + t * sxl]);
+    const float nr = qr * hr - qi * hi + pv * u;
+    const float ni = qr * hi + qi * hr;
+    hr = nr;
+    hi = ni;
+  }
+  float* ho = h_out + (((size_t)b * D + d) * N + n) * 2;
+  ho[0] = hr;
+  ho[1] = hi;
+}
+
+}  // namespace
+
+// Host side: decides whether the MFMA path covers a request and launches it.
+// Returns 1 if handled, 0 if the caller must use the generic path, < 0 on a launch error.
+int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb,
+                 int64_t syd, int64_t syl, const float* p, const float* q, const float* gamma, int is_complex,
+                 const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
+                 int64_t N, int64_t L, int bidirectional, int64_t Lk, int shift, float* acc, float* h_tile,
+                 hipStream_t s) {
+  if (dtype != MEGA_BF16 || N > kNS || Lk > 0 || L < 256) return 0;
+  int layout;
+  if (sxd == 1 && syd == 1 && D % 8 == 0 && sxl % 8 == 0 && syl % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 1;
+  else if (sxl == 1 && syl == 1 && L % 8 == 0 && sxd % 8 == 0 && syd % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 0;
+  else return 0;
+  if (((uintptr_t)x % 16) || ((uintptr_t)y % 16) || (mask && layout == 0 && ((uintptr_t)mask % 8))) return 0;
+  if (B * ceil_div(D, kWaves) >= (int64_t)1 << 31) return 0;
+  constexpr int SEGT = 4;
+  using G = Geo<SEGT>;
+  const int ncb = (int)ceil_div(D, kWaves);
+  MfmaArgs A;
+  A.x = x; A.y = y; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.syb = syb; A.syd = syd; A.syl = syl;
+  A.p = p; A.q = q; A.gamma = gamma; A.mask = mask;
+  A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L; A.is_complex = is_complex;
+  A.xcd_map = (layout == 1 && ncb % 4 == 0 && ((B * ncb / 4) % 8) == 0) ? 1 : 0;
+  // fp32 partial sums between the two directions live in [B, D, L]-shaped storage with y's layout
+  A.sab = layout == 1 ? L * D : D * L;
+  A.sad = layout == 1 ? 1 : L;
+  A.sal = layout == 1 ? D : 1;
+  const dim3 grid((unsigned)(B * ncb));
+  auto launch = [&](const MfmaArgs& a) -> int {
+    auto kern = layout == 1 ? ema_mfma_kernel<SEGT, 2, 1> : ema_mfma_kernel<SEGT, 2, 0>;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[layout]) {
+      hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
+      attr_set[layout] = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(kThreadsM), G::TOTAL, s, a);
+    MEGA_CHECK_LAUNCH("ema_fwd (matrix-core path)");
+    return MEGA_OK;
+  };
+  if (bidirectional) {
+    MfmaArgs Bk = A;
+    Bk.koff = (int)D; Bk.reverse = 1; Bk.lag = shift ? 1 : 0;
+    Bk.omega = nullptr; Bk.h_in = nullptr; Bk.h_tile = nullptr; Bk.acc_in = nullptr; Bk.acc_out = acc;
+    int rc = launch(Bk);
+    if (rc) return rc;
+  }
+  A.koff = 0; A.reverse = 0; A.lag = 0; A.omega = omega; A.h_in = h_in;
+  A.h_tile = h_out ? h_tile : nullptr;
+  A.acc_in = bidirectional ? acc : nullptr; A.acc_out = nullptr;
+  int rc = launch(A);
+  if (rc) return rc;
+  if (h_out) {
+    const int64_t n = B * D * N;
+    hipLaunchKernelGGL(ema_state_tail_kernel<bf16_t>, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s,
+                       (const bf16_t*)x, sxb, sxd, sxl, mask, p, q, h_tile, h_out, (int)B, (int)D, (int)N, (int)L,
+                       is_complex);
+    MEGA_CHECK_LAUNCH("ema_fwd state tail");
+  }
+  return 1;
+}
+
+size_t ema_mfma_workspace_bytes(int64_t B, int64_t D, int64_t L, int bidirectional) {
+  size_t n = align_up((size_t)B * D * kNS * 2 * 4, 256);          // h_tile
+  if (bidirectional) n += align_up((size_t)B * D * L * 4, 256);    // fp32 partial sums
+  return n;
+}
+
+}  // namespace mega

@@ -24,6 +24,14 @@
 #include "common.h"
 
 namespace mega {
+
+// matrix-core path (ema_mfma.hip)
+int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb,
+                 int64_t syd, int64_t syl, const float* p, const float* q, const float* gamma, int is_complex,
+                 const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
+                 int64_t N, int64_t L, int bidirectional, int64_t Lk, int shift, float* acc, float* h_tile,
+                 hipStream_t s);
+
 namespace {
 
 constexpr int kNPT = 4;          // complex states per thread
@@ -273,7 +281,7 @@ __global__ void coef_prep_kernel(const float* __restrict__ p, const float* __res
 
 struct Plan {
   int NP, TPR, Tc, nchunks;
-  size_t coef_bytes, st_bytes, acc_bytes, total;
+  size_t coef_bytes, st_bytes, acc_bytes, tile_bytes, total;
 };
 
 Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_acc) {
@@ -298,7 +306,8 @@ Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_
   pl.st_bytes = align_up((size_t)B * pl.nchunks * D * pl.NP * 2 * 4, 256);
   pl.acc_bytes = need_acc ? align_up((size_t)B * L * D * 4, 256) : 0;
   (void)nsets;
-  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes;
+  pl.tile_bytes = align_up((size_t)B * D * 16 * 2 * 4, 256);      // state after the last whole tile
+  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
   return pl;
 }
 
@@ -486,6 +495,10 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
   float* coef = (float*)w;
   float* st = (float*)(w + pl.coef_bytes);
   float* acc = need_acc ? (float*)(w + pl.coef_bytes + pl.st_bytes) : nullptr;
+  float* h_tile = (float*)(w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes);
+  rc = ema_mfma_try(x, y, dtype, sxb, sxd, sxl, syb, syd, syl, p, q, gamma, is_complex, omega, mask, h_in, h_out, B,
+                    D, N, L, bidirectional, Lk, shift, acc, h_tile, s);
+  if (rc != 0) return rc < 0 ? rc : MEGA_OK;
   const int ndir = bidirectional ? 2 : 1;
   {
     const int64_t n = (int64_t)D * pl.NP * ndir;
