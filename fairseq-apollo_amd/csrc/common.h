@@ -44,15 +44,10 @@ __device__ __forceinline__ float to_float(f16_t v) { return (float)v.h; }
 template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
-  // round to nearest even; NaN stays NaN
-  uint32_t u = __float_as_uint(v);
+  // round to nearest even in hardware (v_cvt_pk_bf16_f32 on gfx950)
+  const __bf16 h = (__bf16)v;
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r.u = (uint16_t)((u >> 16) | 0x0040u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.u = (uint16_t)(u >> 16);
-  }
+  r.u = __builtin_bit_cast(uint16_t, h);
   return r;
 }
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) {

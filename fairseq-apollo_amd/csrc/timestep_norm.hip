@@ -26,7 +26,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kNV = 16;                       // vectors kept in registers per thread
 constexpr int kPartCap = kThreads * kNV;      // vectors per tile
+constexpr int kMaxTT = 64;                    // tokens per tile (16 lanes x 4 tokens in the scan)
 constexpr uint32_t kSpinLimit = 1u << 22;
+constexpr int kLbWords = 2048;                // tile aggregates staged in LDS per look-back round
 
 struct TsnHeader {
   uint32_t ticket;
@@ -51,9 +53,8 @@ struct TsnParams {
   float* cummean;
   float* cumrstd;
   TsnHeader* hdr;
-  uint32_t* flags;   // [B*ntiles]
-  uint32_t* tcnt;    // [B*ntiles] unmasked tokens per tile
-  float* agg;        // [B*ntiles*G*2] (mean, var) of the tile
+  uint32_t* tcnt;              // [B*ntiles] unmasked tokens of the tile + 1 (0 = not published)
+  unsigned long long* agg;     // [B*ntiles*G] (mean, var) of the tile; bit 63 set = published
   int B, L, H, G;
   int TT, ntiles;
   int TPT;           // vectors per token
@@ -61,25 +62,114 @@ struct TsnParams {
   float eps;
 };
 
-template <typename T, int VEC, bool HOIST>
+// ---- lane-group primitives (DPP inside rows of 16 lanes)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141;
+constexpr int kRowMirror = 0x140;
+
+// sum over LPG adjacent lanes (LPG a power of two <= 64); every lane of the group gets the sum
+template <int LPG>
+__device__ __forceinline__ float group_sum(float v) {
+  if (LPG >= 2) v += dpp_f<kXor1>(v);
+  if (LPG >= 4) v += dpp_f<kXor2>(v);
+  if (LPG >= 8) v += dpp_f<kHalfMirror>(v);
+  if (LPG >= 16) v += dpp_f<kRowMirror>(v);
+  if (LPG >= 32) v += __shfl_xor(v, 16);
+  if (LPG >= 64) v += __shfl_xor(v, 32);
+  return v;
+}
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+
+// acc + x0 + x1 and acc + x0^2 + x1^2 for a packed pair of 16-bit values
+template <typename T>
+__device__ __forceinline__ float dot2_ones(uint32_t w, float acc) {
+  if constexpr (sizeof(T) == 2 && !__is_same(T, f16_t)) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3f803f80u),
+                                           acc, false);
+  } else {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, w), __builtin_bit_cast(f16x2_t, 0x3c003c00u), acc, false);
+  }
+}
+template <typename T>
+__device__ __forceinline__ float dot2_self(uint32_t w, float acc) {
+  if constexpr (sizeof(T) == 2 && !__is_same(T, f16_t)) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, w), acc, false);
+  } else {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, w), __builtin_bit_cast(f16x2_t, w), acc, false);
+  }
+}
+
+// merge of two sets of equally weighted steps; one reciprocal per merge
+__device__ __forceinline__ Moments merge(Moments a, Moments b) {
+  const float n = a.n + b.n;
+  const float rn = n > 0.f ? __builtin_amdgcn_rcpf(n) : 0.f;
+  const float cb = b.n * rn, ca = a.n * rn;
+  const float d = b.mean - a.mean;
+  Moments r;
+  r.n = n;
+  r.mean = a.mean + cb * d;
+  r.var = ca * a.var + cb * b.var + (ca * d) * (cb * d);
+  return r;
+}
+
+template <int CTRL>
+__device__ __forceinline__ Moments dpp_m(Moments m) {
+  return Moments{dpp_f<CTRL>(m.n), dpp_f<CTRL>(m.mean), dpp_f<CTRL>(m.var)};
+}
+
+// all 16 lanes of a row get the merge of the row
+__device__ __forceinline__ Moments row_reduce(Moments m) {
+  m = merge(m, dpp_m<kXor1>(m));
+  m = merge(m, dpp_m<kXor2>(m));
+  m = merge(m, dpp_m<kHalfMirror>(m));
+  m = merge(m, dpp_m<kRowMirror>(m));
+  return m;
+}
+
+// inclusive scan over the 16 lanes of a row (lanes shifted in from outside the row are empty sets)
+__device__ __forceinline__ Moments row_scan(Moments m) {
+  m = merge(dpp_m<0x111>(m), m);
+  m = merge(dpp_m<0x112>(m), m);
+  m = merge(dpp_m<0x114>(m), m);
+  m = merge(dpp_m<0x118>(m), m);
+  return m;
+}
+
+__device__ __forceinline__ uint32_t row_sum_u32(uint32_t v) {
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kXor1, 0xf, 0xf, true);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kXor2, 0xf, 0xf, true);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kHalfMirror, 0xf, 0xf, true);
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, kRowMirror, 0xf, 0xf, true);
+  return v;
+}
+
+__device__ __forceinline__ unsigned long long pack_agg(float mean, float var) {
+  return ((unsigned long long)(__float_as_uint(var) | 0x80000000u) << 32) | __float_as_uint(mean);
+}
+
+// LPGT > 0: groups are LPGT adjacent lanes and are reduced with lane shuffles;
+// LPGT == 0: any group size, partial sums go through LDS.
+template <typename T, int VEC, bool HOIST, int LPGT>
 __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) {
   extern __shared__ float smem[];
-  float* part = smem;                              // [kPartCap]
-  float* s_mean = part + kPartCap;                 // [TT*G]
-  float* s_var = s_mean + (size_t)P.TT * P.G;      // [TT*G]
-  float* s_carry = s_var + (size_t)P.TT * P.G;     // [3*G]
-  float* s_slot = s_carry + 3 * (size_t)P.G;       // [3*max(G,256)]
-  float* s_lcnt = s_slot + 3 * (size_t)(P.G > kThreads ? P.G : kThreads);  // [TT]
-  uint8_t* s_mask = (uint8_t*)(s_lcnt + P.TT);     // [TT]
+  float* s_mean = smem;                            // [TT*G]  group mean, later running mean
+  float* s_var = s_mean + (size_t)P.TT * P.G;      // [TT*G]  group var, later running rstd
+  uint8_t* s_mask = (uint8_t*)(s_var + (size_t)P.TT * P.G);   // [TT]
+  unsigned long long* s_lbw = (unsigned long long*)(s_mask + ((P.TT + 15) / 16) * 16);   // [kLbWords]
+  uint32_t* s_lbc = (uint32_t*)(s_lbw + kLbWords);                                       // [kLbWords]
+  float* part = (float*)(s_lbc + kLbWords);                   // [kPartCap] (LPGT == 0 only)
   __shared__ uint32_t s_ticket;
-  __shared__ uint32_t s_prevcnt;
   __shared__ uint32_t s_last;
 
   const int tid = threadIdx.x;
-  if (tid == 0) {
-    s_ticket = atomicAdd(&P.hdr->ticket, 1u);
-    s_prevcnt = 0;
-  }
+  if (tid == 0) s_ticket = atomicAdd(&P.hdr->ticket, 1u);
   __syncthreads();
   const int ticket = (int)s_ticket;
   const int tile = ticket / P.B;
@@ -99,144 +189,210 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
 #pragma unroll
   for (int j = 0; j < kNV; ++j) {
     const int v = j * kThreads + tid;
-    if (v < nvec) xv[j] = xin[v];
+    if (v < nvec) {
+      xv[j] = xin[v];
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xv[j].v[i] = from_float<T>(0.f);
+    }
   }
   for (int t = tid; t < nt; t += kThreads)
     s_mask[t] = P.mask ? (P.mask[(size_t)b * P.L + t0 + t] != 0) : 0;
 
-  // ---- phase 1: group means
+  // ---- moments of every (token, group): mean first, then the variance around it
+  if (LPGT > 0) {
 #pragma unroll
-  for (int j = 0; j < kNV; ++j) {
-    const int v = j * kThreads + tid;
-    if (v < nvec) {
-      float s = 0.f;
+    for (int j = 0; j < kNV; ++j) {
+      const int v = j * kThreads + tid;
+      float m, gv;
+      if constexpr (sizeof(T) == 2 && VEC >= 2) {
+        // 16-bit activations: sum and sum of squares by packed dot products.  The difference
+        // E[x^2] - mean^2 is taken in fp32, which resolves more than the 8 / 11 significant bits
+        // the inputs themselves carry.
+        float s = 0.f, q = 0.f;
+        const uint32_t* w = (const uint32_t*)&xv[j];
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) s += to_float(xv[j].v[i]);
-      part[v] = s;
-    }
-  }
-  __syncthreads();
-  for (int item = tid; item < nt * G; item += kThreads) {
-    const int tok = item / G, g = item - tok * G;
-    const float* pp = part + tok * TPT + g * LPG;
-    float s = 0.f;
-    for (int i = 0; i < LPG; ++i) s += pp[i];
-    s_mean[item] = s * inv_dg;
-  }
-  __syncthreads();
-  // ---- phase 2: group variances around the group mean
+        for (int i = 0; i < VEC / 2; ++i) {
+          s = dot2_ones<T>(w[i], s);
+          q = dot2_self<T>(w[i], q);
+        }
+        m = group_sum<LPGT>(s) * inv_dg;
+        gv = fmaxf(group_sum<LPGT>(q) * inv_dg - m * m, 0.f);
+      } else {
+        float s = 0.f;
 #pragma unroll
-  for (int j = 0; j < kNV; ++j) {
-    const int v = j * kThreads + tid;
-    if (v < nvec) {
-      const int tok = v / TPT;
-      const int g = (v - tok * TPT) / LPG;
-      const float m = s_mean[tok * G + g];
-      float s = 0.f;
+        for (int i = 0; i < VEC; ++i) s += to_float(xv[j].v[i]);
+        m = group_sum<LPGT>(s) * inv_dg;
+        float s2 = 0.f;
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        const float d = to_float(xv[j].v[i]) - m;
-        s += d * d;
+        for (int i = 0; i < VEC; ++i) {
+          const float d = to_float(xv[j].v[i]) - m;
+          s2 += d * d;
+        }
+        gv = group_sum<LPGT>(s2) * inv_dg;
       }
-      part[v] = s;
-    }
-  }
-  __syncthreads();
-  for (int item = tid; item < nt * G; item += kThreads) {
-    const int tok = item / G, g = item - tok * G;
-    const float* pp = part + tok * TPT + g * LPG;
-    float s = 0.f;
-    for (int i = 0; i < LPG; ++i) s += pp[i];
-    s_var[item] = s * inv_dg;
-  }
-  __syncthreads();
-
-  // ---- phase 3: scan over the tile's tokens from a zero state; publish the aggregate
-  const size_t tslot = (size_t)b * P.ntiles + tile;
-  for (int g = tid; g < G; g += kThreads) {
-    Moments st = {0.f, 0.f, 0.f};
-    for (int tok = 0; tok < nt; ++tok) {
-      const float gm = s_mean[tok * G + g];
-      const float gv = s_var[tok * G + g];
-      if (P.group_mean) P.group_mean[((size_t)b * P.L + t0 + tok) * G + g] = gm;
-      if (!s_mask[tok]) st = combine(st, Moments{1.f, gm, gv});
-      s_mean[tok * G + g] = st.mean;
-      s_var[tok * G + g] = st.var;
-      if (g == 0) s_lcnt[tok] = st.n;
-    }
-    publish_f32(&P.agg[(tslot * G + g) * 2 + 0], st.mean);
-    publish_f32(&P.agg[(tslot * G + g) * 2 + 1], st.var);
-    if (g == 0) publish_u32(&P.tcnt[tslot], (uint32_t)st.n);
-  }
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) release_flag(&P.flags[tslot], 1u);
-
-  // ---- phase 4: wait for the earlier tiles of this row, fold them into the carry-in
-  for (int p = tid; p < tile; p += kThreads) {
-    const uint32_t* f = &P.flags[(size_t)b * P.ntiles + p];
-    uint32_t spins = 0;
-    while (acquire_flag(f) == 0u) {
-      __builtin_amdgcn_s_sleep(2);
-      if (++spins > kSpinLimit) {
-        publish_u32(&P.hdr->error, 1u);
-        break;
+      if ((tid & (LPGT - 1)) == 0 && v < nvec) {
+        const int tok = v / TPT;
+        const int g = (v - tok * TPT) / LPGT;
+        s_mean[tok * G + g] = m;
+        s_var[tok * G + g] = gv;
       }
     }
-    atomicAdd(&s_prevcnt, fetch_u32(&P.tcnt[(size_t)b * P.ntiles + p]));
-  }
-  __syncthreads();
-  const int NS = G >= kThreads ? 1 : kThreads / G;
-  for (int item = tid; item < G * NS; item += kThreads) {
-    const int slot = item / G, g = item - slot * G;
-    Moments st = {0.f, 0.f, 0.f};
-    for (int p = slot; p < tile; p += NS) {
-      const size_t ps = (size_t)b * P.ntiles + p;
-      Moments a;
-      a.n = (float)fetch_u32(&P.tcnt[ps]);
-      a.mean = fetch_f32(&P.agg[(ps * G + g) * 2 + 0]);
-      a.var = fetch_f32(&P.agg[(ps * G + g) * 2 + 1]);
-      st = combine(st, a);
+    __syncthreads();
+  } else {
+#pragma unroll
+    for (int j = 0; j < kNV; ++j) {
+      const int v = j * kThreads + tid;
+      if (v < nvec) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s += to_float(xv[j].v[i]);
+        part[v] = s;
+      }
     }
-    s_slot[item * 3 + 0] = st.n;
-    s_slot[item * 3 + 1] = st.mean;
-    s_slot[item * 3 + 2] = st.var;
-  }
-  __syncthreads();
-  for (int g = tid; g < G; g += kThreads) {
-    Moments st = {(float)P.prev_count[b], P.prev_mean[(size_t)b * G + g], P.prev_var[(size_t)b * G + g]};
-    for (int slot = 0; slot < NS; ++slot) {
-      const int item = slot * G + g;
-      st = combine(st, Moments{s_slot[item * 3 + 0], s_slot[item * 3 + 1], s_slot[item * 3 + 2]});
+    __syncthreads();
+    for (int item = tid; item < nt * G; item += kThreads) {
+      const int tok = item / G, g = item - tok * G;
+      const float* pp = part + tok * TPT + g * LPG;
+      float s = 0.f;
+      for (int i = 0; i < LPG; ++i) s += pp[i];
+      s_mean[item] = s * inv_dg;
     }
-    s_carry[g * 3 + 0] = st.n;
-    s_carry[g * 3 + 1] = st.mean;
-    s_carry[g * 3 + 2] = st.var;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kNV; ++j) {
+      const int v = j * kThreads + tid;
+      if (v < nvec) {
+        const int tok = v / TPT;
+        const int g = (v - tok * TPT) / LPG;
+        const float m = s_mean[tok * G + g];
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          const float d = to_float(xv[j].v[i]) - m;
+          s += d * d;
+        }
+        part[v] = s;
+      }
+    }
+    __syncthreads();
+    for (int item = tid; item < nt * G; item += kThreads) {
+      const int tok = item / G, g = item - tok * G;
+      const float* pp = part + tok * TPT + g * LPG;
+      float s = 0.f;
+      for (int i = 0; i < LPG; ++i) s += pp[i];
+      s_var[item] = s * inv_dg;
+    }
+    __syncthreads();
   }
-  __syncthreads();
 
-  // ---- phase 5: running statistics of every token of the tile
+  // ---- running statistics.  A row of 16 lanes owns one group: lane l16 scans its TPL tokens, the
+  // row scans across lanes and publishes the tile aggregate.  The aggregates of the earlier tiles of
+  // this batch row are then fetched as one contiguous block into LDS (every word says by itself
+  // whether it has been published: no fence on either side) and folded into the carry-in.
+  const int row16 = tid >> 4, l16 = tid & 15;
+  const int TPL = (P.TT + 15) >> 4;                 // tokens per lane (<= 4)
+  const size_t trow = (size_t)b * P.ntiles;
   const bool last_tile = tile == P.ntiles - 1;
-  for (int item = tid; item < nt * G; item += kThreads) {
-    const int tok = item / G, g = item - tok * G;
-    const Moments c = {s_carry[g * 3 + 0], s_carry[g * 3 + 1], s_carry[g * 3 + 2]};
-    const Moments st = combine(c, Moments{s_lcnt[tok], s_mean[item], s_var[item]});
-    const float rstd = 1.0f / sqrtf(st.var + P.eps);
-    s_mean[item] = st.mean;
-    s_var[item] = rstd;
-    const size_t o = ((size_t)b * P.L + t0 + tok) * G + g;
-    if (P.cummean) P.cummean[o] = st.mean;
-    if (P.cumrstd) P.cumrstd[o] = rstd;
-    if (last_tile && tok == nt - 1) {
-      P.mean[(size_t)b * G + g] = st.mean;
-      P.var[(size_t)b * G + g] = st.var;
+  const int RT = kLbWords / G > 0 ? kLbWords / G : 1;   // earlier tiles per look-back round
+  for (int gbase = 0; gbase < G; gbase += 16) {
+    const int g = gbase + row16;
+    const bool active = g < G;
+    const int gc = active ? g : G - 1;
+    Moments pref[4];
+    Moments st = {0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int tok = l16 * TPL + u;
+      if (u < TPL && tok < nt) {
+        const float gm = s_mean[tok * G + gc];
+        const float gv = s_var[tok * G + gc];
+        if (P.group_mean && active) P.group_mean[((size_t)b * P.L + t0 + tok) * G + g] = gm;
+        if (!s_mask[tok]) st = merge(st, Moments{1.f, gm, gv});
+      }
+      pref[u] = st;
+    }
+    const Moments inc = row_scan(st);
+    const Moments exc = dpp_m<0x111>(inc);          // exclusive: what the lanes before this one hold
+    if (l16 == 15 && active) {
+      __hip_atomic_store(&P.agg[(trow + tile) * G + g], pack_agg(inc.mean, inc.var), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      if (g == 0) publish_u32(&P.tcnt[trow + tile], (uint32_t)inc.n + 1u);
+    }
+    // earlier tiles, RT per round
+    Moments acc = {0.f, 0.f, 0.f};
+    uint32_t prevcnt = 0;
+    for (int p0 = 0; p0 < tile; p0 += RT) {
+      const int np = min(RT, tile - p0);
+      __syncthreads();                              // the staging buffers are free again
+      for (int i = tid; i < np * G; i += kThreads) {
+        const unsigned long long* src = &P.agg[(trow + p0) * G + i];
+        unsigned long long w = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t spins = 0;
+        while ((w >> 63) == 0ull) {
+          __builtin_amdgcn_s_sleep(1);
+          w = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (++spins > kSpinLimit) {
+            publish_u32(&P.hdr->error, 1u);
+            break;
+          }
+        }
+        s_lbw[i] = w;
+      }
+      for (int i = tid; i < np; i += kThreads) {
+        const uint32_t* src = &P.tcnt[trow + p0 + i];
+        uint32_t c = fetch_u32(src);
+        uint32_t spins = 0;
+        while (c == 0u) {
+          __builtin_amdgcn_s_sleep(1);
+          c = fetch_u32(src);
+          if (++spins > kSpinLimit) {
+            publish_u32(&P.hdr->error, 1u);
+            c = 1u;
+            break;
+          }
+        }
+        s_lbc[i] = c - 1u;
+      }
+      __syncthreads();
+      for (int i = l16; i < np; i += 16) {
+        const unsigned long long w = s_lbw[i * G + gc];
+        Moments a;
+        a.n = (float)s_lbc[i];
+        a.mean = __uint_as_float((uint32_t)w);
+        a.var = __uint_as_float((uint32_t)(w >> 32) & 0x7fffffffu);
+        acc = merge(acc, a);
+        prevcnt += s_lbc[i];
+      }
+    }
+    acc = row_reduce(acc);
+    const uint32_t prevtot = row_sum_u32(prevcnt);    // the lanes hold disjoint sets of earlier tiles
+    const Moments prior = {(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gc], P.prev_var[(size_t)b * G + gc]};
+    const Moments carry = merge(prior, acc);
+    const Moments base = merge(carry, exc);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int tok = l16 * TPL + u;
+      if (u < TPL && tok < nt && active) {
+        const Moments full = merge(base, pref[u]);
+        const float rstd = __builtin_amdgcn_rsqf(full.var + P.eps);
+        s_mean[tok * G + g] = full.mean;
+        s_var[tok * G + g] = rstd;
+        const size_t o = ((size_t)b * P.L + t0 + tok) * G + g;
+        if (P.cummean) P.cummean[o] = full.mean;
+        if (P.cumrstd) P.cumrstd[o] = rstd;
+      }
+    }
+    if (last_tile && l16 == 15 && active) {
+      const Moments fin = merge(carry, inc);
+      P.mean[(size_t)b * G + g] = fin.mean;
+      P.var[(size_t)b * G + g] = fin.var;
+      if (g == 0) P.count[b] = P.prev_count[b] + (int64_t)prevtot + (int64_t)inc.n;
     }
   }
-  if (last_tile && tid == 0)
-    P.count[b] = P.prev_count[b] + (int64_t)s_prevcnt + (int64_t)s_lcnt[nt - 1];
   __syncthreads();
 
-  // ---- phase 6: normalise and store
+  // ---- normalise and store
   float gam[VEC], bet[VEC];
   if (HOIST) {
     const int f0 = (tid % TPT) * VEC;
@@ -264,10 +420,12 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
         }
       }
       V out;
+      const float rr = masked ? 0.f : r;
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        const float val = (to_float(xv[j].v[i]) - m) * r * gam[i] + bet[i];
-        out.v[i] = from_float<T>(masked ? 0.f : val);
+        const float a = rr * gam[i];
+        const float c = masked ? 0.f : bet[i] - m * a;
+        out.v[i] = from_float<T>(to_float(xv[j].v[i]) * a + c);
       }
       yout[v] = out;
     }
@@ -282,7 +440,10 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   }
   __syncthreads();
   if (s_last) {
-    for (int i = tid; i < P.B * P.ntiles; i += kThreads) publish_u32(&P.flags[i], 0u);
+    const int n = P.B * P.ntiles;
+    for (int i = tid; i < n; i += kThreads) publish_u32(&P.tcnt[i], 0u);
+    for (int i = tid; i < n * G; i += kThreads)
+      __hip_atomic_store(&P.agg[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) {
       publish_u32(&P.hdr->ticket, 0u);
       publish_u32(&P.hdr->done, 0u);
@@ -332,7 +493,7 @@ __global__ __launch_bounds__(kThreads) void feature_tsn_kernel(
 }
 
 struct TsnGeom {
-  int vec, tpt, lpg, tt, ntiles;
+  int vec, tpt, lpg, tt, ntiles, lpgt;
   size_t smem;
 };
 
@@ -342,9 +503,9 @@ bool tsn_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, TsnGeom
   int vec = 16 / esize;
   while (vec > 1 && dg % vec != 0) vec /= 2;
   const int64_t tpt = H / vec;
-  if (tpt > kPartCap) return false;
+  if (tpt > kPartCap || G > kLbWords) return false;
   int tt = (int)(kPartCap / tpt);
-  if (tt > 64) tt = 64;
+  if (tt > kMaxTT) tt = kMaxTT;
   while (tt > 8 && B * ceil_div(L, tt) < 512) tt /= 2;
   if (tt > L) tt = (int)L;
   if (tt < 1) tt = 1;
@@ -353,23 +514,39 @@ bool tsn_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, TsnGeom
   g->lpg = (int)(dg / vec);
   g->tt = tt;
   g->ntiles = (int)ceil_div(L, tt);
-  const size_t floats = (size_t)kPartCap + 2 * (size_t)tt * G + 3 * (size_t)G +
-                        3 * (size_t)(G > kThreads ? G : kThreads) + (size_t)tt;
-  g->smem = floats * 4 + align_up((size_t)tt, 16);
+  const int lpg = g->lpg;
+  g->lpgt = (lpg <= 64 && (lpg & (lpg - 1)) == 0) ? lpg : 0;
+  size_t bytes = 2 * (size_t)tt * G * 4 + align_up((size_t)tt, 16) + (size_t)kLbWords * 12;
+  if (g->lpgt == 0) bytes += (size_t)kPartCap * 4;
+  g->smem = bytes;
   return g->smem <= 150 * 1024;
 }
 
-template <typename T, int VEC>
-int launch_group_tsn(const TsnParams& P, const TsnGeom& g, hipStream_t stream) {
+template <typename T, int VEC, int LPGT>
+int launch_group_tsn2(const TsnParams& P, const TsnGeom& g, hipStream_t stream) {
   const bool hoist = (kThreads % g.tpt) == 0;
   const dim3 grid((unsigned)(P.B * P.ntiles));
-  auto kern = hoist ? group_tsn_kernel<T, VEC, true> : group_tsn_kernel<T, VEC, false>;
+  auto kern = hoist ? group_tsn_kernel<T, VEC, true, LPGT> : group_tsn_kernel<T, VEC, false, LPGT>;
   if (g.smem > 64 * 1024) {
-    hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.smem);
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.smem);
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), g.smem, stream, P);
   MEGA_CHECK_LAUNCH("group_timestep_norm_fwd");
   return MEGA_OK;
+}
+
+template <typename T, int VEC>
+int launch_group_tsn(const TsnParams& P, const TsnGeom& g, hipStream_t stream) {
+  switch (g.lpgt) {
+    case 1: return launch_group_tsn2<T, VEC, 1>(P, g, stream);
+    case 2: return launch_group_tsn2<T, VEC, 2>(P, g, stream);
+    case 4: return launch_group_tsn2<T, VEC, 4>(P, g, stream);
+    case 8: return launch_group_tsn2<T, VEC, 8>(P, g, stream);
+    case 16: return launch_group_tsn2<T, VEC, 16>(P, g, stream);
+    case 32: return launch_group_tsn2<T, VEC, 32>(P, g, stream);
+    case 64: return launch_group_tsn2<T, VEC, 64>(P, g, stream);
+    default: return launch_group_tsn2<T, VEC, 0>(P, g, stream);
+  }
 }
 
 template <typename T>
@@ -384,7 +561,7 @@ int dispatch_vec(const TsnParams& P, const TsnGeom& g, hipStream_t s) {
 
 size_t tsn_workspace_bytes(int64_t B, int64_t G, int ntiles) {
   const size_t n = (size_t)B * ntiles;
-  return align_up(sizeof(TsnHeader), 256) + align_up(n * 4, 256) * 2 + align_up(n * G * 2 * 4, 256);
+  return align_up(sizeof(TsnHeader), 256) + align_up(n * 4, 256) + align_up(n * G * 8, 256);
 }
 
 }  // namespace
@@ -441,9 +618,8 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
   P.gamma = gamma; P.beta = beta; P.mask = mask; P.count = count; P.mean = mean; P.var = var;
   P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd;
   P.hdr = (TsnHeader*)w; w += align_up(sizeof(TsnHeader), 256);
-  P.flags = (uint32_t*)w; w += align_up(n * 4, 256);
   P.tcnt = (uint32_t*)w; w += align_up(n * 4, 256);
-  P.agg = (float*)w;
+  P.agg = (unsigned long long*)w;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G;
   P.TT = g.tt; P.ntiles = g.ntiles; P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
   switch (dtype) {
