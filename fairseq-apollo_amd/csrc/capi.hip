@@ -14,4 +14,4 @@ void set_error(const char* fmt, ...) {
 }  // namespace mega
 
 extern "C" const char* mega_last_error(void) { return mega::g_err; }
-extern "C" int mega_abi_version(void) { return 1; }
+extern "C" int mega_abi_version(void) { return 2; }

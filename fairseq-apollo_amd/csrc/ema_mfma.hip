@@ -10,21 +10,24 @@
 //
 // which is the reference's own incremental decomposition (kernel + carried-state bias,
 // fairseq/csrc/ops/ema_parameters.cc:37-77) applied per tile.  K, P, C are 32x32 matrices that
-// depend on the channel only, so they are generated once per wave from a q-power table in LDS
-// (kernel generation fused in) and kept in registers as MFMA A-operands; the B-operands are 16
-// columns of 32 tokens each, i.e. all three products are v_mfma_f32_16x16x32_bf16.
+// depend on the channel only.
 //
-// One wave owns one (batch, channel) row for the whole sequence; a workgroup is 16 waves = 16
-// adjacent channels, so a [B, L, D] activation tensor is streamed as 32-byte pieces per token
-// that the workgroup transposes through LDS (the four workgroups that share a 128-byte line are
-// placed on the same XCD), and a [B, D, L] tensor as contiguous rows.
+// Kernel generation (ema_image_kernel): one wave per coefficient row builds a q-power table in
+// LDS and from it the MFMA A-operand images of K, P, C (bf16, optionally with a second bf16
+// correction term) plus the per-state multipliers q^32 and q^(32 SEGT).  The image is what the
+// reference caches as `_coeffs` / recomputes as the D x L kernel; here it is 9-13 KB per channel
+// whatever L is.
 //
-// A super-chunk of 16 segments x SEGT tiles is resident in LDS.  The 16 MFMA columns are the 16
-// segments, so the tile-to-tile recurrence of the state stays inside a lane:
+// Streaming (ema_mfma_kernel): one wave owns one (batch, channel) row for the whole sequence and
+// keeps the image in registers; a workgroup is 16 waves = 16 adjacent channels, so a [B, L, D]
+// tensor is streamed as 32-byte pieces per token that the workgroup transposes through LDS (the
+// four workgroups that share a 128-byte line are placed on the same XCD), and a [B, D, L] tensor
+// as contiguous rows.  A super-chunk of 16 segments x SEGT tiles is resident in LDS.  The 16
+// MFMA columns are the 16 segments, so the tile-to-tile recurrence stays inside a lane:
 //   sweep 1: segment end states from a zero start            (P products only)
-//   scan   : 16-step serial scan over the segments per state (through LDS, lanes 0..15)
+//   scan   : 16-step serial scan over the segments per state (lanes 0..15, values in registers)
 //   sweep 2: K, P, C products with the true start states; y overwrites x in LDS
-#include "common.h"
+#include "ema_mfma.h"
 
 namespace mega {
 namespace {
@@ -35,14 +38,188 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int kWaves = 16;               // channels per workgroup
 constexpr int kThreadsM = kWaves * 64;
 constexpr int kNS = 16;                  // complex states per channel (zero padded)
+#ifndef MEGA_SEGT
+#define MEGA_SEGT 2
+#endif
+constexpr int kSEGT = MEGA_SEGT;         // tiles per segment: super-chunk = 16 * kSEGT * 32 tokens
+#ifndef MEGA_NWK
+#define MEGA_NWK 2
+#endif
+#ifndef MEGA_NWP
+#define MEGA_NWP 2
+#endif
+#ifndef MEGA_NWC
+#define MEGA_NWC 1
+#endif
+constexpr int kNWK = MEGA_NWK;           // bf16 terms of the Toeplitz operand K
+constexpr int kNWP = MEGA_NWP;           // bf16 terms of the state-input operand P
+constexpr int kNWC = MEGA_NWC;           // bf16 terms of the state-output operand C
+constexpr int kNOPS = 2 * (kNWK + kNWP + kNWC);
+constexpr int kImgSlots = kNOPS + 3;     // + q^32 of the lane's 4 states (2 slots) + scan multiplier
+constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
 
+// ------------------------------------------------------------------------------------------
+// kernel generation
+// ------------------------------------------------------------------------------------------
+struct ImageArgs {
+  const float* p;        // [K, N]
+  const float* q;        // [K, N, 2]
+  const float* gamma;    // [K, N, 2]
+  const float* omega;    // [D] or null
+  uint4* image;          // [K][kImgSlots][64]
+  int K, D, N;
+  int is_complex;
+  int lag_back;          // rows >= D exclude the current sample (backward half with shift)
+};
+
+__device__ __forceinline__ float bf_split(float v, __bf16* h) {
+  *h = (__bf16)v;
+  return v - (float)(*h);
+}
+
+constexpr int kPrepWaves = 4;
+constexpr int kPowB = 33 * kNS * 8;
+constexpr int kAuxB = 64 * 4 + kNS * 4 + kNS * 8;
+
+__global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageArgs A) {
+  __shared__ __attribute__((aligned(16))) char smem[kPrepWaves * (kPowB + kAuxB)];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int kr_raw = blockIdx.x * kPrepWaves + wave;
+  const bool ok = kr_raw < A.K;
+  const int kr = ok ? kr_raw : A.K - 1;
+  const int lag = (kr >= A.D && A.lag_back) ? 1 : 0;
+  float2* pw = (float2*)(smem + wave * kPowB);
+  float* kkt = (float*)(smem + kPrepWaves * kPowB + wave * kAuxB);   // [64]: k[idx] at kkt[32 + idx]
+  float* pbuf = kkt + 64;
+  float2* gbuf = (float2*)(pbuf + kNS);
+  const int r = lane >> 4;
+  {
+    const int n = lane & 15, blk = lane >> 4;
+    float qr = 0.f, qi = 0.f, pv = 0.f, gr = 0.f, gi = 0.f;
+    if (n < A.N) {
+      const size_t o = ((size_t)kr * A.N + n);
+      qr = A.q[o * 2];
+      qi = A.is_complex ? A.q[o * 2 + 1] : 0.f;
+      pv = A.p[o];
+      gr = A.gamma[o * 2];
+      gi = A.is_complex ? A.gamma[o * 2 + 1] : 0.f;
+    }
+    cfloat q1 = {qr, qi};
+    cfloat q2 = cmul(q1, q1), q4 = cmul(q2, q2), q8 = cmul(q4, q4), q16 = cmul(q8, q8), q24 = cmul(q16, q8);
+    cfloat base = blk == 0 ? cfloat{1.f, 0.f} : blk == 1 ? q8 : blk == 2 ? q16 : q24;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      pw[(8 * blk + t) * kNS + n] = make_float2(base.re, base.im);
+      base = cmul(base, q1);
+    }
+    if (blk == 3) pw[32 * kNS + n] = make_float2(base.re, base.im);
+    if (blk == 0) {
+      pbuf[n] = pv;
+      gbuf[n] = make_float2(gr, gi);
+    }
+  }
+  __syncthreads();
+  {
+    // k[e] = Re sum_n p gamma q^e; lag 1 shifts it by one tap; omega joins tap 0 of the forward rows
+    const int e = lane & 31;
+    float s = 0.f;
+#pragma unroll
+    for (int n = 0; n < kNS; ++n) {
+      const float2 w = pw[e * kNS + n];
+      const float2 g = gbuf[n];
+      s += pbuf[n] * (g.x * w.x - g.y * w.y);
+    }
+    const int idx = e + lag;
+    if (lane < 32) {
+      if (idx < 32) kkt[32 + idx] = s;
+      kkt[lane] = 0.f;
+    }
+  }
+  __syncthreads();
+  if (lane == 0) {
+    if (lag) kkt[32] = 0.f;
+    if (A.omega && kr < A.D) kkt[32] += A.omega[kr];
+  }
+  __syncthreads();
+  uint4* img = A.image + (size_t)kr * kImgSlots * 64;
+  const int m = lane & 15, g = lane >> 4;
+  int slot = 0;
+  bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int row = 16 * mb + m;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int k = 8 * g + t;
+      // K: rows = output time, k = input time (Toeplitz)
+      const float kv = kkt[32 + row - k];
+      // P: rows = (state, part), k = input time i: p q^{31-i}
+      float pv;
+      {
+        const int n = row >> 1, part = row & 1;
+        const float2 w = pw[(31 - k) * kNS + n];
+        pv = pbuf[n] * (part ? w.y : w.x);
+      }
+      // C: rows = output time i; k-slot t of block g <-> state 2g + t/2 (t < 4) or 8 + 2g + (t-4)/2,
+      // part t & 1: Re(gamma q^{i+1-lag}) multiplies Re h, -Im(...) multiplies Im h
+      float cv;
+      {
+        const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
+        const int part = t & 1;
+        const float2 w = pw[(row + 1 - lag) * kNS + n];
+        const float2 gm = gbuf[n];
+        const float re = gm.x * w.x - gm.y * w.y;
+        const float im = gm.x * w.y + gm.y * w.x;
+        cv = part ? -im : re;
+      }
+      __bf16 h;
+      float rem = bf_split(kv, &h);
+      Kw[0][mb][t] = h;
+      if (kNWK > 1) Kw[kNWK - 1][mb][t] = (__bf16)rem;
+      rem = bf_split(pv, &h);
+      Pw[0][mb][t] = h;
+      if (kNWP > 1) Pw[kNWP - 1][mb][t] = (__bf16)rem;
+      rem = bf_split(cv, &h);
+      Cw[0][mb][t] = h;
+      if (kNWC > 1) Cw[kNWC - 1][mb][t] = (__bf16)rem;
+    }
+  }
+  if (ok) {
+#pragma unroll
+    for (int w = 0; w < kNWK; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
+#pragma unroll
+    for (int w = 0; w < kNWP; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
+#pragma unroll
+    for (int w = 0; w < kNWC; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
+    // q^32 of this lane's four states (2r, 2r+1, 8+2r, 9+2r)
+    const float2 a = pw[32 * kNS + 2 * r], bq = pw[32 * kNS + 2 * r + 1];
+    const float2 c = pw[32 * kNS + 8 + 2 * r], d = pw[32 * kNS + 9 + 2 * r];
+    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(a.x), __float_as_uint(a.y), __float_as_uint(bq.x),
+                                           __float_as_uint(bq.y));
+    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(c.x), __float_as_uint(c.y), __float_as_uint(d.x),
+                                           __float_as_uint(d.y));
+    // scan multiplier q^(32 SEGT) of state `lane & 15`
+    cfloat R = {1.f, 0.f};
+    const float2 w = pw[32 * kNS + (lane & 15)];
+    for (int t = 0; t < kSEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
+    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// streaming
+// ------------------------------------------------------------------------------------------
 struct MfmaArgs {
   const void* x;
   void* y;
   int64_t sxb, sxd, sxl, syb, syd, syl;
-  const float* p;        // [K, N]
-  const float* q;        // [K, N, 2]
-  const float* gamma;    // [K, N, 2]
+  const uint4* image;    // [K][kImgSlots][64]
   const float* omega;    // [D] or null (null: no residual in this pass)
   const uint8_t* mask;   // [B, L] or null
   const float* h_in;     // [B, D, N, 2] or null
@@ -53,35 +230,30 @@ struct MfmaArgs {
   int B, D, N, L;
   int koff;              // first coefficient row of this direction
   int reverse;           // logical time runs backwards
-  int lag;               // 1: the output at t excludes x[t] (backward half with shift)
   int is_complex;
   int xcd_map;           // 1: sibling channel blocks share an XCD
 };
 
-__device__ __forceinline__ float bf_hi(float v, __bf16* h) {
-  *h = (__bf16)v;
-  return v - (float)(*h);
-}
-
-template <int SEGT>
 struct Geo {
-  static constexpr int SEG = SEGT * 32;            // tokens per segment
+  static constexpr int SEG = kSEGT * 32;           // tokens per segment
   static constexpr int SC = SEG * 16;              // tokens per super-chunk
   static constexpr int SEGB = SEG * 2 + 16;        // bytes per segment in an LDS row (padded)
-  static constexpr int ROWB = SEGB * 16;           // bytes per channel row
+  static constexpr int ROWB = SEGB * 16 + 16;      // bytes per channel row; (ROWB / 4) % 16 == 4
   static constexpr int XBUF = ROWB * kWaves;
-  static constexpr int POWB = 33 * kNS * 8;        // q-power table per channel (setup only, aliases xbuf)
   static constexpr int SCANB = 16 * kNS * 8;       // segment states per channel
-  static constexpr int AUXB = 64 * 4 + kNS * 4 + kNS * 8;   // k table (64), p (16), gamma (16 x 2)
-  static constexpr int TOTAL = XBUF + kWaves * (SCANB + AUXB);
-  static_assert(POWB * kWaves <= XBUF, "power table must fit in the staging buffer");
+  static constexpr int TOTAL = XBUF + kWaves * SCANB;
+  static_assert((ROWB / 4) % 16 == 4, "row stride must spread the four rows of a store over the banks");
   __device__ static __forceinline__ int pos(int t) { return (t / SEG) * SEGB + (t % SEG) * 2; }
 };
 
+__device__ __forceinline__ uint32_t dpp_swap2(uint32_t v) {      // lane ^ 2 within a quad
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true);
+}
+
 // LAYOUT 0: [B, D, L] rows contiguous in time; LAYOUT 1: [B, L, D] channels contiguous.
-template <int SEGT, int NW, int LAYOUT>
+template <int LAYOUT>
 __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
-  using G = Geo<SEGT>;
+  using G = Geo;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -91,7 +263,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   const int ncb = (A.D + kWaves - 1) / kWaves;
   int b, cb;
   {
-    int g = blockIdx.x;
+    const int g = blockIdx.x;
     if (A.xcd_map) {
       const int xcd = g & 7, slot = g >> 3;
       const int s = slot & 3, gi = (slot >> 2) * 8 + xcd;
@@ -105,147 +277,18 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   }
   const int ch = cb * kWaves + wave;
   const bool ch_ok = ch < A.D;
-  const int chc = ch_ok ? ch : A.D - 1;            // clamp: idle waves compute on a valid row, never store
-  const int kr = A.koff + chc;
-
+  const int chc = ch_ok ? ch : A.D - 1;            // idle waves compute on a valid row, never store
   char* xrow = smem + wave * G::ROWB;
-  char* powt = smem + wave * G::POWB;              // aliases the staging buffer during setup
   char* scan = smem + G::XBUF + wave * G::SCANB;
-  char* aux = smem + G::XBUF + kWaves * G::SCANB + wave * G::AUXB;
-  float* kkt = (float*)aux;                        // [64]: k[idx] at kkt[32 + idx], zeros below
-  float* pbuf = kkt + 64;                          // [16]
-  float2* gbuf = (float2*)(pbuf + kNS);            // [16]
 
-  // ================= setup: q powers -> LDS, then K / P / C operands in registers
-  {
-    const int n = lane & 15, blk = lane >> 4;
-    float qr = 0.f, qi = 0.f, pv = 0.f, gr = 0.f, gi = 0.f;
-    if (n < A.N) {
-      const size_t o = ((size_t)kr * A.N + n);
-      qr = A.q[o * 2];
-      qi = A.is_complex ? A.q[o * 2 + 1] : 0.f;
-      pv = A.p[o];
-      gr = A.gamma[o * 2];
-      gi = A.is_complex ? A.gamma[o * 2 + 1] : 0.f;
-    }
-    // q^2, q^4, q^8, q^16, q^24
-    cfloat q1 = {qr, qi};
-    cfloat q2 = cmul(q1, q1), q4 = cmul(q2, q2), q8 = cmul(q4, q4), q16 = cmul(q8, q8), q24 = cmul(q16, q8);
-    cfloat base = blk == 0 ? cfloat{1.f, 0.f} : blk == 1 ? q8 : blk == 2 ? q16 : q24;
-    float2* pw = (float2*)powt;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      pw[(8 * blk + t) * kNS + n] = make_float2(base.re, base.im);
-      base = cmul(base, q1);
-    }
-    if (blk == 3) pw[32 * kNS + n] = make_float2(base.re, base.im);
-    if (blk == 0) {
-      pbuf[n] = pv;
-      gbuf[n] = make_float2(gr, gi);
-    }
-  }
-  __syncthreads();
-  bf16x8 Kw[NW][2], Pw[NW][2], Cw[NW][2];
-  float Qr[4], Qi[4];       // q^32 of this lane's four states
-  float Rr = 0.f, Ri = 0.f; // q^(32*SEGT) of state `lane` (lanes 0..15, segment scan)
-  float Hcr = 0.f, Hci = 0.f;
-  {
-    const float2* pw = (const float2*)powt;
-    // k table: lane e (< 32) sums over the states
-    {
-      const int e = lane & 31;
-      float s = 0.f;
-#pragma unroll
-      for (int n = 0; n < kNS; ++n) {
-        const float2 w = pw[e * kNS + n];
-        const float2 g = gbuf[n];
-        const float pn = pbuf[n];
-        s += pn * (g.x * w.x - g.y * w.y);
-      }
-      // lag 1 shifts the kernel by one tap; omega joins tap 0 of the pass that carries the residual
-      const int idx = e + A.lag;
-      if (lane < 32) {
-        if (idx < 32) kkt[32 + idx] = s;
-        kkt[lane] = 0.f;
-      }
-    }
-    __syncthreads();
-    if (lane == 0) {
-      if (A.lag) kkt[32] = 0.f;
-      if (A.omega) kkt[32] += A.omega[chc];
-    }
-    __syncthreads();
-    const int m = lane & 15, g = lane >> 4;
-    int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float2 w = pw[32 * kNS + nn[u]];
-      Qr[u] = w.x;
-      Qi[u] = w.y;
-    }
-    if (lane < 16) {
-      cfloat R = {1.f, 0.f};
-      const float2 w = pw[32 * kNS + lane];
-      for (int t = 0; t < SEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
-      Rr = R.re;
-      Ri = R.im;
-      if (A.h_in && lane < A.N && ch_ok) {
-        const size_t o = (((size_t)b * A.D + ch) * A.N + lane) * 2;
-        Hcr = A.h_in[o];
-        Hci = A.is_complex ? A.h_in[o + 1] : 0.f;
-      }
-    }
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      float kv[8], pvv[8], cv[8];
-      const int row = 16 * mb + m;
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const int k = 8 * g + t;
-        // K: Toeplitz, rows = output time, k = input time
-        kv[t] = kkt[32 + row - k];
-        // P: rows = (state, part), k = input time i: p q^{31-i}
-        {
-          const int n = row >> 1, part = row & 1;
-          const float2 w = pw[(31 - k) * kNS + n];
-          pvv[t] = pbuf[n] * (part ? w.y : w.x);
-        }
-        // C: rows = output time i, k-slot t of block g <-> state nn[t/2 (+2)] part t&1;
-        // gamma q^{i+1-lag}: real part multiplies Re h, minus imaginary part multiplies Im h
-        {
-          const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
-          const int part = t & 1;
-          const int e = row + 1 - A.lag;
-          const float2 w = pw[e * kNS + n];
-          const float2 gm = gbuf[n];
-          const float re = gm.x * w.x - gm.y * w.y;
-          const float im = gm.x * w.y + gm.y * w.x;
-          cv[t] = part ? -im : re;
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        __bf16 h;
-        float rem = bf_hi(kv[t], &h);
-        Kw[0][mb][t] = h;
-        if (NW > 1) Kw[NW - 1][mb][t] = (__bf16)rem;
-        rem = bf_hi(pvv[t], &h);
-        Pw[0][mb][t] = h;
-        if (NW > 1) Pw[NW - 1][mb][t] = (__bf16)rem;
-        rem = bf_hi(cv[t], &h);
-        Cw[0][mb][t] = h;
-        if (NW > 1) Cw[NW - 1][mb][t] = (__bf16)rem;
-      }
-    }
-  }
-  __syncthreads();      // the power table (aliasing the staging buffer) is dead from here on
-
-  // ================= streaming over super-chunks
   const int nsc = (A.L + G::SC - 1) / G::SC;
   const int last_tile = A.L / 32 - 1;             // global index of the last whole tile
-  constexpr int NLD = G::SC * 2 * kWaves / (kThreadsM * 16);   // 16-byte loads per thread per super-chunk
+  constexpr int NLD = G::SC * 2 * kWaves / (kThreadsM * 16);   // 16-byte pieces per thread per super-chunk
   uint4 pre[NLD];
   const bf16_t* xg = (const bf16_t*)A.x;
+  // LAYOUT 1: a lane pair (lane, lane ^ 2) covers tokens (2m, 2m+1) x 8 channels (half = lane & 1)
+  const int half = tid & 1;
+  const int odd = (tid >> 1) & 1;
 
   auto issue_loads = [&](int sc) {
     const int t0 = sc * G::SC;
@@ -253,9 +296,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     for (int k = 0; k < NLD; ++k) {
       pre[k] = make_uint4(0, 0, 0, 0);
       if (LAYOUT == 1) {
-        // thread -> (token, half of the 16 channels)
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
-        const int half = tid & 1;
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
         if (tau < A.L && c0 < A.D) {
@@ -264,14 +305,12 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
             pre[k] = *(const uint4*)(xg + b * A.sxb + (int64_t)t * A.sxl + c0);
         }
       } else {
-        // wave -> its own row; lane -> 8 consecutive tokens
         const int tk = k * 512 + lane * 8;
         const int tau = t0 + tk;
         if (tau < A.L) {
           const int t = A.reverse ? A.L - 8 - tau : tau;
           uint4 v = *(const uint4*)(xg + b * A.sxb + (int64_t)chc * A.sxd + t);
           if (A.reverse) {
-            // reverse the 8 elements
             uint4 w;
             w.x = (v.w >> 16) | (v.w << 16);
             w.y = (v.z >> 16) | (v.z << 16);
@@ -281,7 +320,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
           }
           if (A.mask) {
             const uint2 mk = *(const uint2*)(A.mask + (size_t)b * A.L + t);
-            uint32_t mm[2] = {mk.x, mk.y};
+            const uint32_t mm[2] = {mk.x, mk.y};
             uint32_t* vv = (uint32_t*)&v;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -297,21 +336,64 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   };
 
   issue_loads(0);
+
+  // ---- operand images of this channel: registers for the whole kernel
+  bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
+  float Qr[4], Qi[4];
+  float Rr, Ri;
+  float Hcr = 0.f, Hci = 0.f;          // carried state of state `lane` (lanes 0..15)
+  {
+    const uint4* img = A.image + (size_t)(A.koff + chc) * kImgSlots * 64 + lane;
+    int slot = 0;
+#pragma unroll
+    for (int w = 0; w < kNWK; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) Kw[w][mb] = __builtin_bit_cast(bf16x8, img[(slot++) * 64]);
+#pragma unroll
+    for (int w = 0; w < kNWP; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) Pw[w][mb] = __builtin_bit_cast(bf16x8, img[(slot++) * 64]);
+#pragma unroll
+    for (int w = 0; w < kNWC; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img[(slot++) * 64]);
+    const uint4 qa = img[(slot++) * 64], qb = img[(slot++) * 64], rr = img[(slot++) * 64];
+    Qr[0] = __uint_as_float(qa.x); Qi[0] = __uint_as_float(qa.y);
+    Qr[1] = __uint_as_float(qa.z); Qi[1] = __uint_as_float(qa.w);
+    Qr[2] = __uint_as_float(qb.x); Qi[2] = __uint_as_float(qb.y);
+    Qr[3] = __uint_as_float(qb.z); Qi[3] = __uint_as_float(qb.w);
+    Rr = __uint_as_float(rr.x);
+    Ri = __uint_as_float(rr.y);
+    if (A.h_in && lane < A.N && ch_ok) {
+      const size_t o = (((size_t)b * A.D + ch) * A.N + lane) * 2;
+      Hcr = A.h_in[o];
+      Hci = A.is_complex ? A.h_in[o + 1] : 0.f;
+    }
+  }
+
   for (int sc = 0; sc < nsc; ++sc) {
     const int t0 = sc * G::SC;
     // ---- stage the prefetched super-chunk into LDS
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
       if (LAYOUT == 1) {
+        // pair exchange: the even-token lane ends up with channels 0..3 of both tokens, the
+        // odd-token lane with channels 4..7, each as dwords (even token | odd token << 16)
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
-        const int half = tid & 1;
-        const uint32_t* vv = (const uint32_t*)&pre[k];
-        char* base = smem + (half * 8) * G::ROWB + G::pos(tk);
+        const uint4 v = pre[k];
+        const uint32_t s0 = odd ? v.x : v.z, s1 = odd ? v.y : v.w;
+        const uint32_t r0 = dpp_swap2(s0), r1 = dpp_swap2(s1);
+        const uint32_t m0 = odd ? v.z : v.x, m1 = odd ? v.w : v.y;
+        const uint32_t e0 = odd ? r0 : m0, e1 = odd ? r1 : m1;      // even token's pair of channels
+        const uint32_t o0 = odd ? m0 : r0, o1 = odd ? m1 : r1;      // odd token's
+        uint32_t w[4];
+        w[0] = (e0 & 0xffffu) | (o0 << 16);
+        w[1] = (e0 >> 16) | (o0 & 0xffff0000u);
+        w[2] = (e1 & 0xffffu) | (o1 << 16);
+        w[3] = (e1 >> 16) | (o1 & 0xffff0000u);
+        char* base = smem + (half * 8 + odd * 4) * G::ROWB + G::pos(tk & ~1);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const uint16_t el = (uint16_t)(vv[e >> 1] >> ((e & 1) * 16));
-          *(uint16_t*)(base + e * G::ROWB) = el;
-        }
+        for (int e = 0; e < 4; ++e) *(uint32_t*)(base + e * G::ROWB) = w[e];
       } else {
         const int tk = k * 512 + lane * 8;
         *(uint4*)(xrow + G::pos(tk)) = pre[k];
@@ -324,11 +406,11 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     float Er[4] = {0.f, 0.f, 0.f, 0.f}, Ei[4] = {0.f, 0.f, 0.f, 0.f};
     const char* xcol = xrow + j * G::SEGB + r * 16;
 #pragma unroll
-    for (int i = 0; i < SEGT; ++i) {
+    for (int i = 0; i < kSEGT; ++i) {
       const bf16x8 X = *(const bf16x8*)(xcol + i * 64);
       f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
+      for (int w = 0; w < kNWP; ++w) {
         S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][0], X, S0, 0, 0, 0);
         S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][1], X, S1, 0, 0, 0);
       }
@@ -344,23 +426,27 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
     // ---- scan over the 16 segments (per state), carried across super-chunks
     {
-      float4* sb = (float4*)scan;     // [16 segments][8 float4]: states (2r, 2r+1) at [j][r], (8+2r, 9+2r) at [j][4+r]
+      float4* sb = (float4*)scan;     // [16 segments][16 states] complex: states (2r, 2r+1) at float4 [j*8 + r]
       sb[j * 8 + r] = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
       sb[j * 8 + 4 + r] = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_wave_barrier();
       if (lane < 16) {
-        float2* s2 = (float2*)scan;   // [16][16] complex, state n of segment jj at s2[jj*16 + slot(n)]
-        const int slot = lane < 8 ? lane : lane;      // states are stored in order 0..15
+        float2* s2 = (float2*)scan;   // state `lane` of segment jj at s2[jj * 16 + lane]
         float hr = Hcr, hi = Hci;
 #pragma unroll
-        for (int jj = 0; jj < 16; ++jj) {
-          const float2 e = s2[jj * 16 + slot];
-          s2[jj * 16 + slot] = make_float2(hr, hi);
-          const float nr = Rr * hr - Ri * hi + e.x;
-          const float ni = Rr * hi + Ri * hr + e.y;
-          hr = nr;
-          hi = ni;
+        for (int half8 = 0; half8 < 2; ++half8) {
+          float2 e[8];
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) e[jj] = s2[(half8 * 8 + jj) * 16 + lane];
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            s2[(half8 * 8 + jj) * 16 + lane] = make_float2(hr, hi);
+            const float nr = Rr * hr - Ri * hi + e[jj].x;
+            const float ni = Rr * hi + Ri * hr + e[jj].y;
+            hr = nr;
+            hi = ni;
+          }
         }
         Hcr = hr;
         Hci = hi;
@@ -378,33 +464,30 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     // ---- sweep 2: outputs
     char* ycol = xrow + j * G::SEGB;
 #pragma unroll
-    for (int i = 0; i < SEGT; ++i) {
+    for (int i = 0; i < kSEGT; ++i) {
       const bf16x8 X = *(const bf16x8*)(xcol + i * 64);
       f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
       f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
-      bf16x8 Hop[NW];
+      bf16x8 Hop;
       {
         const float hv[8] = {Hr[0], Hi[0], Hr[1], Hi[1], Hr[2], Hi[2], Hr[3], Hi[3]};
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          __bf16 h;
-          const float rem = bf_hi(hv[t], &h);
-          Hop[0][t] = h;
-          if (NW > 1) Hop[NW - 1][t] = (__bf16)rem;
-        }
+        for (int t = 0; t < 8; ++t) Hop[t] = (__bf16)hv[t];
       }
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
+      for (int w = 0; w < kNWP; ++w) {
         S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][0], X, S0, 0, 0, 0);
         S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Pw[w][1], X, S1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int w = 0; w < kNWC; ++w) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop, Y1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int w = 0; w < kNWK; ++w) {
         Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][0], X, Y0, 0, 0, 0);
         Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][1], X, Y1, 0, 0, 0);
-        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop[0], Y0, 0, 0, 0);
-        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop[0], Y1, 0, 0, 0);
-      }
-      if (NW > 1) {
-        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[0][0], Hop[NW - 1], Y0, 0, 0, 0);
-        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[0][1], Hop[NW - 1], Y1, 0, 0, 0);
       }
       const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
       const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
@@ -446,29 +529,34 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     for (int k = 0; k < NLD; ++k) {
       if (LAYOUT == 1) {
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
-        const int half = tid & 1;
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
+        // four dwords (even token | odd token << 16) of channels half*8 + odd*4 + {0..3}
+        const char* base = smem + (half * 8 + odd * 4) * G::ROWB + G::pos(tk & ~1);
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = *(const uint32_t*)(base + e * G::ROWB);
+        // what the partner needs of mine: its token's halves of my four channels, as two dwords
+        const uint32_t give0 = odd ? ((w[0] & 0xffffu) | (w[1] << 16)) : ((w[0] >> 16) | (w[1] & 0xffff0000u));
+        const uint32_t give1 = odd ? ((w[2] & 0xffffu) | (w[3] << 16)) : ((w[2] >> 16) | (w[3] & 0xffff0000u));
+        const uint32_t keep0 = odd ? ((w[0] >> 16) | (w[1] & 0xffff0000u)) : ((w[0] & 0xffffu) | (w[1] << 16));
+        const uint32_t keep1 = odd ? ((w[2] >> 16) | (w[3] & 0xffff0000u)) : ((w[2] & 0xffffu) | (w[3] << 16));
+        const uint32_t got0 = dpp_swap2(give0), got1 = dpp_swap2(give1);
+        uint4 o;     // channels c0 .. c0+7 of token tk
+        o.x = odd ? got0 : keep0;
+        o.y = odd ? got1 : keep1;
+        o.z = odd ? keep0 : got0;
+        o.w = odd ? keep1 : got1;
         if (tau < A.L && c0 < A.D) {
           const int t = A.reverse ? A.L - 1 - tau : tau;
-          const char* base = smem + (half * 8) * G::ROWB + G::pos(tk);
-          float v[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            bf16_t el;
-            el.u = *(const uint16_t*)(base + e * G::ROWB);
-            v[e] = to_float(el);
-          }
           const bool direct = !A.acc_in && !A.acc_out && !(A.mask && A.omega);
           if (direct) {
-            uint4 o;
-            uint32_t* oo = (uint32_t*)&o;
-#pragma unroll
-            for (int e = 0; e < 8; e += 2)
-              oo[e >> 1] = (uint32_t)(*(const uint16_t*)(base + e * G::ROWB)) |
-                           ((uint32_t)(*(const uint16_t*)(base + (e + 1) * G::ROWB)) << 16);
             *(uint4*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = o;
           } else {
+            float v[8];
+            const uint32_t* oo = (const uint32_t*)&o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = __uint_as_float((e & 1) ? (oo[e >> 1] & 0xffff0000u) : (oo[e >> 1] << 16));
             if (A.acc_in) {
               const float* ai = A.acc_in + b * A.sab + (int64_t)t * A.sal + c0;
 #pragma unroll
@@ -485,10 +573,10 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
 #pragma unroll
               for (int e = 0; e < 8; ++e) ao[e] = v[e];
             } else {
-              Vec<bf16_t, 8> o;
+              Vec<bf16_t, 8> ov;
 #pragma unroll
-              for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16_t>(v[e]);
-              *(Vec<bf16_t, 8>*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = o;
+              for (int e = 0; e < 8; ++e) ov.v[e] = from_float<bf16_t>(v[e]);
+              *(Vec<bf16_t, 8>*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = ov;
             }
           }
         }
@@ -563,38 +651,47 @@ __global__ void ema_state_tail_kernel(const T* __restrict__ x, int64_t sxb, int6
 
 }  // namespace
 
-// Host side: decides whether the MFMA path covers a request and launches it.
+size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional) {
+  if (N > kNS || D <= 0) return 0;
+  return (size_t)(bidirectional ? 2 * D : D) * kImgRowBytes;
+}
+
+int ema_image_build(const float* p, const float* q, const float* gamma, int is_complex, const float* omega, int64_t D,
+                    int64_t N, int bidirectional, int shift, void* image, hipStream_t s) {
+  ImageArgs A;
+  A.p = p; A.q = q; A.gamma = gamma; A.omega = omega; A.image = (uint4*)image;
+  A.K = (int)(bidirectional ? 2 * D : D); A.D = (int)D; A.N = (int)N; A.is_complex = is_complex;
+  A.lag_back = shift ? 1 : 0;
+  hipLaunchKernelGGL(ema_image_kernel, dim3((unsigned)ceil_div(A.K, kPrepWaves)), dim3(kPrepWaves * 64), 0, s, A);
+  MEGA_CHECK_LAUNCH("ema kernel generation");
+  return MEGA_OK;
+}
+
+// Host side: decides whether the matrix-core path covers a request and launches it.
 // Returns 1 if handled, 0 if the caller must use the generic path, < 0 on a launch error.
 int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb,
-                 int64_t syd, int64_t syl, const float* p, const float* q, const float* gamma, int is_complex,
+                 int64_t syd, int64_t syl, const float* p, const float* q, const void* image, int is_complex,
                  const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
-                 int64_t N, int64_t L, int bidirectional, int64_t Lk, int shift, float* acc, float* h_tile,
-                 hipStream_t s) {
-  if (dtype != MEGA_BF16 || N > kNS || Lk > 0 || L < 256) return 0;
-  int layout;
-  if (sxd == 1 && syd == 1 && D % 8 == 0 && sxl % 8 == 0 && syl % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 1;
-  else if (sxl == 1 && syl == 1 && L % 8 == 0 && sxd % 8 == 0 && syd % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 0;
-  else return 0;
-  if (((uintptr_t)x % 16) || ((uintptr_t)y % 16) || (mask && layout == 0 && ((uintptr_t)mask % 8))) return 0;
-  if (B * ceil_div(D, kWaves) >= (int64_t)1 << 31) return 0;
-  constexpr int SEGT = 4;
-  using G = Geo<SEGT>;
+                 int64_t N, int64_t L, int bidirectional, int64_t Lk, float* acc, float* h_tile, hipStream_t s) {
+  if (!ema_mfma_covers(dtype, sxb, sxd, sxl, syb, syd, syl, x, y, mask, B, D, N, L, Lk)) return 0;
+  const int layout = (sxd == 1 && syd == 1) ? 1 : 0;
+  using G = Geo;
   const int ncb = (int)ceil_div(D, kWaves);
   MfmaArgs A;
   A.x = x; A.y = y; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.syb = syb; A.syd = syd; A.syl = syl;
-  A.p = p; A.q = q; A.gamma = gamma; A.mask = mask;
+  A.image = (const uint4*)image; A.mask = mask;
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L; A.is_complex = is_complex;
-  A.xcd_map = (layout == 1 && ncb % 4 == 0 && ((B * ncb / 4) % 8) == 0) ? 1 : 0;
+  A.xcd_map = (layout == 1 && ncb % 4 == 0 && ((B * ncb) % 32) == 0) ? 1 : 0;
   // fp32 partial sums between the two directions live in [B, D, L]-shaped storage with y's layout
   A.sab = layout == 1 ? L * D : D * L;
   A.sad = layout == 1 ? 1 : L;
   A.sal = layout == 1 ? D : 1;
   const dim3 grid((unsigned)(B * ncb));
   auto launch = [&](const MfmaArgs& a) -> int {
-    auto kern = layout == 1 ? ema_mfma_kernel<SEGT, 2, 1> : ema_mfma_kernel<SEGT, 2, 0>;
+    auto kern = layout == 1 ? ema_mfma_kernel<1> : ema_mfma_kernel<0>;
     static bool attr_set[2] = {false, false};
     if (!attr_set[layout]) {
-      hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
+      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
       attr_set[layout] = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(kThreadsM), G::TOTAL, s, a);
@@ -603,12 +700,12 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
   };
   if (bidirectional) {
     MfmaArgs Bk = A;
-    Bk.koff = (int)D; Bk.reverse = 1; Bk.lag = shift ? 1 : 0;
+    Bk.koff = (int)D; Bk.reverse = 1;
     Bk.omega = nullptr; Bk.h_in = nullptr; Bk.h_tile = nullptr; Bk.acc_in = nullptr; Bk.acc_out = acc;
     int rc = launch(Bk);
     if (rc) return rc;
   }
-  A.koff = 0; A.reverse = 0; A.lag = 0; A.omega = omega; A.h_in = h_in;
+  A.koff = 0; A.reverse = 0; A.omega = omega; A.h_in = h_in;
   A.h_tile = h_out ? h_tile : nullptr;
   A.acc_in = bidirectional ? acc : nullptr; A.acc_out = nullptr;
   int rc = launch(A);
@@ -623,10 +720,17 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
   return 1;
 }
 
-size_t ema_mfma_workspace_bytes(int64_t B, int64_t D, int64_t L, int bidirectional) {
-  size_t n = align_up((size_t)B * D * kNS * 2 * 4, 256);          // h_tile
-  if (bidirectional) n += align_up((size_t)B * D * L * 4, 256);    // fp32 partial sums
-  return n;
+bool ema_mfma_covers(int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb, int64_t syd, int64_t syl,
+                     const void* x, const void* y, const uint8_t* mask, int64_t B, int64_t D, int64_t N, int64_t L,
+                     int64_t Lk) {
+  if (dtype != MEGA_BF16 || N > kNS || Lk > 0 || L < 256) return false;
+  int layout;
+  if (sxd == 1 && syd == 1 && D % 8 == 0 && sxl % 8 == 0 && syl % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 1;
+  else if (sxl == 1 && syl == 1 && L % 8 == 0 && sxd % 8 == 0 && syd % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 0;
+  else return false;
+  if (((uintptr_t)x % 16) || ((uintptr_t)y % 16) || (mask && layout == 0 && ((uintptr_t)mask % 8))) return false;
+  if (B * ceil_div(D, kWaves) >= (int64_t)1 << 31) return false;
+  return true;
 }
 
 }  // namespace mega

@@ -22,15 +22,9 @@
 // states each; rows are laid out channel-fastest so that [B,L,D] activations are read
 // coalesced.
 #include "common.h"
+#include "ema_mfma.h"
 
 namespace mega {
-
-// matrix-core path (ema_mfma.hip)
-int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb,
-                 int64_t syd, int64_t syl, const float* p, const float* q, const float* gamma, int is_complex,
-                 const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
-                 int64_t N, int64_t L, int bidirectional, int64_t Lk, int shift, float* acc, float* h_tile,
-                 hipStream_t s);
 
 namespace {
 
@@ -281,10 +275,10 @@ __global__ void coef_prep_kernel(const float* __restrict__ p, const float* __res
 
 struct Plan {
   int NP, TPR, Tc, nchunks;
-  size_t coef_bytes, st_bytes, acc_bytes, tile_bytes, total;
+  size_t coef_bytes, st_bytes, acc_bytes, tile_bytes, image_bytes, total;
 };
 
-Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_acc) {
+Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_acc, bool bidirectional = false) {
   Plan pl;
   int tpr = 1;
   while (tpr * kNPT < N) tpr <<= 1;
@@ -307,7 +301,8 @@ Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_
   pl.acc_bytes = need_acc ? align_up((size_t)B * L * D * 4, 256) : 0;
   (void)nsets;
   pl.tile_bytes = align_up((size_t)B * D * 16 * 2 * 4, 256);      // state after the last whole tile
-  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
+  pl.image_bytes = align_up(ema_image_bytes(D, N, bidirectional ? 1 : 0), 256);   // when the caller brings none
+  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes + pl.image_bytes;
   return pl;
 }
 
@@ -452,7 +447,23 @@ extern "C" size_t mega_ema_fwd_workspace_bytes(int64_t B, int64_t D, int64_t N, 
   if (B <= 0 || D <= 0 || N <= 0 || L <= 0) return 256;
   const bool trunc = truncation > 0 && truncation < L;
   const bool need_acc = bidirectional || trunc;
-  return make_plan(B, D, N, L, 4, need_acc).total;
+  return make_plan(B, D, N, L, 4, need_acc, bidirectional != 0).total;
+}
+
+extern "C" size_t mega_ema_image_bytes(int64_t D, int64_t N, int bidirectional) {
+  return ema_image_bytes(D, N, bidirectional);
+}
+
+extern "C" int mega_ema_prepare(const float* p, const float* q, const float* gamma, int is_complex,
+                                const float* omega, int64_t D, int64_t N, int bidirectional, int shift,
+                                void* image, size_t image_bytes, void* stream) {
+  MEGA_REQUIRE(D > 0 && N > 0, MEGA_ERR_ARG, "ema_prepare: bad shape D=%ld N=%ld", (long)D, (long)N);
+  const size_t need = ema_image_bytes(D, N, bidirectional);
+  MEGA_REQUIRE(need > 0, MEGA_ERR_UNSUPPORTED, "ema_prepare: ndim=%ld has no operand image (ndim <= 16 only)", (long)N);
+  MEGA_REQUIRE(p && q && gamma && omega && image, MEGA_ERR_ARG, "ema_prepare: null pointer argument");
+  MEGA_REQUIRE(image_bytes >= need && ((uintptr_t)image % 16) == 0, MEGA_ERR_WORKSPACE,
+               "ema_prepare: image of %zu bytes (16-byte aligned) needed", need);
+  return ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, image, (hipStream_t)stream);
 }
 
 extern "C" size_t mega_ema_hidden_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L) {
@@ -475,8 +486,8 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
                             int64_t syb, int64_t syd, int64_t syl, const float* p, const float* q,
                             const float* gamma, int is_complex, const float* omega, const uint8_t* mask,
                             const float* h_in, float* h_out, int64_t B, int64_t D, int64_t N, int64_t L,
-                            int bidirectional, int64_t truncation, int shift, void* workspace,
-                            size_t workspace_bytes, void* stream) {
+                            int bidirectional, int64_t truncation, int shift, const void* image,
+                            void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common("ema_fwd", dtype, B, D, N, L);
   if (rc) return rc;
   MEGA_REQUIRE(!(bidirectional && (h_in || h_out)), MEGA_ERR_ARG,
@@ -487,7 +498,7 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
   MEGA_REQUIRE(!(Lk > 0 && (h_in || h_out)), MEGA_ERR_UNSUPPORTED,
                "ema_fwd: truncation together with incremental state is not supported");
   const bool need_acc = bidirectional || Lk > 0;
-  const Plan pl = make_plan(B, D, N, L, 4, need_acc);
+  const Plan pl = make_plan(B, D, N, L, 4, need_acc, bidirectional != 0);
   MEGA_REQUIRE(workspace && workspace_bytes >= pl.total, MEGA_ERR_WORKSPACE,
                "ema_fwd: workspace of %zu bytes needed", pl.total);
   hipStream_t s = (hipStream_t)stream;
@@ -496,9 +507,19 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
   float* st = (float*)(w + pl.coef_bytes);
   float* acc = need_acc ? (float*)(w + pl.coef_bytes + pl.st_bytes) : nullptr;
   float* h_tile = (float*)(w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes);
-  rc = ema_mfma_try(x, y, dtype, sxb, sxd, sxl, syb, syd, syl, p, q, gamma, is_complex, omega, mask, h_in, h_out, B,
-                    D, N, L, bidirectional, Lk, shift, acc, h_tile, s);
-  if (rc != 0) return rc < 0 ? rc : MEGA_OK;
+  if (ema_mfma_covers(dtype, sxb, sxd, sxl, syb, syd, syl, x, y, mask, B, D, N, L, Lk)) {
+    const void* img = image;
+    if (!img) {
+      // no cached image: kernel generation runs with every call
+      void* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
+      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s);
+      if (rc) return rc;
+      img = wimg;
+    }
+    rc = ema_mfma_try(x, y, dtype, sxb, sxd, sxl, syb, syd, syl, p, q, img, is_complex, omega, mask, h_in, h_out, B,
+                      D, N, L, bidirectional, Lk, acc, h_tile, s);
+    if (rc != 0) return rc < 0 ? rc : MEGA_OK;
+  }
   const int ndir = bidirectional ? 2 : 1;
   {
     const int64_t n = (int64_t)D * pl.NP * ndir;

@@ -299,6 +299,17 @@ class PreparedEMA:
         self.bidirectional = bool(bidirectional)
         self.trunc = 0 if truncation is None or truncation < 1 else int(truncation)
         self.shift = bool(shift)
+        # kernel generation once per set of coefficients (operand images of the matrix-core path)
+        self.image = None
+        lib = _lib.load()
+        nimg = lib.mega_ema_image_bytes(self.D, self.N, 1 if self.bidirectional else 0)
+        if nimg > 0:
+            self.image = torch.empty(nimg, dtype=torch.uint8, device=self.dev)
+            with torch.cuda.device(self.dev):
+                rc = lib.mega_ema_prepare(_ptr(self.p), _ptr(self.q), _ptr(self.gamma), 1 if self.is_complex else 0,
+                                          _ptr(self.omega), self.D, self.N, 1 if self.bidirectional else 0,
+                                          1 if self.shift else 0, _ptr(self.image), nimg, _stream(self.dev))
+            _lib.check(rc, "ema_prepare")
 
     def __call__(self, x: torch.Tensor, padding_mask: Optional[torch.Tensor] = None,
                  h: Optional[torch.Tensor] = None, want_state: bool = False,
@@ -334,7 +345,7 @@ class PreparedEMA:
                                   y.stride(1), y.stride(2), _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
                                   1 if self.is_complex else 0, _ptr(self.omega), _ptr(m8), _ptr(hin), _ptr(hout),
                                   B, D, N, L, 1 if self.bidirectional else 0, self.trunc, 1 if self.shift else 0,
-                                  _ptr(ws), ws.numel(), _stream(dev))
+                                  _ptr(self.image), _ptr(ws), ws.numel(), _stream(dev))
         _lib.check(rc, "ema_fwd")
         hc = None
         if hout is not None:

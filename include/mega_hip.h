@@ -99,7 +99,9 @@ int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_t sxd, int6
  *   h_in    [B,D,N,2] carried state or NULL; h_out [B,D,N,2] or NULL
  *           (both must be NULL when bidirectional)
  *   truncation  <= 0: kernel length L; otherwise min(truncation, L)
- *   shift   bidirectional only: 1 = the backward half starts at lag 1            */
+ *   shift   bidirectional only: 1 = the backward half starts at lag 1
+ *   image   operand images from mega_ema_prepare for the same coefficients, or NULL: then
+ *           kernel generation runs inside this call (into the workspace)                 */
 size_t mega_ema_fwd_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L,
                                     int bidirectional, int64_t truncation);
 int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
@@ -107,7 +109,22 @@ int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
                  const float* gamma, int is_complex, const float* omega,
                  const uint8_t* mask, const float* h_in, float* h_out, int64_t B,
                  int64_t D, int64_t N, int64_t L, int bidirectional, int64_t truncation,
-                 int shift, void* workspace, size_t workspace_bytes, void* stream);
+                 int shift, const void* image, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/* EMA kernel generation for the matrix-core path: from the coefficients to per-channel
+ * operand images (the 32-tap Toeplitz block of k[l] = Re sum_n p gamma q^l, the state
+ * input / output blocks p q^{31-i} and gamma q^{i+1}, and q^32), 9-13 KB per coefficient
+ * row whatever L is.  Stands in for what the reference recomputes or caches per call:
+ * _compute_kernel / ema_parameters (fairseq/modules/complex_exponential_moving_average.py:
+ * 98-109, fairseq/csrc/ops/ema_parameters_kernel.cu:40-66) and the eval-mode `_coeffs`
+ * cache (fairseq/modules/base_moving_average.py:52-58).  The image is valid while p, q,
+ * gamma, omega, bidirectional and shift are unchanged; it only exists for ndim <= 16
+ * (mega_ema_image_bytes returns 0 otherwise).                                            */
+size_t mega_ema_image_bytes(int64_t D, int64_t N, int bidirectional);
+int mega_ema_prepare(const float* p, const float* q, const float* gamma, int is_complex,
+                     const float* omega, int64_t D, int64_t N, int bidirectional, int shift,
+                     void* image, size_t image_bytes, void* stream);
 
 /* One decode step of the same layer: h' = q h + p x, y = Re sum gamma h' + omega x
  * (BaseMovingLayer.one_step, fairseq/modules/base_moving_average.py:105-118, and the

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_argument_checks_need_no_gpu():
     lib = M._lib.load()
-    assert lib.mega_abi_version() == 1
+    assert lib.mega_abi_version() == 2
     # bad dtype is rejected before anything touches a device
     rc = lib.mega_swiglu_fwd(None, None, None, 7, 16, None)
     assert rc == -1 and b"dtype" in lib.mega_last_error()
@@ -36,7 +36,7 @@ def test_argument_checks_need_no_gpu():
                                           None, None, None, None, None, None, None, 0, None)
     assert rc == -1 and b"multiple" in lib.mega_last_error()
     rc = lib.mega_ema_fwd(None, None, 1, 0, 0, 0, 0, 0, 0, None, None, None, 1, None, None, None, None, 2, 8, 64, 16,
-                          0, 0, 1, None, 0, None)
+                          0, 0, 1, None, None, 0, None)
     assert rc == -2 and b"ndim" in lib.mega_last_error()
     assert lib.mega_timestep_norm_workspace_bytes(1, 4, 4096, 1024, 16) > 0
     assert lib.mega_ema_fwd_workspace_bytes(4, 1024, 16, 4096, 0, 0) > 0
