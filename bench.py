@@ -83,6 +83,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
+                    help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
+                         "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -168,6 +172,11 @@ def main():
         reps = max(20, min(args.steps, 200))
         norm_avg, norm_med = timed(NormCall(), reps)
         ema_avg, ema_med = timed(EmaCall(), reps)
+        if args.copy_calibration:
+            dst = torch.empty_like(xs[0])
+            for i in range(args.copy_calibration):
+                dst.copy_(xs[i % NBUF])
+            torch.cuda.synchronize()
     status = M.ops.timestep_norm_status()
 
     tokens = B * L

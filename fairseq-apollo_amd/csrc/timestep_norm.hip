@@ -14,9 +14,11 @@
 //   * it then waits until every earlier tile of the same batch row has published,
 //     folds prior state + earlier aggregates into its carry-in, finishes the
 //     per-token running statistics and writes the normalised block.
-//   Tiles are handed out by an atomic ticket in time-major order, so a tile only ever
-//   waits for tiles whose workgroups are already resident; the wait is bounded and
-//   sets an error word instead of spinning forever.
+//   Tiles map to workgroup ids in time-major order; workgroups are dispatched in id order, so
+//   a tile only ever waits for tiles whose workgroups were dispatched before it; the wait is
+//   bounded and sets an error word instead of spinning forever.  Published words carry the
+//   launch epoch as a tag, so nothing has to be cleared between launches and no single
+//   address is hit by one atomic per workgroup on the way in.
 #include "common.h"
 
 namespace mega {
@@ -28,13 +30,14 @@ constexpr int kNV = 16;                       // vectors kept in registers per t
 constexpr int kPartCap = kThreads * kNV;      // vectors per tile
 constexpr int kMaxTT = 64;                    // tokens per tile (16 lanes x 4 tokens in the scan)
 constexpr uint32_t kSpinLimit = 1u << 22;
-constexpr int kLbWords = 2048;                // tile aggregates staged in LDS per look-back round
+constexpr int kLbWords = 4352;                // 64-bit words staged in LDS per look-back round
 
 struct TsnHeader {
-  uint32_t ticket;
-  uint32_t done;
-  uint32_t error;
+  uint32_t epoch;        // bumped by the last workgroup of every launch
+  uint32_t done2;        // second-level retire counter
+  uint32_t error;        // set when a bounded wait gave up
   uint32_t pad;
+  uint32_t done1[32];    // first-level retire counters (workgroup id mod 32)
 };
 
 struct TsnParams {
@@ -53,8 +56,9 @@ struct TsnParams {
   float* cummean;
   float* cumrstd;
   TsnHeader* hdr;
-  uint32_t* tcnt;              // [B*ntiles] unmasked tokens of the tile + 1 (0 = not published)
-  unsigned long long* agg;     // [B*ntiles*G] (mean, var) of the tile; bit 63 set = published
+  // [B*ntiles][2G+1] 64-bit words, value in the low half, launch tag in the high half:
+  // word 0 = unmasked tokens of the tile, word 1+2g = mean, word 2+2g = variance of group g
+  unsigned long long* rec;
   int B, L, H, G;
   int TT, ntiles;
   int TPT;           // vectors per token
@@ -150,8 +154,14 @@ __device__ __forceinline__ uint32_t row_sum_u32(uint32_t v) {
   return v;
 }
 
-__device__ __forceinline__ unsigned long long pack_agg(float mean, float var) {
-  return ((unsigned long long)(__float_as_uint(var) | 0x80000000u) << 32) | __float_as_uint(mean);
+__device__ __forceinline__ unsigned long long tagged(uint32_t v, uint32_t tag) {
+  return ((unsigned long long)tag << 32) | v;
+}
+__device__ __forceinline__ void put_rec(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long get_rec(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // LPGT > 0: groups are LPGT adjacent lanes and are reduced with lane shuffles;
@@ -163,15 +173,11 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   float* s_var = s_mean + (size_t)P.TT * P.G;      // [TT*G]  group var, later running rstd
   uint8_t* s_mask = (uint8_t*)(s_var + (size_t)P.TT * P.G);   // [TT]
   unsigned long long* s_lbw = (unsigned long long*)(s_mask + ((P.TT + 15) / 16) * 16);   // [kLbWords]
-  uint32_t* s_lbc = (uint32_t*)(s_lbw + kLbWords);                                       // [kLbWords]
-  float* part = (float*)(s_lbc + kLbWords);                   // [kPartCap] (LPGT == 0 only)
-  __shared__ uint32_t s_ticket;
-  __shared__ uint32_t s_last;
+  float* part = (float*)(s_lbw + kLbWords);                   // [kPartCap] (LPGT == 0 only)
 
   const int tid = threadIdx.x;
-  if (tid == 0) s_ticket = atomicAdd(&P.hdr->ticket, 1u);
-  __syncthreads();
-  const int ticket = (int)s_ticket;
+  const int ticket = (int)blockIdx.x;
+  const uint32_t tag = P.hdr->epoch + 1u;
   const int tile = ticket / P.B;
   const int b = ticket - tile * P.B;
   const int t0 = tile * P.TT;
@@ -294,7 +300,8 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   const int TPL = (P.TT + 15) >> 4;                 // tokens per lane (<= 4)
   const size_t trow = (size_t)b * P.ntiles;
   const bool last_tile = tile == P.ntiles - 1;
-  const int RT = kLbWords / G > 0 ? kLbWords / G : 1;   // earlier tiles per look-back round
+  const int W = 2 * G + 1;                          // words per tile record
+  const int RT = kLbWords / W;                      // earlier tiles per look-back round
   for (int gbase = 0; gbase < G; gbase += 16) {
     const int g = gbase + row16;
     const bool active = g < G;
@@ -315,9 +322,10 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     const Moments inc = row_scan(st);
     const Moments exc = dpp_m<0x111>(inc);          // exclusive: what the lanes before this one hold
     if (l16 == 15 && active) {
-      __hip_atomic_store(&P.agg[(trow + tile) * G + g], pack_agg(inc.mean, inc.var), __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
-      if (g == 0) publish_u32(&P.tcnt[trow + tile], (uint32_t)inc.n + 1u);
+      unsigned long long* mine = P.rec + (trow + tile) * W;
+      put_rec(mine + 1 + 2 * g, tagged(__float_as_uint(inc.mean), tag));
+      put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(inc.var), tag));
+      if (g == 0) put_rec(mine, tagged((uint32_t)inc.n, tag));
     }
     // earlier tiles, RT per round
     Moments acc = {0.f, 0.f, 0.f};
@@ -325,13 +333,13 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     for (int p0 = 0; p0 < tile; p0 += RT) {
       const int np = min(RT, tile - p0);
       __syncthreads();                              // the staging buffers are free again
-      for (int i = tid; i < np * G; i += kThreads) {
-        const unsigned long long* src = &P.agg[(trow + p0) * G + i];
-        unsigned long long w = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int i = tid; i < np * W; i += kThreads) {
+        const unsigned long long* src = P.rec + (trow + p0) * W + i;
+        unsigned long long w = get_rec(src);
         uint32_t spins = 0;
-        while ((w >> 63) == 0ull) {
+        while ((uint32_t)(w >> 32) != tag) {
           __builtin_amdgcn_s_sleep(1);
-          w = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          w = get_rec(src);
           if (++spins > kSpinLimit) {
             publish_u32(&P.hdr->error, 1u);
             break;
@@ -339,30 +347,16 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
         }
         s_lbw[i] = w;
       }
-      for (int i = tid; i < np; i += kThreads) {
-        const uint32_t* src = &P.tcnt[trow + p0 + i];
-        uint32_t c = fetch_u32(src);
-        uint32_t spins = 0;
-        while (c == 0u) {
-          __builtin_amdgcn_s_sleep(1);
-          c = fetch_u32(src);
-          if (++spins > kSpinLimit) {
-            publish_u32(&P.hdr->error, 1u);
-            c = 1u;
-            break;
-          }
-        }
-        s_lbc[i] = c - 1u;
-      }
       __syncthreads();
       for (int i = l16; i < np; i += 16) {
-        const unsigned long long w = s_lbw[i * G + gc];
+        const unsigned long long* rw = s_lbw + i * W;
+        const uint32_t c = (uint32_t)rw[0];
         Moments a;
-        a.n = (float)s_lbc[i];
-        a.mean = __uint_as_float((uint32_t)w);
-        a.var = __uint_as_float((uint32_t)(w >> 32) & 0x7fffffffu);
+        a.n = (float)c;
+        a.mean = __uint_as_float((uint32_t)rw[1 + 2 * gc]);
+        a.var = __uint_as_float((uint32_t)rw[2 + 2 * gc]);
         acc = merge(acc, a);
-        prevcnt += s_lbc[i];
+        prevcnt += c;
       }
     }
     acc = row_reduce(acc);
@@ -431,22 +425,19 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     }
   }
 
-  // ---- retire: the last workgroup to finish leaves the workspace zero-filled
-  __syncthreads();
+  // ---- retire: the last workgroup to finish opens the next epoch (two-level count so that no
+  // single address sees one atomic per workgroup)
   if (tid == 0) {
-    const uint32_t total = (uint32_t)(P.B * P.ntiles);
-    const uint32_t prev = atomicAdd(&P.hdr->done, 1u);
-    s_last = (prev == total - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (s_last) {
-    const int n = P.B * P.ntiles;
-    for (int i = tid; i < n; i += kThreads) publish_u32(&P.tcnt[i], 0u);
-    for (int i = tid; i < n * G; i += kThreads)
-      __hip_atomic_store(&P.agg[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (tid == 0) {
-      publish_u32(&P.hdr->ticket, 0u);
-      publish_u32(&P.hdr->done, 0u);
+    const uint32_t total = gridDim.x;
+    const uint32_t k = blockIdx.x & 31u;
+    const uint32_t quota = (total - k + 31u) / 32u;
+    if (atomicAdd(&P.hdr->done1[k], 1u) == quota - 1u) {
+      publish_u32(&P.hdr->done1[k], 0u);
+      const uint32_t classes = total < 32u ? total : 32u;
+      if (atomicAdd(&P.hdr->done2, 1u) == classes - 1u) {
+        publish_u32(&P.hdr->done2, 0u);
+        publish_u32(&P.hdr->epoch, tag == 0xffffffffu ? 0u : tag);
+      }
     }
   }
 }
@@ -503,7 +494,7 @@ bool tsn_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, TsnGeom
   int vec = 16 / esize;
   while (vec > 1 && dg % vec != 0) vec /= 2;
   const int64_t tpt = H / vec;
-  if (tpt > kPartCap || G > kLbWords) return false;
+  if (tpt > kPartCap || 2 * G + 1 > kLbWords) return false;
   int tt = (int)(kPartCap / tpt);
   if (tt > kMaxTT) tt = kMaxTT;
   while (tt > 8 && B * ceil_div(L, tt) < 512) tt /= 2;
@@ -516,7 +507,7 @@ bool tsn_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, TsnGeom
   g->ntiles = (int)ceil_div(L, tt);
   const int lpg = g->lpg;
   g->lpgt = (lpg <= 64 && (lpg & (lpg - 1)) == 0) ? lpg : 0;
-  size_t bytes = 2 * (size_t)tt * G * 4 + align_up((size_t)tt, 16) + (size_t)kLbWords * 12;
+  size_t bytes = 2 * (size_t)tt * G * 4 + align_up((size_t)tt, 16) + (size_t)kLbWords * 8;
   if (g->lpgt == 0) bytes += (size_t)kPartCap * 4;
   g->smem = bytes;
   return g->smem <= 150 * 1024;
@@ -561,7 +552,7 @@ int dispatch_vec(const TsnParams& P, const TsnGeom& g, hipStream_t s) {
 
 size_t tsn_workspace_bytes(int64_t B, int64_t G, int ntiles) {
   const size_t n = (size_t)B * ntiles;
-  return align_up(sizeof(TsnHeader), 256) + align_up(n * 4, 256) + align_up(n * G * 8, 256);
+  return align_up(sizeof(TsnHeader), 256) + align_up(n * (2 * (size_t)G + 1) * 8, 256);
 }
 
 }  // namespace
@@ -611,15 +602,13 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
   MEGA_REQUIRE(workspace != nullptr && workspace_bytes >= tsn_workspace_bytes(B, G, g.ntiles),
                MEGA_ERR_WORKSPACE, "group_timestep_norm_fwd: workspace of %zu bytes needed",
                tsn_workspace_bytes(B, G, g.ntiles));
-  const size_t n = (size_t)B * g.ntiles;
   char* w = (char*)workspace;
   TsnParams P;
   P.x = x; P.y = y; P.prev_count = prev_count; P.prev_mean = prev_mean; P.prev_var = prev_var;
   P.gamma = gamma; P.beta = beta; P.mask = mask; P.count = count; P.mean = mean; P.var = var;
   P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd;
   P.hdr = (TsnHeader*)w; w += align_up(sizeof(TsnHeader), 256);
-  P.tcnt = (uint32_t*)w; w += align_up(n * 4, 256);
-  P.agg = (unsigned long long*)w;
+  P.rec = (unsigned long long*)w;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G;
   P.TT = g.tt; P.ntiles = g.ntiles; P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
   switch (dtype) {

@@ -64,7 +64,8 @@ _tsn_ws = {}
 
 
 def _tsn_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
-    """Zero-filled once; the kernels leave it zero-filled, so it is reused per (device, stream)."""
+    """Zero-filled once, then owned by the TimestepNorm calls (launch epoch + tile records); one per
+    (device, stream)."""
     key = (dev.index, _stream(dev))
     ws = _tsn_ws.get(key)
     if ws is None or ws.numel() < nbytes:

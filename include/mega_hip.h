@@ -11,9 +11,9 @@
  *  - the library never allocates device memory: scratch comes in through
  *    `workspace` (size from the matching *_workspace_bytes query).  A workspace
  *    that is handed to mega_*_timestep_norm_fwd must be zero-filled once when it
- *    is created; the kernels leave it zero-filled again, so it can be reused by
- *    later calls on the same stream.  Calls that share one workspace must not
- *    overlap in time;
+ *    is created and then belongs to these calls (they keep a launch epoch in
+ *    it), so it can be reused by later calls on the same stream.  Calls that
+ *    share one workspace must not overlap in time;
  *  - return value 0 = launched; a negative value = rejected before anything was
  *    launched (MEGA_ERR_*), with a human-readable reason in mega_last_error()
  *    (thread-local).  This mirrors the TORCH_CHECK -> RuntimeError behaviour of
