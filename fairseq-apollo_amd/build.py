@@ -20,6 +20,7 @@ SOURCES = [
     "ema_mfma.hip",
     "elementwise.hip",
     "attention.hip",
+    "attention_mfma.hip",
     "long_conv.hip",
 ]
 

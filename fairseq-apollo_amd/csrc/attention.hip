@@ -8,6 +8,14 @@
 #include "common.h"
 
 namespace mega {
+
+// matrix-core path (attention_mfma.hip)
+bool attention_mfma_covers(int dtype, const void* q, const void* k, const void* v, int64_t B, int64_t L, int64_t Nh,
+                           int64_t H1, int64_t H2);
+size_t attention_mfma_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H2);
+int attention_mfma_run(const void* q, const void* k, const void* v, void* y, void* w, int dtype, int64_t B, int64_t L,
+                       int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, void* ws, hipStream_t s);
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -131,15 +139,27 @@ extern "C" int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int
   return MEGA_OK;
 }
 
+extern "C" size_t mega_attention_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                                                 int64_t H2) {
+  if (B <= 0 || L <= 0 || Nh <= 0 || H1 <= 0 || H2 <= 0 || dtype == MEGA_F32 || H1 % 8 != 0) return 0;
+  return attention_mfma_workspace_bytes(dtype, B, L, Nh, H2);
+}
+
 extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
                                   int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
-                                  int causal, void* stream) {
+                                  int causal, void* workspace, size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "attention_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && Nh > 0 && H1 > 0 && H2 > 0, MEGA_ERR_ARG, "attention_fwd: bad shape");
   if (B == 0 || L == 0) return MEGA_OK;
   MEGA_REQUIRE(q && k && v && y, MEGA_ERR_ARG, "attention_fwd: null pointer argument");
   MEGA_REQUIRE(B * L * Nh < (int64_t)1 << 31, MEGA_ERR_UNSUPPORTED, "attention_fwd: too many rows");
+  if (attention_mfma_covers(dtype, q, k, v, B, L, Nh, H1, H2)) {
+    const size_t need = attention_mfma_workspace_bytes(dtype, B, L, Nh, H2);
+    MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 256) == 0, MEGA_ERR_WORKSPACE,
+                 "attention_fwd: workspace of %zu bytes (256-byte aligned) needed", need);
+    return attention_mfma_run(q, k, v, y, w, dtype, B, L, Nh, H1, H2, scale, causal, workspace, (hipStream_t)stream);
+  }
   const size_t smem = (size_t)(L + H1) * 4;
   MEGA_REQUIRE(smem <= 150 * 1024, MEGA_ERR_UNSUPPORTED, "attention_fwd: L=%ld too long for one chunk", (long)L);
   hipStream_t s = (hipStream_t)stream;

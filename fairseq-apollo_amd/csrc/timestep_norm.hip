@@ -333,19 +333,33 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     for (int p0 = 0; p0 < tile; p0 += RT) {
       const int np = min(RT, tile - p0);
       __syncthreads();                              // the staging buffers are free again
-      for (int i = tid; i < np * W; i += kThreads) {
-        const unsigned long long* src = P.rec + (trow + p0) * W + i;
-        unsigned long long w = get_rec(src);
-        uint32_t spins = 0;
-        while ((uint32_t)(w >> 32) != tag) {
-          __builtin_amdgcn_s_sleep(1);
-          w = get_rec(src);
-          if (++spins > kSpinLimit) {
-            publish_u32(&P.hdr->error, 1u);
-            break;
+      {
+        // all loads of a batch are issued before the first one is looked at
+        constexpr int kBatch = 8;
+        const unsigned long long* src0 = P.rec + (trow + p0) * W;
+        const int nw = np * W;
+        for (int i0 = tid; i0 < nw; i0 += kThreads * kBatch) {
+          unsigned long long w[kBatch];
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * kThreads;
+            w[u] = i < nw ? get_rec(src0 + i) : tagged(0u, tag);
+          }
+#pragma unroll
+          for (int u = 0; u < kBatch; ++u) {
+            const int i = i0 + u * kThreads;
+            uint32_t spins = 0;
+            while ((uint32_t)(w[u] >> 32) != tag) {
+              __builtin_amdgcn_s_sleep(1);
+              w[u] = get_rec(src0 + i);
+              if (++spins > kSpinLimit) {
+                publish_u32(&P.hdr->error, 1u);
+                break;
+              }
+            }
+            if (i < nw) s_lbw[i] = w[u];
           }
         }
-        s_lbw[i] = w;
       }
       __syncthreads();
       for (int i = l16; i < np; i += 16) {

@@ -268,9 +268,12 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
     H2 = vd.shape[3]
     y = torch.empty(B, L, Nh, H2, dtype=qd.dtype, device=dev)
     w = torch.empty(B, Nh, L, L, dtype=qd.dtype, device=dev) if need_weights else None
+    nws = lib.mega_attention_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2)
+    ws = _scratch_buffer(dev, nws) if nws else None
     with torch.cuda.device(dev):
         rc = lib.mega_attention_fwd(_ptr(qd), _ptr(kd), _ptr(vd), _ptr(y), _ptr(w), _dtype_code(qd), B, L, Nh, H1, H2,
-                                    float(scale), 1 if use_causal_mask else 0, _stream(dev))
+                                    float(scale), 1 if use_causal_mask else 0, _ptr(ws), ws.numel() if nws else 0,
+                                    _stream(dev))
     _lib.check(rc, "attention_fwd")
     return y, w
 

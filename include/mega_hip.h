@@ -188,10 +188,15 @@ int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch,
 /* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276),
  * dropout = 0:  q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;
  *   y[b,:,n,:] = softmax_causal(scale q k^T) v per (b, n).  The L x L weights are
- *   not materialised unless w != NULL (w [B,Nh,L,L] of `dtype`).                  */
+ *   not returned unless w != NULL (w [B,Nh,L,L] of `dtype`).
+ *   16-bit activations with H1 % 8 == 0 run on the matrix cores and need the workspace
+ *   (scores in fp32, probabilities and v^T in the activation type); other requests need
+ *   none (mega_attention_workspace_bytes returns 0).                                   */
+size_t mega_attention_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                                      int64_t H2);
 int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
                        int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
-                       int causal, void* stream);
+                       int causal, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* SwiGLU gate: y = silu(a) * b, elementwise over n elements of `dtype`.
