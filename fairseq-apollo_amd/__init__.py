@@ -11,7 +11,13 @@ from .modules import (  # noqa: F401
     TimestepNorm,
 )
 
+from .layers import Mega2Layer, MovingAverageGatedAttention, RMSNorm, RotaryEmbedding  # noqa: F401,E402
+
 __all__ = [
+    "Mega2Layer",
+    "MovingAverageGatedAttention",
+    "RMSNorm",
+    "RotaryEmbedding",
     "ops",
     "AttentionSoftmax",
     "BaseMovingLayer",

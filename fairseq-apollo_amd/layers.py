@@ -1,0 +1,203 @@
+"""Layer glue around the HIP ops: the caller of the hot path in the reference,
+`MovingAverageGatedAttention` (fairseq/modules/moving_average_gated_attention.py:26-470),
+restricted to what Mega2 uses on the causal path (unidirectional, softmax attention through
+the fused rotary / causal op, TimestepNorm, EMA or CEMA), plus the north-star SwiGLU FFN.
+
+The projections are library GEMMs (torch -> hipBLASLt); normalisation, moving average,
+attention and the SwiGLU gate run in libmega_hip.so.  Forward only.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+from torch.nn import Parameter
+
+from . import ops
+from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SwiGLU, TimestepNorm,
+                      _no_grad_only)
+
+
+class RMSNorm(nn.Module):
+    """x / sqrt(mean(x^2) + eps) * weight (fairseq/modules/norm_layer/layer_norm.py:41-59, which
+    wraps apex FusedRMSNorm); plain torch here, it is not on the measured path."""
+
+    def __init__(self, dim: int, elementwise_affine: bool = True, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        if elementwise_affine:
+            self.weight = Parameter(torch.ones(dim))
+        else:
+            self.register_parameter("weight", None)
+
+    def forward(self, x: Tensor) -> Tensor:
+        y = x.float()
+        y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.eps)
+        if self.weight is not None:
+            y = y * self.weight.float()
+        return y.to(x.dtype)
+
+
+class RotaryEmbedding(nn.Module):
+    """fairseq/modules/relative_positional_bias.py:47-97: features (2i, 2i+1) rotate by
+    t * base^(-2i/dim); q may start at an offset (incremental decoding)."""
+
+    def __init__(self, embed_dim: int, max_positions: int, base: Optional[float] = None):
+        super().__init__()
+        assert embed_dim % 2 == 0
+        self.embed_dim = embed_dim
+        self.max_positions = max_positions
+        self.base = 10000 if base is None else base
+        freqs = 1.0 / torch.tensor([self.base ** (j / embed_dim) for j in range(0, embed_dim, 2)], dtype=torch.float32)
+        self.register_buffer("freqs", freqs)
+        self._cis: Optional[Tensor] = None
+
+    def _freqs_cis(self, start: int, end: int) -> Tensor:
+        if self._cis is None or self._cis.shape[0] < end or self._cis.device != self.freqs.device:
+            n = max(end, self.max_positions)
+            t = torch.arange(n, dtype=torch.float32, device=self.freqs.device)
+            ang = torch.outer(t, self.freqs.float())
+            self._cis = torch.polar(torch.ones_like(ang), ang)
+        return self._cis[start:end]
+
+    def rotary(self, x: Tensor, sidx: int) -> Tensor:
+        """x: [..., C, dim] with positions along the second to last axis."""
+        cis = self._freqs_cis(sidx, sidx + x.shape[-2])
+        x_ = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
+        return torch.view_as_real(x_ * cis).flatten(-2).to(x.dtype)
+
+    def forward(self, xq: Tensor, xk: Tensor, qidx: int = 0) -> Tuple[Tensor, Tensor]:
+        return self.rotary(xq, qidx), self.rotary(xk, 0)
+
+
+class MovingAverageGatedAttention(nn.Module, IncrementalState):
+    """Gated attention with a moving-average pre-mixer.  Constructor arguments follow the
+    reference (moving_average_gated_attention.py:31-53) for the supported subset; `num_heads`
+    (default 1 = the reference) splits q, k and v into heads in the [B, L, Nh, H] layout of the
+    fused attention op."""
+
+    def __init__(self, embed_dim, zdim, hdim, ndim, chunk_size=-1, moving_layer='cema', moving_act='rmsnorm',
+                 norm_num_groups=None, norm_affine=True, norm_eps=1e-5, max_positions=1024, num_heads=1,
+                 efficient_attn=True, rel_pos_bias='rotary', bidirectional=False, attention_activation='softmax'):
+        super().__init__()
+        self.init_incremental_state()
+        if bidirectional or not efficient_attn or rel_pos_bias != 'rotary' or attention_activation != 'softmax':
+            raise NotImplementedError("only the causal path with the fused rotary softmax attention is built")
+        assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
+        self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
+        self.chunk_size = chunk_size
+        self.num_heads = num_heads
+        self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=True, scale=1.0)
+        self.norm = TimestepNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
+        if moving_layer == 'ema':
+            self.move = MultiHeadEMA(embed_dim, ndim=ndim)
+        elif moving_layer == 'cema':
+            self.move = MultiHeadComplexEMA(embed_dim, ndim=ndim)
+        else:
+            raise ValueError("Unknown moving type: {}".format(moving_layer))
+        assert moving_act in ['rmsnorm', 'silu']
+        self.move_act = RMSNorm(embed_dim, norm_affine, norm_eps) if moving_act == 'rmsnorm' else nn.SiLU()
+        self.v_proj = nn.Linear(embed_dim, hdim, bias=True)
+        self.mx_proj = nn.Linear(embed_dim, zdim + hdim + 2 * embed_dim, bias=True)
+        self.h_proj = nn.Linear(hdim, embed_dim, bias=False)
+        self.gamma = Parameter(torch.zeros(2, zdim))
+        self.beta = Parameter(torch.zeros(2, zdim))
+        self.max_positions = max_positions if chunk_size < 0 else chunk_size
+        self.rel_pos_bias = RotaryEmbedding(zdim // num_heads, self.max_positions)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        for lin in (self.v_proj, self.mx_proj, self.h_proj):
+            nn.init.normal_(lin.weight, mean=0.0, std=0.02)
+        nn.init.constant_(self.v_proj.bias, 0.0)
+        nn.init.constant_(self.mx_proj.bias, 0.0)
+        nn.init.constant_(self.gamma, 0.0)
+        nn.init.constant_(self.beta, 0.0)
+
+    def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
+                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None):
+        """x: [B, L, D] -> ([B, L, D], None)."""
+        _no_grad_only(self, x)
+        bsz, seq_len, embed_dim = x.size()
+        assert embed_dim == self.embed_dim
+        saved_state = self._get_input_buffer(incremental_state) if incremental_state is not None else None
+        residual = x
+        x = self.norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
+        v = F.silu(self.v_proj(x))
+        mx = self.move(x.transpose(1, 2), padding_mask, incremental_state).transpose(1, 2)
+        mx = self.move_act(mx)
+        base = self.mx_proj(mx)
+        u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
+        u = torch.sigmoid(u)
+        z = F.normalize(z, p=2, dim=-1, eps=1e-5)
+        z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
+        q, k = torch.unbind(z, dim=2)
+        r = F.silu(r)
+        if saved_state is not None:
+            # partial-chunk key / value cache (moving_average_gated_attention.py:332-372)
+            if "prev_key" in saved_state:
+                k = torch.cat([saved_state["prev_key"], k], dim=1)
+                v = torch.cat([saved_state["prev_value"], v], dim=1)
+            if self.chunk_size < 0 or k.size(1) % self.chunk_size != 0:
+                saved_state["prev_key"], saved_state["prev_value"] = k, v
+            else:
+                saved_state.pop("prev_key", None)
+                saved_state.pop("prev_value", None)
+            self._set_input_buffer(incremental_state, saved_state)
+        Nh = self.num_heads
+        ctx_len = k.size(1)
+        if 1 < self.chunk_size < seq_len:
+            nc = seq_len // self.chunk_size
+            q = q.reshape(bsz * nc, self.chunk_size, self.zdim)
+        if 1 < self.chunk_size < ctx_len:
+            nc = ctx_len // self.chunk_size
+            k = k.reshape(bsz * nc, self.chunk_size, self.zdim)
+            v = v.reshape(bsz * nc, self.chunk_size, self.hdim)
+        # [B', C, Nh, H]; rotary positions run along C per head and restart in every chunk
+        q4 = q.reshape(q.size(0), q.size(1), Nh, -1)
+        k4 = k.reshape(k.size(0), k.size(1), Nh, -1)
+        v4 = v.reshape(v.size(0), v.size(1), Nh, -1)
+        qidx = k4.size(1) - q4.size(1)
+        q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), qidx).transpose(1, 2)
+        k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+        if q4.size(1) == k4.size(1):
+            attn = self.efficient_attn(q4, k4, v4)
+        else:
+            # a few new queries against a longer cached context: right-aligned causal softmax
+            s = torch.einsum('bqnh,bknh->bnqk', q4.float(), k4.float()).to(q4.dtype)
+            w = ops.attention_softmax_fwd(s, 0.0, True)
+            attn = torch.einsum('bnqk,bknh->bqnh', w.float(), v4.float()).to(v4.dtype)
+        attn = attn.reshape(bsz, seq_len, self.hdim)
+        h = F.silu(hx + self.h_proj(attn * r))
+        out = torch.addcmul(residual, u, h - residual)
+        return out, None
+
+    def _get_input_buffer(self, incremental_state):
+        result = self.get_incremental_state(incremental_state, "attn_state")
+        return result if result is not None else {}
+
+    def _set_input_buffer(self, incremental_state, buffer):
+        return self.set_incremental_state(incremental_state, "attn_state", buffer)
+
+
+class Mega2Layer(nn.Module):
+    """One Mega2 block of the north-star configuration: gated attention (TimestepNorm -> CEMA ->
+    chunked causal attention) followed by a pre-normalised SwiGLU FFN with a residual."""
+
+    def __init__(self, embed_dim, zdim, hdim, ndim, ffn_dim, chunk_size, norm_num_groups=16, num_heads=1,
+                 moving_act='silu'):
+        super().__init__()
+        self.attn = MovingAverageGatedAttention(embed_dim, zdim, hdim, ndim, chunk_size=chunk_size,
+                                                norm_num_groups=norm_num_groups, num_heads=num_heads,
+                                                moving_act=moving_act)
+        self.ffn_norm = TimestepNorm(embed_dim, num_groups=norm_num_groups)
+        self.ffn = SwiGLU(embed_dim, ffn_dim, bias=False)
+        for lin in (self.ffn.w1, self.ffn.w2, self.ffn.w3):
+            nn.init.normal_(lin.weight, mean=0.0, std=0.02)
+
+    def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, incremental_state=None) -> Tensor:
+        x, _ = self.attn(x, padding_mask, incremental_state)
+        return x + self.ffn(self.ffn_norm(x, padding_mask, incremental_state))

@@ -437,3 +437,55 @@ def rotary(x, base: float = 10000.0):
     out[..., 0::2] = z.real
     out[..., 1::2] = z.imag
     return out
+
+
+def rms_norm(x, weight=None, eps: float = 1e-5):
+    """RMSNorm over the last axis (modules/norm_layer/layer_norm.py:41-59: apex FusedRMSNorm):
+    x / sqrt(mean(x^2) + eps) * weight."""
+    x = np.asarray(x, np.float64)
+    y = x / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
+    return y if weight is None else y * np.asarray(weight, np.float64)
+
+
+def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str = 'silu', eps: float = 1e-5,
+                          num_groups: Optional[int] = None):
+    """MovingAverageGatedAttention.forward, unidirectional, softmax attention through the fused
+    (rotary, causal, scale 1) op: modules/moving_average_gated_attention.py:263-417, step by
+    step.  x: [B, L, D]; P: dict of numpy parameters
+      norm_weight, norm_bias [D]; ema p, q, gamma [D, N], omega [D];
+      v_w [E, D], v_b [E]; mx_w [D+S+E+D, D], mx_b; h_w [D, E]; gamma, beta [2, S];
+      optional rms_weight [D].
+    num_heads > 1 splits q, k (S) and v (E) into heads laid out [B, L, Nh, H] (the layout of the
+    fused op, csrc/ops/attention_kernel.cu:46-50); the reference layer itself is single-head."""
+    x = np.asarray(x, np.float64)
+    B, L, D = x.shape
+    S = P['gamma'].shape[1]
+    E = P['v_w'].shape[0]
+    xn, _, _, _ = timestep_norm(x, np.zeros(B, np.int64), np.zeros((B, num_groups or D)), np.ones((B, num_groups or D)),
+                                np.asarray(P['norm_weight'], np.float64) + 1.0, P['norm_bias'], None, num_groups, eps)
+    v = _silu(xn @ np.asarray(P['v_w'], np.float64).T + P['v_b'])
+    mx, _ = ema_forward(xn.transpose(0, 2, 1), P['p'], P['q'], P['ema_gamma'], P['omega'])
+    mx = mx.transpose(0, 2, 1)
+    mx = _silu(mx) if moving_act == 'silu' else rms_norm(mx, P.get('rms_weight'), eps)
+    base = mx @ np.asarray(P['mx_w'], np.float64).T + P['mx_b']
+    u, z, r, hx = np.split(base, [D, D + S, D + S + E], axis=-1)
+    u = _sigmoid(u)
+    z = z / np.maximum(np.sqrt((z * z).sum(-1, keepdims=True)), 1e-5)
+    g = np.asarray(P['gamma'], np.float64) + 1.0
+    bt = np.asarray(P['beta'], np.float64)
+    q = z * g[0] + bt[0]
+    k = z * g[1] + bt[1]
+    r = _silu(r)
+    nc = L // chunk if 1 < chunk < L else 1
+    C = L // nc
+    H1, H2 = S // num_heads, E // num_heads
+    qc = q.reshape(B * nc, C, num_heads, H1)
+    kc = k.reshape(B * nc, C, num_heads, H1)
+    vc = v.reshape(B * nc, C, num_heads, H2)
+    # rotary on every head's features, positions restart in every chunk
+    qr = rotary(qc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
+    kr = rotary(kc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
+    a, _ = attention(qr, kr, vc, 1.0, True)
+    a = a.reshape(B, L, E)
+    h = _silu(hx + (a * r) @ np.asarray(P['h_w'], np.float64).T)
+    return x + u * (h - x)

@@ -1,0 +1,99 @@
+"""The gated-attention layer (the caller of the hot path) and the full Mega2 block against the
+fp64 oracle restatement of moving_average_gated_attention.py:263-417."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import rel_err
+from gpu_util import DEV, host
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _params(layer):
+    p, q, g = layer.move.coeffs()
+    P = dict(norm_weight=host(layer.norm.weight), norm_bias=host(layer.norm.bias), p=host(p.squeeze(-1)),
+             q=host(q.squeeze(-1)), ema_gamma=host(g), omega=host(layer.move.omega).reshape(-1),
+             v_w=host(layer.v_proj.weight), v_b=host(layer.v_proj.bias), mx_w=host(layer.mx_proj.weight),
+             mx_b=host(layer.mx_proj.bias), h_w=host(layer.h_proj.weight), gamma=host(layer.gamma),
+             beta=host(layer.beta))
+    if isinstance(layer.move_act, M.RMSNorm):
+        P['rms_weight'] = host(layer.move_act.weight)
+    return P
+
+
+def _chain_ok(y, yo, tol):
+    """A layer chains ~10 roundings to the activation type, so the per-op bound (2e-2 for bf16) is
+    applied to the root-mean-square error and a 4x wider bound to the worst element."""
+    e = host(y) - yo
+    rms = np.sqrt(np.mean(yo ** 2))
+    return rel_err(host(y), yo) < 4 * tol and np.sqrt(np.mean(e ** 2)) < tol * rms
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("heads,act,moving", [(1, 'rmsnorm', 'cema'), (4, 'silu', 'cema'), (1, 'silu', 'ema')])
+def test_gated_attention_layer(dtype, tol, heads, act, moving):
+    torch.manual_seed(7)
+    B, L, D, S, E, N, C = 2, 512, 64, 32, 128, 16, 256
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_layer=moving, moving_act=act,
+                                          norm_num_groups=8, num_heads=heads).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.15)
+        layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
+        layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+    P = _params(layer)                       # fp32 master copy of the parameters
+    if dtype != torch.float32:               # the module rounds its projection weights to the activation type
+        for k_ in ('v_w', 'v_b', 'mx_w', 'mx_b', 'h_w', 'gamma', 'beta', 'norm_weight', 'norm_bias', 'rms_weight'):
+            if k_ in P:
+                P[k_] = torch.from_numpy(np.asarray(P[k_], np.float32)).to(dtype).double().numpy()
+    layer = layer.to(dtype)
+    x = torch.randn(B, L, D, device=DEV).to(dtype)
+    with torch.no_grad():
+        y, _ = layer(x)
+    yo = O.gated_attention_layer(host(x), P, chunk=C, num_heads=heads, moving_act=act, num_groups=8)
+    assert _chain_ok(y, yo, tol) if dtype != torch.float32 else rel_err(host(y), yo) < tol
+
+
+def test_incremental_chunks_match_one_shot():
+    torch.manual_seed(8)
+    B, L, D, S, E, N, C = 2, 512, 64, 32, 64, 16, 128
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act='silu', norm_num_groups=8).to(DEV).eval()
+    x = torch.randn(B, L, D, device=DEV)
+    with torch.no_grad():
+        full, _ = layer(x)
+        state = {}
+        parts = [layer(x[:, a:a + C], None, state)[0] for a in range(0, L, C)]
+        state2 = {}
+        odd = [layer(x[:, a:b], None, state2)[0] for a, b in ((0, 100), (100, 128), (128, 131), (131, 256))]
+    assert rel_err(host(torch.cat(parts, 1)), host(full)) < 1e-4
+    assert rel_err(host(torch.cat(odd, 1)), host(full[:, :256])) < 1e-4
+
+
+def test_config4_full_mega2_layer_bf16():
+    """B=1, L=8192, D=2048, z=512, v=4096, chunk 2048, 4 heads, SwiGLU 5632, bf16."""
+    torch.manual_seed(1238)
+    B, L, D, S, E, N, C, Hf = 1, 8192, 2048, 512, 4096, 16, 2048, 5632
+    blk = M.Mega2Layer(D, S, E, N, Hf, C, norm_num_groups=16, num_heads=4, moving_act='silu').to(DEV).eval()
+    P = _params(blk.attn)
+    w1, w2, w3 = host(blk.ffn.w1.weight), host(blk.ffn.w2.weight), host(blk.ffn.w3.weight)
+    blk = blk.to(torch.bfloat16)
+    x = torch.randn(B, L, D, device=DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        y = blk(x)
+        a, _ = blk.attn(x)
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    # oracle on the first two chunks (causal: they do not see the rest), bf16-rounded weights
+    Lo = 2 * C
+    rb = lambda a_: torch.from_numpy(np.asarray(a_, np.float32)).to(torch.bfloat16).double().numpy()
+    Pb = {k_: (rb(v_) if k_ in ('v_w', 'v_b', 'mx_w', 'mx_b', 'h_w', 'gamma', 'beta', 'norm_weight', 'norm_bias')
+               else v_) for k_, v_ in P.items()}
+    ao = O.gated_attention_layer(host(x[:, :Lo]), Pb, chunk=C, num_heads=4, moving_act='silu', num_groups=16)
+    assert _chain_ok(a[:, :Lo], ao, 2e-2)
+    xn, _, _, _ = O.timestep_norm(ao, np.zeros(B, np.int64), np.zeros((B, 16)), np.ones((B, 16)), np.ones(D),
+                                  np.zeros(D), None, 16, 1e-5)
+    yo = ao + O.swiglu_ffn(xn, rb(w1), rb(w3), rb(w2))
+    assert _chain_ok(y[:, :Lo], yo, 2e-2)

@@ -58,3 +58,33 @@ def test_swiglu_and_rotary():
     q = rng.normal(size=(1, 1, 8)).repeat(7, 1); k = rng.normal(size=(1, 1, 8)).repeat(7, 1)
     rq, rk = O.rotary(q), O.rotary(k)
     assert np.isclose(rq[0, 5] @ rk[0, 3], rq[0, 4] @ rk[0, 2])
+
+
+def _layer_params(rng, D, S, E, N):
+    from conftest import mega_init_complex
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    return dict(norm_weight=rng.normal(size=D) * 0.1, norm_bias=rng.normal(size=D) * 0.1, p=p, q=q, ema_gamma=g,
+                omega=rng.normal(size=D), v_w=rng.normal(size=(E, D)) * 0.2, v_b=rng.normal(size=E) * 0.1,
+                mx_w=rng.normal(size=(2 * D + S + E, D)) * 0.2, mx_b=rng.normal(size=2 * D + S + E) * 0.1,
+                h_w=rng.normal(size=(D, E)) * 0.2, gamma=rng.normal(size=(2, S)) * 0.1, beta=rng.normal(size=(2, S)) * 0.1)
+
+
+def test_layer_gate_closed_forms_and_chunk_causality():
+    rng = np.random.default_rng(5)
+    B, L, D, S, E, N = 2, 12, 8, 4, 6, 4
+    P = _layer_params(rng, D, S, E, N)
+    x = rng.normal(size=(B, L, D))
+    y = O.gated_attention_layer(x, P, chunk=4, num_groups=2)
+    # u == 0 (a very negative gate bias) makes the layer the identity
+    P0 = dict(P); P0['mx_b'] = P['mx_b'].copy(); P0['mx_b'][:D] = -1e4; P0['mx_w'] = P['mx_w'].copy(); P0['mx_w'][:D] = 0
+    assert np.allclose(O.gated_attention_layer(x, P0, chunk=4, num_groups=2), x, atol=1e-12)
+    # causal: outputs before t do not see x[t:]
+    x2 = x.copy(); x2[:, 7:] += rng.normal(size=(B, 5, D))
+    y2 = O.gated_attention_layer(x2, P, chunk=4, num_groups=2)
+    assert np.allclose(y2[:, :7], y[:, :7], atol=1e-10) and not np.allclose(y2[:, 7:], y[:, 7:])
+    # head split with one head equals the single-head layer; rms variant follows its formula
+    assert np.allclose(O.gated_attention_layer(x, P, chunk=4, num_heads=1, num_groups=2), y)
+    z = rng.normal(size=(3, 5))
+    assert np.allclose(O.rms_norm(z, None, 1e-5), z / np.sqrt((z ** 2).mean(-1, keepdims=True) + 1e-5))
+    yh = O.gated_attention_layer(x, P, chunk=4, num_heads=2, num_groups=2)
+    assert yh.shape == y.shape and not np.allclose(yh, y)
