@@ -18,6 +18,7 @@ SOURCES = [
     "timestep_norm.hip",
     "ema_scan.hip",
     "ema_mfma.hip",
+    "decode.hip",
     "elementwise.hip",
     "attention.hip",
     "attention_mfma.hip",

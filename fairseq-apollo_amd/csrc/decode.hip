@@ -1,0 +1,146 @@
+// One decode step of the norm -> moving-average pair: streaming TimestepNorm of one token
+// (fairseq/modules/norm_layer/timestep_norm.py:100-139 with L = 1: the WelfordCombine of
+// fairseq/csrc/utils.h:66-76 on the carried (count, mean, var)) followed by the single-step state
+// update h' = q h + p xn, y = Re sum gamma h' + omega xn
+// (fairseq/modules/base_moving_average.py:105-118, 144-160).  One launch per step; a workgroup
+// owns one (stream, group): it reads its slice of x once, the state h once, and writes both back.
+// Traffic per step is the state: 2 * B * D * N * 8 bytes.
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kT = 128;
+
+struct StepArgs {
+  const void* x;
+  void* xn;
+  void* y;
+  const int64_t* prev_count;
+  const float* prev_mean;
+  const float* prev_var;
+  int64_t* count;
+  float* mean;
+  float* var;
+  const float* nw;       // gamma of the norm (weight + 1)
+  const float* nb;
+  const float* p;        // [D, N]
+  const float* q;        // [D, N, 2]
+  const float* g;        // [D, N, 2]
+  const float* omega;    // [D]
+  const float* h_in;     // [B, D, N, 2] or null
+  float* h_out;
+  int B, D, G, N;
+  float eps;
+};
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < kT / 64; ++i) t += red[i];
+  return t;
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kT) void norm_ema_step_kernel(const StepArgs A) {
+  __shared__ float red[kT / 64];
+  const int g = blockIdx.x % A.G, b = blockIdx.x / A.G;
+  const int dg = A.D / A.G;
+  const T* xr = (const T*)A.x + (size_t)b * A.D + (size_t)g * dg;
+  // moments of this token's group
+  float s = 0.f;
+  for (int f = threadIdx.x; f < dg; f += kT) s += to_float(xr[f]);
+  const float gm = block_sum(s, red) / (float)dg;
+  float s2 = 0.f;
+  for (int f = threadIdx.x; f < dg; f += kT) {
+    const float d = to_float(xr[f]) - gm;
+    s2 += d * d;
+  }
+  const float gv = block_sum(s2, red) / (float)dg;
+  // fold into the carried state (one step of weight 1)
+  const int64_t c0 = A.prev_count[b];
+  const float u0 = A.prev_mean[(size_t)b * A.G + g], v0 = A.prev_var[(size_t)b * A.G + g];
+  const float c1 = (float)c0 / (float)(c0 + 1), c2 = 1.0f / (float)(c0 + 1);
+  const float dl = gm - u0;
+  const float u1 = c1 * u0 + c2 * gm;
+  const float v1 = c1 * v0 + c2 * gv + (c1 * dl) * (c2 * dl);
+  const float rstd = 1.0f / sqrtf(v1 + A.eps);
+  __syncthreads();                               // every thread has read the old state
+  if (threadIdx.x == 0) {
+    A.mean[(size_t)b * A.G + g] = u1;
+    A.var[(size_t)b * A.G + g] = v1;
+    if (g == 0) A.count[b] = c0 + 1;
+  }
+  for (int f = threadIdx.x; f < dg; f += kT) {
+    const int d = g * dg + f;
+    const size_t o = (size_t)b * A.D + d;
+    const float xnv_full = (to_float(xr[f]) - u1) * rstd * A.nw[d] + A.nb[d];
+    const T xn_t = from_float<T>(xnv_full);
+    ((T*)A.xn)[o] = xn_t;
+    const float xv = to_float(xn_t);             // the moving average sees the rounded activation
+    float acc = 0.f;
+    const size_t ho = o * A.N * 2;
+    const size_t co = (size_t)d * A.N;
+    for (int n = 0; n < A.N; ++n) {
+      const float qr = A.q[(co + n) * 2], qi = CPLX ? A.q[(co + n) * 2 + 1] : 0.f;
+      const float gr = A.g[(co + n) * 2], gi = CPLX ? A.g[(co + n) * 2 + 1] : 0.f;
+      float hr = 0.f, hi = 0.f;
+      if (A.h_in) {
+        hr = A.h_in[ho + 2 * n];
+        hi = CPLX ? A.h_in[ho + 2 * n + 1] : 0.f;
+      }
+      const float nr = qr * hr - qi * hi + A.p[co + n] * xv;
+      const float ni = qr * hi + qi * hr;
+      A.h_out[ho + 2 * n] = nr;
+      A.h_out[ho + 2 * n + 1] = ni;
+      acc += gr * nr - gi * ni;
+    }
+    ((T*)A.y)[o] = from_float<T>(acc + A.omega[d] * xv);
+  }
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_t* prev_count,
+                                  const float* prev_mean, const float* prev_var, int64_t* count, float* mean,
+                                  float* var, const float* norm_gamma, const float* norm_beta, double eps,
+                                  const float* p, const float* q, const float* gamma, int is_complex,
+                                  const float* omega, const float* h_in, float* h_out, int64_t B, int64_t D,
+                                  int64_t G, int64_t N, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "norm_ema_step: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && D > 0 && G > 0 && N > 0 && D % G == 0, MEGA_ERR_ARG,
+               "norm_ema_step: bad shape B=%ld D=%ld G=%ld N=%ld", (long)B, (long)D, (long)G, (long)N);
+  MEGA_REQUIRE(N <= 32, MEGA_ERR_UNSUPPORTED, "norm_ema_step: ndim=%ld > 32 is not supported", (long)N);
+  MEGA_REQUIRE(B * G < (int64_t)1 << 31, MEGA_ERR_UNSUPPORTED, "norm_ema_step: too many streams");
+  if (B == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && xn && y && prev_count && prev_mean && prev_var && count && mean && var && norm_gamma && norm_beta &&
+                   p && q && gamma && omega && h_out,
+               MEGA_ERR_ARG, "norm_ema_step: null pointer argument");
+  StepArgs A;
+  A.x = x; A.xn = xn; A.y = y; A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var;
+  A.count = count; A.mean = mean; A.var = var; A.nw = norm_gamma; A.nb = norm_beta; A.p = p; A.q = q; A.g = gamma;
+  A.omega = omega; A.h_in = h_in; A.h_out = h_out; A.B = (int)B; A.D = (int)D; A.G = (int)G; A.N = (int)N;
+  A.eps = (float)eps;
+  const dim3 grid((unsigned)(B * G));
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH_NS(T, C) hipLaunchKernelGGL((norm_ema_step_kernel<T, C>), grid, dim3(kT), 0, s, A)
+  if (is_complex) {
+    if (dtype == MEGA_F32) LAUNCH_NS(float, true);
+    else if (dtype == MEGA_BF16) LAUNCH_NS(bf16_t, true);
+    else LAUNCH_NS(f16_t, true);
+  } else {
+    if (dtype == MEGA_F32) LAUNCH_NS(float, false);
+    else if (dtype == MEGA_BF16) LAUNCH_NS(bf16_t, false);
+    else LAUNCH_NS(f16_t, false);
+  }
+#undef LAUNCH_NS
+  MEGA_CHECK_LAUNCH("norm_ema_step");
+  return MEGA_OK;
+}

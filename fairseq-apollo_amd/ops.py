@@ -408,6 +408,48 @@ def ema_step(x_t: torch.Tensor, p, q, gamma, omega, h: Optional[torch.Tensor]):
     return y, (torch.view_as_complex(hout) if is_complex else hout[..., 0])
 
 
+class DecodeStep:
+    """Streaming decode of the norm -> moving-average pair: one launch per token.  Holds the
+    converted coefficients and the carried state (norm count / mean / var, EMA h) on the device
+    and updates them in place."""
+
+    def __init__(self, norm_weight, norm_bias, num_groups: int, eps: float, p, q, gamma, omega, batch_size: int,
+                 prior_count: int = 0):
+        self.dev = _need_gpu(norm_weight, norm_bias, p, q, gamma, omega)
+        self.D, self.N = p.shape[0], p.shape[1]
+        self.G, self.eps, self.B = int(num_groups), float(eps), int(batch_size)
+        self.is_complex = bool(q.is_complex() or gamma.is_complex())
+        self.nw = (_f32c(norm_weight) + 1.0).contiguous()
+        self.nb = _f32c(norm_bias)
+        self.p = _f32c(p).reshape(self.D, self.N)
+        self.q = _cplx_as_f32(q.reshape(self.D, self.N))
+        self.gamma = _cplx_as_f32(gamma.reshape(self.D, self.N))
+        self.omega = _f32c(omega).reshape(self.D)
+        self.count = torch.full((self.B,), prior_count, dtype=torch.int64, device=self.dev)
+        self.mean = torch.zeros(self.B, self.G, dtype=torch.float32, device=self.dev)
+        self.var = torch.ones(self.B, self.G, dtype=torch.float32, device=self.dev)
+        self.h = torch.zeros(self.B, self.D, self.N, 2, dtype=torch.float32, device=self.dev)
+
+    def __call__(self, x_t: torch.Tensor):
+        """x_t: [B, D] -> (xn_t, y_t), both [B, D]."""
+        lib = _lib.load()
+        xd = x_t.detach().contiguous()
+        xn = torch.empty_like(xd)
+        y = torch.empty_like(xd)
+        with torch.cuda.device(self.dev):
+            rc = lib.mega_norm_ema_step(_ptr(xd), _ptr(xn), _ptr(y), _dtype_code(xd), _ptr(self.count), _ptr(self.mean),
+                                        _ptr(self.var), _ptr(self.count), _ptr(self.mean), _ptr(self.var), _ptr(self.nw),
+                                        _ptr(self.nb), self.eps, _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
+                                        1 if self.is_complex else 0, _ptr(self.omega), _ptr(self.h), _ptr(self.h),
+                                        self.B, self.D, self.G, self.N, _stream(self.dev))
+        _lib.check(rc, "norm_ema_step")
+        return xn, y
+
+    @property
+    def state(self) -> torch.Tensor:
+        return torch.view_as_complex(self.h) if self.is_complex else self.h[..., 0]
+
+
 def fftconv(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """Causal long convolution with an explicit kernel k[D, Lk] (fftconv,
     fairseq/modules/fused_ops/fftconv.py:11-27); evaluated in the time domain."""

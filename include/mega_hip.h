@@ -135,6 +135,22 @@ int mega_ema_step(const void* x, void* y, int dtype, const float* p, const float
                   const float* gamma, int is_complex, const float* omega, const float* h_in,
                   float* h_out, int64_t B, int64_t D, int64_t N, void* stream);
 
+/* One decode step of the norm -> moving-average pair in one launch: streaming group
+ * TimestepNorm of a single token (TimestepNorm.forward with L = 1 and incremental state,
+ * fairseq/modules/norm_layer/timestep_norm.py:100-139) followed by mega_ema_step on the
+ * normalised token (BaseMovingLayer.forward with L = 1 and incremental state,
+ * fairseq/modules/base_moving_average.py:144-160).  The reference runs these as two modules
+ * and >= 6 kernels per step.
+ *   x, xn, y [B,D] of `dtype`; norm state in (prev_*) and out (count, mean, var; may alias
+ *   the inputs); norm_gamma (= weight + 1), norm_beta [D]; EMA coefficients as mega_ema_step;
+ *   h_in may be NULL (zero state) and h_out may alias h_in.                              */
+int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_t* prev_count,
+                       const float* prev_mean, const float* prev_var, int64_t* count,
+                       float* mean, float* var, const float* norm_gamma, const float* norm_beta,
+                       double eps, const float* p, const float* q, const float* gamma,
+                       int is_complex, const float* omega, const float* h_in, float* h_out,
+                       int64_t B, int64_t D, int64_t G, int64_t N, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Long convolution with an explicit time-domain kernel                      */
 /* stands in for fftconv(x, k) (fairseq/modules/fused_ops/fftconv.py:11-27, 45-61;

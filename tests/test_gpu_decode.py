@@ -1,0 +1,91 @@
+"""Recurrent decode path: single-step EMA state update plus streaming TimestepNorm, checked against
+the parallel path on the concatenated sequence (both HIP) and against the fp64 oracle."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import mega_init_complex, rel_err
+from gpu_util import DEV, dev, host, rounded
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(B, D, N, G, seed):
+    rng = np.random.default_rng(seed)
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    om = rng.normal(size=D)
+    nw = rng.normal(size=D) * 0.1
+    nb = rng.normal(size=D) * 0.1
+    return rng, p, q, g, om, nw, nb
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_small_streams_against_oracle(dtype, tol):
+    B, D, N, G, T = 3, 96, 16, 4, 200
+    rng, p, q, g, om, nw, nb = _setup(B, D, N, G, 41)
+    x, x64 = rounded(rng.normal(size=(B, T, D)), dtype)
+    step = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    xs, ys = [], []
+    for t in range(T):
+        xn, y = step(x[:, t])
+        xs.append(xn); ys.append(y)
+    xn_s, y_s = torch.stack(xs, 1), torch.stack(ys, 1)
+    torch.cuda.synchronize()
+    xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, None, G)
+    assert rel_err(host(xn_s), xno) < max(tol, 1e-4)
+    yo, ho = O.ema_forward(host(xn_s).transpose(0, 2, 1), p, q, g, om, incremental=True)
+    assert rel_err(host(y_s), yo.transpose(0, 2, 1)) < max(tol, 1e-4)
+    assert step.count.tolist() == [T] * B
+    assert rel_err(host(step.mean), mu) < 1e-4 and rel_err(host(step.var), v) < 1e-4
+    assert rel_err(np.real(host(step.state)), np.real(ho)) < 1e-4
+    # the same tokens through the parallel kernels
+    norm = M.TimestepNorm(D, G).to(DEV).eval()
+    with torch.no_grad():
+        norm.weight.copy_(dev(nw)); norm.bias.copy_(dev(nb))
+        xn_p = norm(x)
+        y_p, h_p = M.ops.ema_forward(xn_p.transpose(1, 2), dev(p), dev(q), dev(g), dev(om), want_state=True)
+    assert rel_err(host(xn_s), host(xn_p)) < tol
+    assert rel_err(host(y_s), host(y_p.transpose(1, 2))) < tol
+
+
+def test_config3_b64_d2048_2048_steps():
+    """B = 64 streams, D = 2048, N = 16, complex q, 2048 consecutive steps, fp32: the recurrent
+    path agrees with the parallel path on the concatenated sequence to 1e-5; four streams are also
+    checked against the fp64 oracle."""
+    B, D, N, G, T = 64, 2048, 16, 16, 2048
+    rng, p, q, g, om, nw, nb = _setup(B, D, N, G, 1237)
+    gen = torch.Generator().manual_seed(1237)
+    x = torch.randn(B, T, D, generator=gen).to(DEV)
+    step = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    xn_s = torch.empty_like(x)
+    y_s = torch.empty_like(x)
+    for t in range(T):
+        xn_s[:, t], y_s[:, t] = step(x[:, t])
+    norm = M.TimestepNorm(D, G).to(DEV).eval()
+    with torch.no_grad():
+        norm.weight.copy_(dev(nw)); norm.bias.copy_(dev(nb))
+        state = {}
+        xn_p = norm(x, None, state)
+        y_p, h_p = M.ops.ema_forward(xn_p.transpose(1, 2), dev(p), dev(q), dev(g), dev(om), want_state=True)
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    def rel(a, b):       # max |a - b| / max(|b|, rms(b)), evaluated on the device
+        rms = b.abs().pow(2).mean().sqrt()
+        return ((a - b).abs() / torch.clamp(b.abs(), min=rms)).max().item()
+
+    e1 = rel(xn_s, xn_p)
+    e2 = rel(y_s, y_p.transpose(1, 2))
+    e3 = rel(step.state, h_p)
+    print(f"recurrent vs parallel: norm {e1:.2e}, ema {e2:.2e}, state {e3:.2e}", flush=True)
+    assert e1 < 1e-5 and e2 < 1e-5 and e3 < 1e-5
+    saved = norm._get_input_buffer(state)
+    assert torch.equal(saved["prev_count"], step.count)
+    assert (saved["prev_mean"] - step.mean).abs().max().item() < 1e-5
+    sel = [0, 17, 40, 63]
+    x64 = x[sel].double().cpu().numpy()
+    xno, _, _, _ = O.timestep_norm(x64, np.zeros(4, np.int64), np.zeros((4, G)), np.ones((4, G)), nw + 1, nb, None, G)
+    assert rel_err(host(xn_s[sel]), xno) < 1e-4
+    yo, _ = O.ema_forward(xno.transpose(0, 2, 1), p, q, g, om)
+    assert rel_err(host(y_s[sel]), yo.transpose(0, 2, 1)) < 1e-4
