@@ -1,0 +1,104 @@
+"""Writes tests/golden/ref_cpu_vectors.npz: inputs and outputs of the reference's own CPU
+operators for this path, produced by oracle/_ref (fairseq/csrc/ops/timestep_norm.cc,
+ema_parameters.cc, ema_hidden.cc compiled in place by `make -C oracle ref`).
+
+    python tests/golden/make_golden.py
+
+The file holds data only (seeded inputs, the reference's outputs); it lets the parity tests
+run where neither the reference tree nor oracle/_ref exist.
+"""
+import importlib.util
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+
+def load_ref():
+    path = os.path.join(ROOT, "oracle", "_ref", "mega2_ref_cpu.so")
+    old = sys.getdlopenflags()
+    sys.setdlopenflags(os.RTLD_LAZY | os.RTLD_GLOBAL)
+    try:
+        spec = importlib.util.spec_from_file_location("mega2_ref_cpu", path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+    finally:
+        sys.setdlopenflags(old)
+    return mod
+
+
+def main():
+    from conftest import mega_init_complex
+    from oracle import mega_oracle as O
+
+    ref = load_ref()
+    out = {}
+    t = torch.from_numpy
+
+    # group TimestepNorm: ragged padding, carried statistics, non-trivial affine
+    rng = np.random.default_rng(20240)
+    for tag, (B, L, H, G, masked) in {"gtsn_a": (3, 37, 48, 4, True), "gtsn_b": (2, 130, 64, 16, False),
+                                      "gtsn_c": (1, 1, 32, 2, False)}.items():
+        x = rng.normal(size=(B, L, H)).astype(np.float32) * 1.7 + 0.3
+        mask = (rng.random((B, L)) < 0.25) if masked else None
+        pc = rng.integers(0, 6, B).astype(np.int64)
+        pm = (rng.normal(size=(B, G)) * 0.2).astype(np.float32)
+        pv = (rng.random((B, G)) + 0.5).astype(np.float32)
+        pm[pc == 0] = 0.0
+        pv[pc == 0] = 1.0
+        gamma = (rng.normal(size=H) + 1).astype(np.float32)
+        beta = rng.normal(size=H).astype(np.float32)
+        y, c, mu, v = ref.group_timestep_norm_fwd(t(x), t(pc), t(pm), t(pv), t(gamma), t(beta),
+                                                  None if mask is None else t(mask), G, 1e-5)[:4]
+        out.update({f"{tag}.x": x, f"{tag}.prev_count": pc, f"{tag}.prev_mean": pm, f"{tag}.prev_var": pv,
+                    f"{tag}.gamma": gamma, f"{tag}.beta": beta, f"{tag}.groups": np.int64(G),
+                    f"{tag}.y": y.numpy(), f"{tag}.count": c.numpy(), f"{tag}.mean": mu.numpy(),
+                    f"{tag}.var": v.numpy()})
+        if mask is not None:
+            out[f"{tag}.mask"] = mask
+
+    # per-feature TimestepNorm
+    B, L, H = 2, 41, 24
+    x = rng.normal(size=(B, L, H)).astype(np.float32)
+    mask = rng.random((B, L)) < 0.2
+    pc = np.array([0, 3], np.int64)
+    pm = np.zeros((B, H), np.float32)
+    pv = np.ones((B, H), np.float32)
+    pm[1] = rng.normal(size=H) * 0.1
+    pv[1] = rng.random(H) + 0.5
+    gamma = (rng.normal(size=H) + 1).astype(np.float32)
+    beta = rng.normal(size=H).astype(np.float32)
+    y, c, mu, v = ref.timestep_norm_fwd(t(x), t(pc), t(pm), t(pv), t(gamma), t(beta), t(mask), 1e-5)[:4]
+    out.update({"tsn.x": x, "tsn.mask": mask, "tsn.prev_count": pc, "tsn.prev_mean": pm, "tsn.prev_var": pv,
+                "tsn.gamma": gamma, "tsn.beta": beta, "tsn.y": y.numpy(), "tsn.count": c.numpy(),
+                "tsn.mean": mu.numpy(), "tsn.var": v.numpy()})
+
+    # kernel generation (with and without a carried state) and the hidden-state update
+    K, N, L, B = 6, 16, 96, 2
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
+    p = p.astype(np.float32)
+    q = q.astype(np.complex64)
+    g = g.astype(np.complex64)
+    h = (rng.normal(size=(B, K, N)) + 1j * rng.normal(size=(B, K, N))).astype(np.complex64)
+    log_q = t(q).log()
+    w, b, _ = ref.ema_parameters_fwd(t(p), log_q, t(g), t(h), L)
+    x = rng.normal(size=(B, K, L)).astype(np.float32)
+    hy, _ = ref.ema_hidden_fwd(t(x), t(p), log_q, t(h))
+    hy0, _ = ref.ema_hidden_fwd(t(x), t(p), log_q, None)
+    out.update({"ema.p": p, "ema.q": q, "ema.log_q": log_q.numpy(), "ema.gamma": g, "ema.h": h, "ema.x": x,
+                "ema.length": np.int64(L), "ema.kernel": w.numpy(), "ema.bias": b.numpy(),
+                "ema.hidden": hy.numpy(), "ema.hidden_zero_start": hy0.numpy()})
+
+    dst = os.path.join(HERE, "ref_cpu_vectors.npz")
+    np.savez_compressed(dst, **out)
+    print(dst, os.path.getsize(dst), "bytes,", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

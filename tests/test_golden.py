@@ -1,0 +1,131 @@
+"""Committed golden vectors (tests/golden/ref_cpu_vectors.npz: outputs of the reference's own CPU
+operators, written by tests/golden/make_golden.py) against the numpy oracle, the C oracle and,
+on a GPU box, the HIP library.  fp32 inputs; tolerance 2e-5 for the fp64/fp32 oracles
+(the vectors are fp32 results), 1e-4 for the HIP fp32 path."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from oracle import mega_oracle as O
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_cpu_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLD, allow_pickle=False)
+
+
+def _case(gold, tag):
+    return {k[len(tag) + 1:]: gold[k] for k in gold.files if k.startswith(tag + ".")}
+
+
+GROUP_CASES = ["gtsn_a", "gtsn_b", "gtsn_c"]
+
+
+@pytest.mark.parametrize("tag", GROUP_CASES)
+def test_oracle_group_norm(gold, tag):
+    c = _case(gold, tag)
+    y, n, mu, v = O.timestep_norm(c["x"], c["prev_count"], c["prev_mean"], c["prev_var"], c["gamma"], c["beta"],
+                                  c.get("mask"), int(c["groups"]), 1e-5)
+    assert rel_err(y, c["y"]) < 2e-5 and np.array_equal(n, c["count"])
+    assert rel_err(mu, c["mean"]) < 2e-5 and rel_err(v, c["var"]) < 2e-5
+
+
+def test_oracle_feature_norm(gold):
+    c = _case(gold, "tsn")
+    y, n, mu, v = O.timestep_norm(c["x"], c["prev_count"], c["prev_mean"], c["prev_var"], c["gamma"], c["beta"],
+                                  c["mask"], None, 1e-5)
+    assert rel_err(y, c["y"]) < 2e-5 and np.array_equal(n, c["count"])
+    assert rel_err(mu, c["mean"]) < 2e-5 and rel_err(v, c["var"]) < 2e-5
+
+
+def test_oracle_ema(gold):
+    c = _case(gold, "ema")
+    L = int(c["length"])
+    p, q, g, h = c["p"].astype(np.float64), c["q"].astype(np.complex128), c["gamma"].astype(np.complex128), c["h"]
+    assert rel_err(O.ema_kernel(p, q, g, L), c["kernel"]) < 2e-5
+    assert rel_err(O.ema_bias(q, g, h, L), c["bias"]) < 2e-5
+    hy = O.ema_hidden(c["x"], p, q, h)
+    assert rel_err(hy.real, c["hidden"].real) < 2e-5 and rel_err(hy.imag, c["hidden"].imag) < 2e-5
+    hy0 = O.ema_hidden(c["x"], p, q, None)
+    assert rel_err(hy0.real, c["hidden_zero_start"].real) < 2e-5
+    assert rel_err(hy0.imag, c["hidden_zero_start"].imag) < 2e-5
+
+
+@pytest.mark.parametrize("tag", GROUP_CASES)
+def test_oracle_c_group_norm(gold, oracle_c, tag):
+    import oracle_c_api as OC
+
+    c = _case(gold, tag)
+    y, n, mu, v = OC.timestep_norm(c["x"], c["prev_count"], c["prev_mean"], c["prev_var"], c["gamma"], c["beta"],
+                                   c.get("mask"), int(c["groups"]), 1e-5, np.float32)
+    assert rel_err(y, c["y"]) < 2e-5 and np.array_equal(n, c["count"])
+    assert rel_err(mu, c["mean"]) < 2e-5 and rel_err(v, c["var"]) < 2e-5
+
+
+def test_oracle_c_kernel(gold, oracle_c):
+    import oracle_c_api as OC
+
+    c = _case(gold, "ema")
+    k = OC.ema_kernel(c["p"], c["q"], c["gamma"], int(c["length"]), np.float32)
+    assert rel_err(k, c["kernel"]) < 2e-5
+
+
+# ----------------------------------------------------------------------------------------------
+# HIP library
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", GROUP_CASES)
+def test_hip_group_norm(gold, tag):
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, tag)
+    mask = None if "mask" not in c else torch.from_numpy(c["mask"]).to("cuda:0")
+    y, n, mu, v = M.ops.group_timestep_norm_fwd(dev(c["x"]), dev(c["prev_count"], torch.int64), dev(c["prev_mean"]),
+                                                dev(c["prev_var"]), dev(c["gamma"]), dev(c["beta"]), mask,
+                                                int(c["groups"]), 1e-5)[:4]
+    assert rel_err(host(y), c["y"]) < 1e-4 and np.array_equal(host(n), c["count"])
+    assert rel_err(host(mu), c["mean"]) < 1e-4 and rel_err(host(v), c["var"]) < 1e-4
+
+
+@pytest.mark.gpu
+def test_hip_feature_norm(gold):
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, "tsn")
+    y, n, mu, v = M.ops.timestep_norm_fwd(dev(c["x"]), dev(c["prev_count"], torch.int64), dev(c["prev_mean"]),
+                                          dev(c["prev_var"]), dev(c["gamma"]), dev(c["beta"]),
+                                          torch.from_numpy(c["mask"]).to("cuda:0"), 1e-5)[:4]
+    assert rel_err(host(y), c["y"]) < 1e-4 and np.array_equal(host(n), c["count"])
+    assert rel_err(host(mu), c["mean"]) < 1e-4 and rel_err(host(v), c["var"]) < 1e-4
+
+
+@pytest.mark.gpu
+def test_hip_ema(gold):
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, "ema")
+    L = int(c["length"])
+    w, b, _ = M.ops.ema_parameters_fwd(dev(c["p"]), dev(c["log_q"]), dev(c["gamma"]), dev(c["h"]), L)
+    assert rel_err(host(w), c["kernel"]) < 1e-4 and rel_err(host(b), c["bias"]) < 1e-4
+    hy, _ = M.ops.ema_hidden_fwd(dev(c["x"]), dev(c["p"]), dev(c["log_q"]), dev(c["h"]))
+    assert rel_err(host(hy).real, c["hidden"].real) < 1e-4 and rel_err(host(hy).imag, c["hidden"].imag) < 1e-4
+    hy0, _ = M.ops.ema_hidden_fwd(dev(c["x"]), dev(c["p"]), dev(c["log_q"]), None)
+    assert rel_err(host(hy0).real, c["hidden_zero_start"].real) < 1e-4
+    assert rel_err(host(hy0).imag, c["hidden_zero_start"].imag) < 1e-4
+    # the whole moving-average layer output from the same coefficients: kernel * x + bias
+    omega = np.zeros(c["p"].shape[0], np.float32)
+    y = M.ops.ema_forward(dev(c["x"]), dev(c["p"]), dev(c["q"]), dev(c["gamma"]), dev(omega), h=dev(c["h"]))
+    y = y[0] if isinstance(y, tuple) else y
+    ref = O.causal_conv_direct(c["x"].astype(np.float64), c["kernel"].astype(np.float64)) + c["bias"]
+    assert rel_err(host(y), ref) < 1e-4
