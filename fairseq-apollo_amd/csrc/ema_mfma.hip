@@ -29,6 +29,12 @@
 //   sweep 2: K, P, C products with the true start states; y overwrites x in LDS
 #include "ema_mfma.h"
 
+// Phase markers of the streaming kernel: a profiling build defines MEGA_TR(k) to stamp the
+// shader clock; here they expand to nothing.
+#ifndef MEGA_TR
+#define MEGA_TR(k)
+#endif
+
 namespace mega {
 namespace {
 
@@ -204,9 +210,9 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
                                            __float_as_uint(bq.y));
     img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(c.x), __float_as_uint(c.y), __float_as_uint(d.x),
                                            __float_as_uint(d.y));
-    // scan multiplier q^(32 SEGT) of state `lane & 15`
+    // scan multiplier q^(32 SEGT) of state `lane >> 2`
     cfloat R = {1.f, 0.f};
-    const float2 w = pw[32 * kNS + (lane & 15)];
+    const float2 w = pw[32 * kNS + (lane >> 2)];
     for (int t = 0; t < kSEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
     img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
   }
@@ -240,7 +246,8 @@ struct Geo {
   static constexpr int SEGB = SEG * 2 + 16;        // bytes per segment in an LDS row (padded)
   static constexpr int ROWB = SEGB * 16 + 16;      // bytes per channel row; (ROWB / 4) % 16 == 4
   static constexpr int XBUF = ROWB * kWaves;
-  static constexpr int SCANB = 16 * kNS * 8;       // segment states per channel
+  static constexpr int SCANJ = 20;                 // complex slots per segment in the scan buffer (16 + 4 pad)
+  static constexpr int SCANB = 16 * SCANJ * 8;     // segment states per channel
   static constexpr int TOTAL = XBUF + kWaves * SCANB;
   static_assert((ROWB / 4) % 16 == 4, "row stride must spread the four rows of a store over the banks");
   __device__ static __forceinline__ int pos(int t) { return (t / SEG) * SEGB + (t % SEG) * 2; }
@@ -251,7 +258,11 @@ __device__ __forceinline__ uint32_t dpp_swap2(uint32_t v) {      // lane ^ 2 wit
 }
 
 // LAYOUT 0: [B, D, L] rows contiguous in time; LAYOUT 1: [B, L, D] channels contiguous.
-template <int LAYOUT>
+// FAST: whole super-chunks and whole channel blocks only, no padding mask, no partial sums:
+// every load and store of the streaming loop is unconditional straight-line code, so the
+// stores of one super-chunk stay in flight under the next one's staging and sweeps (with a
+// branch around them the loop has to drain them before it may consume the prefetched loads).
+template <int LAYOUT, bool FAST>
 __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   using G = Geo;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
   }
   const int ch = cb * kWaves + wave;
-  const bool ch_ok = ch < A.D;
+  const bool ch_ok = FAST || ch < A.D;
   const int chc = ch_ok ? ch : A.D - 1;            // idle waves compute on a valid row, never store
   char* xrow = smem + wave * G::ROWB;
   char* scan = smem + G::XBUF + wave * G::SCANB;
@@ -289,6 +300,12 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   // LAYOUT 1: a lane pair (lane, lane ^ 2) covers tokens (2m, 2m+1) x 8 channels (half = lane & 1)
   const int half = tid & 1;
   const int odd = (tid >> 1) & 1;
+  // byte selectors of v_perm_b32 (source bytes 0..3 = second operand, 4..7 = first operand):
+  // staging packs (even token | odd token << 16) per channel, the store unpacks it again
+  const uint32_t sel_lo = odd ? 0x01000504u : 0x05040100u;
+  const uint32_t sel_hi = odd ? 0x03020706u : 0x07060302u;
+  const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
+  const uint32_t sel_give = odd ? 0x05040100u : 0x07060302u;
 
   auto issue_loads = [&](int sc) {
     const int t0 = sc * G::SC;
@@ -299,7 +316,10 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
-        if (tau < A.L && c0 < A.D) {
+        if (FAST) {
+          const int t = A.reverse ? A.L - 1 - tau : tau;
+          pre[k] = *(const uint4*)(xg + b * A.sxb + (int64_t)t * A.sxl + c0);
+        } else if (tau < A.L && c0 < A.D) {
           const int t = A.reverse ? A.L - 1 - tau : tau;
           if (!(A.mask && A.mask[(size_t)b * A.L + t]))
             pre[k] = *(const uint4*)(xg + b * A.sxb + (int64_t)t * A.sxl + c0);
@@ -307,7 +327,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       } else {
         const int tk = k * 512 + lane * 8;
         const int tau = t0 + tk;
-        if (tau < A.L) {
+        if (FAST || tau < A.L) {
           const int t = A.reverse ? A.L - 8 - tau : tau;
           uint4 v = *(const uint4*)(xg + b * A.sxb + (int64_t)chc * A.sxd + t);
           if (A.reverse) {
@@ -318,7 +338,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
             w.w = (v.x >> 16) | (v.x << 16);
             v = w;
           }
-          if (A.mask) {
+          if (!FAST && A.mask) {
             const uint2 mk = *(const uint2*)(A.mask + (size_t)b * A.L + t);
             const uint32_t mm[2] = {mk.x, mk.y};
             uint32_t* vv = (uint32_t*)&v;
@@ -335,13 +355,16 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
   };
 
+  MEGA_TR(0);
   issue_loads(0);
+  MEGA_TR(1);
 
   // ---- operand images of this channel: registers for the whole kernel
   bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
   float Qr[4], Qi[4];
-  float Rr, Ri;
-  float Hcr = 0.f, Hci = 0.f;          // carried state of state `lane` (lanes 0..15)
+  // segment scan: lane (n = lane >> 2, c = lane & 3) owns state n over segments 4c .. 4c+3
+  float Rr, Ri, R2r, R2i, R3r, R3i, R4r, R4i, R8r, R8i;    // powers of q^(32 SEGT); R4/R8 zeroed where unused
+  float Hcr = 0.f, Hci = 0.f;          // carried state of state n, in the lanes with c == 0 (zero elsewhere)
   {
     const uint4* img = A.image + (size_t)(A.koff + chc) * kImgSlots * 64 + lane;
     int slot = 0;
@@ -364,15 +387,23 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     Qr[3] = __uint_as_float(qb.z); Qi[3] = __uint_as_float(qb.w);
     Rr = __uint_as_float(rr.x);
     Ri = __uint_as_float(rr.y);
-    if (A.h_in && lane < A.N && ch_ok) {
-      const size_t o = (((size_t)b * A.D + ch) * A.N + lane) * 2;
+    R2r = Rr * Rr - Ri * Ri; R2i = 2.f * Rr * Ri;
+    R3r = R2r * Rr - R2i * Ri; R3i = R2r * Ri + R2i * Rr;
+    R4r = R2r * R2r - R2i * R2i; R4i = 2.f * R2r * R2i;
+    R8r = R4r * R4r - R4i * R4i; R8i = 2.f * R4r * R4i;
+    if ((lane & 3) < 1) { R4r = 0.f; R4i = 0.f; }     // quarter 0 has no predecessor
+    if ((lane & 3) < 2) { R8r = 0.f; R8i = 0.f; }     // quarters 0, 1 have none two back
+    if (A.h_in && (lane & 3) == 0 && (lane >> 2) < A.N && ch_ok) {
+      const size_t o = (((size_t)b * A.D + ch) * A.N + (lane >> 2)) * 2;
       Hcr = A.h_in[o];
       Hci = A.is_complex ? A.h_in[o + 1] : 0.f;
     }
   }
 
+  MEGA_TR(2);
   for (int sc = 0; sc < nsc; ++sc) {
     const int t0 = sc * G::SC;
+    MEGA_TR(3 + sc * 9);
     // ---- stage the prefetched super-chunk into LDS
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
@@ -382,15 +413,13 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
         const uint4 v = pre[k];
         const uint32_t s0 = odd ? v.x : v.z, s1 = odd ? v.y : v.w;
-        const uint32_t r0 = dpp_swap2(s0), r1 = dpp_swap2(s1);
-        const uint32_t m0 = odd ? v.z : v.x, m1 = odd ? v.w : v.y;
-        const uint32_t e0 = odd ? r0 : m0, e1 = odd ? r1 : m1;      // even token's pair of channels
-        const uint32_t o0 = odd ? m0 : r0, o1 = odd ? m1 : r1;      // odd token's
+        const uint32_t r0 = dpp_swap2(s0), r1 = dpp_swap2(s1);      // the partner's token, my channels
+        const uint32_t m0 = odd ? v.z : v.x, m1 = odd ? v.w : v.y;  // my token, my channels
         uint32_t w[4];
-        w[0] = (e0 & 0xffffu) | (o0 << 16);
-        w[1] = (e0 >> 16) | (o0 & 0xffff0000u);
-        w[2] = (e1 & 0xffffu) | (o1 << 16);
-        w[3] = (e1 >> 16) | (o1 & 0xffff0000u);
+        w[0] = __builtin_amdgcn_perm(r0, m0, sel_lo);
+        w[1] = __builtin_amdgcn_perm(r0, m0, sel_hi);
+        w[2] = __builtin_amdgcn_perm(r1, m1, sel_lo);
+        w[3] = __builtin_amdgcn_perm(r1, m1, sel_hi);
         char* base = smem + (half * 8 + odd * 4) * G::ROWB + G::pos(tk & ~1);
 #pragma unroll
         for (int e = 0; e < 4; ++e) *(uint32_t*)(base + e * G::ROWB) = w[e];
@@ -399,8 +428,11 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         *(uint4*)(xrow + G::pos(tk)) = pre[k];
       }
     }
+    MEGA_TR(4 + sc * 9);
     __syncthreads();
+    MEGA_TR(5 + sc * 9);
     if (sc + 1 < nsc) issue_loads(sc + 1);
+    MEGA_TR(6 + sc * 9);
 
     // ---- sweep 1: segment end states from a zero start
     float Er[4] = {0.f, 0.f, 0.f, 0.f}, Ei[4] = {0.f, 0.f, 0.f, 0.f};
@@ -418,38 +450,71 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const float nr = Qr[u] * Er[u] - Qi[u] * Ei[u] + sr[u];
-        const float ni = Qr[u] * Ei[u] + Qi[u] * Er[u] + si[u];
+        const float nr = fmaf(Qr[u], Er[u], fmaf(-Qi[u], Ei[u], sr[u]));
+        const float ni = fmaf(Qr[u], Ei[u], fmaf(Qi[u], Er[u], si[u]));
         Er[u] = nr;
         Ei[u] = ni;
       }
     }
+    MEGA_TR(7 + sc * 9);
     // ---- scan over the 16 segments (per state), carried across super-chunks
     {
-      float4* sb = (float4*)scan;     // [16 segments][16 states] complex: states (2r, 2r+1) at float4 [j*8 + r]
-      sb[j * 8 + r] = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
-      sb[j * 8 + 4 + r] = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
+      // [16 segments][SCANJ] complex: states (2r, 2r+1) of segment j at float4 [j * SCANJ/2 + r]
+      float4* sb = (float4*)scan;
+      constexpr int J4 = G::SCANJ / 2;
+      sb[j * J4 + r] = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
+      sb[j * J4 + 4 + r] = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_wave_barrier();
-      if (lane < 16) {
-        float2* s2 = (float2*)scan;   // state `lane` of segment jj at s2[jj * 16 + lane]
-        float hr = Hcr, hi = Hci;
+      {
+        const int n = lane >> 2, c = lane & 3;
+        float2* s2 = (float2*)scan + (4 * c) * G::SCANJ + n;
+        float2 e[4];
 #pragma unroll
-        for (int half8 = 0; half8 < 2; ++half8) {
-          float2 e[8];
+        for (int k = 0; k < 4; ++k) e[k] = s2[k * G::SCANJ];
+        // quarter-local exclusive scan (the carry enters quarter 0 here)
+        float ar = Hcr, ai = Hci, outr[4], outi[4];
 #pragma unroll
-          for (int jj = 0; jj < 8; ++jj) e[jj] = s2[(half8 * 8 + jj) * 16 + lane];
-#pragma unroll
-          for (int jj = 0; jj < 8; ++jj) {
-            s2[(half8 * 8 + jj) * 16 + lane] = make_float2(hr, hi);
-            const float nr = Rr * hr - Ri * hi + e[jj].x;
-            const float ni = Rr * hi + Ri * hr + e[jj].y;
-            hr = nr;
-            hi = ni;
-          }
+        for (int k = 0; k < 4; ++k) {
+          outr[k] = ar;
+          outi[k] = ai;
+          const float nr = fmaf(Rr, ar, fmaf(-Ri, ai, e[k].x));
+          const float ni = fmaf(Rr, ai, fmaf(Ri, ar, e[k].y));
+          ar = nr;
+          ai = ni;
         }
-        Hcr = hr;
-        Hci = hi;
+        // inclusive scan of the quarter totals across the quad (multipliers q^(4 seg), q^(8 seg))
+        {
+          const float xr = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ar), 0x90, 0xf, 0xf, false));
+          const float xi = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ai), 0x90, 0xf, 0xf, false));
+          ar = fmaf(R4r, xr, fmaf(-R4i, xi, ar));
+          ai = fmaf(R4r, xi, fmaf(R4i, xr, ai));
+        }
+        {
+          const float xr = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ar), 0x44, 0xf, 0xf, false));
+          const float xi = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ai), 0x44, 0xf, 0xf, false));
+          ar = fmaf(R8r, xr, fmaf(-R8i, xi, ar));
+          ai = fmaf(R8r, xi, fmaf(R8i, xr, ai));
+        }
+        // carry into this quarter = total up to the previous one (quarter 0 already has its own)
+        float cr = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ar), 0x90, 0xf, 0xf, false));
+        float ci = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ai), 0x90, 0xf, 0xf, false));
+        const float tr = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ar), 0xFF, 0xf, 0xf, false));
+        const float ti = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ai), 0xFF, 0xf, 0xf, false));
+        cr = c == 0 ? 0.f : cr;
+        ci = c == 0 ? 0.f : ci;
+        Hcr = c == 0 ? tr : 0.f;
+        Hci = c == 0 ? ti : 0.f;
+        outr[0] += cr;
+        outi[0] += ci;
+        outr[1] = fmaf(Rr, cr, fmaf(-Ri, ci, outr[1]));
+        outi[1] = fmaf(Rr, ci, fmaf(Ri, cr, outi[1]));
+        outr[2] = fmaf(R2r, cr, fmaf(-R2i, ci, outr[2]));
+        outi[2] = fmaf(R2r, ci, fmaf(R2i, cr, outi[2]));
+        outr[3] = fmaf(R3r, cr, fmaf(-R3i, ci, outr[3]));
+        outi[3] = fmaf(R3r, ci, fmaf(R3i, cr, outi[3]));
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s2[k * G::SCANJ] = make_float2(outr[k], outi[k]);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_wave_barrier();
@@ -457,10 +522,12 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     float Hr[4], Hi[4];
     {
       const float4* sb = (const float4*)scan;
-      const float4 a = sb[j * 8 + r], c = sb[j * 8 + 4 + r];
+      constexpr int J4 = G::SCANJ / 2;
+      const float4 a = sb[j * J4 + r], c = sb[j * J4 + 4 + r];
       Hr[0] = a.x; Hi[0] = a.y; Hr[1] = a.z; Hi[1] = a.w;
       Hr[2] = c.x; Hi[2] = c.y; Hr[3] = c.z; Hi[3] = c.w;
     }
+    MEGA_TR(8 + sc * 9);
     // ---- sweep 2: outputs
     char* ycol = xrow + j * G::SEGB;
 #pragma unroll
@@ -493,12 +560,12 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const float nr = Qr[u] * Hr[u] - Qi[u] * Hi[u] + sr[u];
-        const float ni = Qr[u] * Hi[u] + Qi[u] * Hr[u] + si[u];
+        const float nr = fmaf(Qr[u], Hr[u], fmaf(-Qi[u], Hi[u], sr[u]));
+        const float ni = fmaf(Qr[u], Hi[u], fmaf(Qi[u], Hr[u], si[u]));
         Hr[u] = nr;
         Hi[u] = ni;
       }
-      if (A.h_tile && ch_ok) {
+      if (!FAST && A.h_tile && ch_ok) {
         const int gt = (t0 + j * G::SEG + i * 32) >> 5;
         if (gt == last_tile) {
           float* ho = A.h_tile + (((size_t)b * A.D + ch) * kNS) * 2;
@@ -522,7 +589,9 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         *(uint2*)(ycol + i * 64 + 32 + r * 8) = *(const uint2*)o1;
       }
     }
+    MEGA_TR(9 + sc * 9);
     __syncthreads();
+    MEGA_TR(10 + sc * 9);
     // ---- store the super-chunk
     bf16_t* yg = (bf16_t*)A.y;
 #pragma unroll
@@ -536,18 +605,20 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         uint32_t w[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = *(const uint32_t*)(base + e * G::ROWB);
-        // what the partner needs of mine: its token's halves of my four channels, as two dwords
-        const uint32_t give0 = odd ? ((w[0] & 0xffffu) | (w[1] << 16)) : ((w[0] >> 16) | (w[1] & 0xffff0000u));
-        const uint32_t give1 = odd ? ((w[2] & 0xffffu) | (w[3] << 16)) : ((w[2] >> 16) | (w[3] & 0xffff0000u));
-        const uint32_t keep0 = odd ? ((w[0] >> 16) | (w[1] & 0xffff0000u)) : ((w[0] & 0xffffu) | (w[1] << 16));
-        const uint32_t keep1 = odd ? ((w[2] >> 16) | (w[3] & 0xffff0000u)) : ((w[2] & 0xffffu) | (w[3] << 16));
-        const uint32_t got0 = dpp_swap2(give0), got1 = dpp_swap2(give1);
+        // my token's halves of my four channels stay, the partner token's halves go to the partner
+        const uint32_t keep0 = __builtin_amdgcn_perm(w[1], w[0], sel_keep);
+        const uint32_t keep1 = __builtin_amdgcn_perm(w[3], w[2], sel_keep);
+        const uint32_t got0 = dpp_swap2(__builtin_amdgcn_perm(w[1], w[0], sel_give));
+        const uint32_t got1 = dpp_swap2(__builtin_amdgcn_perm(w[3], w[2], sel_give));
         uint4 o;     // channels c0 .. c0+7 of token tk
         o.x = odd ? got0 : keep0;
         o.y = odd ? got1 : keep1;
         o.z = odd ? keep0 : got0;
         o.w = odd ? keep1 : got1;
-        if (tau < A.L && c0 < A.D) {
+        if (FAST) {
+          const int t = A.reverse ? A.L - 1 - tau : tau;
+          *(uint4*)(yg + b * A.syb + (int64_t)t * A.syl + c0) = o;
+        } else if (tau < A.L && c0 < A.D) {
           const int t = A.reverse ? A.L - 1 - tau : tau;
           const bool direct = !A.acc_in && !A.acc_out && !(A.mask && A.omega);
           if (direct) {
@@ -583,7 +654,19 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       } else {
         const int tk = k * 512 + lane * 8;
         const int tau = t0 + tk;
-        if (tau < A.L && ch_ok) {
+        if (FAST) {
+          const int t = A.reverse ? A.L - 8 - tau : tau;
+          uint4 v = *(const uint4*)(xrow + G::pos(tk));
+          if (A.reverse) {
+            uint4 w;
+            w.x = (v.w >> 16) | (v.w << 16);
+            w.y = (v.z >> 16) | (v.z << 16);
+            w.z = (v.y >> 16) | (v.y << 16);
+            w.w = (v.x >> 16) | (v.x << 16);
+            v = w;
+          }
+          *(uint4*)(yg + b * A.syb + (int64_t)ch * A.syd + t) = v;
+        } else if (tau < A.L && ch_ok) {
           const int t = A.reverse ? A.L - 8 - tau : tau;       // first physical token of the 8
           Vec<bf16_t, 8> in = *(const Vec<bf16_t, 8>*)(xrow + G::pos(tk));
           float v[8];
@@ -615,7 +698,15 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         }
       }
     }
+    MEGA_TR(11 + sc * 9);
     __syncthreads();
+  }
+  MEGA_TR(3 + nsc * 9);
+  if (FAST && A.h_tile && (lane & 3) == 0) {
+    // L is a whole number of super-chunks: the carried scan state is the state at time L
+    float* ho = A.h_tile + (((size_t)b * A.D + ch) * kNS + (lane >> 2)) * 2;
+    ho[0] = Hcr;
+    ho[1] = Hci;
   }
 }
 
@@ -687,12 +778,15 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
   A.sad = layout == 1 ? 1 : L;
   A.sal = layout == 1 ? D : 1;
   const dim3 grid((unsigned)(B * ncb));
+  const bool fast = !bidirectional && !mask && L % G::SC == 0 && D % kWaves == 0;
   auto launch = [&](const MfmaArgs& a) -> int {
-    auto kern = layout == 1 ? ema_mfma_kernel<1> : ema_mfma_kernel<0>;
-    static bool attr_set[2] = {false, false};
-    if (!attr_set[layout]) {
+    auto kern = layout == 1 ? (fast ? ema_mfma_kernel<1, true> : ema_mfma_kernel<1, false>)
+                            : (fast ? ema_mfma_kernel<0, true> : ema_mfma_kernel<0, false>);
+    static bool attr_set[4] = {false, false, false, false};
+    const int ki = layout * 2 + (fast ? 1 : 0);
+    if (!attr_set[ki]) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
-      attr_set[layout] = true;
+      attr_set[ki] = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(kThreadsM), G::TOTAL, s, a);
     MEGA_CHECK_LAUNCH("ema_fwd (matrix-core path)");
