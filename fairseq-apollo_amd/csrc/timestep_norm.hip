@@ -21,6 +21,11 @@
 //   address is hit by one atomic per workgroup on the way in.
 #include "common.h"
 
+// Phase markers: a profiling build defines MEGA_TSN_TR(k) to stamp a clock; no-ops here.
+#ifndef MEGA_TSN_TR
+#define MEGA_TSN_TR(k)
+#endif
+
 namespace mega {
 
 namespace {
@@ -190,6 +195,22 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   const V* xin = (const V*)P.x + ((size_t)b * P.L + t0) * TPT;
   V* yout = (V*)P.y + ((size_t)b * P.L + t0) * TPT;
 
+  MEGA_TSN_TR(0);
+  // ---- everything the tail of the kernel needs from global memory is requested up front, so
+  // that no cold miss sits between the look-back and the stores: the prior state of the first
+  // 16 groups and the affine parameters of this thread's features
+  const int row16 = tid >> 4, l16 = tid & 15;
+  const int gfirst = row16 < G ? row16 : G - 1;
+  const Moments prior0 = {(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gfirst], P.prev_var[(size_t)b * G + gfirst]};
+  float gam[VEC], bet[VEC];
+  if (HOIST) {
+    const int f0 = (tid % TPT) * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      gam[i] = P.gamma[f0 + i];
+      bet[i] = P.beta[f0 + i];
+    }
+  }
   // ---- load the tile (one contiguous block) and the mask bytes
   V xv[kNV];
 #pragma unroll
@@ -296,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   // row scans across lanes and publishes the tile aggregate.  The aggregates of the earlier tiles of
   // this batch row are then fetched as one contiguous block into LDS (every word says by itself
   // whether it has been published: no fence on either side) and folded into the carry-in.
-  const int row16 = tid >> 4, l16 = tid & 15;
+  MEGA_TSN_TR(1);
   const int TPL = (P.TT + 15) >> 4;                 // tokens per lane (<= 4)
   const size_t trow = (size_t)b * P.ntiles;
   const bool last_tile = tile == P.ntiles - 1;
@@ -327,6 +348,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(inc.var), tag));
       if (g == 0) put_rec(mine, tagged((uint32_t)inc.n, tag));
     }
+    MEGA_TSN_TR(2);
     // earlier tiles, RT per round
     Moments acc = {0.f, 0.f, 0.f};
     uint32_t prevcnt = 0;
@@ -373,9 +395,11 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
         prevcnt += c;
       }
     }
+    MEGA_TSN_TR(3);
     acc = row_reduce(acc);
     const uint32_t prevtot = row_sum_u32(prevcnt);    // the lanes hold disjoint sets of earlier tiles
-    const Moments prior = {(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gc], P.prev_var[(size_t)b * G + gc]};
+    Moments prior = prior0;
+    if (gbase != 0) prior = Moments{(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gc], P.prev_var[(size_t)b * G + gc]};
     const Moments carry = merge(prior, acc);
     const Moments base = merge(carry, exc);
 #pragma unroll
@@ -399,17 +423,9 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     }
   }
   __syncthreads();
+  MEGA_TSN_TR(4);
 
   // ---- normalise and store
-  float gam[VEC], bet[VEC];
-  if (HOIST) {
-    const int f0 = (tid % TPT) * VEC;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      gam[i] = P.gamma[f0 + i];
-      bet[i] = P.beta[f0 + i];
-    }
-  }
 #pragma unroll
   for (int j = 0; j < kNV; ++j) {
     const int v = j * kThreads + tid;
@@ -439,6 +455,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     }
   }
 
+  MEGA_TSN_TR(5);
   // ---- retire: the last workgroup to finish opens the next epoch (two-level count so that no
   // single address sees one atomic per workgroup)
   if (tid == 0) {
