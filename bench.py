@@ -77,6 +77,19 @@ def cpu_baseline(params, x_bf16_as_f32, threads):
             "sample": f"the full B{B}xL{L}xD{D} block, median of {len(times)} runs ({t * 1e3:.0f} ms each)"}
 
 
+def measured_traffic():
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE / WRITE_SIZE scaled
+    by a plain copy of known size): lines `traffic_bytes_per_launch <kernel> = <bytes>`."""
+    import re
+
+    out = {}
+    path = os.path.join(ROOT, "profiles", "ema_tsn_block_B4_L4096_D1024_bf16.txt")
+    if os.path.exists(path):
+        for m in re.finditer(r"^traffic_bytes_per_launch\s+(\S+)\s*=\s*(\d+)", open(path).read(), re.M):
+            out[m.group(1)] = int(m.group(2))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,20 +149,23 @@ def main():
         gpu_ms = e0.elapsed_time(e1)
         ms_per_step = max(wall * 1e3, gpu_ms) / args.steps
 
-        # per-operator device time (events on the launch stream around each call)
+        # per-operator device time: HIP events on the launch stream around a run of back-to-back
+        # calls (the queue never drains, so the quotient is the kernel's launch-to-launch period)
         def timed(fn, reps):
-            evs = []
-            for i in range(reps):
-                a = torch.cuda.Event(enable_timing=True)
-                b = torch.cuda.Event(enable_timing=True)
-                arg = fn.prep(i)
-                a.record()
-                fn(arg)
-                b.record()
-                evs.append((a, b))
+            args_ = [fn.prep(i) for i in range(reps)]
+            for i in range(min(reps, 8)):
+                fn(args_[i])
             torch.cuda.synchronize()
-            ts = sorted(a.elapsed_time(b) for a, b in evs)
-            return sum(ts) / len(ts), ts[len(ts) // 2]
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            h0 = time.perf_counter()
+            a.record()
+            for i in range(reps):
+                fn(args_[i])
+            b.record()
+            host = time.perf_counter() - h0
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps, host * 1e3 / reps
 
         class NormCall:
             @staticmethod
@@ -170,8 +186,8 @@ def main():
                 return ema(x)
 
         reps = max(20, min(args.steps, 200))
-        norm_avg, norm_med = timed(NormCall(), reps)
-        ema_avg, ema_med = timed(EmaCall(), reps)
+        norm_avg, norm_host = timed(NormCall(), reps)
+        ema_avg, ema_host = timed(EmaCall(), reps)
         if args.copy_calibration:
             dst = torch.empty_like(xs[0])
             for i in range(args.copy_calibration):
@@ -179,6 +195,7 @@ def main():
             torch.cuda.synchronize()
     status = M.ops.timestep_norm_status()
 
+    traffic = measured_traffic()
     tokens = B * L
     alg_bytes_block = 4 * B * L * D * 2          # norm: read x, write xn; EMA: read xn, write y
     alg_bytes_ema = 2 * B * L * D * 2
@@ -204,12 +221,12 @@ def main():
         "block_hbm_gbs": alg_bytes_block / (ms_per_step * 1e-3) / 1e9,
         "block_hbm_frac": alg_bytes_block / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "kernel": "ema_fwd (every launch of one call)", "achieved": ema_gbs,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg, "median_ms": ema_med},
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS, "traffic": traffic.get("ema_mfma_kernel"),
+                     "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg, "host_enqueue_ms": ema_host},
         "roofline_timestep_norm": {"bound": "hbm", "kernel": "group_tsn_kernel", "achieved": norm_gbs,
                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": norm_gbs / HBM_PEAK_GBS,
                                    "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg,
-                                   "median_ms": norm_med},
+                                   "host_enqueue_ms": norm_host, "traffic": traffic.get("group_tsn_kernel")},
         "timestep_norm_status": status,
     }
     if not args.no_cpu:

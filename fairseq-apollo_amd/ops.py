@@ -44,11 +44,35 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
-def _stream(dev: torch.device):
-    return torch.cuda.current_stream(dev).cuda_stream
+def _stream(dev: torch.device) -> int:
+    """Raw handle of torch's current stream on `dev` (the launch stream of every call)."""
+    return torch._C._cuda_getCurrentRawStream(dev.index)
+
+
+class _on_device:
+    """`with _on_device(dev):` makes `dev` the current HIP device for the launch; free when it
+    already is (the usual case: one process per GPU)."""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, dev: torch.device):
+        self.idx = dev.index
+        self.prev = -1
+
+    def __enter__(self):
+        cur = torch._C._cuda_getDevice()
+        if cur != self.idx:
+            self.prev = cur
+            torch._C._cuda_setDevice(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch._C._cuda_setDevice(self.prev)
+        return False
 
 
 def _f32c(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype is torch.float32 and not t.requires_grad and t.is_contiguous():
+        return t
     return t.detach().to(torch.float32).contiguous()
 
 
@@ -63,10 +87,10 @@ def _cplx_as_f32(t: torch.Tensor) -> torch.Tensor:
 _tsn_ws = {}
 
 
-def _tsn_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+def _tsn_workspace(dev: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
     """Zero-filled once, then owned by the TimestepNorm calls (launch epoch + tile records); one per
     (device, stream)."""
-    key = (dev.index, _stream(dev))
+    key = (dev.index, _stream(dev) if stream is None else stream)
     ws = _tsn_ws.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
@@ -77,10 +101,10 @@ def _tsn_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
 _scratch = {}
 
 
-def _scratch_buffer(dev: torch.device, nbytes: int) -> torch.Tensor:
+def _scratch_buffer(dev: torch.device, nbytes: int, stream: Optional[int] = None) -> torch.Tensor:
     """Grow-only scratch per (device, stream): calls on one stream are ordered, so they can
     share it; its contents never need to survive a call."""
-    key = (dev.index, _stream(dev))
+    key = (dev.index, _stream(dev) if stream is None else stream)
     ws = _scratch.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
@@ -121,7 +145,7 @@ def ema_parameters_fwd(p: torch.Tensor, log_q: torch.Tensor, gamma: torch.Tensor
         B = h.shape[0]
         hb = _cplx_as_f32(h.reshape(B, K, N))
         b = torch.empty(B, K, L, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_ema_parameters_fwd(_ptr(pf), _ptr(lq), _ptr(g), _ptr(hb), B, K, N, L, _ptr(w), _ptr(b),
                                          _stream(dev))
     _lib.check(rc, "ema_parameters_fwd")
@@ -142,7 +166,7 @@ def ema_hidden_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, h: Opt
     nws = lib.mega_ema_hidden_workspace_bytes(B, D, N, L)
     ws = torch.empty(nws, dtype=torch.uint8, device=dev)
     xd = x.detach()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_ema_hidden_fwd(_ptr(xd), _dtype_code(xd), xd.stride(0), xd.stride(1), xd.stride(2), _ptr(pf),
                                      _ptr(lq), _ptr(hb), B, D, N, L, _ptr(out), _ptr(ws), nws, _stream(dev))
     _lib.check(rc, "ema_hidden_fwd")
@@ -150,10 +174,17 @@ def ema_hidden_fwd(x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor, h: Opt
 
 
 def _norm_state(prev_count, prev_mean, prev_var, B, G, dev):
-    pc = prev_count.detach().to(device=dev, dtype=torch.int64).contiguous()
-    pm = _f32c(prev_mean).reshape(B, G)
-    pv = _f32c(prev_var).reshape(B, G)
+    pc = prev_count
+    if not (pc.dtype is torch.int64 and pc.device == dev and pc.is_contiguous()):
+        pc = pc.detach().to(device=dev, dtype=torch.int64).contiguous()
+    pm = _f32c(prev_mean)
+    pv = _f32c(prev_var)
+    if pm.numel() != B * G or pv.numel() != B * G or pc.numel() != B:
+        raise RuntimeError(f"carried state must hold {B} counts and {B}x{G} means / variances")
     return pc, pm, pv
+
+
+_ws_bytes_cache = {}
 
 
 def _mask_u8(mask: Optional[torch.Tensor], B: int, L: int):
@@ -181,7 +212,7 @@ def group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, pad
     G = int(num_groups)
     if G <= 0 or H % G != 0:
         raise RuntimeError(f"num_features={H} is not divisible by num_groups={G}")
-    xd = x.detach().contiguous()
+    xd = x if (x.is_contiguous() and not x.requires_grad) else x.detach().contiguous()
     dt = _dtype_code(xd)
     y = torch.empty_like(xd)
     pc, pm, pv = _norm_state(prev_count, prev_mean, prev_var, B, G, dev)
@@ -193,14 +224,18 @@ def group_timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, pad
         gm = torch.empty(B, L, G, dtype=torch.float32, device=dev)
         cm = torch.empty_like(gm)
         cr = torch.empty_like(gm)
-    nws = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, G)
-    ws = _tsn_workspace(dev, nws)
+    key = ("tsn", dt, B, L, H, G)
+    nws = _ws_bytes_cache.get(key)
+    if nws is None:
+        nws = _ws_bytes_cache[key] = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, G)
+    stream = _stream(dev)
+    ws = _tsn_workspace(dev, nws, stream)
     m8 = _mask_u8(padding_mask, B, L)
     gf, bf = _f32c(gamma), _f32c(beta)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_group_timestep_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf),
                                               _ptr(m8), B, L, H, G, float(eps), _ptr(count), _ptr(mean), _ptr(var),
-                                              _ptr(gm), _ptr(cm), _ptr(cr), _ptr(ws), ws.numel(), _stream(dev))
+                                              _ptr(gm), _ptr(cm), _ptr(cr), _ptr(ws), ws.numel(), stream)
     _lib.check(rc, "group_timestep_norm_fwd")
     return y, count, mean, var, gm, cm, cr
 
@@ -225,7 +260,7 @@ def timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_m
         cr = torch.empty_like(cm)
     m8 = _mask_u8(padding_mask, B, L)
     gf, bf = _f32c(gamma), _f32c(beta)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_timestep_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf),
                                         _ptr(m8), B, L, H, float(eps), _ptr(count), _ptr(mean), _ptr(var), _ptr(cm),
                                         _ptr(cr), None, 0, _stream(dev))
@@ -245,7 +280,7 @@ def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool
     outer, inner = xd.shape[-2], xd.shape[-1]
     batch = xd.numel() // max(outer * inner, 1)
     y = torch.empty_like(xd)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_attention_softmax_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), batch, outer, inner,
                                             1 if use_causal_mask else 0, _stream(dev))
     _lib.check(rc, "attention_softmax_fwd")
@@ -270,7 +305,7 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
     w = torch.empty(B, Nh, L, L, dtype=qd.dtype, device=dev) if need_weights else None
     nws = lib.mega_attention_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2)
     ws = _scratch_buffer(dev, nws) if nws else None
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_attention_fwd(_ptr(qd), _ptr(kd), _ptr(vd), _ptr(y), _ptr(w), _dtype_code(qd), B, L, Nh, H1, H2,
                                     float(scale), 1 if use_causal_mask else 0, _ptr(ws), ws.numel() if nws else 0,
                                     _stream(dev))
@@ -309,7 +344,7 @@ class PreparedEMA:
         nimg = lib.mega_ema_image_bytes(self.D, self.N, 1 if self.bidirectional else 0)
         if nimg > 0:
             self.image = torch.empty(nimg, dtype=torch.uint8, device=self.dev)
-            with torch.cuda.device(self.dev):
+            with _on_device(self.dev):
                 rc = lib.mega_ema_prepare(_ptr(self.p), _ptr(self.q), _ptr(self.gamma), 1 if self.is_complex else 0,
                                           _ptr(self.omega), self.D, self.N, 1 if self.bidirectional else 0,
                                           1 if self.shift else 0, _ptr(self.image), nimg, _stream(self.dev))
@@ -342,14 +377,19 @@ class PreparedEMA:
         N = self.N
         hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
         hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev) if (want_state or h is not None) else None
-        nws = lib.mega_ema_fwd_workspace_bytes(B, D, N, L, 1 if self.bidirectional else 0, self.trunc)
-        ws = _scratch_buffer(dev, nws)
-        with torch.cuda.device(dev):
+        key = ("ema", B, D, N, L, self.bidirectional, self.trunc)
+        nws = _ws_bytes_cache.get(key)
+        if nws is None:
+            nws = _ws_bytes_cache[key] = lib.mega_ema_fwd_workspace_bytes(B, D, N, L, 1 if self.bidirectional else 0,
+                                                                         self.trunc)
+        stream = _stream(dev)
+        ws = _scratch_buffer(dev, nws, stream)
+        with _on_device(dev):
             rc = lib.mega_ema_fwd(_ptr(xd), _ptr(y), dt, xd.stride(0), xd.stride(1), xd.stride(2), y.stride(0),
                                   y.stride(1), y.stride(2), _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
                                   1 if self.is_complex else 0, _ptr(self.omega), _ptr(m8), _ptr(hin), _ptr(hout),
                                   B, D, N, L, 1 if self.bidirectional else 0, self.trunc, 1 if self.shift else 0,
-                                  _ptr(self.image), _ptr(ws), ws.numel(), _stream(dev))
+                                  _ptr(self.image), _ptr(ws), ws.numel(), stream)
         _lib.check(rc, "ema_fwd")
         hc = None
         if hout is not None:
@@ -401,7 +441,7 @@ def ema_step(x_t: torch.Tensor, p, q, gamma, omega, h: Optional[torch.Tensor]):
     of = _f32c(omega).reshape(D)
     hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
     hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_ema_step(_ptr(xd), _ptr(y), _dtype_code(xd), _ptr(pf), _ptr(qf), _ptr(gf),
                                1 if is_complex else 0, _ptr(of), _ptr(hin), _ptr(hout), B, D, N, _stream(dev))
     _lib.check(rc, "ema_step")
@@ -436,7 +476,7 @@ class DecodeStep:
         xd = x_t.detach().contiguous()
         xn = torch.empty_like(xd)
         y = torch.empty_like(xd)
-        with torch.cuda.device(self.dev):
+        with _on_device(self.dev):
             rc = lib.mega_norm_ema_step(_ptr(xd), _ptr(xn), _ptr(y), _dtype_code(xd), _ptr(self.count), _ptr(self.mean),
                                         _ptr(self.var), _ptr(self.count), _ptr(self.mean), _ptr(self.var), _ptr(self.nw),
                                         _ptr(self.nb), self.eps, _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
@@ -471,7 +511,7 @@ def _long_conv(x, k, bidirectional, shift):
         raise RuntimeError("kernel rows do not match the channel count")
     Lk = kf.shape[1]
     y = torch.empty_like(xd)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_long_conv_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), _ptr(kf), B, D, L, Lk,
                                     1 if bidirectional else 0, 1 if shift else 0, _stream(dev))
     _lib.check(rc, "long_conv_fwd")
@@ -486,7 +526,7 @@ def swiglu(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         raise RuntimeError("swiglu: a and b must have the same shape and dtype")
     ad, bd = a.detach().contiguous(), b.detach().contiguous()
     y = torch.empty_like(ad)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.mega_swiglu_fwd(_ptr(ad), _ptr(bd), _ptr(y), _dtype_code(ad), ad.numel(), _stream(dev))
     _lib.check(rc, "swiglu_fwd")
     return y
