@@ -4,8 +4,9 @@ bf16 activations, fp32 parameters and accumulation, on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step = one forward of the block over one batch of synthetic input that already sits in
-HBM: xn = TimestepNorm(x) ([B, L, D], 16 groups), y = CEMA(xn^T) read and written in the same
-[B, L, D] memory layout.  Inputs rotate over several buffers so that a step never finds its
+HBM: xn = TimestepNorm(x) ([B, L, D], 16 groups), y = CEMA(xn^T): xn is read in place through the
+transposed view the layer passes, y is the contiguous [B, D, L] tensor the reference's
+convolution returns.  Inputs rotate over several buffers so that a step never finds its
 input in the 256 MB last-level cache.  Prints one JSON line (tokens/s of the whole job), with
 the HBM roofline of the dominant kernel and the CPU oracle timed on the host cores beside it.
 """

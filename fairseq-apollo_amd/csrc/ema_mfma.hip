@@ -257,12 +257,14 @@ __device__ __forceinline__ uint32_t dpp_swap2(uint32_t v) {      // lane ^ 2 wit
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true);
 }
 
-// LAYOUT 0: [B, D, L] rows contiguous in time; LAYOUT 1: [B, L, D] channels contiguous.
+// Layouts (LIN of x, LOUT of y, independent): 0 = [B, D, L] rows contiguous in time, 1 = [B, L, D]
+// channels contiguous.  LIN 1 / LOUT 0 reads the transposed view the layer passes and writes the
+// rows the reference's convolution returns (rfft / irfft output, fused_ops/fftconv.py:45-61).
 // FAST: whole super-chunks and whole channel blocks only, no padding mask, no partial sums:
 // every load and store of the streaming loop is unconditional straight-line code, so the
 // stores of one super-chunk stay in flight under the next one's staging and sweeps (with a
 // branch around them the loop has to drain them before it may consume the prefetched loads).
-template <int LAYOUT, bool FAST>
+template <int LIN, int LOUT, bool FAST>
 __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   using G = Geo;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   constexpr int NLD = G::SC * 2 * kWaves / (kThreadsM * 16);   // 16-byte pieces per thread per super-chunk
   uint4 pre[NLD];
   const bf16_t* xg = (const bf16_t*)A.x;
-  // LAYOUT 1: a lane pair (lane, lane ^ 2) covers tokens (2m, 2m+1) x 8 channels (half = lane & 1)
+  // layout 1: a lane pair (lane, lane ^ 2) covers tokens (2m, 2m+1) x 8 channels (half = lane & 1)
   const int half = tid & 1;
   const int odd = (tid >> 1) & 1;
   // byte selectors of v_perm_b32 (source bytes 0..3 = second operand, 4..7 = first operand):
@@ -312,7 +314,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
       pre[k] = make_uint4(0, 0, 0, 0);
-      if (LAYOUT == 1) {
+      if (LIN == 1) {
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
@@ -407,7 +409,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     // ---- stage the prefetched super-chunk into LDS
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
-      if (LAYOUT == 1) {
+      if (LIN == 1) {
         // pair exchange: the even-token lane ends up with channels 0..3 of both tokens, the
         // odd-token lane with channels 4..7, each as dwords (even token | odd token << 16)
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
@@ -590,13 +592,14 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       }
     }
     MEGA_TR(9 + sc * 9);
-    __syncthreads();
+    if (LOUT == 1) __syncthreads();      // the channel-contiguous store reads every wave's row; a
+                                         // time-contiguous one only the wave's own
     MEGA_TR(10 + sc * 9);
     // ---- store the super-chunk
     bf16_t* yg = (bf16_t*)A.y;
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
-      if (LAYOUT == 1) {
+      if (LOUT == 1) {
         const int tk = k * (kThreadsM / 2) + (tid >> 1);
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
@@ -635,9 +638,9 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
             }
             if (A.mask && A.omega && A.mask[(size_t)b * A.L + t]) {
               // the residual uses the unmasked input (base_moving_average.py:138)
-              const bf16_t* xo = xg + b * A.sxb + (int64_t)t * A.sxl + c0;
+              const bf16_t* xo = xg + b * A.sxb + (int64_t)t * A.sxl + (int64_t)c0 * A.sxd;
 #pragma unroll
-              for (int e = 0; e < 8; ++e) v[e] += A.omega[c0 + e] * to_float(xo[e]);
+              for (int e = 0; e < 8; ++e) v[e] += A.omega[c0 + e] * to_float(xo[e * A.sxd]);
             }
             if (A.acc_out) {
               float* ao = A.acc_out + b * A.sab + (int64_t)t * A.sal + c0;
@@ -679,11 +682,11 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
           }
           if (A.mask && A.omega) {
             const uint8_t* mk = A.mask + (size_t)b * A.L + t;
-            const bf16_t* xo = xg + b * A.sxb + (int64_t)ch * A.sxd + t;
+            const bf16_t* xo = xg + b * A.sxb + (int64_t)ch * A.sxd + (int64_t)t * A.sxl;
             const float om = A.omega[ch];
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-              if (mk[e]) v[e] += om * to_float(xo[e]);
+              if (mk[e]) v[e] += om * to_float(xo[e * A.sxl]);
           }
           if (A.acc_out) {
             float* ao = A.acc_out + b * A.sab + (int64_t)ch * A.sad + t;
@@ -742,6 +745,14 @@ __global__ void ema_state_tail_kernel(const T* __restrict__ x, int64_t sxb, int6
 
 }  // namespace
 
+// Memory layout of one side of the call: 1 = channels contiguous (16-byte pieces of 8 channels),
+// 0 = time contiguous (pieces of 8 tokens), -1 = neither (the generic path takes it).
+static int side_layout(int64_t sb, int64_t sd, int64_t sl, int64_t D, int64_t L) {
+  if (sd == 1 && D % 8 == 0 && sl % 8 == 0 && sb % 8 == 0) return 1;
+  if (sl == 1 && L % 8 == 0 && sd % 8 == 0 && sb % 8 == 0) return 0;
+  return -1;
+}
+
 size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional) {
   if (N > kNS || D <= 0) return 0;
   return (size_t)(bidirectional ? 2 * D : D) * kImgRowBytes;
@@ -765,25 +776,29 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
                  const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
                  int64_t N, int64_t L, int bidirectional, int64_t Lk, float* acc, float* h_tile, hipStream_t s) {
   if (!ema_mfma_covers(dtype, sxb, sxd, sxl, syb, syd, syl, x, y, mask, B, D, N, L, Lk)) return 0;
-  const int layout = (sxd == 1 && syd == 1) ? 1 : 0;
+  const int lin = side_layout(sxb, sxd, sxl, D, L), lout = side_layout(syb, syd, syl, D, L);
   using G = Geo;
   const int ncb = (int)ceil_div(D, kWaves);
   MfmaArgs A;
   A.x = x; A.y = y; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.syb = syb; A.syd = syd; A.syl = syl;
   A.image = (const uint4*)image; A.mask = mask;
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L; A.is_complex = is_complex;
-  A.xcd_map = (layout == 1 && ncb % 4 == 0 && ((B * ncb) % 32) == 0) ? 1 : 0;
+  A.xcd_map = ((lin == 1 || lout == 1) && ncb % 4 == 0 && ((B * ncb) % 32) == 0) ? 1 : 0;
   // fp32 partial sums between the two directions live in [B, D, L]-shaped storage with y's layout
-  A.sab = layout == 1 ? L * D : D * L;
-  A.sad = layout == 1 ? 1 : L;
-  A.sal = layout == 1 ? D : 1;
+  A.sab = lout == 1 ? L * D : D * L;
+  A.sad = lout == 1 ? 1 : L;
+  A.sal = lout == 1 ? D : 1;
   const dim3 grid((unsigned)(B * ncb));
   const bool fast = !bidirectional && !mask && L % G::SC == 0 && D % kWaves == 0;
   auto launch = [&](const MfmaArgs& a) -> int {
-    auto kern = layout == 1 ? (fast ? ema_mfma_kernel<1, true> : ema_mfma_kernel<1, false>)
-                            : (fast ? ema_mfma_kernel<0, true> : ema_mfma_kernel<0, false>);
-    static bool attr_set[4] = {false, false, false, false};
-    const int ki = layout * 2 + (fast ? 1 : 0);
+    typedef void (*Kern)(const MfmaArgs);
+    static const Kern table[8] = {
+        ema_mfma_kernel<0, 0, false>, ema_mfma_kernel<0, 0, true>, ema_mfma_kernel<0, 1, false>,
+        ema_mfma_kernel<0, 1, true>,  ema_mfma_kernel<1, 0, false>, ema_mfma_kernel<1, 0, true>,
+        ema_mfma_kernel<1, 1, false>, ema_mfma_kernel<1, 1, true>};
+    static bool attr_set[8] = {false, false, false, false, false, false, false, false};
+    const int ki = lin * 4 + lout * 2 + (fast ? 1 : 0);
+    const Kern kern = table[ki];
     if (!attr_set[ki]) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
       attr_set[ki] = true;
@@ -818,11 +833,9 @@ bool ema_mfma_covers(int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t s
                      const void* x, const void* y, const uint8_t* mask, int64_t B, int64_t D, int64_t N, int64_t L,
                      int64_t Lk) {
   if (dtype != MEGA_BF16 || N > kNS || Lk > 0 || L < 256) return false;
-  int layout;
-  if (sxd == 1 && syd == 1 && D % 8 == 0 && sxl % 8 == 0 && syl % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 1;
-  else if (sxl == 1 && syl == 1 && L % 8 == 0 && sxd % 8 == 0 && syd % 8 == 0 && sxb % 8 == 0 && syb % 8 == 0) layout = 0;
-  else return false;
-  if (((uintptr_t)x % 16) || ((uintptr_t)y % 16) || (mask && layout == 0 && ((uintptr_t)mask % 8))) return false;
+  const int lin = side_layout(sxb, sxd, sxl, D, L), lout = side_layout(syb, syd, syl, D, L);
+  if (lin < 0 || lout < 0) return false;
+  if (((uintptr_t)x % 16) || ((uintptr_t)y % 16) || (mask && lin == 0 && ((uintptr_t)mask % 8))) return false;
   if (B * ceil_div(D, kWaves) >= (int64_t)1 << 31) return false;
   return true;
 }

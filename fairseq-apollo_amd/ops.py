@@ -352,7 +352,11 @@ class PreparedEMA:
 
     def __call__(self, x: torch.Tensor, padding_mask: Optional[torch.Tensor] = None,
                  h: Optional[torch.Tensor] = None, want_state: bool = False,
-                 out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                 out: Optional[torch.Tensor] = None, out_layout: str = "rows"
+                 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """x: [B, D, L] with any strides.  The result is a contiguous [B, D, L] tensor (rows in time, what
+        the reference's convolution returns, fused_ops/fftconv.py:45-61) unless `out` is given or
+        out_layout == "input" asks for x's own strides."""
         dev = self.dev
         _need_gpu(x, padding_mask, h)
         lib = _lib.load()
@@ -369,10 +373,12 @@ class PreparedEMA:
             y = out
             if y.shape != xd.shape or y.dtype != xd.dtype:
                 raise RuntimeError("out must match x in shape and dtype")
-        elif _dense(xd):
+        elif out_layout == "input" and _dense(xd):
             y = torch.empty_strided(xd.shape, xd.stride(), dtype=xd.dtype, device=dev)
+        elif out_layout in ("rows", "input"):
+            y = torch.empty(xd.shape, dtype=xd.dtype, device=dev)
         else:
-            y = torch.empty_like(xd, memory_format=torch.contiguous_format)
+            raise RuntimeError(f"out_layout must be 'rows' or 'input', got {out_layout!r}")
         m8 = _mask_u8(padding_mask, B, L)
         N = self.N
         hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
@@ -400,16 +406,18 @@ class PreparedEMA:
 def ema_forward(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, omega: torch.Tensor,
                 padding_mask: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
                 want_state: bool = False, bidirectional: bool = False, truncation: Optional[int] = None,
-                shift: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                shift: bool = True, out_layout: str = "rows") -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Whole moving-average layer in one call (BaseMovingLayer.forward,
     fairseq/modules/base_moving_average.py:120-172).
 
     x: [B, D, L] (any strides; a transposed view of a [B, L, D] tensor is read in place);
     p: [K, N]; q, gamma: [K, N] real or complex; omega: [D]; h: [B, D, N] carried state.
-    Returns (y, h') with y shaped [B, D, L] in x's memory layout and h' complex64 (or None).
+    Returns (y, h') with y a contiguous [B, D, L] tensor (out_layout="input": x's strides) and h'
+    complex64 (or None).
     """
     _need_gpu(x)
-    return PreparedEMA(p, q, gamma, omega, bidirectional, truncation, shift)(x, padding_mask, h, want_state)
+    return PreparedEMA(p, q, gamma, omega, bidirectional, truncation, shift)(x, padding_mask, h, want_state,
+                                                                            out_layout=out_layout)
 
 
 def _dense(t: torch.Tensor) -> bool:

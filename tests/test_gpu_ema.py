@@ -50,7 +50,7 @@ def test_time_major_layout_and_mask(dtype):
     xt, x64t = rounded(rng.normal(size=(B, L, D)), dtype)
     mask = np.zeros((B, L), bool); mask[0, 250:] = True; mask[1, 17] = True
     y, _ = _run(xt.transpose(1, 2), p, q, g, om, padding_mask=dev(mask, torch.bool))
-    assert y.shape == (B, D, L) and y.transpose(1, 2).is_contiguous()
+    assert y.shape == (B, D, L) and y.is_contiguous()      # the reference's convolution output layout
     yo, _ = O.ema_forward(x64t.transpose(0, 2, 1), p, q, g, om, mask)
     assert rel_err(host(y), yo) < TOL[dtype]
 

@@ -28,12 +28,13 @@ def _check(y, yo, tol=2e-2, med=3e-3):
     assert np.median(e) < med * rms, (np.median(e), rms)
 
 
+@pytest.mark.parametrize("out_layout", ["rows", "input"])
 @pytest.mark.parametrize("time_major", [False, True])
 @pytest.mark.parametrize("cplx", [True, False])
 @pytest.mark.parametrize("B,D,N,L", [(2, 32, 16, 2048), (1, 24, 16, 1000), (2, 16, 7, 5000), (3, 40, 2, 256),
                                      (1, 8, 16, 4352)])
-def test_causal(time_major, cplx, B, D, N, L):
-    print(f"case time_major={time_major} cplx={cplx} B={B} D={D} N={N} L={L}", flush=True)
+def test_causal(out_layout, time_major, cplx, B, D, N, L):
+    print(f"case out={out_layout} time_major={time_major} cplx={cplx} B={B} D={D} N={N} L={L}", flush=True)
     rng = np.random.default_rng(31)
     p, q, g = _coeffs(rng, D, N, cplx)
     om = rng.normal(size=D)
@@ -45,11 +46,13 @@ def test_causal(time_major, cplx, B, D, N, L):
     mask = np.zeros((B, L), bool)
     mask[0, L - L // 5:] = True
     mask[-1, 3] = True
-    y, _ = M.ops.ema_forward(x, dev(p), dev(q), dev(g), dev(om), padding_mask=dev(mask, torch.bool))
+    y, _ = M.ops.ema_forward(x, dev(p), dev(q), dev(g), dev(om), padding_mask=dev(mask, torch.bool),
+                             out_layout=out_layout)
     torch.cuda.synchronize()
+    assert y.stride() == (x.stride() if out_layout == "input" else (D * L, L, 1))
     yo, _ = O.ema_forward(x64, p, q, g, om, mask)
     _check(y, yo)
-    y2, _ = M.ops.ema_forward(x, dev(p), dev(q), dev(g), dev(om))
+    y2, _ = M.ops.ema_forward(x, dev(p), dev(q), dev(g), dev(om), out_layout=out_layout)
     yo2, _ = O.ema_forward(x64, p, q, g, om)
     _check(y2, yo2)
 
