@@ -33,6 +33,7 @@
 // shader clock; here they expand to nothing.
 #ifndef MEGA_TR
 #define MEGA_TR(k)
+#define MEGA_TR_FLUSH()
 #endif
 
 namespace mega {
@@ -264,7 +265,7 @@ __device__ __forceinline__ uint32_t dpp_swap2(uint32_t v) {      // lane ^ 2 wit
 // every load and store of the streaming loop is unconditional straight-line code, so the
 // stores of one super-chunk stay in flight under the next one's staging and sweeps (with a
 // branch around them the loop has to drain them before it may consume the prefetched loads).
-template <int LIN, int LOUT, bool FAST>
+template <int LIN, int LOUT, int MODE>
 __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   using G = Geo;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -289,6 +290,8 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
   }
   const int ch = cb * kWaves + wave;
+  // MODE 0: general; 1: FAST; 2: FAST with an even number of super-chunks, two of them in flight
+  constexpr bool FAST = MODE != 0;
   const bool ch_ok = FAST || ch < A.D;
   const int chc = ch_ok ? ch : A.D - 1;            // idle waves compute on a valid row, never store
   char* xrow = smem + wave * G::ROWB;
@@ -297,7 +300,12 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   const int nsc = (A.L + G::SC - 1) / G::SC;
   const int last_tile = A.L / 32 - 1;             // global index of the last whole tile
   constexpr int NLD = G::SC * 2 * kWaves / (kThreadsM * 16);   // 16-byte pieces per thread per super-chunk
-  uint4 pre[NLD];
+  // MODE 2 keeps two super-chunks of loads in flight (one register set each): the 32-byte pieces
+  // make a load take longer from issue to arrival than one super-chunk takes to compute.  Its loop
+  // has no branch around a load or a store (loads past the end fetch token 0 again and are never
+  // used), so every wait inside the loop counts exactly what may stay in flight.
+  constexpr int DEPTH = MODE == 2 ? 2 : 1;
+  uint4 preA[NLD], preB[NLD];
   const bf16_t* xg = (const bf16_t*)A.x;
   // layout 1: a lane pair (lane, lane ^ 2) covers tokens (2m, 2m+1) x 8 channels (half = lane & 1)
   const int half = tid & 1;
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
   const uint32_t sel_give = odd ? 0x05040100u : 0x07060302u;
 
-  auto issue_loads = [&](int sc) {
+  auto issue_loads = [&](int sc, uint4 (&pre)[NLD]) {
     const int t0 = sc * G::SC;
 #pragma unroll
     for (int k = 0; k < NLD; ++k) {
@@ -319,7 +327,8 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         const int tau = t0 + tk;
         const int c0 = cb * kWaves + half * 8;
         if (FAST) {
-          const int t = A.reverse ? A.L - 1 - tau : tau;
+          int t = A.reverse ? A.L - 1 - tau : tau;
+          if (MODE == 2) t = sc < nsc ? t : 0;
           pre[k] = *(const uint4*)(xg + b * A.sxb + (int64_t)t * A.sxl + c0);
         } else if (tau < A.L && c0 < A.D) {
           const int t = A.reverse ? A.L - 1 - tau : tau;
@@ -330,7 +339,8 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         const int tk = k * 512 + lane * 8;
         const int tau = t0 + tk;
         if (FAST || tau < A.L) {
-          const int t = A.reverse ? A.L - 8 - tau : tau;
+          int t = A.reverse ? A.L - 8 - tau : tau;
+          if (MODE == 2) t = sc < nsc ? t : 0;
           uint4 v = *(const uint4*)(xg + b * A.sxb + (int64_t)chc * A.sxd + t);
           if (A.reverse) {
             uint4 w;
@@ -358,14 +368,13 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
   };
 
   MEGA_TR(0);
-  issue_loads(0);
-  MEGA_TR(1);
+  issue_loads(0, preA);
 
   // ---- operand images of this channel: registers for the whole kernel
   bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
   float Qr[4], Qi[4];
   // segment scan: lane (n = lane >> 2, c = lane & 3) owns state n over segments 4c .. 4c+3
-  float Rr, Ri, R2r, R2i, R3r, R3i, R4r, R4i, R8r, R8i;    // powers of q^(32 SEGT); R4/R8 zeroed where unused
+  float Rr, Ri;                        // q^(32 SEGT) of state n: the scan's multiplier
   float Hcr = 0.f, Hci = 0.f;          // carried state of state n, in the lanes with c == 0 (zero elsewhere)
   {
     const uint4* img = A.image + (size_t)(A.koff + chc) * kImgSlots * 64 + lane;
@@ -389,21 +398,37 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     Qr[3] = __uint_as_float(qb.z); Qi[3] = __uint_as_float(qb.w);
     Rr = __uint_as_float(rr.x);
     Ri = __uint_as_float(rr.y);
-    R2r = Rr * Rr - Ri * Ri; R2i = 2.f * Rr * Ri;
-    R3r = R2r * Rr - R2i * Ri; R3i = R2r * Ri + R2i * Rr;
-    R4r = R2r * R2r - R2i * R2i; R4i = 2.f * R2r * R2i;
-    R8r = R4r * R4r - R4i * R4i; R8i = 2.f * R4r * R4i;
-    if ((lane & 3) < 1) { R4r = 0.f; R4i = 0.f; }     // quarter 0 has no predecessor
-    if ((lane & 3) < 2) { R8r = 0.f; R8i = 0.f; }     // quarters 0, 1 have none two back
     if (A.h_in && (lane & 3) == 0 && (lane >> 2) < A.N && ch_ok) {
       const size_t o = (((size_t)b * A.D + ch) * A.N + (lane >> 2)) * 2;
       Hcr = A.h_in[o];
       Hci = A.is_complex ? A.h_in[o + 1] : 0.f;
     }
   }
+  MEGA_TR(1);
+  if (DEPTH == 2) issue_loads(1, preB);
+  // The first super-chunk and the images are consumed here, outside the loop (only the second
+  // super-chunk's loads stay pending): a wait for them placed inside the loop would also drain the
+  // loads that are meant to stay in flight across iterations.
+  {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    auto pin = [](bf16x8& v) {
+      u32x4 t = __builtin_bit_cast(u32x4, v);
+      asm volatile("" : "+v"(t));
+      v = __builtin_bit_cast(bf16x8, t);
+    };
+#pragma unroll
+    for (int w = 0; w < kNWK; ++w) { pin(Kw[w][0]); pin(Kw[w][1]); }
+#pragma unroll
+    for (int w = 0; w < kNWP; ++w) { pin(Pw[w][0]); pin(Pw[w][1]); }
+#pragma unroll
+    for (int w = 0; w < kNWC; ++w) { pin(Cw[w][0]); pin(Cw[w][1]); }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(Qr[u]), "+v"(Qi[u]));
+    asm volatile("" : "+v"(Rr), "+v"(Ri), "+v"(Hcr), "+v"(Hci));
+  }
 
   MEGA_TR(2);
-  for (int sc = 0; sc < nsc; ++sc) {
+  auto body = [&](const int sc, uint4 (&pre)[NLD]) {
     const int t0 = sc * G::SC;
     MEGA_TR(3 + sc * 9);
     // ---- stage the prefetched super-chunk into LDS
@@ -433,7 +458,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     MEGA_TR(4 + sc * 9);
     __syncthreads();
     MEGA_TR(5 + sc * 9);
-    if (sc + 1 < nsc) issue_loads(sc + 1);
+    if (MODE == 2 || sc + DEPTH < nsc) issue_loads(sc + DEPTH, pre);      // the staged registers are free again
     MEGA_TR(6 + sc * 9);
 
     // ---- sweep 1: segment end states from a zero start
@@ -470,6 +495,16 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       __builtin_amdgcn_wave_barrier();
       {
         const int n = lane >> 2, c = lane & 3;
+        // powers of the multiplier, rebuilt here rather than held in registers across the loop
+        // (the opaque copy keeps the compiler from hoisting them back out)
+        float Tr = Rr, Ti = Ri;
+        asm volatile("" : "+v"(Tr), "+v"(Ti));
+        const float R2r = Tr * Tr - Ti * Ti, R2i = 2.f * Tr * Ti;
+        const float R3r = R2r * Tr - R2i * Ti, R3i = R2r * Ti + R2i * Tr;
+        float R4r = R2r * R2r - R2i * R2i, R4i = 2.f * R2r * R2i;
+        float R8r = R4r * R4r - R4i * R4i, R8i = 2.f * R4r * R4i;
+        if (c < 1) { R4r = 0.f; R4i = 0.f; }     // quarter 0 has no predecessor
+        if (c < 2) { R8r = 0.f; R8i = 0.f; }     // quarters 0, 1 have none two back
         float2* s2 = (float2*)scan + (4 * c) * G::SCANJ + n;
         float2 e[4];
 #pragma unroll
@@ -703,8 +738,17 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
     MEGA_TR(11 + sc * 9);
     __syncthreads();
+  };
+  if (DEPTH == 2) {
+    for (int sc = 0; sc < nsc; sc += 2) {
+      body(sc, preA);
+      body(sc + 1, preB);
+    }
+  } else {
+    for (int sc = 0; sc < nsc; ++sc) body(sc, preA);
   }
   MEGA_TR(3 + nsc * 9);
+  MEGA_TR_FLUSH();
   if (FAST && A.h_tile && (lane & 3) == 0) {
     // L is a whole number of super-chunks: the carried scan state is the state at time L
     float* ho = A.h_tile + (((size_t)b * A.D + ch) * kNS + (lane >> 2)) * 2;
@@ -792,12 +836,14 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
   const bool fast = !bidirectional && !mask && L % G::SC == 0 && D % kWaves == 0;
   auto launch = [&](const MfmaArgs& a) -> int {
     typedef void (*Kern)(const MfmaArgs);
-    static const Kern table[8] = {
-        ema_mfma_kernel<0, 0, false>, ema_mfma_kernel<0, 0, true>, ema_mfma_kernel<0, 1, false>,
-        ema_mfma_kernel<0, 1, true>,  ema_mfma_kernel<1, 0, false>, ema_mfma_kernel<1, 0, true>,
-        ema_mfma_kernel<1, 1, false>, ema_mfma_kernel<1, 1, true>};
-    static bool attr_set[8] = {false, false, false, false, false, false, false, false};
-    const int ki = lin * 4 + lout * 2 + (fast ? 1 : 0);
+    static const Kern table[12] = {
+        ema_mfma_kernel<0, 0, 0>, ema_mfma_kernel<0, 0, 1>, ema_mfma_kernel<0, 0, 2>,
+        ema_mfma_kernel<0, 1, 0>, ema_mfma_kernel<0, 1, 1>, ema_mfma_kernel<0, 1, 2>,
+        ema_mfma_kernel<1, 0, 0>, ema_mfma_kernel<1, 0, 1>, ema_mfma_kernel<1, 0, 2>,
+        ema_mfma_kernel<1, 1, 0>, ema_mfma_kernel<1, 1, 1>, ema_mfma_kernel<1, 1, 2>};
+    static bool attr_set[12] = {false, false, false, false, false, false, false, false, false, false, false, false};
+    const int mode = fast ? ((L / G::SC) % 2 == 0 ? 2 : 1) : 0;
+    const int ki = (lin * 2 + lout) * 3 + mode;
     const Kern kern = table[ki];
     if (!attr_set[ki]) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
