@@ -221,15 +221,23 @@ def main():
                    "input_buffers_rotated": NBUF},
         "block_hbm_gbs": alg_bytes_block / (ms_per_step * 1e-3) / 1e9,
         "block_hbm_frac": alg_bytes_block / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "roofline": {"bound": "hbm", "kernel": "ema_fwd (every launch of one call)", "achieved": ema_gbs,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS, "traffic": traffic.get("ema_mfma_kernel"),
-                     "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg, "host_enqueue_ms": ema_host},
-        "roofline_timestep_norm": {"bound": "hbm", "kernel": "group_tsn_kernel", "achieved": norm_gbs,
-                                   "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": norm_gbs / HBM_PEAK_GBS,
-                                   "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg,
-                                   "host_enqueue_ms": norm_host, "traffic": traffic.get("group_tsn_kernel")},
+        "roofline": None,
+        "kernels": {
+            "ema_mfma_kernel": {"bound": "hbm", "kernel": "ema_mfma_kernel (the EMA call)", "achieved": ema_gbs,
+                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS,
+                                "traffic": traffic.get("ema_mfma_kernel"),
+                                "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg,
+                                "host_enqueue_ms": ema_host},
+            "group_tsn_kernel": {"bound": "hbm", "kernel": "group_tsn_kernel (the TimestepNorm call)",
+                                 "achieved": norm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": norm_gbs / HBM_PEAK_GBS, "traffic": traffic.get("group_tsn_kernel"),
+                                 "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg,
+                                 "host_enqueue_ms": norm_host},
+        },
         "timestep_norm_status": status,
     }
+    # the dominant kernel = the one with the longer launch (both are HBM-bound)
+    out["roofline"] = max(out["kernels"].values(), key=lambda k: k["avg_ms"])
     if not args.no_cpu:
         threads = min(os.cpu_count() or 1, 16)
         x_host = xs[0].float().cpu().numpy()
