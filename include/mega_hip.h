@@ -90,7 +90,8 @@ int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_t sxd, int6
  * ema_hidden and the omega residual in one pass over x.  The D x L kernel is
  * never materialised.
  *   x, y    [B,D,L] of `dtype` with element strides (sxb,sxd,sxl) / (syb,syd,syl);
- *           any of the two contiguous layouts [B,D,L] or [B,L,D] is streamed coalesced
+ *           x and y may each use either contiguous layout, [B,D,L] or [B,L,D], independently
+ *           (the reference's convolution returns [B,D,L] rows for a transposed [B,L,D] input)
  *   p       [K,N] real, q [K,N,2] complex (q itself, not its log), gamma [K,N,2]
  *           complex already scaled by sqrt(1/N); K = D, or 2D when bidirectional
  *   is_complex   0: imaginary parts are ignored / assumed zero (real EMA)
