@@ -91,6 +91,95 @@ def measured_traffic():
     return out
 
 
+def bench_decode(args):
+    """configs[3]: B = 64 streams, D = 2048, N = 16, 16 norm groups: one fused TimestepNorm + EMA decode
+    step per token (state-traffic bound: the complex64 state h[B, D, N] is read and written once)."""
+    import numpy as np
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    Bd, Dd, Nd, Gd = 64, 2048, 16, 16
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1237)
+    import oracle.mega_oracle as O  # coefficient formulas only (host-side set-up of synthetic parameters)
+    from conftest import mega_init_complex
+
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, Dd, Nd))
+    t = lambda a, dt=torch.float32: torch.from_numpy(np.ascontiguousarray(a)).to(dt).to(dev)
+    tq = torch.from_numpy(q.astype(np.complex64)).to(dev)
+    tg = torch.from_numpy(g.astype(np.complex64)).to(dev)
+    step = M.ops.DecodeStep(t(rng.normal(size=Dd) * 0.1), t(rng.normal(size=Dd) * 0.1), Gd, 1e-5, t(p), tq, tg,
+                            t(rng.normal(size=Dd)), Bd)
+    xs = [torch.randn(Bd, Dd, device=dev).to(torch.bfloat16) for _ in range(16)]
+    with torch.no_grad():
+        for i in range(args.warmup):
+            step(xs[i % 16])
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        a.record()
+        for i in range(args.steps):
+            step(xs[i % 16])
+        b.record()
+        host = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms = max(wall * 1e3, a.elapsed_time(b)) / args.steps
+    dev_ms = a.elapsed_time(b) / args.steps
+    alg = 2 * Bd * Dd * Nd * 8 + 3 * Bd * Dd * 2 + 4 * Bd * Gd * 4
+    gbs = alg / (dev_ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "decode tokens/sec @B64xD2048, fused TimestepNorm + EMA step", "value": Bd / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[3]: 64 streams, D=2048, N=16 complex, 16 norm groups, one token per step"},
+        "roofline": {"bound": "hbm", "kernel": "norm_ema_step_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg, "avg_ms": dev_ms, "host_enqueue_ms": host * 1e3 / args.steps},
+    }))
+
+
+def bench_attention(args):
+    """configs[4]'s attention: 4 chunks of 2048 tokens, 4 heads, H1 = 128, H2 = 1024, bf16, causal
+    (matrix-core bound).  Flops are counted for the causal half only: 2 * C^2/2 * (H1 + H2) per chunk-head."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    Bc, C, Nh, H1, H2 = 4, 2048, 4, 128, 1024
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(1238)
+    mk = lambda *sh: torch.randn(*sh, generator=gen).to(torch.bfloat16).to(dev)
+    q, k, v = mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H2)
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            M.ops.attention_fwd(q, k, v, 1.0 / H1 ** 0.5, 0.0, True)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        a.record()
+        for _ in range(args.steps):
+            M.ops.attention_fwd(q, k, v, 1.0 / H1 ** 0.5, 0.0, True)
+        b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms = max(wall * 1e3, a.elapsed_time(b)) / args.steps
+    dev_ms = a.elapsed_time(b) / args.steps
+    flops_causal = Bc * Nh * (C * (C + 1)) * (H1 + H2)          # 2 flops x C(C+1)/2 pairs x (H1 + H2)
+    flops_full = 2 * Bc * Nh * C * C * (H1 + H2)
+    tf = flops_causal / (dev_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "attention chunk tokens/sec @4x2048, 4 heads, H1=128, H2=1024", "value": Bc * C / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[4] attention: causal softmax(q k^T) v per 2048-token chunk and head"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel x2 + softmax_f32_kernel + transpose_v_kernel",
+                     "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0, "traffic": None,
+                     "algorithmic_flops_per_call": flops_causal, "full_square_flops": flops_full, "avg_ms": dev_ms},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -101,10 +190,18 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
+    ap.add_argument("--workload", choices=["block", "decode", "attention"], default="block",
+                    help="block: the headline TimestepNorm -> EMA block (default); decode / attention: the "
+                         "decode step of configs[3] / the chunk attention of configs[4], one JSON line each")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "decode":
+        return bench_decode(args)
+    if args.workload == "attention":
+        return bench_attention(args)
 
     import numpy as np
     import torch

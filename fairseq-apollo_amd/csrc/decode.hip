@@ -102,6 +102,88 @@ __global__ __launch_bounds__(kT) void norm_ema_step_kernel(const StepArgs A) {
   }
 }
 
+// Same step with the state streamed as 32-byte pieces: NP = N / 4 adjacent lanes own one channel,
+// each lane four states (two 16-byte loads of h, q, gamma, one of p), so a wave reads and writes
+// the state as one contiguous 2 KB block; the output sum is finished across the NP lanes.
+constexpr int kTV = 256;
+
+template <typename T, int NP>
+__global__ __launch_bounds__(kTV) void norm_ema_step_vec_kernel(const StepArgs A) {
+  __shared__ float red[kTV / 64];
+  const int g = blockIdx.x % A.G, b = blockIdx.x / A.G;
+  const int dg = A.D / A.G;
+  const T* xr = (const T*)A.x + (size_t)b * A.D + (size_t)g * dg;
+  const int64_t c0 = A.prev_count[b];
+  const float u0 = A.prev_mean[(size_t)b * A.G + g], v0 = A.prev_var[(size_t)b * A.G + g];
+  auto wg_sum = [&](float v) {
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < kTV / 64; ++i) t += red[i];
+    return t;
+  };
+  float s = 0.f;
+  for (int f = threadIdx.x; f < dg; f += kTV) s += to_float(xr[f]);
+  const float gm = wg_sum(s) / (float)dg;
+  float s2 = 0.f;
+  for (int f = threadIdx.x; f < dg; f += kTV) {
+    const float d = to_float(xr[f]) - gm;
+    s2 += d * d;
+  }
+  const float gv = wg_sum(s2) / (float)dg;
+  const float c1 = (float)c0 / (float)(c0 + 1), c2 = 1.0f / (float)(c0 + 1);
+  const float dl = gm - u0;
+  const float u1 = c1 * u0 + c2 * gm;
+  const float v1 = c1 * v0 + c2 * gv + (c1 * dl) * (c2 * dl);
+  const float rstd = 1.0f / sqrtf(v1 + A.eps);
+  __syncthreads();                               // every thread has read the old state
+  if (threadIdx.x == 0) {
+    A.mean[(size_t)b * A.G + g] = u1;
+    A.var[(size_t)b * A.G + g] = v1;
+    if (g == 0) A.count[b] = c0 + 1;
+  }
+  const int items = dg * NP;                     // a multiple of NP, so the lanes of a channel stay together
+  for (int it0 = 0; it0 < items; it0 += kTV) {
+    const int it = it0 + threadIdx.x;
+    const bool ok = it < items;
+    const int f = ok ? it / NP : 0, part = it % NP;
+    const int d = g * dg + f;
+    const size_t o = (size_t)b * A.D + d;
+    const float xnv_full = (to_float(xr[f]) - u1) * rstd * A.nw[d] + A.nb[d];
+    const T xn_t = from_float<T>(xnv_full);
+    const float xv = to_float(xn_t);             // the moving average sees the rounded activation
+    const size_t ho = (o * A.N + 4 * part) * 2;
+    const size_t co = (size_t)d * A.N + 4 * part;
+    float4 h0 = make_float4(0.f, 0.f, 0.f, 0.f), h1 = h0;
+    if (A.h_in) {
+      h0 = *(const float4*)(A.h_in + ho);
+      h1 = *(const float4*)(A.h_in + ho + 4);
+    }
+    const float4 q0 = *(const float4*)(A.q + co * 2), q1 = *(const float4*)(A.q + co * 2 + 4);
+    const float4 g0 = *(const float4*)(A.g + co * 2), g1 = *(const float4*)(A.g + co * 2 + 4);
+    const float4 pp = *(const float4*)(A.p + co);
+    float4 n0, n1;
+    n0.x = q0.x * h0.x - q0.y * h0.y + pp.x * xv;  n0.y = q0.x * h0.y + q0.y * h0.x;
+    n0.z = q0.z * h0.z - q0.w * h0.w + pp.y * xv;  n0.w = q0.z * h0.w + q0.w * h0.z;
+    n1.x = q1.x * h1.x - q1.y * h1.y + pp.z * xv;  n1.y = q1.x * h1.y + q1.y * h1.x;
+    n1.z = q1.z * h1.z - q1.w * h1.w + pp.w * xv;  n1.w = q1.z * h1.w + q1.w * h1.z;
+    float acc = (g0.x * n0.x - g0.y * n0.y) + (g0.z * n0.z - g0.w * n0.w) + (g1.x * n1.x - g1.y * n1.y) +
+                (g1.z * n1.z - g1.w * n1.w);
+#pragma unroll
+    for (int m = 1; m < NP; m <<= 1) acc += __shfl_xor(acc, m);
+    if (ok) {
+      *(float4*)(A.h_out + ho) = n0;
+      *(float4*)(A.h_out + ho + 4) = n1;
+      if (part == 0) {
+        ((T*)A.xn)[o] = xn_t;
+        ((T*)A.y)[o] = from_float<T>(acc + A.omega[d] * xv);
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -130,6 +212,24 @@ extern "C" int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, c
   A.eps = (float)eps;
   const dim3 grid((unsigned)(B * G));
   hipStream_t s = (hipStream_t)stream;
+  // vector path: complex coefficient storage (always), 4 | N, N / 4 a power of two, aligned pointers
+  const int np = (int)(N / 4);
+  if (is_complex && N % 4 == 0 && (np & (np - 1)) == 0 && ((uintptr_t)h_out % 16) == 0 && (!h_in || ((uintptr_t)h_in % 16) == 0) &&
+      ((uintptr_t)q % 16) == 0 && ((uintptr_t)gamma % 16) == 0 && ((uintptr_t)p % 16) == 0) {
+#define LAUNCH_NV(T)                                                                                     \
+  switch (np) {                                                                                          \
+    case 1: hipLaunchKernelGGL((norm_ema_step_vec_kernel<T, 1>), grid, dim3(kTV), 0, s, A); break;       \
+    case 2: hipLaunchKernelGGL((norm_ema_step_vec_kernel<T, 2>), grid, dim3(kTV), 0, s, A); break;       \
+    case 4: hipLaunchKernelGGL((norm_ema_step_vec_kernel<T, 4>), grid, dim3(kTV), 0, s, A); break;       \
+    default: hipLaunchKernelGGL((norm_ema_step_vec_kernel<T, 8>), grid, dim3(kTV), 0, s, A); break;      \
+  }
+    if (dtype == MEGA_F32) { LAUNCH_NV(float) }
+    else if (dtype == MEGA_BF16) { LAUNCH_NV(bf16_t) }
+    else { LAUNCH_NV(f16_t) }
+#undef LAUNCH_NV
+    MEGA_CHECK_LAUNCH("norm_ema_step");
+    return MEGA_OK;
+  }
 #define LAUNCH_NS(T, C) hipLaunchKernelGGL((norm_ema_step_kernel<T, C>), grid, dim3(kT), 0, s, A)
   if (is_complex) {
     if (dtype == MEGA_F32) LAUNCH_NS(float, true);
