@@ -9,7 +9,7 @@
 //                          the reduction stops at the diagonal
 //
 // The GEMM: 128 x 128 output tile per workgroup (4 waves, 64 x 64 each as 4 x 4 MFMA blocks),
-// K step 32, operands staged through LDS with an 80-byte row pitch (conflict-free 16-byte reads),
+// K step 64, operands staged through LDS with a 144-byte row pitch (conflict-free 16-byte reads),
 // register prefetch of the next K step.
 #include "common.h"
 
@@ -20,8 +20,10 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int BM = 128, BN = 128, BK = 32;
-constexpr int PITCH = 80;                 // bytes per LDS row of 32 16-bit elements (+ 16 pad)
+constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int PITCH = BK * 2 + 16;        // bytes per LDS row of BK 16-bit elements (+ 16 pad)
+constexpr int KP = BK / 8;                // 16-byte pieces per operand row and K step
+constexpr int NLP = BM * KP / 256;        // pieces per thread, operand and K step
 
 struct GemmArgs {
   const void* A;      // [batch][M][K] rows with pitch lda (elements), batch stride sa
@@ -35,6 +37,10 @@ struct GemmArgs {
   float alpha;
   int causal;         // 1: S = q k^T (skip tiles with n0 > m0 + BM - 1); 2: y = P v (K stops at m0 + BM)
   int kshift;         // causal offset: row m sees columns <= m + kshift
+  // xcd != 0: one-dimensional grid; every tile of a batch entry runs on one XCD (workgroup ids go
+  // round-robin over the 8 XCDs), so both operands of a batch entry are fetched into one L2 only;
+  // the long (late) row tiles of a causal product come first
+  int xcd, mt, nt;
 };
 
 template <typename T>
@@ -53,9 +59,22 @@ template <typename TIn, typename TOut>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
   __shared__ __attribute__((aligned(16))) char lds[2 * (BM + BN) * PITCH];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  int m0, n0, bz;
+  if (G.xcd) {
+    int rest = (int)blockIdx.x >> 3;
+    const int ntile = rest % G.nt;
+    rest /= G.nt;
+    const int mtile = G.mt - 1 - rest % G.mt;
+    rest /= G.mt;
+    bz = rest * 8 + ((int)blockIdx.x & 7);
+    m0 = mtile * BM;
+    n0 = ntile * BN;
+  } else {
+    m0 = blockIdx.y * BM;
+    n0 = blockIdx.x * BN;
+    bz = blockIdx.z;
+  }
   if (G.causal == 1 && n0 > m0 + BM - 1 + G.kshift) return;      // entirely above the diagonal
-  const int bz = blockIdx.z;
   const int bo = bz / G.nin, bi = bz - bo * G.nin;
   const TIn* A = (const TIn*)G.A + bo * G.sa + bi * G.sai;
   const TIn* Bm = (const TIn*)G.Bm + bo * G.sb + bi * G.sbi;
@@ -65,14 +84,14 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
   if (Kend < 0) Kend = 0;
   const int nk = (Kend + BK - 1) / BK;
 
-  // global -> register staging: thread covers 2 x 16 bytes of A and of B per K step
-  const int lrow = tid >> 2, lcol = (tid & 3) * 8;               // rows 0..63 (+64), 8 elements each
-  uint4 ra[2], rb[2];
+  // global -> register staging: thread covers NLP x 16 bytes of A and of B per K step
+  const int lrow = tid / KP, lcol = (tid % KP) * 8;              // rows 0 .. 256/KP - 1 (+ h * 256/KP)
+  uint4 ra[NLP], rb[NLP];
   auto gload = [&](int kt) {
     const int k = kt * BK + lcol;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lrow + h * 64;
+    for (int h = 0; h < NLP; ++h) {
+      const int r = lrow + h * (256 / KP);
       ra[h] = make_uint4(0, 0, 0, 0);
       rb[h] = make_uint4(0, 0, 0, 0);
       if (m0 + r < G.M && k < Kend) ra[h] = *(const uint4*)(A + (int64_t)(m0 + r) * G.lda + k);
@@ -83,8 +102,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
     char* la = lds + buf * (BM + BN) * PITCH;
     char* lb = la + BM * PITCH;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int r = lrow + h * 64;
+    for (int h = 0; h < NLP; ++h) {
+      const int r = lrow + h * (256 / KP);
       *(uint4*)(la + r * PITCH + lcol * 2) = ra[h];
       *(uint4*)(lb + r * PITCH + lcol * 2) = rb[h];
     }
@@ -107,15 +126,18 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
     if (kt + 1 < nk) gload(kt + 1);
     const char* la = lds + buf * (BM + BN) * PITCH;
     const char* lb = la + BM * PITCH;
-    uint4 fa[4], fb[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + fk);
+    for (int kk = 0; kk < BK / 32; ++kk) {
+      uint4 fa[4], fb[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + fk);
+      for (int i = 0; i < 4; ++i) fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + kk * 64 + fk);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 4; ++j) fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + kk * 64 + fk);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<TIn>(fa[i], fb[j], acc[i][j]);
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<TIn>(fa[i], fb[j], acc[i][j]);
+    }
     if (kt + 1 < nk) lstore(buf ^ 1);
     __syncthreads();
   }
@@ -135,38 +157,69 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
     }
 }
 
-// v [B][L][Nh][H2] -> vt [B][Nh][H2][Lp] (Lp = L rounded up to 8, zero padded)
+// v [B][L][Nh][H2] -> vt [B][Nh][H2][Lp] (Lp = L rounded up to 8, zero padded).  64 x 64 tiles:
+// 16-byte loads along H2, 2-byte gathers from LDS, 16-byte stores along L.  `vec` = H2 % 8 == 0 and
+// v 16-byte aligned (otherwise element-wise loads).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_v_kernel(const T* __restrict__ v, T* __restrict__ vt, int L, int Nh,
-                                                          int H2, int Lp) {
-  __shared__ T tile[32][33];
+                                                          int H2, int Lp, int vec) {
+  constexpr int TP = 66;                                         // LDS row pitch in elements (33 dwords)
+  __shared__ T tile[64 * TP];
   const int bn = blockIdx.z;
   const int b = bn / Nh, n = bn - b * Nh;
-  const int l0 = blockIdx.x * 32, h0 = blockIdx.y * 32;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;      // 32 x 8
-  for (int i = ty; i < 32; i += 8) {
-    const int l = l0 + i, h = h0 + tx;
-    T val = from_float<T>(0.f);
-    if (l < L && h < H2) val = v[(((int64_t)b * L + l) * Nh + n) * H2 + h];
-    tile[i][tx] = val;
+  const int l0 = blockIdx.x * 64, h0 = blockIdx.y * 64;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int pi = threadIdx.x + u * 256;
+    const int li = pi >> 3, hc = (pi & 7) * 8;
+    const int l = l0 + li, h = h0 + hc;
+    Vec<T, 8> val;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) val.v[e] = from_float<T>(0.f);
+    if (l < L) {
+      const T* src = v + (((int64_t)b * L + l) * Nh + n) * H2 + h;
+      if (vec && h + 8 <= H2) {
+        val = *(const Vec<T, 8>*)src;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (h + e < H2) val.v[e] = src[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tile[li * TP + hc + e] = val.v[e];
   }
   __syncthreads();
-  for (int i = ty; i < 32; i += 8) {
-    const int h = h0 + i, l = l0 + tx;
-    if (h < H2 && l < Lp) vt[(((int64_t)b * Nh + n) * H2 + h) * Lp + l] = tile[tx][i];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int pi = threadIdx.x + u * 256;
+    const int hi = pi >> 3, lc = (pi & 7) * 8;
+    const int h = h0 + hi, l = l0 + lc;
+    if (h < H2 && l < Lp) {
+      Vec<T, 8> out;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out.v[e] = tile[(lc + e) * TP + hi];
+      *(Vec<T, 8>*)(vt + (((int64_t)b * Nh + n) * H2 + h) * Lp + l) = out;     // Lp % 8 == 0: whole pieces
+    }
   }
 }
 
 // causal softmax of fp32 scores into 16-bit probabilities; rows [outer][inner], pitch in elements
+// (multiples of 4).  The row is read once into registers (up to 16 values per thread, longer rows
+// loop); columns past the causal limit are written as zeros only up to `zcols`, the end of the
+// 128-column block the diagonal falls into (the second product never reads beyond it), unless the
+// caller wants the whole weight matrix (zero_all).
 template <typename TOut>
 __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restrict__ s, TOut* __restrict__ p, int outer,
                                                           int inner, int64_t spitch, int64_t ppitch, int pcols,
-                                                          int causal) {
+                                                          int causal, int zero_all) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int r = (int)(row % outer);
   int n = causal ? inner - outer + r + 1 : inner;
   if (n < 0) n = 0;
+  int zcols = pcols;
+  if (causal && !zero_all) zcols = min(pcols, ((n + BM - 1) / BM + 1) * BM);
   const float* sp = s + row * spitch;
   TOut* pp = p + row * ppitch;
   auto reduce = [&](float v, bool is_max) {
@@ -181,18 +234,62 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restric
     for (int i = 1; i < 4; ++i) t = is_max ? fmaxf(t, red[i]) : t + red[i];
     return t;
   };
+  constexpr int NV = 4;                              // float4 per thread held in registers: 4096 columns
+  const bool in_regs = n <= 256 * 4 * NV;
+  float4 v[NV];
   float m = -INFINITY;
-  for (int j = threadIdx.x; j < n; j += 256) m = fmaxf(m, sp[j]);
+  if (in_regs) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int j = (u * 256 + threadIdx.x) * 4;
+      v[u] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      if (j < n) {
+        v[u] = *(const float4*)(sp + j);
+        if (j + 1 >= n) v[u].y = -INFINITY;
+        if (j + 2 >= n) v[u].z = -INFINITY;
+        if (j + 3 >= n) v[u].w = -INFINITY;
+      }
+      m = fmaxf(m, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+    }
+  } else {
+    for (int j = threadIdx.x; j < n; j += 256) m = fmaxf(m, sp[j]);
+  }
   m = reduce(m, true);
   const bool dead = !(m > -INFINITY) || !(m < INFINITY);
   float sum = 0.f;
-  if (!dead)
-    for (int j = threadIdx.x; j < n; j += 256) sum += __expf(sp[j] - m);
+  if (!dead) {
+    if (in_regs) {
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        v[u].x = __expf(v[u].x - m); v[u].y = __expf(v[u].y - m);
+        v[u].z = __expf(v[u].z - m); v[u].w = __expf(v[u].w - m);
+        sum += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+      }
+    } else {
+      for (int j = threadIdx.x; j < n; j += 256) sum += __expf(sp[j] - m);
+    }
+  }
   sum = reduce(sum, false);
   const float c = (dead || sum == 0.f) ? 0.f : 1.0f / sum;
-  for (int j = threadIdx.x; j < pcols; j += 256) {
-    const float e = (j < n && !dead) ? __expf(sp[j] - m) * c : 0.f;
-    pp[j] = from_float<TOut>(e);
+  if (in_regs && sizeof(TOut) == 2) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int j = (u * 256 + threadIdx.x) * 4;
+      if (j < zcols) {
+        const bool live = !dead && j < n;             // exp(-inf) = 0 covers the tail of a partial quad
+        TOut o0 = from_float<TOut>(live ? v[u].x * c : 0.f), o1 = from_float<TOut>(live ? v[u].y * c : 0.f);
+        TOut o2 = from_float<TOut>(live ? v[u].z * c : 0.f), o3 = from_float<TOut>(live ? v[u].w * c : 0.f);
+        uint2 w;
+        w.x = (uint32_t)__builtin_bit_cast(uint16_t, o0) | ((uint32_t)__builtin_bit_cast(uint16_t, o1) << 16);
+        w.y = (uint32_t)__builtin_bit_cast(uint16_t, o2) | ((uint32_t)__builtin_bit_cast(uint16_t, o3) << 16);
+        *(uint2*)(pp + j) = w;
+      }
+    }
+  } else {
+    for (int j = threadIdx.x; j < zcols; j += 256) {
+      const float e = (j < n && !dead) ? __expf(sp[j] - m) * c : 0.f;
+      pp[j] = from_float<TOut>(e);
+    }
   }
 }
 
@@ -207,8 +304,10 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   ws += align_up((size_t)BN_ * L * Lp * sizeof(T), 256);
   T* Vt = (T*)ws;                                  // [B*Nh][H2][Lp]
   {
-    const dim3 grid((unsigned)ceil_div(Lp, 32), (unsigned)ceil_div(H2, 32), (unsigned)BN_);
-    hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, (const T*)v, Vt, (int)L, (int)Nh, (int)H2, (int)Lp);
+    const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(H2, 64), (unsigned)BN_);
+    const int vec = (H2 % 8 == 0 && ((uintptr_t)v % 16) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, (const T*)v, Vt, (int)L, (int)Nh, (int)H2, (int)Lp,
+                       vec);
   }
   GemmArgs G;
   // S[b,n] = scale q[b,:,n,:] k[b,:,n,:]^T
@@ -216,12 +315,15 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   G.lda = Nh * H1; G.ldb = Nh * H1; G.ldc = Lp;
   G.sa = L * Nh * H1; G.sai = H1; G.sb = L * Nh * H1; G.sbi = H1; G.sc = Nh * L * Lp; G.sci = L * Lp;
   G.nin = (int)Nh; G.M = (int)L; G.N = (int)L; G.K = (int)H1; G.alpha = scale; G.causal = causal ? 1 : 0; G.kshift = 0;
+  const bool xcd = BN_ % 8 == 0;
   {
-    const dim3 grid((unsigned)ceil_div(L, BN), (unsigned)ceil_div(L, BM), (unsigned)BN_);
-    hipLaunchKernelGGL((gemm_nt_kernel<T, float>), grid, dim3(256), 0, s, G);
+    G.xcd = xcd ? 1 : 0; G.mt = (int)ceil_div(L, BM); G.nt = (int)ceil_div(L, BN);
+    const dim3 grid3((unsigned)G.nt, (unsigned)G.mt, (unsigned)BN_);
+    const dim3 grid1((unsigned)(G.nt * G.mt * BN_));
+    hipLaunchKernelGGL((gemm_nt_kernel<T, float>), xcd ? grid1 : grid3, dim3(256), 0, s, G);
   }
   hipLaunchKernelGGL(softmax_f32_kernel<T>, dim3((unsigned)(BN_ * L)), dim3(256), 0, s, S, P, (int)L, (int)L, Lp, Lp,
-                     (int)Lp, causal);
+                     (int)Lp, causal, w ? 1 : 0);
   if (w) {
     // the weights the reference returns: [B, Nh, L, L]
     hipMemcpy2DAsync(w, (size_t)L * sizeof(T), P, (size_t)Lp * sizeof(T), (size_t)L * sizeof(T), (size_t)(BN_ * L),
@@ -233,8 +335,10 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = Nh * H2 * Lp; G.sbi = H2 * Lp; G.sc = L * Nh * H2; G.sci = H2;
   G.M = (int)L; G.N = (int)H2; G.K = (int)Lp; G.alpha = 1.0f; G.causal = causal ? 2 : 0;
   {
-    const dim3 grid((unsigned)ceil_div(H2, BN), (unsigned)ceil_div(L, BM), (unsigned)BN_);
-    hipLaunchKernelGGL((gemm_nt_kernel<T, T>), grid, dim3(256), 0, s, G);
+    G.xcd = xcd ? 1 : 0; G.mt = (int)ceil_div(L, BM); G.nt = (int)ceil_div(H2, BN);
+    const dim3 grid3((unsigned)G.nt, (unsigned)G.mt, (unsigned)BN_);
+    const dim3 grid1((unsigned)(G.nt * G.mt * BN_));
+    hipLaunchKernelGGL((gemm_nt_kernel<T, T>), xcd ? grid1 : grid3, dim3(256), 0, s, G);
   }
   MEGA_CHECK_LAUNCH("attention_fwd (matrix-core path)");
   return MEGA_OK;

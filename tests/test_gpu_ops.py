@@ -87,6 +87,31 @@ def test_attention(dtype, B, L, Nh, H1, H2, causal):
         assert torch.equal(ym, y[:, :, 0])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,Nh,H1,H2", [(2, 300, 2, 64, 256), (1, 1000, 1, 128, 512), (1, 129, 3, 32, 256),
+                                          (1, 64, 1, 96, 256)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_no_weights(dtype, B, L, Nh, H1, H2, causal):
+    """No weights requested (the inference call of the layer), at sizes where the matrix-core GEMMs
+    run many tiles; also against the call that returns the weights."""
+    print(f"case {dtype} B={B} L={L} Nh={Nh} H1={H1} H2={H2} causal={causal}", flush=True)
+    rng = np.random.default_rng(26)
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    scale = 1.0 / np.sqrt(H1) * 2.0
+    y, w = M.ops.attention_fwd(q, k, v, scale, 0.0, causal)
+    assert w is None
+    torch.cuda.synchronize()
+    yo, _ = O.attention(q64, k64, v64, scale, causal)
+    # the probabilities enter the second product rounded to 16 bits (as the reference's do: its softmax
+    # output has the activation dtype): over 10^5..10^6 outputs the largest deviation sits ~5 sigma out,
+    # so the denominator floor of the error measure is 2 rms here (eps = 2) instead of 1 rms
+    assert rel_err(host(y), yo, eps=2.0) < TOL[dtype]
+    y2, _ = M.ops.attention_fwd(q, k, v, scale, 0.0, causal, need_weights=True)
+    assert rel_err(host(y), host(y2), eps=2.0) < 2 * TOL[dtype]      # two 16-bit results
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n", [1, 7, 4096, 100003])
 def test_swiglu(dtype, n):
