@@ -143,6 +143,31 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
   }
   // D layout: column = lane & 15, rows 4 (lane >> 4) + {0..3}
   const int cn = lane & 15, cr = (lane >> 4) * 4;
+  constexpr int VW = 16 / (int)sizeof(TOut);                     // elements per 16-byte piece
+  const bool wide = (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + BN <= G.N;
+  if (wide) {
+    // whole tile through LDS (the operand buffers are free after the last barrier): rows leave as
+    // 16-byte pieces, BN * sizeof(TOut) contiguous bytes each
+    constexpr int CP = BN + VW;                                  // row pitch in elements
+    TOut* Cs = (TOut*)lds;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          Cs[(wm + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
+    __syncthreads();
+    constexpr int PPR = BN / VW;                                 // pieces per row
+#pragma unroll
+    for (int u = 0; u < BM * PPR / 256; ++u) {
+      const int pi = tid + u * 256;
+      const int r = pi / PPR, pc = pi - r * PPR;
+      if (m0 + r < G.M)
+        *(uint4*)(C + (int64_t)(m0 + r) * G.ldc + n0 + pc * VW) = *(const uint4*)(Cs + r * CP + pc * VW);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
