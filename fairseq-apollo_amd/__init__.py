@@ -11,11 +11,18 @@ from .modules import (  # noqa: F401
     TimestepNorm,
 )
 
-from .layers import Mega2Layer, MovingAverageGatedAttention, RMSNorm, RotaryEmbedding  # noqa: F401,E402
+from .layers import (  # noqa: F401,E402
+    Mega2Layer,
+    MovingAverageGatedAttention,
+    NormalizedFeedForwardNetwork,
+    RMSNorm,
+    RotaryEmbedding,
+)
 
 __all__ = [
     "Mega2Layer",
     "MovingAverageGatedAttention",
+    "NormalizedFeedForwardNetwork",
     "RMSNorm",
     "RotaryEmbedding",
     "ops",

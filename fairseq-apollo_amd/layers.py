@@ -41,6 +41,64 @@ class RMSNorm(nn.Module):
         return y.to(x.dtype)
 
 
+class NormalizedFeedForwardNetwork(nn.Module):
+    """The reference's position-wise block, `x + fc2(silu(fc1(norm(x))))` with an optional
+    per-feature layer scale (fairseq/modules/normalized_feedforward_network.py:13-93; same
+    constructor arguments, parameter names and initialisation; dropout is inference-mode identity).
+    The two projections are library GEMMs; norm and activation are elementwise glue."""
+
+    def __init__(self, embed_dim, ffn_hidden_dim, dropout=0.0, hidden_dropout=0.0, norm_type='layernorm',
+                 norm_affine=True, norm_eps=1e-5, layer_scale=None, init_mode='bert', export=False):
+        super().__init__()
+        self.embedding_dim = embed_dim
+        self.hidden_dim = ffn_hidden_dim
+        self.act_fn = 'silu'
+        self.init_mode = init_mode
+        self.layer_scale = layer_scale
+        if dropout or hidden_dropout:
+            raise RuntimeError("NormalizedFeedForwardNetwork: dropout (training) is not implemented; pass 0")
+        if norm_type == 'layernorm':
+            self.norm = nn.LayerNorm(embed_dim, eps=norm_eps, elementwise_affine=norm_affine)
+        elif norm_type == 'rmsnorm':
+            self.norm = RMSNorm(embed_dim, elementwise_affine=norm_affine, eps=norm_eps)
+        else:
+            raise ValueError('unknown norm type: {}'.format(norm_type))
+        self.fc1 = nn.Linear(embed_dim, ffn_hidden_dim, bias=True)
+        self.fc2 = nn.Linear(ffn_hidden_dim, embed_dim, bias=False)
+        if layer_scale is None:
+            self.register_parameter('layerscale_weight', None)
+        else:
+            assert layer_scale > 0., 'Layer scale init value should be positive.'
+            self.layerscale_weight = Parameter(torch.Tensor(embed_dim))
+        assert init_mode in ['bert', 'xavier', 'he']
+        self.reset_parameters(init_mode)
+
+    def reset_parameters(self, mode):
+        if mode == 'bert':
+            nn.init.normal_(self.fc1.weight, mean=0.0, std=0.02)
+            nn.init.normal_(self.fc2.weight, mean=0.0, std=0.02)
+        elif mode == 'he':
+            nn.init.kaiming_normal_(self.fc1.weight, a=math.sqrt(5.0))
+            nn.init.kaiming_normal_(self.fc2.weight, a=math.sqrt(5.0))
+        else:
+            nn.init.xavier_uniform_(self.fc1.weight)
+            nn.init.xavier_uniform_(self.fc2.weight)
+        nn.init.constant_(self.fc1.bias, 0.0)
+        if self.layerscale_weight is not None:
+            nn.init.constant_(self.layerscale_weight, self.layer_scale)
+
+    def forward(self, x: Tensor) -> Tensor:
+        _no_grad_only(self, x)
+        h = self.fc2(F.silu(self.fc1(self.norm(x))))
+        if self.layerscale_weight is not None:
+            h = h * self.layerscale_weight
+        return h + x
+
+    def extra_repr(self) -> str:
+        return 'edim={}, hdim={}, act={}, init={}, layerscale={}'.format(self.embedding_dim, self.hidden_dim,
+                                                                         self.act_fn, self.init_mode, self.layer_scale)
+
+
 class RotaryEmbedding(nn.Module):
     """fairseq/modules/relative_positional_bias.py:47-97: features (2i, 2i+1) rotate by
     t * base^(-2i/dim); q may start at an offset (incremental decoding)."""

@@ -97,3 +97,29 @@ def test_config4_full_mega2_layer_bf16():
                                   np.zeros(D), None, 16, 1e-5)
     yo = ao + O.swiglu_ffn(xn, rb(w1), rb(w3), rb(w2))
     assert _chain_ok(y[:, :Lo], yo, 2e-2)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("norm_type,layer_scale", [("rmsnorm", None), ("layernorm", 0.1)])
+def test_normalized_feed_forward(dtype, tol, norm_type, layer_scale):
+    """The reference's position-wise block against the oracle (normalized_feedforward_network.py:77-93)."""
+    torch.manual_seed(11)
+    B, L, D, Hd = 2, 96, 64, 160
+    ffn = M.NormalizedFeedForwardNetwork(D, Hd, norm_type=norm_type, layer_scale=layer_scale, init_mode='xavier')
+    with torch.no_grad():
+        ffn.fc1.bias.normal_(0, 0.1)
+    ffn = ffn.to(DEV).to(dtype).eval()
+    x = torch.randn(B, L, D).to(dtype).to(DEV)
+    with torch.no_grad():
+        y = ffn(x)
+    x64 = host(x)
+    if norm_type == "rmsnorm":
+        xn = O.rms_norm(x64, host(ffn.norm.weight))
+    else:
+        mu = x64.mean(-1, keepdims=True)
+        xn = (x64 - mu) / np.sqrt(x64.var(-1, keepdims=True) + 1e-5) * host(ffn.norm.weight) + host(ffn.norm.bias)
+    w2 = host(ffn.fc2.weight)
+    if layer_scale is not None:
+        w2 = w2 * host(ffn.layerscale_weight)[:, None]
+    yo = O.silu_ffn(xn, host(ffn.fc1.weight), host(ffn.fc1.bias), w2, 0.0) - xn + x64
+    assert _chain_ok(y, yo, tol)
