@@ -101,16 +101,12 @@ def bench_decode(args):
 
     Bd, Dd, Nd, Gd = 64, 2048, 16, 16
     dev = torch.device("cuda:0")
-    rng = np.random.default_rng(1237)
-    import oracle.mega_oracle as O  # coefficient formulas only (host-side set-up of synthetic parameters)
-    from conftest import mega_init_complex
-
-    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, Dd, Nd))
-    t = lambda a, dt=torch.float32: torch.from_numpy(np.ascontiguousarray(a)).to(dt).to(dev)
-    tq = torch.from_numpy(q.astype(np.complex64)).to(dev)
-    tg = torch.from_numpy(g.astype(np.complex64)).to(dev)
-    step = M.ops.DecodeStep(t(rng.normal(size=Dd) * 0.1), t(rng.normal(size=Dd) * 0.1), Gd, 1e-5, t(p), tq, tg,
-                            t(rng.normal(size=Dd)), Bd)
+    torch.manual_seed(1237)
+    ema = M.MultiHeadComplexEMA(Dd, ndim=Nd).to(dev).eval()          # the module's own initialisation
+    with torch.no_grad():
+        p, q, g = ema.coeffs()
+        step = M.ops.DecodeStep(torch.randn(Dd, device=dev) * 0.1, torch.randn(Dd, device=dev) * 0.1, Gd, 1e-5,
+                                p.squeeze(-1), q.squeeze(-1), g, ema.omega.reshape(-1), Bd)
     xs = [torch.randn(Bd, Dd, device=dev).to(torch.bfloat16) for _ in range(16)]
     with torch.no_grad():
         for i in range(args.warmup):

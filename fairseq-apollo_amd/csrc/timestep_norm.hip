@@ -202,9 +202,14 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   const int row16 = tid >> 4, l16 = tid & 15;
   const int gfirst = row16 < G ? row16 : G - 1;
   const Moments prior0 = {(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gfirst], P.prev_var[(size_t)b * G + gfirst]};
+  // HOIST (kThreads is a multiple of the vectors per token): vector j of a thread belongs to token
+  // tok0 + j * tps and always to the same features, so the loops below need no division
+  const int tok0 = tid / TPT, vi0 = tid - tok0 * TPT, tps = kThreads / TPT;
+  int g0;
+  if constexpr (LPGT > 0) g0 = vi0 / LPGT; else g0 = vi0 / LPG;
   float gam[VEC], bet[VEC];
   if (HOIST) {
-    const int f0 = (tid % TPT) * VEC;
+    const int f0 = vi0 * VEC;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
       gam[i] = P.gamma[f0 + i];
@@ -259,8 +264,8 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
         gv = group_sum<LPGT>(s2) * inv_dg;
       }
       if ((tid & (LPGT - 1)) == 0 && v < nvec) {
-        const int tok = v / TPT;
-        const int g = (v - tok * TPT) / LPGT;
+        const int tok = HOIST ? tok0 + j * tps : v / TPT;
+        const int g = HOIST ? g0 : (v - tok * TPT) / LPGT;
         s_mean[tok * G + g] = m;
         s_var[tok * G + g] = gv;
       }
@@ -367,18 +372,27 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
             const int i = i0 + u * kThreads;
             w[u] = i < nw ? get_rec(src0 + i) : tagged(0u, tag);
           }
+          // words that are not there yet are asked for again together, one round trip per round
+          uint32_t spins = 0;
+          for (;;) {
+            bool pending = false;
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) pending |= (uint32_t)(w[u] >> 32) != tag;
+            if (!pending) break;
+            if (++spins > kSpinLimit) {
+              publish_u32(&P.hdr->error, 1u);
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+              const int i = i0 + u * kThreads;
+              if ((uint32_t)(w[u] >> 32) != tag) w[u] = get_rec(src0 + i);
+            }
+          }
 #pragma unroll
           for (int u = 0; u < kBatch; ++u) {
             const int i = i0 + u * kThreads;
-            uint32_t spins = 0;
-            while ((uint32_t)(w[u] >> 32) != tag) {
-              __builtin_amdgcn_s_sleep(1);
-              w[u] = get_rec(src0 + i);
-              if (++spins > kSpinLimit) {
-                publish_u32(&P.hdr->error, 1u);
-                break;
-              }
-            }
             if (i < nw) s_lbw[i] = w[u];
           }
         }
@@ -430,9 +444,9 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   for (int j = 0; j < kNV; ++j) {
     const int v = j * kThreads + tid;
     if (v < nvec) {
-      const int tok = v / TPT;
-      const int vi = v - tok * TPT;
-      const int g = vi / LPG;
+      const int tok = HOIST ? tok0 + j * tps : v / TPT;
+      const int vi = HOIST ? vi0 : v - tok * TPT;
+      const int g = HOIST ? g0 : vi / LPG;
       const float m = s_mean[tok * G + g];
       const float r = s_var[tok * G + g];
       const bool masked = s_mask[tok] != 0;
