@@ -20,10 +20,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BM = 128, BN = 128, BK = 64;      // BM: block size of the causal bookkeeping and the small tile
 constexpr int PITCH = BK * 2 + 16;        // bytes per LDS row of BK 16-bit elements (+ 16 pad)
 constexpr int KP = BK / 8;                // 16-byte pieces per operand row and K step
-constexpr int NLP = BM * KP / 256;        // pieces per thread, operand and K step
 
 struct GemmArgs {
   const void* A;      // [batch][M][K] rows with pitch lda (elements), batch stride sa
@@ -54,10 +53,15 @@ __device__ __forceinline__ f32x4 mfma16<f16_t>(uint4 a, uint4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// C = alpha A B^T; TIn 16-bit, TOut float or TIn
-template <typename TIn, typename TOut>
-__global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
-  __shared__ __attribute__((aligned(16))) char lds[2 * (BM + BN) * PITCH];
+// C = alpha A B^T; TIn 16-bit, TOut float or TIn.  WM x WN waves, each a 64 x 64 block of the
+// (64 WM) x (64 WN) output tile.  The operand traffic from L2 per flop falls with the tile edge:
+// 2 x 2 waves (128 x 128) need 1/64 byte per flop, 4 x 4 waves (256 x 256) half of that.
+template <typename TIn, typename TOut, int WM, int WN>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G) {
+  constexpr int TM = 64 * WM, TN = 64 * WN, NT = 64 * WM * WN;
+  constexpr int NLA = TM * KP / NT, NLB = TN * KP / NT;          // 16-byte pieces per thread and K step
+  static_assert(TM * KP % NT == 0 && TN * KP % NT == 0, "tile rows must divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) char lds[];     // 2 x (TM + TN) x PITCH
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int m0, n0, bz;
   if (G.xcd) {
@@ -67,53 +71,55 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
     const int mtile = G.mt - 1 - rest % G.mt;
     rest /= G.mt;
     bz = rest * 8 + ((int)blockIdx.x & 7);
-    m0 = mtile * BM;
-    n0 = ntile * BN;
+    m0 = mtile * TM;
+    n0 = ntile * TN;
   } else {
-    m0 = blockIdx.y * BM;
-    n0 = blockIdx.x * BN;
+    m0 = blockIdx.y * TM;
+    n0 = blockIdx.x * TN;
     bz = blockIdx.z;
   }
-  if (G.causal == 1 && n0 > m0 + BM - 1 + G.kshift) return;      // entirely above the diagonal
+  if (G.causal == 1 && n0 > m0 + TM - 1 + G.kshift) return;      // entirely above the diagonal
   const int bo = bz / G.nin, bi = bz - bo * G.nin;
   const TIn* A = (const TIn*)G.A + bo * G.sa + bi * G.sai;
   const TIn* Bm = (const TIn*)G.Bm + bo * G.sb + bi * G.sbi;
   TOut* C = (TOut*)G.C + bo * G.sc + bi * G.sci;
   int Kend = G.K;
-  if (G.causal == 2) Kend = min(G.K, m0 + BM + G.kshift);
+  if (G.causal == 2) Kend = min(G.K, m0 + TM + G.kshift);
   if (Kend < 0) Kend = 0;
   const int nk = (Kend + BK - 1) / BK;
 
-  // global -> register staging: thread covers NLP x 16 bytes of A and of B per K step
-  const int lrow = tid / KP, lcol = (tid % KP) * 8;              // rows 0 .. 256/KP - 1 (+ h * 256/KP)
-  uint4 ra[NLP], rb[NLP];
+  // global -> register staging
+  const int lrow = tid / KP, lcol = (tid % KP) * 8;              // rows 0 .. NT/KP - 1 (+ h * NT/KP)
+  uint4 ra[NLA], rb[NLB];
   auto gload = [&](int kt) {
     const int k = kt * BK + lcol;
 #pragma unroll
-    for (int h = 0; h < NLP; ++h) {
-      const int r = lrow + h * (256 / KP);
+    for (int h = 0; h < NLA; ++h) {
+      const int r = lrow + h * (NT / KP);
       ra[h] = make_uint4(0, 0, 0, 0);
-      rb[h] = make_uint4(0, 0, 0, 0);
       if (m0 + r < G.M && k < Kend) ra[h] = *(const uint4*)(A + (int64_t)(m0 + r) * G.lda + k);
+    }
+#pragma unroll
+    for (int h = 0; h < NLB; ++h) {
+      const int r = lrow + h * (NT / KP);
+      rb[h] = make_uint4(0, 0, 0, 0);
       if (n0 + r < G.N && k < Kend) rb[h] = *(const uint4*)(Bm + (int64_t)(n0 + r) * G.ldb + k);
     }
   };
   auto lstore = [&](int buf) {
-    char* la = lds + buf * (BM + BN) * PITCH;
-    char* lb = la + BM * PITCH;
+    char* la = lds + buf * (TM + TN) * PITCH;
+    char* lb = la + TM * PITCH;
 #pragma unroll
-    for (int h = 0; h < NLP; ++h) {
-      const int r = lrow + h * (256 / KP);
-      *(uint4*)(la + r * PITCH + lcol * 2) = ra[h];
-      *(uint4*)(lb + r * PITCH + lcol * 2) = rb[h];
-    }
+    for (int h = 0; h < NLA; ++h) *(uint4*)(la + (lrow + h * (NT / KP)) * PITCH + lcol * 2) = ra[h];
+#pragma unroll
+    for (int h = 0; h < NLB; ++h) *(uint4*)(lb + (lrow + h * (NT / KP)) * PITCH + lcol * 2) = rb[h];
   };
   f32x4 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int wm = (wave / WN) * 64, wn = (wave % WN) * 64;
   const int fr = lane & 15, fk = (lane >> 4) * 16;                // fragment row, byte offset of the k block
 
   if (nk > 0) {
@@ -124,8 +130,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) gload(kt + 1);
-    const char* la = lds + buf * (BM + BN) * PITCH;
-    const char* lb = la + BM * PITCH;
+    const char* la = lds + buf * (TM + TN) * PITCH;
+    const char* lb = la + TM * PITCH;
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
       uint4 fa[4], fb[4];
@@ -144,11 +150,12 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
   // D layout: column = lane & 15, rows 4 (lane >> 4) + {0..3}
   const int cn = lane & 15, cr = (lane >> 4) * 4;
   constexpr int VW = 16 / (int)sizeof(TOut);                     // elements per 16-byte piece
-  const bool wide = (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + BN <= G.N;
+  constexpr int CP = TN + VW;                                    // row pitch of the staged tile in elements
+  constexpr bool fits = (size_t)TM * CP * sizeof(TOut) <= (size_t)2 * (TM + TN) * PITCH;
+  const bool wide = fits && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
   if (wide) {
     // whole tile through LDS (the operand buffers are free after the last barrier): rows leave as
-    // 16-byte pieces, BN * sizeof(TOut) contiguous bytes each
-    constexpr int CP = BN + VW;                                  // row pitch in elements
+    // 16-byte pieces, TN * sizeof(TOut) contiguous bytes each
     TOut* Cs = (TOut*)lds;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -158,10 +165,10 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
         for (int u = 0; u < 4; ++u)
           Cs[(wm + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
     __syncthreads();
-    constexpr int PPR = BN / VW;                                 // pieces per row
+    constexpr int PPR = TN / VW;                                 // pieces per row
 #pragma unroll
-    for (int u = 0; u < BM * PPR / 256; ++u) {
-      const int pi = tid + u * 256;
+    for (int u = 0; u < TM * PPR / NT; ++u) {
+      const int pi = tid + u * NT;
       const int r = pi / PPR, pc = pi - r * PPR;
       if (m0 + r < G.M)
         *(uint4*)(C + (int64_t)(m0 + r) * G.ldc + n0 + pc * VW) = *(const uint4*)(Cs + r * CP + pc * VW);
@@ -180,6 +187,24 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs G) {
         if (m < G.M) C[(int64_t)m * G.ldc + n] = from_float<TOut>(acc[i][j][u] * G.alpha);
       }
     }
+}
+
+template <typename TIn, typename TOut, int WM, int WN>
+void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hipStream_t s) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
+  constexpr int smem = 2 * (TM + TN) * PITCH;
+  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN>;
+  static bool attr_set = false;
+  if (!attr_set && smem > 64 * 1024) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    attr_set = true;
+  }
+  G.xcd = xcd ? 1 : 0;
+  G.mt = (int)ceil_div(M, TM);
+  G.nt = (int)ceil_div(N, TN);
+  const dim3 grid3((unsigned)G.nt, (unsigned)G.mt, (unsigned)batches);
+  const dim3 grid1((unsigned)((int64_t)G.nt * G.mt * batches));
+  hipLaunchKernelGGL(kern, xcd ? grid1 : grid3, dim3(64 * WM * WN), smem, s, G);
 }
 
 // v [B][L][Nh][H2] -> vt [B][Nh][H2][Lp] (Lp = L rounded up to 8, zero padded).  64 x 64 tiles:
@@ -230,43 +255,40 @@ __global__ __launch_bounds__(256) void transpose_v_kernel(const T* __restrict__ 
 }
 
 // causal softmax of fp32 scores into 16-bit probabilities; rows [outer][inner], pitch in elements
-// (multiples of 4).  The row is read once into registers (up to 16 values per thread, longer rows
-// loop); columns past the causal limit are written as zeros only up to `zcols`, the end of the
-// 128-column block the diagonal falls into (the second product never reads beyond it), unless the
-// caller wants the whole weight matrix (zero_all).
+// (multiples of 4).  One wave per row, four rows per workgroup: the row is read once into registers
+// (up to 32 values per lane = 2048 columns; longer rows are read three times), reductions stay
+// inside the wave.  Columns past the causal limit are written as zeros only up to `zcols`, the end of
+// the 256-column block the diagonal falls into (the second product, with row tiles of 128 or 256,
+// never reads beyond it), unless the caller wants the whole weight matrix (zero_all).
 template <typename TOut>
 __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restrict__ s, TOut* __restrict__ p, int outer,
                                                           int inner, int64_t spitch, int64_t ppitch, int pcols,
-                                                          int causal, int zero_all) {
-  __shared__ float red[4];
-  const int64_t row = blockIdx.x;
+                                                          int causal, int zero_all, int64_t nrows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
   const int r = (int)(row % outer);
   int n = causal ? inner - outer + r + 1 : inner;
   if (n < 0) n = 0;
   int zcols = pcols;
-  if (causal && !zero_all) zcols = min(pcols, ((n + BM - 1) / BM + 1) * BM);
+  if (causal && !zero_all) zcols = min(pcols, ((n + 255) / 256) * 256);
   const float* sp = s + row * spitch;
   TOut* pp = p + row * ppitch;
-  auto reduce = [&](float v, bool is_max) {
-    for (int m = 32; m >= 1; m >>= 1) {
-      const float o = __shfl_xor(v, m);
-      v = is_max ? fmaxf(v, o) : v + o;
-    }
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float t = red[0];
-    for (int i = 1; i < 4; ++i) t = is_max ? fmaxf(t, red[i]) : t + red[i];
-    return t;
+  auto wave_max = [](float v) {
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    return v;
   };
-  constexpr int NV = 4;                              // float4 per thread held in registers: 4096 columns
-  const bool in_regs = n <= 256 * 4 * NV;
-  float4 v[NV];
-  float m = -INFINITY;
-  if (in_regs) {
+  auto wave_sum = [](float v) {
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    return v;
+  };
+  constexpr int NV = 8;                              // float4 per lane held in registers: 2048 columns
+  if (n <= 64 * 4 * NV && sizeof(TOut) == 2) {
+    float4 v[NV];
+    float m = -INFINITY;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int j = (u * 256 + threadIdx.x) * 4;
+      const int j = (u * 64 + lane) * 4;
       v[u] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
       if (j < n) {
         v[u] = *(const float4*)(sp + j);
@@ -276,45 +298,48 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restric
       }
       m = fmaxf(m, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
     }
-  } else {
-    for (int j = threadIdx.x; j < n; j += 256) m = fmaxf(m, sp[j]);
-  }
-  m = reduce(m, true);
-  const bool dead = !(m > -INFINITY) || !(m < INFINITY);
-  float sum = 0.f;
-  if (!dead) {
-    if (in_regs) {
+    m = wave_max(m);
+    const bool dead = !(m > -INFINITY) || !(m < INFINITY);
+    float sum = 0.f;
+    if (!dead) {
 #pragma unroll
       for (int u = 0; u < NV; ++u) {
         v[u].x = __expf(v[u].x - m); v[u].y = __expf(v[u].y - m);
         v[u].z = __expf(v[u].z - m); v[u].w = __expf(v[u].w - m);
         sum += (v[u].x + v[u].y) + (v[u].z + v[u].w);
       }
-    } else {
-      for (int j = threadIdx.x; j < n; j += 256) sum += __expf(sp[j] - m);
     }
-  }
-  sum = reduce(sum, false);
-  const float c = (dead || sum == 0.f) ? 0.f : 1.0f / sum;
-  if (in_regs && sizeof(TOut) == 2) {
+    sum = wave_sum(sum);
+    const float c = (dead || sum == 0.f) ? 0.f : 1.0f / sum;
+    // live columns from registers (exp(-inf) = 0 covers the tail of a partial quad) ...
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int j = (u * 256 + threadIdx.x) * 4;
-      if (j < zcols) {
-        const bool live = !dead && j < n;             // exp(-inf) = 0 covers the tail of a partial quad
-        TOut o0 = from_float<TOut>(live ? v[u].x * c : 0.f), o1 = from_float<TOut>(live ? v[u].y * c : 0.f);
-        TOut o2 = from_float<TOut>(live ? v[u].z * c : 0.f), o3 = from_float<TOut>(live ? v[u].w * c : 0.f);
+      const int j = (u * 64 + lane) * 4;
+      if (j < zcols && j < n) {
+        TOut o0 = from_float<TOut>(v[u].x * c), o1 = from_float<TOut>(v[u].y * c);
+        TOut o2 = from_float<TOut>(v[u].z * c), o3 = from_float<TOut>(v[u].w * c);
         uint2 w;
         w.x = (uint32_t)__builtin_bit_cast(uint16_t, o0) | ((uint32_t)__builtin_bit_cast(uint16_t, o1) << 16);
         w.y = (uint32_t)__builtin_bit_cast(uint16_t, o2) | ((uint32_t)__builtin_bit_cast(uint16_t, o3) << 16);
         *(uint2*)(pp + j) = w;
       }
     }
-  } else {
-    for (int j = threadIdx.x; j < zcols; j += 256) {
-      const float e = (j < n && !dead) ? __expf(sp[j] - m) * c : 0.f;
-      pp[j] = from_float<TOut>(e);
-    }
+    // ... and zeros from the first whole quad past the limit up to zcols
+    for (int j = ((n + 3) / 4 + lane) * 4; j < zcols; j += 256) *(uint2*)(pp + j) = make_uint2(0u, 0u);
+    return;
+  }
+  float m = -INFINITY;
+  for (int j = lane; j < n; j += 64) m = fmaxf(m, sp[j]);
+  m = wave_max(m);
+  const bool dead = !(m > -INFINITY) || !(m < INFINITY);
+  float sum = 0.f;
+  if (!dead)
+    for (int j = lane; j < n; j += 64) sum += __expf(sp[j] - m);
+  sum = wave_sum(sum);
+  const float c = (dead || sum == 0.f) ? 0.f : 1.0f / sum;
+  for (int j = lane; j < zcols; j += 64) {
+    const float e = (j < n && !dead) ? __expf(sp[j] - m) * c : 0.f;
+    pp[j] = from_float<TOut>(e);
   }
 }
 
@@ -341,14 +366,9 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   G.sa = L * Nh * H1; G.sai = H1; G.sb = L * Nh * H1; G.sbi = H1; G.sc = Nh * L * Lp; G.sci = L * Lp;
   G.nin = (int)Nh; G.M = (int)L; G.N = (int)L; G.K = (int)H1; G.alpha = scale; G.causal = causal ? 1 : 0; G.kshift = 0;
   const bool xcd = BN_ % 8 == 0;
-  {
-    G.xcd = xcd ? 1 : 0; G.mt = (int)ceil_div(L, BM); G.nt = (int)ceil_div(L, BN);
-    const dim3 grid3((unsigned)G.nt, (unsigned)G.mt, (unsigned)BN_);
-    const dim3 grid1((unsigned)(G.nt * G.mt * BN_));
-    hipLaunchKernelGGL((gemm_nt_kernel<T, float>), xcd ? grid1 : grid3, dim3(256), 0, s, G);
-  }
-  hipLaunchKernelGGL(softmax_f32_kernel<T>, dim3((unsigned)(BN_ * L)), dim3(256), 0, s, S, P, (int)L, (int)L, Lp, Lp,
-                     (int)Lp, causal, w ? 1 : 0);
+  launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  hipLaunchKernelGGL(softmax_f32_kernel<T>, dim3((unsigned)ceil_div(BN_ * L, 4)), dim3(256), 0, s, S, P, (int)L, (int)L,
+                     Lp, Lp, (int)Lp, causal, w ? 1 : 0, (int64_t)(BN_ * L));
   if (w) {
     // the weights the reference returns: [B, Nh, L, L]
     hipMemcpy2DAsync(w, (size_t)L * sizeof(T), P, (size_t)Lp * sizeof(T), (size_t)L * sizeof(T), (size_t)(BN_ * L),
@@ -359,12 +379,9 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   G.lda = Lp; G.ldb = Lp; G.ldc = Nh * H2;
   G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = Nh * H2 * Lp; G.sbi = H2 * Lp; G.sc = L * Nh * H2; G.sci = H2;
   G.M = (int)L; G.N = (int)H2; G.K = (int)Lp; G.alpha = 1.0f; G.causal = causal ? 2 : 0;
-  {
-    G.xcd = xcd ? 1 : 0; G.mt = (int)ceil_div(L, BM); G.nt = (int)ceil_div(H2, BN);
-    const dim3 grid3((unsigned)G.nt, (unsigned)G.mt, (unsigned)BN_);
-    const dim3 grid1((unsigned)(G.nt * G.mt * BN_));
-    hipLaunchKernelGGL((gemm_nt_kernel<T, T>), xcd ? grid1 : grid3, dim3(256), 0, s, G);
-  }
+  // the second product carries the flops: 256 x 256 tiles when the problem has that many rows and columns
+  if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4>(G, L, H2, BN_, xcd, s);
+  else launch_gemm<T, T, 2, 2>(G, L, H2, BN_, xcd, s);
   MEGA_CHECK_LAUNCH("attention_fwd (matrix-core path)");
   return MEGA_OK;
 }
