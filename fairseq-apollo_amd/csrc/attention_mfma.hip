@@ -8,9 +8,10 @@
 //   y = P v                the same NT GEMM against v^T (v is transposed once through LDS); causal:
 //                          the reduction stops at the diagonal
 //
-// The GEMM: 128 x 128 output tile per workgroup (4 waves, 64 x 64 each as 4 x 4 MFMA blocks),
+// The GEMM: (64 WM) x (64 WN) output tile per workgroup of WM x WN waves (64 x 64 each as 4 x 4 MFMA
+// blocks): 128 x 128 for the scores, 256 x 256 for the second product, which carries the flops.
 // K step 64, operands staged through LDS with a 144-byte row pitch (conflict-free 16-byte reads),
-// register prefetch of the next K step.
+// register prefetch of the next K step, all tiles of one batch entry on one XCD, epilogue through LDS.
 #include "common.h"
 
 namespace mega {
