@@ -58,7 +58,7 @@ def test_causal(out_layout, time_major, cplx, B, D, N, L):
 
 
 @pytest.mark.parametrize("time_major", [False, True])
-@pytest.mark.parametrize("L1,L2", [(1024, 512), (1000, 1048), (288, 300)])
+@pytest.mark.parametrize("L1,L2", [(1024, 512), (1000, 1048), (288, 300), (2048, 4096)])
 def test_carried_state(time_major, L1, L2):
     rng = np.random.default_rng(32)
     B, D, N = 2, 32, 16
