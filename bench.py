@@ -176,6 +176,50 @@ def bench_attention(args):
     }))
 
 
+def bench_layer(args):
+    """configs[4]: one Mega2 layer forward (TimestepNorm -> CEMA -> chunked causal attention with
+    rotary -> gates, then TimestepNorm -> SwiGLU), L = 8192, D = 2048, S = 512, E = 4096, chunk 2048,
+    4 heads, SwiGLU hidden 5632, bf16.  The projections are library GEMMs; the rest runs in the HIP
+    library.  Flops: the dense projections plus the causal half of the attention products."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    L4, D4, S4, E4, N4, Hf, C4, heads = 8192, 2048, 512, 4096, 16, 5632, 2048, 4
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1238)
+    blk = M.Mega2Layer(D4, S4, E4, N4, Hf, C4, norm_num_groups=16, num_heads=heads, moving_act='silu')
+    blk = blk.to(dev).to(torch.bfloat16).eval()
+    xs = [torch.randn(1, L4, D4, device=dev).to(torch.bfloat16) for _ in range(4)]
+    with torch.no_grad():
+        for i in range(args.warmup):
+            blk(xs[i % 4])
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        a.record()
+        for i in range(args.steps):
+            blk(xs[i % 4])
+        b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms = max(wall * 1e3, a.elapsed_time(b)) / args.steps
+    gemm = 2 * L4 * D4 * (E4 + (S4 + E4 + 2 * D4)) + 2 * L4 * E4 * D4 + 3 * 2 * L4 * D4 * Hf
+    nchunk = L4 // C4
+    attn = nchunk * heads * C4 * (C4 + 1) * (S4 // heads + E4 // heads)
+    tf = (gemm + attn) / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "Mega2 layer tokens/sec @B1xL8192xD2048", "value": L4 / (ms * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[4]: one Mega2 layer, L=8192 D=2048 z=512 h=4096 chunk=2048 4 heads, "
+                               "SwiGLU 5632"},
+        "roofline": {"bound": "mfma", "kernel": "whole layer (library GEMMs + HIP kernels)", "achieved": tf,
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0, "traffic": None,
+                     "gemm_flops": gemm, "attention_flops_causal": attn},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,9 +230,10 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention"], default="block",
-                    help="block: the headline TimestepNorm -> EMA block (default); decode / attention: the "
-                         "decode step of configs[3] / the chunk attention of configs[4], one JSON line each")
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer"], default="block",
+                    help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
+                         "the decode step of configs[3] / the chunk attention / the whole layer of configs[4], "
+                         "one JSON line each")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -198,6 +243,8 @@ def main():
         return bench_decode(args)
     if args.workload == "attention":
         return bench_attention(args)
+    if args.workload == "layer":
+        return bench_layer(args)
 
     import numpy as np
     import torch

@@ -185,7 +185,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         residual = x
         x = self.norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
         v = F.silu(self.v_proj(x))
-        mx = self.move(x.transpose(1, 2), padding_mask, incremental_state).transpose(1, 2)
+        mx = self.move(x.transpose(1, 2), padding_mask, incremental_state, out_layout="input").transpose(1, 2)
         mx = self.move_act(mx)
         base = self.mx_proj(mx)
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)

@@ -126,8 +126,11 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         return y.unsqueeze(-1), h
 
     def forward(self, x, padding_mask: Optional[Tensor] = None,
-                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None) -> Tensor:
-        """x: [B, D, L]; padding_mask: [B, L] with 1 / True at padding; returns [B, D, L]."""
+                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None,
+                out_layout: str = "rows") -> Tensor:
+        """x: [B, D, L]; padding_mask: [B, L] with 1 / True at padding; returns [B, D, L]: contiguous
+        rows (what the reference returns) or, with out_layout="input", in x's own strides (a caller
+        that hands over a transposed [B, L, D] view and transposes back gets a contiguous result)."""
         _no_grad_only(self, x)
         bsz, embed_dim, seq_len = x.size()
         assert embed_dim == self.embed_dim
@@ -137,11 +140,11 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         if incremental_state is not None:
             saved_state = self._get_input_buffer(incremental_state)
             h = saved_state['prev_state'] if 'prev_state' in saved_state else None
-            out, h = layer(x, padding_mask, h, want_state=True)
+            out, h = layer(x, padding_mask, h, want_state=True, out_layout=out_layout)
             saved_state['prev_state'] = h
             self._set_input_buffer(incremental_state, saved_state)
         else:
-            out, _ = layer(x, padding_mask, None, want_state=False)
+            out, _ = layer(x, padding_mask, None, want_state=False, out_layout=out_layout)
         return out
 
     def _prepared_layer(self) -> "ops.PreparedEMA":
