@@ -20,6 +20,7 @@ SOURCES = [
     "ema_mfma.hip",
     "decode.hip",
     "elementwise.hip",
+    "gate_glue.hip",
     "attention.hip",
     "attention_mfma.hip",
     "long_conv.hip",

@@ -1,0 +1,307 @@
+// Elementwise and per-token glue of the gated-attention layer
+// (fairseq/modules/moving_average_gated_attention.py:322-330, 407-412): the pieces between the
+// projections and the attention product.  Every kernel is a single streaming pass in fp32
+// registers with one rounding at the store; operands are rows of a wider projection output, so
+// each takes its own row stride and the split of that output never needs a copy.
+//
+//   rms_norm   y = x / sqrt(mean(x^2) + eps) * weight                      (one wave per token)
+//   gate_qk    q, k = rotary(normalize(z) * gamma[i] + beta[i])             (one wave per token)
+//   gate_mul   y = a * silu(r)
+//   gate_out   y = residual + sigmoid(u) * (silu(hx + hp) - residual)
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kRowThreads = 256;                 // 4 waves, one token each
+constexpr int kRowsPerWg = kRowThreads / 64;
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(kRowThreads) void rms_norm_kernel(const T* __restrict__ x, int64_t xs,
+                                                               const float* __restrict__ w, T* __restrict__ y,
+                                                               int64_t T_, int D, float eps) {
+  using V = Vec<T, VEC>;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const T* row = x + t * xs;
+  float ss = 0.f;
+  for (int j = lane * VEC; j < D; j += 64 * VEC) {
+    const V v = *(const V*)(row + j);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float f = to_float(v.v[i]);
+      ss = fmaf(f, f, ss);
+    }
+  }
+  const float r = rsqrtf(wave_sum(ss) / (float)D + eps);
+  T* out = y + t * (int64_t)D;
+  for (int j = lane * VEC; j < D; j += 64 * VEC) {
+    const V v = *(const V*)(row + j);   // second read of a row this wave has just pulled in
+    V o;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float g = w ? w[j + i] : 1.0f;
+      o.v[i] = from_float<T>(to_float(v.v[i]) * r * g);
+    }
+    *(V*)(out + j) = o;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One wave per token: L2 norm over the S features, the two affine maps, then the rotation of
+// feature pairs (2i, 2i+1) of each head by pos * freqs[i]  (relative_positional_bias.py:86-92),
+// pos = pos0 + token index within its chunk.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kRowThreads) void gate_qk_kernel(const T* __restrict__ z, int64_t zs,
+                                                              const float* __restrict__ gamma,
+                                                              const float* __restrict__ beta,
+                                                              const float* __restrict__ freqs, T* __restrict__ q,
+                                                              T* __restrict__ k, int64_t T_, int S, int Hd,
+                                                              int64_t chunk, int64_t pos0, float eps) {
+  using V = Vec<T, VEC>;
+  static_assert(VEC % 2 == 0, "pairs of features stay inside one vector");
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (t >= T_) return;
+  const T* row = z + t * zs;
+  float ss = 0.f;
+  for (int j = lane * VEC; j < S; j += 64 * VEC) {
+    const V v = *(const V*)(row + j);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float f = to_float(v.v[i]);
+      ss = fmaf(f, f, ss);
+    }
+  }
+  const float inv = 1.0f / fmaxf(sqrtf(wave_sum(ss)), eps);   // F.normalize: x / max(|x|, eps)
+  const float pos = (float)(pos0 + t % chunk);
+  T* qo = q + t * (int64_t)S;
+  T* ko = k + t * (int64_t)S;
+  for (int j = lane * VEC; j < S; j += 64 * VEC) {
+    const V v = *(const V*)(row + j);
+    V oq, ok;
+#pragma unroll
+    for (int i = 0; i < VEC; i += 2) {
+      const int f = j + i;
+      float sn, cs;
+      sincosf(pos * freqs[(f % Hd) >> 1], &sn, &cs);
+      const float z0 = to_float(v.v[i]) * inv, z1 = to_float(v.v[i + 1]) * inv;
+      const float q0 = fmaf(z0, gamma[f], beta[f]), q1 = fmaf(z1, gamma[f + 1], beta[f + 1]);
+      const float k0 = fmaf(z0, gamma[S + f], beta[S + f]), k1 = fmaf(z1, gamma[S + f + 1], beta[S + f + 1]);
+      oq.v[i] = from_float<T>(q0 * cs - q1 * sn);
+      oq.v[i + 1] = from_float<T>(q0 * sn + q1 * cs);
+      ok.v[i] = from_float<T>(k0 * cs - k1 * sn);
+      ok.v[i + 1] = from_float<T>(k0 * sn + k1 * cs);
+    }
+    *(V*)(qo + j) = oq;
+    *(V*)(ko + j) = ok;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Row-strided elementwise kernels: blockIdx.x walks rows, threads walk the row in vectors.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_mul_kernel(const T* __restrict__ a, int64_t as, const T* __restrict__ r,
+                                                       int64_t rs, T* __restrict__ y, int64_t T_, int E) {
+  using V = Vec<T, VEC>;
+  for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
+    const T* ar = a + t * as;
+    const T* rr = r + t * rs;
+    T* yr = y + t * (int64_t)E;
+    for (int j = threadIdx.x * VEC; j < E; j += 256 * VEC) {
+      const V av = *(const V*)(ar + j);
+      const V rv = *(const V*)(rr + j);
+      V o;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) o.v[i] = from_float<T>(to_float(av.v[i]) * silu_f(to_float(rv.v[i])));
+      *(V*)(yr + j) = o;
+    }
+  }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_out_kernel(const T* __restrict__ res, int64_t ress,
+                                                       const T* __restrict__ u, int64_t us, const T* __restrict__ hx,
+                                                       int64_t hxs, const T* __restrict__ hp, int64_t hps,
+                                                       T* __restrict__ y, int64_t T_, int D) {
+  using V = Vec<T, VEC>;
+  for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
+    const T* r0 = res + t * ress;
+    const T* u0 = u + t * us;
+    const T* x0 = hx + t * hxs;
+    const T* p0 = hp + t * hps;
+    T* yr = y + t * (int64_t)D;
+    for (int j = threadIdx.x * VEC; j < D; j += 256 * VEC) {
+      const V rv = *(const V*)(r0 + j);
+      const V uv = *(const V*)(u0 + j);
+      const V xv = *(const V*)(x0 + j);
+      const V pv = *(const V*)(p0 + j);
+      V o;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float rr = to_float(rv.v[i]);
+        const float h = silu_f(to_float(xv.v[i]) + to_float(pv.v[i]));
+        o.v[i] = from_float<T>(fmaf(sigmoid_f(to_float(uv.v[i])), h - rr, rr));
+      }
+      *(V*)(yr + j) = o;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+inline bool vec_ok(const void* p, int64_t stride, size_t elem, int vec) {
+  return ((uintptr_t)p % (elem * vec)) == 0 && stride % vec == 0;
+}
+
+inline unsigned row_grid(int64_t T_) {
+  const int64_t cap = 256 * 16;
+  return (unsigned)(T_ < cap ? T_ : cap);
+}
+
+template <typename T>
+int launch_rms_norm(const void* x, int64_t xs, const float* w, void* y, int64_t T_, int64_t D, float eps,
+                    hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const unsigned grid = (unsigned)ceil_div(T_, kRowsPerWg);
+  if (D % VEC == 0 && vec_ok(x, xs, sizeof(T), VEC) && vec_ok(y, D, sizeof(T), VEC))
+    hipLaunchKernelGGL((rms_norm_kernel<T, VEC>), dim3(grid), dim3(kRowThreads), 0, s, (const T*)x, xs, w, (T*)y, T_,
+                       (int)D, eps);
+  else
+    hipLaunchKernelGGL((rms_norm_kernel<T, 1>), dim3(grid), dim3(kRowThreads), 0, s, (const T*)x, xs, w, (T*)y, T_,
+                       (int)D, eps);
+  MEGA_CHECK_LAUNCH("rms_norm_fwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_gate_qk(const void* z, int64_t zs, const float* gamma, const float* beta, const float* freqs, void* q,
+                   void* k, int64_t T_, int64_t S, int64_t Hd, int64_t chunk, int64_t pos0, float eps,
+                   hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const unsigned grid = (unsigned)ceil_div(T_, kRowsPerWg);
+  if (S % VEC == 0 && vec_ok(z, zs, sizeof(T), VEC) && vec_ok(q, S, sizeof(T), VEC) && vec_ok(k, S, sizeof(T), VEC))
+    hipLaunchKernelGGL((gate_qk_kernel<T, VEC>), dim3(grid), dim3(kRowThreads), 0, s, (const T*)z, zs, gamma, beta,
+                       freqs, (T*)q, (T*)k, T_, (int)S, (int)Hd, chunk, pos0, eps);
+  else {
+    MEGA_REQUIRE(vec_ok(z, zs, sizeof(T), 2) && vec_ok(q, S, sizeof(T), 2) && vec_ok(k, S, sizeof(T), 2), MEGA_ERR_ARG,
+                 "gate_qk_fwd: rows must start on an even element (feature pairs are moved together)");
+    hipLaunchKernelGGL((gate_qk_kernel<T, 2>), dim3(grid), dim3(kRowThreads), 0, s, (const T*)z, zs, gamma, beta,
+                       freqs, (T*)q, (T*)k, T_, (int)S, (int)Hd, chunk, pos0, eps);
+  }
+  MEGA_CHECK_LAUNCH("gate_qk_fwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_gate_mul(const void* a, int64_t as, const void* r, int64_t rs, void* y, int64_t T_, int64_t E,
+                    hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  if (E % VEC == 0 && vec_ok(a, as, sizeof(T), VEC) && vec_ok(r, rs, sizeof(T), VEC) && vec_ok(y, E, sizeof(T), VEC))
+    hipLaunchKernelGGL((gate_mul_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)a, as, (const T*)r,
+                       rs, (T*)y, T_, (int)E);
+  else
+    hipLaunchKernelGGL((gate_mul_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)a, as, (const T*)r, rs,
+                       (T*)y, T_, (int)E);
+  MEGA_CHECK_LAUNCH("gate_mul_fwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_gate_out(const void* res, int64_t ress, const void* u, int64_t us, const void* hx, int64_t hxs,
+                    const void* hp, int64_t hps, void* y, int64_t T_, int64_t D, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  if (D % VEC == 0 && vec_ok(res, ress, sizeof(T), VEC) && vec_ok(u, us, sizeof(T), VEC) &&
+      vec_ok(hx, hxs, sizeof(T), VEC) && vec_ok(hp, hps, sizeof(T), VEC) && vec_ok(y, D, sizeof(T), VEC))
+    hipLaunchKernelGGL((gate_out_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)res, ress,
+                       (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)y, T_, (int)D);
+  else
+    hipLaunchKernelGGL((gate_out_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)res, ress, (const T*)u,
+                       us, (const T*)hx, hxs, (const T*)hp, hps, (T*)y, T_, (int)D);
+  MEGA_CHECK_LAUNCH("gate_out_fwd");
+  return MEGA_OK;
+}
+
+bool known_dtype(int dtype) { return dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16; }
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+#define MEGA_GLUE_DISPATCH(fn, ...)                 \
+  switch (dtype) {                                  \
+    case MEGA_F32: return fn<float>(__VA_ARGS__);   \
+    case MEGA_BF16: return fn<bf16_t>(__VA_ARGS__); \
+    default: return fn<f16_t>(__VA_ARGS__);         \
+  }
+
+extern "C" int mega_rms_norm_fwd(const void* x, int64_t x_stride, const float* weight, void* y, int dtype, int64_t T_,
+                                 int64_t D, double eps, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "rms_norm_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && D >= 1 && D < (1ll << 30), MEGA_ERR_ARG, "rms_norm_fwd: bad sizes T=%lld D=%lld",
+               (long long)T_, (long long)D);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && y, MEGA_ERR_ARG, "rms_norm_fwd: null pointer argument");
+  MEGA_REQUIRE(x_stride >= D, MEGA_ERR_ARG, "rms_norm_fwd: row stride %lld below the row length %lld",
+               (long long)x_stride, (long long)D);
+  MEGA_REQUIRE(ceil_div(T_, kRowsPerWg) < (1ll << 31), MEGA_ERR_ARG, "rms_norm_fwd: too many rows");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_rms_norm, x, x_stride, weight, y, T_, D, (float)eps, s);
+}
+
+extern "C" int mega_gate_qk_fwd(const void* z, int64_t z_stride, const float* gamma, const float* beta,
+                                const float* freqs, void* q, void* k, int dtype, int64_t T_, int64_t S,
+                                int64_t heads, int64_t chunk, int64_t pos0, double eps, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_qk_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && S >= 2 && S < (1ll << 30) && heads >= 1 && chunk >= 1 && pos0 >= 0, MEGA_ERR_ARG,
+               "gate_qk_fwd: bad sizes T=%lld S=%lld heads=%lld chunk=%lld pos0=%lld", (long long)T_, (long long)S,
+               (long long)heads, (long long)chunk, (long long)pos0);
+  MEGA_REQUIRE(S % heads == 0 && (S / heads) % 2 == 0, MEGA_ERR_ARG,
+               "gate_qk_fwd: S=%lld must split into %lld heads of even size", (long long)S, (long long)heads);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(z && gamma && beta && freqs && q && k, MEGA_ERR_ARG, "gate_qk_fwd: null pointer argument");
+  MEGA_REQUIRE(z_stride >= S, MEGA_ERR_ARG, "gate_qk_fwd: row stride %lld below the row length %lld",
+               (long long)z_stride, (long long)S);
+  MEGA_REQUIRE(ceil_div(T_, kRowsPerWg) < (1ll << 31), MEGA_ERR_ARG, "gate_qk_fwd: too many rows");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_gate_qk, z, z_stride, gamma, beta, freqs, q, k, T_, S, S / heads, chunk, pos0, (float)eps,
+                     s);
+}
+
+extern "C" int mega_gate_mul_fwd(const void* a, int64_t a_stride, const void* r, int64_t r_stride, void* y, int dtype,
+                                 int64_t T_, int64_t E, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_mul_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && E >= 1 && E < (1ll << 30), MEGA_ERR_ARG, "gate_mul_fwd: bad sizes T=%lld E=%lld",
+               (long long)T_, (long long)E);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(a && r && y, MEGA_ERR_ARG, "gate_mul_fwd: null pointer argument");
+  MEGA_REQUIRE(a_stride >= E && r_stride >= E, MEGA_ERR_ARG, "gate_mul_fwd: a row stride is below the row length");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_gate_mul, a, a_stride, r, r_stride, y, T_, E, s);
+}
+
+extern "C" int mega_gate_out_fwd(const void* residual, int64_t residual_stride, const void* u, int64_t u_stride,
+                                 const void* hx, int64_t hx_stride, const void* hp, int64_t hp_stride, void* y,
+                                 int dtype, int64_t T_, int64_t D, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_out_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && D >= 1 && D < (1ll << 30), MEGA_ERR_ARG, "gate_out_fwd: bad sizes T=%lld D=%lld",
+               (long long)T_, (long long)D);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(residual && u && hx && hp && y, MEGA_ERR_ARG, "gate_out_fwd: null pointer argument");
+  MEGA_REQUIRE(residual_stride >= D && u_stride >= D && hx_stride >= D && hp_stride >= D, MEGA_ERR_ARG,
+               "gate_out_fwd: a row stride is below the row length");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_gate_out, residual, residual_stride, u, u_stride, hx, hx_stride, hp, hp_stride, y, T_, D,
+                     s);
+}

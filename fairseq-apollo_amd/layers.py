@@ -23,7 +23,7 @@ from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA,
 
 class RMSNorm(nn.Module):
     """x / sqrt(mean(x^2) + eps) * weight (fairseq/modules/norm_layer/layer_norm.py:41-59, which
-    wraps apex FusedRMSNorm); plain torch here, it is not on the measured path."""
+    wraps apex FusedRMSNorm); one wave per token in the HIP library."""
 
     def __init__(self, dim: int, elementwise_affine: bool = True, eps: float = 1e-5):
         super().__init__()
@@ -34,11 +34,8 @@ class RMSNorm(nn.Module):
             self.register_parameter("weight", None)
 
     def forward(self, x: Tensor) -> Tensor:
-        y = x.float()
-        y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.eps)
-        if self.weight is not None:
-            y = y * self.weight.float()
-        return y.to(x.dtype)
+        _no_grad_only(self, x)
+        return ops.rms_norm_fwd(x, self.weight, self.eps)
 
 
 class NormalizedFeedForwardNetwork(nn.Module):
@@ -189,23 +186,40 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         mx = self.move_act(mx)
         base = self.mx_proj(mx)
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
-        u = torch.sigmoid(u)
+        Nh = self.num_heads
+        if saved_state is None:
+            # whole chunks, nothing cached: q, k come out of one pass over z (normalise, the two
+            # affine maps, rotary with positions restarting in every chunk)
+            C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
+            nc = seq_len // C
+            q, k = ops.gate_qk_fwd(z, self.gamma + 1.0, self.beta, self.rel_pos_bias.freqs, Nh, C)
+            attn = self.efficient_attn(q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1),
+                                       v.reshape(bsz * nc, C, Nh, -1))
+        else:
+            attn = self._cached_attention(z, v, saved_state, incremental_state)
+        # the gates are applied where their operands are consumed: r on the way into the output
+        # projection, u and the residual mix after it
+        hp = self.h_proj(ops.gate_mul_fwd(attn.reshape(bsz, seq_len, self.hdim), r))
+        return ops.gate_out_fwd(residual, u, hx, hp), None
+
+    def _cached_attention(self, z: Tensor, v: Tensor, saved_state, incremental_state) -> Tensor:
+        """Attention with the partial-chunk key / value cache
+        (moving_average_gated_attention.py:332-372): keys are cached before the rotation, so the
+        whole context is rotated again at every call."""
+        bsz, seq_len = z.shape[:2]
+        Nh = self.num_heads
         z = F.normalize(z, p=2, dim=-1, eps=1e-5)
         z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
         q, k = torch.unbind(z, dim=2)
-        r = F.silu(r)
-        if saved_state is not None:
-            # partial-chunk key / value cache (moving_average_gated_attention.py:332-372)
-            if "prev_key" in saved_state:
-                k = torch.cat([saved_state["prev_key"], k], dim=1)
-                v = torch.cat([saved_state["prev_value"], v], dim=1)
-            if self.chunk_size < 0 or k.size(1) % self.chunk_size != 0:
-                saved_state["prev_key"], saved_state["prev_value"] = k, v
-            else:
-                saved_state.pop("prev_key", None)
-                saved_state.pop("prev_value", None)
-            self._set_input_buffer(incremental_state, saved_state)
-        Nh = self.num_heads
+        if "prev_key" in saved_state:
+            k = torch.cat([saved_state["prev_key"], k], dim=1)
+            v = torch.cat([saved_state["prev_value"], v], dim=1)
+        if self.chunk_size < 0 or k.size(1) % self.chunk_size != 0:
+            saved_state["prev_key"], saved_state["prev_value"] = k, v
+        else:
+            saved_state.pop("prev_key", None)
+            saved_state.pop("prev_value", None)
+        self._set_input_buffer(incremental_state, saved_state)
         ctx_len = k.size(1)
         if 1 < self.chunk_size < seq_len:
             nc = seq_len // self.chunk_size
@@ -222,16 +236,11 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), qidx).transpose(1, 2)
         k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
         if q4.size(1) == k4.size(1):
-            attn = self.efficient_attn(q4, k4, v4)
-        else:
-            # a few new queries against a longer cached context: right-aligned causal softmax
-            s = torch.einsum('bqnh,bknh->bnqk', q4.float(), k4.float()).to(q4.dtype)
-            w = ops.attention_softmax_fwd(s, 0.0, True)
-            attn = torch.einsum('bnqk,bknh->bqnh', w.float(), v4.float()).to(v4.dtype)
-        attn = attn.reshape(bsz, seq_len, self.hdim)
-        h = F.silu(hx + self.h_proj(attn * r))
-        out = torch.addcmul(residual, u, h - residual)
-        return out, None
+            return self.efficient_attn(q4, k4, v4)
+        # a few new queries against a longer cached context: right-aligned causal softmax
+        s = torch.einsum('bqnh,bknh->bnqk', q4.float(), k4.float()).to(q4.dtype)
+        w = ops.attention_softmax_fwd(s, 0.0, True)
+        return torch.einsum('bnqk,bknh->bqnh', w.float(), v4.float()).to(v4.dtype)
 
     def _get_input_buffer(self, incremental_state):
         result = self.get_incremental_state(incremental_state, "attn_state")

@@ -538,3 +538,98 @@ def swiglu(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         rc = lib.mega_swiglu_fwd(_ptr(ad), _ptr(bd), _ptr(y), _dtype_code(ad), ad.numel(), _stream(dev))
     _lib.check(rc, "swiglu_fwd")
     return y
+
+
+# ------------------------------------------------------------------------------------------------
+# per-token glue of the gated-attention layer (rows of a wider projection output are passed in
+# place: every input carries its own row stride)
+# ------------------------------------------------------------------------------------------------
+def _rows(t: torch.Tensor):
+    """(tensor whose data_ptr is the first row, row stride in elements) of a [..., W] tensor whose
+    leading axes walk memory uniformly; anything else is made contiguous first."""
+    t = t.detach()
+    ok = t.stride(-1) == 1 or t.shape[-1] == 1
+    for i in range(t.dim() - 2):
+        ok = ok and (t.shape[i] == 1 or t.stride(i) == t.stride(i + 1) * t.shape[i + 1])
+    if not ok:
+        t = t.contiguous()
+    if t.dim() == 1:
+        return t, t.shape[-1]
+    return t, t.stride(-2) if t.shape[-2] > 1 else max(t.stride(-2), t.shape[-1])
+
+
+def _ntok(t: torch.Tensor) -> int:
+    return t.numel() // t.shape[-1] if t.shape[-1] else 0
+
+
+def rms_norm_fwd(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """x * rsqrt(mean(x^2, -1) + eps) * weight (fairseq/modules/norm_layer/layer_norm.py:51-59)."""
+    dev = _need_gpu(x)
+    lib = _lib.load()
+    xr, xs = _rows(x)
+    w = None if weight is None else _f32c(weight)
+    if w is not None and w.numel() != x.shape[-1]:
+        raise RuntimeError("rms_norm_fwd: weight must hold one value per feature")
+    y = torch.empty(x.shape, dtype=x.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_rms_norm_fwd(_ptr(xr), xs, _ptr(w), _ptr(y), _dtype_code(xr), _ntok(x), x.shape[-1], float(eps),
+                                   _stream(dev))
+    _lib.check(rc, "rms_norm_fwd")
+    return y
+
+
+def gate_qk_fwd(z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, freqs: torch.Tensor, num_heads: int,
+                chunk: int, pos0: int = 0, eps: float = 1e-5):
+    """q, k = rotary(normalize(z) * gamma[i] + beta[i]), i = 0, 1
+    (moving_average_gated_attention.py:324-328, relative_positional_bias.py:86-97 with qidx = 0).
+    z: [..., S]; gamma, beta: [2, S] (gamma is the multiplier, "+ 1" included); freqs: [S/heads/2];
+    the position of a token is pos0 + its index modulo `chunk` along the flattened leading axes."""
+    dev = _need_gpu(z)
+    lib = _lib.load()
+    S = z.shape[-1]
+    zr, zs = _rows(z)
+    g, b, f = _f32c(gamma), _f32c(beta), _f32c(freqs)
+    if g.shape != (2, S) or b.shape != (2, S) or num_heads < 1 or S % num_heads or f.numel() * 2 * num_heads != S:
+        raise RuntimeError("gate_qk_fwd: gamma, beta must be [2, S] and freqs [S / heads / 2]")
+    q = torch.empty(z.shape, dtype=z.dtype, device=dev)
+    k = torch.empty(z.shape, dtype=z.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_gate_qk_fwd(_ptr(zr), zs, _ptr(g), _ptr(b), _ptr(f), _ptr(q), _ptr(k), _dtype_code(zr), _ntok(z),
+                                  S, num_heads, int(chunk), int(pos0), float(eps), _stream(dev))
+    _lib.check(rc, "gate_qk_fwd")
+    return q, k
+
+
+def gate_mul_fwd(a: torch.Tensor, r: torch.Tensor) -> torch.Tensor:
+    """a * silu(r) (moving_average_gated_attention.py:330, 407)."""
+    dev = _need_gpu(a, r)
+    lib = _lib.load()
+    if a.shape != r.shape or a.dtype != r.dtype:
+        raise RuntimeError("gate_mul_fwd: a and r must have the same shape and dtype")
+    ar, as_ = _rows(a)
+    rr, rs = _rows(r)
+    y = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_gate_mul_fwd(_ptr(ar), as_, _ptr(rr), rs, _ptr(y), _dtype_code(ar), _ntok(a), a.shape[-1],
+                                   _stream(dev))
+    _lib.check(rc, "gate_mul_fwd")
+    return y
+
+
+def gate_out_fwd(residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: torch.Tensor) -> torch.Tensor:
+    """residual + sigmoid(u) * (silu(hx + hp) - residual)
+    (moving_average_gated_attention.py:322, 409, 412)."""
+    dev = _need_gpu(residual, u, hx, hp)
+    lib = _lib.load()
+    if not (residual.shape == u.shape == hx.shape == hp.shape) or len({residual.dtype, u.dtype, hx.dtype, hp.dtype}) != 1:
+        raise RuntimeError("gate_out_fwd: all four operands must have the same shape and dtype")
+    r0, rs = _rows(residual)
+    u0, us = _rows(u)
+    x0, xs = _rows(hx)
+    p0, ps = _rows(hp)
+    y = torch.empty(residual.shape, dtype=residual.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_gate_out_fwd(_ptr(r0), rs, _ptr(u0), us, _ptr(x0), xs, _ptr(p0), ps, _ptr(y), _dtype_code(r0),
+                                   _ntok(residual), residual.shape[-1], _stream(dev))
+    _lib.check(rc, "gate_out_fwd")
+    return y

@@ -222,6 +222,34 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, voi
  * the reference's F.silu.                                                         */
 int mega_swiglu_fwd(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
 
+/* ------------------------------------------------------------------------ */
+/* Per-token glue of the gated-attention layer.  Inputs are [T, *] row-major with an
+ * element stride per row (so a slice of a wider projection output is passed in place);
+ * outputs are contiguous [T, *] of the same `dtype`; arithmetic in fp32.
+ *
+ * mega_rms_norm_fwd stands in for FusedRMSNorm.forward
+ *   (fairseq/modules/norm_layer/layer_norm.py:51-59): y = x * rsqrt(mean(x^2) + eps) * weight,
+ *   weight [D] fp32 or NULL.
+ * mega_gate_qk_fwd stands in for moving_average_gated_attention.py:324-328 followed by
+ *   RotaryEmbedding.forward (relative_positional_bias.py:86-97) with qidx = 0:
+ *   zn = z / max(|z|_2, eps); q = rot(zn * gamma[0] + beta[0]); k = rot(zn * gamma[1] + beta[1]);
+ *   gamma, beta [2, S] fp32 (gamma already holds the "+ 1"); rot turns features (2i, 2i+1) of
+ *   each of the `heads` slices of S/heads features by (pos0 + t % chunk) * freqs[i],
+ *   freqs [S/heads/2] fp32 (the module's buffer).
+ * mega_gate_mul_fwd: y = a * silu(r)                      (lines 330 and 407)
+ * mega_gate_out_fwd: y = residual + sigmoid(u) * (silu(hx + hp) - residual)
+ *                                                          (lines 322, 409 and 412)        */
+int mega_rms_norm_fwd(const void* x, int64_t x_stride, const float* weight, void* y, int dtype,
+                      int64_t T, int64_t D, double eps, void* stream);
+int mega_gate_qk_fwd(const void* z, int64_t z_stride, const float* gamma, const float* beta,
+                     const float* freqs, void* q, void* k, int dtype, int64_t T, int64_t S,
+                     int64_t heads, int64_t chunk, int64_t pos0, double eps, void* stream);
+int mega_gate_mul_fwd(const void* a, int64_t a_stride, const void* r, int64_t r_stride, void* y,
+                      int dtype, int64_t T, int64_t E, void* stream);
+int mega_gate_out_fwd(const void* residual, int64_t residual_stride, const void* u,
+                      int64_t u_stride, const void* hx, int64_t hx_stride, const void* hp,
+                      int64_t hp_stride, void* y, int dtype, int64_t T, int64_t D, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -119,3 +119,72 @@ def test_swiglu(dtype, n):
     a, a64 = rounded(rng.normal(size=n) * 3, dtype)
     b, b64 = rounded(rng.normal(size=n), dtype)
     assert rel_err(host(M.ops.swiglu(a, b)), O.swiglu(a64, b64)) < TOL[dtype]
+
+
+# ----------------------------------------------------------------------------------------------
+# per-token glue of the gated-attention layer; operands are slices of a wider row (the layout the
+# layer hands over) and odd sizes take the element-wise fallback
+# ----------------------------------------------------------------------------------------------
+def _wide(rng, shape, width, off, dtype):
+    """A [..., W] slice starting at column `off` of a [..., width] tensor, and its values."""
+    t, t64 = rounded(rng.normal(size=shape[:-1] + (width,)) * 1.5, dtype)
+    return t[..., off:off + shape[-1]], t64[..., off:off + shape[-1]]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,width,off", [((2, 33, 256), 256, 0), ((3, 17, 1024), 1304, 24), ((5, 77), 91, 3)])
+def test_rms_norm(dtype, shape, width, off):
+    rng = np.random.default_rng(41)
+    x, x64 = _wide(rng, shape, width, off, dtype)
+    w = rng.normal(size=shape[-1]) + 1
+    assert rel_err(host(M.ops.rms_norm_fwd(x, dev(w), 1e-5)), O.rms_norm(x64, w, 1e-5)) < TOL[dtype]
+    assert rel_err(host(M.ops.rms_norm_fwd(x, None, 1e-3)), O.rms_norm(x64, None, 1e-3)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,S,heads,chunk,width,off", [(2, 64, 128, 1, 64, 128, 0), (1, 96, 64, 4, 32, 200, 72),
+                                                         (3, 40, 36, 2, 40, 50, 6), (1, 4096, 512, 4, 2048, 512, 0)])
+def test_gate_qk(dtype, B, L, S, heads, chunk, width, off):
+    rng = np.random.default_rng(42)
+    z, z64 = _wide(rng, (B, L, S), width, off, dtype)
+    g = rng.normal(size=(2, S)) * 0.3 + 1
+    b = rng.normal(size=(2, S)) * 0.3
+    Hd = S // heads
+    freqs = (1.0 / (10000.0 ** (np.arange(0, Hd, 2) / Hd))).astype(np.float32)
+    q, k = M.ops.gate_qk_fwd(z, dev(g), dev(b), dev(freqs), heads, chunk)
+    zn = z64 / np.maximum(np.sqrt((z64 * z64).sum(-1, keepdims=True)), 1e-5)
+    for got, i in ((q, 0), (k, 1)):
+        a = (zn * g[i] + b[i]).reshape(B * (L // chunk), chunk, heads, Hd)
+        ref = O.rotary(a.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3).reshape(B, L, S)
+        # positions reach 2047 rad in fp32: the angle itself carries ~1e-4 absolute error there
+        assert rel_err(host(got), ref) < max(TOL[dtype], 5e-4)
+    # a zero row stays finite (the norm is clamped at eps)
+    zz = torch.zeros(1, 2, S, dtype=dtype, device=DEV)
+    q0, k0 = M.ops.gate_qk_fwd(zz, dev(g), dev(b), dev(freqs), heads, 2)
+    assert torch.isfinite(q0).all() and torch.isfinite(k0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,width,off", [((2, 50, 512), 1100, 80), ((4, 9, 35), 35, 0), ((1, 5000, 64), 72, 8)])
+def test_gate_mul_and_out(dtype, shape, width, off):
+    rng = np.random.default_rng(43)
+    a, a64 = rounded(rng.normal(size=shape), dtype)
+    r, r64 = _wide(rng, shape, width, off, dtype)
+    assert rel_err(host(M.ops.gate_mul_fwd(a, r)), a64 * O._silu(r64)) < TOL[dtype]
+    u, u64 = _wide(rng, shape, width, 0, dtype)
+    hx, hx64 = _wide(rng, shape, width, off, dtype)
+    hp, hp64 = rounded(rng.normal(size=shape), dtype)
+    res, res64 = rounded(rng.normal(size=shape), dtype)
+    ref = res64 + O._sigmoid(u64) * (O._silu(hx64 + hp64) - res64)
+    assert rel_err(host(M.ops.gate_out_fwd(res, u, hx, hp)), ref) < TOL[dtype]
+
+
+def test_glue_rejects_bad_arguments():
+    z = torch.zeros(2, 4, 30, device=DEV)
+    g = torch.ones(2, 30, device=DEV)
+    with pytest.raises(RuntimeError):
+        M.ops.gate_qk_fwd(z, g, g, torch.ones(5, device=DEV), 4, 4)       # 30 does not split into 4 heads
+    with pytest.raises(RuntimeError):
+        M.ops.gate_mul_fwd(torch.zeros(2, 8, device=DEV), torch.zeros(2, 9, device=DEV))
+    with pytest.raises(RuntimeError):
+        M.ops.rms_norm_fwd(torch.zeros(2, 8), None, 1e-5)                  # CPU tensor: no CPU path
