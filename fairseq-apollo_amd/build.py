@@ -16,6 +16,7 @@ LIB = os.path.join(HERE, "libmega_hip.so")
 SOURCES = [
     "capi.hip",
     "timestep_norm.hip",
+    "timestep_norm_bwd.hip",
     "ema_scan.hip",
     "ema_mfma.hip",
     "decode.hip",

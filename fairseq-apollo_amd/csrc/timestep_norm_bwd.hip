@@ -1,0 +1,408 @@
+// TimestepNorm backward (group and per-feature variants).
+//
+// Reference recurrences: fairseq/csrc/ops/timestep_norm.cc:318-450 (group) and :104-217
+// (per-feature, which is the group form with one channel per group and group_mean = x).
+// Walking the tokens of one (batch row, group) from the last to the first, the pair
+// (u_grad, v_grad) is carried; at an unmasked token with running count n, c1 = (n-1)/n, c2 = 1/n,
+// delta = group_mean - previous cumulative mean, r = cumrstd, ds = sum dy (x - cummean) w,
+// db = sum dy w over the group's channels:
+//     du = u_grad - r db,  dv = v_grad - r^3 ds / 2
+//     dux = c2 du + 2 c1 c2 dv delta,  dvx = c2 dv
+//     dx = dy r w + (dux + 2 dvx (x - group_mean)) / D
+//     u_grad <- c1 du - 2 c1 c2 dv delta,  v_grad <- c1 dv
+// The update of (u_grad, v_grad) is an affine map [[a, m], [0, a]] (.) + (bu, bv); such maps
+// compose into maps of the same shape, so the walk is split over token tiles:
+//   1. tsn_bwd_tile_kernel<.., 0>: per tile, ds / db per (token, group), the tile's composed map,
+//      and the tile's share of the gamma / beta gradients;
+//   2. tsn_bwd_carry_kernel: one thread per (row, group) walks the tile maps from the last tile
+//      to the first and leaves the pair that enters every tile (and the prev_mean / prev_var
+//      gradients at the end);
+//   3. tsn_bwd_tile_kernel<.., 1>: per tile, the same ds / db again, the walk inside the tile from
+//      its entering pair, then dx;
+//   4. tsn_bwd_param_kernel: sums the per-tile gamma / beta shares.
+// Masked tokens are skipped by the walk (identity map, dx = 0).  "Previous cumulative mean" is
+// cummean[t-1]; the forward kernels of this library store the carried mean at masked tokens, so
+// this is the state before token t also behind a masked token.
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxTileCells = 4096;   // tokens-per-tile * groups held in LDS
+
+struct TsnBwdParams {
+  const void* dy;
+  const void* x;
+  void* dx;
+  const float* mean_grad;
+  const float* var_grad;
+  const float* prev_mean;
+  const int64_t* count;
+  const float* group_mean;
+  const float* cummean;
+  const float* cumrstd;
+  const float* gamma;
+  const uint8_t* mask;
+  float* agg;     // [B, nt, G, 4]  composed map of every tile
+  float* state;   // [B, nt, G, 2]  (u_grad, v_grad) entering every tile (from the right)
+  float* part;    // [B * nt, 2, H] gamma / beta shares
+  float* prev_mean_grad;
+  float* prev_var_grad;
+  float* gamma_grad;
+  float* beta_grad;
+  int B, L, H, G, Dg, TT, nt;
+  int LPG;     // lanes that share one (token, group)
+  int PER;     // vectors per lane
+  int slots;   // lanes per token = G * LPG
+};
+
+// PHASE 0: tile maps + parameter shares; PHASE 1: dx.
+template <typename T, int VEC, int PHASE>
+__global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdParams P) {
+  using V = Vec<T, VEC>;
+  extern __shared__ float smem[];
+  const int G = P.G, H = P.H, TT = P.TT, Dg = P.Dg;
+  const int cells = TT * G;
+  float* s_r = smem;
+  float* s_u = s_r + cells;
+  float* s_ux = s_u + cells;
+  float* s_ds = s_ux + cells;    // PHASE 1: dux after the walk
+  float* s_db = s_ds + cells;    // PHASE 1: dvx after the walk
+  float* s_up0 = s_db + cells;   // [G] cumulative mean before the tile's first token
+  float* s_wg = s_up0 + G;       // [H] PHASE 0 only
+  float* s_bg = s_wg + H;
+  int* s_mask = (int*)(PHASE == 0 ? s_bg + H : s_up0 + G);   // [TT] + 1 counter
+  const int tid = threadIdx.x;
+  const int tile = blockIdx.x % P.nt;
+  const int b = blockIdx.x / P.nt;
+  const int t0 = tile * TT;
+  const int ntok = min(TT, P.L - t0);
+  const T* dy = (const T*)P.dy + ((size_t)b * P.L + t0) * H;
+  const T* x = (const T*)P.x + ((size_t)b * P.L + t0) * H;
+
+  // ---- statistics of the tile, mask, tokens that count after the tile
+  for (int i = tid; i < cells; i += kThreads) {
+    const int tok = i / G;
+    if (tok < ntok) {
+      const size_t o = ((size_t)b * P.L + t0) * G + i;
+      s_r[i] = P.cumrstd[o];
+      s_u[i] = P.cummean[o];
+      s_ux[i] = P.group_mean ? P.group_mean[o] : 0.f;
+    }
+  }
+  for (int g = tid; g < G; g += kThreads)
+    s_up0[g] = t0 == 0 ? P.prev_mean[(size_t)b * G + g] : P.cummean[((size_t)b * P.L + t0 - 1) * G + g];
+  if (PHASE == 0)
+    for (int c = tid; c < H; c += kThreads) { s_wg[c] = 0.f; s_bg[c] = 0.f; }
+  if (tid == 0) s_mask[TT] = 0;
+  for (int tok = tid; tok < TT; tok += kThreads)
+    s_mask[tok] = (tok >= ntok) || (P.mask && P.mask[(size_t)b * P.L + t0 + tok]);
+  __syncthreads();
+  if (P.mask) {
+    int later = 0;   // unmasked tokens behind this tile
+    for (int t = t0 + TT + tid; t < P.L; t += kThreads) later += P.mask[(size_t)b * P.L + t] ? 0 : 1;
+    if (later) atomicAdd(&s_mask[TT], later);
+  }
+
+  // ---- ds, db (and the group mean when it was not handed in) per (token, group)
+  const int items = ntok * P.slots;
+  const int span = VEC * P.PER;          // channels per lane
+  for (int i0 = 0; i0 < items; i0 += kThreads) {
+    const int i = i0 + tid;
+    const bool live = i < items;
+    const int tok = live ? i / P.slots : 0;
+    const int slot = live ? i - tok * P.slots : 0;
+    const int g = slot / P.LPG;
+    const int c0 = g * Dg + (slot - g * P.LPG) * span;
+    const int cell = tok * G + g;
+    float ds = 0.f, db = 0.f, sx = 0.f;
+    if (live) {
+      const float u = s_u[cell], r = s_r[cell];
+      const bool keep = !s_mask[tok];
+      for (int k = 0; k < P.PER; ++k) {
+        const int c = c0 + k * VEC;
+        const V dv = *(const V*)(dy + (size_t)tok * H + c);
+        const V xv = *(const V*)(x + (size_t)tok * H + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float d = to_float(dv.v[e]), xe = to_float(xv.v[e]), w = P.gamma[c + e];
+          ds = fmaf(d * (xe - u), w, ds);
+          db = fmaf(d, w, db);
+          sx += xe;
+          if (PHASE == 0 && keep) {
+            atomicAdd(&s_wg[c + e], d * (xe - u) * r);
+            atomicAdd(&s_bg[c + e], d);
+          }
+        }
+      }
+    }
+    for (int o = 1; o < P.LPG; o <<= 1) {
+      ds += __shfl_xor(ds, o);
+      db += __shfl_xor(db, o);
+      sx += __shfl_xor(sx, o);
+    }
+    if (live && slot == g * P.LPG) {
+      s_ds[cell] = ds;
+      s_db[cell] = db;
+      if (!P.group_mean) s_ux[cell] = sx / (float)Dg;
+    }
+  }
+  __syncthreads();
+
+  // ---- the walk over the tile's tokens, last to first, one thread per group
+  const int64_t n_end = P.count[b] - (P.mask ? s_mask[TT] : max(0, P.L - t0 - TT));
+  for (int g = tid; g < G; g += kThreads) {
+    int64_t n = n_end;                         // running count at the tile's last unmasked token
+    float a = 1.f, m = 0.f, bu = 0.f, bv = 0.f;
+    float ug = 0.f, vg = 0.f;
+    if (PHASE == 1) {
+      const size_t so = (((size_t)b * P.nt + tile) * G + g) * 2;
+      ug = P.state[so];
+      vg = P.state[so + 1];
+    }
+    for (int tok = ntok - 1; tok >= 0; --tok) {
+      const int cell = tok * G + g;
+      if (s_mask[tok]) {
+        if (PHASE == 1) { s_ds[cell] = 0.f; s_db[cell] = 0.f; }
+        continue;
+      }
+      const float c2 = 1.0f / (float)n, c1 = (float)(n - 1) * c2;
+      --n;
+      const float r = s_r[cell];
+      const float up = tok == 0 ? s_up0[g] : s_u[cell - G];
+      const float delta = s_ux[cell] - up;
+      const float e = 0.5f * r * r * r * s_ds[cell];
+      const float rdb = r * s_db[cell];
+      const float mj = -2.0f * c1 * c2 * delta;
+      if (PHASE == 0) {
+        const float buj = -c1 * rdb - mj * e, bvj = -c1 * e;
+        // this token's map after the maps of the tokens behind it
+        const float na = c1 * a, nm = c1 * m + mj * a;
+        const float nbu = c1 * bu + mj * bv + buj, nbv = c1 * bv + bvj;
+        a = na; m = nm; bu = nbu; bv = nbv;
+      } else {
+        const float du = ug - rdb, dv = vg - e;
+        s_ds[cell] = c2 * du - mj * dv;      // dux = c2 du + 2 c1 c2 dv delta
+        s_db[cell] = c2 * dv;                // dvx
+        ug = c1 * du + mj * dv;
+        vg = c1 * dv;
+      }
+    }
+    if (PHASE == 0) {
+      float4* dst = (float4*)P.agg + ((size_t)b * P.nt + tile) * G + g;
+      *dst = make_float4(a, m, bu, bv);
+    }
+  }
+  __syncthreads();
+
+  if (PHASE == 0) {
+    float* dst = P.part + ((size_t)b * P.nt + tile) * 2 * H;
+    for (int c = tid; c < H; c += kThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
+  } else {
+    T* dx = (T*)P.dx + ((size_t)b * P.L + t0) * H;
+    const float cg = 1.0f / (float)Dg;
+    for (int i = tid; i < items; i += kThreads) {
+      const int tok = i / P.slots;
+      const int slot = i - tok * P.slots;
+      const int g = slot / P.LPG;
+      const int c0 = g * Dg + (slot - g * P.LPG) * span;
+      const int cell = tok * G + g;
+      const float r = s_r[cell], ux = s_ux[cell];
+      const float a0 = s_ds[cell] * cg, a1 = 2.0f * s_db[cell] * cg;
+      const bool keep = !s_mask[tok];
+      for (int k = 0; k < P.PER; ++k) {
+        const int c = c0 + k * VEC;
+        const V dv = *(const V*)(dy + (size_t)tok * H + c);
+        const V xv = *(const V*)(x + (size_t)tok * H + c);
+        V o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float v = fmaf(to_float(dv.v[e]) * r, P.gamma[c + e], fmaf(a1, to_float(xv.v[e]) - ux, a0));
+          o.v[e] = from_float<T>(keep ? v : 0.f);
+        }
+        *(V*)(dx + (size_t)tok * H + c) = o;
+      }
+    }
+  }
+}
+
+__global__ void tsn_bwd_carry_kernel(const TsnBwdParams P) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P.B * P.G) return;
+  const int b = i / P.G, g = i - b * P.G;
+  float ug = P.mean_grad ? P.mean_grad[i] : 0.f;
+  float vg = P.var_grad ? P.var_grad[i] : 0.f;
+  for (int tile = P.nt - 1; tile >= 0; --tile) {
+    const size_t o = ((size_t)b * P.nt + tile) * P.G + g;
+    P.state[o * 2] = ug;
+    P.state[o * 2 + 1] = vg;
+    const float4 mp = ((const float4*)P.agg)[o];
+    const float nu = fmaf(mp.x, ug, fmaf(mp.y, vg, mp.z));
+    vg = fmaf(mp.x, vg, mp.w);
+    ug = nu;
+  }
+  P.prev_mean_grad[i] = ug;
+  P.prev_var_grad[i] = vg;
+}
+
+__global__ void tsn_bwd_param_kernel(const TsnBwdParams P) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;   // over 2 * H
+  if (c >= 2 * P.H) return;
+  const int ntile = P.B * P.nt;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int t = 0;
+  for (; t + 4 <= ntile; t += 4) {
+    s0 += P.part[(size_t)t * 2 * P.H + c];
+    s1 += P.part[(size_t)(t + 1) * 2 * P.H + c];
+    s2 += P.part[(size_t)(t + 2) * 2 * P.H + c];
+    s3 += P.part[(size_t)(t + 3) * 2 * P.H + c];
+  }
+  for (; t < ntile; ++t) s0 += P.part[(size_t)t * 2 * P.H + c];
+  const float s = (s0 + s1) + (s2 + s3);
+  if (c < P.H) P.gamma_grad[c] = s;
+  else P.beta_grad[c - P.H] = s;
+}
+
+struct BwdGeom {
+  int tt, nt, vec, lpg, per;
+  size_t agg_bytes, state_bytes, part_bytes;
+};
+
+bool bwd_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, BwdGeom* g) {
+  if (G > kMaxTileCells || H > 8192 || B * L >= (int64_t)1 << 31) return false;
+  const int64_t Dg = H / G;
+  const int full = dtype == MEGA_F32 ? 4 : 8;
+  g->vec = (Dg % full == 0) ? full : 1;
+  int64_t vecs = Dg / g->vec;          // vectors per (token, group)
+  int lpg = 1;
+  while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
+  g->lpg = lpg;
+  g->per = (int)(vecs / lpg);
+  int tt = (int)(kMaxTileCells / G);
+  if (tt > 32) tt = 32;
+  if (tt < 1) tt = 1;
+  g->tt = tt;
+  g->nt = (int)ceil_div(L, tt);
+  if (B * g->nt >= (int64_t)1 << 31) return false;
+  g->agg_bytes = align_up((size_t)B * g->nt * G * 16, 256);
+  g->state_bytes = align_up((size_t)B * g->nt * G * 8, 256);
+  g->part_bytes = align_up((size_t)B * g->nt * 2 * H * 4, 256);
+  return true;
+}
+
+template <typename T, int VEC>
+int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
+  const size_t cells = (size_t)P.TT * P.G;
+  const size_t lds0 = (5 * cells + P.G + 2 * (size_t)P.H) * 4 + (P.TT + 1) * 4;
+  const size_t lds1 = (5 * cells + P.G) * 4 + (P.TT + 1) * 4;
+  static bool attr0 = false, attr1 = false;
+  if (!attr0) {
+    (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    attr0 = true;
+  }
+  if (!attr1) {
+    (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              160 * 1024);
+    attr1 = true;
+  }
+  const dim3 grid((unsigned)(P.B * P.nt));
+  hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0>), grid, dim3(kThreads), lds0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (tile maps)");
+  hipLaunchKernelGGL(tsn_bwd_carry_kernel, dim3((unsigned)ceil_div((int64_t)P.B * P.G, 64)), dim3(64), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (carry)");
+  hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 1>), grid, dim3(kThreads), lds1, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (dx)");
+  hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 256)), dim3(256), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (parameters)");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_bwd(const TsnBwdParams& P, int vec, hipStream_t s) {
+  constexpr int FULL = 16 / (int)sizeof(T);
+  return vec == FULL ? launch_tiles<T, FULL>(P, s) : launch_tiles<T, 1>(P, s);
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" size_t mega_timestep_norm_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G) {
+  BwdGeom g;
+  if (B <= 0 || L <= 0 || H <= 0 || G <= 0 || H % G != 0 || !bwd_geometry(dtype, B, L, H, G, &g)) return 256;
+  return g.agg_bytes + g.state_bytes + g.part_bytes;
+}
+
+extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,
+                                            const void* x, int dtype, const float* prev_mean, const int64_t* count,
+                                            const float* group_mean, const float* cummean, const float* cumrstd,
+                                            const float* gamma, const uint8_t* mask, int64_t B, int64_t L, int64_t H,
+                                            int64_t G, void* x_grad, float* prev_mean_grad, float* prev_var_grad,
+                                            float* gamma_grad, float* beta_grad, void* workspace,
+                                            size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "timestep_norm_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && L >= 0 && H > 0 && G > 0 && H % G == 0, MEGA_ERR_ARG,
+               "timestep_norm_bwd: bad shape B=%ld L=%ld H=%ld G=%ld", (long)B, (long)L, (long)H, (long)G);
+  MEGA_REQUIRE(prev_mean_grad && prev_var_grad && gamma_grad && beta_grad, MEGA_ERR_ARG,
+               "timestep_norm_bwd: null gradient output");
+  hipStream_t s = (hipStream_t)stream;
+  if (B == 0 || L == 0) {
+    // nothing between the incoming state gradients and the outgoing ones
+    if (B > 0) {
+      if (mean_grad) hipMemcpyAsync(prev_mean_grad, mean_grad, (size_t)B * G * 4, hipMemcpyDeviceToDevice, s);
+      else hipMemsetAsync(prev_mean_grad, 0, (size_t)B * G * 4, s);
+      if (var_grad) hipMemcpyAsync(prev_var_grad, var_grad, (size_t)B * G * 4, hipMemcpyDeviceToDevice, s);
+      else hipMemsetAsync(prev_var_grad, 0, (size_t)B * G * 4, s);
+    }
+    hipMemsetAsync(gamma_grad, 0, (size_t)H * 4, s);
+    hipMemsetAsync(beta_grad, 0, (size_t)H * 4, s);
+    return MEGA_OK;
+  }
+  MEGA_REQUIRE(y_grad && x && x_grad && prev_mean && count && cummean && cumrstd && gamma, MEGA_ERR_ARG,
+               "timestep_norm_bwd: null pointer argument");
+  BwdGeom g;
+  MEGA_REQUIRE(bwd_geometry(dtype, B, L, H, G, &g), MEGA_ERR_UNSUPPORTED,
+               "timestep_norm_bwd: H=%ld G=%ld outside the supported envelope (H <= 8192, G <= %d)", (long)H, (long)G,
+               kMaxTileCells);
+  if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad) % 16) != 0)) {
+    g.vec = 1;
+    int64_t vecs = H / G;
+    int lpg = 1;
+    while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
+    g.lpg = lpg;
+    g.per = (int)(vecs / lpg);
+  }
+  const size_t need = g.agg_bytes + g.state_bytes + g.part_bytes;
+  MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
+               "timestep_norm_bwd: workspace of %zu bytes (16-byte aligned) needed", need);
+  char* w = (char*)workspace;
+  TsnBwdParams P;
+  P.dy = y_grad; P.x = x; P.dx = x_grad; P.mean_grad = mean_grad; P.var_grad = var_grad; P.prev_mean = prev_mean;
+  P.count = count; P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd; P.gamma = gamma; P.mask = mask;
+  P.agg = (float*)w; w += g.agg_bytes;
+  P.state = (float*)w; w += g.state_bytes;
+  P.part = (float*)w;
+  P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
+  P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
+  P.LPG = g.lpg; P.PER = g.per; P.slots = (int)G * g.lpg;
+  switch (dtype) {
+    case MEGA_F32: return launch_bwd<float>(P, g.vec, s);
+    case MEGA_BF16: return launch_bwd<bf16_t>(P, g.vec, s);
+    default: return launch_bwd<f16_t>(P, g.vec, s);
+  }
+}
+
+extern "C" int mega_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad, const void* x,
+                                      int dtype, const float* prev_mean, const int64_t* count, const float* cummean,
+                                      const float* cumrstd, const float* gamma, const uint8_t* mask, int64_t B,
+                                      int64_t L, int64_t H, void* x_grad, float* prev_mean_grad, float* prev_var_grad,
+                                      float* gamma_grad, float* beta_grad, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+  return mega_group_timestep_norm_bwd(y_grad, mean_grad, var_grad, x, dtype, prev_mean, count, nullptr, cummean,
+                                      cumrstd, gamma, mask, B, L, H, H, x_grad, prev_mean_grad, prev_var_grad,
+                                      gamma_grad, beta_grad, workspace, workspace_bytes, stream);
+}

@@ -272,6 +272,43 @@ class MultiHeadComplexEMA(BaseMovingLayer):
         return p, q, gamma
 
 
+class TimestepNormFunc(torch.autograd.Function):
+    """fairseq/modules/norm_layer/timestep_norm.py:14-66: the forward keeps (group_mean,) cummean,
+    cumrstd for the backward pass; count is an integer output without a gradient."""
+
+    @staticmethod
+    def forward(ctx, x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask=None, num_groups=None,
+                eps: float = 1e-5):
+        if num_groups is None:
+            y, count, mean, var, cummean, cumrstd = ops.timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma,
+                                                                          beta, padding_mask, eps)
+            ctx.save_for_backward(x, prev_mean, count, cummean, cumrstd, gamma, padding_mask)
+        else:
+            y, count, mean, var, group_mean, cummean, cumrstd = ops.group_timestep_norm_fwd(
+                x, prev_count, prev_mean, prev_var, gamma, beta, padding_mask, num_groups, eps)
+            ctx.save_for_backward(x, prev_mean, count, group_mean, cummean, cumrstd, gamma, padding_mask)
+        ctx.num_groups = num_groups
+        ctx.mark_non_differentiable(count)
+        return y, count, mean, var
+
+    @staticmethod
+    def backward(ctx, y_grad, _, mean_grad, var_grad):
+        if ctx.num_groups is None:
+            x, prev_mean, count, cummean, cumrstd, gamma, padding_mask = ctx.saved_tensors
+            grads = ops.timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma,
+                                          padding_mask)
+        else:
+            x, prev_mean, count, group_mean, cummean, cumrstd, gamma, padding_mask = ctx.saved_tensors
+            grads = ops.group_timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, group_mean, cummean,
+                                                cumrstd, gamma, padding_mask, ctx.num_groups)
+        x_grad, prev_mean_grad, prev_var_grad, gamma_grad, beta_grad = grads
+        return (x_grad, None, prev_mean_grad.to(prev_mean.dtype).view_as(prev_mean), prev_var_grad.view_as(prev_mean),
+                gamma_grad.to(gamma.dtype), beta_grad, None, None, None)
+
+
+timestep_norm = TimestepNormFunc.apply
+
+
 class TimestepNorm(nn.Module, IncrementalState):
     """Streaming cumulative (group) normalisation with a carried (count, mean, var) state
     (fairseq/modules/norm_layer/timestep_norm.py:71-167).  mean / var are carried in fp32."""
@@ -303,8 +340,8 @@ class TimestepNorm(nn.Module, IncrementalState):
 
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
                 incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None) -> Tensor:
-        _no_grad_only(self, x)
         batch_size = x.size(0)
+        train = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
         prev_mean = prev_var = prev_count = None
         saved_state = None
         if incremental_state is not None:
@@ -315,10 +352,19 @@ class TimestepNorm(nn.Module, IncrementalState):
                 prev_var = saved_state['prev_var']
                 prev_count = saved_state['prev_count']
         if prev_count is None or prev_mean is None or prev_var is None:
-            d_count, d_mean, d_var = self._prior_state(batch_size)
+            d_count, d_mean, d_var = self._prior_state(batch_size, train)
             prev_count = d_count if prev_count is None else prev_count
             prev_mean = d_mean if prev_mean is None else prev_mean
             prev_var = d_var if prev_var is None else prev_var
+        if train:
+            # the autograd path of the reference (timestep_norm.py:129-136): prior, weight + 1 and
+            # bias stay in the graph; statistics for the backward pass are kept
+            out, count, mean, var = timestep_norm(x, prev_count, prev_mean, prev_var, self.weight.float() + 1.0,
+                                                  self.bias.float(), padding_mask, self.num_groups, self.eps)
+            if incremental_state is not None:
+                saved_state['prev_mean'], saved_state['prev_var'], saved_state['prev_count'] = mean, var, count
+                self._set_input_buffer(incremental_state, saved_state)
+            return out
         gamma, beta = self._affine()
         if self.num_groups is None:
             out, count, mean, var, _, _ = ops.timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta,
@@ -334,8 +380,12 @@ class TimestepNorm(nn.Module, IncrementalState):
             self._set_input_buffer(incremental_state, saved_state)
         return out
 
-    def _prior_state(self, batch_size: int):
+    def _prior_state(self, batch_size: int, differentiable: bool = False):
         """(count[B], mean[B,G], var[B,G]) of the prior (timestep_norm.py:122-127); cached in eval mode."""
+        if differentiable:
+            return (self.prior_count.expand(batch_size).contiguous(),
+                    self.prior_mean.float().expand(batch_size, -1),
+                    torch.exp(self.prior_logv.float()).expand(batch_size, -1))
         key = batch_size
         if not self.training and key in self._prior_cache:
             return self._prior_cache[key]

@@ -268,6 +268,63 @@ def timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_m
     return y, count, mean, var, cm, cr
 
 
+def _tsn_bwd(name, y_grad, mean_grad, var_grad, x, prev_mean, count, group_mean, cummean, cumrstd, gamma,
+             padding_mask, G: int):
+    dev = _need_gpu(y_grad, mean_grad, var_grad, x, prev_mean, count, group_mean, cummean, cumrstd, gamma,
+                    padding_mask)
+    lib = _lib.load()
+    if x.dim() != 3 or y_grad.shape != x.shape:
+        raise RuntimeError(f"{name}: x and y_grad must be [B, L, H] of the same shape")
+    B, L, H = x.shape
+    if G <= 0 or H % G != 0:
+        raise RuntimeError(f"num_features={H} is not divisible by num_groups={G}")
+    xd = x.detach().contiguous()
+    dyd = y_grad.detach().to(xd.dtype).contiguous()
+    dt = _dtype_code(xd)
+    for nm, t in (("cummean", cummean), ("cumrstd", cumrstd)) + ((("group_mean", group_mean),) if group_mean is not None else ()):
+        if t.shape != (B, L, G) or t.dtype is not torch.float32:
+            raise RuntimeError(f"{name}: {nm} must be the forward's [B, L, G] float32 output")
+    f32 = lambda t: None if t is None else _f32c(t).reshape(B, G)
+    mg, vg, pm = f32(mean_grad), f32(var_grad), f32(prev_mean)
+    cnt = count.detach().to(torch.int64).contiguous()
+    if cnt.numel() != B:
+        raise RuntimeError(f"{name}: count must be [B]")
+    dx = torch.empty_like(xd)
+    dpm = torch.empty(B, G, dtype=torch.float32, device=dev)
+    dpv = torch.empty(B, G, dtype=torch.float32, device=dev)
+    dg = torch.empty(H, dtype=torch.float32, device=dev)
+    db = torch.empty(H, dtype=torch.float32, device=dev)
+    nws = lib.mega_timestep_norm_bwd_workspace_bytes(dt, B, L, H, G)
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, nws, stream)
+    m8 = _mask_u8(padding_mask, B, L)
+    gm = None if group_mean is None else group_mean.contiguous()
+    with _on_device(dev):
+        rc = lib.mega_group_timestep_norm_bwd(_ptr(dyd), _ptr(mg), _ptr(vg), _ptr(xd), dt, _ptr(pm), _ptr(cnt),
+                                              _ptr(gm), _ptr(cummean.contiguous()), _ptr(cumrstd.contiguous()),
+                                              _ptr(_f32c(gamma)), _ptr(m8), B, L, H, G, _ptr(dx), _ptr(dpm),
+                                              _ptr(dpv), _ptr(dg), _ptr(db), _ptr(ws), ws.numel(), stream)
+    _lib.check(rc, name)
+    return dx, dpm, dpv, dg, db
+
+
+def group_timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, group_mean, cummean, cumrstd, gamma,
+                            padding_mask, num_groups: int):
+    """-> (x_grad, prev_mean_grad[B,G], prev_var_grad[B,G], gamma_grad[H], beta_grad[H]); the state
+    and parameter gradients are fp32.  Reference: group_timestep_norm_bwd,
+    fairseq/csrc/ops/timestep_norm.cc:638-708 (recurrences at :318-450).  mean_grad / var_grad may
+    be None (zeros)."""
+    return _tsn_bwd("group_timestep_norm_bwd", y_grad, mean_grad, var_grad, x, prev_mean, count, group_mean, cummean,
+                    cumrstd, gamma, padding_mask, int(num_groups))
+
+
+def timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma, padding_mask):
+    """Per-feature form of group_timestep_norm_bwd.  Reference: timestep_norm_bwd,
+    fairseq/csrc/ops/timestep_norm.cc:512-566 (recurrences at :104-217)."""
+    return _tsn_bwd("timestep_norm_bwd", y_grad, mean_grad, var_grad, x, prev_mean, count, None, cummean, cumrstd,
+                    gamma, padding_mask, x.shape[-1])
+
+
 def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
     """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18."""
     if dropout != 0.0:

@@ -193,6 +193,32 @@ int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* pre
                            float* cummean, float* cumrstd, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/* backward: stands in for group_timestep_norm_bwd and timestep_norm_bwd
+ * (fairseq/csrc/ops/timestep_norm.cc:318-450 and :104-217, CUDA side
+ * ops/timestep_norm_kernel.cu; caller norm_layer/timestep_norm.py:45-66).
+ *   y_grad, x, x_grad [B,L,H] contiguous of `dtype`; mean_grad, var_grad [B,G] fp32 or NULL
+ *   (zeros); prev_mean [B,G]; count [B] = the forward's count output; group_mean (NULL:
+ *   recomputed from x), cummean, cumrstd [B,L,G] fp32 as the forward wrote them (at a masked
+ *   token cummean must hold the carried mean, which is what this library's forward stores);
+ *   gamma [H] fp32 (weight + 1).  Outputs: x_grad, prev_mean_grad, prev_var_grad [B,G],
+ *   gamma_grad, beta_grad [H] fp32.  The per-feature form has H in place of G.           */
+size_t mega_timestep_norm_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G);
+int mega_group_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,
+                                 const void* x, int dtype, const float* prev_mean,
+                                 const int64_t* count, const float* group_mean,
+                                 const float* cummean, const float* cumrstd, const float* gamma,
+                                 const uint8_t* mask, int64_t B, int64_t L, int64_t H, int64_t G,
+                                 void* x_grad, float* prev_mean_grad, float* prev_var_grad,
+                                 float* gamma_grad, float* beta_grad, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+int mega_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,
+                           const void* x, int dtype, const float* prev_mean, const int64_t* count,
+                           const float* cummean, const float* cumrstd, const float* gamma,
+                           const uint8_t* mask, int64_t B, int64_t L, int64_t H, void* x_grad,
+                           float* prev_mean_grad, float* prev_var_grad, float* gamma_grad,
+                           float* beta_grad, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Attention softmax and the fused attention op                              */
 /* stands in for attention_softmax_fwd (fairseq/csrc/ops/attention_softmax.cc:6-18,

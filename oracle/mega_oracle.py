@@ -365,6 +365,77 @@ def timestep_norm_closed_form(x, padding_mask=None, num_groups: Optional[int] = 
     return y, mu, var
 
 
+def timestep_norm_saved(x, prev_count, prev_mean, prev_var, padding_mask=None, num_groups: Optional[int] = None,
+                        eps: float = 1e-5):
+    """What the forward keeps for the backward pass (csrc/ops/timestep_norm.cc:283-300):
+    (count[B], group_mean, cummean, cumrstd), the last three [B, L, G].  At a masked token
+    cummean / cumrstd hold the carried (unchanged) state, which is what "the cumulative mean before
+    the next token" must be for the backward recurrences to be the derivative of the forward."""
+    x = np.asarray(x, np.float64)
+    B, L, H = x.shape
+    G = H if num_groups is None else num_groups
+    xg = x.reshape(B, L, G, H // G)
+    gmean, gvar = xg.mean(-1), xg.var(-1)
+    cm = np.zeros((B, L, G))
+    cr = np.zeros((B, L, G))
+    count = np.array(prev_count, np.int64).copy()
+    for b in range(B):
+        m0 = int(count[b])
+        u = np.array(prev_mean, np.float64).reshape(B, G)[b].copy()
+        v = np.array(prev_var, np.float64).reshape(B, G)[b].copy()
+        for t in range(L):
+            if padding_mask is not None and bool(padding_mask[b][t]):
+                cm[b, t], cr[b, t] = u, 1.0 / np.sqrt(v + eps)
+                continue
+            _, u, v = _welford_combine(m0, u, v, 1, gmean[b, t], gvar[b, t])
+            m0 += 1
+            cm[b, t], cr[b, t] = u, 1.0 / np.sqrt(v + eps)
+        count[b] = m0
+    return count, gmean, cm, cr
+
+
+def timestep_norm_bwd(dy, dmean, dvar, x, prev_mean, count, group_mean, cummean, cumrstd, gamma,
+                      padding_mask=None, num_groups: Optional[int] = None):
+    """Group variant: csrc/ops/timestep_norm.cc:318-450, the literal reverse-time loop; the
+    per-feature variant (:104-217) is the same recurrence with one channel per group and
+    group_mean = x.  Returns (dx, dprev_mean, dprev_var, dgamma, dbeta)."""
+    dy = np.asarray(dy, np.float64)
+    x = np.asarray(x, np.float64)
+    B, L, H = x.shape
+    G = H if num_groups is None else num_groups
+    D = H // G
+    w = np.asarray(gamma, np.float64).reshape(G, D)
+    dyg, xg = dy.reshape(B, L, G, D), x.reshape(B, L, G, D)
+    gm = xg.mean(-1) if group_mean is None else np.asarray(group_mean, np.float64)
+    dx = np.zeros((B, L, G, D))
+    dw = np.zeros((G, D))
+    dbeta = np.zeros((G, D))
+    ug = np.zeros((B, G)) if dmean is None else np.array(dmean, np.float64).reshape(B, G).copy()
+    vg = np.zeros((B, G)) if dvar is None else np.array(dvar, np.float64).reshape(B, G).copy()
+    pm = np.asarray(prev_mean, np.float64).reshape(B, G)
+    for b in range(B):
+        m0 = int(count[b])
+        for j in range(L - 1, -1, -1):
+            if padding_mask is not None and bool(padding_mask[b][j]):
+                continue
+            c1, c2 = (m0 - 1) / m0, 1.0 / m0
+            m0 -= 1
+            prev_u = pm[b] if j == 0 else cummean[b, j - 1]
+            u, r, ux = cummean[b, j], cumrstd[b, j], gm[b, j]
+            ds = (dyg[b, j] * (xg[b, j] - u[:, None]) * w).sum(-1)
+            db = (dyg[b, j] * w).sum(-1)
+            du = ug[b] - r * db
+            dv = vg[b] - 0.5 * r ** 3 * ds
+            dux = c2 * du + 2 * c1 * c2 * dv * (ux - prev_u)
+            dvx = c2 * dv
+            dx[b, j] = dyg[b, j] * r[:, None] * w + (dux[:, None] + 2 * dvx[:, None] * (xg[b, j] - ux[:, None])) / D
+            dw += dyg[b, j] * (xg[b, j] - u[:, None]) * r[:, None]
+            dbeta += dyg[b, j]
+            ug[b] = c1 * du - 2 * c1 * c2 * dv * (ux - prev_u)
+            vg[b] = c1 * dv
+    return dx.reshape(B, L, H), ug, vg, dw.reshape(H), dbeta.reshape(H)
+
+
 # --------------------------------------------------------------------------
 # A9/A10: attention softmax and the fused attention op
 # --------------------------------------------------------------------------

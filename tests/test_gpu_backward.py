@@ -1,0 +1,103 @@
+"""Backward kernels on the GPU against the fp64 oracle's backward restatements (which the CPU
+suite pins by finite differences of the oracle's forward and by the reference's own CPU
+operators' outputs in tests/golden)."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import mega_init_complex, rel_err
+from gpu_util import DEV, TOL, dev, host, rounded
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _tsn_case(rng, B, L, H, G, masked, prior, dtype):
+    GG = H if G is None else G
+    x, x64 = rounded(rng.normal(size=(B, L, H)) * 1.3 + 0.2, dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, L, H)), dtype)
+    mask = (rng.random((B, L)) < 0.25) if masked else None
+    pc = rng.integers(1, 5, B).astype(np.int64) if prior else np.zeros(B, np.int64)
+    pm = (rng.normal(size=(B, GG)) * 0.2 * prior).astype(np.float32).astype(np.float64)
+    pv = (rng.random((B, GG)) + 0.5 if prior else np.ones((B, GG))).astype(np.float32).astype(np.float64)
+    gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32).astype(np.float64)
+    beta = rng.normal(size=H).astype(np.float32).astype(np.float64)
+    dm = rng.normal(size=(B, GG)).astype(np.float32).astype(np.float64)
+    dv = rng.normal(size=(B, GG)).astype(np.float32).astype(np.float64)
+    return x, x64, dy, dy64, mask, pc, pm, pv, gamma, beta, dm, dv
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H,G,masked,prior", [
+    (2, 37, 64, 4, True, True),        # ragged tile, interior padding, carried statistics
+    (3, 130, 128, 16, False, False),   # several tiles per row, 8 channels per group
+    (1, 96, 1024, 16, False, False),   # the headline geometry (64 channels per group)
+    (2, 50, 48, 2, True, False),       # 24 channels per group: three vectors per lane
+    (2, 33, 30, 5, True, True),        # 6 channels per group: element-wise path
+    (2, 45, 24, None, True, True),     # per-feature statistics
+])
+def test_timestep_norm_bwd(dtype, B, L, H, G, masked, prior):
+    rng = np.random.default_rng(51)
+    x, x64, dy, dy64, mask, pc, pm, pv, gamma, beta, dm, dv = _tsn_case(rng, B, L, H, G, masked, prior, dtype)
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    if G is None:
+        y, cnt, mu, var, cm, cr = M.ops.timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma),
+                                                          dev(beta), tm, 1e-5)
+        got = M.ops.timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, cm, cr, dev(gamma), tm)
+    else:
+        y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv),
+                                                                    dev(gamma), dev(beta), tm, G, 1e-5)
+        got = M.ops.group_timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, gm, cm, cr, dev(gamma), tm, G)
+        # without the saved group means the kernel recomputes them
+        got2 = M.ops.group_timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, None, cm, cr, dev(gamma), tm, G)
+        assert rel_err(host(got2[0]), host(got[0])) < 1e-5
+    ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm, pv, mask, G, 1e-5)
+    assert np.array_equal(host(cnt), ocnt)
+    ref = O.timestep_norm_bwd(dy64, dm, dv, x64, pm, ocnt, ogm if G else None, ocm, ocr, gamma, mask, G)
+    tol = TOL[dtype]
+    assert rel_err(host(got[0]), ref[0]) < tol                       # dx, rounded once to the activation type
+    for a, b in zip(got[1:], ref[1:]):                                # fp32 sums over tokens / channels
+        assert rel_err(host(a), b) < 2e-4
+
+
+def test_timestep_norm_bwd_zero_upstream_state_grads():
+    rng = np.random.default_rng(52)
+    x, x64, dy, dy64, mask, pc, pm, pv, gamma, beta, _, _ = _tsn_case(rng, 2, 40, 32, 4, False, True, torch.float32)
+    y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma),
+                                                                dev(beta), None, 4, 1e-5)
+    got = M.ops.group_timestep_norm_bwd(dy, None, None, x, dev(pm), cnt, gm, cm, cr, dev(gamma), None, 4)
+    ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm, pv, None, 4, 1e-5)
+    ref = O.timestep_norm_bwd(dy64, None, None, x64, pm, ocnt, ogm, ocm, ocr, gamma, None, 4)
+    for a, b in zip(got, ref):
+        assert rel_err(host(a), b) < 2e-4
+
+
+@pytest.mark.parametrize("groups,prior_count", [(8, 0), (None, 2), (4, 3)])
+def test_timestep_norm_module_autograd(groups, prior_count):
+    """loss = sum(y * w): gradients of x, weight, bias (and the prior when it is a parameter)."""
+    rng = np.random.default_rng(53)
+    B, L, H = 2, 70, 32
+    mod = M.TimestepNorm(H, groups, prior_count=prior_count).to(DEV).train()
+    with torch.no_grad():
+        mod.weight.normal_(0, 0.2); mod.bias.normal_(0, 0.2)
+        if prior_count > 0:
+            mod.prior_mean.normal_(0, 0.2); mod.prior_logv.normal_(0, 0.2)
+    x64 = rng.normal(size=(B, L, H)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, L, H)).astype(np.float32).astype(np.float64)
+    x = dev(x64).requires_grad_(True)
+    y = mod(x)
+    (y * dev(w64)).sum().backward()
+    G = H if groups is None else groups
+    pc = np.full(B, prior_count, np.int64)
+    pm = np.broadcast_to(host(mod.prior_mean), (B, G)).copy()
+    pv = np.broadcast_to(np.exp(host(mod.prior_logv)), (B, G)).copy()
+    gamma = host(mod.weight) + 1.0
+    ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm, pv, None, groups, 1e-5)
+    dx, dpm, dpv, dg, db = O.timestep_norm_bwd(w64, None, None, x64, pm, ocnt, ogm if groups else None, ocm, ocr,
+                                               gamma, None, groups)
+    assert rel_err(host(x.grad), dx) < 2e-4
+    assert rel_err(host(mod.weight.grad), dg) < 2e-4 and rel_err(host(mod.bias.grad), db) < 2e-4
+    if prior_count > 0:
+        assert rel_err(host(mod.prior_mean.grad), dpm.sum(0)) < 2e-4
+        assert rel_err(host(mod.prior_logv.grad), (dpv * pv).sum(0)) < 2e-4
