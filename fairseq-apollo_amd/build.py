@@ -19,6 +19,7 @@ SOURCES = [
     "timestep_norm_bwd.hip",
     "ema_scan.hip",
     "ema_mfma.hip",
+    "ema_bwd.hip",
     "decode.hip",
     "elementwise.hip",
     "gate_glue.hip",

@@ -62,6 +62,29 @@ def _no_grad_only(module: nn.Module, *tensors):
         )
 
 
+class MovingAverageFunc(torch.autograd.Function):
+    """The whole unidirectional moving-average layer as one differentiable operator: the
+    reference chains EMAParametersFunc (fused_ops/ema_parameters.py:11-33) and FFTConvFunc
+    (fused_ops/fftconv.py:13-41) plus the residual; here neither the kernel nor its gradient is
+    materialised.  Inputs (x [B, D, L], p, q, gamma, omega) as BaseMovingLayer holds them."""
+
+    @staticmethod
+    def forward(ctx, x, p, q, gamma, omega, padding_mask, out_layout):
+        layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1))
+        y, _ = layer(x, padding_mask, None, want_state=False, out_layout=out_layout)
+        ctx.layer = layer
+        ctx.save_for_backward(x, p, q, gamma, omega, padding_mask)
+        return y
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        x, p, q, gamma, omega, padding_mask = ctx.saved_tensors
+        dx, dp, dq, dg, dom = ops.ema_backward(y_grad, x, p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1),
+                                               padding_mask, layer=ctx.layer)
+        return (dx, dp.to(p.dtype).view_as(p), dq.to(q.dtype).view_as(q), dg.to(gamma.dtype).view_as(gamma),
+                dom.to(omega.dtype).view_as(omega), None, None)
+
+
 class BaseMovingLayer(nn.Module, IncrementalState):
     """fairseq/modules/base_moving_average.py:18-197."""
 
@@ -131,11 +154,17 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         """x: [B, D, L]; padding_mask: [B, L] with 1 / True at padding; returns [B, D, L]: contiguous
         rows (what the reference returns) or, with out_layout="input", in x's own strides (a caller
         that hands over a transposed [B, L, D] view and transposes back gets a contiguous result)."""
-        _no_grad_only(self, x)
         bsz, embed_dim, seq_len = x.size()
         assert embed_dim == self.embed_dim
         assert not self.bidirectional or incremental_state is None, \
             'Bidirectional EMA does not support incremental state'
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            if self.bidirectional or incremental_state is not None or (self.truncation is not None and self.truncation >= 1):
+                raise NotImplementedError(
+                    f"{type(self).__name__}: the backward pass covers the unidirectional layer without carried "
+                    "state or truncation; call other configurations under torch.no_grad()")
+            p, q, gamma = self._calc_coeffs()           # stays in the graph
+            return MovingAverageFunc.apply(x, p, q, gamma, self.omega, padding_mask, out_layout)
         layer = self._prepared_layer()
         if incremental_state is not None:
             saved_state = self._get_input_buffer(incremental_state)

@@ -460,6 +460,48 @@ class PreparedEMA:
         return y, hc
 
 
+    def adjoint(self, y_grad: torch.Tensor, padding_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Gradient of the layer output with respect to its input x (unidirectional layer):
+        dx[t] = (1 - mask[t]) sum_{s >= t} k[s - t] dy[s] + omega dy[t], the same layer run backwards
+        in time.  A channel-contiguous y_grad ([B, L, D] memory) is read in place with negated
+        token strides; rows in time are flipped through a copy.  The result has y_grad's layout."""
+        if self.bidirectional or self.trunc:
+            raise NotImplementedError("adjoint: unidirectional layers without truncation only")
+        dev = self.dev
+        _need_gpu(y_grad, padding_mask)
+        lib = _lib.load()
+        B, D, L = y_grad.shape
+        if D != self.D:
+            raise RuntimeError("y_grad must be [B, D, L] of this layer")
+        g = y_grad.detach()
+        if L == 0 or B == 0:
+            return torch.empty_like(g)
+        if g.stride(1) != 1 or not _dense(g):
+            # time is the fast axis (or the layout is irregular): flip, run forwards, flip back
+            out, _ = self(g.flip(-1))
+            dx = out.flip(-1)
+        else:
+            dx = torch.empty_strided(g.shape, g.stride(), dtype=g.dtype, device=dev)
+            es = g.element_size()
+            key = ("ema", B, D, self.N, L, False, 0)
+            nws = _ws_bytes_cache.get(key)
+            if nws is None:
+                nws = _ws_bytes_cache[key] = lib.mega_ema_fwd_workspace_bytes(B, D, self.N, L, 0, 0)
+            stream = _stream(dev)
+            ws = _scratch_buffer(dev, nws, stream)
+            sl = g.stride(2)
+            with _on_device(dev):
+                rc = lib.mega_ema_fwd(g.data_ptr() + (L - 1) * sl * es, dx.data_ptr() + (L - 1) * sl * es,
+                                      _dtype_code(g), g.stride(0), g.stride(1), -sl, dx.stride(0), dx.stride(1), -sl,
+                                      _ptr(self.p), _ptr(self.q), _ptr(self.gamma), 1 if self.is_complex else 0,
+                                      _ptr(self.omega), None, None, None, B, D, self.N, L, 0, 0,
+                                      1 if self.shift else 0, _ptr(self.image), _ptr(ws), ws.numel(), stream)
+            _lib.check(rc, "ema_fwd (adjoint)")
+        if padding_mask is not None:
+            dx = torch.where(padding_mask.to(torch.bool).unsqueeze(1), self.omega.to(g.dtype).view(1, D, 1) * g, dx)
+        return dx
+
+
 def ema_forward(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, omega: torch.Tensor,
                 padding_mask: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
                 want_state: bool = False, bidirectional: bool = False, truncation: Optional[int] = None,
@@ -690,3 +732,46 @@ def gate_out_fwd(residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: 
                                    _ntok(residual), residual.shape[-1], _stream(dev))
     _lib.check(rc, "gate_out_fwd")
     return y
+
+
+def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor,
+                 omega: torch.Tensor, padding_mask: Optional[torch.Tensor] = None,
+                 layer: Optional[PreparedEMA] = None):
+    """Backward of ema_forward (unidirectional, no carried state, no truncation):
+    -> (x_grad, p_grad [D,N], q_grad [D,N], gamma_grad [D,N], omega_grad [D]); q_grad / gamma_grad are
+    complex for the complex layer, in torch's convention for a real loss (dL = Re(conj(grad) dz)).
+    It replaces fftconv_bwd + ema_parameters_bwd of the reference
+    (fairseq/modules/fused_ops/fftconv.py:32-41, fused_ops/ema_parameters.py:23-33,
+    csrc/ops/ema_parameters.cc:80-97) without forming the kernel or its gradient."""
+    dev = _need_gpu(y_grad, x, p, q, gamma, omega, padding_mask)
+    lib = _lib.load()
+    if x.dim() != 3 or y_grad.shape != x.shape:
+        raise RuntimeError("x and y_grad must be [B, D, L] of the same shape")
+    B, D, L = x.shape
+    if layer is None:
+        layer = PreparedEMA(p, q, gamma, omega)
+    N = layer.N
+    xd = x.detach()
+    g = y_grad.detach().to(xd.dtype)
+    if 0 in g.stride() and g.numel() > 0:
+        g = g.contiguous()
+    dx = layer.adjoint(g, padding_mask)
+    sums = torch.empty(B, D, N, 4, dtype=torch.float32, device=dev)
+    dyx = torch.empty(B, D, dtype=torch.float32, device=dev)
+    m8 = _mask_u8(padding_mask, B, L)
+    with _on_device(dev):
+        rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
+                                     xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.q), _ptr(m8), B, D, N, L,
+                                     _ptr(sums), _ptr(dyx), _stream(dev))
+    _lib.check(rc, "ema_param_grad")
+    tot = sums.sum(0)                                   # [D, N, 4]
+    s2 = torch.complex(tot[..., 0], tot[..., 1])
+    s1 = torch.complex(tot[..., 2], tot[..., 3])
+    pc = layer.p.to(torch.complex64)
+    gc = torch.view_as_complex(layer.gamma)
+    dp = (s2 * gc).real
+    dq = torch.conj(s1 * pc * gc)
+    dg = torch.conj(s2 * pc)
+    if not layer.is_complex:
+        dq, dg = dq.real, dg.real
+    return dx, dp, dq, dg, dyx.sum(0)

@@ -251,6 +251,45 @@ def ema_forward(x, p, q, gamma, omega, padding_mask=None, h=None,
     return out + residual, h_new
 
 
+def ema_kernel_bwd(dk, p, q, gamma):
+    """RowwiseEMAWeightCPUBwd, csrc/ops/ema_parameters.cc:80-97: from the kernel gradient
+    dk [D, L] to (dp [D,N] real, dq [D,N], dgamma [D,N]) with
+    sum1 = sum_l dk[l] l q^(l-1), sum2 = sum_l dk[l] q^l; dp = Re(sum2 gamma),
+    dq = conj(sum1 p gamma), dgamma = conj(sum2 p)."""
+    dk = np.asarray(dk, np.float64)
+    p = np.asarray(p, np.float64)
+    q = np.asarray(q, np.complex128)
+    gamma = np.asarray(gamma, np.complex128)
+    L = dk.shape[-1]
+    l = np.arange(L)
+    qw2 = q[..., None] ** l                                             # q^l
+    qw1 = np.where(l > 0, q[..., None] ** np.maximum(l - 1, 0), 0.0)    # q^(l-1), 0 at l = 0
+    sum1 = (dk[:, None, :] * qw1 * l).sum(-1)
+    sum2 = (dk[:, None, :] * qw2).sum(-1)
+    return (sum2 * gamma).real, np.conj(sum1 * p * gamma), np.conj(sum2 * p)
+
+
+def ema_backward(dy, x, p, q, gamma, omega, padding_mask=None):
+    """Backward of ema_forward (unidirectional, no carried state): the reference's chain
+    fftconv backward (modules/fused_ops/fftconv.py:66-88: dx = correlation of dy with k,
+    dk = sum over the batch of the correlation of dy with x) -> ema_kernel_bwd, with the
+    correlations written out directly.  Returns (dx, dp, dq, dgamma, domega)."""
+    dy = np.asarray(dy, np.float64)
+    x = np.asarray(x, np.float64)
+    B, D, L = x.shape
+    keep = np.ones((B, 1, L)) if padding_mask is None else 1.0 - np.asarray(padding_mask, np.float64)[:, None, :]
+    xm = x * keep
+    k = ema_kernel(p, q, gamma, L)
+    dxc = np.zeros_like(x)
+    dk = np.zeros((D, L))
+    for l in range(L):
+        dxc[:, :, :L - l] += dy[:, :, l:] * k[None, :, l:l + 1]
+        dk[:, l] = (dy[:, :, l:] * xm[:, :, :L - l]).sum(axis=(0, 2))
+    om = np.asarray(omega, np.float64).reshape(1, D, 1)
+    dp, dq, dg = ema_kernel_bwd(dk, p, q, gamma)
+    return dxc * keep + om * dy, dp, dq, dg, (dy * x).sum(axis=(0, 2))
+
+
 def ema_one_step(x_t, p, q, gamma, omega, h=None):
     """BaseMovingLayer.one_step, modules/base_moving_average.py:105-118, plus the
     residual the caller adds.  x_t: [B, D]; h: [B, D, N]."""

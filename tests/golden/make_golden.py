@@ -95,6 +95,56 @@ def main():
                 "ema.length": np.int64(L), "ema.kernel": w.numpy(), "ema.bias": b.numpy(),
                 "ema.hidden": hy.numpy(), "ema.hidden_zero_start": hy0.numpy()})
 
+    # backward operators (own generator, so the arrays above keep their values).  TimestepNorm
+    # cases have padding at the end of the rows only: behind an interior masked token the
+    # reference's CPU forward stores a cumulative mean that includes the masked token
+    # (timestep_norm.cc:291-296), and its backward then differentiates a different function.
+    rng = np.random.default_rng(20241)
+    for tag, (B, L, H, G, pad) in {"gtsn_bwd_a": (2, 45, 48, 4, True), "gtsn_bwd_b": (3, 70, 64, 16, False),
+                                   "tsn_bwd": (2, 33, 24, None, True)}.items():
+        GG = H if G is None else G
+        x = (rng.normal(size=(B, L, H)) * 1.4 + 0.2).astype(np.float32)
+        mask = None
+        if pad:
+            mask = np.zeros((B, L), bool)
+            for b in range(B):
+                mask[b, L - int(rng.integers(1, 9)):] = True
+        pc = rng.integers(1, 6, B).astype(np.int64)
+        pm = (rng.normal(size=(B, GG)) * 0.2).astype(np.float32)
+        pv = (rng.random((B, GG)) + 0.5).astype(np.float32)
+        gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32)
+        beta = rng.normal(size=H).astype(np.float32)
+        dy = rng.normal(size=(B, L, H)).astype(np.float32)
+        dm = rng.normal(size=(B, GG)).astype(np.float32)
+        dv = rng.normal(size=(B, GG)).astype(np.float32)
+        tm = None if mask is None else t(mask)
+        if G is None:
+            y, c, mu, v, cm, cr = ref.timestep_norm_fwd(t(x), t(pc), t(pm), t(pv), t(gamma), t(beta), tm, 1e-5)
+            gr = ref.timestep_norm_bwd(t(dy), t(dm), t(dv), t(x), t(pm), c, cm, cr, t(gamma), tm)
+        else:
+            y, c, mu, v, gm, cm, cr = ref.group_timestep_norm_fwd(t(x), t(pc), t(pm), t(pv), t(gamma), t(beta), tm, G,
+                                                                  1e-5)
+            gr = ref.group_timestep_norm_bwd(t(dy), t(dm), t(dv), t(x), t(pm), c, gm, cm, cr, t(gamma), tm, G)
+        out.update({f"{tag}.x": x, f"{tag}.prev_count": pc, f"{tag}.prev_mean": pm, f"{tag}.prev_var": pv,
+                    f"{tag}.gamma": gamma, f"{tag}.beta": beta, f"{tag}.groups": np.int64(0 if G is None else G),
+                    f"{tag}.y_grad": dy, f"{tag}.mean_grad": dm, f"{tag}.var_grad": dv,
+                    f"{tag}.x_grad": gr[0].numpy(), f"{tag}.prev_mean_grad": gr[1].numpy(),
+                    f"{tag}.prev_var_grad": gr[2].numpy(), f"{tag}.gamma_grad": gr[3].numpy(),
+                    f"{tag}.beta_grad": gr[4].numpy()})
+        if mask is not None:
+            out[f"{tag}.mask"] = mask
+
+    # kernel gradient -> coefficient gradients
+    K, N, L = 5, 16, 80
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
+    p, q, g = p.astype(np.float32), q.astype(np.complex64), g.astype(np.complex64)
+    dk = rng.normal(size=(K, L)).astype(np.float32)
+    log_q = t(q).log()
+    w, _, vander = ref.ema_parameters_fwd(t(p), log_q, t(g), None, L)
+    dp, dq, dg, _ = ref.ema_parameters_bwd(t(dk), None, t(p), log_q, t(g), None, vander)
+    out.update({"ema_bwd.p": p, "ema_bwd.q": q, "ema_bwd.gamma": g, "ema_bwd.kernel_grad": dk,
+                "ema_bwd.p_grad": dp.numpy(), "ema_bwd.q_grad": dq.numpy(), "ema_bwd.gamma_grad": dg.numpy()})
+
     dst = os.path.join(HERE, "ref_cpu_vectors.npz")
     np.savez_compressed(dst, **out)
     print(dst, os.path.getsize(dst), "bytes,", len(out), "arrays")

@@ -129,3 +129,46 @@ def test_hip_ema(gold):
     y = y[0] if isinstance(y, tuple) else y
     ref = O.causal_conv_direct(c["x"].astype(np.float64), c["kernel"].astype(np.float64)) + c["bias"]
     assert rel_err(host(y), ref) < 1e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", ["gtsn_bwd_a", "gtsn_bwd_b", "tsn_bwd"])
+def test_hip_timestep_norm_bwd(gold, tag):
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, tag)
+    G = int(c["groups"])
+    mask = None if "mask" not in c else torch.from_numpy(c["mask"]).to("cuda:0")
+    x, pm, gamma = dev(c["x"]), dev(c["prev_mean"]), dev(c["gamma"])
+    fwd_args = (x, dev(c["prev_count"], torch.int64), pm, dev(c["prev_var"]), gamma, dev(c["beta"]), mask)
+    if G:
+        _, cnt, _, _, gm, cm, cr = M.ops.group_timestep_norm_fwd(*fwd_args, G, 1e-5)
+        got = M.ops.group_timestep_norm_bwd(dev(c["y_grad"]), dev(c["mean_grad"]), dev(c["var_grad"]), x, pm, cnt, gm,
+                                            cm, cr, gamma, mask, G)
+    else:
+        _, cnt, _, _, cm, cr = M.ops.timestep_norm_fwd(*fwd_args, 1e-5)
+        got = M.ops.timestep_norm_bwd(dev(c["y_grad"]), dev(c["mean_grad"]), dev(c["var_grad"]), x, pm, cnt, cm, cr,
+                                      gamma, mask)
+    for a, name in zip(got, ("x_grad", "prev_mean_grad", "prev_var_grad", "gamma_grad", "beta_grad")):
+        assert rel_err(host(a), c[name]) < 1e-4, name
+
+
+@pytest.mark.gpu
+def test_hip_ema_backward_against_kernel_gradient_vectors(gold):
+    """With x a unit impulse at t = 0 the kernel gradient sum_t dy[t] x[t - l] is dy itself, so the
+    fused backward must return what the reference's ema_parameters_bwd returned for dk = dy."""
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, "ema_bwd")
+    K, L = c["kernel_grad"].shape
+    x = np.zeros((1, K, L), np.float32)
+    x[:, :, 0] = 1.0
+    _, dp, dq, dg, _ = M.ops.ema_backward(dev(c["kernel_grad"][None]), dev(x), dev(c["p"]), dev(c["q"]),
+                                          dev(c["gamma"]), dev(np.zeros(K, np.float32)))
+    assert rel_err(host(dp), c["p_grad"]) < 1e-4
+    for a, b in ((host(dq), c["q_grad"]), (host(dg), c["gamma_grad"])):
+        assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4

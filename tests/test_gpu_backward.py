@@ -101,3 +101,92 @@ def test_timestep_norm_module_autograd(groups, prior_count):
     if prior_count > 0:
         assert rel_err(host(mod.prior_mean.grad), dpm.sum(0)) < 2e-4
         assert rel_err(host(mod.prior_logv.grad), (dpv * pv).sum(0)) < 2e-4
+
+
+# ----------------------------------------------------------------------------------------------
+# moving-average layer
+# ----------------------------------------------------------------------------------------------
+def _ema_coeffs(rng, D, N, cplx):
+    if cplx:
+        return O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    alpha, delta = rng.normal(size=(D, N)) * 0.2, rng.normal(size=(D, N)) * 0.2
+    beta = rng.normal(size=(D, N)) * 0.02 + np.where(np.arange(N) % 2 == 0, 1.0, -1.0)
+    return O.ema_coeffs_real(alpha, delta, beta, rng.normal(size=(D, N)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,D,N,L,cplx,layout,masked", [
+    (2, 32, 16, 2048, True, "bld", False),    # matrix-core path backwards in time, channels contiguous
+    (1, 16, 16, 1024, True, "bdl", False),    # rows in time: flipped through a copy
+    (2, 24, 16, 300, True, "bld", True),      # generic path, padding
+    (3, 20, 2, 77, False, "bdl", True),       # real layer, two states
+    (2, 40, 7, 129, True, "bld", False),      # odd state count
+])
+def test_ema_backward(dtype, B, D, N, L, cplx, layout, masked):
+    rng = np.random.default_rng(61)
+    p, q, g = _ema_coeffs(rng, D, N, cplx)
+    p, g = p.astype(np.float32).astype(np.float64), (g.astype(np.complex64).astype(np.complex128) if cplx else
+                                                      g.astype(np.float32).astype(np.float64))
+    q = q.astype(np.complex64).astype(np.complex128) if cplx else q.astype(np.float32).astype(np.float64)
+    om = rng.normal(size=D).astype(np.float32).astype(np.float64)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    if layout == "bld":
+        x = x.transpose(1, 2).contiguous().transpose(1, 2)
+        dy = dy.transpose(1, 2).contiguous().transpose(1, 2)
+    mask = (rng.random((B, L)) < 0.2) if masked else None
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    got = M.ops.ema_backward(dy, x, dev(p), dev(q), dev(g), dev(om), tm)
+    ref = O.ema_backward(dy64, x64, p, q, g, om, mask)
+    assert got[0].stride() == dy.stride()
+    # dx is one moving average of dy: same bound as the forward layer
+    assert rel_err(host(got[0]), ref[0]) < TOL[dtype]
+    for a, b, name in zip(got[1:], ref[1:], ("dp", "dq", "dgamma", "domega")):
+        a = host(a)
+        if np.iscomplexobj(b):
+            assert rel_err(a.real, b.real) < 5e-4 and rel_err(a.imag, b.imag) < 5e-4, name
+        else:
+            assert rel_err(a, np.real(b)) < 5e-4, name
+
+
+@pytest.mark.parametrize("cls,N", [("cema", 16), ("ema", 2)])
+def test_moving_average_module_autograd(cls, N):
+    """Gradients of the raw parameters (alpha, delta, theta | beta, gamma, omega) and of x through
+    autograd of the coefficient formulas + the backward operator, against central differences of
+    the fp64 oracle."""
+    rng = np.random.default_rng(62)
+    B, D, L = 2, 16, 96
+    torch.manual_seed(5)
+    mod = (M.MultiHeadComplexEMA if cls == "cema" else M.MultiHeadEMA)(D, ndim=N).to(DEV).train()
+    x64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    x = dev(x64).requires_grad_(True)
+    (mod(x) * dev(w64)).sum().backward()
+
+    names = ["alpha", "delta", "theta" if cls == "cema" else "beta", "gamma", "omega"]
+    P = {n: host(getattr(mod, n)) for n in names}
+
+    def loss(Pd, xx):
+        if cls == "cema":
+            p, q, g = O.ema_coeffs_complex(Pd["alpha"], Pd["delta"], Pd["theta"], Pd["gamma"])
+        else:
+            p, q, g = O.ema_coeffs_real(Pd["alpha"], Pd["delta"], Pd["beta"], Pd["gamma"])
+        return (O.ema_forward(xx, p, q, g, Pd["omega"].reshape(-1))[0] * w64).sum()
+
+    eps = 1e-5
+    for n in names:
+        grad = host(getattr(mod, n).grad)
+        scale = np.abs(grad).max() + 1e-6
+        for _ in range(4):
+            idx = tuple(rng.integers(0, s) for s in P[n].shape)
+            Pp = {k: v.copy() for k, v in P.items()}; Pp[n][idx] += eps
+            Pm = {k: v.copy() for k, v in P.items()}; Pm[n][idx] -= eps
+            fd = (loss(Pp, x64) - loss(Pm, x64)) / (2 * eps)
+            assert abs(fd - grad[idx]) < 2e-3 * scale, (n, idx, fd, grad[idx])
+    dxo = O.ema_backward(w64, x64, *_module_coeffs(mod, cls), host(mod.omega).reshape(-1))[0]
+    assert rel_err(host(x.grad), dxo) < 1e-4
+
+
+def _module_coeffs(mod, cls):
+    p, q, g = mod.coeffs()
+    return host(p.squeeze(-1)), host(q.squeeze(-1)), host(g)

@@ -1,0 +1,101 @@
+"""Pins of the oracle's backward restatements (CPU only):
+  * central differences of the oracle's own fp64 forward (a dropped term, a wrong sign or a
+    transposed index in the backward fails these);
+  * the outputs of the reference's own CPU operators (tests/golden/ref_cpu_vectors.npz)."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import mega_init_complex, rel_err
+from oracle import mega_oracle as O
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_cpu_vectors.npz")
+
+
+def _fd(f, arr, idx, unit=1.0, e=1e-6):
+    a1, a2 = arr.copy(), arr.copy()
+    a1[idx] += e * unit
+    a2[idx] -= e * unit
+    return (f(a1) - f(a2)) / (2 * e)
+
+
+@pytest.mark.parametrize("G,masked,prior", [(4, True, 3), (None, True, 2), (2, False, 0), (8, True, 0)])
+def test_timestep_norm_bwd_matches_finite_differences(G, masked, prior):
+    rng = np.random.default_rng(7)
+    B, L, H = 2, 11, 8
+    GG = H if G is None else G
+    x = rng.normal(size=(B, L, H))
+    gamma, beta = rng.normal(size=H) + 1, rng.normal(size=H)
+    mask = (rng.random((B, L)) < 0.3) if masked else None      # interior padding included
+    pc = np.array([prior, prior + 1]) if prior else np.zeros(B, np.int64)
+    pm, pv = rng.normal(size=(B, GG)) * 0.3, rng.random((B, GG)) + 0.5
+    wy, wm, wv = rng.normal(size=(B, L, H)), rng.normal(size=(B, GG)), rng.normal(size=(B, GG))
+
+    def loss(x_, pm_, pv_, g_, b_):
+        y, _, mu, v = O.timestep_norm(x_, pc, pm_, pv_, g_, b_, mask, G, 1e-5)
+        return (y * wy).sum() + (mu * wm).sum() + (v * wv).sum()
+
+    cnt, gm, cm, cr = O.timestep_norm_saved(x, pc, pm, pv, mask, G, 1e-5)
+    grads = O.timestep_norm_bwd(wy, wm, wv, x, pm, cnt, gm if G else None, cm, cr, gamma, mask, G)
+    args = [x, pm, pv, gamma, beta]
+    for which, g in enumerate(grads):
+        if which in (1, 2) and prior == 0:
+            continue                                           # count 0: the prior has no weight
+        for _ in range(8):
+            idx = tuple(rng.integers(0, s) for s in args[which].shape)
+            f = lambda a: loss(*[a if i == which else args[i] for i in range(5)])
+            assert abs(_fd(f, args[which], idx) - g[idx]) < 1e-6
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_ema_backward_matches_finite_differences(masked):
+    rng = np.random.default_rng(8)
+    D, N, L, B = 3, 4, 13, 2
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    om = rng.normal(size=D)
+    x, wy = rng.normal(size=(B, D, L)), rng.normal(size=(B, D, L))
+    mask = (rng.random((B, L)) < 0.3) if masked else None
+    loss = lambda x_, p_, q_, g_, o_: (O.ema_forward(x_, p_, q_, g_, o_, mask)[0] * wy).sum()
+    dx, dp, dq, dg, dom = O.ema_backward(wy, x, p, q, g, om, mask)
+    for _ in range(6):
+        i = tuple(rng.integers(0, s) for s in x.shape)
+        j = tuple(rng.integers(0, s) for s in p.shape)
+        d = (int(rng.integers(0, D)),)
+        assert abs(_fd(lambda a: loss(a, p, q, g, om), x, i) - dx[i]) < 1e-6
+        assert abs(_fd(lambda a: loss(x, a, q, g, om), p, j) - dp[j]) < 1e-6
+        assert abs(_fd(lambda a: loss(x, p, q, g, a), om, d) - dom[d]) < 1e-6
+        # complex gradients: real part = d/dRe, imaginary part = d/dIm
+        assert abs(_fd(lambda a: loss(x, p, a, g, om), q, j) - dq[j].real) < 1e-6
+        assert abs(_fd(lambda a: loss(x, p, a, g, om), q, j, 1j) - dq[j].imag) < 1e-6
+        assert abs(_fd(lambda a: loss(x, p, q, a, om), g, j) - dg[j].real) < 1e-6
+        assert abs(_fd(lambda a: loss(x, p, q, a, om), g, j, 1j) - dg[j].imag) < 1e-6
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLD, allow_pickle=False)
+
+
+def _case(gold, tag):
+    return {k[len(tag) + 1:]: gold[k] for k in gold.files if k.startswith(tag + ".")}
+
+
+@pytest.mark.parametrize("tag", ["gtsn_bwd_a", "gtsn_bwd_b", "tsn_bwd"])
+def test_timestep_norm_bwd_matches_reference_vectors(gold, tag):
+    c = _case(gold, tag)
+    G = int(c["groups"]) or None
+    mask = c.get("mask")
+    cnt, gm, cm, cr = O.timestep_norm_saved(c["x"], c["prev_count"], c["prev_mean"], c["prev_var"], mask, G, 1e-5)
+    got = O.timestep_norm_bwd(c["y_grad"], c["mean_grad"], c["var_grad"], c["x"], c["prev_mean"], cnt,
+                              gm if G else None, cm, cr, c["gamma"], mask, G)
+    for a, name in zip(got, ("x_grad", "prev_mean_grad", "prev_var_grad", "gamma_grad", "beta_grad")):
+        assert rel_err(a, c[name]) < 5e-5, name            # the vectors are fp32 results
+
+
+def test_ema_kernel_bwd_matches_reference_vectors(gold):
+    c = _case(gold, "ema_bwd")
+    dp, dq, dg = O.ema_kernel_bwd(c["kernel_grad"], c["p"], c["q"], c["gamma"])
+    assert rel_err(dp, c["p_grad"]) < 5e-5
+    for a, b in ((dq, c["q_grad"]), (dg, c["gamma_grad"])):
+        assert rel_err(a.real, b.real) < 5e-5 and rel_err(a.imag, b.imag) < 5e-5
