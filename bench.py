@@ -136,6 +136,85 @@ def bench_decode(args):
     }))
 
 
+def bench_block_bwd(args):
+    """Backward of the headline block at configs[2]'s shape: moving-average backward (input
+    gradient + parameter-gradient sums) followed by the TimestepNorm backward, per operator with HIP
+    events around back-to-back launches."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1237)
+    ema = M.MultiHeadComplexEMA(D, ndim=N).to(dev).eval()
+    with torch.no_grad():
+        p, q, g = ema.coeffs()
+        layer = M.ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), g, ema.omega.reshape(-1))
+    gamma = torch.randn(D, device=dev) * 0.1 + 1.0
+    beta = torch.randn(D, device=dev) * 0.1
+    pc = torch.zeros(B, dtype=torch.int64, device=dev)
+    pm = torch.zeros(B, G, device=dev)
+    pv = torch.ones(B, G, device=dev)
+    nbuf = 4
+    xs = [torch.randn(B, L, D, device=dev).to(torch.bfloat16) for _ in range(nbuf)]
+    dys = [torch.randn(B, L, D, device=dev).to(torch.bfloat16) for _ in range(nbuf)]
+    saved = []
+    with torch.no_grad():
+        for x in xs:
+            xn, cnt, _, _, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, pc, pm, pv, gamma, beta, None, G, 1e-5)
+            saved.append((xn, cnt, gm, cm, cr))
+
+    def ema_bwd(i):
+        xn = saved[i % nbuf][0]
+        return M.ops.ema_backward(dys[i % nbuf].transpose(1, 2), xn.transpose(1, 2), p.squeeze(-1), q.squeeze(-1), g,
+                                  ema.omega.reshape(-1), None, layer=layer)
+
+    def tsn_bwd(i, dxn):
+        _, cnt, gm, cm, cr = saved[i % nbuf]
+        return M.ops.group_timestep_norm_bwd(dxn, None, None, xs[i % nbuf], pm, cnt, gm, cm, cr, gamma, None, G)
+
+    def timed(fn):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for i in range(args.steps):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / args.steps
+
+    with torch.no_grad():
+        dxn = None
+        for i in range(max(args.warmup, 1)):
+            dxn = ema_bwd(i)[0].transpose(1, 2)
+            tsn_bwd(i, dxn)
+        ms_ema = timed(ema_bwd)
+        ms_tsn = timed(lambda i: tsn_bwd(i, dxn))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            tsn_bwd(i, ema_bwd(i)[0].transpose(1, 2))
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    act = B * L * D * 2
+    # algorithmic bytes: EMA backward reads dy twice (input gradient, sums) and x once, writes dx;
+    # the norm backward reads dy and x twice (tile maps, then dx) and writes dx
+    alg_ema, alg_tsn = 4 * act, 5 * act
+    print(json.dumps({
+        "metric": "backward tokens/sec @B4xL4096xD1024, CEMA backward + TimestepNorm backward", "value": B * L / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[2] shape, backward of TimestepNorm(16 groups) -> complex EMA (N=16)"},
+        "kernels": {
+            "ema_backward": {"avg_ms": ms_ema, "algorithmic_bytes": alg_ema, "GBps": alg_ema / (ms_ema * 1e-3) / 1e9},
+            "group_timestep_norm_bwd": {"avg_ms": ms_tsn, "algorithmic_bytes": alg_tsn,
+                                        "GBps": alg_tsn / (ms_tsn * 1e-3) / 1e9}},
+        "roofline": {"bound": "hbm", "kernel": "ema_backward (adjoint + parameter sums)",
+                     "achieved": alg_ema / (ms_ema * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg_ema / (ms_ema * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None},
+    }))
+
+
 def bench_attention(args):
     """configs[4]'s attention: 4 chunks of 2048 tokens, 4 heads, H1 = 128, H2 = 1024, bf16, causal
     (matrix-core bound).  Flops are counted for the causal half only: 2 * C^2/2 * (H1 + H2) per chunk-head."""
@@ -230,7 +309,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer"], default="block",
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd"], default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4], "
                          "one JSON line each")
@@ -241,6 +320,8 @@ def main():
 
     if args.workload == "decode":
         return bench_decode(args)
+    if args.workload == "block_bwd":
+        return bench_block_bwd(args)
     if args.workload == "attention":
         return bench_attention(args)
     if args.workload == "layer":

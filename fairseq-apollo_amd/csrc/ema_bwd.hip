@@ -60,15 +60,25 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
   float sr = 0.f, si = 0.f, gr = 0.f, gi = 0.f;          // s[t], g[t]
   float a2r = 0.f, a2i = 0.f, a1r = 0.f, a1i = 0.f, ax = 0.f;
 
+  // Tile moves are branch-free (clamped addresses, validity applied when the value is parked in
+  // LDS) so that all loads of a tile are in flight together and stay in flight across the
+  // arithmetic of the previous tile.
   float px[kPerThread], pg[kPerThread];
+  int ex[kPerThread], eg[kPerThread];       // (channel << 16 | token) of every element this thread moves
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const int e = tid + k * kBwdThreads;
+    ex[k] = x_chan_fast ? ((e % kCh) << 16 | (e / kCh)) : ((e / kTk) << 16 | (e % kTk));
+    eg[k] = g_chan_fast ? ((e % kCh) << 16 | (e / kCh)) : ((e / kTk) << 16 | (e % kTk));
+  }
+  const int dmax = A.D - 1 - c0, lmax = A.L - 1;
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int k = 0; k < kPerThread; ++k) {
-      const int e = tid + k * kBwdThreads;
-      const int cx = x_chan_fast ? e % kCh : e / kTk, tx = x_chan_fast ? e / kCh : e % kTk;
-      const int cg = g_chan_fast ? e % kCh : e / kTk, tg = g_chan_fast ? e / kCh : e % kTk;
-      px[k] = (c0 + cx < A.D && t0 + tx < A.L) ? to_float(xg[(int64_t)(c0 + cx) * A.sxd + (int64_t)(t0 + tx) * A.sxl]) : 0.f;
-      pg[k] = (c0 + cg < A.D && t0 + tg < A.L) ? to_float(gg[(int64_t)(c0 + cg) * A.sgd + (int64_t)(t0 + tg) * A.sgl]) : 0.f;
+      const int cx = min(ex[k] >> 16, dmax), tx = min(t0 + (ex[k] & 0xffff), lmax);
+      const int cg = min(eg[k] >> 16, dmax), tg = min(t0 + (eg[k] & 0xffff), lmax);
+      px[k] = to_float(xg[(int64_t)(c0 + cx) * A.sxd + (int64_t)tx * A.sxl]);
+      pg[k] = to_float(gg[(int64_t)(c0 + cg) * A.sgd + (int64_t)tg * A.sgl]);
     }
   };
   fetch(0);
@@ -76,15 +86,17 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
     __syncthreads();    // the previous tile has been consumed
 #pragma unroll
     for (int k = 0; k < kPerThread; ++k) {
-      const int e = tid + k * kBwdThreads;
-      const int cx = x_chan_fast ? e % kCh : e / kTk, tx = x_chan_fast ? e / kCh : e % kTk;
-      const int cg = g_chan_fast ? e % kCh : e / kTk, tg = g_chan_fast ? e / kCh : e % kTk;
-      s_x[cx][tx] = px[k];
-      s_g[cg][tg] = pg[k];
+      const int cx = ex[k] >> 16, tx = ex[k] & 0xffff, cg = eg[k] >> 16, tg = eg[k] & 0xffff;
+      s_x[cx][tx] = (cx <= dmax && t0 + tx <= lmax) ? px[k] : 0.f;
+      s_g[cg][tg] = (cg <= dmax && t0 + tg <= lmax) ? pg[k] : 0.f;
     }
-    if (tid < kTk) s_keep[tid] = (A.mask && t0 + tid < A.L && A.mask[(size_t)b * A.L + t0 + tid]) ? 0.f : 1.f;
+    if (tid < kTk) {
+      const int tm = min(t0 + tid, lmax);
+      const uint8_t mk = A.mask ? A.mask[(size_t)b * A.L + tm] : (uint8_t)0;
+      s_keep[tid] = mk ? 0.f : 1.f;
+    }
     __syncthreads();
-    if (t0 + kTk < A.L) fetch(t0 + kTk);    // in flight while this tile is worked through
+    fetch(t0 + kTk);    // the next tile (clamped past the end) is in flight while this one is worked through
 #pragma unroll 4
     for (int t = 0; t < kTk; t += 4) {
       const float4 xv = *(const float4*)&s_x[ch][t];
@@ -132,6 +144,11 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
                "ema_param_grad: shape too large");
   if (B == 0) return MEGA_OK;
   MEGA_REQUIRE(q && sums && dyx && (L == 0 || (dy && x)), MEGA_ERR_ARG, "ema_param_grad: null pointer argument");
+  if (L == 0) {
+    hipMemsetAsync(sums, 0, (size_t)B * D * N * 16, (hipStream_t)stream);
+    hipMemsetAsync(dyx, 0, (size_t)B * D * 4, (hipStream_t)stream);
+    return MEGA_OK;
+  }
   MEGA_REQUIRE(((uintptr_t)sums % 16) == 0, MEGA_ERR_ARG, "ema_param_grad: sums must be 16-byte aligned");
   EmaGradArgs A;
   A.dy = dy; A.x = x; A.sgb = sgb; A.sgd = sgd; A.sgl = sgl; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl;

@@ -14,7 +14,7 @@
 // compose into maps of the same shape, so the walk is split over token tiles:
 //   1. tsn_bwd_tile_kernel<.., 0>: per tile, ds / db per (token, group), the tile's composed map,
 //      and the tile's share of the gamma / beta gradients;
-//   2. tsn_bwd_carry_kernel: one thread per (row, group) walks the tile maps from the last tile
+//   2. tsn_bwd_carry_kernel: one wave per (row, group) scans the tile maps from the last tile
 //      to the first and leaves the pair that enters every tile (and the prev_mean / prev_var
 //      gradients at the end);
 //   3. tsn_bwd_tile_kernel<.., 1>: per tile, the same ds / db again, the walk inside the tile from
@@ -58,7 +58,10 @@ struct TsnBwdParams {
 };
 
 // PHASE 0: tile maps + parameter shares; PHASE 1: dx.
-template <typename T, int VEC, int PHASE>
+// FIXED (PHASE 0 only): slots divides the workgroup size and every lane moves one vector, so a
+// thread meets the same VEC channels at every token it visits and keeps their gamma / beta shares
+// in registers; otherwise the shares are added into LDS element by element.
+template <typename T, int VEC, int PHASE, bool FIXED = false>
 __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdParams P) {
   using V = Vec<T, VEC>;
   extern __shared__ float smem[];
@@ -108,6 +111,9 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   // ---- ds, db (and the group mean when it was not handed in) per (token, group)
   const int items = ntok * P.slots;
   const int span = VEC * P.PER;          // channels per lane
+  float rw[VEC], rb[VEC];                // FIXED: this thread's gamma / beta shares
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) { rw[e] = 0.f; rb[e] = 0.f; }
   for (int i0 = 0; i0 < items; i0 += kThreads) {
     const int i = i0 + tid;
     const bool live = i < items;
@@ -131,8 +137,13 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
           db = fmaf(d, w, db);
           sx += xe;
           if (PHASE == 0 && keep) {
-            atomicAdd(&s_wg[c + e], d * (xe - u) * r);
-            atomicAdd(&s_bg[c + e], d);
+            if (FIXED) {
+              rw[e] = fmaf(d * (xe - u), r, rw[e]);
+              rb[e] += d;
+            } else {
+              atomicAdd(&s_wg[c + e], d * (xe - u) * r);
+              atomicAdd(&s_bg[c + e], d);
+            }
           }
         }
       }
@@ -197,6 +208,19 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   __syncthreads();
 
   if (PHASE == 0) {
+    if (FIXED) {
+      // the kThreads / slots threads of one slot add up in a fixed order
+      const int slot = tid % P.slots;
+      const int g = slot / P.LPG;
+      const int c0 = g * Dg + (slot - g * P.LPG) * VEC;
+      for (int turn = 0; turn < kThreads / P.slots; ++turn) {
+        if (tid / P.slots == turn) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) { s_wg[c0 + e] += rw[e]; s_bg[c0 + e] += rb[e]; }
+        }
+        __syncthreads();
+      }
+    }
     float* dst = P.part + ((size_t)b * P.nt + tile) * 2 * H;
     for (int c = tid; c < H; c += kThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
   } else {
@@ -227,41 +251,78 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   }
 }
 
-__global__ void tsn_bwd_carry_kernel(const TsnBwdParams P) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= P.B * P.G) return;
-  const int b = i / P.G, g = i - b * P.G;
-  float ug = P.mean_grad ? P.mean_grad[i] : 0.f;
-  float vg = P.var_grad ? P.var_grad[i] : 0.f;
-  for (int tile = P.nt - 1; tile >= 0; --tile) {
-    const size_t o = ((size_t)b * P.nt + tile) * P.G + g;
-    P.state[o * 2] = ug;
-    P.state[o * 2 + 1] = vg;
-    const float4 mp = ((const float4*)P.agg)[o];
-    const float nu = fmaf(mp.x, ug, fmaf(mp.y, vg, mp.z));
-    vg = fmaf(mp.x, vg, mp.w);
-    ug = nu;
-  }
-  P.prev_mean_grad[i] = ug;
-  P.prev_var_grad[i] = vg;
+struct TileMap { float a, m, bu, bv; };
+// first `f`, then `s`
+__device__ __forceinline__ TileMap then(const TileMap f, const TileMap s) {
+  return TileMap{s.a * f.a, fmaf(s.a, f.m, s.m * f.a), fmaf(s.a, f.bu, fmaf(s.m, f.bv, s.bu)), fmaf(s.a, f.bv, s.bv)};
 }
 
-__global__ void tsn_bwd_param_kernel(const TsnBwdParams P) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;   // over 2 * H
-  if (c >= 2 * P.H) return;
-  const int ntile = P.B * P.nt;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  int t = 0;
-  for (; t + 4 <= ntile; t += 4) {
-    s0 += P.part[(size_t)t * 2 * P.H + c];
-    s1 += P.part[(size_t)(t + 1) * 2 * P.H + c];
-    s2 += P.part[(size_t)(t + 2) * 2 * P.H + c];
-    s3 += P.part[(size_t)(t + 3) * 2 * P.H + c];
+// One wave per (row, group).  The tiles are walked from the last to the first; lane l owns the
+// l-th run of `per` tiles in that order, composes its run, the runs are combined by a scan over
+// the lanes, and every lane then replays its run from the pair that enters it.
+__global__ __launch_bounds__(64) void tsn_bwd_carry_kernel(const TsnBwdParams P) {
+  const int i = blockIdx.x;               // (row, group)
+  const int b = i / P.G, g = i - b * P.G;
+  const int lane = threadIdx.x;
+  const int per = (P.nt + 63) / 64;
+  const int first = lane * per;           // position in walk order; tile = nt - 1 - position
+  const float4* agg = (const float4*)P.agg + (size_t)b * P.nt * P.G + g;
+  TileMap run{1.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < per; ++k) {
+    const int pos = first + k;
+    if (pos < P.nt) {
+      const float4 v = agg[(size_t)(P.nt - 1 - pos) * P.G];
+      run = then(run, TileMap{v.x, v.y, v.z, v.w});
+    }
   }
-  for (; t < ntile; ++t) s0 += P.part[(size_t)t * 2 * P.H + c];
-  const float s = (s0 + s1) + (s2 + s3);
-  if (c < P.H) P.gamma_grad[c] = s;
-  else P.beta_grad[c - P.H] = s;
+  TileMap inc = run;                      // inclusive scan over the lanes
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    TileMap prev{__shfl_up(inc.a, o), __shfl_up(inc.m, o), __shfl_up(inc.bu, o), __shfl_up(inc.bv, o)};
+    if (lane >= o) inc = then(prev, inc);
+  }
+  TileMap exc{__shfl_up(inc.a, 1), __shfl_up(inc.m, 1), __shfl_up(inc.bu, 1), __shfl_up(inc.bv, 1)};
+  if (lane == 0) exc = TileMap{1.f, 0.f, 0.f, 0.f};
+  const float u0 = P.mean_grad ? P.mean_grad[i] : 0.f;
+  const float v0 = P.var_grad ? P.var_grad[i] : 0.f;
+  float ug = fmaf(exc.a, u0, fmaf(exc.m, v0, exc.bu));
+  float vg = fmaf(exc.a, v0, exc.bv);
+  for (int k = 0; k < per; ++k) {
+    const int pos = first + k;
+    if (pos < P.nt) {
+      const size_t o = ((size_t)b * P.nt + (P.nt - 1 - pos)) * P.G + g;
+      P.state[o * 2] = ug;
+      P.state[o * 2 + 1] = vg;
+      const float4 v = ((const float4*)P.agg)[o];
+      const float nu = fmaf(v.x, ug, fmaf(v.y, vg, v.z));
+      vg = fmaf(v.x, vg, v.w);
+      ug = nu;
+    }
+  }
+  if (lane == 63) {
+    P.prev_mean_grad[i] = fmaf(inc.a, u0, fmaf(inc.m, v0, inc.bu));
+    P.prev_var_grad[i] = fmaf(inc.a, v0, inc.bv);
+  }
+}
+
+// gamma / beta: 32 columns x 8 tile lanes per workgroup
+__global__ __launch_bounds__(256) void tsn_bwd_param_kernel(const TsnBwdParams P) {
+  __shared__ float s_acc[8][33];
+  const int cl = threadIdx.x & 31, tl = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + cl;     // over 2 * H
+  const int ntile = P.B * P.nt;
+  float s = 0.f;
+  if (c < 2 * P.H)
+    for (int t = tl; t < ntile; t += 8) s += P.part[(size_t)t * 2 * P.H + c];
+  s_acc[tl][cl] = s;
+  __syncthreads();
+  if (tl == 0 && c < 2 * P.H) {
+    float r = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) r += s_acc[k][cl];
+    if (c < P.H) P.gamma_grad[c] = r;
+    else P.beta_grad[c - P.H] = r;
+  }
 }
 
 struct BwdGeom {
@@ -298,8 +359,10 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
   const size_t lds1 = (5 * cells + P.G) * 4 + (P.TT + 1) * 4;
   static bool attr0 = false, attr1 = false;
   if (!attr0) {
-    (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024);
+    (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0, false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0, true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     attr0 = true;
   }
   if (!attr1) {
@@ -308,13 +371,15 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
     attr1 = true;
   }
   const dim3 grid((unsigned)(P.B * P.nt));
-  hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0>), grid, dim3(kThreads), lds0, s, P);
+  const bool fixed = P.PER == 1 && P.slots <= kThreads && kThreads % P.slots == 0;
+  if (fixed) hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, true>), grid, dim3(kThreads), lds0, s, P);
+  else hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, false>), grid, dim3(kThreads), lds0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (tile maps)");
-  hipLaunchKernelGGL(tsn_bwd_carry_kernel, dim3((unsigned)ceil_div((int64_t)P.B * P.G, 64)), dim3(64), 0, s, P);
+  hipLaunchKernelGGL(tsn_bwd_carry_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (carry)");
   hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 1>), grid, dim3(kThreads), lds1, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (dx)");
-  hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 256)), dim3(256), 0, s, P);
+  hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 32)), dim3(256), 0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (parameters)");
   return MEGA_OK;
 }
