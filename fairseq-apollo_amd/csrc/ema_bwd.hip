@@ -11,8 +11,9 @@
 // two recurrences of the forward kind run next to each other.  One workgroup owns 16 channels of
 // one batch row: thread = (channel, state n), 12 fused multiply-adds per token on the vector
 // ALUs; x and dy tiles pass through LDS so that every layout is read with its own coalescing.
-// Output: per batch row (the sum over rows is left to the caller: B terms, deterministic)
-//   sums [B, D, N, 4] = (Re sum2, Im sum2, Re sum1, Im sum1),  dyx [B, D] = sum_t dy x (for omega).
+// Per batch row the kernel leaves sums [B, D, N, 4] = (Re sum2, Im sum2, Re sum1, Im sum1) and
+// dyx [B, D] = sum_t dy x in the workspace; ema_grad_finalize_kernel adds the rows up in a fixed
+// order and forms dp, dq, dgamma and domega.
 #include "common.h"
 
 namespace mega {
@@ -36,7 +37,7 @@ struct EmaGradArgs {
   int B, D, N, L;
 };
 
-template <typename T>
+template <typename T, bool MASKED>
 __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGradArgs A) {
   __shared__ float s_x[kCh][kTk + 4];
   __shared__ float s_g[kCh][kTk + 4];
@@ -72,13 +73,23 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
     eg[k] = g_chan_fast ? ((e % kCh) << 16 | (e / kCh)) : ((e / kTk) << 16 | (e % kTk));
   }
   const int dmax = A.D - 1 - c0, lmax = A.L - 1;
+  // per element: pointer at tile 0 and pointer of the row's last token (what a token past the end reads)
+  const T* bx[kPerThread]; const T* lx[kPerThread];
+  const T* bg[kPerThread]; const T* lg[kPerThread];
+#pragma unroll
+  for (int k = 0; k < kPerThread; ++k) {
+    const int cx = min(ex[k] >> 16, dmax), cg = min(eg[k] >> 16, dmax);
+    bx[k] = xg + (int64_t)(c0 + cx) * A.sxd + (int64_t)(ex[k] & 0xffff) * A.sxl;
+    lx[k] = xg + (int64_t)(c0 + cx) * A.sxd + (int64_t)lmax * A.sxl;
+    bg[k] = gg + (int64_t)(c0 + cg) * A.sgd + (int64_t)(eg[k] & 0xffff) * A.sgl;
+    lg[k] = gg + (int64_t)(c0 + cg) * A.sgd + (int64_t)lmax * A.sgl;
+  }
   auto fetch = [&](int t0) {
+    const int64_t ox = (int64_t)t0 * A.sxl, og = (int64_t)t0 * A.sgl;
 #pragma unroll
     for (int k = 0; k < kPerThread; ++k) {
-      const int cx = min(ex[k] >> 16, dmax), tx = min(t0 + (ex[k] & 0xffff), lmax);
-      const int cg = min(eg[k] >> 16, dmax), tg = min(t0 + (eg[k] & 0xffff), lmax);
-      px[k] = to_float(xg[(int64_t)(c0 + cx) * A.sxd + (int64_t)tx * A.sxl]);
-      pg[k] = to_float(gg[(int64_t)(c0 + cg) * A.sgd + (int64_t)tg * A.sgl]);
+      px[k] = to_float(*(t0 + (ex[k] & 0xffff) <= lmax ? bx[k] + ox : lx[k]));
+      pg[k] = to_float(*(t0 + (eg[k] & 0xffff) <= lmax ? bg[k] + og : lg[k]));
     }
   };
   fetch(0);
@@ -90,25 +101,22 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
       s_x[cx][tx] = (cx <= dmax && t0 + tx <= lmax) ? px[k] : 0.f;
       s_g[cg][tg] = (cg <= dmax && t0 + tg <= lmax) ? pg[k] : 0.f;
     }
-    if (tid < kTk) {
-      const int tm = min(t0 + tid, lmax);
-      const uint8_t mk = A.mask ? A.mask[(size_t)b * A.L + tm] : (uint8_t)0;
-      s_keep[tid] = mk ? 0.f : 1.f;
-    }
+    if (MASKED && tid < kTk) s_keep[tid] = A.mask[(size_t)b * A.L + min(t0 + tid, lmax)] ? 0.f : 1.f;
     __syncthreads();
     fetch(t0 + kTk);    // the next tile (clamped past the end) is in flight while this one is worked through
 #pragma unroll 4
     for (int t = 0; t < kTk; t += 4) {
       const float4 xv = *(const float4*)&s_x[ch][t];
       const float4 gv = *(const float4*)&s_g[ch][t];
-      const float4 kv = *(const float4*)&s_keep[t];
+      float4 kv = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (MASKED) kv = *(const float4*)&s_keep[t];
       const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ds[4] = {gv.x, gv.y, gv.z, gv.w}, ks[4] = {kv.x, kv.y, kv.z, kv.w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // g[t] = q g[t-1] + s[t-1];  s[t] = q s[t-1] + x[t] (masked tokens enter as zero)
         const float ngr = fmaf(qr, gr, fmaf(-qi, gi, sr));
         const float ngi = fmaf(qr, gi, fmaf(qi, gr, si));
-        const float nsr = fmaf(qr, sr, fmaf(-qi, si, xs[j] * ks[j]));
+        const float nsr = fmaf(qr, sr, fmaf(-qi, si, MASKED ? xs[j] * ks[j] : xs[j]));
         const float nsi = fmaf(qr, si, qi * sr);
         gr = ngr; gi = ngi; sr = nsr; si = nsi;
         a2r = fmaf(ds[j], sr, a2r);
@@ -126,41 +134,88 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
   }
 }
 
+// thread = (channel, state): rows summed in order, then the products of ema_parameters.cc:95-96
+__global__ void ema_grad_finalize_kernel(const float* __restrict__ sums, const float* __restrict__ dyx,
+                                         const float* __restrict__ p, const float* __restrict__ gamma, int B, int D,
+                                         int N, float* __restrict__ dp, float* __restrict__ dq,
+                                         float* __restrict__ dgamma, float* __restrict__ domega) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;   // over D * N
+  if (i >= D * N) return;
+  float s2r = 0.f, s2i = 0.f, s1r = 0.f, s1i = 0.f;
+  for (int b = 0; b < B; ++b) {
+    const float4 v = ((const float4*)sums)[(size_t)b * D * N + i];
+    s2r += v.x; s2i += v.y; s1r += v.z; s1i += v.w;
+  }
+  const float pr = p[i], gr = gamma[2 * i], gi = gamma[2 * i + 1];
+  dp[i] = s2r * gr - s2i * gi;                       // Re(sum2 gamma)
+  dq[2 * i] = pr * (s1r * gr - s1i * gi);            // conj(sum1 p gamma)
+  dq[2 * i + 1] = -pr * (s1r * gi + s1i * gr);
+  dgamma[2 * i] = pr * s2r;                          // conj(sum2 p)
+  dgamma[2 * i + 1] = -pr * s2i;
+  if (i % N == 0) {
+    const int d = i / N;
+    float o = 0.f;
+    for (int b = 0; b < B; ++b) o += dyx[(size_t)b * D + d];
+    domega[d] = o;
+  }
+}
+
 }  // namespace
 }  // namespace mega
 
 using namespace mega;
 
+extern "C" size_t mega_ema_param_grad_workspace_bytes(int64_t B, int64_t D, int64_t N) {
+  if (B <= 0 || D <= 0 || N <= 0) return 256;
+  return align_up((size_t)B * D * N * 16, 256) + align_up((size_t)B * D * 4, 256);
+}
+
 extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, int64_t sgd, int64_t sgl,
-                                   int64_t sxb, int64_t sxd, int64_t sxl, const float* q, const uint8_t* mask,
-                                   int64_t B, int64_t D, int64_t N, int64_t L, float* sums, float* dyx,
-                                   void* stream) {
+                                   int64_t sxb, int64_t sxd, int64_t sxl, const float* p, const float* q,
+                                   const float* gamma, const uint8_t* mask, int64_t B, int64_t D, int64_t N,
+                                   int64_t L, float* dp, float* dq, float* dgamma, float* domega, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "ema_param_grad: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && D > 0 && N > 0 && L >= 0, MEGA_ERR_ARG, "ema_param_grad: bad shape B=%ld D=%ld N=%ld L=%ld",
                (long)B, (long)D, (long)N, (long)L);
   MEGA_REQUIRE(N <= kNs, MEGA_ERR_UNSUPPORTED, "ema_param_grad: ndim=%ld > %d is not supported", (long)N, kNs);
-  MEGA_REQUIRE(B * ceil_div(D, kCh) < (int64_t)1 << 31 && L < (int64_t)1 << 30, MEGA_ERR_UNSUPPORTED,
-               "ema_param_grad: shape too large");
-  if (B == 0) return MEGA_OK;
-  MEGA_REQUIRE(q && sums && dyx && (L == 0 || (dy && x)), MEGA_ERR_ARG, "ema_param_grad: null pointer argument");
-  if (L == 0) {
-    hipMemsetAsync(sums, 0, (size_t)B * D * N * 16, (hipStream_t)stream);
-    hipMemsetAsync(dyx, 0, (size_t)B * D * 4, (hipStream_t)stream);
+  MEGA_REQUIRE(B * ceil_div(D, kCh) < (int64_t)1 << 31 && L < (int64_t)1 << 30 && D * N < (int64_t)1 << 31,
+               MEGA_ERR_UNSUPPORTED, "ema_param_grad: shape too large");
+  MEGA_REQUIRE(p && q && gamma && dp && dq && dgamma && domega, MEGA_ERR_ARG, "ema_param_grad: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  if (B == 0 || L == 0) {
+    (void)hipMemsetAsync(dp, 0, (size_t)D * N * 4, s);
+    (void)hipMemsetAsync(dq, 0, (size_t)D * N * 8, s);
+    (void)hipMemsetAsync(dgamma, 0, (size_t)D * N * 8, s);
+    (void)hipMemsetAsync(domega, 0, (size_t)D * 4, s);
     return MEGA_OK;
   }
-  MEGA_REQUIRE(((uintptr_t)sums % 16) == 0, MEGA_ERR_ARG, "ema_param_grad: sums must be 16-byte aligned");
+  MEGA_REQUIRE(dy && x, MEGA_ERR_ARG, "ema_param_grad: null dy / x");
+  const size_t need = mega_ema_param_grad_workspace_bytes(B, D, N);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
+               "ema_param_grad: workspace of %zu bytes (16-byte aligned) needed", need);
   EmaGradArgs A;
   A.dy = dy; A.x = x; A.sgb = sgb; A.sgd = sgd; A.sgl = sgl; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl;
-  A.q = q; A.mask = mask; A.sums = sums; A.dyx = dyx;
+  A.q = q; A.mask = mask;
+  A.sums = (float*)workspace;
+  A.dyx = (float*)((char*)workspace + align_up((size_t)B * D * N * 16, 256));
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
   const dim3 grid((unsigned)(B * ceil_div(D, kCh)));
-  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH_PG(T)                                                                                   \
+  do {                                                                                                 \
+    if (mask) hipLaunchKernelGGL((ema_param_grad_kernel<T, true>), grid, dim3(kBwdThreads), 0, s, A);  \
+    else hipLaunchKernelGGL((ema_param_grad_kernel<T, false>), grid, dim3(kBwdThreads), 0, s, A);      \
+  } while (0)
   switch (dtype) {
-    case MEGA_F32: hipLaunchKernelGGL(ema_param_grad_kernel<float>, grid, dim3(kBwdThreads), 0, s, A); break;
-    case MEGA_BF16: hipLaunchKernelGGL(ema_param_grad_kernel<bf16_t>, grid, dim3(kBwdThreads), 0, s, A); break;
-    default: hipLaunchKernelGGL(ema_param_grad_kernel<f16_t>, grid, dim3(kBwdThreads), 0, s, A); break;
+    case MEGA_F32: LAUNCH_PG(float); break;
+    case MEGA_BF16: LAUNCH_PG(bf16_t); break;
+    default: LAUNCH_PG(f16_t); break;
   }
+#undef LAUNCH_PG
   MEGA_CHECK_LAUNCH("ema_param_grad");
+  hipLaunchKernelGGL(ema_grad_finalize_kernel, dim3((unsigned)ceil_div(D * N, 256)), dim3(256), 0, s, A.sums, A.dyx, p,
+                     gamma, (int)B, (int)D, (int)N, dp, dq, dgamma, domega);
+  MEGA_CHECK_LAUNCH("ema_param_grad (finalize)");
   return MEGA_OK;
 }

@@ -55,7 +55,30 @@ struct TsnBwdParams {
   int LPG;     // lanes that share one (token, group)
   int PER;     // vectors per lane
   int slots;   // lanes per token = G * LPG
+  int lpg_shift;     // log2(LPG)
+  int slots_shift;   // log2(slots), or -1 when slots is not a power of two
 };
+
+// item -> (token, slot): a shift when the lane count per token is a power of two
+__device__ __forceinline__ void split_item(const TsnBwdParams& P, int i, int& tok, int& slot) {
+  if (P.slots_shift >= 0) {
+    tok = i >> P.slots_shift;
+    slot = i & (P.slots - 1);
+  } else {
+    tok = i / P.slots;
+    slot = i - tok * P.slots;
+  }
+}
+
+struct TileMap { float a, m, bu, bv; };
+// first `f`, then `s`
+__device__ __forceinline__ TileMap then(const TileMap f, const TileMap s) {
+  return TileMap{s.a * f.a, fmaf(s.a, f.m, s.m * f.a), fmaf(s.a, f.bu, fmaf(s.m, f.bv, s.bu)), fmaf(s.a, f.bv, s.bv)};
+}
+
+__device__ __forceinline__ TileMap shfl_up32(const TileMap v, int o) {
+  return TileMap{__shfl_up(v.a, o, 32), __shfl_up(v.m, o, 32), __shfl_up(v.bu, o, 32), __shfl_up(v.bv, o, 32)};
+}
 
 // PHASE 0: tile maps + parameter shares; PHASE 1: dx.
 // FIXED (PHASE 0 only): slots divides the workgroup size and every lane moves one vector, so a
@@ -114,6 +137,61 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   float rw[VEC], rb[VEC];                // FIXED: this thread's gamma / beta shares
 #pragma unroll
   for (int e = 0; e < VEC; ++e) { rw[e] = 0.f; rb[e] = 0.f; }
+  if (P.PER == 1) {
+    // one vector per lane: four items per thread are loaded before any of them is used
+    constexpr int U = 4;
+    for (int i0 = 0; i0 < items; i0 += U * kThreads) {
+      V dvv[U], xvv[U];
+      int tokk[U], cc[U], cellk[U];
+      bool livek[U], leadk[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * kThreads + tid;
+        livek[u] = i < items;
+        int tok, slot;
+        split_item(P, livek[u] ? i : 0, tok, slot);
+        const int g = slot >> P.lpg_shift;
+        tokk[u] = tok;
+        cc[u] = g * Dg + (slot - (g << P.lpg_shift)) * VEC;
+        cellk[u] = tok * G + g;
+        leadk[u] = livek[u] && slot == (g << P.lpg_shift);
+        dvv[u] = *(const V*)(dy + (size_t)tok * H + cc[u]);
+        xvv[u] = *(const V*)(x + (size_t)tok * H + cc[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float u_ = s_u[cellk[u]], r = s_r[cellk[u]];
+        const bool keep = livek[u] && !s_mask[tokk[u]];
+        float ds = 0.f, db = 0.f, sx = 0.f;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float d = livek[u] ? to_float(dvv[u].v[e]) : 0.f, xe = to_float(xvv[u].v[e]), w = P.gamma[cc[u] + e];
+          ds = fmaf(d * (xe - u_), w, ds);
+          db = fmaf(d, w, db);
+          sx += xe;
+          if (PHASE == 0 && keep) {
+            if (FIXED) {
+              rw[e] = fmaf(d * (xe - u_), r, rw[e]);
+              rb[e] += d;
+            } else {
+              atomicAdd(&s_wg[cc[u] + e], d * (xe - u_) * r);
+              atomicAdd(&s_bg[cc[u] + e], d);
+            }
+          }
+        }
+        for (int o = 1; o < P.LPG; o <<= 1) {
+          ds += __shfl_xor(ds, o);
+          db += __shfl_xor(db, o);
+          sx += __shfl_xor(sx, o);
+        }
+        if (leadk[u]) {
+          s_ds[cellk[u]] = ds;
+          s_db[cellk[u]] = db;
+          if (!P.group_mean) s_ux[cellk[u]] = sx / (float)Dg;
+        }
+      }
+    }
+  } else {
   for (int i0 = 0; i0 < items; i0 += kThreads) {
     const int i = i0 + tid;
     const bool live = i < items;
@@ -137,13 +215,8 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
           db = fmaf(d, w, db);
           sx += xe;
           if (PHASE == 0 && keep) {
-            if (FIXED) {
-              rw[e] = fmaf(d * (xe - u), r, rw[e]);
-              rb[e] += d;
-            } else {
-              atomicAdd(&s_wg[c + e], d * (xe - u) * r);
-              atomicAdd(&s_bg[c + e], d);
-            }
+            atomicAdd(&s_wg[c + e], d * (xe - u) * r);
+            atomicAdd(&s_bg[c + e], d);
           }
         }
       }
@@ -159,10 +232,60 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
       if (!P.group_mean) s_ux[cell] = sx / (float)Dg;
     }
   }
+  }
   __syncthreads();
 
   // ---- the walk over the tile's tokens, last to first, one thread per group
   const int64_t n_end = P.count[b] - (P.mask ? s_mask[TT] : max(0, P.L - t0 - TT));
+  if (TT >= 16) {
+    // 32 lanes per group, lane = position in walk order (0 = the tile's last token): every token's
+    // map at once, then a scan over the positions
+    const int pos = tid & 31;
+    const int tok = ntok - 1 - pos;
+    for (int g0 = 0; g0 < G; g0 += kThreads / 32) {
+      const int g = g0 + (tid >> 5);
+      const bool valid = g < G;
+      const bool has = valid && tok >= 0 && !s_mask[max(tok, 0)];
+      const unsigned long long bal = __ballot(has);
+      const unsigned half = (unsigned)(bal >> (tid & 32));
+      const int64_t n = n_end - __popc(half & ((1u << pos) - 1u));
+      const int cell = max(tok, 0) * G + (valid ? g : 0);
+      float c2 = 0.f, e = 0.f, rdb = 0.f, mj = 0.f;
+      TileMap own{1.f, 0.f, 0.f, 0.f};
+      if (has) {
+        c2 = 1.0f / (float)n;
+        const float c1 = (float)(n - 1) * c2;
+        const float r = s_r[cell];
+        const float up = tok == 0 ? s_up0[g] : s_u[cell - G];
+        const float delta = s_ux[cell] - up;
+        e = 0.5f * r * r * r * s_ds[cell];
+        rdb = r * s_db[cell];
+        mj = -2.0f * c1 * c2 * delta;
+        own = TileMap{c1, mj, -c1 * rdb - mj * e, -c1 * e};
+      }
+      TileMap inc = own;
+#pragma unroll
+      for (int o = 1; o < 32; o <<= 1) {
+        const TileMap prev = shfl_up32(inc, o);
+        if (pos >= o) inc = then(prev, inc);
+      }
+      if (PHASE == 0) {
+        if (valid && pos == 31) ((float4*)P.agg)[((size_t)b * P.nt + tile) * G + g] = make_float4(inc.a, inc.m, inc.bu, inc.bv);
+      } else {
+        TileMap exc = shfl_up32(inc, 1);
+        if (pos == 0) exc = TileMap{1.f, 0.f, 0.f, 0.f};
+        if (valid && tok >= 0) {
+          const size_t so = (((size_t)b * P.nt + tile) * G + g) * 2;
+          const float u0 = P.state[so], v0 = P.state[so + 1];
+          const float ug = fmaf(exc.a, u0, fmaf(exc.m, v0, exc.bu));
+          const float vg = fmaf(exc.a, v0, exc.bv);
+          const float du = ug - rdb, dv = vg - e;
+          s_ds[cell] = has ? c2 * du - mj * dv : 0.f;      // dux
+          s_db[cell] = has ? c2 * dv : 0.f;                // dvx
+        }
+      }
+    }
+  } else
   for (int g = tid; g < G; g += kThreads) {
     int64_t n = n_end;                         // running count at the tile's last unmasked token
     float a = 1.f, m = 0.f, bu = 0.f, bv = 0.f;
@@ -226,35 +349,65 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   } else {
     T* dx = (T*)P.dx + ((size_t)b * P.L + t0) * H;
     const float cg = 1.0f / (float)Dg;
-    for (int i = tid; i < items; i += kThreads) {
-      const int tok = i / P.slots;
-      const int slot = i - tok * P.slots;
-      const int g = slot / P.LPG;
-      const int c0 = g * Dg + (slot - g * P.LPG) * span;
-      const int cell = tok * G + g;
-      const float r = s_r[cell], ux = s_ux[cell];
-      const float a0 = s_ds[cell] * cg, a1 = 2.0f * s_db[cell] * cg;
-      const bool keep = !s_mask[tok];
-      for (int k = 0; k < P.PER; ++k) {
-        const int c = c0 + k * VEC;
-        const V dv = *(const V*)(dy + (size_t)tok * H + c);
-        const V xv = *(const V*)(x + (size_t)tok * H + c);
-        V o;
+    if (P.PER == 1) {
+      constexpr int U = 4;
+      for (int i0 = 0; i0 < items; i0 += U * kThreads) {
+        V dvv[U], xvv[U];
+        int tokk[U], cc[U], cellk[U];
+        bool livek[U];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const float v = fmaf(to_float(dv.v[e]) * r, P.gamma[c + e], fmaf(a1, to_float(xv.v[e]) - ux, a0));
-          o.v[e] = from_float<T>(keep ? v : 0.f);
+        for (int u = 0; u < U; ++u) {
+          const int i = i0 + u * kThreads + tid;
+          livek[u] = i < items;
+          int tok, slot;
+          split_item(P, livek[u] ? i : 0, tok, slot);
+          const int g = slot >> P.lpg_shift;
+          tokk[u] = tok;
+          cc[u] = g * Dg + (slot - (g << P.lpg_shift)) * VEC;
+          cellk[u] = tok * G + g;
+          dvv[u] = *(const V*)(dy + (size_t)tok * H + cc[u]);
+          xvv[u] = *(const V*)(x + (size_t)tok * H + cc[u]);
         }
-        *(V*)(dx + (size_t)tok * H + c) = o;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const float r = s_r[cellk[u]], ux = s_ux[cellk[u]];
+          const float a0 = s_ds[cellk[u]] * cg, a1 = 2.0f * s_db[cellk[u]] * cg;
+          const bool keep = !s_mask[tokk[u]];
+          V o;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float v = fmaf(to_float(dvv[u].v[e]) * r, P.gamma[cc[u] + e],
+                                 fmaf(a1, to_float(xvv[u].v[e]) - ux, a0));
+            o.v[e] = from_float<T>(keep ? v : 0.f);
+          }
+          if (livek[u]) *(V*)(dx + (size_t)tokk[u] * H + cc[u]) = o;
+        }
+      }
+    } else {
+      for (int i = tid; i < items; i += kThreads) {
+        const int tok = i / P.slots;
+        const int slot = i - tok * P.slots;
+        const int g = slot / P.LPG;
+        const int c0 = g * Dg + (slot - g * P.LPG) * span;
+        const int cell = tok * G + g;
+        const float r = s_r[cell], ux = s_ux[cell];
+        const float a0 = s_ds[cell] * cg, a1 = 2.0f * s_db[cell] * cg;
+        const bool keep = !s_mask[tok];
+        for (int k = 0; k < P.PER; ++k) {
+          const int c = c0 + k * VEC;
+          const V dv = *(const V*)(dy + (size_t)tok * H + c);
+          const V xv = *(const V*)(x + (size_t)tok * H + c);
+          V o;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float v = fmaf(to_float(dv.v[e]) * r, P.gamma[c + e], fmaf(a1, to_float(xv.v[e]) - ux, a0));
+            o.v[e] = from_float<T>(keep ? v : 0.f);
+          }
+          *(V*)(dx + (size_t)tok * H + c) = o;
+        }
       }
     }
   }
-}
-
-struct TileMap { float a, m, bu, bv; };
-// first `f`, then `s`
-__device__ __forceinline__ TileMap then(const TileMap f, const TileMap s) {
-  return TileMap{s.a * f.a, fmaf(s.a, f.m, s.m * f.a), fmaf(s.a, f.bu, fmaf(s.m, f.bv, s.bu)), fmaf(s.a, f.bv, s.bv)};
 }
 
 // One wave per (row, group).  The tiles are walked from the last to the first; lane l owns the
@@ -312,8 +465,17 @@ __global__ __launch_bounds__(256) void tsn_bwd_param_kernel(const TsnBwdParams P
   const int c = blockIdx.x * 32 + cl;     // over 2 * H
   const int ntile = P.B * P.nt;
   float s = 0.f;
-  if (c < 2 * P.H)
-    for (int t = tl; t < ntile; t += 8) s += P.part[(size_t)t * 2 * P.H + c];
+  if (c < 2 * P.H) {
+    int t = tl;
+    for (; t + 56 < ntile; t += 64) {       // eight loads in flight
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = P.part[(size_t)(t + 8 * k) * 2 * P.H + c];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; t < ntile; t += 8) s += P.part[(size_t)t * 2 * P.H + c];
+  }
   s_acc[tl][cl] = s;
   __syncthreads();
   if (tl == 0 && c < 2 * P.H) {
@@ -454,6 +616,13 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
   P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
   P.LPG = g.lpg; P.PER = g.per; P.slots = (int)G * g.lpg;
+  P.lpg_shift = 0;
+  while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
+  P.slots_shift = -1;
+  if ((P.slots & (P.slots - 1)) == 0) {
+    P.slots_shift = 0;
+    while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
+  }
   switch (dtype) {
     case MEGA_F32: return launch_bwd<float>(P, g.vec, s);
     case MEGA_BF16: return launch_bwd<bf16_t>(P, g.vec, s);

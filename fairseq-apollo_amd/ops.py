@@ -756,22 +756,19 @@ def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torc
     if 0 in g.stride() and g.numel() > 0:
         g = g.contiguous()
     dx = layer.adjoint(g, padding_mask)
-    sums = torch.empty(B, D, N, 4, dtype=torch.float32, device=dev)
-    dyx = torch.empty(B, D, dtype=torch.float32, device=dev)
+    dp = torch.empty(D, N, dtype=torch.float32, device=dev)
+    dq = torch.empty(D, N, 2, dtype=torch.float32, device=dev)
+    dg = torch.empty(D, N, 2, dtype=torch.float32, device=dev)
+    dom = torch.empty(D, dtype=torch.float32, device=dev)
     m8 = _mask_u8(padding_mask, B, L)
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, lib.mega_ema_param_grad_workspace_bytes(B, D, N), stream)
     with _on_device(dev):
         rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
-                                     xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.q), _ptr(m8), B, D, N, L,
-                                     _ptr(sums), _ptr(dyx), _stream(dev))
+                                     xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.p), _ptr(layer.q),
+                                     _ptr(layer.gamma), _ptr(m8), B, D, N, L, _ptr(dp), _ptr(dq), _ptr(dg), _ptr(dom),
+                                     _ptr(ws), ws.numel(), stream)
     _lib.check(rc, "ema_param_grad")
-    tot = sums.sum(0)                                   # [D, N, 4]
-    s2 = torch.complex(tot[..., 0], tot[..., 1])
-    s1 = torch.complex(tot[..., 2], tot[..., 3])
-    pc = layer.p.to(torch.complex64)
-    gc = torch.view_as_complex(layer.gamma)
-    dp = (s2 * gc).real
-    dq = torch.conj(s1 * pc * gc)
-    dg = torch.conj(s2 * pc)
-    if not layer.is_complex:
-        dq, dg = dq.real, dg.real
-    return dx, dp, dq, dg, dyx.sum(0)
+    if layer.is_complex:
+        return dx, dp, torch.view_as_complex(dq), torch.view_as_complex(dg), dom
+    return dx, dp, dq[..., 0], dg[..., 0], dom

@@ -158,19 +158,22 @@ int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_
  * x = y_grad, pointers at the last token and negated token strides (the kernel is
  * k[l] for l >= 0, so dx[t] = sum_{s>=t} k[s-t] dy[s] + omega dy[t]).
  * mega_ema_param_grad stands in for the kernel-gradient half of fftconv_bwd
- * (fairseq/modules/fused_ops/fftconv.py:66-88) followed by the sums of
- * ema_parameters_bwd (fairseq/csrc/ops/ema_parameters.cc:80-97), without forming dk:
- *   sums[b,d,n] = (Re, Im of sum_t dy[t] s[t]; Re, Im of sum_t dy[t] g[t]),
+ * (fairseq/modules/fused_ops/fftconv.py:66-88) followed by ema_parameters_bwd
+ * (fairseq/csrc/ops/ema_parameters.cc:80-97) for a layer without carried state, without
+ * forming dk:
+ *   S2[d,n] = sum_{b,t} dy[t] s[t],  S1[d,n] = sum_{b,t} dy[t] g[t],
  *   s[t] = q s[t-1] + x[t] (masked x enters as 0), g[t] = q g[t-1] + s[t-1];
- *   dyx[b,d] = sum_t dy[t] x[t] (the gradient of omega).
- * The caller sums over b and forms dp = Re(S2 gamma), dq = conj(S1 p gamma),
- * dgamma = conj(S2 p) (ema_parameters.cc:95-96).
- *   dy, x [B,D,L] of `dtype` with element strides; q [D,N,2] fp32 (imaginary part 0 for the
- *   real layer); mask [B,L] or NULL; sums [B,D,N,4], dyx [B,D] fp32; N <= 16.           */
+ *   dp = Re(S2 gamma), dq = conj(S1 p gamma), dgamma = conj(S2 p) (ema_parameters.cc:95-96),
+ *   domega[d] = sum_{b,t} dy[t] x[t].
+ *   dy, x [B,D,L] of `dtype` with element strides; p [D,N], q, gamma [D,N,2] fp32 (imaginary
+ *   parts 0 for the real layer); mask [B,L] or NULL; outputs dp [D,N], dq, dgamma [D,N,2],
+ *   domega [D] fp32; N <= 16; workspace of mega_ema_param_grad_workspace_bytes(B, D, N).   */
+size_t mega_ema_param_grad_workspace_bytes(int64_t B, int64_t D, int64_t N);
 int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, int64_t sgd,
-                        int64_t sgl, int64_t sxb, int64_t sxd, int64_t sxl, const float* q,
-                        const uint8_t* mask, int64_t B, int64_t D, int64_t N, int64_t L,
-                        float* sums, float* dyx, void* stream);
+                        int64_t sgl, int64_t sxb, int64_t sxd, int64_t sxl, const float* p,
+                        const float* q, const float* gamma, const uint8_t* mask, int64_t B,
+                        int64_t D, int64_t N, int64_t L, float* dp, float* dq, float* dgamma,
+                        float* domega, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Long convolution with an explicit time-domain kernel                      */
