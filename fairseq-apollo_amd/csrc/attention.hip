@@ -108,6 +108,68 @@ __global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restri
   }
 }
 
+// Softmax backward (fairseq/csrc/softmax.cuh AttentionSoftmaxBwdKernel, called from
+// ops/attention_softmax_kernel.cu and ops/attention_kernel.cu:195-203):
+//   dx[r, c] = scale * y[r, c] * (dy[r, c] - sum_c' y[r, c'] dy[r, c']).
+// One wave per row, four rows per workgroup; columns behind the causal limit hold y = 0 and are
+// written as zeros without being read.  dx may alias dy.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const T* dy, const T* __restrict__ y,
+                                                          T* dx, int64_t rows, int outer, int inner, int causal,
+                                                          float scale) {
+  using V = Vec<T, VEC>;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int r = (int)(row % outer);
+  int limit = causal ? inner - outer + r + 1 : inner;     // columns that can be non-zero
+  if (limit < 0) limit = 0;
+  if (limit > inner) limit = inner;
+  const T* dyr = dy + row * inner;
+  const T* yr = y + row * inner;
+  T* dxr = dx + row * inner;
+  float dot = 0.f;
+  for (int c = lane * VEC; c < limit; c += 64 * VEC) {
+    const V a = *(const V*)(dyr + c);
+    const V b = *(const V*)(yr + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+      if (c + e < limit) dot = fmaf(to_float(a.v[e]), to_float(b.v[e]), dot);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
+  for (int c = lane * VEC; c < inner; c += 64 * VEC) {
+    V o;
+    if (c < limit) {
+      const V a = *(const V*)(dyr + c);
+      const V b = *(const V*)(yr + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        o.v[e] = from_float<T>(c + e < limit ? scale * to_float(b.v[e]) * (to_float(a.v[e]) - dot) : 0.f);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o.v[e] = from_float<T>(0.f);
+    }
+    *(V*)(dxr + c) = o;
+  }
+}
+
+template <typename T>
+int launch_softmax_bwd(const void* dy, const void* y, void* dx, int64_t rows, int64_t outer, int64_t inner, int causal,
+                       float scale, hipStream_t s) {
+  constexpr int FULL = 16 / (int)sizeof(T);
+  const dim3 grid((unsigned)ceil_div(rows, 4));
+  const bool vec = inner % FULL == 0 && ((((uintptr_t)dy | (uintptr_t)y | (uintptr_t)dx) % 16) == 0);
+  if (vec)
+    hipLaunchKernelGGL((softmax_bwd_kernel<T, FULL>), grid, dim3(256), 0, s, (const T*)dy, (const T*)y, (T*)dx, rows,
+                       (int)outer, (int)inner, causal, scale);
+  else
+    hipLaunchKernelGGL((softmax_bwd_kernel<T, 1>), grid, dim3(256), 0, s, (const T*)dy, (const T*)y, (T*)dx, rows,
+                       (int)outer, (int)inner, causal, scale);
+  MEGA_CHECK_LAUNCH("attention_softmax_bwd");
+  return MEGA_OK;
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -180,4 +242,22 @@ extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, v
 #undef LAUNCH_ATT
   MEGA_CHECK_LAUNCH("attention_fwd");
   return MEGA_OK;
+}
+
+extern "C" int mega_attention_softmax_bwd(const void* y_grad, const void* y, void* x_grad, int dtype, int64_t batch,
+                                          int64_t outer, int64_t inner, int causal, float scale, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "attention_softmax_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(batch >= 0 && outer >= 0 && inner >= 0, MEGA_ERR_ARG, "attention_softmax_bwd: negative size");
+  const int64_t rows = batch * outer;
+  if (rows == 0 || inner == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && y && x_grad, MEGA_ERR_ARG, "attention_softmax_bwd: null pointer argument");
+  MEGA_REQUIRE(rows < (int64_t)1 << 33 && inner < (int64_t)1 << 30 && outer < (int64_t)1 << 30, MEGA_ERR_UNSUPPORTED,
+               "attention_softmax_bwd: shape too large");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MEGA_F32: return launch_softmax_bwd<float>(y_grad, y, x_grad, rows, outer, inner, causal, scale, s);
+    case MEGA_BF16: return launch_softmax_bwd<bf16_t>(y_grad, y, x_grad, rows, outer, inner, causal, scale, s);
+    default: return launch_softmax_bwd<f16_t>(y_grad, y, x_grad, rows, outer, inner, causal, scale, s);
+  }
 }

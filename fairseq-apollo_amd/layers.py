@@ -4,7 +4,10 @@ restricted to what Mega2 uses on the causal path (unidirectional, softmax attent
 the fused rotary / causal op, TimestepNorm, EMA or CEMA), plus the north-star SwiGLU FFN.
 
 The projections are library GEMMs (torch -> hipBLASLt); normalisation, moving average,
-attention and the SwiGLU gate run in libmega_hip.so.  Forward only.
+attention and the SwiGLU gate run in libmega_hip.so.  Under autograd the normalisation, the
+moving average and the attention (softmax backward in libmega_hip.so, batched library GEMMs) keep
+their own backward operators; the element-wise glue then runs as torch operations so that the
+graph is complete.
 """
 from __future__ import annotations
 
@@ -18,7 +21,7 @@ from torch.nn import Parameter
 
 from . import ops
 from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SwiGLU, TimestepNorm,
-                      _no_grad_only)
+                      _training_call)
 
 
 class RMSNorm(nn.Module):
@@ -34,7 +37,12 @@ class RMSNorm(nn.Module):
             self.register_parameter("weight", None)
 
     def forward(self, x: Tensor) -> Tensor:
-        _no_grad_only(self, x)
+        if _training_call(self, x):
+            y = x.float()
+            y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.eps)
+            if self.weight is not None:
+                y = y * self.weight.float()
+            return y.to(x.dtype)
         return ops.rms_norm_fwd(x, self.weight, self.eps)
 
 
@@ -85,7 +93,6 @@ class NormalizedFeedForwardNetwork(nn.Module):
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 
     def forward(self, x: Tensor) -> Tensor:
-        _no_grad_only(self, x)
         h = self.fc2(F.silu(self.fc1(self.norm(x))))
         if self.layerscale_weight is not None:
             h = h * self.layerscale_weight
@@ -175,7 +182,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
                 incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None):
         """x: [B, L, D] -> ([B, L, D], None)."""
-        _no_grad_only(self, x)
+        if _training_call(self, x):
+            return self._forward_autograd(x, padding_mask, incremental_state), None
         bsz, seq_len, embed_dim = x.size()
         assert embed_dim == self.embed_dim
         saved_state = self._get_input_buffer(incremental_state) if incremental_state is not None else None
@@ -201,6 +209,35 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         # projection, u and the residual mix after it
         hp = self.h_proj(ops.gate_mul_fwd(attn.reshape(bsz, seq_len, self.hdim), r))
         return ops.gate_out_fwd(residual, u, hx, hp), None
+
+    def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
+        """The same layer with a complete autograd graph (moving_average_gated_attention.py:263-417,
+        whole chunks, no cache): TimestepNorm, the moving average and the attention carry their own
+        backward operators, the element-wise steps are torch operations."""
+        if incremental_state is not None:
+            raise NotImplementedError("MovingAverageGatedAttention: incremental state is an inference feature; "
+                                      "call it under torch.no_grad()")
+        bsz, seq_len, _ = x.size()
+        residual = x
+        x = self.norm(x, padding_mask=padding_mask)
+        v = F.silu(self.v_proj(x))
+        mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
+        base = self.mx_proj(self.move_act(mx))
+        u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
+        z = F.normalize(z, p=2, dim=-1, eps=1e-5)
+        z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
+        q, k = torch.unbind(z, dim=2)
+        Nh = self.num_heads
+        C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
+        nc = seq_len // C
+        q4 = q.reshape(bsz * nc, C, Nh, -1)
+        k4 = k.reshape(bsz * nc, C, Nh, -1)
+        v4 = v.reshape(bsz * nc, C, Nh, -1)
+        q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
+        k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+        attn = self.efficient_attn(q4, k4, v4).reshape(bsz, seq_len, self.hdim)
+        h = F.silu(hx + self.h_proj(attn * F.silu(r)))
+        return torch.addcmul(residual, torch.sigmoid(u), h - residual)
 
     def _cached_attention(self, z: Tensor, v: Tensor, saved_state, incremental_state) -> Tensor:
         """Attention with the partial-chunk key / value cache

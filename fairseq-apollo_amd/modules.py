@@ -51,17 +51,6 @@ class IncrementalState(object):
         return incremental_state
 
 
-def _no_grad_only(module: nn.Module, *tensors):
-    if torch.is_grad_enabled() and (
-        any(t is not None and t.requires_grad for t in tensors)
-        or any(p.requires_grad for p in module.parameters())
-    ):
-        raise RuntimeError(
-            f"{type(module).__name__}: the HIP path implements the forward pass only; "
-            "call it under torch.no_grad() (inference)"
-        )
-
-
 class MovingAverageFunc(torch.autograd.Function):
     """The whole unidirectional moving-average layer as one differentiable operator: the
     reference chains EMAParametersFunc (fused_ops/ema_parameters.py:11-33) and FFTConvFunc
@@ -83,6 +72,12 @@ class MovingAverageFunc(torch.autograd.Function):
                                                padding_mask, layer=ctx.layer)
         return (dx, dp.to(p.dtype).view_as(p), dq.to(q.dtype).view_as(q), dg.to(gamma.dtype).view_as(gamma),
                 dom.to(omega.dtype).view_as(omega), None, None)
+
+
+def _training_call(module: nn.Module, *tensors) -> bool:
+    """True when the call must build an autograd graph."""
+    return torch.is_grad_enabled() and (any(t is not None and t.requires_grad for t in tensors)
+                                        or any(p.requires_grad for p in module.parameters()))
 
 
 class BaseMovingLayer(nn.Module, IncrementalState):
@@ -466,6 +461,50 @@ class TimestepNorm(nn.Module, IncrementalState):
             **self.__dict__)
 
 
+class AttentionSoftmaxFunc(torch.autograd.Function):
+    """fairseq/modules/attention_softmax.py:11-39 (dropout = 0)."""
+
+    @staticmethod
+    def forward(ctx, x, dropout: float = 0.0, use_causal_mask: bool = True, training: bool = True):
+        y = ops.attention_softmax_fwd(x, dropout if training else 0.0, use_causal_mask)
+        ctx.save_for_backward(y)
+        ctx.use_causal_mask = use_causal_mask
+        return y
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        y, = ctx.saved_tensors
+        return ops.attention_softmax_bwd(y_grad, y, ctx.use_causal_mask), None, None, None
+
+
+class AttentionFunc(torch.autograd.Function):
+    """fairseq/modules/efficient_attention.py:11-40 (dropout = 0): the forward keeps the L x L
+    weights for the backward pass, as the reference does."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale: float = 1.0, dropout: float = 0.0, use_causal_mask: bool = True,
+                training: bool = True):
+        y, w = ops.attention_fwd(q, k, v, scale, dropout if training else 0.0, use_causal_mask, need_weights=True)
+        ctx.save_for_backward(q, k, v, w)
+        ctx.scale = scale
+        ctx.use_causal_mask = use_causal_mask
+        return y
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        q, k, v, w = ctx.saved_tensors
+        q_grad, k_grad, v_grad = ops.attention_bwd(y_grad, q, k, v, w, ctx.scale, ctx.use_causal_mask)
+        return q_grad, k_grad, v_grad, None, None, None, None
+
+
+attention_softmax = AttentionSoftmaxFunc.apply
+attention = AttentionFunc.apply
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
 class AttentionSoftmax(nn.Module):
     """fairseq/modules/attention_softmax.py:44-56."""
 
@@ -475,7 +514,8 @@ class AttentionSoftmax(nn.Module):
         self._causal = use_causal_mask
 
     def forward(self, x: Tensor) -> Tensor:
-        _no_grad_only(self, x)
+        if _wants_grad(x):
+            return attention_softmax(x, self._dropout, self._causal, self.training)
         return ops.attention_softmax_fwd(x, self._dropout if self.training else 0.0, self._causal)
 
     def extra_repr(self) -> str:
@@ -493,11 +533,13 @@ class EfficientAttention(nn.Module):
         self._causal = use_causal_mask
 
     def forward(self, q: Tensor, k: Tensor, v: Tensor) -> Tensor:
-        _no_grad_only(self, q, k, v)
         squeeze = q.dim() == 3
         if squeeze:
             q, k, v = q.unsqueeze(2), k.unsqueeze(2), v.unsqueeze(2)
-        out, _ = ops.attention_fwd(q, k, v, self._scale, self._dropout if self.training else 0.0, self._causal)
+        if _wants_grad(q, k, v):
+            out = attention(q, k, v, self._scale, self._dropout, self._causal, self.training)
+        else:
+            out, _ = ops.attention_fwd(q, k, v, self._scale, self._dropout if self.training else 0.0, self._causal)
         return out.squeeze(2) if squeeze else out
 
     def extra_repr(self) -> str:
@@ -515,5 +557,6 @@ class SwiGLU(nn.Module):
         self.w2 = nn.Linear(hidden_dim, embed_dim, bias=bias)
 
     def forward(self, x: Tensor) -> Tensor:
-        _no_grad_only(self, x)
+        if _training_call(self, x):
+            return self.w2(F.silu(self.w1(x)) * self.w3(x))      # autograd: element-wise gate in torch
         return self.w2(ops.swiglu(self.w1(x), self.w3(x)))

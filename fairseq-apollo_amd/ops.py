@@ -370,6 +370,44 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
     return y, w
 
 
+def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask: bool, scale: float = 1.0,
+                          inplace: bool = False) -> torch.Tensor:
+    """x_grad = scale * y * (y_grad - sum(y * y_grad, -1)).  Reference: attention_softmax_bwd,
+    fairseq/csrc/ops/attention_softmax.cc:20-26 (scale = 1); `inplace` overwrites y_grad, as the
+    reference's attention backward does with its weight gradient."""
+    dev = _need_gpu(y_grad, y)
+    lib = _lib.load()
+    if y_grad.shape != y.shape or y.dim() < 2:
+        raise RuntimeError("attention_softmax_bwd: y_grad and y must have the same shape (>= 2 dimensions)")
+    yd = y.detach().contiguous()
+    gd = y_grad.detach().to(yd.dtype).contiguous()
+    outer, inner = yd.shape[-2], yd.shape[-1]
+    batch = yd.numel() // max(outer * inner, 1)
+    dx = gd if inplace else torch.empty_like(yd)
+    with _on_device(dev):
+        rc = lib.mega_attention_softmax_bwd(_ptr(gd), _ptr(yd), _ptr(dx), _dtype_code(yd), batch, outer, inner,
+                                            1 if use_causal_mask else 0, float(scale), _stream(dev))
+    _lib.check(rc, "attention_softmax_bwd")
+    return dx
+
+
+def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool):
+    """-> (q_grad, k_grad, v_grad).  Reference: attention_bwd, fairseq/csrc/ops/attention_kernel.cu:133-255:
+    four batched library GEMMs around the softmax backward, which runs in place on the weight
+    gradient; w [B, Nh, L, L] are the forward's weights."""
+    dev = _need_gpu(y_grad, q, k, v, w)
+    if q.dim() != 4 or w is None or w.dim() != 4:
+        raise RuntimeError("attention_bwd: q, k, v must be [B,L,N,H] and w [B,N,L,L]")
+    g = y_grad.detach().to(q.dtype)
+    qd, kd, vd, wd = q.detach(), k.detach(), v.detach(), w.detach()
+    v_grad = torch.einsum('bnqk,bqnh->bknh', wd, g)
+    w_grad = torch.einsum('bqnh,bknh->bnqk', g, vd).contiguous()
+    s_grad = attention_softmax_bwd(w_grad, wd, use_causal_mask, scale=float(scale), inplace=True)
+    k_grad = torch.einsum('bnqk,bqnh->bknh', s_grad, qd)
+    q_grad = torch.einsum('bnqk,bknh->bqnh', s_grad, kd)
+    return q_grad, k_grad, v_grad
+
+
 # --------------------------------------------------------------------------------------
 # fused inference entry points used by the modules
 # --------------------------------------------------------------------------------------

@@ -250,6 +250,14 @@ int mega_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const flo
  *   inner - outer + r + 1 columns; a fully masked row becomes zeros.              */
 int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch, int64_t outer,
                                int64_t inner, int causal, void* stream);
+/* stands in for attention_softmax_bwd (fairseq/csrc/ops/attention_softmax.cc:20-26,
+ * softmax.cuh AttentionSoftmaxBwdKernel; also the middle step of attention_bwd,
+ * ops/attention_kernel.cu:195-203):
+ *   x_grad = scale * y * (y_grad - rowsum(y * y_grad)); columns behind the causal limit are 0.
+ *   x_grad may be the same buffer as y_grad.                                            */
+int mega_attention_softmax_bwd(const void* y_grad, const void* y, void* x_grad, int dtype,
+                               int64_t batch, int64_t outer, int64_t inner, int causal,
+                               float scale, void* stream);
 
 /* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276),
  * dropout = 0:  q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;

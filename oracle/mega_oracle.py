@@ -510,6 +510,30 @@ def attention(q, k, v, scale: float = 1.0, causal: bool = True):
     return y, w
 
 
+def attention_softmax_bwd(dy, y):
+    """csrc/softmax.cuh AttentionSoftmaxBwdKernel: dx = y (dy - sum(y dy, -1)); masked columns hold
+    y = 0 and get dx = 0."""
+    dy = np.asarray(dy, np.float64)
+    y = np.asarray(y, np.float64)
+    return y * (dy - (y * dy).sum(-1, keepdims=True))
+
+
+def attention_bwd(dy, q, k, v, scale: float = 1.0, causal: bool = True):
+    """csrc/ops/attention_kernel.cu:133-255: dv = w^T dy, dw = dy v^T, ds = softmax_bwd(dw, w),
+    dk = scale ds^T q, dq = scale ds k per (batch, head).  Returns (dq, dk, dv)."""
+    dy = np.asarray(dy, np.float64)
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    _, w = attention(q, k, v, scale, causal)
+    dv = np.einsum('bnlm,blnh->bmnh', w, dy)
+    dw = np.einsum('blnh,bmnh->bnlm', dy, v)
+    ds = attention_softmax_bwd(dw, w)
+    dk = scale * np.einsum('bnlm,blnh->bmnh', ds, q)
+    dq = scale * np.einsum('bnlm,bmnh->blnh', ds, k)
+    return dq, dk, dv
+
+
 # --------------------------------------------------------------------------
 # A11/A12: layer glue (spec-level restatement)
 # --------------------------------------------------------------------------

@@ -190,3 +190,95 @@ def test_moving_average_module_autograd(cls, N):
 def _module_coeffs(mod, cls):
     p, q, g = mod.coeffs()
     return host(p.squeeze(-1)), host(q.squeeze(-1)), host(g)
+
+
+# ----------------------------------------------------------------------------------------------
+# attention
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,causal", [((3, 40, 40), True), ((2, 3, 17, 50), True), ((4, 64, 256), False),
+                                          ((2, 33, 33), False)])
+def test_attention_softmax_bwd(dtype, shape, causal):
+    rng = np.random.default_rng(71)
+    x, x64 = rounded(rng.normal(size=shape) * 2, dtype)
+    dy, dy64 = rounded(rng.normal(size=shape), dtype)
+    y = M.ops.attention_softmax_fwd(x, 0.0, causal)
+    y64 = host(y)                                          # the weights the backward is handed
+    dx = M.ops.attention_softmax_bwd(dy, y, causal)
+    assert rel_err(host(dx), O.attention_softmax_bwd(dy64, y64)) < TOL[dtype]
+    # module-level autograd
+    xg = x.clone().requires_grad_(True)
+    (M.AttentionSoftmax(0.0, causal)(xg) * dy).sum().backward()
+    assert rel_err(host(xg.grad), host(dx)) < 1e-6
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2), (torch.float16, 4e-3)])
+@pytest.mark.parametrize("B,L,Nh,H1,H2", [(2, 64, 2, 16, 32), (1, 256, 4, 32, 64), (3, 50, 1, 8, 24)])
+def test_attention_autograd(dtype, tol, B, L, Nh, H1, H2):
+    """q, k, v gradients through AttentionFunc.  As in the reference (attention_kernel.cu:148, 195-203)
+    the weight gradient dy v^T is stored in the activation type before its row mean under the weights
+    is subtracted, so q and k gradients carry that rounding amplified by the cancellation: the
+    per-op bound applies to their root-mean-square error and 4x the bound to the worst element."""
+    rng = np.random.default_rng(72)
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    y = M.EfficientAttention(scale=0.5)(q, k, v)
+    (y * dy).sum().backward()
+    assert rel_err(host(y), O.attention(q64, k64, v64, 0.5, True)[0]) < TOL[dtype]
+    for got, ref in zip((q.grad, k.grad, v.grad), O.attention_bwd(dy64, q64, k64, v64, 0.5, True)):
+        e = host(got) - ref
+        rms = np.sqrt((ref ** 2).mean())
+        assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
+
+
+@pytest.mark.parametrize("heads,act,moving", [(1, 'rmsnorm', 'cema'), (2, 'silu', 'ema')])
+def test_gated_attention_layer_trains(heads, act, moving):
+    """The whole layer under autograd (fp32): parameter and input gradients against central
+    differences of the fp64 layer oracle."""
+    from test_gpu_layer import _params
+    rng = np.random.default_rng(73)
+    B, L, D, S, E, N, C = 2, 32, 16, 8, 24, 4, 16
+    torch.manual_seed(11)
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_layer=moving, moving_act=act,
+                                          norm_num_groups=4, num_heads=heads).to(DEV).train()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.3)
+        layer.gamma.normal_(0, 0.3); layer.beta.normal_(0, 0.3)
+        layer.norm.weight.normal_(0, 0.2); layer.norm.bias.normal_(0, 0.2)
+    x64 = rng.normal(size=(B, L, D)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, L, D)).astype(np.float32).astype(np.float64)
+    x = dev(x64).requires_grad_(True)
+    out, _ = layer(x)
+    (out * dev(w64)).sum().backward()
+    P = _params(layer)
+    loss = lambda Pd, xx: (O.gated_attention_layer(xx, Pd, chunk=C, num_heads=heads, moving_act=act,
+                                                   num_groups=4) * w64).sum()
+    assert rel_err(host(out), O.gated_attention_layer(x64, P, chunk=C, num_heads=heads, moving_act=act,
+                                                      num_groups=4)) < 1e-4
+    eps = 1e-5
+    checks = [("v_w", layer.v_proj.weight), ("mx_w", layer.mx_proj.weight), ("mx_b", layer.mx_proj.bias),
+              ("h_w", layer.h_proj.weight), ("gamma", layer.gamma), ("beta", layer.beta),
+              ("norm_weight", layer.norm.weight), ("norm_bias", layer.norm.bias)]
+    for name, prm in checks:
+        grad = host(prm.grad)
+        scale = np.abs(grad).max() + 1e-6
+        for _ in range(3):
+            idx = tuple(rng.integers(0, s) for s in P[name].shape)
+            Pp = dict(P); Pp[name] = P[name].copy(); Pp[name][idx] += eps
+            Pm = dict(P); Pm[name] = P[name].copy(); Pm[name][idx] -= eps
+            fd = (loss(Pp, x64) - loss(Pm, x64)) / (2 * eps)
+            assert abs(fd - grad[idx]) < 3e-3 * scale, (name, idx, fd, grad[idx])
+    gx = host(x.grad)
+    for _ in range(4):
+        idx = tuple(rng.integers(0, s) for s in x64.shape)
+        xp, xm = x64.copy(), x64.copy()
+        xp[idx] += eps; xm[idx] -= eps
+        fd = (loss(P, xp) - loss(P, xm)) / (2 * eps)
+        assert abs(fd - gx[idx]) < 3e-3 * (np.abs(gx).max() + 1e-6), (idx, fd, gx[idx])
+    # the moving-average parameters get gradients as well
+    for prm in (layer.move.alpha, layer.move.delta, layer.move.gamma, layer.move.omega):
+        assert prm.grad is not None and torch.isfinite(prm.grad).all() and prm.grad.abs().max() > 0

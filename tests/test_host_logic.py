@@ -65,12 +65,12 @@ def test_incremental_state_keys_are_per_module():
     assert torch.equal(e._get_input_buffer(inc)["prev_state"], torch.tensor([[4., 5.], [0., 1.]]))
 
 
-def test_modules_without_a_backward_refuse_autograd():
-    """The moving average (unidirectional) and TimestepNorm have backward kernels; everything
-    else still says so instead of returning tensors that silently carry no graph."""
+def test_configurations_without_a_backward_refuse_autograd():
+    """The unidirectional moving average, TimestepNorm and the attention have backward operators;
+    what has none says so instead of returning tensors that silently carry no graph."""
     e = M.MultiHeadComplexEMA(4, ndim=2, bidirectional=True)
     with pytest.raises(NotImplementedError, match="backward pass covers"):
         e(torch.zeros(1, 4, 8))
-    a = M.EfficientAttention()
-    with pytest.raises(RuntimeError, match="forward pass only"):
-        a(torch.zeros(1, 8, 4, requires_grad=True), torch.zeros(1, 8, 4), torch.zeros(1, 8, 4))
+    layer = M.MovingAverageGatedAttention(8, 4, 8, 2, chunk_size=4, norm_num_groups=2)
+    with pytest.raises(NotImplementedError, match="incremental state"):
+        layer(torch.zeros(1, 4, 8), None, {})

@@ -72,6 +72,29 @@ def test_ema_backward_matches_finite_differences(masked):
         assert abs(_fd(lambda a: loss(x, p, q, a, om), g, j, 1j) - dg[j].imag) < 1e-6
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_bwd_matches_finite_differences(causal):
+    rng = np.random.default_rng(9)
+    B, L, Nh, H1, H2 = 2, 7, 2, 4, 5
+    q, k = rng.normal(size=(B, L, Nh, H1)), rng.normal(size=(B, L, Nh, H1))
+    v, wy = rng.normal(size=(B, L, Nh, H2)), rng.normal(size=(B, L, Nh, H2))
+    loss = lambda q_, k_, v_: (O.attention(q_, k_, v_, 0.7, causal)[0] * wy).sum()
+    dq, dk, dv = O.attention_bwd(wy, q, k, v, 0.7, causal)
+    for _ in range(8):
+        i = tuple(rng.integers(0, s) for s in q.shape)
+        j = tuple(rng.integers(0, s) for s in v.shape)
+        assert abs(_fd(lambda a: loss(a, k, v), q, i) - dq[i]) < 1e-6
+        assert abs(_fd(lambda a: loss(q, a, v), k, i) - dk[i]) < 1e-6
+        assert abs(_fd(lambda a: loss(q, k, a), v, j) - dv[j]) < 1e-6
+    # the softmax step alone: derivative of sum(softmax(x) * w)
+    x, w = rng.normal(size=(3, 5, 9)), rng.normal(size=(3, 5, 9))
+    y = O.attention_softmax(x, causal)
+    dx = O.attention_softmax_bwd(w, y)
+    for _ in range(8):
+        i = tuple(rng.integers(0, s) for s in x.shape)
+        assert abs(_fd(lambda a: (O.attention_softmax(a, causal) * w).sum(), x, i) - dx[i]) < 1e-6
+
+
 @pytest.fixture(scope="module")
 def gold():
     return np.load(GOLD, allow_pickle=False)
