@@ -268,17 +268,27 @@ def bench_layer(args):
     dev = torch.device("cuda:0")
     torch.manual_seed(1238)
     blk = M.Mega2Layer(D4, S4, E4, N4, Hf, C4, norm_num_groups=16, num_heads=heads, moving_act='silu')
-    blk = blk.to(dev).to(torch.bfloat16).eval()
+    train = args.workload == "layer_train"
+    blk = blk.to(dev).to(torch.bfloat16)
+    blk = blk.train() if train else blk.eval()
     xs = [torch.randn(1, L4, D4, device=dev).to(torch.bfloat16) for _ in range(4)]
-    with torch.no_grad():
-        for i in range(args.warmup):
+    ws = torch.randn(1, L4, D4, device=dev).to(torch.bfloat16)
+
+    def step(i):
+        if train:                      # forward + backward of sum(y * w); gradients accumulate in .grad
+            (blk(xs[i % 4]) * ws).sum().backward()
+        else:
             blk(xs[i % 4])
+
+    with torch.set_grad_enabled(train):
+        for i in range(args.warmup):
+            step(i)
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         a.record()
         for i in range(args.steps):
-            blk(xs[i % 4])
+            step(i)
         b.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
@@ -286,9 +296,12 @@ def bench_layer(args):
     gemm = 2 * L4 * D4 * (E4 + (S4 + E4 + 2 * D4)) + 2 * L4 * E4 * D4 + 3 * 2 * L4 * D4 * Hf
     nchunk = L4 // C4
     attn = nchunk * heads * C4 * (C4 + 1) * (S4 // heads + E4 // heads)
+    if train:                          # two more products per forward product; the backward attention is dense
+        gemm, attn = 3 * gemm, attn + 2 * nchunk * heads * 2 * C4 * C4 * (S4 // heads + E4 // heads)
     tf = (gemm + attn) / (ms * 1e-3) / 1e12
     print(json.dumps({
-        "metric": "Mega2 layer tokens/sec @B1xL8192xD2048", "value": L4 / (ms * 1e-3), "unit": "tokens/s",
+        "metric": ("Mega2 layer training tokens/sec (forward + backward) @B1xL8192xD2048" if train else
+                   "Mega2 layer tokens/sec @B1xL8192xD2048"), "value": L4 / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[4]: one Mega2 layer, L=8192 D=2048 z=512 h=4096 chunk=2048 4 heads, "
@@ -309,7 +322,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd"], default="block",
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train"], default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4], "
                          "one JSON line each")
@@ -324,7 +337,7 @@ def main():
         return bench_block_bwd(args)
     if args.workload == "attention":
         return bench_attention(args)
-    if args.workload == "layer":
+    if args.workload in ("layer", "layer_train"):
         return bench_layer(args)
 
     import numpy as np
