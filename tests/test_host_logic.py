@@ -74,3 +74,28 @@ def test_configurations_without_a_backward_refuse_autograd():
     layer = M.MovingAverageGatedAttention(8, 4, 8, 2, chunk_size=4, norm_num_groups=2)
     with pytest.raises(NotImplementedError, match="incremental state"):
         layer(torch.zeros(1, 4, 8), None, {})
+
+
+def test_gated_attention_state_dict_matches_reference_names():
+    """Parameter / buffer names and shapes a reference checkpoint of the layer holds
+    (moving_average_gated_attention.py:84-113; complex_exponential_moving_average.py:31-36;
+    norm_layer/timestep_norm.py:91-101; norm_layer/layer_norm.py:41-49; relative_positional_bias.py:55),
+    so load_state_dict takes a reference state dict as is."""
+    D, S, E, N, G = 16, 8, 24, 4, 4
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=8, moving_layer='cema', moving_act='rmsnorm',
+                                          norm_num_groups=G)
+    want = {
+        "norm.prior_count": (), "norm.prior_mean": (G,), "norm.prior_logv": (G,), "norm.weight": (D,), "norm.bias": (D,),
+        "move.alpha": (D, N, 1), "move.delta": (D, N, 1), "move.theta": (D, 1, 1), "move.gamma": (D, N, 2),
+        "move.omega": (D, 1),
+        "move_act.weight": (D,),
+        "v_proj.weight": (E, D), "v_proj.bias": (E,),
+        "mx_proj.weight": (S + E + 2 * D, D), "mx_proj.bias": (S + E + 2 * D,),
+        "h_proj.weight": (D, E),
+        "gamma": (2, S), "beta": (2, S),
+        "rel_pos_bias.freqs": (S // 2,),
+    }
+    got = {k: tuple(v.shape) for k, v in layer.state_dict().items()}
+    assert got == want
+    ffn = M.NormalizedFeedForwardNetwork(D, 32, norm_type='rmsnorm')
+    assert set(ffn.state_dict()) == {"norm.weight", "fc1.weight", "fc1.bias", "fc2.weight"}
