@@ -7,6 +7,7 @@ from .modules import (  # noqa: F401
     EfficientAttention,
     MultiHeadComplexEMA,
     MultiHeadEMA,
+    SequenceNorm,
     SwiGLU,
     TimestepNorm,
 )
@@ -31,6 +32,7 @@ __all__ = [
     "EfficientAttention",
     "MultiHeadComplexEMA",
     "MultiHeadEMA",
+    "SequenceNorm",
     "SwiGLU",
     "TimestepNorm",
 ]

@@ -17,6 +17,7 @@ SOURCES = [
     "capi.hip",
     "timestep_norm.hip",
     "timestep_norm_bwd.hip",
+    "sequence_norm.hip",
     "ema_scan.hip",
     "ema_mfma.hip",
     "ema_bwd.hip",

@@ -1,0 +1,372 @@
+// SequenceNorm forward (group and per-feature variants, [B, L, H] and [B, H, L] layouts):
+// the statistics of one (batch row, group) are the mean and the biased variance over all unmasked
+// tokens and the group's channels; y = (x - mean) * rstd * gamma + beta, masked tokens become 0.
+// Reference: fairseq/csrc/ops/sequence_norm.cc:258-372 (per feature), :531-656 (groups); the
+// per-feature form is the group form with one channel per group.
+//
+// Three launches, all deterministic (no floating-point atomics):
+//   1. moments: partial (count, mean, M2) per (row, token tile, group) for [B, L, H], per
+//      (row, channel) for [B, H, L]  (sums of x and x^2 over at most a tile in fp32);
+//   2. combine: one wave per (row, group) merges the partials pairwise (Chan et al.) and writes
+//      mean, rstd and the row's token count;
+//   3. apply: the same tiling as 1, one streaming pass.
+// HBM traffic: x twice, y once.
+#include "common.h"
+
+namespace mega {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxCells = 4096;     // tokens-per-tile * groups held in LDS
+
+struct SeqNormParams {
+  const void* x;
+  void* y;
+  const float* gamma;
+  const float* beta;
+  const uint8_t* mask;
+  float* part;        // [B, np, G, 3] ([B, L, H]) or [B, H, 3] ([B, H, L]): (n, mean, M2)
+  int64_t* count;
+  float* mean;
+  float* rstd;
+  int B, L, H, G, Dg, TT, nt;
+  int LPG, PER, slots, lpg_shift, slots_shift;
+  float eps;
+};
+
+__device__ __forceinline__ void split_item(const SeqNormParams& P, int i, int& tok, int& slot) {
+  if (P.slots_shift >= 0) {
+    tok = i >> P.slots_shift;
+    slot = i & (P.slots - 1);
+  } else {
+    tok = i / P.slots;
+    slot = i - tok * P.slots;
+  }
+}
+
+// Chan et al.: (na, ma, Ma) + (nb, mb, Mb)
+__device__ __forceinline__ void merge3(float& n, float& m, float& M2, float nb, float mb, float Mb) {
+  const float nt = n + nb;
+  if (nt > 0.f) {
+    const float d = mb - m, f = nb / nt;
+    m = fmaf(d, f, m);
+    M2 = M2 + Mb + d * d * n * f;
+  }
+  n = nt;
+}
+
+// ---------------------------------------------------------------- [B, L, H]: channels contiguous
+// APPLY = false: partial moments of the tile; APPLY = true: normalise the tile.
+template <typename T, int VEC, bool APPLY>
+__global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormParams P) {
+  using V = Vec<T, VEC>;
+  extern __shared__ float smem[];
+  const int G = P.G, H = P.H, TT = P.TT, Dg = P.Dg;
+  float* s_a = smem;                  // moments: sum per (token, group);  apply: mean per group
+  float* s_b = s_a + (APPLY ? G : TT * G);   // moments: sum of squares;  apply: rstd per group
+  int* s_mask = (int*)(s_b + (APPLY ? G : TT * G));
+  const int tid = threadIdx.x;
+  const int tile = blockIdx.x % P.nt, b = blockIdx.x / P.nt;
+  const int t0 = tile * TT;
+  const int ntok = min(TT, P.L - t0);
+  const T* x = (const T*)P.x + ((size_t)b * P.L + t0) * H;
+  for (int tok = tid; tok < TT; tok += kThreads)
+    s_mask[tok] = (tok >= ntok) || (P.mask && P.mask[(size_t)b * P.L + t0 + tok]);
+  if (APPLY)
+    for (int g = tid; g < G; g += kThreads) {
+      s_a[g] = P.mean[(size_t)b * G + g];
+      s_b[g] = P.rstd[(size_t)b * G + g];
+    }
+  __syncthreads();
+  const int items = ntok * P.slots;
+  const int span = VEC * P.PER;
+  for (int i0 = 0; i0 < items; i0 += kThreads) {
+    const int i = i0 + tid;
+    const bool live = i < items;
+    int tok, slot;
+    split_item(P, live ? i : 0, tok, slot);
+    const int g = slot >> P.lpg_shift;
+    const int c0 = g * Dg + (slot - (g << P.lpg_shift)) * span;
+    if (APPLY) {
+      if (live) {
+        const float mu = s_a[g], r = s_b[g];
+        const bool keep = !s_mask[tok];
+        T* y = (T*)P.y + ((size_t)b * P.L + t0 + tok) * H;
+        for (int k = 0; k < P.PER; ++k) {
+          const int c = c0 + k * VEC;
+          const V xv = *(const V*)(x + (size_t)tok * H + c);
+          V o;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            o.v[e] = from_float<T>(keep ? fmaf((to_float(xv.v[e]) - mu) * r, P.gamma[c + e], P.beta[c + e]) : 0.f);
+          *(V*)(y + c) = o;
+        }
+      }
+    } else {
+      float s1 = 0.f, s2 = 0.f;
+      if (live && !s_mask[tok]) {
+        for (int k = 0; k < P.PER; ++k) {
+          const V xv = *(const V*)(x + (size_t)tok * H + c0 + k * VEC);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float f = to_float(xv.v[e]);
+            s1 += f;
+            s2 = fmaf(f, f, s2);
+          }
+        }
+      }
+      for (int o = 1; o < P.LPG; o <<= 1) {
+        s1 += __shfl_xor(s1, o);
+        s2 += __shfl_xor(s2, o);
+      }
+      if (live && slot == (g << P.lpg_shift)) {
+        s_a[tok * G + g] = s1;
+        s_b[tok * G + g] = s2;
+      }
+    }
+  }
+  if (!APPLY) {
+    __syncthreads();
+    int nkeep = 0;
+    for (int tok = 0; tok < ntok; ++tok) nkeep += s_mask[tok] ? 0 : 1;
+    for (int g = tid; g < G; g += kThreads) {
+      float s1 = 0.f, s2 = 0.f;
+      for (int tok = 0; tok < ntok; ++tok) {      // masked tokens hold zeros
+        s1 += s_a[tok * G + g];
+        s2 += s_b[tok * G + g];
+      }
+      const float n = (float)nkeep * (float)Dg;
+      const float m = n > 0.f ? s1 / n : 0.f;
+      float* dst = P.part + (((size_t)b * P.nt + tile) * G + g) * 3;
+      dst[0] = n;
+      dst[1] = m;
+      dst[2] = fmaxf(s2 - n * m * m, 0.f);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- [B, H, L]: time contiguous
+// one workgroup per (row, channel)
+template <typename T, int VEC, bool APPLY>
+__global__ __launch_bounds__(kThreads) void seqnorm_bhl_kernel(const SeqNormParams P) {
+  using V = Vec<T, VEC>;
+  __shared__ float s_red[2][kThreads / 64];
+  __shared__ int s_cnt[kThreads / 64];
+  const int tid = threadIdx.x;
+  const int c = blockIdx.x % P.H, b = blockIdx.x / P.H;
+  const T* x = (const T*)P.x + ((size_t)b * P.H + c) * P.L;
+  const uint8_t* mk = P.mask ? P.mask + (size_t)b * P.L : nullptr;
+  if (APPLY) {
+    const int g = c / P.Dg;
+    const float mu = P.mean[(size_t)b * P.G + g], r = P.rstd[(size_t)b * P.G + g];
+    const float w = P.gamma[c] * r, sh = P.beta[c] - mu * w;
+    T* y = (T*)P.y + ((size_t)b * P.H + c) * P.L;
+    for (int t = tid * VEC; t < P.L; t += kThreads * VEC) {
+      const V xv = *(const V*)(x + t);
+      V o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        o.v[e] = from_float<T>((mk && mk[t + e]) ? 0.f : fmaf(to_float(xv.v[e]), w, sh));
+      *(V*)(y + t) = o;
+    }
+    return;
+  }
+  float s1 = 0.f, s2 = 0.f;
+  int n = 0;
+  for (int t = tid * VEC; t < P.L; t += kThreads * VEC) {
+    const V xv = *(const V*)(x + t);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if (!(mk && mk[t + e])) {
+        const float f = to_float(xv.v[e]);
+        s1 += f;
+        s2 = fmaf(f, f, s2);
+        ++n;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    s1 += __shfl_xor(s1, o);
+    s2 += __shfl_xor(s2, o);
+    n += __shfl_xor(n, o);
+  }
+  if ((tid & 63) == 0) { s_red[0][tid >> 6] = s1; s_red[1][tid >> 6] = s2; s_cnt[tid >> 6] = n; }
+  __syncthreads();
+  if (tid == 0) {
+    float a1 = 0.f, a2 = 0.f;
+    int nn = 0;
+    for (int k = 0; k < kThreads / 64; ++k) { a1 += s_red[0][k]; a2 += s_red[1][k]; nn += s_cnt[k]; }
+    const float fn = (float)nn, m = nn > 0 ? a1 / fn : 0.f;
+    float* dst = P.part + ((size_t)b * P.H + c) * 3;
+    dst[0] = fn;
+    dst[1] = m;
+    dst[2] = fmaxf(a2 - fn * m * m, 0.f);
+  }
+}
+
+// one wave per (row, group): partial p of the group sits at part[(b * np_outer + p_outer) ...];
+// both layouts are walked with (first, stride, count).
+__global__ __launch_bounds__(64) void seqnorm_combine_kernel(const SeqNormParams P, int np, int64_t row_stride,
+                                                            int64_t g_stride, int64_t p_stride) {
+  const int i = blockIdx.x;
+  const int b = i / P.G, g = i - b * P.G;
+  const int lane = threadIdx.x;
+  const float* base = P.part + (size_t)b * row_stride + (size_t)g * g_stride;
+  float n = 0.f, m = 0.f, M2 = 0.f;
+  for (int p = lane; p < np; p += 64) {
+    const float* q = base + (size_t)p * p_stride;
+    merge3(n, m, M2, q[0], q[1], q[2]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float nb = __shfl_xor(n, o), mb = __shfl_xor(m, o), Mb = __shfl_xor(M2, o);
+    // both partners must end with the same bits: merge in a fixed (low lane, high lane) order
+    float an = (lane & o) ? nb : n, am = (lane & o) ? mb : m, aM = (lane & o) ? Mb : M2;
+    const float bn = (lane & o) ? n : nb, bm = (lane & o) ? m : mb, bM = (lane & o) ? M2 : Mb;
+    merge3(an, am, aM, bn, bm, bM);
+    n = an; m = am; M2 = aM;
+  }
+  if (lane == 0) {
+    const float var = n > 0.f ? M2 / n : 0.f;
+    P.mean[i] = m;
+    P.rstd[i] = rsqrtf(var + P.eps);
+    if (g == 0) P.count[b] = (int64_t)llrintf(n / (float)P.Dg);
+  }
+}
+
+struct SeqGeom {
+  int tt, nt, vec, lpg, per;
+  size_t part_bytes;
+};
+
+bool seq_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, int length_last, SeqGeom* g) {
+  if (B * L >= (int64_t)1 << 31 || B * H >= (int64_t)1 << 31 || G > kMaxCells) return false;
+  const int full = dtype == MEGA_F32 ? 4 : 8;
+  if (length_last) {
+    g->vec = (L % full == 0) ? full : 1;
+    g->tt = 0; g->nt = 0; g->lpg = 1; g->per = 1;
+    g->part_bytes = align_up((size_t)B * H * 12, 256);
+    return true;
+  }
+  const int64_t Dg = H / G;
+  g->vec = (Dg % full == 0) ? full : 1;
+  const int64_t vecs = Dg / g->vec;
+  int lpg = 1;
+  while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
+  g->lpg = lpg;
+  g->per = (int)(vecs / lpg);
+  int tt = (int)(kMaxCells / G);
+  if (tt > 32) tt = 32;
+  if (tt < 1) tt = 1;
+  g->tt = tt;
+  g->nt = (int)ceil_div(L, tt);
+  if (B * g->nt >= (int64_t)1 << 31) return false;
+  g->part_bytes = align_up((size_t)B * g->nt * G * 12, 256);
+  return true;
+}
+
+template <typename T>
+int launch_seqnorm(SeqNormParams P, const SeqGeom& g, int length_last, bool aligned, hipStream_t s) {
+  constexpr int FULL = 16 / (int)sizeof(T);
+  const bool vec = g.vec == FULL && aligned;
+  if (length_last) {
+    const dim3 grid((unsigned)(P.B * P.H));
+    if (vec) hipLaunchKernelGGL((seqnorm_bhl_kernel<T, FULL, false>), grid, dim3(kThreads), 0, s, P);
+    else hipLaunchKernelGGL((seqnorm_bhl_kernel<T, 1, false>), grid, dim3(kThreads), 0, s, P);
+    MEGA_CHECK_LAUNCH("sequence_norm_fwd (moments)");
+    hipLaunchKernelGGL(seqnorm_combine_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P, P.Dg,
+                       (int64_t)P.H * 3, (int64_t)P.Dg * 3, (int64_t)3);
+    MEGA_CHECK_LAUNCH("sequence_norm_fwd (combine)");
+    if (vec) hipLaunchKernelGGL((seqnorm_bhl_kernel<T, FULL, true>), grid, dim3(kThreads), 0, s, P);
+    else hipLaunchKernelGGL((seqnorm_bhl_kernel<T, 1, true>), grid, dim3(kThreads), 0, s, P);
+    MEGA_CHECK_LAUNCH("sequence_norm_fwd (apply)");
+    return MEGA_OK;
+  }
+  const dim3 grid((unsigned)(P.B * P.nt));
+  const size_t lds_m = ((size_t)2 * P.TT * P.G + P.TT) * 4, lds_a = ((size_t)2 * P.G + P.TT) * 4;
+  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, false>), grid, dim3(kThreads), lds_m, s, P);
+  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, false>), grid, dim3(kThreads), lds_m, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_fwd (moments)");
+  hipLaunchKernelGGL(seqnorm_combine_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P, P.nt,
+                     (int64_t)P.nt * P.G * 3, (int64_t)3, (int64_t)P.G * 3);
+  MEGA_CHECK_LAUNCH("sequence_norm_fwd (combine)");
+  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, true>), grid, dim3(kThreads), lds_a, s, P);
+  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, true>), grid, dim3(kThreads), lds_a, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_fwd (apply)");
+  return MEGA_OK;
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+extern "C" size_t mega_sequence_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G,
+                                                     int length_last) {
+  SeqGeom g;
+  if (B <= 0 || L <= 0 || H <= 0 || G <= 0 || H % G != 0 || !seq_geometry(dtype, B, L, H, G, length_last, &g))
+    return 256;
+  return g.part_bytes;
+}
+
+extern "C" int mega_group_sequence_norm_fwd(const void* x, void* y, int dtype, const float* gamma, const float* beta,
+                                            const uint8_t* mask, int64_t B, int64_t L, int64_t H, int64_t G,
+                                            double eps, int length_last, int64_t* count, float* mean, float* rstd,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "sequence_norm_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && L >= 0 && H > 0 && G > 0 && H % G == 0, MEGA_ERR_ARG,
+               "sequence_norm_fwd: bad shape B=%ld L=%ld H=%ld G=%ld", (long)B, (long)L, (long)H, (long)G);
+  if (B == 0) return MEGA_OK;
+  MEGA_REQUIRE(gamma && beta && count && mean && rstd && (L == 0 || (x && y)), MEGA_ERR_ARG,
+               "sequence_norm_fwd: null pointer argument");
+  SeqGeom g;
+  MEGA_REQUIRE(seq_geometry(dtype, B, L > 0 ? L : 1, H, G, length_last, &g), MEGA_ERR_UNSUPPORTED,
+               "sequence_norm_fwd: shape outside the supported envelope (G <= %d)", kMaxCells);
+  MEGA_REQUIRE(L > 0, MEGA_ERR_UNSUPPORTED, "sequence_norm_fwd: empty sequences have no statistics");
+  MEGA_REQUIRE(workspace && workspace_bytes >= g.part_bytes, MEGA_ERR_WORKSPACE,
+               "sequence_norm_fwd: workspace of %zu bytes needed", g.part_bytes);
+  SeqNormParams P;
+  P.x = x; P.y = y; P.gamma = gamma; P.beta = beta; P.mask = mask; P.part = (float*)workspace;
+  P.count = count; P.mean = mean; P.rstd = rstd;
+  P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
+  P.LPG = g.lpg; P.PER = g.per; P.slots = (int)G * g.lpg; P.eps = (float)eps;
+  P.lpg_shift = 0;
+  while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
+  P.slots_shift = -1;
+  if ((P.slots & (P.slots - 1)) == 0) {
+    P.slots_shift = 0;
+    while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
+  }
+  const bool aligned = ((((uintptr_t)x | (uintptr_t)y) % 16) == 0);
+  if (!aligned && !length_last && g.vec > 1) {
+    // element-wise tiling when the buffers are not 16-byte aligned
+    g.vec = 1;
+    int64_t vecs = H / G;
+    int lpg = 1;
+    while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
+    P.LPG = lpg; P.PER = (int)(vecs / lpg); P.slots = (int)G * lpg;
+    P.lpg_shift = 0;
+    while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
+    P.slots_shift = -1;
+    if ((P.slots & (P.slots - 1)) == 0) {
+      P.slots_shift = 0;
+      while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
+    }
+  }
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MEGA_F32: return launch_seqnorm<float>(P, g, length_last, aligned, s);
+    case MEGA_BF16: return launch_seqnorm<bf16_t>(P, g, length_last, aligned, s);
+    default: return launch_seqnorm<f16_t>(P, g, length_last, aligned, s);
+  }
+}
+
+extern "C" int mega_sequence_norm_fwd(const void* x, void* y, int dtype, const float* gamma, const float* beta,
+                                      const uint8_t* mask, int64_t B, int64_t L, int64_t H, double eps,
+                                      int length_last, int64_t* count, float* mean, float* rstd, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  return mega_group_sequence_norm_fwd(x, y, dtype, gamma, beta, mask, B, L, H, H, eps, length_last, count, mean,
+                                      rstd, workspace, workspace_bytes, stream);
+}

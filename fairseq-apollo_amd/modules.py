@@ -461,6 +461,32 @@ class TimestepNorm(nn.Module, IncrementalState):
             **self.__dict__)
 
 
+class SequenceNorm(nn.Module):
+    """Whole-sequence (group) normalisation of bidirectional layers
+    (fairseq/modules/norm_layer/sequence_norm.py:54-74): x [B, H, L], statistics per (row, group)
+    over the unmasked tokens.  Forward only."""
+
+    def __init__(self, num_features: int, num_groups: Optional[int] = None, eps: float = 1e-5) -> None:
+        super().__init__()
+        self.num_features = num_features
+        self.num_groups = num_groups
+        assert self.num_groups is None or self.num_features % self.num_groups == 0
+        self.register_parameter("weight", Parameter(torch.zeros(num_features), requires_grad=True))
+        self.register_parameter("bias", Parameter(torch.zeros(num_features), requires_grad=True))
+        self.eps = eps
+
+    def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, length_last: bool = True) -> Tensor:
+        if _training_call(self, x):
+            raise NotImplementedError("SequenceNorm: the backward pass is not built; call it under torch.no_grad()")
+        gamma, beta = self.weight.float() + 1.0, self.bias.float()
+        if self.num_groups is None:
+            return ops.sequence_norm_fwd(x, gamma, beta, padding_mask, self.eps, length_last)[0]
+        return ops.group_sequence_norm_fwd(x, gamma, beta, padding_mask, self.num_groups, self.eps, length_last)[0]
+
+    def extra_repr(self) -> str:
+        return 'num_features={num_features}, num_groups={num_groups}, eps={eps}'.format(**self.__dict__)
+
+
 class AttentionSoftmaxFunc(torch.autograd.Function):
     """fairseq/modules/attention_softmax.py:11-39 (dropout = 0)."""
 

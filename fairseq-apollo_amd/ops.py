@@ -325,6 +325,42 @@ def timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean,
                     gamma, padding_mask, x.shape[-1])
 
 
+def group_sequence_norm_fwd(x, gamma, beta, padding_mask, num_groups: int, eps: float, length_last: bool = False):
+    """-> (y, count[B] int64, mean[B,G], rstd[B,G]).  x: [B, L, H], or [B, H, L] with length_last.
+    Reference: group_sequence_norm_fwd, fairseq/csrc/ops/sequence_norm.cc:953-1010."""
+    dev = _need_gpu(x, gamma, beta, padding_mask)
+    lib = _lib.load()
+    if x.dim() != 3:
+        raise RuntimeError("x must be [B, L, H] (or [B, H, L] with length_last)")
+    B = x.shape[0]
+    H, L = (x.shape[1], x.shape[2]) if length_last else (x.shape[2], x.shape[1])
+    G = int(num_groups)
+    if G <= 0 or H % G != 0:
+        raise RuntimeError(f"num_features={H} is not divisible by num_groups={G}")
+    xd = x.detach().contiguous()
+    dt = _dtype_code(xd)
+    y = torch.empty_like(xd)
+    count = torch.empty(B, dtype=torch.int64, device=dev)
+    mean = torch.empty(B, G, dtype=torch.float32, device=dev)
+    rstd = torch.empty(B, G, dtype=torch.float32, device=dev)
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, lib.mega_sequence_norm_workspace_bytes(dt, B, L, H, G, 1 if length_last else 0), stream)
+    m8 = _mask_u8(padding_mask, B, L)
+    with _on_device(dev):
+        rc = lib.mega_group_sequence_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(_f32c(gamma)), _ptr(_f32c(beta)), _ptr(m8),
+                                              B, L, H, G, float(eps), 1 if length_last else 0, _ptr(count),
+                                              _ptr(mean), _ptr(rstd), _ptr(ws), ws.numel(), stream)
+    _lib.check(rc, "group_sequence_norm_fwd")
+    return y, count, mean, rstd
+
+
+def sequence_norm_fwd(x, gamma, beta, padding_mask, eps: float, length_last: bool = False):
+    """Per-feature form: -> (y, count[B], mean[B,H], rstd[B,H]).  Reference: sequence_norm_fwd,
+    fairseq/csrc/ops/sequence_norm.cc:844-900."""
+    H = x.shape[1] if length_last else x.shape[2]
+    return group_sequence_norm_fwd(x, gamma, beta, padding_mask, H, eps, length_last)
+
+
 def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
     """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18."""
     if dropout != 0.0:

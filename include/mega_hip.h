@@ -243,6 +243,28 @@ int mega_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const flo
                            void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* SequenceNorm (the whole-sequence twin of TimestepNorm, used by bidirectional layers)      */
+/* stands in for group_sequence_norm_fwd and sequence_norm_fwd
+ * (fairseq/csrc/ops/sequence_norm.cc:953-1010 and :844-900; loops at :531-656, :258-372;
+ * caller norm_layer/sequence_norm.py:14-33).
+ *   x, y   [B,L,H] (length_last = 0) or [B,H,L] (length_last = 1) contiguous of `dtype`
+ *   gamma, beta [H] fp32 (gamma is weight + 1); mask [B,L] bytes, non-zero = padding, or NULL
+ *   count [B] int64 = unmasked tokens; mean, rstd [B,G] fp32: statistics over the unmasked
+ *   tokens and the group's channels (biased variance); masked tokens of y are 0.
+ * The per-feature form has H in place of G.                                                 */
+size_t mega_sequence_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G,
+                                          int length_last);
+int mega_group_sequence_norm_fwd(const void* x, void* y, int dtype, const float* gamma,
+                                 const float* beta, const uint8_t* mask, int64_t B, int64_t L,
+                                 int64_t H, int64_t G, double eps, int length_last,
+                                 int64_t* count, float* mean, float* rstd, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+int mega_sequence_norm_fwd(const void* x, void* y, int dtype, const float* gamma, const float* beta,
+                           const uint8_t* mask, int64_t B, int64_t L, int64_t H, double eps,
+                           int length_last, int64_t* count, float* mean, float* rstd,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Attention softmax and the fused attention op                              */
 /* stands in for attention_softmax_fwd (fairseq/csrc/ops/attention_softmax.cc:6-18,
  * ops/attention_softmax_kernel.cu:22-64, softmax.cuh:90-153), dropout = 0.

@@ -404,6 +404,36 @@ def timestep_norm_closed_form(x, padding_mask=None, num_groups: Optional[int] = 
     return y, mu, var
 
 
+def sequence_norm(x, gamma, beta, padding_mask=None, num_groups: Optional[int] = None, eps: float = 1e-5,
+                  length_last: bool = False):
+    """csrc/ops/sequence_norm.cc:531-656 (groups) and :258-372 (per feature): statistics of one
+    (row, group) over all unmasked tokens and the group's channels (biased variance),
+    y = (x - mean) rstd gamma + beta, masked tokens 0.  x: [B, L, H], or [B, H, L] with length_last.
+    Returns (y, count[B], mean[B,G], rstd[B,G])."""
+    x = np.asarray(x, np.float64)
+    xl = x.transpose(0, 2, 1) if length_last else x
+    B, L, H = xl.shape
+    G = H if num_groups is None else num_groups
+    D = H // G
+    keep = np.ones((B, L), bool) if padding_mask is None else ~np.asarray(padding_mask, bool)
+    y = np.zeros_like(xl)
+    count = keep.sum(1).astype(np.int64)
+    mean = np.zeros((B, G))
+    rstd = np.zeros((B, G))
+    gw = np.asarray(gamma, np.float64)
+    bw = np.asarray(beta, np.float64)
+    for b in range(B):
+        xg = xl[b][keep[b]].reshape(-1, G, D)
+        for g in range(G):
+            v = xg[:, g, :]
+            mean[b, g] = v.mean() if v.size else 0.0
+            rstd[b, g] = 1.0 / np.sqrt((v.var() if v.size else 0.0) + eps)
+        yb = (xl[b].reshape(L, G, D) - mean[b][None, :, None]) * rstd[b][None, :, None]
+        y[b] = yb.reshape(L, H) * gw + bw
+        y[b][~keep[b]] = 0.0
+    return (y.transpose(0, 2, 1) if length_last else y), count, mean, rstd
+
+
 def timestep_norm_saved(x, prev_count, prev_mean, prev_var, padding_mask=None, num_groups: Optional[int] = None,
                         eps: float = 1e-5):
     """What the forward keeps for the backward pass (csrc/ops/timestep_norm.cc:283-300):

@@ -1,6 +1,6 @@
-// Test infrastructure only. Python entry point for a CPU-only build of three of
+// Test infrastructure only. Python entry point for a CPU-only build of four of
 // the reference's own translation units (ops/timestep_norm.cc,
-// ops/ema_parameters.cc, ops/ema_hidden.cc), compiled where they lie under
+// ops/ema_parameters.cc, ops/ema_hidden.cc, ops/sequence_norm.cc), compiled where they lie under
 // /root/reference by oracle/Makefile. Nothing of the reference is copied: this
 // file only registers the op tables those translation units already define.
 // The CUDA entry points they dispatch to stay unresolved (lazy binding); they
@@ -9,6 +9,7 @@
 
 #include "ops/ema_hidden.h"
 #include "ops/ema_parameters.h"
+#include "ops/sequence_norm.h"
 #include "ops/timestep_norm.h"
 
 PYBIND11_MODULE(mega2_ref_cpu, m) {
@@ -16,4 +17,5 @@ PYBIND11_MODULE(mega2_ref_cpu, m) {
   mega2::ops::DefineTimestepNormOp(m);
   mega2::ops::DefineEMAParametersOp(m);
   mega2::ops::DefineEMAHiddenOp(m);
+  mega2::ops::DefineSequenceNormOp(m);
 }

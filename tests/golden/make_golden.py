@@ -1,6 +1,6 @@
 """Writes tests/golden/ref_cpu_vectors.npz: inputs and outputs of the reference's own CPU
 operators for this path, produced by oracle/_ref (fairseq/csrc/ops/timestep_norm.cc,
-ema_parameters.cc, ema_hidden.cc compiled in place by `make -C oracle ref`).
+ema_parameters.cc, ema_hidden.cc, sequence_norm.cc compiled in place by `make -C oracle ref`).
 
     python tests/golden/make_golden.py
 
@@ -144,6 +144,26 @@ def main():
     dp, dq, dg, _ = ref.ema_parameters_bwd(t(dk), None, t(p), log_q, t(g), None, vander)
     out.update({"ema_bwd.p": p, "ema_bwd.q": q, "ema_bwd.gamma": g, "ema_bwd.kernel_grad": dk,
                 "ema_bwd.p_grad": dp.numpy(), "ema_bwd.q_grad": dq.numpy(), "ema_bwd.gamma_grad": dg.numpy()})
+
+    # SequenceNorm: both layouts, group and per-feature, ragged padding
+    rng = np.random.default_rng(20242)
+    for tag, (B, L, H, G, last, masked) in {"gsn_a": (3, 37, 48, 4, False, True), "gsn_b": (2, 130, 64, 16, True, True),
+                                           "gsn_c": (2, 50, 32, 2, True, False), "sn_a": (2, 41, 24, None, True, True),
+                                           "sn_b": (2, 33, 20, None, False, False)}.items():
+        x = (rng.normal(size=(B, H, L) if last else (B, L, H)) * 1.6 + 0.4).astype(np.float32)
+        mask = (rng.random((B, L)) < 0.25) if masked else None
+        gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32)
+        beta = rng.normal(size=H).astype(np.float32)
+        tm = None if mask is None else t(mask)
+        if G is None:
+            y, c, mu, r = ref.sequence_norm_fwd(t(x), t(gamma), t(beta), tm, 1e-5, last)
+        else:
+            y, c, mu, r = ref.group_sequence_norm_fwd(t(x), t(gamma), t(beta), tm, G, 1e-5, last)
+        out.update({f"{tag}.x": x, f"{tag}.gamma": gamma, f"{tag}.beta": beta, f"{tag}.groups": np.int64(0 if G is None else G),
+                    f"{tag}.length_last": np.int64(1 if last else 0), f"{tag}.y": y.numpy(), f"{tag}.count": c.numpy(),
+                    f"{tag}.mean": mu.numpy(), f"{tag}.rstd": r.numpy()})
+        if mask is not None:
+            out[f"{tag}.mask"] = mask
 
     dst = os.path.join(HERE, "ref_cpu_vectors.npz")
     np.savez_compressed(dst, **out)

@@ -172,3 +172,35 @@ def test_hip_ema_backward_against_kernel_gradient_vectors(gold):
     assert rel_err(host(dp), c["p_grad"]) < 1e-4
     for a, b in ((host(dq), c["q_grad"]), (host(dg), c["gamma_grad"])):
         assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4
+
+
+SEQ_CASES = ["gsn_a", "gsn_b", "gsn_c", "sn_a", "sn_b"]
+
+
+@pytest.mark.parametrize("tag", SEQ_CASES)
+def test_oracle_sequence_norm(gold, tag):
+    c = _case(gold, tag)
+    G = int(c["groups"]) or None
+    y, n, mu, r = O.sequence_norm(c["x"], c["gamma"], c["beta"], c.get("mask"), G, 1e-5, bool(c["length_last"]))
+    assert rel_err(y, c["y"]) < 2e-5 and np.array_equal(n, c["count"])
+    assert rel_err(mu, c["mean"]) < 2e-5 and rel_err(r, c["rstd"]) < 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", SEQ_CASES)
+def test_hip_sequence_norm(gold, tag):
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, tag)
+    G = int(c["groups"])
+    mask = None if "mask" not in c else torch.from_numpy(c["mask"]).to("cuda:0")
+    last = bool(c["length_last"])
+    if G:
+        y, n, mu, r = M.ops.group_sequence_norm_fwd(dev(c["x"]), dev(c["gamma"]), dev(c["beta"]), mask, G, 1e-5, last)
+    else:
+        y, n, mu, r = M.ops.sequence_norm_fwd(dev(c["x"]), dev(c["gamma"]), dev(c["beta"]), mask, 1e-5, last)
+    assert rel_err(host(y), c["y"]) < 1e-4 and np.array_equal(host(n), c["count"])
+    assert rel_err(host(mu), c["mean"]) < 1e-4 and rel_err(host(r), c["rstd"]) < 1e-4

@@ -188,3 +188,56 @@ def test_glue_rejects_bad_arguments():
         M.ops.gate_mul_fwd(torch.zeros(2, 8, device=DEV), torch.zeros(2, 9, device=DEV))
     with pytest.raises(RuntimeError):
         M.ops.rms_norm_fwd(torch.zeros(2, 8), None, 1e-5)                  # CPU tensor: no CPU path
+
+
+# ----------------------------------------------------------------------------------------------
+# SequenceNorm
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H,G,last,masked", [
+    (2, 100, 64, 8, False, True),       # [B, L, H], vectors of 8 channels inside a group
+    (1, 4096, 1024, 16, False, False),  # the headline geometry, 128 tiles to combine
+    (2, 70, 48, 2, False, True),        # 24 channels per group
+    (3, 33, 30, 5, False, True),        # 6 channels per group: element-wise path
+    (2, 45, 24, None, False, True),     # per feature
+    (2, 256, 64, 8, True, True),        # [B, H, L], 16-byte rows
+    (2, 77, 40, 4, True, True),         # [B, H, L], odd row length
+    (1, 16384, 32, None, True, False),  # long rows, per feature
+])
+def test_sequence_norm(dtype, B, L, H, G, last, masked):
+    rng = np.random.default_rng(81)
+    x, x64 = rounded(rng.normal(size=(B, H, L) if last else (B, L, H)) * 1.5 + 0.7, dtype)
+    gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32)
+    beta = rng.normal(size=H).astype(np.float32)
+    mask = (rng.random((B, L)) < 0.3) if masked else None
+    if mask is not None:
+        mask[0, :] = False
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    if G is None:
+        y, n, mu, r = M.ops.sequence_norm_fwd(x, dev(gamma), dev(beta), tm, 1e-5, last)
+    else:
+        y, n, mu, r = M.ops.group_sequence_norm_fwd(x, dev(gamma), dev(beta), tm, G, 1e-5, last)
+    yo, no, muo, ro = O.sequence_norm(x64, gamma, beta, mask, G, 1e-5, last)
+    assert np.array_equal(host(n), no)
+    assert rel_err(host(mu), muo) < 1e-4 and rel_err(host(r), ro) < 1e-4
+    assert rel_err(host(y), yo) < TOL[dtype]
+
+
+def test_sequence_norm_module_and_edge_cases():
+    rng = np.random.default_rng(82)
+    B, H, L = 2, 32, 60
+    mod = M.SequenceNorm(H, 4).to(DEV).eval()
+    with torch.no_grad():
+        mod.weight.normal_(0, 0.2); mod.bias.normal_(0, 0.2)
+    x64 = rng.normal(size=(B, H, L))
+    mask = np.zeros((B, L), bool)
+    mask[1, :] = True                                     # a fully padded row: zeros out, finite statistics
+    mask[0, 50:] = True
+    with torch.no_grad():
+        y = mod(dev(x64), torch.from_numpy(mask).to(DEV))
+    yo = O.sequence_norm(x64.astype(np.float32).astype(np.float64), host(mod.weight) + 1, host(mod.bias), mask, 4, 1e-5, True)[0]
+    assert rel_err(host(y), yo) < 1e-4 and torch.isfinite(y).all() and float(y[1].abs().max()) == 0.0
+    with pytest.raises(NotImplementedError):
+        mod.train()(dev(x64).requires_grad_(True))
+    with pytest.raises(RuntimeError):
+        M.ops.group_sequence_norm_fwd(dev(x64), dev(np.ones(H)), dev(np.zeros(H)), None, 5, 1e-5, True)
