@@ -215,6 +215,43 @@ def bench_block_bwd(args):
     }))
 
 
+def bench_seqnorm(args):
+    """SequenceNorm (16 groups) at configs[2]'s activation shape, both layouts."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1237)
+    gamma = torch.randn(D, device=dev) * 0.1 + 1.0
+    beta = torch.randn(D, device=dev) * 0.1
+    res = {}
+    for name, last in (("blh", False), ("bhl", True)):
+        xs = [torch.randn((B, D, L) if last else (B, L, D), device=dev).to(torch.bfloat16) for _ in range(NBUF)]
+        for i in range(max(args.warmup, 1)):
+            M.ops.group_sequence_norm_fwd(xs[i % NBUF], gamma, beta, None, G, 1e-5, last)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for i in range(args.steps):
+            M.ops.group_sequence_norm_fwd(xs[i % NBUF], gamma, beta, None, G, 1e-5, last)
+        b.record()
+        torch.cuda.synchronize()
+        res[name] = a.elapsed_time(b) / args.steps
+    alg = 2 * B * L * D * 2              # x read once, y written once
+    ms = res["bhl"]                      # the layout the reference module uses
+    print(json.dumps({
+        "metric": "SequenceNorm tokens/sec @B4xL4096xD1024 ([B, H, L], 16 groups)", "value": B * L / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "SequenceNorm(16 groups) at configs[2]'s activation shape"},
+        "kernels": {"blh_ms": res["blh"], "bhl_ms": res["bhl"]},
+        "roofline": {"bound": "hbm", "kernel": "seqnorm moments + combine + apply", "achieved": alg / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_step": alg},
+    }))
+
+
 def bench_attention(args):
     """configs[4]'s attention: 4 chunks of 2048 tokens, 4 heads, H1 = 128, H2 = 1024, bf16, causal
     (matrix-core bound).  Flops are counted for the causal half only: 2 * C^2/2 * (H1 + H2) per chunk-head."""
@@ -322,7 +359,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train"], default="block",
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm"], default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4], "
                          "one JSON line each")
@@ -333,6 +370,8 @@ def main():
 
     if args.workload == "decode":
         return bench_decode(args)
+    if args.workload == "seqnorm":
+        return bench_seqnorm(args)
     if args.workload == "block_bwd":
         return bench_block_bwd(args)
     if args.workload == "attention":

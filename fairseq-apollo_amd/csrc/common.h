@@ -56,6 +56,21 @@ template <> __device__ __forceinline__ f16_t from_float<f16_t>(float v) {
   return r;
 }
 
+// VEC consecutive fp32 parameters (16-byte pieces when VEC is a multiple of 4 and p is aligned to it)
+template <int VEC>
+__device__ __forceinline__ void load_params(const float* __restrict__ p, float (&out)[VEC]) {
+  if constexpr (VEC % 4 == 0) {
+#pragma unroll
+    for (int i = 0; i < VEC / 4; ++i) {
+      const float4 v = ((const float4*)p)[i];
+      out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) out[i] = p[i];
+  }
+}
+
 // a naturally aligned vector of VEC elements, moved with one memory instruction
 template <typename T, int VEC>
 struct alignas(sizeof(T) * VEC) Vec {

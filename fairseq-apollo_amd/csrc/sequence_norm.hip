@@ -95,10 +95,13 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
         for (int k = 0; k < P.PER; ++k) {
           const int c = c0 + k * VEC;
           const V xv = *(const V*)(x + (size_t)tok * H + c);
+          float gw[VEC], bw[VEC];
+          load_params<VEC>(P.gamma + c, gw);
+          load_params<VEC>(P.beta + c, bw);
           V o;
 #pragma unroll
           for (int e = 0; e < VEC; ++e)
-            o.v[e] = from_float<T>(keep ? fmaf((to_float(xv.v[e]) - mu) * r, P.gamma[c + e], P.beta[c + e]) : 0.f);
+            o.v[e] = from_float<T>(keep ? fmaf((to_float(xv.v[e]) - mu) * r, gw[e], bw[e]) : 0.f);
           *(V*)(y + c) = o;
         }
       }
@@ -339,7 +342,7 @@ extern "C" int mega_group_sequence_norm_fwd(const void* x, void* y, int dtype, c
     P.slots_shift = 0;
     while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
   }
-  const bool aligned = ((((uintptr_t)x | (uintptr_t)y) % 16) == 0);
+  const bool aligned = ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta) % 16) == 0);
   if (!aligned && !length_last && g.vec > 1) {
     // element-wise tiling when the buffers are not 16-byte aligned
     g.vec = 1;

@@ -163,9 +163,11 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
         const float u_ = s_u[cellk[u]], r = s_r[cellk[u]];
         const bool keep = livek[u] && !s_mask[tokk[u]];
         float ds = 0.f, db = 0.f, sx = 0.f;
+        float gw[VEC];
+        load_params<VEC>(P.gamma + cc[u], gw);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-          const float d = livek[u] ? to_float(dvv[u].v[e]) : 0.f, xe = to_float(xvv[u].v[e]), w = P.gamma[cc[u] + e];
+          const float d = livek[u] ? to_float(dvv[u].v[e]) : 0.f, xe = to_float(xvv[u].v[e]), w = gw[e];
           ds = fmaf(d * (xe - u_), w, ds);
           db = fmaf(d, w, db);
           sx += xe;
@@ -374,9 +376,11 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
           const float a0 = s_ds[cellk[u]] * cg, a1 = 2.0f * s_db[cellk[u]] * cg;
           const bool keep = !s_mask[tokk[u]];
           V o;
+          float gw[VEC];
+          load_params<VEC>(P.gamma + cc[u], gw);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
-            const float v = fmaf(to_float(dvv[u].v[e]) * r, P.gamma[cc[u] + e],
+            const float v = fmaf(to_float(dvv[u].v[e]) * r, gw[e],
                                  fmaf(a1, to_float(xvv[u].v[e]) - ux, a0));
             o.v[e] = from_float<T>(keep ? v : 0.f);
           }
@@ -595,7 +599,7 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
   MEGA_REQUIRE(bwd_geometry(dtype, B, L, H, G, &g), MEGA_ERR_UNSUPPORTED,
                "timestep_norm_bwd: H=%ld G=%ld outside the supported envelope (H <= 8192, G <= %d)", (long)H, (long)G,
                kMaxTileCells);
-  if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad) % 16) != 0)) {
+  if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad | (uintptr_t)gamma) % 16) != 0)) {
     g.vec = 1;
     int64_t vecs = H / G;
     int lpg = 1;
