@@ -238,6 +238,139 @@ __global__ __launch_bounds__(64) void seqnorm_combine_kernel(const SeqNormParams
   }
 }
 
+// ---------------------------------------------------------------- backward, [B, H, L]
+// Reference: sequence_norm.cc:756-842 (groups, time last), :459-529 (per feature).  Per (row, channel)
+// ds = sum dy x, db = sum dy over the unmasked tokens; per (row, group) dsw = sum ds gamma,
+// dbw = sum db gamma, n = count * D, dv = r^3 (u dbw - dsw) / 2, du = -r dbw;
+// dx = r gamma dy + (2 (x - u) dv + du) / n;  dgamma = sum_rows r (ds - u db), dbeta = sum_rows db.
+struct SeqBwdParams {
+  const void* dy;
+  const void* x;
+  void* dx;
+  const int64_t* count;
+  const float* mean;
+  const float* rstd;
+  const float* gamma;
+  const uint8_t* mask;
+  float* part;     // [B, H, 2]  (ds, db)
+  float* coef;     // [B, G, 2]  (2 dv / n, du / n)
+  float* gamma_grad;
+  float* beta_grad;
+  int B, L, H, G, Dg;
+};
+
+template <typename T, int VEC, bool APPLY>
+__global__ __launch_bounds__(kThreads) void seqnorm_bwd_bhl_kernel(const SeqBwdParams P) {
+  using V = Vec<T, VEC>;
+  __shared__ float s_red[2][kThreads / 64];
+  const int tid = threadIdx.x;
+  const int c = blockIdx.x % P.H, b = blockIdx.x / P.H;
+  const T* x = (const T*)P.x + ((size_t)b * P.H + c) * P.L;
+  const T* dy = (const T*)P.dy + ((size_t)b * P.H + c) * P.L;
+  const uint8_t* mk = P.mask ? P.mask + (size_t)b * P.L : nullptr;
+  if (APPLY) {
+    const int g = c / P.Dg;
+    const float u = P.mean[(size_t)b * P.G + g], r = P.rstd[(size_t)b * P.G + g];
+    const float a1 = P.coef[((size_t)b * P.G + g) * 2], a0 = P.coef[((size_t)b * P.G + g) * 2 + 1];
+    const float rw = r * P.gamma[c], sh = a0 - a1 * u;
+    T* dx = (T*)P.dx + ((size_t)b * P.H + c) * P.L;
+    for (int t = tid * VEC; t < P.L; t += kThreads * VEC) {
+      const V xv = *(const V*)(x + t);
+      const V gv = *(const V*)(dy + t);
+      V o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        o.v[e] = from_float<T>((mk && mk[t + e]) ? 0.f : fmaf(rw, to_float(gv.v[e]), fmaf(a1, to_float(xv.v[e]), sh)));
+      *(V*)(dx + t) = o;
+    }
+    return;
+  }
+  float ds = 0.f, db = 0.f;
+  for (int t = tid * VEC; t < P.L; t += kThreads * VEC) {
+    const V xv = *(const V*)(x + t);
+    const V gv = *(const V*)(dy + t);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if (!(mk && mk[t + e])) {
+        const float d = to_float(gv.v[e]);
+        ds = fmaf(d, to_float(xv.v[e]), ds);
+        db += d;
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ds += __shfl_xor(ds, o);
+    db += __shfl_xor(db, o);
+  }
+  if ((tid & 63) == 0) { s_red[0][tid >> 6] = ds; s_red[1][tid >> 6] = db; }
+  __syncthreads();
+  if (tid == 0) {
+    float a = 0.f, d = 0.f;
+    for (int k = 0; k < kThreads / 64; ++k) { a += s_red[0][k]; d += s_red[1][k]; }
+    P.part[((size_t)b * P.H + c) * 2] = a;
+    P.part[((size_t)b * P.H + c) * 2 + 1] = d;
+  }
+}
+
+// one wave per (row, group): the two coefficients of dx
+__global__ __launch_bounds__(64) void seqnorm_bwd_combine_kernel(const SeqBwdParams P) {
+  const int i = blockIdx.x;
+  const int b = i / P.G, g = i - b * P.G;
+  const int lane = threadIdx.x;
+  float dsw = 0.f, dbw = 0.f;
+  for (int k = lane; k < P.Dg; k += 64) {
+    const int c = g * P.Dg + k;
+    const float w = P.gamma[c];
+    dsw = fmaf(P.part[((size_t)b * P.H + c) * 2], w, dsw);
+    dbw = fmaf(P.part[((size_t)b * P.H + c) * 2 + 1], w, dbw);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    dsw += __shfl_xor(dsw, o);
+    dbw += __shfl_xor(dbw, o);
+  }
+  if (lane == 0) {
+    const float n = (float)P.count[b] * (float)P.Dg;
+    const float u = P.mean[i], r = P.rstd[i];
+    const float dv = 0.5f * r * r * r * (u * dbw - dsw), du = -r * dbw;
+    P.coef[(size_t)i * 2] = n > 0.f ? 2.0f * dv / n : 0.f;
+    P.coef[(size_t)i * 2 + 1] = n > 0.f ? du / n : 0.f;
+  }
+}
+
+// thread per channel: parameter gradients summed over the rows in order
+__global__ void seqnorm_bwd_param_kernel(const SeqBwdParams P) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= P.H) return;
+  const int g = c / P.Dg;
+  float gw = 0.f, gb = 0.f;
+  for (int b = 0; b < P.B; ++b) {
+    const float ds = P.part[((size_t)b * P.H + c) * 2], db = P.part[((size_t)b * P.H + c) * 2 + 1];
+    gw = fmaf(P.rstd[(size_t)b * P.G + g], ds - P.mean[(size_t)b * P.G + g] * db, gw);
+    gb += db;
+  }
+  P.gamma_grad[c] = gw;
+  P.beta_grad[c] = gb;
+}
+
+template <typename T>
+int launch_seqnorm_bwd(const SeqBwdParams& P, bool vec, hipStream_t s) {
+  constexpr int FULL = 16 / (int)sizeof(T);
+  const dim3 grid((unsigned)(P.B * P.H));
+  if (vec) hipLaunchKernelGGL((seqnorm_bwd_bhl_kernel<T, FULL, false>), grid, dim3(kThreads), 0, s, P);
+  else hipLaunchKernelGGL((seqnorm_bwd_bhl_kernel<T, 1, false>), grid, dim3(kThreads), 0, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_bwd (sums)");
+  hipLaunchKernelGGL(seqnorm_bwd_combine_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_bwd (combine)");
+  hipLaunchKernelGGL(seqnorm_bwd_param_kernel, dim3((unsigned)ceil_div(P.H, 256)), dim3(256), 0, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_bwd (parameters)");
+  if (vec) hipLaunchKernelGGL((seqnorm_bwd_bhl_kernel<T, FULL, true>), grid, dim3(kThreads), 0, s, P);
+  else hipLaunchKernelGGL((seqnorm_bwd_bhl_kernel<T, 1, true>), grid, dim3(kThreads), 0, s, P);
+  MEGA_CHECK_LAUNCH("sequence_norm_bwd (dx)");
+  return MEGA_OK;
+}
+
 struct SeqGeom {
   int tt, nt, vec, lpg, per;
   size_t part_bytes;
@@ -372,4 +505,47 @@ extern "C" int mega_sequence_norm_fwd(const void* x, void* y, int dtype, const f
                                       size_t workspace_bytes, void* stream) {
   return mega_group_sequence_norm_fwd(x, y, dtype, gamma, beta, mask, B, L, H, H, eps, length_last, count, mean,
                                       rstd, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t mega_sequence_norm_bwd_workspace_bytes(int64_t B, int64_t H, int64_t G) {
+  if (B <= 0 || H <= 0 || G <= 0) return 256;
+  return align_up((size_t)B * H * 8, 256) + align_up((size_t)B * G * 8, 256);
+}
+
+extern "C" int mega_group_sequence_norm_bwd(const void* y_grad, const void* x, int dtype, const int64_t* count,
+                                            const float* mean, const float* rstd, const float* gamma,
+                                            const uint8_t* mask, int64_t B, int64_t L, int64_t H, int64_t G,
+                                            void* x_grad, float* gamma_grad, float* beta_grad, void* workspace,
+                                            size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "sequence_norm_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && L > 0 && H > 0 && G > 0 && H % G == 0, MEGA_ERR_ARG,
+               "sequence_norm_bwd: bad shape B=%ld L=%ld H=%ld G=%ld", (long)B, (long)L, (long)H, (long)G);
+  MEGA_REQUIRE(B * H < (int64_t)1 << 31 && L < (int64_t)1 << 30, MEGA_ERR_UNSUPPORTED,
+               "sequence_norm_bwd: shape too large");
+  MEGA_REQUIRE(gamma_grad && beta_grad, MEGA_ERR_ARG, "sequence_norm_bwd: null gradient output");
+  hipStream_t s = (hipStream_t)stream;
+  if (B == 0) {
+    (void)hipMemsetAsync(gamma_grad, 0, (size_t)H * 4, s);
+    (void)hipMemsetAsync(beta_grad, 0, (size_t)H * 4, s);
+    return MEGA_OK;
+  }
+  MEGA_REQUIRE(y_grad && x && x_grad && count && mean && rstd && gamma, MEGA_ERR_ARG,
+               "sequence_norm_bwd: null pointer argument");
+  const size_t need = mega_sequence_norm_bwd_workspace_bytes(B, H, G);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need, MEGA_ERR_WORKSPACE,
+               "sequence_norm_bwd: workspace of %zu bytes needed", need);
+  SeqBwdParams P;
+  P.dy = y_grad; P.x = x; P.dx = x_grad; P.count = count; P.mean = mean; P.rstd = rstd; P.gamma = gamma; P.mask = mask;
+  P.part = (float*)workspace;
+  P.coef = (float*)((char*)workspace + align_up((size_t)B * H * 8, 256));
+  P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
+  P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G);
+  const int full = dtype == MEGA_F32 ? 4 : 8;
+  const bool vec = L % full == 0 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad) % 16) == 0);
+  switch (dtype) {
+    case MEGA_F32: return launch_seqnorm_bwd<float>(P, vec, s);
+    case MEGA_BF16: return launch_seqnorm_bwd<bf16_t>(P, vec, s);
+    default: return launch_seqnorm_bwd<f16_t>(P, vec, s);
+  }
 }

@@ -461,10 +461,33 @@ class TimestepNorm(nn.Module, IncrementalState):
             **self.__dict__)
 
 
+class SequenceNormFunc(torch.autograd.Function):
+    """fairseq/modules/norm_layer/sequence_norm.py:12-49."""
+
+    @staticmethod
+    def forward(ctx, x, gamma, beta, padding_mask=None, num_groups=None, eps: float = 1e-5, length_last: bool = False):
+        G = (x.shape[1] if length_last else x.shape[2]) if num_groups is None else num_groups
+        y, count, mean, rstd = ops.group_sequence_norm_fwd(x, gamma, beta, padding_mask, G, eps, length_last)
+        ctx.save_for_backward(x, count, mean, rstd, gamma, padding_mask)
+        ctx.groups = G
+        ctx.length_last = length_last
+        return y
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        x, count, mean, rstd, gamma, padding_mask = ctx.saved_tensors
+        dx, dg, db = ops.group_sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, ctx.groups,
+                                                 ctx.length_last)
+        return dx, dg.to(gamma.dtype), db, None, None, None, None
+
+
+sequence_norm = SequenceNormFunc.apply
+
+
 class SequenceNorm(nn.Module):
     """Whole-sequence (group) normalisation of bidirectional layers
     (fairseq/modules/norm_layer/sequence_norm.py:54-74): x [B, H, L], statistics per (row, group)
-    over the unmasked tokens.  Forward only."""
+    over the unmasked tokens."""
 
     def __init__(self, num_features: int, num_groups: Optional[int] = None, eps: float = 1e-5) -> None:
         super().__init__()
@@ -477,7 +500,8 @@ class SequenceNorm(nn.Module):
 
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, length_last: bool = True) -> Tensor:
         if _training_call(self, x):
-            raise NotImplementedError("SequenceNorm: the backward pass is not built; call it under torch.no_grad()")
+            return sequence_norm(x, self.weight.float() + 1.0, self.bias.float(), padding_mask, self.num_groups,
+                                 self.eps, length_last)
         gamma, beta = self.weight.float() + 1.0, self.bias.float()
         if self.num_groups is None:
             return ops.sequence_norm_fwd(x, gamma, beta, padding_mask, self.eps, length_last)[0]

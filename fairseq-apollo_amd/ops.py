@@ -361,6 +361,47 @@ def sequence_norm_fwd(x, gamma, beta, padding_mask, eps: float, length_last: boo
     return group_sequence_norm_fwd(x, gamma, beta, padding_mask, H, eps, length_last)
 
 
+def group_sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, num_groups: int,
+                            length_last: bool = False):
+    """-> (x_grad, gamma_grad[H], beta_grad[H]) (parameter gradients in fp32).  Reference:
+    group_sequence_norm_bwd, fairseq/csrc/ops/sequence_norm.cc:1012-1063.  The kernels work on
+    [B, H, L]; a [B, L, H] call goes through transposed copies."""
+    dev = _need_gpu(y_grad, x, count, mean, rstd, gamma, padding_mask)
+    lib = _lib.load()
+    if x.dim() != 3 or y_grad.shape != x.shape:
+        raise RuntimeError("x and y_grad must have the same 3-D shape")
+    if not length_last:
+        dx, dg, db = group_sequence_norm_bwd(y_grad.transpose(1, 2), x.transpose(1, 2), count, mean, rstd, gamma,
+                                             padding_mask, num_groups, True)
+        return dx.transpose(1, 2).contiguous(), dg, db
+    B, H, L = x.shape
+    G = int(num_groups)
+    if G <= 0 or H % G != 0:
+        raise RuntimeError(f"num_features={H} is not divisible by num_groups={G}")
+    xd = x.detach().contiguous()
+    gd = y_grad.detach().to(xd.dtype).contiguous()
+    dx = torch.empty_like(xd)
+    dg = torch.empty(H, dtype=torch.float32, device=dev)
+    db = torch.empty(H, dtype=torch.float32, device=dev)
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, lib.mega_sequence_norm_bwd_workspace_bytes(B, H, G), stream)
+    m8 = _mask_u8(padding_mask, B, L)
+    cnt = count.detach().to(torch.int64).contiguous()
+    with _on_device(dev):
+        rc = lib.mega_group_sequence_norm_bwd(_ptr(gd), _ptr(xd), _dtype_code(xd), _ptr(cnt),
+                                              _ptr(_f32c(mean).reshape(B, G)), _ptr(_f32c(rstd).reshape(B, G)),
+                                              _ptr(_f32c(gamma)), _ptr(m8), B, L, H, G, _ptr(dx), _ptr(dg), _ptr(db),
+                                              _ptr(ws), ws.numel(), stream)
+    _lib.check(rc, "group_sequence_norm_bwd")
+    return dx, dg, db
+
+
+def sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, length_last: bool = False):
+    """Per-feature form.  Reference: sequence_norm_bwd, fairseq/csrc/ops/sequence_norm.cc:902-951."""
+    H = x.shape[1] if length_last else x.shape[2]
+    return group_sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, H, length_last)
+
+
 def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
     """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18."""
     if dropout != 0.0:

@@ -263,6 +263,17 @@ int mega_sequence_norm_fwd(const void* x, void* y, int dtype, const float* gamma
                            const uint8_t* mask, int64_t B, int64_t L, int64_t H, double eps,
                            int length_last, int64_t* count, float* mean, float* rstd,
                            void* workspace, size_t workspace_bytes, void* stream);
+/* backward for the [B,H,L] layout (the one the reference module uses): stands in for
+ * group_sequence_norm_bwd / sequence_norm_bwd with length_last = true
+ * (fairseq/csrc/ops/sequence_norm.cc:756-842, :459-529; pass G = H for the per-feature form).
+ *   y_grad, x, x_grad [B,H,L] contiguous of `dtype`; count, mean, rstd as the forward wrote
+ *   them; outputs x_grad, gamma_grad, beta_grad [H] fp32.                                 */
+size_t mega_sequence_norm_bwd_workspace_bytes(int64_t B, int64_t H, int64_t G);
+int mega_group_sequence_norm_bwd(const void* y_grad, const void* x, int dtype, const int64_t* count,
+                                 const float* mean, const float* rstd, const float* gamma,
+                                 const uint8_t* mask, int64_t B, int64_t L, int64_t H, int64_t G,
+                                 void* x_grad, float* gamma_grad, float* beta_grad,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Attention softmax and the fused attention op                              */

@@ -434,6 +434,38 @@ def sequence_norm(x, gamma, beta, padding_mask=None, num_groups: Optional[int] =
     return (y.transpose(0, 2, 1) if length_last else y), count, mean, rstd
 
 
+def sequence_norm_bwd(dy, x, gamma, padding_mask=None, num_groups: Optional[int] = None, eps: float = 1e-5,
+                      length_last: bool = False):
+    """csrc/ops/sequence_norm.cc:657-754 (and the time-last twin :756-842): per (row, channel)
+    ds = sum dy x, db = sum dy over unmasked tokens; per group dsw = sum ds gamma, dbw = sum db gamma;
+    dv = r^3 (u dbw - dsw) / 2, du = -r dbw; dx = r gamma dy + (2 (x - u) dv + du) / (count D);
+    dgamma = sum_rows r (ds - u db), dbeta = sum_rows db.  Returns (dx, dgamma, dbeta)."""
+    dy = np.asarray(dy, np.float64)
+    x = np.asarray(x, np.float64)
+    if length_last:
+        dy, x = dy.transpose(0, 2, 1), x.transpose(0, 2, 1)
+    B, L, H = x.shape
+    G = H if num_groups is None else num_groups
+    D = H // G
+    _, count, mean, rstd = sequence_norm(x, gamma, np.zeros(H), padding_mask, num_groups, eps, False)
+    keep = np.ones((B, L)) if padding_mask is None else 1.0 - np.asarray(padding_mask, np.float64)
+    w = np.asarray(gamma, np.float64)
+    dym = dy * keep[..., None]
+    ds = (dym * x).sum(1)                                  # [B, H]
+    db = dym.sum(1)
+    dsw = (ds * w).reshape(B, G, D).sum(-1)
+    dbw = (db * w).reshape(B, G, D).sum(-1)
+    dv = 0.5 * rstd ** 3 * (mean * dbw - dsw)
+    du = -rstd * dbw
+    n = np.maximum(count[:, None] * D, 1)
+    ue, re_ = np.repeat(mean, D, 1), np.repeat(rstd, D, 1)
+    dx = re_[:, None, :] * w * dy + (2 * (x - ue[:, None, :]) * np.repeat(dv / n, D, 1)[:, None, :]
+                                     + np.repeat(du / n, D, 1)[:, None, :])
+    dx = dx * keep[..., None]
+    dg = (re_ * (ds - ue * db)).sum(0)
+    return (dx.transpose(0, 2, 1) if length_last else dx), dg, db.sum(0)
+
+
 def timestep_norm_saved(x, prev_count, prev_mean, prev_var, padding_mask=None, num_groups: Optional[int] = None,
                         eps: float = 1e-5):
     """What the forward keeps for the backward pass (csrc/ops/timestep_norm.cc:283-300):

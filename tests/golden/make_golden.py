@@ -165,6 +165,28 @@ def main():
         if mask is not None:
             out[f"{tag}.mask"] = mask
 
+    # SequenceNorm backward
+    rng = np.random.default_rng(20243)
+    for tag, (B, L, H, G, last, masked) in {"gsn_bwd_a": (2, 45, 48, 4, True, True), "gsn_bwd_b": (3, 40, 32, 8, False, True),
+                                           "sn_bwd": (2, 33, 24, None, True, False)}.items():
+        x = (rng.normal(size=(B, H, L) if last else (B, L, H)) * 1.3 + 0.3).astype(np.float32)
+        dy = rng.normal(size=x.shape).astype(np.float32)
+        mask = (rng.random((B, L)) < 0.25) if masked else None
+        gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32)
+        beta = rng.normal(size=H).astype(np.float32)
+        tm = None if mask is None else t(mask)
+        if G is None:
+            y, c, mu, r = ref.sequence_norm_fwd(t(x), t(gamma), t(beta), tm, 1e-5, last)
+            gr = ref.sequence_norm_bwd(t(dy), t(x), c, mu, r, t(gamma), tm, last)
+        else:
+            y, c, mu, r = ref.group_sequence_norm_fwd(t(x), t(gamma), t(beta), tm, G, 1e-5, last)
+            gr = ref.group_sequence_norm_bwd(t(dy), t(x), c, mu, r, t(gamma), tm, G, last)
+        out.update({f"{tag}.x": x, f"{tag}.y_grad": dy, f"{tag}.gamma": gamma, f"{tag}.beta": beta,
+                    f"{tag}.groups": np.int64(0 if G is None else G), f"{tag}.length_last": np.int64(1 if last else 0),
+                    f"{tag}.x_grad": gr[0].numpy(), f"{tag}.gamma_grad": gr[1].numpy(), f"{tag}.beta_grad": gr[2].numpy()})
+        if mask is not None:
+            out[f"{tag}.mask"] = mask
+
     dst = os.path.join(HERE, "ref_cpu_vectors.npz")
     np.savez_compressed(dst, **out)
     print(dst, os.path.getsize(dst), "bytes,", len(out), "arrays")

@@ -72,6 +72,24 @@ def test_ema_backward_matches_finite_differences(masked):
         assert abs(_fd(lambda a: loss(x, p, q, a, om), g, j, 1j) - dg[j].imag) < 1e-6
 
 
+@pytest.mark.parametrize("G,last,masked", [(4, False, True), (None, True, True), (2, True, False)])
+def test_sequence_norm_bwd_matches_finite_differences(G, last, masked):
+    rng = np.random.default_rng(10)
+    B, L, H = 2, 9, 8
+    x = rng.normal(size=(B, H, L) if last else (B, L, H))
+    wy = rng.normal(size=x.shape)
+    gamma, beta = rng.normal(size=H) + 1, rng.normal(size=H)
+    mask = (rng.random((B, L)) < 0.3) if masked else None
+    loss = lambda x_, g_, b_: (O.sequence_norm(x_, g_, b_, mask, G, 1e-5, last)[0] * wy).sum()
+    dx, dg, db = O.sequence_norm_bwd(wy, x, gamma, mask, G, 1e-5, last)
+    for _ in range(10):
+        i = tuple(rng.integers(0, s) for s in x.shape)
+        c = (int(rng.integers(0, H)),)
+        assert abs(_fd(lambda a: loss(a, gamma, beta), x, i) - dx[i]) < 1e-6
+        assert abs(_fd(lambda a: loss(x, a, beta), gamma, c) - dg[c]) < 1e-6
+        assert abs(_fd(lambda a: loss(x, gamma, a), beta, c) - db[c]) < 1e-6
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_bwd_matches_finite_differences(causal):
     rng = np.random.default_rng(9)
@@ -122,3 +140,11 @@ def test_ema_kernel_bwd_matches_reference_vectors(gold):
     assert rel_err(dp, c["p_grad"]) < 5e-5
     for a, b in ((dq, c["q_grad"]), (dg, c["gamma_grad"])):
         assert rel_err(a.real, b.real) < 5e-5 and rel_err(a.imag, b.imag) < 5e-5
+
+
+@pytest.mark.parametrize("tag", ["gsn_bwd_a", "gsn_bwd_b", "sn_bwd"])
+def test_sequence_norm_bwd_matches_reference_vectors(gold, tag):
+    c = _case(gold, tag)
+    G = int(c["groups"]) or None
+    dx, dg, db = O.sequence_norm_bwd(c["y_grad"], c["x"], c["gamma"], c.get("mask"), G, 1e-5, bool(c["length_last"]))
+    assert rel_err(dx, c["x_grad"]) < 5e-5 and rel_err(dg, c["gamma_grad"]) < 5e-5 and rel_err(db, c["beta_grad"]) < 5e-5
