@@ -20,8 +20,8 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SwiGLU, TimestepNorm,
-                      _training_call)
+from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
+                      TimestepNorm, _training_call)
 
 
 class RMSNorm(nn.Module):
@@ -143,21 +143,28 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
 
     def __init__(self, embed_dim, zdim, hdim, ndim, chunk_size=-1, moving_layer='cema', moving_act='rmsnorm',
                  norm_num_groups=None, norm_affine=True, norm_eps=1e-5, max_positions=1024, num_heads=1,
-                 efficient_attn=True, rel_pos_bias='rotary', bidirectional=False, attention_activation='softmax'):
+                 efficient_attn=True, rel_pos_bias='rotary', bidirectional=False, attention_activation='softmax',
+                 truncation=None):
         super().__init__()
         self.init_incremental_state()
-        if bidirectional or not efficient_attn or rel_pos_bias != 'rotary' or attention_activation != 'softmax':
-            raise NotImplementedError("only the causal path with the fused rotary softmax attention is built")
+        if not efficient_attn or rel_pos_bias != 'rotary' or attention_activation != 'softmax':
+            raise NotImplementedError("only the rotary softmax attention through the fused ops is built")
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
         self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
         self.chunk_size = chunk_size
         self.num_heads = num_heads
-        self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=True, scale=1.0)
-        self.norm = TimestepNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
+        self.bidirectional = bidirectional
+        # causal layers: the fused causal op; bidirectional layers (moving_average_gated_attention.py:70-75,
+        # 84-92): full softmax over every chunk, SequenceNorm, a two-sided moving average
+        self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=not bidirectional, scale=1.0)
+        if bidirectional:
+            self.norm = SequenceNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
+        else:
+            self.norm = TimestepNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
         if moving_layer == 'ema':
-            self.move = MultiHeadEMA(embed_dim, ndim=ndim)
+            self.move = MultiHeadEMA(embed_dim, ndim=ndim, bidirectional=bidirectional, truncation=truncation)
         elif moving_layer == 'cema':
-            self.move = MultiHeadComplexEMA(embed_dim, ndim=ndim)
+            self.move = MultiHeadComplexEMA(embed_dim, ndim=ndim, bidirectional=bidirectional, truncation=truncation)
         else:
             raise ValueError("Unknown moving type: {}".format(moving_layer))
         assert moving_act in ['rmsnorm', 'silu']
@@ -188,7 +195,11 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         assert embed_dim == self.embed_dim
         saved_state = self._get_input_buffer(incremental_state) if incremental_state is not None else None
         residual = x
-        x = self.norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
+        if self.bidirectional:
+            assert incremental_state is None, 'a bidirectional layer has no incremental state'
+            x = self.norm(x, padding_mask, length_last=False)      # the statistics do not depend on the layout
+        else:
+            x = self.norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
         v = F.silu(self.v_proj(x))
         mx = self.move(x.transpose(1, 2), padding_mask, incremental_state, out_layout="input").transpose(1, 2)
         mx = self.move_act(mx)
@@ -201,14 +212,28 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
             nc = seq_len // C
             q, k = ops.gate_qk_fwd(z, self.gamma + 1.0, self.beta, self.rel_pos_bias.freqs, Nh, C)
-            attn = self.efficient_attn(q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1),
-                                       v.reshape(bsz * nc, C, Nh, -1))
+            q4, k4, v4 = q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1), v.reshape(bsz * nc, C, Nh, -1)
+            if self.bidirectional and padding_mask is not None:
+                attn = self._padded_attention(q4, k4, v4, padding_mask.reshape(bsz * nc, C))
+            else:
+                attn = self.efficient_attn(q4, k4, v4)
         else:
             attn = self._cached_attention(z, v, saved_state, incremental_state)
         # the gates are applied where their operands are consumed: r on the way into the output
         # projection, u and the residual mix after it
         hp = self.h_proj(ops.gate_mul_fwd(attn.reshape(bsz, seq_len, self.hdim), r))
         return ops.gate_out_fwd(residual, u, hx, hp), None
+
+    def _padded_attention(self, q4: Tensor, k4: Tensor, v4: Tensor, key_padding: Tensor) -> Tensor:
+        """Full softmax over a chunk with padded keys excluded
+        (moving_average_gated_attention.py:232-248): scores of padded keys are -inf except in chunks
+        that consist of padding only; library GEMMs around the softmax op."""
+        pad = key_padding.to(torch.bool)
+        pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
+        s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
+        s = s.masked_fill(pad[:, None, None, :], float('-inf'))
+        w = ops.attention_softmax_fwd(s, 0.0, False)
+        return torch.einsum('bnqk,bknh->bqnh', w, v4)
 
     def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
         """The same layer with a complete autograd graph (moving_average_gated_attention.py:263-417,
@@ -217,6 +242,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if incremental_state is not None:
             raise NotImplementedError("MovingAverageGatedAttention: incremental state is an inference feature; "
                                       "call it under torch.no_grad()")
+        if self.bidirectional:
+            raise NotImplementedError("MovingAverageGatedAttention: the two-sided moving average has no backward "
+                                      "pass yet; call a bidirectional layer under torch.no_grad()")
         bsz, seq_len, _ = x.size()
         residual = x
         x = self.norm(x, padding_mask=padding_mask)

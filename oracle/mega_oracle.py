@@ -644,7 +644,7 @@ def rms_norm(x, weight=None, eps: float = 1e-5):
 
 
 def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str = 'silu', eps: float = 1e-5,
-                          num_groups: Optional[int] = None):
+                          num_groups: Optional[int] = None, bidirectional: bool = False, padding_mask=None):
     """MovingAverageGatedAttention.forward, unidirectional, softmax attention through the fused
     (rotary, causal, scale 1) op: modules/moving_average_gated_attention.py:263-417, step by
     step.  x: [B, L, D]; P: dict of numpy parameters
@@ -657,10 +657,17 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     B, L, D = x.shape
     S = P['gamma'].shape[1]
     E = P['v_w'].shape[0]
-    xn, _, _, _ = timestep_norm(x, np.zeros(B, np.int64), np.zeros((B, num_groups or D)), np.ones((B, num_groups or D)),
-                                np.asarray(P['norm_weight'], np.float64) + 1.0, P['norm_bias'], None, num_groups, eps)
+    if bidirectional:
+        # moving_average_gated_attention.py:84-87, 297-302: SequenceNorm, two-sided moving average
+        xn = sequence_norm(x, np.asarray(P['norm_weight'], np.float64) + 1.0, P['norm_bias'], padding_mask, num_groups,
+                           eps)[0]
+    else:
+        xn, _, _, _ = timestep_norm(x, np.zeros(B, np.int64), np.zeros((B, num_groups or D)),
+                                    np.ones((B, num_groups or D)), np.asarray(P['norm_weight'], np.float64) + 1.0,
+                                    P['norm_bias'], padding_mask, num_groups, eps)
     v = _silu(xn @ np.asarray(P['v_w'], np.float64).T + P['v_b'])
-    mx, _ = ema_forward(xn.transpose(0, 2, 1), P['p'], P['q'], P['ema_gamma'], P['omega'])
+    mx, _ = ema_forward(xn.transpose(0, 2, 1), P['p'], P['q'], P['ema_gamma'], P['omega'], padding_mask,
+                        bidirectional=bidirectional)
     mx = mx.transpose(0, 2, 1)
     mx = _silu(mx) if moving_act == 'silu' else rms_norm(mx, P.get('rms_weight'), eps)
     base = mx @ np.asarray(P['mx_w'], np.float64).T + P['mx_b']
@@ -681,7 +688,16 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     # rotary on every head's features, positions restart in every chunk
     qr = rotary(qc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
     kr = rotary(kc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
-    a, _ = attention(qr, kr, vc, 1.0, True)
+    if bidirectional:
+        # full softmax per chunk; padded keys excluded unless the whole chunk is padding (:232-248)
+        sc = np.einsum('blnh,bmnh->bnlm', qr, kr)
+        if padding_mask is not None:
+            pad = np.asarray(padding_mask, bool).reshape(B * nc, C)
+            pad = pad & ~pad.all(-1, keepdims=True)
+            sc = np.where(pad[:, None, None, :], -np.inf, sc)
+        a = np.einsum('bnlm,bmnh->blnh', attention_softmax(sc, False), vc)
+    else:
+        a, _ = attention(qr, kr, vc, 1.0, True)
     a = a.reshape(B, L, E)
     h = _silu(hx + (a * r) @ np.asarray(P['h_w'], np.float64).T)
     return x + u * (h - x)

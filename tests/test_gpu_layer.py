@@ -123,3 +123,46 @@ def test_normalized_feed_forward(dtype, tol, norm_type, layer_scale):
         w2 = w2 * host(ffn.layerscale_weight)[:, None]
     yo = O.silu_ffn(xn, host(ffn.fc1.weight), host(ffn.fc1.bias), w2, 0.0) - xn + x64
     assert _chain_ok(y, yo, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("heads,act,moving,masked", [(1, 'rmsnorm', 'cema', True), (2, 'silu', 'cema', False),
+                                                     (1, 'silu', 'ema', True)])
+def test_bidirectional_gated_attention_layer(dtype, tol, heads, act, moving, masked):
+    """The encoder form of the layer: SequenceNorm, two-sided moving average, full softmax per
+    chunk with padded keys excluded (one row ends in a chunk that is padding only)."""
+    torch.manual_seed(9)
+    B, L, D, S, E, N, C = 2, 512, 64, 32, 128, 16, 128
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_layer=moving, moving_act=act,
+                                          norm_num_groups=8, num_heads=heads, bidirectional=True).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.15)
+        layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
+        layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+    P = _params(layer)
+    if dtype != torch.float32:
+        for k_ in ('v_w', 'v_b', 'mx_w', 'mx_b', 'h_w', 'gamma', 'beta', 'norm_weight', 'norm_bias', 'rms_weight'):
+            if k_ in P:
+                P[k_] = torch.from_numpy(np.asarray(P[k_], np.float32)).to(dtype).double().numpy()
+    layer = layer.to(dtype)
+    x = torch.randn(B, L, D, device=DEV).to(dtype)
+    mask = None
+    if masked:
+        mask = np.zeros((B, L), bool)
+        mask[0, 300:] = True                   # the last chunk of row 0 is padding only
+        mask[1, 500:] = True
+    with torch.no_grad():
+        y, _ = layer(x, None if mask is None else torch.from_numpy(mask).to(DEV))
+    yo = O.gated_attention_layer(host(x), P, chunk=C, num_heads=heads, moving_act=act, num_groups=8,
+                                 bidirectional=True, padding_mask=mask)
+    keep = np.ones((B, L), bool) if mask is None else ~mask     # padded positions carry no meaning
+    got, ref = host(y)[keep], yo[keep]
+    if dtype == torch.float32:
+        assert rel_err(got, ref) < tol
+    else:
+        e = got - ref
+        rms = np.sqrt((ref ** 2).mean())
+        assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
+    with pytest.raises(NotImplementedError):
+        layer.train()(x.requires_grad_(True))
