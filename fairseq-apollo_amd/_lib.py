@@ -37,7 +37,7 @@ SIGNATURES = {
                                   _p, _i64, _i64, _i64, _i64, _p]),
     "mega_ema_param_grad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "mega_ema_param_grad": (_int, [_p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64,
-                                   _i64, _p, _p, _p, _p, _p, _sz, _p]),
+                                   _i64, _int, _int, _p, _p, _p, _p, _p, _sz, _p]),
     "mega_long_conv_fwd": (_int, [_p, _p, _int, _p, _i64, _i64, _i64, _i64, _int, _int, _p]),
     "mega_timestep_norm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "mega_group_timestep_norm_fwd": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, C.c_double,

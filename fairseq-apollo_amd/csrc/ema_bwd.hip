@@ -35,9 +35,13 @@ struct EmaGradArgs {
   float* sums;              // [B, D, N, 4]
   float* dyx;               // [B, D]
   int B, D, N, L;
+  int reverse;   // walk the tokens from the last to the first (the backward half of a two-sided layer)
 };
 
-template <typename T, bool MASKED>
+// LAG1: the sums pair dy[t] with the state before token t (kernel lags start at 1: the backward
+// half of a two-sided layer with shift).  A.reverse: x and dy arrive with negated token strides and
+// pointers at the last token; only the mask needs the index turned round here.
+template <typename T, bool MASKED, bool LAG1>
 __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGradArgs A) {
   __shared__ float s_x[kCh][kTk + 4];
   __shared__ float s_g[kCh][kTk + 4];
@@ -101,7 +105,10 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
       s_x[cx][tx] = (cx <= dmax && t0 + tx <= lmax) ? px[k] : 0.f;
       s_g[cg][tg] = (cg <= dmax && t0 + tg <= lmax) ? pg[k] : 0.f;
     }
-    if (MASKED && tid < kTk) s_keep[tid] = A.mask[(size_t)b * A.L + min(t0 + tid, lmax)] ? 0.f : 1.f;
+    if (MASKED && tid < kTk) {
+      const int tm = min(t0 + tid, lmax);
+      s_keep[tid] = A.mask[(size_t)b * A.L + (A.reverse ? lmax - tm : tm)] ? 0.f : 1.f;
+    }
     __syncthreads();
     fetch(t0 + kTk);    // the next tile (clamped past the end) is in flight while this one is worked through
 #pragma unroll 4
@@ -118,11 +125,19 @@ __global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGr
         const float ngi = fmaf(qr, gi, fmaf(qi, gr, si));
         const float nsr = fmaf(qr, sr, fmaf(-qi, si, MASKED ? xs[j] * ks[j] : xs[j]));
         const float nsi = fmaf(qr, si, qi * sr);
+        if (LAG1) {
+          a2r = fmaf(ds[j], sr, a2r);
+          a2i = fmaf(ds[j], si, a2i);
+          a1r = fmaf(ds[j], gr, a1r);
+          a1i = fmaf(ds[j], gi, a1i);
+        }
         gr = ngr; gi = ngi; sr = nsr; si = nsi;
-        a2r = fmaf(ds[j], sr, a2r);
-        a2i = fmaf(ds[j], si, a2i);
-        a1r = fmaf(ds[j], gr, a1r);
-        a1i = fmaf(ds[j], gi, a1i);
+        if (!LAG1) {
+          a2r = fmaf(ds[j], sr, a2r);
+          a2i = fmaf(ds[j], si, a2i);
+          a1r = fmaf(ds[j], gr, a1r);
+          a1i = fmaf(ds[j], gi, a1i);
+        }
         ax = fmaf(ds[j], xs[j], ax);
       }
     }
@@ -173,8 +188,8 @@ extern "C" size_t mega_ema_param_grad_workspace_bytes(int64_t B, int64_t D, int6
 extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, int64_t sgd, int64_t sgl,
                                    int64_t sxb, int64_t sxd, int64_t sxl, const float* p, const float* q,
                                    const float* gamma, const uint8_t* mask, int64_t B, int64_t D, int64_t N,
-                                   int64_t L, float* dp, float* dq, float* dgamma, float* domega, void* workspace,
-                                   size_t workspace_bytes, void* stream) {
+                                   int64_t L, int reverse_time, int lag_one, float* dp, float* dq, float* dgamma,
+                                   float* domega, void* workspace, size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "ema_param_grad: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && D > 0 && N > 0 && L >= 0, MEGA_ERR_ARG, "ema_param_grad: bad shape B=%ld D=%ld N=%ld L=%ld",
@@ -197,15 +212,24 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
                "ema_param_grad: workspace of %zu bytes (16-byte aligned) needed", need);
   EmaGradArgs A;
   A.dy = dy; A.x = x; A.sgb = sgb; A.sgd = sgd; A.sgl = sgl; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl;
-  A.q = q; A.mask = mask;
+  A.q = q; A.mask = mask; A.reverse = reverse_time ? 1 : 0;
+  if (reverse_time) {
+    const int64_t es = dtype == MEGA_F32 ? 4 : 2;
+    A.dy = (const char*)dy + (L - 1) * sgl * es;
+    A.x = (const char*)x + (L - 1) * sxl * es;
+    A.sgl = -sgl;
+    A.sxl = -sxl;
+  }
   A.sums = (float*)workspace;
   A.dyx = (float*)((char*)workspace + align_up((size_t)B * D * N * 16, 256));
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
   const dim3 grid((unsigned)(B * ceil_div(D, kCh)));
-#define LAUNCH_PG(T)                                                                                   \
-  do {                                                                                                 \
-    if (mask) hipLaunchKernelGGL((ema_param_grad_kernel<T, true>), grid, dim3(kBwdThreads), 0, s, A);  \
-    else hipLaunchKernelGGL((ema_param_grad_kernel<T, false>), grid, dim3(kBwdThreads), 0, s, A);      \
+#define LAUNCH_PG(T)                                                                                        \
+  do {                                                                                                      \
+    typedef void (*Kern)(const EmaGradArgs);                                                               \
+    static const Kern table[4] = {ema_param_grad_kernel<T, false, false>, ema_param_grad_kernel<T, false, true>, \
+                                  ema_param_grad_kernel<T, true, false>, ema_param_grad_kernel<T, true, true>};  \
+    hipLaunchKernelGGL(table[(mask ? 2 : 0) + (lag_one ? 1 : 0)], grid, dim3(kBwdThreads), 0, s, A);        \
   } while (0)
   switch (dtype) {
     case MEGA_F32: LAUNCH_PG(float); break;

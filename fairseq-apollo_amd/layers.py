@@ -20,7 +20,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
+from .modules import (AttentionSoftmax, EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
                       TimestepNorm, _training_call)
 
 
@@ -157,6 +157,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         # causal layers: the fused causal op; bidirectional layers (moving_average_gated_attention.py:70-75,
         # 84-92): full softmax over every chunk, SequenceNorm, a two-sided moving average
         self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=not bidirectional, scale=1.0)
+        self.attn_softmax = AttentionSoftmax(dropout=0.0, use_causal_mask=False) if bidirectional else None
         if bidirectional:
             self.norm = SequenceNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
         else:
@@ -242,12 +243,12 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if incremental_state is not None:
             raise NotImplementedError("MovingAverageGatedAttention: incremental state is an inference feature; "
                                       "call it under torch.no_grad()")
-        if self.bidirectional:
-            raise NotImplementedError("MovingAverageGatedAttention: the two-sided moving average has no backward "
-                                      "pass yet; call a bidirectional layer under torch.no_grad()")
         bsz, seq_len, _ = x.size()
         residual = x
-        x = self.norm(x, padding_mask=padding_mask)
+        if self.bidirectional:
+            x = self.norm(x, padding_mask, length_last=False)
+        else:
+            x = self.norm(x, padding_mask=padding_mask)
         v = F.silu(self.v_proj(x))
         mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
         base = self.mx_proj(self.move_act(mx))
@@ -263,7 +264,14 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         v4 = v.reshape(bsz * nc, C, Nh, -1)
         q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
         k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
-        attn = self.efficient_attn(q4, k4, v4).reshape(bsz, seq_len, self.hdim)
+        if self.bidirectional and padding_mask is not None:
+            pad = padding_mask.reshape(bsz * nc, C).to(torch.bool)
+            pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
+            s = torch.einsum('bqnh,bknh->bnqk', q4, k4).masked_fill(pad[:, None, None, :], float('-inf'))
+            attn = torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
+        else:
+            attn = self.efficient_attn(q4, k4, v4)
+        attn = attn.reshape(bsz, seq_len, self.hdim)
         h = F.silu(hx + self.h_proj(attn * F.silu(r)))
         return torch.addcmul(residual, torch.sigmoid(u), h - residual)
 

@@ -52,14 +52,14 @@ class IncrementalState(object):
 
 
 class MovingAverageFunc(torch.autograd.Function):
-    """The whole unidirectional moving-average layer as one differentiable operator: the
+    """The whole moving-average layer (one- or two-sided) as one differentiable operator: the
     reference chains EMAParametersFunc (fused_ops/ema_parameters.py:11-33) and FFTConvFunc
     (fused_ops/fftconv.py:13-41) plus the residual; here neither the kernel nor its gradient is
     materialised.  Inputs (x [B, D, L], p, q, gamma, omega) as BaseMovingLayer holds them."""
 
     @staticmethod
-    def forward(ctx, x, p, q, gamma, omega, padding_mask, out_layout):
-        layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1))
+    def forward(ctx, x, p, q, gamma, omega, padding_mask, out_layout, bidirectional=False, shift=True):
+        layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1), bidirectional, None, shift)
         y, _ = layer(x, padding_mask, None, want_state=False, out_layout=out_layout)
         ctx.layer = layer
         ctx.save_for_backward(x, p, q, gamma, omega, padding_mask)
@@ -71,7 +71,7 @@ class MovingAverageFunc(torch.autograd.Function):
         dx, dp, dq, dg, dom = ops.ema_backward(y_grad, x, p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1),
                                                padding_mask, layer=ctx.layer)
         return (dx, dp.to(p.dtype).view_as(p), dq.to(q.dtype).view_as(q), dg.to(gamma.dtype).view_as(gamma),
-                dom.to(omega.dtype).view_as(omega), None, None)
+                dom.to(omega.dtype).view_as(omega), None, None, None, None)
 
 
 def _training_call(module: nn.Module, *tensors) -> bool:
@@ -154,12 +154,13 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         assert not self.bidirectional or incremental_state is None, \
             'Bidirectional EMA does not support incremental state'
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
-            if self.bidirectional or incremental_state is not None or (self.truncation is not None and self.truncation >= 1):
+            if incremental_state is not None or (self.truncation is not None and self.truncation >= 1):
                 raise NotImplementedError(
-                    f"{type(self).__name__}: the backward pass covers the unidirectional layer without carried "
-                    "state or truncation; call other configurations under torch.no_grad()")
+                    f"{type(self).__name__}: the backward pass covers layers without carried state or kernel "
+                    "truncation; call other configurations under torch.no_grad()")
             p, q, gamma = self._calc_coeffs()           # stays in the graph
-            return MovingAverageFunc.apply(x, p, q, gamma, self.omega, padding_mask, out_layout)
+            return MovingAverageFunc.apply(x, p, q, gamma, self.omega, padding_mask, out_layout, self.bidirectional,
+                                           self.shift)
         layer = self._prepared_layer()
         if incremental_state is not None:
             saved_state = self._get_input_buffer(incremental_state)

@@ -576,12 +576,13 @@ class PreparedEMA:
 
 
     def adjoint(self, y_grad: torch.Tensor, padding_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Gradient of the layer output with respect to its input x (unidirectional layer):
-        dx[t] = (1 - mask[t]) sum_{s >= t} k[s - t] dy[s] + omega dy[t], the same layer run backwards
-        in time.  A channel-contiguous y_grad ([B, L, D] memory) is read in place with negated
-        token strides; rows in time are flipped through a copy.  The result has y_grad's layout."""
-        if self.bidirectional or self.trunc:
-            raise NotImplementedError("adjoint: unidirectional layers without truncation only")
+        """Gradient of the layer output with respect to its input x:
+        dx[t] = (1 - mask[t]) sum_s k(s - t) dy[s] + omega dy[t], the same layer (one- or two-sided)
+        run backwards in time.  A channel-contiguous y_grad ([B, L, D] memory) is read in place with
+        negated token strides; rows in time are flipped through a copy.  The result has y_grad's
+        layout."""
+        if self.trunc:
+            raise NotImplementedError("adjoint: layers without kernel truncation only")
         dev = self.dev
         _need_gpu(y_grad, padding_mask)
         lib = _lib.load()
@@ -598,10 +599,11 @@ class PreparedEMA:
         else:
             dx = torch.empty_strided(g.shape, g.stride(), dtype=g.dtype, device=dev)
             es = g.element_size()
-            key = ("ema", B, D, self.N, L, False, 0)
+            bi = 1 if self.bidirectional else 0
+            key = ("ema", B, D, self.N, L, self.bidirectional, 0)
             nws = _ws_bytes_cache.get(key)
             if nws is None:
-                nws = _ws_bytes_cache[key] = lib.mega_ema_fwd_workspace_bytes(B, D, self.N, L, 0, 0)
+                nws = _ws_bytes_cache[key] = lib.mega_ema_fwd_workspace_bytes(B, D, self.N, L, bi, 0)
             stream = _stream(dev)
             ws = _scratch_buffer(dev, nws, stream)
             sl = g.stride(2)
@@ -609,7 +611,7 @@ class PreparedEMA:
                 rc = lib.mega_ema_fwd(g.data_ptr() + (L - 1) * sl * es, dx.data_ptr() + (L - 1) * sl * es,
                                       _dtype_code(g), g.stride(0), g.stride(1), -sl, dx.stride(0), dx.stride(1), -sl,
                                       _ptr(self.p), _ptr(self.q), _ptr(self.gamma), 1 if self.is_complex else 0,
-                                      _ptr(self.omega), None, None, None, B, D, self.N, L, 0, 0,
+                                      _ptr(self.omega), None, None, None, B, D, self.N, L, bi, 0,
                                       1 if self.shift else 0, _ptr(self.image), _ptr(ws), ws.numel(), stream)
             _lib.check(rc, "ema_fwd (adjoint)")
         if padding_mask is not None:
@@ -852,8 +854,8 @@ def gate_out_fwd(residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: 
 def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor,
                  omega: torch.Tensor, padding_mask: Optional[torch.Tensor] = None,
                  layer: Optional[PreparedEMA] = None):
-    """Backward of ema_forward (unidirectional, no carried state, no truncation):
-    -> (x_grad, p_grad [D,N], q_grad [D,N], gamma_grad [D,N], omega_grad [D]); q_grad / gamma_grad are
+    """Backward of ema_forward (one- or two-sided, no carried state, no truncation):
+    -> (x_grad, p_grad [K,N], q_grad [K,N], gamma_grad [K,N], omega_grad [D]); q_grad / gamma_grad are
     complex for the complex layer, in torch's convention for a real loss (dL = Re(conj(grad) dz)).
     It replaces fftconv_bwd + ema_parameters_bwd of the reference
     (fairseq/modules/fused_ops/fftconv.py:32-41, fused_ops/ema_parameters.py:23-33,
@@ -864,26 +866,33 @@ def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torc
         raise RuntimeError("x and y_grad must be [B, D, L] of the same shape")
     B, D, L = x.shape
     if layer is None:
-        layer = PreparedEMA(p, q, gamma, omega)
+        layer = PreparedEMA(p, q, gamma, omega, bidirectional=p.shape[0] == 2 * D)
     N = layer.N
     xd = x.detach()
     g = y_grad.detach().to(xd.dtype)
     if 0 in g.stride() and g.numel() > 0:
         g = g.contiguous()
     dx = layer.adjoint(g, padding_mask)
-    dp = torch.empty(D, N, dtype=torch.float32, device=dev)
-    dq = torch.empty(D, N, 2, dtype=torch.float32, device=dev)
-    dg = torch.empty(D, N, 2, dtype=torch.float32, device=dev)
+    K = layer.K                                           # D, or 2 D for a two-sided layer
+    dp = torch.empty(K, N, dtype=torch.float32, device=dev)
+    dq = torch.empty(K, N, 2, dtype=torch.float32, device=dev)
+    dg = torch.empty(K, N, 2, dtype=torch.float32, device=dev)
     dom = torch.empty(D, dtype=torch.float32, device=dev)
     m8 = _mask_u8(padding_mask, B, L)
     stream = _stream(dev)
     ws = _scratch_buffer(dev, lib.mega_ema_param_grad_workspace_bytes(B, D, N), stream)
+    # first D rows: the causal half; second D rows (two-sided layers): the same sums over the tokens
+    # walked backwards, lags starting at 1 when the layer shifts its backward kernel
+    halves = [(0, 0, 0)] + ([(D, 1, 1 if layer.shift else 0)] if layer.bidirectional else [])
+    scratch_om = dom if not layer.bidirectional else torch.empty_like(dom)
     with _on_device(dev):
-        rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
-                                     xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.p), _ptr(layer.q),
-                                     _ptr(layer.gamma), _ptr(m8), B, D, N, L, _ptr(dp), _ptr(dq), _ptr(dg), _ptr(dom),
-                                     _ptr(ws), ws.numel(), stream)
-    _lib.check(rc, "ema_param_grad")
+        for off, rev, lag in halves:
+            rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
+                                         xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.p[off:]),
+                                         _ptr(layer.q[off:]), _ptr(layer.gamma[off:]), _ptr(m8), B, D, N, L, rev, lag,
+                                         _ptr(dp[off:]), _ptr(dq[off:]), _ptr(dg[off:]),
+                                         _ptr(dom if off == 0 else scratch_om), _ptr(ws), ws.numel(), stream)
+            _lib.check(rc, "ema_param_grad")
     if layer.is_complex:
         return dx, dp, torch.view_as_complex(dq), torch.view_as_complex(dg), dom
     return dx, dp, dq[..., 0], dg[..., 0], dom

@@ -167,13 +167,17 @@ int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_
  *   domega[d] = sum_{b,t} dy[t] x[t].
  *   dy, x [B,D,L] of `dtype` with element strides; p [D,N], q, gamma [D,N,2] fp32 (imaginary
  *   parts 0 for the real layer); mask [B,L] or NULL; outputs dp [D,N], dq, dgamma [D,N,2],
- *   domega [D] fp32; N <= 16; workspace of mega_ema_param_grad_workspace_bytes(B, D, N).   */
+ *   domega [D] fp32; N <= 16; workspace of mega_ema_param_grad_workspace_bytes(B, D, N).
+ *   A two-sided layer takes two calls: its first D coefficient rows as above; its second D rows
+ *   with reverse_time = 1 (the tokens are walked from the last to the first) and lag_one = shift
+ *   (dy[t] is paired with the state before token t: kernel lags start at 1).               */
 size_t mega_ema_param_grad_workspace_bytes(int64_t B, int64_t D, int64_t N);
 int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, int64_t sgd,
                         int64_t sgl, int64_t sxb, int64_t sxd, int64_t sxl, const float* p,
                         const float* q, const float* gamma, const uint8_t* mask, int64_t B,
-                        int64_t D, int64_t N, int64_t L, float* dp, float* dq, float* dgamma,
-                        float* domega, void* workspace, size_t workspace_bytes, void* stream);
+                        int64_t D, int64_t N, int64_t L, int reverse_time, int lag_one, float* dp,
+                        float* dq, float* dgamma, float* domega, void* workspace,
+                        size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Long convolution with an explicit time-domain kernel                      */

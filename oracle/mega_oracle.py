@@ -269,11 +269,13 @@ def ema_kernel_bwd(dk, p, q, gamma):
     return (sum2 * gamma).real, np.conj(sum1 * p * gamma), np.conj(sum2 * p)
 
 
-def ema_backward(dy, x, p, q, gamma, omega, padding_mask=None):
-    """Backward of ema_forward (unidirectional, no carried state): the reference's chain
-    fftconv backward (modules/fused_ops/fftconv.py:66-88: dx = correlation of dy with k,
-    dk = sum over the batch of the correlation of dy with x) -> ema_kernel_bwd, with the
-    correlations written out directly.  Returns (dx, dp, dq, dgamma, domega)."""
+def ema_backward(dy, x, p, q, gamma, omega, padding_mask=None, bidirectional: bool = False, shift: bool = True):
+    """Backward of ema_forward (no carried state): the reference's chain fftconv backward
+    (modules/fused_ops/fftconv.py:66-88, 85-100: dx = correlation of dy with k, dk = sum over the
+    batch of the correlation of dy with x) -> ema_kernel_bwd, with the correlations written out
+    directly.  Two-sided layers: y[t] = sum_{j>=0} k1[j] x[t-j] + sum_{m>=1} k2[m-1] x[t+m] (shift) or
+    sum_{m>=0} k2[m] x[t+m] (no shift), k1 / k2 from the first / second D coefficient rows.
+    Returns (dx, dp, dq, dgamma, domega)."""
     dy = np.asarray(dy, np.float64)
     x = np.asarray(x, np.float64)
     B, D, L = x.shape
@@ -281,10 +283,16 @@ def ema_backward(dy, x, p, q, gamma, omega, padding_mask=None):
     xm = x * keep
     k = ema_kernel(p, q, gamma, L)
     dxc = np.zeros_like(x)
-    dk = np.zeros((D, L))
+    dk = np.zeros((k.shape[0], L))
     for l in range(L):
-        dxc[:, :, :L - l] += dy[:, :, l:] * k[None, :, l:l + 1]
-        dk[:, l] = (dy[:, :, l:] * xm[:, :, :L - l]).sum(axis=(0, 2))
+        # forward lags: y[t] += k1[l] x[t - l]
+        dxc[:, :, :L - l] += dy[:, :, l:] * k[None, :D, l:l + 1]
+        dk[:D, l] = (dy[:, :, l:] * xm[:, :, :L - l]).sum(axis=(0, 2))
+        if bidirectional:
+            m = l + 1 if shift else l                       # backward lags: y[t] += k2[l] x[t + m]
+            if m < L:
+                dxc[:, :, m:] += dy[:, :, :L - m] * k[None, D:, l:l + 1]
+                dk[D:, l] = (dy[:, :, :L - m] * xm[:, :, m:]).sum(axis=(0, 2))
     om = np.asarray(omega, np.float64).reshape(1, D, 1)
     dp, dq, dg = ema_kernel_bwd(dk, p, q, gamma)
     return dxc * keep + om * dy, dp, dq, dg, (dy * x).sum(axis=(0, 2))

@@ -149,6 +149,64 @@ def test_ema_backward(dtype, B, D, N, L, cplx, layout, masked):
             assert rel_err(a, np.real(b)) < 5e-4, name
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,D,N,L,shift,layout,masked", [
+    (2, 32, 16, 2048, True, "bld", False),    # matrix-core path, both directions
+    (2, 24, 16, 300, True, "bld", True),
+    (1, 16, 4, 150, False, "bdl", True),      # backward kernel with its lag-0 tap
+])
+def test_ema_backward_two_sided(dtype, B, D, N, L, shift, layout, masked):
+    rng = np.random.default_rng(63)
+    p, q, g = _ema_coeffs(rng, 2 * D, N, True)
+    p, q, g = p.astype(np.float32).astype(np.float64), q.astype(np.complex64).astype(np.complex128), \
+        g.astype(np.complex64).astype(np.complex128)
+    om = rng.normal(size=D).astype(np.float32).astype(np.float64)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    if layout == "bld":
+        x = x.transpose(1, 2).contiguous().transpose(1, 2)
+        dy = dy.transpose(1, 2).contiguous().transpose(1, 2)
+    mask = (rng.random((B, L)) < 0.2) if masked else None
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om), True, None, shift)
+    got = M.ops.ema_backward(dy, x, dev(p), dev(q), dev(g), dev(om), tm, layer=layer)
+    ref = O.ema_backward(dy64, x64, p, q, g, om, mask, True, shift)
+    assert rel_err(host(got[0]), ref[0]) < TOL[dtype]
+    for a, b, name in zip(got[1:], ref[1:], ("dp", "dq", "dgamma", "domega")):
+        a = host(a)
+        if np.iscomplexobj(b):
+            assert rel_err(a.real, b.real) < 5e-4 and rel_err(a.imag, b.imag) < 5e-4, name
+        else:
+            assert rel_err(a, np.real(b)) < 5e-4, name
+
+
+def test_two_sided_module_autograd():
+    rng = np.random.default_rng(64)
+    B, D, N, L = 2, 16, 8, 80
+    torch.manual_seed(6)
+    mod = M.MultiHeadComplexEMA(D, ndim=N, bidirectional=True).to(DEV).train()
+    x64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    x = dev(x64).requires_grad_(True)
+    (mod(x) * dev(w64)).sum().backward()
+    P = {n: host(getattr(mod, n)) for n in ("alpha", "delta", "theta", "gamma", "omega")}
+
+    def loss(Pd):
+        p, q, g = O.ema_coeffs_complex(Pd["alpha"], Pd["delta"], Pd["theta"], Pd["gamma"])
+        return (O.ema_forward(x64, p, q, g, Pd["omega"].reshape(-1), bidirectional=True)[0] * w64).sum()
+
+    eps = 1e-5
+    for n in P:
+        grad = host(getattr(mod, n).grad)
+        scale = np.abs(grad).max() + 1e-6
+        for _ in range(4):
+            idx = tuple(rng.integers(0, s) for s in P[n].shape)
+            Pp = {k: v.copy() for k, v in P.items()}; Pp[n][idx] += eps
+            Pm = {k: v.copy() for k, v in P.items()}; Pm[n][idx] -= eps
+            fd = (loss(Pp) - loss(Pm)) / (2 * eps)
+            assert abs(fd - grad[idx]) < 2e-3 * scale, (n, idx, fd, grad[idx])
+
+
 @pytest.mark.parametrize("cls,N", [("cema", 16), ("ema", 2)])
 def test_moving_average_module_autograd(cls, N):
     """Gradients of the raw parameters (alpha, delta, theta | beta, gamma, omega) and of x through
@@ -234,16 +292,22 @@ def test_attention_autograd(dtype, tol, B, L, Nh, H1, H2):
         assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
 
 
-@pytest.mark.parametrize("heads,act,moving", [(1, 'rmsnorm', 'cema'), (2, 'silu', 'ema')])
-def test_gated_attention_layer_trains(heads, act, moving):
-    """The whole layer under autograd (fp32): parameter and input gradients against central
-    differences of the fp64 layer oracle."""
+@pytest.mark.parametrize("heads,act,moving,bidir", [(1, 'rmsnorm', 'cema', False), (2, 'silu', 'ema', False),
+                                                    (1, 'silu', 'cema', True), (2, 'rmsnorm', 'cema', "padded")])
+def test_gated_attention_layer_trains(heads, act, moving, bidir):
+    """The whole layer under autograd (fp32), causal and bidirectional (also with padding):
+    parameter and input gradients against central differences of the fp64 layer oracle."""
     from test_gpu_layer import _params
     rng = np.random.default_rng(73)
     B, L, D, S, E, N, C = 2, 32, 16, 8, 24, 4, 16
     torch.manual_seed(11)
     layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_layer=moving, moving_act=act,
-                                          norm_num_groups=4, num_heads=heads).to(DEV).train()
+                                          norm_num_groups=4, num_heads=heads, bidirectional=bool(bidir)).to(DEV).train()
+    mask = None
+    if bidir == "padded":
+        mask = np.zeros((B, L), bool)
+        mask[0, 27:] = True
+        mask[1, 12:] = True                    # the second chunk of row 1 is padding only
     with torch.no_grad():
         for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
             prm.normal_(0, 0.3)
@@ -251,14 +315,16 @@ def test_gated_attention_layer_trains(heads, act, moving):
         layer.norm.weight.normal_(0, 0.2); layer.norm.bias.normal_(0, 0.2)
     x64 = rng.normal(size=(B, L, D)).astype(np.float32).astype(np.float64)
     w64 = rng.normal(size=(B, L, D)).astype(np.float32).astype(np.float64)
+    if mask is not None:
+        w64 = w64 * (~mask)[..., None]         # padded positions carry no loss
     x = dev(x64).requires_grad_(True)
-    out, _ = layer(x)
+    out, _ = layer(x, None if mask is None else torch.from_numpy(mask).to(DEV))
     (out * dev(w64)).sum().backward()
     P = _params(layer)
-    loss = lambda Pd, xx: (O.gated_attention_layer(xx, Pd, chunk=C, num_heads=heads, moving_act=act,
-                                                   num_groups=4) * w64).sum()
-    assert rel_err(host(out), O.gated_attention_layer(x64, P, chunk=C, num_heads=heads, moving_act=act,
-                                                      num_groups=4)) < 1e-4
+    okw = dict(chunk=C, num_heads=heads, moving_act=act, num_groups=4, bidirectional=bool(bidir), padding_mask=mask)
+    loss = lambda Pd, xx: (O.gated_attention_layer(xx, Pd, **okw) * w64).sum()
+    keep = np.ones((B, L), bool) if mask is None else ~mask
+    assert rel_err(host(out)[keep], O.gated_attention_layer(x64, P, **okw)[keep]) < 1e-4
     eps = 1e-5
     checks = [("v_w", layer.v_proj.weight), ("mx_w", layer.mx_proj.weight), ("mx_b", layer.mx_proj.bias),
               ("h_w", layer.h_proj.weight), ("gamma", layer.gamma), ("beta", layer.beta),

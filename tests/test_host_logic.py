@@ -68,7 +68,7 @@ def test_incremental_state_keys_are_per_module():
 def test_configurations_without_a_backward_refuse_autograd():
     """The unidirectional moving average, TimestepNorm and the attention have backward operators;
     what has none says so instead of returning tensors that silently carry no graph."""
-    e = M.MultiHeadComplexEMA(4, ndim=2, bidirectional=True)
+    e = M.MultiHeadComplexEMA(4, ndim=2, bidirectional=True, truncation=4)
     with pytest.raises(NotImplementedError, match="backward pass covers"):
         e(torch.zeros(1, 4, 8))
     layer = M.MovingAverageGatedAttention(8, 4, 8, 2, chunk_size=4, norm_num_groups=2)

@@ -48,16 +48,18 @@ def test_timestep_norm_bwd_matches_finite_differences(G, masked, prior):
             assert abs(_fd(f, args[which], idx) - g[idx]) < 1e-6
 
 
-@pytest.mark.parametrize("masked", [False, True])
-def test_ema_backward_matches_finite_differences(masked):
+@pytest.mark.parametrize("masked,bidir,shift", [(False, False, True), (True, False, True), (True, True, True),
+                                                (False, True, False)])
+def test_ema_backward_matches_finite_differences(masked, bidir, shift):
     rng = np.random.default_rng(8)
     D, N, L, B = 3, 4, 13, 2
-    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, 2 * D if bidir else D, N))
     om = rng.normal(size=D)
     x, wy = rng.normal(size=(B, D, L)), rng.normal(size=(B, D, L))
     mask = (rng.random((B, L)) < 0.3) if masked else None
-    loss = lambda x_, p_, q_, g_, o_: (O.ema_forward(x_, p_, q_, g_, o_, mask)[0] * wy).sum()
-    dx, dp, dq, dg, dom = O.ema_backward(wy, x, p, q, g, om, mask)
+    loss = lambda x_, p_, q_, g_, o_: (O.ema_forward(x_, p_, q_, g_, o_, mask, bidirectional=bidir,
+                                                     shift=shift)[0] * wy).sum()
+    dx, dp, dq, dg, dom = O.ema_backward(wy, x, p, q, g, om, mask, bidir, shift)
     for _ in range(6):
         i = tuple(rng.integers(0, s) for s in x.shape)
         j = tuple(rng.integers(0, s) for s in p.shape)
