@@ -67,6 +67,9 @@ SIGNATURES = {
     "mega_gate_qk_fwd": (_int, [_p, _i64, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_double, _p]),
     "mega_gate_mul_fwd": (_int, [_p, _i64, _p, _i64, _p, _int, _i64, _i64, _p]),
     "mega_gate_out_fwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _int, _i64, _i64, _p]),
+    "mega_gate_mul_bwd": (_int, [_p, _p, _i64, _p, _i64, _p, _p, _int, _i64, _i64, _p]),
+    "mega_gate_out_bwd": (_int, [_p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _int, _i64, _i64, _p]),
+    "mega_swiglu_bwd": (_int, [_p, _p, _p, _p, _p, _int, _i64, _p]),
 }
 
 _lib = None

@@ -160,6 +160,100 @@ __global__ __launch_bounds__(256) void gate_out_kernel(const T* __restrict__ res
 }
 
 // ---------------------------------------------------------------------------------------------
+// Backward of the three element-wise gates.  silu'(a) = s (1 + a (1 - s)), s = sigmoid(a).
+__device__ __forceinline__ float dsilu_f(float a) {
+  const float sg = sigmoid_f(a);
+  return sg * fmaf(a, 1.0f - sg, 1.0f);
+}
+
+// y = a * silu(r):  da = dy silu(r),  dr = dy a silu'(r)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_mul_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ a,
+                                                           int64_t as, const T* __restrict__ r, int64_t rs,
+                                                           T* __restrict__ da, T* __restrict__ dr, int64_t T_, int E) {
+  using V = Vec<T, VEC>;
+  for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
+    for (int j = threadIdx.x * VEC; j < E; j += 256 * VEC) {
+      const V gv = *(const V*)(dy + t * (int64_t)E + j);
+      const V av = *(const V*)(a + t * as + j);
+      const V rv = *(const V*)(r + t * rs + j);
+      V oa, orr;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float g = to_float(gv.v[i]), rr = to_float(rv.v[i]);
+        oa.v[i] = from_float<T>(g * silu_f(rr));
+        orr.v[i] = from_float<T>(g * to_float(av.v[i]) * dsilu_f(rr));
+      }
+      *(V*)(da + t * (int64_t)E + j) = oa;
+      *(V*)(dr + t * (int64_t)E + j) = orr;
+    }
+  }
+}
+
+// y = res + sigmoid(u) (silu(hx + hp) - res):
+//   dres = dy (1 - s),  du = dy (h - res) s (1 - s),  da = dy s silu'(hx + hp)  (da serves hx and hp)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void gate_out_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ res,
+                                                           int64_t ress, const T* __restrict__ u, int64_t us,
+                                                           const T* __restrict__ hx, int64_t hxs,
+                                                           const T* __restrict__ hp, int64_t hps, T* __restrict__ dres,
+                                                           T* __restrict__ du, T* __restrict__ da, int64_t T_, int D) {
+  using V = Vec<T, VEC>;
+  for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
+    for (int j = threadIdx.x * VEC; j < D; j += 256 * VEC) {
+      const V gv = *(const V*)(dy + t * (int64_t)D + j);
+      const V rv = *(const V*)(res + t * ress + j);
+      const V uv = *(const V*)(u + t * us + j);
+      const V xv = *(const V*)(hx + t * hxs + j);
+      const V pv = *(const V*)(hp + t * hps + j);
+      V o0, o1, o2;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float g = to_float(gv.v[i]), rr = to_float(rv.v[i]);
+        const float sg = sigmoid_f(to_float(uv.v[i]));
+        const float a = to_float(xv.v[i]) + to_float(pv.v[i]);
+        o0.v[i] = from_float<T>(g * (1.0f - sg));
+        o1.v[i] = from_float<T>(g * (silu_f(a) - rr) * sg * (1.0f - sg));
+        o2.v[i] = from_float<T>(g * sg * dsilu_f(a));
+      }
+      *(V*)(dres + t * (int64_t)D + j) = o0;
+      *(V*)(du + t * (int64_t)D + j) = o1;
+      *(V*)(da + t * (int64_t)D + j) = o2;
+    }
+  }
+}
+
+// y = silu(a) * b:  da = dy b silu'(a),  db = dy silu(a)   (contiguous operands)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ a,
+                                                         const T* __restrict__ b, T* __restrict__ da,
+                                                         T* __restrict__ db, int64_t n) {
+  using V = Vec<T, VEC>;
+  const int64_t nv = n / VEC;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+    const V gv = ((const V*)dy)[i];
+    const V av = ((const V*)a)[i];
+    const V bv = ((const V*)b)[i];
+    V oa, ob;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float g = to_float(gv.v[k]), aa = to_float(av.v[k]);
+      oa.v[k] = from_float<T>(g * to_float(bv.v[k]) * dsilu_f(aa));
+      ob.v[k] = from_float<T>(g * silu_f(aa));
+    }
+    ((V*)da)[i] = oa;
+    ((V*)db)[i] = ob;
+  }
+  const int64_t t = nv * VEC + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) {
+    const float g = to_float(dy[t]), aa = to_float(a[t]);
+    da[t] = from_float<T>(g * to_float(b[t]) * dsilu_f(aa));
+    db[t] = from_float<T>(g * silu_f(aa));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 inline bool vec_ok(const void* p, int64_t stride, size_t elem, int vec) {
   return ((uintptr_t)p % (elem * vec)) == 0 && stride % vec == 0;
 }
@@ -229,6 +323,59 @@ int launch_gate_out(const void* res, int64_t ress, const void* u, int64_t us, co
     hipLaunchKernelGGL((gate_out_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)res, ress, (const T*)u,
                        us, (const T*)hx, hxs, (const T*)hp, hps, (T*)y, T_, (int)D);
   MEGA_CHECK_LAUNCH("gate_out_fwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_gate_mul_bwd(const void* dy, const void* a, int64_t as, const void* r, int64_t rs, void* da, void* dr,
+                        int64_t T_, int64_t E, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool v = E % VEC == 0 && vec_ok(dy, E, sizeof(T), VEC) && vec_ok(a, as, sizeof(T), VEC) &&
+                 vec_ok(r, rs, sizeof(T), VEC) && vec_ok(da, E, sizeof(T), VEC) && vec_ok(dr, E, sizeof(T), VEC);
+  if (v)
+    hipLaunchKernelGGL((gate_mul_bwd_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)a,
+                       as, (const T*)r, rs, (T*)da, (T*)dr, T_, (int)E);
+  else
+    hipLaunchKernelGGL((gate_mul_bwd_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)a, as,
+                       (const T*)r, rs, (T*)da, (T*)dr, T_, (int)E);
+  MEGA_CHECK_LAUNCH("gate_mul_bwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_gate_out_bwd(const void* dy, const void* res, int64_t ress, const void* u, int64_t us, const void* hx,
+                        int64_t hxs, const void* hp, int64_t hps, void* dres, void* du, void* da, int64_t T_,
+                        int64_t D, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool v = D % VEC == 0 && vec_ok(dy, D, sizeof(T), VEC) && vec_ok(res, ress, sizeof(T), VEC) &&
+                 vec_ok(u, us, sizeof(T), VEC) && vec_ok(hx, hxs, sizeof(T), VEC) && vec_ok(hp, hps, sizeof(T), VEC) &&
+                 vec_ok(dres, D, sizeof(T), VEC) && vec_ok(du, D, sizeof(T), VEC) && vec_ok(da, D, sizeof(T), VEC);
+  if (v)
+    hipLaunchKernelGGL((gate_out_bwd_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)res,
+                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, (T*)da, T_,
+                       (int)D);
+  else
+    hipLaunchKernelGGL((gate_out_bwd_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)res,
+                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, (T*)da, T_,
+                       (int)D);
+  MEGA_CHECK_LAUNCH("gate_out_bwd");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_swiglu_bwd(const void* dy, const void* a, const void* b, void* da, void* db, int64_t n, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool aligned = (((uintptr_t)dy | (uintptr_t)a | (uintptr_t)b | (uintptr_t)da | (uintptr_t)db) % 16) == 0;
+  int64_t blocks = ceil_div(ceil_div(n, VEC), 256);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  if (aligned)
+    hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)dy, (const T*)a,
+                       (const T*)b, (T*)da, (T*)db, n);
+  else
+    hipLaunchKernelGGL((swiglu_bwd_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)dy, (const T*)a,
+                       (const T*)b, (T*)da, (T*)db, n);
+  MEGA_CHECK_LAUNCH("swiglu_bwd");
   return MEGA_OK;
 }
 
@@ -304,4 +451,43 @@ extern "C" int mega_gate_out_fwd(const void* residual, int64_t residual_stride, 
   hipStream_t s = (hipStream_t)stream;
   MEGA_GLUE_DISPATCH(launch_gate_out, residual, residual_stride, u, u_stride, hx, hx_stride, hp, hp_stride, y, T_, D,
                      s);
+}
+
+extern "C" int mega_gate_mul_bwd(const void* y_grad, const void* a, int64_t a_stride, const void* r, int64_t r_stride,
+                                 void* a_grad, void* r_grad, int dtype, int64_t T_, int64_t E, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_mul_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && E >= 1 && E < (1ll << 30), MEGA_ERR_ARG, "gate_mul_bwd: bad sizes T=%lld E=%lld",
+               (long long)T_, (long long)E);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && a && r && a_grad && r_grad, MEGA_ERR_ARG, "gate_mul_bwd: null pointer argument");
+  MEGA_REQUIRE(a_stride >= E && r_stride >= E, MEGA_ERR_ARG, "gate_mul_bwd: a row stride is below the row length");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_gate_mul_bwd, y_grad, a, a_stride, r, r_stride, a_grad, r_grad, T_, E, s);
+}
+
+extern "C" int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual_stride, const void* u,
+                                 int64_t u_stride, const void* hx, int64_t hx_stride, const void* hp,
+                                 int64_t hp_stride, void* residual_grad, void* u_grad, void* h_grad, int dtype,
+                                 int64_t T_, int64_t D, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_out_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && D >= 1 && D < (1ll << 30), MEGA_ERR_ARG, "gate_out_bwd: bad sizes T=%lld D=%lld",
+               (long long)T_, (long long)D);
+  if (T_ == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && residual && u && hx && hp && residual_grad && u_grad && h_grad, MEGA_ERR_ARG,
+               "gate_out_bwd: null pointer argument");
+  MEGA_REQUIRE(residual_stride >= D && u_stride >= D && hx_stride >= D && hp_stride >= D, MEGA_ERR_ARG,
+               "gate_out_bwd: a row stride is below the row length");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_gate_out_bwd, y_grad, residual, residual_stride, u, u_stride, hx, hx_stride, hp, hp_stride,
+                     residual_grad, u_grad, h_grad, T_, D, s);
+}
+
+extern "C" int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_grad, void* b_grad, int dtype,
+                               int64_t n, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "swiglu_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(n >= 0, MEGA_ERR_ARG, "swiglu_bwd: negative size");
+  if (n == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && a && b && a_grad && b_grad, MEGA_ERR_ARG, "swiglu_bwd: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  MEGA_GLUE_DISPATCH(launch_swiglu_bwd, y_grad, a, b, a_grad, b_grad, n, s);
 }

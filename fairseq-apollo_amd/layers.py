@@ -1,13 +1,15 @@
 """Layer glue around the HIP ops: the caller of the hot path in the reference,
 `MovingAverageGatedAttention` (fairseq/modules/moving_average_gated_attention.py:26-470),
-restricted to what Mega2 uses on the causal path (unidirectional, softmax attention through
-the fused rotary / causal op, TimestepNorm, EMA or CEMA), plus the north-star SwiGLU FFN.
+restricted to the rotary softmax attention through the fused ops (causal with TimestepNorm and a
+one-sided EMA / CEMA, or bidirectional with SequenceNorm and a two-sided one), plus the north-star
+SwiGLU FFN.
 
 The projections are library GEMMs (torch -> hipBLASLt); normalisation, moving average,
 attention and the SwiGLU gate run in libmega_hip.so.  Under autograd the normalisation, the
 moving average and the attention (softmax backward in libmega_hip.so, batched library GEMMs) keep
-their own backward operators; the element-wise glue then runs as torch operations so that the
-graph is complete.
+their own backward operators, and so do the r gate, the output gate and the SwiGLU gate; the
+remaining element-wise steps (q / k map, activations of v and of the moving average) run as torch
+operations so that the graph is complete.
 """
 from __future__ import annotations
 
@@ -20,7 +22,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (AttentionSoftmax, EfficientAttention, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
+from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
                       TimestepNorm, _training_call)
 
 
@@ -271,9 +273,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             attn = torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
         else:
             attn = self.efficient_attn(q4, k4, v4)
-        attn = attn.reshape(bsz, seq_len, self.hdim)
-        h = F.silu(hx + self.h_proj(attn * F.silu(r)))
-        return torch.addcmul(residual, torch.sigmoid(u), h - residual)
+        hp = self.h_proj(GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r))
+        return GateOutFunc.apply(residual, u, hx, hp)
 
     def _cached_attention(self, z: Tensor, v: Tensor, saved_state, incremental_state) -> Tensor:
         """Attention with the partial-chunk key / value cache

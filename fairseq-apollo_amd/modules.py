@@ -512,6 +512,47 @@ class SequenceNorm(nn.Module):
         return 'num_features={num_features}, num_groups={num_groups}, eps={eps}'.format(**self.__dict__)
 
 
+class GateMulFunc(torch.autograd.Function):
+    """a * silu(r) with its own backward (moving_average_gated_attention.py:330, 407)."""
+
+    @staticmethod
+    def forward(ctx, a, r):
+        ctx.save_for_backward(a, r)
+        return ops.gate_mul_fwd(a, r)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        return ops.gate_mul_bwd(y_grad, *ctx.saved_tensors)
+
+
+class GateOutFunc(torch.autograd.Function):
+    """residual + sigmoid(u) * (silu(hx + hp) - residual) with its own backward
+    (moving_average_gated_attention.py:322, 409, 412)."""
+
+    @staticmethod
+    def forward(ctx, residual, u, hx, hp):
+        ctx.save_for_backward(residual, u, hx, hp)
+        return ops.gate_out_fwd(residual, u, hx, hp)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        dres, du, dh = ops.gate_out_bwd(y_grad, *ctx.saved_tensors)
+        return dres, du, dh, dh
+
+
+class SwiGLUFunc(torch.autograd.Function):
+    """silu(a) * b with its own backward."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        ctx.save_for_backward(a, b)
+        return ops.swiglu(a, b)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        return ops.swiglu_bwd(y_grad, *ctx.saved_tensors)
+
+
 class AttentionSoftmaxFunc(torch.autograd.Function):
     """fairseq/modules/attention_softmax.py:11-39 (dropout = 0)."""
 
@@ -609,5 +650,5 @@ class SwiGLU(nn.Module):
 
     def forward(self, x: Tensor) -> Tensor:
         if _training_call(self, x):
-            return self.w2(F.silu(self.w1(x)) * self.w3(x))      # autograd: element-wise gate in torch
+            return self.w2(SwiGLUFunc.apply(self.w1(x), self.w3(x)))
         return self.w2(ops.swiglu(self.w1(x), self.w3(x)))

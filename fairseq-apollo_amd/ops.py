@@ -896,3 +896,51 @@ def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torc
     if layer.is_complex:
         return dx, dp, torch.view_as_complex(dq), torch.view_as_complex(dg), dom
     return dx, dp, dq[..., 0], dg[..., 0], dom
+
+
+def gate_mul_bwd(y_grad: torch.Tensor, a: torch.Tensor, r: torch.Tensor):
+    """Backward of gate_mul_fwd: -> (a_grad, r_grad)."""
+    dev = _need_gpu(y_grad, a, r)
+    lib = _lib.load()
+    ar, as_ = _rows(a)
+    rr, rs = _rows(r)
+    g = y_grad.detach().to(a.dtype).contiguous()
+    da = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    dr = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_gate_mul_bwd(_ptr(g), _ptr(ar), as_, _ptr(rr), rs, _ptr(da), _ptr(dr), _dtype_code(ar),
+                                   _ntok(a), a.shape[-1], _stream(dev))
+    _lib.check(rc, "gate_mul_bwd")
+    return da, dr
+
+
+def gate_out_bwd(y_grad: torch.Tensor, residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: torch.Tensor):
+    """Backward of gate_out_fwd: -> (residual_grad, u_grad, h_grad); h_grad is the gradient of hx and of hp."""
+    dev = _need_gpu(y_grad, residual, u, hx, hp)
+    lib = _lib.load()
+    r0, rs = _rows(residual)
+    u0, us = _rows(u)
+    x0, xs = _rows(hx)
+    p0, ps = _rows(hp)
+    g = y_grad.detach().to(residual.dtype).contiguous()
+    outs = [torch.empty(residual.shape, dtype=residual.dtype, device=dev) for _ in range(3)]
+    with _on_device(dev):
+        rc = lib.mega_gate_out_bwd(_ptr(g), _ptr(r0), rs, _ptr(u0), us, _ptr(x0), xs, _ptr(p0), ps, _ptr(outs[0]),
+                                   _ptr(outs[1]), _ptr(outs[2]), _dtype_code(r0), _ntok(residual), residual.shape[-1],
+                                   _stream(dev))
+    _lib.check(rc, "gate_out_bwd")
+    return tuple(outs)
+
+
+def swiglu_bwd(y_grad: torch.Tensor, a: torch.Tensor, b: torch.Tensor):
+    """Backward of swiglu: -> (a_grad, b_grad)."""
+    dev = _need_gpu(y_grad, a, b)
+    lib = _lib.load()
+    ad, bd = a.detach().contiguous(), b.detach().contiguous()
+    g = y_grad.detach().to(ad.dtype).contiguous()
+    da, db = torch.empty_like(ad), torch.empty_like(ad)
+    with _on_device(dev):
+        rc = lib.mega_swiglu_bwd(_ptr(g), _ptr(ad), _ptr(bd), _ptr(da), _ptr(db), _dtype_code(ad), ad.numel(),
+                                 _stream(dev))
+    _lib.check(rc, "swiglu_bwd")
+    return da, db

@@ -343,6 +343,22 @@ int mega_gate_mul_fwd(const void* a, int64_t a_stride, const void* r, int64_t r_
 int mega_gate_out_fwd(const void* residual, int64_t residual_stride, const void* u,
                       int64_t u_stride, const void* hx, int64_t hx_stride, const void* hp,
                       int64_t hp_stride, void* y, int dtype, int64_t T, int64_t D, void* stream);
+/* Backward of the element-wise gates (in the reference these are autograd graphs of torch
+ * element-wise operations over the same lines); gradients are contiguous [T, *] of `dtype`:
+ *   mega_gate_mul_bwd: a_grad = y_grad silu(r), r_grad = y_grad a silu'(r)
+ *   mega_gate_out_bwd: residual_grad = y_grad (1 - s), u_grad = y_grad (h - residual) s (1 - s),
+ *                      h_grad = y_grad s silu'(hx + hp) (the gradient of hx and of hp),
+ *                      s = sigmoid(u), h = silu(hx + hp)
+ *   mega_swiglu_bwd:   a_grad = y_grad b silu'(a), b_grad = y_grad silu(a)                 */
+int mega_gate_mul_bwd(const void* y_grad, const void* a, int64_t a_stride, const void* r,
+                      int64_t r_stride, void* a_grad, void* r_grad, int dtype, int64_t T, int64_t E,
+                      void* stream);
+int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual_stride,
+                      const void* u, int64_t u_stride, const void* hx, int64_t hx_stride,
+                      const void* hp, int64_t hp_stride, void* residual_grad, void* u_grad,
+                      void* h_grad, int dtype, int64_t T, int64_t D, void* stream);
+int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_grad, void* b_grad,
+                    int dtype, int64_t n, void* stream);
 
 #ifdef __cplusplus
 }

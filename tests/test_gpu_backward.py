@@ -428,3 +428,36 @@ def test_sequence_norm_module_autograd_and_golden():
         dx, dg, db = M.ops.group_sequence_norm_bwd(dev(c["y_grad"]), dev(c["x"]), n, mu, r, dev(c["gamma"]), tm, G, last)
         assert rel_err(host(dx), c["x_grad"]) < 1e-4, tag
         assert rel_err(host(dg), c["gamma_grad"]) < 1e-4 and rel_err(host(db), c["beta_grad"]) < 1e-4, tag
+
+
+# ----------------------------------------------------------------------------------------------
+# element-wise gates
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,width,off", [((2, 50, 512), 1100, 80), ((4, 9, 35), 35, 0)])
+def test_gate_backwards(dtype, shape, width, off):
+    """gate_mul, gate_out and swiglu backward against the closed-form derivatives in fp64
+    (silu'(a) = s (1 + a (1 - s)), s = sigmoid(a)); operands that are slices of a wider row."""
+    from test_gpu_ops import _wide
+    rng = np.random.default_rng(95)
+    sg = O._sigmoid
+    dsilu = lambda a_: sg(a_) * (1 + a_ * (1 - sg(a_)))
+    a, a64 = rounded(rng.normal(size=shape), dtype)
+    r, r64 = _wide(rng, shape, width, off, dtype)
+    dy, dy64 = rounded(rng.normal(size=shape), dtype)
+    da, dr = M.ops.gate_mul_bwd(dy, a, r)
+    assert rel_err(host(da), dy64 * O._silu(r64)) < TOL[dtype]
+    assert rel_err(host(dr), dy64 * a64 * dsilu(r64)) < TOL[dtype]
+    u, u64 = _wide(rng, shape, width, 0, dtype)
+    hx, hx64 = _wide(rng, shape, width, off, dtype)
+    hp, hp64 = rounded(rng.normal(size=shape), dtype)
+    res, res64 = rounded(rng.normal(size=shape), dtype)
+    dres, du, dh = M.ops.gate_out_bwd(dy, res, u, hx, hp)
+    s, aa = sg(u64), hx64 + hp64
+    assert rel_err(host(dres), dy64 * (1 - s)) < TOL[dtype]
+    assert rel_err(host(du), dy64 * (O._silu(aa) - res64) * s * (1 - s)) < TOL[dtype]
+    assert rel_err(host(dh), dy64 * s * dsilu(aa)) < TOL[dtype]
+    b, b64 = rounded(rng.normal(size=shape), dtype)
+    ga, gb = M.ops.swiglu_bwd(dy, a, b)
+    assert rel_err(host(ga), dy64 * b64 * dsilu(a64)) < TOL[dtype]
+    assert rel_err(host(gb), dy64 * O._silu(a64)) < TOL[dtype]
