@@ -19,11 +19,9 @@
 namespace mega {
 namespace {
 
-constexpr int kCh = 16;        // channels per workgroup
 constexpr int kNs = 16;        // state lanes per channel
 constexpr int kTk = 128;       // tokens per LDS tile
-constexpr int kBwdThreads = kCh * kNs;
-constexpr int kPerThread = kCh * kTk / kBwdThreads;   // elements of one tile a thread moves
+constexpr int kPerThread = kTk / kNs;   // elements of one tile a thread moves (CH * kTk / (CH * kNs))
 
 struct EmaGradArgs {
   const void* dy;
@@ -41,8 +39,11 @@ struct EmaGradArgs {
 // LAG1: the sums pair dy[t] with the state before token t (kernel lags start at 1: the backward
 // half of a two-sided layer with shift).  A.reverse: x and dy arrive with negated token strides and
 // pointers at the last token; only the mask needs the index turned round here.
-template <typename T, bool MASKED, bool LAG1>
-__global__ __launch_bounds__(kBwdThreads) void ema_param_grad_kernel(const EmaGradArgs A) {
+// CH channels per workgroup (16, or 8 when 16 would leave compute units without a workgroup).
+template <typename T, bool MASKED, bool LAG1, int CH>
+__global__ __launch_bounds__(CH * kNs) void ema_param_grad_kernel(const EmaGradArgs A) {
+  constexpr int kCh = CH;
+  constexpr int kBwdThreads = CH * kNs;
   __shared__ float s_x[kCh][kTk + 4];
   __shared__ float s_g[kCh][kTk + 4];
   __shared__ float s_keep[kTk];
@@ -195,7 +196,7 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
   MEGA_REQUIRE(B >= 0 && D > 0 && N > 0 && L >= 0, MEGA_ERR_ARG, "ema_param_grad: bad shape B=%ld D=%ld N=%ld L=%ld",
                (long)B, (long)D, (long)N, (long)L);
   MEGA_REQUIRE(N <= kNs, MEGA_ERR_UNSUPPORTED, "ema_param_grad: ndim=%ld > %d is not supported", (long)N, kNs);
-  MEGA_REQUIRE(B * ceil_div(D, kCh) < (int64_t)1 << 31 && L < (int64_t)1 << 30 && D * N < (int64_t)1 << 31,
+  MEGA_REQUIRE(B * ceil_div(D, 8) < (int64_t)1 << 31 && L < (int64_t)1 << 30 && D * N < (int64_t)1 << 31,
                MEGA_ERR_UNSUPPORTED, "ema_param_grad: shape too large");
   MEGA_REQUIRE(p && q && gamma && dp && dq && dgamma && domega, MEGA_ERR_ARG, "ema_param_grad: null pointer argument");
   hipStream_t s = (hipStream_t)stream;
@@ -223,13 +224,32 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
   A.sums = (float*)workspace;
   A.dyx = (float*)((char*)workspace + align_up((size_t)B * D * N * 16, 256));
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
-  const dim3 grid((unsigned)(B * ceil_div(D, kCh)));
-#define LAUNCH_PG(T)                                                                                        \
-  do {                                                                                                      \
-    typedef void (*Kern)(const EmaGradArgs);                                                               \
-    static const Kern table[4] = {ema_param_grad_kernel<T, false, false>, ema_param_grad_kernel<T, false, true>, \
-                                  ema_param_grad_kernel<T, true, false>, ema_param_grad_kernel<T, true, true>};  \
-    hipLaunchKernelGGL(table[(mask ? 2 : 0) + (lag_one ? 1 : 0)], grid, dim3(kBwdThreads), 0, s, A);        \
+  // 16 channels per workgroup, 8 when that would leave compute units idle
+  static int cu_count[64] = {0};     // per device, queried once
+  int cus = 256;
+  {
+    int dev_id = 0;
+    if (hipGetDevice(&dev_id) == hipSuccess && dev_id >= 0 && dev_id < 64) {
+      if (cu_count[dev_id] == 0) {
+        int n = 0;
+        cu_count[dev_id] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev_id) == hipSuccess && n > 0) ? n : 256;
+      }
+      cus = cu_count[dev_id];
+    }
+  }
+  const bool narrow = B * ceil_div(D, 16) < cus;
+  const int ch = narrow ? 8 : 16;
+  const dim3 grid((unsigned)(B * ceil_div(D, ch)));
+#define LAUNCH_PG(T)                                                                                          \
+  do {                                                                                                        \
+    typedef void (*Kern)(const EmaGradArgs);                                                                 \
+    static const Kern table[8] = {                                                                            \
+        ema_param_grad_kernel<T, false, false, 16>, ema_param_grad_kernel<T, false, true, 16>,                \
+        ema_param_grad_kernel<T, true, false, 16>,  ema_param_grad_kernel<T, true, true, 16>,                 \
+        ema_param_grad_kernel<T, false, false, 8>,  ema_param_grad_kernel<T, false, true, 8>,                 \
+        ema_param_grad_kernel<T, true, false, 8>,   ema_param_grad_kernel<T, true, true, 8>};                 \
+    hipLaunchKernelGGL(table[(narrow ? 4 : 0) + (mask ? 2 : 0) + (lag_one ? 1 : 0)], grid, dim3(ch * kNs), 0, \
+                       s, A);                                                                                 \
   } while (0)
   switch (dtype) {
     case MEGA_F32: LAUNCH_PG(float); break;
