@@ -14,6 +14,8 @@
 // Per batch row the kernel leaves sums [B, D, N, 4] = (Re sum2, Im sum2, Re sum1, Im sum1) and
 // dyx [B, D] = sum_t dy x in the workspace; ema_grad_finalize_kernel adds the rows up in a fixed
 // order and forms dp, dq, dgamma and domega.
+#include <type_traits>
+
 #include "common.h"
 
 namespace mega {
@@ -21,7 +23,7 @@ namespace {
 
 constexpr int kNs = 16;        // state lanes per channel
 constexpr int kTk = 128;       // tokens per LDS tile
-constexpr int kPerThread = kTk / kNs;   // elements of one tile a thread moves (CH * kTk / (CH * kNs))
+
 
 struct EmaGradArgs {
   const void* dy;
@@ -40,10 +42,15 @@ struct EmaGradArgs {
 // half of a two-sided layer with shift).  A.reverse: x and dy arrive with negated token strides and
 // pointers at the last token; only the mask needs the index turned round here.
 // CH channels per workgroup (16, or 8 when 16 would leave compute units without a workgroup).
-template <typename T, bool MASKED, bool LAG1, int CH>
-__global__ __launch_bounds__(CH * kNs) void ema_param_grad_kernel(const EmaGradArgs A) {
+// ROLES = 2: a second set of CH * 16 threads shares the tiles; the first set runs s and the sum2
+// pair, the second s, g and the sum1 pair.  That is 17 instead of 13 multiply-adds per token and
+// state, but two waves per SIMD issue about 1.6 times faster than one wave alone, so it pays
+// whenever the grid would otherwise leave every SIMD with a single wave.
+template <typename T, bool MASKED, bool LAG1, int CH, int ROLES>
+__global__ __launch_bounds__(CH * kNs * ROLES) void ema_param_grad_kernel(const EmaGradArgs A) {
   constexpr int kCh = CH;
-  constexpr int kBwdThreads = CH * kNs;
+  constexpr int kBwdThreads = CH * kNs * ROLES;
+  constexpr int kPerThread = kTk / kNs / ROLES;   // elements of one tile a thread moves
   __shared__ float s_x[kCh][kTk + 4];
   __shared__ float s_g[kCh][kTk + 4];
   __shared__ float s_keep[kTk];
@@ -51,7 +58,8 @@ __global__ __launch_bounds__(CH * kNs) void ema_param_grad_kernel(const EmaGradA
   const int ncb = (A.D + kCh - 1) / kCh;
   const int b = blockIdx.x / ncb;
   const int c0 = (blockIdx.x - b * ncb) * kCh;
-  const int ch = tid / kNs, n = tid % kNs;
+  const int role = tid / (CH * kNs);             // wave-uniform
+  const int ch = (tid % (CH * kNs)) / kNs, n = tid % kNs;
   const bool state_lane = n < A.N && c0 + ch < A.D;
   const T* xg = (const T*)A.x + b * A.sxb;
   const T* gg = (const T*)A.dy + b * A.sgb;
@@ -112,41 +120,51 @@ __global__ __launch_bounds__(CH * kNs) void ema_param_grad_kernel(const EmaGradA
     }
     __syncthreads();
     fetch(t0 + kTk);    // the next tile (clamped past the end) is in flight while this one is worked through
+    auto work = [&](auto do_a2, auto do_g) {
+      constexpr bool A2 = decltype(do_a2)::value, G = decltype(do_g)::value;
 #pragma unroll 4
-    for (int t = 0; t < kTk; t += 4) {
-      const float4 xv = *(const float4*)&s_x[ch][t];
-      const float4 gv = *(const float4*)&s_g[ch][t];
-      float4 kv = make_float4(1.f, 1.f, 1.f, 1.f);
-      if (MASKED) kv = *(const float4*)&s_keep[t];
-      const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ds[4] = {gv.x, gv.y, gv.z, gv.w}, ks[4] = {kv.x, kv.y, kv.z, kv.w};
+      for (int t = 0; t < kTk; t += 4) {
+        const float4 xv = *(const float4*)&s_x[ch][t];
+        const float4 gv = *(const float4*)&s_g[ch][t];
+        float4 kv = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (MASKED) kv = *(const float4*)&s_keep[t];
+        const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, ds[4] = {gv.x, gv.y, gv.z, gv.w}, ks[4] = {kv.x, kv.y, kv.z, kv.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // g[t] = q g[t-1] + s[t-1];  s[t] = q s[t-1] + x[t] (masked tokens enter as zero)
-        const float ngr = fmaf(qr, gr, fmaf(-qi, gi, sr));
-        const float ngi = fmaf(qr, gi, fmaf(qi, gr, si));
-        const float nsr = fmaf(qr, sr, fmaf(-qi, si, MASKED ? xs[j] * ks[j] : xs[j]));
-        const float nsi = fmaf(qr, si, qi * sr);
-        if (LAG1) {
-          a2r = fmaf(ds[j], sr, a2r);
-          a2i = fmaf(ds[j], si, a2i);
-          a1r = fmaf(ds[j], gr, a1r);
-          a1i = fmaf(ds[j], gi, a1i);
+        for (int j = 0; j < 4; ++j) {
+          // g[t] = q g[t-1] + s[t-1];  s[t] = q s[t-1] + x[t] (masked tokens enter as zero)
+          float ngr = 0.f, ngi = 0.f;
+          if (G) {
+            ngr = fmaf(qr, gr, fmaf(-qi, gi, sr));
+            ngi = fmaf(qr, gi, fmaf(qi, gr, si));
+          }
+          const float nsr = fmaf(qr, sr, fmaf(-qi, si, MASKED ? xs[j] * ks[j] : xs[j]));
+          const float nsi = fmaf(qr, si, qi * sr);
+          if (LAG1) {
+            if (A2) { a2r = fmaf(ds[j], sr, a2r); a2i = fmaf(ds[j], si, a2i); }
+            if (G) { a1r = fmaf(ds[j], gr, a1r); a1i = fmaf(ds[j], gi, a1i); }
+          }
+          gr = ngr; gi = ngi; sr = nsr; si = nsi;
+          if (!LAG1) {
+            if (A2) { a2r = fmaf(ds[j], sr, a2r); a2i = fmaf(ds[j], si, a2i); }
+            if (G) { a1r = fmaf(ds[j], gr, a1r); a1i = fmaf(ds[j], gi, a1i); }
+          }
+          if (A2) ax = fmaf(ds[j], xs[j], ax);
         }
-        gr = ngr; gi = ngi; sr = nsr; si = nsi;
-        if (!LAG1) {
-          a2r = fmaf(ds[j], sr, a2r);
-          a2i = fmaf(ds[j], si, a2i);
-          a1r = fmaf(ds[j], gr, a1r);
-          a1i = fmaf(ds[j], gi, a1i);
-        }
-        ax = fmaf(ds[j], xs[j], ax);
       }
-    }
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+    if (ROLES == 1) work(Yes{}, Yes{});
+    else if (role == 0) work(Yes{}, No{});
+    else work(No{}, Yes{});
   }
   if (state_lane) {
-    float4* dst = (float4*)A.sums + ((size_t)b * A.D + c0 + ch) * A.N + n;
-    *dst = make_float4(a2r, a2i, a1r, a1i);
-    if (n == 0) A.dyx[(size_t)b * A.D + c0 + ch] = ax;
+    float2* dst = (float2*)A.sums + (((size_t)b * A.D + c0 + ch) * A.N + n) * 2;
+    if (ROLES == 1 || role == 0) {
+      dst[0] = make_float2(a2r, a2i);
+      if (n == 0) A.dyx[(size_t)b * A.D + c0 + ch] = ax;
+    }
+    if (ROLES == 1 || role == 1) dst[1] = make_float2(a1r, a1i);
   }
 }
 
@@ -237,19 +255,26 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
       cus = cu_count[dev_id];
     }
   }
+  // one role set per workgroup only when the grid fills every SIMD with several waves anyway
   const bool narrow = B * ceil_div(D, 16) < cus;
   const int ch = narrow ? 8 : 16;
-  const dim3 grid((unsigned)(B * ceil_div(D, ch)));
+  const int64_t wgs = B * ceil_div(D, ch);
+  const bool split = wgs * (ch * kNs / 64) <= (int64_t)cus * 4;     // at most one wave per SIMD without it
+  const dim3 grid((unsigned)wgs);
 #define LAUNCH_PG(T)                                                                                          \
   do {                                                                                                        \
     typedef void (*Kern)(const EmaGradArgs);                                                                 \
-    static const Kern table[8] = {                                                                            \
-        ema_param_grad_kernel<T, false, false, 16>, ema_param_grad_kernel<T, false, true, 16>,                \
-        ema_param_grad_kernel<T, true, false, 16>,  ema_param_grad_kernel<T, true, true, 16>,                 \
-        ema_param_grad_kernel<T, false, false, 8>,  ema_param_grad_kernel<T, false, true, 8>,                 \
-        ema_param_grad_kernel<T, true, false, 8>,   ema_param_grad_kernel<T, true, true, 8>};                 \
-    hipLaunchKernelGGL(table[(narrow ? 4 : 0) + (mask ? 2 : 0) + (lag_one ? 1 : 0)], grid, dim3(ch * kNs), 0, \
-                       s, A);                                                                                 \
+    static const Kern table[16] = {                                                                           \
+        ema_param_grad_kernel<T, false, false, 16, 1>, ema_param_grad_kernel<T, false, true, 16, 1>,          \
+        ema_param_grad_kernel<T, true, false, 16, 1>,  ema_param_grad_kernel<T, true, true, 16, 1>,           \
+        ema_param_grad_kernel<T, false, false, 8, 1>,  ema_param_grad_kernel<T, false, true, 8, 1>,           \
+        ema_param_grad_kernel<T, true, false, 8, 1>,   ema_param_grad_kernel<T, true, true, 8, 1>,            \
+        ema_param_grad_kernel<T, false, false, 16, 2>, ema_param_grad_kernel<T, false, true, 16, 2>,          \
+        ema_param_grad_kernel<T, true, false, 16, 2>,  ema_param_grad_kernel<T, true, true, 16, 2>,           \
+        ema_param_grad_kernel<T, false, false, 8, 2>,  ema_param_grad_kernel<T, false, true, 8, 2>,           \
+        ema_param_grad_kernel<T, true, false, 8, 2>,   ema_param_grad_kernel<T, true, true, 8, 2>};           \
+    hipLaunchKernelGGL(table[(split ? 8 : 0) + (narrow ? 4 : 0) + (mask ? 2 : 0) + (lag_one ? 1 : 0)], grid,  \
+                       dim3(ch * kNs * (split ? 2 : 1)), 0, s, A);                                            \
   } while (0)
   switch (dtype) {
     case MEGA_F32: LAUNCH_PG(float); break;
