@@ -14,14 +14,20 @@ from .modules import (  # noqa: F401
 
 from .layers import (  # noqa: F401,E402
     Mega2Layer,
+    MegaDecoderLayer,
+    MegaEncoderLayer,
     MovingAverageGatedAttention,
     NormalizedFeedForwardNetwork,
     RMSNorm,
     RotaryEmbedding,
+    streamed_forward,
 )
 
 __all__ = [
     "Mega2Layer",
+    "MegaDecoderLayer",
+    "MegaEncoderLayer",
+    "streamed_forward",
     "MovingAverageGatedAttention",
     "NormalizedFeedForwardNetwork",
     "RMSNorm",

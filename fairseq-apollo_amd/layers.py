@@ -342,3 +342,95 @@ class Mega2Layer(nn.Module):
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, incremental_state=None) -> Tensor:
         x, _ = self.attn(x, padding_mask, incremental_state)
         return x + self.ffn(self.ffn_norm(x, padding_mask, incremental_state))
+
+
+def _arg(args, name, default):
+    return getattr(args, name, default)
+
+
+class MegaDecoderLayer(nn.Module):
+    """fairseq/modules/mega_layer.py:81-202 without the cross attention (a language-model layer):
+    `mega_layer` (causal MovingAverageGatedAttention) followed by `nffn`
+    (NormalizedFeedForwardNetwork) when args.decoder_ffn_embed_dim > 0.  `args` is the reference's
+    namespace (fairseq/models/mega_lm.py:51-121); submodule names, and therefore state-dict keys,
+    are the reference's."""
+
+    def __init__(self, args, no_cross_attention: bool = True, layer_scale: Optional[float] = None):
+        super().__init__()
+        if not no_cross_attention:
+            raise NotImplementedError("MegaDecoderLayer: the gated cross attention is not built")
+        self.embed_dim = args.decoder_embed_dim
+        trunc = _arg(args, 'truncation_length', 0)
+        self.mega_layer = MovingAverageGatedAttention(
+            self.embed_dim, args.decoder_z_dim, args.decoder_hidden_dim, args.decoder_n_dim,
+            chunk_size=_arg(args, 'decoder_chunk_size', -1), moving_layer=_arg(args, 'moving_layer', 'cema'),
+            moving_act=_arg(args, 'moving_act', 'rmsnorm'), norm_num_groups=_arg(args, 'norm_num_groups', None),
+            norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
+            max_positions=_arg(args, 'max_target_positions', 1024), num_heads=_arg(args, 'num_heads', 1),
+            efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
+            bidirectional=False, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
+            truncation=trunc if trunc and trunc > 0 else None)
+        self.cross_attn = None
+        if _arg(args, 'decoder_ffn_embed_dim', 0) > 0:
+            self.nffn = NormalizedFeedForwardNetwork(
+                self.embed_dim, args.decoder_ffn_embed_dim, norm_type=_arg(args, 'norm_type', 'layernorm'),
+                norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
+                layer_scale=layer_scale, init_mode=_arg(args, 'init_mode', 'bert'))
+        else:
+            self.nffn = None
+
+    def forward(self, x: Tensor, encoder_out=None, encoder_padding_mask=None, incremental_state=None, attn_mask=None,
+                decoder_padding_mask: Optional[Tensor] = None, need_attn: bool = False):
+        """x: [B, L, D] -> (x, None, None), the reference's return triple."""
+        x, attn = self.mega_layer(x, decoder_padding_mask, incremental_state)
+        if self.nffn is not None:
+            x = self.nffn(x)
+        return x, attn, None
+
+
+class MegaEncoderLayer(nn.Module):
+    """fairseq/modules/mega_layer.py:11-78: bidirectional `mega_layer` followed by `nffn`."""
+
+    def __init__(self, args, layer_scale: Optional[float] = None):
+        super().__init__()
+        self.embed_dim = args.encoder_embed_dim
+        trunc = _arg(args, 'truncation_length', 0)
+        self.mega_layer = MovingAverageGatedAttention(
+            self.embed_dim, args.encoder_z_dim, args.encoder_hidden_dim, args.encoder_n_dim,
+            chunk_size=_arg(args, 'encoder_chunk_size', -1), moving_layer=_arg(args, 'moving_layer', 'cema'),
+            moving_act=_arg(args, 'moving_act', 'rmsnorm'), norm_num_groups=_arg(args, 'norm_num_groups', None),
+            norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
+            max_positions=_arg(args, 'max_source_positions', 1024), num_heads=_arg(args, 'num_heads', 1),
+            efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
+            bidirectional=True, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
+            truncation=trunc if trunc and trunc > 0 else None)
+        if _arg(args, 'encoder_ffn_embed_dim', 0) > 0:
+            self.nffn = NormalizedFeedForwardNetwork(
+                self.embed_dim, args.encoder_ffn_embed_dim, norm_type=_arg(args, 'norm_type', 'layernorm'),
+                norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
+                layer_scale=layer_scale, init_mode=_arg(args, 'init_mode', 'bert'))
+        else:
+            self.nffn = None
+
+    def forward(self, x: Tensor, encoder_padding_mask: Optional[Tensor] = None) -> Tensor:
+        x, _ = self.mega_layer(x, encoder_padding_mask)
+        if self.nffn is not None:
+            x = self.nffn(x)
+        return x
+
+
+def streamed_forward(layers, x: Tensor, chunk_size: int, padding_mask: Optional[Tensor] = None) -> Tensor:
+    """Run a stack of decoder layers over x [B, L, D] chunk by chunk with carried state, the way the
+    reference's validation streams documents (fairseq_cli/train.py:406-417: one incremental-state
+    dictionary per document, consecutive slices of `chunk_size` tokens).  Equals the one-shot result
+    for causal layers."""
+    incremental_states: Dict[str, Dict[str, Optional[Tensor]]] = {}
+    outs = []
+    for a in range(0, x.size(1), chunk_size):
+        h = x[:, a:a + chunk_size]
+        pm = None if padding_mask is None else padding_mask[:, a:a + chunk_size]
+        for layer in layers:
+            out = layer(h, incremental_state=incremental_states, decoder_padding_mask=pm)
+            h = out[0] if isinstance(out, tuple) else out
+        outs.append(h)
+    return torch.cat(outs, dim=1)

@@ -164,3 +164,60 @@ def test_bidirectional_gated_attention_layer(dtype, tol, heads, act, moving, mas
         e = got - ref
         rms = np.sqrt((ref ** 2).mean())
         assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
+
+
+def _lm_args(**kw):
+    import types
+    base = dict(decoder_embed_dim=64, decoder_z_dim=32, decoder_hidden_dim=128, decoder_n_dim=16,
+                decoder_chunk_size=128, decoder_ffn_embed_dim=160, norm_num_groups=8, norm_type='rmsnorm',
+                moving_layer='cema', moving_act='rmsnorm', efficient_attention=True, rel_pos_bias='rotary')
+    base.update(kw)
+    return types.SimpleNamespace(**base)
+
+
+def test_decoder_stack_streams_like_the_reference_validation():
+    """Three MegaDecoderLayers: a document streamed in chunk-sized slices with one incremental-state
+    dictionary equals the one-shot forward (fp32: the recurrences agree to ~1e-5), also when the
+    slices are half chunks."""
+    torch.manual_seed(21)
+    args = _lm_args()
+    layers = torch.nn.ModuleList([M.MegaDecoderLayer(args) for _ in range(3)]).to(DEV).eval()
+    with torch.no_grad():
+        for lyr in layers:
+            for prm in (lyr.mega_layer.v_proj.weight, lyr.mega_layer.mx_proj.weight, lyr.mega_layer.h_proj.weight,
+                        lyr.nffn.fc1.weight, lyr.nffn.fc2.weight):
+                prm.normal_(0, 0.1)
+    x = torch.randn(2, 512, 64, device=DEV)
+    with torch.no_grad():
+        full = x
+        for lyr in layers:
+            full = lyr(full)[0]
+        streamed = M.streamed_forward(layers, x, 128)
+        halves = M.streamed_forward(layers, x, 64)
+    assert rel_err(host(streamed), host(full)) < 5e-5
+    assert rel_err(host(halves), host(full)) < 5e-5
+    assert M.ops.timestep_norm_status() == 0
+
+
+def test_decoder_and_encoder_layer_names_and_training():
+    args = _lm_args()
+    dec = M.MegaDecoderLayer(args).to(DEV).train()
+    keys = set(dec.state_dict())
+    assert {"mega_layer.norm.weight", "mega_layer.move.alpha", "mega_layer.mx_proj.weight", "mega_layer.gamma",
+            "mega_layer.move_act.weight", "mega_layer.rel_pos_bias.freqs", "nffn.norm.weight", "nffn.fc1.weight",
+            "nffn.fc1.bias", "nffn.fc2.weight"} <= keys
+    x = torch.randn(2, 256, 64, device=DEV, requires_grad=True)
+    dec(x)[0].square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in dec.parameters())
+    import types
+    eargs = types.SimpleNamespace(encoder_embed_dim=64, encoder_z_dim=32, encoder_hidden_dim=128, encoder_n_dim=16,
+                                  encoder_chunk_size=128, encoder_ffn_embed_dim=160, norm_num_groups=8,
+                                  norm_type='layernorm', moving_act='silu')
+    enc = M.MegaEncoderLayer(eargs).to(DEV).train()
+    assert isinstance(enc.mega_layer.norm, M.SequenceNorm) and enc.mega_layer.move.bidirectional
+    mask = torch.zeros(2, 256, dtype=torch.bool, device=DEV)
+    mask[1, 200:] = True
+    xe = torch.randn(2, 256, 64, device=DEV, requires_grad=True)
+    (enc(xe, mask) * (~mask)[..., None]).square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in enc.parameters())
+    assert torch.isfinite(xe.grad).all()
