@@ -137,6 +137,26 @@ class RotaryEmbedding(nn.Module):
         return self.rotary(xq, qidx), self.rotary(xk, 0)
 
 
+class SimpleRelativePositionalBias(nn.Module):
+    """fairseq/modules/relative_positional_bias.py:13-45: one learned bias per relative offset;
+    forward(L) is the L x L Toeplitz matrix with entry (i, j) = rel_pos_bias[max_positions - 1 + j - i]."""
+
+    def __init__(self, max_positions: int):
+        super().__init__()
+        self.max_positions = max_positions
+        self.rel_pos_bias = Parameter(torch.Tensor(2 * max_positions - 1))
+        nn.init.normal_(self.rel_pos_bias, mean=0, std=0.02)
+
+    def forward(self, seq_len: int) -> Tensor:
+        if seq_len > self.max_positions:
+            raise ValueError('Sequence length {} going beyond max length {}'.format(seq_len, self.max_positions))
+        pos = torch.arange(seq_len, device=self.rel_pos_bias.device)
+        return self.rel_pos_bias[(self.max_positions - 1) + pos[None, :] - pos[:, None]]
+
+    def extra_repr(self) -> str:
+        return 'max positions={}'.format(self.max_positions)
+
+
 class MovingAverageGatedAttention(nn.Module, IncrementalState):
     """Gated attention with a moving-average pre-mixer.  Constructor arguments follow the
     reference (moving_average_gated_attention.py:31-53) for the supported subset; `num_heads`
@@ -149,8 +169,10 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
                  truncation=None):
         super().__init__()
         self.init_incremental_state()
-        if not efficient_attn or rel_pos_bias != 'rotary' or attention_activation != 'softmax':
-            raise NotImplementedError("only the rotary softmax attention through the fused ops is built")
+        if attention_activation != 'softmax':
+            raise NotImplementedError("only the softmax attention is built (no relu2 / laplace)")
+        if rel_pos_bias not in ('rotary', 'simple'):
+            raise ValueError('unknown relative position bias: {}'.format(rel_pos_bias))
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
         self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
         self.chunk_size = chunk_size
@@ -159,7 +181,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         # causal layers: the fused causal op; bidirectional layers (moving_average_gated_attention.py:70-75,
         # 84-92): full softmax over every chunk, SequenceNorm, a two-sided moving average
         self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=not bidirectional, scale=1.0)
-        self.attn_softmax = AttentionSoftmax(dropout=0.0, use_causal_mask=False) if bidirectional else None
+        self.attn_softmax = AttentionSoftmax(dropout=0.0, use_causal_mask=not bidirectional)
         if bidirectional:
             self.norm = SequenceNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
         else:
@@ -178,7 +200,12 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         self.gamma = Parameter(torch.zeros(2, zdim))
         self.beta = Parameter(torch.zeros(2, zdim))
         self.max_positions = max_positions if chunk_size < 0 else chunk_size
-        self.rel_pos_bias = RotaryEmbedding(zdim // num_heads, self.max_positions)
+        if rel_pos_bias == 'rotary':
+            self.rel_pos_bias = RotaryEmbedding(zdim // num_heads, self.max_positions)
+        else:
+            # moving_average_gated_attention.py:109-110, 212-219: scores = q k^T + bias[j - i], no rotation
+            self.rel_pos_bias = SimpleRelativePositionalBias(self.max_positions)
+            self.register_buffer("_no_rotation", torch.zeros(zdim // num_heads // 2), persistent=False)
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -214,10 +241,13 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             # affine maps, rotary with positions restarting in every chunk)
             C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
             nc = seq_len // C
-            q, k = ops.gate_qk_fwd(z, self.gamma + 1.0, self.beta, self.rel_pos_bias.freqs, Nh, C)
+            simple = isinstance(self.rel_pos_bias, SimpleRelativePositionalBias)
+            freqs = self._no_rotation if simple else self.rel_pos_bias.freqs      # zero angles: no rotation
+            q, k = ops.gate_qk_fwd(z, self.gamma + 1.0, self.beta, freqs, Nh, C)
             q4, k4, v4 = q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1), v.reshape(bsz * nc, C, Nh, -1)
-            if self.bidirectional and padding_mask is not None:
-                attn = self._padded_attention(q4, k4, v4, padding_mask.reshape(bsz * nc, C))
+            if simple or (self.bidirectional and padding_mask is not None):
+                attn = self._padded_attention(q4, k4, v4, None if padding_mask is None or not self.bidirectional
+                                              else padding_mask.reshape(bsz * nc, C))
             else:
                 attn = self.efficient_attn(q4, k4, v4)
         else:
@@ -228,14 +258,18 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         return ops.gate_out_fwd(residual, u, hx, hp), None
 
     def _padded_attention(self, q4: Tensor, k4: Tensor, v4: Tensor, key_padding: Tensor) -> Tensor:
-        """Full softmax over a chunk with padded keys excluded
-        (moving_average_gated_attention.py:232-248): scores of padded keys are -inf except in chunks
-        that consist of padding only; library GEMMs around the softmax op."""
-        pad = key_padding.to(torch.bool)
-        pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
+        """Softmax attention outside the fused op (moving_average_gated_attention.py:210-256): the
+        learned relative bias is added to the scores, scores of padded keys are -inf except in chunks
+        that consist of padding only; library GEMMs around the softmax op (causal for one-sided
+        layers)."""
         s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
-        s = s.masked_fill(pad[:, None, None, :], float('-inf'))
-        w = ops.attention_softmax_fwd(s, 0.0, False)
+        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias):
+            s = s + self.rel_pos_bias(q4.size(1)).to(s.dtype)
+        if key_padding is not None:
+            pad = key_padding.to(torch.bool)
+            pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
+            s = s.masked_fill(pad[:, None, None, :], float('-inf'))
+        w = ops.attention_softmax_fwd(s, 0.0, not self.bidirectional)
         return torch.einsum('bnqk,bknh->bqnh', w, v4)
 
     def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
@@ -264,12 +298,18 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         q4 = q.reshape(bsz * nc, C, Nh, -1)
         k4 = k.reshape(bsz * nc, C, Nh, -1)
         v4 = v.reshape(bsz * nc, C, Nh, -1)
-        q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
-        k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
-        if self.bidirectional and padding_mask is not None:
-            pad = padding_mask.reshape(bsz * nc, C).to(torch.bool)
-            pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
-            s = torch.einsum('bqnh,bknh->bnqk', q4, k4).masked_fill(pad[:, None, None, :], float('-inf'))
+        simple = isinstance(self.rel_pos_bias, SimpleRelativePositionalBias)
+        if not simple:
+            q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
+            k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+        if simple or (self.bidirectional and padding_mask is not None):
+            s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
+            if simple:
+                s = s + self.rel_pos_bias(C).to(s.dtype)
+            if self.bidirectional and padding_mask is not None:
+                pad = padding_mask.reshape(bsz * nc, C).to(torch.bool)
+                pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
+                s = s.masked_fill(pad[:, None, None, :], float('-inf'))
             attn = torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
         else:
             attn = self.efficient_attn(q4, k4, v4)
@@ -280,6 +320,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         """Attention with the partial-chunk key / value cache
         (moving_average_gated_attention.py:332-372): keys are cached before the rotation, so the
         whole context is rotated again at every call."""
+        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias):
+            raise NotImplementedError("MovingAverageGatedAttention: incremental decoding is built for the rotary "
+                                      "position encoding only")
         bsz, seq_len = z.shape[:2]
         Nh = self.num_heads
         z = F.normalize(z, p=2, dim=-1, eps=1e-5)

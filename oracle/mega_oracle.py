@@ -652,7 +652,8 @@ def rms_norm(x, weight=None, eps: float = 1e-5):
 
 
 def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str = 'silu', eps: float = 1e-5,
-                          num_groups: Optional[int] = None, bidirectional: bool = False, padding_mask=None):
+                          num_groups: Optional[int] = None, bidirectional: bool = False, padding_mask=None,
+                          simple_bias=None):
     """MovingAverageGatedAttention.forward, unidirectional, softmax attention through the fused
     (rotary, causal, scale 1) op: modules/moving_average_gated_attention.py:263-417, step by
     step.  x: [B, L, D]; P: dict of numpy parameters
@@ -693,17 +694,27 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     qc = q.reshape(B * nc, C, num_heads, H1)
     kc = k.reshape(B * nc, C, num_heads, H1)
     vc = v.reshape(B * nc, C, num_heads, H2)
-    # rotary on every head's features, positions restart in every chunk
-    qr = rotary(qc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
-    kr = rotary(kc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
-    if bidirectional:
-        # full softmax per chunk; padded keys excluded unless the whole chunk is padding (:232-248)
+    if simple_bias is None:
+        # rotary on every head's features, positions restart in every chunk
+        qr = rotary(qc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
+        kr = rotary(kc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
+    else:
+        qr, kr = qc, kc
+    if bidirectional or simple_bias is not None:
+        # softmax outside the fused op (:210-256): learned bias per relative offset j - i
+        # (relative_positional_bias.py:25-42; simple_bias has 2 * max_positions - 1 entries), padded keys
+        # excluded unless the whole chunk is padding, causal for one-sided layers
         sc = np.einsum('blnh,bmnh->bnlm', qr, kr)
-        if padding_mask is not None:
+        if simple_bias is not None:
+            sb = np.asarray(simple_bias, np.float64)
+            mp = (sb.shape[0] + 1) // 2
+            pos = np.arange(C)
+            sc = sc + sb[(mp - 1) + pos[None, :] - pos[:, None]]
+        if bidirectional and padding_mask is not None:
             pad = np.asarray(padding_mask, bool).reshape(B * nc, C)
             pad = pad & ~pad.all(-1, keepdims=True)
             sc = np.where(pad[:, None, None, :], -np.inf, sc)
-        a = np.einsum('bnlm,bmnh->blnh', attention_softmax(sc, False), vc)
+        a = np.einsum('bnlm,bmnh->blnh', attention_softmax(sc, not bidirectional), vc)
     else:
         a, _ = attention(qr, kr, vc, 1.0, True)
     a = a.reshape(B, L, E)

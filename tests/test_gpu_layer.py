@@ -221,3 +221,40 @@ def test_decoder_and_encoder_layer_names_and_training():
     (enc(xe, mask) * (~mask)[..., None]).square().mean().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in enc.parameters())
     assert torch.isfinite(xe.grad).all()
+
+
+@pytest.mark.parametrize("bidir", [False, True])
+def test_simple_relative_bias_layer(bidir):
+    """rel_pos_bias='simple' (moving_average_gated_attention.py:109-110): scores = q k^T + bias[j - i],
+    no rotation; forward against the layer oracle and a training step against central differences
+    of the bias parameter."""
+    torch.manual_seed(31)
+    B, L, D, S, E, N, C = 2, 128, 32, 16, 48, 8, 64
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act='silu', norm_num_groups=4,
+                                          rel_pos_bias='simple', bidirectional=bidir).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.2)
+        layer.gamma.normal_(0, 0.3); layer.beta.normal_(0, 0.3)
+        layer.rel_pos_bias.rel_pos_bias.normal_(0, 0.5)
+    P = _params(layer)
+    sb = host(layer.rel_pos_bias.rel_pos_bias)
+    assert sb.shape == (2 * C - 1,)
+    x = torch.randn(B, L, D, device=DEV)
+    okw = dict(chunk=C, num_heads=1, moving_act='silu', num_groups=4, bidirectional=bidir)
+    with torch.no_grad():
+        y, _ = layer(x)
+    assert rel_err(host(y), O.gated_attention_layer(host(x), P, simple_bias=sb, **okw)) < 2e-4
+    w = torch.randn(B, L, D, device=DEV)
+    layer.train()
+    out, _ = layer(x)
+    (out * w).sum().backward()
+    g = host(layer.rel_pos_bias.rel_pos_bias.grad)
+    rng = np.random.default_rng(3)
+    for _ in range(4):
+        i = int(rng.integers(C - 20, C + 19))              # offsets that occur often
+        sp, sm = sb.copy(), sb.copy()
+        sp[i] += 1e-5; sm[i] -= 1e-5
+        fd = ((O.gated_attention_layer(host(x), P, simple_bias=sp, **okw) * host(w)).sum()
+              - (O.gated_attention_layer(host(x), P, simple_bias=sm, **okw) * host(w)).sum()) / 2e-5
+        assert abs(fd - g[i]) < 3e-3 * (np.abs(g).max() + 1e-6), (i, fd, g[i])
