@@ -461,3 +461,47 @@ def test_gate_backwards(dtype, shape, width, off):
     ga, gb = M.ops.swiglu_bwd(dy, a, b)
     assert rel_err(host(ga), dy64 * b64 * dsilu(a64)) < TOL[dtype]
     assert rel_err(host(gb), dy64 * O._silu(a64)) < TOL[dtype]
+
+
+def test_backward_edge_shapes():
+    """Single-token and single-row inputs, channel counts that are not multiples of the tile sizes."""
+    rng = np.random.default_rng(99)
+    # TimestepNorm backward, one token
+    x, x64 = rounded(rng.normal(size=(1, 1, 8)), torch.float32)
+    dy, dy64 = rounded(rng.normal(size=(1, 1, 8)), torch.float32)
+    gamma, beta = np.ones(8), np.zeros(8)
+    pc, pm, pv = np.array([2], np.int64), rng.normal(size=(1, 2)) * 0.1, np.ones((1, 2))
+    y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma),
+                                                                dev(beta), None, 2, 1e-5)
+    got = M.ops.group_timestep_norm_bwd(dy, None, None, x, dev(pm), cnt, gm, cm, cr, dev(gamma), None, 2)
+    ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm.astype(np.float32).astype(np.float64), pv, None, 2, 1e-5)
+    ref = O.timestep_norm_bwd(dy64, None, None, x64, pm.astype(np.float32).astype(np.float64), ocnt, ogm, ocm, ocr,
+                              gamma, None, 2)
+    for a, b in zip(got, ref):
+        assert rel_err(host(a), b) < 2e-4
+    # moving-average backward: one token, then a tile boundary plus one, 5 channels, 3 states
+    for L in (1, 129):
+        p, q, g = _ema_coeffs(rng, 5, 3, True)
+        p, q, g = p.astype(np.float32).astype(np.float64), q.astype(np.complex64).astype(np.complex128), \
+            g.astype(np.complex64).astype(np.complex128)
+        om = rng.normal(size=5).astype(np.float32).astype(np.float64)
+        x, x64 = rounded(rng.normal(size=(2, 5, L)), torch.float32)
+        dy, dy64 = rounded(rng.normal(size=(2, 5, L)), torch.float32)
+        got = M.ops.ema_backward(dy, x, dev(p), dev(q), dev(g), dev(om))
+        ref = O.ema_backward(dy64, x64, p, q, g, om)
+        assert rel_err(host(got[0]), ref[0]) < 1e-4
+        for a, b in zip(got[1:], ref[1:]):
+            a = host(a)
+            assert rel_err(np.real(a), np.real(b)) < 5e-4 and rel_err(np.imag(a), np.imag(b)) < 5e-4
+    # SequenceNorm forward + backward, one token per row
+    x, x64 = rounded(rng.normal(size=(2, 6, 1)), torch.float32)
+    dy, dy64 = rounded(rng.normal(size=(2, 6, 1)), torch.float32)
+    gam = rng.normal(size=6) + 1
+    y, n, mu, r = M.ops.group_sequence_norm_fwd(x, dev(gam), dev(np.zeros(6)), None, 2, 1e-5, True)
+    assert rel_err(host(y), O.sequence_norm(x64, gam.astype(np.float32), np.zeros(6), None, 2, 1e-5, True)[0]) < 1e-4
+    dx, dg, db = M.ops.group_sequence_norm_bwd(dy, x, n, mu, r, dev(gam), None, 2, True)
+    rx, rg, rb = O.sequence_norm_bwd(dy64, x64, gam.astype(np.float32).astype(np.float64), None, 2, 1e-5, True)
+    assert rel_err(host(dx), rx) < 1e-4 and rel_err(host(dg), rg) < 2e-4 and rel_err(host(db), rb) < 2e-4
+    # softmax backward on a single column
+    yv = M.ops.attention_softmax_fwd(dev(rng.normal(size=(3, 1, 1))), 0.0, True)
+    assert float(M.ops.attention_softmax_bwd(dev(rng.normal(size=(3, 1, 1))), yv, True).abs().max()) < 1e-6
