@@ -393,7 +393,7 @@ bool seq_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, int len
   g->lpg = lpg;
   g->per = (int)(vecs / lpg);
   int tt = (int)(kMaxCells / G);
-  if (tt > 32) tt = 32;
+  if (tt > 16) tt = 16;
   if (tt < 1) tt = 1;
   g->tt = tt;
   g->nt = (int)ceil_div(L, tt);
