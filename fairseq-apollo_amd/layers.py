@@ -175,6 +175,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             raise ValueError('unknown relative position bias: {}'.format(rel_pos_bias))
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
         self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
+        self._qk_cache = None
         self.chunk_size = chunk_size
         self.num_heads = num_heads
         self.bidirectional = bidirectional
@@ -242,8 +243,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
             nc = seq_len // C
             simple = isinstance(self.rel_pos_bias, SimpleRelativePositionalBias)
-            freqs = self._no_rotation if simple else self.rel_pos_bias.freqs      # zero angles: no rotation
-            q, k = ops.gate_qk_fwd(z, self.gamma + 1.0, self.beta, freqs, Nh, C)
+            qk_gamma, qk_beta, freqs = self._qk_constants(simple)
+            q, k = ops.gate_qk_fwd(z, qk_gamma, qk_beta, freqs, Nh, C)
             q4, k4, v4 = q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1), v.reshape(bsz * nc, C, Nh, -1)
             if simple or (self.bidirectional and padding_mask is not None):
                 attn = self._padded_attention(q4, k4, v4, None if padding_mask is None or not self.bidirectional
@@ -256,6 +257,25 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         # projection, u and the residual mix after it
         hp = self.h_proj(ops.gate_mul_fwd(attn.reshape(bsz, seq_len, self.hdim), r))
         return ops.gate_out_fwd(residual, u, hx, hp), None
+
+    def _qk_constants(self, simple: bool):
+        """(gamma + 1, beta, rotation frequencies) in fp32 for the q / k kernel; kept in eval mode
+        (dropped by train() and by .to() / .half())."""
+        if not self.training and self._qk_cache is not None:
+            return self._qk_cache
+        with torch.no_grad():
+            freqs = self._no_rotation if simple else self.rel_pos_bias.freqs      # zero angles: no rotation
+            c = ((self.gamma.float() + 1.0).contiguous(), self.beta.float().contiguous(), freqs.float().contiguous())
+        self._qk_cache = None if self.training else c
+        return c
+
+    def train(self, mode: bool = True):
+        self._qk_cache = None
+        return super().train(mode)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._qk_cache = None
+        return super()._apply(fn, *args, **kwargs)
 
     def _padded_attention(self, q4: Tensor, k4: Tensor, v4: Tensor, key_padding: Tensor) -> Tensor:
         """Softmax attention outside the fused op (moving_average_gated_attention.py:210-256): the
