@@ -33,6 +33,45 @@ void set_error(const char* fmt, ...);
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
 
+// ---------------------------------------------------------------- row tiling of [tokens, H] tiles
+// How the channel vectors of one token are spread over threads in the kernels that walk
+// [tokens, H] tiles with per-group reductions: LPG consecutive lanes (a power of two) share one
+// (token, group) and move PER vectors of `vec` channels each; `slots` = lanes per token.
+struct RowTiling {
+  int LPG, PER, slots;
+  int lpg_shift;     // log2(LPG)
+  int slots_shift;   // log2(slots), or -1 when slots is not a power of two
+};
+
+static inline RowTiling make_row_tiling(int64_t G, int64_t Dg, int vec) {
+  RowTiling R;
+  const int64_t vecs = Dg / vec;          // vectors per (token, group)
+  int lpg = 1;
+  while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
+  R.LPG = lpg;
+  R.PER = (int)(vecs / lpg);
+  R.slots = (int)G * lpg;
+  R.lpg_shift = 0;
+  while ((1 << R.lpg_shift) < R.LPG) ++R.lpg_shift;
+  R.slots_shift = -1;
+  if ((R.slots & (R.slots - 1)) == 0) {
+    R.slots_shift = 0;
+    while ((1 << R.slots_shift) < R.slots) ++R.slots_shift;
+  }
+  return R;
+}
+
+// item -> (token, slot): a shift when the lane count per token is a power of two
+__device__ __forceinline__ void split_item(const RowTiling& R, int i, int& tok, int& slot) {
+  if (R.slots_shift >= 0) {
+    tok = i >> R.slots_shift;
+    slot = i & (R.slots - 1);
+  } else {
+    tok = i / R.slots;
+    slot = i - tok * R.slots;
+  }
+}
+
 // ---------------------------------------------------------------- element types
 struct bf16_t { uint16_t u; };
 struct f16_t { _Float16 h; };

@@ -30,19 +30,9 @@ struct SeqNormParams {
   float* mean;
   float* rstd;
   int B, L, H, G, Dg, TT, nt;
-  int LPG, PER, slots, lpg_shift, slots_shift;
+  RowTiling R;
   float eps;
 };
-
-__device__ __forceinline__ void split_item(const SeqNormParams& P, int i, int& tok, int& slot) {
-  if (P.slots_shift >= 0) {
-    tok = i >> P.slots_shift;
-    slot = i & (P.slots - 1);
-  } else {
-    tok = i / P.slots;
-    slot = i - tok * P.slots;
-  }
-}
 
 // Chan et al.: (na, ma, Ma) + (nb, mb, Mb)
 __device__ __forceinline__ void merge3(float& n, float& m, float& M2, float nb, float mb, float Mb) {
@@ -78,21 +68,21 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
       s_b[g] = P.rstd[(size_t)b * G + g];
     }
   __syncthreads();
-  const int items = ntok * P.slots;
-  const int span = VEC * P.PER;
+  const int items = ntok * P.R.slots;
+  const int span = VEC * P.R.PER;
   for (int i0 = 0; i0 < items; i0 += kThreads) {
     const int i = i0 + tid;
     const bool live = i < items;
     int tok, slot;
-    split_item(P, live ? i : 0, tok, slot);
-    const int g = slot >> P.lpg_shift;
-    const int c0 = g * Dg + (slot - (g << P.lpg_shift)) * span;
+    split_item(P.R, live ? i : 0, tok, slot);
+    const int g = slot >> P.R.lpg_shift;
+    const int c0 = g * Dg + (slot - (g << P.R.lpg_shift)) * span;
     if (APPLY) {
       if (live) {
         const float mu = s_a[g], r = s_b[g];
         const bool keep = !s_mask[tok];
         T* y = (T*)P.y + ((size_t)b * P.L + t0 + tok) * H;
-        for (int k = 0; k < P.PER; ++k) {
+        for (int k = 0; k < P.R.PER; ++k) {
           const int c = c0 + k * VEC;
           const V xv = *(const V*)(x + (size_t)tok * H + c);
           float gw[VEC], bw[VEC];
@@ -108,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
     } else {
       float s1 = 0.f, s2 = 0.f;
       if (live && !s_mask[tok]) {
-        for (int k = 0; k < P.PER; ++k) {
+        for (int k = 0; k < P.R.PER; ++k) {
           const V xv = *(const V*)(x + (size_t)tok * H + c0 + k * VEC);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
@@ -118,11 +108,11 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
           }
         }
       }
-      for (int o = 1; o < P.LPG; o <<= 1) {
+      for (int o = 1; o < P.R.LPG; o <<= 1) {
         s1 += __shfl_xor(s1, o);
         s2 += __shfl_xor(s2, o);
       }
-      if (live && slot == (g << P.lpg_shift)) {
+      if (live && slot == (g << P.R.lpg_shift)) {
         s_a[tok * G + g] = s1;
         s_b[tok * G + g] = s2;
       }
@@ -372,7 +362,7 @@ int launch_seqnorm_bwd(const SeqBwdParams& P, bool vec, hipStream_t s) {
 }
 
 struct SeqGeom {
-  int tt, nt, vec, lpg, per;
+  int tt, nt, vec;
   size_t part_bytes;
 };
 
@@ -381,17 +371,12 @@ bool seq_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, int len
   const int full = dtype == MEGA_F32 ? 4 : 8;
   if (length_last) {
     g->vec = (L % full == 0) ? full : 1;
-    g->tt = 0; g->nt = 0; g->lpg = 1; g->per = 1;
+    g->tt = 0; g->nt = 0;
     g->part_bytes = align_up((size_t)B * H * 12, 256);
     return true;
   }
   const int64_t Dg = H / G;
   g->vec = (Dg % full == 0) ? full : 1;
-  const int64_t vecs = Dg / g->vec;
-  int lpg = 1;
-  while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
-  g->lpg = lpg;
-  g->per = (int)(vecs / lpg);
   int tt = (int)(kMaxCells / G);
   if (tt > 16) tt = 16;
   if (tt < 1) tt = 1;
@@ -467,30 +452,10 @@ extern "C" int mega_group_sequence_norm_fwd(const void* x, void* y, int dtype, c
   P.x = x; P.y = y; P.gamma = gamma; P.beta = beta; P.mask = mask; P.part = (float*)workspace;
   P.count = count; P.mean = mean; P.rstd = rstd;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
-  P.LPG = g.lpg; P.PER = g.per; P.slots = (int)G * g.lpg; P.eps = (float)eps;
-  P.lpg_shift = 0;
-  while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
-  P.slots_shift = -1;
-  if ((P.slots & (P.slots - 1)) == 0) {
-    P.slots_shift = 0;
-    while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
-  }
+  P.eps = (float)eps;
   const bool aligned = ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)gamma | (uintptr_t)beta) % 16) == 0);
-  if (!aligned && !length_last && g.vec > 1) {
-    // element-wise tiling when the buffers are not 16-byte aligned
-    g.vec = 1;
-    int64_t vecs = H / G;
-    int lpg = 1;
-    while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
-    P.LPG = lpg; P.PER = (int)(vecs / lpg); P.slots = (int)G * lpg;
-    P.lpg_shift = 0;
-    while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
-    P.slots_shift = -1;
-    if ((P.slots & (P.slots - 1)) == 0) {
-      P.slots_shift = 0;
-      while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
-    }
-  }
+  if (!aligned) g.vec = 1;                 // element-wise tiling when a buffer is not 16-byte aligned
+  P.R = make_row_tiling(G, H / G, length_last ? 1 : g.vec);
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case MEGA_F32: return launch_seqnorm<float>(P, g, length_last, aligned, s);

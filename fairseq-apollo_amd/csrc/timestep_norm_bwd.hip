@@ -52,23 +52,8 @@ struct TsnBwdParams {
   float* gamma_grad;
   float* beta_grad;
   int B, L, H, G, Dg, TT, nt;
-  int LPG;     // lanes that share one (token, group)
-  int PER;     // vectors per lane
-  int slots;   // lanes per token = G * LPG
-  int lpg_shift;     // log2(LPG)
-  int slots_shift;   // log2(slots), or -1 when slots is not a power of two
+  RowTiling R;
 };
-
-// item -> (token, slot): a shift when the lane count per token is a power of two
-__device__ __forceinline__ void split_item(const TsnBwdParams& P, int i, int& tok, int& slot) {
-  if (P.slots_shift >= 0) {
-    tok = i >> P.slots_shift;
-    slot = i & (P.slots - 1);
-  } else {
-    tok = i / P.slots;
-    slot = i - tok * P.slots;
-  }
-}
 
 struct TileMap { float a, m, bu, bv; };
 // first `f`, then `s`
@@ -132,12 +117,12 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   }
 
   // ---- ds, db (and the group mean when it was not handed in) per (token, group)
-  const int items = ntok * P.slots;
-  const int span = VEC * P.PER;          // channels per lane
+  const int items = ntok * P.R.slots;
+  const int span = VEC * P.R.PER;          // channels per lane
   float rw[VEC], rb[VEC];                // FIXED: this thread's gamma / beta shares
 #pragma unroll
   for (int e = 0; e < VEC; ++e) { rw[e] = 0.f; rb[e] = 0.f; }
-  if (P.PER == 1) {
+  if (P.R.PER == 1) {
     // one vector per lane: four items per thread are loaded before any of them is used
     constexpr int U = 4;
     for (int i0 = 0; i0 < items; i0 += U * kThreads) {
@@ -149,12 +134,12 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
         const int i = i0 + u * kThreads + tid;
         livek[u] = i < items;
         int tok, slot;
-        split_item(P, livek[u] ? i : 0, tok, slot);
-        const int g = slot >> P.lpg_shift;
+        split_item(P.R, livek[u] ? i : 0, tok, slot);
+        const int g = slot >> P.R.lpg_shift;
         tokk[u] = tok;
-        cc[u] = g * Dg + (slot - (g << P.lpg_shift)) * VEC;
+        cc[u] = g * Dg + (slot - (g << P.R.lpg_shift)) * VEC;
         cellk[u] = tok * G + g;
-        leadk[u] = livek[u] && slot == (g << P.lpg_shift);
+        leadk[u] = livek[u] && slot == (g << P.R.lpg_shift);
         dvv[u] = *(const V*)(dy + (size_t)tok * H + cc[u]);
         xvv[u] = *(const V*)(x + (size_t)tok * H + cc[u]);
       }
@@ -181,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
             }
           }
         }
-        for (int o = 1; o < P.LPG; o <<= 1) {
+        for (int o = 1; o < P.R.LPG; o <<= 1) {
           ds += __shfl_xor(ds, o);
           db += __shfl_xor(db, o);
           sx += __shfl_xor(sx, o);
@@ -197,16 +182,16 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   for (int i0 = 0; i0 < items; i0 += kThreads) {
     const int i = i0 + tid;
     const bool live = i < items;
-    const int tok = live ? i / P.slots : 0;
-    const int slot = live ? i - tok * P.slots : 0;
-    const int g = slot / P.LPG;
-    const int c0 = g * Dg + (slot - g * P.LPG) * span;
+    const int tok = live ? i / P.R.slots : 0;
+    const int slot = live ? i - tok * P.R.slots : 0;
+    const int g = slot / P.R.LPG;
+    const int c0 = g * Dg + (slot - g * P.R.LPG) * span;
     const int cell = tok * G + g;
     float ds = 0.f, db = 0.f, sx = 0.f;
     if (live) {
       const float u = s_u[cell], r = s_r[cell];
       const bool keep = !s_mask[tok];
-      for (int k = 0; k < P.PER; ++k) {
+      for (int k = 0; k < P.R.PER; ++k) {
         const int c = c0 + k * VEC;
         const V dv = *(const V*)(dy + (size_t)tok * H + c);
         const V xv = *(const V*)(x + (size_t)tok * H + c);
@@ -223,12 +208,12 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
         }
       }
     }
-    for (int o = 1; o < P.LPG; o <<= 1) {
+    for (int o = 1; o < P.R.LPG; o <<= 1) {
       ds += __shfl_xor(ds, o);
       db += __shfl_xor(db, o);
       sx += __shfl_xor(sx, o);
     }
-    if (live && slot == g * P.LPG) {
+    if (live && slot == g * P.R.LPG) {
       s_ds[cell] = ds;
       s_db[cell] = db;
       if (!P.group_mean) s_ux[cell] = sx / (float)Dg;
@@ -335,11 +320,11 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   if (PHASE == 0) {
     if (FIXED) {
       // the kThreads / slots threads of one slot add up in a fixed order
-      const int slot = tid % P.slots;
-      const int g = slot / P.LPG;
-      const int c0 = g * Dg + (slot - g * P.LPG) * VEC;
-      for (int turn = 0; turn < kThreads / P.slots; ++turn) {
-        if (tid / P.slots == turn) {
+      const int slot = tid % P.R.slots;
+      const int g = slot / P.R.LPG;
+      const int c0 = g * Dg + (slot - g * P.R.LPG) * VEC;
+      for (int turn = 0; turn < kThreads / P.R.slots; ++turn) {
+        if (tid / P.R.slots == turn) {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) { s_wg[c0 + e] += rw[e]; s_bg[c0 + e] += rb[e]; }
         }
@@ -351,7 +336,7 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   } else {
     T* dx = (T*)P.dx + ((size_t)b * P.L + t0) * H;
     const float cg = 1.0f / (float)Dg;
-    if (P.PER == 1) {
+    if (P.R.PER == 1) {
       constexpr int U = 4;
       for (int i0 = 0; i0 < items; i0 += U * kThreads) {
         V dvv[U], xvv[U];
@@ -362,10 +347,10 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
           const int i = i0 + u * kThreads + tid;
           livek[u] = i < items;
           int tok, slot;
-          split_item(P, livek[u] ? i : 0, tok, slot);
-          const int g = slot >> P.lpg_shift;
+          split_item(P.R, livek[u] ? i : 0, tok, slot);
+          const int g = slot >> P.R.lpg_shift;
           tokk[u] = tok;
-          cc[u] = g * Dg + (slot - (g << P.lpg_shift)) * VEC;
+          cc[u] = g * Dg + (slot - (g << P.R.lpg_shift)) * VEC;
           cellk[u] = tok * G + g;
           dvv[u] = *(const V*)(dy + (size_t)tok * H + cc[u]);
           xvv[u] = *(const V*)(x + (size_t)tok * H + cc[u]);
@@ -389,15 +374,15 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
       }
     } else {
       for (int i = tid; i < items; i += kThreads) {
-        const int tok = i / P.slots;
-        const int slot = i - tok * P.slots;
-        const int g = slot / P.LPG;
-        const int c0 = g * Dg + (slot - g * P.LPG) * span;
+        const int tok = i / P.R.slots;
+        const int slot = i - tok * P.R.slots;
+        const int g = slot / P.R.LPG;
+        const int c0 = g * Dg + (slot - g * P.R.LPG) * span;
         const int cell = tok * G + g;
         const float r = s_r[cell], ux = s_ux[cell];
         const float a0 = s_ds[cell] * cg, a1 = 2.0f * s_db[cell] * cg;
         const bool keep = !s_mask[tok];
-        for (int k = 0; k < P.PER; ++k) {
+        for (int k = 0; k < P.R.PER; ++k) {
           const int c = c0 + k * VEC;
           const V dv = *(const V*)(dy + (size_t)tok * H + c);
           const V xv = *(const V*)(x + (size_t)tok * H + c);
@@ -492,7 +477,7 @@ __global__ __launch_bounds__(256) void tsn_bwd_param_kernel(const TsnBwdParams P
 }
 
 struct BwdGeom {
-  int tt, nt, vec, lpg, per;
+  int tt, nt, vec;
   size_t agg_bytes, state_bytes, part_bytes;
 };
 
@@ -501,11 +486,6 @@ bool bwd_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, BwdGeom
   const int64_t Dg = H / G;
   const int full = dtype == MEGA_F32 ? 4 : 8;
   g->vec = (Dg % full == 0) ? full : 1;
-  int64_t vecs = Dg / g->vec;          // vectors per (token, group)
-  int lpg = 1;
-  while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
-  g->lpg = lpg;
-  g->per = (int)(vecs / lpg);
   int tt = (int)(kMaxTileCells / G);
   if (tt > 32) tt = 32;
   if (tt < 1) tt = 1;
@@ -537,7 +517,7 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
     attr1 = true;
   }
   const dim3 grid((unsigned)(P.B * P.nt));
-  const bool fixed = P.PER == 1 && P.slots <= kThreads && kThreads % P.slots == 0;
+  const bool fixed = P.R.PER == 1 && P.R.slots <= kThreads && kThreads % P.R.slots == 0;
   if (fixed) hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, true>), grid, dim3(kThreads), lds0, s, P);
   else hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, false>), grid, dim3(kThreads), lds0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (tile maps)");
@@ -599,14 +579,8 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
   MEGA_REQUIRE(bwd_geometry(dtype, B, L, H, G, &g), MEGA_ERR_UNSUPPORTED,
                "timestep_norm_bwd: H=%ld G=%ld outside the supported envelope (H <= 8192, G <= %d)", (long)H, (long)G,
                kMaxTileCells);
-  if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad | (uintptr_t)gamma) % 16) != 0)) {
-    g.vec = 1;
-    int64_t vecs = H / G;
-    int lpg = 1;
-    while (lpg < 64 && vecs % (2 * lpg) == 0) lpg *= 2;
-    g.lpg = lpg;
-    g.per = (int)(vecs / lpg);
-  }
+  if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad | (uintptr_t)gamma) % 16) != 0))
+    g.vec = 1;                             // element-wise tiling when a buffer is not 16-byte aligned
   const size_t need = g.agg_bytes + g.state_bytes + g.part_bytes;
   MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
                "timestep_norm_bwd: workspace of %zu bytes (16-byte aligned) needed", need);
@@ -619,14 +593,7 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
   P.part = (float*)w;
   P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
-  P.LPG = g.lpg; P.PER = g.per; P.slots = (int)G * g.lpg;
-  P.lpg_shift = 0;
-  while ((1 << P.lpg_shift) < P.LPG) ++P.lpg_shift;
-  P.slots_shift = -1;
-  if ((P.slots & (P.slots - 1)) == 0) {
-    P.slots_shift = 0;
-    while ((1 << P.slots_shift) < P.slots) ++P.slots_shift;
-  }
+  P.R = make_row_tiling(G, H / G, g.vec);
   switch (dtype) {
     case MEGA_F32: return launch_bwd<float>(P, g.vec, s);
     case MEGA_BF16: return launch_bwd<bf16_t>(P, g.vec, s);
