@@ -944,3 +944,52 @@ def swiglu_bwd(y_grad: torch.Tensor, a: torch.Tensor, b: torch.Tensor):
                                  _stream(dev))
     _lib.check(rc, "swiglu_bwd")
     return da, db
+
+
+def ema_parameters_bwd(w_grad: torch.Tensor, b_grad: Optional[torch.Tensor], p: torch.Tensor, log_q: torch.Tensor,
+                       gamma: torch.Tensor, h: Optional[torch.Tensor], v: Optional[torch.Tensor] = None):
+    """-> (p_grad [D,N], q_grad [D,N] complex, gamma_grad [D,N] complex, h_grad [B,D,N] complex or None):
+    the gradients of ema_parameters_fwd's kernel w [D, L] (and bias b [B, D, L]) outputs.
+    Reference: ema_parameters_bwd, fairseq/csrc/ops/ema_parameters.cc:80-186 (`v`, the Vandermonde
+    matrix its CUDA path keeps, is not needed).  The power sums sum_l g[l] q^l and sum_l g[l] l q^(l-1)
+    come from the parameter-sum kernel of the fused backward: fed a unit impulse as x, its state
+    is q^t, so the "kernel gradient" it sees is g itself."""
+    dev = _need_gpu(w_grad, b_grad, p, log_q, gamma, h)
+    D, N = p.shape
+    L = w_grad.shape[-1]
+    q = torch.exp(log_q.detach().to(torch.complex64)).reshape(D, N)
+    pf = _f32c(p).reshape(D, N)
+    gc = gamma.detach().to(torch.complex64).reshape(D, N)
+    one = torch.ones(D, N, dtype=torch.float32, device=dev)
+    zero = torch.zeros(D, dtype=torch.float32, device=dev)
+
+    def power_sums(g: torch.Tensor):
+        """g [R, D, L] -> (S2, S1) [R, D, N] complex: sum_l g q^l, sum_l g l q^(l-1) per row."""
+        R = g.shape[0]
+        imp = torch.zeros(1, D, L, dtype=torch.float32, device=dev)
+        imp[:, :, 0] = 1.0
+        s2, s1 = [], []
+        for r in range(R):                      # the kernel adds rows up; here every row is wanted by itself
+            _, _, dq, dg, _ = ema_backward(g[r:r + 1].float(), imp, one, q, one.to(torch.complex64), zero)
+            s2.append(torch.conj(dg))           # with p = gamma = 1: dgamma = conj(S2), dq = conj(S1)
+            s1.append(torch.conj(dq))
+        return torch.stack(s2), torch.stack(s1)
+
+    S2, S1 = power_sums(w_grad.detach().reshape(1, D, L))
+    S2, S1 = S2[0], S1[0]
+    p_grad = (S2 * gc).real
+    q_grad = torch.conj(S1 * pf * gc)
+    gamma_grad = torch.conj(S2 * pf)
+    h_grad = None
+    if b_grad is not None:
+        if h is None:
+            raise RuntimeError("ema_parameters_bwd: b_grad needs the carried state h")
+        hc = h.detach().to(torch.complex64).reshape(-1, D, N)
+        T2, T1 = power_sums(b_grad.detach().reshape(-1, D, L))
+        # the bias uses q^(l+1): sum_l g q^(l+1) = q T2, sum_l g (l+1) q^l = T2 + q T1   (ema_parameters.cc:100-116)
+        sum2 = q * T2
+        sum1 = T2 + q * T1
+        q_grad = q_grad + torch.conj(sum1 * gc * hc).sum(0)
+        gamma_grad = gamma_grad + torch.conj(sum2 * hc).sum(0)
+        h_grad = torch.conj(sum2 * gc)
+    return p_grad, q_grad, gamma_grad, h_grad

@@ -269,6 +269,24 @@ def ema_kernel_bwd(dk, p, q, gamma):
     return (sum2 * gamma).real, np.conj(sum1 * p * gamma), np.conj(sum2 * p)
 
 
+def ema_bias_bwd(db, q, gamma, h):
+    """RowwiseEMABiasCPUBwd, csrc/ops/ema_parameters.cc:99-116: the bias is
+    b[b,d,l] = Re sum_n q^(l+1) gamma h; with sum1 = sum_l db[l] (l+1) q^l and sum2 = sum_l db[l] q^(l+1)
+    per batch row: dq = sum_rows conj(sum1 gamma h), dgamma = sum_rows conj(sum2 h), dh = conj(sum2 gamma).
+    db: [B, D, L]; h: [B, D, N].  Returns (dq [D,N], dgamma [D,N], dh [B,D,N])."""
+    db = np.asarray(db, np.float64)
+    q = np.asarray(q, np.complex128)
+    gamma = np.asarray(gamma, np.complex128)
+    h = np.asarray(h, np.complex128)
+    L = db.shape[-1]
+    l = np.arange(L)
+    qw1 = q[..., None] ** l                     # q^l
+    qw2 = qw1 * q[..., None]                    # q^(l+1)
+    sum1 = (db[:, :, None, :] * qw1[None] * (l + 1)).sum(-1)
+    sum2 = (db[:, :, None, :] * qw2[None]).sum(-1)
+    return np.conj(sum1 * gamma * h).sum(0), np.conj(sum2 * h).sum(0), np.conj(sum2 * gamma)
+
+
 def ema_backward(dy, x, p, q, gamma, omega, padding_mask=None, bidirectional: bool = False, shift: bool = True):
     """Backward of ema_forward (no carried state): the reference's chain fftconv backward
     (modules/fused_ops/fftconv.py:66-88, 85-100: dx = correlation of dy with k, dk = sum over the

@@ -144,6 +144,13 @@ def main():
     dp, dq, dg, _ = ref.ema_parameters_bwd(t(dk), None, t(p), log_q, t(g), None, vander)
     out.update({"ema_bwd.p": p, "ema_bwd.q": q, "ema_bwd.gamma": g, "ema_bwd.kernel_grad": dk,
                 "ema_bwd.p_grad": dp.numpy(), "ema_bwd.q_grad": dq.numpy(), "ema_bwd.gamma_grad": dg.numpy()})
+    # the same with a carried state: the bias gradient adds to dq, dgamma and gives dh
+    hb = (rng.normal(size=(2, K, N)) + 1j * rng.normal(size=(2, K, N))).astype(np.complex64)
+    db = rng.normal(size=(2, K, L)).astype(np.float32)
+    _, _, vander = ref.ema_parameters_fwd(t(p), log_q, t(g), t(hb), L)
+    dp2, dq2, dg2, dh2 = ref.ema_parameters_bwd(t(dk), t(db), t(p), log_q, t(g), t(hb), vander)
+    out.update({"ema_bwd.h": hb, "ema_bwd.bias_grad": db, "ema_bwd.p_grad_b": dp2.numpy(), "ema_bwd.q_grad_b": dq2.numpy(),
+                "ema_bwd.gamma_grad_b": dg2.numpy(), "ema_bwd.h_grad_b": dh2.numpy()})
 
     # SequenceNorm: both layouts, group and per-feature, ragged padding
     rng = np.random.default_rng(20242)

@@ -204,3 +204,25 @@ def test_hip_sequence_norm(gold, tag):
         y, n, mu, r = M.ops.sequence_norm_fwd(dev(c["x"]), dev(c["gamma"]), dev(c["beta"]), mask, 1e-5, last)
     assert rel_err(host(y), c["y"]) < 1e-4 and np.array_equal(host(n), c["count"])
     assert rel_err(host(mu), c["mean"]) < 1e-4 and rel_err(host(r), c["rstd"]) < 1e-4
+
+
+@pytest.mark.gpu
+def test_hip_ema_parameters_bwd(gold):
+    """The operator under the reference's name: kernel gradient (and bias gradient with a carried
+    state) to coefficient gradients."""
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, "ema_bwd")
+    log_q = torch.from_numpy(c["q"]).log().to("cuda:0")
+    dp, dq, dg, dh = M.ops.ema_parameters_bwd(dev(c["kernel_grad"]), None, dev(c["p"]), log_q, dev(c["gamma"]), None)
+    assert dh is None and rel_err(host(dp), c["p_grad"]) < 1e-4
+    for a, b in ((host(dq), c["q_grad"]), (host(dg), c["gamma_grad"])):
+        assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4
+    dp, dq, dg, dh = M.ops.ema_parameters_bwd(dev(c["kernel_grad"]), dev(c["bias_grad"]), dev(c["p"]), log_q,
+                                              dev(c["gamma"]), dev(c["h"]))
+    assert rel_err(host(dp), c["p_grad_b"]) < 1e-4
+    for a, b in ((host(dq), c["q_grad_b"]), (host(dg), c["gamma_grad_b"]), (host(dh), c["h_grad_b"])):
+        assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4

@@ -150,3 +150,26 @@ def test_sequence_norm_bwd_matches_reference_vectors(gold, tag):
     G = int(c["groups"]) or None
     dx, dg, db = O.sequence_norm_bwd(c["y_grad"], c["x"], c["gamma"], c.get("mask"), G, 1e-5, bool(c["length_last"]))
     assert rel_err(dx, c["x_grad"]) < 5e-5 and rel_err(dg, c["gamma_grad"]) < 5e-5 and rel_err(db, c["beta_grad"]) < 5e-5
+
+
+def test_ema_bias_bwd_matches_finite_differences_and_reference_vectors(gold):
+    rng = np.random.default_rng(11)
+    D, N, L, B = 3, 4, 9, 2
+    _, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    h = rng.normal(size=(B, D, N)) + 1j * rng.normal(size=(B, D, N))
+    wb = rng.normal(size=(B, D, L))
+    loss = lambda q_, g_, h_: (O.ema_bias(q_, g_, h_, L) * wb).sum()
+    dq, dg, dh = O.ema_bias_bwd(wb, q, g, h)
+    for _ in range(6):
+        j = tuple(rng.integers(0, s) for s in q.shape)
+        i = tuple(rng.integers(0, s) for s in h.shape)
+        for unit, part in ((1.0, "real"), (1j, "imag")):
+            assert abs(_fd(lambda a: loss(a, g, h), q, j, unit) - getattr(dq[j], part)) < 1e-6
+            assert abs(_fd(lambda a: loss(q, a, h), g, j, unit) - getattr(dg[j], part)) < 1e-6
+            assert abs(_fd(lambda a: loss(q, g, a), h, i, unit) - getattr(dh[i], part)) < 1e-6
+    c = _case(gold, "ema_bwd")
+    dp, dq, dg = O.ema_kernel_bwd(c["kernel_grad"], c["p"], c["q"], c["gamma"])
+    bq, bg, bh = O.ema_bias_bwd(c["bias_grad"], c["q"], c["gamma"], c["h"])
+    assert rel_err(dp, c["p_grad_b"]) < 5e-5
+    for a, b in ((dq + bq, c["q_grad_b"]), (dg + bg, c["gamma_grad_b"]), (bh, c["h_grad_b"])):
+        assert rel_err(a.real, b.real) < 5e-5 and rel_err(a.imag, b.imag) < 5e-5
