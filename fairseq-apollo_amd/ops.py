@@ -80,7 +80,7 @@ def _cplx_as_f32(t: torch.Tensor) -> torch.Tensor:
     """complex [...] -> float32 [..., 2]; real [...] -> [..., 2] with a zero imaginary part."""
     t = t.detach()
     if t.is_complex():
-        return torch.view_as_real(t.to(torch.complex64).contiguous()).contiguous()
+        return torch.view_as_real(t.to(torch.complex64).resolve_conj().contiguous()).contiguous()
     return torch.stack([t.to(torch.float32), torch.zeros_like(t, dtype=torch.float32)], dim=-1).contiguous()
 
 
@@ -993,3 +993,44 @@ def ema_parameters_bwd(w_grad: torch.Tensor, b_grad: Optional[torch.Tensor], p: 
         gamma_grad = gamma_grad + torch.conj(sum2 * hc).sum(0)
         h_grad = torch.conj(sum2 * gc)
     return p_grad, q_grad, gamma_grad, h_grad
+
+
+def ema_hidden_bwd(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, log_q: torch.Tensor,
+                   h: Optional[torch.Tensor], v: Optional[torch.Tensor] = None):
+    """-> (x_grad [B,D,L], p_grad [D,N], q_grad [D,N] complex, h_grad [B,D,N] complex or None): the
+    gradients of ema_hidden_fwd, h' = q^L h + sum_j p q^(L-1-j) x[j].
+    Reference: ema_hidden_bwd, fairseq/csrc/ops/ema_hidden.cc:66-159.  Built from two existing
+    kernels: x_grad is the layer's kernel with conj(y_grad) in the place of gamma, read backwards
+    (kernel generation); the power sums sum_j x[j] q^(L-1-j) and sum_j x[j] (L-1-j) q^(L-2-j) are the
+    state and its q-derivative at the last token, which the parameter-sum kernel returns when its
+    "y_grad" is a unit impulse there."""
+    dev = _need_gpu(y_grad, x, p, log_q, h)
+    B, D, L = x.shape
+    N = p.shape[1]
+    lq = log_q.detach().to(torch.complex64).reshape(D, N)
+    q = torch.exp(lq)
+    pf = _f32c(p).reshape(D, N)
+    dyc = torch.conj(y_grad.detach().to(torch.complex64).reshape(B, D, N))
+    one = torch.ones(D, N, dtype=torch.float32, device=dev)
+    zero = torch.zeros(D, dtype=torch.float32, device=dev)
+    imp = torch.zeros(1, D, L, dtype=torch.float32, device=dev)
+    imp[:, :, L - 1] = 1.0
+    xg = torch.empty(B, D, L, dtype=x.dtype, device=dev)
+    p_grad = torch.zeros(D, N, dtype=torch.float32, device=dev)
+    sum2 = torch.zeros(D, N, dtype=torch.complex64, device=dev)
+    xf = x.detach().float()
+    for b in range(B):
+        w, _, _ = ema_parameters_fwd(pf, lq, dyc[b], None, L)          # Re sum_n p q^l conj(dy): lag l = L-1-j
+        xg[b] = w.flip(-1).to(x.dtype)
+        _, _, dq1, dg1, _ = ema_backward(imp, xf[b:b + 1], one, q, one.to(torch.complex64), zero)
+        s_end, g_end = torch.conj(dg1), torch.conj(dq1)                # with p = gamma = 1
+        p_grad += (dyc[b] * s_end).real
+        sum2 += dyc[b] * pf * g_end
+    q_grad = torch.conj(sum2)
+    h_grad = None
+    if h is not None:
+        hc = h.detach().to(torch.complex64).reshape(B, D, N)
+        qL1 = torch.exp(lq * (L - 1))
+        q_grad = q_grad + torch.conj((dyc * hc).sum(0) * qL1 * L)
+        h_grad = torch.conj(dyc * qL1 * q)
+    return xg, p_grad, q_grad, h_grad

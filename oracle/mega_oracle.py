@@ -269,6 +269,31 @@ def ema_kernel_bwd(dk, p, q, gamma):
     return (sum2 * gamma).real, np.conj(sum1 * p * gamma), np.conj(sum2 * p)
 
 
+def ema_hidden_bwd(dy, x, p, q, h=None):
+    """EMAHiddenCPUBwdImpl, csrc/ops/ema_hidden.cc:66-159, for h' = q^L h + sum_j p q^(L-1-j) x[j]
+    (dy: gradient of h', complex [B, D, N]):
+    dx[j] = Re sum_n conj(dy) p q^(L-1-j); dp = Re sum_{b,j} conj(dy) x[j] q^(L-1-j);
+    dq = conj(sum_{b,j} conj(dy) x[j] p (L-1-j) q^(L-2-j) + sum_b conj(dy) h L q^(L-1)); dh = conj(conj(dy) q^L).
+    Returns (dx, dp, dq, dh or None)."""
+    x = np.asarray(x, np.float64)
+    p = np.asarray(p, np.float64)
+    q = np.asarray(q, np.complex128)
+    dyc = np.conj(np.asarray(dy, np.complex128))
+    B, D, L = x.shape
+    e = L - 1 - np.arange(L)                                         # exponent of q at token j
+    qw = q[..., None] ** e                                           # [D, N, L]
+    qd = np.where(e > 0, e * q[..., None] ** np.maximum(e - 1, 0), 0.0)
+    dx = np.real(np.einsum('bdn,dn,dnl->bdl', dyc, p, qw))
+    dp = np.real(np.einsum('bdn,bdl,dnl->dn', dyc, x, qw))
+    s2 = np.einsum('bdn,bdl,dn,dnl->dn', dyc, x, p, qd)
+    dh = None
+    if h is not None:
+        h = np.asarray(h, np.complex128)
+        s2 = s2 + (dyc * h).sum(0) * L * q ** (L - 1)
+        dh = np.conj(dyc * q ** L)
+    return dx, dp, np.conj(s2), dh
+
+
 def ema_bias_bwd(db, q, gamma, h):
     """RowwiseEMABiasCPUBwd, csrc/ops/ema_parameters.cc:99-116: the bias is
     b[b,d,l] = Re sum_n q^(l+1) gamma h; with sum1 = sum_l db[l] (l+1) q^l and sum2 = sum_l db[l] q^(l+1)

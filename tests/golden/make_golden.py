@@ -152,6 +152,17 @@ def main():
     out.update({"ema_bwd.h": hb, "ema_bwd.bias_grad": db, "ema_bwd.p_grad_b": dp2.numpy(), "ema_bwd.q_grad_b": dq2.numpy(),
                 "ema_bwd.gamma_grad_b": dg2.numpy(), "ema_bwd.h_grad_b": dh2.numpy()})
 
+    # hidden-state update backward (with a carried state)
+    B2, L2 = 2, 40
+    xh = rng.normal(size=(B2, K, L2)).astype(np.float32)
+    hh = (rng.normal(size=(B2, K, N)) + 1j * rng.normal(size=(B2, K, N))).astype(np.complex64)
+    dhy = (rng.normal(size=(B2, K, N)) + 1j * rng.normal(size=(B2, K, N))).astype(np.complex64)
+    _, vh = ref.ema_hidden_fwd(t(xh), t(p), log_q, t(hh))
+    gx, gp, gq, gh = ref.ema_hidden_bwd(t(dhy), t(xh), t(p), log_q, t(hh), vh)
+    out.update({"hid_bwd.x": xh, "hid_bwd.h": hh, "hid_bwd.y_grad": dhy, "hid_bwd.p": p, "hid_bwd.q": q,
+                "hid_bwd.x_grad": gx.numpy(), "hid_bwd.p_grad": gp.numpy(), "hid_bwd.q_grad": gq.numpy(),
+                "hid_bwd.h_grad": gh.numpy()})
+
     # SequenceNorm: both layouts, group and per-feature, ragged padding
     rng = np.random.default_rng(20242)
     for tag, (B, L, H, G, last, masked) in {"gsn_a": (3, 37, 48, 4, False, True), "gsn_b": (2, 130, 64, 16, True, True),

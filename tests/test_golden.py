@@ -226,3 +226,20 @@ def test_hip_ema_parameters_bwd(gold):
     assert rel_err(host(dp), c["p_grad_b"]) < 1e-4
     for a, b in ((host(dq), c["q_grad_b"]), (host(dg), c["gamma_grad_b"]), (host(dh), c["h_grad_b"])):
         assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4
+
+
+@pytest.mark.gpu
+def test_hip_ema_hidden_bwd(gold):
+    import torch
+
+    import fairseq_apollo_amd as M
+    from gpu_util import dev, host
+
+    c = _case(gold, "hid_bwd")
+    log_q = torch.from_numpy(c["q"]).log().to("cuda:0")
+    dx, dp, dq, dh = M.ops.ema_hidden_bwd(dev(c["y_grad"]), dev(c["x"]), dev(c["p"]), log_q, dev(c["h"]))
+    assert rel_err(host(dx), c["x_grad"]) < 1e-4 and rel_err(host(dp), c["p_grad"]) < 1e-4
+    for a, b in ((host(dq), c["q_grad"]), (host(dh), c["h_grad"])):
+        assert rel_err(a.real, b.real) < 1e-4 and rel_err(a.imag, b.imag) < 1e-4
+    dx0, dp0, dq0, dh0 = M.ops.ema_hidden_bwd(dev(c["y_grad"]), dev(c["x"]), dev(c["p"]), log_q, None)
+    assert dh0 is None and rel_err(host(dx0), c["x_grad"]) < 1e-4 and rel_err(host(dp0), c["p_grad"]) < 1e-4

@@ -173,3 +173,28 @@ def test_ema_bias_bwd_matches_finite_differences_and_reference_vectors(gold):
     assert rel_err(dp, c["p_grad_b"]) < 5e-5
     for a, b in ((dq + bq, c["q_grad_b"]), (dg + bg, c["gamma_grad_b"]), (bh, c["h_grad_b"])):
         assert rel_err(a.real, b.real) < 5e-5 and rel_err(a.imag, b.imag) < 5e-5
+
+
+def test_ema_hidden_bwd_matches_finite_differences_and_reference_vectors(gold):
+    rng = np.random.default_rng(12)
+    D, N, L, B = 3, 4, 10, 2
+    p, q, _ = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    x = rng.normal(size=(B, D, L))
+    h = rng.normal(size=(B, D, N)) + 1j * rng.normal(size=(B, D, N))
+    w = rng.normal(size=(B, D, N)) + 1j * rng.normal(size=(B, D, N))      # loss = Re sum conj(w) h'
+    loss = lambda x_, p_, q_, h_: np.real(np.conj(w) * O.ema_hidden(x_, p_, q_, h_)).sum()
+    dx, dp, dq, dh = O.ema_hidden_bwd(w, x, p, q, h)
+    for _ in range(6):
+        i = tuple(rng.integers(0, s) for s in x.shape)
+        j = tuple(rng.integers(0, s) for s in p.shape)
+        k = tuple(rng.integers(0, s) for s in h.shape)
+        assert abs(_fd(lambda a: loss(a, p, q, h), x, i) - dx[i]) < 1e-6
+        assert abs(_fd(lambda a: loss(x, a, q, h), p, j) - dp[j]) < 1e-6
+        for unit, part in ((1.0, "real"), (1j, "imag")):
+            assert abs(_fd(lambda a: loss(x, p, a, h), q, j, unit) - getattr(dq[j], part)) < 1e-6
+            assert abs(_fd(lambda a: loss(x, p, q, a), h, k, unit) - getattr(dh[k], part)) < 1e-6
+    c = _case(gold, "hid_bwd")
+    dx, dp, dq, dh = O.ema_hidden_bwd(c["y_grad"], c["x"], c["p"], c["q"], c["h"])
+    assert rel_err(dx, c["x_grad"]) < 5e-5 and rel_err(dp, c["p_grad"]) < 5e-5
+    for a, b in ((dq, c["q_grad"]), (dh, c["h_grad"])):
+        assert rel_err(a.real, b.real) < 5e-5 and rel_err(a.imag, b.imag) < 5e-5
