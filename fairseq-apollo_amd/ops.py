@@ -714,10 +714,45 @@ class DecodeStep:
         return torch.view_as_complex(self.h) if self.is_complex else self.h[..., 0]
 
 
+class _CausalConvFunc(torch.autograd.Function):
+    """fairseq/modules/fused_ops/fftconv.py:11-41 (FFTConvFunc) with the kernel in the time domain."""
+
+    @staticmethod
+    def forward(ctx, x, k):
+        ctx.save_for_backward(x, k)
+        return _long_conv(x, k, False, True)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        x, k = ctx.saved_tensors
+        x_grad, k_grad = fftconv_bwd(y_grad, x, k)
+        return x_grad, k_grad.to(k.dtype)
+
+
 def fftconv(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """Causal long convolution with an explicit kernel k[D, Lk] (fftconv,
-    fairseq/modules/fused_ops/fftconv.py:11-27); evaluated in the time domain."""
+    fairseq/modules/fused_ops/fftconv.py:11-27); evaluated in the time domain.  Differentiable."""
+    if torch.is_grad_enabled() and (x.requires_grad or k.requires_grad):
+        return _CausalConvFunc.apply(x, k)
     return _long_conv(x, k, False, True)
+
+
+def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor):
+    """-> (x_grad [B,D,L], k_grad [D,Lk] fp32) of y = fftconv(x, k): the two correlations of
+    fused_ops/fftconv.py:66-88 (x_grad[t] = sum_l k[l] dy[t+l], k_grad[l] = sum_{b,t} dy[t] x[t-l]) as
+    causal convolutions of the time-reversed gradient, through the same explicit-kernel op (a
+    correctness path, O(L Lk) per row; the modules use ema_backward, which forms neither k nor k_grad)."""
+    _need_gpu(y_grad, x, k)
+    B, D, L = x.shape
+    Lk = k.shape[1]
+    r = y_grad.detach().to(x.dtype).flip(-1).contiguous()              # r[t] = dy[L-1-t]
+    x_grad = _long_conv(r, k, False, True).flip(-1)
+    k_grad = torch.zeros(D, L, dtype=torch.float32, device=x.device)
+    xf = x.detach().float()
+    for b in range(B):
+        # y[t] = sum_j x_b[j] r_b[t-j] = sum_j x_b[j] dy_b[L-1-t+j]  ->  k_grad[l] += y[L-1-l]
+        k_grad += _long_conv(r[b:b + 1].float(), xf[b], False, True)[0].flip(-1)
+    return x_grad, k_grad[:, :Lk].contiguous()
 
 
 def bidirectional_fftconv(x: torch.Tensor, k: torch.Tensor, shift: bool = True) -> torch.Tensor:

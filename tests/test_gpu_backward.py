@@ -505,3 +505,23 @@ def test_backward_edge_shapes():
     # softmax backward on a single column
     yv = M.ops.attention_softmax_fwd(dev(rng.normal(size=(3, 1, 1))), 0.0, True)
     assert float(M.ops.attention_softmax_bwd(dev(rng.normal(size=(3, 1, 1))), yv, True).abs().max()) < 1e-6
+
+
+def test_explicit_kernel_convolution_autograd():
+    """ops.fftconv(x, k) under autograd against the oracle's correlations (dk restricted to Lk lags)."""
+    rng = np.random.default_rng(97)
+    B, D, L, Lk = 2, 6, 70, 40
+    x64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    k64 = rng.normal(size=(D, Lk)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    x = dev(x64).requires_grad_(True)
+    k = dev(k64).requires_grad_(True)
+    y = M.ops.fftconv(x, k)
+    assert rel_err(host(y), O.causal_conv_direct(x64, k64)) < 1e-4
+    (y * dev(w64)).sum().backward()
+    dx = np.zeros_like(x64)
+    dk = np.zeros_like(k64)
+    for l in range(Lk):
+        dx[:, :, :L - l] += w64[:, :, l:] * k64[None, :, l:l + 1]
+        dk[:, l] = (w64[:, :, l:] * x64[:, :, :L - l]).sum(axis=(0, 2))
+    assert rel_err(host(x.grad), dx) < 1e-4 and rel_err(host(k.grad), dk) < 1e-4
