@@ -23,7 +23,10 @@ from .layers import (  # noqa: F401,E402
     streamed_forward,
 )
 
+from .model import MegaDecoderNoCrossAttn  # noqa: F401,E402
+
 __all__ = [
+    "MegaDecoderNoCrossAttn",
     "Mega2Layer",
     "MegaDecoderLayer",
     "MegaEncoderLayer",

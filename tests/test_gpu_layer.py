@@ -258,3 +258,35 @@ def test_simple_relative_bias_layer(bidir):
         fd = ((O.gated_attention_layer(host(x), P, simple_bias=sp, **okw) * host(w)).sum()
               - (O.gated_attention_layer(host(x), P, simple_bias=sm, **okw) * host(w)).sum()) / 2e-5
         assert abs(fd - g[i]) < 3e-3 * (np.abs(g).max() + 1e-6), (i, fd, g[i])
+
+
+def test_decoder_model_names_streaming_and_training():
+    """MegaDecoderNoCrossAttn: reference state-dict names, logits streamed chunk by chunk equal to
+    the one-shot logits (also for a length that is not a whole number of chunks), and a
+    cross-entropy training step."""
+    torch.manual_seed(41)
+    args = _lm_args(decoder_layers=2, share_decoder_input_output_embed=True, layer_scale=True, norm_eps=1e-5)
+    vocab, pad = 50, 1
+    emb = torch.nn.Embedding(vocab, 64, padding_idx=pad)
+    model = M.MegaDecoderNoCrossAttn(args, vocab, emb).to(DEV).eval()
+    keys = set(model.state_dict())
+    assert {"version", "embed_tokens.weight", "layers.0.mega_layer.norm.weight", "layers.1.mega_layer.move.alpha",
+            "layers.0.nffn.fc1.weight", "layers.1.nffn.layerscale_weight", "final_norm.weight", "final_norm.bias",
+            "output_projection.weight"} <= keys
+    assert model.output_projection.weight is model.embed_tokens.weight
+    with torch.no_grad():
+        for lyr in model.layers:
+            for prm in (lyr.mega_layer.v_proj.weight, lyr.mega_layer.mx_proj.weight, lyr.mega_layer.h_proj.weight):
+                prm.normal_(0, 0.1)
+    tokens = torch.randint(2, vocab, (2, 512), device=DEV)
+    with torch.no_grad():
+        full = model(tokens)[0]
+        streamed = model.streamed(tokens)
+        odd = model(tokens[:, :300])[0]                  # padded up to 384 tokens inside, cut back to 300
+    assert full.shape == (2, 512, vocab) and rel_err(host(streamed), host(full)) < 5e-5
+    assert odd.shape == (2, 300, vocab) and rel_err(host(odd[:, :256]), host(full[:, :256])) < 5e-5
+    model.train()
+    logits = model(tokens[:, :-1])[0]
+    loss = torch.nn.functional.cross_entropy(logits.reshape(-1, vocab).float(), tokens[:, 1:].reshape(-1))
+    loss.backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
