@@ -14,7 +14,8 @@ bool attention_mfma_covers(int dtype, const void* q, const void* k, const void* 
                            int64_t H1, int64_t H2);
 size_t attention_mfma_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H2);
 int attention_mfma_run(const void* q, const void* k, const void* v, void* y, void* w, int dtype, int64_t B, int64_t L,
-                       int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, void* ws, hipStream_t s);
+                       int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, float dropout, uint64_t seed,
+                       void* ws, hipStream_t s);
 
 namespace {
 
@@ -34,10 +35,17 @@ __device__ __forceinline__ float block_reduce(float v, float* red, bool is_max) 
   return r;
 }
 
+// DropKey (fairseq/csrc/softmax.cuh:157-185): a score whose uniform draw falls below `dropout` is
+// replaced by -inf before the softmax, so the surviving keys of the row still sum to one.
+__device__ __forceinline__ float drop_key(float v, float dropout, uint64_t seed, uint64_t idx) {
+  return (dropout > 0.f && hash_uniform(seed, idx) < dropout) ? -INFINITY : v;
+}
+
 // one workgroup per row
 template <typename T>
 __global__ __launch_bounds__(kBlock) void softmax_kernel(const T* __restrict__ x, T* __restrict__ y,
-                                                         int64_t outer, int64_t inner, int causal) {
+                                                         int64_t outer, int64_t inner, int causal, float dropout,
+                                                         uint64_t seed) {
   __shared__ float red[kBlock / 64];
   const int64_t row = blockIdx.x;
   const int64_t r = row % outer;
@@ -45,17 +53,19 @@ __global__ __launch_bounds__(kBlock) void softmax_kernel(const T* __restrict__ x
   if (n < 0) n = 0;
   const T* xp = x + row * inner;
   T* yp = y + row * inner;
+  const uint64_t e0 = (uint64_t)row * (uint64_t)inner;
   float m = -INFINITY;
-  for (int64_t j = threadIdx.x; j < n; j += kBlock) m = fmaxf(m, to_float(xp[j]));
+  for (int64_t j = threadIdx.x; j < n; j += kBlock) m = fmaxf(m, drop_key(to_float(xp[j]), dropout, seed, e0 + j));
   m = block_reduce(m, red, true);
   const bool dead = !(m > -INFINITY) || !(m < INFINITY);
   float s = 0.f;
   if (!dead)
-    for (int64_t j = threadIdx.x; j < n; j += kBlock) s += __expf(to_float(xp[j]) - m);
+    for (int64_t j = threadIdx.x; j < n; j += kBlock)
+      s += __expf(drop_key(to_float(xp[j]), dropout, seed, e0 + j) - m);
   s = block_reduce(s, red, false);
   const float c = (dead || s == 0.f) ? 0.f : 1.0f / s;
   for (int64_t j = threadIdx.x; j < inner; j += kBlock) {
-    const float e = (j < n && !dead) ? __expf(to_float(xp[j]) - m) * c : 0.f;
+    const float e = (j < n && !dead) ? __expf(drop_key(to_float(xp[j]), dropout, seed, e0 + j) - m) * c : 0.f;
     yp[j] = from_float<T>(e);
   }
 }
@@ -65,7 +75,8 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                                const T* __restrict__ v, T* __restrict__ y,
                                                                T* __restrict__ w, int B, int L, int Nh, int H1,
-                                                               int H2, float scale, int causal) {
+                                                               int H2, float scale, int causal, float dropout,
+                                                               uint64_t seed) {
   extern __shared__ float sc[];     // [L] scores, then [H1] the query row
   __shared__ float red[kBlock / 64];
   float* qs = sc + L;
@@ -74,6 +85,7 @@ __global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restri
   const int b = blockIdx.x / (L * Nh);
   const int nk = causal ? l + 1 : L;
   const T* qp = q + (((size_t)b * L + l) * Nh + n) * H1;
+  const uint64_t e0 = (((uint64_t)b * Nh + n) * L + l) * L;     // the row's place in the [B,Nh,L,L] weights
   for (int i = threadIdx.x; i < H1; i += kBlock) qs[i] = to_float(qp[i]);
   __syncthreads();
   float m = -INFINITY;
@@ -81,7 +93,7 @@ __global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restri
     const T* kp = k + (((size_t)b * L + j) * Nh + n) * H1;
     float s = 0.f;
     for (int i = 0; i < H1; ++i) s += qs[i] * to_float(kp[i]);
-    s *= scale;
+    s = drop_key(s * scale, dropout, seed, e0 + j);
     sc[j] = s;
     m = fmaxf(m, s);
   }
@@ -89,7 +101,7 @@ __global__ __launch_bounds__(kBlock) void attention_row_kernel(const T* __restri
   const bool dead = !(m > -INFINITY) || !(m < INFINITY);
   float s = 0.f;
   for (int j = threadIdx.x; j < nk; j += kBlock) {
-    const float e = dead ? 0.f : __expf(sc[j] - m);
+    const float e = dead ? 0.f : __expf(sc[j] - m);     // exp(-inf - m) = 0 for a dropped key
     sc[j] = e;
     s += e;
   }
@@ -176,10 +188,12 @@ int launch_softmax_bwd(const void* dy, const void* y, void* dx, int64_t rows, in
 using namespace mega;
 
 extern "C" int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch, int64_t outer,
-                                          int64_t inner, int causal, void* stream) {
+                                          int64_t inner, int causal, float dropout, uint64_t seed, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "attention_softmax_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(batch >= 0 && outer >= 0 && inner >= 0, MEGA_ERR_ARG, "attention_softmax_fwd: negative size");
+  MEGA_REQUIRE(dropout >= 0.f && dropout <= 1.f, MEGA_ERR_ARG, "attention_softmax_fwd: dropout %g outside [0, 1]",
+               (double)dropout);
   const int64_t rows = batch * outer;
   if (rows == 0 || inner == 0) return MEGA_OK;
   MEGA_REQUIRE(x && y, MEGA_ERR_ARG, "attention_softmax_fwd: null pointer argument");
@@ -188,13 +202,16 @@ extern "C" int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int
   const dim3 grid((unsigned)rows);
   switch (dtype) {
     case MEGA_F32:
-      hipLaunchKernelGGL(softmax_kernel<float>, grid, dim3(kBlock), 0, s, (const float*)x, (float*)y, outer, inner, causal);
+      hipLaunchKernelGGL(softmax_kernel<float>, grid, dim3(kBlock), 0, s, (const float*)x, (float*)y, outer, inner, causal,
+                         dropout, seed);
       break;
     case MEGA_BF16:
-      hipLaunchKernelGGL(softmax_kernel<bf16_t>, grid, dim3(kBlock), 0, s, (const bf16_t*)x, (bf16_t*)y, outer, inner, causal);
+      hipLaunchKernelGGL(softmax_kernel<bf16_t>, grid, dim3(kBlock), 0, s, (const bf16_t*)x, (bf16_t*)y, outer, inner, causal,
+                         dropout, seed);
       break;
     default:
-      hipLaunchKernelGGL(softmax_kernel<f16_t>, grid, dim3(kBlock), 0, s, (const f16_t*)x, (f16_t*)y, outer, inner, causal);
+      hipLaunchKernelGGL(softmax_kernel<f16_t>, grid, dim3(kBlock), 0, s, (const f16_t*)x, (f16_t*)y, outer, inner, causal,
+                         dropout, seed);
       break;
   }
   MEGA_CHECK_LAUNCH("attention_softmax_fwd");
@@ -209,9 +226,12 @@ extern "C" size_t mega_attention_workspace_bytes(int dtype, int64_t B, int64_t L
 
 extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
                                   int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
-                                  int causal, void* workspace, size_t workspace_bytes, void* stream) {
+                                  int causal, float dropout, uint64_t seed, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "attention_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(dropout >= 0.f && dropout <= 1.f, MEGA_ERR_ARG, "attention_fwd: dropout %g outside [0, 1]",
+               (double)dropout);
   MEGA_REQUIRE(B >= 0 && L >= 0 && Nh > 0 && H1 > 0 && H2 > 0, MEGA_ERR_ARG, "attention_fwd: bad shape");
   if (B == 0 || L == 0) return MEGA_OK;
   MEGA_REQUIRE(q && k && v && y, MEGA_ERR_ARG, "attention_fwd: null pointer argument");
@@ -220,7 +240,8 @@ extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, v
     const size_t need = attention_mfma_workspace_bytes(dtype, B, L, Nh, H2);
     MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 256) == 0, MEGA_ERR_WORKSPACE,
                  "attention_fwd: workspace of %zu bytes (256-byte aligned) needed", need);
-    return attention_mfma_run(q, k, v, y, w, dtype, B, L, Nh, H1, H2, scale, causal, workspace, (hipStream_t)stream);
+    return attention_mfma_run(q, k, v, y, w, dtype, B, L, Nh, H1, H2, scale, causal, dropout, seed, workspace,
+                              (hipStream_t)stream);
   }
   const size_t smem = (size_t)(L + H1) * 4;
   MEGA_REQUIRE(smem <= 150 * 1024, MEGA_ERR_UNSUPPORTED, "attention_fwd: L=%ld too long for one chunk", (long)L);
@@ -232,7 +253,8 @@ extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, v
       hipFuncSetAttribute((const void*)attention_row_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                           (int)smem);                                                                      \
     hipLaunchKernelGGL(attention_row_kernel<T>, grid, dim3(kBlock), smem, s, (const T*)q, (const T*)k,     \
-                       (const T*)v, (T*)y, (T*)w, (int)B, (int)L, (int)Nh, (int)H1, (int)H2, scale, causal); \
+                       (const T*)v, (T*)y, (T*)w, (int)B, (int)L, (int)Nh, (int)H1, (int)H2, scale, causal,  \
+                       dropout, seed);                                                                     \
   } while (0)
   switch (dtype) {
     case MEGA_F32: LAUNCH_ATT(float); break;

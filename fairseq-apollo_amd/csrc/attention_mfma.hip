@@ -309,6 +309,10 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restric
         v[u].z = __expf(v[u].z - m); v[u].w = __expf(v[u].w - m);
         sum += (v[u].x + v[u].y) + (v[u].z + v[u].w);
       }
+    } else {
+      // every key masked or dropped: the registers hold -inf, and -inf * 0 would be NaN
+#pragma unroll
+      for (int u = 0; u < NV; ++u) v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     sum = wave_sum(sum);
     const float c = (dead || sum == 0.f) ? 0.f : 1.0f / sum;
@@ -344,9 +348,27 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(const float* __restric
   }
 }
 
+// DropKey on the fp32 scores, in place, ahead of the softmax: element (row, j) of the [B*Nh*L, L]
+// score matrix becomes -inf when its uniform draw falls below `dropout`.  Launched only when
+// dropout > 0, so the inference path does not pay for it.
+__global__ __launch_bounds__(256) void dropkey_f32_kernel(float* __restrict__ s, int outer, int inner, int64_t spitch,
+                                                          int causal, float dropout, uint64_t seed, int64_t nrows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
+  const int r = (int)(row % outer);
+  int n = causal ? inner - outer + r + 1 : inner;
+  if (n > inner) n = inner;
+  float* sp = s + row * spitch;
+  const uint64_t e0 = (uint64_t)row * (uint64_t)inner;
+  for (int j = lane; j < n; j += 64)
+    if (hash_uniform(seed, e0 + j) < dropout) sp[j] = -INFINITY;
+}
+
 template <typename T>
 int run_attention(const void* q, const void* k, const void* v, void* y, void* w, int64_t B, int64_t L, int64_t Nh,
-                  int64_t H1, int64_t H2, float scale, int causal, char* ws, hipStream_t s) {
+                  int64_t H1, int64_t H2, float scale, int causal, float dropout, uint64_t seed, char* ws,
+                  hipStream_t s) {
   const int64_t Lp = (L + 7) / 8 * 8;
   const int64_t BN_ = B * Nh;
   float* S = (float*)ws;
@@ -368,6 +390,9 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   G.nin = (int)Nh; G.M = (int)L; G.N = (int)L; G.K = (int)H1; G.alpha = scale; G.causal = causal ? 1 : 0; G.kshift = 0;
   const bool xcd = BN_ % 8 == 0;
   launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  if (dropout > 0.f)
+    hipLaunchKernelGGL(dropkey_f32_kernel, dim3((unsigned)ceil_div(BN_ * L, 4)), dim3(256), 0, s, S, (int)L, (int)L, Lp,
+                       causal, dropout, seed, (int64_t)(BN_ * L));
   hipLaunchKernelGGL(softmax_f32_kernel<T>, dim3((unsigned)ceil_div(BN_ * L, 4)), dim3(256), 0, s, S, P, (int)L, (int)L,
                      Lp, Lp, (int)Lp, causal, w ? 1 : 0, (int64_t)(BN_ * L));
   if (w) {
@@ -407,9 +432,11 @@ size_t attention_mfma_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t N
 }
 
 int attention_mfma_run(const void* q, const void* k, const void* v, void* y, void* w, int dtype, int64_t B, int64_t L,
-                       int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, void* ws, hipStream_t s) {
-  if (dtype == MEGA_BF16) return run_attention<bf16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
-  return run_attention<f16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
+                       int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, float dropout, uint64_t seed,
+                       void* ws, hipStream_t s) {
+  if (dtype == MEGA_BF16)
+    return run_attention<bf16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, dropout, seed, (char*)ws, s);
+  return run_attention<f16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, dropout, seed, (char*)ws, s);
 }
 
 }  // namespace mega

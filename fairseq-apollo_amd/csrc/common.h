@@ -116,6 +116,19 @@ struct alignas(sizeof(T) * VEC) Vec {
   T v[VEC];
 };
 
+// ---------------------------------------------------------------- counter-based random numbers
+// Uniform number in [0, 1) that depends only on (seed, idx): the 64-bit finaliser of splitmix64 on
+// seed + (idx + 1) * golden ratio, top 24 bits.  Every kernel that drops keys calls it with the
+// element's position in the [B, Nh, L, L] weight tensor, so the fused and the unfused attention
+// draw the same mask from the same seed, and a mask can be restated on the host bit for bit.
+__host__ __device__ inline float hash_uniform(uint64_t seed, uint64_t idx) {
+  uint64_t z = seed + (idx + 1) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
 // ---------------------------------------------------------------- complex
 struct cfloat {
   float re, im;

@@ -51,8 +51,8 @@ class RMSNorm(nn.Module):
 class NormalizedFeedForwardNetwork(nn.Module):
     """The reference's position-wise block, `x + fc2(silu(fc1(norm(x))))` with an optional
     per-feature layer scale (fairseq/modules/normalized_feedforward_network.py:13-93; same
-    constructor arguments, parameter names and initialisation; dropout is inference-mode identity).
-    The two projections are library GEMMs; norm and activation are elementwise glue."""
+    constructor arguments, parameter names and initialisation; the two dropouts act in training
+    mode only).  The two projections are library GEMMs; norm and activation are elementwise glue."""
 
     def __init__(self, embed_dim, ffn_hidden_dim, dropout=0.0, hidden_dropout=0.0, norm_type='layernorm',
                  norm_affine=True, norm_eps=1e-5, layer_scale=None, init_mode='bert', export=False):
@@ -62,8 +62,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
         self.act_fn = 'silu'
         self.init_mode = init_mode
         self.layer_scale = layer_scale
-        if dropout or hidden_dropout:
-            raise RuntimeError("NormalizedFeedForwardNetwork: dropout (training) is not implemented; pass 0")
+        self.dropout_p, self.hidden_dropout_p = float(dropout), float(hidden_dropout)
         if norm_type == 'layernorm':
             self.norm = nn.LayerNorm(embed_dim, eps=norm_eps, elementwise_affine=norm_affine)
         elif norm_type == 'rmsnorm':
@@ -95,7 +94,8 @@ class NormalizedFeedForwardNetwork(nn.Module):
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 
     def forward(self, x: Tensor) -> Tensor:
-        h = self.fc2(F.silu(self.fc1(self.norm(x))))
+        h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
+        h = F.dropout(self.fc2(h), self.dropout_p, self.training)
         if self.layerscale_weight is not None:
             h = h * self.layerscale_weight
         return h + x
@@ -166,9 +166,13 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def __init__(self, embed_dim, zdim, hdim, ndim, chunk_size=-1, moving_layer='cema', moving_act='rmsnorm',
                  norm_num_groups=None, norm_affine=True, norm_eps=1e-5, max_positions=1024, num_heads=1,
                  efficient_attn=True, rel_pos_bias='rotary', bidirectional=False, attention_activation='softmax',
-                 truncation=None):
+                 truncation=None, dropout=0.0, attention_dropout=0.0, hidden_dropout=0.0):
         super().__init__()
         self.init_incremental_state()
+        # moving_average_gated_attention.py:64-79: element dropout after the output activation and on the
+        # two hidden activations, DropKey inside the attention softmax; all three act in training mode only
+        self.dropout_p, self.hidden_dropout_p = float(dropout), float(hidden_dropout)
+        self.attention_dropout_p = float(attention_dropout)
         if attention_activation != 'softmax':
             raise NotImplementedError("only the softmax attention is built (no relu2 / laplace)")
         if rel_pos_bias not in ('rotary', 'simple'):
@@ -181,8 +185,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         self.bidirectional = bidirectional
         # causal layers: the fused causal op; bidirectional layers (moving_average_gated_attention.py:70-75,
         # 84-92): full softmax over every chunk, SequenceNorm, a two-sided moving average
-        self.efficient_attn = EfficientAttention(dropout=0.0, use_causal_mask=not bidirectional, scale=1.0)
-        self.attn_softmax = AttentionSoftmax(dropout=0.0, use_causal_mask=not bidirectional)
+        self.efficient_attn = EfficientAttention(dropout=attention_dropout, use_causal_mask=not bidirectional,
+                                                 scale=1.0)
+        self.attn_softmax = AttentionSoftmax(dropout=attention_dropout, use_causal_mask=not bidirectional)
         if bidirectional:
             self.norm = SequenceNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
         else:
@@ -220,7 +225,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
                 incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None):
         """x: [B, L, D] -> ([B, L, D], None)."""
-        if _training_call(self, x):
+        if _training_call(self, x) or (self.training and self._drops()):
             return self._forward_autograd(x, padding_mask, incremental_state), None
         bsz, seq_len, embed_dim = x.size()
         assert embed_dim == self.embed_dim
@@ -258,6 +263,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         hp = self.h_proj(ops.gate_mul_fwd(attn.reshape(bsz, seq_len, self.hdim), r))
         return ops.gate_out_fwd(residual, u, hx, hp), None
 
+    def _drops(self) -> bool:
+        return self.dropout_p > 0 or self.hidden_dropout_p > 0 or self.attention_dropout_p > 0
+
     def _qk_constants(self, simple: bool):
         """(gamma + 1, beta, rotation frequencies) in fp32 for the q / k kernel; kept in eval mode
         (dropped by train() and by .to() / .half())."""
@@ -289,8 +297,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             pad = key_padding.to(torch.bool)
             pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
             s = s.masked_fill(pad[:, None, None, :], float('-inf'))
-        w = ops.attention_softmax_fwd(s, 0.0, not self.bidirectional)
-        return torch.einsum('bnqk,bknh->bqnh', w, v4)
+        return torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
 
     def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
         """The same layer with a complete autograd graph (moving_average_gated_attention.py:263-417,
@@ -307,7 +314,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             x = self.norm(x, padding_mask=padding_mask)
         v = F.silu(self.v_proj(x))
         mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
-        base = self.mx_proj(self.move_act(mx))
+        base = self.mx_proj(F.dropout(self.move_act(mx), self.hidden_dropout_p, self.training))
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
         z = F.normalize(z, p=2, dim=-1, eps=1e-5)
         z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
@@ -333,7 +340,13 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             attn = torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
         else:
             attn = self.efficient_attn(q4, k4, v4)
-        hp = self.h_proj(GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r))
+        gated = GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r)
+        hp = self.h_proj(F.dropout(gated, self.hidden_dropout_p, self.training))
+        if self.training and self.dropout_p > 0:
+            # the output dropout sits between the activation and the residual mix
+            # (moving_average_gated_attention.py:409-412), so the fused gate is taken apart
+            h = F.dropout(F.silu(hx + hp), self.dropout_p, True)
+            return torch.addcmul(residual, torch.sigmoid(u), h - residual)
         return GateOutFunc.apply(residual, u, hx, hp)
 
     def _cached_attention(self, z: Tensor, v: Tensor, saved_state, incremental_state) -> Tensor:
@@ -432,11 +445,13 @@ class MegaDecoderLayer(nn.Module):
             max_positions=_arg(args, 'max_target_positions', 1024), num_heads=_arg(args, 'num_heads', 1),
             efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
             bidirectional=False, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
-            truncation=trunc if trunc and trunc > 0 else None)
+            truncation=trunc if trunc and trunc > 0 else None, dropout=_arg(args, 'dropout', 0.0),
+            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0))
         self.cross_attn = None
         if _arg(args, 'decoder_ffn_embed_dim', 0) > 0:
             self.nffn = NormalizedFeedForwardNetwork(
-                self.embed_dim, args.decoder_ffn_embed_dim, norm_type=_arg(args, 'norm_type', 'layernorm'),
+                self.embed_dim, args.decoder_ffn_embed_dim, dropout=_arg(args, 'dropout', 0.0),
+                hidden_dropout=_arg(args, 'activation_dropout', 0.0), norm_type=_arg(args, 'norm_type', 'layernorm'),
                 norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
                 layer_scale=layer_scale, init_mode=_arg(args, 'init_mode', 'bert'))
         else:
@@ -466,10 +481,12 @@ class MegaEncoderLayer(nn.Module):
             max_positions=_arg(args, 'max_source_positions', 1024), num_heads=_arg(args, 'num_heads', 1),
             efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
             bidirectional=True, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
-            truncation=trunc if trunc and trunc > 0 else None)
+            truncation=trunc if trunc and trunc > 0 else None, dropout=_arg(args, 'dropout', 0.0),
+            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0))
         if _arg(args, 'encoder_ffn_embed_dim', 0) > 0:
             self.nffn = NormalizedFeedForwardNetwork(
-                self.embed_dim, args.encoder_ffn_embed_dim, norm_type=_arg(args, 'norm_type', 'layernorm'),
+                self.embed_dim, args.encoder_ffn_embed_dim, dropout=_arg(args, 'dropout', 0.0),
+                hidden_dropout=_arg(args, 'activation_dropout', 0.0), norm_type=_arg(args, 'norm_type', 'layernorm'),
                 norm_affine=not _arg(args, 'no_affine_norm', False), norm_eps=_arg(args, 'norm_eps', 1e-5),
                 layer_scale=layer_scale, init_mode=_arg(args, 'init_mode', 'bert'))
         else:

@@ -554,11 +554,12 @@ class SwiGLUFunc(torch.autograd.Function):
 
 
 class AttentionSoftmaxFunc(torch.autograd.Function):
-    """fairseq/modules/attention_softmax.py:11-39 (dropout = 0)."""
+    """fairseq/modules/attention_softmax.py:11-39.  The saved output already holds zeros at the
+    dropped keys, so the backward needs no mask.  `seed` (not in the reference) pins the mask."""
 
     @staticmethod
-    def forward(ctx, x, dropout: float = 0.0, use_causal_mask: bool = True, training: bool = True):
-        y = ops.attention_softmax_fwd(x, dropout if training else 0.0, use_causal_mask)
+    def forward(ctx, x, dropout: float = 0.0, use_causal_mask: bool = True, training: bool = True, seed=None):
+        y = ops.attention_softmax_fwd(x, dropout if training else 0.0, use_causal_mask, seed)
         ctx.save_for_backward(y)
         ctx.use_causal_mask = use_causal_mask
         return y
@@ -566,17 +567,19 @@ class AttentionSoftmaxFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, y_grad):
         y, = ctx.saved_tensors
-        return ops.attention_softmax_bwd(y_grad, y, ctx.use_causal_mask), None, None, None
+        return ops.attention_softmax_bwd(y_grad, y, ctx.use_causal_mask), None, None, None, None
 
 
 class AttentionFunc(torch.autograd.Function):
-    """fairseq/modules/efficient_attention.py:11-40 (dropout = 0): the forward keeps the L x L
-    weights for the backward pass, as the reference does."""
+    """fairseq/modules/efficient_attention.py:11-40: the forward keeps the L x L weights (after
+    DropKey) for the backward pass, as the reference does.  `seed` (not in the reference) pins
+    the mask."""
 
     @staticmethod
     def forward(ctx, q, k, v, scale: float = 1.0, dropout: float = 0.0, use_causal_mask: bool = True,
-                training: bool = True):
-        y, w = ops.attention_fwd(q, k, v, scale, dropout if training else 0.0, use_causal_mask, need_weights=True)
+                training: bool = True, seed=None):
+        y, w = ops.attention_fwd(q, k, v, scale, dropout if training else 0.0, use_causal_mask, need_weights=True,
+                                 seed=seed)
         ctx.save_for_backward(q, k, v, w)
         ctx.scale = scale
         ctx.use_causal_mask = use_causal_mask
@@ -586,7 +589,7 @@ class AttentionFunc(torch.autograd.Function):
     def backward(ctx, y_grad):
         q, k, v, w = ctx.saved_tensors
         q_grad, k_grad, v_grad = ops.attention_bwd(y_grad, q, k, v, w, ctx.scale, ctx.use_causal_mask)
-        return q_grad, k_grad, v_grad, None, None, None, None
+        return q_grad, k_grad, v_grad, None, None, None, None, None
 
 
 attention_softmax = AttentionSoftmaxFunc.apply

@@ -5,7 +5,7 @@ argument order and return tuples, plus the fused inference entry points the modu
 Every function takes torch tensors that live on a HIP device, allocates its outputs with
 torch (so they belong to the caller, as torch::empty_like does in the reference), and
 enqueues the HIP kernels of libmega_hip.so on torch's current stream.  CPU tensors are
-rejected: there is no fallback.  Forward only (inference); dropout must be 0.
+rejected: there is no fallback.
 """
 from __future__ import annotations
 
@@ -402,10 +402,24 @@ def sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, length_
     return group_sequence_norm_bwd(y_grad, x, count, mean, rstd, gamma, padding_mask, H, length_last)
 
 
-def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool) -> torch.Tensor:
-    """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18."""
-    if dropout != 0.0:
-        raise RuntimeError("attention_softmax_fwd: DropKey dropout (training) is not implemented; pass 0")
+def _dropkey_seed(dropout: float, seed: Optional[int]) -> int:
+    """The 64-bit seed that names a DropKey mask: the caller's, or one drawn from torch's CPU
+    generator (so torch.manual_seed makes a run repeatable, as it does for the reference's Philox
+    offsets, fairseq/csrc/ops/attention_softmax_kernel.cu:44-55)."""
+    if not 0.0 <= dropout <= 1.0:
+        raise RuntimeError("dropout must lie in [0, 1]")
+    if dropout == 0.0:
+        return 0
+    if seed is None:
+        seed = int(torch.randint(0, 2 ** 62, (1,), dtype=torch.int64).item())
+    return seed & (2 ** 64 - 1)
+
+
+def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool,
+                          seed: Optional[int] = None) -> torch.Tensor:
+    """Reference: attention_softmax_fwd, fairseq/csrc/ops/attention_softmax.cc:6-18.  `dropout` is
+    DropKey (scores set to -inf with that probability before the softmax); `seed` names the mask."""
+    seed = _dropkey_seed(dropout, seed)
     dev = _need_gpu(x)
     lib = _lib.load()
     if x.dim() < 2:
@@ -416,16 +430,18 @@ def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool
     y = torch.empty_like(xd)
     with _on_device(dev):
         rc = lib.mega_attention_softmax_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), batch, outer, inner,
-                                            1 if use_causal_mask else 0, _stream(dev))
+                                            1 if use_causal_mask else 0, float(dropout), seed, _stream(dev))
     _lib.check(rc, "attention_softmax_fwd")
     return y
 
 
-def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, need_weights: bool = False):
+def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, need_weights: bool = False,
+                  seed: Optional[int] = None):
     """-> (y[B,L,Nh,H2], w[B,Nh,L,L] or None).  Reference: attention_fwd,
-    fairseq/csrc/ops/attention_kernel.cu:40-131; the L x L weights are only written on request."""
-    if dropout != 0.0:
-        raise RuntimeError("attention_fwd: dropout (training) is not implemented; pass 0")
+    fairseq/csrc/ops/attention_kernel.cu:40-131; the L x L weights are only written on request.
+    `dropout` is DropKey on the scaled scores, `seed` names the mask (shared with
+    attention_softmax_fwd on the [B,Nh,L,L] scores)."""
+    seed = _dropkey_seed(dropout, seed)
     dev = _need_gpu(q, k, v)
     lib = _lib.load()
     if q.dim() != 4 or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
@@ -441,8 +457,8 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
     ws = _scratch_buffer(dev, nws) if nws else None
     with _on_device(dev):
         rc = lib.mega_attention_fwd(_ptr(qd), _ptr(kd), _ptr(vd), _ptr(y), _ptr(w), _dtype_code(qd), B, L, Nh, H1, H2,
-                                    float(scale), 1 if use_causal_mask else 0, _ptr(ws), ws.numel() if nws else 0,
-                                    _stream(dev))
+                                    float(scale), 1 if use_causal_mask else 0, float(dropout), seed, _ptr(ws),
+                                    ws.numel() if nws else 0, _stream(dev))
     _lib.check(rc, "attention_fwd")
     return y, w
 

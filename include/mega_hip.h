@@ -282,11 +282,17 @@ int mega_group_sequence_norm_bwd(const void* y_grad, const void* x, int dtype, c
 /* ------------------------------------------------------------------------ */
 /* Attention softmax and the fused attention op                              */
 /* stands in for attention_softmax_fwd (fairseq/csrc/ops/attention_softmax.cc:6-18,
- * ops/attention_softmax_kernel.cu:22-64, softmax.cuh:90-153), dropout = 0.
+ * ops/attention_softmax_kernel.cu:22-64, softmax.cuh:90-185).
  *   x, y [batch, outer, inner] contiguous of `dtype`; causal: row r keeps the first
- *   inner - outer + r + 1 columns; a fully masked row becomes zeros.              */
+ *   inner - outer + r + 1 columns; a fully masked row becomes zeros.
+ *   dropout in [0, 1] is DropKey (softmax.cuh:157-185): each score is replaced by -inf with
+ *   that probability before the softmax.  The reference draws from the Philox stream of its
+ *   CUDA generator; here the draw for element e of the flattened input is a counter-based hash
+ *   of (seed, e), so one seed names one mask, for this op and for mega_attention_fwd alike.
+ *   dropout = 0 ignores the seed.                                                       */
 int mega_attention_softmax_fwd(const void* x, void* y, int dtype, int64_t batch, int64_t outer,
-                               int64_t inner, int causal, void* stream);
+                               int64_t inner, int causal, float dropout, uint64_t seed,
+                               void* stream);
 /* stands in for attention_softmax_bwd (fairseq/csrc/ops/attention_softmax.cc:20-26,
  * softmax.cuh AttentionSoftmaxBwdKernel; also the middle step of attention_bwd,
  * ops/attention_kernel.cu:195-203):
@@ -296,10 +302,12 @@ int mega_attention_softmax_bwd(const void* y_grad, const void* y, void* x_grad, 
                                int64_t batch, int64_t outer, int64_t inner, int causal,
                                float scale, void* stream);
 
-/* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276),
- * dropout = 0:  q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;
+/* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276):
+ *   q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;
  *   y[b,:,n,:] = softmax_causal(scale q k^T) v per (b, n).  The L x L weights are
  *   not returned unless w != NULL (w [B,Nh,L,L] of `dtype`).
+ *   dropout, seed: DropKey on the scaled scores, as in mega_attention_softmax_fwd; element
+ *   e is the score's place in the [B,Nh,L,L] weights.
  *   16-bit activations with H1 % 8 == 0 run on the matrix cores and need the workspace
  *   (scores in fp32, probabilities and v^T in the activation type); other requests need
  *   none (mega_attention_workspace_bytes returns 0).                                   */
@@ -307,7 +315,8 @@ size_t mega_attention_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t N
                                       int64_t H2);
 int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, void* w, int dtype,
                        int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
-                       int causal, void* workspace, size_t workspace_bytes, void* stream);
+                       int causal, float dropout, uint64_t seed, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* SwiGLU gate: y = silu(a) * b, elementwise over n elements of `dtype`.

@@ -593,12 +593,29 @@ def timestep_norm_bwd(dy, dmean, dvar, x, prev_mean, count, group_mean, cummean,
 # --------------------------------------------------------------------------
 
 
-def attention_softmax(x, causal: bool = False):
-    """csrc/softmax.cuh:90-153: softmax over the last axis of x[..., R, C]; causal keeps
-    columns [0, C - R + r] of row r; a row whose maximum is -inf (or whose sum is 0)
-    becomes zeros."""
+def dropkey_draws(seed: int, shape):
+    """The uniform draws in [0, 1) the HIP kernels use for DropKey: draw e (the element's place in
+    the flattened score tensor) is the splitmix64 finaliser of seed + (e + 1) * golden ratio, top
+    24 bits.  The reference draws from Philox (csrc/softmax.cuh:157-185); which generator names the
+    mask is not part of the op's contract, only `draw < dropout -> -inf` is.  Restated here so a
+    test can hand the same mask to the fp64 softmax below."""
+    n = int(np.prod(shape))
+    with np.errstate(over='ignore'):
+        z = np.uint64(seed & (2 ** 64 - 1)) + (np.arange(n, dtype=np.uint64) + np.uint64(1)) * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    return ((z >> np.uint64(40)).astype(np.float64) / 16777216.0).reshape(shape)
+
+
+def attention_softmax(x, causal: bool = False, drop=None):
+    """csrc/softmax.cuh:90-185: softmax over the last axis of x[..., R, C]; causal keeps
+    columns [0, C - R + r] of row r; `drop` (boolean, x's shape) marks the keys DropKey replaces
+    by -inf first; a row whose maximum is -inf (or whose sum is 0) becomes zeros."""
     x = np.asarray(x, np.float64)
     R, C = x.shape[-2], x.shape[-1]
+    if drop is not None:
+        x = np.where(np.asarray(drop, bool), -np.inf, x)
     if causal:
         r = np.arange(R)[:, None]
         c = np.arange(C)[None, :]
@@ -611,14 +628,15 @@ def attention_softmax(x, causal: bool = False):
     return np.where(s > 0, e / np.where(s > 0, s, 1.0), 0.0)
 
 
-def attention(q, k, v, scale: float = 1.0, causal: bool = True):
+def attention(q, k, v, scale: float = 1.0, causal: bool = True, drop=None):
     """csrc/ops/attention_kernel.cu:40-131: q, k: [B, L, Nh, H1]; v: [B, L, Nh, H2];
-    w[b,n] = softmax_causal(scale q k^T); y[b,:,n,:] = w v.  Returns (y, w)."""
+    w[b,n] = softmax_causal(scale q k^T) with the keys marked in drop[B, Nh, L, L] removed;
+    y[b,:,n,:] = w v.  Returns (y, w)."""
     q = np.asarray(q, np.float64)
     k = np.asarray(k, np.float64)
     v = np.asarray(v, np.float64)
     s = np.einsum('blnh,bmnh->bnlm', q, k) * scale
-    w = attention_softmax(s, causal)
+    w = attention_softmax(s, causal, drop)
     y = np.einsum('bnlm,bmnh->blnh', w, v)
     return y, w
 
@@ -631,14 +649,14 @@ def attention_softmax_bwd(dy, y):
     return y * (dy - (y * dy).sum(-1, keepdims=True))
 
 
-def attention_bwd(dy, q, k, v, scale: float = 1.0, causal: bool = True):
+def attention_bwd(dy, q, k, v, scale: float = 1.0, causal: bool = True, drop=None):
     """csrc/ops/attention_kernel.cu:133-255: dv = w^T dy, dw = dy v^T, ds = softmax_bwd(dw, w),
     dk = scale ds^T q, dq = scale ds k per (batch, head).  Returns (dq, dk, dv)."""
     dy = np.asarray(dy, np.float64)
     q = np.asarray(q, np.float64)
     k = np.asarray(k, np.float64)
     v = np.asarray(v, np.float64)
-    _, w = attention(q, k, v, scale, causal)
+    _, w = attention(q, k, v, scale, causal, drop)
     dv = np.einsum('bnlm,blnh->bmnh', w, dy)
     dw = np.einsum('blnh,bmnh->bnlm', dy, v)
     ds = attention_softmax_bwd(dw, w)

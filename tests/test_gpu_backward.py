@@ -525,3 +525,34 @@ def test_explicit_kernel_convolution_autograd():
         dx[:, :, :L - l] += w64[:, :, l:] * k64[None, :, l:l + 1]
         dk[:, l] = (w64[:, :, l:] * x64[:, :, :L - l]).sum(axis=(0, 2))
     assert rel_err(host(x.grad), dx) < 1e-4 and rel_err(host(k.grad), dk) < 1e-4
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])
+def test_attention_dropkey_autograd(dtype, tol):
+    """Training with DropKey: the backward runs on the saved weights, which hold zeros at the dropped
+    keys, so the gradients are those of the oracle with the same mask."""
+    rng = np.random.default_rng(74)
+    B, L, Nh, H1, H2 = 2, 64, 2, 16, 32
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    p, seed = 0.25, 424242
+    drop = O.dropkey_draws(seed, (B, Nh, L, L)) < p
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    y = M.modules.attention(q, k, v, 0.5, p, True, True, seed)
+    (y * dy).sum().backward()
+    assert rel_err(host(y), O.attention(q64, k64, v64, 0.5, True, drop)[0]) < TOL[dtype]
+    for got, ref in zip((q.grad, k.grad, v.grad), O.attention_bwd(dy64, q64, k64, v64, 0.5, True, drop)):
+        e = host(got) - ref
+        rms = np.sqrt((ref ** 2).mean())
+        assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
+    # the softmax op alone
+    x, x64 = rounded(rng.normal(size=(3, 20, 20)) * 2, dtype)
+    g, g64 = rounded(rng.normal(size=(3, 20, 20)), dtype)
+    xg = x.clone().requires_grad_(True)
+    yy = M.modules.attention_softmax(xg, p, False, True, seed)
+    (yy * g).sum().backward()
+    ref = O.attention_softmax_bwd(g64, host(yy))
+    assert rel_err(host(xg.grad), ref) < TOL[dtype]
+    assert np.all(host(xg.grad)[O.dropkey_draws(seed, (3, 20, 20)) < p] == 0)

@@ -290,3 +290,38 @@ def test_decoder_model_names_streaming_and_training():
     loss = torch.nn.functional.cross_entropy(logits.reshape(-1, vocab).float(), tokens[:, 1:].reshape(-1))
     loss.backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+def test_layer_dropouts_act_in_training_only():
+    """dropout / hidden_dropout / attention_dropout (moving_average_gated_attention.py:64-79, 316,
+    407-410): identity in eval mode; in training mode they change the output, follow torch's seed,
+    and with all three at zero the training path equals the inference path."""
+    torch.manual_seed(3)
+    D, S, E, N, C = 32, 16, 48, 4, 16
+    kw = dict(chunk_size=C, norm_num_groups=4, moving_act='silu')
+    plain = M.MovingAverageGatedAttention(D, S, E, N, **kw).to(DEV)
+    drop = M.MovingAverageGatedAttention(D, S, E, N, dropout=0.1, attention_dropout=0.2, hidden_dropout=0.1,
+                                         **kw).to(DEV)
+    drop.load_state_dict(plain.state_dict())
+    x = torch.randn(2, 64, D, device=DEV)
+    with torch.no_grad():
+        ref = plain.eval()(x)[0]
+        assert torch.equal(drop.eval()(x)[0], ref)
+        torch.manual_seed(7)
+        a = drop.train()(x)[0]
+        torch.manual_seed(7)
+        b = drop(x)[0]
+        assert torch.equal(a, b) and not torch.allclose(a, ref, atol=1e-4)
+        assert torch.isfinite(a).all()
+    # each dropout alone reaches the output, and gradients flow through the dropped layer
+    for name in ('dropout', 'attention_dropout', 'hidden_dropout'):
+        one = M.MovingAverageGatedAttention(D, S, E, N, **{name: 0.3}, **kw).to(DEV).train()
+        one.load_state_dict(plain.state_dict())
+        xg = x.clone().requires_grad_(True)
+        y = one(xg)[0]
+        assert not torch.allclose(y.detach(), ref, atol=1e-5), name
+        y.square().sum().backward()
+        assert torch.isfinite(xg.grad).all() and all(torch.isfinite(p.grad).all() for p in one.parameters()
+                                                     if p.grad is not None)
+    f = M.NormalizedFeedForwardNetwork(D, 64, dropout=0.2, hidden_dropout=0.2).to(DEV)
+    assert torch.equal(f.eval()(x), f(x)) and not torch.equal(f.train()(x), f.eval()(x))

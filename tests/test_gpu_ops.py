@@ -239,3 +239,65 @@ def test_sequence_norm_module_and_edge_cases():
     assert rel_err(host(y), yo) < 1e-4 and torch.isfinite(y).all() and float(y[1].abs().max()) == 0.0
     with pytest.raises(RuntimeError):
         M.ops.group_sequence_norm_fwd(dev(x64), dev(np.ones(H)), dev(np.zeros(H)), None, 5, 1e-5, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape,causal", [((3, 5, 40, 40), True), ((2, 17, 300), False), ((2, 64, 2048), True)])
+def test_attention_softmax_dropkey(dtype, shape, causal):
+    """DropKey (softmax.cuh:157-185): the keys whose draw falls below `dropout` get weight zero, the
+    others the softmax over the survivors; the mask is the one the seed names."""
+    rng = np.random.default_rng(27)
+    x, x64 = rounded(rng.normal(size=shape) * 2, dtype)
+    p, seed = 0.3, 0x1234_5678_9ABC_DEF1
+    y = M.ops.attention_softmax_fwd(x, p, causal, seed=seed)
+    drop = O.dropkey_draws(seed, shape) < p
+    yo = O.attention_softmax(x64, causal, drop)
+    assert np.abs(host(y) - yo).max() < (1e-5 if dtype == torch.float32 else 4e-3)
+    assert np.all(host(y)[drop] == 0)
+    assert torch.equal(y, M.ops.attention_softmax_fwd(x, p, causal, seed=seed))
+    y2 = M.ops.attention_softmax_fwd(x, p, causal, seed=seed + 1)
+    assert not torch.equal(y, y2)
+    # the mask has the asked-for rate and does not repeat from row to row
+    assert abs(drop.mean() - p) < 5 * np.sqrt(p * (1 - p) / drop.size) + 1e-3
+    d2 = drop.reshape(-1, shape[-1])
+    assert abs((d2[:-1] & d2[1:]).mean() - p * p) < 0.01
+    # eval mode and dropout = 0 ignore it
+    mod = M.AttentionSoftmax(dropout=p, use_causal_mask=causal)
+    assert torch.equal(mod.eval()(x), M.ops.attention_softmax_fwd(x, 0.0, causal))
+    torch.manual_seed(5)
+    a = mod.train()(x)
+    torch.manual_seed(5)
+    assert torch.equal(a, mod(x)) and not torch.equal(a, mod(x))
+
+
+def test_attention_softmax_dropkey_extremes():
+    x = torch.randn(2, 8, 8, device=DEV)
+    assert torch.all(M.ops.attention_softmax_fwd(x, 1.0, False, seed=3) == 0)      # every key dropped: zero rows
+    with pytest.raises(RuntimeError):
+        M.ops.attention_softmax_fwd(x, 1.5, False)
+    with pytest.raises(RuntimeError):
+        M.ops.attention_fwd(x[..., None], x[..., None], x[..., None], 1.0, -0.1, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,Nh,H1,H2", [(2, 50, 1, 16, 24), (1, 130, 4, 32, 64), (2, 300, 2, 64, 256)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_dropkey(dtype, B, L, Nh, H1, H2, causal):
+    """The fused op (row kernel for fp32, matrix-core path for bf16) drops the same keys as the softmax
+    op does on the [B,Nh,L,L] scores."""
+    rng = np.random.default_rng(28)
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    p, seed = 0.2, 987654321
+    drop = O.dropkey_draws(seed, (B, Nh, L, L)) < p
+    y, w = M.ops.attention_fwd(q, k, v, 0.8, p, causal, need_weights=True, seed=seed)
+    yo, wo = O.attention(q64, k64, v64, 0.8, causal, drop)
+    assert rel_err(host(y), yo, eps=2.0) < TOL[dtype]
+    assert np.abs(host(w) - wo).max() < (1e-5 if dtype == torch.float32 else 4e-3)
+    assert np.all(host(w)[drop] == 0)
+    y1, _ = M.ops.attention_fwd(q, k, v, 0.8, p, causal, seed=seed)
+    assert rel_err(host(y1), host(y), eps=2.0) < 2 * TOL[dtype]
+    # no dropout afterwards: the workspace keeps nothing of the mask
+    y0, _ = M.ops.attention_fwd(q, k, v, 0.8, 0.0, causal)
+    assert rel_err(host(y0), O.attention(q64, k64, v64, 0.8, causal)[0], eps=2.0) < TOL[dtype]

@@ -88,3 +88,47 @@ def test_layer_gate_closed_forms_and_chunk_causality():
     assert np.allclose(O.rms_norm(z, None, 1e-5), z / np.sqrt((z ** 2).mean(-1, keepdims=True) + 1e-5))
     yh = O.gated_attention_layer(x, P, chunk=4, num_heads=2, num_groups=2)
     assert yh.shape == y.shape and not np.allclose(yh, y)
+
+
+def test_dropkey_draws_and_masked_softmax(tmp_path):
+    """The draws: against a C restatement of the hash (64-bit wrap-around and the 24-bit float
+    conversion are where numpy could differ), uniform, independent from row to row.  The masked
+    softmax: equal to the plain softmax over the surviving keys, zeros at dropped keys and in rows
+    that lose every key (softmax.cuh:157-185)."""
+    import subprocess
+    src = tmp_path / "h.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <stdint.h>
+int main(void) {
+  const uint64_t seeds[2] = {12345ull, 0xFEDCBA9876543210ull};
+  for (int s = 0; s < 2; ++s)
+    for (uint64_t i = 0; i < 64; ++i) {
+      uint64_t z = seeds[s] + (i + 1) * 0x9E3779B97F4A7C15ull;
+      z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+      z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+      z ^= z >> 31;
+      printf("%.9g\n", (float)(z >> 40) * (1.0f / 16777216.0f));
+    }
+  return 0;
+}''')
+    exe = tmp_path / "h"
+    subprocess.run(["gcc", "-O1", str(src), "-o", str(exe)], check=True)
+    out = np.array([float(t) for t in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                     text=True).stdout.split()])
+    got = np.concatenate([O.dropkey_draws(12345, (64,)), O.dropkey_draws(0xFEDCBA9876543210, (8, 8)).ravel()])
+    assert np.array_equal(out, got)
+    d = O.dropkey_draws(99, (2000, 500))
+    assert 0 <= d.min() and d.max() < 1 and abs(d.mean() - 0.5) < 2e-3 and abs(d.var() - 1 / 12) < 1e-3
+    assert abs(np.corrcoef(d[:-1].ravel(), d[1:].ravel())[0, 1]) < 5e-3
+    assert abs(np.corrcoef(d[:, :-1].ravel(), d[:, 1:].ravel())[0, 1]) < 5e-3
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(3, 6, 9))
+    drop = O.dropkey_draws(7, x.shape) < 0.4
+    drop[1, 2] = True                                   # a row that loses every key
+    y = O.attention_softmax(x, False, drop)
+    assert np.all(y[drop] == 0) and np.all(y[1, 2] == 0)
+    for b, r in [(0, 0), (2, 5), (1, 3)]:
+        keep = ~drop[b, r]
+        e = np.exp(x[b, r, keep] - x[b, r, keep].max())
+        assert np.allclose(y[b, r, keep], e / e.sum(), atol=1e-15)
