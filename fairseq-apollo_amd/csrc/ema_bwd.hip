@@ -19,6 +19,15 @@
 #include "common.h"
 
 namespace mega {
+
+// matrix-core form of the sums (ema_bwd_tile.hip)
+bool ema_param_grad_tile_covers(int dtype, const void* dy, const void* x, int64_t sgb, int64_t sgd, int64_t sgl,
+                                int64_t sxb, int64_t sxd, int64_t sxl, const uint8_t* mask, int64_t B, int64_t D,
+                                int64_t N, int64_t L, int lag_one);
+void ema_param_grad_tile_launch(const void* dy, const void* x, int64_t sgb, int64_t sgd, int64_t sgl, int64_t sxb,
+                                int64_t sxd, int64_t sxl, const float* q, int64_t B, int64_t D, int64_t N, int64_t L,
+                                float* sums, float* dyx, hipStream_t s);
+
 namespace {
 
 constexpr int kNs = 16;        // state lanes per channel
@@ -242,6 +251,15 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
   A.sums = (float*)workspace;
   A.dyx = (float*)((char*)workspace + align_up((size_t)B * D * N * 16, 256));
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+  if (ema_param_grad_tile_covers(dtype, A.dy, A.x, A.sgb, A.sgd, A.sgl, A.sxb, A.sxd, A.sxl, mask, B, D, N, L,
+                                 lag_one)) {
+    ema_param_grad_tile_launch(A.dy, A.x, A.sgb, A.sgd, A.sgl, A.sxb, A.sxd, A.sxl, q, B, D, N, L, A.sums, A.dyx, s);
+    MEGA_CHECK_LAUNCH("ema_param_grad (matrix-core form)");
+    hipLaunchKernelGGL(ema_grad_finalize_kernel, dim3((unsigned)ceil_div(D * N, 256)), dim3(256), 0, s, A.sums, A.dyx,
+                       p, gamma, (int)B, (int)D, (int)N, dp, dq, dgamma, domega);
+    MEGA_CHECK_LAUNCH("ema_param_grad (finalize)");
+    return MEGA_OK;
+  }
   // 16 channels per workgroup, 8 when that would leave compute units idle
   static int cu_count[64] = {0};     // per device, queried once
   int cus = 256;

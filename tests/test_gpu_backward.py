@@ -121,6 +121,8 @@ def _ema_coeffs(rng, D, N, cplx):
     (2, 24, 16, 300, True, "bld", True),      # generic path, padding
     (3, 20, 2, 77, False, "bdl", True),       # real layer, two states
     (2, 40, 7, 129, True, "bld", False),      # odd state count
+    (2, 16, 16, 1544, True, "mixed", False),  # x with channels contiguous, dy with rows in time; a partial last step
+    (1, 8, 16, 520, False, "bdl", False),     # real coefficients on the matrix-core sums
 ])
 def test_ema_backward(dtype, B, D, N, L, cplx, layout, masked):
     rng = np.random.default_rng(61)
@@ -131,8 +133,9 @@ def test_ema_backward(dtype, B, D, N, L, cplx, layout, masked):
     om = rng.normal(size=D).astype(np.float32).astype(np.float64)
     x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
     dy, dy64 = rounded(rng.normal(size=(B, D, L)), dtype)
-    if layout == "bld":
+    if layout in ("bld", "mixed"):
         x = x.transpose(1, 2).contiguous().transpose(1, 2)
+    if layout == "bld":
         dy = dy.transpose(1, 2).contiguous().transpose(1, 2)
     mask = (rng.random((B, L)) < 0.2) if masked else None
     tm = None if mask is None else torch.from_numpy(mask).to(DEV)
@@ -154,6 +157,7 @@ def test_ema_backward(dtype, B, D, N, L, cplx, layout, masked):
     (2, 32, 16, 2048, True, "bld", False),    # matrix-core path, both directions
     (2, 24, 16, 300, True, "bld", True),
     (1, 16, 4, 150, False, "bdl", True),      # backward kernel with its lag-0 tap
+    (2, 32, 16, 1100, False, "bld", False),   # lag-0 tap, no padding: the reversed half on the matrix-core sums
 ])
 def test_ema_backward_two_sided(dtype, B, D, N, L, shift, layout, masked):
     rng = np.random.default_rng(63)
