@@ -72,6 +72,7 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
   __shared__ __attribute__((aligned(16))) char s_x[kTCh * kRowB];
   __shared__ __attribute__((aligned(16))) char s_g[kTCh * kRowB];
   __shared__ __attribute__((aligned(16))) char s_out[kTCh * 16 * kTileB];
+  __shared__ __attribute__((aligned(16))) char s_zero[kStep];     // what the unused k slots of the data product read
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int col = lane & 15, r = lane >> 4;
   // workgroups that share the lines of a channel-contiguous operand get ids on one XCD
@@ -173,6 +174,7 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
   const char* grow = s_g + wave * kRowB;
   char* orow = s_out + wave * 16 * kTileB;
 
+  s_zero[tid] = 0;
   fetch(0);
   for (int t0 = 0; t0 < A.L; t0 += kStep) {
     park(s_x, px, A.x_chan_fast, xtok, t0 + xtok <= xlast);
@@ -185,32 +187,37 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
     const bf16x8 G = *(const bf16x8*)(grow + (32 * col + 8 * r) * 2);
     f32x4 Sa[2], Sad[2], Sb[2], Sbd[2];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      Sa[rb] = Sad[rb] = Sb[rb] = Sbd[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < 2; ++rb) Sa[rb] = Sad[rb] = Sb[rb] = Sbd[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // term by term, so that products into the same accumulator sit eight instructions apart
 #pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        Sa[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ta[w][rb], G, Sa[rb], 0, 0, 0);
-        Sad[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Tad[w][rb], G, Sad[rb], 0, 0, 0);
+    for (int w = 0; w < 2; ++w)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
         Sb[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Tb[w][rb], X, Sb[rb], 0, 0, 0);
         Sbd[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Tbd[w][rb], X, Sbd[rb], 0, 0, 0);
+        Sa[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ta[w][rb], G, Sa[rb], 0, 0, 0);
+        Sad[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Tad[w][rb], G, Sad[rb], 0, 0, 0);
       }
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
       // states 8 rb + 2r and + 1 of tile `col`: (b re, b im, bd re, bd im)
       char* o = orow + col * kTileB + (8 * rb + 2 * r) * 16;
       *(float4*)o = make_float4(Sb[rb][0], Sb[rb][1], Sbd[rb][0], Sbd[rb][1]);
       *(float4*)(o + 16) = make_float4(Sb[rb][2], Sb[rb][3], Sbd[rb][2], Sbd[rb][3]);
     }
-    // tile-local correlation: contraction over the 16 tiles (k slots 16..31 are zero)
+    // tile-local correlation: contraction over the 16 tiles; the k slots 16..31 (lanes with r >= 2)
+    // read a row of zeros
     {
+      const char* gsrc = r < 2 ? grow + (32 * 8 * r + col) * 2 : s_zero;
+      const char* xsrc = r < 2 ? xrow + (32 * 8 * r + col) * 2 : s_zero;
       bf16x8 Gt[2], Xt[2];
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const int off = (32 * (8 * (r & 1) + e) + 16 * hf + col) * 2;
-          const uint16_t gv = *(const uint16_t*)(grow + off);
-          const uint16_t xv = *(const uint16_t*)(xrow + off);
-          Gt[hf][e] = __builtin_bit_cast(__bf16, (uint16_t)(r < 2 ? gv : 0));
-          Xt[hf][e] = __builtin_bit_cast(__bf16, (uint16_t)(r < 2 ? xv : 0));
+          const int off = (32 * e + 16 * hf) * 2;
+          Gt[hf][e] = __builtin_bit_cast(__bf16, *(const uint16_t*)(gsrc + off));
+          Xt[hf][e] = __builtin_bit_cast(__bf16, *(const uint16_t*)(xsrc + off));
         }
       }
 #pragma unroll
@@ -224,15 +231,27 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
     // ---- scan over the 16 tiles: leave the state before each tile where its (b, bd) was
     if (tid < kTCh * 16) {
       char* o = s_out + sch * 16 * kTileB + sn * 16;
-#pragma unroll 4
-      for (int k = 0; k < 16; ++k) {
-        const float4 in = *(const float4*)(o + k * kTileB);
-        *(float4*)(o + k * kTileB) = make_float4(h.re, h.im, hd.re, hd.im);
-        const cfloat nhd = {fmaf(Q.re, hd.re, fmaf(-Q.im, hd.im, fmaf(Qd.re, h.re, fmaf(-Qd.im, h.im, in.z)))),
-                            fmaf(Q.re, hd.im, fmaf(Q.im, hd.re, fmaf(Qd.re, h.im, fmaf(Qd.im, h.re, in.w))))};
-        const cfloat nh = {fmaf(Q.re, h.re, fmaf(-Q.im, h.im, in.x)), fmaf(Q.re, h.im, fmaf(Q.im, h.re, in.y))};
-        h = nh;
-        hd = nhd;
+      // groups of four tiles: the next group's (b, bd) are on their way while this one is walked
+      float4 in[4], nx[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) in[i] = *(const float4*)(o + i * kTileB);
+#pragma unroll
+      for (int kg = 0; kg < 4; ++kg) {
+        if (kg < 3) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) nx[i] = *(const float4*)(o + (4 * kg + 4 + i) * kTileB);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          *(float4*)(o + (4 * kg + i) * kTileB) = make_float4(h.re, h.im, hd.re, hd.im);
+          const cfloat nhd = {fmaf(Q.re, hd.re, fmaf(-Q.im, hd.im, fmaf(Qd.re, h.re, fmaf(-Qd.im, h.im, in[i].z)))),
+                              fmaf(Q.re, hd.im, fmaf(Q.im, hd.re, fmaf(Qd.re, h.im, fmaf(Qd.im, h.re, in[i].w))))};
+          const cfloat nh = {fmaf(Q.re, h.re, fmaf(-Q.im, h.im, in[i].x)), fmaf(Q.re, h.im, fmaf(Q.im, h.re, in[i].y))};
+          h = nh;
+          hd = nhd;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) in[i] = nx[i];
       }
     }
     __syncthreads();
