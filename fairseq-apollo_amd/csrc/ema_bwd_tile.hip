@@ -83,6 +83,35 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
   const int c0 = (v - b * ncb) * kTCh;
   const int d = c0 + wave;                                  // this wave's channel
 
+  // ---- loads: one 16-byte piece of x and of dy per thread and step
+  // channel-contiguous operand: thread <-> token, the piece holds the 8 channels;
+  // time-contiguous operand: thread <-> (channel, group of 8 tokens)
+  const int lmax = A.L - 1;
+  const uint16_t* xb = A.x + (int64_t)b * A.sxb + (A.x_chan_fast ? (int64_t)c0 : (int64_t)(c0 + (tid >> 6)) * A.sxd);
+  const uint16_t* gb = A.dy + (int64_t)b * A.sgb + (A.g_chan_fast ? (int64_t)c0 : (int64_t)(c0 + (tid >> 6)) * A.sgd);
+  const int xtok = A.x_chan_fast ? tid : 8 * (tid & 63);      // first token of the piece inside a step
+  const int gtok = A.g_chan_fast ? tid : 8 * (tid & 63);
+  const int xlast = A.x_chan_fast ? lmax : A.L - 8;           // last valid first-token
+  const int glast = A.g_chan_fast ? lmax : A.L - 8;
+  uint4 px, pg;
+  auto fetch = [&](int t0) {
+    px = *(const uint4*)(xb + (int64_t)min(t0 + xtok, xlast) * A.sxl);
+    pg = *(const uint4*)(gb + (int64_t)min(t0 + gtok, glast) * A.sgl);
+  };
+  auto park = [&](char* base, const uint4& p, bool chan_fast, int tok, bool valid) {
+    const uint4 z = valid ? p : make_uint4(0u, 0u, 0u, 0u);
+    if (chan_fast) {
+      const uint32_t w[4] = {z.x, z.y, z.z, z.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        *(uint16_t*)(base + e * kRowB + tok * 2) = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
+    } else {
+      *(uint4*)(base + (tid >> 6) * kRowB + tok * 2) = z;
+    }
+  };
+
+  fetch(0);                                  // in flight while the tables are built
+
   // ---- constant operands: rows = (state, re | im), 16 rows per block, columns = token in tile
   bf16x8 Ta[2][2], Tad[2][2], Tb[2][2], Tbd[2][2];          // [term][row block]
 #pragma unroll
@@ -135,33 +164,6 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
     Qd = {32.f * q31.re, 32.f * q31.im};
   }
 
-  // ---- loads: one 16-byte piece of x and of dy per thread and step
-  // channel-contiguous operand: thread <-> token, the piece holds the 8 channels;
-  // time-contiguous operand: thread <-> (channel, group of 8 tokens)
-  const int lmax = A.L - 1;
-  const uint16_t* xb = A.x + (int64_t)b * A.sxb + (A.x_chan_fast ? (int64_t)c0 : (int64_t)(c0 + (tid >> 6)) * A.sxd);
-  const uint16_t* gb = A.dy + (int64_t)b * A.sgb + (A.g_chan_fast ? (int64_t)c0 : (int64_t)(c0 + (tid >> 6)) * A.sgd);
-  const int xtok = A.x_chan_fast ? tid : 8 * (tid & 63);      // first token of the piece inside a step
-  const int gtok = A.g_chan_fast ? tid : 8 * (tid & 63);
-  const int xlast = A.x_chan_fast ? lmax : A.L - 8;           // last valid first-token
-  const int glast = A.g_chan_fast ? lmax : A.L - 8;
-  uint4 px, pg;
-  auto fetch = [&](int t0) {
-    px = *(const uint4*)(xb + (int64_t)min(t0 + xtok, xlast) * A.sxl);
-    pg = *(const uint4*)(gb + (int64_t)min(t0 + gtok, glast) * A.sgl);
-  };
-  auto park = [&](char* base, const uint4& p, bool chan_fast, int tok, bool valid) {
-    const uint4 z = valid ? p : make_uint4(0u, 0u, 0u, 0u);
-    if (chan_fast) {
-      const uint32_t w[4] = {z.x, z.y, z.z, z.w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        *(uint16_t*)(base + e * kRowB + tok * 2) = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
-    } else {
-      *(uint4*)(base + (tid >> 6) * kRowB + tok * 2) = z;
-    }
-  };
-
   f32x4 S2a[2], S1a[2];                      // per row block: (state 2r: re, im, state 2r+1: re, im) partial sums
   f32x4 M[2][2];                             // tile-local correlation, blocks [dy half][x half]
 #pragma unroll
@@ -175,7 +177,6 @@ __global__ __launch_bounds__(kTThreads) void ema_param_grad_tile_kernel(const Ti
   char* orow = s_out + wave * 16 * kTileB;
 
   s_zero[tid] = 0;
-  fetch(0);
   for (int t0 = 0; t0 < A.L; t0 += kStep) {
     park(s_x, px, A.x_chan_fast, xtok, t0 + xtok <= xlast);
     park(s_g, pg, A.g_chan_fast, gtok, t0 + gtok <= glast);
