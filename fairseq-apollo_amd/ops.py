@@ -753,12 +753,60 @@ def fftconv(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     return _long_conv(x, k, False, True)
 
 
-def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor):
-    """-> (x_grad [B,D,L], k_grad [D,Lk] fp32) of y = fftconv(x, k): the two correlations of
+def _rfft_len(L: int) -> int:
+    """Length of the real transform the reference's convolution uses: 2 * pow2ceil(L)
+    (fused_ops/fftconv.py:17-18, 47)."""
+    N = L if (L & (L - 1)) == 0 else (1 << L.bit_length())
+    return 2 * N
+
+
+def rfft(x: torch.Tensor, flip: bool = False) -> torch.Tensor:
+    """Reference: rfft, fairseq/csrc/ops/fftconv.cc:6-8 (ops/fftconv_kernel.cu:23-44, 169-212): the
+    unnormalised real transform of length 2 * pow2ceil(L) over the last axis, of the time-reversed
+    signal when `flip` -> [..., pow2ceil(L) + 1] complex64.  The kernels of this library work in the
+    time domain; the operator exists for callers written against the reference's extension and runs
+    the library transform."""
+    _need_gpu(x)
+    xf = x.detach().float()
+    return torch.fft.rfft(xf.flip(-1) if flip else xf, n=_rfft_len(x.size(-1)))
+
+
+def _from_spectrum(t_f: torch.Tensor, L: int, what: str) -> torch.Tensor:
+    n = _rfft_len(L)
+    if not t_f.is_complex() or t_f.size(-1) != n // 2 + 1:
+        raise RuntimeError(f"{what} must be a complex spectrum with {n // 2 + 1} bins for L = {L}")
+    return torch.fft.irfft(t_f, n=n)[..., :L]
+
+
+def fftconv_fwd(x: torch.Tensor, k_f: torch.Tensor):
+    """-> (y [B,H,L] of x's dtype, x_f [B,H,pow2ceil(L)+1] complex64).  Reference: fftconv_fwd,
+    fairseq/csrc/ops/fftconv.cc:10-13 (ops/fftconv_kernel.cu:46-78, 214-269): the causal convolution
+    with the kernel given as its spectrum k_f = rfft(k).  The first L taps are taken back out of the
+    spectrum and the convolution runs in the time domain; x_f is produced because the reference's
+    autograd function saves it.  No L <= 8192 limit."""
+    _need_gpu(x, k_f)
+    if x.dim() != 3:
+        raise RuntimeError("fftconv_fwd: x must be [B, H, L]")
+    L = x.size(-1)
+    k = _from_spectrum(k_f, L, "k_f").float().contiguous()
+    return _long_conv(x, k, False, True), rfft(x, False)
+
+
+def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, k_dtype: Optional[torch.dtype] = None):
+    """-> (x_grad [B,D,L], k_grad [D,Lk]) of y = fftconv(x, k): the two correlations of
     fused_ops/fftconv.py:66-88 (x_grad[t] = sum_l k[l] dy[t+l], k_grad[l] = sum_{b,t} dy[t] x[t-l]) as
     causal convolutions of the time-reversed gradient, through the same explicit-kernel op (a
-    correctness path, O(L Lk) per row; the modules use ema_backward, which forms neither k nor k_grad)."""
+    correctness path, O(L Lk) per row; the modules use ema_backward, which forms neither k nor k_grad).
+    Two call forms: (y_grad, x, k) in the time domain (k_grad in fp32), and the reference's
+    fftconv_bwd(y_grad, x_f, k_f, k_dtype) (fairseq/csrc/ops/fftconv.cc:15-20) with the spectra its
+    forward saved, k_grad [D, L] in k_dtype."""
     _need_gpu(y_grad, x, k)
+    if x.is_complex() or k.is_complex():
+        L = y_grad.size(-1)
+        xt = _from_spectrum(x, L, "x_f").to(y_grad.dtype)
+        kt = _from_spectrum(k, L, "k_f").float().contiguous()
+        x_grad, k_grad = fftconv_bwd(y_grad, xt, kt)
+        return x_grad, k_grad.to(k_dtype if k_dtype is not None else torch.float32)
     B, D, L = x.shape
     Lk = k.shape[1]
     r = y_grad.detach().to(x.dtype).flip(-1).contiguous()              # r[t] = dy[L-1-t]

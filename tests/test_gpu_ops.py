@@ -301,3 +301,39 @@ def test_attention_dropkey(dtype, B, L, Nh, H1, H2, causal):
     # no dropout afterwards: the workspace keeps nothing of the mask
     y0, _ = M.ops.attention_fwd(q, k, v, 0.8, 0.0, causal)
     assert rel_err(host(y0), O.attention(q64, k64, v64, 0.8, causal)[0], eps=2.0) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L", [700, 1024, 33])
+def test_spectral_convolution_operators(dtype, L):
+    """rfft / fftconv_fwd / fftconv_bwd under the reference's names and call forms
+    (fused_ops/fftconv.py:14-41): spectra are unnormalised transforms of length 2 * pow2ceil(L)."""
+    rng = np.random.default_rng(29)
+    B, D = 2, 6
+    n = 2 * O.pow2ceil(L)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    k = (rng.normal(size=(D, L)) * 0.2).astype(np.float32)
+    dy, dy64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    k_f = M.ops.rfft(dev(k), False)
+    assert k_f.shape == (D, n // 2 + 1) and k_f.dtype == torch.complex64
+    ref = np.fft.rfft(k.astype(np.float64), n=n)
+    assert rel_err(host(k_f).real, ref.real) < 1e-5 and rel_err(host(k_f).imag, ref.imag) < 1e-5
+    refl = np.fft.rfft(x64[..., ::-1], n=n)
+    got = host(M.ops.rfft(x, True))
+    assert rel_err(got.real, refl.real) < 1e-5 and rel_err(got.imag, refl.imag) < 1e-5
+    y, x_f = M.ops.fftconv_fwd(x, k_f)
+    assert y.dtype == dtype and x_f.shape == (B, D, n // 2 + 1)
+    assert rel_err(host(y), O.causal_conv(x64, k.astype(np.float64))) < TOL[dtype]
+    assert rel_err(host(x_f).real, np.fft.rfft(x64, n=n).real) < 1e-5
+    x_grad, k_grad = M.ops.fftconv_bwd(dy, x_f, k_f, torch.float32)
+    assert x_grad.dtype == dtype and k_grad.shape == (D, L) and k_grad.dtype == torch.float32
+    # x_grad[t] = sum_l k[l] dy[t+l]: the causal convolution of the reversed gradient, reversed
+    ref_xg = O.causal_conv(dy64[..., ::-1], k.astype(np.float64))[..., ::-1]
+    assert rel_err(host(x_grad), ref_xg) < TOL[dtype]
+    # k_grad[l] = sum_{b,t} dy[t] x[t-l]
+    ref_kg = np.stack([sum(np.correlate(dy64[b, d], x64[b, d], "full")[L - 1:] for b in range(B)) for d in range(D)])
+    assert rel_err(host(k_grad), ref_kg) < 2e-4
+    xt, kt = M.ops.fftconv_bwd(dy, x, dev(k))
+    assert rel_err(host(xt), host(x_grad)) < TOL[dtype] and rel_err(host(kt), host(k_grad)) < 1e-4
+    with pytest.raises(RuntimeError):
+        M.ops.fftconv_fwd(x, k_f[:, :-1])
