@@ -399,6 +399,20 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def _set_input_buffer(self, incremental_state, buffer):
         return self.set_incremental_state(incremental_state, "attn_state", buffer)
 
+    def reorder_incremental_state(self, incremental_state, new_order: Tensor):
+        """The cached keys / values follow a beam reordering
+        (moving_average_gated_attention.py:430-443); the norm and the moving average reorder their
+        own entries."""
+        input_buffer = self._get_input_buffer(incremental_state)
+        for name in list(input_buffer.keys()):
+            if input_buffer[name] is not None:
+                input_buffer[name] = input_buffer[name].index_select(0, new_order)
+        return self._set_input_buffer(incremental_state, input_buffer)
+
+    def extra_repr(self) -> str:
+        return 'edim={}, zdim={}, hdim={}, ndim={}, chunk={}, heads={}, bidir={}'.format(
+            self.embed_dim, self.zdim, self.hdim, self.ndim, self.chunk_size, self.num_heads, self.bidirectional)
+
 
 class Mega2Layer(nn.Module):
     """One Mega2 block of the north-star configuration: gated attention (TimestepNorm -> CEMA ->

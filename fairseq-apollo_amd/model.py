@@ -94,6 +94,14 @@ class MegaDecoderNoCrossAttn(nn.Module):
             x = x[:, :seq_len]
         return x, {"inner_states": inner_states}
 
+    def reorder_incremental_state(self, incremental_state, new_order: Tensor) -> None:
+        """Beam search keeps a subset / permutation of the streams: every module that carries state
+        reorders its own entries (fairseq/models/fairseq_incremental_decoder.py:82-96 walks the
+        module tree the same way)."""
+        for module in self.modules():
+            if module is not self and hasattr(module, 'reorder_incremental_state'):
+                module.reorder_incremental_state(incremental_state, new_order)
+
     def streamed(self, tokens: Tensor, chunk_size: Optional[int] = None) -> Tensor:
         """Logits of a document evaluated slice by slice with one incremental-state dictionary
         (fairseq_cli/train.py:406-417)."""

@@ -325,3 +325,25 @@ def test_layer_dropouts_act_in_training_only():
                                                      if p.grad is not None)
     f = M.NormalizedFeedForwardNetwork(D, 64, dropout=0.2, hidden_dropout=0.2).to(DEV)
     assert torch.equal(f.eval()(x), f(x)) and not torch.equal(f.train()(x), f.eval()(x))
+
+
+def test_decoder_model_beam_reorder():
+    """reorder_incremental_state: after some tokens the streams are permuted / duplicated as beam
+    search does (fairseq_incremental_decoder.py:82-96); decoding on equals decoding the reordered
+    streams from the start.  Single tokens, so the K/V chunk cache, the norm state and the
+    moving-average state all carry entries."""
+    torch.manual_seed(43)
+    args = _lm_args(decoder_layers=2, norm_eps=1e-5)
+    vocab = 40
+    model = M.MegaDecoderNoCrossAttn(args, vocab, torch.nn.Embedding(vocab, 64, padding_idx=1)).to(DEV).eval()
+    tokens = torch.randint(2, vocab, (3, 40), device=DEV)
+    order = torch.tensor([2, 0, 2], device=DEV)
+    with torch.no_grad():
+        state = {}
+        for t in range(25):
+            model(tokens[:, t:t + 1], incremental_state=state)
+        model.reorder_incremental_state(state, order)
+        got = torch.cat([model(tokens[order][:, t:t + 1], incremental_state=state)[0] for t in range(25, 40)], dim=1)
+        ref_state = {}
+        ref = torch.cat([model(tokens[order][:, t:t + 1], incremental_state=ref_state)[0] for t in range(40)], dim=1)
+    assert rel_err(host(got), host(ref[:, 25:])) < 1e-5
