@@ -31,6 +31,10 @@ void set_error(const char* fmt, ...);
   } while (0)
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Clears `bytes` (a multiple of 4) with a small kernel (elementwise.hip).  Used instead of a memset
+// node so that a caller may record any entry point into a HIP graph.
+void zero_async(void* p, size_t bytes, hipStream_t s);
 static inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
 
 // ---------------------------------------------------------------- row tiling of [tokens, H] tiles

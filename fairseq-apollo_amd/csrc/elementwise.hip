@@ -47,7 +47,20 @@ int launch_swiglu(const void* a, const void* b, void* y, int64_t n, hipStream_t 
   return MEGA_OK;
 }
 
+// zeros for small outputs of degenerate calls
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* __restrict__ p, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 }  // namespace
+
+void zero_async(void* p, size_t bytes, hipStream_t s) {
+  const size_t n = bytes / 4;
+  if (n == 0) return;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)ceil_div((int64_t)n, 256)), dim3(256), 0, s, (uint32_t*)p, n);
+}
+
 }  // namespace mega
 
 using namespace mega;

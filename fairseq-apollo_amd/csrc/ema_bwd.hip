@@ -228,10 +228,10 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
   MEGA_REQUIRE(p && q && gamma && dp && dq && dgamma && domega, MEGA_ERR_ARG, "ema_param_grad: null pointer argument");
   hipStream_t s = (hipStream_t)stream;
   if (B == 0 || L == 0) {
-    (void)hipMemsetAsync(dp, 0, (size_t)D * N * 4, s);
-    (void)hipMemsetAsync(dq, 0, (size_t)D * N * 8, s);
-    (void)hipMemsetAsync(dgamma, 0, (size_t)D * N * 8, s);
-    (void)hipMemsetAsync(domega, 0, (size_t)D * 4, s);
+    zero_async(dp, (size_t)D * N * 4, s);
+    zero_async(dq, (size_t)D * N * 8, s);
+    zero_async(dgamma, (size_t)D * N * 8, s);
+    zero_async(domega, (size_t)D * 4, s);
     return MEGA_OK;
   }
   MEGA_REQUIRE(dy && x, MEGA_ERR_ARG, "ema_param_grad: null dy / x");

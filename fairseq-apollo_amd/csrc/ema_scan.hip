@@ -569,7 +569,7 @@ extern "C" int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_
   hipStream_t s = (hipStream_t)stream;
   if (L == 0) {
     if (h) hipMemcpyAsync(h_out, h, (size_t)B * D * N * 8, hipMemcpyDeviceToDevice, s);
-    else hipMemsetAsync(h_out, 0, (size_t)B * D * N * 8, s);
+    else zero_async(h_out, (size_t)B * D * N * 8, s);
     return MEGA_OK;
   }
   const Plan pl = make_plan(B, D, N, L, 1, false);

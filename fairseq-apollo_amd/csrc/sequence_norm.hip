@@ -491,8 +491,8 @@ extern "C" int mega_group_sequence_norm_bwd(const void* y_grad, const void* x, i
   MEGA_REQUIRE(gamma_grad && beta_grad, MEGA_ERR_ARG, "sequence_norm_bwd: null gradient output");
   hipStream_t s = (hipStream_t)stream;
   if (B == 0) {
-    (void)hipMemsetAsync(gamma_grad, 0, (size_t)H * 4, s);
-    (void)hipMemsetAsync(beta_grad, 0, (size_t)H * 4, s);
+    zero_async(gamma_grad, (size_t)H * 4, s);
+    zero_async(beta_grad, (size_t)H * 4, s);
     return MEGA_OK;
   }
   MEGA_REQUIRE(y_grad && x && x_grad && count && mean && rstd && gamma, MEGA_ERR_ARG,

@@ -565,12 +565,12 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
     // nothing between the incoming state gradients and the outgoing ones
     if (B > 0) {
       if (mean_grad) hipMemcpyAsync(prev_mean_grad, mean_grad, (size_t)B * G * 4, hipMemcpyDeviceToDevice, s);
-      else hipMemsetAsync(prev_mean_grad, 0, (size_t)B * G * 4, s);
+      else zero_async(prev_mean_grad, (size_t)B * G * 4, s);
       if (var_grad) hipMemcpyAsync(prev_var_grad, var_grad, (size_t)B * G * 4, hipMemcpyDeviceToDevice, s);
-      else hipMemsetAsync(prev_var_grad, 0, (size_t)B * G * 4, s);
+      else zero_async(prev_var_grad, (size_t)B * G * 4, s);
     }
-    hipMemsetAsync(gamma_grad, 0, (size_t)H * 4, s);
-    hipMemsetAsync(beta_grad, 0, (size_t)H * 4, s);
+    zero_async(gamma_grad, (size_t)H * 4, s);
+    zero_async(beta_grad, (size_t)H * 4, s);
     return MEGA_OK;
   }
   MEGA_REQUIRE(y_grad && x && x_grad && prev_mean && count && cummean && cumrstd && gamma, MEGA_ERR_ARG,
