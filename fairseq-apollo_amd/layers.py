@@ -173,8 +173,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         # two hidden activations, DropKey inside the attention softmax; all three act in training mode only
         self.dropout_p, self.hidden_dropout_p = float(dropout), float(hidden_dropout)
         self.attention_dropout_p = float(attention_dropout)
-        if attention_activation != 'softmax':
-            raise NotImplementedError("only the softmax attention is built (no relu2 / laplace)")
+        if attention_activation not in ('softmax', 'relu2', 'laplace'):
+            raise ValueError('Unknown attention activation function: {}'.format(attention_activation))
+        self.attention_activation = attention_activation
         if rel_pos_bias not in ('rotary', 'simple'):
             raise ValueError('unknown relative position bias: {}'.format(rel_pos_bias))
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
@@ -251,7 +252,10 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             qk_gamma, qk_beta, freqs = self._qk_constants(simple)
             q, k = ops.gate_qk_fwd(z, qk_gamma, qk_beta, freqs, Nh, C)
             q4, k4, v4 = q.view(bsz * nc, C, Nh, -1), k.view(bsz * nc, C, Nh, -1), v.reshape(bsz * nc, C, Nh, -1)
-            if simple or (self.bidirectional and padding_mask is not None):
+            if self.attention_activation != 'softmax':
+                attn = self._element_attention(q4, k4, v4, None if padding_mask is None
+                                               else padding_mask.reshape(bsz * nc, C))
+            elif simple or (self.bidirectional and padding_mask is not None):
                 attn = self._padded_attention(q4, k4, v4, None if padding_mask is None or not self.bidirectional
                                               else padding_mask.reshape(bsz * nc, C))
             else:
@@ -299,6 +303,37 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             s = s.masked_fill(pad[:, None, None, :], float('-inf'))
         return torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
 
+    def _element_attention(self, q4: Tensor, k4: Tensor, v4: Tensor, key_padding: Optional[Tensor]) -> Tensor:
+        """The element-wise attention of moving_average_gated_attention.py:153-208 (relu2 / laplace in place
+        of the softmax): scores scaled by 1 / sqrt(number of keys a query sees), the learned bias added for
+        the simple position encoding, weights of padded keys and, in one-sided layers, of future keys set
+        to zero after the activation; plain dropout on the weights.  Library GEMMs and torch element-wise
+        operations."""
+        C = q4.size(1)
+        s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
+        if not self.bidirectional:
+            # the reference's lower-triangular attn_mask (models/mega_lm.py:391-410): query i sees i + 1 keys
+            scale = torch.rsqrt(torch.arange(1, C + 1, device=s.device, dtype=torch.float32)).to(s.dtype)[:, None]
+        elif key_padding is not None:
+            lengths = C - key_padding.to(torch.float32).sum(dim=-1)
+            scale = torch.rsqrt(lengths.clamp(min=1.0)).to(s.dtype)[:, None, None, None]
+        else:
+            scale = 1.0 / math.sqrt(C)
+        s = s * scale
+        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias):
+            s = s + self.rel_pos_bias(C).to(s.dtype)
+        if self.attention_activation == 'relu2':
+            w = torch.square(F.relu(s))
+        else:
+            # fairseq/utils.py:451-457: the logistic approximation of the Laplace attention function
+            w = torch.sigmoid((s - 0.707107) * (1.702 / 0.282095))
+        if key_padding is not None:
+            w = w * (~key_padding.to(torch.bool)).to(w.dtype)[:, None, None, :]
+        if not self.bidirectional:
+            w = w * torch.ones(C, C, device=w.device, dtype=w.dtype).tril_()
+        w = F.dropout(w, self.attention_dropout_p, self.training)
+        return torch.einsum('bnqk,bknh->bqnh', w, v4)
+
     def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
         """The same layer with a complete autograd graph (moving_average_gated_attention.py:263-417,
         whole chunks, no cache): TimestepNorm, the moving average and the attention carry their own
@@ -329,7 +364,10 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if not simple:
             q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
             k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
-        if simple or (self.bidirectional and padding_mask is not None):
+        if self.attention_activation != 'softmax':
+            attn = self._element_attention(q4, k4, v4, None if padding_mask is None
+                                           else padding_mask.reshape(bsz * nc, C))
+        elif simple or (self.bidirectional and padding_mask is not None):
             s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
             if simple:
                 s = s + self.rel_pos_bias(C).to(s.dtype)
@@ -353,9 +391,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         """Attention with the partial-chunk key / value cache
         (moving_average_gated_attention.py:332-372): keys are cached before the rotation, so the
         whole context is rotated again at every call."""
-        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias):
+        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias) or self.attention_activation != 'softmax':
             raise NotImplementedError("MovingAverageGatedAttention: incremental decoding is built for the rotary "
-                                      "position encoding only")
+                                      "position encoding and the softmax attention only")
         bsz, seq_len = z.shape[:2]
         Nh = self.num_heads
         z = F.normalize(z, p=2, dim=-1, eps=1e-5)

@@ -714,7 +714,7 @@ def rms_norm(x, weight=None, eps: float = 1e-5):
 
 def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str = 'silu', eps: float = 1e-5,
                           num_groups: Optional[int] = None, bidirectional: bool = False, padding_mask=None,
-                          simple_bias=None):
+                          simple_bias=None, attention_activation: str = 'softmax'):
     """MovingAverageGatedAttention.forward, unidirectional, softmax attention through the fused
     (rotary, causal, scale 1) op: modules/moving_average_gated_attention.py:263-417, step by
     step.  x: [B, L, D]; P: dict of numpy parameters
@@ -761,7 +761,29 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
         kr = rotary(kc.transpose(0, 2, 1, 3)).transpose(0, 2, 1, 3)
     else:
         qr, kr = qc, kc
-    if bidirectional or simple_bias is not None:
+    if attention_activation != 'softmax':
+        # element-wise attention (:153-208): scores over sqrt(keys seen), bias, relu^2 or the logistic
+        # approximation of the Laplace function (fairseq/utils.py:444-457), then the masks as factors
+        sc = np.einsum('blnh,bmnh->bnlm', qr, kr)
+        pad = None if padding_mask is None else np.asarray(padding_mask, bool).reshape(B * nc, C)
+        if not bidirectional:
+            sc = sc / np.sqrt(np.arange(1, C + 1))[:, None]
+        elif pad is not None:
+            sc = sc / np.sqrt(np.maximum(C - pad.sum(-1), 1.0))[:, None, None, None]
+        else:
+            sc = sc / np.sqrt(C)
+        if simple_bias is not None:
+            sb = np.asarray(simple_bias, np.float64)
+            mp = (sb.shape[0] + 1) // 2
+            pos = np.arange(C)
+            sc = sc + sb[(mp - 1) + pos[None, :] - pos[:, None]]
+        w = np.maximum(sc, 0.0) ** 2 if attention_activation == 'relu2' else _sigmoid((sc - 0.707107) * (1.702 / 0.282095))
+        if pad is not None:
+            w = w * (~pad)[:, None, None, :]
+        if not bidirectional:
+            w = w * np.tril(np.ones((C, C)))
+        a = np.einsum('bnlm,bmnh->blnh', w, vc)
+    elif bidirectional or simple_bias is not None:
         # softmax outside the fused op (:210-256): learned bias per relative offset j - i
         # (relative_positional_bias.py:25-42; simple_bias has 2 * max_positions - 1 entries), padded keys
         # excluded unless the whole chunk is padding, causal for one-sided layers

@@ -347,3 +347,52 @@ def test_decoder_model_beam_reorder():
         ref_state = {}
         ref = torch.cat([model(tokens[order][:, t:t + 1], incremental_state=ref_state)[0] for t in range(40)], dim=1)
     assert rel_err(host(got), host(ref[:, 25:])) < 1e-5
+
+
+@pytest.mark.parametrize("act", ['laplace', 'relu2'])
+@pytest.mark.parametrize("bidir,bias,masked", [(False, 'rotary', False), (True, 'simple', True), (True, 'rotary', True),
+                                               (False, 'simple', True)])
+def test_element_attention_layer(act, bidir, bias, masked):
+    """attention_activation = relu2 / laplace (moving_average_gated_attention.py:153-208): forward in
+    inference and in training mode against the layer oracle, and the gradient of the q / k scale
+    against central differences of the oracle."""
+    torch.manual_seed(37)
+    B, L, D, S, E, N, C = 2, 128, 32, 16, 48, 8, 64
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act='silu', norm_num_groups=4,
+                                          rel_pos_bias=bias, bidirectional=bidir,
+                                          attention_activation=act).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.2)
+        layer.gamma.normal_(0, 0.5); layer.beta.normal_(0, 0.5)
+        if bias == 'simple':
+            layer.rel_pos_bias.rel_pos_bias.normal_(0, 0.5)
+    P = _params(layer)
+    sb = host(layer.rel_pos_bias.rel_pos_bias) if bias == 'simple' else None
+    x = torch.randn(B, L, D, device=DEV)
+    mask = None
+    if masked:
+        mask = np.zeros((B, L), bool)
+        mask[0, 100:] = True
+        mask[1, 60:] = True                     # the second chunk of row 1 is padding only
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    okw = dict(chunk=C, num_heads=1, moving_act='silu', num_groups=4, bidirectional=bidir, padding_mask=mask,
+               simple_bias=sb, attention_activation=act)
+    yo = O.gated_attention_layer(host(x), P, **okw)
+    keep = np.ones((B, L), bool) if mask is None else ~mask
+    with torch.no_grad():
+        y, _ = layer(x, tm)
+    assert rel_err(host(y)[keep], yo[keep]) < 2e-4
+    layer.train()
+    w = torch.randn(B, L, D, device=DEV) * torch.from_numpy(keep).to(DEV)[..., None]
+    out, _ = layer(x, tm)
+    assert rel_err(host(out)[keep], yo[keep]) < 2e-4
+    (out * w).sum().backward()
+    g = host(layer.gamma.grad)
+    for (a, i) in [(0, 3), (1, 11)]:
+        Pp, Pm = dict(P), dict(P)
+        Pp['gamma'] = P['gamma'].copy(); Pm['gamma'] = P['gamma'].copy()
+        Pp['gamma'][a, i] += 1e-5; Pm['gamma'][a, i] -= 1e-5
+        fd = ((O.gated_attention_layer(host(x), Pp, **okw) * host(w)).sum()
+              - (O.gated_attention_layer(host(x), Pm, **okw) * host(w)).sum()) / 2e-5
+        assert abs(fd - g[a, i]) < 3e-3 * (np.abs(g).max() + 1e-6), (a, i, fd, g[a, i])
