@@ -181,6 +181,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
         self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
         self._qk_cache = None
+        self._keep_weights, self._last_weights = False, None
         self.chunk_size = chunk_size
         self.num_heads = num_heads
         self.bidirectional = bidirectional
@@ -224,8 +225,26 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         nn.init.constant_(self.beta, 0.0)
 
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None,
-                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None):
-        """x: [B, L, D] -> ([B, L, D], None)."""
+                incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None,
+                need_weights: bool = False, attn_mask: Optional[Tensor] = None, before_attn_fn: bool = False):
+        """x: [B, L, D] -> ([B, L, D], weights or None); the reference's signature
+        (moving_average_gated_attention.py:263-271).  One-sided layers mask the future themselves, so the
+        `attn_mask` the reference's decoder hands them (models/mega_lm.py:353-360: always that mask) is not
+        looked at; need_weights returns the [B * chunks, (Nh,) C, C] weights of a whole-sequence call."""
+        if before_attn_fn:
+            raise NotImplementedError("MovingAverageGatedAttention: before_attn_fn (raw scores) is not built")
+        if attn_mask is not None and self.bidirectional:
+            raise NotImplementedError("MovingAverageGatedAttention: attn_mask on a bidirectional layer is not built")
+        if need_weights:
+            if incremental_state is not None:
+                raise NotImplementedError("MovingAverageGatedAttention: need_weights with incremental state")
+            self._keep_weights = True
+            try:
+                out = self._forward_autograd(x, padding_mask, None)
+                w = self._last_weights
+            finally:
+                self._keep_weights, self._last_weights = False, None
+            return out, (w.squeeze(1) if self.num_heads == 1 else w)
         if _training_call(self, x) or (self.training and self._drops()):
             return self._forward_autograd(x, padding_mask, incremental_state), None
         bsz, seq_len, embed_dim = x.size()
@@ -332,6 +351,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if not self.bidirectional:
             w = w * torch.ones(C, C, device=w.device, dtype=w.dtype).tril_()
         w = F.dropout(w, self.attention_dropout_p, self.training)
+        if self._keep_weights:
+            self._last_weights = w
         return torch.einsum('bnqk,bknh->bqnh', w, v4)
 
     def _forward_autograd(self, x: Tensor, padding_mask: Optional[Tensor], incremental_state) -> Tensor:
@@ -367,7 +388,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if self.attention_activation != 'softmax':
             attn = self._element_attention(q4, k4, v4, None if padding_mask is None
                                            else padding_mask.reshape(bsz * nc, C))
-        elif simple or (self.bidirectional and padding_mask is not None):
+        elif simple or self._keep_weights or (self.bidirectional and padding_mask is not None):
             s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
             if simple:
                 s = s + self.rel_pos_bias(C).to(s.dtype)
@@ -375,7 +396,10 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
                 pad = padding_mask.reshape(bsz * nc, C).to(torch.bool)
                 pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
                 s = s.masked_fill(pad[:, None, None, :], float('-inf'))
-            attn = torch.einsum('bnqk,bknh->bqnh', self.attn_softmax(s), v4)
+            w = self.attn_softmax(s)
+            if self._keep_weights:
+                self._last_weights = w
+            attn = torch.einsum('bnqk,bknh->bqnh', w, v4)
         else:
             attn = self.efficient_attn(q4, k4, v4)
         gated = GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r)
@@ -512,7 +536,7 @@ class MegaDecoderLayer(nn.Module):
     def forward(self, x: Tensor, encoder_out=None, encoder_padding_mask=None, incremental_state=None, attn_mask=None,
                 decoder_padding_mask: Optional[Tensor] = None, need_attn: bool = False):
         """x: [B, L, D] -> (x, None, None), the reference's return triple."""
-        x, attn = self.mega_layer(x, decoder_padding_mask, incremental_state)
+        x, attn = self.mega_layer(x, decoder_padding_mask, incremental_state, need_weights=need_attn)
         if self.nffn is not None:
             x = self.nffn(x)
         return x, attn, None

@@ -396,3 +396,29 @@ def test_element_attention_layer(act, bidir, bias, masked):
         fd = ((O.gated_attention_layer(host(x), Pp, **okw) * host(w)).sum()
               - (O.gated_attention_layer(host(x), Pm, **okw) * host(w)).sum()) / 2e-5
         assert abs(fd - g[a, i]) < 3e-3 * (np.abs(g).max() + 1e-6), (a, i, fd, g[a, i])
+
+
+@pytest.mark.parametrize("heads", [1, 2])
+def test_need_weights_returns_the_chunk_attention(heads):
+    """need_weights (moving_average_gated_attention.py:266, 414-417): same output as the fused call, weights
+    per chunk with rows that sum to one and no weight on future keys."""
+    torch.manual_seed(39)
+    B, L, D, S, E, N, C = 2, 128, 32, 16, 48, 8, 64
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act='silu', norm_num_groups=4,
+                                          num_heads=heads).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.2)
+        x = torch.randn(B, L, D, device=DEV)
+        y0, none = layer(x)
+        y1, w = layer(x, need_weights=True, attn_mask=torch.ones(C, C, device=DEV).tril())
+    assert none is None and rel_err(host(y1), host(y0)) < 1e-5
+    assert w.shape == ((B * L // C, C, C) if heads == 1 else (B * L // C, heads, C, C))
+    assert torch.allclose(w.sum(-1), torch.ones_like(w.sum(-1)), atol=1e-5)
+    assert torch.all(w.triu(1) == 0)
+    dec = M.MegaDecoderLayer(_lm_args()).to(DEV).eval()
+    with torch.no_grad():
+        out, attn, _ = dec(torch.randn(1, 256, 64, device=DEV), need_attn=True)
+    assert attn.shape == (2, 128, 128)
+    with pytest.raises(NotImplementedError):
+        layer(x, before_attn_fn=True)
