@@ -166,9 +166,13 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def __init__(self, embed_dim, zdim, hdim, ndim, chunk_size=-1, moving_layer='cema', moving_act='rmsnorm',
                  norm_num_groups=None, norm_affine=True, norm_eps=1e-5, max_positions=1024, num_heads=1,
                  efficient_attn=True, rel_pos_bias='rotary', bidirectional=False, attention_activation='softmax',
-                 truncation=None, dropout=0.0, attention_dropout=0.0, hidden_dropout=0.0):
+                 truncation=None, dropout=0.0, attention_dropout=0.0, hidden_dropout=0.0, init_mode='bert'):
         super().__init__()
         self.init_incremental_state()
+        self.init_mode = init_mode
+        # efficient_attn=False (moving_average_gated_attention.py:66-79) changes one thing: the attention
+        # dropout is plain dropout on the softmax weights instead of DropKey inside the softmax
+        self._weight_dropout = (not efficient_attn) and attention_activation == 'softmax' and attention_dropout > 0
         # moving_average_gated_attention.py:64-79: element dropout after the output activation and on the
         # two hidden activations, DropKey inside the attention softmax; all three act in training mode only
         self.dropout_p, self.hidden_dropout_p = float(dropout), float(hidden_dropout)
@@ -187,9 +191,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         self.bidirectional = bidirectional
         # causal layers: the fused causal op; bidirectional layers (moving_average_gated_attention.py:70-75,
         # 84-92): full softmax over every chunk, SequenceNorm, a two-sided moving average
-        self.efficient_attn = EfficientAttention(dropout=attention_dropout, use_causal_mask=not bidirectional,
-                                                 scale=1.0)
-        self.attn_softmax = AttentionSoftmax(dropout=attention_dropout, use_causal_mask=not bidirectional)
+        dropkey = 0.0 if not efficient_attn else attention_dropout
+        self.efficient_attn = EfficientAttention(dropout=dropkey, use_causal_mask=not bidirectional, scale=1.0)
+        self.attn_softmax = AttentionSoftmax(dropout=dropkey, use_causal_mask=not bidirectional)
         if bidirectional:
             self.norm = SequenceNorm(embed_dim, num_groups=norm_num_groups, eps=norm_eps)
         else:
@@ -214,11 +218,19 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             # moving_average_gated_attention.py:109-110, 212-219: scores = q k^T + bias[j - i], no rotation
             self.rel_pos_bias = SimpleRelativePositionalBias(self.max_positions)
             self.register_buffer("_no_rotation", torch.zeros(zdim // num_heads // 2), persistent=False)
-        self.reset_parameters()
+        self.reset_parameters(init_mode)
 
-    def reset_parameters(self):
+    def reset_parameters(self, mode='bert'):
+        """moving_average_gated_attention.py:128-151."""
         for lin in (self.v_proj, self.mx_proj, self.h_proj):
-            nn.init.normal_(lin.weight, mean=0.0, std=0.02)
+            if mode == 'bert':
+                nn.init.normal_(lin.weight, mean=0.0, std=0.02)
+            elif mode == 'he':
+                nn.init.kaiming_normal_(lin.weight, a=math.sqrt(5.0))
+            elif mode == 'xavier':
+                nn.init.xavier_uniform_(lin.weight)
+            else:
+                raise ValueError('Unknown init mode: {}'.format(mode))
         nn.init.constant_(self.v_proj.bias, 0.0)
         nn.init.constant_(self.mx_proj.bias, 0.0)
         nn.init.constant_(self.gamma, 0.0)
@@ -388,7 +400,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if self.attention_activation != 'softmax':
             attn = self._element_attention(q4, k4, v4, None if padding_mask is None
                                            else padding_mask.reshape(bsz * nc, C))
-        elif simple or self._keep_weights or (self.bidirectional and padding_mask is not None):
+        elif simple or self._keep_weights or (self.bidirectional and padding_mask is not None) or \
+                (self._weight_dropout and self.training):
             s = torch.einsum('bqnh,bknh->bnqk', q4, k4)
             if simple:
                 s = s + self.rel_pos_bias(C).to(s.dtype)
@@ -397,6 +410,8 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
                 pad = torch.logical_and(pad, ~pad.all(dim=-1, keepdim=True))
                 s = s.masked_fill(pad[:, None, None, :], float('-inf'))
             w = self.attn_softmax(s)
+            if self._weight_dropout:
+                w = F.dropout(w, self.attention_dropout_p, self.training)
             if self._keep_weights:
                 self._last_weights = w
             attn = torch.einsum('bnqk,bknh->bqnh', w, v4)
@@ -522,7 +537,8 @@ class MegaDecoderLayer(nn.Module):
             efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
             bidirectional=False, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
             truncation=trunc if trunc and trunc > 0 else None, dropout=_arg(args, 'dropout', 0.0),
-            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0))
+            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0),
+            init_mode=_arg(args, 'init_mode', 'bert'))
         self.cross_attn = None
         if _arg(args, 'decoder_ffn_embed_dim', 0) > 0:
             self.nffn = NormalizedFeedForwardNetwork(
@@ -558,7 +574,8 @@ class MegaEncoderLayer(nn.Module):
             efficient_attn=_arg(args, 'efficient_attention', True), rel_pos_bias=_arg(args, 'rel_pos_bias', 'rotary'),
             bidirectional=True, attention_activation=_arg(args, 'attention_activation_fn', 'softmax'),
             truncation=trunc if trunc and trunc > 0 else None, dropout=_arg(args, 'dropout', 0.0),
-            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0))
+            attention_dropout=_arg(args, 'attention_dropout', 0.0), hidden_dropout=_arg(args, 'hidden_dropout', 0.0),
+            init_mode=_arg(args, 'init_mode', 'bert'))
         if _arg(args, 'encoder_ffn_embed_dim', 0) > 0:
             self.nffn = NormalizedFeedForwardNetwork(
                 self.embed_dim, args.encoder_ffn_embed_dim, dropout=_arg(args, 'dropout', 0.0),

@@ -325,6 +325,15 @@ def test_layer_dropouts_act_in_training_only():
                                                      if p.grad is not None)
     f = M.NormalizedFeedForwardNetwork(D, 64, dropout=0.2, hidden_dropout=0.2).to(DEV)
     assert torch.equal(f.eval()(x), f(x)) and not torch.equal(f.train()(x), f.eval()(x))
+    # efficient_attn=False: plain dropout on the softmax weights instead of DropKey (:66-79, 244-247)
+    wd = M.MovingAverageGatedAttention(D, S, E, N, attention_dropout=0.3, efficient_attn=False, **kw).to(DEV)
+    wd.load_state_dict(plain.state_dict())
+    with torch.no_grad():
+        assert torch.equal(wd.eval()(x)[0], ref)
+        _, w = wd.train()(x, need_weights=True)
+    zeros = (w.tril() == 0) & (torch.ones_like(w).tril() > 0)
+    assert 0.2 < zeros.float().sum() / torch.ones_like(w).tril().sum() < 0.4
+    assert (w.sum(-1) - 1).abs().max() > 0.05           # survivors are scaled by 1 / (1 - p), rows no longer sum to one
 
 
 def test_decoder_model_beam_reorder():

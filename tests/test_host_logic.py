@@ -99,3 +99,17 @@ def test_gated_attention_state_dict_matches_reference_names():
     assert got == want
     ffn = M.NormalizedFeedForwardNetwork(D, 32, norm_type='rmsnorm')
     assert set(ffn.state_dict()) == {"norm.weight", "fc1.weight", "fc1.bias", "fc2.weight"}
+
+
+def test_layer_constructor_follows_the_reference():
+    """init_mode (moving_average_gated_attention.py:128-145) and the attention activations are checked at
+    construction."""
+    kw = dict(chunk_size=4, norm_num_groups=2)
+    for mode in ('bert', 'he', 'xavier'):
+        layer = M.MovingAverageGatedAttention(8, 4, 8, 2, init_mode=mode, **kw)
+        assert layer.init_mode == mode and torch.all(layer.gamma == 0) and torch.all(layer.v_proj.bias == 0)
+    with pytest.raises(ValueError, match="init mode"):
+        M.MovingAverageGatedAttention(8, 4, 8, 2, init_mode='orthogonal', **kw)
+    with pytest.raises(ValueError, match="attention activation"):
+        M.MovingAverageGatedAttention(8, 4, 8, 2, attention_activation='gelu', **kw)
+    assert 'chunk=4' in repr(M.MovingAverageGatedAttention(8, 4, 8, 2, **kw))
