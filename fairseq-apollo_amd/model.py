@@ -1,8 +1,8 @@
 """Decoder-only Mega language-model body: token embedding -> MegaDecoderLayer stack ->
 TimestepNorm -> output projection, with the reference's submodule names so that the `decoder.*`
 entries of a reference `mega_lm` checkpoint load with `load_state_dict`
-(fairseq/models/mega_lm.py:188-300, MegaDecoderNoCrossAttn).  Dictionary handling, dropout,
-adaptive softmax and the fairseq task / trainer plumbing are not part of it.
+(fairseq/models/mega_lm.py:188-300, MegaDecoderNoCrossAttn).  Dictionary handling, adaptive softmax
+and the fairseq task / trainer plumbing are not part of it.
 """
 from __future__ import annotations
 
@@ -36,6 +36,7 @@ class MegaDecoderNoCrossAttn(nn.Module):
         self.chunk_size = _arg(args, 'decoder_chunk_size', -1)
         self.embed_tokens = embed_tokens
         self.embed_scale = None if _arg(args, 'no_scale_embedding', False) else math.sqrt(embed_dim)
+        self.embedding_dropout = nn.Dropout(_arg(args, 'dropout', 0.0))
         depth = args.decoder_layers
         lsw = [0.1 * (0.5 ** i) for i in range(depth)] if _arg(args, 'layer_scale', False) else [None] * depth
         self.layers = nn.ModuleList([MegaDecoderLayer(args, no_cross_attention=True, layer_scale=lsw[i])
@@ -47,7 +48,8 @@ class MegaDecoderNoCrossAttn(nn.Module):
         if rep is not None:
             self.num_features = rep
             self.pre_logits = nn.Sequential(OrderedDict([('fc', nn.Linear(embed_dim, rep, bias=True)),
-                                                         ('act', nn.SiLU())]))
+                                                         ('act', nn.SiLU()),
+                                                         ('dropout', nn.Dropout(_arg(args, 'dropout', 0.0)))]))
         else:
             self.num_features = embed_dim
             self.pre_logits = nn.Identity()
@@ -65,8 +67,16 @@ class MegaDecoderNoCrossAttn(nn.Module):
                 features_only: bool = False) -> Tuple[Tensor, Dict[str, List[Tensor]]]:
         x, extra = self.extract_features(prev_output_tokens, incremental_state)
         if not features_only:
-            x = self.output_projection(x)
+            x = self.output_layer(x)
         return x, extra
+
+    def output_layer(self, features: Tensor) -> Tensor:
+        """Project features to the vocabulary (mega_lm.py:379-385)."""
+        return self.output_projection(features)
+
+    def max_positions(self) -> int:
+        """Longest sequence the decoder is configured for (mega_lm.py:387-389)."""
+        return self.max_target_positions
 
     def extract_features(self, prev_output_tokens: Tensor, incremental_state=None):
         """mega_lm.py:313-386: tokens are padded up to a whole number of chunks, padded positions are
@@ -82,6 +92,7 @@ class MegaDecoderNoCrossAttn(nn.Module):
         decoder_padding_mask = prev_output_tokens.eq(self.padding_idx) if self.padding_idx is not None else None
         if decoder_padding_mask is not None and not decoder_padding_mask.any():
             decoder_padding_mask = None
+        x = self.embedding_dropout(x)
         inner_states: List[Tensor] = [x]
         for layer in self.layers:
             x, _, _ = layer(x, incremental_state=incremental_state, decoder_padding_mask=decoder_padding_mask)
