@@ -23,10 +23,11 @@ from .layers import (  # noqa: F401,E402
     streamed_forward,
 )
 
-from .model import MegaDecoderNoCrossAttn  # noqa: F401,E402
+from .model import MegaDecoderNoCrossAttn, validate_stream  # noqa: F401,E402
 
 __all__ = [
     "MegaDecoderNoCrossAttn",
+    "validate_stream",
     "Mega2Layer",
     "MegaDecoderLayer",
     "MegaEncoderLayer",

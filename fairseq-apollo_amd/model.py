@@ -120,3 +120,27 @@ class MegaDecoderNoCrossAttn(nn.Module):
         state: Dict[str, Dict[str, Optional[Tensor]]] = {}
         outs = [self(tokens[:, a:a + chunk], incremental_state=state)[0] for a in range(0, tokens.size(1), chunk)]
         return torch.cat(outs, dim=1)
+
+
+def validate_stream(model: MegaDecoderNoCrossAttn, src_tokens: Tensor, target: Tensor, pad_idx: int,
+                    chunk_size: Optional[int] = None) -> Tuple[Tensor, Tensor]:
+    """Chunk-wise evaluation of one batch of documents the way the reference validates a Mega language
+    model (fairseq_cli/train.py:395-417): consecutive slices of `chunk_size` tokens go through the
+    model with one incremental-state dictionary per batch, and every slice adds its summed negative
+    log-likelihood and its count of non-padding targets.  -> (nll_sum, ntokens); perplexity is
+    exp(nll_sum / ntokens) (base e)."""
+    chunk = chunk_size or model.chunk_size
+    if chunk <= 0:
+        chunk = src_tokens.size(1)
+    state: Dict[str, Dict[str, Optional[Tensor]]] = {}
+    nll = torch.zeros((), dtype=torch.float64, device=src_tokens.device)
+    ntok = torch.zeros((), dtype=torch.int64, device=src_tokens.device)
+    with torch.no_grad():
+        for a in range(0, src_tokens.size(1), chunk):
+            logits = model(src_tokens[:, a:a + chunk], incremental_state=state)[0]
+            tgt = target[:, a:a + chunk]
+            lp = F.log_softmax(logits.float(), dim=-1)
+            nll += F.nll_loss(lp.reshape(-1, lp.size(-1)), tgt.reshape(-1), ignore_index=pad_idx,
+                              reduction='sum').double()
+            ntok += tgt.ne(pad_idx).sum()
+    return nll, ntok

@@ -431,3 +431,23 @@ def test_need_weights_returns_the_chunk_attention(heads):
     assert attn.shape == (2, 128, 128)
     with pytest.raises(NotImplementedError):
         layer(x, before_attn_fn=True)
+
+
+def test_chunkwise_validation_equals_one_shot_loss():
+    """validate_stream (fairseq_cli/train.py:395-417): the summed loss over chunk-wise slices with carried
+    state equals the loss of the whole documents in one forward; padded targets are not counted."""
+    torch.manual_seed(45)
+    args = _lm_args(decoder_layers=2, norm_eps=1e-5)
+    vocab, pad = 40, 1
+    model = M.MegaDecoderNoCrossAttn(args, vocab, torch.nn.Embedding(vocab, 64, padding_idx=pad)).to(DEV).eval()
+    tokens = torch.randint(2, vocab, (3, 513), device=DEV)
+    src, tgt = tokens[:, :-1].clone(), tokens[:, 1:].clone()
+    src[1, 400:] = pad
+    tgt[1, 399:] = pad                                   # a document that ends early
+    nll, ntok = M.validate_stream(model, src, tgt, pad)
+    with torch.no_grad():
+        logits = model(src)[0]
+    ref = torch.nn.functional.cross_entropy(logits.reshape(-1, vocab).float(), tgt.reshape(-1), ignore_index=pad,
+                                            reduction='sum')
+    assert int(ntok) == int(tgt.ne(pad).sum()) == 2 * 512 + 399
+    assert abs(float(nll) - float(ref)) < 1e-4 * float(ref)
