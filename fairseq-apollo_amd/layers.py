@@ -430,9 +430,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         """Attention with the partial-chunk key / value cache
         (moving_average_gated_attention.py:332-372): keys are cached before the rotation, so the
         whole context is rotated again at every call."""
-        if isinstance(self.rel_pos_bias, SimpleRelativePositionalBias) or self.attention_activation != 'softmax':
-            raise NotImplementedError("MovingAverageGatedAttention: incremental decoding is built for the rotary "
-                                      "position encoding and the softmax attention only")
+        simple = isinstance(self.rel_pos_bias, SimpleRelativePositionalBias)
         bsz, seq_len = z.shape[:2]
         Nh = self.num_heads
         z = F.normalize(z, p=2, dim=-1, eps=1e-5)
@@ -460,14 +458,27 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         k4 = k.reshape(k.size(0), k.size(1), Nh, -1)
         v4 = v.reshape(v.size(0), v.size(1), Nh, -1)
         qidx = k4.size(1) - q4.size(1)
-        q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), qidx).transpose(1, 2)
-        k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
-        if q4.size(1) == k4.size(1):
-            return self.efficient_attn(q4, k4, v4)
-        # a few new queries against a longer cached context: right-aligned causal softmax
-        s = torch.einsum('bqnh,bknh->bnqk', q4.float(), k4.float()).to(q4.dtype)
-        w = ops.attention_softmax_fwd(s, 0.0, True)
-        return torch.einsum('bnqk,bknh->bqnh', w.float(), v4.float()).to(v4.dtype)
+        if not simple:
+            q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), qidx).transpose(1, 2)
+            k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+            if q4.size(1) == k4.size(1) and self.attention_activation == 'softmax':
+                return self.efficient_attn(q4, k4, v4)
+        # new queries at positions qidx .. ctx-1 against the cached context (a whole chunk when qidx = 0):
+        # right-aligned causal weights; the bias rows are those of the query positions
+        # (moving_average_gated_attention.py:170-178, 212-221: `bias[-1:]` for one new token)
+        ctx = k4.size(1)
+        s = torch.einsum('bqnh,bknh->bnqk', q4.float(), k4.float())
+        if self.attention_activation != 'softmax':
+            s = s * torch.rsqrt(torch.arange(qidx + 1, ctx + 1, device=s.device, dtype=torch.float32))[:, None]
+        if simple:
+            s = s + self.rel_pos_bias(ctx)[qidx:].float()
+        if self.attention_activation == 'softmax':
+            w = ops.attention_softmax_fwd(s.to(q4.dtype), 0.0, True).float()
+        else:
+            w = torch.square(F.relu(s)) if self.attention_activation == 'relu2' else \
+                torch.sigmoid((s - 0.707107) * (1.702 / 0.282095))
+            w = w * torch.ones(ctx, ctx, device=w.device, dtype=w.dtype).tril_()[qidx:]
+        return torch.einsum('bnqk,bknh->bqnh', w, v4.float()).to(v4.dtype)
 
     def _get_input_buffer(self, incremental_state):
         result = self.get_incremental_state(incremental_state, "attn_state")

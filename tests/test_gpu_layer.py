@@ -451,3 +451,26 @@ def test_chunkwise_validation_equals_one_shot_loss():
                                             reduction='sum')
     assert int(ntok) == int(tgt.ne(pad).sum()) == 2 * 512 + 399
     assert abs(float(nll) - float(ref)) < 1e-4 * float(ref)
+
+
+@pytest.mark.parametrize("bias,act", [('simple', 'softmax'), ('rotary', 'laplace'), ('simple', 'relu2')])
+@pytest.mark.parametrize("step", [1, 16, 64])
+def test_incremental_decoding_with_learned_bias_and_element_attention(bias, act, step):
+    """The key / value chunk cache with the learned position bias (rows of the new positions,
+    moving_average_gated_attention.py:212-221) and with the element-wise attention: a sequence fed in
+    slices of `step` tokens (1: token by token; 64: whole chunks) equals the one-shot forward."""
+    torch.manual_seed(47)
+    B, L, D, S, E, N, C = 2, 160, 32, 16, 48, 8, 64
+    layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act='silu', norm_num_groups=4,
+                                          rel_pos_bias=bias, attention_activation=act).to(DEV).eval()
+    with torch.no_grad():
+        for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+            prm.normal_(0, 0.2)
+        layer.gamma.normal_(0, 0.5); layer.beta.normal_(0, 0.5)
+        if bias == 'simple':
+            layer.rel_pos_bias.rel_pos_bias.normal_(0, 0.5)
+        x = torch.randn(B, 128, D, device=DEV)
+        full, _ = layer(x)
+        state = {}
+        parts = [layer(x[:, a:a + step], incremental_state=state)[0] for a in range(0, 128, step)]
+    assert rel_err(host(torch.cat(parts, dim=1)), host(full)) < 2e-5
