@@ -28,7 +28,7 @@
 namespace mega {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kMaxTileCells = 4096;   // tokens-per-tile * groups held in LDS
 
 struct TsnBwdParams {
