@@ -16,7 +16,8 @@
 namespace mega {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;        // [B, H, L] kernels: one workgroup per row, rows are plentiful
+constexpr int kTileThreads = 512;    // [B, L, H] tile kernel: two tiles per compute unit, four waves per SIMD
 constexpr int kMaxCells = 4096;     // tokens-per-tile * groups held in LDS
 
 struct SeqNormParams {
@@ -48,7 +49,7 @@ __device__ __forceinline__ void merge3(float& n, float& m, float& M2, float nb, 
 // ---------------------------------------------------------------- [B, L, H]: channels contiguous
 // APPLY = false: partial moments of the tile; APPLY = true: normalise the tile.
 template <typename T, int VEC, bool APPLY>
-__global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormParams P) {
+__global__ __launch_bounds__(kTileThreads) void seqnorm_blh_kernel(const SeqNormParams P) {
   using V = Vec<T, VEC>;
   extern __shared__ float smem[];
   const int G = P.G, H = P.H, TT = P.TT, Dg = P.Dg;
@@ -60,17 +61,17 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
   const int t0 = tile * TT;
   const int ntok = min(TT, P.L - t0);
   const T* x = (const T*)P.x + ((size_t)b * P.L + t0) * H;
-  for (int tok = tid; tok < TT; tok += kThreads)
+  for (int tok = tid; tok < TT; tok += kTileThreads)
     s_mask[tok] = (tok >= ntok) || (P.mask && P.mask[(size_t)b * P.L + t0 + tok]);
   if (APPLY)
-    for (int g = tid; g < G; g += kThreads) {
+    for (int g = tid; g < G; g += kTileThreads) {
       s_a[g] = P.mean[(size_t)b * G + g];
       s_b[g] = P.rstd[(size_t)b * G + g];
     }
   __syncthreads();
   const int items = ntok * P.R.slots;
   const int span = VEC * P.R.PER;
-  for (int i0 = 0; i0 < items; i0 += kThreads) {
+  for (int i0 = 0; i0 < items; i0 += kTileThreads) {
     const int i = i0 + tid;
     const bool live = i < items;
     int tok, slot;
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void seqnorm_blh_kernel(const SeqNormPara
     __syncthreads();
     int nkeep = 0;
     for (int tok = 0; tok < ntok; ++tok) nkeep += s_mask[tok] ? 0 : 1;
-    for (int g = tid; g < G; g += kThreads) {
+    for (int g = tid; g < G; g += kTileThreads) {
       float s1 = 0.f, s2 = 0.f;
       for (int tok = 0; tok < ntok; ++tok) {      // masked tokens hold zeros
         s1 += s_a[tok * G + g];
@@ -406,14 +407,14 @@ int launch_seqnorm(SeqNormParams P, const SeqGeom& g, int length_last, bool alig
   }
   const dim3 grid((unsigned)(P.B * P.nt));
   const size_t lds_m = ((size_t)2 * P.TT * P.G + P.TT) * 4, lds_a = ((size_t)2 * P.G + P.TT) * 4;
-  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, false>), grid, dim3(kThreads), lds_m, s, P);
-  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, false>), grid, dim3(kThreads), lds_m, s, P);
+  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, false>), grid, dim3(kTileThreads), lds_m, s, P);
+  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, false>), grid, dim3(kTileThreads), lds_m, s, P);
   MEGA_CHECK_LAUNCH("sequence_norm_fwd (moments)");
   hipLaunchKernelGGL(seqnorm_combine_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P, P.nt,
                      (int64_t)P.nt * P.G * 3, (int64_t)3, (int64_t)P.G * 3);
   MEGA_CHECK_LAUNCH("sequence_norm_fwd (combine)");
-  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, true>), grid, dim3(kThreads), lds_a, s, P);
-  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, true>), grid, dim3(kThreads), lds_a, s, P);
+  if (vec) hipLaunchKernelGGL((seqnorm_blh_kernel<T, FULL, true>), grid, dim3(kTileThreads), lds_a, s, P);
+  else hipLaunchKernelGGL((seqnorm_blh_kernel<T, 1, true>), grid, dim3(kTileThreads), lds_a, s, P);
   MEGA_CHECK_LAUNCH("sequence_norm_fwd (apply)");
   return MEGA_OK;
 }
