@@ -65,6 +65,9 @@ SIGNATURES = {
     "mega_swiglu_fwd": (_int, [_p, _p, _p, _int, _i64, _p]),
     "mega_rms_norm_fwd": (_int, [_p, _i64, _p, _p, _int, _i64, _i64, C.c_double, _p]),
     "mega_gate_qk_fwd": (_int, [_p, _i64, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_double, _p]),
+    "mega_gate_qk_bwd_workspace_bytes": (_sz, [_i64, _i64]),
+    "mega_gate_qk_bwd": (_int, [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_double,
+                                _p, _sz, _p]),
     "mega_gate_mul_fwd": (_int, [_p, _i64, _p, _i64, _p, _int, _i64, _i64, _p]),
     "mega_gate_out_fwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _int, _i64, _i64, _p]),
     "mega_gate_mul_bwd": (_int, [_p, _p, _i64, _p, _i64, _p, _p, _int, _i64, _i64, _p]),

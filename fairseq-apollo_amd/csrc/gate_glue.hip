@@ -109,6 +109,138 @@ __global__ __launch_bounds__(kRowThreads) void gate_qk_kernel(const T* __restric
   }
 }
 
+// Backward of the q / k map.  One wave per token, a wave walks tokens t, t + waves, ...; lane l owns
+// the same NV vectors of features at every token, so the four parameter sums (d gamma, d beta of the
+// q and of the k map) stay in registers until the end:
+//   dq_pre = rot^T(dq), dk_pre = rot^T(dk)                         (rotation by -pos * freq)
+//   dbeta_q += dq_pre, dgamma_q += dq_pre zn   (and the same for k)
+//   dzn = dq_pre gamma_q + dk_pre gamma_k
+//   dz  = (dzn - zn (zn . dzn)) / |z|      (|z| > eps)      or      dzn / eps      (|z| <= eps)
+// The workgroup's four waves then add their sums in LDS, one after the other, and leave one row
+// per workgroup in `part` [workgroups][4][S]; gate_qk_param_kernel adds the rows in order.
+template <typename T, int VEC, int NV>
+__global__ __launch_bounds__(kRowThreads) void gate_qk_bwd_kernel(
+    const T* __restrict__ dq, const T* __restrict__ dk, const T* __restrict__ z, int64_t zs,
+    const float* __restrict__ gamma, const float* __restrict__ freqs, T* __restrict__ dz, float* __restrict__ part,
+    int64_t T_, int S, int Hd, int64_t chunk, int64_t pos0, float eps) {
+  using V = Vec<T, VEC>;
+  static_assert(VEC % 2 == 0, "pairs of features stay inside one vector");
+  extern __shared__ float s_acc[];                     // [4][S]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float agq[NV][VEC], abq[NV][VEC], agk[NV][VEC], abk[NV][VEC];
+  float gq[NV][VEC], gk[NV][VEC], fr[NV][VEC / 2];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int j = (u * 64 + lane) * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      agq[u][i] = abq[u][i] = agk[u][i] = abk[u][i] = 0.f;
+      gq[u][i] = j + i < S ? gamma[j + i] : 0.f;
+      gk[u][i] = j + i < S ? gamma[S + j + i] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < VEC / 2; ++i) fr[u][i] = j + 2 * i < S ? freqs[((j + 2 * i) % Hd) >> 1] : 0.f;
+  }
+  const int64_t stride = (int64_t)gridDim.x * kRowsPerWg;
+  for (int64_t t = (int64_t)blockIdx.x * kRowsPerWg + wave; t < T_; t += stride) {
+    const T* row = z + t * zs;
+    float zf[NV][VEC], aq[NV][VEC], ak[NV][VEC];
+    float ss = 0.f;
+    const float pos = (float)(pos0 + t % chunk);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int j = (u * 64 + lane) * VEC;
+      if (j < S) {
+        const V v = *(const V*)(row + j);
+        const V a = *(const V*)(dq + t * (int64_t)S + j);
+        const V b = *(const V*)(dk + t * (int64_t)S + j);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          zf[u][i] = to_float(v.v[i]);
+          ss = fmaf(zf[u][i], zf[u][i], ss);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; i += 2) {
+          float sn, cs;
+          sincosf(pos * fr[u][i >> 1], &sn, &cs);
+          const float a0 = to_float(a.v[i]), a1 = to_float(a.v[i + 1]);
+          const float b0 = to_float(b.v[i]), b1 = to_float(b.v[i + 1]);
+          aq[u][i] = a0 * cs + a1 * sn;
+          aq[u][i + 1] = a1 * cs - a0 * sn;
+          ak[u][i] = b0 * cs + b1 * sn;
+          ak[u][i + 1] = b1 * cs - b0 * sn;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) zf[u][i] = aq[u][i] = ak[u][i] = 0.f;
+      }
+    }
+    const float nrm = sqrtf(wave_sum(ss));
+    const bool clamped = !(nrm > eps);
+    const float inv = 1.0f / fmaxf(nrm, eps);
+    float dot = 0.f;
+    float dzn[NV][VEC];
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float zn = zf[u][i] * inv;
+        abq[u][i] += aq[u][i];
+        agq[u][i] = fmaf(aq[u][i], zn, agq[u][i]);
+        abk[u][i] += ak[u][i];
+        agk[u][i] = fmaf(ak[u][i], zn, agk[u][i]);
+        dzn[u][i] = fmaf(aq[u][i], gq[u][i], ak[u][i] * gk[u][i]);
+        dot = fmaf(zn, dzn[u][i], dot);
+        zf[u][i] = zn;
+      }
+    dot = clamped ? 0.f : wave_sum(dot);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int j = (u * 64 + lane) * VEC;
+      if (j < S) {
+        V o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = from_float<T>((dzn[u][i] - zf[u][i] * dot) * inv);
+        *(V*)(dz + t * (int64_t)S + j) = o;
+      }
+    }
+  }
+  // the four waves add up in a fixed order
+  for (int turn = 0; turn < kRowsPerWg; ++turn) {
+    if (wave == turn) {
+#pragma unroll
+      for (int u = 0; u < NV; ++u) {
+        const int j = (u * 64 + lane) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          if (j + i < S) {
+            if (turn == 0) {
+              s_acc[j + i] = agq[u][i]; s_acc[S + j + i] = agk[u][i];
+              s_acc[2 * S + j + i] = abq[u][i]; s_acc[3 * S + j + i] = abk[u][i];
+            } else {
+              s_acc[j + i] += agq[u][i]; s_acc[S + j + i] += agk[u][i];
+              s_acc[2 * S + j + i] += abq[u][i]; s_acc[3 * S + j + i] += abk[u][i];
+            }
+          }
+      }
+    }
+    __syncthreads();
+  }
+  float* dst = part + (size_t)blockIdx.x * 4 * S;
+  for (int i = threadIdx.x; i < 4 * S; i += kRowThreads) dst[i] = s_acc[i];
+}
+
+// dgamma [2, S] = rows 0, 1 of the sums, dbeta [2, S] = rows 2, 3
+__global__ __launch_bounds__(256) void gate_qk_param_kernel(const float* __restrict__ part, int rows, int S,
+                                                            float* __restrict__ dgamma, float* __restrict__ dbeta) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= 4 * S) return;
+  float a = 0.f;
+  for (int r = 0; r < rows; ++r) a += part[(size_t)r * 4 * S + i];
+  if (i < 2 * S) dgamma[i] = a;
+  else dbeta[i - 2 * S] = a;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Row-strided elementwise kernels: blockIdx.x walks rows, threads walk the row in vectors.
 template <typename T, int VEC>
@@ -297,6 +429,38 @@ int launch_gate_qk(const void* z, int64_t zs, const float* gamma, const float* b
   return MEGA_OK;
 }
 
+constexpr int kQkBwdMaxWgs = 512;
+
+inline int64_t gate_qk_bwd_wgs(int64_t T_) {
+  const int64_t w = ceil_div(T_, kRowsPerWg);
+  return w < kQkBwdMaxWgs ? w : kQkBwdMaxWgs;
+}
+
+template <typename T>
+int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs, const float* gamma,
+                       const float* freqs, void* dz, float* dgamma, float* dbeta, float* part, int64_t T_, int64_t S,
+                       int64_t Hd, int64_t chunk, int64_t pos0, float eps, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  MEGA_REQUIRE(S % VEC == 0 && S <= 2 * 64 * VEC && vec_ok(z, zs, sizeof(T), VEC) && vec_ok(dq, S, sizeof(T), VEC) &&
+                   vec_ok(dk, S, sizeof(T), VEC) && vec_ok(dz, S, sizeof(T), VEC),
+               MEGA_ERR_UNSUPPORTED,
+               "gate_qk_bwd: S=%lld must be a multiple of %d, at most %d, with 16-byte aligned rows", (long long)S, VEC,
+               2 * 64 * VEC);
+  const unsigned grid = (unsigned)gate_qk_bwd_wgs(T_);
+  const size_t lds = (size_t)4 * S * sizeof(float);
+  if (S <= 64 * VEC)
+    hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 1>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
+                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
+  else
+    hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 2>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
+                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
+  MEGA_CHECK_LAUNCH("gate_qk_bwd");
+  hipLaunchKernelGGL(gate_qk_param_kernel, dim3((unsigned)ceil_div(4 * S, 256)), dim3(256), 0, s, part, (int)grid,
+                     (int)S, dgamma, dbeta);
+  MEGA_CHECK_LAUNCH("gate_qk_bwd (parameter sums)");
+  return MEGA_OK;
+}
+
 template <typename T>
 int launch_gate_mul(const void* a, int64_t as, const void* r, int64_t rs, void* y, int64_t T_, int64_t E,
                     hipStream_t s) {
@@ -424,6 +588,38 @@ extern "C" int mega_gate_qk_fwd(const void* z, int64_t z_stride, const float* ga
   hipStream_t s = (hipStream_t)stream;
   MEGA_GLUE_DISPATCH(launch_gate_qk, z, z_stride, gamma, beta, freqs, q, k, T_, S, S / heads, chunk, pos0, (float)eps,
                      s);
+}
+
+extern "C" size_t mega_gate_qk_bwd_workspace_bytes(int64_t T_, int64_t S) {
+  if (T_ <= 0 || S <= 0) return 256;
+  return align_up((size_t)gate_qk_bwd_wgs(T_) * 4 * (size_t)S * sizeof(float), 256);
+}
+
+extern "C" int mega_gate_qk_bwd(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
+                                const float* gamma, const float* freqs, void* z_grad, float* gamma_grad,
+                                float* beta_grad, int dtype, int64_t T_, int64_t S, int64_t heads, int64_t chunk,
+                                int64_t pos0, double eps, void* workspace, size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_qk_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(T_ >= 0 && S >= 2 && S < (1ll << 30) && heads >= 1 && chunk >= 1 && pos0 >= 0, MEGA_ERR_ARG,
+               "gate_qk_bwd: bad sizes T=%lld S=%lld heads=%lld chunk=%lld pos0=%lld", (long long)T_, (long long)S,
+               (long long)heads, (long long)chunk, (long long)pos0);
+  MEGA_REQUIRE(S % heads == 0 && (S / heads) % 2 == 0, MEGA_ERR_ARG,
+               "gate_qk_bwd: S=%lld must split into %lld heads of even size", (long long)S, (long long)heads);
+  MEGA_REQUIRE(gamma_grad && beta_grad, MEGA_ERR_ARG, "gate_qk_bwd: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  if (T_ == 0) {
+    zero_async(gamma_grad, (size_t)2 * S * 4, s);
+    zero_async(beta_grad, (size_t)2 * S * 4, s);
+    return MEGA_OK;
+  }
+  MEGA_REQUIRE(q_grad && k_grad && z && gamma && freqs && z_grad, MEGA_ERR_ARG, "gate_qk_bwd: null pointer argument");
+  MEGA_REQUIRE(z_stride >= S, MEGA_ERR_ARG, "gate_qk_bwd: row stride %lld below the row length %lld",
+               (long long)z_stride, (long long)S);
+  const size_t need = mega_gate_qk_bwd_workspace_bytes(T_, S);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
+               "gate_qk_bwd: workspace of %zu bytes (16-byte aligned) needed", need);
+  MEGA_GLUE_DISPATCH(launch_gate_qk_bwd, q_grad, k_grad, z, z_stride, gamma, freqs, z_grad, gamma_grad, beta_grad,
+                     (float*)workspace, T_, S, S / heads, chunk, pos0, (float)eps, s);
 }
 
 extern "C" int mega_gate_mul_fwd(const void* a, int64_t a_stride, const void* r, int64_t r_stride, void* y, int dtype,

@@ -22,7 +22,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
+from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
                       TimestepNorm, _training_call)
 
 
@@ -384,19 +384,27 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
         base = self.mx_proj(F.dropout(self.move_act(mx), self.hidden_dropout_p, self.training))
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
-        z = F.normalize(z, p=2, dim=-1, eps=1e-5)
-        z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
-        q, k = torch.unbind(z, dim=2)
         Nh = self.num_heads
         C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
         nc = seq_len // C
-        q4 = q.reshape(bsz * nc, C, Nh, -1)
-        k4 = k.reshape(bsz * nc, C, Nh, -1)
-        v4 = v.reshape(bsz * nc, C, Nh, -1)
         simple = isinstance(self.rel_pos_bias, SimpleRelativePositionalBias)
-        if not simple:
-            q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
-            k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+        v4 = v.reshape(bsz * nc, C, Nh, -1)
+        vec = 16 // z.element_size()
+        if self.zdim % vec == 0 and self.zdim <= 128 * vec:
+            # one kernel forward, one backward (rows of whole 16-byte vectors, at most two per lane)
+            freqs = self._no_rotation if simple else self.rel_pos_bias.freqs
+            q, k = GateQKFunc.apply(z, self.gamma, self.beta, freqs.detach().float().contiguous(), Nh, C)
+            q4 = q.view(bsz * nc, C, Nh, -1)
+            k4 = k.view(bsz * nc, C, Nh, -1)
+        else:
+            z = F.normalize(z, p=2, dim=-1, eps=1e-5)
+            z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
+            q, k = torch.unbind(z, dim=2)
+            q4 = q.reshape(bsz * nc, C, Nh, -1)
+            k4 = k.reshape(bsz * nc, C, Nh, -1)
+            if not simple:
+                q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
+                k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
         if self.attention_activation != 'softmax':
             attn = self._element_attention(q4, k4, v4, None if padding_mask is None
                                            else padding_mask.reshape(bsz * nc, C))

@@ -512,6 +512,26 @@ class SequenceNorm(nn.Module):
         return 'num_features={num_features}, num_groups={num_groups}, eps={eps}'.format(**self.__dict__)
 
 
+class GateQKFunc(torch.autograd.Function):
+    """q, k = rotary(normalize(z) * (gamma + 1) + beta) in one pass over z, with one backward pass
+    (moving_average_gated_attention.py:324-328, relative_positional_bias.py:86-97).  gamma, beta are
+    the layer's [2, S] parameters; freqs holds zeros when the layer does not rotate."""
+
+    @staticmethod
+    def forward(ctx, z, gamma, beta, freqs, num_heads, chunk):
+        g1 = gamma.detach().float() + 1.0
+        ctx.save_for_backward(z, g1, freqs)
+        ctx.num_heads, ctx.chunk = num_heads, chunk
+        ctx.param_dtypes = (gamma.dtype, beta.dtype)
+        return ops.gate_qk_fwd(z, g1, beta.detach().float(), freqs, num_heads, chunk)
+
+    @staticmethod
+    def backward(ctx, q_grad, k_grad):
+        z, g1, freqs = ctx.saved_tensors
+        dz, dgamma, dbeta = ops.gate_qk_bwd(q_grad, k_grad, z, g1, freqs, ctx.num_heads, ctx.chunk)
+        return dz, dgamma.to(ctx.param_dtypes[0]), dbeta.to(ctx.param_dtypes[1]), None, None, None
+
+
 class GateMulFunc(torch.autograd.Function):
     """a * silu(r) with its own backward (moving_average_gated_attention.py:330, 407)."""
 

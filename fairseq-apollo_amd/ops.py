@@ -915,6 +915,39 @@ def gate_qk_fwd(z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, freqs:
     return q, k
 
 
+def gate_qk_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, freqs: torch.Tensor,
+                num_heads: int, chunk: int, pos0: int = 0, eps: float = 1e-5):
+    """Backward of gate_qk_fwd: -> (z_grad [..., S] in z's dtype, gamma_grad [2, S] fp32, beta_grad [2, S] fp32).
+    The autograd graph it replaces is normalize -> affine -> rotary
+    (moving_average_gated_attention.py:324-328, relative_positional_bias.py:86-97)."""
+    dev = _need_gpu(q_grad, k_grad, z)
+    lib = _lib.load()
+    S = z.shape[-1]
+    zr, zs = _rows(z)
+    if (zs * zr.element_size()) % 16 or zr.data_ptr() % 16:
+        zr, zs = z.detach().contiguous(), S        # the kernel reads whole 16-byte vectors
+    g, f = _f32c(gamma), _f32c(freqs)
+    if g.shape != (2, S) or num_heads < 1 or S % num_heads or f.numel() * 2 * num_heads != S:
+        raise RuntimeError("gate_qk_bwd: gamma must be [2, S] and freqs [S / heads / 2]")
+    if q_grad.shape != z.shape or k_grad.shape != z.shape:
+        raise RuntimeError("gate_qk_bwd: q_grad, k_grad must have z's shape")
+    dq = q_grad.detach().to(z.dtype).contiguous()
+    dk = k_grad.detach().to(z.dtype).contiguous()
+    dz = torch.empty(z.shape, dtype=z.dtype, device=dev)
+    dgamma = torch.empty(2, S, dtype=torch.float32, device=dev)
+    dbeta = torch.empty(2, S, dtype=torch.float32, device=dev)
+    T = _ntok(z)
+    nws = lib.mega_gate_qk_bwd_workspace_bytes(T, S)
+    with _on_device(dev):
+        stream = _stream(dev)
+        ws = _scratch_buffer(dev, nws, stream)
+        rc = lib.mega_gate_qk_bwd(_ptr(dq), _ptr(dk), _ptr(zr), zs, _ptr(g), _ptr(f), _ptr(dz), _ptr(dgamma),
+                                  _ptr(dbeta), _dtype_code(zr), T, S, num_heads, int(chunk), int(pos0), float(eps),
+                                  _ptr(ws), ws.numel(), stream)
+    _lib.check(rc, "gate_qk_bwd")
+    return dz, dgamma, dbeta
+
+
 def gate_mul_fwd(a: torch.Tensor, r: torch.Tensor) -> torch.Tensor:
     """a * silu(r) (moving_average_gated_attention.py:330, 407)."""
     dev = _need_gpu(a, r)

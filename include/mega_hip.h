@@ -359,6 +359,17 @@ int mega_gate_out_fwd(const void* residual, int64_t residual_stride, const void*
  *                      h_grad = y_grad s silu'(hx + hp) (the gradient of hx and of hp),
  *                      s = sigmoid(u), h = silu(hx + hp)
  *   mega_swiglu_bwd:   a_grad = y_grad b silu'(a), b_grad = y_grad silu(a)                 */
+/* Backward of mega_gate_qk_fwd (the autograd graph of moving_average_gated_attention.py:324-328
+ * and of the rotation, relative_positional_bias.py:86-97): q_grad, k_grad, z_grad contiguous [T, S]
+ * of `dtype`, z as in the forward call; gamma [2, S] (holding the "+ 1"); gamma_grad, beta_grad
+ * [2, S] fp32.  S a multiple of 16 bytes' worth of elements, at most 1024 (bf16, fp16) or 512 (fp32)
+ * features.  The workspace holds one row of partial parameter sums per workgroup.          */
+size_t mega_gate_qk_bwd_workspace_bytes(int64_t T, int64_t S);
+int mega_gate_qk_bwd(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
+                     const float* gamma, const float* freqs, void* z_grad, float* gamma_grad,
+                     float* beta_grad, int dtype, int64_t T, int64_t S, int64_t heads,
+                     int64_t chunk, int64_t pos0, double eps, void* workspace,
+                     size_t workspace_bytes, void* stream);
 int mega_gate_mul_bwd(const void* y_grad, const void* a, int64_t a_stride, const void* r,
                       int64_t r_stride, void* a_grad, void* r_grad, int dtype, int64_t T, int64_t E,
                       void* stream);

@@ -467,6 +467,66 @@ def test_gate_backwards(dtype, shape, width, off):
     assert rel_err(host(gb), dy64 * O._silu(a64)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,S,heads,chunk,width,off", [(2, 64, 128, 1, 64, 128, 0), (1, 96, 64, 4, 32, 200, 72),
+                                                         (3, 40, 40, 2, 40, 56, 8), (1, 4096, 512, 4, 2048, 512, 0),
+                                                         (2, 300, 512, 2, 100, 1024, 512)])
+def test_gate_qk_bwd(dtype, B, L, S, heads, chunk, width, off):
+    """Backward of the q / k map against fp64 autograd through normalize -> affine -> rotation written
+    with torch operations on the CPU; z a slice of a wider row, one all-zero row (clamped norm)."""
+    from test_gpu_ops import _wide
+    rng = np.random.default_rng(97)
+    z, z64 = _wide(rng, (B, L, S), width, off, dtype)
+    with torch.no_grad():
+        z[0, 1].zero_()
+    z64[0, 1] = 0
+    g = rng.normal(size=(2, S)) * 0.3 + 1
+    b = rng.normal(size=(2, S)) * 0.3
+    Hd = S // heads
+    freqs = (1.0 / (10000.0 ** (np.arange(0, Hd, 2) / Hd))).astype(np.float32)
+    up = rng.normal(size=(2, B, L, S))
+    up[:, 0, 1] *= 1e-2                    # the clamped row scales its gradient by 1 / eps: keep it inside fp16
+    dq, dq64 = rounded(up[0], dtype)
+    dk, dk64 = rounded(up[1], dtype)
+    dz, dg, db = M.ops.gate_qk_bwd(dq, dk, z, dev(g), dev(freqs), heads, chunk)
+    # arbiter
+    tz = torch.from_numpy(z64).requires_grad_(True)
+    tg = torch.from_numpy(g).requires_grad_(True)
+    tb = torch.from_numpy(b).requires_grad_(True)
+    zn = tz / tz.norm(dim=-1, keepdim=True).clamp_min(1e-5)
+    ang = torch.arange(chunk, dtype=torch.float64)[:, None] * torch.from_numpy(freqs.astype(np.float64))[None, :]
+    cs, sn = torch.cos(ang)[None, :, None, :], torch.sin(ang)[None, :, None, :]
+    loss = 0
+    for i, up in ((0, dq64), (1, dk64)):
+        a = (zn * tg[i] + tb[i]).reshape(B * (L // chunk), chunk, heads, Hd // 2, 2)
+        a0, a1 = a[..., 0], a[..., 1]
+        rot = torch.stack([a0 * cs - a1 * sn, a0 * sn + a1 * cs], dim=-1).reshape(B, L, S)
+        loss = loss + (rot * torch.from_numpy(up)).sum()
+    loss.backward()
+    # a clamped row has gradient dzn / eps = 1e5 dzn: compare it apart from the others
+    ref = tz.grad.numpy()
+    got = host(dz)
+    keep = np.ones((B, L), bool); keep[0, 1] = False
+    tol = max(TOL[dtype], 5e-4)
+    assert rel_err(got[keep], ref[keep]) < tol
+    assert rel_err(got[0, 1], ref[0, 1]) < tol
+    # sums over all tokens of bf16-rounded products: fp32 accumulation, inputs exact
+    assert rel_err(host(dg), tg.grad.numpy()) < 5e-4 and rel_err(host(db), tb.grad.numpy()) < 5e-4
+
+
+def test_gate_qk_bwd_rejects_bad_arguments():
+    z = torch.zeros(2, 4, 36, device=DEV, dtype=torch.bfloat16)
+    g = torch.ones(2, 36, device=DEV)
+    with pytest.raises(RuntimeError):                                   # rows of 36 bf16 are not whole vectors
+        M.ops.gate_qk_bwd(z, z, z, g, torch.ones(9, device=DEV), 2, 4)
+    z = torch.zeros(2, 4, 2048, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):                                   # more than two vectors per lane
+        M.ops.gate_qk_bwd(z, z, z, torch.ones(2, 2048, device=DEV), torch.ones(1024, device=DEV), 1, 4)
+    z = torch.zeros(0, 64, device=DEV)
+    dz, dg, db = M.ops.gate_qk_bwd(z, z, z, torch.ones(2, 64, device=DEV), torch.ones(32, device=DEV), 1, 4)
+    assert dz.shape == (0, 64) and float(dg.abs().sum()) == 0 and float(db.abs().sum()) == 0
+
+
 def test_backward_edge_shapes():
     """Single-token and single-row inputs, channel counts that are not multiples of the tile sizes."""
     rng = np.random.default_rng(99)
