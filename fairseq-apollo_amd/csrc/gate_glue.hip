@@ -230,15 +230,37 @@ __global__ __launch_bounds__(kRowThreads) void gate_qk_bwd_kernel(
   for (int i = threadIdx.x; i < 4 * S; i += kRowThreads) dst[i] = s_acc[i];
 }
 
-// dgamma [2, S] = rows 0, 1 of the sums, dbeta [2, S] = rows 2, 3
-__global__ __launch_bounds__(256) void gate_qk_param_kernel(const float* __restrict__ part, int rows, int S,
-                                                            float* __restrict__ dgamma, float* __restrict__ dbeta) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= 4 * S) return;
-  float a = 0.f;
-  for (int r = 0; r < rows; ++r) a += part[(size_t)r * 4 * S + i];
-  if (i < 2 * S) dgamma[i] = a;
-  else dbeta[i - 2 * S] = a;
+// dgamma [2, S] = rows 0, 1 of the sums, dbeta [2, S] = rows 2, 3.  A workgroup owns 64 adjacent
+// columns; its 16 waves each add every 16th row (independent loads in flight, a fixed order inside
+// the wave), then the 16 sums of a column are added in wave order.
+constexpr int kParamSlices = 16;
+__global__ __launch_bounds__(64 * kParamSlices) void gate_qk_param_kernel(const float* __restrict__ part, int rows,
+                                                                          int S, float* __restrict__ dgamma,
+                                                                          float* __restrict__ dbeta) {
+  __shared__ float s_sum[kParamSlices][64];
+  const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  const size_t W = (size_t)4 * S;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  if (i < 4 * S) {
+    int r = slice;
+    for (; r + 3 * kParamSlices < rows; r += 4 * kParamSlices) {
+      a0 += part[(size_t)r * W + i];
+      a1 += part[(size_t)(r + kParamSlices) * W + i];
+      a2 += part[(size_t)(r + 2 * kParamSlices) * W + i];
+      a3 += part[(size_t)(r + 3 * kParamSlices) * W + i];
+    }
+    for (; r < rows; r += kParamSlices) a0 += part[(size_t)r * W + i];
+  }
+  s_sum[slice][lane] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (slice == 0 && i < 4 * S) {
+    float a = 0.f;
+#pragma unroll
+    for (int w = 0; w < kParamSlices; ++w) a += s_sum[w][lane];
+    if (i < 2 * S) dgamma[i] = a;
+    else dbeta[i - 2 * S] = a;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -455,7 +477,8 @@ int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs
     hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 2>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
                        (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
   MEGA_CHECK_LAUNCH("gate_qk_bwd");
-  hipLaunchKernelGGL(gate_qk_param_kernel, dim3((unsigned)ceil_div(4 * S, 256)), dim3(256), 0, s, part, (int)grid,
+  hipLaunchKernelGGL(gate_qk_param_kernel, dim3((unsigned)ceil_div(4 * S, 64)), dim3(64 * kParamSlices), 0, s, part,
+                     (int)grid,
                      (int)S, dgamma, dbeta);
   MEGA_CHECK_LAUNCH("gate_qk_bwd (parameter sums)");
   return MEGA_OK;
