@@ -20,7 +20,8 @@
 //
 // Thread mapping: TPR = ceil(N/4) lanes share one (batch, channel) row, 4 complex
 // states each; rows are laid out channel-fastest so that [B,L,D] activations are read
-// coalesced.
+// coalesced.  Activations with a contiguous time axis ([B,D,L]) take the *_rows kernels,
+// which stage sub-tiles of time through LDS.
 #include "common.h"
 #include "ema_mfma.h"
 
@@ -53,12 +54,25 @@ struct PassArgs {
   int before;              // output uses the state before absorbing the current sample
   int tshift;              // the filter input is delayed by tshift samples
   // output stage
-  const float* acc_in;     // [B, L, D] fp32 partial sums from earlier pass sets, or null
-  float* acc_out;          // [B, L, D] fp32, or null when this pass set writes y
+  const float* acc_in;     // fp32 partial sums from earlier pass sets, or null: [B, L, D], or [B, D, L]
+  float* acc_out;          // when the passes run on time-contiguous rows; null when this pass set writes y
   void* y;
   int64_t syb, syd, syl;
   const float* omega;      // [D]
 };
+
+// sum over the TPR (1, 2, 4 or 8) adjacent lanes of a unit, left in every one of them: lane exchanges
+// inside quads, then between the two quads of an 8-lane half (data-parallel primitives, no LDS traffic)
+template <int CTRL>
+__device__ __forceinline__ float lane_swap(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float unit_sum(float v, int tpr) {
+  if (tpr >= 2) v += lane_swap<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  if (tpr >= 4) v += lane_swap<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  if (tpr >= 8) v += lane_swap<0x141>(v);    // mirror inside each half row of 8 lanes
+  return v;
+}
 
 template <typename T>
 __device__ __forceinline__ float load_u(const PassArgs& A, int b, int d, int tau) {
@@ -112,46 +126,110 @@ __global__ __launch_bounds__(kBlock) void chunk_state_kernel(const PassArgs A) {
   }
 }
 
-// one thread per (b, d, state): serial over the chunks
+// Exclusive scan of the chunk states.  A (batch, channel) row is owned by G lane groups of NP
+// threads (thread = one state of one group); a group owns a run of consecutive chunks.  Pass 1 folds
+// the run into one aggregate (loads in batches, all of a batch in flight), the groups' aggregates
+// meet in LDS and every thread folds the earlier groups' into its start state, pass 2 walks the
+// run again and leaves the state at the start of every chunk in place of the chunk's own sum.
+// G is a power of two (1 when there are few chunks, then a workgroup owns 256 / NP rows).
+constexpr int kScanBatch = 8;
+
 template <bool CPLX>
-__global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A) {
-  const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int64_t total = (int64_t)A.B * A.D * A.NP;
-  if (gid >= total) return;
-  const int n = (int)(gid % A.NP);
-  const int d = (int)((gid / A.NP) % A.D);
-  const int b = (int)(gid / ((int64_t)A.NP * A.D));
+__global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A, const int G) {
+  __shared__ float s_agg[kBlock * 2];
+  const int n = threadIdx.x % A.NP;
+  const int grp = (threadIdx.x / A.NP) % G;
+  const int rloc = threadIdx.x / (A.NP * G);
+  const int rows_per_wg = kBlock / (A.NP * G);
+  const int64_t row = (int64_t)blockIdx.x * rows_per_wg + rloc;
+  const bool live = row < (int64_t)A.B * A.D;
+  const int d = live ? (int)(row % A.D) : 0;
+  const int b = live ? (int)(row / A.D) : 0;
   const size_t oc = ((size_t)d * A.NP + n) * 2;
   const double qr = A.coef.q[oc], qi = CPLX ? A.coef.q[oc + 1] : 0.0;
   const float p = A.coef.p[(size_t)d * A.NP + n];
   double Qr, Qi;
   cpow_int(qr, qi, A.Tc, &Qr, &Qi);
+  const float fQr = (float)Qr, fQi = (float)Qi;
+  const int cpg = (A.nchunks + G - 1) / G;
+  const int cb = min(grp * cpg, A.nchunks), ce = live ? min(cb + cpg, A.nchunks) : cb;
+  const size_t cstride = (size_t)A.D * A.NP * 2;
+  float* base = A.st + (((size_t)b * A.nchunks) * A.D + d) * A.NP * 2 + (size_t)n * 2;
+  // pass 1: the run's aggregate from a zero start
   float hr = 0.f, hi = 0.f;
-  if (A.h_in && n < A.N) {
+  for (int c = cb; c < ce; c += kScanBatch) {
+    float sr[kScanBatch], si[kScanBatch];
+#pragma unroll
+    for (int k = 0; k < kScanBatch; ++k) {
+      const bool ok = c + k < ce;
+      const float* sp = base + (size_t)(ok ? c + k : c) * cstride;
+      sr[k] = sp[0];
+      si[k] = CPLX ? sp[1] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < kScanBatch; ++k)
+      if (c + k < ce) {
+        const float nr = fQr * hr - fQi * hi + p * sr[k];
+        const float ni = fQr * hi + fQi * hr + p * si[k];
+        hr = nr;
+        hi = ni;
+      }
+  }
+  s_agg[threadIdx.x * 2] = hr;
+  s_agg[threadIdx.x * 2 + 1] = hi;
+  __syncthreads();
+  // start state of the run: the carried state pushed through the earlier runs
+  hr = 0.f;
+  hi = 0.f;
+  if (live && A.h_in && n < A.N) {
     const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
     hr = A.h_in[oh];
     hi = CPLX ? A.h_in[oh + 1] : 0.f;
   }
-  const float fQr = (float)Qr, fQi = (float)Qi;
-  for (int c = 0; c < A.nchunks; ++c) {
-    float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + n) * 2;
-    const float sr = sp[0], si = sp[1];
-    sp[0] = hr;
-    sp[1] = hi;
-    float Ar = fQr, Ai = fQi;
-    if (c == A.nchunks - 1) {
-      // the last chunk may be shorter
-      double lr, li;
-      cpow_int(qr, qi, A.L - c * A.Tc, &lr, &li);
-      Ar = (float)lr;
-      Ai = (float)li;
+  if (grp > 0) {
+    double Gr, Gi;
+    cpow_int(qr, qi, (int64_t)A.Tc * cpg, &Gr, &Gi);
+    const float fGr = (float)Gr, fGi = (float)Gi;
+    for (int j = 0; j < grp; ++j) {
+      const int o = (threadIdx.x - (grp - j) * A.NP) * 2;
+      const float nr = fGr * hr - fGi * hi + s_agg[o];
+      const float ni = fGr * hi + fGi * hr + s_agg[o + 1];
+      hr = nr;
+      hi = ni;
     }
-    const float nr = Ar * hr - Ai * hi + p * sr;
-    const float ni = Ar * hi + Ai * hr + p * si;
-    hr = nr;
-    hi = ni;
   }
-  if (A.h_out && n < A.N) {
+  // pass 2: chunk-start states in place; the last chunk of the row may be shorter
+  float Lr = fQr, Li = fQi;
+  if (ce == A.nchunks && ce > cb) {
+    double lr, li;
+    cpow_int(qr, qi, A.L - (int64_t)(A.nchunks - 1) * A.Tc, &lr, &li);
+    Lr = (float)lr;
+    Li = (float)li;
+  }
+  for (int c = cb; c < ce; c += kScanBatch) {
+    float sr[kScanBatch], si[kScanBatch];
+#pragma unroll
+    for (int k = 0; k < kScanBatch; ++k) {
+      const bool ok = c + k < ce;
+      const float* sp = base + (size_t)(ok ? c + k : c) * cstride;
+      sr[k] = sp[0];
+      si[k] = CPLX ? sp[1] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < kScanBatch; ++k)
+      if (c + k < ce) {
+        float* sp = base + (size_t)(c + k) * cstride;
+        sp[0] = hr;
+        sp[1] = hi;
+        const bool last = c + k == A.nchunks - 1;
+        const float Ar = last ? Lr : fQr, Ai = last ? Li : fQi;
+        const float nr = Ar * hr - Ai * hi + p * sr[k];
+        const float ni = Ar * hi + Ai * hr + p * si[k];
+        hr = nr;
+        hi = ni;
+      }
+  }
+  if (A.h_out && n < A.N && ce == A.nchunks && ce > cb) {
     const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
     A.h_out[oh] = hr;
     A.h_out[oh + 1] = hi;
@@ -207,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
 #pragma unroll
       for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
     }
-    for (int m = 1; m < A.TPR; m <<= 1) acc += __shfl_xor(acc, m);
+    acc = unit_sum(acc, A.TPR);
     if (ns == 0 && live) {
       const int t = A.reverse ? A.L - 1 - tau : tau;
       const size_t oa = ((size_t)b * A.L + t) * A.D + d;
@@ -220,6 +298,189 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
         ((T*)A.y)[b * A.syb + d * A.syd + t * A.syl] = from_float<T>(acc + om * xr);
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same two passes for activations whose time axis is contiguous ([B, D, L] rows): the units of
+// a workgroup (unit = one chunk of one row, TPR lanes) are consecutive (row, chunk) pairs, their
+// samples are staged through LDS in sub-tiles of kTS steps with loads and stores that run along
+// time, and the partial sums of earlier pass sets are kept as [B, D, L] as well.
+constexpr int kTS = 32;
+constexpr int kTSP = kTS + 1;      // row pitch of the LDS tile: units of a wave fall into different banks
+
+struct UnitMap {
+  float* tile;
+  int* ub;
+  int* ud;
+  int* ut0;
+};
+
+__device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds, int U) {
+  UnitMap m;
+  m.tile = lds;
+  m.ub = (int*)(lds + (size_t)U * kTSP);
+  m.ud = m.ub + U;
+  m.ut0 = m.ud + U;
+  const int64_t units = (int64_t)A.B * A.D * A.nchunks;
+  for (int u = threadIdx.x; u < U; u += kBlock) {
+    const int64_t g = (int64_t)blockIdx.x * U + u;
+    if (g < units) {
+      const int64_t row = g / A.nchunks;
+      m.ub[u] = (int)(row / A.D);
+      m.ud[u] = (int)(row % A.D);
+      m.ut0[u] = (int)(g % A.nchunks) * A.Tc;
+    } else {
+      m.ub[u] = 0;
+      m.ud[u] = 0;
+      m.ut0[u] = -1;
+    }
+  }
+  return m;
+}
+
+// logical steps of the unit that fall into the sub-tile starting s0 steps into the chunk
+__device__ __forceinline__ int unit_steps(const PassArgs& A, int t0, int s0) {
+  if (t0 < 0) return 0;
+  const int n = min(A.Tc - s0, A.L - (t0 + s0));
+  return n < 0 ? 0 : (n > kTS ? kTS : n);
+}
+
+template <typename T>
+__device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m, int U, int s0) {
+  for (int i = threadIdx.x; i < U * kTS; i += kBlock) {
+    const int u = i / kTS, off = i % kTS;
+    const int t0 = m.ut0[u];
+    float v = 0.f;
+    if (off < unit_steps(A, t0, s0)) v = load_u<T>(A, m.ub[u], m.ud[u], t0 + s0 + off);
+    m.tile[u * kTSP + off] = v;
+  }
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs A) {
+  extern __shared__ float lds[];
+  const int U = kBlock / A.TPR;
+  const UnitMap m = unit_map(A, lds, U);
+  __syncthreads();
+  const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
+  const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
+  float qr[kNPT], qi[kNPT], hr[kNPT], hi[kNPT];
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    qr[k] = A.coef.q[o];
+    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    hr[k] = 0.f;
+    hi[k] = 0.f;
+  }
+  for (int s0 = 0; s0 < A.Tc; s0 += kTS) {
+    stage_inputs<T>(A, m, U, s0);
+    __syncthreads();
+    const int steps = unit_steps(A, t0, s0);
+    const float* row = m.tile + u * kTSP;
+    for (int i = 0; i < steps; ++i) {
+      const float x = row[i];
+#pragma unroll
+      for (int k = 0; k < kNPT; ++k) {
+        if (CPLX) {
+          const float nr = qr[k] * hr[k] - qi[k] * hi[k] + x;
+          const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+          hr[k] = nr;
+          hi[k] = ni;
+        } else {
+          hr[k] = qr[k] * hr[k] + x;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  if (t0 < 0) return;
+  const int c = t0 / A.Tc;
+  float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + ns * kNPT) * 2;
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    sp[2 * k] = hr[k];
+    sp[2 * k + 1] = hi[k];
+  }
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs A) {
+  extern __shared__ float lds[];
+  const int U = kBlock / A.TPR;
+  const UnitMap m = unit_map(A, lds, U);
+  __syncthreads();
+  const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
+  const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
+  float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], pp[kNPT], hr[kNPT], hi[kNPT];
+  const int c = t0 < 0 ? 0 : t0 / A.Tc;
+  const float* sp = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + ns * kNPT) * 2;
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    qr[k] = A.coef.q[o];
+    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    cr[k] = A.coef.c[o];
+    ci[k] = CPLX ? A.coef.c[o + 1] : 0.f;
+    pp[k] = A.coef.p[o / 2];
+    hr[k] = sp[2 * k];
+    hi[k] = sp[2 * k + 1];
+  }
+  for (int s0 = 0; s0 < A.Tc; s0 += kTS) {
+    stage_inputs<T>(A, m, U, s0);
+    __syncthreads();
+    const int steps = unit_steps(A, t0, s0);
+    float* row = m.tile + u * kTSP;
+    for (int i = 0; i < steps; ++i) {
+      const float x = row[i];
+      float acc = 0.f;
+      if (A.before) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+      }
+#pragma unroll
+      for (int k = 0; k < kNPT; ++k) {
+        const float pu = pp[k] * x;
+        if (CPLX) {
+          const float nr = qr[k] * hr[k] - qi[k] * hi[k] + pu;
+          const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+          hr[k] = nr;
+          hi[k] = ni;
+        } else {
+          hr[k] = qr[k] * hr[k] + pu;
+        }
+      }
+      if (!A.before) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+      }
+      acc = unit_sum(acc, A.TPR);
+      if (ns == 0) row[i] = acc;          // the sample of this step has been consumed by every lane of the unit
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < U * kTS; i += kBlock) {
+      const int uu = i / kTS, off = i % kTS;
+      const int tt0 = m.ut0[uu];
+      if (off >= unit_steps(A, tt0, s0)) continue;
+      const int tau = tt0 + s0 + off;
+      const int t = A.reverse ? A.L - 1 - tau : tau;
+      const int bb = m.ub[uu], dd = m.ud[uu];
+      float acc = m.tile[uu * kTSP + off];
+      const size_t oa = ((size_t)bb * A.D + dd) * A.L + t;
+      if (A.acc_in) acc += A.acc_in[oa];
+      if (A.acc_out) {
+        A.acc_out[oa] = acc;
+      } else {
+        float xr = 0.f, om = 0.f;
+        if (A.omega) {
+          om = A.omega[dd];
+          xr = to_float(((const T*)A.x)[bb * A.sxb + dd * A.sxd + t * A.sxl]);
+        }
+        ((T*)A.y)[bb * A.syb + dd * A.syd + t * A.syl] = from_float<T>(acc + om * xr);
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -306,23 +567,42 @@ Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_
   return pl;
 }
 
-template <typename T>
-int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
+// lane groups per row of the chunk scan: enough that a group's run is a few load batches
+inline int scan_groups(int NP, int nchunks) {
+  int g = 1;
+  while (g * NP < kBlock && g * 2 * kScanBatch <= nchunks) g <<= 1;
+  return g;
+}
+
+template <typename T, bool CPLX>
+int run_pass_set_t(PassArgs& A, bool state_only, hipStream_t s) {
   const int64_t tA = (int64_t)A.B * A.nchunks * A.D * A.TPR;
-  const int64_t tB = (int64_t)A.B * A.D * A.NP;
-  if (cplx) {
-    hipLaunchKernelGGL((chunk_state_kernel<T, true>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
-    hipLaunchKernelGGL((chunk_scan_kernel<true>), dim3((unsigned)ceil_div(tB, kBlock)), dim3(kBlock), 0, s, A);
-    if (!state_only)
-      hipLaunchKernelGGL((chunk_apply_kernel<T, true>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
-  } else {
-    hipLaunchKernelGGL((chunk_state_kernel<T, false>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
-    hipLaunchKernelGGL((chunk_scan_kernel<false>), dim3((unsigned)ceil_div(tB, kBlock)), dim3(kBlock), 0, s, A);
-    if (!state_only)
-      hipLaunchKernelGGL((chunk_apply_kernel<T, false>), dim3((unsigned)ceil_div(tA, kBlock)), dim3(kBlock), 0, s, A);
+  // time-contiguous activations take the LDS-staged passes
+  const bool rows = A.sxl == 1 && A.L > 1 && (state_only || A.syl == 1);
+  const int U = kBlock / A.TPR;
+  const size_t lds = (size_t)U * (kTSP + 3) * 4;
+  const dim3 gridA((unsigned)ceil_div(tA, kBlock));
+  if (rows)
+    hipLaunchKernelGGL((chunk_state_rows_kernel<T, CPLX>), gridA, dim3(kBlock), lds, s, A);
+  else
+    hipLaunchKernelGGL((chunk_state_kernel<T, CPLX>), gridA, dim3(kBlock), 0, s, A);
+  const int G = scan_groups(A.NP, A.nchunks);
+  const int rows_per_wg = kBlock / (A.NP * G);
+  hipLaunchKernelGGL((chunk_scan_kernel<CPLX>), dim3((unsigned)ceil_div((int64_t)A.B * A.D, rows_per_wg)),
+                     dim3(kBlock), 0, s, A, G);
+  if (!state_only) {
+    if (rows)
+      hipLaunchKernelGGL((chunk_apply_rows_kernel<T, CPLX>), gridA, dim3(kBlock), lds, s, A);
+    else
+      hipLaunchKernelGGL((chunk_apply_kernel<T, CPLX>), gridA, dim3(kBlock), 0, s, A);
   }
   MEGA_CHECK_LAUNCH("ema pass");
   return MEGA_OK;
+}
+
+template <typename T>
+int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
+  return cplx ? run_pass_set_t<T, true>(A, state_only, s) : run_pass_set_t<T, false>(A, state_only, s);
 }
 
 int run_pass_set_dtype(int dtype, PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
