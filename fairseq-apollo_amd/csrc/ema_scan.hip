@@ -304,27 +304,37 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
 // ---------------------------------------------------------------------------------------------
 // The same two passes for activations whose time axis is contiguous ([B, D, L] rows): the units of
 // a workgroup (unit = one chunk of one row, TPR lanes) are consecutive (row, chunk) pairs, their
-// samples are staged through LDS in sub-tiles of kTS steps with loads and stores that run along
+// samples are staged through LDS one sub-tile of steps at a time with loads and stores that run along
 // time, and the partial sums of earlier pass sets are kept as [B, D, L] as well.
-constexpr int kTS = 32;
-constexpr int kTSP = kTS + 1;      // row pitch of the LDS tile: units of a wave fall into different banks
+// A sub-tile is 64 steps (32 when the chunks are no longer than that, or when a unit is a single
+// lane and a workgroup holds 256 units).
+__host__ __device__ inline int rows_ts_log2(int tpr, int tc) { return tpr >= 2 && tc > 32 ? 6 : 5; }
+__host__ __device__ inline size_t rows_lds_bytes(int tpr, int tc) {
+  const int U = kBlock / tpr;
+  return (size_t)U * ((1 << rows_ts_log2(tpr, tc)) + 1 + 3) * 4;
+}
 
 struct UnitMap {
-  float* tile;
+  float* tile;     // [U][pitch], pitch = ts + 1: the units of a wave fall into different banks
   int* ub;
   int* ud;
   int* ut0;
+  int U, tsl, ts, pitch;
 };
 
-__device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds, int U) {
+__device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds) {
   UnitMap m;
+  m.U = kBlock / A.TPR;
+  m.tsl = rows_ts_log2(A.TPR, A.Tc);
+  m.ts = 1 << m.tsl;
+  m.pitch = m.ts + 1;
   m.tile = lds;
-  m.ub = (int*)(lds + (size_t)U * kTSP);
-  m.ud = m.ub + U;
-  m.ut0 = m.ud + U;
+  m.ub = (int*)(lds + (size_t)m.U * m.pitch);
+  m.ud = m.ub + m.U;
+  m.ut0 = m.ud + m.U;
   const int64_t units = (int64_t)A.B * A.D * A.nchunks;
-  for (int u = threadIdx.x; u < U; u += kBlock) {
-    const int64_t g = (int64_t)blockIdx.x * U + u;
+  for (int u = threadIdx.x; u < m.U; u += kBlock) {
+    const int64_t g = (int64_t)blockIdx.x * m.U + u;
     if (g < units) {
       const int64_t row = g / A.nchunks;
       m.ub[u] = (int)(row / A.D);
@@ -340,28 +350,44 @@ __device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds, int U
 }
 
 // logical steps of the unit that fall into the sub-tile starting s0 steps into the chunk
-__device__ __forceinline__ int unit_steps(const PassArgs& A, int t0, int s0) {
+__device__ __forceinline__ int unit_steps(const PassArgs& A, const UnitMap& m, int t0, int s0) {
   if (t0 < 0) return 0;
   const int n = min(A.Tc - s0, A.L - (t0 + s0));
-  return n < 0 ? 0 : (n > kTS ? kTS : n);
+  return n < 0 ? 0 : (n > m.ts ? m.ts : n);
 }
 
+// samples beyond a unit's steps are staged as zeros; a thread's elements go in batches whose loads
+// are all issued before the first of them is used
+constexpr int kStageBatch = 8;
+
 template <typename T>
-__device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m, int U, int s0) {
-  for (int i = threadIdx.x; i < U * kTS; i += kBlock) {
-    const int u = i / kTS, off = i % kTS;
-    const int t0 = m.ut0[u];
-    float v = 0.f;
-    if (off < unit_steps(A, t0, s0)) v = load_u<T>(A, m.ub[u], m.ud[u], t0 + s0 + off);
-    m.tile[u * kTSP + off] = v;
+__device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m, int s0) {
+  const int per_thread = (m.U << m.tsl) / kBlock;          // ts / TPR: 4 or a multiple of the batch
+  for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
+    float v[kStageBatch];
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j) {
+      const int i = (e0 + j) * kBlock + threadIdx.x;
+      const int u = i >> m.tsl, off = i & (m.ts - 1);
+      const int t0 = e0 + j < per_thread ? m.ut0[u] : -1;
+      v[j] = 0.f;
+      if (e0 + j < per_thread && off < unit_steps(A, m, t0, s0))
+        v[j] = load_u<T>(A, m.ub[u], m.ud[u], t0 + s0 + off);
+    }
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j) {
+      const int i = (e0 + j) * kBlock + threadIdx.x;
+      if (e0 + j < per_thread) m.tile[(i >> m.tsl) * m.pitch + (i & (m.ts - 1))] = v[j];
+    }
   }
 }
+
+constexpr int kStepBlock = 8;      // steps whose samples are fetched from LDS together
 
 template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs A) {
   extern __shared__ float lds[];
-  const int U = kBlock / A.TPR;
-  const UnitMap m = unit_map(A, lds, U);
+  const UnitMap m = unit_map(A, lds);
   __syncthreads();
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
   const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
@@ -374,22 +400,29 @@ __global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs
     hr[k] = 0.f;
     hi[k] = 0.f;
   }
-  for (int s0 = 0; s0 < A.Tc; s0 += kTS) {
-    stage_inputs<T>(A, m, U, s0);
+  for (int s0 = 0; s0 < A.Tc; s0 += m.ts) {
+    stage_inputs<T>(A, m, s0);
     __syncthreads();
-    const int steps = unit_steps(A, t0, s0);
-    const float* row = m.tile + u * kTSP;
-    for (int i = 0; i < steps; ++i) {
-      const float x = row[i];
+    const int steps = unit_steps(A, m, t0, s0);
+    const float* row = m.tile + u * m.pitch;
+    for (int i0 = 0; i0 < steps; i0 += kStepBlock) {
+      float xs[kStepBlock];
 #pragma unroll
-      for (int k = 0; k < kNPT; ++k) {
-        if (CPLX) {
-          const float nr = qr[k] * hr[k] - qi[k] * hi[k] + x;
-          const float ni = qr[k] * hi[k] + qi[k] * hr[k];
-          hr[k] = nr;
-          hi[k] = ni;
-        } else {
-          hr[k] = qr[k] * hr[k] + x;
+      for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];      // inside the row: ts is a multiple of the block
+#pragma unroll
+      for (int j = 0; j < kStepBlock; ++j) {
+        if (i0 + j < steps) {                                        // the state must not run past the last step
+#pragma unroll
+          for (int k = 0; k < kNPT; ++k) {
+            if (CPLX) {
+              const float nr = qr[k] * hr[k] - qi[k] * hi[k] + xs[j];
+              const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+              hr[k] = nr;
+              hi[k] = ni;
+            } else {
+              hr[k] = qr[k] * hr[k] + xs[j];
+            }
+          }
         }
       }
     }
@@ -408,8 +441,7 @@ __global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs
 template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs A) {
   extern __shared__ float lds[];
-  const int U = kBlock / A.TPR;
-  const UnitMap m = unit_map(A, lds, U);
+  const UnitMap m = unit_map(A, lds);
   __syncthreads();
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
   const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
@@ -427,57 +459,82 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs
     hr[k] = sp[2 * k];
     hi[k] = sp[2 * k + 1];
   }
-  for (int s0 = 0; s0 < A.Tc; s0 += kTS) {
-    stage_inputs<T>(A, m, U, s0);
+  for (int s0 = 0; s0 < A.Tc; s0 += m.ts) {
+    stage_inputs<T>(A, m, s0);
     __syncthreads();
-    const int steps = unit_steps(A, t0, s0);
-    float* row = m.tile + u * kTSP;
-    for (int i = 0; i < steps; ++i) {
-      const float x = row[i];
-      float acc = 0.f;
-      if (A.before) {
+    const int steps = unit_steps(A, m, t0, s0);
+    float* row = m.tile + u * m.pitch;
+    // whole blocks of steps: the zeros staged past the last step only touch a state that is not
+    // used again (a short sub-tile is the unit's last) and outputs that the store below skips
+    for (int i0 = 0; i0 < steps; i0 += kStepBlock) {
+      float xs[kStepBlock];
 #pragma unroll
-        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
-      }
+      for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
 #pragma unroll
-      for (int k = 0; k < kNPT; ++k) {
-        const float pu = pp[k] * x;
-        if (CPLX) {
-          const float nr = qr[k] * hr[k] - qi[k] * hi[k] + pu;
-          const float ni = qr[k] * hi[k] + qi[k] * hr[k];
-          hr[k] = nr;
-          hi[k] = ni;
-        } else {
-          hr[k] = qr[k] * hr[k] + pu;
+      for (int j = 0; j < kStepBlock; ++j) {
+        float acc = 0.f;
+        if (A.before) {
+#pragma unroll
+          for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
         }
-      }
-      if (!A.before) {
 #pragma unroll
-        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+        for (int k = 0; k < kNPT; ++k) {
+          const float pu = pp[k] * xs[j];
+          if (CPLX) {
+            const float nr = qr[k] * hr[k] - qi[k] * hi[k] + pu;
+            const float ni = qr[k] * hi[k] + qi[k] * hr[k];
+            hr[k] = nr;
+            hi[k] = ni;
+          } else {
+            hr[k] = qr[k] * hr[k] + pu;
+          }
+        }
+        if (!A.before) {
+#pragma unroll
+          for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+        }
+        xs[j] = unit_sum(acc, A.TPR);
       }
-      acc = unit_sum(acc, A.TPR);
-      if (ns == 0) row[i] = acc;          // the sample of this step has been consumed by every lane of the unit
+      if (ns == 0) {                      // the samples of these steps have been consumed by every lane of the unit
+#pragma unroll
+        for (int j = 0; j < kStepBlock; ++j) row[i0 + j] = xs[j];
+      }
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < U * kTS; i += kBlock) {
-      const int uu = i / kTS, off = i % kTS;
-      const int tt0 = m.ut0[uu];
-      if (off >= unit_steps(A, tt0, s0)) continue;
-      const int tau = tt0 + s0 + off;
-      const int t = A.reverse ? A.L - 1 - tau : tau;
-      const int bb = m.ub[uu], dd = m.ud[uu];
-      float acc = m.tile[uu * kTSP + off];
-      const size_t oa = ((size_t)bb * A.D + dd) * A.L + t;
-      if (A.acc_in) acc += A.acc_in[oa];
-      if (A.acc_out) {
-        A.acc_out[oa] = acc;
-      } else {
-        float xr = 0.f, om = 0.f;
-        if (A.omega) {
-          om = A.omega[dd];
-          xr = to_float(((const T*)A.x)[bb * A.sxb + dd * A.sxd + t * A.sxl]);
+    const int per_thread = (m.U << m.tsl) / kBlock;
+    for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
+      float acc[kStageBatch], xr[kStageBatch], om[kStageBatch];
+      int64_t oy[kStageBatch];
+      size_t oa[kStageBatch];
+      bool on[kStageBatch];
+#pragma unroll
+      for (int j = 0; j < kStageBatch; ++j) {
+        const int i = (e0 + j) * kBlock + threadIdx.x;
+        const int uu = i >> m.tsl, off = i & (m.ts - 1);
+        const bool mine = e0 + j < per_thread;
+        const int tt0 = mine ? m.ut0[uu] : -1;
+        on[j] = mine && off < unit_steps(A, m, tt0, s0);
+        const int tau = tt0 + s0 + off;
+        const int t = A.reverse ? A.L - 1 - tau : tau;
+        const int bb = mine ? m.ub[uu] : 0, dd = mine ? m.ud[uu] : 0;
+        acc[j] = mine ? m.tile[uu * m.pitch + off] : 0.f;
+        oa[j] = ((size_t)bb * A.D + dd) * A.L + t;
+        oy[j] = bb * A.syb + dd * A.syd + t * A.syl;
+        xr[j] = 0.f;
+        om[j] = 0.f;
+        if (on[j]) {
+          if (A.acc_in) acc[j] += A.acc_in[oa[j]];
+          if (!A.acc_out && A.omega) {
+            om[j] = A.omega[dd];
+            xr[j] = to_float(((const T*)A.x)[bb * A.sxb + dd * A.sxd + t * A.sxl]);
+          }
         }
-        ((T*)A.y)[bb * A.syb + dd * A.syd + t * A.syl] = from_float<T>(acc + om * xr);
+      }
+#pragma unroll
+      for (int j = 0; j < kStageBatch; ++j) {
+        if (!on[j]) continue;
+        if (A.acc_out) A.acc_out[oa[j]] = acc[j];
+        else ((T*)A.y)[oy[j]] = from_float<T>(acc[j] + om[j] * xr[j]);
       }
     }
     __syncthreads();
@@ -579,8 +636,7 @@ int run_pass_set_t(PassArgs& A, bool state_only, hipStream_t s) {
   const int64_t tA = (int64_t)A.B * A.nchunks * A.D * A.TPR;
   // time-contiguous activations take the LDS-staged passes
   const bool rows = A.sxl == 1 && A.L > 1 && (state_only || A.syl == 1);
-  const int U = kBlock / A.TPR;
-  const size_t lds = (size_t)U * (kTSP + 3) * 4;
+  const size_t lds = rows_lds_bytes(A.TPR, A.Tc);
   const dim3 gridA((unsigned)ceil_div(tA, kBlock));
   if (rows)
     hipLaunchKernelGGL((chunk_state_rows_kernel<T, CPLX>), gridA, dim3(kBlock), lds, s, A);
