@@ -252,6 +252,86 @@ def bench_seqnorm(args):
     }))
 
 
+def bench_ema_real(args):
+    """configs[0] and configs[1]: the real MultiHeadEMA forward in fp32 on [B, D, L] rows (one-sided,
+    B2 x D512 x L1024; two-sided with a right-padding mask, B1 x D256 x L16384).  The value is
+    configs[1]'s; the CPU leg is the oracle's FFT convolution of the same call."""
+    import numpy as np
+    import torch
+
+    import fairseq_apollo_amd as M
+    from conftest import mega_init_real, rel_err
+    from oracle import mega_oracle as O
+
+    dev = torch.device("cuda:0")
+    out = {}
+    for name, (b, d, l, bidir, seed) in (("configs[0]", (2, 512, 1024, False, 1234)),
+                                         ("configs[1]", (1, 256, 16384, True, 1235))):
+        rng = np.random.default_rng(seed)
+        K = 2 * d if bidir else d
+        alpha, delta, beta, gamma = mega_init_real(rng, K, N)
+        omega = rng.normal(0, 1.0, d)
+        m = M.MultiHeadEMA(d, ndim=N, bidirectional=bidir).to(dev).eval()
+        with torch.no_grad():
+            for prm, v in ((m.alpha, alpha), (m.delta, delta), (m.beta, beta), (m.gamma, gamma), (m.omega, omega)):
+                prm.copy_(torch.from_numpy(np.asarray(v, np.float32)).reshape(prm.shape))
+        x = rng.normal(size=(b, d, l)).astype(np.float32)
+        mask = None
+        if bidir:
+            mask = np.zeros((b, l), bool)
+            for i in range(b):
+                mask[i, l - int(rng.integers(0, l // 4 + 1)):] = True
+        nbuf = 4
+        xs = [torch.from_numpy(x).to(dev) for _ in range(nbuf)]
+        tm = None if mask is None else torch.from_numpy(mask).to(dev)
+        with torch.no_grad():
+            for i in range(max(args.warmup, 1)):
+                y = m(xs[i % nbuf], tm)
+            a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            a.record()
+            for i in range(args.steps):
+                y = m(xs[i % nbuf], tm)
+            e.record()
+            torch.cuda.synchronize()
+        ms = a.elapsed_time(e) / args.steps
+        p_, q_, g_ = O.ema_coeffs_real(alpha.astype(np.float32), delta.astype(np.float32), beta.astype(np.float32),
+                                       gamma.astype(np.float32))
+        cpu = None
+        ref = None
+        if not args.no_cpu:
+            times = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                ref, _ = O.ema_forward(x, p_, q_, g_, omega.astype(np.float32), padding_mask=mask, bidirectional=bidir)
+                times.append(time.perf_counter() - t0)
+            cpu = sorted(times)[1]
+        alg = 2 * b * d * l * 4
+        out[name] = {"ms": ms, "tokens_per_s": b * l / (ms * 1e-3), "algorithmic_bytes": alg,
+                     "hbm_gbs": alg / (ms * 1e-3) / 1e9, "cpu_ms": None if cpu is None else cpu * 1e3,
+                     "rel_err_vs_oracle": None if ref is None else rel_err(y.float().cpu().numpy(), ref)}
+    c1 = out["configs[1]"]
+    line = {
+        "metric": "real MultiHeadEMA forward tokens/sec @B1xL16384xD256 (bidirectional, fp32)",
+        "value": c1["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": c1["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: bidirectional real MultiHeadEMA (N=16), B=1 L=16384 D=256, fp32, "
+                               "right-padding mask; configs[0] beside it"},
+        "roofline": {"bound": "hbm", "kernel": "chunk_state_rows + chunk_scan + chunk_apply_rows, both directions",
+                     "achieved": c1["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": c1["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_step": c1["algorithmic_bytes"]},
+        "cases": out,
+    }
+    if c1["cpu_ms"] is not None:
+        line["cpu_baseline"] = {"value": 16384 / (c1["cpu_ms"] * 1e-3), "unit": "tokens/s",
+                                "cores": 1, "kind": "port",
+                                "sample": "the whole configs[1] call through the oracle's numpy kernel generation "
+                                          "and FFT convolution (fp64, one thread), median of 3"}
+    print(json.dumps(line))
+
+
 def bench_attention(args):
     """configs[4]'s attention: 4 chunks of 2048 tokens, 4 heads, H1 = 128, H2 = 1024, bf16, causal
     (matrix-core bound).  Flops are counted for the causal half only: 2 * C^2/2 * (H1 + H2) per chunk-head."""
@@ -359,10 +439,11 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm"], default="block",
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real"],
+                    default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
-                         "the decode step of configs[3] / the chunk attention / the whole layer of configs[4], "
-                         "one JSON line each")
+                         "the decode step of configs[3] / the chunk attention / the whole layer of configs[4]; "
+                         "ema_real: the fp32 real-EMA calls of configs[0] and configs[1]; one JSON line each")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -370,6 +451,8 @@ def main():
 
     if args.workload == "decode":
         return bench_decode(args)
+    if args.workload == "ema_real":
+        return bench_ema_real(args)
     if args.workload == "seqnorm":
         return bench_seqnorm(args)
     if args.workload == "block_bwd":

@@ -80,8 +80,10 @@ __device__ __forceinline__ float load_u(const PassArgs& A, int b, int d, int tau
   const int ts = tau - A.tshift;
   if (ts < 0) return 0.f;
   const int t = A.reverse ? A.L - 1 - ts : ts;
-  if (A.mask && A.mask[(size_t)b * A.L + t]) return 0.f;
-  return to_float(((const T*)A.x)[b * A.sxb + d * A.sxd + t * A.sxl]);
+  // both loads are issued before either is looked at: one round trip, not two
+  const T v = ((const T*)A.x)[b * A.sxb + d * A.sxd + t * A.sxl];
+  const uint8_t pad = A.mask ? A.mask[(size_t)b * A.L + t] : (uint8_t)0;
+  return pad ? 0.f : to_float(v);
 }
 
 template <typename T, bool CPLX>
