@@ -310,14 +310,17 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
 // time, and the partial sums of earlier pass sets are kept as [B, D, L] as well.
 // A sub-tile is 64 steps (32 when the chunks are no longer than that, or when a unit is a single
 // lane and a workgroup holds 256 units).
+constexpr int kUnitWords = 7;      // 32-bit words of the unit map per unit
 __host__ __device__ inline int rows_ts_log2(int tpr, int tc) { return tpr >= 2 && tc > 32 ? 6 : 5; }
 __host__ __device__ inline size_t rows_lds_bytes(int tpr, int tc) {
   const int U = kBlock / tpr;
-  return (size_t)U * ((1 << rows_ts_log2(tpr, tc)) + 1 + 3) * 4;
+  return (size_t)U * ((1 << rows_ts_log2(tpr, tc)) + 1 + kUnitWords) * 4;
 }
 
 struct UnitMap {
   float* tile;     // [U][pitch], pitch = ts + 1: the units of a wave fall into different banks
+  int64_t* uxo;    // offset of the unit's row in x (time stride 1), and in y
+  int64_t* uyo;
   int* ub;
   int* ud;
   int* ut0;
@@ -331,24 +334,39 @@ __device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds) {
   m.ts = 1 << m.tsl;
   m.pitch = m.ts + 1;
   m.tile = lds;
-  m.ub = (int*)(lds + (size_t)m.U * m.pitch);
+  m.uxo = (int64_t*)(lds + (size_t)m.U * m.pitch);       // U is a multiple of 32: 8-byte aligned
+  m.uyo = m.uxo + m.U;
+  m.ub = (int*)(m.uyo + m.U);
   m.ud = m.ub + m.U;
   m.ut0 = m.ud + m.U;
   const int64_t units = (int64_t)A.B * A.D * A.nchunks;
   for (int u = threadIdx.x; u < m.U; u += kBlock) {
     const int64_t g = (int64_t)blockIdx.x * m.U + u;
+    int b = 0, d = 0, t0 = -1;
     if (g < units) {
       const int64_t row = g / A.nchunks;
-      m.ub[u] = (int)(row / A.D);
-      m.ud[u] = (int)(row % A.D);
-      m.ut0[u] = (int)(g % A.nchunks) * A.Tc;
-    } else {
-      m.ub[u] = 0;
-      m.ud[u] = 0;
-      m.ut0[u] = -1;
+      b = (int)(row / A.D);
+      d = (int)(row % A.D);
+      t0 = (int)(g % A.nchunks) * A.Tc;
     }
+    m.ub[u] = b;
+    m.ud[u] = d;
+    m.ut0[u] = t0;
+    m.uxo[u] = b * A.sxb + d * A.sxd;
+    m.uyo[u] = b * A.syb + d * A.syd;
   }
   return m;
+}
+
+// logical sample tau of the (delayed, masked) filter input of a time-contiguous row at offset xo
+template <typename T>
+__device__ __forceinline__ float load_row_u(const PassArgs& A, int64_t xo, int b, int tau) {
+  const int ts = tau - A.tshift;
+  if (ts < 0) return 0.f;
+  const int t = A.reverse ? A.L - 1 - ts : ts;
+  const T v = ((const T*)A.x)[xo + t];
+  const uint8_t pad = A.mask ? A.mask[(size_t)b * A.L + t] : (uint8_t)0;
+  return pad ? 0.f : to_float(v);
 }
 
 // logical steps of the unit that fall into the sub-tile starting s0 steps into the chunk
@@ -374,7 +392,7 @@ __device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m
       const int t0 = e0 + j < per_thread ? m.ut0[u] : -1;
       v[j] = 0.f;
       if (e0 + j < per_thread && off < unit_steps(A, m, t0, s0))
-        v[j] = load_u<T>(A, m.ub[u], m.ud[u], t0 + s0 + off);
+        v[j] = load_row_u<T>(A, m.uxo[u], m.ub[u], t0 + s0 + off);
     }
 #pragma unroll
     for (int j = 0; j < kStageBatch; ++j) {
@@ -521,14 +539,14 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs
         const int bb = mine ? m.ub[uu] : 0, dd = mine ? m.ud[uu] : 0;
         acc[j] = mine ? m.tile[uu * m.pitch + off] : 0.f;
         oa[j] = ((size_t)bb * A.D + dd) * A.L + t;
-        oy[j] = bb * A.syb + dd * A.syd + t * A.syl;
+        oy[j] = (mine ? m.uyo[uu] : 0) + t;
         xr[j] = 0.f;
         om[j] = 0.f;
         if (on[j]) {
           if (A.acc_in) acc[j] += A.acc_in[oa[j]];
           if (!A.acc_out && A.omega) {
             om[j] = A.omega[dd];
-            xr[j] = to_float(((const T*)A.x)[bb * A.sxb + dd * A.sxd + t * A.sxl]);
+            xr[j] = to_float(((const T*)A.x)[m.uxo[uu] + t]);
           }
         }
       }
@@ -540,6 +558,211 @@ __global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs
       }
     }
     __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Two-sided layers on time-contiguous rows whose chunks fit one sub-tile: both directions share the
+// staged samples.  The direction that runs back in time uses the same chunk boundaries as the forward
+// one (its chunk j is the forward chunk nchunks - 1 - j, walked from its last sample to its first);
+// the only chunk that can be short is then the first it meets, where the state is still zero, so the
+// scan's uniform factor q^Tc holds for it as well.  `rc`, `st_r`: coefficients and chunk states of
+// that direction; `before`: its output at a sample excludes the sample itself (fftconv.py:85-100
+// with shift).
+__host__ __device__ inline size_t bidir_lds_bytes(int tpr, int tc) {
+  const int U = kBlock / tpr;
+  return (size_t)U * (2 * ((1 << rows_ts_log2(tpr, tc)) + 1) + kUnitWords) * 4;
+}
+
+// h <- q h + x (the imaginary parts are untouched for real coefficients)
+template <bool CPLX>
+__device__ __forceinline__ void state_step(float qr, float qi, float& hr, float& hi, float x) {
+  if (CPLX) {
+    const float nr = qr * hr - qi * hi + x;
+    hi = qr * hi + qi * hr;
+    hr = nr;
+  } else {
+    hr = fmaf(qr, hr, x);
+  }
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void bidir_state_rows_kernel(const PassArgs A, const PassCoef rc,
+                                                                  float* __restrict__ st_r) {
+  extern __shared__ float lds[];
+  const UnitMap m = unit_map(A, lds);
+  __syncthreads();
+  const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
+  const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
+  float fr[kNPT], fi[kNPT], br[kNPT], bi[kNPT], hr[kNPT], hi[kNPT], gr[kNPT], gi[kNPT];
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    fr[k] = A.coef.q[o];
+    fi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    br[k] = rc.q[o];
+    bi[k] = CPLX ? rc.q[o + 1] : 0.f;
+    hr[k] = hi[k] = gr[k] = gi[k] = 0.f;
+  }
+  stage_inputs<T>(A, m, 0);
+  __syncthreads();
+  const int steps = unit_steps(A, m, t0, 0);
+  const float* row = m.tile + u * m.pitch;
+  // whole blocks of steps run unguarded; the block that holds the last step checks every step
+  const int whole = steps / kStepBlock * kStepBlock;
+  for (int i0 = 0; i0 < steps; i0 += kStepBlock) {
+    float xs[kStepBlock];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
+    if (i0 < whole) {
+#pragma unroll
+      for (int j = 0; j < kStepBlock; ++j)
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) state_step<CPLX>(fr[k], fi[k], hr[k], hi[k], xs[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kStepBlock; ++j)
+        if (i0 + j < steps) {
+#pragma unroll
+          for (int k = 0; k < kNPT; ++k) state_step<CPLX>(fr[k], fi[k], hr[k], hi[k], xs[j]);
+        }
+    }
+  }
+  for (int i0 = ((steps - 1) / kStepBlock) * kStepBlock; i0 >= 0 && steps > 0; i0 -= kStepBlock) {
+    float xs[kStepBlock];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
+    if (i0 < whole) {
+#pragma unroll
+      for (int j = kStepBlock - 1; j >= 0; --j)
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) state_step<CPLX>(br[k], bi[k], gr[k], gi[k], xs[j]);
+    } else {
+#pragma unroll
+      for (int j = kStepBlock - 1; j >= 0; --j)
+        if (i0 + j < steps) {
+#pragma unroll
+          for (int k = 0; k < kNPT; ++k) state_step<CPLX>(br[k], bi[k], gr[k], gi[k], xs[j]);
+        }
+    }
+  }
+  if (t0 < 0) return;
+  const int c = t0 / A.Tc;
+  float* sf = A.st + ((((size_t)b * A.nchunks + c) * A.D + d) * A.NP + ns * kNPT) * 2;
+  float* sr = st_r + ((((size_t)b * A.nchunks + (A.nchunks - 1 - c)) * A.D + d) * A.NP + ns * kNPT) * 2;
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    sf[2 * k] = hr[k];
+    sf[2 * k + 1] = hi[k];
+    sr[2 * k] = gr[k];
+    sr[2 * k + 1] = gi[k];
+  }
+}
+
+// One direction of the apply pass over the unit's staged samples (ASC: forward in time, its outputs
+// are stored to out[]; otherwise from the last sample to the first, added to out[]).  The state is
+// carried as h / p, so a step is h <- q h + x and the output coefficient is c p: one multiply per
+// state and step less (padded states have p = c = 0 and stay zero).
+template <bool CPLX, bool ASC, bool BEFORE>
+__device__ __forceinline__ void bidir_sweep(const PassCoef& cf, const float* st, int d, int NP, int ns, int tpr,
+                                            const float* row, float* out, int steps) {
+  float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], hr[kNPT], hi[kNPT];
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * NP + ns * kNPT + k) * 2;
+    qr[k] = cf.q[o];
+    qi[k] = CPLX ? cf.q[o + 1] : 0.f;
+    const float p = cf.p[o / 2];
+    const float ip = p != 0.f ? 1.0f / p : 0.f;
+    cr[k] = cf.c[o] * p;
+    ci[k] = CPLX ? cf.c[o + 1] * p : 0.f;
+    hr[k] = st[2 * k] * ip;
+    hi[k] = CPLX ? st[2 * k + 1] * ip : 0.f;
+  }
+  if (steps <= 0) return;
+  const int last = ((steps - 1) / kStepBlock) * kStepBlock;
+  for (int i0 = ASC ? 0 : last; ASC ? i0 <= last : i0 >= 0; i0 += ASC ? kStepBlock : -kStepBlock) {
+    float xs[kStepBlock];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
+    // walking back, the zeros staged past the last step come first: they must leave the state alone
+    const bool tail = !ASC && i0 == last;
+#pragma unroll
+    for (int jj = 0; jj < kStepBlock; ++jj) {
+      const int j = ASC ? jj : kStepBlock - 1 - jj;
+      float acc = 0.f;
+      if (BEFORE) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+      }
+      if (!tail || i0 + j < steps) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) state_step<CPLX>(qr[k], qi[k], hr[k], hi[k], xs[j]);
+      }
+      if (!BEFORE) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+      }
+      xs[j] = unit_sum(acc, tpr);
+    }
+    if (ns == 0) {
+#pragma unroll
+      for (int j = 0; j < kStepBlock; ++j) {
+        if (ASC) out[i0 + j] = xs[j];
+        else out[i0 + j] += xs[j];
+      }
+    }
+  }
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void bidir_apply_rows_kernel(const PassArgs A, const PassCoef rc,
+                                                                  const float* __restrict__ st_r, const int before) {
+  extern __shared__ float lds[];
+  UnitMap m = unit_map(A, lds + (size_t)(kBlock / A.TPR) * ((1 << rows_ts_log2(A.TPR, A.Tc)) + 1));
+  float* outs = lds;                      // [U][pitch] sums of both directions (every step that is read back
+  __syncthreads();                        // is first stored by the forward sweep); the samples follow it
+  const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
+  const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
+  const int c = t0 < 0 ? 0 : t0 / A.Tc;
+  stage_inputs<T>(A, m, 0);
+  __syncthreads();
+  const int steps = unit_steps(A, m, t0, 0);
+  const float* row = m.tile + u * m.pitch;
+  float* out = outs + u * m.pitch;
+  const size_t so = (((size_t)b * A.nchunks) * A.D + d) * A.NP + ns * kNPT;
+  const size_t cs = (size_t)A.D * A.NP;
+  bidir_sweep<CPLX, true, false>(A.coef, A.st + (so + (size_t)c * cs) * 2, d, A.NP, ns, A.TPR, row, out, steps);
+  const float* sr = st_r + (so + (size_t)(A.nchunks - 1 - c) * cs) * 2;
+  if (before) bidir_sweep<CPLX, false, true>(rc, sr, d, A.NP, ns, A.TPR, row, out, steps);
+  else bidir_sweep<CPLX, false, false>(rc, sr, d, A.NP, ns, A.TPR, row, out, steps);
+  __syncthreads();
+  const int per_thread = (m.U << m.tsl) / kBlock;
+  for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
+    float acc[kStageBatch], xr[kStageBatch], om[kStageBatch];
+    int64_t oy[kStageBatch];
+    bool on[kStageBatch];
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j) {
+      const int i = (e0 + j) * kBlock + threadIdx.x;
+      const int uu = i >> m.tsl, off = i & (m.ts - 1);
+      const bool mine = e0 + j < per_thread;
+      const int tt0 = mine ? m.ut0[uu] : -1;
+      on[j] = mine && off < unit_steps(A, m, tt0, 0);
+      const int t = tt0 + off;
+      const int dd = mine ? m.ud[uu] : 0;
+      acc[j] = mine ? outs[uu * m.pitch + off] : 0.f;
+      oy[j] = (mine ? m.uyo[uu] : 0) + t;
+      xr[j] = 0.f;
+      om[j] = 0.f;
+      if (on[j]) {
+        om[j] = A.omega[dd];
+        xr[j] = to_float(((const T*)A.x)[m.uxo[uu] + t]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j)
+      if (on[j]) ((T*)A.y)[oy[j]] = from_float<T>(acc[j] + om[j] * xr[j]);
   }
 }
 
@@ -617,7 +840,8 @@ Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_
   pl.nchunks = (int)ceil_div(L, tc);
   if (pl.nchunks < 1) pl.nchunks = 1;
   pl.coef_bytes = align_up((size_t)D * pl.NP * 5 * 4 * 4, 256);   // 4 sets
-  pl.st_bytes = align_up((size_t)B * pl.nchunks * D * pl.NP * 2 * 4, 256);
+  // chunk states; a two-sided layer may keep both directions' at once
+  pl.st_bytes = align_up((size_t)B * pl.nchunks * D * pl.NP * 2 * 4, 256) * (bidirectional ? 2 : 1);
   pl.acc_bytes = need_acc ? align_up((size_t)B * L * D * 4, 256) : 0;
   (void)nsets;
   pl.tile_bytes = align_up((size_t)B * D * 16 * 2 * 4, 256);      // state after the last whole tile
@@ -661,6 +885,44 @@ int run_pass_set_t(PassArgs& A, bool state_only, hipStream_t s) {
 template <typename T>
 int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
   return cplx ? run_pass_set_t<T, true>(A, state_only, s) : run_pass_set_t<T, false>(A, state_only, s);
+}
+
+// both directions of a two-sided layer in four launches (state, two scans, apply); see the kernels
+inline bool bidir_rows_ok(const PassArgs& A) {
+  return A.sxl == 1 && A.syl == 1 && A.L > 1 && A.Tc <= (1 << rows_ts_log2(A.TPR, A.Tc));
+}
+
+template <typename T, bool CPLX>
+int run_bidir_rows_t(PassArgs& A, const PassCoef& rc, float* st_r, int before, hipStream_t s) {
+  const int64_t tA = (int64_t)A.B * A.nchunks * A.D * A.TPR;
+  const dim3 gridA((unsigned)ceil_div(tA, kBlock));
+  hipLaunchKernelGGL((bidir_state_rows_kernel<T, CPLX>), gridA, dim3(kBlock), rows_lds_bytes(A.TPR, A.Tc), s, A, rc,
+                     st_r);
+  const int G = scan_groups(A.NP, A.nchunks);
+  const int rows_per_wg = kBlock / (A.NP * G);
+  const dim3 gridB((unsigned)ceil_div((int64_t)A.B * A.D, rows_per_wg));
+  PassArgs R = A;
+  R.coef = rc;
+  R.st = st_r;
+  R.h_in = nullptr;
+  R.h_out = nullptr;
+  hipLaunchKernelGGL((chunk_scan_kernel<CPLX>), gridB, dim3(kBlock), 0, s, A, G);
+  hipLaunchKernelGGL((chunk_scan_kernel<CPLX>), gridB, dim3(kBlock), 0, s, R, G);
+  hipLaunchKernelGGL((bidir_apply_rows_kernel<T, CPLX>), gridA, dim3(kBlock), bidir_lds_bytes(A.TPR, A.Tc), s, A, rc,
+                     (const float*)st_r, before);
+  MEGA_CHECK_LAUNCH("ema two-sided passes");
+  return MEGA_OK;
+}
+
+int run_bidir_rows(int dtype, PassArgs& A, const PassCoef& rc, float* st_r, int before, bool cplx, hipStream_t s) {
+#define MEGA_BIDIR(T) \
+  return cplx ? run_bidir_rows_t<T, true>(A, rc, st_r, before, s) : run_bidir_rows_t<T, false>(A, rc, st_r, before, s)
+  switch (dtype) {
+    case MEGA_F32: MEGA_BIDIR(float);
+    case MEGA_BF16: MEGA_BIDIR(bf16_t);
+    default: MEGA_BIDIR(f16_t);
+  }
+#undef MEGA_BIDIR
 }
 
 int run_pass_set_dtype(int dtype, PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
@@ -864,6 +1126,21 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     hipLaunchKernelGGL(coef_prep_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, p, q, gamma, 0,
                        is_complex ? 1 : 0, (int)D, (int)N, pl.NP, ndir, Lk, coef);
     MEGA_CHECK_LAUNCH("ema_fwd coefficient prep");
+  }
+  if (bidirectional && Lk == 0) {
+    PassArgs A;
+    A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
+    A.coef = coef_of(coef, 0, D, pl.NP);
+    A.h_in = nullptr; A.h_out = nullptr; A.st = st;
+    A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+    A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
+    A.reverse = 0; A.before = 0; A.tshift = 0;
+    A.acc_in = nullptr; A.acc_out = nullptr;
+    A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
+    A.omega = omega;
+    if (bidir_rows_ok(A))
+      return run_bidir_rows(dtype, A, coef_of(coef, 2, D, pl.NP), (float*)((char*)st + pl.st_bytes / 2), shift ? 1 : 0,
+                            is_complex != 0, s);
   }
   // list of pass sets; the last one writes y
   struct SetDesc { int set, reverse, before, tshift; };

@@ -78,13 +78,14 @@ def test_incremental_chunks_and_state(cplx):
 @pytest.mark.parametrize("shift", [True, False])
 @pytest.mark.parametrize("trunc", [None, 40])
 @pytest.mark.parametrize("cplx", [False, True])
-def test_bidirectional(shift, trunc, cplx):
+@pytest.mark.parametrize("L", [150, 256, 1000])
+def test_bidirectional(shift, trunc, cplx, L):
     rng = np.random.default_rng(14)
-    B, D, N, L = 2, 12, 16, 150
+    B, D, N = 2, 12, 16
     p, q, g = _coeffs(rng, 2 * D, N, cplx)
     om = rng.normal(size=D)
     x, x64 = rounded(rng.normal(size=(B, D, L)), torch.float32)
-    mask = np.zeros((B, L), bool); mask[1, 120:] = True
+    mask = np.zeros((B, L), bool); mask[1, L - 30:] = True
     y, _ = _run(x, p, q, g, om, padding_mask=dev(mask, torch.bool), bidirectional=True, truncation=trunc, shift=shift)
     yo, _ = O.ema_forward(x64, p, q, g, om, mask, bidirectional=True, truncation=trunc, shift=shift)
     assert rel_err(host(y), yo) < 1e-4
