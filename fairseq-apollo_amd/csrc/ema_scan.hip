@@ -137,8 +137,7 @@ __global__ __launch_bounds__(kBlock) void chunk_state_kernel(const PassArgs A) {
 constexpr int kScanBatch = 8;
 
 template <bool CPLX>
-__global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A, const int G) {
-  __shared__ float s_agg[kBlock * 2];
+__device__ __forceinline__ void chunk_scan_body(const PassArgs& A, const int G, float* s_agg) {
   const int n = threadIdx.x % A.NP;
   const int grp = (threadIdx.x / A.NP) % G;
   const int rloc = threadIdx.x / (A.NP * G);
@@ -238,6 +237,20 @@ __global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A, co
   }
 }
 
+template <bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_scan_kernel(const PassArgs A, const int G) {
+  __shared__ float s_agg[kBlock * 2];
+  chunk_scan_body<CPLX>(A, G, s_agg);
+}
+
+// the scans of the two directions of a two-sided layer in one launch (blockIdx.y picks the direction)
+template <bool CPLX>
+__global__ __launch_bounds__(kBlock) void chunk_scan2_kernel(const PassArgs A, const PassArgs R, const int G) {
+  __shared__ float s_agg[kBlock * 2];
+  if (blockIdx.y == 0) chunk_scan_body<CPLX>(A, G, s_agg);
+  else chunk_scan_body<CPLX>(R, G, s_agg);
+}
+
 template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void chunk_apply_kernel(const PassArgs A) {
   const int64_t gid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -327,10 +340,10 @@ struct UnitMap {
   int U, tsl, ts, pitch;
 };
 
-__device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds) {
+__device__ __forceinline__ UnitMap unit_map(const PassArgs& A, float* lds, int lanes, int tsl) {
   UnitMap m;
-  m.U = kBlock / A.TPR;
-  m.tsl = rows_ts_log2(A.TPR, A.Tc);
+  m.U = kBlock / lanes;
+  m.tsl = tsl;
   m.ts = 1 << m.tsl;
   m.pitch = m.ts + 1;
   m.tile = lds;
@@ -378,15 +391,16 @@ __device__ __forceinline__ int unit_steps(const PassArgs& A, const UnitMap& m, i
 
 // samples beyond a unit's steps are staged as zeros; a thread's elements go in batches whose loads
 // are all issued before the first of them is used
-constexpr int kStageBatch = 8;
+constexpr int kStageBatch = 8;       // elements per thread and batch of the store phases
+constexpr int kLoadBatch = 16;       // of the staging loads
 
 template <typename T>
 __device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m, int s0) {
   const int per_thread = (m.U << m.tsl) / kBlock;          // ts / TPR: 4 or a multiple of the batch
-  for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
-    float v[kStageBatch];
+  for (int e0 = 0; e0 < per_thread; e0 += kLoadBatch) {
+    float v[kLoadBatch];
 #pragma unroll
-    for (int j = 0; j < kStageBatch; ++j) {
+    for (int j = 0; j < kLoadBatch; ++j) {
       const int i = (e0 + j) * kBlock + threadIdx.x;
       const int u = i >> m.tsl, off = i & (m.ts - 1);
       const int t0 = e0 + j < per_thread ? m.ut0[u] : -1;
@@ -395,7 +409,7 @@ __device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m
         v[j] = load_row_u<T>(A, m.uxo[u], m.ub[u], t0 + s0 + off);
     }
 #pragma unroll
-    for (int j = 0; j < kStageBatch; ++j) {
+    for (int j = 0; j < kLoadBatch; ++j) {
       const int i = (e0 + j) * kBlock + threadIdx.x;
       if (e0 + j < per_thread) m.tile[(i >> m.tsl) * m.pitch + (i & (m.ts - 1))] = v[j];
     }
@@ -407,7 +421,7 @@ constexpr int kStepBlock = 8;      // steps whose samples are fetched from LDS t
 template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs A) {
   extern __shared__ float lds[];
-  const UnitMap m = unit_map(A, lds);
+  const UnitMap m = unit_map(A, lds, A.TPR, rows_ts_log2(A.TPR, A.Tc));
   __syncthreads();
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
   const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
@@ -461,7 +475,7 @@ __global__ __launch_bounds__(kBlock) void chunk_state_rows_kernel(const PassArgs
 template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void chunk_apply_rows_kernel(const PassArgs A) {
   extern __shared__ float lds[];
-  const UnitMap m = unit_map(A, lds);
+  const UnitMap m = unit_map(A, lds, A.TPR, rows_ts_log2(A.TPR, A.Tc));
   __syncthreads();
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
   const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
@@ -590,7 +604,7 @@ template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void bidir_state_rows_kernel(const PassArgs A, const PassCoef rc,
                                                                   float* __restrict__ st_r) {
   extern __shared__ float lds[];
-  const UnitMap m = unit_map(A, lds);
+  const UnitMap m = unit_map(A, lds, A.TPR, rows_ts_log2(A.TPR, A.Tc));
   __syncthreads();
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
   const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
@@ -719,7 +733,8 @@ template <typename T, bool CPLX>
 __global__ __launch_bounds__(kBlock) void bidir_apply_rows_kernel(const PassArgs A, const PassCoef rc,
                                                                   const float* __restrict__ st_r, const int before) {
   extern __shared__ float lds[];
-  UnitMap m = unit_map(A, lds + (size_t)(kBlock / A.TPR) * ((1 << rows_ts_log2(A.TPR, A.Tc)) + 1));
+  UnitMap m = unit_map(A, lds + (size_t)(kBlock / A.TPR) * ((1 << rows_ts_log2(A.TPR, A.Tc)) + 1), A.TPR,
+                       rows_ts_log2(A.TPR, A.Tc));
   float* outs = lds;                      // [U][pitch] sums of both directions (every step that is read back
   __syncthreads();                        // is first stored by the forward sweep); the samples follow it
   const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
@@ -887,7 +902,7 @@ int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
   return cplx ? run_pass_set_t<T, true>(A, state_only, s) : run_pass_set_t<T, false>(A, state_only, s);
 }
 
-// both directions of a two-sided layer in four launches (state, two scans, apply); see the kernels
+// both directions of a two-sided layer in three launches (state, scans, apply); see the kernels
 inline bool bidir_rows_ok(const PassArgs& A) {
   return A.sxl == 1 && A.syl == 1 && A.L > 1 && A.Tc <= (1 << rows_ts_log2(A.TPR, A.Tc));
 }
@@ -900,14 +915,13 @@ int run_bidir_rows_t(PassArgs& A, const PassCoef& rc, float* st_r, int before, h
                      st_r);
   const int G = scan_groups(A.NP, A.nchunks);
   const int rows_per_wg = kBlock / (A.NP * G);
-  const dim3 gridB((unsigned)ceil_div((int64_t)A.B * A.D, rows_per_wg));
+  const dim3 gridB((unsigned)ceil_div((int64_t)A.B * A.D, rows_per_wg), 2);
   PassArgs R = A;
   R.coef = rc;
   R.st = st_r;
   R.h_in = nullptr;
   R.h_out = nullptr;
-  hipLaunchKernelGGL((chunk_scan_kernel<CPLX>), gridB, dim3(kBlock), 0, s, A, G);
-  hipLaunchKernelGGL((chunk_scan_kernel<CPLX>), gridB, dim3(kBlock), 0, s, R, G);
+  hipLaunchKernelGGL((chunk_scan2_kernel<CPLX>), gridB, dim3(kBlock), 0, s, A, R, G);
   hipLaunchKernelGGL((bidir_apply_rows_kernel<T, CPLX>), gridA, dim3(kBlock), bidir_lds_bytes(A.TPR, A.Tc), s, A, rc,
                      (const float*)st_r, before);
   MEGA_CHECK_LAUNCH("ema two-sided passes");
