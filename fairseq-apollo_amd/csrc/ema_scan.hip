@@ -781,6 +781,145 @@ __global__ __launch_bounds__(kBlock) void bidir_apply_rows_kernel(const PassArgs
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// One-sided layers on time-contiguous rows short enough that all chunks of a row are units of one
+// workgroup (L <= 64 * U): the three passes in one kernel.  Chunk sums meet in LDS, every unit folds
+// the sums of the row's earlier chunks into its start state (all of them whole chunks), then runs the
+// recurrence over the samples that are still staged.  A.Tc is the sub-tile length and A.nchunks a
+// power of two that divides the units of a workgroup, so a workgroup holds whole rows.
+__host__ __device__ inline size_t fused_lds_bytes(int tpr, int tsl) {
+  const int U = kBlock / tpr;
+  return ((size_t)U * ((1 << tsl) + 1 + kUnitWords) + (size_t)kBlock * kNPT * 2) * 4;
+}
+
+template <typename T, bool CPLX>
+__global__ __launch_bounds__(kBlock) void ema_rows_fused_kernel(const PassArgs A, const int tsl) {
+  extern __shared__ float lds[];
+  const UnitMap m = unit_map(A, lds, A.TPR, tsl);
+  float* agg = (float*)(m.ut0 + m.U);                 // [kBlock][kNPT][2] chunk sums
+  __syncthreads();
+  const int u = threadIdx.x / A.TPR, ns = threadIdx.x % A.TPR;
+  const int t0 = m.ut0[u], d = m.ud[u], b = m.ub[u];
+  float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], pp[kNPT], hr[kNPT], hi[kNPT];
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
+    qr[k] = A.coef.q[o];
+    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
+    cr[k] = A.coef.c[o];
+    ci[k] = CPLX ? A.coef.c[o + 1] : 0.f;
+    pp[k] = A.coef.p[o / 2];
+    hr[k] = 0.f;
+    hi[k] = 0.f;
+  }
+  stage_inputs<T>(A, m, 0);
+  __syncthreads();
+  const int steps = unit_steps(A, m, t0, 0);
+  const int whole = steps / kStepBlock * kStepBlock;
+  float* row = m.tile + u * m.pitch;
+  // chunk sums from a zero start
+  for (int i0 = 0; i0 < steps; i0 += kStepBlock) {
+    float xs[kStepBlock];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j)
+      if (i0 < whole || i0 + j < steps) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) state_step<CPLX>(qr[k], qi[k], hr[k], hi[k], xs[j]);
+      }
+  }
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    agg[(threadIdx.x * kNPT + k) * 2] = hr[k];
+    agg[(threadIdx.x * kNPT + k) * 2 + 1] = hi[k];
+  }
+  __syncthreads();
+  // start state: the carried state pushed through the row's earlier chunks
+  const int cidx = u & (A.nchunks - 1);
+#pragma unroll
+  for (int k = 0; k < kNPT; ++k) {
+    const int n = ns * kNPT + k;
+    float sr = 0.f, si = 0.f;
+    if (A.h_in && n < A.N && t0 >= 0) {
+      const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
+      sr = A.h_in[oh];
+      si = CPLX ? A.h_in[oh + 1] : 0.f;
+    }
+    double Qr, Qi;
+    cpow_int((double)qr[k], (double)qi[k], A.Tc, &Qr, &Qi);
+    const float fQr = (float)Qr, fQi = (float)Qi;
+    for (int j = 0; j < cidx; ++j) {
+      const float* a = agg + ((size_t)(threadIdx.x - (cidx - j) * A.TPR) * kNPT + k) * 2;
+      const float nr = fQr * sr - fQi * si + pp[k] * a[0];
+      const float ni = fQr * si + fQi * sr + pp[k] * a[1];
+      sr = nr;
+      si = ni;
+    }
+    hr[k] = sr;
+    hi[k] = si;
+  }
+  // outputs; the state must be exact after the last step (it may be the carried state that is returned)
+  for (int i0 = 0; i0 < steps; i0 += kStepBlock) {
+    float xs[kStepBlock];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) xs[j] = row[i0 + j];
+#pragma unroll
+    for (int j = 0; j < kStepBlock; ++j) {
+      if (i0 < whole || i0 + j < steps) {
+#pragma unroll
+        for (int k = 0; k < kNPT; ++k) state_step<CPLX>(qr[k], qi[k], hr[k], hi[k], pp[k] * xs[j]);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int k = 0; k < kNPT; ++k) acc += CPLX ? (cr[k] * hr[k] - ci[k] * hi[k]) : cr[k] * hr[k];
+      xs[j] = unit_sum(acc, A.TPR);
+    }
+    if (ns == 0) {
+#pragma unroll
+      for (int j = 0; j < kStepBlock; ++j) row[i0 + j] = xs[j];
+    }
+  }
+  if (A.h_out && t0 >= 0 && t0 < A.L && t0 + A.Tc >= A.L) {
+#pragma unroll
+    for (int k = 0; k < kNPT; ++k) {
+      const int n = ns * kNPT + k;
+      if (n < A.N) {
+        const size_t oh = (((size_t)b * A.D + d) * A.N + n) * 2;
+        A.h_out[oh] = hr[k];
+        A.h_out[oh + 1] = hi[k];
+      }
+    }
+  }
+  __syncthreads();
+  const int per_thread = (m.U << m.tsl) / kBlock;
+  for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
+    float acc[kStageBatch], xr[kStageBatch], om[kStageBatch];
+    int64_t oy[kStageBatch];
+    bool on[kStageBatch];
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j) {
+      const int i = (e0 + j) * kBlock + threadIdx.x;
+      const int uu = i >> m.tsl, off = i & (m.ts - 1);
+      const bool mine = e0 + j < per_thread;
+      const int tt0 = mine ? m.ut0[uu] : -1;
+      on[j] = mine && off < unit_steps(A, m, tt0, 0);
+      const int t = tt0 + off;
+      acc[j] = mine ? m.tile[uu * m.pitch + off] : 0.f;
+      oy[j] = (mine ? m.uyo[uu] : 0) + t;
+      xr[j] = 0.f;
+      om[j] = 0.f;
+      if (on[j]) {
+        om[j] = A.omega[m.ud[uu]];
+        xr[j] = to_float(((const T*)A.x)[m.uxo[uu] + t]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kStageBatch; ++j)
+      if (on[j]) ((T*)A.y)[oy[j]] = from_float<T>(acc[j] + om[j] * xr[j]);
+  }
+}
+
 // builds the padded coefficient images of up to 4 pass sets:
 //   set 0: forward rows [0,D)            set 1: forward tail  (c = -gamma q^Lk)
 //   set 2: backward rows [D,2D)          set 3: backward tail
@@ -900,6 +1039,33 @@ int run_pass_set_t(PassArgs& A, bool state_only, hipStream_t s) {
 template <typename T>
 int run_pass_set(PassArgs& A, bool cplx, bool state_only, hipStream_t s) {
   return cplx ? run_pass_set_t<T, true>(A, state_only, s) : run_pass_set_t<T, false>(A, state_only, s);
+}
+
+// one-sided, untruncated layers on short time-contiguous rows: one kernel (see ema_rows_fused_kernel)
+inline bool fused_rows_plan(const PassArgs& A, int* tsl, int* nch) {
+  if (!(A.sxl == 1 && A.syl == 1 && A.L > 1)) return false;
+  const int U = kBlock / A.TPR;
+  int l2 = 5;
+  if ((int64_t)A.L > (int64_t)U << l2) l2 = A.TPR >= 2 ? 6 : 5;
+  if ((int64_t)A.L > (int64_t)U << l2) return false;
+  int n = 1;
+  while (((int64_t)n << l2) < A.L) n <<= 1;
+  *tsl = l2;
+  *nch = n;
+  return true;
+}
+
+template <typename T>
+int run_fused_rows(PassArgs& A, bool cplx, int tsl, int nch, hipStream_t s) {
+  A.Tc = 1 << tsl;
+  A.nchunks = nch;
+  const int U = kBlock / A.TPR;
+  const dim3 grid((unsigned)ceil_div((int64_t)A.B * A.D * nch, U));
+  const size_t lds = fused_lds_bytes(A.TPR, tsl);
+  if (cplx) hipLaunchKernelGGL((ema_rows_fused_kernel<T, true>), grid, dim3(kBlock), lds, s, A, tsl);
+  else hipLaunchKernelGGL((ema_rows_fused_kernel<T, false>), grid, dim3(kBlock), lds, s, A, tsl);
+  MEGA_CHECK_LAUNCH("ema fused row pass");
+  return MEGA_OK;
 }
 
 // both directions of a two-sided layer in three launches (state, scans, apply); see the kernels
@@ -1155,6 +1321,26 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     if (bidir_rows_ok(A))
       return run_bidir_rows(dtype, A, coef_of(coef, 2, D, pl.NP), (float*)((char*)st + pl.st_bytes / 2), shift ? 1 : 0,
                             is_complex != 0, s);
+  }
+  if (!bidirectional && Lk == 0) {
+    PassArgs A;
+    A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
+    A.coef = coef_of(coef, 0, D, pl.NP);
+    A.h_in = h_in; A.h_out = h_out; A.st = st;
+    A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+    A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
+    A.reverse = 0; A.before = 0; A.tshift = 0;
+    A.acc_in = nullptr; A.acc_out = nullptr;
+    A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
+    A.omega = omega;
+    int tsl = 0, nch = 0;
+    if (fused_rows_plan(A, &tsl, &nch)) {
+      switch (dtype) {
+        case MEGA_F32: return run_fused_rows<float>(A, is_complex != 0, tsl, nch, s);
+        case MEGA_BF16: return run_fused_rows<bf16_t>(A, is_complex != 0, tsl, nch, s);
+        default: return run_fused_rows<f16_t>(A, is_complex != 0, tsl, nch, s);
+      }
+    }
   }
   // list of pass sets; the last one writes y
   struct SetDesc { int set, reverse, before, tshift; };
