@@ -75,6 +75,34 @@ def test_incremental_chunks_and_state(cplx):
         assert rel_err(np.imag(hh), np.imag(ho)) < 1e-4
 
 
+@pytest.mark.parametrize("cplx", [False, True])
+@pytest.mark.parametrize("B,D,L", [(2, 24, 3000), (16, 256, 4100)])
+def test_long_rows_with_state_and_mask(cplx, B, D, L):
+    """fp32 [B, D, L] rows on the vector-ALU path: 3000 steps is the single-kernel form with 64-step
+    chunks; 16 x 256 rows of 4100 steps is the three-pass form with chunks of several sub-tiles (the
+    last one partial), one-sided with a carried state in and out, and two-sided with a mask."""
+    rng = np.random.default_rng(15)
+    N = 16
+    p, q, g = _coeffs(rng, 2 * D, N, cplx)
+    om = rng.normal(size=D)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), torch.float32)
+    # the carried state goes in only at the small shape (its bias term is a [B, D, N, L] array in the oracle)
+    h0 = None
+    if B * D < 100:
+        h0 = (rng.normal(size=(B, D, N)) + (1j * rng.normal(size=(B, D, N)) if cplx else 0)).astype(np.complex64)
+    mask = np.zeros((B, L), bool); mask[0, L - 77:] = True; mask[B - 1, 5] = True
+    y, h = _run(x, p[:D], q[:D], g[:D], om, padding_mask=dev(mask, torch.bool), h=None if h0 is None else dev(h0),
+                want_state=True)
+    yo, ho = O.ema_forward(x64, p[:D], q[:D], g[:D], om, mask, h=h0, incremental=True)
+    assert rel_err(host(y), yo) < 1e-4
+    assert rel_err(np.real(host(h)), np.real(ho)) < 1e-4
+    if cplx:
+        assert rel_err(np.imag(host(h)), np.imag(ho)) < 1e-4
+    y2, _ = _run(x, p, q, g, om, padding_mask=dev(mask, torch.bool), bidirectional=True, shift=False)
+    yo2, _ = O.ema_forward(x64, p, q, g, om, mask, bidirectional=True, shift=False)
+    assert rel_err(host(y2), yo2) < 1e-4
+
+
 @pytest.mark.parametrize("shift", [True, False])
 @pytest.mark.parametrize("trunc", [None, 40])
 @pytest.mark.parametrize("cplx", [False, True])
