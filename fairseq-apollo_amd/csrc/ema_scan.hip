@@ -389,6 +389,45 @@ __device__ __forceinline__ int unit_steps(const PassArgs& A, const UnitMap& m, i
   return n < 0 ? 0 : (n > m.ts ? m.ts : n);
 }
 
+// values that are the same in every lane of a wave, moved to scalar registers
+__device__ __forceinline__ int uniform_i32(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+constexpr int kWaves = kBlock / 64;
+constexpr int kUnitBatch = 8;        // units per wave whose loads are in flight together (U / kWaves is a multiple)
+
+// y = sums + omega x for 64-step sub-tiles: the store phase of the single-sub-tile kernels, one unit
+// per wave and pass (wave-uniform unit entries as in stage_inputs)
+template <typename T>
+__device__ __forceinline__ void store_outputs64(const PassArgs& A, const UnitMap& m, const float* sums) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int ub = 0; ub < m.U / kWaves; ub += kUnitBatch) {
+    float acc[kUnitBatch], xr[kUnitBatch], om[kUnitBatch];
+#pragma unroll
+    for (int j = 0; j < kUnitBatch; ++j) {
+      const int u = (ub + j) * kWaves + wave;
+      const int t0 = uniform_i32(m.ut0[u]);
+      acc[j] = sums[u * m.pitch + lane];
+      xr[j] = 0.f;
+      om[j] = 0.f;
+      if (lane < unit_steps(A, m, t0, 0)) {
+        om[j] = A.omega[uniform_i32(m.ud[u])];
+        xr[j] = to_float(((const T*)A.x)[uniform_i64(m.uxo[u]) + t0 + lane]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kUnitBatch; ++j) {
+      const int u = (ub + j) * kWaves + wave;
+      const int t0 = uniform_i32(m.ut0[u]);
+      if (lane < unit_steps(A, m, t0, 0))
+        ((T*)A.y)[uniform_i64(m.uyo[u]) + t0 + lane] = from_float<T>(acc[j] + om[j] * xr[j]);
+    }
+  }
+}
+
 // samples beyond a unit's steps are staged as zeros; a thread's elements go in batches whose loads
 // are all issued before the first of them is used
 constexpr int kStageBatch = 8;       // elements per thread and batch of the store phases
@@ -396,6 +435,25 @@ constexpr int kLoadBatch = 16;       // of the staging loads
 
 template <typename T>
 __device__ __forceinline__ void stage_inputs(const PassArgs& A, const UnitMap& m, int s0) {
+  if (m.tsl == 6) {
+    // a wave covers one unit per pass: the unit's entries of the map are wave-uniform (scalar
+    // registers), a lane only adds its own step to the addresses
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int ub = 0; ub < m.U / kWaves; ub += kUnitBatch) {
+      float v[kUnitBatch];
+#pragma unroll
+      for (int j = 0; j < kUnitBatch; ++j) {
+        const int u = (ub + j) * kWaves + wave;
+        const int t0 = uniform_i32(m.ut0[u]);
+        v[j] = 0.f;
+        if (lane < unit_steps(A, m, t0, s0))
+          v[j] = load_row_u<T>(A, uniform_i64(m.uxo[u]), uniform_i32(m.ub[u]), t0 + s0 + lane);
+      }
+#pragma unroll
+      for (int j = 0; j < kUnitBatch; ++j) m.tile[((ub + j) * kWaves + wave) * m.pitch + lane] = v[j];
+    }
+    return;
+  }
   const int per_thread = (m.U << m.tsl) / kBlock;          // ts / TPR: 4 or a multiple of the batch
   for (int e0 = 0; e0 < per_thread; e0 += kLoadBatch) {
     float v[kLoadBatch];
@@ -752,6 +810,10 @@ __global__ __launch_bounds__(kBlock) void bidir_apply_rows_kernel(const PassArgs
   if (before) bidir_sweep<CPLX, false, true>(rc, sr, d, A.NP, ns, A.TPR, row, out, steps);
   else bidir_sweep<CPLX, false, false>(rc, sr, d, A.NP, ns, A.TPR, row, out, steps);
   __syncthreads();
+  if (m.tsl == 6) {
+    store_outputs64<T>(A, m, outs);
+    return;
+  }
   const int per_thread = (m.U << m.tsl) / kBlock;
   for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
     float acc[kStageBatch], xr[kStageBatch], om[kStageBatch];
@@ -892,6 +954,10 @@ __global__ __launch_bounds__(kBlock) void ema_rows_fused_kernel(const PassArgs A
     }
   }
   __syncthreads();
+  if (m.tsl == 6) {
+    store_outputs64<T>(A, m, m.tile);
+    return;
+  }
   const int per_thread = (m.U << m.tsl) / kBlock;
   for (int e0 = 0; e0 < per_thread; e0 += kStageBatch) {
     float acc[kStageBatch], xr[kStageBatch], om[kStageBatch];
