@@ -439,6 +439,8 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
+    ap.add_argument("--standalone", action="store_true",
+                    help="block workload: also time each operator alone, back to back on cold inputs")
     ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
@@ -506,8 +508,29 @@ def main():
         gpu_ms = e0.elapsed_time(e1)
         ms_per_step = max(wall * 1e3, gpu_ms) / args.steps
 
-        # per-operator device time: HIP events on the launch stream around a run of back-to-back
-        # calls (the queue never drains, so the quotient is the kernel's launch-to-launch period)
+        # per-kernel device time inside the block: the same steps again with an event between the two
+        # calls (the EMA finds its input where the norm has just left it, as in the timed region)
+        reps = max(20, min(args.steps, 200))
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
+        h0 = time.perf_counter()
+        for i in range(reps):
+            a, b, c = evs[i]
+            a.record()
+            xn = norm(xs[i % NBUF])
+            b.record()
+            ema(xn.transpose(1, 2))
+            c.record()
+        host_step = (time.perf_counter() - h0) * 1e3 / reps
+        torch.cuda.synchronize()
+        norm_ev = sum(a.elapsed_time(b) for a, b, _ in evs) / reps
+        ema_ev = sum(b.elapsed_time(c) for _, b, c in evs) / reps
+        # the event packets between the kernels cost about a microsecond each: a kernel's time is its
+        # share of the step measured above, split in the proportion of the event intervals
+        # (launch gaps included, so slightly above the kernel trace of the same run)
+        norm_avg = ms_per_step * norm_ev / (norm_ev + ema_ev)
+        ema_avg = ms_per_step * ema_ev / (norm_ev + ema_ev)
+
+        # optionally each operator alone, back to back on inputs that are cold in every cache
         def timed(fn, reps):
             args_ = [fn.prep(i) for i in range(reps)]
             for i in range(min(reps, 8)):
@@ -532,8 +555,6 @@ def main():
             def __call__(self, x):
                 return norm(x)
 
-        xns = [norm(x) for x in xs]
-
         class EmaCall:
             @staticmethod
             def prep(i):
@@ -542,9 +563,13 @@ def main():
             def __call__(self, x):
                 return ema(x)
 
-        reps = max(20, min(args.steps, 200))
-        norm_avg, norm_host = timed(NormCall(), reps)
-        ema_avg, ema_host = timed(EmaCall(), reps)
+        standalone = None
+        if args.standalone:
+            xns = [norm(x) for x in xs]
+            n_avg, n_host = timed(NormCall(), reps)
+            e_avg, e_host = timed(EmaCall(), reps)
+            standalone = {"group_tsn_kernel": {"avg_ms": n_avg, "host_enqueue_ms": n_host},
+                          "ema_mfma_kernel": {"avg_ms": e_avg, "host_enqueue_ms": e_host}}
         if args.copy_calibration:
             dst = torch.empty_like(xs[0])
             for i in range(args.copy_calibration):
@@ -582,16 +607,18 @@ def main():
             "ema_mfma_kernel": {"bound": "hbm", "kernel": "ema_mfma_kernel (the EMA call)", "achieved": ema_gbs,
                                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS,
                                 "traffic": traffic.get("ema_mfma_kernel"),
-                                "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg,
-                                "host_enqueue_ms": ema_host},
+                                "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg},
             "group_tsn_kernel": {"bound": "hbm", "kernel": "group_tsn_kernel (the TimestepNorm call)",
                                  "achieved": norm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": norm_gbs / HBM_PEAK_GBS, "traffic": traffic.get("group_tsn_kernel"),
-                                 "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg,
-                                 "host_enqueue_ms": norm_host},
+                                 "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg},
         },
+        "host_enqueue_ms_per_step": host_step,
+        "event_intervals_ms": {"group_tsn_kernel": norm_ev, "ema_mfma_kernel": ema_ev},
         "timestep_norm_status": status,
     }
+    if standalone is not None:
+        out["standalone_cold"] = standalone
     # the dominant kernel = the one with the longer launch (both are HBM-bound)
     out["roofline"] = max(out["kernels"].values(), key=lambda k: k["avg_ms"])
     if not args.no_cpu:
