@@ -107,16 +107,17 @@ def test_long_rows_with_state_and_mask(cplx, B, D, L):
 @pytest.mark.parametrize("trunc", [None, 40])
 @pytest.mark.parametrize("cplx", [False, True])
 @pytest.mark.parametrize("L", [150, 256, 1000])
-def test_bidirectional(shift, trunc, cplx, L):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_bidirectional(shift, trunc, cplx, L, dtype):
     rng = np.random.default_rng(14)
     B, D, N = 2, 12, 16
     p, q, g = _coeffs(rng, 2 * D, N, cplx)
     om = rng.normal(size=D)
-    x, x64 = rounded(rng.normal(size=(B, D, L)), torch.float32)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
     mask = np.zeros((B, L), bool); mask[1, L - 30:] = True
     y, _ = _run(x, p, q, g, om, padding_mask=dev(mask, torch.bool), bidirectional=True, truncation=trunc, shift=shift)
     yo, _ = O.ema_forward(x64, p, q, g, om, mask, bidirectional=True, truncation=trunc, shift=shift)
-    assert rel_err(host(y), yo) < 1e-4
+    assert rel_err(host(y), yo) < TOL[dtype]
 
 
 def test_modules_forward():
