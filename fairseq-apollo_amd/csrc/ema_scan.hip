@@ -21,7 +21,11 @@
 // Thread mapping: TPR = ceil(N/4) lanes share one (batch, channel) row, 4 complex
 // states each; rows are laid out channel-fastest so that [B,L,D] activations are read
 // coalesced.  Activations with a contiguous time axis ([B,D,L]) take the *_rows kernels,
-// which stage sub-tiles of time through LDS.
+// which stage sub-tiles of time through LDS.  On such rows, a one-sided untruncated layer
+// whose rows fit one workgroup's units runs the three passes in one kernel
+// (ema_rows_fused_kernel), and a two-sided untruncated layer whose chunks fit one sub-tile
+// runs both directions from the same staged samples (bidir_*_rows_kernel, one launch for
+// both chunk scans) instead of one pass set per direction.
 #include "common.h"
 #include "ema_mfma.h"
 
