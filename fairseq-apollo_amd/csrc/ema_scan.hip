@@ -858,8 +858,13 @@ __host__ __device__ inline size_t fused_lds_bytes(int tpr, int tsl) {
   return ((size_t)U * ((1 << tsl) + 1 + kUnitWords) + (size_t)kBlock * kNPT * 2) * 4;
 }
 
+// The coefficients come straight from the caller's arrays (p [D, N], q and gamma [D, N, 2]); states
+// beyond N are zero.
 template <typename T, bool CPLX>
-__global__ __launch_bounds__(kBlock) void ema_rows_fused_kernel(const PassArgs A, const int tsl) {
+__global__ __launch_bounds__(kBlock) void ema_rows_fused_kernel(const PassArgs A, const int tsl,
+                                                                const float* __restrict__ p_raw,
+                                                                const float* __restrict__ q_raw,
+                                                                const float* __restrict__ g_raw) {
   extern __shared__ float lds[];
   const UnitMap m = unit_map(A, lds, A.TPR, tsl);
   float* agg = (float*)(m.ut0 + m.U);                 // [kBlock][kNPT][2] chunk sums
@@ -869,12 +874,14 @@ __global__ __launch_bounds__(kBlock) void ema_rows_fused_kernel(const PassArgs A
   float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], pp[kNPT], hr[kNPT], hi[kNPT];
 #pragma unroll
   for (int k = 0; k < kNPT; ++k) {
-    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
-    qr[k] = A.coef.q[o];
-    qi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
-    cr[k] = A.coef.c[o];
-    ci[k] = CPLX ? A.coef.c[o + 1] : 0.f;
-    pp[k] = A.coef.p[o / 2];
+    const int n = ns * kNPT + k;
+    const bool real_state = n < A.N;
+    const size_t o = ((size_t)d * A.N + (real_state ? n : 0)) * 2;
+    qr[k] = real_state ? q_raw[o] : 0.f;
+    qi[k] = CPLX && real_state ? q_raw[o + 1] : 0.f;
+    cr[k] = real_state ? g_raw[o] : 0.f;
+    ci[k] = CPLX && real_state ? g_raw[o + 1] : 0.f;
+    pp[k] = real_state ? p_raw[o / 2] : 0.f;
     hr[k] = 0.f;
     hi[k] = 0.f;
   }
@@ -1126,14 +1133,15 @@ inline bool fused_rows_plan(const PassArgs& A, int* tsl, int* nch) {
 }
 
 template <typename T>
-int run_fused_rows(PassArgs& A, bool cplx, int tsl, int nch, hipStream_t s) {
+int run_fused_rows(PassArgs& A, bool cplx, int tsl, int nch, const float* p, const float* q, const float* gamma,
+                   hipStream_t s) {
   A.Tc = 1 << tsl;
   A.nchunks = nch;
   const int U = kBlock / A.TPR;
   const dim3 grid((unsigned)ceil_div((int64_t)A.B * A.D * nch, U));
   const size_t lds = fused_lds_bytes(A.TPR, tsl);
-  if (cplx) hipLaunchKernelGGL((ema_rows_fused_kernel<T, true>), grid, dim3(kBlock), lds, s, A, tsl);
-  else hipLaunchKernelGGL((ema_rows_fused_kernel<T, false>), grid, dim3(kBlock), lds, s, A, tsl);
+  if (cplx) hipLaunchKernelGGL((ema_rows_fused_kernel<T, true>), grid, dim3(kBlock), lds, s, A, tsl, p, q, gamma);
+  else hipLaunchKernelGGL((ema_rows_fused_kernel<T, false>), grid, dim3(kBlock), lds, s, A, tsl, p, q, gamma);
   MEGA_CHECK_LAUNCH("ema fused row pass");
   return MEGA_OK;
 }
@@ -1370,6 +1378,26 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
                       D, N, L, bidirectional, Lk, acc, h_tile, s);
     if (rc != 0) return rc < 0 ? rc : MEGA_OK;
   }
+  if (!bidirectional && Lk == 0) {
+    PassArgs A;
+    A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
+    A.coef = coef_of(coef, 0, D, pl.NP);
+    A.h_in = h_in; A.h_out = h_out; A.st = st;
+    A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+    A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
+    A.reverse = 0; A.before = 0; A.tshift = 0;
+    A.acc_in = nullptr; A.acc_out = nullptr;
+    A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
+    A.omega = omega;
+    int tsl = 0, nch = 0;
+    if (fused_rows_plan(A, &tsl, &nch)) {
+      switch (dtype) {
+        case MEGA_F32: return run_fused_rows<float>(A, is_complex != 0, tsl, nch, p, q, gamma, s);
+        case MEGA_BF16: return run_fused_rows<bf16_t>(A, is_complex != 0, tsl, nch, p, q, gamma, s);
+        default: return run_fused_rows<f16_t>(A, is_complex != 0, tsl, nch, p, q, gamma, s);
+      }
+    }
+  }
   const int ndir = bidirectional ? 2 : 1;
   {
     const int64_t n = (int64_t)D * pl.NP * ndir;
@@ -1391,26 +1419,6 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     if (bidir_rows_ok(A))
       return run_bidir_rows(dtype, A, coef_of(coef, 2, D, pl.NP), (float*)((char*)st + pl.st_bytes / 2), shift ? 1 : 0,
                             is_complex != 0, s);
-  }
-  if (!bidirectional && Lk == 0) {
-    PassArgs A;
-    A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
-    A.coef = coef_of(coef, 0, D, pl.NP);
-    A.h_in = h_in; A.h_out = h_out; A.st = st;
-    A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
-    A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
-    A.reverse = 0; A.before = 0; A.tshift = 0;
-    A.acc_in = nullptr; A.acc_out = nullptr;
-    A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
-    A.omega = omega;
-    int tsl = 0, nch = 0;
-    if (fused_rows_plan(A, &tsl, &nch)) {
-      switch (dtype) {
-        case MEGA_F32: return run_fused_rows<float>(A, is_complex != 0, tsl, nch, s);
-        case MEGA_BF16: return run_fused_rows<bf16_t>(A, is_complex != 0, tsl, nch, s);
-        default: return run_fused_rows<f16_t>(A, is_complex != 0, tsl, nch, s);
-      }
-    }
   }
   // list of pass sets; the last one writes y
   struct SetDesc { int set, reverse, before, tshift; };
