@@ -38,10 +38,17 @@ constexpr int kBlock = 256;
 
 // coefficient image of one pass set, padded to NP = TPR*4 states per row (zeros beyond N)
 struct PassCoef {
-  const float* q;   // [Drows, NP, 2]
-  const float* c;   // [Drows, NP, 2]  output coefficient (gamma, or -gamma q^Lk)
-  const float* p;   // [Drows, NP]     input coefficient
+  const float* q;   // [Drows, np, 2]
+  const float* c;   // [Drows, np, 2]  output coefficient (gamma, or -gamma q^Lk)
+  const float* p;   // [Drows, np]     input coefficient
+  int np;           // states per row in memory: NP for the padded images, N for the caller's own arrays
 };
+
+// element offset of state n of row d, or -1 for a padded state that the arrays do not hold (all of its
+// coefficients are zero); the kernels of the two-sided row passes and the chunk scan read through it
+__device__ __forceinline__ int64_t coef_at(const PassCoef& cf, int d, int n) {
+  return n < cf.np ? (int64_t)d * cf.np + n : -1;
+}
 
 struct PassArgs {
   const void* x;
@@ -150,9 +157,9 @@ __device__ __forceinline__ void chunk_scan_body(const PassArgs& A, const int G, 
   const bool live = row < (int64_t)A.B * A.D;
   const int d = live ? (int)(row % A.D) : 0;
   const int b = live ? (int)(row / A.D) : 0;
-  const size_t oc = ((size_t)d * A.NP + n) * 2;
-  const double qr = A.coef.q[oc], qi = CPLX ? A.coef.q[oc + 1] : 0.0;
-  const float p = A.coef.p[(size_t)d * A.NP + n];
+  const int64_t oc = coef_at(A.coef, d, n);
+  const double qr = oc >= 0 ? A.coef.q[oc * 2] : 0.0, qi = CPLX && oc >= 0 ? A.coef.q[oc * 2 + 1] : 0.0;
+  const float p = oc >= 0 ? A.coef.p[oc] : 0.f;
   double Qr, Qi;
   cpow_int(qr, qi, A.Tc, &Qr, &Qi);
   const float fQr = (float)Qr, fQi = (float)Qi;
@@ -673,11 +680,11 @@ __global__ __launch_bounds__(kBlock) void bidir_state_rows_kernel(const PassArgs
   float fr[kNPT], fi[kNPT], br[kNPT], bi[kNPT], hr[kNPT], hi[kNPT], gr[kNPT], gi[kNPT];
 #pragma unroll
   for (int k = 0; k < kNPT; ++k) {
-    const size_t o = ((size_t)d * A.NP + ns * kNPT + k) * 2;
-    fr[k] = A.coef.q[o];
-    fi[k] = CPLX ? A.coef.q[o + 1] : 0.f;
-    br[k] = rc.q[o];
-    bi[k] = CPLX ? rc.q[o + 1] : 0.f;
+    const int64_t o = coef_at(A.coef, d, ns * kNPT + k);
+    fr[k] = o >= 0 ? A.coef.q[o * 2] : 0.f;
+    fi[k] = CPLX && o >= 0 ? A.coef.q[o * 2 + 1] : 0.f;
+    br[k] = o >= 0 ? rc.q[o * 2] : 0.f;
+    bi[k] = CPLX && o >= 0 ? rc.q[o * 2 + 1] : 0.f;
     hr[k] = hi[k] = gr[k] = gi[k] = 0.f;
   }
   stage_inputs<T>(A, m, 0);
@@ -745,13 +752,13 @@ __device__ __forceinline__ void bidir_sweep(const PassCoef& cf, const float* st,
   float qr[kNPT], qi[kNPT], cr[kNPT], ci[kNPT], hr[kNPT], hi[kNPT];
 #pragma unroll
   for (int k = 0; k < kNPT; ++k) {
-    const size_t o = ((size_t)d * NP + ns * kNPT + k) * 2;
-    qr[k] = cf.q[o];
-    qi[k] = CPLX ? cf.q[o + 1] : 0.f;
-    const float p = cf.p[o / 2];
+    const int64_t o = coef_at(cf, d, ns * kNPT + k);
+    qr[k] = o >= 0 ? cf.q[o * 2] : 0.f;
+    qi[k] = CPLX && o >= 0 ? cf.q[o * 2 + 1] : 0.f;
+    const float p = o >= 0 ? cf.p[o] : 0.f;
     const float ip = p != 0.f ? 1.0f / p : 0.f;
-    cr[k] = cf.c[o] * p;
-    ci[k] = CPLX ? cf.c[o + 1] * p : 0.f;
+    cr[k] = o >= 0 ? cf.c[o * 2] * p : 0.f;
+    ci[k] = CPLX && o >= 0 ? cf.c[o * 2 + 1] * p : 0.f;
     hr[k] = st[2 * k] * ip;
     hi[k] = CPLX ? st[2 * k + 1] * ip : 0.f;
   }
@@ -1194,7 +1201,7 @@ int run_pass_set_dtype(int dtype, PassArgs& A, bool cplx, bool state_only, hipSt
 PassCoef coef_of(float* base, int set, int64_t D, int NP) {
   const size_t per = (size_t)D * NP;
   float* o = base + (size_t)set * per * 5;
-  return PassCoef{o, o + per * 2, o + per * 4};
+  return PassCoef{o, o + per * 2, o + per * 4, NP};
 }
 
 // ---------------------------------------------------------------- single decode step
@@ -1398,17 +1405,11 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
       }
     }
   }
-  const int ndir = bidirectional ? 2 : 1;
-  {
-    const int64_t n = (int64_t)D * pl.NP * ndir;
-    hipLaunchKernelGGL(coef_prep_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, p, q, gamma, 0,
-                       is_complex ? 1 : 0, (int)D, (int)N, pl.NP, ndir, Lk, coef);
-    MEGA_CHECK_LAUNCH("ema_fwd coefficient prep");
-  }
   if (bidirectional && Lk == 0) {
     PassArgs A;
     A.x = x; A.sxb = sxb; A.sxd = sxd; A.sxl = sxl; A.mask = mask;
-    A.coef = coef_of(coef, 0, D, pl.NP);
+    // both directions read the caller's arrays: rows [0, D) run forward, rows [D, 2D) back in time
+    A.coef = PassCoef{q, gamma, p, (int)N};
     A.h_in = nullptr; A.h_out = nullptr; A.st = st;
     A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
     A.NP = pl.NP; A.TPR = pl.TPR; A.Tc = pl.Tc; A.nchunks = pl.nchunks;
@@ -1417,8 +1418,16 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     A.y = y; A.syb = syb; A.syd = syd; A.syl = syl;
     A.omega = omega;
     if (bidir_rows_ok(A))
-      return run_bidir_rows(dtype, A, coef_of(coef, 2, D, pl.NP), (float*)((char*)st + pl.st_bytes / 2), shift ? 1 : 0,
+      return run_bidir_rows(dtype, A, PassCoef{q + D * N * 2, gamma + D * N * 2, p + D * N, (int)N},
+                            (float*)((char*)st + pl.st_bytes / 2), shift ? 1 : 0,
                             is_complex != 0, s);
+  }
+  const int ndir = bidirectional ? 2 : 1;
+  {
+    const int64_t n = (int64_t)D * pl.NP * ndir;
+    hipLaunchKernelGGL(coef_prep_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, s, p, q, gamma, 0,
+                       is_complex ? 1 : 0, (int)D, (int)N, pl.NP, ndir, Lk, coef);
+    MEGA_CHECK_LAUNCH("ema_fwd coefficient prep");
   }
   // list of pass sets; the last one writes y
   struct SetDesc { int set, reverse, before, tshift; };
