@@ -36,6 +36,11 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // node so that a caller may record any entry point into a HIP graph.
 void zero_async(void* p, size_t bytes, hipStream_t s);
 static inline size_t align_up(size_t a, size_t b) { return (a + b - 1) / b * b; }
+// do the byte ranges [a, a + na) and [b, b + nb) share a byte?
+static inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
+  const uintptr_t ua = (uintptr_t)a, ub = (uintptr_t)b;
+  return ua < ub + nb && ub < ua + na;
+}
 
 // ---------------------------------------------------------------- row tiling of [tokens, H] tiles
 // How the channel vectors of one token are spread over threads in the kernels that walk

@@ -205,6 +205,12 @@ extern "C" int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, c
   MEGA_REQUIRE(x && xn && y && prev_count && prev_mean && prev_var && count && mean && var && norm_gamma && norm_beta &&
                    p && q && gamma && omega && h_out,
                MEGA_ERR_ARG, "norm_ema_step: null pointer argument");
+  // Every workgroup (stream, group) of a launch reads prev_count[stream] and the workgroup of group 0 writes
+  // count[stream]: with the two in one buffer a late workgroup could read the count of the step being
+  // written.  mean / var words and the state h have one owning workgroup each, so those may be updated in place.
+  MEGA_REQUIRE(!ranges_overlap(prev_count, (size_t)B * 8, count, (size_t)B * 8), MEGA_ERR_ARG,
+               "norm_ema_step: count must not overlap prev_count (every group of a stream reads prev_count "
+               "while one of them writes count); alternate between two count buffers");
   StepArgs A;
   A.x = x; A.xn = xn; A.y = y; A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var;
   A.count = count; A.mean = mean; A.var = var; A.nw = norm_gamma; A.nb = norm_beta; A.p = p; A.q = q; A.g = gamma;

@@ -631,6 +631,13 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
   if (B == 0) return MEGA_OK;
   MEGA_REQUIRE(prev_count && prev_mean && prev_var && gamma && beta && count && mean && var, MEGA_ERR_ARG,
                "group_timestep_norm_fwd: null state / parameter pointer");
+  // every tile of a row reads the prior state while the row's last tile writes the new one
+  MEGA_REQUIRE(!ranges_overlap(prev_count, (size_t)B * 8, count, (size_t)B * 8) &&
+                   !ranges_overlap(prev_mean, (size_t)B * G * 4, mean, (size_t)B * G * 4) &&
+                   !ranges_overlap(prev_var, (size_t)B * G * 4, var, (size_t)B * G * 4),
+               MEGA_ERR_ARG,
+               "group_timestep_norm_fwd: count / mean / var must not overlap prev_count / prev_mean / prev_var "
+               "(the state is not updated in place)");
   hipStream_t s = (hipStream_t)stream;
   if (L == 0) {
     hipMemcpyAsync(count, prev_count, (size_t)B * 8, hipMemcpyDeviceToDevice, s);
@@ -678,6 +685,9 @@ extern "C" int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const i
   if (B == 0) return MEGA_OK;
   MEGA_REQUIRE(prev_count && prev_mean && prev_var && gamma && beta && count && mean && var, MEGA_ERR_ARG,
                "timestep_norm_fwd: null state / parameter pointer");
+  // every block of features of a row reads prev_count while the first one writes count
+  MEGA_REQUIRE(!ranges_overlap(prev_count, (size_t)B * 8, count, (size_t)B * 8), MEGA_ERR_ARG,
+               "timestep_norm_fwd: count must not overlap prev_count");
   MEGA_REQUIRE(L == 0 || (x && y), MEGA_ERR_ARG, "timestep_norm_fwd: null x / y");
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)ceil_div(H, kThreads), (unsigned)B);

@@ -705,7 +705,10 @@ class DecodeStep:
         self.q = _cplx_as_f32(q.reshape(self.D, self.N))
         self.gamma = _cplx_as_f32(gamma.reshape(self.D, self.N))
         self.omega = _f32c(omega).reshape(self.D)
+        # two count buffers used in turn: every (stream, group) workgroup of a launch reads the old
+        # count while one workgroup per stream writes the new one, so the two must not share memory
         self.count = torch.full((self.B,), prior_count, dtype=torch.int64, device=self.dev)
+        self._count_next = torch.empty_like(self.count)
         self.mean = torch.zeros(self.B, self.G, dtype=torch.float32, device=self.dev)
         self.var = torch.ones(self.B, self.G, dtype=torch.float32, device=self.dev)
         self.h = torch.zeros(self.B, self.D, self.N, 2, dtype=torch.float32, device=self.dev)
@@ -718,11 +721,12 @@ class DecodeStep:
         y = torch.empty_like(xd)
         with _on_device(self.dev):
             rc = lib.mega_norm_ema_step(_ptr(xd), _ptr(xn), _ptr(y), _dtype_code(xd), _ptr(self.count), _ptr(self.mean),
-                                        _ptr(self.var), _ptr(self.count), _ptr(self.mean), _ptr(self.var), _ptr(self.nw),
+                                        _ptr(self.var), _ptr(self._count_next), _ptr(self.mean), _ptr(self.var), _ptr(self.nw),
                                         _ptr(self.nb), self.eps, _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
                                         1 if self.is_complex else 0, _ptr(self.omega), _ptr(self.h), _ptr(self.h),
                                         self.B, self.D, self.G, self.N, _stream(self.dev))
         _lib.check(rc, "norm_ema_step")
+        self.count, self._count_next = self._count_next, self.count
         return xn, y
 
     @property

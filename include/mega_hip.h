@@ -142,9 +142,13 @@ int mega_ema_step(const void* x, void* y, int dtype, const float* p, const float
  * normalised token (BaseMovingLayer.forward with L = 1 and incremental state,
  * fairseq/modules/base_moving_average.py:144-160).  The reference runs these as two modules
  * and >= 6 kernels per step.
- *   x, xn, y [B,D] of `dtype`; norm state in (prev_*) and out (count, mean, var; may alias
- *   the inputs); norm_gamma (= weight + 1), norm_beta [D]; EMA coefficients as mega_ema_step;
- *   h_in may be NULL (zero state) and h_out may alias h_in.                              */
+ *   x, xn, y [B,D] of `dtype`; norm state in (prev_*) and out (count, mean, var);
+ *   norm_gamma (= weight + 1), norm_beta [D]; EMA coefficients as mega_ema_step;
+ *   h_in may be NULL (zero state).
+ *   In-place update: mean / var may be the prev_mean / prev_var buffers and h_out may be h_in
+ *   (one workgroup owns each of those words: it reads, then writes).  count must NOT overlap
+ *   prev_count (MEGA_ERR_ARG): all G workgroups of a stream read prev_count[b] while one of
+ *   them writes count[b]; a streaming caller alternates between two count buffers.         */
 int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_t* prev_count,
                        const float* prev_mean, const float* prev_var, int64_t* count,
                        float* mean, float* var, const float* norm_gamma, const float* norm_beta,
@@ -199,7 +203,10 @@ int mega_long_conv_fwd(const void* x, void* y, int dtype, const float* k, int64_
  *   prev_count   [B] int64; prev_mean, prev_var [B,G] fp32
  *   gamma, beta  [H] fp32 (gamma is weight + 1, as the module passes it)
  *   mask         [B,L] bytes, non-zero = padding, or NULL
- *   count [B] int64, mean, var [B,G] fp32: state after the last token
+ *   count [B] int64, mean, var [B,G] fp32: state after the last token; they must not overlap
+ *   prev_count / prev_mean / prev_var (MEGA_ERR_ARG): every time tile of a row reads the prior
+ *   state while the row's last tile writes the new one (per-feature variant: count must not
+ *   overlap prev_count; mean / var may be updated in place there)
  *   group_mean, cummean, cumrstd: [B,L,G] fp32 each, or NULL to skip (they exist for
  *   the backward pass only)
  * per-feature variant (G == H): stands in for timestep_norm_fwd

@@ -42,6 +42,26 @@ def test_argument_checks_need_no_gpu():
     assert lib.mega_ema_fwd_workspace_bytes(4, 1024, 16, 4096, 0, 0) > 0
 
 
+def test_state_aliasing_rules_answer_without_a_gpu():
+    """The decode step and the norms reject a count that overlaps prev_count (several workgroups
+    read the old value while one writes the new one); the check runs before anything is launched,
+    so made-up addresses are enough."""
+    lib = M._lib.load()
+    a = 0x10000   # never dereferenced
+    step = lambda pc, c: lib.mega_norm_ema_step(a, a, a, 1, pc, a, a, c, a, a, a, a, 1e-5, a, a, a, 1, a, a, a,
+                                                4, 64, 4, 16, None)
+    assert step(0x20000, 0x20000) == -1 and b"overlap" in lib.mega_last_error()
+    assert step(0x20000, 0x20000 + 24) == -1          # partial overlap of the 4 x 8 bytes
+    gtsn = lambda pc, pm, pv, c, m, v: lib.mega_group_timestep_norm_fwd(
+        a, a, 1, pc, pm, pv, a, a, None, 2, 8, 64, 4, 1e-5, c, m, v, None, None, None, None, 0, None)
+    assert gtsn(0x20000, 0x30000, 0x40000, 0x20000, 0x50000, 0x60000) == -1 and b"overlap" in lib.mega_last_error()
+    assert gtsn(0x20000, 0x30000, 0x40000, 0x70000, 0x30000, 0x60000) == -1
+    assert gtsn(0x20000, 0x30000, 0x40000, 0x70000, 0x50000, 0x40000 + 28) == -1
+    ftsn = lib.mega_timestep_norm_fwd(a, a, 1, 0x20000, a, a, a, a, None, 2, 8, 64, 1e-5, 0x20008, a, a, None, None,
+                                      None, 0, None)
+    assert ftsn == -1 and b"overlap" in lib.mega_last_error()
+
+
 def test_ops_reject_cpu_tensors():
     import torch
     x = torch.zeros(1, 4, 8)
