@@ -42,6 +42,8 @@ SIGNATURES = {
     "mega_timestep_norm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "mega_group_timestep_norm_fwd": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, C.c_double,
                                             _p, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "mega_group_timestep_norm_fwd_noalloc": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64,
+                                                    C.c_double, _p, _p, _p, _p, _p, _p, _p]),
     "mega_timestep_norm_fwd": (_int, [_p, _p, _int, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, C.c_double,
                                       _p, _p, _p, _p, _p, _p, _sz, _p]),
     "mega_timestep_norm_bwd_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),

@@ -612,14 +612,12 @@ extern "C" size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64
   return tsn_workspace_bytes(B, G, g.ntiles);
 }
 
-extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
-                                            const int64_t* prev_count, const float* prev_mean,
-                                            const float* prev_var, const float* gamma,
-                                            const float* beta, const uint8_t* mask, int64_t B,
-                                            int64_t L, int64_t H, int64_t G, double eps,
-                                            int64_t* count, float* mean, float* var,
-                                            float* group_mean, float* cummean, float* cumrstd,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* prev_count,
+                              const float* prev_mean, const float* prev_var, const float* gamma,
+                              const float* beta, const uint8_t* mask, int64_t B, int64_t L, int64_t H,
+                              int64_t G, double eps, int64_t* count, float* mean, float* var,
+                              float* group_mean, float* cummean, float* cumrstd, void* workspace,
+                              size_t workspace_bytes, bool fixed_scratch, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "group_timestep_norm_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && H > 0 && G > 0, MEGA_ERR_ARG,
@@ -651,6 +649,13 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
   TsnGeom g;
   MEGA_REQUIRE(tsn_geometry(dtype, B, L, H, G, &g), MEGA_ERR_UNSUPPORTED,
                "group_timestep_norm_fwd: H=%ld G=%ld outside the supported envelope", (long)H, (long)G);
+  if (fixed_scratch) {
+    MEGA_REQUIRE(workspace_bytes >= tsn_workspace_bytes(B, G, g.ntiles), MEGA_ERR_UNSUPPORTED,
+                 "group_timestep_norm_fwd_noalloc: B=%ld L=%ld G=%ld needs %zu bytes of tile records, the library's "
+                 "fixed scratch array holds %zu (B * ceil(L / %d) * (2 G + 1) * 8 + 256 must fit); use "
+                 "mega_group_timestep_norm_fwd with a caller workspace",
+                 (long)B, (long)L, (long)G, tsn_workspace_bytes(B, G, g.ntiles), workspace_bytes, g.tt);
+  }
   MEGA_REQUIRE(workspace != nullptr && workspace_bytes >= tsn_workspace_bytes(B, G, g.ntiles),
                MEGA_ERR_WORKSPACE, "group_timestep_norm_fwd: workspace of %zu bytes needed",
                tsn_workspace_bytes(B, G, g.ntiles));
@@ -668,6 +673,67 @@ extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
     case MEGA_BF16: return dispatch_vec<bf16_t>(P, g, s);
     default: return dispatch_vec<f16_t>(P, g, s);
   }
+}
+
+extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,
+                                            const int64_t* prev_count, const float* prev_mean,
+                                            const float* prev_var, const float* gamma,
+                                            const float* beta, const uint8_t* mask, int64_t B,
+                                            int64_t L, int64_t H, int64_t G, double eps,
+                                            int64_t* count, float* mean, float* var,
+                                            float* group_mean, float* cummean, float* cumrstd,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  return group_tsn_fwd_impl(x, y, dtype, prev_count, prev_mean, prev_var, gamma, beta, mask, B, L, H, G, eps, count,
+                            mean, var, group_mean, cummean, cumrstd, workspace, workspace_bytes, false, stream);
+}
+
+// ---------------------------------------------------------------- the same call without a workspace argument
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc): the launch epoch, retire counters and tile records live in a
+// file-scope device array instead of a caller workspace.  Every GPU holds its own copy of the array
+// at its own address; host code never uses the array's name as an address (it is a host-side
+// stand-in), only the pointer hipGetSymbolAddress returns for the current device, looked up once per
+// device.  The array starts zero-filled (device globals do), which is the "zero once" the workspace
+// protocol asks for; after that every launch leaves the header consistent and the records carry
+// launch tags, so nothing is cleared between calls even when the shape changes.  All calls on one
+// GPU share the array: calls that can overlap in time (two streams) race.
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)1 << 20;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];   // per device: the address of that device's copy, 0 = not looked up yet
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  MEGA_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, MEGA_ERR_LAUNCH,
+               "group_timestep_norm_fwd_noalloc: no current HIP device (%s)", hipGetErrorString(e));
+  void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    MEGA_REQUIRE(e == hipSuccess && p != nullptr, MEGA_ERR_LAUNCH,
+                 "group_timestep_norm_fwd_noalloc: hipGetSymbolAddress failed on device %d: %s", dev,
+                 hipGetErrorString(e));
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);   // two threads racing here store the same address
+  }
+  *out = p;
+  return MEGA_OK;
+}
+
+extern "C" int mega_group_timestep_norm_fwd_noalloc(const void* x, void* y, int dtype,
+                                                    const int64_t* prev_count, const float* prev_mean,
+                                                    const float* prev_var, const float* gamma,
+                                                    const float* beta, const uint8_t* mask, int64_t B,
+                                                    int64_t L, int64_t H, int64_t G, double eps,
+                                                    int64_t* count, float* mean, float* var,
+                                                    float* group_mean, float* cummean, float* cumrstd,
+                                                    void* stream) {
+  void* ptr = nullptr;
+  const int rc = static_scratch(&ptr);
+  if (rc != MEGA_OK) return rc;
+  return group_tsn_fwd_impl(x, y, dtype, prev_count, prev_mean, prev_var, gamma, beta, mask, B, L, H, G, eps, count,
+                            mean, var, group_mean, cummean, cumrstd, ptr, kStaticScratchBytes, true, stream);
 }
 
 extern "C" int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* prev_count,

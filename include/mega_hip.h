@@ -227,6 +227,30 @@ int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* pre
                            float* cummean, float* cumrstd, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/* mega_group_timestep_norm_fwd without the workspace arguments.  No counterpart in the
+ * reference: it exists for callers that cannot allocate device memory or hand one over --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The
+ * launch epoch, retire counters and tile records live in a 1 MiB device array inside the
+ * library (each GPU the library runs on holds its own copy until the process ends); the call
+ * itself allocates and frees nothing.  Same arguments, results and errors as
+ * mega_group_timestep_norm_fwd, plus:
+ *   - MEGA_ERR_UNSUPPORTED when the tile records do not fit:
+ *     256 + B * ceil(L / TT) * (2 G + 1) * 8 bytes <= 1 MiB, TT = tokens per tile (<= 64;
+ *     mega_timestep_norm_workspace_bytes returns the exact figure for a shape);
+ *   - the first call on a device looks the array's address up (hipGetSymbolAddress): make
+ *     that call outside stream capture;
+ *   - all calls on one GPU share the array and it keeps the previous call's contents (the
+ *     records carry launch tags, so nothing needs clearing, also when the shape changes):
+ *     calls that can overlap in time on one GPU -- two streams, two host threads -- race.   */
+int mega_group_timestep_norm_fwd_noalloc(const void* x, void* y, int dtype,
+                                         const int64_t* prev_count, const float* prev_mean,
+                                         const float* prev_var, const float* gamma,
+                                         const float* beta, const uint8_t* mask, int64_t B,
+                                         int64_t L, int64_t H, int64_t G, double eps,
+                                         int64_t* count, float* mean, float* var,
+                                         float* group_mean, float* cummean, float* cumrstd,
+                                         void* stream);
+
 /* backward: stands in for group_timestep_norm_bwd and timestep_norm_bwd
  * (fairseq/csrc/ops/timestep_norm.cc:318-450 and :104-217, CUDA side
  * ops/timestep_norm_kernel.cu; caller norm_layer/timestep_norm.py:45-66).
