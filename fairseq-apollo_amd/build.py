@@ -20,6 +20,7 @@ SOURCES = [
     "sequence_norm.hip",
     "ema_scan.hip",
     "ema_mfma.hip",
+    "norm_ema_fused.hip",
     "ema_bwd.hip", "ema_bwd_tile.hip",
     "decode.hip",
     "elementwise.hip",

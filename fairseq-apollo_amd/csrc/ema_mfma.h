@@ -4,6 +4,38 @@
 
 namespace mega {
 
+// ---- layout of the per-channel operand image (written by ema_image_kernel): kImgSlots slots of
+// 64 lanes x 16 bytes.  Slots [0, kNOPS): the MFMA A operands K (Toeplitz of k[0..31]), P (p q^(31-i)),
+// C (gamma q^(i+1)), each as kNW* bf16 terms x 2 row blocks.  Then, per lane (j = lane & 15, r = lane >> 4)
+// for the four states (2r, 2r+1, 8+2r, 9+2r) as (re, im) pairs, two slots each:
+//   kSlotQ32  q^32      kSlotRS  q^64      kSlotRJ  (q^64)^j      kSlotRW  q^1024      kSlotRWJ  (q^1024)^j
+// and one slot in the layout of the 64-lane segment scan (kSlotScan: q^(32 kSEGT) of state lane >> 2).
+constexpr int kNS = 16;                  // complex states per channel (zero padded)
+#ifndef MEGA_SEGT
+#define MEGA_SEGT 2
+#endif
+constexpr int kSEGT = MEGA_SEGT;         // tiles per segment: super-chunk = 16 * kSEGT * 32 tokens
+#ifndef MEGA_NWK
+#define MEGA_NWK 2
+#endif
+#ifndef MEGA_NWP
+#define MEGA_NWP 2
+#endif
+#ifndef MEGA_NWC
+#define MEGA_NWC 1
+#endif
+constexpr int kNWK = MEGA_NWK;           // bf16 terms of the Toeplitz operand K
+constexpr int kNWP = MEGA_NWP;           // bf16 terms of the state-input operand P
+constexpr int kNWC = MEGA_NWC;           // bf16 terms of the state-output operand C
+constexpr int kNOPS = 2 * (kNWK + kNWP + kNWC);
+constexpr int kSlotK = 0, kSlotP = 2 * kNWK, kSlotC = 2 * (kNWK + kNWP);
+constexpr int kSlotQ32 = kNOPS, kSlotScan = kNOPS + 2, kSlotRS = kNOPS + 3, kSlotRJ = kNOPS + 5, kSlotRW = kNOPS + 7,
+              kSlotRWJ = kNOPS + 9, kSlotCmp = kNOPS + 11;
+constexpr int kImgSlots = kNOPS + 12;
+// kSlotCmp: per-state multipliers once each, six tables of 16 complex values (128 bytes = one line):
+enum { kCmpQ32 = 0, kCmpRS = 1, kCmpRS2 = 2, kCmpRS4 = 3, kCmpRS8 = 4, kCmpRW = 5 };
+constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
+
 // bytes of the per-channel operand images for a layer (0: the layer is outside the fast path)
 size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional);
 

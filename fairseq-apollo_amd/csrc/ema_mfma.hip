@@ -44,26 +44,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kWaves = 16;               // channels per workgroup
 constexpr int kThreadsM = kWaves * 64;
-constexpr int kNS = 16;                  // complex states per channel (zero padded)
-#ifndef MEGA_SEGT
-#define MEGA_SEGT 2
-#endif
-constexpr int kSEGT = MEGA_SEGT;         // tiles per segment: super-chunk = 16 * kSEGT * 32 tokens
-#ifndef MEGA_NWK
-#define MEGA_NWK 2
-#endif
-#ifndef MEGA_NWP
-#define MEGA_NWP 2
-#endif
-#ifndef MEGA_NWC
-#define MEGA_NWC 1
-#endif
-constexpr int kNWK = MEGA_NWK;           // bf16 terms of the Toeplitz operand K
-constexpr int kNWP = MEGA_NWP;           // bf16 terms of the state-input operand P
-constexpr int kNWC = MEGA_NWC;           // bf16 terms of the state-output operand C
-constexpr int kNOPS = 2 * (kNWK + kNWP + kNWC);
-constexpr int kImgSlots = kNOPS + 3;     // + q^32 of the lane's 4 states (2 slots) + scan multiplier
-constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
 
 // ------------------------------------------------------------------------------------------
 // kernel generation
@@ -216,6 +196,52 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     const float2 w = pw[32 * kNS + (lane >> 2)];
     for (int t = 0; t < kSEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
     img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
+    // multipliers in the matrix-core lane layout (lane = segment j + 16 r, states 2r, 2r+1, 8+2r, 9+2r), for the
+    // kernel that scans 16 segments of 64 tokens across the lanes of a row: per state q^64, (q^64)^j,
+    // (q^64)^16 = q^1024 (the step from one 1024-token block to the next) and (q^1024)^j
+    const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
+    cfloat RS[4], RJ[4], RW[4], RWJ[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float2 w32 = pw[32 * kNS + nn[u]];
+      RS[u] = cmul(cfloat{w32.x, w32.y}, cfloat{w32.x, w32.y});
+      cfloat a = {1.f, 0.f};
+      for (int t = 0; t < (lane & 15); ++t) a = cmul(a, RS[u]);
+      RJ[u] = a;
+      cfloat w = RS[u];
+      for (int t = 0; t < 4; ++t) w = cmul(w, w);
+      RW[u] = w;
+      cfloat c = {1.f, 0.f};
+      for (int t = 0; t < (lane & 15); ++t) c = cmul(c, w);
+      RWJ[u] = c;
+    }
+    auto put2 = [&](const cfloat (&v)[4]) {
+      img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(v[0].re), __float_as_uint(v[0].im),
+                                             __float_as_uint(v[1].re), __float_as_uint(v[1].im));
+      img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(v[2].re), __float_as_uint(v[2].im),
+                                             __float_as_uint(v[3].re), __float_as_uint(v[3].im));
+    };
+    put2(RS);
+    put2(RJ);
+    put2(RW);
+    put2(RWJ);
+    if (lane < kNS) {
+      // the same multipliers once per state (a lane of the streaming kernels reads 16 bytes = two states)
+      float2* cmp = (float2*)(img + (size_t)kSlotCmp * 64);
+      const float2 w32 = pw[32 * kNS + lane];
+      cfloat v = {w32.x, w32.y};
+      cmp[kCmpQ32 * kNS + lane] = make_float2(v.re, v.im);
+      v = cmul(v, v);
+      cmp[kCmpRS * kNS + lane] = make_float2(v.re, v.im);
+      v = cmul(v, v);
+      cmp[kCmpRS2 * kNS + lane] = make_float2(v.re, v.im);
+      v = cmul(v, v);
+      cmp[kCmpRS4 * kNS + lane] = make_float2(v.re, v.im);
+      v = cmul(v, v);
+      cmp[kCmpRS8 * kNS + lane] = make_float2(v.re, v.im);
+      v = cmul(v, v);
+      cmp[kCmpRW * kNS + lane] = make_float2(v.re, v.im);
+    }
   }
 }
 

@@ -1,0 +1,917 @@
+// TimestepNorm -> moving-average layer in one kernel (gfx950, bf16 activations, 64 channels per
+// norm group, ndim <= 16): what MovingAverageGatedAttention.forward does at
+// fairseq/modules/moving_average_gated_attention.py:304-315 (x = norm(x); mx = move(x^T)) with
+// TimestepNorm per fairseq/csrc/ops/timestep_norm.cc:218-316 and the layer per
+// fairseq/modules/base_moving_average.py:120-172.  x is read once, xn (the norm's output, which the
+// layer also feeds to v_proj) and y are written once.
+//
+// A workgroup (16 waves) owns one (batch row, norm group, block of 1024 tokens): whole 128-byte
+// lines of x, xn and -- with [B, D, L] rows -- y.
+//   1. load the block, per-token moments of the group (packed dot products + DPP), Welford scan over
+//      the block's tokens, publish the block aggregate, fold the earlier blocks' aggregates of the
+//      same (row, group) and the prior state into the carry-in, finish mean / rstd per token;
+//   2. normalise from registers, store xn, and stage xn (bf16, as the layer sees it) into LDS
+//      transposed to channel rows;
+//   3. per channel (4 per wave), with the operand images of ema_image_kernel:
+//        sweep 1: end states of the 16 segments (64 tokens = 2 tiles each) from a zero start on the
+//                 matrix cores, scanned across the 16 lanes of a DPP row; the block's end state from a
+//                 zero start is published, the segments' start states are parked as bf16;
+//      look-back: the earlier blocks' end states (and the caller's carried state) folded into the
+//                 block's start state, h_start = sum_d (q^1024)^d E_{s-1-d};
+//        sweep 2: y_tile = K x_tile + C (h_seg + (q^64)^j h_start), bf16, back into LDS over x, and
+//                 out as whole rows.
+// Blocks map to workgroup ids time-major and workgroups are dispatched in id order, so a block only
+// waits for blocks dispatched before it; every wait is bounded and poisons the block's outputs with
+// NaN (and sets the error word of the workspace header) when it gives up.
+#include "ema_mfma.h"
+#include "tsn_common.h"
+
+// Phase markers: a profiling build defines MEGA_FTR(k) to stamp a clock per workgroup; no-ops here.
+#ifndef MEGA_FTR
+#define MEGA_FTR(k)
+#define MEGA_FTR_END()
+#endif
+#ifndef MEGA_FTR2
+#define MEGA_FTR2(k)
+#endif
+
+namespace mega {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kFW = 16;                       // waves per workgroup
+constexpr int kFT = kFW * 64;                 // threads
+constexpr int kFC = 64;                       // channels per workgroup = per norm group
+constexpr int kFSeg = 1024;                   // tokens per block: 16 segments x 2 tiles x 32
+constexpr int kFCPW = kFC / kFW;              // channels per wave
+constexpr int kFNLD = kFSeg * 8 / kFT;        // 16-byte pieces per thread
+constexpr int kFRow = kFSeg * 2;              // bytes of one channel row in LDS
+constexpr int kFTile = kFC * kFRow + (kFC / 4) * 16;
+constexpr int kFRecW = 4 + kFC * kNS * 2;     // 64-bit words per block record: n, mean, var, pad, end states
+constexpr int kFMaxBlocks = 16;               // terms of the look-back sum (earlier blocks + the carried state): one per lane of a row
+constexpr int kFTabs = 2;                     // per-state multiplier tables kept in LDS: q^32, q^64
+constexpr size_t kFSmem = (size_t)kFTile + 2 * kFSeg * 4 + 64 + (size_t)kFTabs * kFC * 128;
+
+static_assert(kSEGT == 2, "the fused kernel uses the q^64 segment multipliers of the image");
+static_assert(kFSmem <= 160 * 1024, "LDS of one workgroup");
+
+// the MFMA A operands of one channel
+struct ImgSet {
+  bf16x8 P[kNWP][2], K[kNWK][2], C[kNWC][2];
+};
+
+struct FusedArgs {
+  const bf16_t* x;       // [B, L, D]
+  bf16_t* xn;            // [B, L, D]
+  bf16_t* y;             // strides (syb, syd, syl): [B, D, L] rows (syl == 1) or [B, L, D] (syd == 1)
+  int64_t syb, syd, syl;
+  const int64_t* prev_count;
+  const float* prev_mean;
+  const float* prev_var;
+  int64_t* count;
+  float* mean;
+  float* var;
+  const float* gamma;    // [D] (weight + 1)
+  const float* beta;     // [D]
+  const uint4* image;    // [D][kImgSlots][64]
+  const float* h_in;     // [B, D, N, 2] or null
+  float* h_out;          // [B, D, N, 2] or null
+  TsnHeader* hdr;
+  unsigned long long* rec;   // [B * G][S][kFRecW]
+  int B, L, D, G, N, S;
+  float eps;
+  int is_complex;
+  int xcd_map;
+};
+
+__device__ __forceinline__ int row_base(int c) { return c * kFRow + (c >> 2) * 16; }
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ float lane_bcast(float v, int src_lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
+}
+
+// one step of the inclusive scan of h_j = R h_{j-1} + e_j across the 16 lanes of a row: lanes take the
+// value SH lanes to the left (zero outside the row) times R^SH
+template <int CTRL>
+__device__ __forceinline__ void scan_step(float (&er)[4], float (&ei)[4], const float (&rr)[4], const float (&ri)[4]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const float tr = dpp_f<CTRL>(er[u]), ti = dpp_f<CTRL>(ei[u]);
+    const float nri = -ri[u];
+    er[u] = fmaf(tr, rr[u], er[u]);
+    er[u] = fmaf(ti, nri, er[u]);
+    ei[u] = fmaf(ti, rr[u], ei[u]);
+    ei[u] = fmaf(tr, ri[u], ei[u]);
+  }
+}
+
+__device__ __forceinline__ void csquare(const float (&ar)[4], const float (&ai)[4], float (&br)[4], float (&bi)[4]) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    br[u] = ar[u] * ar[u] - ai[u] * ai[u];
+    bi[u] = 2.f * ar[u] * ai[u];
+  }
+}
+
+// activations leave once and are not read again by this kernel: streaming (non-temporal) stores
+#ifndef MEGA_FUSED_NT
+#define MEGA_FUSED_NT 1
+#endif
+__device__ __forceinline__ void store_stream(uint4* p, uint4 v) {
+#if MEGA_FUSED_NT
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), (u32x4*)p);
+#else
+  *p = v;
+#endif
+}
+
+// slot `slot` of an operand image: uniform base, 32-bit lane offset (scalar-base addressing)
+__device__ __forceinline__ uint4 img_slot(const char* base, int slot, uint32_t lane_off) {
+  return *(const uint4*)(base + slot * 1024 + lane_off);
+}
+
+__device__ __forceinline__ void load_c4(const char* base, int slot, uint32_t lane_off, float (&re)[4], float (&im)[4]) {
+  const uint4 a = img_slot(base, slot, lane_off), b = img_slot(base, slot + 1, lane_off);
+  re[0] = __uint_as_float(a.x); im[0] = __uint_as_float(a.y);
+  re[1] = __uint_as_float(a.z); im[1] = __uint_as_float(a.w);
+  re[2] = __uint_as_float(b.x); im[2] = __uint_as_float(b.y);
+  re[3] = __uint_as_float(b.z); im[3] = __uint_as_float(b.w);
+}
+
+// the four states of row block r from table `tab` of the compact slot: two 16-byte pieces that the 16 lanes of
+// a row share (one line per table leaves the cache, not a slot)
+__device__ __forceinline__ void load_cmp(const char* base, int tab, uint32_t r_off, float (&re)[4], float (&im)[4]) {
+  const uint4 a = *(const uint4*)(base + kSlotCmp * 1024 + tab * 128 + r_off);
+  const uint4 b = *(const uint4*)(base + kSlotCmp * 1024 + tab * 128 + 64 + r_off);
+  re[0] = __uint_as_float(a.x); im[0] = __uint_as_float(a.y);
+  re[1] = __uint_as_float(a.z); im[1] = __uint_as_float(a.w);
+  re[2] = __uint_as_float(b.x); im[2] = __uint_as_float(b.y);
+  re[3] = __uint_as_float(b.z); im[3] = __uint_as_float(b.w);
+}
+
+// the same from the copy of tables 0..2 in LDS
+__device__ __forceinline__ void lds_cmp(const char* s_tab, int tab, int c, uint32_t r_off, float (&re)[4], float (&im)[4]) {
+  const float4 a = *(const float4*)(s_tab + (tab * kFC + c) * 128 + r_off);
+  const float4 b = *(const float4*)(s_tab + (tab * kFC + c) * 128 + 64 + r_off);
+  re[0] = a.x; im[0] = a.y; re[1] = a.z; im[1] = a.w;
+  re[2] = b.x; im[2] = b.y; re[3] = b.z; im[3] = b.w;
+}
+
+// LOUT 0: y as [B, D, L] rows; 1: y as [B, L, D]
+template <int LOUT>
+__global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* tile = smem;
+  float* s_gm = (float*)(smem + kFTile);      // [kFSeg] group mean of a token, later the running mean
+  float* s_gv = s_gm + kFSeg;                 // [kFSeg] group variance, later the running rstd
+  float* s_wt = s_gv + kFSeg;                 // [4][4] totals of the four scanning waves
+  float* s_end = s_gm;                        // [kFC][kNS][2] block end states from a zero start (after step 2)
+  char* s_tab = (char*)(s_wt + 16);           // [kFTabs][kFC][kNS] complex: q^32, q^64 of every channel
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: channel rows and image addresses stay scalar
+  const int G = A.G;
+  const int BG = A.B * G;
+  const int s = (int)blockIdx.x / BG, local = (int)blockIdx.x - s * BG;
+  int b, g;
+  if (A.xcd_map) {
+    // consecutive workgroup ids go to the 8 XCDs in turn: keep a group's blocks (and with them the operand
+    // images of its 64 channels) on one XCD, G / 8 groups per XCD
+    const int gp = G >> 3, xcd = local & 7, slot = local >> 3;
+    g = xcd * gp + slot % gp;
+    b = slot / gp;
+  } else {
+    b = local / G;
+    g = local - b * G;
+  }
+  const uint32_t tag = A.hdr->epoch + 1u;
+  const int t0 = s * kFSeg;
+  const int piece = tid & 7, tokl = tid >> 3;            // 16-byte piece of the 128-byte line, token 0..127
+  // addresses of the block's lines: a uniform base per 128-token round plus one 32-bit lane offset
+  const size_t xblk = ((size_t)b * A.L + t0) * A.D + (size_t)g * kFC;
+  const uint32_t toff = (uint32_t)tokl * (uint32_t)A.D + piece * 8;
+  const size_t brow = (size_t)b * G + g;
+  unsigned long long* const myrec = A.rec + (brow * A.S + s) * kFRecW;
+  bool poison = false;
+
+  MEGA_FTR(0);
+  // ---- everything the norm needs from memory is requested before the block itself
+  const Moments prior = {(float)A.prev_count[b], A.prev_mean[brow], A.prev_var[brow]};
+  float gam[8], bet[8];
+  load_params<8>(A.gamma + g * kFC + piece * 8, gam);
+  load_params<8>(A.beta + g * kFC + piece * 8, bet);
+  uint4 xv[kFNLD];
+#pragma unroll
+  for (int k = 0; k < kFNLD; ++k) xv[k] = *(const uint4*)(A.x + xblk + (size_t)k * 128 * A.D + toff);
+
+  // the per-state multipliers of the group's 64 channels (three lines per channel) go to LDS once
+  {
+    static_assert(kCmpQ32 == 0 && kCmpRS == 1 && kFTabs == 2, "tables 0..1 of the compact slot are staged");
+    const char* ibase = (const char*)A.image + (size_t)g * kFC * kImgRowBytes + kSlotCmp * 1024;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int idx = it * kFT + tid;               // (table, channel, 16-byte piece)
+      if (idx < kFTabs * kFC * 8) {
+        const int t = idx / (kFC * 8), rem = idx - t * (kFC * 8), c = rem >> 3, pc = rem & 7;
+        *(uint4*)(s_tab + (t * kFC + c) * 128 + pc * 16) =
+            *(const uint4*)(ibase + (size_t)c * kImgRowBytes + t * 128 + pc * 16);
+      }
+    }
+  }
+
+  // ---- moments of every token's group (64 channels = the 8 lanes of a line)
+#pragma unroll
+  for (int k = 0; k < kFNLD; ++k) {
+    const uint32_t w[4] = {xv[k].x, xv[k].y, xv[k].z, xv[k].w};
+    float sm = 0.f, sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sm = dot2_ones<bf16_t>(w[i], sm);
+      sq = dot2_self<bf16_t>(w[i], sq);
+    }
+    const float m = group_sum<8>(sm) * (1.0f / kFC);
+    const float v = fmaxf(group_sum<8>(sq) * (1.0f / kFC) - m * m, 0.f);
+    if (piece == 0) {
+      s_gm[k * 128 + tokl] = m;
+      s_gv[k * 128 + tokl] = v;
+    }
+  }
+  __syncthreads();
+  MEGA_FTR(1);
+
+  // ---- running statistics: waves 0..3 scan 256 tokens each (4 per lane), the wave totals meet in LDS
+  Moments pref[4], lane_exc = {0.f, 0.f, 0.f};
+  if (wave < 4) {
+    const float4 m4 = *(const float4*)(s_gm + wave * 256 + lane * 4);
+    const float4 v4 = *(const float4*)(s_gv + wave * 256 + lane * 4);
+    const float mm[4] = {m4.x, m4.y, m4.z, m4.w}, vv[4] = {v4.x, v4.y, v4.z, v4.w};
+    Moments st = {1.f, mm[0], vv[0]};
+    pref[0] = st;
+#pragma unroll
+    for (int u = 1; u < 4; ++u) {
+      st = merge(st, Moments{1.f, mm[u], vv[u]});
+      pref[u] = st;
+    }
+    const Moments inc = row_scan(st);
+    const Moments exc = dpp_m<0x111>(inc);
+    Moments acc = {0.f, 0.f, 0.f}, rp = {0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const Moments t = {__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, inc.n), 16 * r + 15)),
+                         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, inc.mean), 16 * r + 15)),
+                         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, inc.var), 16 * r + 15))};
+      if ((lane >> 4) == r) rp = acc;
+      acc = merge(acc, t);
+    }
+    lane_exc = merge(rp, exc);
+    if (lane == 0) {
+      s_wt[wave * 4] = acc.n;
+      s_wt[wave * 4 + 1] = acc.mean;
+      s_wt[wave * 4 + 2] = acc.var;
+    }
+  }
+  __syncthreads();
+  if (wave < 4) {
+    Moments wpre = {0.f, 0.f, 0.f}, tot = {0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w == wave) wpre = tot;
+      tot = merge(tot, Moments{s_wt[w * 4], s_wt[w * 4 + 1], s_wt[w * 4 + 2]});
+    }
+    if (wave == 0 && lane == 0) {
+      put_rec(myrec, tagged((uint32_t)tot.n, tag));
+      put_rec(myrec + 1, tagged(__float_as_uint(tot.mean), tag));
+      put_rec(myrec + 2, tagged(__float_as_uint(tot.var), tag));
+    }
+    MEGA_FTR(2);
+    // earlier blocks of this (row, group): lane i fetches block i's aggregate
+    Moments accp = {0.f, 0.f, 0.f};
+    if (s > 0) {
+      const unsigned long long* rp = A.rec + (brow * A.S + (lane < s ? lane : s - 1)) * kFRecW;
+      unsigned long long w0, w1, w2;
+      uint32_t spins = 0;
+      for (;;) {
+        w0 = get_rec(rp);
+        w1 = get_rec(rp + 1);
+        w2 = get_rec(rp + 2);
+        const bool ok = (uint32_t)(w0 >> 32) == tag && (uint32_t)(w1 >> 32) == tag && (uint32_t)(w2 >> 32) == tag;
+        if (__all(ok)) break;
+        if (++spins > kSpinLimit) {
+          poison = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      for (int i = 0; i < s; ++i) {
+        const Moments t = {(float)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)w0, i),
+                           __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)(uint32_t)w1, i)),
+                           __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)(uint32_t)w2, i))};
+        accp = merge(accp, t);
+      }
+    }
+    MEGA_FTR(3);
+    Moments carry = merge(prior, accp);
+    if (poison) {
+      carry.mean = __builtin_nanf("");
+      if (lane == 0) publish_u32(&A.hdr->error, 1u);
+    }
+    const Moments base = merge(carry, merge(wpre, lane_exc));
+    Moments full = base;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      full = merge(base, pref[u]);
+      s_gm[wave * 256 + lane * 4 + u] = full.mean;
+      s_gv[wave * 256 + lane * 4 + u] = __builtin_amdgcn_rsqf(full.var + A.eps);
+    }
+    if (s == A.S - 1 && wave == 3 && lane == 63) {
+      A.mean[brow] = full.mean;
+      A.var[brow] = full.var;
+      if (g == 0) A.count[b] = poison ? (int64_t)-1 : A.prev_count[b] + (int64_t)A.L;
+    }
+  }
+  __syncthreads();
+
+  // the operands of the wave's first channel travel under the normalisation
+  const uint32_t loff0 = (uint32_t)lane * 16;
+  // the P operand of channel c (requested one channel ahead)
+  auto load_p = [&](const int c, ImgSet& I) {
+    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    uint32_t loff = loff0;
+    asm volatile("" : "+v"(loff));
+#pragma unroll
+    for (int w = 0; w < kNWP; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) I.P[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotP + 2 * w + mb, loff));
+  };
+  auto load_kc = [&](const int c, ImgSet& I) {
+    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    uint32_t loff = loff0;
+    asm volatile("" : "+v"(loff));
+#pragma unroll
+    for (int w = 0; w < kNWK; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) I.K[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotK + 2 * w + mb, loff));
+#pragma unroll
+    for (int w = 0; w < kNWC; ++w)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) I.C[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
+  };
+  ImgSet img_set[2];
+  load_p(wave, img_set[0]);
+  load_kc(wave, img_set[0]);
+
+  // ---- normalise from registers and stage xn (bf16, as the layer sees it) transposed: channel rows of 16
+  // segments x 128 bytes, 16-byte chunk c of segment j at chunk c ^ (j >> 1) (the 16 lanes of a matrix-core
+  // operand load then cover all banks); the lanes of tokens (2m, 2m+1) swap halves so that each writes dwords
+  // (even token | odd token << 16) of four channels
+  {
+    const int odd = tokl & 1;
+    const uint32_t sel_lo = odd ? 0x01000504u : 0x05040100u;
+    const uint32_t sel_hi = odd ? 0x03020706u : 0x07060302u;
+    const int tl = tokl & ~1;
+    char* wbase = tile + row_base(piece * 8 + odd * 4) + (tl >> 6) * 128 + ((tl & 7) >> 1) * 4;
+    const int c8 = (tl & 63) >> 3;
+#pragma unroll
+    for (int k = 0; k < kFNLD; ++k) {
+      const int tok = k * 128 + tokl;
+      const float m = s_gm[tok], r = s_gv[tok];
+      const float mr = m * r;
+      const uint32_t w[4] = {xv[k].x, xv[k].y, xv[k].z, xv[k].w};
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float lo = fmaf(__uint_as_float(w[i] << 16), r, -mr);
+        const float hi = fmaf(__uint_as_float(w[i] & 0xffff0000u), r, -mr);
+        o[i] = pack_bf16(fmaf(lo, gam[2 * i], bet[2 * i]), fmaf(hi, gam[2 * i + 1], bet[2 * i + 1]));
+      }
+#ifndef MEGA_X_NOXN
+      store_stream((uint4*)(A.xn + xblk + (size_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
+#endif
+      const uint32_t s0 = odd ? o[0] : o[2], s1 = odd ? o[1] : o[3];
+      const uint32_t r0 = dpp_u<0x128>(s0), r1 = dpp_u<0x128>(s1);       // row_ror:8 = the partner token's lane
+      const uint32_t m0 = odd ? o[2] : o[0], m1 = odd ? o[3] : o[1];
+      char* wp = wbase + (2 * k) * 128 + ((c8 ^ k) << 4);
+      *(uint32_t*)(wp) = __builtin_amdgcn_perm(r0, m0, sel_lo);
+      *(uint32_t*)(wp + kFRow) = __builtin_amdgcn_perm(r0, m0, sel_hi);
+      *(uint32_t*)(wp + 2 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_lo);
+      *(uint32_t*)(wp + 3 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_hi);
+    }
+  }
+  __syncthreads();
+
+  MEGA_FTR(4);
+  // ---- moving average.  MFMA lane layout: column j = lane & 15 is segment j, r = lane >> 4 holds the
+  // states (2r, 2r+1, 8+2r, 9+2r) of the 32-row state products.
+  const int j = lane & 15, r = lane >> 4;
+  const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
+  const bool last_block = s == A.S - 1;
+#ifdef MEGA_X_ONEWAVE
+  const int nterms = 0;
+#else
+  const int nterms = s + (A.h_in ? 1 : 0);
+#endif
+  const uint32_t roff0 = (uint32_t)r * 16;
+
+  // the wave's own row leaves as whole lines ([B, D, L] rows)
+  auto store_row = [&](const int c) {
+    // LDS operations of one wave are performed in order: the lanes' writes above are visible to the
+    // reads below without waiting for anything else (a release fence would also wait for the wave's
+    // outstanding global stores)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const char* rb = tile + row_base(c);
+    bf16_t* yr = A.y + (size_t)b * A.syb + (size_t)(g * kFC + c) * A.syd + t0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int q = k * 64 + lane;                 // 16-byte chunk of the row: segment q >> 3, chunk q & 7
+      const uint4 v = *(const uint4*)(rb + (q >> 3) * 128 + (((q & 7) ^ (q >> 4)) << 4));
+      store_stream((uint4*)(yr + q * 8), v);
+    }
+  };
+
+  // pass 1 over channel c, everything that does not need the earlier blocks: end states of the 16 segments
+  // from a zero start (P products), scanned across the row; the block's end state from a zero start is
+  // published; y = K x + C (segment start state from a zero block start) goes back into LDS over x as bf16
+  auto pass1 = [&](const int c, const int cnext, ImgSet& cur, ImgSet& nxt) {
+    uint32_t roff = roff0;
+    asm volatile("" : "+v"(roff));
+    float Qr[4], Qi[4];
+    lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
+    char* row = tile + row_base(c) + j * 128;
+    float Er[4], Ei[4], Fr[4], Fi[4];              // F: state after the segment's first tile from a zero segment start
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const bf16x8 X = *(const bf16x8*)(row + (((4 * t + r) ^ (j >> 1)) << 4));
+      f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < kNWP; ++w) {
+        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.P[w][0], X, S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.P[w][1], X, S1, 0, 0, 0);
+      }
+      const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
+      const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (t == 0) {
+          Fr[u] = sr[u];
+          Fi[u] = si[u];
+        } else {
+          Er[u] = fmaf(Qr[u], Fr[u], fmaf(-Qi[u], Fi[u], sr[u]));
+          Ei[u] = fmaf(Qr[u], Fi[u], fmaf(Qi[u], Fr[u], si[u]));
+        }
+      }
+    }
+    MEGA_FTR2(0);
+    // the next channel's P operand is requested as soon as this one's is used up
+    __builtin_amdgcn_sched_barrier(0);
+    if (cnext >= 0) load_p(cnext, nxt);
+    __builtin_amdgcn_sched_barrier(0);
+#ifndef MEGA_X_NOSCAN
+    {
+      float Rr[4], Ri[4], R2r[4], R2i[4];
+      lds_cmp(s_tab, kCmpRS, c, roff, Rr, Ri);
+      scan_step<0x111>(Er, Ei, Rr, Ri);
+      csquare(Rr, Ri, R2r, R2i);
+      scan_step<0x112>(Er, Ei, R2r, R2i);
+      csquare(R2r, R2i, Rr, Ri);
+      scan_step<0x114>(Er, Ei, Rr, Ri);
+      csquare(Rr, Ri, R2r, R2i);
+      scan_step<0x118>(Er, Ei, R2r, R2i);
+    }
+#endif
+    MEGA_FTR2(1);
+    // lane 15 of a row holds the block's end state from a zero start: parked in LDS, published for the later
+    // blocks after the wave's last channel (and kept for the carried state the last block returns)
+    if (j == 15) {
+      *(float4*)(s_end + (c * kNS + 2 * r) * 2) = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
+      *(float4*)(s_end + (c * kNS + 8 + 2 * r) * 2) = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
+    }
+    MEGA_FTR2(2);
+    // ... and its K and C operands a whole pass before they are needed
+    __builtin_amdgcn_sched_barrier(0);
+    if (cnext >= 0) load_kc(cnext, nxt);
+    __builtin_amdgcn_sched_barrier(0);
+    MEGA_FTR2(3);
+    // start state of segment j = inclusive value of segment j - 1; of its second tile: q^32 times that + F
+    float hr[4], hi[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      hr[u] = dpp_f<0x111>(Er[u]);
+      hi[u] = dpp_f<0x111>(Ei[u]);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const bf16x8 X = *(const bf16x8*)(row + (((4 * t + r) ^ (j >> 1)) << 4));
+      bf16x8 Hop;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        Hop[2 * u] = (__bf16)hr[u];
+        Hop[2 * u + 1] = (__bf16)hi[u];
+      }
+      f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < kNWC; ++w) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.C[w][0], Hop, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.C[w][1], Hop, Y1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int w = 0; w < kNWK; ++w) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.K[w][0], X, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.K[w][1], X, Y1, 0, 0, 0);
+      }
+      if (t == 0) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float nr = fmaf(Qr[u], hr[u], fmaf(-Qi[u], hi[u], Fr[u]));
+          hi[u] = fmaf(Qr[u], hi[u], fmaf(Qi[u], hr[u], Fi[u]));
+          hr[u] = nr;
+        }
+      }
+      // y (bf16) over x: tokens 32 t + 4 r + {0..3} and 32 t + 16 + 4 r + {0..3} of segment j
+      const uint2 o0 = make_uint2(pack_bf16(Y0[0], Y0[1]), pack_bf16(Y0[2], Y0[3]));
+      const uint2 o1 = make_uint2(pack_bf16(Y1[0], Y1[1]), pack_bf16(Y1[2], Y1[3]));
+      *(uint2*)(row + (((4 * t + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) = o0;
+      *(uint2*)(row + (((4 * t + 2 + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) = o1;
+    }
+  };
+
+  MEGA_FTR(5);
+#ifdef MEGA_X_ONEWAVE
+  if (wave < 4)
+#endif
+  {
+#pragma unroll
+    for (int i = 0; i < kFCPW; ++i) {
+      pass1(wave + kFW * i, i + 1 < kFCPW ? wave + kFW * (i + 1) : -1, img_set[i & 1], img_set[(i + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      MEGA_FTR(6 + i);
+    }
+  }
+  if (!last_block) {
+    // the wave's four channels x 16 states x (re, im) = 128 words: two per lane
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    const int cp = wave + kFW * (lane >> 4);
+    const float2 v = *(const float2*)(s_end + (cp * kNS + (lane & 15)) * 2);
+    unsigned long long* e = myrec + 4 + ((size_t)cp * kNS + (lane & 15)) * 2;
+    put_rec(e, tagged(__float_as_uint(v.x), tag));
+    put_rec(e + 1, tagged(__float_as_uint(v.y), tag));
+  }
+  if (LOUT == 0 && nterms == 0) {                    // nothing comes in from earlier blocks: y is final
+#pragma unroll
+    for (int i = 0; i < kFCPW; ++i) store_row(wave + kFW * i);
+  }
+
+  if (nterms > 0) {
+    // ---- start state of the block: h_start = sum_{d >= 0} (q^1024)^d E_{s-1-d} (+ (q^1024)^s h_in).  Lane (j, r)
+    // works for channel wave + 16 (j >> 2) and takes the terms d = (j & 3) + 4 k; the four lanes of a quad add up.
+    // the operands of pass 2's first channel are requested before the wait for the earlier blocks
+    auto load2 = [&](const int c, bf16x8 (&Cw)[kNWC][2], float (&Jr)[4], float (&Ji)[4]) {
+      const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+      uint32_t loff = loff0;
+      asm volatile("" : "+v"(loff));
+#pragma unroll
+      for (int w = 0; w < kNWC; ++w)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
+      load_c4(img, kSlotRJ, loff, Jr, Ji);
+    };
+    bf16x8 Cn[kNWC][2];
+    float Jnr[4], Jni[4];
+    load2(wave, Cn, Jnr, Jni);
+    float Cr[4] = {0.f, 0.f, 0.f, 0.f}, Ci[4] = {0.f, 0.f, 0.f, 0.f};
+    {
+      const int cl = wave + kFW * (j >> 2);
+      const int chl = g * kFC + cl;
+      const char* wimg = (const char*)A.image + (size_t)chl * kImgRowBytes;
+      for (int d0 = 0; d0 < nterms; d0 += 4) {
+        const int d = d0 + (j & 3);
+        const bool have = d < nterms;
+        const bool from_state = d == s;              // the caller's carried state enters behind block 0
+        const bool from_rec = have && !from_state;
+        const unsigned long long* e =
+            A.rec + (brow * A.S + (from_rec ? s - 1 - d : 0)) * kFRecW + 4 + (size_t)cl * kNS * 2 + 4 * r;
+        float Wr[4], Wi[4];
+        load_c4(wimg, kSlotRWJ, (uint32_t)(((r << 4) | (have ? d : 0)) * 16), Wr, Wi);      // (q^1024)^d
+        unsigned long long w[8];
+        uint32_t spins = 0;
+        for (;;) {
+          bool ok = true;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {              // states (2r, 2r+1) and (8+2r, 9+2r): two runs of four words
+            w[u] = from_rec ? get_rec(e + u) : tagged(0u, tag);
+            w[4 + u] = from_rec ? get_rec(e + 16 + u) : tagged(0u, tag);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) ok &= (uint32_t)(w[u] >> 32) == tag;
+          if (__all(ok)) break;
+          if (++spins > kSpinLimit) {
+            poison = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+        float er[4], ei[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          er[u] = __uint_as_float((uint32_t)w[2 * u]);
+          ei[u] = __uint_as_float((uint32_t)w[2 * u + 1]);
+        }
+        if (have && from_state) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            er[u] = ei[u] = 0.f;
+            if (nn[u] < A.N) {
+              const size_t o = (((size_t)b * A.D + chl) * A.N + nn[u]) * 2;
+              er[u] = A.h_in[o];
+              ei[u] = A.is_complex ? A.h_in[o + 1] : 0.f;
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          Cr[u] = fmaf(Wr[u], er[u], fmaf(-Wi[u], ei[u], Cr[u]));
+          Ci[u] = fmaf(Wr[u], ei[u], fmaf(Wi[u], er[u], Ci[u]));
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        Cr[u] = group_sum<4>(Cr[u]);
+        Ci[u] = group_sum<4>(Ci[u]);
+      }
+      if (poison) {
+        Cr[0] = __builtin_nanf("");
+        if (lane == 0) publish_u32(&A.hdr->error, 1u);
+      }
+    }
+    MEGA_FTR(10);
+
+    // ---- pass 2: add C ((q^64)^j h_start) (one more factor q^32 for a segment's second tile) to y and send it out;
+    // the operands of the next channel travel under the current one
+#pragma unroll
+    for (int i = 0; i < kFCPW; ++i) {
+      const int c = wave + kFW * i;
+      const int ch = g * kFC + c;
+      const char* img = (const char*)A.image + (size_t)ch * kImgRowBytes;
+      uint32_t roff = roff0;
+      asm volatile("" : "+v"(roff));
+      bf16x8 Cw[kNWC][2];
+      float Qr[4], Qi[4], Jr[4], Ji[4], ar[4], ai[4], br[4], bi[4];
+#pragma unroll
+      for (int w = 0; w < kNWC; ++w)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = Cn[w][mb];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        Jr[u] = Jnr[u];
+        Ji[u] = Jni[u];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (i + 1 < kFCPW) load2(wave + kFW * (i + 1), Cn, Jnr, Jni);
+      __builtin_amdgcn_sched_barrier(0);
+      lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {                  // the quad i of every row holds this channel's start state
+        br[u] = lane_bcast(Cr[u], (lane & 48) | (4 * i));
+        bi[u] = lane_bcast(Ci[u], (lane & 48) | (4 * i));
+        ar[u] = Jr[u] * br[u] - Ji[u] * bi[u];
+        ai[u] = Jr[u] * bi[u] + Ji[u] * br[u];
+      }
+      char* row = tile + row_base(c) + j * 128;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        bf16x8 Hop;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          Hop[2 * u] = (__bf16)ar[u];
+          Hop[2 * u + 1] = (__bf16)ai[u];
+        }
+        f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < kNWC; ++w) {
+          Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop, Y0, 0, 0, 0);
+          Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop, Y1, 0, 0, 0);
+        }
+        if (t == 0) {
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const float nr = Qr[u] * ar[u] - Qi[u] * ai[u];
+            ai[u] = Qr[u] * ai[u] + Qi[u] * ar[u];
+            ar[u] = nr;
+          }
+        }
+        uint2* p0 = (uint2*)(row + (((4 * t + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8);
+        uint2* p1 = (uint2*)(row + (((4 * t + 2 + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8);
+        const uint2 a0 = *p0, a1 = *p1;
+        *p0 = make_uint2(pack_bf16(Y0[0] + __uint_as_float(a0.x << 16), Y0[1] + __uint_as_float(a0.x & 0xffff0000u)),
+                         pack_bf16(Y0[2] + __uint_as_float(a0.y << 16), Y0[3] + __uint_as_float(a0.y & 0xffff0000u)));
+        *p1 = make_uint2(pack_bf16(Y1[0] + __uint_as_float(a1.x << 16), Y1[1] + __uint_as_float(a1.x & 0xffff0000u)),
+                         pack_bf16(Y1[2] + __uint_as_float(a1.y << 16), Y1[3] + __uint_as_float(a1.y & 0xffff0000u)));
+      }
+      if (last_block && A.h_out && j == 15) {
+        // state after the block's last token: end state from a zero start + (q^1024) h_start
+        float Rr[4], Ri[4];
+        load_cmp(img, kCmpRW, roff, Rr, Ri);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (nn[u] < A.N) {
+            const float er = s_end[(c * kNS + nn[u]) * 2], ei = s_end[(c * kNS + nn[u]) * 2 + 1];
+            const size_t o = (((size_t)b * A.D + ch) * A.N + nn[u]) * 2;
+            A.h_out[o] = fmaf(Rr[u], br[u], fmaf(-Ri[u], bi[u], er));
+            A.h_out[o + 1] = fmaf(Rr[u], bi[u], fmaf(Ri[u], br[u], ei));
+          }
+        }
+      }
+      if (LOUT == 0) store_row(c);
+      __builtin_amdgcn_sched_barrier(0);
+      MEGA_FTR(11 + i);
+    }
+  } else if (last_block && A.h_out && j == 15) {
+    // a single block without a carried state: its end state from a zero start is the state to return
+#pragma unroll
+    for (int i = 0; i < kFCPW; ++i) {
+      const int c = wave + kFW * i;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (nn[u] < A.N) {
+          const size_t o = (((size_t)b * A.D + g * kFC + c) * A.N + nn[u]) * 2;
+          A.h_out[o] = s_end[(c * kNS + nn[u]) * 2];
+          A.h_out[o + 1] = s_end[(c * kNS + nn[u]) * 2 + 1];
+        }
+      }
+    }
+  }
+  if (LOUT == 1) {
+    // [B, L, D]: the inverse of the staging step, whole lines of 64 channels per token
+    __syncthreads();
+    const int odd = tokl & 1;
+    const uint32_t sel_keep = odd ? 0x07060302u : 0x05040100u;
+    const uint32_t sel_give = odd ? 0x05040100u : 0x07060302u;
+    const int tl = tokl & ~1;
+    const char* rbase = tile + row_base(piece * 8 + odd * 4) + (tl >> 6) * 128 + ((tl & 7) >> 1) * 4;
+    const int c8 = (tl & 63) >> 3;
+    bf16_t* yb = A.y + (size_t)b * A.syb + (size_t)(g * kFC + piece * 8) * A.syd;
+#pragma unroll
+    for (int k = 0; k < kFNLD; ++k) {
+      const int tok = k * 128 + tokl;
+      const char* rp = rbase + (2 * k) * 128 + ((c8 ^ k) << 4);
+      uint32_t w[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = *(const uint32_t*)(rp + e * kFRow);
+      const uint32_t keep0 = __builtin_amdgcn_perm(w[1], w[0], sel_keep);
+      const uint32_t keep1 = __builtin_amdgcn_perm(w[3], w[2], sel_keep);
+      const uint32_t got0 = dpp_u<0x128>(__builtin_amdgcn_perm(w[1], w[0], sel_give));
+      const uint32_t got1 = dpp_u<0x128>(__builtin_amdgcn_perm(w[3], w[2], sel_give));
+      uint4 o;
+      o.x = odd ? got0 : keep0;
+      o.y = odd ? got1 : keep1;
+      o.z = odd ? keep0 : got0;
+      o.w = odd ? keep1 : got1;
+      store_stream((uint4*)(yb + (size_t)(t0 + tok) * A.syl), o);
+    }
+  }
+
+  MEGA_FTR_END();
+  // ---- retire: the last workgroup to finish opens the next epoch
+  if (tid == 0) {
+    const uint32_t total = gridDim.x;
+    const uint32_t k = blockIdx.x & 31u;
+    const uint32_t quota = (total - k + 31u) / 32u;
+    if (atomicAdd(&A.hdr->done1[k], 1u) == quota - 1u) {
+      publish_u32(&A.hdr->done1[k], 0u);
+      const uint32_t classes = total < 32u ? total : 32u;
+      if (atomicAdd(&A.hdr->done2, 1u) == classes - 1u) {
+        publish_u32(&A.hdr->done2, 0u);
+        publish_u32(&A.hdr->epoch, tag == 0xffffffffu ? 0u : tag);
+      }
+    }
+  }
+}
+
+size_t fused_ws_bytes(int64_t B, int64_t G, int64_t S) {
+  return align_up(sizeof(TsnHeader), 256) + align_up((size_t)B * G * S * kFRecW * 8, 256);
+}
+
+bool fused_covers(int dtype, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N, const void* x, const void* xn,
+                  const void* y, int64_t syb, int64_t syd, int64_t syl, const uint8_t* mask, const float* h_in) {
+  if (dtype != MEGA_BF16 || mask || G <= 0 || D != G * kFC || N > kNS || N <= 0) return false;
+  if (L <= 0 || L % kFSeg != 0 || L / kFSeg + (h_in ? 1 : 0) > kFMaxBlocks) return false;
+  if (((uintptr_t)x % 16) || ((uintptr_t)xn % 16) || ((uintptr_t)y % 16)) return false;
+  const bool rows = syl == 1 && syd % 8 == 0 && syb % 8 == 0;
+  const bool lines = syd == 1 && syl % 8 == 0 && syb % 8 == 0;
+  if (!rows && !lines) return false;
+  if (B * G * (L / kFSeg) >= (int64_t)1 << 31) return false;
+  return true;
+}
+
+}  // namespace
+}  // namespace mega
+
+using namespace mega;
+
+// workspace (zero once, then owned by these calls): launch header + the records of whichever route a shape takes
+extern "C" size_t mega_norm_ema_fwd_workspace_bytes(int64_t B, int64_t L, int64_t D, int64_t G, int64_t N) {
+  (void)N;
+  if (B <= 0 || L <= 0 || D <= 0 || G <= 0) return 256;
+  const size_t fused = fused_ws_bytes(B, G, ceil_div(L, kFSeg));
+  const size_t tsn = mega_timestep_norm_workspace_bytes(MEGA_BF16, B, L, D, G);
+  return fused > tsn ? fused : tsn;
+}
+
+// scratch (no initialisation, contents never survive a call): the moving average's own workspace when the two
+// operators run one after the other, or room for kernel generation when no image is passed
+extern "C" size_t mega_norm_ema_fwd_scratch_bytes(int64_t B, int64_t L, int64_t D, int64_t G, int64_t N) {
+  (void)G;
+  if (B <= 0 || L <= 0 || D <= 0 || N <= 0) return 256;
+  const size_t ema = mega_ema_fwd_workspace_bytes(B, D, N, L, 0, 0);
+  const size_t img = mega_ema_image_bytes(D, N, 0);
+  return align_up(ema > img ? ema : img, 256);
+}
+
+extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd, int64_t syl,
+                                 const int64_t* prev_count, const float* prev_mean, const float* prev_var,
+                                 const float* norm_gamma, const float* norm_beta, const uint8_t* mask, double eps,
+                                 int64_t* count, float* mean, float* var, const float* p, const float* q,
+                                 const float* gamma, int is_complex, const float* omega, const float* h_in,
+                                 float* h_out, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N,
+                                 const void* image, void* workspace, size_t workspace_bytes, void* scratch,
+                                 size_t scratch_bytes, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "norm_ema_fwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && L >= 0 && D > 0 && G > 0 && N > 0 && D % G == 0, MEGA_ERR_ARG,
+               "norm_ema_fwd: bad shape B=%ld L=%ld D=%ld G=%ld N=%ld", (long)B, (long)L, (long)D, (long)G, (long)N);
+  if (B == 0) return MEGA_OK;
+  const size_t need = mega_norm_ema_fwd_workspace_bytes(B, L > 0 ? L : 1, D, G, N);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need, MEGA_ERR_WORKSPACE, "norm_ema_fwd: workspace of %zu bytes needed",
+               need);
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t S = ceil_div(L > 0 ? L : 1, kFSeg);
+  char* w = (char*)workspace;
+  const bool one_kernel = L > 0 && (image || mega_ema_image_bytes(D, N, 0) > 0) &&
+                          fused_covers(dtype, B, L, D, G, N, x, xn, y, syb, syd, syl, mask, h_in);
+  if (!one_kernel || !image) {
+    const size_t sneed = mega_norm_ema_fwd_scratch_bytes(B, L > 0 ? L : 1, D, G, N);
+    MEGA_REQUIRE(scratch && scratch_bytes >= sneed, MEGA_ERR_WORKSPACE, "norm_ema_fwd: scratch of %zu bytes needed",
+                 sneed);
+  }
+  if (one_kernel) {
+    MEGA_REQUIRE(x && xn && y && prev_count && prev_mean && prev_var && norm_gamma && norm_beta && count && mean &&
+                     var && p && q && gamma && omega,
+                 MEGA_ERR_ARG, "norm_ema_fwd: null pointer argument");
+    MEGA_REQUIRE(!ranges_overlap(prev_count, (size_t)B * 8, count, (size_t)B * 8) &&
+                     !ranges_overlap(prev_mean, (size_t)B * G * 4, mean, (size_t)B * G * 4) &&
+                     !ranges_overlap(prev_var, (size_t)B * G * 4, var, (size_t)B * G * 4),
+                 MEGA_ERR_ARG, "norm_ema_fwd: count / mean / var must not overlap prev_count / prev_mean / prev_var");
+    MEGA_REQUIRE(!h_in || !h_out || !ranges_overlap(h_in, (size_t)B * D * N * 8, h_out, (size_t)B * D * N * 8),
+                 MEGA_ERR_ARG, "norm_ema_fwd: h_out must not overlap h_in (every block reads h_in, the last writes h_out)");
+    const void* img = image;
+    if (!img) {
+      // no cached image: kernel generation runs with every call
+      const int rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, 0, 1, scratch, s);
+      if (rc) return rc;
+      img = scratch;
+    }
+    FusedArgs A;
+    A.x = (const bf16_t*)x; A.xn = (bf16_t*)xn; A.y = (bf16_t*)y; A.syb = syb; A.syd = syd; A.syl = syl;
+    A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var; A.count = count; A.mean = mean;
+    A.var = var; A.gamma = norm_gamma; A.beta = norm_beta; A.image = (const uint4*)img; A.h_in = h_in; A.h_out = h_out;
+    A.hdr = (TsnHeader*)w; A.rec = (unsigned long long*)(w + align_up(sizeof(TsnHeader), 256));
+    A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
+    A.is_complex = is_complex;
+    A.xcd_map = (G % 8 == 0) ? 1 : 0;
+    const dim3 grid((unsigned)(B * G * S));
+    typedef void (*Kern)(const FusedArgs);
+    const int lout = syl == 1 ? 0 : 1;
+    const Kern kern = lout == 0 ? norm_ema_fused_kernel<0> : norm_ema_fused_kernel<1>;
+    static bool attr_set[2] = {false, false};
+    if (!attr_set[lout]) {
+      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFSmem);
+      attr_set[lout] = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(kFT), kFSmem, s, A);
+    MEGA_CHECK_LAUNCH("norm_ema_fwd");
+    return MEGA_OK;
+  }
+  // outside the one-kernel envelope: the two operators one after the other
+  // (x -> xn by the norm, xn read through its transposed view by the moving average); the norm keeps its
+  // launch header and tile records in the same workspace (same header, same protocol)
+  int rc = mega_group_timestep_norm_fwd(x, xn, dtype, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, mask, B, L,
+                                        D, G, eps, count, mean, var, nullptr, nullptr, nullptr, workspace,
+                                        workspace_bytes, stream);
+  if (rc) return rc;
+  return mega_ema_fwd(xn, y, dtype, L * D, 1, D, syb, syd, syl, p, q, gamma, is_complex, omega, mask, h_in, h_out, B, D,
+                      N, L, 0, 0, 1, image, scratch, scratch_bytes, stream);
+}

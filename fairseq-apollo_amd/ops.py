@@ -591,6 +591,63 @@ class PreparedEMA:
         return y, hc
 
 
+    def norm_forward(self, x: torch.Tensor, prev_count, prev_mean, prev_var, norm_gamma, norm_beta,
+                     num_groups: int, eps: float, padding_mask: Optional[torch.Tensor] = None,
+                     h: Optional[torch.Tensor] = None, want_state: bool = False, out_layout: str = "rows"):
+        """TimestepNorm followed by this layer in one call (moving_average_gated_attention.py:304-315:
+        x = norm(x); mx = move(x^T)).  x: [B, L, D].  -> (xn [B, L, D], y, count, mean, var, h_out); y is a
+        contiguous [B, D, L] tensor (out_layout "rows", what the reference's convolution returns) or a
+        [B, D, L] view of [B, L, D] memory (out_layout "input").  Covered shapes run as one kernel, the
+        rest as the two operators one after the other (mega_norm_ema_fwd)."""
+        dev = self.dev
+        _need_gpu(x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, padding_mask, h)
+        if self.bidirectional or self.trunc:
+            raise RuntimeError("norm_forward: one-sided layers without kernel truncation only")
+        lib = _lib.load()
+        if x.dim() != 3 or x.shape[2] != self.D:
+            raise RuntimeError(f"x must be [B, L, {self.D}]")
+        B, L, D = x.shape
+        G = int(num_groups)
+        if G <= 0 or D % G != 0:
+            raise RuntimeError(f"num_features={D} is not divisible by num_groups={G}")
+        xd = x if (x.is_contiguous() and not x.requires_grad) else x.detach().contiguous()
+        dt = _dtype_code(xd)
+        xn = torch.empty_like(xd)
+        if out_layout == "rows":
+            y = torch.empty(B, D, L, dtype=xd.dtype, device=dev)
+        elif out_layout == "input":
+            y = torch.empty(B, L, D, dtype=xd.dtype, device=dev).transpose(1, 2)
+        else:
+            raise RuntimeError(f"out_layout must be 'rows' or 'input', got {out_layout!r}")
+        pc, pm, pv = _norm_state(prev_count, prev_mean, prev_var, B, G, dev)
+        count = torch.empty(B, dtype=torch.int64, device=dev)
+        mean = torch.empty(B, G, dtype=torch.float32, device=dev)
+        var = torch.empty(B, G, dtype=torch.float32, device=dev)
+        N = self.N
+        hin = None if h is None else _cplx_as_f32(h.reshape(B, D, N))
+        hout = torch.empty(B, D, N, 2, dtype=torch.float32, device=dev) if (want_state or h is not None) else None
+        key = ("norm_ema", B, L, D, G, N)
+        sizes = _ws_bytes_cache.get(key)
+        if sizes is None:
+            sizes = _ws_bytes_cache[key] = (lib.mega_norm_ema_fwd_workspace_bytes(B, L, D, G, N),
+                                            lib.mega_norm_ema_fwd_scratch_bytes(B, L, D, G, N))
+        stream = _stream(dev)
+        ws = _tsn_workspace(dev, sizes[0], stream)
+        sc = _scratch_buffer(dev, sizes[1], stream)
+        m8 = _mask_u8(padding_mask, B, L)
+        gf, bf = _f32c(norm_gamma), _f32c(norm_beta)
+        with _on_device(dev):
+            rc = lib.mega_norm_ema_fwd(_ptr(xd), _ptr(xn), _ptr(y), dt, y.stride(0), y.stride(1), y.stride(2),
+                                       _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf), _ptr(m8), float(eps),
+                                       _ptr(count), _ptr(mean), _ptr(var), _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
+                                       1 if self.is_complex else 0, _ptr(self.omega), _ptr(hin), _ptr(hout), B, L, D, G,
+                                       N, _ptr(self.image), _ptr(ws), ws.numel(), _ptr(sc), sc.numel(), stream)
+        _lib.check(rc, "norm_ema_fwd")
+        hc = None
+        if hout is not None:
+            hc = torch.view_as_complex(hout) if self.is_complex else hout[..., 0]
+        return xn, y, count, mean, var, hc
+
     def adjoint(self, y_grad: torch.Tensor, padding_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Gradient of the layer output with respect to its input x:
         dx[t] = (1 - mask[t]) sum_s k(s - t) dy[s] + omega dy[t], the same layer (one- or two-sided)

@@ -156,6 +156,36 @@ int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_
                        int is_complex, const float* omega, const float* h_in, float* h_out,
                        int64_t B, int64_t D, int64_t G, int64_t N, void* stream);
 
+/* TimestepNorm followed by the moving-average layer in one call: what
+ * MovingAverageGatedAttention.forward does with x at
+ * fairseq/modules/moving_average_gated_attention.py:304-315 (x = norm(x), then
+ * mx = move(x^T)), i.e. mega_group_timestep_norm_fwd (x -> xn, [B,L,D]) followed by
+ * mega_ema_fwd on the transposed view of xn (-> y).  xn is an output too: the layer also
+ * feeds it to v_proj.
+ *   x, xn      [B,L,D] contiguous of `dtype`; y of `dtype` with element strides
+ *              (syb, syd, syl) over (batch, channel, time): [B,D,L] rows, which is what the
+ *              reference's convolution returns, or [B,L,D]
+ *   norm state / parameters / mask as mega_group_timestep_norm_fwd (norm_gamma = weight + 1);
+ *   moving-average coefficients, h_in / h_out and `image` as mega_ema_fwd (unidirectional,
+ *   no truncation); h_out must not overlap h_in.
+ * bf16 activations with 64 channels per norm group (D = 64 G), ndim <= 16, no mask, L a
+ * multiple of 1024 with L / 1024 (+ 1 with h_in) <= 16 run as ONE kernel that reads x once and
+ * writes xn and y once; everything else runs the two operators one after the other.
+ * `workspace` (launch epoch, block / tile records) must be zero-filled once and then belongs to
+ * these calls, exactly like the TimestepNorm workspace (the two may be the same buffer);
+ * `scratch` needs no initialisation and is used only when the two operators run one after the
+ * other or when image == NULL (kernel generation inside the call).                          */
+size_t mega_norm_ema_fwd_workspace_bytes(int64_t B, int64_t L, int64_t D, int64_t G, int64_t N);
+size_t mega_norm_ema_fwd_scratch_bytes(int64_t B, int64_t L, int64_t D, int64_t G, int64_t N);
+int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd,
+                      int64_t syl, const int64_t* prev_count, const float* prev_mean,
+                      const float* prev_var, const float* norm_gamma, const float* norm_beta,
+                      const uint8_t* mask, double eps, int64_t* count, float* mean, float* var,
+                      const float* p, const float* q, const float* gamma, int is_complex,
+                      const float* omega, const float* h_in, float* h_out, int64_t B, int64_t L,
+                      int64_t D, int64_t G, int64_t N, const void* image, void* workspace,
+                      size_t workspace_bytes, void* scratch, size_t scratch_bytes, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Moving-average backward (unidirectional, no carried state)                  */
 /* The input gradient is the same layer run backwards in time: call mega_ema_fwd with
