@@ -10,6 +10,8 @@ namespace mega {
 // for the four states (2r, 2r+1, 8+2r, 9+2r) as (re, im) pairs, two slots each:
 //   kSlotQ32  q^32      kSlotRS  q^64      kSlotRJ  (q^64)^j      kSlotRW  q^1024      kSlotRWJ  (q^1024)^j
 // and one slot in the layout of the 64-lane segment scan (kSlotScan: q^(32 kSEGT) of state lane >> 2).
+// kSlotKT (kNWK slots): the K operand once per distinct content, 56 vectors of 16 bytes per term; lane (m, g) of
+// row block mb finds its vector at byte 16 (16 mb + m - 8 g + 24).
 constexpr int kNS = 16;                  // complex states per channel (zero padded)
 #ifndef MEGA_SEGT
 #define MEGA_SEGT 2
@@ -30,10 +32,13 @@ constexpr int kNWC = MEGA_NWC;           // bf16 terms of the state-output opera
 constexpr int kNOPS = 2 * (kNWK + kNWP + kNWC);
 constexpr int kSlotK = 0, kSlotP = 2 * kNWK, kSlotC = 2 * (kNWK + kNWP);
 constexpr int kSlotQ32 = kNOPS, kSlotScan = kNOPS + 2, kSlotRS = kNOPS + 3, kSlotRJ = kNOPS + 5, kSlotRW = kNOPS + 7,
-              kSlotRWJ = kNOPS + 9, kSlotCmp = kNOPS + 11;
-constexpr int kImgSlots = kNOPS + 12;
+              kSlotRWJ = kNOPS + 9, kSlotCmp = kNOPS + 11, kSlotKT = kNOPS + 12;
+constexpr int kImgSlots = kNOPS + 12 + kNWK;
 // kSlotCmp: per-state multipliers once each, six tables of 16 complex values (128 bytes = one line):
-enum { kCmpQ32 = 0, kCmpRS = 1, kCmpRS2 = 2, kCmpRS4 = 3, kCmpRS8 = 4, kCmpRW = 5 };
+// and one line of reach figures (how far the slowest pole of the channel carries before |q|^t < 2^-24):
+//   word 0: how many of the doubling steps 64, 128, 256, 512 tokens still matter (0..4)
+//   word 1: how many blocks of 1024 tokens back a block has to look (1..16)
+enum { kCmpQ32 = 0, kCmpRS = 1, kCmpRS2 = 2, kCmpRS4 = 3, kCmpRS8 = 4, kCmpRW = 5, kCmpReach = 6 };
 constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
 
 // bytes of the per-channel operand images for a layer (0: the layer is outside the fast path)

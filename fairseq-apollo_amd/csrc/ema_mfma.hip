@@ -242,6 +242,50 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       v = cmul(v, v);
       cmp[kCmpRW * kNS + lane] = make_float2(v.re, v.im);
     }
+    if (lane < 56) {
+      // the K operand once per distinct content: lane (m, g) of row block mb holds k[16 mb + m - 8 g - t], t = 0..7,
+      // which depends on delta = 16 mb + m - 8 g (-24..31) only; vector delta + 24 of term w sits at byte
+      // 16 (delta + 24) of slot kSlotKT + w (7 lines per term instead of 16)
+      const int delta = lane - 24;
+#pragma unroll
+      for (int w = 0; w < kNWK; ++w) {
+        bf16x8 v;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          __bf16 h;
+          const float rem = bf_split(kkt[32 + delta - t], &h);
+          v[t] = w == 0 ? h : (__bf16)rem;
+        }
+        img[(size_t)(kSlotKT + w) * 64 + lane] = __builtin_bit_cast(uint4, v);
+      }
+    }
+    {
+      // reach of the channel's slowest pole: m = max |q|^64; a contribution over t tokens is dropped by the
+      // streaming kernels once |q|^t < 2^-24 (below fp32 resolution of what it is added to)
+      const float2 w32 = pw[32 * kNS + (lane & 15)];
+      float m = w32.x * w32.x + w32.y * w32.y;             // |q^32|^2 = |q|^64
+#pragma unroll
+      for (int o = 8; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      const float lim = 0x1p-24f;
+      float md = m;
+      int nsteps = 0;
+      for (int t = 0; t < 4; ++t) {                         // |q|^(64 d) for d = 1, 2, 4, 8
+        if (md >= lim) nsteps = t + 1;
+        md *= md;
+      }
+      // md = |q|^1024 now
+      int nlook = 1;
+      float w = md;
+      while (nlook < 16 && w >= lim) {
+        w *= md;
+        ++nlook;
+      }
+      if (lane == 0) {
+        uint32_t* rw = (uint32_t*)(img + (size_t)kSlotCmp * 64) + kCmpReach * kNS * 2;
+        rw[0] = (uint32_t)nsteps;
+        rw[1] = (uint32_t)nlook;
+      }
+    }
   }
 }
 

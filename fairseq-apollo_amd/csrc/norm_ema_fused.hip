@@ -346,6 +346,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 
   // the operands of the wave's first channel travel under the normalisation
   const uint32_t loff0 = (uint32_t)lane * 16;
+  const uint32_t koff0 = (uint32_t)(((lane & 15) - 8 * (lane >> 4) + 24) * 16);
   // the P operand of channel c (requested one channel ahead)
   auto load_p = [&](const int c, ImgSet& I) {
     const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
@@ -360,10 +361,14 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
+    // K from the slot that holds each distinct vector once: 7 lines per term leave the cache instead of 16
+    uint32_t koff = koff0;
+    asm volatile("" : "+v"(koff));
 #pragma unroll
     for (int w = 0; w < kNWK; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) I.K[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotK + 2 * w + mb, loff));
+      for (int mb = 0; mb < 2; ++mb)
+        I.K[w][mb] = __builtin_bit_cast(bf16x8, *(const uint4*)(img + (kSlotKT + w) * 1024 + mb * 256 + koff));
 #pragma unroll
     for (int w = 0; w < kNWC; ++w)
 #pragma unroll
@@ -397,9 +402,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         const float hi = fmaf(__uint_as_float(w[i] & 0xffff0000u), r, -mr);
         o[i] = pack_bf16(fmaf(lo, gam[2 * i], bet[2 * i]), fmaf(hi, gam[2 * i + 1], bet[2 * i + 1]));
       }
-#ifndef MEGA_X_NOXN
       store_stream((uint4*)(A.xn + xblk + (size_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
-#endif
       const uint32_t s0 = odd ? o[0] : o[2], s1 = odd ? o[1] : o[3];
       const uint32_t r0 = dpp_u<0x128>(s0), r1 = dpp_u<0x128>(s1);       // row_ror:8 = the partner token's lane
       const uint32_t m0 = odd ? o[2] : o[0], m1 = odd ? o[3] : o[1];
@@ -418,12 +421,17 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   const int j = lane & 15, r = lane >> 4;
   const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
   const bool last_block = s == A.S - 1;
-#ifdef MEGA_X_ONEWAVE
-  const int nterms = 0;
-#else
   const int nterms = s + (A.h_in ? 1 : 0);
-#endif
   const uint32_t roff0 = (uint32_t)r * 16;
+  // how far the channels' slowest poles reach (figures of the operand image, uniform per wave and channel)
+  int nsteps[kFCPW], nlook[kFCPW];
+#pragma unroll
+  for (int i = 0; i < kFCPW; ++i) {
+    const uint2 rw = *(const uint2*)((const char*)A.image + (size_t)(g * kFC + wave + kFW * i) * kImgRowBytes +
+                                     kSlotCmp * 1024 + kCmpReach * 128);
+    nsteps[i] = __builtin_amdgcn_readfirstlane((int)rw.x);
+    nlook[i] = __builtin_amdgcn_readfirstlane((int)rw.y);
+  }
 
   // the wave's own row leaves as whole lines ([B, D, L] rows)
   auto store_row = [&](const int c) {
@@ -445,7 +453,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   // pass 1 over channel c, everything that does not need the earlier blocks: end states of the 16 segments
   // from a zero start (P products), scanned across the row; the block's end state from a zero start is
   // published; y = K x + C (segment start state from a zero block start) goes back into LDS over x as bf16
-  auto pass1 = [&](const int c, const int cnext, ImgSet& cur, ImgSet& nxt) {
+  auto pass1 = [&](const int c, const int cnext, const int steps, ImgSet& cur, ImgSet& nxt) {
     uint32_t roff = roff0;
     asm volatile("" : "+v"(roff));
     float Qr[4], Qi[4];
@@ -479,19 +487,25 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     __builtin_amdgcn_sched_barrier(0);
     if (cnext >= 0) load_p(cnext, nxt);
     __builtin_amdgcn_sched_barrier(0);
-#ifndef MEGA_X_NOSCAN
-    {
+    // inclusive scan over the 16 segments by doubling; a step over d segments is skipped (uniform branch) when
+    // |q|^(64 d) < 2^-24 for every state of the channel: what it would add is below fp32 resolution
+    if (steps > 0) {
       float Rr[4], Ri[4], R2r[4], R2i[4];
       lds_cmp(s_tab, kCmpRS, c, roff, Rr, Ri);
       scan_step<0x111>(Er, Ei, Rr, Ri);
-      csquare(Rr, Ri, R2r, R2i);
-      scan_step<0x112>(Er, Ei, R2r, R2i);
-      csquare(R2r, R2i, Rr, Ri);
-      scan_step<0x114>(Er, Ei, Rr, Ri);
-      csquare(Rr, Ri, R2r, R2i);
-      scan_step<0x118>(Er, Ei, R2r, R2i);
+      if (steps > 1) {
+        csquare(Rr, Ri, R2r, R2i);
+        scan_step<0x112>(Er, Ei, R2r, R2i);
+        if (steps > 2) {
+          csquare(R2r, R2i, Rr, Ri);
+          scan_step<0x114>(Er, Ei, Rr, Ri);
+          if (steps > 3) {
+            csquare(Rr, Ri, R2r, R2i);
+            scan_step<0x118>(Er, Ei, R2r, R2i);
+          }
+        }
+      }
     }
-#endif
     MEGA_FTR2(1);
     // lane 15 of a row holds the block's end state from a zero start: parked in LDS, published for the later
     // blocks after the wave's last channel (and kept for the carried state the last block returns)
@@ -549,13 +563,10 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   };
 
   MEGA_FTR(5);
-#ifdef MEGA_X_ONEWAVE
-  if (wave < 4)
-#endif
   {
 #pragma unroll
     for (int i = 0; i < kFCPW; ++i) {
-      pass1(wave + kFW * i, i + 1 < kFCPW ? wave + kFW * (i + 1) : -1, img_set[i & 1], img_set[(i + 1) & 1]);
+      pass1(wave + kFW * i, i + 1 < kFCPW ? wave + kFW * (i + 1) : -1, nsteps[i], img_set[i & 1], img_set[(i + 1) & 1]);
       __builtin_amdgcn_sched_barrier(0);
       MEGA_FTR(6 + i);
     }
@@ -579,7 +590,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     // ---- start state of the block: h_start = sum_{d >= 0} (q^1024)^d E_{s-1-d} (+ (q^1024)^s h_in).  Lane (j, r)
     // works for channel wave + 16 (j >> 2) and takes the terms d = (j & 3) + 4 k; the four lanes of a quad add up.
     // the operands of pass 2's first channel are requested before the wait for the earlier blocks
-    auto load2 = [&](const int c, bf16x8 (&Cw)[kNWC][2], float (&Jr)[4], float (&Ji)[4]) {
+    auto load2 = [&](const int c, const int steps, bf16x8 (&Cw)[kNWC][2], float (&Jr)[4], float (&Ji)[4]) {
       const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
       uint32_t loff = loff0;
       asm volatile("" : "+v"(loff));
@@ -587,19 +598,26 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       for (int w = 0; w < kNWC; ++w)
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
-      load_c4(img, kSlotRJ, loff, Jr, Ji);
+      if (steps > 1) load_c4(img, kSlotRJ, loff, Jr, Ji);      // else (q^64)^j is 1, q^64, then nothing
     };
     bf16x8 Cn[kNWC][2];
-    float Jnr[4], Jni[4];
-    load2(wave, Cn, Jnr, Jni);
+    float Jnr[4] = {0.f, 0.f, 0.f, 0.f}, Jni[4] = {0.f, 0.f, 0.f, 0.f};
+    load2(wave, nsteps[0], Cn, Jnr, Jni);
     float Cr[4] = {0.f, 0.f, 0.f, 0.f}, Ci[4] = {0.f, 0.f, 0.f, 0.f};
     {
       const int cl = wave + kFW * (j >> 2);
       const int chl = g * kFC + cl;
+      int look = 0;                                  // blocks back that still reach this lane's channel
+#pragma unroll
+      for (int i = 0; i < kFCPW; ++i) look = (j >> 2) == i ? nlook[i] : look;
       const char* wimg = (const char*)A.image + (size_t)chl * kImgRowBytes;
-      for (int d0 = 0; d0 < nterms; d0 += 4) {
+      int maxlook = 0;
+#pragma unroll
+      for (int i = 0; i < kFCPW; ++i) maxlook = nlook[i] > maxlook ? nlook[i] : maxlook;
+      const int nrounds = nterms < maxlook ? nterms : maxlook;
+      for (int d0 = 0; d0 < nrounds; d0 += 4) {
         const int d = d0 + (j & 3);
-        const bool have = d < nterms;
+        const bool have = d < nterms && d < look;
         const bool from_state = d == s;              // the caller's carried state enters behind block 0
         const bool from_rec = have && !from_state;
         const unsigned long long* e =
@@ -680,9 +698,18 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         Ji[u] = Jni[u];
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (i + 1 < kFCPW) load2(wave + kFW * (i + 1), Cn, Jnr, Jni);
+      if (i + 1 < kFCPW) load2(wave + kFW * (i + 1), nsteps[i + 1 < kFCPW ? i + 1 : i], Cn, Jnr, Jni);
       __builtin_amdgcn_sched_barrier(0);
       lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
+      if (nsteps[i] <= 1) {                          // |q|^128 < 2^-24: the start state reaches two segments
+        float Sr[4], Si[4];
+        lds_cmp(s_tab, kCmpRS, c, roff, Sr, Si);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          Jr[u] = j == 0 ? 1.f : (j == 1 ? Sr[u] : 0.f);
+          Ji[u] = j == 1 ? Si[u] : 0.f;
+        }
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {                  // the quad i of every row holds this channel's start state
         br[u] = lane_bcast(Cr[u], (lane & 48) | (4 * i));
