@@ -4,11 +4,13 @@ bf16 activations, fp32 parameters and accumulation, on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step = one forward of the block over one batch of synthetic input that already sits in
-HBM: xn = TimestepNorm(x) ([B, L, D], 16 groups), y = CEMA(xn^T): xn is read in place through the
-transposed view the layer passes, y is the contiguous [B, D, L] tensor the reference's
-convolution returns.  Inputs rotate over several buffers so that a step never finds its
-input in the 256 MB last-level cache.  Prints one JSON line (tokens/s of the whole job), with
-the HBM roofline of the dominant kernel and the CPU oracle timed on the host cores beside it.
+HBM: xn = TimestepNorm(x) ([B, L, D], 16 groups), y = CEMA(xn^T), both results written (the layer
+needs xn for its value projection), y as the contiguous [B, D, L] tensor the reference's convolution
+returns.  The timed step is one library call (one kernel); the same block as two module calls and
+the step with the kernel generation inside the call are timed beside it.  Inputs rotate over several
+buffers so that a step never finds its input in the 256 MB last-level cache.  Prints one JSON line
+(tokens/s of the whole job), with the HBM roofline of the dominant kernel and the CPU oracle timed
+on the host cores beside it.
 """
 import argparse
 import json
@@ -88,6 +90,19 @@ def measured_traffic():
     if os.path.exists(path):
         for m in re.finditer(r"^traffic_bytes_per_launch\s+(\S+)\s*=\s*(\d+)", open(path).read(), re.M):
             out[m.group(1)] = int(m.group(2))
+    return out
+
+
+def profiled_durations():
+    """Average kernel durations (ms) of the committed rocprofv3 --kernel-trace --stats summary of this
+    command: lines `avg_duration_us <kernel> = <microseconds>`."""
+    import re
+
+    out = {}
+    path = os.path.join(ROOT, "profiles", "ema_tsn_block_B4_L4096_D1024_bf16.txt")
+    if os.path.exists(path):
+        for m in re.finditer(r"^avg_duration_us\s+(\S+)\s*=\s*([0-9.]+)", open(path).read(), re.M):
+            out[m.group(1)] = float(m.group(2)) * 1e-3
     return out
 
 
@@ -439,8 +454,6 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--standalone", action="store_true",
-                    help="block workload: also time each operator alone, back to back on cold inputs")
     ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
@@ -487,32 +500,40 @@ def main():
     xs = [torch.randn(B, L, D, generator=gen, dtype=torch.float32).to(torch.bfloat16).to(dev) for _ in range(NBUF)]
 
     def step(i):
-        x = xs[i % NBUF]
-        xn = norm(x)
-        y = ema(xn.transpose(1, 2))
-        return xn, y
+        # the head of the layer as one library call: x read once, xn and y written once
+        return M.norm_then_move(norm, ema, xs[i % NBUF])
 
-    with torch.no_grad():
-        for i in range(args.warmup):
-            step(i)
+    def step_two_modules(i):
+        # the same block across the module boundary: two kernels, xn travels through HBM in between
+        xn = norm(xs[i % NBUF])
+        return xn, ema(xn.transpose(1, 2))
+
+    def timed(fn, steps, warmup):
+        """(device ms per step from events on the launch stream, wall ms per step, host enqueue ms per step)"""
+        for i in range(warmup):
+            fn(i)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
         e0.record()
-        for i in range(args.steps):
-            step(i)
+        for i in range(steps):
+            fn(i)
         e1.record()
+        host = time.perf_counter() - t0
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-        gpu_ms = e0.elapsed_time(e1)
-        ms_per_step = max(wall * 1e3, gpu_ms) / args.steps
+        return e0.elapsed_time(e1) / steps, wall * 1e3 / steps, host * 1e3 / steps
 
-        # per-kernel device time inside the block: the same steps again with an event between the two
-        # calls (the EMA finds its input where the norm has just left it, as in the timed region)
+    with torch.no_grad():
+        gpu_ms, wall_ms, host_step = timed(step, args.steps, args.warmup)
+        ms_per_step = max(wall_ms, gpu_ms)
         reps = max(20, min(args.steps, 200))
+        two_ms, _, two_host = timed(step_two_modules, reps, 8)
+
+        # per-kernel device time of the two-module variant: an event between the two calls (the EMA finds
+        # its input where the norm has just left it)
         evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
-        h0 = time.perf_counter()
         for i in range(reps):
             a, b, c = evs[i]
             a.record()
@@ -520,56 +541,23 @@ def main():
             b.record()
             ema(xn.transpose(1, 2))
             c.record()
-        host_step = (time.perf_counter() - h0) * 1e3 / reps
         torch.cuda.synchronize()
         norm_ev = sum(a.elapsed_time(b) for a, b, _ in evs) / reps
         ema_ev = sum(b.elapsed_time(c) for _, b, c in evs) / reps
         # the event packets between the kernels cost about a microsecond each: a kernel's time is its
-        # share of the step measured above, split in the proportion of the event intervals
-        # (launch gaps included, so slightly above the kernel trace of the same run)
-        norm_avg = ms_per_step * norm_ev / (norm_ev + ema_ev)
-        ema_avg = ms_per_step * ema_ev / (norm_ev + ema_ev)
+        # share of the two-module step, split in the proportion of the event intervals
+        norm_avg = two_ms * norm_ev / (norm_ev + ema_ev)
+        ema_avg = two_ms * ema_ev / (norm_ev + ema_ev)
 
-        # optionally each operator alone, back to back on inputs that are cold in every cache
-        def timed(fn, reps):
-            args_ = [fn.prep(i) for i in range(reps)]
-            for i in range(min(reps, 8)):
-                fn(args_[i])
-            torch.cuda.synchronize()
-            a = torch.cuda.Event(enable_timing=True)
-            b = torch.cuda.Event(enable_timing=True)
-            h0 = time.perf_counter()
-            a.record()
-            for i in range(reps):
-                fn(args_[i])
-            b.record()
-            host = time.perf_counter() - h0
-            torch.cuda.synchronize()
-            return a.elapsed_time(b) / reps, host * 1e3 / reps
+        # kernel generation inside the call (what a training forward does, where the coefficients change every
+        # step: complex_exponential_moving_average.py:98-109): the prepared operand images are withheld, the
+        # call builds them from (p, q, gamma) into its workspace first
+        layer = ema._prepared_layer()
+        saved_image = layer.image
+        layer.image = None
+        gen_ms, _, gen_host = timed(step, reps, 8)
+        layer.image = saved_image
 
-        class NormCall:
-            @staticmethod
-            def prep(i):
-                return xs[i % NBUF]
-
-            def __call__(self, x):
-                return norm(x)
-
-        class EmaCall:
-            @staticmethod
-            def prep(i):
-                return xns[i % NBUF].transpose(1, 2)
-
-            def __call__(self, x):
-                return ema(x)
-
-        standalone = None
-        if args.standalone:
-            xns = [norm(x) for x in xs]
-            n_avg, n_host = timed(NormCall(), reps)
-            e_avg, e_host = timed(EmaCall(), reps)
-            standalone = {"group_tsn_kernel": {"avg_ms": n_avg, "host_enqueue_ms": n_host},
-                          "ema_mfma_kernel": {"avg_ms": e_avg, "host_enqueue_ms": e_host}}
         if args.copy_calibration:
             dst = torch.empty_like(xs[0])
             for i in range(args.copy_calibration):
@@ -578,12 +566,22 @@ def main():
     status = M.ops.timestep_norm_status()
 
     traffic = measured_traffic()
+    prof = profiled_durations()
     tokens = B * L
-    alg_bytes_block = 4 * B * L * D * 2          # norm: read x, write xn; EMA: read xn, write y
+    alg_bytes_block = 4 * B * L * D * 2          # module boundary kept: norm reads x, writes xn; EMA reads xn, writes y
+    alg_bytes_fused = 3 * B * L * D * 2          # what one kernel has to move: x in, xn and y out
     alg_bytes_ema = 2 * B * L * D * 2
     alg_bytes_norm = 2 * B * L * D * 2
     ema_gbs = alg_bytes_ema / (ema_avg * 1e-3) / 1e9
     norm_gbs = alg_bytes_norm / (norm_avg * 1e-3) / 1e9
+    fused_gbs = alg_bytes_block / (gpu_ms * 1e-3) / 1e9
+
+    def kern(name, what, gbs, alg, avg):
+        return {"bound": "hbm", "kernel": what, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": gbs / HBM_PEAK_GBS, "traffic": traffic.get(name), "algorithmic_bytes_per_launch": alg,
+                "avg_ms": avg, "avg_ms_source": "HIP events on the launch stream around the timed steps / steps",
+                "rocprof_avg_ms": prof.get(name)}
+
     out = {
         "metric": "EMA+norm block tokens/sec @B4xL4096xD1024; achieved HBM GB/s vs peak",
         "value": tokens / (ms_per_step * 1e-3),
@@ -598,29 +596,35 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "configs[2]: TimestepNorm(16 groups) -> complex EMA (N=16), B=4 L=4096 D=1024, "
-                               "bf16 activations, fp32 parameters/accumulation, forward",
+                               "bf16 activations, fp32 parameters/accumulation, forward, one library call "
+                               "(xn and y both written)",
                    "input_buffers_rotated": NBUF},
         "block_hbm_gbs": alg_bytes_block / (ms_per_step * 1e-3) / 1e9,
         "block_hbm_frac": alg_bytes_block / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "roofline": None,
-        "kernels": {
-            "ema_mfma_kernel": {"bound": "hbm", "kernel": "ema_mfma_kernel (the EMA call)", "achieved": ema_gbs,
-                                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ema_gbs / HBM_PEAK_GBS,
-                                "traffic": traffic.get("ema_mfma_kernel"),
-                                "algorithmic_bytes_per_launch": alg_bytes_ema, "avg_ms": ema_avg},
-            "group_tsn_kernel": {"bound": "hbm", "kernel": "group_tsn_kernel (the TimestepNorm call)",
-                                 "achieved": norm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                 "frac": norm_gbs / HBM_PEAK_GBS, "traffic": traffic.get("group_tsn_kernel"),
-                                 "algorithmic_bytes_per_launch": alg_bytes_norm, "avg_ms": norm_avg},
-        },
+        # the dominant (only) kernel of the step; `achieved` prices the block at the bytes of the two-module
+        # boundary (x, xn twice, y), the figure the metric is defined on; `kernel_bytes` is what this kernel moves
+        "roofline": dict(kern("norm_ema_fused_kernel", "norm_ema_fused_kernel (TimestepNorm and EMA in one launch)",
+                              fused_gbs, alg_bytes_block, gpu_ms),
+                         kernel_bytes=alg_bytes_fused,
+                         achieved_on_kernel_bytes=alg_bytes_fused / (gpu_ms * 1e-3) / 1e9,
+                         frac_on_kernel_bytes=alg_bytes_fused / (gpu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS),
+        "device_ms_per_step": gpu_ms,
         "host_enqueue_ms_per_step": host_step,
-        "event_intervals_ms": {"group_tsn_kernel": norm_ev, "ema_mfma_kernel": ema_ev},
+        "two_module_variant": {
+            "ms_per_step": two_ms, "host_enqueue_ms_per_step": two_host,
+            "block_hbm_frac": alg_bytes_block / (two_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "kernels": {
+                "ema_mfma_kernel": kern("ema_mfma_kernel", "ema_mfma_kernel (the EMA call)", ema_gbs, alg_bytes_ema,
+                                        ema_avg),
+                "group_tsn_kernel": kern("group_tsn_kernel", "group_tsn_kernel (the TimestepNorm call)", norm_gbs,
+                                         alg_bytes_norm, norm_avg)},
+            "event_intervals_ms": {"group_tsn_kernel": norm_ev, "ema_mfma_kernel": ema_ev}},
+        "kernel_generation_in_call": {
+            "ms_per_step": gen_ms, "host_enqueue_ms_per_step": gen_host, "tokens_per_s": tokens / (gen_ms * 1e-3),
+            "what": "the same step with the prepared operand images withheld (image = NULL): the call generates "
+                    "them from (p, q, gamma) before the block kernel"},
         "timestep_norm_status": status,
     }
-    if standalone is not None:
-        out["standalone_cold"] = standalone
-    # the dominant kernel = the one with the longer launch (both are HBM-bound)
-    out["roofline"] = max(out["kernels"].values(), key=lambda k: k["avg_ms"])
     if not args.no_cpu:
         threads = min(os.cpu_count() or 1, 16)
         x_host = xs[0].float().cpu().numpy()

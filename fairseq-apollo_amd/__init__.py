@@ -10,6 +10,7 @@ from .modules import (  # noqa: F401
     SequenceNorm,
     SwiGLU,
     TimestepNorm,
+    norm_then_move,
 )
 
 from .layers import (  # noqa: F401,E402
@@ -45,4 +46,5 @@ __all__ = [
     "SequenceNorm",
     "SwiGLU",
     "TimestepNorm",
+    "norm_then_move",
 ]

@@ -22,7 +22,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU,
+from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU, norm_then_move,
                       TimestepNorm, _training_call)
 
 
@@ -266,11 +266,13 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if self.bidirectional:
             assert incremental_state is None, 'a bidirectional layer has no incremental state'
             x = self.norm(x, padding_mask, length_last=False)      # the statistics do not depend on the layout
+            mx = None
         else:
-            x = self.norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
+            x, mx = norm_then_move(self.norm, self.move, x, padding_mask, incremental_state, out_layout="input")
         v = F.silu(self.v_proj(x))
-        mx = self.move(x.transpose(1, 2), padding_mask, incremental_state, out_layout="input").transpose(1, 2)
-        mx = self.move_act(mx)
+        if mx is None:
+            mx = self.move(x.transpose(1, 2), padding_mask, incremental_state, out_layout="input")
+        mx = self.move_act(mx.transpose(1, 2))
         base = self.mx_proj(mx)
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
         Nh = self.num_heads

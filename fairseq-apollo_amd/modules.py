@@ -19,7 +19,7 @@ from __future__ import annotations
 import math
 import uuid
 from collections import OrderedDict
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 import torch.nn.functional as F
@@ -460,6 +460,47 @@ class TimestepNorm(nn.Module, IncrementalState):
     def extra_repr(self) -> str:
         return 'num_features={num_features}, num_groups={num_groups}, prior_count={_prior_count}, eps={eps}'.format(
             **self.__dict__)
+
+
+def norm_then_move(norm: nn.Module, move: nn.Module, x: Tensor, padding_mask: Optional[Tensor] = None,
+                   incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None,
+                   out_layout: str = "rows") -> Tuple[Tensor, Tensor]:
+    """x = norm(x); mx = move(x^T), the head of the layer (moving_average_gated_attention.py:304-315).
+    x: [B, L, D] -> (xn [B, L, D], mx [B, D, L] in `out_layout`).  A group TimestepNorm in front of a
+    one-sided layer without kernel truncation, called without autograd, goes to the library as one call
+    (x is read once, xn and mx are written once); both modules' incremental state is kept exactly as the
+    two calls keep it.  Every other combination runs the two modules one after the other."""
+    one_call = (isinstance(norm, TimestepNorm) and norm.num_groups is not None and isinstance(move, BaseMovingLayer)
+                and not move.bidirectional and (move.truncation is None or move.truncation < 1)
+                and x.is_cuda and x.dim() == 3 and x.size(0) > 0 and x.size(1) > 0
+                and not _training_call(norm, x) and not _training_call(move, x))
+    if not one_call:
+        xn = norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
+        return xn, move(xn.transpose(1, 2), padding_mask, incremental_state, out_layout=out_layout)
+    batch_size = x.size(0)
+    norm_state = move_state = None
+    prev_count = prev_mean = prev_var = h = None
+    if incremental_state is not None:
+        norm_state = norm._get_input_buffer(incremental_state)
+        if 'prev_mean' in norm_state:
+            prev_mean, prev_var, prev_count = norm_state['prev_mean'], norm_state['prev_var'], norm_state['prev_count']
+        move_state = move._get_input_buffer(incremental_state)
+        h = move_state.get('prev_state')
+    if prev_count is None or prev_mean is None or prev_var is None:
+        d_count, d_mean, d_var = norm._prior_state(batch_size)
+        prev_count = d_count if prev_count is None else prev_count
+        prev_mean = d_mean if prev_mean is None else prev_mean
+        prev_var = d_var if prev_var is None else prev_var
+    gamma, beta = norm._affine()
+    xn, y, count, mean, var, h_out = move._prepared_layer().norm_forward(
+        x, prev_count, prev_mean, prev_var, gamma, beta, norm.num_groups, norm.eps, padding_mask, h,
+        want_state=incremental_state is not None, out_layout=out_layout)
+    if incremental_state is not None:
+        norm_state['prev_mean'], norm_state['prev_var'], norm_state['prev_count'] = mean, var, count
+        norm._set_input_buffer(incremental_state, norm_state)
+        move_state['prev_state'] = h_out
+        move._set_input_buffer(incremental_state, move_state)
+    return xn, y
 
 
 class SequenceNormFunc(torch.autograd.Function):

@@ -197,3 +197,38 @@ def test_kernel_generation_inside_the_call():
     got = _run(layer, x, G, nw, nb)
     layer.image = saved
     assert torch.equal(ref[0], got[0]) and torch.equal(ref[1], got[1])
+
+
+def test_module_pair_keeps_both_incremental_states():
+    """norm_then_move(norm, move, x, ...) equals the two modules called one after the other, chunk by chunk with
+    incremental state (1024 tokens in one kernel, then 300 as two operators, then a single token)."""
+    B, G, N = 2, 2, 16
+    D = 64 * G
+    torch.manual_seed(56)
+    norm = M.TimestepNorm(D, G).to(DEV).eval()
+    move = M.MultiHeadComplexEMA(D, ndim=N).to(DEV).eval()
+    with torch.no_grad():
+        norm.weight.normal_(0, 0.1)
+        norm.bias.normal_(0, 0.1)
+    x = torch.randn(B, 1325, D, device=DEV).to(BF)
+    inc_a, inc_b = {}, {}
+    with torch.no_grad():
+        for lo, hi in ((0, 1024), (1024, 1324), (1324, 1325)):
+            xc = x[:, lo:hi].contiguous()
+            xn_a, y_a = M.norm_then_move(norm, move, xc, None, inc_a, out_layout="input")
+            xn_b = norm(xc, incremental_state=inc_b)
+            y_b = move(xn_b.transpose(1, 2), None, inc_b, out_layout="input")
+            torch.cuda.synchronize()
+            assert y_a.shape == y_b.shape == (B, D, hi - lo)
+            assert rel_err(host(xn_a), host(xn_b)) < 1e-2
+            assert rel_err(host(y_a), host(y_b)) < 2e-2
+    sa, sb = norm._get_input_buffer(inc_a), norm._get_input_buffer(inc_b)
+    assert sa['prev_count'].tolist() == sb['prev_count'].tolist() == [1325] * B
+    assert rel_err(host(sa['prev_mean']), host(sb['prev_mean'])) < 1e-5
+    assert rel_err(host(sa['prev_var']), host(sb['prev_var'])) < 1e-5
+    ha, hb = move._get_input_buffer(inc_a)['prev_state'], move._get_input_buffer(inc_b)['prev_state']
+    assert rel_err(np.real(host(ha)), np.real(host(hb))) < 2e-3
+    # with autograd the pair runs as the two modules
+    xg = x[:, :64].float().requires_grad_(True)
+    xn_g, y_g = M.norm_then_move(norm, move, xg)
+    assert y_g.requires_grad and xn_g.requires_grad
