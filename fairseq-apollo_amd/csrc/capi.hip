@@ -15,3 +15,90 @@ void set_error(const char* fmt, ...) {
 
 extern "C" const char* mega_last_error(void) { return mega::g_err; }
 extern "C" int mega_abi_version(void) { return 2; }
+
+// ------------------------------------------------------------------------------------------------
+// Status of the bounded waits.  One word of pinned, device-mapped host memory per device: a kernel that
+// gives up stores 1 into it (system scope); the entry points that launch such kernels look at it first and
+// refuse the call once, the way a sticky launch error surfaces on the next call
+// (C10_CUDA_KERNEL_LAUNCH_CHECK(), fairseq/csrc/ops/timestep_norm_kernel.cu:641).
+#include <atomic>
+#include <mutex>
+
+namespace mega {
+namespace {
+constexpr int kMaxDevices = 64;
+constexpr uint32_t kDefaultSpinLimit = 1u << 22;
+struct StatusSlot {
+  volatile uint32_t* host = nullptr;   // what the host reads
+  uint32_t* dev = nullptr;             // the same word as the kernels address it
+  bool tried = false;
+};
+StatusSlot g_status[kMaxDevices];
+volatile uint32_t g_plain[kMaxDevices];   // stands in where no pinned word exists (no device, allocation refused)
+std::mutex g_status_mu;
+std::atomic<uint32_t> g_spin_limit{kDefaultSpinLimit};
+std::atomic<int> g_withhold_first{0};
+
+int current_slot() {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) {
+    (void)hipGetLastError();
+    d = 0;
+  }
+  return d >= 0 && d < kMaxDevices ? d : 0;
+}
+
+StatusSlot& slot_of(int d, bool may_allocate) {
+  std::lock_guard<std::mutex> lock(g_status_mu);
+  StatusSlot& s = g_status[d];
+  if (!s.host) s.host = &g_plain[d];
+  if (!s.dev && !s.tried && may_allocate) {
+    s.tried = true;
+    void* h = nullptr;
+    void* dv = nullptr;
+    if (hipHostMalloc(&h, 64, hipHostMallocMapped) == hipSuccess && h &&
+        hipHostGetDevicePointer(&dv, h, 0) == hipSuccess && dv) {
+      *(volatile uint32_t*)h = g_plain[d];
+      s.host = (volatile uint32_t*)h;
+      s.dev = (uint32_t*)dv;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+  return s;
+}
+}  // namespace
+
+LookbackLaunch lookback_launch(bool may_allocate) {
+  StatusSlot& s = slot_of(current_slot(), may_allocate);
+  LookbackLaunch l;
+  l.status = s.dev;
+  l.spin_limit = g_spin_limit.load();
+  l.withhold_first = g_withhold_first.load();
+  return l;
+}
+
+int lookback_pending(const char* entry) {
+  StatusSlot& s = slot_of(current_slot(), false);
+  if (*s.host == 0u) return MEGA_OK;
+  *s.host = 0u;
+  set_error("%s: an earlier launch on this device gave up waiting for the words of an earlier tile (workgroups "
+            "not dispatched in id order, or a workspace shared by launches that overlap); it has written NaN into "
+            "the outputs and statistics that depended on them.  This call was not launched; the status is now clear",
+            entry);
+  return MEGA_ERR_LAUNCH;
+}
+}  // namespace mega
+
+extern "C" int mega_lookback_status(int clear) {
+  auto& s = mega::slot_of(mega::current_slot(), false);
+  const int v = (int)*s.host;
+  if (clear) *s.host = 0u;
+  return v;
+}
+
+extern "C" void mega_test_lookback(unsigned spin_limit, int withhold_first, int raise) {
+  mega::g_spin_limit.store(spin_limit ? spin_limit : mega::kDefaultSpinLimit);
+  mega::g_withhold_first.store(withhold_first ? 1 : 0);
+  if (raise) *mega::slot_of(mega::current_slot(), false).host = 1u;
+}

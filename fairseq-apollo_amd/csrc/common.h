@@ -13,6 +13,19 @@ namespace mega {
 // ---------------------------------------------------------------- errors
 void set_error(const char* fmt, ...);
 
+// ---- give-ups of the bounded waits between workgroups (look-back of the streaming kernels).
+// A kernel that gives up writes NaN into what depended on the missing words and sets two words: `error` of its
+// workspace header and the host-mapped status word of its device, which the host reads without synchronising.
+struct LookbackLaunch {
+  uint32_t* status;      // device address of the device's host-mapped status word (null: none could be set up)
+  uint32_t spin_limit;   // polls before a wait gives up
+  int withhold_first;    // test hook: the first tile of every row publishes nothing
+};
+// `may_allocate`: the status word may be created (pinned host memory) if the device has none yet
+LookbackLaunch lookback_launch(bool may_allocate);
+// MEGA_ERR_LAUNCH (message set, word cleared) when a launch on the current device has given up since the last check
+int lookback_pending(const char* entry);
+
 #define MEGA_REQUIRE(cond, code, ...)  \
   do {                                 \
     if (!(cond)) {                     \

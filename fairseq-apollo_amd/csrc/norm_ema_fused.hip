@@ -84,6 +84,7 @@ struct FusedArgs {
   float eps;
   int is_complex;
   int xcd_map;
+  LookbackLaunch lb;     // status word, poll limit, test hook
 };
 
 __device__ __forceinline__ int row_base(int c) { return c * kFRow + (c >> 2) * 16; }
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       if (w == wave) wpre = tot;
       tot = merge(tot, Moments{s_wt[w * 4], s_wt[w * 4 + 1], s_wt[w * 4 + 2]});
     }
-    if (wave == 0 && lane == 0) {
+    if (wave == 0 && lane == 0 && !(A.lb.withhold_first && s == 0)) {
       put_rec(myrec, tagged((uint32_t)tot.n, tag));
       put_rec(myrec + 1, tagged(__float_as_uint(tot.mean), tag));
       put_rec(myrec + 2, tagged(__float_as_uint(tot.var), tag));
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         w2 = get_rec(rp + 2);
         const bool ok = (uint32_t)(w0 >> 32) == tag && (uint32_t)(w1 >> 32) == tag && (uint32_t)(w2 >> 32) == tag;
         if (__all(ok)) break;
-        if (++spins > kSpinLimit) {
+        if (++spins > A.lb.spin_limit) {
           poison = true;
           break;
         }
@@ -326,7 +327,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     Moments carry = merge(prior, accp);
     if (poison) {
       carry.mean = __builtin_nanf("");
-      if (lane == 0) publish_u32(&A.hdr->error, 1u);
+      if (lane == 0) report_give_up(A.hdr, A.lb.status);
     }
     const Moments base = merge(carry, merge(wpre, lane_exc));
     Moments full = base;
@@ -571,7 +572,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       MEGA_FTR(6 + i);
     }
   }
-  if (!last_block) {
+  if (!last_block && !(A.lb.withhold_first && s == 0)) {
     // the wave's four channels x 16 states x (re, im) = 128 words: two per lane
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
@@ -636,7 +637,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 #pragma unroll
           for (int u = 0; u < 8; ++u) ok &= (uint32_t)(w[u] >> 32) == tag;
           if (__all(ok)) break;
-          if (++spins > kSpinLimit) {
+          if (++spins > A.lb.spin_limit) {
             poison = true;
             break;
           }
@@ -672,7 +673,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       }
       if (poison) {
         Cr[0] = __builtin_nanf("");
-        if (lane == 0) publish_u32(&A.hdr->error, 1u);
+        if (lane == 0) report_give_up(A.hdr, A.lb.status);
       }
     }
     MEGA_FTR(10);
@@ -876,6 +877,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
                                  float* h_out, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N,
                                  const void* image, void* workspace, size_t workspace_bytes, void* scratch,
                                  size_t scratch_bytes, void* stream) {
+  if (const int rc = lookback_pending("norm_ema_fwd")) return rc;
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "norm_ema_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && D > 0 && G > 0 && N > 0 && D % G == 0, MEGA_ERR_ARG,
@@ -919,6 +921,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
     A.is_complex = is_complex;
     A.xcd_map = (G % 8 == 0) ? 1 : 0;
+    A.lb = lookback_launch(true);
     const dim3 grid((unsigned)(B * G * S));
     typedef void (*Kern)(const FusedArgs);
     const int lout = syl == 1 ? 0 : 1;

@@ -60,6 +60,7 @@ struct TsnParams {
   int TPT;           // vectors per token
   int LPG;           // vectors per group
   float eps;
+  LookbackLaunch lb; // status word, poll limit, test hook
 };
 
 // LPGT > 0: groups are LPGT adjacent lanes and are reduced with lane shuffles;
@@ -73,7 +74,9 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   unsigned long long* s_lbw = (unsigned long long*)(s_mask + ((P.TT + 15) / 16) * 16);   // [kLbWords]
   float* part = (float*)(s_lbw + kLbWords);                   // [kPartCap] (LPGT == 0 only)
 
+  __shared__ uint32_t s_gave_up;                   // a wait of this workgroup ran into the poll limit
   const int tid = threadIdx.x;
+  if (tid == 0) s_gave_up = 0u;
   const int ticket = (int)blockIdx.x;
   const uint32_t tag = P.hdr->epoch + 1u;
   const int tile = ticket / P.B;
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     }
     const Moments inc = row_scan(st);
     const Moments exc = dpp_m<0x111>(inc);          // exclusive: what the lanes before this one hold
-    if (l16 == 15 && active) {
+    if (l16 == 15 && active && !(P.lb.withhold_first && tile == 0)) {
       unsigned long long* mine = P.rec + (trow + tile) * W;
       put_rec(mine + 1 + 2 * g, tagged(__float_as_uint(inc.mean), tag));
       put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(inc.var), tag));
@@ -272,8 +275,9 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) pending |= (uint32_t)(w[u] >> 32) != tag;
             if (!pending) break;
-            if (++spins > kSpinLimit) {
-              publish_u32(&P.hdr->error, 1u);
+            if (++spins > P.lb.spin_limit) {
+              s_gave_up = 1u;
+              report_give_up(P.hdr, P.lb.status);
               break;
             }
             __builtin_amdgcn_s_sleep(1);
@@ -304,6 +308,9 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     }
     MEGA_TSN_TR(3);
     acc = row_reduce(acc);
+    // words that never came: everything this tile derives from the earlier tiles is NaN, not a partial sum
+    const bool poison = s_gave_up != 0u;
+    if (poison) acc.mean = __builtin_nanf("");
     const uint32_t prevtot = row_sum_u32(prevcnt);    // the lanes hold disjoint sets of earlier tiles
     Moments prior = prior0;
     if (gbase != 0) prior = Moments{(float)P.prev_count[b], P.prev_mean[(size_t)b * G + gc], P.prev_var[(size_t)b * G + gc]};
@@ -326,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       const Moments fin = merge(carry, inc);
       P.mean[(size_t)b * G + g] = fin.mean;
       P.var[(size_t)b * G + g] = fin.var;
-      if (g == 0) P.count[b] = P.prev_count[b] + (int64_t)prevtot + (int64_t)inc.n;
+      if (g == 0) P.count[b] = poison ? (int64_t)-1 : P.prev_count[b] + (int64_t)prevtot + (int64_t)inc.n;
     }
   }
   __syncthreads();
@@ -511,6 +518,7 @@ static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* 
                               int64_t G, double eps, int64_t* count, float* mean, float* var,
                               float* group_mean, float* cummean, float* cumrstd, void* workspace,
                               size_t workspace_bytes, bool fixed_scratch, void* stream) {
+  if (const int rc = lookback_pending("group_timestep_norm_fwd")) return rc;
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "group_timestep_norm_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && H > 0 && G > 0, MEGA_ERR_ARG,
@@ -561,6 +569,7 @@ static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* 
   P.rec = (unsigned long long*)w;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G;
   P.TT = g.tt; P.ntiles = g.ntiles; P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
+  P.lb = lookback_launch(!fixed_scratch);
   switch (dtype) {
     case MEGA_F32: return dispatch_vec<float>(P, g, s);
     case MEGA_BF16: return dispatch_vec<bf16_t>(P, g, s);

@@ -6,8 +6,6 @@
 namespace mega {
 namespace {
 
-constexpr uint32_t kSpinLimit = 1u << 22;     // bounded wait for another tile's published words
-
 struct TsnHeader {
   uint32_t epoch;        // bumped by the last workgroup of every launch
   uint32_t done2;        // second-level retire counter
@@ -15,6 +13,12 @@ struct TsnHeader {
   uint32_t pad;
   uint32_t done1[32];    // first-level retire counters (workgroup id mod 32)
 };
+
+// a bounded wait gave up: the workspace header and the device's host-mapped status word say so
+__device__ __forceinline__ void report_give_up(TsnHeader* hdr, uint32_t* status) {
+  publish_u32(&hdr->error, 1u);
+  if (status) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // ---- lane-group primitives (DPP inside rows of 16 lanes)
 template <int CTRL>

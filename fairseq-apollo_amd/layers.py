@@ -627,4 +627,6 @@ def streamed_forward(layers, x: Tensor, chunk_size: int, padding_mask: Optional[
             out = layer(h, incremental_state=incremental_states, decoder_padding_mask=pm)
             h = out[0] if isinstance(out, tuple) else out
         outs.append(h)
+    if x.is_cuda:
+        ops.check_lookback("streamed_forward")
     return torch.cat(outs, dim=1)

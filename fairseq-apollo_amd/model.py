@@ -14,6 +14,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
+from . import ops
 from .layers import MegaDecoderLayer, _arg
 from .modules import TimestepNorm
 
@@ -143,4 +144,6 @@ def validate_stream(model: MegaDecoderNoCrossAttn, src_tokens: Tensor, target: T
             nll += F.nll_loss(lp.reshape(-1, lp.size(-1)), tgt.reshape(-1), ignore_index=pad_idx,
                               reduction='sum').double()
             ntok += tgt.ne(pad_idx).sum()
+    if src_tokens.is_cuda:
+        ops.check_lookback("validate_stream")
     return nll, ntok

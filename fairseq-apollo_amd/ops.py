@@ -112,14 +112,34 @@ def _scratch_buffer(dev: torch.device, nbytes: int, stream: Optional[int] = None
     return ws
 
 
-def timestep_norm_status(dev=None) -> int:
+def timestep_norm_status(dev=None, clear: bool = False) -> int:
     """Error word of the TimestepNorm workspaces of `dev` (non-zero: a tile gave up waiting for
-    an earlier tile).  Synchronises; meant for tests and debugging."""
+    an earlier tile).  Synchronises; meant for tests and debugging (lookback_status is the view
+    that does not synchronise)."""
     bad = 0
     for (idx, _), ws in _tsn_ws.items():
         if dev is None or torch.device(dev).index in (None, idx):
             bad |= int(ws[8:12].view(torch.int32).item())
+            if clear:
+                ws[8:12].zero_()
     return bad
+
+
+def lookback_status(clear: bool = False) -> int:
+    """Status word of the current device's bounded waits (mega_lookback_status): non-zero once a tile of a
+    TimestepNorm or block launch has given up waiting for an earlier tile.  Does not synchronise: a launch that
+    is still running may set it later."""
+    return int(_lib.load().mega_lookback_status(1 if clear else 0))
+
+
+def check_lookback(where: str = "") -> None:
+    """Raise (and clear the status) if a launch has given up since the last check.  The library does the same
+    at the start of the calls that launch such kernels; streaming helpers call this once more when they are
+    done, so that a failure in their last chunks does not wait for an unrelated later call."""
+    if lookback_status(clear=True):
+        raise RuntimeError(f"{where or 'mega'}: a TimestepNorm / moving-average launch gave up waiting for an "
+                           "earlier time tile and has written NaN into the outputs and statistics that depended on "
+                           "it (workgroups not dispatched in id order, or one workspace used by overlapping launches)")
 
 
 # --------------------------------------------------------------------------------------

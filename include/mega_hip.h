@@ -43,7 +43,7 @@ enum {
   MEGA_ERR_ARG = -1,       /* bad shape / pointer / flag                     */
   MEGA_ERR_UNSUPPORTED = -2, /* valid request outside the implemented envelope */
   MEGA_ERR_WORKSPACE = -3, /* workspace missing or too small                 */
-  MEGA_ERR_LAUNCH = -4     /* hipLaunchKernel reported an error              */
+  MEGA_ERR_LAUNCH = -4     /* hipLaunchKernel reported an error, or an earlier launch gave up a bounded wait */
 };
 
 /* reason for the last negative return on this thread (never NULL) */
@@ -51,6 +51,26 @@ const char* mega_last_error(void);
 
 /* library version, bumped when a signature changes */
 int mega_abi_version(void);
+
+/* Bounded waits between workgroups.  The group TimestepNorm kernel and the one-kernel TimestepNorm -> moving
+ * average block let a time tile wait for the words of the earlier tiles of its row; they count on the
+ * hardware starting workgroups in id order, and the wait is bounded.  A tile that gives up writes NaN into
+ * every output and statistic that depended on the missing words (count becomes -1), sets the error word of
+ * its workspace and a host-mapped status word of its device.  The entry points that launch these kernels
+ * (mega_group_timestep_norm_fwd, mega_norm_ema_fwd) look at that word before anything else: if it is set they
+ * clear it and return MEGA_ERR_LAUNCH without launching, so a give-up surfaces on the next call the way a
+ * sticky launch error does (C10_CUDA_KERNEL_LAUNCH_CHECK(), fairseq/csrc/ops/timestep_norm_kernel.cu:641).
+ * mega_lookback_status reads the word of the current device without synchronising (a launch still running
+ * may set it later; after a synchronisation it is final); clear != 0 resets it.
+ * mega_group_timestep_norm_fwd_noalloc passes the word to its kernel only once another entry point has
+ * created it (creating it allocates pinned host memory).                                            */
+int mega_lookback_status(int clear);
+
+/* Test hook for the failure path, so that it can be exercised with every kernel exiting normally:
+ * spin_limit = polls before a wait gives up (0 = the default, 2^22); withhold_first != 0 makes the first
+ * tile of every row publish nothing, so the later tiles of the row run into the limit; raise != 0 sets the
+ * status word of the current device from the host.  Not for production use.                         */
+void mega_test_lookback(unsigned spin_limit, int withhold_first, int raise);
 
 /* ------------------------------------------------------------------------ */
 /* EMA coefficients -> convolution kernel and carried-state bias            */

@@ -69,3 +69,33 @@ def test_ops_reject_cpu_tensors():
         M.ops.swiglu(x, x)
     with pytest.raises(RuntimeError, match="HIP device"):
         M.ops.attention_softmax_fwd(x, 0.0, True)
+
+
+def test_give_up_status_is_reported_once_by_the_next_call():
+    """Host logic of the bounded-wait status: a raised status word makes the next call of an entry point that
+    launches a look-back kernel return MEGA_ERR_LAUNCH before anything else is looked at, and clears the
+    word; the call after that is judged on its own arguments again.  (On a box without a GPU a plain host
+    word stands in for the pinned one the kernels write.)"""
+    lib = M._lib.load()
+    a = 0x10000   # never dereferenced
+    gtsn = lambda: lib.mega_group_timestep_norm_fwd(None, None, 1, None, None, None, None, None, None, 2, 8, 30, 4,
+                                                    1e-5, None, None, None, None, None, None, None, 0, None)
+    fused = lambda: lib.mega_norm_ema_fwd(a, a, a, 9, 0, 0, 0, a, a, a, a, a, None, 1e-5, a, a, a, a, a, a, 1, a,
+                                          None, None, 1, 1024, 64, 1, 16, None, None, 0, None, 0, None)
+    assert lib.mega_lookback_status(0) == 0
+    try:
+        for call, plain_rc in ((gtsn, -1), (fused, -1)):
+            lib.mega_test_lookback(0, 0, 1)
+            assert lib.mega_lookback_status(0) == 1
+            assert call() == -4 and b"gave up" in lib.mega_last_error()
+            assert lib.mega_lookback_status(0) == 0          # reported once
+            assert call() == plain_rc and b"gave up" not in lib.mega_last_error()
+        lib.mega_test_lookback(0, 0, 1)
+        assert lib.mega_lookback_status(1) == 1 and lib.mega_lookback_status(0) == 0
+        lib.mega_test_lookback(0, 0, 1)
+        with pytest.raises(RuntimeError, match="gave up"):
+            M.ops.check_lookback("test")
+        M.ops.check_lookback("test")                         # cleared
+    finally:
+        lib.mega_test_lookback(0, 0, 0)
+        lib.mega_lookback_status(1)
