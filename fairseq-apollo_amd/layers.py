@@ -23,7 +23,7 @@ from torch.nn import Parameter
 
 from . import ops
 from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU, norm_then_move,
-                      TimestepNorm, _training_call)
+                      TimestepNorm, _tensor_versions, _training_call)
 
 
 class RMSNorm(nn.Module):
@@ -185,6 +185,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         assert zdim % num_heads == 0 and hdim % num_heads == 0 and (zdim // num_heads) % 2 == 0
         self.embed_dim, self.zdim, self.hdim, self.ndim = embed_dim, zdim, hdim, ndim
         self._qk_cache = None
+        self._qk_key = None
         self._keep_weights, self._last_weights = False, None
         self.chunk_size = chunk_size
         self.num_heads = num_heads
@@ -306,8 +307,12 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
     def _qk_constants(self, simple: bool):
         """(gamma + 1, beta, rotation frequencies) in fp32 for the q / k kernel; kept in eval mode
         (dropped by train() and by .to() / .half())."""
-        if not self.training and self._qk_cache is not None:
-            return self._qk_cache
+        if not self.training:
+            key = _tensor_versions(self, self.rel_pos_bias)
+            if key != self._qk_key:
+                self._qk_cache, self._qk_key = None, key
+            if self._qk_cache is not None:
+                return self._qk_cache
         with torch.no_grad():
             freqs = self._no_rotation if simple else self.rel_pos_bias.freqs      # zero angles: no rotation
             c = ((self.gamma.float() + 1.0).contiguous(), self.beta.float().contiguous(), freqs.float().contiguous())

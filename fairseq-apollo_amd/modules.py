@@ -80,6 +80,17 @@ def _training_call(module: nn.Module, *tensors) -> bool:
                                         or any(p.requires_grad for p in module.parameters()))
 
 
+def _tensor_versions(*modules: nn.Module) -> tuple:
+    """Storage address and in-place version of the modules' own parameters and buffers.  An eval-mode cache
+    derived from them is stale once this tuple changes: load_state_dict copies into the parameters, an
+    optimiser step or an in-place edit under no_grad bumps the version, `.to()` moves the storage.  (The
+    reference recomputes weight + 1, the prior state and the q / k affine on every call,
+    timestep_norm.py:118-131, and caches only the moving-average coefficients in eval mode,
+    base_moving_average.py:52-58.)"""
+    return tuple((t.data_ptr(), t._version) for m in modules
+                 for t in (*m._parameters.values(), *m._buffers.values()) if t is not None)
+
+
 class BaseMovingLayer(nn.Module, IncrementalState):
     """fairseq/modules/base_moving_average.py:18-197."""
 
@@ -93,6 +104,7 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         self.shift = shift
         self._coeffs = None
         self._prepared = None
+        self._cache_key = None
         assert self.bidirectional or (self.truncation is None or self.truncation < 1), \
             'one directional moving average should not have positive trunction: {}'.format(truncation)
 
@@ -111,9 +123,18 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         with torch.no_grad():           # forward only: coefficients never carry a graph
             if self.training:
                 return self._calc_coeffs()
+            self._drop_stale_cache()
             if self._coeffs is None:
                 self._coeffs = self._calc_coeffs()
             return self._coeffs
+
+    def _drop_stale_cache(self):
+        """The eval-mode caches follow the parameters they were computed from."""
+        key = _tensor_versions(self)
+        if key != self._cache_key:
+            self._coeffs = None
+            self._prepared = None
+            self._cache_key = key
 
     def train(self, mode: bool = True):
         self._coeffs = None
@@ -174,8 +195,10 @@ class BaseMovingLayer(nn.Module, IncrementalState):
 
     def _prepared_layer(self) -> "ops.PreparedEMA":
         """Coefficients in the library's layout; kept while the eval-mode coefficient cache lives."""
-        if not self.training and self._prepared is not None and self._coeffs is not None:
-            return self._prepared
+        if not self.training:
+            self._drop_stale_cache()
+            if self._prepared is not None and self._coeffs is not None:
+                return self._prepared
         p, q, gamma = self.coeffs()
         layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, self.omega.reshape(-1), self.bidirectional,
                                 self.truncation, self.shift)
@@ -347,6 +370,7 @@ class TimestepNorm(nn.Module, IncrementalState):
         self._prior_count = prior_count
         self._prior_cache = {}
         self._affine_cache = None
+        self._cache_key = None
         if num_groups is None or num_groups == num_features:
             num_groups = num_features
             assert prior_count > 1
@@ -412,8 +436,10 @@ class TimestepNorm(nn.Module, IncrementalState):
                     self.prior_mean.float().expand(batch_size, -1),
                     torch.exp(self.prior_logv.float()).expand(batch_size, -1))
         key = batch_size
-        if not self.training and key in self._prior_cache:
-            return self._prior_cache[key]
+        if not self.training:
+            self._drop_stale_cache()
+            if key in self._prior_cache:
+                return self._prior_cache[key]
         with torch.no_grad():
             st = (self.prior_count.expand(batch_size).contiguous(),
                   self.prior_mean.float().expand(batch_size, -1).contiguous(),
@@ -424,12 +450,22 @@ class TimestepNorm(nn.Module, IncrementalState):
 
     def _affine(self):
         """(weight + 1, bias) in fp32, as the reference passes them (timestep_norm.py:129-131)."""
-        if not self.training and self._affine_cache is not None:
-            return self._affine_cache
+        if not self.training:
+            self._drop_stale_cache()
+            if self._affine_cache is not None:
+                return self._affine_cache
         with torch.no_grad():
             ab = (self.weight.float() + 1.0, self.bias.float().contiguous())
         self._affine_cache = None if self.training else ab
         return ab
+
+    def _drop_stale_cache(self):
+        """The eval-mode caches follow the parameters and buffers they were computed from."""
+        key = _tensor_versions(self)
+        if key != self._cache_key:
+            self._prior_cache = {}
+            self._affine_cache = None
+            self._cache_key = key
 
     def train(self, mode: bool = True):
         self._prior_cache = {}

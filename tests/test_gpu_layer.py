@@ -474,3 +474,30 @@ def test_incremental_decoding_with_learned_bias_and_element_attention(bias, act,
         state = {}
         parts = [layer(x[:, a:a + step], incremental_state=state)[0] for a in range(0, 128, step)]
     assert rel_err(host(torch.cat(parts, dim=1)), host(full)) < 2e-5
+
+
+def test_weights_loaded_after_an_eval_forward_take_effect():
+    """The eval-mode caches (moving-average coefficients and operand images, weight + 1 / bias of the norm,
+    the q / k affine) are rebuilt when load_state_dict or an in-place edit changes the parameters."""
+    B, L, D, S, E, N, C = 1, 1024, 64, 32, 128, 16, 256
+    mk = lambda seed: (torch.manual_seed(seed), M.MovingAverageGatedAttention(
+        D, S, E, N, chunk_size=C, norm_num_groups=1).to(DEV).to(torch.bfloat16).eval())[1]
+    a, b = mk(11), mk(12)
+    with torch.no_grad():
+        for layer in (a, b):
+            layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
+            layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+    x = torch.randn(B, L, D, device=DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        ya, _ = a(x)
+        yb, _ = b(x)
+        assert not torch.equal(ya, yb)
+        a.load_state_dict(b.state_dict())
+        ya2, _ = a(x)
+        assert torch.equal(ya2, yb)
+        a.move.alpha.add_(0.3); b.move.alpha.add_(0.3)
+        a.norm.weight.mul_(0.5); b.norm.weight.mul_(0.5)
+        b.train(); b.eval()                  # b recomputes everything
+        ya3, _ = a(x)
+        yb3, _ = b(x)
+        assert torch.equal(ya3, yb3) and not torch.equal(ya3, ya2)

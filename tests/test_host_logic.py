@@ -113,3 +113,39 @@ def test_layer_constructor_follows_the_reference():
     with pytest.raises(ValueError, match="attention activation"):
         M.MovingAverageGatedAttention(8, 4, 8, 2, attention_activation='gelu', **kw)
     assert 'chunk=4' in repr(M.MovingAverageGatedAttention(8, 4, 8, 2, **kw))
+
+
+def test_eval_caches_follow_the_parameters():
+    """Weights loaded (or edited in place) after a first eval-mode use: the cached coefficients, weight + 1 /
+    bias and the prior state are recomputed, as the reference computes them on every call
+    (timestep_norm.py:118-131) or from the parameters it was given (base_moving_average.py:52-58)."""
+    import copy
+
+    torch.manual_seed(3)
+    ema = M.MultiHeadComplexEMA(8, ndim=4).eval()
+    p0, q0, g0 = [t.clone() for t in ema.coeffs()]
+    assert ema.coeffs()[0] is ema.coeffs()[0]                    # cached while nothing changes
+    other = M.MultiHeadComplexEMA(8, ndim=4)
+    ema.load_state_dict(copy.deepcopy(other.state_dict()))
+    p1, q1, g1 = ema.coeffs()
+    po, qo, go = other.eval().coeffs()
+    assert torch.equal(p1, po) and torch.equal(q1, qo) and torch.equal(g1, go)
+    assert not torch.equal(p1, p0)
+    with torch.no_grad():
+        ema.alpha.add_(0.5)
+    assert not torch.equal(ema.coeffs()[0], p1)
+
+    norm = M.TimestepNorm(16, 4, prior_count=2).eval()
+    g_a, b_a = norm._affine()
+    c_a, m_a, v_a = norm._prior_state(3)
+    assert norm._affine()[0] is g_a and norm._prior_state(3)[1] is m_a
+    sd = copy.deepcopy(norm.state_dict())
+    sd["weight"] = torch.randn(16)
+    sd["bias"] = torch.randn(16)
+    sd["prior_mean"] = torch.randn(4)
+    sd["prior_logv"] = torch.randn(4)
+    norm.load_state_dict(sd)
+    g_b, b_b = norm._affine()
+    c_b, m_b, v_b = norm._prior_state(3)
+    assert torch.equal(g_b, sd["weight"] + 1.0) and torch.equal(b_b, sd["bias"])
+    assert torch.equal(m_b, sd["prior_mean"].expand(3, -1)) and torch.allclose(v_b, sd["prior_logv"].exp().expand(3, -1))
