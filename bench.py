@@ -140,6 +140,29 @@ def bench_decode(args):
     dev_ms = a.elapsed_time(b) / args.steps
     alg = 2 * Bd * Dd * Nd * 8 + 3 * Bd * Dd * 2 + 4 * Bd * Gd * 4
     gbs = alg / (dev_ms * 1e-3) / 1e9
+    # K tokens of every stream per launch (chunk-wise streaming of given inputs, not autoregressive
+    # generation): the state crosses HBM once per launch
+    multi = {}
+    with torch.no_grad():
+        for K in (4, 16, 64):
+            chunks = [torch.randn(Bd, K, Dd, device=dev).to(torch.bfloat16) for _ in range(4)]
+            n = max(20, args.steps // 4)
+            for i in range(5):
+                step.steps(chunks[i % 4])
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            a.record()
+            for i in range(n):
+                step.steps(chunks[i % 4])
+            b.record()
+            torch.cuda.synchronize()
+            wall_k = (time.perf_counter() - t0) * 1e3 / n
+            dev_k = a.elapsed_time(b) / n
+            alg_k = 2 * Bd * Dd * Nd * 8 + 3 * Bd * K * Dd * 2 + 4 * Bd * Gd * 4
+            multi[f"K={K}"] = {"ms_per_launch": max(wall_k, dev_k), "device_ms_per_launch": dev_k,
+                               "tokens_per_s": Bd * K / (max(wall_k, dev_k) * 1e-3),
+                               "hbm_gbs": alg_k / (dev_k * 1e-3) / 1e9, "algorithmic_bytes_per_launch": alg_k}
     print(json.dumps({
         "metric": "decode tokens/sec @B64xD2048, fused TimestepNorm + EMA step", "value": Bd / (ms * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
@@ -148,6 +171,7 @@ def bench_decode(args):
         "roofline": {"bound": "hbm", "kernel": "norm_ema_step_kernel", "achieved": gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": alg, "avg_ms": dev_ms, "host_enqueue_ms": host * 1e3 / args.steps},
+        "tokens_per_launch": multi,
     }))
 
 

@@ -37,6 +37,8 @@ SIGNATURES = {
     "mega_ema_step": (_int, [_p, _p, _int, _p, _p, _p, _int, _p, _p, _p, _i64, _i64, _i64, _p]),
     "mega_norm_ema_step": (_int, [_p, _p, _p, _int, _p, _p, _p, _p, _p, _p, _p, _p, C.c_double, _p, _p, _p, _int, _p, _p,
                                   _p, _i64, _i64, _i64, _i64, _p]),
+    "mega_norm_ema_steps": (_int, [_p, _p, _p, _int, _i64, _p, _p, _p, _p, _p, _p, _p, _p, C.c_double, _p, _p, _p, _int,
+                                   _p, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "mega_norm_ema_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mega_norm_ema_fwd_scratch_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mega_norm_ema_fwd": (_int, [_p, _p, _p, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, C.c_double, _p, _p, _p,

@@ -31,6 +31,8 @@ struct StepArgs {
   const float* h_in;     // [B, D, N, 2] or null
   float* h_out;
   int B, D, G, N;
+  int K;                 // tokens per stream in this launch (the multi-token kernel)
+  int MB;                // tokens per batch staged in LDS
   float eps;
 };
 
@@ -184,6 +186,170 @@ __global__ __launch_bounds__(kTV) void norm_ema_step_vec_kernel(const StepArgs A
   }
 }
 
+// K consecutive tokens of every stream in one launch: x, xn, y are [B, K, D].  The state h of a channel stays in
+// registers over the K tokens (read once, written once per launch instead of once per token), the norm
+// statistics of the (stream, group) advance token by token exactly as K single steps would advance them.
+// Tokens are taken in batches of A.MB that fit in LDS: the group's slice of the batch is staged there with its
+// moments (one wave per token, no workgroup barrier per token), every thread then walks the batch for its
+// channels out of LDS (no global access inside the token loop), and xn, y leave as whole rows.
+constexpr int kStepsLdsBytes = 32 * 1024;     // per workgroup, so that four of them share a CU
+constexpr int kStepsIT = 2;                     // channels-parts a thread advances side by side
+
+struct StepMoments {
+  float n, mean, var;
+};
+// Welford merge of two runs (fairseq/csrc/utils.h:66-76 for general weights)
+__device__ __forceinline__ StepMoments step_merge(StepMoments a, StepMoments b) {
+  const float n = a.n + b.n;
+  const float rn = n > 0.f ? 1.0f / n : 0.f;
+  const float ca = a.n * rn, cb = b.n * rn;
+  const float d = b.mean - a.mean;
+  return StepMoments{n, a.mean + cb * d, ca * a.var + cb * b.var + (ca * d) * (cb * d)};
+}
+
+template <typename T, int NP>
+__global__ __launch_bounds__(kTV) void norm_ema_steps_kernel(const StepArgs A) {
+  extern __shared__ float s_dyn[];
+  const int dg = A.D / A.G;
+  const int MB = A.MB;                           // <= 64
+  float* s_mu = s_dyn;                           // [MB] group mean of the token, then running mean
+  float* s_rs = s_mu + MB;                       // [MB] group variance, then running 1 / sqrt(var + eps)
+  float* s_x = s_rs + MB;                        // [MB][dg] x, then xn (as rounded to T)
+  float* s_y = s_x + (size_t)MB * dg;            // [MB][dg] y
+  const int g = blockIdx.x % A.G, b = blockIdx.x / A.G;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* xb = (const T*)A.x + (size_t)b * A.K * A.D + (size_t)g * dg;
+  T* xnb = (T*)A.xn + (size_t)b * A.K * A.D + (size_t)g * dg;
+  T* yb = (T*)A.y + (size_t)b * A.K * A.D + (size_t)g * dg;
+  const int64_t c_in = A.prev_count[b];
+  // the statistics carried into the current batch (every thread keeps a copy)
+  StepMoments carry = {(float)c_in, A.prev_mean[(size_t)b * A.G + g], A.prev_var[(size_t)b * A.G + g]};
+  const float inv_dg = 1.0f / (float)dg;
+  const int items = dg * NP;                     // a multiple of NP, so the lanes of a channel stay together
+  for (int k0 = 0; k0 < A.K; k0 += MB) {
+    const int nk = min(MB, A.K - k0);
+    __syncthreads();                             // the previous batch has left LDS
+    for (int k = wave; k < nk; k += kTV / 64) {
+      const T* xr = xb + (size_t)(k0 + k) * A.D;
+      float* sx = s_x + (size_t)k * dg;
+      float s = 0.f;
+      for (int f = lane; f < dg; f += 64) {
+        const float xv = to_float(xr[f]);
+        sx[f] = xv;
+        s += xv;
+      }
+      for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m);
+      const float gm = s * inv_dg;
+      float s2 = 0.f;
+      for (int f = lane; f < dg; f += 64) {
+        const float d = sx[f] - gm;              // this lane's own stores
+        s2 += d * d;
+      }
+      for (int m = 32; m >= 1; m >>= 1) s2 += __shfl_xor(s2, m);
+      if (lane == 0) {
+        s_mu[k] = gm;
+        s_rs[k] = s2 * inv_dg;
+      }
+    }
+    __syncthreads();
+    // running statistics after every token of the batch: an inclusive scan of Welford merges over the tokens
+    // (lane = token), every wave for itself; the same merge tree for every wave, so all threads agree
+    StepMoments m = {0.f, 0.f, 0.f};
+    if (lane < nk) m = StepMoments{1.f, s_mu[lane], s_rs[lane]};
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const StepMoments p = {__shfl_up(m.n, o), __shfl_up(m.mean, o), __shfl_up(m.var, o)};
+      if (lane >= o) m = step_merge(p, m);
+    }
+    const StepMoments run = step_merge(carry, m);
+    __syncthreads();                             // every wave has read the group moments
+    if (wave == 0 && lane < nk) {
+      s_mu[lane] = run.mean;
+      s_rs[lane] = 1.0f / sqrtf(run.var + A.eps);
+    }
+    {
+      const StepMoments last = {__shfl(run.n, nk - 1), __shfl(run.mean, nk - 1), __shfl(run.var, nk - 1)};
+      carry = last;
+    }
+    __syncthreads();
+    for (int it0 = 0; it0 < items; it0 += kTV * kStepsIT) {
+      bool ok[kStepsIT];
+      int f[kStepsIT], part[kStepsIT];
+      size_t ho[kStepsIT];
+      float4 h0[kStepsIT], h1[kStepsIT], q0[kStepsIT], q1[kStepsIT], g0[kStepsIT], g1[kStepsIT], pp[kStepsIT];
+      float nw[kStepsIT], nb[kStepsIT], om[kStepsIT];
+      const float* hsrc = k0 == 0 ? A.h_in : A.h_out;          // later batches continue from what this thread wrote
+#pragma unroll
+      for (int i = 0; i < kStepsIT; ++i) {
+        const int it = it0 + i * kTV + threadIdx.x;
+        ok[i] = it < items;
+        f[i] = ok[i] ? it / NP : 0;
+        part[i] = it % NP;
+        const int d = g * dg + f[i];
+        ho[i] = (((size_t)b * A.D + d) * A.N + 4 * part[i]) * 2;
+        const size_t co = (size_t)d * A.N + 4 * part[i];
+        h0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        h1[i] = h0[i];
+        if (hsrc) {
+          h0[i] = *(const float4*)(hsrc + ho[i]);
+          h1[i] = *(const float4*)(hsrc + ho[i] + 4);
+        }
+        q0[i] = *(const float4*)(A.q + co * 2);
+        q1[i] = *(const float4*)(A.q + co * 2 + 4);
+        g0[i] = *(const float4*)(A.g + co * 2);
+        g1[i] = *(const float4*)(A.g + co * 2 + 4);
+        pp[i] = *(const float4*)(A.p + co);
+        nw[i] = A.nw[d];
+        nb[i] = A.nb[d];
+        om[i] = A.omega[d];
+      }
+      for (int k = 0; k < nk; ++k) {
+        const float mu = s_mu[k], rs = s_rs[k];
+#pragma unroll
+        for (int i = 0; i < kStepsIT; ++i) {
+          float* sx = s_x + (size_t)k * dg + f[i];
+          const T xn_t = from_float<T>((*sx - mu) * rs * nw[i] + nb[i]);
+          const float xv = to_float(xn_t);         // the moving average sees the rounded activation
+          float4 n0, n1;
+          n0.x = q0[i].x * h0[i].x - q0[i].y * h0[i].y + pp[i].x * xv;  n0.y = q0[i].x * h0[i].y + q0[i].y * h0[i].x;
+          n0.z = q0[i].z * h0[i].z - q0[i].w * h0[i].w + pp[i].y * xv;  n0.w = q0[i].z * h0[i].w + q0[i].w * h0[i].z;
+          n1.x = q1[i].x * h1[i].x - q1[i].y * h1[i].y + pp[i].z * xv;  n1.y = q1[i].x * h1[i].y + q1[i].y * h1[i].x;
+          n1.z = q1[i].z * h1[i].z - q1[i].w * h1[i].w + pp[i].w * xv;  n1.w = q1[i].z * h1[i].w + q1[i].w * h1[i].z;
+          h0[i] = n0;
+          h1[i] = n1;
+          float acc = (g0[i].x * n0.x - g0[i].y * n0.y) + (g0[i].z * n0.z - g0[i].w * n0.w) +
+                      (g1[i].x * n1.x - g1[i].y * n1.y) + (g1[i].z * n1.z - g1[i].w * n1.w);
+#pragma unroll
+          for (int mm = 1; mm < NP; mm <<= 1) acc += __shfl_xor(acc, mm);
+          if (ok[i] && part[i] == 0) {             // the NP lanes of the channel have read *sx (same wave)
+            *sx = xv;
+            s_y[(size_t)k * dg + f[i]] = acc + om[i] * xv;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kStepsIT; ++i) {
+        if (ok[i]) {
+          *(float4*)(A.h_out + ho[i]) = h0[i];
+          *(float4*)(A.h_out + ho[i] + 4) = h1[i];
+        }
+      }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nk * dg; i += kTV) {
+      const int k = i / dg, f = i - k * dg;
+      const size_t o = (size_t)(k0 + k) * A.D + f;
+      xnb[o] = from_float<T>(s_x[i]);              // exact: the value was rounded to T before it was stored
+      yb[o] = from_float<T>(s_y[i]);
+    }
+  }
+  if (threadIdx.x == 0) {
+    A.mean[(size_t)b * A.G + g] = carry.mean;
+    A.var[(size_t)b * A.G + g] = carry.var;
+    if (g == 0) A.count[b] = c_in + (int64_t)A.K;
+  }
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -215,6 +381,7 @@ extern "C" int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, c
   A.x = x; A.xn = xn; A.y = y; A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var;
   A.count = count; A.mean = mean; A.var = var; A.nw = norm_gamma; A.nb = norm_beta; A.p = p; A.q = q; A.g = gamma;
   A.omega = omega; A.h_in = h_in; A.h_out = h_out; A.B = (int)B; A.D = (int)D; A.G = (int)G; A.N = (int)N;
+  A.K = 1;
   A.eps = (float)eps;
   const dim3 grid((unsigned)(B * G));
   hipStream_t s = (hipStream_t)stream;
@@ -248,5 +415,63 @@ extern "C" int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, c
   }
 #undef LAUNCH_NS
   MEGA_CHECK_LAUNCH("norm_ema_step");
+  return MEGA_OK;
+}
+
+extern "C" int mega_norm_ema_steps(const void* x, void* xn, void* y, int dtype, int64_t K, const int64_t* prev_count,
+                                   const float* prev_mean, const float* prev_var, int64_t* count, float* mean,
+                                   float* var, const float* norm_gamma, const float* norm_beta, double eps,
+                                   const float* p, const float* q, const float* gamma, int is_complex,
+                                   const float* omega, const float* h_in, float* h_out, int64_t B, int64_t D,
+                                   int64_t G, int64_t N, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "norm_ema_steps: unknown dtype %d", dtype);
+  MEGA_REQUIRE(B >= 0 && K >= 0 && D > 0 && G > 0 && N > 0 && D % G == 0, MEGA_ERR_ARG,
+               "norm_ema_steps: bad shape B=%ld K=%ld D=%ld G=%ld N=%ld", (long)B, (long)K, (long)D, (long)G, (long)N);
+  MEGA_REQUIRE(B * G < (int64_t)1 << 31 && K < (int64_t)1 << 24 && B * K * D < (int64_t)1 << 40, MEGA_ERR_UNSUPPORTED,
+               "norm_ema_steps: shape too large");
+  const int np = (int)(N / 4);
+  MEGA_REQUIRE(is_complex && N % 4 == 0 && N <= 32 && (np & (np - 1)) == 0, MEGA_ERR_UNSUPPORTED,
+               "norm_ema_steps: complex coefficient storage with ndim in {4, 8, 16, 32} only (ndim=%ld, is_complex=%d); "
+               "call mega_norm_ema_step once per token",
+               (long)N, is_complex);
+  if (B == 0 || K == 0) return MEGA_OK;
+  MEGA_REQUIRE(x && xn && y && prev_count && prev_mean && prev_var && count && mean && var && norm_gamma && norm_beta &&
+                   p && q && gamma && omega && h_out,
+               MEGA_ERR_ARG, "norm_ema_steps: null pointer argument");
+  MEGA_REQUIRE(((uintptr_t)h_out % 16) == 0 && (!h_in || ((uintptr_t)h_in % 16) == 0) && ((uintptr_t)q % 16) == 0 &&
+                   ((uintptr_t)gamma % 16) == 0 && ((uintptr_t)p % 16) == 0,
+               MEGA_ERR_ARG, "norm_ema_steps: h, p, q, gamma must be 16-byte aligned");
+  MEGA_REQUIRE(!ranges_overlap(prev_count, (size_t)B * 8, count, (size_t)B * 8), MEGA_ERR_ARG,
+               "norm_ema_steps: count must not overlap prev_count (every group of a stream reads prev_count "
+               "while one of them writes count); alternate between two count buffers");
+  StepArgs A;
+  A.x = x; A.xn = xn; A.y = y; A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var;
+  A.count = count; A.mean = mean; A.var = var; A.nw = norm_gamma; A.nb = norm_beta; A.p = p; A.q = q; A.g = gamma;
+  A.omega = omega; A.h_in = h_in; A.h_out = h_out; A.B = (int)B; A.D = (int)D; A.G = (int)G; A.N = (int)N;
+  A.K = (int)K;
+  A.eps = (float)eps;
+  // tokens per batch: what fits in LDS beside the moments (x / xn and y of the group's slice as fp32)
+  const int64_t dg = D / G;
+  int64_t mb = (kStepsLdsBytes - 0) / (dg * 8 + 8);
+  MEGA_REQUIRE(mb >= 1, MEGA_ERR_UNSUPPORTED, "norm_ema_steps: %ld channels per group do not fit in LDS", (long)dg);
+  if (mb > 64) mb = 64;
+  if (mb > K) mb = K;
+  A.MB = (int)mb;
+  const size_t smem = (size_t)mb * (dg * 8 + 8);
+  const dim3 grid((unsigned)(B * G));
+  hipStream_t s = (hipStream_t)stream;
+#define LAUNCH_NK(T)                                                                                  \
+  switch (np) {                                                                                       \
+    case 1: hipLaunchKernelGGL((norm_ema_steps_kernel<T, 1>), grid, dim3(kTV), smem, s, A); break;       \
+    case 2: hipLaunchKernelGGL((norm_ema_steps_kernel<T, 2>), grid, dim3(kTV), smem, s, A); break;       \
+    case 4: hipLaunchKernelGGL((norm_ema_steps_kernel<T, 4>), grid, dim3(kTV), smem, s, A); break;       \
+    default: hipLaunchKernelGGL((norm_ema_steps_kernel<T, 8>), grid, dim3(kTV), smem, s, A); break;      \
+  }
+  if (dtype == MEGA_F32) { LAUNCH_NK(float) }
+  else if (dtype == MEGA_BF16) { LAUNCH_NK(bf16_t) }
+  else { LAUNCH_NK(f16_t) }
+#undef LAUNCH_NK
+  MEGA_CHECK_LAUNCH("norm_ema_steps");
   return MEGA_OK;
 }

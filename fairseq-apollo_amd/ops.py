@@ -806,6 +806,35 @@ class DecodeStep:
         self.count, self._count_next = self._count_next, self.count
         return xn, y
 
+    def steps(self, x: torch.Tensor):
+        """x: [B, K, D], K consecutive tokens of every stream -> (xn, y), both [B, K, D]: the same as K calls,
+        in one launch (the state is read and written once).  Coefficient shapes the multi-token kernel does not
+        cover take K single steps."""
+        lib = _lib.load()
+        if x.dim() != 3 or x.shape[0] != self.B or x.shape[2] != self.D:
+            raise RuntimeError(f"x must be [{self.B}, K, {self.D}]")
+        K = x.shape[1]
+        np_ = self.N // 4
+        if not (self.is_complex and self.N % 4 == 0 and self.N <= 32 and np_ & (np_ - 1) == 0):
+            outs = [self(x[:, k]) for k in range(K)]
+            if not outs:
+                return torch.empty_like(x), torch.empty_like(x)
+            return torch.stack([o[0] for o in outs], 1), torch.stack([o[1] for o in outs], 1)
+        xd = x.detach().contiguous()
+        xn = torch.empty_like(xd)
+        y = torch.empty_like(xd)
+        if K == 0:
+            return xn, y
+        with _on_device(self.dev):
+            rc = lib.mega_norm_ema_steps(_ptr(xd), _ptr(xn), _ptr(y), _dtype_code(xd), K, _ptr(self.count),
+                                         _ptr(self.mean), _ptr(self.var), _ptr(self._count_next), _ptr(self.mean),
+                                         _ptr(self.var), _ptr(self.nw), _ptr(self.nb), self.eps, _ptr(self.p), _ptr(self.q),
+                                         _ptr(self.gamma), 1, _ptr(self.omega), _ptr(self.h), _ptr(self.h), self.B, self.D,
+                                         self.G, self.N, _stream(self.dev))
+        _lib.check(rc, "norm_ema_steps")
+        self.count, self._count_next = self._count_next, self.count
+        return xn, y
+
     @property
     def state(self) -> torch.Tensor:
         return torch.view_as_complex(self.h) if self.is_complex else self.h[..., 0]

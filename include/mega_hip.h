@@ -176,6 +176,22 @@ int mega_norm_ema_step(const void* x, void* xn, void* y, int dtype, const int64_
                        int is_complex, const float* omega, const float* h_in, float* h_out,
                        int64_t B, int64_t D, int64_t G, int64_t N, void* stream);
 
+/* K consecutive tokens of every stream in one launch: the same result as K calls of
+ * mega_norm_ema_step on x[:, k] (the reference's chunk-wise streaming, fairseq_cli/train.py:406-417,
+ * with chunks of K tokens through TimestepNorm.forward and BaseMovingLayer.forward with incremental
+ * state, timestep_norm.py:100-139 and base_moving_average.py:144-160), but the state h is read and
+ * written once per launch, not once per token, and the host enqueues one kernel instead of K.
+ *   x, xn, y [B,K,D] of `dtype` (contiguous); everything else as mega_norm_ema_step, the same
+ *   in-place rules (count must not overlap prev_count; count advances by K).
+ *   Covered: complex coefficient storage (is_complex != 0), ndim in {4, 8, 16, 32}, 16-byte aligned
+ *   p, q, gamma, h; MEGA_ERR_UNSUPPORTED otherwise (call mega_norm_ema_step per token).        */
+int mega_norm_ema_steps(const void* x, void* xn, void* y, int dtype, int64_t K,
+                        const int64_t* prev_count, const float* prev_mean, const float* prev_var,
+                        int64_t* count, float* mean, float* var, const float* norm_gamma,
+                        const float* norm_beta, double eps, const float* p, const float* q,
+                        const float* gamma, int is_complex, const float* omega, const float* h_in,
+                        float* h_out, int64_t B, int64_t D, int64_t G, int64_t N, void* stream);
+
 /* TimestepNorm followed by the moving-average layer in one call: what
  * MovingAverageGatedAttention.forward does with x at
  * fairseq/modules/moving_average_gated_attention.py:304-315 (x = norm(x), then

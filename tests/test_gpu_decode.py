@@ -94,3 +94,61 @@ def test_config3_b64_d2048_2048_steps():
     assert rel_err(host(step.mean[sel]), mu_o) < 1e-5 and rel_err(host(step.var[sel]), v_o) < 1e-5
     yo, _ = O.ema_forward(xno.transpose(0, 2, 1), p, q, g, om)
     assert rel_err(host(y_s[sel]), yo.transpose(0, 2, 1)) < 1e-4
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B,D,N,G,chunks", [(3, 96, 16, 4, (1, 7, 64, 65, 130)), (2, 256, 8, 2, (16, 16)),
+                                            (5, 64, 4, 1, (3, 200))])
+def test_multi_token_launch_equals_single_steps(dtype, tol, B, D, N, G, chunks):
+    """K tokens per launch (mega_norm_ema_steps) against the same tokens one launch each, chunk after chunk with the
+    state carried (chunks shorter, equal to and longer than the kernel's batch of 64 tokens), and against the fp64
+    oracle on the whole sequence."""
+    rng, p, q, g, om, nw, nb = _setup(B, D, N, G, 43)
+    T = sum(chunks)
+    x, x64 = rounded(rng.normal(size=(B, T, D)) + 0.2, dtype)
+    mk = lambda: M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    one, many = mk(), mk()
+    xs, ys = [], []
+    for t in range(T):
+        xn, y = one(x[:, t])
+        xs.append(xn); ys.append(y)
+    xn_1, y_1 = torch.stack(xs, 1), torch.stack(ys, 1)
+    xk, yk, a = [], [], 0
+    for K in chunks:
+        print(f"case B={B} D={D} N={N} G={G} chunk K={K} at {a}", flush=True)
+        xn, y = many.steps(x[:, a:a + K])
+        assert xn.shape == y.shape == (B, K, D)
+        xk.append(xn); yk.append(y)
+        a += K
+    xn_k, y_k = torch.cat(xk, 1), torch.cat(yk, 1)
+    torch.cuda.synchronize()
+    assert many.count.tolist() == one.count.tolist() == [T] * B
+    assert rel_err(host(many.mean), host(one.mean)) < 1e-5 and rel_err(host(many.var), host(one.var)) < 1e-5
+    assert rel_err(host(xn_k), host(xn_1)) < (1e-5 if dtype is torch.float32 else 1e-2)
+    assert rel_err(host(y_k), host(y_1)) < tol
+    assert rel_err(np.real(host(many.state)), np.real(host(one.state))) < 1e-4
+    assert rel_err(np.imag(host(many.state)), np.imag(host(one.state))) < 1e-4
+    xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, None, G)
+    assert rel_err(host(xn_k), xno) < max(tol, 1e-4)
+    yo, ho = O.ema_forward(host(xn_k).transpose(0, 2, 1), p, q, g, om, incremental=True)
+    assert rel_err(host(y_k), yo.transpose(0, 2, 1)) < max(tol, 1e-4)
+    assert rel_err(np.real(host(many.state)), np.real(ho)) < 1e-4
+
+
+def test_multi_token_launch_other_coefficient_shapes_take_single_steps():
+    """ndim = 6 is outside the multi-token kernel: the C entry point says so, DecodeStep.steps runs K single steps."""
+    B, D, N, G, K = 2, 64, 6, 2, 5
+    rng, p, q, g, om, nw, nb = _setup(B, D, N, G, 44)
+    x, _ = rounded(rng.normal(size=(B, K, D)), torch.float32)
+    a = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    b = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    xn_a, y_a = a.steps(x)
+    outs = [b(x[:, k]) for k in range(K)]
+    torch.cuda.synchronize()
+    assert torch.equal(y_a, torch.stack([o[1] for o in outs], 1)) and torch.equal(a.h, b.h)
+    lib = M._lib.load()
+    ptr = lambda t: t.data_ptr()
+    rc = lib.mega_norm_ema_steps(ptr(x), ptr(xn_a), ptr(y_a), 0, K, ptr(a.count), ptr(a.mean), ptr(a.var),
+                                 ptr(a._count_next), ptr(a.mean), ptr(a.var), ptr(a.nw), ptr(a.nb), 1e-5, ptr(a.p), ptr(a.q),
+                                 ptr(a.gamma), 1, ptr(a.omega), ptr(a.h), ptr(a.h), B, D, G, N, None)
+    assert rc == -2 and b"ndim" in lib.mega_last_error()
