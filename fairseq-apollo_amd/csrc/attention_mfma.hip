@@ -365,6 +365,394 @@ __global__ __launch_bounds__(256) void dropkey_f32_kernel(float* __restrict__ s,
     if (hash_uniform(seed, e0 + j) < dropout) sp[j] = -INFINITY;
 }
 
+// ---------------------------------------------------------------------------------------------
+// One kernel for the whole op when the weights are not wanted: scores, causal softmax and the
+// second product per tile of 64 keys, with running row maxima and sums (no L x L array in memory).
+// The products are formed transposed, S^T = k q^T and y^T = v^T P^T, so that a query is a column
+// (lane & 15) of every accumulator: the running maximum, the rescaling of y and the row sum are
+// per-lane scalars, and the probabilities go from the accumulators of the first product straight
+// into the B operand of the second (the keys of a 32-key block are assigned to MFMA rows so that a
+// lane ends up with eight consecutive keys).  A workgroup of 8 waves owns 256 queries of one
+// (batch, head) and 256 columns of v; a wave owns 32 queries.  k and v tiles go from global memory
+// straight into LDS (global_load ... lds), two buffers, the next tile in flight under the current
+// tile's products; no staging registers, so the 128 accumulator registers of y leave room for the rest.
+// v stays in its own layout (keys x columns): the A operand of the second product, v^T, is formed by the
+// transposing LDS reads of gfx950 (ds_read_b64_tr_b16), so no transposed copy of v is made.
+// Phase clocks: a profiling build defines these to add up the cycles a wave spends per phase; no-ops here.
+#ifndef MEGA_ATR
+#define MEGA_ATR_BEGIN()
+#define MEGA_ATR(k)
+#define MEGA_ATR_END()
+#endif
+constexpr int FBM = 256, FBN = 64, FBD = 256, FNW = 8;
+
+struct FlashArgs {
+  const void* q;      // [B, L, Nh, H1]
+  const void* k;      // [B, L, Nh, H1]
+  const void* v;      // [B, L, Nh, H2]
+  void* y;            // [B, L, Nh, H2]
+  int L, Nh, H1, H2;
+  float scale_log2;   // scale * log2(e)
+  int causal;
+  int xcd, mt, ns;
+};
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+  const v2 v = {(__bf16)a, (__bf16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 v2;
+  const v2 v = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename T, int KS, int FQB>    // KS = H1 / 32 reduction steps of the first product, FQB blocks of 16 queries per wave
+__global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) {
+  constexpr int H1 = 32 * KS;
+  constexpr int QW = 16 * FQB;              // queries per wave
+  constexpr int KROW = H1 * 2;              // bytes per k row in LDS (dense; 16-byte pieces XOR-swizzled by the row)
+  constexpr int KPC = H1 / 8;               // pieces per k row (8 or 16)
+  constexpr int KB = FBN * KROW, VB = FBD * FBN * 2, BUF = KB + VB;
+  constexpr int NKL = FBN * KPC / (64 * FNW);            // 16-byte pieces of a k tile per lane
+  constexpr int NVL = FBD * (FBN / 8) / (64 * FNW);      // of a v^T tile
+  static_assert(NKL >= 1 && FBN * KPC % (64 * FNW) == 0 && FBD * (FBN / 8) % (64 * FNW) == 0,
+                "the tiles must divide over the lanes");
+  extern __shared__ __attribute__((aligned(16))) char lds[];     // 2 x BUF
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int bz, mtile, slab;
+  {
+    int rest = A.xcd ? (int)blockIdx.x >> 3 : (int)blockIdx.x;
+    slab = rest % A.ns;
+    rest /= A.ns;
+    mtile = A.mt - 1 - rest % A.mt;                      // the long (late) query tiles of a causal call first
+    rest /= A.mt;
+    bz = A.xcd ? rest * 8 + ((int)blockIdx.x & 7) : rest;
+  }
+  const int b = bz / A.Nh, h = bz - b * A.Nh;
+  const int m0 = mtile * FBM, d0 = slab * FBD;
+  const int qw0 = m0 + wave * QW;
+  const int n = lane & 15, g = lane >> 4;
+  const T* qb = (const T*)A.q + ((int64_t)b * A.L * A.Nh + h) * H1;
+  const T* kb_ = (const T*)A.k + ((int64_t)b * A.L * A.Nh + h) * H1;
+  const T* vb = (const T*)A.v + ((int64_t)b * A.L * A.Nh + h) * A.H2 + d0;
+  const int64_t vs = (int64_t)A.Nh * A.H2;               // row stride of v in elements
+  const int64_t rs = (int64_t)A.Nh * H1;                 // row stride of q and k in elements
+
+  // q^T as B operand: lane (n, g) holds q[query n of the block][32 s + 8 g ..]
+  uint4 Qr[FQB][KS];
+#pragma unroll
+  for (int j = 0; j < FQB; ++j) {
+    const int qi = qw0 + 16 * j + n;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      Qr[j][s] = make_uint4(0, 0, 0, 0);
+      if (qi < A.L) Qr[j][s] = *(const uint4*)(qb + (int64_t)qi * rs + 32 * s + 8 * g);
+    }
+  }
+  // tiles of keys this workgroup / this wave has to look at
+  const int klim_wg = A.causal ? min(A.L, m0 + FBM) : A.L;         // keys < klim
+  const int klim_w = A.causal ? min(A.L, qw0 + QW) : A.L;
+  const int nkt = (klim_wg + FBN - 1) / FBN;
+
+  // ---- tiles travel from global memory straight into LDS (no staging registers): lane i of a load
+  // instruction supplies the 16 bytes that belong at the i-th piece of the wave's 1 KB of the tile image, so
+  // every lane fetches the piece its LDS position stands for.  k image: row lrow = 16 (2 a + hb) + 4 gg + t holds
+  // key 32 a + 8 gg + 4 hb + t (MFMA row block 2 a + hb then leaves lane (n, g) with keys 32 a + 8 g + 4 hb + {0..3}),
+  // piece c at position c ^ (lrow & 15) (128-byte rows: c ^ ((lrow >> 1) & 7)).  v^T image: row r (128 bytes), piece c at position c ^ ((r >> 1) & 7).
+  // Rows and columns past the end are fetched from the last valid one: their scores are masked, and a
+  // probability of zero meets a finite value.
+  // common case (whole tile inside the sequence, whole slab inside v): one per-lane byte offset per operand,
+  // everything else is uniform (load u of a lane is 32 u keys / 64 u rows of v^T further on)
+  uint32_t koff0, voff0;
+  {
+    const int lrow = tid / KPC, pp = tid % KPC;
+    const int a = lrow >> 5, hb = (lrow >> 4) & 1, gg = (lrow >> 2) & 3, t = lrow & 3;
+    const int key = 32 * a + 8 * gg + 4 * hb + t;
+    const int kc = (pp ^ (KPC == 16 ? (lrow & 15) : ((lrow >> 1) & 7))) * 8;
+    koff0 = (uint32_t)((key * (int)rs + kc) * 2);
+    // v image: row = key (512 bytes), 16-byte piece p at position (((p >> 1) ^ vswz(row)) << 1) | (p & 1): the
+    // 32-byte spans are XOR-swizzled so that the transposing reads of a fragment (four rows, four 8-byte
+    // columns per group of 16 lanes) fall on different banks
+    const int r = tid / (FBD / 8), vp = tid % (FBD / 8);
+    const int p = ((((vp >> 1) ^ ((r & 3) + 4 * ((r >> 3) & 1))) << 1) | (vp & 1));
+    voff0 = (uint32_t)((r * (int)vs + p * 8) * 2);
+  }
+  static_assert(64 * FNW / KPC == 32 || NKL == 1, "load u of the k tile starts 32 u keys further on");
+  static_assert(64 * FNW / (FBD / 8) == 16, "load u of the v tile starts 16 u keys further on");
+  const bool whole_slab = d0 + FBD <= A.H2;
+  auto issue_tile = [&](int kt, int buf) {
+    const int k0 = kt * FBN;
+    char* lk = lds + buf * BUF + wave * 1024;
+    char* lv = lds + buf * BUF + KB + wave * 1024;
+    if (whole_slab && k0 + FBN <= A.L) {
+      const char* kbase = (const char*)(kb_ + (int64_t)k0 * rs);
+      const char* vbase = (const char*)(vb + (int64_t)k0 * vs);
+#pragma unroll
+      for (int u = 0; u < NKL; ++u)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kbase + (int64_t)u * 32 * rs * 2 + koff0),
+                                         (__attribute__((address_space(3))) void*)(lk + u * 1024 * FNW), 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < NVL; ++u)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vbase + (int64_t)u * 16 * vs * 2 + voff0),
+                                         (__attribute__((address_space(3))) void*)(lv + u * 1024 * FNW), 16, 0, 0);
+      return;
+    }
+    // the last tile of a sequence / a partial slab: rows and columns past the end come from the last valid one
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < NKL; ++u) {
+      const int P = u * 64 * FNW + tid;
+      const int lrow = P / KPC, pp = P % KPC;
+      const int a = lrow >> 5, hb = (lrow >> 4) & 1, gg = (lrow >> 2) & 3, t = lrow & 3;
+      const int key = min(k0 + 32 * a + 8 * gg + 4 * hb + t, A.L - 1);
+      const int kc = (pp ^ (KPC == 16 ? (lrow & 15) : ((lrow >> 1) & 7))) * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb_ + (int64_t)key * rs + kc),
+                                       (__attribute__((address_space(3))) void*)(lk + u * 1024 * FNW), 16, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < NVL; ++u) {
+      const int P = u * 64 * FNW + tid;
+      const int r = P / (FBD / 8), pp = P % (FBD / 8);
+      const int key = min(k0 + r, A.L - 1);
+      const int pc = ((((pp >> 1) ^ ((r & 3) + 4 * ((r >> 3) & 1))) << 1) | (pp & 1));
+      const int col = min(pc * 8, A.H2 - d0 - 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + (int64_t)key * vs + col),
+                                       (__attribute__((address_space(3))) void*)(lv + u * 1024 * FNW), 16, 0, 0);
+    }
+  };
+
+  f32x4 O[FBD / 16][FQB];
+#pragma unroll
+  for (int i = 0; i < FBD / 16; ++i)
+#pragma unroll
+    for (int j = 0; j < FQB; ++j) O[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float mrun[FQB], lrun[FQB], pend[FQB];
+#pragma unroll
+  for (int j = 0; j < FQB; ++j) {
+    mrun[j] = -INFINITY;
+    lrun[j] = 0.f;
+    pend[j] = 1.0f;
+  }
+
+  uint4 Pb[2][FQB];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int j = 0; j < FQB; ++j) Pb[a][j] = make_uint4(0, 0, 0, 0);
+  if (nkt > 0) issue_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): this wave's pieces have landed
+  __syncthreads();
+  MEGA_ATR_BEGIN();
+  for (int kt = 0; kt < nkt; ++kt) {
+    if (kt + 1 < nkt) issue_tile(kt + 1, (kt + 1) & 1);  // lands under this tile's products
+    const int k0 = kt * FBN;
+    const bool valid = k0 < klim_w;                      // wave-uniform: some key of the tile is visible
+    const char* lk = lds + (kt & 1) * BUF;
+    const char* lv = lk + KB;
+    MEGA_ATR(5);
+    {
+      if (valid) {
+      f32x4 S[4][FQB];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int j = 0; j < FQB; ++j) S[kb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      {
+        // fragment f = 4 s + kb: row 16 kb + n, piece 4 s + g at position (4 s + g) ^ n; two fragments ahead
+        const char* kfrag = lk + n * KROW;
+        const int ksw = KPC == 16 ? n : ((n >> 1) & 7);
+        auto kaddr = [&](int f) { return kfrag + (f & 3) * 16 * KROW + (((f >> 2) * 4 + g) ^ ksw) * 16; };
+        // the order below is kept as written (the fragment reads run DK fragments ahead of the products that
+        // use them, so that the LDS latency is covered): no scheduling across the markers
+        constexpr int DK = 4;
+        uint4 fk[DK + 1];
+#pragma unroll
+        for (int f = 0; f < DK; ++f) fk[f] = *(const uint4*)kaddr(f);
+#pragma unroll
+        for (int f = 0; f < 4 * KS; ++f) {
+          const int s = f >> 2, kb = f & 3;
+          if (f + DK < 4 * KS) fk[(f + DK) % (DK + 1)] = *(const uint4*)kaddr(f + DK);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < FQB; ++j) S[kb][j] = mfma16<T>(fk[f % (DK + 1)], Qr[j][s], S[kb][j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      MEGA_ATR(0);
+      // mask, running maximum and sum; key of S[kb][j][u]: k0 + 32 (kb >> 1) + 8 g + 4 (kb & 1) + u
+      const bool edge = (A.causal && k0 + FBN - 1 > qw0) || k0 + FBN > A.L;
+#pragma unroll
+      for (int j = 0; j < FQB; ++j) {
+        const int qi = qw0 + 16 * j + n;
+        const int lim = A.causal ? min(qi, A.L - 1) : A.L - 1;      // last visible key
+        if (edge) {
+          // only the tiles on the diagonal and the last one carry this code (kept a branch: the empty asm
+          // statement stops the compiler from turning it into selects executed on every tile)
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int key = k0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + u;
+              S[kb][j][u] = key <= lim ? S[kb][j][u] : -INFINITY;
+            }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) tmax = fmaxf(tmax, S[kb][j][u]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        tmax *= A.scale_log2;                                        // scale > 0: the maximum commutes with it
+        // the running maximum moves only when a tile exceeds it by more than 2^8: probabilities up to 256
+        // are as exact as those below 1, and y is rescaled on few tiles
+        const float mnew = tmax > mrun[j] + 8.0f ? tmax : mrun[j];
+        const float muse = mnew == -INFINITY ? 0.f : mnew;
+        const float corr = __builtin_amdgcn_exp2f(mrun[j] - muse);
+        mrun[j] = mnew;
+        float psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const float pv = __builtin_amdgcn_exp2f(fmaf(S[kb][j][u], A.scale_log2, -muse));
+            S[kb][j][u] = pv;
+            psum += pv;
+          }
+        lrun[j] = lrun[j] * corr + psum;
+        pend[j] = corr;                                              // y is rescaled where it is next touched
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+          Pb[a][j] = make_uint4(pack2<T>(S[2 * a][j][0], S[2 * a][j][1]), pack2<T>(S[2 * a][j][2], S[2 * a][j][3]),
+                                pack2<T>(S[2 * a + 1][j][0], S[2 * a + 1][j][1]),
+                                pack2<T>(S[2 * a + 1][j][2], S[2 * a + 1][j][3]));
+      }
+      MEGA_ATR(1);
+      }
+      if (valid) {
+#pragma unroll
+      for (int j = 0; j < FQB; ++j) {
+        if (__any(pend[j] != 1.0f)) {
+#pragma unroll
+          for (int i = 0; i < FBD / 16; ++i)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) O[i][j][u] *= pend[j];
+        }
+      }
+      {
+        // fragment f = 2 i + a: the A operand v^T[d = 16 i + n][keys 32 a + 8 g ..+7] out of the key-major tile by two
+        // transposing reads (ds_read_b64_tr_b16: lane s of a group of 16 supplies 8 bytes = 4 columns of one row;
+        // lane l receives element l & 3 of the lanes (l >> 2) + 4 x, x = 0..3).  Source lane s points at row
+        // 32 a + 8 g + 4 hh + (s >> 2), columns 16 i + 4 (s & 3): the result is 4 consecutive keys of column 16 i + n.
+        const int sr = n >> 2, sc = n & 3;
+        const char* vsrc = lv + (8 * g + sr) * (FBD * 2) + sc * 8;
+        const int vsw = sr + 4 * (g & 1);
+        typedef __attribute__((ext_vector_type(4))) short s4v;
+        auto vread = [&](int f) {
+          const int i = f >> 1, a = f & 1;
+          const char* q0 = vsrc + a * 32 * (FBD * 2) + ((i ^ vsw) * 32);
+          const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0));
+          const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0 + 4 * (FBD * 2)));
+          const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+          return make_uint4(l2.x, l2.y, h2.x, h2.y);
+        };
+        constexpr int NF = 2 * (FBD / 16);
+        constexpr int DV = 6;                            // fragments in flight ahead of the products
+        uint4 fv[DV + 1];
+#pragma unroll
+        for (int f = 0; f < DV; ++f) fv[f] = vread(f);
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          const int i = f >> 1, a = f & 1;
+          if (f + DV < NF) fv[(f + DV) % (DV + 1)] = vread(f + DV);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < FQB; ++j) O[i][j] = mfma16<T>(fv[f % (DV + 1)], Pb[a][j], O[i][j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      MEGA_ATR(2);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): the next tile's pieces of this wave have landed
+    MEGA_ATR(3);
+    __syncthreads();
+    MEGA_ATR(4);
+  }
+  MEGA_ATR_END();
+  // ---- 1 / row sum, then the wave's block of y leaves through LDS as whole 512-byte rows
+  constexpr int OP = FBD * 2 + 16;                       // pitch of a staged row
+  static_assert(16 * OP <= 2 * BUF / FNW, "a wave stages 16 rows at a time in its share of LDS");
+  __syncthreads();                                       // the last products have read their tiles
+  char* stage = lds + wave * (2 * BUF / FNW);
+  T* yb = (T*)A.y + ((int64_t)b * A.L * A.Nh + h) * A.H2 + d0;
+  const int64_t ys = (int64_t)A.Nh * A.H2;
+#pragma unroll
+  for (int j = 0; j < FQB; ++j) {
+    float l = lrun[j];
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;          // a row without a visible key gives zeros
+#pragma unroll
+    for (int i = 0; i < FBD / 16; ++i) {
+      const uint2 w = make_uint2(pack2<T>(O[i][j][0] * inv, O[i][j][1] * inv), pack2<T>(O[i][j][2] * inv, O[i][j][3] * inv));
+      *(uint2*)(stage + n * OP + (16 * i + 4 * g) * 2) = w;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < 16 * (FBD / 8) / 64; ++u) {
+      const int pi = lane + u * 64;
+      const int r = pi / (FBD / 8), c = pi % (FBD / 8);
+      const int qi = qw0 + 16 * j + r;
+      if (qi < A.L && d0 + c * 8 < A.H2) *(uint4*)(yb + (int64_t)qi * ys + c * 8) = *(const uint4*)(stage + r * OP + c * 16);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <typename T>
+bool flash_covers(const void* v, const void* y, int64_t L, int64_t H1, int64_t H2) {
+  return (H1 == 64 || H1 == 128) && H2 % 8 == 0 && H2 >= 64 && L >= 64 && ((uintptr_t)y % 16) == 0 &&
+         ((uintptr_t)v % 16) == 0;
+}
+
+template <typename T>
+void launch_flash(const void* q, const void* k, const void* v, void* y, int64_t B, int64_t L, int64_t Nh,
+                  int64_t H1, int64_t H2, float scale, int causal, hipStream_t s) {
+  FlashArgs F;
+  F.q = q; F.k = k; F.v = v; F.y = y;
+  F.L = (int)L; F.Nh = (int)Nh; F.H1 = (int)H1; F.H2 = (int)H2;
+  F.scale_log2 = scale * 1.4426950408889634f;
+  F.causal = causal ? 1 : 0;
+  F.mt = (int)ceil_div(L, FBM);
+  F.ns = (int)ceil_div(H2, FBD);
+  const int64_t BN_ = B * Nh;
+  F.xcd = BN_ % 8 == 0 ? 1 : 0;
+  const dim3 grid((unsigned)(BN_ * F.mt * F.ns));
+  const int ks = (int)(H1 / 32);
+  const size_t smem = 2 * ((size_t)FBN * H1 * 2 + (size_t)FBD * FBN * 2);
+#define MEGA_FLASH(KS_)                                                                                       \
+  {                                                                                                           \
+    auto kern = flash_fwd_kernel<T, KS_, FBM / FNW / 16>;                                                                     \
+    static bool attr_set = false;                                                                             \
+    if (!attr_set) {                                                                                          \
+      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);    \
+      attr_set = true;                                                                                        \
+    }                                                                                                         \
+    hipLaunchKernelGGL(kern, grid, dim3(64 * FNW), smem, s, F);                                               \
+  }
+  if (ks == 2) MEGA_FLASH(2) else MEGA_FLASH(4)
+#undef MEGA_FLASH
+}
+
 template <typename T>
 int run_attention(const void* q, const void* k, const void* v, void* y, void* w, int64_t B, int64_t L, int64_t Nh,
                   int64_t H1, int64_t H2, float scale, int causal, float dropout, uint64_t seed, char* ws,
@@ -376,6 +764,11 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   T* P = (T*)ws;                                   // [B*Nh][L][Lp]
   ws += align_up((size_t)BN_ * L * Lp * sizeof(T), 256);
   T* Vt = (T*)ws;                                  // [B*Nh][H2][Lp]
+  if (!w && dropout <= 0.f && scale > 0.f && flash_covers<T>(v, y, L, H1, H2)) {
+    launch_flash<T>(q, k, v, y, B, L, Nh, H1, H2, scale, causal, s);
+    MEGA_CHECK_LAUNCH("attention_fwd (one-kernel path)");
+    return MEGA_OK;
+  }
   {
     const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(H2, 64), (unsigned)BN_);
     const int vec = (H2 % 8 == 0 && ((uintptr_t)v % 16) == 0) ? 1 : 0;
