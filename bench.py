@@ -291,6 +291,62 @@ def bench_seqnorm(args):
     }))
 
 
+def bench_tsn_feature(args):
+    """Per-feature TimestepNorm (every feature its own group) at configs[2]'s activation shape: the three kernels
+    parallel over time tiles, and the one-thread-per-feature kernel (the same entry point without a workspace)."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1238)
+    gamma = torch.randn(D, device=dev) * 0.1 + 1.0
+    beta = torch.randn(D, device=dev) * 0.1
+    pc = torch.zeros(B, dtype=torch.int64, device=dev)
+    pm = torch.zeros(B, D, device=dev)
+    pv = torch.ones(B, D, device=dev)
+    xs = [torch.randn(B, L, D, device=dev).to(torch.bfloat16) for _ in range(NBUF)]
+
+    def timed(fn, n):
+        for i in range(3):
+            fn(i)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for i in range(n):
+            fn(i)
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    par = timed(lambda i: M.ops.timestep_norm_fwd(xs[i % NBUF], pc, pm, pv, gamma, beta, None, 1e-5, need_stats=False),
+                args.steps)
+    lib = M._lib.load()
+    y = torch.empty_like(xs[0])
+    cnt = torch.empty(B, dtype=torch.int64, device=dev)
+    mean, var = torch.empty(B, D, device=dev), torch.empty(B, D, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def serial(i):
+        rc = lib.mega_timestep_norm_fwd(xs[i % NBUF].data_ptr(), y.data_ptr(), 1, pc.data_ptr(), pm.data_ptr(), pv.data_ptr(),
+                                        gamma.data_ptr(), beta.data_ptr(), None, B, L, D, 1e-5, cnt.data_ptr(),
+                                        mean.data_ptr(), var.data_ptr(), None, None, None, 0, stream)
+        assert rc == 0
+
+    ser = timed(serial, max(5, args.steps // 10))
+    alg = 2 * B * L * D * 2              # x read once, y written once
+    print(json.dumps({
+        "metric": "per-feature TimestepNorm tokens/sec @B4xL4096xD1024", "value": B * L / (par * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": par,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "TimestepNorm without groups (every feature its own statistics) at configs[2]'s activation shape"},
+        "kernels": {"time_tiles_ms": par, "one_thread_per_feature_ms": ser},
+        "roofline": {"bound": "hbm", "kernel": "feature_tile_moments + feature_tile_scan + feature_tile_apply",
+                     "achieved": alg / (par * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg / (par * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": alg},
+    }))
+
+
 def bench_ema_real(args):
     """configs[0] and configs[1]: the real MultiHeadEMA forward in fp32 on [B, D, L] rows (one-sided,
     B2 x D512 x L1024; two-sided with a right-padding mask, B1 x D256 x L16384).  The value is
@@ -478,7 +534,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real"],
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4]; "
@@ -494,6 +550,8 @@ def main():
         return bench_ema_real(args)
     if args.workload == "seqnorm":
         return bench_seqnorm(args)
+    if args.workload == "tsn_feature":
+        return bench_tsn_feature(args)
     if args.workload == "block_bwd":
         return bench_block_bwd(args)
     if args.workload == "attention":

@@ -428,6 +428,185 @@ __global__ __launch_bounds__(kThreads) void feature_tsn_kernel(
   if (h == 0) count[b] = m0;
 }
 
+// ---- the per-feature variant in parallel over time (fairseq/csrc/ops/timestep_norm_kernel.cu:73-185 scans time
+// in parallel as well).  Time is cut into tiles of kFeatTT tokens:
+//   feature_tile_moments   one thread per (row, tile, feature): Welford state of the tile from an empty start
+//   feature_tile_scan      one thread per (row, feature): the states become "everything before the tile",
+//                          prior included (WelfordCombine, fairseq/csrc/utils.h:66-76), in place
+//   feature_tile_apply     one thread per (row, tile, feature): the per-element update of the serial kernel from
+//                          that start, normalise, store; the last tile writes the final state
+// x is read twice and y written once; the states are 12 bytes per feature and tile.
+#ifndef MEGA_FEAT_TT
+#define MEGA_FEAT_TT 64
+#endif
+constexpr int kFeatTT = MEGA_FEAT_TT;
+
+struct FeatArgs {
+  const void* x;
+  void* y;
+  const int64_t* prev_count;
+  const float* prev_mean;
+  const float* prev_var;
+  const float* gamma;
+  const float* beta;
+  const uint8_t* mask;
+  int64_t* count;
+  float* mean;
+  float* var;
+  float* cummean;
+  float* cumrstd;
+  float* agg;            // [B][ntiles][3][H]: count (as float; after the scan: as int bits), mean, variance
+  int B, L, H, ntiles;
+  float eps;
+};
+
+// V features per thread (16-byte loads when the row length allows it)
+template <typename T, int V>
+__global__ __launch_bounds__(kThreads) void feature_tile_moments(const FeatArgs A) {
+  const int h = (blockIdx.x * kThreads + threadIdx.x) * V;
+  const int tile = blockIdx.y, b = blockIdx.z;
+  if (h >= A.H) return;
+  const int t0 = tile * kFeatTT, t1 = min(A.L, t0 + kFeatTT);
+  const T* x = (const T*)A.x;
+  int m0 = 0;
+  float u[V], v[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) u[i] = v[i] = 0.f;
+  constexpr int kB = 8;                              // tokens requested together (the loads do not wait for each other)
+  for (int tb = t0; tb < t1; tb += kB) {
+    Vec<T, V> xv[kB];
+    bool skip[kB];
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+      const int t = min(tb + k, t1 - 1);
+      xv[k] = *(const Vec<T, V>*)(x + ((size_t)b * A.L + t) * A.H + h);
+      skip[k] = tb + k >= t1 || (A.mask && A.mask[(size_t)b * A.L + t]);
+    }
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+      if (skip[k]) continue;
+      const float coef = 1.0f / (float)(m0 + 1);
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float xf = to_float(xv[k].v[i]);
+        const float d1 = xf - u[i];
+        const float m1 = u[i] + coef * d1;
+        v[i] = v[i] + coef * (d1 * (xf - m1) - v[i]);
+        u[i] = m1;
+      }
+      ++m0;
+    }
+  }
+  float* a = A.agg + (((size_t)b * A.ntiles + tile) * 3) * A.H + h;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    a[i] = (float)m0;
+    a[(size_t)A.H + i] = u[i];
+    a[2 * (size_t)A.H + i] = v[i];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void feature_tile_scan(const FeatArgs A) {
+  const int h = blockIdx.x * kThreads + threadIdx.x;
+  const int b = blockIdx.y;
+  if (h >= A.H) return;
+  int64_t cnt = A.prev_count[b];
+  Moments run = {(float)cnt, A.prev_mean[(size_t)b * A.H + h], A.prev_var[(size_t)b * A.H + h]};
+  constexpr int kB = 8;                                // tiles requested together
+  const int64_t c0 = cnt;
+  for (int tb = 0; tb < A.ntiles; tb += kB) {
+    Moments own[kB];
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+      const int tile = min(tb + k, A.ntiles - 1);
+      const float* a = A.agg + (((size_t)b * A.ntiles + tile) * 3) * A.H + h;
+      own[k] = Moments{a[0], a[(size_t)A.H], a[2 * (size_t)A.H]};
+    }
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+      const int tile = tb + k;
+      if (tile >= A.ntiles) break;
+      float* a = A.agg + (((size_t)b * A.ntiles + tile) * 3) * A.H + h;
+      a[0] = __int_as_float((int)(cnt - c0));              // tokens of this call before the tile (exact)
+      a[(size_t)A.H] = run.mean;
+      a[2 * (size_t)A.H] = run.var;
+      if (own[k].n > 0.f) run = combine(run, own[k]);      // a fully masked tile leaves the state as it is
+      cnt += (int64_t)own[k].n;
+    }
+  }
+}
+
+template <typename T, int V>
+__global__ __launch_bounds__(kThreads) void feature_tile_apply(const FeatArgs A) {
+  const int h = (blockIdx.x * kThreads + threadIdx.x) * V;
+  const int tile = blockIdx.y, b = blockIdx.z;
+  if (h >= A.H) return;
+  const int t0 = tile * kFeatTT, t1 = min(A.L, t0 + kFeatTT);
+  const T* x = (const T*)A.x;
+  T* y = (T*)A.y;
+  const float* a = A.agg + (((size_t)b * A.ntiles + tile) * 3) * A.H + h;
+  int64_t m0 = A.prev_count[b] + (int64_t)__float_as_int(a[0]);
+  float u[V], v[V], w[V], bb[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    u[i] = a[(size_t)A.H + i];
+    v[i] = a[2 * (size_t)A.H + i];
+    w[i] = A.gamma[h + i];
+    bb[i] = A.beta[h + i];
+  }
+  constexpr int kB = 8;                              // tokens requested together
+  for (int tb = t0; tb < t1; tb += kB) {
+    Vec<T, V> xq[kB];
+    bool mk[kB];
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+      const int t = min(tb + k, t1 - 1);
+      xq[k] = *(const Vec<T, V>*)(x + ((size_t)b * A.L + t) * A.H + h);
+      mk[k] = A.mask && A.mask[(size_t)b * A.L + t];
+    }
+#pragma unroll
+    for (int k = 0; k < kB; ++k) {
+    const int t = tb + k;
+    if (t >= t1) break;
+    const size_t o = ((size_t)b * A.L + t) * A.H + h;
+    const bool masked = mk[k];
+    const Vec<T, V> xv = xq[k];
+    const float coef = 1.0f / (float)(m0 + 1);
+    Vec<T, V> out;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float xf = to_float(xv.v[i]);
+      const float d1 = xf - u[i];
+      const float m1 = u[i] + coef * d1;
+      const float m2 = v[i] + coef * (d1 * (xf - m1) - v[i]);
+      const float rstd = __builtin_amdgcn_rsqf(m2 + A.eps);
+      out.v[i] = from_float<T>(masked ? 0.f : (xf - m1) * rstd * w[i] + bb[i]);
+      if (!masked) {
+        u[i] = m1;
+        v[i] = m2;
+      }
+      if (A.cummean) A.cummean[o + i] = masked ? u[i] : m1;
+      if (A.cumrstd) A.cumrstd[o + i] = masked ? __builtin_amdgcn_rsqf(v[i] + A.eps) : rstd;
+    }
+    *(Vec<T, V>*)(y + o) = out;
+    if (!masked) ++m0;
+    }
+  }
+  if (tile == A.ntiles - 1) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      A.mean[(size_t)b * A.H + h + i] = u[i];
+      A.var[(size_t)b * A.H + h + i] = v[i];
+    }
+    if (h == 0) A.count[b] = m0;
+  }
+}
+
+size_t feature_tsn_workspace_bytes(int64_t B, int64_t L, int64_t H) {
+  if (L <= 2 * kFeatTT) return 0;                     // short sequences take the serial kernel
+  return (size_t)B * (size_t)ceil_div(L, kFeatTT) * 3 * (size_t)H * 4;
+}
+
 struct TsnGeom {
   int vec, tpt, lpg, tt, ntiles, lpgt;
   size_t smem;
@@ -507,6 +686,10 @@ size_t tsn_workspace_bytes(int64_t B, int64_t G, int ntiles) {
 using namespace mega;
 
 extern "C" size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G) {
+  if (B > 0 && L > 0 && H > 0 && G == H && H > 1) {
+    const size_t f = feature_tsn_workspace_bytes(B, L, H);   // the per-feature variant (mega_timestep_norm_fwd)
+    return f > 256 ? f : 256;
+  }
   TsnGeom g;
   if (B <= 0 || L <= 0 || H <= 0 || G <= 0 || H % G != 0 || !tsn_geometry(dtype, B, L, H, G, &g)) return 256;
   return tsn_workspace_bytes(B, G, g.ntiles);
@@ -644,8 +827,6 @@ extern "C" int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const i
                                       int64_t B, int64_t L, int64_t H, double eps, int64_t* count,
                                       float* mean, float* var, float* cummean, float* cumrstd,
                                       void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace;
-  (void)workspace_bytes;
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "timestep_norm_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && H > 0, MEGA_ERR_ARG, "timestep_norm_fwd: bad shape");
@@ -658,6 +839,46 @@ extern "C" int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const i
                "timestep_norm_fwd: count must not overlap prev_count");
   MEGA_REQUIRE(L == 0 || (x && y), MEGA_ERR_ARG, "timestep_norm_fwd: null x / y");
   hipStream_t s = (hipStream_t)stream;
+  {
+    // with a workspace: three kernels parallel over time tiles; without (or for short sequences): one thread per
+    // (row, feature) walks the whole sequence
+    const size_t need = feature_tsn_workspace_bytes(B, L, H);
+    const int64_t ntiles = ceil_div(L, kFeatTT);
+    if (need > 0 && workspace && workspace_bytes >= need && ((uintptr_t)workspace % 4) == 0 && ntiles < 65536) {
+      // mean / var may be the prior buffers (the scan has consumed the prior before the last tile writes), count not
+      FeatArgs A;
+      A.x = x; A.y = y; A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var; A.gamma = gamma;
+      A.beta = beta; A.mask = mask; A.count = count; A.mean = mean; A.var = var; A.cummean = cummean;
+      A.cumrstd = cumrstd; A.agg = (float*)workspace; A.B = (int)B; A.L = (int)L; A.H = (int)H; A.ntiles = (int)ntiles;
+      A.eps = (float)eps;
+      const int es = dtype == MEGA_F32 ? 4 : 2;
+      // 8-byte pieces per thread: enough threads to fill the chip at 64 tokens per tile
+      const bool wide = H % (8 / es) == 0 && ((uintptr_t)x % 8) == 0 && ((uintptr_t)y % 8) == 0;
+      const int64_t hv = wide ? H / (8 / es) : H;                  // threads along the features
+      const dim3 gt((unsigned)ceil_div(hv, kThreads), (unsigned)ntiles, (unsigned)B);
+      const dim3 gs((unsigned)ceil_div(H, kThreads), (unsigned)B);
+#define LAUNCH_FPAR(T, V)                                                                \
+  hipLaunchKernelGGL((feature_tile_moments<T, V>), gt, dim3(kThreads), 0, s, A);         \
+  hipLaunchKernelGGL(feature_tile_scan, gs, dim3(kThreads), 0, s, A);                    \
+  hipLaunchKernelGGL((feature_tile_apply<T, V>), gt, dim3(kThreads), 0, s, A)
+      if (wide) {
+        switch (dtype) {
+          case MEGA_F32: LAUNCH_FPAR(float, 2); break;
+          case MEGA_BF16: LAUNCH_FPAR(bf16_t, 4); break;
+          default: LAUNCH_FPAR(f16_t, 4); break;
+        }
+      } else {
+        switch (dtype) {
+          case MEGA_F32: LAUNCH_FPAR(float, 1); break;
+          case MEGA_BF16: LAUNCH_FPAR(bf16_t, 1); break;
+          default: LAUNCH_FPAR(f16_t, 1); break;
+        }
+      }
+#undef LAUNCH_FPAR
+      MEGA_CHECK_LAUNCH("timestep_norm_fwd (time tiles)");
+      return MEGA_OK;
+    }
+  }
   const dim3 grid((unsigned)ceil_div(H, kThreads), (unsigned)B);
 #define LAUNCH_FTSN(T)                                                                            \
   hipLaunchKernelGGL(feature_tsn_kernel<T>, grid, dim3(kThreads), 0, s, (const T*)x, (T*)y,       \

@@ -280,10 +280,16 @@ def timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_m
         cr = torch.empty_like(cm)
     m8 = _mask_u8(padding_mask, B, L)
     gf, bf = _f32c(gamma), _f32c(beta)
+    key = ("tsn_feat", dt, B, L, H)
+    nws = _ws_bytes_cache.get(key)
+    if nws is None:
+        nws = _ws_bytes_cache[key] = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, H) if H > 1 else 0
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, nws, stream) if nws else None      # tile states of the time-parallel kernels
     with _on_device(dev):
         rc = lib.mega_timestep_norm_fwd(_ptr(xd), _ptr(y), dt, _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf),
                                         _ptr(m8), B, L, H, float(eps), _ptr(count), _ptr(mean), _ptr(var), _ptr(cm),
-                                        _ptr(cr), None, 0, _stream(dev))
+                                        _ptr(cr), _ptr(ws), ws.numel() if ws is not None else 0, stream)
     _lib.check(rc, "timestep_norm_fwd")
     return y, count, mean, var, cm, cr
 
