@@ -347,6 +347,43 @@ def bench_tsn_feature(args):
     }))
 
 
+def bench_long_conv(args):
+    """Explicit-kernel causal convolution (ops.fftconv) at configs[2]'s shape: x [B, D, L], k [D, L]."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1239)
+    res = {}
+    for name, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+        xs = [torch.randn(B, D, L, device=dev).to(dt) for _ in range(4)]
+        k = torch.randn(D, L, device=dev) * torch.exp(-torch.arange(L, device=dev) / 300.0)
+        for i in range(3):
+            M.ops.fftconv(xs[i % 4], k)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for i in range(args.steps):
+            M.ops.fftconv(xs[i % 4], k)
+        b.record()
+        torch.cuda.synchronize()
+        res[name] = a.elapsed_time(b) / args.steps
+    ms = res["bf16"]
+    alg = 2 * B * L * D * 2 + D * L * 4              # x read, y written, the kernel read once
+    print(json.dumps({
+        "metric": "explicit-kernel causal convolution tokens/sec @B4xD1024xL4096, Lk=4096", "value": B * L / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "fftconv(x, k) with a materialised kernel of L lags at configs[2]'s shape"},
+        "kernels": {"bf16_ms": res["bf16"], "f32_ms": res["f32"]},
+        "roofline": {"bound": "hbm", "kernel": "long_conv_fft_kernel", "achieved": alg / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_step": alg,
+                     "direct_form_flops": 2 * B * D * L * (L + 1) // 2},
+    }))
+
+
 def bench_ema_real(args):
     """configs[0] and configs[1]: the real MultiHeadEMA forward in fp32 on [B, D, L] rows (one-sided,
     B2 x D512 x L1024; two-sided with a right-padding mask, B1 x D256 x L16384).  The value is
@@ -534,7 +571,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature"],
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature", "long_conv"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4]; "
@@ -552,6 +589,8 @@ def main():
         return bench_seqnorm(args)
     if args.workload == "tsn_feature":
         return bench_tsn_feature(args)
+    if args.workload == "long_conv":
+        return bench_long_conv(args)
     if args.workload == "block_bwd":
         return bench_block_bwd(args)
     if args.workload == "attention":

@@ -63,6 +63,147 @@ __global__ __launch_bounds__(kT) void long_conv_kernel(const T* __restrict__ x, 
   if (t < L) y[(size_t)row * L + t] = from_float<T>(acc);
 }
 
+// ---- the same convolutions through a Fourier transform held in LDS, O(M log M) per row instead of
+// O(L Lk): the reference's route (fftconv_kernel.cu:40-78 with the shuffle FFT of fft.cuh:461-533; n = 2 *
+// pow2ceil(L), fused_ops/fftconv.py:45-61).  M = pow2ceil(L + Lk) points, complex fp32, one workgroup of 1024
+// threads per channel: the (real) kernel row is transformed once and its spectrum kept in registers; the
+// batch rows of the channel go through in pairs, row b in the real and row b + 1 in the imaginary part (the
+// kernel is real, so the two convolutions do not mix).  Forward transform by decimation in frequency (natural
+// order in, bit-reversed out), product with the spectrum in that order, inverse by decimation in time
+// (bit-reversed in, natural out): no reordering pass.  Twiddle factors come from v_sin_f32 / v_cos_f32 (argument
+// in revolutions, exact fractions j / 2^s).
+#ifndef MEGA_LC_FFT_MIN
+#define MEGA_LC_FFT_MIN 512        // shortest kernel that takes the transform
+#endif
+constexpr int kFT = 1024;
+constexpr int kFftMaxLog = 14;            // M <= 16384: 128 KB of LDS
+
+__device__ __forceinline__ float2 cmulf(float2 a, float2 b) {
+  return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);
+}
+
+// forward: natural order -> bit-reversed order
+__device__ __forceinline__ void fft_dif(float2* buf, int logm) {
+  const int M = 1 << logm;
+  for (int s = logm - 1; s >= 0; --s) {
+    const int half = 1 << s;
+    const float inv = 1.0f / (float)(2 * half);
+    __syncthreads();
+    for (int j = threadIdx.x; j < M / 2; j += kFT) {
+      const int pos = j & (half - 1);
+      const int i0 = ((j >> s) << (s + 1)) + pos, i1 = i0 + half;
+      const float2 a = buf[i0], b = buf[i1];
+      const float fr = (float)pos * inv;
+      const float2 w = make_float2(__builtin_amdgcn_cosf(fr), -__builtin_amdgcn_sinf(fr));
+      buf[i0] = make_float2(a.x + b.x, a.y + b.y);
+      buf[i1] = cmulf(make_float2(a.x - b.x, a.y - b.y), w);
+    }
+  }
+  __syncthreads();
+}
+
+// inverse (unscaled): bit-reversed order -> natural order
+__device__ __forceinline__ void fft_dit_inverse(float2* buf, int logm) {
+  const int M = 1 << logm;
+  for (int s = 0; s < logm; ++s) {
+    const int half = 1 << s;
+    const float inv = 1.0f / (float)(2 * half);
+    __syncthreads();
+    for (int j = threadIdx.x; j < M / 2; j += kFT) {
+      const int pos = j & (half - 1);
+      const int i0 = ((j >> s) << (s + 1)) + pos, i1 = i0 + half;
+      const float fr = (float)pos * inv;
+      const float2 w = make_float2(__builtin_amdgcn_cosf(fr), __builtin_amdgcn_sinf(fr));
+      const float2 a = buf[i0], t = cmulf(buf[i1], w);
+      buf[i0] = make_float2(a.x + t.x, a.y + t.y);
+      buf[i1] = make_float2(a.x - t.x, a.y - t.y);
+    }
+  }
+  __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFT) void long_conv_fft_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                            const float* __restrict__ k, int B, int D, int L, int Lk,
+                                                            int logm, int bidirectional, int shift) {
+  extern __shared__ float2 fbuf[];                   // M complex values
+  const int M = 1 << logm;
+  const int d = blockIdx.x;
+  constexpr int kPer = (1 << kFftMaxLog) / kFT;      // spectrum values per thread at the largest M
+  // ---- the kernel row(s) of the channel as one sequence of period M: lags 0 .. Lk - 1 at the front, the
+  // anti-causal taps of the second row at the back (offset m at index M - m)
+  for (int i = threadIdx.x; i < M; i += kFT) fbuf[i] = make_float2(i < Lk ? k[(size_t)d * Lk + i] : 0.f, 0.f);
+  if (bidirectional) {
+    __syncthreads();
+    const float* k2 = k + (size_t)(D + d) * Lk;
+    for (int tap = threadIdx.x; tap < Lk; tap += kFT) {
+      const int m = tap + (shift ? 1 : 0);           // x[t + m] meets tap m - 1 (shift) or m
+      const int idx = (M - m) & (M - 1);
+      fbuf[idx].x += k2[tap];
+    }
+  }
+  fft_dif(fbuf, logm);
+  float2 Kf[kPer];
+  const float scale = 1.0f / (float)M;
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) {
+    const int i = threadIdx.x + e * kFT;
+    Kf[e] = i < M ? make_float2(fbuf[i].x * scale, fbuf[i].y * scale) : make_float2(0.f, 0.f);
+  }
+  // ---- the rows of the channel, two at a time
+  for (int b = blockIdx.y * 2; b < B; b += 2 * gridDim.y) {
+    const bool two = b + 1 < B;
+    const T* x0 = x + ((size_t)b * D + d) * L;
+    const T* x1 = x + ((size_t)(b + 1) * D + d) * L;
+    __syncthreads();
+    for (int i = threadIdx.x; i < M; i += kFT)
+      fbuf[i] = i < L ? make_float2(to_float(x0[i]), two ? to_float(x1[i]) : 0.f) : make_float2(0.f, 0.f);
+    fft_dif(fbuf, logm);
+#pragma unroll
+    for (int e = 0; e < kPer; ++e) {
+      const int i = threadIdx.x + e * kFT;
+      if (i < M) fbuf[i] = cmulf(fbuf[i], Kf[e]);
+    }
+    fft_dit_inverse(fbuf, logm);
+    T* y0 = y + ((size_t)b * D + d) * L;
+    T* y1 = y + ((size_t)(b + 1) * D + d) * L;
+    for (int i = threadIdx.x; i < L; i += kFT) {
+      const float2 v = fbuf[i];
+      y0[i] = from_float<T>(v.x);
+      if (two) y1[i] = from_float<T>(v.y);
+    }
+  }
+}
+
+// the transform pays off once the kernel is long; it needs M = pow2ceil(L + Lk) complex values in LDS
+bool long_conv_fft_plan(int64_t L, int64_t Lk, int* logm) {
+  if (Lk < MEGA_LC_FFT_MIN) return false;
+  int lg = 0;
+  while (((int64_t)1 << lg) < L + Lk) ++lg;
+  if (lg > kFftMaxLog || lg < 11) return false;
+  *logm = lg;
+  return true;
+}
+
+template <typename T>
+int launch_long_conv_fft(const void* x, void* y, const float* k, int64_t B, int64_t D, int64_t L, int64_t Lk, int logm,
+                         int bidirectional, int shift, hipStream_t s) {
+  auto kern = long_conv_fft_kernel<T>;
+  const size_t smem = ((size_t)8) << logm;
+  static bool attr_set = false;
+  if (!attr_set) {
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 8 << kFftMaxLog);
+    attr_set = true;
+  }
+  // enough workgroups to fill the chip: split the batch when there are few channels
+  int64_t nb = 1;
+  while (D * nb < 512 && nb * 2 <= (B + 1) / 2) nb *= 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)D, (unsigned)nb), dim3(kFT), smem, s, (const T*)x, (T*)y, k, (int)B, (int)D,
+                     (int)L, (int)Lk, logm, bidirectional, shift);
+  MEGA_CHECK_LAUNCH("long_conv_fwd (transform path)");
+  return MEGA_OK;
+}
+
 }  // namespace
 }  // namespace mega
 
@@ -79,6 +220,14 @@ extern "C" int mega_long_conv_fwd(const void* x, void* y, int dtype, const float
   MEGA_REQUIRE(x && y && k, MEGA_ERR_ARG, "long_conv_fwd: null pointer argument");
   MEGA_REQUIRE(B * D < (int64_t)1 << 31 && L < (int64_t)65535 * kT, MEGA_ERR_UNSUPPORTED, "long_conv_fwd: shape too large");
   hipStream_t s = (hipStream_t)stream;
+  int logm = 0;
+  if (D < 65536 && long_conv_fft_plan(L, Lk, &logm)) {
+    switch (dtype) {
+      case MEGA_F32: return launch_long_conv_fft<float>(x, y, k, B, D, L, Lk, logm, bidirectional, shift, s);
+      case MEGA_BF16: return launch_long_conv_fft<bf16_t>(x, y, k, B, D, L, Lk, logm, bidirectional, shift, s);
+      default: return launch_long_conv_fft<f16_t>(x, y, k, B, D, L, Lk, logm, bidirectional, shift, s);
+    }
+  }
   const dim3 grid((unsigned)(B * D), (unsigned)ceil_div(L, kT));
   switch (dtype) {
     case MEGA_F32:

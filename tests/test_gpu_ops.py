@@ -57,6 +57,29 @@ def test_long_conv(dtype, Lk):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,D,L,Lk", [(3, 5, 4096, 4096), (1, 4, 5000, 3000), (2, 3, 8192, 8192), (5, 2, 1500, 512),
+                                      (2, 600, 2048, 2048)])
+def test_long_conv_transform_path(dtype, B, D, L, Lk):
+    """Kernels of 512 lags and more go through the Fourier transform in LDS (M = pow2ceil(L + Lk) <= 16384 points):
+    odd batch sizes (rows travel in pairs), M from 2048 to 16384, many channels; against numpy's convolution."""
+    print(f"case {dtype} B={B} D={D} L={L} Lk={Lk}", flush=True)
+    rng = np.random.default_rng(27)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    k = (rng.normal(size=(2 * D, Lk)) * np.exp(-np.arange(Lk) / 300.0) * 0.3).astype(np.float32)
+    sel = slice(0, min(D, 8))                      # the oracle's convolution is O(L Lk) per row
+    y = M.ops.fftconv(x, dev(k[:D]))
+    ref = O.causal_conv(x64[:, sel], np.pad(k[:D][sel].astype(np.float64), ((0, 0), (0, L - Lk))))
+    assert rel_err(host(y)[:, sel], ref) < TOL[dtype]
+    for shift in (True, False):
+        y = M.ops.bidirectional_fftconv(x, dev(k), shift)
+        kk = np.concatenate([k[:D][sel], k[D:][sel]], 0).astype(np.float64)
+        assert rel_err(host(y)[:, sel], O.bidirectional_conv(x64[:, sel], kk, shift)) < TOL[dtype]
+    if D > 8:                                      # the remaining channels against the first ones' code path: linearity
+        y2 = M.ops.fftconv(2 * x, dev(k[:D]))
+        assert rel_err(host(y2), 2 * host(M.ops.fftconv(x, dev(k[:D])))) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(3, 5, 40, 40), (2, 17, 300), (2, 64, 2048), (1, 6, 3)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_attention_softmax(dtype, shape, causal):
