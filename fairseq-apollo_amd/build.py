@@ -21,6 +21,7 @@ SOURCES = [
     "ema_scan.hip",
     "ema_mfma.hip",
     "norm_ema_fused.hip",
+    "ema_rows.hip",
     "ema_bwd.hip", "ema_bwd_tile.hip",
     "decode.hip",
     "elementwise.hip",

@@ -12,6 +12,8 @@ namespace mega {
 // and one slot in the layout of the 64-lane segment scan (kSlotScan: q^(32 kSEGT) of state lane >> 2).
 // kSlotKT (kNWK slots): the K operand once per distinct content, 56 vectors of 16 bytes per term; lane (m, g) of
 // row block mb finds its vector at byte 16 (16 mb + m - 8 g + 24).
+// kSlotK16 / kSlotP16 / kSlotC16 (4 slots each: term w, row block mb at 2 w + mb): the same three operands as two
+// fp16 terms (22 significant bits), for the kernel that serves fp32 / fp16 activations.
 constexpr int kNS = 16;                  // complex states per channel (zero padded)
 #ifndef MEGA_SEGT
 #define MEGA_SEGT 2
@@ -32,8 +34,9 @@ constexpr int kNWC = MEGA_NWC;           // bf16 terms of the state-output opera
 constexpr int kNOPS = 2 * (kNWK + kNWP + kNWC);
 constexpr int kSlotK = 0, kSlotP = 2 * kNWK, kSlotC = 2 * (kNWK + kNWP);
 constexpr int kSlotQ32 = kNOPS, kSlotScan = kNOPS + 2, kSlotRS = kNOPS + 3, kSlotRJ = kNOPS + 5, kSlotRW = kNOPS + 7,
-              kSlotRWJ = kNOPS + 9, kSlotCmp = kNOPS + 11, kSlotKT = kNOPS + 12;
-constexpr int kImgSlots = kNOPS + 12 + kNWK;
+              kSlotRWJ = kNOPS + 9, kSlotCmp = kNOPS + 11, kSlotKT = kNOPS + 12, kSlotK16 = kNOPS + 12 + kNWK,
+              kSlotP16 = kSlotK16 + 4, kSlotC16 = kSlotP16 + 4;
+constexpr int kImgSlots = kSlotC16 + 4;
 // kSlotCmp: per-state multipliers once each, six tables of 16 complex values (128 bytes = one line):
 // and one line of reach figures (how far the slowest pole of the channel carries before |q|^t < 2^-24):
 //   word 0: how many of the doubling steps 64, 128, 256, 512 tokens still matter (0..4)
@@ -58,5 +61,14 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
                  int64_t syd, int64_t syl, const float* p, const float* q, const void* image, int is_complex,
                  const float* omega, const uint8_t* mask, const float* h_in, float* h_out, int64_t B, int64_t D,
                  int64_t N, int64_t L, int bidirectional, int64_t Lk, float* acc, float* h_tile, hipStream_t s);
+
+// ---- [B, D, L] rows of any activation type, parallel over blocks of 1024 tokens (csrc/ema_rows.hip)
+size_t ema_rows_record_bytes(int64_t B, int64_t D, int64_t L, int bidirectional);
+bool ema_rows_covers(int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb, int64_t syd, int64_t syl,
+                     int64_t B, int64_t D, int64_t N, int64_t L, int64_t Lk, const float* h_out);
+int ema_rows_run(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t syb, int64_t syd,
+                 const void* image, int is_complex, const float* omega, const uint8_t* mask, const float* h_in,
+                 float* h_out, int64_t B, int64_t D, int64_t N, int64_t L, int bidirectional, float* acc, float* rec,
+                 hipStream_t s);
 
 }  // namespace mega

@@ -132,6 +132,8 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
   const int m = lane & 15, g = lane >> 4;
   int slot = 0;
   bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
+  typedef __attribute__((ext_vector_type(8))) _Float16 f16x8v;
+  f16x8v H16[3][2][2];                    // K, P, C as two fp16 terms
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int row = 16 * mb + m;
@@ -169,6 +171,15 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       rem = bf_split(cv, &h);
       Cw[0][mb][t] = h;
       if (kNWC > 1) Cw[kNWC - 1][mb][t] = (__bf16)rem;
+      {
+        const float vals[3] = {kv, pv, cv};
+#pragma unroll
+        for (int o = 0; o < 3; ++o) {
+          const _Float16 h16 = (_Float16)vals[o];
+          H16[o][0][mb][t] = h16;
+          H16[o][1][mb][t] = (_Float16)(vals[o] - (float)h16);
+        }
+      }
     }
   }
   if (ok) {
@@ -242,6 +253,13 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       v = cmul(v, v);
       cmp[kCmpRW * kNS + lane] = make_float2(v.re, v.im);
     }
+#pragma unroll
+    for (int o = 0; o < 3; ++o)
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+          img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
     if (lane < 56) {
       // the K operand once per distinct content: lane (m, g) of row block mb holds k[16 mb + m - 8 g - t], t = 0..7,
       // which depends on delta = 16 mb + m - 8 g (-24..31) only; vector delta + 24 of term w sits at byte

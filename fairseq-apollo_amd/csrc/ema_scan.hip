@@ -1056,7 +1056,7 @@ __global__ void coef_prep_kernel(const float* __restrict__ p, const float* __res
 
 struct Plan {
   int NP, TPR, Tc, nchunks;
-  size_t coef_bytes, st_bytes, acc_bytes, tile_bytes, image_bytes, total;
+  size_t coef_bytes, st_bytes, acc_bytes, tile_bytes, image_bytes, rows_bytes, total;
 };
 
 Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_acc, bool bidirectional = false) {
@@ -1084,7 +1084,8 @@ Plan make_plan(int64_t B, int64_t D, int64_t N, int64_t L, int nsets, bool need_
   (void)nsets;
   pl.tile_bytes = align_up((size_t)B * D * 16 * 2 * 4, 256);      // state after the last whole tile
   pl.image_bytes = align_up(ema_image_bytes(D, N, bidirectional ? 1 : 0), 256);   // when the caller brings none
-  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes + pl.image_bytes;
+  pl.rows_bytes = align_up(ema_rows_record_bytes(B, D, L, bidirectional ? 1 : 0), 256);   // block end states of the rows path
+  pl.total = pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes + pl.image_bytes + pl.rows_bytes;
   return pl;
 }
 
@@ -1372,7 +1373,22 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
   float* st = (float*)(w + pl.coef_bytes);
   float* acc = need_acc ? (float*)(w + pl.coef_bytes + pl.st_bytes) : nullptr;
   float* h_tile = (float*)(w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes);
-  if (ema_mfma_covers(dtype, sxb, sxd, sxl, syb, syd, syl, x, y, mask, B, D, N, L, Lk)) {
+  // [B, D, L] rows: fp32 / fp16 always, bf16 when the streaming kernel (one workgroup per 16 channels, the whole
+  // sequence) would leave most of the chip idle
+  const bool stream_ok = ema_mfma_covers(dtype, sxb, sxd, sxl, syb, syd, syl, x, y, mask, B, D, N, L, Lk);
+  if (ema_rows_covers(dtype, sxb, sxd, sxl, syb, syd, syl, B, D, N, L, Lk, h_out) &&
+      (!stream_ok || B * ceil_div(D, 16) < 128)) {
+    const void* img = image;
+    char* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
+    if (!img) {
+      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s);
+      if (rc) return rc;
+      img = wimg;
+    }
+    return ema_rows_run(x, y, dtype, sxb, sxd, syb, syd, img, is_complex, omega, mask, h_in, h_out, B, D, N, L,
+                        bidirectional, acc, (float*)(wimg + pl.image_bytes), s);
+  }
+  if (stream_ok) {
     const void* img = image;
     if (!img) {
       // no cached image: kernel generation runs with every call
