@@ -450,7 +450,7 @@ def bench_ema_real(args):
         "data": "synthetic",
         "config": {"workload": "configs[1]: bidirectional real MultiHeadEMA (N=16), B=1 L=16384 D=256, fp32, "
                                "right-padding mask; configs[0] beside it"},
-        "roofline": {"bound": "hbm", "kernel": "chunk_state_rows + chunk_scan + chunk_apply_rows, both directions",
+        "roofline": {"bound": "hbm", "kernel": "ema_rows_kernel: block end states, then both directions of every block (matrix cores, fp16 terms)",
                      "achieved": c1["hbm_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": c1["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_step": c1["algorithmic_bytes"]},

@@ -41,6 +41,8 @@ struct RowsArgs {
   int reverse;           // tokens are walked from the last to the first
   int B, D, N, L, S, R;
   int is_complex;
+  int both;              // both directions in this launch: forward as given, backward with rows D .. 2D - 1
+  int64_t rec_dir;       // floats from the forward records to the backward ones
 };
 
 __device__ __forceinline__ uint4 img_slot(const char* base, int slot, uint32_t lane_off) {
@@ -114,29 +116,52 @@ __device__ __forceinline__ int plane_off(int i) {
   return j * 128 + ((c8 ^ (j >> 1)) << 4) + e * 2;
 }
 
-// STATE: only the block's end state is wanted (first kernel).  NX: terms of x; F16: fp16 operands; VEC: rows, mask
-// and partial sums are aligned for four tokens per access and L is a multiple of 4
-template <typename T, int NX, bool F16, bool STATE, bool VEC>
+// STATE: only the block's end state is wanted (first kernel; with A.both the grid holds both directions).  NX: terms
+// of x; F16: fp16 operands; VEC: rows, mask and partial sums are aligned for four tokens per access and L is a
+// multiple of 4.  BOTH (second kernel, L a multiple of 1024, VEC): a wave forms both directions of its 1024 tokens
+// of memory, backward first, and adds them up in LDS, so that y is written once and no partial sums pass
+// through memory.
+template <typename T, int NX, bool F16, bool STATE, bool VEC, bool BOTH>
 __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A) {
-  __shared__ __attribute__((aligned(16))) char lds[kRW * kRWaveLds];
+  constexpr int kWaveLds = (BOTH ? 2 : 1) * kRWaveLds;
+  __shared__ __attribute__((aligned(16))) char lds[kRW * kWaveLds];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int nrg = (A.R + kRW - 1) / kRW;
-  const int s = (int)blockIdx.x / nrg;                  // time-major: the early blocks of all rows first
-  const int row = ((int)blockIdx.x - s * nrg) * kRW + wave;
+  int bid = (int)blockIdx.x, dirsel = 0;
+  if (STATE && A.both) {
+    const int per = nrg * (A.S - 1);
+    dirsel = bid >= per ? 1 : 0;
+    bid -= dirsel * per;
+  }
+  const int sm = bid / nrg;                             // time-major: the early blocks of all rows first
+  const int row = (bid - sm * nrg) * kRW + wave;
   if (row >= A.R) return;
   const int b = row / A.D, d = row - b * A.D;
   const int j = lane & 15, r = lane >> 4;
-  char* plane = lds + wave * kRWaveLds;                 // hi plane at 0, lo plane at 2048
+  char* plane = lds + wave * kWaveLds;                  // hi plane at 0, lo plane at 2048
+  float* ys = (float*)(plane + (BOTH ? kRWaveLds : 0)); // y as fp32 (over the used-up x unless both directions meet here)
   const T* xr = (const T*)A.x + (size_t)b * A.sxb + (size_t)d * A.sxd;
-  const int i0 = s * kRBlk;                             // first token of the block in walking order
-  const char* img = (const char*)A.image + (size_t)(A.koff + d) * kImgRowBytes;
   const uint32_t loff = (uint32_t)lane * 16, roff = (uint32_t)r * 16;
+  constexpr int NL = 8;                                // loads in flight per lane and round (element-wise path)
+  const uint8_t* mrow = A.mask ? A.mask + (size_t)b * A.L : nullptr;
+  int reverse = 0, i0 = 0;
+#pragma unroll 1
+  for (int pass = 0; pass < (BOTH ? 2 : 1); ++pass) {
+  // this pass's direction: its block in walking order, coefficient rows, records and carried states
+  const bool back = BOTH ? pass == 0 : (STATE && dirsel) ? true : A.reverse != 0;
+  const bool second = BOTH || (STATE && A.both);         // the launch covers both directions
+  reverse = back ? 1 : 0;
+  const int s = (BOTH && back) ? A.S - 1 - sm : sm;
+  const int koff = second ? (back ? A.D : 0) : A.koff;
+  float* rec = A.rec + ((second && back) ? A.rec_dir : 0);
+  const float* h_in = (second && back) ? nullptr : A.h_in;
+  float* h_out = (second && back) ? nullptr : A.h_out;
+  i0 = s * kRBlk;                                       // first token of the block in walking order
+  const char* img = (const char*)A.image + (size_t)(koff + d) * kImgRowBytes;
 
   // ---- the block of x into LDS as two 16-bit planes (masked and out-of-range tokens as zeros); every load of
   // the block is requested before the first one is used
-  constexpr int NL = 8;                                // loads in flight per lane and round (element-wise path)
-  const uint8_t* mrow = A.mask ? A.mask + (size_t)b * A.L : nullptr;
   if (VEC) {
     // four consecutive tokens per lane and access, all requested at once
     Vec<T, 4> xq[4];
@@ -145,7 +170,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
     for (int m = 0; m < 4; ++m) {
       const int w = i0 + m * 256 + 4 * lane;
       const int wc = w < A.L ? w : A.L - 4;
-      const int t = A.reverse ? A.L - 4 - wc : wc;       // first of the four in memory
+      const int t = reverse ? A.L - 4 - wc : wc;         // first of the four in memory
       xq[m] = *(const Vec<T, 4>*)(xr + t);
       mq[m] = mrow ? *(const uint32_t*)(mrow + t) : 0u;
     }
@@ -156,7 +181,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
       uint16_t hi[4], lo[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int src = A.reverse ? 3 - e : e;           // memory element of walking token e
+        const int src = reverse ? 3 - e : e;             // memory element of walking token e
         const bool masked = ((mq[m] >> (8 * src)) & 0xffu) != 0u;
         const float v = (in && !masked) ? to_float(xq[m].v[src]) : 0.f;
         split16<F16>(v, &hi[e], &lo[e]);
@@ -174,7 +199,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
     for (int k = 0; k < NL; ++k) {
       const int w = i0 + (k0 + k) * 64 + lane;
       const int wc = w < A.L ? w : A.L - 1;
-      const int t = A.reverse ? A.L - 1 - wc : wc;
+      const int t = reverse ? A.L - 1 - wc : wc;
       xv[k] = to_float(xr[t]);
       mk[k] = mrow ? mrow[t] : (uint8_t)0;
     }
@@ -205,7 +230,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
   load_cmp(img, kCmpRS, roff, RSr, RSi);
   const uint2 reach = *(const uint2*)(img + kSlotCmp * 1024 + kCmpReach * 128);
   const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
-  const int nterms = s + (A.h_in ? 1 : 0);
+  const int nterms = s + (h_in ? 1 : 0);
   float RWJr[4], RWJi[4], RWr[4], RWi[4], RJr[4], RJi[4], tr[4], ti[4];
   uint4 Kw[2][2], Cw[NC][2];
   if (!STATE) {
@@ -216,17 +241,17 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
 #pragma unroll
     for (int u = 0; u < 4; ++u) tr[u] = ti[u] = 0.f;
     if (j < s) {
-      const float* e = A.rec + ((size_t)row * A.S + (s - 1 - j)) * kRecF;
+      const float* e = rec + ((size_t)row * A.S + (s - 1 - j)) * kRecF;
       const float4 a = *(const float4*)(e + (2 * r) * 2), c = *(const float4*)(e + (8 + 2 * r) * 2);
       tr[0] = a.x; ti[0] = a.y; tr[1] = a.z; ti[1] = a.w;
       tr[2] = c.x; ti[2] = c.y; tr[3] = c.z; ti[3] = c.w;
-    } else if (A.h_in && j == s) {
+    } else if (h_in && j == s) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         if (nn[u] < A.N) {
           const size_t o = (((size_t)b * A.D + d) * A.N + nn[u]) * 2;
-          tr[u] = A.h_in[o];
-          ti[u] = A.is_complex ? A.h_in[o + 1] : 0.f;
+          tr[u] = h_in[o];
+          ti[u] = A.is_complex ? h_in[o + 1] : 0.f;
         }
       }
     }
@@ -305,7 +330,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
   if (STATE) {
     // lane 15 of a row holds the block's end state from a zero start
     if (j == 15) {
-      float* e = A.rec + ((size_t)row * A.S + s) * kRecF;
+      float* e = rec + ((size_t)row * A.S + s) * kRecF;
       *(float4*)(e + (2 * r) * 2) = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
       *(float4*)(e + (8 + 2 * r) * 2) = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
     }
@@ -325,14 +350,14 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
       Ci[u] = group_sum<16>(have ? ci : 0.f);
     }
   }
-  if (A.h_out && s == A.S - 1 && j == 15) {
+  if (h_out && s == A.S - 1 && j == 15) {
     // state after the last token: the block's own end state plus q^1024 times what it inherited
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       if (nn[u] < A.N) {
         const size_t o = (((size_t)b * A.D + d) * A.N + nn[u]) * 2;
-        A.h_out[o] = fmaf(RWr[u], Cr[u], fmaf(-RWi[u], Ci[u], Er[u]));
-        A.h_out[o + 1] = fmaf(RWr[u], Ci[u], fmaf(RWi[u], Cr[u], Ei[u]));
+        h_out[o] = fmaf(RWr[u], Cr[u], fmaf(-RWi[u], Ci[u], Er[u]));
+        h_out[o + 1] = fmaf(RWr[u], Ci[u], fmaf(RWi[u], Cr[u], Ei[u]));
       }
     }
   }
@@ -400,13 +425,31 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
   // XOR-swizzled by the segment so that the 16 segments' stores fall on different banks) and out in whole runs
   // of 64 tokens
   __builtin_amdgcn_wave_barrier();
-  float* ys = (float*)plane;
+  if (BOTH && back) {
+    // in the order of memory: walking piece (j, c) is piece (15 - j, 15 - c) there, its four tokens reversed
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
-      *(float4*)(ys + j * 64 + (((t * 8 + h * 4 + r) ^ j) & 15) * 4) = make_float4(Y[t][h][0], Y[t][h][1], Y[t][h][2], Y[t][h][3]);
+      for (int h = 0; h < 2; ++h) {
+        const int jm = 15 - j, cm = 15 - (t * 8 + h * 4 + r);
+        *(float4*)(ys + jm * 64 + ((cm ^ jm) & 15) * 4) = make_float4(Y[t][h][3], Y[t][h][2], Y[t][h][1], Y[t][h][0]);
+      }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float4* at = (float4*)(ys + j * 64 + (((t * 8 + h * 4 + r) ^ j) & 15) * 4);
+        float4 v = make_float4(Y[t][h][0], Y[t][h][1], Y[t][h][2], Y[t][h][3]);
+        if (BOTH) {
+          const float4 o = *at;
+          v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+        }
+        *at = v;
+      }
+  }
   __builtin_amdgcn_wave_barrier();
+  }  // pass
   T* yr = (T*)A.y + (size_t)b * A.syb + (size_t)d * A.syd;
   float* ar = A.acc ? A.acc + ((size_t)b * A.D + d) * A.L : nullptr;
   const bool resid = A.omega && A.mask;                  // masked tokens keep their residual omega x
@@ -417,7 +460,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
     for (int m = 0; m < 4; ++m) {
       const int w = i0 + m * 256 + 4 * lane;
       const int wc = w < A.L ? w : A.L - 4;
-      const int t = A.reverse ? A.L - 4 - wc : wc;
+      const int t = reverse ? A.L - 4 - wc : wc;
       add[m] = make_float4(0.f, 0.f, 0.f, 0.f);
       if (A.acc_mode == 2) add[m] = *(const float4*)(ar + t);
       if (resid) {
@@ -434,10 +477,10 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
       const int i = m * 256 + 4 * lane;
       const int w = i0 + i;
       if (w < A.L) {
-        const int t = A.reverse ? A.L - 4 - w : w;
+        const int t = reverse ? A.L - 4 - w : w;
         const float4 yv = *(const float4*)(ys + (i & ~63) + (((((i & 63) >> 2) ^ (i >> 6)) & 15) << 2));
         // memory order: the four walking tokens reversed when time runs backwards
-        float4 v = A.reverse ? make_float4(yv.w, yv.z, yv.y, yv.x) : yv;
+        float4 v = reverse ? make_float4(yv.w, yv.z, yv.y, yv.x) : yv;
         v.x += add[m].x; v.y += add[m].y; v.z += add[m].z; v.w += add[m].w;
         if (A.acc_mode == 1) {
           *(float4*)(ar + t) = v;
@@ -457,7 +500,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
     for (int k = 0; k < NL; ++k) {
       const int w = i0 + (k0 + k) * 64 + lane;
       const int wc = w < A.L ? w : A.L - 1;
-      const int t = A.reverse ? A.L - 1 - wc : wc;
+      const int t = reverse ? A.L - 1 - wc : wc;
       add[k] = 0.f;
       if (A.acc_mode == 2) add[k] = ar[t];
       if (resid) {                                       // both loads unconditional: no load waits for another
@@ -471,7 +514,7 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
       const int i = (k0 + k) * 64 + lane;
       const int w = i0 + i;
       if (w < A.L) {
-        const int t = A.reverse ? A.L - 1 - w : w;
+        const int t = reverse ? A.L - 1 - w : w;
         const float v = ys[(i & ~63) + (((((i & 63) >> 2) ^ (i >> 6)) & 15) << 2) + (i & 3)] + add[k];
         if (A.acc_mode == 1) ar[t] = v;
         else yr[t] = from_float<T>(v);
@@ -483,23 +526,34 @@ __global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A)
 template <typename T, int NX, bool F16, bool VEC>
 int launch_rows_v(const RowsArgs& A, hipStream_t s) {
   const int nrg = (A.R + kRW - 1) / kRW;
+  const unsigned per_state = (unsigned)(nrg * (A.S - 1)), per_apply = (unsigned)(nrg * A.S);
   if (A.S > 1) {
-    // end states of the blocks 0 .. S - 2 (nobody inherits from the last one)
-    hipLaunchKernelGGL((ema_rows_kernel<T, NX, F16, true, VEC>), dim3((unsigned)(nrg * (A.S - 1))), dim3(64 * kRW), 0, s, A);
+    // end states of the blocks 0 .. S - 2 (nobody inherits from the last one), of both directions when asked
+    hipLaunchKernelGGL((ema_rows_kernel<T, NX, F16, true, VEC, false>), dim3(per_state * (A.both ? 2 : 1)), dim3(64 * kRW),
+                       0, s, A);
   }
-  hipLaunchKernelGGL((ema_rows_kernel<T, NX, F16, false, VEC>), dim3((unsigned)(nrg * A.S)), dim3(64 * kRW), 0, s, A);
+  if (A.both) {
+    if constexpr (VEC)
+      hipLaunchKernelGGL((ema_rows_kernel<T, NX, F16, false, true, true>), dim3(per_apply), dim3(64 * kRW), 0, s, A);
+  } else {
+    hipLaunchKernelGGL((ema_rows_kernel<T, NX, F16, false, VEC, false>), dim3(per_apply), dim3(64 * kRW), 0, s, A);
+  }
   MEGA_CHECK_LAUNCH("ema_fwd (rows on the matrix cores)");
   return MEGA_OK;
 }
 
+// four tokens per access when every row, the mask and the partial sums start on such a boundary
+template <typename T>
+bool rows_vec_ok(const RowsArgs& A) {
+  const size_t al = 4 * sizeof(T);
+  return A.L % 4 == 0 && A.L >= 4 && ((uintptr_t)A.x % al) == 0 && ((uintptr_t)A.y % al) == 0 &&
+         A.sxb % 4 == 0 && A.sxd % 4 == 0 && A.syb % 4 == 0 && A.syd % 4 == 0 &&
+         (!A.mask || ((uintptr_t)A.mask % 4) == 0) && (!A.acc || ((uintptr_t)A.acc % 16) == 0);
+}
+
 template <typename T, int NX, bool F16>
 int launch_rows(const RowsArgs& A, hipStream_t s) {
-  // four tokens per access when every row, the mask and the partial sums start on such a boundary
-  const size_t al = 4 * sizeof(T);
-  const bool vec = A.L % 4 == 0 && A.L >= 4 && ((uintptr_t)A.x % al) == 0 && ((uintptr_t)A.y % al) == 0 &&
-                   A.sxb % 4 == 0 && A.sxd % 4 == 0 && A.syb % 4 == 0 && A.syd % 4 == 0 &&
-                   (!A.mask || ((uintptr_t)A.mask % 4) == 0) && (!A.acc || ((uintptr_t)A.acc % 16) == 0);
-  return vec ? launch_rows_v<T, NX, F16, true>(A, s) : launch_rows_v<T, NX, F16, false>(A, s);
+  return rows_vec_ok<T>(A) ? launch_rows_v<T, NX, F16, true>(A, s) : launch_rows_v<T, NX, F16, false>(A, s);
 }
 
 }  // namespace
@@ -516,7 +570,7 @@ bool ema_rows_covers(int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t s
   if (N > kNS || Lk > 0 || sxl != 1 || syl != 1 || L < 64) return false;
   if (ceil_div(L, kRBlk) > 16) return false;
   if (h_out && L % kRBlk != 0) return false;           // the state after the last token of a partial block
-  if (B * D >= (int64_t)1 << 28) return false;
+  if (B * D >= (int64_t)1 << 26) return false;          // the grids stay below 2^31 workgroups
   (void)dtype; (void)sxb; (void)sxd; (void)syb; (void)syd;
   return true;
 }
@@ -529,6 +583,7 @@ int ema_rows_run(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
   A.x = x; A.y = y; A.sxb = sxb; A.sxd = sxd; A.syb = syb; A.syd = syd; A.mask = mask;
   A.image = (const uint4*)image; A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
   A.S = (int)ceil_div(L, kRBlk); A.R = (int)(B * D); A.is_complex = is_complex;
+  A.both = 0; A.rec_dir = (int64_t)B * D * A.S * kRecF;
   auto launch = [&](const RowsArgs& a) -> int {
     switch (dtype) {
       case MEGA_F32: return launch_rows<float, 2, true>(a, s);
@@ -536,18 +591,24 @@ int ema_rows_run(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
       default: return launch_rows<bf16_t, 1, false>(a, s);
     }
   };
+  A.koff = 0; A.reverse = 0; A.omega = mask ? omega : nullptr; A.h_in = h_in; A.h_out = h_out;
+  A.acc = nullptr; A.acc_mode = 0; A.rec = rec;
   if (bidirectional) {
+    const bool vec = dtype == MEGA_F32 ? rows_vec_ok<float>(A) : rows_vec_ok<bf16_t>(A);
+    if (vec && L % kRBlk == 0) {
+      // whole blocks: the two directions of a block of memory meet inside one wave
+      A.both = 1;
+      return launch(A);
+    }
     // the direction back in time first, into the fp32 partial sums
     RowsArgs Bk = A;
     Bk.koff = (int)D; Bk.reverse = 1; Bk.omega = nullptr; Bk.h_in = nullptr; Bk.h_out = nullptr;
     Bk.acc = acc; Bk.acc_mode = 1;
-    Bk.rec = rec + (size_t)B * D * A.S * kRecF;
+    Bk.rec = rec + A.rec_dir;
     const int rc = launch(Bk);
     if (rc) return rc;
+    A.acc = acc; A.acc_mode = 2;
   }
-  A.koff = 0; A.reverse = 0; A.omega = mask ? omega : nullptr; A.h_in = h_in; A.h_out = h_out;
-  A.acc = bidirectional ? acc : nullptr; A.acc_mode = bidirectional ? 2 : 0;
-  A.rec = rec;
   return launch(A);
 }
 

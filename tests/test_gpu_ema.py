@@ -120,6 +120,28 @@ def test_bidirectional(shift, trunc, cplx, L, dtype):
     assert rel_err(host(y), yo) < TOL[dtype]
 
 
+@pytest.mark.parametrize("shift", [True, False])
+@pytest.mark.parametrize("cplx", [False, True])
+@pytest.mark.parametrize("L", [1024, 3072])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_bidirectional_whole_blocks(shift, cplx, L, dtype):
+    """Whole blocks of 1024 tokens: the two directions of a block are formed by one wave and meet before y is
+    written; masked tokens in the middle of the rows, not only at their ends."""
+    rng = np.random.default_rng(15)
+    B, D, N = 2, 10, 16
+    p, q, g = _coeffs(rng, 2 * D, N, cplx)
+    om = rng.normal(size=D)
+    x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+    mask = rng.random((B, L)) < 0.05
+    mask[1, L - 100:] = True
+    y, _ = _run(x, p, q, g, om, padding_mask=dev(mask, torch.bool), bidirectional=True, shift=shift)
+    yo, _ = O.ema_forward(x64, p, q, g, om, mask, bidirectional=True, shift=shift)
+    assert rel_err(host(y), yo) < TOL[dtype]
+    y2, _ = _run(x, p, q, g, om, bidirectional=True, shift=shift)
+    yo2, _ = O.ema_forward(x64, p, q, g, om, None, bidirectional=True, shift=shift)
+    assert rel_err(host(y2), yo2) < TOL[dtype]
+
+
 def test_modules_forward():
     torch.manual_seed(3)
     B, D, N, L = 2, 32, 16, 128
