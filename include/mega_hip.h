@@ -122,7 +122,12 @@ int mega_ema_hidden_fwd(const void* x, int dtype, int64_t sxb, int64_t sxd, int6
  *   truncation  <= 0: kernel length L; otherwise min(truncation, L)
  *   shift   bidirectional only: 1 = the backward half starts at lag 1
  *   image   operand images from mega_ema_prepare for the same coefficients, or NULL: then
- *           kernel generation runs inside this call (into the workspace)                 */
+ *           kernel generation runs inside this call (into the workspace)
+ * All three activation types run on the matrix cores for ndim <= 16 without truncation, as the
+ * reference's convolution serves them alike (ops/fftconv_kernel.cu:214-269): bf16 in either
+ * layout; fp32 / fp16 on [B,D,L] rows (sxl = syl = 1) of up to 16384 tokens, where fp32 values
+ * and operands travel as two fp16 terms (error ~ 2^-22 of the largest term, accumulation in
+ * fp32).  Other cases take the chunked scan on the vector ALUs.                            */
 size_t mega_ema_fwd_workspace_bytes(int64_t B, int64_t D, int64_t N, int64_t L,
                                     int bidirectional, int64_t truncation);
 int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, int64_t sxl,
@@ -135,8 +140,8 @@ int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
 
 /* EMA kernel generation for the matrix-core path: from the coefficients to per-channel
  * operand images (the 32-tap Toeplitz block of k[l] = Re sum_n p gamma q^l, the state
- * input / output blocks p q^{31-i} and gamma q^{i+1}, and q^32), 9-13 KB per coefficient
- * row whatever L is.  Stands in for what the reference recomputes or caches per call:
+ * input / output blocks p q^{31-i} and gamma q^{i+1} as bf16 and as fp16 terms, and the
+ * powers of q that join tiles, segments and blocks), 36 KB per coefficient row whatever L is.  Stands in for what the reference recomputes or caches per call:
  * _compute_kernel / ema_parameters (fairseq/modules/complex_exponential_moving_average.py:
  * 98-109, fairseq/csrc/ops/ema_parameters_kernel.cu:40-66) and the eval-mode `_coeffs`
  * cache (fairseq/modules/base_moving_average.py:52-58).  The image is valid while p, q,
@@ -255,7 +260,10 @@ int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, i
  * fused CUDA op fftconv_fwd, ops/fftconv_kernel.cu:431-470) and
  * bidirectional_fftconv (fused_ops/fftconv.py:85-100).
  *   x, y [B,D,L] contiguous of `dtype`; k [K,Lk] fp32, K = D (causal) or 2D
- *   (bidirectional), Lk <= L.                                                    */
+ *   (bidirectional), Lk <= L.  Kernels of 512 lags and more with L + Lk <= 16384
+ *   go through a Fourier transform held in LDS (fp32, two batch rows per complex
+ *   transform, as fftconv_kernel.cu does with registers and shared memory); shorter
+ *   kernels and longer rows take the direct sum.                                  */
 int mega_long_conv_fwd(const void* x, void* y, int dtype, const float* k, int64_t B,
                        int64_t D, int64_t L, int64_t Lk, int bidirectional, int shift,
                        void* stream);
