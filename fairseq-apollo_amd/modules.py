@@ -176,9 +176,7 @@ class BaseMovingLayer(nn.Module, IncrementalState):
             'Bidirectional EMA does not support incremental state'
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
             if incremental_state is not None or (self.truncation is not None and self.truncation >= 1):
-                raise NotImplementedError(
-                    f"{type(self).__name__}: the backward pass covers layers without carried state or kernel "
-                    "truncation; call other configurations under torch.no_grad()")
+                return self._chained_forward(x, padding_mask, incremental_state, out_layout)
             p, q, gamma = self._calc_coeffs()           # stays in the graph
             return MovingAverageFunc.apply(x, p, q, gamma, self.omega, padding_mask, out_layout, self.bidirectional,
                                            self.shift)
@@ -191,6 +189,36 @@ class BaseMovingLayer(nn.Module, IncrementalState):
             self._set_input_buffer(incremental_state, saved_state)
         else:
             out, _ = layer(x, padding_mask, None, want_state=False, out_layout=out_layout)
+        return out
+
+    def _chained_forward(self, x, padding_mask, incremental_state, out_layout):
+        """Training with a carried state or a truncated kernel: the reference's own chain of differentiable
+        operators (base_moving_average.py:139-171): kernel and state bias from ema_parameters, the explicit
+        convolution, ema_hidden for the next state.  The kernel [K, L] is materialised here; the one-operator
+        path of the common case (no state, no truncation) never forms it."""
+        bsz, embed_dim, seq_len = x.size()
+        p, q, gamma = self._calc_coeffs()
+        p, q = p.squeeze(-1), q.squeeze(-1)
+        residual = x * self.omega.reshape(1, -1, 1).to(x.dtype)
+        xm = x if padding_mask is None else x * (1.0 - padding_mask.unsqueeze(1).to(x.dtype))
+        if incremental_state is not None:
+            saved_state = self._get_input_buffer(incremental_state)
+            h = saved_state['prev_state'] if 'prev_state' in saved_state else None
+            k, b = ops.ema_parameters(p, q, gamma, h, seq_len)
+            out = ops.fftconv(xm, k)
+            if b is not None:
+                out = out + b.to(out.dtype)
+            saved_state['prev_state'] = ops.ema_hidden(xm, p, q, h)
+            self._set_input_buffer(incremental_state, saved_state)
+        else:
+            kernel_size = min(self.truncation, seq_len)
+            k, _ = ops.ema_parameters(p, q, gamma, None, kernel_size)
+            out = ops.bidirectional_fftconv(xm, k, self.shift) if self.bidirectional else ops.fftconv(xm, k)
+        out = out + residual
+        if out_layout == "input" and out.stride() != x.stride():
+            y = torch.empty_like(x)                     # keeps x's strides
+            y.copy_(out)
+            return y
         return out
 
     def _prepared_layer(self) -> "ops.PreparedEMA":

@@ -869,6 +869,69 @@ def fftconv(x: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     return _long_conv(x, k, False, True)
 
 
+class _EMAParametersFunc(torch.autograd.Function):
+    """fairseq/modules/fused_ops/ema_parameters.py:11-35 (EMAParametersFunc): kernel and carried-state bias
+    from the coefficients, differentiable in p, q, gamma and h."""
+
+    @staticmethod
+    def forward(ctx, p, q, gamma, h, length):
+        log_q = q.detach().log()
+        w, b, _ = ema_parameters_fwd(p, log_q, gamma, h, length)
+        ctx.save_for_backward(p, log_q, gamma, h)
+        return w, b
+
+    @staticmethod
+    def backward(ctx, w_grad, b_grad):
+        p, log_q, gamma, h = ctx.saved_tensors
+        if h is None:
+            b_grad = None
+        elif b_grad is None:
+            b_grad = torch.zeros(h.shape[0], p.shape[0], w_grad.shape[-1], dtype=torch.float32, device=w_grad.device)
+        p_grad, q_grad, gamma_grad, h_grad = ema_parameters_bwd(w_grad, b_grad, p, log_q, gamma, h)
+        return (_like_input(p_grad, p), _like_input(q_grad, log_q, p.shape), _like_input(gamma_grad, gamma),
+                None if h is None else _like_input(h_grad, h), None)
+
+
+class _EMAHiddenFunc(torch.autograd.Function):
+    """fairseq/modules/fused_ops/ema_hidden.py:8-30 (EMAHiddenFunc): the state after the last token,
+    differentiable in x, p, q and h."""
+
+    @staticmethod
+    def forward(ctx, x, p, q, h):
+        log_q = q.detach().log()
+        y, _ = ema_hidden_fwd(x, p, log_q, h)
+        ctx.save_for_backward(x, p, log_q, h)
+        return y if log_q.is_complex() else y.real.contiguous()
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        x, p, log_q, h = ctx.saved_tensors
+        x_grad, p_grad, q_grad, h_grad = ema_hidden_bwd(y_grad, x, p, log_q, h)
+        return (x_grad.to(x.dtype), _like_input(p_grad, p), _like_input(q_grad, log_q, p.shape),
+                None if h is None else _like_input(h_grad, h))
+
+
+def _like_input(g: torch.Tensor, t: torch.Tensor, shape=None) -> torch.Tensor:
+    """A gradient in the type (real or complex) and shape of the input it belongs to."""
+    if not t.is_complex() and g.is_complex():
+        g = g.real
+    g = g.to(torch.complex64 if t.is_complex() else t.dtype)
+    return g.reshape(t.shape if shape is None else shape).contiguous()
+
+
+def ema_parameters(p: torch.Tensor, q: torch.Tensor, gamma: torch.Tensor, h: Optional[torch.Tensor], length: int):
+    """-> (k [K, length] fp32, b [B, K, length] fp32 or None): k[l] = Re sum_n p gamma q^l and the carried
+    state's contribution b[l] = Re sum_n gamma q^(l+1) h, differentiable (ema_parameters,
+    fairseq/modules/fused_ops/ema_parameters.py:11-35).  p, q: [K, N]; gamma: [K, N]; h: [B, K, N] or None."""
+    return _EMAParametersFunc.apply(p, q, gamma, h, length)
+
+
+def ema_hidden(x: torch.Tensor, p: torch.Tensor, q: torch.Tensor, h: Optional[torch.Tensor]) -> torch.Tensor:
+    """-> h' [B, D, N] = q^L h + sum_j p q^(L-1-j) x[j], differentiable (ema_hidden,
+    fairseq/modules/fused_ops/ema_hidden.py:8-30); real for real coefficients."""
+    return _EMAHiddenFunc.apply(x, p, q, h)
+
+
 def _rfft_len(L: int) -> int:
     """Length of the real transform the reference's convolution uses: 2 * pow2ceil(L)
     (fused_ops/fftconv.py:17-18, 47)."""
@@ -936,7 +999,17 @@ def fftconv_bwd(y_grad: torch.Tensor, x: torch.Tensor, k: torch.Tensor, k_dtype:
 
 
 def bidirectional_fftconv(x: torch.Tensor, k: torch.Tensor, shift: bool = True) -> torch.Tensor:
-    """bidirectional_fftconv, fairseq/modules/fused_ops/fftconv.py:85-100; k is [2D, Lk]."""
+    """bidirectional_fftconv, fairseq/modules/fused_ops/fftconv.py:85-100; k is [2D, Lk]:
+    y[t] = sum_l k1[l] x[t-l] + sum_l k2[l] x[t+l+1] (shift) or x[t+l] (no shift).  Under autograd the two
+    halves run as two causal convolutions, the second one over reversed time (the reference's is plain
+    torch.fft and differentiable the same way)."""
+    if torch.is_grad_enabled() and (x.requires_grad or k.requires_grad):
+        D = x.size(1)
+        fwd = fftconv(x, k[:D])
+        back = fftconv(x.flip(-1), k[D:]).flip(-1)
+        if shift:
+            back = torch.nn.functional.pad(back[..., 1:], (0, 1))
+        return fwd + back
     return _long_conv(x, k, True, shift)
 
 

@@ -249,6 +249,94 @@ def test_moving_average_module_autograd(cls, N):
     assert rel_err(host(x.grad), dxo) < 1e-4
 
 
+def _fd_check(rng, names, P, grads, loss, eps=1e-5, tol=2e-3, picks=4):
+    for n in names:
+        grad = grads[n]
+        scale = np.abs(grad).max() + 1e-6
+        for _ in range(picks):
+            idx = tuple(rng.integers(0, s) for s in P[n].shape)
+            Pp = {k: v.copy() for k, v in P.items()}; Pp[n][idx] += eps
+            Pm = {k: v.copy() for k, v in P.items()}; Pm[n][idx] -= eps
+            fd = (loss(Pp) - loss(Pm)) / (2 * eps)
+            assert abs(fd - grad[idx]) < tol * scale, (n, idx, fd, grad[idx])
+
+
+@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("cls,N", [("cema", 16), ("ema", 4)])
+def test_training_with_carried_state(cls, N, masked):
+    """Two chunks in training mode with the state carried between them (base_moving_average.py:139-160: kernel and
+    bias from ema_parameters, ema_hidden for the next state): outputs against the oracle on the whole sequence,
+    gradients of the raw parameters and of x (through both chunks and the state) against central differences of
+    the fp64 oracle."""
+    rng = np.random.default_rng(71)
+    B, D, L1, L2 = 2, 8, 40, 56
+    torch.manual_seed(6)
+    mod = (M.MultiHeadComplexEMA if cls == "cema" else M.MultiHeadEMA)(D, ndim=N).to(DEV).train()
+    x64 = rng.normal(size=(B, D, L1 + L2)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, D, L1 + L2)).astype(np.float32).astype(np.float64)
+    mask = None
+    if masked:
+        mask = np.zeros((B, L1 + L2), bool); mask[0, 30:35] = True; mask[1, L1 + 20:] = True
+    x = dev(x64).requires_grad_(True)
+    state = {}
+    tm = None if mask is None else dev(mask, torch.bool)
+    y1 = mod(x[:, :, :L1], None if tm is None else tm[:, :L1], incremental_state=state)
+    y2 = mod(x[:, :, L1:], None if tm is None else tm[:, L1:], incremental_state=state)
+    y = torch.cat([y1, y2], dim=-1)
+    names = ["alpha", "delta", "theta" if cls == "cema" else "beta", "gamma", "omega"]
+    P = {n: host(getattr(mod, n)) for n in names}
+    P["x"] = x64
+
+    def run(Pd):
+        if cls == "cema":
+            p, q, g = O.ema_coeffs_complex(Pd["alpha"], Pd["delta"], Pd["theta"], Pd["gamma"])
+        else:
+            p, q, g = O.ema_coeffs_real(Pd["alpha"], Pd["delta"], Pd["beta"], Pd["gamma"])
+        return O.ema_forward(Pd["x"], p, q, g, Pd["omega"].reshape(-1), mask)[0]
+
+    assert rel_err(host(y), run(P)) < 1e-4          # the chunked call equals the whole sequence
+    (y * dev(w64)).sum().backward()
+    grads = {n: host(getattr(mod, n).grad) for n in names}
+    grads["x"] = host(x.grad)
+    _fd_check(rng, names + ["x"], P, grads, lambda Pd: (run(Pd) * w64).sum())
+
+
+@pytest.mark.parametrize("shift", [True, False])
+@pytest.mark.parametrize("cls,N", [("cema", 16), ("ema", 4)])
+def test_training_with_truncated_kernel(cls, N, shift):
+    """A two-sided layer whose kernel is cut to `truncation` lags, in training mode: output against the oracle,
+    gradients against its central differences."""
+    rng = np.random.default_rng(72)
+    B, D, L, trunc = 2, 6, 90, 24
+    torch.manual_seed(7)
+    mod = (M.MultiHeadComplexEMA if cls == "cema" else M.MultiHeadEMA)(D, ndim=N, bidirectional=True, truncation=trunc,
+                                                                      shift=shift).to(DEV).train()
+    x64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    w64 = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64)
+    mask = np.zeros((B, L), bool); mask[1, L - 17:] = True
+    x = dev(x64).requires_grad_(True)
+    y = mod(x, dev(mask, torch.bool))
+    names = ["alpha", "delta", "theta" if cls == "cema" else "beta", "gamma", "omega"]
+    P = {n: host(getattr(mod, n)) for n in names}
+    P["x"] = x64
+
+    def run(Pd):
+        if cls == "cema":
+            p, q, g = O.ema_coeffs_complex(Pd["alpha"], Pd["delta"], Pd["theta"], Pd["gamma"])
+        else:
+            p, q, g = O.ema_coeffs_real(Pd["alpha"], Pd["delta"], Pd["beta"], Pd["gamma"])
+        return O.ema_forward(Pd["x"], p, q, g, Pd["omega"].reshape(-1), mask, bidirectional=True, truncation=trunc,
+                             shift=shift)[0]
+
+    assert rel_err(host(y), run(P)) < 1e-4
+    with torch.no_grad():
+        assert rel_err(host(mod(x.detach(), dev(mask, torch.bool))), run(P)) < 1e-4   # the inference kernels agree
+    (y * dev(w64)).sum().backward()
+    grads = {n: host(getattr(mod, n).grad) for n in names}
+    grads["x"] = host(x.grad)
+    _fd_check(rng, names + ["x"], P, grads, lambda Pd: (run(Pd) * w64).sum())
+
+
 def _module_coeffs(mod, cls):
     p, q, g = mod.coeffs()
     return host(p.squeeze(-1)), host(q.squeeze(-1)), host(g)
