@@ -66,7 +66,18 @@ __device__ __forceinline__ float bf_split(float v, __bf16* h) {
 
 constexpr int kPrepWaves = 4;
 constexpr int kPowB = 33 * kNS * 8;
-constexpr int kAuxB = 64 * 4 + kNS * 4 + kNS * 8;
+constexpr int kAuxB = 64 * 4 + kNS * 4 + kNS * 8 + kNS * 16;
+
+// The powers of q are formed in double precision and rounded once: a power q^L formed by fp32 products carries L
+// roundings of q, which at L = 15 * 1024 and |q| = 1 - 3e-5 is 4e-4 of a term that still matters (the reference
+// takes exp(l log q), complex_exponential_moving_average.py:103-106, whose error does not grow with l either).
+struct cdouble {
+  double re, im;
+};
+__device__ __forceinline__ cdouble cmuld(cdouble a, cdouble b) {
+  return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+__device__ __forceinline__ cfloat to_cfloat(cdouble a) { return {(float)a.re, (float)a.im}; }
 
 __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageArgs A) {
   __shared__ __attribute__((aligned(16))) char smem[kPrepWaves * (kPowB + kAuxB)];
@@ -79,6 +90,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
   float* kkt = (float*)(smem + kPrepWaves * kPowB + wave * kAuxB);   // [64]: k[idx] at kkt[32 + idx]
   float* pbuf = kkt + 64;
   float2* gbuf = (float2*)(pbuf + kNS);
+  double2* q32d = (double2*)(gbuf + kNS);                             // [kNS]: q^32 before rounding
   const int r = lane >> 4;
   {
     const int n = lane & 15, blk = lane >> 4;
@@ -91,15 +103,18 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       gr = A.gamma[o * 2];
       gi = A.is_complex ? A.gamma[o * 2 + 1] : 0.f;
     }
-    cfloat q1 = {qr, qi};
-    cfloat q2 = cmul(q1, q1), q4 = cmul(q2, q2), q8 = cmul(q4, q4), q16 = cmul(q8, q8), q24 = cmul(q16, q8);
-    cfloat base = blk == 0 ? cfloat{1.f, 0.f} : blk == 1 ? q8 : blk == 2 ? q16 : q24;
+    const cdouble q1 = {(double)qr, (double)qi};
+    const cdouble q2 = cmuld(q1, q1), q4 = cmuld(q2, q2), q8 = cmuld(q4, q4), q16 = cmuld(q8, q8), q24 = cmuld(q16, q8);
+    cdouble base = blk == 0 ? cdouble{1.0, 0.0} : blk == 1 ? q8 : blk == 2 ? q16 : q24;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-      pw[(8 * blk + t) * kNS + n] = make_float2(base.re, base.im);
-      base = cmul(base, q1);
+      pw[(8 * blk + t) * kNS + n] = make_float2((float)base.re, (float)base.im);
+      base = cmuld(base, q1);
     }
-    if (blk == 3) pw[32 * kNS + n] = make_float2(base.re, base.im);
+    if (blk == 3) {
+      pw[32 * kNS + n] = make_float2((float)base.re, (float)base.im);
+      q32d[n] = make_double2(base.re, base.im);
+    }
     if (blk == 0) {
       pbuf[n] = pv;
       gbuf[n] = make_float2(gr, gi);
@@ -203,9 +218,10 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(c.x), __float_as_uint(c.y), __float_as_uint(d.x),
                                            __float_as_uint(d.y));
     // scan multiplier q^(32 SEGT) of state `lane >> 2`
-    cfloat R = {1.f, 0.f};
-    const float2 w = pw[32 * kNS + (lane >> 2)];
-    for (int t = 0; t < kSEGT; ++t) R = cmul(R, cfloat{w.x, w.y});
+    cdouble Rd = {1.0, 0.0};
+    const double2 w = q32d[lane >> 2];
+    for (int t = 0; t < kSEGT; ++t) Rd = cmuld(Rd, cdouble{w.x, w.y});
+    const cfloat R = to_cfloat(Rd);
     img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
     // multipliers in the matrix-core lane layout (lane = segment j + 16 r, states 2r, 2r+1, 8+2r, 9+2r), for the
     // kernel that scans 16 segments of 64 tokens across the lanes of a row: per state q^64, (q^64)^j,
@@ -214,17 +230,18 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     cfloat RS[4], RJ[4], RW[4], RWJ[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const float2 w32 = pw[32 * kNS + nn[u]];
-      RS[u] = cmul(cfloat{w32.x, w32.y}, cfloat{w32.x, w32.y});
-      cfloat a = {1.f, 0.f};
-      for (int t = 0; t < (lane & 15); ++t) a = cmul(a, RS[u]);
-      RJ[u] = a;
-      cfloat w = RS[u];
-      for (int t = 0; t < 4; ++t) w = cmul(w, w);
-      RW[u] = w;
-      cfloat c = {1.f, 0.f};
-      for (int t = 0; t < (lane & 15); ++t) c = cmul(c, w);
-      RWJ[u] = c;
+      const double2 w32 = q32d[nn[u]];
+      const cdouble rs = cmuld(cdouble{w32.x, w32.y}, cdouble{w32.x, w32.y});
+      RS[u] = to_cfloat(rs);
+      cdouble a = {1.0, 0.0};
+      for (int t = 0; t < (lane & 15); ++t) a = cmuld(a, rs);
+      RJ[u] = to_cfloat(a);
+      cdouble w = rs;
+      for (int t = 0; t < 4; ++t) w = cmuld(w, w);
+      RW[u] = to_cfloat(w);
+      cdouble c = {1.0, 0.0};
+      for (int t = 0; t < (lane & 15); ++t) c = cmuld(c, w);
+      RWJ[u] = to_cfloat(c);
     }
     auto put2 = [&](const cfloat (&v)[4]) {
       img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(v[0].re), __float_as_uint(v[0].im),
@@ -239,19 +256,19 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     if (lane < kNS) {
       // the same multipliers once per state (a lane of the streaming kernels reads 16 bytes = two states)
       float2* cmp = (float2*)(img + (size_t)kSlotCmp * 64);
-      const float2 w32 = pw[32 * kNS + lane];
-      cfloat v = {w32.x, w32.y};
-      cmp[kCmpQ32 * kNS + lane] = make_float2(v.re, v.im);
-      v = cmul(v, v);
-      cmp[kCmpRS * kNS + lane] = make_float2(v.re, v.im);
-      v = cmul(v, v);
-      cmp[kCmpRS2 * kNS + lane] = make_float2(v.re, v.im);
-      v = cmul(v, v);
-      cmp[kCmpRS4 * kNS + lane] = make_float2(v.re, v.im);
-      v = cmul(v, v);
-      cmp[kCmpRS8 * kNS + lane] = make_float2(v.re, v.im);
-      v = cmul(v, v);
-      cmp[kCmpRW * kNS + lane] = make_float2(v.re, v.im);
+      const double2 w32 = q32d[lane];
+      cdouble v = {w32.x, w32.y};
+      cmp[kCmpQ32 * kNS + lane] = make_float2((float)v.re, (float)v.im);
+      v = cmuld(v, v);
+      cmp[kCmpRS * kNS + lane] = make_float2((float)v.re, (float)v.im);
+      v = cmuld(v, v);
+      cmp[kCmpRS2 * kNS + lane] = make_float2((float)v.re, (float)v.im);
+      v = cmuld(v, v);
+      cmp[kCmpRS4 * kNS + lane] = make_float2((float)v.re, (float)v.im);
+      v = cmuld(v, v);
+      cmp[kCmpRS8 * kNS + lane] = make_float2((float)v.re, (float)v.im);
+      v = cmuld(v, v);
+      cmp[kCmpRW * kNS + lane] = make_float2((float)v.re, (float)v.im);
     }
 #pragma unroll
     for (int o = 0; o < 3; ++o)
