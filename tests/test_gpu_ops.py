@@ -135,6 +135,26 @@ def test_attention_no_weights(dtype, B, L, Nh, H1, H2, causal):
     assert rel_err(host(y), host(y2), eps=2.0) < 2 * TOL[dtype]      # two 16-bit results
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("gain", [6.0, 20.0])
+def test_attention_wide_score_range(gain, causal):
+    """Scores that spread over tens to hundreds of units and whose row maximum keeps rising along the keys (a
+    drift in k): the running maximum of the one-kernel path moves by more than its rescaling threshold many times
+    per row, late keys dominate early ones by far more than 2^24."""
+    rng = np.random.default_rng(27)
+    B, L, Nh, H1, H2 = 1, 1536, 2, 128, 256
+    drift = np.linspace(0.0, 1.0, L)[None, :, None, None]
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5 + 0.3, torch.bfloat16)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5 + 0.3 * drift, torch.bfloat16)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), torch.bfloat16)
+    scale = gain / np.sqrt(H1)
+    y, _ = M.ops.attention_fwd(q, k, v, scale, 0.0, causal)
+    torch.cuda.synchronize()
+    yo, _ = O.attention(q64, k64, v64, scale, causal)
+    assert np.isfinite(host(y)).all()
+    assert rel_err(host(y), yo, eps=2.0) < TOL[torch.bfloat16]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n", [1, 7, 4096, 100003])
 def test_swiglu(dtype, n):
