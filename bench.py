@@ -430,6 +430,35 @@ def bench_ema_real(args):
                 torch.cuda.synchronize()
                 regions.append(a.elapsed_time(e) / args.steps)
         ms = min(regions)
+        # the same call replayed from a HIP graph (no Python, no launch calls on the host): tells whether the host
+        # or the device's own dispatch of back-to-back launches bounds a call this small; the replay must
+        # reproduce the eager result
+        graph_ms = None
+        with torch.no_grad():
+            xg = xs[0].clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    m(xg, tm)
+            torch.cuda.current_stream().wait_stream(side)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                yg = m(xg, tm)
+            g.replay()
+            torch.cuda.synchronize()
+            if torch.equal(yg, m(xg, tm)):
+                reg = []
+                for _ in range(3):
+                    a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    torch.cuda.synchronize()
+                    a.record()
+                    for i in range(args.steps):
+                        g.replay()
+                    e.record()
+                    torch.cuda.synchronize()
+                    reg.append(a.elapsed_time(e) / args.steps)
+                graph_ms = min(reg)
         p_, q_, g_ = O.ema_coeffs_real(alpha.astype(np.float32), delta.astype(np.float32), beta.astype(np.float32),
                                        gamma.astype(np.float32))
         cpu = None
@@ -445,7 +474,8 @@ def bench_ema_real(args):
         out[name] = {"ms": ms, "tokens_per_s": b * l / (ms * 1e-3), "algorithmic_bytes": alg,
                      "hbm_gbs": alg / (ms * 1e-3) / 1e9, "cpu_ms": None if cpu is None else cpu * 1e3,
                      "rel_err_vs_oracle": None if ref is None else rel_err(y.float().cpu().numpy(), ref),
-                     "timed_regions_ms": regions}
+                     "timed_regions_ms": regions, "graph_replay_ms": graph_ms,
+                     "graph_replay_hbm_gbs": None if graph_ms is None else alg / (graph_ms * 1e-3) / 1e9}
     c1 = out["configs[1]"]
     line = {
         "metric": "real MultiHeadEMA forward tokens/sec @B1xL16384xD256 (bidirectional, fp32)",
