@@ -64,7 +64,9 @@ __device__ __forceinline__ float dot2_self(uint32_t w, float acc) {
   }
 }
 
-// merge of two sets of equally weighted steps; one reciprocal per merge
+// merge of two sets of equally weighted steps; one reciprocal per merge.  Two empty sets keep the first one's
+// mean and variance: a row that has seen no valid step yet still carries the caller's prior statistics, which
+// the reference hands back unchanged (timestep_norm.cc:283-311: u, v only move on unmasked steps).
 __device__ __forceinline__ Moments merge(Moments a, Moments b) {
   const float n = a.n + b.n;
   const float rn = n > 0.f ? __builtin_amdgcn_rcpf(n) : 0.f;
@@ -73,7 +75,7 @@ __device__ __forceinline__ Moments merge(Moments a, Moments b) {
   Moments r;
   r.n = n;
   r.mean = a.mean + cb * d;
-  r.var = ca * a.var + cb * b.var + (ca * d) * (cb * d);
+  r.var = n > 0.f ? ca * a.var + cb * b.var + (ca * d) * (cb * d) : a.var;
   return r;
 }
 

@@ -1,0 +1,177 @@
+"""Seeded random sweeps across the shape boundaries where the library changes kernels: every case is one call
+of a public operator checked against the fp64 oracle.  The moving average draws its type, layout, lengths around
+64 / 256 / 1024 / 4096 tokens, channel counts around the 16-channel blocks, 1..16 (or 32) states, mask, carried
+state, direction and truncation; the TimestepNorm draws group and per-feature variants, masks, priors and tile
+boundaries; the norm -> moving-average call draws shapes inside and outside its one-kernel envelope."""
+import numpy as np
+import pytest
+import torch
+
+import fairseq_apollo_amd as M
+from conftest import mega_init_complex, mega_init_real, rel_err
+from gpu_util import DEV, TOL, dev, host, rounded
+from oracle import mega_oracle as O
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+LENGTHS = [1, 2, 31, 63, 64, 65, 100, 255, 256, 257, 511, 1000, 1023, 1024, 1025, 2047, 2048, 2052, 3000, 4096, 4100]
+
+
+def _state_err(h, ho):
+    """rel_err with a floor: behind a long masked tail the state has decayed below what fp32 holds at all."""
+    a, b = np.asarray(h, np.float64), np.asarray(ho, np.float64)
+    den = np.maximum(np.abs(b), float(np.sqrt(np.mean(b * b))) + 1e-30)
+    return float(np.max(np.abs(a - b) / den))
+
+
+def _coeffs(rng, K, N, cplx):
+    if cplx:
+        return O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
+    return O.ema_coeffs_real(*mega_init_real(rng, K, N))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_moving_average_sweep(seed):
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(12):
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        L = int(rng.choice(LENGTHS))
+        D = int(rng.choice([1, 3, 15, 16, 17, 32, 48, 130]))
+        B = int(rng.choice([1, 2, 3, 5]))
+        if B * D * L > 3_000_000:
+            B, D = 1, min(D, 32)
+        N = int(rng.choice([1, 2, 5, 8, 15, 16, 32])) if L <= 2052 else int(rng.choice([2, 16]))
+        cplx = bool(rng.integers(0, 2))
+        bidir = bool(rng.integers(0, 2))
+        time_major = bool(rng.integers(0, 2))
+        masked = bool(rng.integers(0, 2))
+        shift = bool(rng.integers(0, 2))
+        trunc = int(rng.choice([0, 0, 7, 40, 300])) if bidir else 0
+        with_state = (not bidir) and bool(rng.integers(0, 2)) and B * D * N * L < 4_000_000
+        out_layout = "input" if rng.integers(0, 3) == 0 else "rows"
+        tag = (f"seed {seed} case {case}: {dtype} B={B} D={D} L={L} N={N} cplx={cplx} bidir={bidir} shift={shift} "
+               f"trunc={trunc} time_major={time_major} masked={masked} state={with_state} out={out_layout}")
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, 2 * D if bidir else D, N, cplx)
+        om = rng.normal(size=D)
+        if time_major:
+            xt, xt64 = rounded(rng.normal(size=(B, L, D)), dtype)
+            x, x64 = xt.transpose(1, 2), xt64.transpose(0, 2, 1)
+        else:
+            x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+        mask = None
+        if masked:
+            mask = rng.random((B, L)) < 0.1
+            mask[0, L - L // 5:] = True
+        h0 = None
+        if with_state:
+            h0 = rng.normal(size=(B, D, N)) + (1j * rng.normal(size=(B, D, N)) if cplx else 0)
+            h0 = h0.astype(np.complex64) if cplx else h0.astype(np.float32)
+        y, h = M.ops.ema_forward(x, dev(p), dev(q), dev(g), dev(om),
+                                 padding_mask=None if mask is None else dev(mask, torch.bool),
+                                 h=None if h0 is None else dev(h0), want_state=with_state, bidirectional=bidir,
+                                 truncation=trunc if trunc else None, shift=shift, out_layout=out_layout)
+        torch.cuda.synchronize()
+        yo, ho = O.ema_forward(x64, p, q, g, om, mask, h=h0, bidirectional=bidir, truncation=trunc if trunc else None,
+                               shift=shift, incremental=with_state)
+        assert y.shape == (B, D, L), tag
+        assert rel_err(host(y), yo) < TOL[dtype], tag
+        if with_state:
+            tol = 1e-4 if dtype is torch.float32 else 2e-3
+            assert _state_err(np.real(host(h)), np.real(ho)) < tol, tag
+            if cplx:
+                assert _state_err(np.imag(host(h)), np.imag(ho)) < tol, tag
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_timestep_norm_sweep(seed):
+    rng = np.random.default_rng(2000 + seed)
+    for case in range(10):
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 2, 7, 8, 15, 16, 17, 33, 64, 100, 257, 1000, 1024, 2049]))
+        feature = rng.integers(0, 4) == 0
+        if feature:
+            H = int(rng.choice([1, 4, 12, 64, 200]))
+            G = None
+        else:
+            G = int(rng.choice([1, 2, 3, 4, 16]))
+            H = G * int(rng.choice([1, 2, 8, 24, 64, 128]))
+        B = int(rng.choice([1, 2, 5]))
+        masked = bool(rng.integers(0, 2))
+        prior = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: {dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior}"
+        print(tag, flush=True)
+        Gn = H if G is None else G
+        x, x64 = rounded(rng.normal(size=(B, L, H)) * 2.0 + 0.5, dtype)
+        gam = rng.normal(size=H) * 0.2 + 1.0
+        bet = rng.normal(size=H) * 0.2
+        mask = None
+        if masked:
+            mask = rng.random((B, L)) < 0.15
+            mask[B - 1, L // 2:] = True
+        pc = rng.integers(1, 50, size=B) if prior else np.zeros(B, np.int64)
+        pm = rng.normal(size=(B, Gn)) if prior else np.zeros((B, Gn))
+        pv = rng.random((B, Gn)) + 0.5 if prior else np.ones((B, Gn))
+        pm, pv = pm.astype(np.float32).astype(np.float64), pv.astype(np.float32).astype(np.float64)
+        args = (x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gam), dev(bet), None if mask is None else dev(mask, torch.bool))
+        if feature:
+            out = M.ops.timestep_norm_fwd(*args, 1e-5)
+        else:
+            out = M.ops.group_timestep_norm_fwd(*args, G, 1e-5)
+        torch.cuda.synchronize()
+        y, cnt, mean, var = out[0], out[1], out[2], out[3]
+        gam32, bet32 = gam.astype(np.float32).astype(np.float64), bet.astype(np.float32).astype(np.float64)
+        yo, co, mo, vo = O.timestep_norm(x64, pc, pm, pv, gam32, bet32, mask, G)
+        assert cnt.tolist() == co.tolist(), tag
+        assert rel_err(host(y), yo) < TOL[dtype], tag
+        assert rel_err(host(mean), mo) < 1e-4 and rel_err(host(var), vo) < 1e-4, tag
+    assert M.ops.timestep_norm_status() == 0
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_norm_then_moving_average_sweep(seed):
+    rng = np.random.default_rng(3000 + seed)
+    for case in range(6):
+        G = int(rng.choice([1, 2, 4]))
+        dg = int(rng.choice([64, 64, 32, 16]))
+        D = G * dg
+        L = int(rng.choice([64, 300, 1024, 2048, 2050, 3072]))
+        B = int(rng.choice([1, 2, 3]))
+        N = int(rng.choice([2, 7, 16]))
+        cplx = bool(rng.integers(0, 2))
+        masked = rng.integers(0, 3) == 0
+        with_state = bool(rng.integers(0, 2))
+        out_layout = "input" if rng.integers(0, 2) else "rows"
+        tag = (f"seed {seed} case {case}: B={B} L={L} D={D} G={G} N={N} cplx={cplx} masked={masked} "
+               f"state={with_state} out={out_layout}")
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, D, N, cplx)
+        om = rng.normal(size=D)
+        gam = (rng.normal(size=D) * 0.1 + 1.0).astype(np.float32).astype(np.float64)
+        bet = (rng.normal(size=D) * 0.1).astype(np.float32).astype(np.float64)
+        x, x64 = rounded(rng.normal(size=(B, L, D)) * 1.5 + 0.3, torch.bfloat16)
+        mask = None
+        if masked:
+            mask = np.zeros((B, L), bool); mask[0, L - L // 4:] = True
+        h0 = None
+        if with_state:
+            h0 = (rng.normal(size=(B, D, N)) + (1j * rng.normal(size=(B, D, N)) if cplx else 0))
+            h0 = h0.astype(np.complex64) if cplx else h0.astype(np.float32)
+        pc = rng.integers(0, 30, size=B)
+        pm = rng.normal(size=(B, G)).astype(np.float32).astype(np.float64)
+        pv = (rng.random((B, G)) + 0.5).astype(np.float32).astype(np.float64)
+        layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+        xn, y, cnt, mean, var, h = layer.norm_forward(
+            x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gam), dev(bet), G, 1e-5,
+            padding_mask=None if mask is None else dev(mask, torch.bool), h=None if h0 is None else dev(h0),
+            want_state=with_state, out_layout=out_layout)
+        torch.cuda.synchronize()
+        xno, co, mo, vo = O.timestep_norm(x64, pc, pm, pv, gam, bet, mask, G)
+        assert cnt.tolist() == co.tolist(), tag
+        assert rel_err(host(xn), xno) < 2e-2, tag
+        assert rel_err(host(mean), mo) < 1e-4 and rel_err(host(var), vo) < 1e-4, tag
+        yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, mask, h=h0, incremental=with_state)
+        assert rel_err(host(y), yo) < 2e-2, tag
+        if with_state:
+            assert _state_err(np.real(host(h)), np.real(ho)) < 2e-3, tag
+    assert M.ops.timestep_norm_status() == 0
