@@ -66,10 +66,11 @@ def test_incremental_state_keys_are_per_module():
 
 
 def test_configurations_without_a_backward_refuse_autograd():
-    """The unidirectional moving average, TimestepNorm and the attention have backward operators;
-    what has none says so instead of returning tensors that silently carry no graph."""
+    """The moving average (with a truncated kernel or a carried state through the chained operators),
+    TimestepNorm and the attention have backward operators; what has none says so instead of returning tensors
+    that silently carry no graph.  None of them has a CPU path: host tensors are refused by name."""
     e = M.MultiHeadComplexEMA(4, ndim=2, bidirectional=True, truncation=4)
-    with pytest.raises(NotImplementedError, match="backward pass covers"):
+    with pytest.raises(RuntimeError, match="no CPU path"):
         e(torch.zeros(1, 4, 8))
     layer = M.MovingAverageGatedAttention(8, 4, 8, 2, chunk_size=4, norm_num_groups=2)
     with pytest.raises(NotImplementedError, match="incremental state"):
