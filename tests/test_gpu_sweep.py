@@ -175,3 +175,95 @@ def test_norm_then_moving_average_sweep(seed):
         if with_state:
             assert _state_err(np.real(host(h)), np.real(ho)) < 2e-3, tag
     assert M.ops.timestep_norm_status() == 0
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_attention_sweep(seed):
+    """EfficientAttention's forward with and without the weights: head sizes on both sides of what the one-kernel
+    path takes (H1 64 / 128, H2 a multiple of 8 from 64 on, L from 64 on), lengths that end inside a tile."""
+    rng = np.random.default_rng(4000 + seed)
+    for case in range(6):
+        dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 5, 63, 64, 65, 200, 256, 257, 700, 1024, 1300]))
+        Nh = int(rng.choice([1, 2, 3]))
+        H1 = int(rng.choice([8, 32, 64, 96, 128]))
+        H2 = int(rng.choice([8, 24, 64, 72, 256, 264, 512]))
+        B = int(rng.choice([1, 2]))
+        causal = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: {dtype} B={B} L={L} Nh={Nh} H1={H1} H2={H2} causal={causal}"
+        print(tag, flush=True)
+        q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+        k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+        v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+        scale = float(rng.choice([0.5, 1.0, 3.0])) / np.sqrt(H1)
+        yo, wo = O.attention(q64, k64, v64, scale, causal)
+        y, w = M.ops.attention_fwd(q, k, v, scale, 0.0, causal)
+        torch.cuda.synchronize()
+        assert w is None, tag
+        assert rel_err(host(y), yo, eps=2.0) < TOL[dtype], tag
+        y2, w2 = M.ops.attention_fwd(q, k, v, scale, 0.0, causal, need_weights=True)
+        torch.cuda.synchronize()
+        assert rel_err(host(y2), yo, eps=2.0) < TOL[dtype], tag
+        assert np.abs(host(w2) - wo).max() < (1e-5 if dtype is torch.float32 else 4e-3), tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_sequence_norm_sweep(seed):
+    rng = np.random.default_rng(5000 + seed)
+    for case in range(8):
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 2, 17, 64, 100, 513, 2048]))
+        feature = rng.integers(0, 3) == 0
+        G = None if feature else int(rng.choice([1, 2, 4, 16]))
+        H = int(rng.choice([1, 8, 40, 200])) if feature else G * int(rng.choice([1, 4, 8, 64]))
+        B = int(rng.choice([1, 3]))
+        last = bool(rng.integers(0, 2))
+        masked = bool(rng.integers(0, 2))
+        if L * (H // (H if G is None else G)) < 8:
+            L = 17              # a statistic over one or two values has variance ~ 0: rstd = eps^-1/2 amplifies rounding
+        tag = f"seed {seed} case {case}: {dtype} B={B} L={L} H={H} G={G} length_last={last} masked={masked}"
+        print(tag, flush=True)
+        x, x64 = rounded(rng.normal(size=(B, H, L) if last else (B, L, H)) * 2.0 + 0.5, dtype)
+        gam = (rng.normal(size=H) * 0.2 + 1.0).astype(np.float32).astype(np.float64)
+        bet = (rng.normal(size=H) * 0.2).astype(np.float32).astype(np.float64)
+        mask = None
+        if masked and L > 1:
+            mask = rng.random((B, L)) < 0.2
+            mask[:, 0] = False                              # at least one valid token per row
+        tm = None if mask is None else dev(mask, torch.bool)
+        if feature:
+            y, cnt, mean, rstd = M.ops.sequence_norm_fwd(x, dev(gam), dev(bet), tm, 1e-5, last)
+        else:
+            y, cnt, mean, rstd = M.ops.group_sequence_norm_fwd(x, dev(gam), dev(bet), tm, G, 1e-5, last)
+        torch.cuda.synchronize()
+        yo, co, mo, ro = O.sequence_norm(x64, gam, bet, mask, G, 1e-5, last)
+        assert cnt.tolist() == co.tolist(), tag
+        assert rel_err(host(y), yo) < TOL[dtype], tag
+        assert rel_err(host(mean), mo) < 1e-4 and rel_err(host(rstd), ro) < 1e-3, tag
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_explicit_kernel_convolution_sweep(seed):
+    """fftconv / bidirectional_fftconv with an explicit kernel: kernel lengths on both sides of the 512 lags from
+    which the transform path takes over, row lengths up to its 16384-point limit and beyond."""
+    rng = np.random.default_rng(6000 + seed)
+    for case in range(5):
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 33, 511, 512, 513, 1000, 2048, 3000, 8192, 9000]))
+        Lk = min(L, int(rng.choice([1, 7, 64, 511, 512, 600, 2048, 8192])))
+        D = int(rng.choice([1, 3, 8]))
+        B = int(rng.choice([1, 2, 3]))
+        bidir = bool(rng.integers(0, 2))
+        shift = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: {dtype} B={B} D={D} L={L} Lk={Lk} bidir={bidir} shift={shift}"
+        print(tag, flush=True)
+        x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+        k = (rng.normal(size=(2 * D if bidir else D, Lk)) * np.exp(-np.arange(Lk) / 200.0) * 0.3).astype(np.float32)
+        if bidir:
+            y = M.ops.bidirectional_fftconv(x, dev(k), shift)
+            ref = O.bidirectional_conv(x64, k.astype(np.float64), shift)
+        else:
+            y = M.ops.fftconv(x, dev(k))
+            ref = O.causal_conv(x64, np.pad(k.astype(np.float64), ((0, 0), (0, L - Lk))))
+        torch.cuda.synchronize()
+        assert rel_err(host(y), ref) < TOL[dtype], tag
