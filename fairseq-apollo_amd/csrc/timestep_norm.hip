@@ -686,13 +686,19 @@ size_t tsn_workspace_bytes(int64_t B, int64_t G, int ntiles) {
 using namespace mega;
 
 extern "C" size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G) {
+  // G == H names both the per-feature variant (mega_timestep_norm_fwd) and the group variant with one channel per
+  // group (mega_group_timestep_norm_fwd): the size covers whichever entry point the workspace is handed to
+  size_t need = 256;
   if (B > 0 && L > 0 && H > 0 && G == H && H > 1) {
-    const size_t f = feature_tsn_workspace_bytes(B, L, H);   // the per-feature variant (mega_timestep_norm_fwd)
-    return f > 256 ? f : 256;
+    const size_t f = feature_tsn_workspace_bytes(B, L, H);
+    need = f > need ? f : need;
   }
   TsnGeom g;
-  if (B <= 0 || L <= 0 || H <= 0 || G <= 0 || H % G != 0 || !tsn_geometry(dtype, B, L, H, G, &g)) return 256;
-  return tsn_workspace_bytes(B, G, g.ntiles);
+  if (B > 0 && L > 0 && H > 0 && G > 0 && H % G == 0 && tsn_geometry(dtype, B, L, H, G, &g)) {
+    const size_t t = tsn_workspace_bytes(B, G, g.ntiles);
+    need = t > need ? t : need;
+  }
+  return need;
 }
 
 static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* prev_count,

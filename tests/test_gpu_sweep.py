@@ -267,3 +267,95 @@ def test_explicit_kernel_convolution_sweep(seed):
             ref = O.causal_conv(x64, np.pad(k.astype(np.float64), ((0, 0), (0, L - Lk))))
         torch.cuda.synchronize()
         assert rel_err(host(y), ref) < TOL[dtype], tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_moving_average_backward_sweep(seed):
+    """ema_backward (input gradient + parameter-gradient sums) for one- and two-sided layers in both layouts."""
+    rng = np.random.default_rng(7000 + seed)
+    for case in range(6):
+        dtype = [torch.float32, torch.bfloat16][int(rng.integers(0, 2))]
+        L = int(rng.choice([1, 31, 64, 100, 256, 300, 511, 1024, 1100, 1544, 2048]))
+        D = int(rng.choice([1, 5, 16, 24, 40]))
+        B = int(rng.choice([1, 2, 3]))
+        N = int(rng.choice([1, 2, 7, 16]))
+        cplx = bool(rng.integers(0, 2))
+        bidir = bool(rng.integers(0, 2))
+        shift = bool(rng.integers(0, 2))
+        layout = str(rng.choice(["bdl", "bld", "mixed"]))
+        masked = bool(rng.integers(0, 2))
+        tag = (f"seed {seed} case {case}: {dtype} B={B} D={D} N={N} L={L} cplx={cplx} bidir={bidir} shift={shift} "
+               f"layout={layout} masked={masked}")
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, 2 * D if bidir else D, N, cplx)
+        p = p.astype(np.float32).astype(np.float64)
+        if cplx:
+            q, g = q.astype(np.complex64).astype(np.complex128), g.astype(np.complex64).astype(np.complex128)
+        else:
+            q, g = q.astype(np.float32).astype(np.float64), g.astype(np.float32).astype(np.float64)
+        om = rng.normal(size=D).astype(np.float32).astype(np.float64)
+        x, x64 = rounded(rng.normal(size=(B, D, L)), dtype)
+        dy, dy64 = rounded(rng.normal(size=(B, D, L)), dtype)
+        if layout in ("bld", "mixed"):
+            x = x.transpose(1, 2).contiguous().transpose(1, 2)
+        if layout == "bld":
+            dy = dy.transpose(1, 2).contiguous().transpose(1, 2)
+        mask = (rng.random((B, L)) < 0.2) if masked else None
+        tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+        layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om), bidir, None, shift)
+        got = M.ops.ema_backward(dy, x, dev(p), dev(q), dev(g), dev(om), tm, layer=layer)
+        torch.cuda.synchronize()
+        ref = O.ema_backward(dy64, x64, p, q, g, om, mask, bidir, shift)
+        assert rel_err(host(got[0]), ref[0]) < TOL[dtype], tag
+        for a, b, name in zip(got[1:], ref[1:], ("dp", "dq", "dgamma", "domega")):
+            a = host(a)
+            if np.iscomplexobj(b) and cplx:
+                assert rel_err(a.real, b.real) < 5e-4 and rel_err(a.imag, b.imag) < 5e-4, (tag, name)
+            else:
+                assert rel_err(np.real(a), np.real(b)) < 5e-4, (tag, name)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_timestep_norm_backward_sweep(seed):
+    rng = np.random.default_rng(8000 + seed)
+    for case in range(6):
+        dtype = DTYPES[int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 2, 15, 16, 17, 37, 96, 130, 257, 1000]))
+        feature = rng.integers(0, 4) == 0
+        G = None if feature else int(rng.choice([1, 2, 4, 5, 16]))
+        H = int(rng.choice([1, 6, 24, 100])) if feature else G * int(rng.choice([1, 6, 8, 24, 64]))
+        B = int(rng.choice([1, 2, 3]))
+        masked = bool(rng.integers(0, 2))
+        prior = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: {dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior}"
+        print(tag, flush=True)
+        GG = H if G is None else G
+        x, x64 = rounded(rng.normal(size=(B, L, H)) * 1.3 + 0.2, dtype)
+        dy, dy64 = rounded(rng.normal(size=(B, L, H)), dtype)
+        mask = (rng.random((B, L)) < 0.25) if masked else None
+        if mask is not None:
+            mask[:, 0] = False
+        pc = rng.integers(1, 5, B).astype(np.int64) if prior else np.zeros(B, np.int64)
+        pm = (rng.normal(size=(B, GG)) * 0.2 * prior).astype(np.float32).astype(np.float64)
+        pv = (rng.random((B, GG)) + 0.5 if prior else np.ones((B, GG))).astype(np.float32).astype(np.float64)
+        gamma = (rng.normal(size=H) * 0.3 + 1).astype(np.float32).astype(np.float64)
+        beta = rng.normal(size=H).astype(np.float32).astype(np.float64)
+        dm = rng.normal(size=(B, GG)).astype(np.float32).astype(np.float64)
+        dv = rng.normal(size=(B, GG)).astype(np.float32).astype(np.float64)
+        tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+        if G is None:
+            y, cnt, mu, var, cm, cr = M.ops.timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma),
+                                                              dev(beta), tm, 1e-5)
+            got = M.ops.timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, cm, cr, dev(gamma), tm)
+        else:
+            y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv),
+                                                                        dev(gamma), dev(beta), tm, G, 1e-5)
+            got = M.ops.group_timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, gm, cm, cr, dev(gamma), tm, G)
+        torch.cuda.synchronize()
+        ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm, pv, mask, G, 1e-5)
+        assert np.array_equal(host(cnt), ocnt), tag
+        ref = O.timestep_norm_bwd(dy64, dm, dv, x64, pm, ocnt, ogm if G else None, ocm, ocr, gamma, mask, G)
+        assert rel_err(host(got[0]), ref[0]) < TOL[dtype], tag
+        for a, b in zip(got[1:], ref[1:]):
+            assert rel_err(host(a), b) < 2e-4, tag
+    assert M.ops.timestep_norm_status() == 0
