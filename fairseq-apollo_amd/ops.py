@@ -1092,6 +1092,8 @@ def gate_qk_fwd(z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, freqs:
     lib = _lib.load()
     S = z.shape[-1]
     zr, zs = _rows(z)
+    if zs % 2 or zr.data_ptr() % (2 * zr.element_size()):
+        zr, zs = z.detach().contiguous(), S        # the kernel moves feature pairs: rows must start on an even element
     g, b, f = _f32c(gamma), _f32c(beta), _f32c(freqs)
     if g.shape != (2, S) or b.shape != (2, S) or num_heads < 1 or S % num_heads or f.numel() * 2 * num_heads != S:
         raise RuntimeError("gate_qk_fwd: gamma, beta must be [2, S] and freqs [S / heads / 2]")

@@ -359,3 +359,70 @@ def test_timestep_norm_backward_sweep(seed):
         for a, b in zip(got[1:], ref[1:]):
             assert rel_err(host(a), b) < 2e-4, tag
     assert M.ops.timestep_norm_status() == 0
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_gated_attention_layer_sweep(seed):
+    """The whole MovingAverageGatedAttention forward in fp32 (a tight bound shows any wrong glue): widths that are
+    not multiples of the vector sizes of the gate kernels, heads, chunk sizes above, at and below the length,
+    both activations of the moving average, one- and two-sided layers with padding."""
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(4):
+        heads = int(rng.choice([1, 2, 4]))
+        S = heads * int(rng.choice([2, 6, 8, 16]))
+        E = heads * int(rng.choice([4, 10, 16, 24, 64]))
+        G = int(rng.choice([1, 2, 4]))
+        D = G * int(rng.choice([3, 8, 10, 16, 64]))
+        N = int(rng.choice([1, 4, 16]))
+        C = int(rng.choice([16, 64, 128]))
+        nchunks = int(rng.choice([1, 1, 2, 5]))
+        L = C * nchunks if nchunks > 1 else int(rng.choice([C, C // 2 + 3, 7]))
+        B = int(rng.choice([1, 2, 3]))
+        act = str(rng.choice(['silu', 'rmsnorm']))
+        moving = str(rng.choice(['cema', 'ema']))
+        bidir = bool(rng.integers(0, 2))
+        masked = bidir and bool(rng.integers(0, 2))
+        tag = (f"seed {seed} case {case}: B={B} L={L} D={D} S={S} E={E} N={N} G={G} C={C} heads={heads} act={act} "
+               f"moving={moving} bidir={bidir} masked={masked}")
+        print(tag, flush=True)
+        torch.manual_seed(9000 + 10 * seed + case)
+        layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_layer=moving, moving_act=act,
+                                              norm_num_groups=G, num_heads=heads, bidirectional=bidir).to(DEV).eval()
+        with torch.no_grad():
+            for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+                prm.normal_(0, 0.15)
+            layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
+            layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+        p, q, g = layer.move.coeffs()
+        P = dict(norm_weight=host(layer.norm.weight), norm_bias=host(layer.norm.bias), p=host(p.squeeze(-1)),
+                 q=host(q.squeeze(-1)), ema_gamma=host(g), omega=host(layer.move.omega).reshape(-1),
+                 v_w=host(layer.v_proj.weight), v_b=host(layer.v_proj.bias), mx_w=host(layer.mx_proj.weight),
+                 mx_b=host(layer.mx_proj.bias), h_w=host(layer.h_proj.weight), gamma=host(layer.gamma),
+                 beta=host(layer.beta))
+        if isinstance(layer.move_act, M.RMSNorm):
+            P['rms_weight'] = host(layer.move_act.weight)
+        x = torch.randn(B, L, D, device=DEV)
+        mask = None
+        if masked:
+            mask = np.zeros((B, L), bool); mask[0, L - max(L // 4, 1):] = True
+        with torch.no_grad():
+            y, _ = layer(x, None if mask is None else dev(mask, torch.bool))
+        torch.cuda.synchronize()
+        yo = O.gated_attention_layer(host(x), P, chunk=C, num_heads=heads, moving_act=act, num_groups=G,
+                                     bidirectional=bidir, padding_mask=mask)
+        keep = np.ones((B, L), bool) if mask is None else ~mask
+        assert rel_err(host(y)[keep], yo[keep]) < 2e-4, tag
+        # the training path (autograd functions and backward kernels) sees the same shapes: same output, and
+        # gradients that are finite and not all zero
+        layer.train()
+        xg = x.clone().requires_grad_(True)
+        yt, _ = layer(xg, None if mask is None else dev(mask, torch.bool))
+        assert rel_err(host(yt)[keep], host(y)[keep]) < 2e-4, tag
+        wgt = torch.randn_like(yt)
+        if mask is not None:
+            wgt = wgt * dev(~mask).unsqueeze(-1)
+        (yt * wgt).sum().backward()
+        torch.cuda.synchronize()
+        grads = [xg.grad] + [prm.grad for prm in layer.parameters() if prm.requires_grad]
+        assert all(gr is not None and torch.isfinite(gr).all() for gr in grads), tag
+        assert xg.grad.abs().max().item() > 0, tag
