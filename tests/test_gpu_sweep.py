@@ -426,3 +426,46 @@ def test_gated_attention_layer_sweep(seed):
         grads = [xg.grad] + [prm.grad for prm in layer.parameters() if prm.requires_grad]
         assert all(gr is not None and torch.isfinite(gr).all() for gr in grads), tag
         assert xg.grad.abs().max().item() > 0, tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_decode_sweep(seed):
+    """Streaming decode of the norm -> moving-average pair: tokens arrive one at a time and in batches of random
+    sizes (the multi-token kernel where the coefficient shape allows it), against the oracle on the whole sequence."""
+    rng = np.random.default_rng(10000 + seed)
+    for case in range(4):
+        dtype = [torch.float32, torch.bfloat16, torch.float16][int(rng.integers(0, 3))]
+        G = int(rng.choice([1, 2, 3, 8]))
+        D = G * int(rng.choice([1, 4, 24, 64]))
+        N = int(rng.choice([1, 2, 4, 6, 8, 16, 32]))
+        B = int(rng.choice([1, 2, 5]))
+        cplx = bool(rng.integers(0, 2))
+        T = int(rng.choice([1, 9, 70, 150]))
+        tag = f"seed {seed} case {case}: {dtype} B={B} D={D} G={G} N={N} cplx={cplx} T={T}"
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, D, N, cplx)
+        om = rng.normal(size=D)
+        nw = (rng.normal(size=D) * 0.1).astype(np.float32).astype(np.float64)
+        nb = (rng.normal(size=D) * 0.1).astype(np.float32).astype(np.float64)
+        x, x64 = rounded(rng.normal(size=(B, T, D)) + 0.2, dtype)
+        step = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+        xs, ys, a = [], [], 0
+        while a < T:
+            K = min(T - a, int(rng.choice([1, 1, 2, 5, 64, 100])))
+            if K == 1 and rng.integers(0, 2):
+                xn, y = step(x[:, a])
+                xn, y = xn.unsqueeze(1), y.unsqueeze(1)
+            else:
+                xn, y = step.steps(x[:, a:a + K])
+            xs.append(xn); ys.append(y)
+            a += K
+        xn_s, y_s = torch.cat(xs, 1), torch.cat(ys, 1)
+        torch.cuda.synchronize()
+        tol = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 4e-3}[dtype]
+        xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, None, G)
+        assert step.count.tolist() == [T] * B, tag
+        assert rel_err(host(xn_s), xno) < tol, tag
+        assert rel_err(host(step.mean), mu) < 1e-4 and rel_err(host(step.var), v) < 1e-4, tag
+        yo, ho = O.ema_forward(host(xn_s).transpose(0, 2, 1), p, q, g, om, incremental=True)
+        assert rel_err(host(y_s), yo.transpose(0, 2, 1)) < tol, tag
+        assert _state_err(np.real(host(step.state)), np.real(ho)) < 1e-4, tag
