@@ -469,3 +469,54 @@ def test_decode_sweep(seed):
         yo, ho = O.ema_forward(host(xn_s).transpose(0, 2, 1), p, q, g, om, incremental=True)
         assert rel_err(host(y_s), yo.transpose(0, 2, 1)) < tol, tag
         assert _state_err(np.real(host(step.state)), np.real(ho)) < 1e-4, tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_streaming_equals_one_shot_sweep(seed):
+    """A causal gated-attention layer fed slices of random lengths with carried state (norm statistics, moving-
+    average state, the partial chunk's keys and values) gives what one call on the whole sequence gives; a batch
+    of bf16 follows the fp32 result."""
+    rng = np.random.default_rng(11000 + seed)
+    for case in range(3):
+        heads = int(rng.choice([1, 2]))
+        S = heads * int(rng.choice([4, 8, 16]))
+        E = heads * int(rng.choice([8, 24, 64]))
+        G = int(rng.choice([1, 2, 4]))
+        D = G * int(rng.choice([8, 16, 64]))
+        N = int(rng.choice([2, 16]))
+        C = int(rng.choice([16, 64, 128]))
+        L = C * int(rng.choice([1, 2, 4])) + int(rng.choice([0, 0, 5]))
+        B = int(rng.choice([1, 2]))
+        act = str(rng.choice(['silu', 'rmsnorm']))
+        tag = f"seed {seed} case {case}: B={B} L={L} D={D} S={S} E={E} N={N} G={G} C={C} heads={heads} act={act}"
+        print(tag, flush=True)
+        torch.manual_seed(11000 + 10 * seed + case)
+        layer = M.MovingAverageGatedAttention(D, S, E, N, chunk_size=C, moving_act=act, norm_num_groups=G,
+                                              num_heads=heads).to(DEV).eval()
+        with torch.no_grad():
+            for prm in (layer.v_proj.weight, layer.mx_proj.weight, layer.h_proj.weight):
+                prm.normal_(0, 0.15)
+        x = torch.randn(B, L, D, device=DEV)
+        # slices the reference's cache logic takes (moving_average_gated_attention.py:332-387): whole chunks from
+        # a chunk boundary, or a piece that stays inside the current chunk
+        cuts = [0]
+        while cuts[-1] < L:
+            a = cuts[-1]
+            room = C - a % C
+            if a % C == 0:
+                step = int(rng.choice([1, 3, C // 2, C, 2 * C]))
+                step = step if (step <= C or a + step <= L - L % C) else C
+            else:
+                step = int(rng.choice([1, 2, room]))
+            cuts.append(min(L, a + min(step, room if step < C else step)))
+        with torch.no_grad():
+            if L % C == 0 or L < C:
+                full, _ = layer(x)
+            else:                                   # a one-shot call wants whole chunks: the whole part, then the rest
+                st = {}
+                full = torch.cat([layer(x[:, :L - L % C], None, st)[0], layer(x[:, L - L % C:], None, st)[0]], 1)
+            state = {}
+            parts = [layer(x[:, a:b], None, state)[0] for a, b in zip(cuts[:-1], cuts[1:])]
+        torch.cuda.synchronize()
+        assert rel_err(host(torch.cat(parts, 1)), host(full)) < 2e-4, (tag, cuts)
+    assert M.ops.timestep_norm_status() == 0
