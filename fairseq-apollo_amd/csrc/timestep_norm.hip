@@ -35,6 +35,8 @@ constexpr int kNV = 16;                       // vectors kept in registers per t
 constexpr int kPartCap = kThreads * kNV;      // vectors per tile
 constexpr int kMaxTT = 64;                    // tokens per tile (16 lanes x 4 tokens in the scan)
 constexpr int kLbWords = 4352;                // 64-bit words staged in LDS per look-back round
+constexpr int kLbBlock = 32;                  // tiles per block record: a tile looks back over the whole blocks before
+                                              // it and the earlier tiles of its own block, not over every earlier tile
 
 struct TsnParams {
   const void* x;
@@ -55,8 +57,11 @@ struct TsnParams {
   // [B*ntiles][2G+1] 64-bit words, value in the low half, launch tag in the high half:
   // word 0 = unmasked tokens of the tile, word 1+2g = mean, word 2+2g = variance of group g
   unsigned long long* rec;
+  // [B*nblk][2G+1] words of the same form: the aggregate of kLbBlock consecutive tiles, left by the block's last
+  // tile once it has seen the others
+  unsigned long long* brec;
   int B, L, H, G;
-  int TT, ntiles;
+  int TT, ntiles, nblk;
   int TPT;           // vectors per token
   int LPG;           // vectors per group
   float eps;
@@ -250,23 +255,34 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       if (g == 0) put_rec(mine, tagged((uint32_t)inc.n, tag));
     }
     MEGA_TSN_TR(2);
-    // earlier tiles, RT per round
-    Moments acc = {0.f, 0.f, 0.f};
+    // what came before: the records of the kblk whole blocks of tiles before this one, then those of the itile
+    // earlier tiles of its own block (a row of 1024 tiles costs its last tile 31 + 31 records, not 1023), RT per round
+    const int kblk = tile / kLbBlock, itile = tile - kblk * kLbBlock;
+    const int nprev = kblk + itile;
+    const unsigned long long* bsrc = P.brec + (size_t)b * P.nblk * W;
+    const unsigned long long* tsrc = P.rec + (trow + (size_t)kblk * kLbBlock) * W;
+    const int nwb = kblk * W;                         // words of the block records
+    Moments accB = {0.f, 0.f, 0.f}, accT = {0.f, 0.f, 0.f};
     uint32_t prevcnt = 0;
-    for (int p0 = 0; p0 < tile; p0 += RT) {
-      const int np = min(RT, tile - p0);
+    auto fetch = [&](const int r0, const int r1) {      // records r0 .. r1 - 1 of the list
+    for (int p0 = r0; p0 < r1; p0 += RT) {
+      const int np = min(RT, r1 - p0);
       __syncthreads();                              // the staging buffers are free again
       {
         // all loads of a batch are issued before the first one is looked at
         constexpr int kBatch = 8;
-        const unsigned long long* src0 = P.rec + (trow + p0) * W;
+        const int w0 = p0 * W;                        // first word of this round in the list of all records
         const int nw = np * W;
+        auto word = [&](const int i) -> const unsigned long long* {
+          const int gw = w0 + i;
+          return gw < nwb ? bsrc + gw : tsrc + (gw - nwb);
+        };
         for (int i0 = tid; i0 < nw; i0 += kThreads * kBatch) {
           unsigned long long w[kBatch];
 #pragma unroll
           for (int u = 0; u < kBatch; ++u) {
             const int i = i0 + u * kThreads;
-            w[u] = i < nw ? get_rec(src0 + i) : tagged(0u, tag);
+            w[u] = i < nw ? get_rec(word(i)) : tagged(0u, tag);
           }
           // words that are not there yet are asked for again together, one round trip per round
           uint32_t spins = 0;
@@ -284,7 +300,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
               const int i = i0 + u * kThreads;
-              if ((uint32_t)(w[u] >> 32) != tag) w[u] = get_rec(src0 + i);
+              if ((uint32_t)(w[u] >> 32) != tag) w[u] = get_rec(word(i));
             }
           }
 #pragma unroll
@@ -302,12 +318,33 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
         a.n = (float)c;
         a.mean = __uint_as_float((uint32_t)rw[1 + 2 * gc]);
         a.var = __uint_as_float((uint32_t)rw[2 + 2 * gc]);
-        acc = merge(acc, a);
+        if (p0 + i < kblk) accB = merge(accB, a);
+        else accT = merge(accT, a);
         prevcnt += c;
       }
     }
+    };
+    // the last tile of a block first collects the block's own tiles and leaves the block's aggregate for the tiles
+    // of the later blocks, then turns to the earlier blocks: a block record never waits for another block record.
+    // A tile that gave up leaves nothing, so that the later ones give up as well instead of building on a partial sum
+    const bool closes_block = itile == kLbBlock - 1;
+    if (closes_block) {
+      fetch(kblk, nprev);
+      accT = row_reduce(accT);
+      if (l16 == 15 && active && s_gave_up == 0u) {
+        unsigned long long* mine = P.brec + ((size_t)b * P.nblk + kblk) * W;
+        const Moments ba = merge(accT, inc);
+        put_rec(mine + 1 + 2 * g, tagged(__float_as_uint(ba.mean), tag));
+        put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(ba.var), tag));
+        if (g == 0) put_rec(mine, tagged((uint32_t)ba.n, tag));
+      }
+      fetch(0, kblk);
+    } else {
+      fetch(0, nprev);
+      accT = row_reduce(accT);
+    }
     MEGA_TSN_TR(3);
-    acc = row_reduce(acc);
+    Moments acc = merge(row_reduce(accB), accT);
     // words that never came: everything this tile derives from the earlier tiles is NaN, not a partial sum
     const bool poison = s_gave_up != 0u;
     if (poison) acc.mean = __builtin_nanf("");
@@ -674,8 +711,9 @@ int dispatch_vec(const TsnParams& P, const TsnGeom& g, hipStream_t s) {
   return launch_group_tsn<T, 1>(P, g, s);
 }
 
+// header, tile records, block records
 size_t tsn_workspace_bytes(int64_t B, int64_t G, int ntiles) {
-  const size_t n = (size_t)B * ntiles;
+  const size_t n = (size_t)B * ntiles + (size_t)B * ceil_div(ntiles, kLbBlock);
   return align_up(sizeof(TsnHeader), 256) + align_up(n * (2 * (size_t)G + 1) * 8, 256);
 }
 
@@ -742,7 +780,7 @@ static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* 
   if (fixed_scratch) {
     MEGA_REQUIRE(workspace_bytes >= tsn_workspace_bytes(B, G, g.ntiles), MEGA_ERR_UNSUPPORTED,
                  "group_timestep_norm_fwd_noalloc: B=%ld L=%ld G=%ld needs %zu bytes of tile records, the library's "
-                 "fixed scratch array holds %zu (B * ceil(L / %d) * (2 G + 1) * 8 + 256 must fit); use "
+                 "fixed scratch array holds %zu (B * (T + ceil(T / 32)) * (2 G + 1) * 8 + 256 with T = ceil(L / %d) must fit); use "
                  "mega_group_timestep_norm_fwd with a caller workspace",
                  (long)B, (long)L, (long)G, tsn_workspace_bytes(B, G, g.ntiles), workspace_bytes, g.tt);
   }
@@ -756,8 +794,9 @@ static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* 
   P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd;
   P.hdr = (TsnHeader*)w; w += align_up(sizeof(TsnHeader), 256);
   P.rec = (unsigned long long*)w;
+  P.brec = P.rec + (size_t)B * g.ntiles * (2 * (size_t)G + 1);
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G;
-  P.TT = g.tt; P.ntiles = g.ntiles; P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
+  P.TT = g.tt; P.ntiles = g.ntiles; P.nblk = (int)ceil_div(g.ntiles, kLbBlock); P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
   P.lb = lookback_launch(!fixed_scratch);
   switch (dtype) {
     case MEGA_F32: return dispatch_vec<float>(P, g, s);

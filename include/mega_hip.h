@@ -309,7 +309,8 @@ int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* pre
  * itself allocates and frees nothing.  Same arguments, results and errors as
  * mega_group_timestep_norm_fwd, plus:
  *   - MEGA_ERR_UNSUPPORTED when the tile records do not fit:
- *     256 + B * ceil(L / TT) * (2 G + 1) * 8 bytes <= 1 MiB, TT = tokens per tile (<= 64;
+ *     256 + B * (T + ceil(T / 32)) * (2 G + 1) * 8 bytes <= 1 MiB with T = ceil(L / TT) tiles,
+ *     TT = tokens per tile (<= 64; one more record per 32 tiles holds their aggregate;
  *     mega_timestep_norm_workspace_bytes returns the exact figure for a shape);
  *   - the first call on a device looks the array's address up (hipGetSymbolAddress): make
  *     that call outside stream capture;

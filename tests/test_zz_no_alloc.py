@@ -61,7 +61,7 @@ def test_noalloc_matches_workspace_entry_twice_then_rejects_oversize():
         for a, b, name in zip(got, ref, ("y", "count", "mean", "var", "group_mean", "cummean", "cumrstd")):
             assert torch.equal(a, b), f"{name} differs at shape {(B, L, H, G)}"
         assert not torch.isnan(got[0].float()).any()
-    # tile records beyond the array: 256 + B * ceil(L / TT) * (2 G + 1) * 8 > 1 MiB
+    # tile and block records beyond the array: 256 + B * (T + ceil(T / 32)) * (2 G + 1) * 8 > 1 MiB, T = ceil(L / TT)
     need = lib.mega_timestep_norm_workspace_bytes(1, 64, 16384, 1024, 16)
     assert need > (1 << 20)
     a = 0x10000
