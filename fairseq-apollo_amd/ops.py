@@ -1203,19 +1203,37 @@ def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torc
     dom = torch.empty(D, dtype=torch.float32, device=dev)
     m8 = _mask_u8(padding_mask, B, L)
     stream = _stream(dev)
-    ws = _scratch_buffer(dev, lib.mega_ema_param_grad_workspace_bytes(B, D, N), stream)
     # first D rows: the causal half; second D rows (two-sided layers): the same sums over the tokens
     # walked backwards, lags starting at 1 when the layer shifts its backward kernel
     halves = [(0, 0, 0)] + ([(D, 1, 1 if layer.shift else 0)] if layer.bidirectional else [])
-    scratch_om = dom if not layer.bidirectional else torch.empty_like(dom)
+    # the sums of one state do not involve the others: more than 16 states go through the kernel 16 at a time
+    NS = 16
+    scratch_om = dom if (not layer.bidirectional and N <= NS) else torch.empty_like(dom)
     with _on_device(dev):
         for off, rev, lag in halves:
-            rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
-                                         xd.stride(0), xd.stride(1), xd.stride(2), _ptr(layer.p[off:]),
-                                         _ptr(layer.q[off:]), _ptr(layer.gamma[off:]), _ptr(m8), B, D, N, L, rev, lag,
-                                         _ptr(dp[off:]), _ptr(dq[off:]), _ptr(dg[off:]),
-                                         _ptr(dom if off == 0 else scratch_om), _ptr(ws), ws.numel(), stream)
-            _lib.check(rc, "ema_param_grad")
+            for n0 in range(0, N, NS):
+                n1 = min(N, n0 + NS)
+                whole = n0 == 0 and n1 == N
+                pp = layer.p[off:off + D] if whole else layer.p[off:off + D, n0:n1].contiguous()
+                qq = layer.q[off:off + D] if whole else layer.q[off:off + D, n0:n1].contiguous()
+                gg = layer.gamma[off:off + D] if whole else layer.gamma[off:off + D, n0:n1].contiguous()
+                if whole:
+                    tp, tq, tg = dp[off:], dq[off:], dg[off:]
+                else:
+                    tp = torch.empty(D, n1 - n0, dtype=torch.float32, device=dev)
+                    tq = torch.empty(D, n1 - n0, 2, dtype=torch.float32, device=dev)
+                    tg = torch.empty(D, n1 - n0, 2, dtype=torch.float32, device=dev)
+                ws = _scratch_buffer(dev, lib.mega_ema_param_grad_workspace_bytes(B, D, n1 - n0), stream)
+                rc = lib.mega_ema_param_grad(_ptr(g), _ptr(xd), _dtype_code(xd), g.stride(0), g.stride(1), g.stride(2),
+                                             xd.stride(0), xd.stride(1), xd.stride(2), _ptr(pp), _ptr(qq), _ptr(gg),
+                                             _ptr(m8), B, D, n1 - n0, L, rev, lag, _ptr(tp), _ptr(tq), _ptr(tg),
+                                             _ptr(dom if (off == 0 and n0 == 0) else scratch_om), _ptr(ws), ws.numel(),
+                                             stream)
+                _lib.check(rc, "ema_param_grad")
+                if not whole:
+                    dp[off:off + D, n0:n1] = tp
+                    dq[off:off + D, n0:n1] = tq
+                    dg[off:off + D, n0:n1] = tg
     if layer.is_complex:
         return dx, dp, torch.view_as_complex(dq), torch.view_as_complex(dg), dom
     return dx, dp, dq[..., 0], dg[..., 0], dom

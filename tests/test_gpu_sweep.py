@@ -278,7 +278,7 @@ def test_moving_average_backward_sweep(seed):
         L = int(rng.choice([1, 31, 64, 100, 256, 300, 511, 1024, 1100, 1544, 2048]))
         D = int(rng.choice([1, 5, 16, 24, 40]))
         B = int(rng.choice([1, 2, 3]))
-        N = int(rng.choice([1, 2, 7, 16]))
+        N = int(rng.choice([1, 2, 7, 16, 24, 32]))
         cplx = bool(rng.integers(0, 2))
         bidir = bool(rng.integers(0, 2))
         shift = bool(rng.integers(0, 2))
@@ -520,3 +520,58 @@ def test_streaming_equals_one_shot_sweep(seed):
         torch.cuda.synchronize()
         assert rel_err(host(torch.cat(parts, 1)), host(full)) < 2e-4, (tag, cuts)
     assert M.ops.timestep_norm_status() == 0
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_kernel_generation_and_state_operators_sweep(seed):
+    """ema_parameters (kernel and carried-state bias) and ema_hidden (state after the last token), forward and
+    backward, at operator level (fairseq/csrc/ops/ema_parameters.cc:80-286, ema_hidden.cc:66-194): state counts
+    from 1 to 32, lengths from 1 to past a tile, with and without a carried state."""
+    rng = np.random.default_rng(12000 + seed)
+    for case in range(5):
+        D = int(rng.choice([1, 3, 16, 40]))
+        N = int(rng.choice([1, 2, 7, 16, 32]))
+        L = int(rng.choice([1, 2, 31, 64, 100, 513]))
+        B = int(rng.choice([1, 2, 3]))
+        with_h = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: B={B} D={D} N={N} L={L} h={with_h}"
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, D, N, True)
+        p = p.astype(np.float32).astype(np.float64)
+        q, g = q.astype(np.complex64).astype(np.complex128), g.astype(np.complex64).astype(np.complex128)
+        h = None
+        if with_h:
+            h = (rng.normal(size=(B, D, N)) + 1j * rng.normal(size=(B, D, N))).astype(np.complex64).astype(np.complex128)
+        x, x64 = rounded(rng.normal(size=(B, D, L)), torch.float32)
+        tq = dev(q)
+        th = None if h is None else dev(h)
+        w, bias, _ = M.ops.ema_parameters_fwd(dev(p), tq.log(), dev(g), th, L)
+        assert rel_err(host(w), O.ema_kernel(p, q, g, L)) < 1e-4, tag
+        if with_h:
+            assert rel_err(host(bias), O.ema_bias(q, g, h, L)) < 1e-4, tag
+        hy, _ = M.ops.ema_hidden_fwd(x, dev(p), tq.log(), th)
+        ho = O.ema_hidden(x64, p, q, h)
+        assert rel_err(np.real(host(hy)), np.real(ho)) < 1e-4 and rel_err(np.imag(host(hy)), np.imag(ho)) < 1e-4, tag
+        # backward of both
+        dk = rng.normal(size=(D, L)).astype(np.float32).astype(np.float64)
+        db = rng.normal(size=(B, D, L)).astype(np.float32).astype(np.float64) if with_h else None
+        dp, dq, dg, dh = M.ops.ema_parameters_bwd(dev(dk), None if db is None else dev(db), dev(p), tq.log(), dev(g), th)
+        rp, rq, rg = O.ema_kernel_bwd(dk, p, q, g)
+        if with_h:
+            bq, bg, bh = O.ema_bias_bwd(db, q, g, h)
+            rq, rg = rq + bq, rg + bg
+            assert _state_err(np.real(host(dh)), np.real(bh)) < 5e-4 and _state_err(np.imag(host(dh)), np.imag(bh)) < 5e-4, tag
+        assert rel_err(host(dp), rp) < 5e-4, tag
+        for a, r_, name in ((dq, rq, "dq"), (dg, rg, "dgamma")):
+            a = host(a)
+            assert rel_err(a.real, r_.real) < 5e-4 and rel_err(a.imag, r_.imag) < 5e-4, (tag, name)
+        dy = (rng.normal(size=(B, D, N)) + 1j * rng.normal(size=(B, D, N))).astype(np.complex64).astype(np.complex128)
+        dx, dp2, dq2, dh2 = M.ops.ema_hidden_bwd(dev(dy), x, dev(p), tq.log(), th)
+        torch.cuda.synchronize()
+        ox, op_, oq, oh = O.ema_hidden_bwd(dy, x64, p, q, h)
+        assert rel_err(host(dx), ox) < 5e-4 and rel_err(host(dp2), op_) < 5e-4, tag
+        a = host(dq2)
+        assert rel_err(a.real, oq.real) < 5e-4 and rel_err(a.imag, oq.imag) < 5e-4, tag
+        if with_h:
+            a = host(dh2)
+            assert _state_err(a.real, oh.real) < 5e-4 and _state_err(a.imag, oh.imag) < 5e-4, tag
