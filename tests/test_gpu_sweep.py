@@ -426,6 +426,26 @@ def test_gated_attention_layer_sweep(seed):
         grads = [xg.grad] + [prm.grad for prm in layer.parameters() if prm.requires_grad]
         assert all(gr is not None and torch.isfinite(gr).all() for gr in grads), tag
         assert xg.grad.abs().max().item() > 0, tag
+        if L <= 128:
+            # a few entries of the input and projection gradients against central differences of the oracle
+            okw = dict(chunk=C, num_heads=heads, moving_act=act, num_groups=G, bidirectional=bidir, padding_mask=mask)
+            w64, x64 = host(wgt), host(x)
+            loss = lambda Pd, xx: (O.gated_attention_layer(xx, Pd, **okw) * w64).sum()
+            eps = 1e-5
+            gx = host(xg.grad)
+            for _ in range(2):
+                idx = tuple(int(rng.integers(0, n)) for n in x64.shape)
+                xp, xm = x64.copy(), x64.copy()
+                xp[idx] += eps; xm[idx] -= eps
+                fd = (loss(P, xp) - loss(P, xm)) / (2 * eps)
+                assert abs(fd - gx[idx]) < 3e-3 * (np.abs(gx).max() + 1e-6), (tag, "x", idx, fd, gx[idx])
+            for name, prm in (("mx_w", layer.mx_proj.weight), ("gamma", layer.gamma), ("norm_weight", layer.norm.weight)):
+                gp = host(prm.grad)
+                idx = tuple(int(rng.integers(0, n)) for n in P[name].shape)
+                Pp = dict(P); Pp[name] = P[name].copy(); Pp[name][idx] += eps
+                Pm = dict(P); Pm[name] = P[name].copy(); Pm[name][idx] -= eps
+                fd = (loss(Pp, x64) - loss(Pm, x64)) / (2 * eps)
+                assert abs(fd - gp[idx]) < 3e-3 * (np.abs(gp).max() + 1e-6), (tag, name, idx, fd, gp[idx])
 
 
 @pytest.mark.parametrize("seed", range(8))
