@@ -426,6 +426,22 @@ def test_gated_attention_layer_sweep(seed):
         grads = [xg.grad] + [prm.grad for prm in layer.parameters() if prm.requires_grad]
         assert all(gr is not None and torch.isfinite(gr).all() for gr in grads), tag
         assert xg.grad.abs().max().item() > 0, tag
+        # the 16-bit kernels (other vector widths and alignment rules) on the same shape: close to the fp32 result
+        # in the root mean square, and a training step that runs
+        import copy
+        for dt16 in (torch.bfloat16, torch.float16):
+            l16 = copy.deepcopy(layer).to(dt16).eval()
+            with torch.no_grad():
+                y16, _ = l16(x.to(dt16), None if mask is None else dev(mask, torch.bool))
+            e = (host(y16) - host(y))[keep]
+            assert np.isfinite(e).all() and np.sqrt(np.mean(e ** 2)) < 5e-2 * np.sqrt(np.mean(host(y)[keep] ** 2)), (tag, dt16)
+            l16.train()
+            x16 = x.to(dt16).requires_grad_(True)
+            yt16, _ = l16(x16, None if mask is None else dev(mask, torch.bool))
+            (yt16.float() * wgt).sum().backward()
+            torch.cuda.synchronize()
+            e = (host(x16.grad) - host(xg.grad))
+            assert np.isfinite(e).all() and np.sqrt(np.mean(e ** 2)) < 0.1 * np.sqrt(np.mean(host(xg.grad) ** 2)) + 1e-6, (tag, dt16)
         if L <= 128:
             # a few entries of the input and projection gradients against central differences of the oracle
             okw = dict(chunk=C, num_heads=heads, moving_act=act, num_groups=G, bidirectional=bidir, padding_mask=mask)
