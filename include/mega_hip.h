@@ -242,7 +242,9 @@ int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, 
  *   domega[d] = sum_{b,t} dy[t] x[t].
  *   dy, x [B,D,L] of `dtype` with element strides; p [D,N], q, gamma [D,N,2] fp32 (imaginary
  *   parts 0 for the real layer); mask [B,L] or NULL; outputs dp [D,N], dq, dgamma [D,N,2],
- *   domega [D] fp32; N <= 16; workspace of mega_ema_param_grad_workspace_bytes(B, D, N).
+ *   domega [D] fp32; N <= 16 per call (the sums of one state do not involve the others: a layer
+ *   with more states passes slices of 16 columns of p, q, gamma); workspace of
+ *   mega_ema_param_grad_workspace_bytes(B, D, N).
  *   A two-sided layer takes two calls: its first D coefficient rows as above; its second D rows
  *   with reverse_time = 1 (the tokens are walked from the last to the first) and lag_one = shift
  *   (dy[t] is paired with the state before token t: kernel lags start at 1).               */
