@@ -37,6 +37,11 @@ constexpr int kMaxTT = 64;                    // tokens per tile (16 lanes x 4 t
 constexpr int kLbWords = 4352;                // 64-bit words staged in LDS per look-back round
 constexpr int kLbBlock = 32;                  // tiles per block record: a tile looks back over the whole blocks before
                                               // it and the earlier tiles of its own block, not over every earlier tile
+#ifndef MEGA_TSN_LBDIRECT
+#define MEGA_TSN_LBDIRECT 128
+#endif
+constexpr int kLbDirect = MEGA_TSN_LBDIRECT;  // rows of up to this many tiles look back over the tiles themselves: one
+                                              // round of records, and no wait for a block's last tile to add its block up
 
 struct TsnParams {
   const void* x;
@@ -257,10 +262,11 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     MEGA_TSN_TR(2);
     // what came before: the records of the kblk whole blocks of tiles before this one, then those of the itile
     // earlier tiles of its own block (a row of 1024 tiles costs its last tile 31 + 31 records, not 1023), RT per round
-    const int kblk = tile / kLbBlock, itile = tile - kblk * kLbBlock;
+    const int lbb = P.ntiles > kLbDirect ? kLbBlock : P.ntiles;   // tiles per block record (the whole row: none)
+    const int kblk = tile / lbb, itile = tile - kblk * lbb;
     const int nprev = kblk + itile;
     const unsigned long long* bsrc = P.brec + (size_t)b * P.nblk * W;
-    const unsigned long long* tsrc = P.rec + (trow + (size_t)kblk * kLbBlock) * W;
+    const unsigned long long* tsrc = P.rec + (trow + (size_t)kblk * lbb) * W;
     const int nwb = kblk * W;                         // words of the block records
     Moments accB = {0.f, 0.f, 0.f}, accT = {0.f, 0.f, 0.f};
     uint32_t prevcnt = 0;
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     // the last tile of a block first collects the block's own tiles and leaves the block's aggregate for the tiles
     // of the later blocks, then turns to the earlier blocks: a block record never waits for another block record.
     // A tile that gave up leaves nothing, so that the later ones give up as well instead of building on a partial sum
-    const bool closes_block = itile == kLbBlock - 1;
+    const bool closes_block = itile == lbb - 1 && P.ntiles > kLbDirect;
     if (closes_block) {
       fetch(kblk, nprev);
       accT = row_reduce(accT);
