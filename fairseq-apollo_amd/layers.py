@@ -22,7 +22,7 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU, norm_then_move,
+from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU, linear_residual, norm_then_move,
                       TimestepNorm, _tensor_versions, _training_call)
 
 
@@ -95,6 +95,8 @@ class NormalizedFeedForwardNetwork(nn.Module):
 
     def forward(self, x: Tensor) -> Tensor:
         h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
+        if self.layerscale_weight is None and not (self.training and self.dropout_p > 0):
+            return linear_residual(self.fc2, h, x)      # the residual rides in the product
         h = F.dropout(self.fc2(h), self.dropout_p, self.training)
         if self.layerscale_weight is not None:
             h = h * self.layerscale_weight
@@ -534,7 +536,7 @@ class Mega2Layer(nn.Module):
 
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, incremental_state=None) -> Tensor:
         x, _ = self.attn(x, padding_mask, incremental_state)
-        return x + self.ffn(self.ffn_norm(x, padding_mask, incremental_state))
+        return self.ffn(self.ffn_norm(x, padding_mask, incremental_state), residual=x)
 
 
 def _arg(args, name, default):

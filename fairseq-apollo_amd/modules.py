@@ -766,6 +766,17 @@ class EfficientAttention(nn.Module):
         return 'causal={}, dropout={}'.format(self._causal, self._dropout)
 
 
+def linear_residual(lin: nn.Linear, h: Tensor, residual: Optional[Tensor]) -> Tensor:
+    """lin(h) + residual as one library GEMM (the residual is the accumulator's start, rounded once with the
+    product); lin(h) when there is no residual."""
+    if residual is None:
+        return lin(h)
+    if lin.bias is not None or residual.dtype != h.dtype or not residual.is_contiguous():
+        return lin(h) + residual
+    out = torch.addmm(residual.reshape(-1, residual.shape[-1]), h.reshape(-1, h.shape[-1]), lin.weight.t())
+    return out.view(residual.shape)
+
+
 class SwiGLU(nn.Module):
     """W2 (silu(W1 x) * W3 x) with the gate evaluated by the HIP kernel; the three
     projections are library GEMMs."""
@@ -776,7 +787,8 @@ class SwiGLU(nn.Module):
         self.w3 = nn.Linear(embed_dim, hidden_dim, bias=bias)
         self.w2 = nn.Linear(hidden_dim, embed_dim, bias=bias)
 
-    def forward(self, x: Tensor) -> Tensor:
-        if _training_call(self, x):
-            return self.w2(SwiGLUFunc.apply(self.w1(x), self.w3(x)))
-        return self.w2(ops.swiglu(self.w1(x), self.w3(x)))
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+        """W2 (silu(W1 x) * W3 x) (+ residual, which then enters the last product as its accumulator start: no
+        separate addition pass over the activations)."""
+        gate = SwiGLUFunc.apply(self.w1(x), self.w3(x)) if _training_call(self, x) else ops.swiglu(self.w1(x), self.w3(x))
+        return linear_residual(self.w2, gate, residual)
