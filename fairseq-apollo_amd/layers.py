@@ -80,16 +80,13 @@ class NormalizedFeedForwardNetwork(nn.Module):
         self.reset_parameters(init_mode)
 
     def reset_parameters(self, mode):
-        if mode == 'bert':
-            nn.init.normal_(self.fc1.weight, mean=0.0, std=0.02)
-            nn.init.normal_(self.fc2.weight, mean=0.0, std=0.02)
-        elif mode == 'he':
-            nn.init.kaiming_normal_(self.fc1.weight, a=math.sqrt(5.0))
-            nn.init.kaiming_normal_(self.fc2.weight, a=math.sqrt(5.0))
-        else:
-            nn.init.xavier_uniform_(self.fc1.weight)
-            nn.init.xavier_uniform_(self.fc2.weight)
-        nn.init.constant_(self.fc1.bias, 0.0)
+        """'bert': N(0, 0.02); 'he': Kaiming normal with a = sqrt(5); otherwise Xavier uniform; zero bias; the layer
+        scale starts at its given value (normalized_feedforward_network.py:56-75)."""
+        init = {'bert': lambda w: nn.init.normal_(w, mean=0.0, std=0.02),
+                'he': lambda w: nn.init.kaiming_normal_(w, a=math.sqrt(5.0))}.get(mode, nn.init.xavier_uniform_)
+        for lin in (self.fc1, self.fc2):
+            init(lin.weight)
+        nn.init.zeros_(self.fc1.bias)
         if self.layerscale_weight is not None:
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 

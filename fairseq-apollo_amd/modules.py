@@ -279,25 +279,22 @@ class MultiHeadEMA(BaseMovingLayer):
         self.reset_parameters()
 
     def reset_parameters(self):
+        """alpha, delta ~ N(0, 0.2); beta = +1, -1, +1, ... along the states plus N(0, 0.02); gamma, omega ~ N(0, 1)
+        (exponential_moving_average.py:47-69)."""
         with torch.no_grad():
-            nn.init.normal_(self.alpha, mean=0.0, std=0.2)
-            nn.init.normal_(self.delta, mean=0.0, std=0.2)
-            # beta alternates +1 / -1 around a small normal perturbation
-            val = torch.ones(self.ndim, 1)
-            if self.ndim > 1:
-                val[1::2] = -1.0
-            self.beta.normal_(mean=0.0, std=0.02).add_(val)
-            nn.init.normal_(self.gamma, mean=0.0, std=1.0)
-            nn.init.normal_(self.omega, mean=0.0, std=1.0)
+            self.alpha.normal_(0.0, 0.2)
+            self.delta.normal_(0.0, 0.2)
+            signs = 1.0 - 2.0 * (torch.arange(self.ndim) % 2).to(self.beta.dtype)
+            self.beta.normal_(0.0, 0.02).add_(signs.view(1, self.ndim, 1))
+            self.gamma.normal_(0.0, 1.0)
+            self.omega.normal_(0.0, 1.0)
 
     def _calc_coeffs(self):
+        """p = sigmoid(alpha) beta, q = 1 - sigmoid(alpha) sigmoid(delta), gamma scaled by sqrt(1 / N)
+        (exponential_moving_average.py:71-80)."""
         self._coeffs = None
-        alpha = torch.sigmoid(self.alpha.float())
-        delta = torch.sigmoid(self.delta.float())
-        q = 1.0 - alpha * delta
-        p = alpha * self.beta.float()
-        gamma = self.gamma.float() * self.scale
-        return p, q, gamma
+        a = torch.sigmoid(self.alpha.float())
+        return a * self.beta.float(), 1.0 - a * torch.sigmoid(self.delta.float()), self.gamma.float() * self.scale
 
 
 class MultiHeadComplexEMA(BaseMovingLayer):
@@ -321,31 +318,31 @@ class MultiHeadComplexEMA(BaseMovingLayer):
         self.reset_parameters()
 
     def reset_parameters(self):
+        """Initial values as the reference draws them (complex_exponential_moving_average.py:47-77): alpha, delta
+        ~ N(0, 0.2); theta = logit of the base frequencies D^(-j / D), j = 1..D, shuffled over the channels (both
+        directions of a two-sided layer share them); gamma real-valued ~ N(0, 1); omega ~ N(0, 1)."""
+        D = self.embed_dim
         with torch.no_grad():
-            nn.init.normal_(self.alpha, mean=0.0, std=0.2)
-            nn.init.normal_(self.delta, mean=0.0, std=0.2)
-            # theta: logit of a random permutation of exp(-j ln(D) / D), j = 1..D
-            freqs = math.log(self.embed_dim) / self.embed_dim
-            freqs = torch.exp(torch.arange(1, self.embed_dim + 1) * -freqs)
-            freqs = freqs[torch.randperm(self.embed_dim)].to(self.theta).view(self.embed_dim, 1, 1)
-            if self.bidirectional:
-                freqs = freqs.repeat(2, 1, 1)
-            self.theta.copy_(torch.log(freqs / (1.0 - freqs)))
-            nn.init.normal_(self.gamma, mean=0.0, std=1.0)
-            self.gamma[:, :, 1] = 0.
-            nn.init.normal_(self.omega, mean=0.0, std=1.0)
+            self.alpha.normal_(0.0, 0.2)
+            self.delta.normal_(0.0, 0.2)
+            base = torch.exp(torch.arange(1, D + 1) * (-math.log(D) / D))
+            base = base[torch.randperm(D)].to(self.theta).view(D, 1, 1)
+            self.theta.copy_(torch.logit(base.repeat(2, 1, 1) if self.bidirectional else base))
+            self.gamma.normal_(0.0, 1.0)
+            self.gamma[..., 1].zero_()
+            self.omega.normal_(0.0, 1.0)
 
     def _calc_coeffs(self):
+        """p = sigmoid(alpha); q: state n of a channel shrinks by 1 - sigmoid(alpha) sigmoid(delta) and turns by
+        (n + 1) sigmoid(theta) 2 pi / N per token; gamma complex, scaled by sqrt(1 / N)
+        (complex_exponential_moving_average.py:79-96)."""
         self._coeffs = None
-        theta = torch.sigmoid(self.theta.float()) * (2 * math.pi / self.ndim)
-        wavelets = torch.arange(1, self.ndim + 1, dtype=theta.dtype, device=theta.device).view(1, self.ndim)
-        theta = wavelets.unsqueeze(2) * theta
-        alpha = torch.sigmoid(self.alpha.float())
-        delta = torch.sigmoid(self.delta.float())
-        p = alpha
-        q = torch.polar(1.0 - alpha * delta, theta)
-        gamma = torch.view_as_complex(self.gamma.float().contiguous()) * self.scale
-        return p, q, gamma
+        a = torch.sigmoid(self.alpha.float())
+        d = torch.sigmoid(self.delta.float())
+        turn = torch.sigmoid(self.theta.float()) * (2.0 * math.pi / self.ndim)                      # [K, 1, 1]
+        harmonic = torch.arange(1, self.ndim + 1, dtype=turn.dtype, device=turn.device).view(1, self.ndim, 1)
+        q = torch.polar(1.0 - a * d, harmonic * turn)
+        return a, q, torch.view_as_complex(self.gamma.float().contiguous()) * self.scale
 
 
 class TimestepNormFunc(torch.autograd.Function):
