@@ -73,6 +73,7 @@ SIGNATURES = {
     "mega_attention_fwd": (_int, [_p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_float, _int, C.c_float,
                                   C.c_uint64, _p, _sz, _p]),
     "mega_swiglu_fwd": (_int, [_p, _p, _p, _int, _i64, _p]),
+    "mega_silu_fwd": (_int, [_p, _p, _int, _i64, _p]),
     "mega_rms_norm_fwd": (_int, [_p, _i64, _p, _p, _int, _i64, _i64, C.c_double, _p]),
     "mega_gate_qk_fwd": (_int, [_p, _i64, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_double, _p]),
     "mega_gate_qk_bwd_workspace_bytes": (_sz, [_i64, _i64]),

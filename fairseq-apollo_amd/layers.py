@@ -91,7 +91,10 @@ class NormalizedFeedForwardNetwork(nn.Module):
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 
     def forward(self, x: Tensor) -> Tensor:
-        h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
+        if _training_call(self, x):
+            h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
+        else:
+            h = ops.silu(self.fc1(self.norm(x)), inplace=True)
         if self.layerscale_weight is None and not (self.training and self.dropout_p > 0):
             return linear_residual(self.fc2, h, x)      # the residual rides in the product
         h = F.dropout(self.fc2(h), self.dropout_p, self.training)
@@ -269,10 +272,11 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             mx = None
         else:
             x, mx = norm_then_move(self.norm, self.move, x, padding_mask, incremental_state, out_layout="input")
-        v = F.silu(self.v_proj(x))
+        v = ops.silu(self.v_proj(x), inplace=True)
         if mx is None:
             mx = self.move(x.transpose(1, 2), padding_mask, incremental_state, out_layout="input")
-        mx = self.move_act(mx.transpose(1, 2))
+        mx = mx.transpose(1, 2)
+        mx = self.move_act(mx) if isinstance(self.move_act, RMSNorm) else ops.silu(mx, inplace=True)
         base = self.mx_proj(mx)
         u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
         Nh = self.num_heads

@@ -1044,6 +1044,21 @@ def swiglu(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return y
 
 
+def silu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
+    """x / (1 + exp(-x)), elementwise (F.silu; moving_average_gated_attention.py:303-316,
+    normalized_feedforward_network.py:82); `inplace` overwrites a contiguous x."""
+    dev = _need_gpu(x)
+    lib = _lib.load()
+    xd = x.detach()
+    if not xd.is_contiguous():
+        xd, inplace = xd.contiguous(), True
+    y = xd if inplace else torch.empty_like(xd)
+    with _on_device(dev):
+        rc = lib.mega_silu_fwd(_ptr(xd), _ptr(y), _dtype_code(xd), xd.numel(), _stream(dev))
+    _lib.check(rc, "silu_fwd")
+    return y
+
+
 # ------------------------------------------------------------------------------------------------
 # per-token glue of the gated-attention layer (rows of a wider projection output are passed in
 # place: every input carries its own row stride)

@@ -433,6 +433,13 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, voi
  * the reference's F.silu.                                                         */
 int mega_swiglu_fwd(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
 
+/* The activation alone: y = silu(a) = a / (1 + exp(-a)), elementwise over n elements of `dtype`
+ * (arithmetic in fp32); y may be a itself.  Stands in for the F.silu calls of the layer on the
+ * value projection and the moving-average output
+ * (fairseq/modules/moving_average_gated_attention.py:303, 308, 316 with moving_act = silu) and of
+ * the feed-forward block (fairseq/modules/normalized_feedforward_network.py:82).                              */
+int mega_silu_fwd(const void* a, void* y, int dtype, int64_t n, void* stream);
+
 /* ------------------------------------------------------------------------ */
 /* Per-token glue of the gated-attention layer.  Inputs are [T, *] row-major with an
  * element stride per row (so a slice of a wider projection output is passed in place);

@@ -157,6 +157,22 @@ def test_attention_wide_score_range(gain, causal):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_silu(dtype, n):
+    """The activation alone, out of place, in place, and on a view that starts off the 16-byte boundary."""
+    rng = np.random.default_rng(28)
+    a, a64 = rounded(rng.normal(size=n + 3) * 3, dtype)
+    ref = a64 / (1.0 + np.exp(-a64))
+    tol = 1e-6 if dtype is torch.float32 else TOL[dtype]
+    y = M.ops.silu(a)
+    assert y.data_ptr() != a.data_ptr() and rel_err(host(y), ref) < tol
+    view = a[1:n + 1]
+    assert rel_err(host(M.ops.silu(view)), ref[1:n + 1]) < tol
+    b = a.clone()
+    assert M.ops.silu(b, inplace=True).data_ptr() == b.data_ptr() and rel_err(host(b), ref) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
 def test_swiglu(dtype, n):
     rng = np.random.default_rng(26)
     a, a64 = rounded(rng.normal(size=n) * 3, dtype)
