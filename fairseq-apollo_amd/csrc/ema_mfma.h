@@ -47,9 +47,12 @@ constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
 // bytes of the per-channel operand images for a layer (0: the layer is outside the fast path)
 size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional);
 
-// kernel generation: coefficients -> operand images
+// kernel generation: coefficients -> operand images.  parts: 1 = the bf16 K / P / C operands, 2 = the fp16 ones, 3 =
+// both (an image that is kept and may serve any activation type); a call that generates the image for itself asks
+// for the operands its own kernel reads
+constexpr int kImgBf16 = 1, kImgF16 = 2, kImgAll = 3;
 int ema_image_build(const float* p, const float* q, const float* gamma, int is_complex, const float* omega, int64_t D,
-                    int64_t N, int bidirectional, int shift, void* image, hipStream_t s);
+                    int64_t N, int bidirectional, int shift, void* image, hipStream_t s, int parts = kImgAll);
 
 // true when the streaming kernel handles this request (dtype, layout, alignment, sizes)
 bool ema_mfma_covers(int dtype, int64_t sxb, int64_t sxd, int64_t sxl, int64_t syb, int64_t syd, int64_t syl,

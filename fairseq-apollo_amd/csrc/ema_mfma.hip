@@ -57,6 +57,7 @@ struct ImageArgs {
   int K, D, N;
   int is_complex;
   int lag_back;          // rows >= D exclude the current sample (backward half with shift)
+  int parts;             // 1: the bf16 K / P / C operands are wanted, 2: the fp16 ones (the tables always are)
 };
 
 __device__ __forceinline__ float bf_split(float v, __bf16* h) {
@@ -198,18 +199,22 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     }
   }
   if (ok) {
+    if (A.parts & 1) {
 #pragma unroll
-    for (int w = 0; w < kNWK; ++w)
+      for (int w = 0; w < kNWK; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
+        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
 #pragma unroll
-    for (int w = 0; w < kNWP; ++w)
+      for (int w = 0; w < kNWP; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
+        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
 #pragma unroll
-    for (int w = 0; w < kNWC; ++w)
+      for (int w = 0; w < kNWC; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
+        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
+    } else {
+      slot += 2 * (kNWK + kNWP + kNWC);
+    }
     // q^32 of this lane's four states (2r, 2r+1, 8+2r, 9+2r)
     const float2 a = pw[32 * kNS + 2 * r], bq = pw[32 * kNS + 2 * r + 1];
     const float2 c = pw[32 * kNS + 8 + 2 * r], d = pw[32 * kNS + 9 + 2 * r];
@@ -270,14 +275,16 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       v = cmuld(v, v);
       cmp[kCmpRW * kNS + lane] = make_float2((float)v.re, (float)v.im);
     }
+    if (A.parts & 2) {
 #pragma unroll
-    for (int o = 0; o < 3; ++o)
+      for (int o = 0; o < 3; ++o)
 #pragma unroll
-      for (int w = 0; w < 2; ++w)
+        for (int w = 0; w < 2; ++w)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-          img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
-    if (lane < 56) {
+          for (int mb = 0; mb < 2; ++mb)
+            img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
+    }
+    if (lane < 56 && (A.parts & 1)) {
       // the K operand once per distinct content: lane (m, g) of row block mb holds k[16 mb + m - 8 g - t], t = 0..7,
       // which depends on delta = 16 mb + m - 8 g (-24..31) only; vector delta + 24 of term w sits at byte
       // 16 (delta + 24) of slot kSlotKT + w (7 lines per term instead of 16)
@@ -908,8 +915,9 @@ size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional) {
 }
 
 int ema_image_build(const float* p, const float* q, const float* gamma, int is_complex, const float* omega, int64_t D,
-                    int64_t N, int bidirectional, int shift, void* image, hipStream_t s) {
+                    int64_t N, int bidirectional, int shift, void* image, hipStream_t s, int parts) {
   ImageArgs A;
+  A.parts = parts;
   A.p = p; A.q = q; A.gamma = gamma; A.omega = omega; A.image = (uint4*)image;
   A.K = (int)(bidirectional ? 2 * D : D); A.D = (int)D; A.N = (int)N; A.is_complex = is_complex;
   A.lag_back = shift ? 1 : 0;

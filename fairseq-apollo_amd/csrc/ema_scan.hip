@@ -1381,7 +1381,8 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     const void* img = image;
     char* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
     if (!img) {
-      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s);
+      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s,
+                           dtype == MEGA_BF16 ? kImgBf16 : kImgF16);
       if (rc) return rc;
       img = wimg;
     }
@@ -1393,7 +1394,7 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     if (!img) {
       // no cached image: kernel generation runs with every call
       void* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
-      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s);
+      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s, kImgBf16);
       if (rc) return rc;
       img = wimg;
     }

@@ -909,7 +909,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     const void* img = image;
     if (!img) {
       // no cached image: kernel generation runs with every call
-      const int rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, 0, 1, scratch, s);
+      const int rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, 0, 1, scratch, s, kImgBf16);
       if (rc) return rc;
       img = scratch;
     }

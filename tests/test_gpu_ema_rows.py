@@ -109,3 +109,26 @@ def test_slow_poles_reach_across_all_blocks():
     yo, ho = O.ema_forward(x64, p, q, g, om, incremental=True)
     assert rel_err(host(y), yo) < 1e-4
     assert rel_err(np.real(host(h)), np.real(ho)) < 1e-4
+
+
+@pytest.mark.parametrize("dtype,B,D,layout", [(torch.float32, 2, 24, "rows"), (torch.float16, 1, 8, "rows"),
+                                              (torch.bfloat16, 1, 16, "rows"), (torch.bfloat16, 2, 64, "time_major")])
+def test_kernel_generation_inside_the_call(dtype, B, D, layout):
+    """Without a prepared image the call generates the operands its own kernel reads (the fp16 terms for fp32 /
+    fp16 rows, the bf16 terms for bf16 on either kernel): the same result as with the prepared image."""
+    rng = np.random.default_rng(35)
+    N, L = 16, 2048
+    p, q, g = _coeffs(rng, D, N, True)
+    om = rng.normal(size=D)
+    if layout == "rows":
+        x, _ = rounded(rng.normal(size=(B, D, L)), dtype)
+    else:
+        xt, _ = rounded(rng.normal(size=(B, L, D)), dtype)
+        x = xt.transpose(1, 2)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+    y0, h0 = layer(x, None, None, want_state=True)
+    saved, layer.image = layer.image, None
+    y1, h1 = layer(x, None, None, want_state=True)
+    layer.image = saved
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1) and torch.equal(torch.view_as_real(h0), torch.view_as_real(h1))
