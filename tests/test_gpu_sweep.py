@@ -99,6 +99,8 @@ def test_timestep_norm_sweep(seed):
         B = int(rng.choice([1, 2, 5]))
         masked = bool(rng.integers(0, 2))
         prior = bool(rng.integers(0, 2))
+        if H // (H if G is None else G) == 1 and L < 8:
+            L = 17              # one value per statistic and hardly any steps: the variance is 0, rstd = eps^-1/2 amplifies rounding
         tag = f"seed {seed} case {case}: {dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior}"
         print(tag, flush=True)
         Gn = H if G is None else G
