@@ -381,10 +381,11 @@ __global__ __launch_bounds__(256) void dropkey_f32_kernel(float* __restrict__ s,
 // Phase clocks: a profiling build defines these to add up the cycles a wave spends per phase; no-ops here.
 #ifndef MEGA_ATR
 #define MEGA_ATR_BEGIN()
+#define MEGA_ATR_MARK()
 #define MEGA_ATR(k)
 #define MEGA_ATR_END()
 #endif
-constexpr int FBM = 256, FBN = 64, FBD = 256, FNW = 8;
+constexpr int FBN = 64, FNW = 8;        // keys per tile, waves per workgroup
 
 struct FlashArgs {
   const void* q;      // [B, L, Nh, H1]
@@ -412,8 +413,32 @@ __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <typename T, int KS, int FQB>    // KS = H1 / 32 reduction steps of the first product, FQB blocks of 16 queries per wave
+// 16 bytes per lane from global memory straight into LDS (lane i of the wave lands at lds_base + 16 i).  Written as
+// assembly on purpose: the compiler cannot tell which LDS reads a tile in flight may alias and would make every
+// wave wait for the loads it has just issued (vmcnt(0)) before its first read of the current tile.  Here the
+// loads are invisible to that bookkeeping; the kernel waits for them itself (vmcnt(0), then the workgroup barrier)
+// before anybody reads the buffer they fill.
+__device__ __forceinline__ void lds_dma16(const void* base /* wave-uniform */, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_off), "s"(base), "s"(lds_base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma16(const void* addr /* per lane */, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(addr), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// KS = H1 / 32 reduction steps of the first product, FQB blocks of 16 queries per wave, FBD columns of v per
+// workgroup (FQB * FBD = 512: 128 accumulator registers per lane either way).  Launched as 32 queries x 256 columns
+// per wave; 16 queries x 512 columns (half as many workgroups repeat the score product and the softmax of a query
+// tile, twice the LDS reads per matrix instruction) measured the same within 3 % from H2 = 512 to 2048
+template <typename T, int KS, int FQB, int FBD>
 __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) {
+  constexpr int FBM = 16 * FNW * FQB;       // queries per workgroup
+  constexpr int VR = 64 * FNW / (FBD / 8);  // rows of the v tile one load instruction of the workgroup covers
   constexpr int H1 = 32 * KS;
   constexpr int QW = 16 * FQB;              // queries per wave
   constexpr int KROW = H1 * 2;              // bytes per k row in LDS (dense; 16-byte pieces XOR-swizzled by the row)
@@ -423,7 +448,7 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
   constexpr int NVL = FBD * (FBN / 8) / (64 * FNW);      // of a v^T tile
   static_assert(NKL >= 1 && FBN * KPC % (64 * FNW) == 0 && FBD * (FBN / 8) % (64 * FNW) == 0,
                 "the tiles must divide over the lanes");
-  extern __shared__ __attribute__((aligned(16))) char lds[];     // 2 x BUF
+  extern __shared__ __attribute__((aligned(16))) char lds[];     // two k tiles, then two v tiles
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int bz, mtile, slab;
@@ -470,8 +495,8 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
   // probability of zero meets a finite value.
   // common case (whole tile inside the sequence, whole slab inside v): one per-lane byte offset per operand,
   // everything else is uniform (load u of a lane is 32 u keys / 64 u rows of v^T further on)
-  uint32_t koff0, voff0;
-  {
+  uint32_t koff0, voffu[2];                  // v: loads of even / odd number (they differ in bit 3 of the row when a
+  {                                          // load covers 8 rows, and the swizzle looks at that bit)
     const int lrow = tid / KPC, pp = tid % KPC;
     const int a = lrow >> 5, hb = (lrow >> 4) & 1, gg = (lrow >> 2) & 3, t = lrow & 3;
     const int key = 32 * a + 8 * gg + 4 * hb + t;
@@ -481,27 +506,27 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
     // 32-byte spans are XOR-swizzled so that the transposing reads of a fragment (four rows, four 8-byte
     // columns per group of 16 lanes) fall on different banks
     const int r = tid / (FBD / 8), vp = tid % (FBD / 8);
-    const int p = ((((vp >> 1) ^ ((r & 3) + 4 * ((r >> 3) & 1))) << 1) | (vp & 1));
-    voff0 = (uint32_t)((r * (int)vs + p * 8) * 2);
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      const int rr = r + VR * par;             // a row of the loads with this parity
+      const int p = ((((vp >> 1) ^ ((rr & 3) + 4 * ((rr >> 3) & 1))) << 1) | (vp & 1));
+      voffu[par] = (uint32_t)((r * (int)vs + p * 8) * 2);
+    }
   }
   static_assert(64 * FNW / KPC == 32 || NKL == 1, "load u of the k tile starts 32 u keys further on");
-  static_assert(64 * FNW / (FBD / 8) == 16, "load u of the v tile starts 16 u keys further on");
+  static_assert(VR * NVL == FBN, "the loads of the v tile cover its rows in turn");
   const bool whole_slab = d0 + FBD <= A.H2;
-  auto issue_tile = [&](int kt, int buf) {
+  auto issue_tile = [&](int kt) {
     const int k0 = kt * FBN;
-    char* lk = lds + buf * BUF + wave * 1024;
-    char* lv = lds + buf * BUF + KB + wave * 1024;
+    const uint32_t lk = lds_addr(lds) + (kt & 1) * KB + wave * 1024;
+    const uint32_t lv = lds_addr(lds) + 2 * KB + (kt & 1) * VB + wave * 1024;
     if (whole_slab && k0 + FBN <= A.L) {
       const char* kbase = (const char*)(kb_ + (int64_t)k0 * rs);
       const char* vbase = (const char*)(vb + (int64_t)k0 * vs);
 #pragma unroll
-      for (int u = 0; u < NKL; ++u)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kbase + (int64_t)u * 32 * rs * 2 + koff0),
-                                         (__attribute__((address_space(3))) void*)(lk + u * 1024 * FNW), 16, 0, 0);
+      for (int u = 0; u < NKL; ++u) lds_dma16(kbase + (int64_t)u * 32 * rs * 2, koff0, lk + u * 1024 * FNW);
 #pragma unroll
-      for (int u = 0; u < NVL; ++u)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vbase + (int64_t)u * 16 * vs * 2 + voff0),
-                                         (__attribute__((address_space(3))) void*)(lv + u * 1024 * FNW), 16, 0, 0);
+      for (int u = 0; u < NVL; ++u) lds_dma16(vbase + (int64_t)u * VR * vs * 2, voffu[u & 1], lv + u * 1024 * FNW);
       return;
     }
     // the last tile of a sequence / a partial slab: rows and columns past the end come from the last valid one
@@ -513,8 +538,7 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
       const int a = lrow >> 5, hb = (lrow >> 4) & 1, gg = (lrow >> 2) & 3, t = lrow & 3;
       const int key = min(k0 + 32 * a + 8 * gg + 4 * hb + t, A.L - 1);
       const int kc = (pp ^ (KPC == 16 ? (lrow & 15) : ((lrow >> 1) & 7))) * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kb_ + (int64_t)key * rs + kc),
-                                       (__attribute__((address_space(3))) void*)(lk + u * 1024 * FNW), 16, 0, 0);
+      lds_dma16(kb_ + (int64_t)key * rs + kc, lk + u * 1024 * FNW);
     }
 #pragma unroll
     for (int u = 0; u < NVL; ++u) {
@@ -523,8 +547,7 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
       const int key = min(k0 + r, A.L - 1);
       const int pc = ((((pp >> 1) ^ ((r & 3) + 4 * ((r >> 3) & 1))) << 1) | (pp & 1));
       const int col = min(pc * 8, A.H2 - d0 - 8);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vb + (int64_t)key * vs + col),
-                                       (__attribute__((address_space(3))) void*)(lv + u * 1024 * FNW), 16, 0, 0);
+      lds_dma16(vb + (int64_t)key * vs + col, lv + u * 1024 * FNW);
     }
   };
 
@@ -546,142 +569,152 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
   for (int a = 0; a < 2; ++a)
 #pragma unroll
     for (int j = 0; j < FQB; ++j) Pb[a][j] = make_uint4(0, 0, 0, 0);
-  if (nkt > 0) issue_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): this wave's pieces have landed
-  __syncthreads();
   MEGA_ATR_BEGIN();
-  for (int kt = 0; kt < nkt; ++kt) {
-    if (kt + 1 < nkt) issue_tile(kt + 1, (kt + 1) & 1);  // lands under this tile's products
+  // ---- the two phases of a key tile.  scores: S^T = k q^T, mask, running maximum and sum; leaves the probabilities
+  // (Pb) and the factor y has to be rescaled by (pend).  second: y^T += v^T P^T.
+  auto scores = [&](int kt) {
     const int k0 = kt * FBN;
-    const bool valid = k0 < klim_w;                      // wave-uniform: some key of the tile is visible
-    const char* lk = lds + (kt & 1) * BUF;
-    const char* lv = lk + KB;
-    MEGA_ATR(5);
+    if (k0 >= klim_w) return;                            // wave-uniform: no key of the tile is visible
+    const char* lk = lds + (kt & 1) * KB;
+    f32x4 S[4][FQB];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int j = 0; j < FQB; ++j) S[kb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     {
-      if (valid) {
-      f32x4 S[4][FQB];
+      // fragment f = 4 s + kb: row 16 kb + n, piece 4 s + g at position (4 s + g) ^ n; two fragments ahead
+      const char* kfrag = lk + n * KROW;
+      const int ksw = KPC == 16 ? n : ((n >> 1) & 7);
+      auto kaddr = [&](int f) { return kfrag + (f & 3) * 16 * KROW + (((f >> 2) * 4 + g) ^ ksw) * 16; };
+      // the order below is kept as written (the fragment reads run DK fragments ahead of the products that
+      // use them, so that the LDS latency is covered): no scheduling across the markers
+      constexpr int DK = 4;
+      uint4 fk[DK + 1];
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
+      for (int f = 0; f < DK; ++f) fk[f] = *(const uint4*)kaddr(f);
 #pragma unroll
-        for (int j = 0; j < FQB; ++j) S[kb][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      {
-        // fragment f = 4 s + kb: row 16 kb + n, piece 4 s + g at position (4 s + g) ^ n; two fragments ahead
-        const char* kfrag = lk + n * KROW;
-        const int ksw = KPC == 16 ? n : ((n >> 1) & 7);
-        auto kaddr = [&](int f) { return kfrag + (f & 3) * 16 * KROW + (((f >> 2) * 4 + g) ^ ksw) * 16; };
-        // the order below is kept as written (the fragment reads run DK fragments ahead of the products that
-        // use them, so that the LDS latency is covered): no scheduling across the markers
-        constexpr int DK = 4;
-        uint4 fk[DK + 1];
+      for (int f = 0; f < 4 * KS; ++f) {
+        const int s = f >> 2, kb = f & 3;
+        if (f + DK < 4 * KS) fk[(f + DK) % (DK + 1)] = *(const uint4*)kaddr(f + DK);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int f = 0; f < DK; ++f) fk[f] = *(const uint4*)kaddr(f);
-#pragma unroll
-        for (int f = 0; f < 4 * KS; ++f) {
-          const int s = f >> 2, kb = f & 3;
-          if (f + DK < 4 * KS) fk[(f + DK) % (DK + 1)] = *(const uint4*)kaddr(f + DK);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int j = 0; j < FQB; ++j) S[kb][j] = mfma16<T>(fk[f % (DK + 1)], Qr[j][s], S[kb][j]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+        for (int j = 0; j < FQB; ++j) S[kb][j] = mfma16<T>(fk[f % (DK + 1)], Qr[j][s], S[kb][j]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      MEGA_ATR(0);
-      // mask, running maximum and sum; key of S[kb][j][u]: k0 + 32 (kb >> 1) + 8 g + 4 (kb & 1) + u
-      const bool edge = (A.causal && k0 + FBN - 1 > qw0) || k0 + FBN > A.L;
+    }
+    MEGA_ATR(0);
+    // mask, running maximum and sum; key of S[kb][j][u]: k0 + 32 (kb >> 1) + 8 g + 4 (kb & 1) + u
+    const bool edge = (A.causal && k0 + FBN - 1 > qw0) || k0 + FBN > A.L;
 #pragma unroll
-      for (int j = 0; j < FQB; ++j) {
-        const int qi = qw0 + 16 * j + n;
-        const int lim = A.causal ? min(qi, A.L - 1) : A.L - 1;      // last visible key
-        if (edge) {
-          // only the tiles on the diagonal and the last one carry this code (kept a branch: the empty asm
-          // statement stops the compiler from turning it into selects executed on every tile)
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              const int key = k0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + u;
-              S[kb][j][u] = key <= lim ? S[kb][j][u] : -INFINITY;
-            }
-        }
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int u = 0; u < 4; ++u) tmax = fmaxf(tmax, S[kb][j][u]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-        tmax *= A.scale_log2;                                        // scale > 0: the maximum commutes with it
-        // the running maximum moves only when a tile exceeds it by more than 2^8: probabilities up to 256
-        // are as exact as those below 1, and y is rescaled on few tiles
-        const float mnew = tmax > mrun[j] + 8.0f ? tmax : mrun[j];
-        const float muse = mnew == -INFINITY ? 0.f : mnew;
-        const float corr = __builtin_amdgcn_exp2f(mrun[j] - muse);
-        mrun[j] = mnew;
-        float psum = 0.f;
+    for (int j = 0; j < FQB; ++j) {
+      const int qi = qw0 + 16 * j + n;
+      const int lim = A.causal ? min(qi, A.L - 1) : A.L - 1;      // last visible key
+      if (edge) {
+        // only the tiles on the diagonal and the last one carry this code (kept a branch: the empty asm
+        // statement stops the compiler from turning it into selects executed on every tile)
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
-            const float pv = __builtin_amdgcn_exp2f(fmaf(S[kb][j][u], A.scale_log2, -muse));
-            S[kb][j][u] = pv;
-            psum += pv;
+            const int key = k0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + u;
+            S[kb][j][u] = key <= lim ? S[kb][j][u] : -INFINITY;
           }
-        lrun[j] = lrun[j] * corr + psum;
-        pend[j] = corr;                                              // y is rescaled where it is next touched
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-          Pb[a][j] = make_uint4(pack2<T>(S[2 * a][j][0], S[2 * a][j][1]), pack2<T>(S[2 * a][j][2], S[2 * a][j][3]),
-                                pack2<T>(S[2 * a + 1][j][0], S[2 * a + 1][j][1]),
-                                pack2<T>(S[2 * a + 1][j][2], S[2 * a + 1][j][3]));
       }
-      MEGA_ATR(1);
-      }
-      if (valid) {
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int j = 0; j < FQB; ++j) {
-        if (__any(pend[j] != 1.0f)) {
+      for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-          for (int i = 0; i < FBD / 16; ++i)
+        for (int u = 0; u < 4; ++u) tmax = fmaxf(tmax, S[kb][j][u]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      tmax *= A.scale_log2;                                        // scale > 0: the maximum commutes with it
+      // the running maximum moves only when a tile exceeds it by more than 2^8: probabilities up to 256
+      // are as exact as those below 1, and y is rescaled on few tiles
+      const float mnew = tmax > mrun[j] + 8.0f ? tmax : mrun[j];
+      const float muse = mnew == -INFINITY ? 0.f : mnew;
+      const float corr = __builtin_amdgcn_exp2f(mrun[j] - muse);
+      mrun[j] = mnew;
+      float psum = 0.f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) O[i][j][u] *= pend[j];
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float pv = __builtin_amdgcn_exp2f(fmaf(S[kb][j][u], A.scale_log2, -muse));
+          S[kb][j][u] = pv;
+          psum += pv;
         }
-      }
-      {
-        // fragment f = 2 i + a: the A operand v^T[d = 16 i + n][keys 32 a + 8 g ..+7] out of the key-major tile by two
-        // transposing reads (ds_read_b64_tr_b16: lane s of a group of 16 supplies 8 bytes = 4 columns of one row;
-        // lane l receives element l & 3 of the lanes (l >> 2) + 4 x, x = 0..3).  Source lane s points at row
-        // 32 a + 8 g + 4 hh + (s >> 2), columns 16 i + 4 (s & 3): the result is 4 consecutive keys of column 16 i + n.
-        const int sr = n >> 2, sc = n & 3;
-        const char* vsrc = lv + (8 * g + sr) * (FBD * 2) + sc * 8;
-        const int vsw = sr + 4 * (g & 1);
-        typedef __attribute__((ext_vector_type(4))) short s4v;
-        auto vread = [&](int f) {
-          const int i = f >> 1, a = f & 1;
-          const char* q0 = vsrc + a * 32 * (FBD * 2) + ((i ^ vsw) * 32);
-          const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0));
-          const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0 + 4 * (FBD * 2)));
-          const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
-          return make_uint4(l2.x, l2.y, h2.x, h2.y);
-        };
-        constexpr int NF = 2 * (FBD / 16);
-        constexpr int DV = 6;                            // fragments in flight ahead of the products
-        uint4 fv[DV + 1];
+      lrun[j] = lrun[j] * corr + psum;
+      pend[j] = corr;                                              // y is rescaled where it is next touched
 #pragma unroll
-        for (int f = 0; f < DV; ++f) fv[f] = vread(f);
+      for (int a = 0; a < 2; ++a)
+        Pb[a][j] = make_uint4(pack2<T>(S[2 * a][j][0], S[2 * a][j][1]), pack2<T>(S[2 * a][j][2], S[2 * a][j][3]),
+                              pack2<T>(S[2 * a + 1][j][0], S[2 * a + 1][j][1]),
+                              pack2<T>(S[2 * a + 1][j][2], S[2 * a + 1][j][3]));
+    }
+    MEGA_ATR(1);
+  };
+  auto second = [&](int kt) {
+    if (kt * FBN >= klim_w) return;
+    int vbo = (kt & 1) * VB;
+    asm volatile("" : "+s"(vbo));                        // per step: keeps the fragment addresses out of loop-invariant registers
+    const char* lv = lds + 2 * KB + vbo;
 #pragma unroll
-        for (int f = 0; f < NF; ++f) {
-          const int i = f >> 1, a = f & 1;
-          if (f + DV < NF) fv[(f + DV) % (DV + 1)] = vread(f + DV);
-          __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < FQB; ++j) {
+      if (__any(pend[j] != 1.0f)) {
 #pragma unroll
-          for (int j = 0; j < FQB; ++j) O[i][j] = mfma16<T>(fv[f % (DV + 1)], Pb[a][j], O[i][j]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      MEGA_ATR(2);
+        for (int i = 0; i < FBD / 16; ++i)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) O[i][j][u] *= pend[j];
       }
     }
+    // fragment f = 2 i + a: the A operand v^T[d = 16 i + n][keys 32 a + 8 g ..+7] out of the key-major tile by two
+    // transposing reads (ds_read_b64_tr_b16: lane s of a group of 16 supplies 8 bytes = 4 columns of one row;
+    // lane l receives element l & 3 of the lanes (l >> 2) + 4 x, x = 0..3).  Source lane s points at row
+    // 32 a + 8 g + 4 hh + (s >> 2), columns 16 i + 4 (s & 3): the result is 4 consecutive keys of column 16 i + n.
+    const int sr = n >> 2, sc = n & 3;
+    const char* vsrc = lv + (8 * g + sr) * (FBD * 2) + sc * 8;
+    const int vsw = sr + 4 * (g & 1);
+    // the swizzle touches the low three bits of the column block only: eight per-lane addresses, the rest of a
+    // fragment's position is an immediate offset
+    const char* va[8];
+#pragma unroll
+    for (int il = 0; il < 8; ++il) va[il] = vsrc + ((il ^ vsw) * 32);
+    typedef __attribute__((ext_vector_type(4))) short s4v;
+    auto vread = [&](int f) {
+      const int i = f >> 1, a = f & 1;
+      const char* q0 = va[i & 7] + a * 32 * (FBD * 2) + (i >> 3) * 256;
+      const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0));
+      const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0 + 4 * (FBD * 2)));
+      const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+      return make_uint4(l2.x, l2.y, h2.x, h2.y);
+    };
+    constexpr int NF = 2 * (FBD / 16);
+    constexpr int DV = 6;                            // fragments in flight ahead of the products
+    uint4 fv[DV + 1];
+#pragma unroll
+    for (int f = 0; f < DV; ++f) fv[f] = vread(f);
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      const int i = f >> 1, a = f & 1;
+      if (f + DV < NF) fv[(f + DV) % (DV + 1)] = vread(f + DV);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < FQB; ++j) O[i][j] = mfma16<T>(fv[f % (DV + 1)], Pb[a][j], O[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    MEGA_ATR(2);
+  };
+
+  if (nkt > 0) issue_tile(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): this wave's pieces have landed
+  __syncthreads();
+  MEGA_ATR_MARK();
+  for (int kt = 0; kt < nkt; ++kt) {
+    if (kt + 1 < nkt) issue_tile(kt + 1);                // lands under this tile's products
+    MEGA_ATR(5);
+    scores(kt);
+    second(kt);
     __builtin_amdgcn_s_waitcnt(0x0F70);                  // vmcnt(0): the next tile's pieces of this wave have landed
     MEGA_ATR(3);
     __syncthreads();
@@ -727,21 +760,22 @@ bool flash_covers(const void* v, const void* y, int64_t L, int64_t H1, int64_t H
 template <typename T>
 void launch_flash(const void* q, const void* k, const void* v, void* y, int64_t B, int64_t L, int64_t Nh,
                   int64_t H1, int64_t H2, float scale, int causal, hipStream_t s) {
+  constexpr int fqb = 2, fbd = 256, fbm = 16 * FNW * fqb;
   FlashArgs F;
   F.q = q; F.k = k; F.v = v; F.y = y;
   F.L = (int)L; F.Nh = (int)Nh; F.H1 = (int)H1; F.H2 = (int)H2;
   F.scale_log2 = scale * 1.4426950408889634f;
   F.causal = causal ? 1 : 0;
-  F.mt = (int)ceil_div(L, FBM);
-  F.ns = (int)ceil_div(H2, FBD);
+  F.mt = (int)ceil_div(L, fbm);
+  F.ns = (int)ceil_div(H2, fbd);
   const int64_t BN_ = B * Nh;
   F.xcd = BN_ % 8 == 0 ? 1 : 0;
   const dim3 grid((unsigned)(BN_ * F.mt * F.ns));
   const int ks = (int)(H1 / 32);
-  const size_t smem = 2 * ((size_t)FBN * H1 * 2 + (size_t)FBD * FBN * 2);
+  const size_t smem = 2 * ((size_t)FBN * H1 * 2 + (size_t)fbd * FBN * 2);
 #define MEGA_FLASH(KS_)                                                                                       \
   {                                                                                                           \
-    auto kern = flash_fwd_kernel<T, KS_, FBM / FNW / 16>;                                                                     \
+    auto kern = flash_fwd_kernel<T, KS_, fqb, fbd>;                                                           \
     static bool attr_set = false;                                                                             \
     if (!attr_set) {                                                                                          \
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);    \

@@ -112,7 +112,9 @@ def test_attention(dtype, B, L, Nh, H1, H2, causal):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,L,Nh,H1,H2", [(2, 300, 2, 64, 256), (1, 1000, 1, 128, 512), (1, 129, 3, 32, 256),
-                                          (1, 64, 1, 96, 256), (1, 2048, 2, 128, 320), (3, 520, 1, 64, 72)])
+                                          (1, 64, 1, 96, 256), (1, 2048, 2, 128, 320), (3, 520, 1, 64, 72),
+                                          (2, 700, 2, 128, 1024), (1, 300, 1, 64, 520), (1, 1100, 3, 128, 768),
+                                          (1, 2048, 1, 64, 1024)])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_no_weights(dtype, B, L, Nh, H1, H2, causal):
     """No weights requested (the inference call of the layer), at sizes where the matrix-core GEMMs
