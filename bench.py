@@ -534,6 +534,40 @@ def bench_attention(args):
     }))
 
 
+def bench_attention_bwd(args):
+    """The backward of configs[4]'s attention (q, k, v gradients from y_grad and the forward's weights) through
+    mega_attention_bwd: four products on the library's matrix-core kernel, the softmax backward and the transposed
+    copies the products need.  Flops for the causal half of the four products: twice the forward's."""
+    import torch
+
+    import fairseq_apollo_amd as M
+
+    Bc, C, Nh, H1, H2 = 4, 2048, 4, 128, 1024
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(1239)
+    mk = lambda *sh: torch.randn(*sh, generator=gen).to(torch.bfloat16).to(dev)
+    q, k, v, dy = mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H2), mk(Bc, C, Nh, H2)
+    scale = 1.0 / H1 ** 0.5
+    with torch.no_grad():
+        _, w = M.ops.attention_fwd(q, k, v, scale, 0.0, True, need_weights=True)
+        run = lambda i: M.ops.attention_bwd(dy, q, k, v, w, scale, True)
+        for _ in range(args.warmup):
+            run(0)
+        dev_ms, wall_ms, _ = best_region(run, args.steps)
+    ms = max(wall_ms, dev_ms)
+    flops_causal = 2 * Bc * Nh * (C * (C + 1)) * (H1 + H2)
+    tf = flops_causal / (dev_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "attention backward chunk tokens/sec @4x2048, 4 heads, H1=128, H2=1024", "value": Bc * C / (ms * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[4] attention backward: q, k, v gradients per 2048-token chunk and head"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel x 4 + softmax_bwd_f32_kernel + transpose_v_kernel x 5",
+                     "achieved": tf, "peak": 2500.0, "unit": "TFLOP/s", "frac": tf / 2500.0, "traffic": None,
+                     "algorithmic_flops_per_call": flops_causal, "avg_ms": dev_ms},
+    }))
+
+
 def bench_layer(args):
     """configs[4]: one Mega2 layer forward (TimestepNorm -> CEMA -> chunked causal attention with
     rotary -> gates, then TimestepNorm -> SwiGLU), L = 8192, D = 2048, S = 512, E = 4096, chunk 2048,
@@ -593,7 +627,7 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
-    ap.add_argument("--workload", choices=["block", "decode", "attention", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature", "long_conv"],
+    ap.add_argument("--workload", choices=["block", "decode", "attention", "attention_bwd", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature", "long_conv"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "
                          "the decode step of configs[3] / the chunk attention / the whole layer of configs[4]; "
@@ -615,6 +649,8 @@ def main():
         return bench_long_conv(args)
     if args.workload == "block_bwd":
         return bench_block_bwd(args)
+    if args.workload == "attention_bwd":
+        return bench_attention_bwd(args)
     if args.workload == "attention":
         return bench_attention(args)
     if args.workload in ("layer", "layer_train"):

@@ -16,6 +16,13 @@ size_t attention_mfma_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t N
 int attention_mfma_run(const void* q, const void* k, const void* v, void* y, void* w, int dtype, int64_t B, int64_t L,
                        int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, float dropout, uint64_t seed,
                        void* ws, hipStream_t s);
+bool attention_mfma_bwd_covers(int dtype, const void* dy, const void* q, const void* k, const void* v, const void* dq,
+                               const void* dk, const void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                               int64_t H2);
+size_t attention_mfma_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2);
+int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq,
+                           void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
+                           float scale, int causal, void* ws, hipStream_t s);
 
 namespace {
 
@@ -282,4 +289,31 @@ extern "C" int mega_attention_softmax_bwd(const void* y_grad, const void* y, voi
     case MEGA_BF16: return launch_softmax_bwd<bf16_t>(y_grad, y, x_grad, rows, outer, inner, causal, scale, s);
     default: return launch_softmax_bwd<f16_t>(y_grad, y, x_grad, rows, outer, inner, causal, scale, s);
   }
+}
+
+extern "C" size_t mega_attention_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                                                     int64_t H2) {
+  if (B <= 0 || L <= 0 || Nh <= 0 || H1 <= 0 || H2 <= 0 || dtype == MEGA_F32 || H1 % 8 != 0 || H2 % 8 != 0) return 0;
+  if (B * Nh > 65535 || L >= (int64_t)1 << 15) return 0;
+  return attention_mfma_bwd_workspace_bytes(dtype, B, L, Nh, H1, H2);
+}
+
+extern "C" int mega_attention_bwd(const void* y_grad, const void* q, const void* k, const void* v, const void* w,
+                                  void* q_grad, void* k_grad, void* v_grad, int dtype, int64_t B, int64_t L,
+                                  int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_BF16 || dtype == MEGA_F16, dtype == MEGA_F32 ? MEGA_ERR_UNSUPPORTED : MEGA_ERR_ARG,
+               "attention_bwd: 16-bit activations only (dtype %d)", dtype);
+  MEGA_REQUIRE(B >= 0 && L >= 0 && Nh > 0 && H1 > 0 && H2 > 0, MEGA_ERR_ARG, "attention_bwd: bad shape");
+  if (B == 0 || L == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && q && k && v && w && q_grad && k_grad && v_grad, MEGA_ERR_ARG,
+               "attention_bwd: null pointer argument");
+  MEGA_REQUIRE(attention_mfma_bwd_covers(dtype, y_grad, q, k, v, q_grad, k_grad, v_grad, B, L, Nh, H1, H2),
+               MEGA_ERR_UNSUPPORTED,
+               "attention_bwd: needs H1 %% 8 == 0, H2 %% 8 == 0, 16-byte aligned tensors, B * Nh <= 65535, L < 32768");
+  const size_t need = attention_mfma_bwd_workspace_bytes(dtype, B, L, Nh, H1, H2);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 256) == 0, MEGA_ERR_WORKSPACE,
+               "attention_bwd: workspace of %zu bytes (256-byte aligned) needed", need);
+  return attention_mfma_bwd_run(y_grad, q, k, v, w, q_grad, k_grad, v_grad, dtype, B, L, Nh, H1, H2, scale, causal,
+                                workspace, (hipStream_t)stream);
 }

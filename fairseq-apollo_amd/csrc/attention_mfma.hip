@@ -8,6 +8,13 @@
 //   y = P v                the same NT GEMM against v^T (v is transposed once through LDS); causal:
 //                          the reduction stops at the diagonal
 //
+// Backward (fairseq/csrc/ops/attention_kernel.cu:133-255), with the forward's weights w:
+//   dW = dy v^T            NT GEMM, fp32 out; causal: tiles above the diagonal are skipped
+//   dS = scale w (dW - rowsum(w dW))       one wave per row, zeros behind the causal limit
+//   dv = w^T dy, dk = dS^T q               NT GEMMs against transposed copies (w^T, dS^T, dy^T, q^T); causal: the
+//                                          reduction starts at the diagonal
+//   dq = dS k                              NT GEMM against k^T; causal: the reduction stops at the diagonal
+//
 // The GEMM: (64 WM) x (64 WN) output tile per workgroup of WM x WN waves (64 x 64 each as 4 x 4 MFMA
 // blocks): 128 x 128 for the scores, 256 x 256 for the second product, which carries the flops.
 // K step 64, operands staged through LDS with a 144-byte row pitch (conflict-free 16-byte reads),
@@ -35,8 +42,9 @@ struct GemmArgs {
   int nin;
   int M, N, K;
   float alpha;
-  int causal;         // 1: S = q k^T (skip tiles with n0 > m0 + BM - 1); 2: y = P v (K stops at m0 + BM)
-  int kshift;         // causal offset: row m sees columns <= m + kshift
+  int causal;         // 1: S = q k^T (skip tiles with n0 > m0 + BM - 1); 2: y = P v (K stops at m0 + BM);
+                      // 3: y = P^T v (row m of the product is column m of P: K starts at m0)
+  int kshift;         // causal offset: row m (of P) sees columns <= m + kshift
   // xcd != 0: one-dimensional grid; every tile of a batch entry runs on one XCD (workgroup ids go
   // round-robin over the 8 XCDs), so both operands of a batch entry are fetched into one L2 only;
   // the long (late) row tiles of a causal product come first
@@ -88,6 +96,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   if (G.causal == 2) Kend = min(G.K, m0 + TM + G.kshift);
   if (Kend < 0) Kend = 0;
   const int nk = (Kend + BK - 1) / BK;
+  const int kt0 = G.causal == 3 ? max(0, m0 - G.kshift) / BK : 0;      // first K step that can hold a non-zero
 
   // global -> register staging
   const int lrow = tid / KP, lcol = (tid % KP) * 8;              // rows 0 .. NT/KP - 1 (+ h * NT/KP)
@@ -123,13 +132,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   const int wm = (wave / WN) * 64, wn = (wave % WN) * 64;
   const int fr = lane & 15, fk = (lane >> 4) * 16;                // fragment row, byte offset of the k block
 
-  if (nk > 0) {
-    gload(0);
+  if (nk > kt0) {
+    gload(kt0);
     lstore(0);
   }
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
+  for (int kt = kt0; kt < nk; ++kt) {
+    const int buf = (kt - kt0) & 1;
     if (kt + 1 < nk) gload(kt + 1);
     const char* la = lds + buf * (TM + TN) * PITCH;
     const char* lb = la + TM * PITCH;
@@ -365,6 +374,52 @@ __global__ __launch_bounds__(256) void dropkey_f32_kernel(float* __restrict__ s,
     if (hash_uniform(seed, e0 + j) < dropout) sp[j] = -INFINITY;
 }
 
+// Softmax backward on the fp32 weight gradient of the first backward product
+// (fairseq/csrc/ops/attention_kernel.cu:195-203, softmax.cuh AttentionSoftmaxBwdKernel):
+//   ds[r, c] = scale * w[r, c] * (dw[r, c] - sum_c' w[r, c'] dw[r, c']),
+// w rows of `wpitch` elements, dw and ds rows of `pitch` (a multiple of 8, >= inner).  One wave per row, four rows
+// per workgroup.  Columns behind the causal limit are not read (the product skips tiles above the diagonal and leaves
+// them unwritten) and every column of ds from the limit to the end of the pitch is written as zero: the products
+// that follow read whole rows and whole columns of ds.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void softmax_bwd_f32_kernel(const float* __restrict__ dw, const T* __restrict__ w,
+                                                              T* __restrict__ ds, int outer, int inner, int64_t wpitch,
+                                                              int64_t pitch, int causal, float scale, int64_t nrows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
+  const int r = (int)(row % outer);
+  int limit = causal ? inner - outer + r + 1 : inner;
+  if (limit < 0) limit = 0;
+  if (limit > inner) limit = inner;
+  const float* dwr = dw + row * pitch;
+  const T* wr = w + row * wpitch;
+  T* dsr = ds + row * pitch;
+  float dot = 0.f;
+  for (int c = lane * VEC; c < limit; c += 64 * VEC) {
+    const Vec<float, VEC> a = *(const Vec<float, VEC>*)(dwr + c);
+    const Vec<T, VEC> b = *(const Vec<T, VEC>*)(wr + c);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+      if (c + e < limit) dot = fmaf(a.v[e], to_float(b.v[e]), dot);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
+  for (int c = lane * VEC; c < (int)pitch; c += 64 * VEC) {
+    Vec<T, VEC> o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.v[e] = from_float<T>(0.f);
+    if (c < limit) {
+      const Vec<float, VEC> a = *(const Vec<float, VEC>*)(dwr + c);
+      const Vec<T, VEC> b = *(const Vec<T, VEC>*)(wr + c);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if (c + e < limit) o.v[e] = from_float<T>(scale * to_float(b.v[e]) * (a.v[e] - dot));
+    }
+    *(Vec<T, VEC>*)(dsr + c) = o;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // One kernel for the whole op when the weights are not wanted: scores, causal softmax and the
 // second product per tile of 64 keys, with running row maxima and sums (no L x L array in memory).
@@ -418,14 +473,30 @@ __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
 // wave wait for the loads it has just issued (vmcnt(0)) before its first read of the current tile.  Here the
 // loads are invisible to that bookkeeping; the kernel waits for them itself (vmcnt(0), then the workgroup barrier)
 // before anybody reads the buffer they fill.
+// M0 (the LDS base of such a load) is put back afterwards: the compiler does not honour a clobber of it.
 __device__ __forceinline__ void lds_dma16(const void* base /* wave-uniform */, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(lane_off), "s"(base), "s"(lds_base)
-               : "memory", "m0");
+  uint32_t keep;
+  asm volatile(
+      "s_mov_b32 %[keep], m0\n\t"
+      "s_mov_b32 m0, %[lds]\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %[off], %[base]\n\t"
+      "s_mov_b32 m0, %[keep]"
+      : [keep] "=&s"(keep)
+      : [off] "v"(lane_off), [base] "s"(base), [lds] "s"(lds_base)
+      : "memory");
 }
 __device__ __forceinline__ void lds_dma16(const void* addr /* per lane */, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(addr), "s"(lds_base) : "memory", "m0");
+  uint32_t keep;
+  asm volatile(
+      "s_mov_b32 %[keep], m0\n\t"
+      "s_mov_b32 m0, %[lds]\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %[addr], off\n\t"
+      "s_mov_b32 m0, %[keep]"
+      : [keep] "=&s"(keep)
+      : [addr] "v"(addr), [lds] "s"(lds_base)
+      : "memory");
 }
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
@@ -839,6 +910,103 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   return MEGA_OK;
 }
 
+// workspace of the backward, in this order (each part 256-byte aligned)
+struct BwdWs {
+  size_t dw, ds, wt, dst, dyt, qt, kt, total;
+};
+BwdWs bwd_workspace(size_t es, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2) {
+  const int64_t Lp = (L + 7) / 8 * 8, BN_ = B * Nh;
+  BwdWs W;
+  size_t o = 0;
+  auto take = [&](size_t bytes) {
+    const size_t at = o;
+    o += align_up(bytes, 256);
+    return at;
+  };
+  W.dw = take((size_t)BN_ * L * Lp * 4);       // fp32 [BN][L][Lp]
+  W.ds = take((size_t)BN_ * L * Lp * es);      // [BN][L][Lp]
+  W.wt = take((size_t)BN_ * L * Lp * es);      // w^T [BN][L][Lp]
+  W.dst = take((size_t)BN_ * Lp * Lp * es);    // dS^T [BN][Lp][Lp] (rows past L are zero)
+  W.dyt = take((size_t)BN_ * H2 * Lp * es);    // dy^T [BN][H2][Lp]
+  W.qt = take((size_t)BN_ * H1 * Lp * es);     // q^T [BN][H1][Lp]
+  W.kt = take((size_t)BN_ * H1 * Lp * es);     // k^T
+  W.total = o;
+  return W;
+}
+
+template <typename T>
+void launch_transpose(const T* src, T* dst, int64_t batches, int64_t rows, int64_t nin, int64_t cols, int64_t Lp,
+                      hipStream_t s) {
+  // src [batches / nin][rows][nin][cols] -> dst [batches][cols][Lp]
+  const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(cols, 64), (unsigned)batches);
+  const int vec = (cols % 8 == 0 && ((uintptr_t)src % 16) == 0) ? 1 : 0;
+  hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, src, dst, (int)rows, (int)nin, (int)cols, (int)Lp,
+                     vec);
+}
+
+template <typename T>
+int run_attention_bwd(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq, void* dk,
+                      void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale, int causal,
+                      char* ws, hipStream_t s) {
+  const int64_t Lp = (L + 7) / 8 * 8, BN_ = B * Nh;
+  const BwdWs W = bwd_workspace(sizeof(T), B, L, Nh, H1, H2);
+  float* dW = (float*)(ws + W.dw);
+  T* dS = (T*)(ws + W.ds);
+  T* Wt = (T*)(ws + W.wt);
+  T* dSt = (T*)(ws + W.dst);
+  T* dYt = (T*)(ws + W.dyt);
+  T* Qt = (T*)(ws + W.qt);
+  T* Kt = (T*)(ws + W.kt);
+  const bool xcd = BN_ % 8 == 0;
+  // transposed copies of the operands that enter a product through their columns
+  launch_transpose<T>((const T*)dy, dYt, BN_, L, Nh, H2, Lp, s);
+  launch_transpose<T>((const T*)q, Qt, BN_, L, Nh, H1, Lp, s);
+  launch_transpose<T>((const T*)k, Kt, BN_, L, Nh, H1, Lp, s);
+  launch_transpose<T>((const T*)w, Wt, BN_, L, 1, L, Lp, s);
+  GemmArgs G;
+  G.nin = (int)Nh; G.kshift = 0;
+  // dW[b,n] = dy[b,:,n,:] v[b,:,n,:]^T (attention_kernel.cu:176-193)
+  G.A = dy; G.Bm = v; G.C = dW;
+  G.lda = Nh * H2; G.ldb = Nh * H2; G.ldc = Lp;
+  G.sa = L * Nh * H2; G.sai = H2; G.sb = L * Nh * H2; G.sbi = H2; G.sc = Nh * L * Lp; G.sci = L * Lp;
+  G.M = (int)L; G.N = (int)L; G.K = (int)H2; G.alpha = 1.0f; G.causal = causal ? 1 : 0;
+  launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  // dS = scale w (dW - rowsum(w dW)) (attention_kernel.cu:195-203)
+  {
+    const int64_t nrows = BN_ * L;
+    const dim3 grid((unsigned)ceil_div(nrows, 4));
+    const bool vec = L % 4 == 0 && ((uintptr_t)w % 8) == 0;
+    if (vec)
+      hipLaunchKernelGGL((softmax_bwd_f32_kernel<T, 4>), grid, dim3(256), 0, s, dW, (const T*)w, dS, (int)L, (int)L, L, Lp,
+                         causal, scale, nrows);
+    else
+      hipLaunchKernelGGL((softmax_bwd_f32_kernel<T, 1>), grid, dim3(256), 0, s, dW, (const T*)w, dS, (int)L, (int)L, L, Lp,
+                         causal, scale, nrows);
+  }
+  // dS [BN][L][Lp] -> dS^T [BN][Lp][Lp]
+  launch_transpose<T>(dS, dSt, BN_, L, 1, Lp, Lp, s);
+  // dv[b,:,n,:] = w[b,n]^T dy[b,:,n,:] (attention_kernel.cu:155-174): rows of w^T against rows of dy^T
+  G.A = Wt; G.Bm = dYt; G.C = dv;
+  G.lda = Lp; G.ldb = Lp; G.ldc = Nh * H2;
+  G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = Nh * H2 * Lp; G.sbi = H2 * Lp; G.sc = L * Nh * H2; G.sci = H2;
+  G.M = (int)L; G.N = (int)H2; G.K = (int)Lp; G.alpha = 1.0f; G.causal = causal ? 3 : 0;
+  if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4>(G, L, H2, BN_, xcd, s);
+  else launch_gemm<T, T, 2, 2>(G, L, H2, BN_, xcd, s);
+  // dq[b,:,n,:] = dS[b,n] k[b,:,n,:] (attention_kernel.cu:205-222)
+  G.A = dS; G.Bm = Kt; G.C = dq;
+  G.lda = Lp; G.ldb = Lp; G.ldc = Nh * H1;
+  G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = Nh * H1 * Lp; G.sbi = H1 * Lp; G.sc = L * Nh * H1; G.sci = H1;
+  G.M = (int)L; G.N = (int)H1; G.K = (int)Lp; G.causal = causal ? 2 : 0;
+  launch_gemm<T, T, 2, 2>(G, L, H1, BN_, xcd, s);
+  // dk[b,:,n,:] = dS[b,n]^T q[b,:,n,:] (attention_kernel.cu:224-241)
+  G.A = dSt; G.Bm = Qt;  G.C = dk;
+  G.sa = Nh * Lp * Lp; G.sai = Lp * Lp;
+  G.causal = causal ? 3 : 0;
+  launch_gemm<T, T, 2, 2>(G, L, H1, BN_, xcd, s);
+  MEGA_CHECK_LAUNCH("attention_bwd");
+  return MEGA_OK;
+}
+
 }  // namespace
 
 bool attention_mfma_covers(int dtype, const void* q, const void* k, const void* v, int64_t B, int64_t L, int64_t Nh,
@@ -864,6 +1032,30 @@ int attention_mfma_run(const void* q, const void* k, const void* v, void* y, voi
   if (dtype == MEGA_BF16)
     return run_attention<bf16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, dropout, seed, (char*)ws, s);
   return run_attention<f16_t>(q, k, v, y, w, B, L, Nh, H1, H2, scale, causal, dropout, seed, (char*)ws, s);
+}
+
+bool attention_mfma_bwd_covers(int dtype, const void* dy, const void* q, const void* k, const void* v, const void* dq,
+                               const void* dk, const void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                               int64_t H2) {
+  if (dtype == MEGA_F32) return false;
+  if (H1 % 8 != 0 || H2 % 8 != 0) return false;                // 16-byte operand and result rows
+  const uintptr_t all = (uintptr_t)dy | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dq | (uintptr_t)dk |
+                        (uintptr_t)dv;
+  if (all % 16) return false;
+  if (B * Nh > 65535 || L >= (int64_t)1 << 15) return false;   // L x L x batch index arithmetic in the transposes
+  return true;
+}
+
+size_t attention_mfma_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2) {
+  return bwd_workspace(dtype == MEGA_F32 ? 4 : 2, B, L, Nh, H1, H2).total;
+}
+
+int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq,
+                           void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
+                           float scale, int causal, void* ws, hipStream_t s) {
+  if (dtype == MEGA_BF16)
+    return run_attention_bwd<bf16_t>(dy, q, k, v, w, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
+  return run_attention_bwd<f16_t>(dy, q, k, v, w, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
 }
 
 }  // namespace mega

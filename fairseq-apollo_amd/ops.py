@@ -512,13 +512,32 @@ def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask
 
 def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool):
     """-> (q_grad, k_grad, v_grad).  Reference: attention_bwd, fairseq/csrc/ops/attention_kernel.cu:133-255:
-    four batched library GEMMs around the softmax backward, which runs in place on the weight
-    gradient; w [B, Nh, L, L] are the forward's weights."""
+    four batched products around the softmax backward; w [B, Nh, L, L] are the forward's weights.
+    16-bit activations with head sizes that are multiples of 8 run through the library's own matrix-core
+    products (mega_attention_bwd: head-strided operands read in place, the causal half of every product
+    skipped); fp32 and odd head sizes through four batched library GEMMs around mega_attention_softmax_bwd."""
     dev = _need_gpu(y_grad, q, k, v, w)
     if q.dim() != 4 or w is None or w.dim() != 4:
         raise RuntimeError("attention_bwd: q, k, v must be [B,L,N,H] and w [B,N,L,L]")
-    g = y_grad.detach().to(q.dtype)
-    qd, kd, vd, wd = q.detach(), k.detach(), v.detach(), w.detach()
+    qd, kd, vd, wd = (t.detach().contiguous() for t in (q, k, v, w))
+    g = y_grad.detach().to(qd.dtype).contiguous()
+    B, L, Nh, H1 = qd.shape
+    H2 = vd.shape[3]
+    if kd.shape != qd.shape or vd.shape[:3] != qd.shape[:3] or g.shape != vd.shape or wd.shape != (B, Nh, L, L):
+        raise RuntimeError("attention_bwd: q, k [B,L,N,H1], v and y_grad [B,L,N,H2], w [B,N,L,L] expected")
+    if not (qd.dtype == kd.dtype == vd.dtype == wd.dtype):
+        raise RuntimeError("attention_bwd: q, k, v, w must share one dtype")
+    lib = _lib.load()
+    nws = lib.mega_attention_bwd_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2) if qd.numel() else 0
+    if nws:
+        q_grad, k_grad, v_grad = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+        ws = _scratch_buffer(dev, nws)
+        with _on_device(dev):
+            rc = lib.mega_attention_bwd(_ptr(g), _ptr(qd), _ptr(kd), _ptr(vd), _ptr(wd), _ptr(q_grad), _ptr(k_grad),
+                                        _ptr(v_grad), _dtype_code(qd), B, L, Nh, H1, H2, float(scale),
+                                        1 if use_causal_mask else 0, _ptr(ws), ws.numel(), _stream(dev))
+        _lib.check(rc, "attention_bwd")
+        return q_grad, k_grad, v_grad
     v_grad = torch.einsum('bnqk,bqnh->bknh', wd, g)
     w_grad = torch.einsum('bqnh,bknh->bnqk', g, vd).contiguous()
     s_grad = attention_softmax_bwd(w_grad, wd, use_causal_mask, scale=float(scale), inplace=True)

@@ -425,6 +425,22 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, voi
                        int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
                        int causal, float dropout, uint64_t seed, void* workspace,
                        size_t workspace_bytes, void* stream);
+/* stands in for attention_bwd (fairseq/csrc/ops/attention_kernel.cu:133-255, 278-296): the gradients of
+ * mega_attention_fwd with respect to q, k and v from y_grad [B,L,Nh,H2] and the forward's weights
+ * w [B,Nh,L,L] (the reference keeps them for the backward as well):
+ *   w_grad = y_grad v^T;  s_grad = scale w (w_grad - rowsum(w w_grad));
+ *   v_grad = w^T y_grad;  q_grad = s_grad k;  k_grad = s_grad^T q           per (b, n),
+ * with the causal half of every product skipped when causal != 0.  Weights that DropKey zeroed in
+ * the forward give zero gradients by the same formulas.  16-bit activations with H1 % 8 == 0 and
+ * H2 % 8 == 0, 16-byte aligned tensors, B * Nh <= 65535, L < 32768 (MEGA_ERR_UNSUPPORTED otherwise;
+ * mega_attention_bwd_workspace_bytes returns 0 for such a request).  The workspace holds the fp32
+ * weight gradient, s_grad and the transposed copies of w, s_grad, y_grad, q and k.       */
+size_t mega_attention_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,
+                                          int64_t H2);
+int mega_attention_bwd(const void* y_grad, const void* q, const void* k, const void* v,
+                       const void* w, void* q_grad, void* k_grad, void* v_grad, int dtype,
+                       int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
+                       int causal, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* SwiGLU gate: y = silu(a) * b, elementwise over n elements of `dtype`.

@@ -384,6 +384,58 @@ def test_attention_autograd(dtype, tol, B, L, Nh, H1, H2):
         assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float16, 4e-3)])
+@pytest.mark.parametrize("B,L,Nh,H1,H2,causal", [
+    (1, 300, 2, 64, 136, True),      # several key tiles, v columns not a multiple of 64
+    (2, 77, 3, 8, 24, True),         # rows of the weights that are not a multiple of 8 long
+    (1, 640, 1, 128, 256, True),     # row tiles of 256 in the v gradient, reductions that start past the first K step
+    (2, 130, 2, 16, 40, False),      # no mask: whole products
+    (1, 1030, 2, 64, 64, True),      # more than one row tile of every product, ragged last tile
+])
+def test_attention_bwd_entry_point(dtype, tol, B, L, Nh, H1, H2, causal):
+    """mega_attention_bwd (the four products on the library's own matrix-core kernel, operands read head-strided in
+    place, the causal half skipped) against the oracle's fp64 gradients (attention_kernel.cu:133-255), from the
+    weights the forward returned.  The weight gradient stays in fp32 here (the reference rounds it to the activation
+    type), so the bound of the per-op tolerance holds for the root-mean-square error and 4x for the worst element."""
+    rng = np.random.default_rng(1000 + L)
+    q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.5, dtype)
+    v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    dy, dy64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+    scale = 1.0 / np.sqrt(H1)
+    lib = M._lib.load()
+    assert lib.mega_attention_bwd_workspace_bytes(M.ops._dtype_code(q), B, L, Nh, H1, H2) > 0
+    y, w = M.ops.attention_fwd(q, k, v, scale, 0.0, causal, need_weights=True)
+    got = M.ops.attention_bwd(dy, q, k, v, w, scale, causal)
+    want = O.attention_bwd(dy64, q64, k64, v64, scale, causal)
+    for name, g, ref in zip("qkv", got, want):
+        assert g.shape == ref.shape and g.dtype == dtype
+        e = host(g) - ref
+        rms = np.sqrt((ref ** 2).mean())
+        assert np.isfinite(host(g)).all(), name
+        assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max()), name
+
+
+def test_attention_bwd_entry_point_refuses_what_it_does_not_cover():
+    """fp32 and head sizes that are not multiples of 8 take the batched library products in ops.attention_bwd; the
+    entry point itself says so instead of computing something else."""
+    lib = M._lib.load()
+    assert lib.mega_attention_bwd_workspace_bytes(0, 1, 64, 1, 16, 16) == 0        # fp32
+    assert lib.mega_attention_bwd_workspace_bytes(1, 1, 64, 1, 12, 16) == 0        # bf16, H1 = 12
+    rng = np.random.default_rng(5)
+    q = dev(rng.normal(size=(1, 64, 1, 12))).to(torch.bfloat16)
+    v = dev(rng.normal(size=(1, 64, 1, 16))).to(torch.bfloat16)
+    y, w = M.ops.attention_fwd(q, q, v, 0.3, 0.0, True, need_weights=True)
+    gq, gk, gv = M.ops.attention_bwd(torch.ones_like(v), q, q, v, w, 0.3, True)       # library products
+    ref = O.attention_bwd(np.ones((1, 64, 1, 16)), host(q), host(q), host(v), 0.3, True)
+    assert rel_err(host(gv), ref[2]) < 2e-2
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=q.device)
+    rc = lib.mega_attention_bwd(M.ops._ptr(v), M.ops._ptr(q), M.ops._ptr(q), M.ops._ptr(v), M.ops._ptr(w),
+                                M.ops._ptr(gq), M.ops._ptr(gk), M.ops._ptr(gv), 1, 1, 64, 1, 12, 16, 0.3, 1,
+                                M.ops._ptr(ws), ws.numel(), None)
+    assert rc == -2                                     # MEGA_ERR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("heads,act,moving,bidir", [(1, 'rmsnorm', 'cema', False), (2, 'silu', 'ema', False),
                                                     (1, 'silu', 'cema', True), (2, 'rmsnorm', 'cema', "padded")])
 def test_gated_attention_layer_trains(heads, act, moving, bidir):
