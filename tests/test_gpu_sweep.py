@@ -210,6 +210,40 @@ def test_attention_sweep(seed):
 
 
 @pytest.mark.parametrize("seed", range(8))
+def test_attention_backward_sweep(seed):
+    """ops.attention_bwd from the forward's weights against the oracle's fp64 gradients: head sizes on both sides of
+    what mega_attention_bwd takes (multiples of 8; the others go through the library products), lengths around the
+    128- and 256-row tiles of its products and lengths that are not a multiple of 8, with and without the mask."""
+    rng = np.random.default_rng(4500 + seed)
+    for case in range(5):
+        dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        L = int(rng.choice([1, 5, 63, 64, 65, 127, 129, 200, 255, 257, 300, 515, 770]))
+        Nh = int(rng.choice([1, 2, 3]))
+        H1 = int(rng.choice([8, 12, 32, 64, 128]))
+        H2 = int(rng.choice([8, 20, 24, 64, 72, 256, 264]))
+        B = int(rng.choice([1, 2]))
+        causal = bool(rng.integers(0, 2))
+        tag = f"seed {seed} case {case}: {dtype} B={B} L={L} Nh={Nh} H1={H1} H2={H2} causal={causal}"
+        print(tag, flush=True)
+        q, q64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+        k, k64 = rounded(rng.normal(size=(B, L, Nh, H1)) * 0.7, dtype)
+        v, v64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+        dy, dy64 = rounded(rng.normal(size=(B, L, Nh, H2)), dtype)
+        scale = float(rng.choice([0.5, 1.0, 2.0])) / np.sqrt(H1)
+        _, w = M.ops.attention_fwd(q, k, v, scale, 0.0, causal, need_weights=True)
+        got = M.ops.attention_bwd(dy, q, k, v, w, scale, causal)
+        torch.cuda.synchronize()
+        want = O.attention_bwd(dy64, q64, k64, v64, scale, causal)
+        tol = {torch.float32: 2e-4, torch.bfloat16: 2e-2, torch.float16: 4e-3}[dtype]
+        for name, g, ref in zip("qkv", got, want):
+            e = host(g) - ref
+            rms = np.sqrt((ref ** 2).mean())
+            assert np.isfinite(host(g)).all(), tag + " " + name
+            assert np.sqrt((e ** 2).mean()) < tol * max(rms, 1e-3), tag + " " + name
+            assert np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max(), 1e-3), tag + " " + name
+
+
+@pytest.mark.parametrize("seed", range(8))
 def test_sequence_norm_sweep(seed):
     rng = np.random.default_rng(5000 + seed)
     for case in range(8):
