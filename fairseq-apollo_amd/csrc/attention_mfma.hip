@@ -866,7 +866,9 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   const int64_t BN_ = B * Nh;
   float* S = (float*)ws;
   ws += align_up((size_t)BN_ * L * Lp * 4, 256);
-  T* P = (T*)ws;                                   // [B*Nh][L][Lp]
+  // probabilities [B*Nh][L][Lp]; when the caller wants the weights and their rows need no padding, they are written
+  // where the caller wants them and the second product reads them there
+  T* P = (w && Lp == L && ((uintptr_t)w % 16) == 0) ? (T*)w : (T*)ws;
   ws += align_up((size_t)BN_ * L * Lp * sizeof(T), 256);
   T* Vt = (T*)ws;                                  // [B*Nh][H2][Lp]
   if (!w && dropout <= 0.f && scale > 0.f && flash_covers<T>(v, y, L, H1, H2)) {
@@ -893,7 +895,7 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
                        causal, dropout, seed, (int64_t)(BN_ * L));
   hipLaunchKernelGGL(softmax_f32_kernel<T>, dim3((unsigned)ceil_div(BN_ * L, 4)), dim3(256), 0, s, S, P, (int)L, (int)L,
                      Lp, Lp, (int)Lp, causal, w ? 1 : 0, (int64_t)(BN_ * L));
-  if (w) {
+  if (w && (void*)P != w) {
     // the weights the reference returns: [B, Nh, L, L]
     hipMemcpy2DAsync(w, (size_t)L * sizeof(T), P, (size_t)Lp * sizeof(T), (size_t)L * sizeof(T), (size_t)(BN_ * L),
                      hipMemcpyDeviceToDevice, s);
