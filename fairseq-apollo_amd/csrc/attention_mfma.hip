@@ -47,7 +47,7 @@ struct GemmArgs {
   int kshift;         // causal offset: row m (of P) sees columns <= m + kshift
   // xcd != 0: one-dimensional grid; every tile of a batch entry runs on one XCD (workgroup ids go
   // round-robin over the 8 XCDs), so both operands of a batch entry are fetched into one L2 only;
-  // the long (late) row tiles of a causal product come first
+  // the long row tiles of a causal product come first
   int xcd, mt, nt;
 };
 
@@ -77,7 +77,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     int rest = (int)blockIdx.x >> 3;
     const int ntile = rest % G.nt;
     rest /= G.nt;
-    const int mtile = G.mt - 1 - rest % G.mt;
+    // the long row tiles first: the late rows of a causal product, the early ones when the reduction starts at
+    // the diagonal (mode 3)
+    const int mtile = G.causal == 3 ? rest % G.mt : G.mt - 1 - rest % G.mt;
     rest /= G.mt;
     bz = rest * 8 + ((int)blockIdx.x & 7);
     m0 = mtile * TM;
@@ -161,27 +163,35 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   const int cn = lane & 15, cr = (lane >> 4) * 4;
   constexpr int VW = 16 / (int)sizeof(TOut);                     // elements per 16-byte piece
   constexpr int CP = TN + VW;                                    // row pitch of the staged tile in elements
-  constexpr bool fits = (size_t)TM * CP * sizeof(TOut) <= (size_t)2 * (TM + TN) * PITCH;
-  const bool wide = fits && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
-  if (wide) {
-    // whole tile through LDS (the operand buffers are free after the last barrier): rows leave as
-    // 16-byte pieces, TN * sizeof(TOut) contiguous bytes each
+  // the tile leaves through LDS (the operand buffers are free after the last barrier) as 16-byte pieces, TN *
+  // sizeof(TOut) contiguous bytes per row: whole, or in NH slices of rows when it is larger than the operand buffers
+  constexpr size_t lds_bytes = (size_t)2 * (TM + TN) * PITCH;
+  constexpr int NH = (size_t)TM * CP * sizeof(TOut) <= lds_bytes ? 1 : (size_t)(TM / 2) * CP * sizeof(TOut) <= lds_bytes ? 2 : 0;
+  const bool wide = NH > 0 && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
+  if (NH > 0 && wide) {
+    constexpr int HR = TM / (NH > 0 ? NH : 1);                   // rows per slice (a multiple of a wave's 64)
     TOut* Cs = (TOut*)lds;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int h = 0; h < NH; ++h) {
+      if (h > 0) __syncthreads();                                // the previous slice has left
+      if (wm / HR == h) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          Cs[(wm + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
-    __syncthreads();
-    constexpr int PPR = TN / VW;                                 // pieces per row
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int u = 0; u < TM * PPR / NT; ++u) {
-      const int pi = tid + u * NT;
-      const int r = pi / PPR, pc = pi - r * PPR;
-      if (m0 + r < G.M)
-        *(uint4*)(C + (int64_t)(m0 + r) * G.ldc + n0 + pc * VW) = *(const uint4*)(Cs + r * CP + pc * VW);
+            for (int u = 0; u < 4; ++u)
+              Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
+      }
+      __syncthreads();
+      constexpr int PPR = TN / VW;                               // pieces per row
+#pragma unroll
+      for (int u = 0; u < HR * PPR / NT; ++u) {
+        const int pi = tid + u * NT;
+        const int r = pi / PPR, pc = pi - r * PPR;
+        if (m0 + h * HR + r < G.M)
+          *(uint4*)(C + (int64_t)(m0 + h * HR + r) * G.ldc + n0 + pc * VW) = *(const uint4*)(Cs + r * CP + pc * VW);
+      }
     }
     return;
   }
@@ -972,7 +982,8 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
   G.lda = Nh * H2; G.ldb = Nh * H2; G.ldc = Lp;
   G.sa = L * Nh * H2; G.sai = H2; G.sb = L * Nh * H2; G.sbi = H2; G.sc = Nh * L * Lp; G.sci = L * Lp;
   G.M = (int)L; G.N = (int)L; G.K = (int)H2; G.alpha = 1.0f; G.causal = causal ? 1 : 0;
-  launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  if (L >= 512) launch_gemm<T, float, 4, 4>(G, L, L, BN_, xcd, s);
+  else launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
   // dS = scale w (dW - rowsum(w dW)) (attention_kernel.cu:195-203)
   {
     const int64_t nrows = BN_ * L;
