@@ -29,7 +29,13 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int BM = 128, BN = 128, BK = 64;      // BM: block size of the causal bookkeeping and the small tile
-constexpr int PITCH = BK * 2 + 16;        // bytes per LDS row of BK 16-bit elements (+ 16 pad)
+#ifndef MEGA_GEMM_SWZ
+#define MEGA_GEMM_SWZ 1
+#endif
+// bytes per LDS row of BK 16-bit elements: dense rows whose 16-byte pieces are XOR-swizzled by the row
+// (piece c of row r sits at c ^ ((r >> 1) & 7): the 16 rows a fragment read touches cover every bank once)
+constexpr int PITCH = MEGA_GEMM_SWZ ? BK * 2 : BK * 2 + 16;
+__device__ __forceinline__ int lds_piece(int row, int piece) { return MEGA_GEMM_SWZ ? (piece ^ ((row >> 1) & 7)) : piece; }
 constexpr int KP = BK / 8;                // 16-byte pieces per operand row and K step
 
 struct GemmArgs {
@@ -122,9 +128,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     char* la = lds + buf * (TM + TN) * PITCH;
     char* lb = la + TM * PITCH;
 #pragma unroll
-    for (int h = 0; h < NLA; ++h) *(uint4*)(la + (lrow + h * (NT / KP)) * PITCH + lcol * 2) = ra[h];
+    for (int h = 0; h < NLA; ++h) {
+      const int r = lrow + h * (NT / KP);
+      *(uint4*)(la + r * PITCH + lds_piece(r, tid % KP) * 16) = ra[h];
+    }
 #pragma unroll
-    for (int h = 0; h < NLB; ++h) *(uint4*)(lb + (lrow + h * (NT / KP)) * PITCH + lcol * 2) = rb[h];
+    for (int h = 0; h < NLB; ++h) {
+      const int r = lrow + h * (NT / KP);
+      *(uint4*)(lb + r * PITCH + lds_piece(r, tid % KP) * 16) = rb[h];
+    }
   };
   f32x4 acc[4][4];
 #pragma unroll
@@ -132,7 +144,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int wm = (wave / WN) * 64, wn = (wave % WN) * 64;
-  const int fr = lane & 15, fk = (lane >> 4) * 16;                // fragment row, byte offset of the k block
+  const int fr = lane & 15;                                       // fragment row; lane >> 4 is its 16-byte k block
 
   if (nk > kt0) {
     gload(kt0);
@@ -148,9 +160,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     for (int kk = 0; kk < BK / 32; ++kk) {
       uint4 fa[4], fb[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + kk * 64 + fk);
+      for (int i = 0; i < 4; ++i)
+        fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + lds_piece(wm + i * 16 + fr, kk * 4 + (lane >> 4)) * 16);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + kk * 64 + fk);
+      for (int j = 0; j < 4; ++j)
+        fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -166,7 +180,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   // the tile leaves through LDS (the operand buffers are free after the last barrier) as 16-byte pieces, TN *
   // sizeof(TOut) contiguous bytes per row: whole, or in NH slices of rows when it is larger than the operand buffers
   constexpr size_t lds_bytes = (size_t)2 * (TM + TN) * PITCH;
-  constexpr int NH = (size_t)TM * CP * sizeof(TOut) <= lds_bytes ? 1 : (size_t)(TM / 2) * CP * sizeof(TOut) <= lds_bytes ? 2 : 0;
+  constexpr size_t tile_bytes = (size_t)TM * CP * sizeof(TOut);
+  constexpr int NH = tile_bytes <= lds_bytes ? 1 : tile_bytes / 2 <= lds_bytes ? 2 : (tile_bytes / 4 <= lds_bytes && TM >= 256) ? 4 : 0;
   const bool wide = NH > 0 && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
   if (NH > 0 && wide) {
     constexpr int HR = TM / (NH > 0 ? NH : 1);                   // rows per slice (a multiple of a wave's 64)
