@@ -5,20 +5,23 @@
 //                          above the diagonal are skipped
 //   P = softmax_causal(S)  one workgroup per row, fp32 in, 16-bit out (right-aligned mask, a fully
 //                          masked row gives zeros: fairseq/csrc/softmax.cuh:90-153)
-//   y = P v                the same NT GEMM against v^T (v is transposed once through LDS); causal:
-//                          the reduction stops at the diagonal
+//   y = P v                the same kernel with v read in place as a K-major operand (its tile goes to LDS as it
+//                          lies in memory, the fragments come out of transposing LDS reads); causal: the
+//                          reduction stops at the diagonal.  v rows that are not whole 16-byte pieces go
+//                          through a transposed copy instead
 //
 // Backward (fairseq/csrc/ops/attention_kernel.cu:133-255), with the forward's weights w:
-//   dW = dy v^T            NT GEMM, fp32 out; causal: tiles above the diagonal are skipped
+//   dW = dy v^T            fp32 out; causal: tiles above the diagonal are skipped
 //   dS = scale w (dW - rowsum(w dW))       one wave per row, zeros behind the causal limit
-//   dv = w^T dy, dk = dS^T q               NT GEMMs against transposed copies (w^T, dS^T, dy^T, q^T); causal: the
-//                                          reduction starts at the diagonal
-//   dq = dS k                              NT GEMM against k^T; causal: the reduction stops at the diagonal
+//   dv = w^T dy, dk = dS^T q               both operands K-major (w, dS, dy, q read in place); causal: the
+//                                          reduction starts at the diagonal, long row tiles first
+//   dq = dS k                              k K-major; causal: the reduction stops at the diagonal
+//   (rows of w that are not whole 16-byte pieces: transposed, zero-padded copies of w, dS, dy, q, k instead)
 //
 // The GEMM: (64 WM) x (64 WN) output tile per workgroup of WM x WN waves (64 x 64 each as 4 x 4 MFMA
 // blocks): 128 x 128 for the scores, 256 x 256 for the second product, which carries the flops.
-// K step 64, operands staged through LDS with a 144-byte row pitch (conflict-free 16-byte reads),
-// register prefetch of the next K step, all tiles of one batch entry on one XCD, epilogue through LDS.
+// K step 64, operands staged through LDS as dense 128-byte rows with XOR-swizzled 16-byte pieces (no bank
+// conflicts), register prefetch of the next K step, all tiles of one batch entry on one XCD, epilogue through LDS.
 #include "common.h"
 
 namespace mega {
@@ -68,10 +71,33 @@ __device__ __forceinline__ f32x4 mfma16<f16_t>(uint4 a, uint4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// A K-major operand tile in LDS (an operand that enters the product through its columns: BK rows of W 16-bit elements,
+// row k = the W values the tile's rows / columns have at reduction index k): dense rows whose 32-byte spans are
+// XOR-swizzled by the row, so that the transposing fragment reads (ds_read_b64_tr_b16: four rows, four 8-byte columns
+// per group of 16 lanes) fall on different banks.  The XOR touches the low three bits of the span index only.
+__device__ __forceinline__ int kmajor_piece(int row, int piece) {
+  const int vs = (row & 3) + 4 * ((row >> 3) & 1);
+  return (((piece >> 1) ^ vs) << 1) | (piece & 1);
+}
+// the MFMA operand fragment (16 rows or columns x 32 reduction indices) of a K-major tile: lane (n, g) ends up with
+// the eight consecutive reduction indices 8 g .. 8 g + 7 of tile column 16 span + n.  base = tile + the lane's part
+// (kmajor_lane), rowbytes = 2 W
+__device__ __forceinline__ uint4 kmajor_frag(const char* base, int rowbytes, int span, int vsw) {
+  typedef __attribute__((ext_vector_type(4))) short s4v;
+  const char* q0 = base + (((span & 7) ^ vsw) * 32) + (span >> 3) * 256;
+  const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0));
+  const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*)(q0 + 4 * rowbytes));
+  const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+  return make_uint4(l2.x, l2.y, h2.x, h2.y);
+}
+
 // C = alpha A B^T; TIn 16-bit, TOut float or TIn.  WM x WN waves, each a 64 x 64 block of the
 // (64 WM) x (64 WN) output tile.  The operand traffic from L2 per flop falls with the tile edge:
 // 2 x 2 waves (128 x 128) need 1/64 byte per flop, 4 x 4 waves (256 x 256) half of that.
-template <typename TIn, typename TOut, int WM, int WN>
+// AT / BT: the operand is stored K-major, [K][M] with pitch lda / [K][N] with pitch ldb (C = A^T-stored ... : the
+// product reduces over the operand's rows), and is read in place: its tile goes to LDS as it lies in memory and the
+// fragments come out of transposing LDS reads.  M (N) must be a multiple of 8 then.
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G) {
   constexpr int TM = 64 * WM, TN = 64 * WN, NT = 64 * WM * WN;
   constexpr int NLA = TM * KP / NT, NLB = TN * KP / NT;          // 16-byte pieces per thread and K step
@@ -113,15 +139,25 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     const int k = kt * BK + lcol;
 #pragma unroll
     for (int h = 0; h < NLA; ++h) {
-      const int r = lrow + h * (NT / KP);
       ra[h] = make_uint4(0, 0, 0, 0);
-      if (m0 + r < G.M && k < Kend) ra[h] = *(const uint4*)(A + (int64_t)(m0 + r) * G.lda + k);
+      if (AT) {
+        const int pi = tid + h * NT, kr = kt * BK + pi / (TM / 8), mc = m0 + (pi % (TM / 8)) * 8;
+        if (kr < Kend && mc < G.M) ra[h] = *(const uint4*)(A + (int64_t)kr * G.lda + mc);
+      } else {
+        const int r = lrow + h * (NT / KP);
+        if (m0 + r < G.M && k < Kend) ra[h] = *(const uint4*)(A + (int64_t)(m0 + r) * G.lda + k);
+      }
     }
 #pragma unroll
     for (int h = 0; h < NLB; ++h) {
-      const int r = lrow + h * (NT / KP);
       rb[h] = make_uint4(0, 0, 0, 0);
-      if (n0 + r < G.N && k < Kend) rb[h] = *(const uint4*)(Bm + (int64_t)(n0 + r) * G.ldb + k);
+      if (BT) {
+        const int pi = tid + h * NT, kr = kt * BK + pi / (TN / 8), nc = n0 + (pi % (TN / 8)) * 8;
+        if (kr < Kend && nc < G.N) rb[h] = *(const uint4*)(Bm + (int64_t)kr * G.ldb + nc);
+      } else {
+        const int r = lrow + h * (NT / KP);
+        if (n0 + r < G.N && k < Kend) rb[h] = *(const uint4*)(Bm + (int64_t)(n0 + r) * G.ldb + k);
+      }
     }
   };
   auto lstore = [&](int buf) {
@@ -129,13 +165,23 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     char* lb = la + TM * PITCH;
 #pragma unroll
     for (int h = 0; h < NLA; ++h) {
-      const int r = lrow + h * (NT / KP);
-      *(uint4*)(la + r * PITCH + lds_piece(r, tid % KP) * 16) = ra[h];
+      if (AT) {
+        const int pi = tid + h * NT, kr = pi / (TM / 8), mp = pi % (TM / 8);
+        *(uint4*)(la + kr * (TM * 2) + kmajor_piece(kr, mp) * 16) = ra[h];
+      } else {
+        const int r = lrow + h * (NT / KP);
+        *(uint4*)(la + r * PITCH + lds_piece(r, tid % KP) * 16) = ra[h];
+      }
     }
 #pragma unroll
     for (int h = 0; h < NLB; ++h) {
-      const int r = lrow + h * (NT / KP);
-      *(uint4*)(lb + r * PITCH + lds_piece(r, tid % KP) * 16) = rb[h];
+      if (BT) {
+        const int pi = tid + h * NT, kr = pi / (TN / 8), np = pi % (TN / 8);
+        *(uint4*)(lb + kr * (TN * 2) + kmajor_piece(kr, np) * 16) = rb[h];
+      } else {
+        const int r = lrow + h * (NT / KP);
+        *(uint4*)(lb + r * PITCH + lds_piece(r, tid % KP) * 16) = rb[h];
+      }
     }
   };
   f32x4 acc[4][4];
@@ -145,6 +191,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int wm = (wave / WN) * 64, wn = (wave % WN) * 64;
   const int fr = lane & 15;                                       // fragment row; lane >> 4 is its 16-byte k block
+  // the lane's part of a K-major fragment address: row 8 g + (n >> 2) of the 32-row block, 8-byte column n & 3
+  const int ksr = fr >> 2, kvsw = ksr + 4 * ((lane >> 4) & 1);
+  const int klane_a = (8 * (lane >> 4) + ksr) * (TM * 2) + (fr & 3) * 8;
+  const int klane_b = (8 * (lane >> 4) + ksr) * (TN * 2) + (fr & 3) * 8;
+  static_assert(!(AT || BT) || PITCH == BK * 2, "a K-major tile takes the room of its row-major form");
+  static_assert(!AT || TM == 128 || TM == 256, "a K-major tile row is 256 or 512 bytes");
+  static_assert(!BT || TN == 128 || TN == 256, "a K-major tile row is 256 or 512 bytes");
 
   if (nk > kt0) {
     gload(kt0);
@@ -160,11 +213,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     for (int kk = 0; kk < BK / 32; ++kk) {
       uint4 fa[4], fb[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + lds_piece(wm + i * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+      for (int i = 0; i < 4; ++i) {
+        if (AT)
+          fa[i] = kmajor_frag(la + kk * 32 * (TM * 2) + klane_a, TM * 2, (wm >> 4) + i, kvsw);
+        else
+          fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + lds_piece(wm + i * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+      }
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+      for (int j = 0; j < 4; ++j) {
+        if (BT)
+          fb[j] = kmajor_frag(lb + kk * 32 * (TN * 2) + klane_b, TN * 2, (wn >> 4) + j, kvsw);
+        else
+          fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -224,11 +285,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     }
 }
 
-template <typename TIn, typename TOut, int WM, int WN>
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false>
 void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hipStream_t s) {
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr int smem = 2 * (TM + TN) * PITCH;
-  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN>;
+  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT>;
   static bool attr_set = false;
   if (!attr_set && smem > 64 * 1024) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -901,11 +962,13 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
     MEGA_CHECK_LAUNCH("attention_fwd (one-kernel path)");
     return MEGA_OK;
   }
-  {
+  // v enters the second product through its columns: read in place (K-major form of the kernel) when its rows are
+  // whole 16-byte pieces, through a transposed, zero-padded copy otherwise
+  const bool v_inplace = H2 % 8 == 0 && ((uintptr_t)v % 16) == 0;
+  if (!v_inplace) {
     const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(H2, 64), (unsigned)BN_);
-    const int vec = (H2 % 8 == 0 && ((uintptr_t)v % 16) == 0) ? 1 : 0;
     hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, (const T*)v, Vt, (int)L, (int)Nh, (int)H2, (int)Lp,
-                       vec);
+                       0);
   }
   GemmArgs G;
   // S[b,n] = scale q[b,:,n,:] k[b,:,n,:]^T
@@ -926,13 +989,20 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
                      hipMemcpyDeviceToDevice, s);
   }
   // y[b,:,n,:] = P[b,n] v[b,:,n,:]  ==  P (v^T)^T
-  G.A = P; G.Bm = Vt; G.C = y;
-  G.lda = Lp; G.ldb = Lp; G.ldc = Nh * H2;
-  G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = Nh * H2 * Lp; G.sbi = H2 * Lp; G.sc = L * Nh * H2; G.sci = H2;
-  G.M = (int)L; G.N = (int)H2; G.K = (int)Lp; G.alpha = 1.0f; G.causal = causal ? 2 : 0;
+  G.A = P; G.C = y;
+  G.lda = Lp; G.ldc = Nh * H2;
+  G.sa = Nh * L * Lp; G.sai = L * Lp; G.sc = L * Nh * H2; G.sci = H2;
+  G.M = (int)L; G.N = (int)H2; G.alpha = 1.0f; G.causal = causal ? 2 : 0;
   // the second product carries the flops: 256 x 256 tiles when the problem has that many rows and columns
-  if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4>(G, L, H2, BN_, xcd, s);
-  else launch_gemm<T, T, 2, 2>(G, L, H2, BN_, xcd, s);
+  if (v_inplace) {
+    G.Bm = v; G.ldb = Nh * H2; G.sb = L * Nh * H2; G.sbi = H2; G.K = (int)L;
+    if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4, false, true>(G, L, H2, BN_, xcd, s);
+    else launch_gemm<T, T, 2, 2, false, true>(G, L, H2, BN_, xcd, s);
+  } else {
+    G.Bm = Vt; G.ldb = Lp; G.sb = Nh * H2 * Lp; G.sbi = H2 * Lp; G.K = (int)Lp;
+    if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4>(G, L, H2, BN_, xcd, s);
+    else launch_gemm<T, T, 2, 2>(G, L, H2, BN_, xcd, s);
+  }
   MEGA_CHECK_LAUNCH("attention_fwd (matrix-core path)");
   return MEGA_OK;
 }
@@ -985,11 +1055,15 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
   T* Qt = (T*)(ws + W.qt);
   T* Kt = (T*)(ws + W.kt);
   const bool xcd = BN_ % 8 == 0;
-  // transposed copies of the operands that enter a product through their columns
-  launch_transpose<T>((const T*)dy, dYt, BN_, L, Nh, H2, Lp, s);
-  launch_transpose<T>((const T*)q, Qt, BN_, L, Nh, H1, Lp, s);
-  launch_transpose<T>((const T*)k, Kt, BN_, L, Nh, H1, Lp, s);
-  launch_transpose<T>((const T*)w, Wt, BN_, L, 1, L, Lp, s);
+  // operands that enter a product through their columns (w, dS, dy, q, k) are read in place by the K-major form of
+  // the kernel when their rows are whole 16-byte pieces; otherwise through transposed, zero-padded copies
+  const bool inplace = L % 8 == 0 && ((uintptr_t)w % 16) == 0;
+  if (!inplace) {
+    launch_transpose<T>((const T*)dy, dYt, BN_, L, Nh, H2, Lp, s);
+    launch_transpose<T>((const T*)q, Qt, BN_, L, Nh, H1, Lp, s);
+    launch_transpose<T>((const T*)k, Kt, BN_, L, Nh, H1, Lp, s);
+    launch_transpose<T>((const T*)w, Wt, BN_, L, 1, L, Lp, s);
+  }
   GemmArgs G;
   G.nin = (int)Nh; G.kshift = 0;
   // dW[b,n] = dy[b,:,n,:] v[b,:,n,:]^T (attention_kernel.cu:176-193)
@@ -1010,6 +1084,27 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
     else
       hipLaunchKernelGGL((softmax_bwd_f32_kernel<T, 1>), grid, dim3(256), 0, s, dW, (const T*)w, dS, (int)L, (int)L, L, Lp,
                          causal, scale, nrows);
+  }
+  if (inplace) {
+    // dv[b,:,n,:] = w[b,n]^T dy[b,:,n,:] (attention_kernel.cu:155-174): both operands K-major
+    G.A = w; G.Bm = dy; G.C = dv;
+    G.lda = L; G.ldb = Nh * H2; G.ldc = Nh * H2;
+    G.sa = Nh * L * L; G.sai = L * L; G.sb = L * Nh * H2; G.sbi = H2; G.sc = L * Nh * H2; G.sci = H2;
+    G.M = (int)L; G.N = (int)H2; G.K = (int)L; G.alpha = 1.0f; G.causal = causal ? 3 : 0;
+    if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4, true, true>(G, L, H2, BN_, xcd, s);
+    else launch_gemm<T, T, 2, 2, true, true>(G, L, H2, BN_, xcd, s);
+    // dq[b,:,n,:] = dS[b,n] k[b,:,n,:] (attention_kernel.cu:205-222): k K-major
+    G.A = dS; G.Bm = k; G.C = dq;
+    G.lda = Lp; G.ldb = Nh * H1; G.ldc = Nh * H1;
+    G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = L * Nh * H1; G.sbi = H1; G.sc = L * Nh * H1; G.sci = H1;
+    G.N = (int)H1; G.causal = causal ? 2 : 0;
+    launch_gemm<T, T, 2, 2, false, true>(G, L, H1, BN_, xcd, s);
+    // dk[b,:,n,:] = dS[b,n]^T q[b,:,n,:] (attention_kernel.cu:224-241): both operands K-major
+    G.Bm = q; G.C = dk;
+    G.causal = causal ? 3 : 0;
+    launch_gemm<T, T, 2, 2, true, true>(G, L, H1, BN_, xcd, s);
+    MEGA_CHECK_LAUNCH("attention_bwd");
+    return MEGA_OK;
   }
   // dS [BN][L][Lp] -> dS^T [BN][Lp][Lp]
   launch_transpose<T>(dS, dSt, BN_, L, 1, Lp, Lp, s);

@@ -391,6 +391,9 @@ def test_attention_autograd(dtype, tol, B, L, Nh, H1, H2):
     (1, 640, 1, 128, 256, True),     # row tiles of 256 in the v gradient, reductions that start past the first K step
     (2, 130, 2, 16, 40, False),      # no mask: whole products
     (1, 1030, 2, 64, 64, True),      # more than one row tile of every product, ragged last tile
+    (2, 264, 2, 72, 136, False),     # rows of whole 16-byte pieces: operands read in place (K-major), no mask
+    (1, 1024, 2, 64, 320, True),     # the same with the mask: several row tiles, reductions that start at the diagonal
+    (3, 72, 1, 8, 8, True),          # in place, smallest head sizes
 ])
 def test_attention_bwd_entry_point(dtype, tol, B, L, Nh, H1, H2, causal):
     """mega_attention_bwd (the four products on the library's own matrix-core kernel, operands read head-strided in
