@@ -550,8 +550,8 @@ def bench_attention_bwd(args):
     q, k, v, dy = mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H1), mk(Bc, C, Nh, H2), mk(Bc, C, Nh, H2)
     scale = 1.0 / H1 ** 0.5
     with torch.no_grad():
-        _, w = M.ops.attention_fwd(q, k, v, scale, 0.0, True, need_weights=True)
-        run = lambda i: M.ops.attention_bwd(dy, q, k, v, w, scale, True)
+        y, w = M.ops.attention_fwd(q, k, v, scale, 0.0, True, need_weights=True)
+        run = lambda i: M.ops.attention_bwd(dy, q, k, v, w, scale, True, y=None if args.no_y else y)
         for _ in range(args.warmup):
             run(0)
         dev_ms, wall_ms, _ = best_region(run, args.steps)
@@ -628,6 +628,8 @@ def main():
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings are scaled by")
+    ap.add_argument("--no-y", action="store_true",
+                    help="attention_bwd: call the backward as the reference does, without the forward's output")
     ap.add_argument("--workload", choices=["block", "decode", "attention", "attention_bwd", "layer", "block_bwd", "layer_train", "seqnorm", "ema_real", "tsn_feature", "long_conv"],
                     default="block",
                     help="block: the headline TimestepNorm -> EMA block (default); decode / attention / layer: "

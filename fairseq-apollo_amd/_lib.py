@@ -69,7 +69,7 @@ SIGNATURES = {
                                             _p, _sz, _p]),
     "mega_attention_softmax_fwd": (_int, [_p, _p, _int, _i64, _i64, _i64, _int, C.c_float, C.c_uint64, _p]),
     "mega_attention_bwd_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _i64]),
-    "mega_attention_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_float, _int,
+    "mega_attention_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, C.c_float, _int,
                                   _p, _sz, _p]),
     "mega_attention_softmax_bwd": (_int, [_p, _p, _p, _int, _i64, _i64, _i64, _int, C.c_float, _p]),
     "mega_attention_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _i64]),

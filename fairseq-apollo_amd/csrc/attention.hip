@@ -20,8 +20,8 @@ bool attention_mfma_bwd_covers(int dtype, const void* dy, const void* q, const v
                                const void* dk, const void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1,
                                int64_t H2);
 size_t attention_mfma_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2);
-int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq,
-                           void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
+int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, const void* y,
+                           void* dq, void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
                            float scale, int causal, void* ws, hipStream_t s);
 
 namespace {
@@ -299,7 +299,7 @@ extern "C" size_t mega_attention_bwd_workspace_bytes(int dtype, int64_t B, int64
 }
 
 extern "C" int mega_attention_bwd(const void* y_grad, const void* q, const void* k, const void* v, const void* w,
-                                  void* q_grad, void* k_grad, void* v_grad, int dtype, int64_t B, int64_t L,
+                                  const void* y, void* q_grad, void* k_grad, void* v_grad, int dtype, int64_t B, int64_t L,
                                   int64_t Nh, int64_t H1, int64_t H2, float scale, int causal, void* workspace,
                                   size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(dtype == MEGA_BF16 || dtype == MEGA_F16, dtype == MEGA_F32 ? MEGA_ERR_UNSUPPORTED : MEGA_ERR_ARG,
@@ -314,6 +314,6 @@ extern "C" int mega_attention_bwd(const void* y_grad, const void* q, const void*
   const size_t need = attention_mfma_bwd_workspace_bytes(dtype, B, L, Nh, H1, H2);
   MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 256) == 0, MEGA_ERR_WORKSPACE,
                "attention_bwd: workspace of %zu bytes (256-byte aligned) needed", need);
-  return attention_mfma_bwd_run(y_grad, q, k, v, w, q_grad, k_grad, v_grad, dtype, B, L, Nh, H1, H2, scale, causal,
+  return attention_mfma_bwd_run(y_grad, q, k, v, w, y, q_grad, k_grad, v_grad, dtype, B, L, Nh, H1, H2, scale, causal,
                                 workspace, (hipStream_t)stream);
 }

@@ -58,6 +58,12 @@ struct GemmArgs {
   // round-robin over the 8 XCDs), so both operands of a batch entry are fetched into one L2 only;
   // the long row tiles of a causal product come first
   int xcd, mt, nt;
+  // softmax-backward epilogue (EPI = 1): C holds elements of the input type, C[m][n] = alpha E[m][n] (acc - rowdot[m])
+  // with zeros behind the causal limit; E has C's batch layout with pitch lde and strides se / sei, rowdot is
+  // [batch][M] fp32
+  const void* E = nullptr;
+  const float* rowdot = nullptr;
+  int64_t lde = 0, se = 0, sei = 0;
 };
 
 template <typename T>
@@ -97,8 +103,9 @@ __device__ __forceinline__ uint4 kmajor_frag(const char* base, int rowbytes, int
 // AT / BT: the operand is stored K-major, [K][M] with pitch lda / [K][N] with pitch ldb (C = A^T-stored ... : the
 // product reduces over the operand's rows), and is read in place: its tile goes to LDS as it lies in memory and the
 // fragments come out of transposing LDS reads.  M (N) must be a multiple of 8 then.
-template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false>
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G) {
+  static_assert(EPI == 0 || sizeof(TOut) == 4, "the softmax-backward epilogue stages fp32");
   constexpr int TM = 64 * WM, TN = 64 * WN, NT = 64 * WM * WN;
   constexpr int NLA = TM * KP / NT, NLB = TN * KP / NT;          // 16-byte pieces per thread and K step
   static_assert(TM * KP % NT == 0 && TN * KP % NT == 0, "tile rows must divide over the threads");
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   const int bo = bz / G.nin, bi = bz - bo * G.nin;
   const TIn* A = (const TIn*)G.A + bo * G.sa + bi * G.sai;
   const TIn* Bm = (const TIn*)G.Bm + bo * G.sb + bi * G.sbi;
-  TOut* C = (TOut*)G.C + bo * G.sc + bi * G.sci;
+  TOut* C = (TOut*)G.C + bo * G.sc + bi * G.sci;     // EPI = 1: unused, the result goes out as TIn (below)
   int Kend = G.K;
   if (G.causal == 2) Kend = min(G.K, m0 + TM + G.kshift);
   if (Kend < 0) Kend = 0;
@@ -243,6 +250,67 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   constexpr size_t lds_bytes = (size_t)2 * (TM + TN) * PITCH;
   constexpr size_t tile_bytes = (size_t)TM * CP * sizeof(TOut);
   constexpr int NH = tile_bytes <= lds_bytes ? 1 : tile_bytes / 2 <= lds_bytes ? 2 : (tile_bytes / 4 <= lds_bytes && TM >= 256) ? 4 : 0;
+  if constexpr (EPI == 1) {
+    TIn* D = (TIn*)G.C + bo * G.sc + bi * G.sci;
+    const TIn* Ep = (const TIn*)G.E + bo * G.se + bi * G.sei;
+    const float* rd = G.rowdot + (int64_t)bz * G.M;
+    auto value = [&](float a, float e, float rdv, int m, int n) {
+      return (!G.causal || n <= m + G.kshift) ? G.alpha * e * (a - rdv) : 0.f;
+    };
+    const bool wide4 = NH > 0 && (G.ldc % 4) == 0 && (G.lde % 4) == 0 && ((((uintptr_t)D) | ((uintptr_t)Ep)) % 8) == 0 &&
+                       n0 + TN <= G.N;
+    if (NH > 0 && wide4) {
+      constexpr int HR = TM / (NH > 0 ? NH : 1);
+      float* Cs = (float*)lds;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        if (h > 0) __syncthreads();
+        if (wm / HR == h) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+              for (int u = 0; u < 4; ++u) Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = acc[i][j][u];
+        }
+        __syncthreads();
+        constexpr int PPR = TN / 4;
+#pragma unroll
+        for (int u = 0; u < HR * PPR / NT; ++u) {
+          const int pi = tid + u * NT;
+          const int r = pi / PPR, pc = pi - r * PPR;
+          const int m = m0 + h * HR + r, n = n0 + pc * 4;
+          if (m < G.M) {
+            const float4 a = *(const float4*)(Cs + r * CP + pc * 4);
+            const Vec<TIn, 4> e = *(const Vec<TIn, 4>*)(Ep + (int64_t)m * G.lde + n);
+            const float rdv = rd[m];
+            Vec<TIn, 4> o;
+            o.v[0] = from_float<TIn>(value(a.x, to_float(e.v[0]), rdv, m, n));
+            o.v[1] = from_float<TIn>(value(a.y, to_float(e.v[1]), rdv, m, n + 1));
+            o.v[2] = from_float<TIn>(value(a.z, to_float(e.v[2]), rdv, m, n + 2));
+            o.v[3] = from_float<TIn>(value(a.w, to_float(e.v[3]), rdv, m, n + 3));
+            *(Vec<TIn, 4>*)(D + (int64_t)m * G.ldc + n) = o;
+          }
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wn + j * 16 + cn;
+        if (n >= G.N) continue;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int m = m0 + wm + i * 16 + cr + u;
+          if (m < G.M)
+            D[(int64_t)m * G.ldc + n] =
+                from_float<TIn>(value(acc[i][j][u], to_float(Ep[(int64_t)m * G.lde + n]), rd[m], m, n));
+        }
+      }
+    return;
+  }
   const bool wide = NH > 0 && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
   if (NH > 0 && wide) {
     constexpr int HR = TM / (NH > 0 ? NH : 1);                   // rows per slice (a multiple of a wave's 64)
@@ -285,11 +353,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     }
 }
 
-template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false>
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0>
 void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hipStream_t s) {
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr int smem = 2 * (TM + TN) * PITCH;
-  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT>;
+  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT, EPI>;
   static bool attr_set = false;
   if (!attr_set && smem > 64 * 1024) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -458,6 +526,33 @@ __global__ __launch_bounds__(256) void dropkey_f32_kernel(float* __restrict__ s,
   const uint64_t e0 = (uint64_t)row * (uint64_t)inner;
   for (int j = lane; j < n; j += 64)
     if (hash_uniform(seed, e0 + j) < dropout) sp[j] = -INFINITY;
+}
+
+// rowdot[b, n, l] = sum_d dy[b, l, n, d] y[b, l, n, d]: with y = w v this is sum_j w[l, j] (dy v^T)[l, j], the row
+// sum the softmax backward subtracts (attention_kernel.cu:195-203), without the L x L weight gradient in memory.
+// One wave per (b, l, n) row of H2 elements (H2 % 8 == 0, 16-byte aligned rows), four rows per workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void rowdot_kernel(const T* __restrict__ dy, const T* __restrict__ y,
+                                                     float* __restrict__ out, int L, int Nh, int H2, int64_t nrows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
+  const int n = (int)(row % Nh);
+  const int64_t bl = row / Nh;
+  const int l = (int)(bl % L);
+  const int64_t b = bl / L;
+  const T* a = dy + row * H2;
+  const T* c = y + row * H2;
+  float acc = 0.f;
+  for (int p = lane * 8; p < H2; p += 512) {
+    const Vec<T, 8> x = *(const Vec<T, 8>*)(a + p);
+    const Vec<T, 8> z = *(const Vec<T, 8>*)(c + p);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = fmaf(to_float(x.v[e]), to_float(z.v[e]), acc);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if (lane == 0) out[(b * Nh + n) * L + l] = acc;
 }
 
 // Softmax backward on the fp32 weight gradient of the first backward product
@@ -1009,7 +1104,7 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
 
 // workspace of the backward, in this order (each part 256-byte aligned)
 struct BwdWs {
-  size_t dw, ds, wt, dst, dyt, qt, kt, total;
+  size_t dw, ds, wt, dst, dyt, qt, kt, rowdot, total;
 };
 BwdWs bwd_workspace(size_t es, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2) {
   const int64_t Lp = (L + 7) / 8 * 8, BN_ = B * Nh;
@@ -1027,6 +1122,7 @@ BwdWs bwd_workspace(size_t es, int64_t B, int64_t L, int64_t Nh, int64_t H1, int
   W.dyt = take((size_t)BN_ * H2 * Lp * es);    // dy^T [BN][H2][Lp]
   W.qt = take((size_t)BN_ * H1 * Lp * es);     // q^T [BN][H1][Lp]
   W.kt = take((size_t)BN_ * H1 * Lp * es);     // k^T
+  W.rowdot = take((size_t)BN_ * L * 4);        // fp32 [BN][L]
   W.total = o;
   return W;
 }
@@ -1042,9 +1138,9 @@ void launch_transpose(const T* src, T* dst, int64_t batches, int64_t rows, int64
 }
 
 template <typename T>
-int run_attention_bwd(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq, void* dk,
-                      void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale, int causal,
-                      char* ws, hipStream_t s) {
+int run_attention_bwd(const void* dy, const void* q, const void* k, const void* v, const void* w, const void* y,
+                      void* dq, void* dk, void* dv, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
+                      int causal, char* ws, hipStream_t s) {
   const int64_t Lp = (L + 7) / 8 * 8, BN_ = B * Nh;
   const BwdWs W = bwd_workspace(sizeof(T), B, L, Nh, H1, H2);
   float* dW = (float*)(ws + W.dw);
@@ -1071,10 +1167,24 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
   G.lda = Nh * H2; G.ldb = Nh * H2; G.ldc = Lp;
   G.sa = L * Nh * H2; G.sai = H2; G.sb = L * Nh * H2; G.sbi = H2; G.sc = Nh * L * Lp; G.sci = L * Lp;
   G.M = (int)L; G.N = (int)L; G.K = (int)H2; G.alpha = 1.0f; G.causal = causal ? 1 : 0;
-  if (L >= 512) launch_gemm<T, float, 4, 4>(G, L, L, BN_, xcd, s);
-  else launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  // with the forward's y at hand the row sum of the softmax backward is dy . y, known before the product, and dS
+  // leaves the product's epilogue directly: no fp32 weight gradient in memory, no softmax-backward pass
+  const bool fused = inplace && y != nullptr && ((uintptr_t)y % 16) == 0;
+  if (fused) {
+    float* rd = (float*)(ws + W.rowdot);
+    const int64_t nrows = B * L * Nh;
+    hipLaunchKernelGGL(rowdot_kernel<T>, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, s, (const T*)dy, (const T*)y, rd,
+                       (int)L, (int)Nh, (int)H2, nrows);
+    G.C = dS; G.E = w; G.rowdot = rd; G.lde = L; G.se = Nh * L * L; G.sei = L * L; G.alpha = scale;
+    if (L >= 512) launch_gemm<T, float, 4, 4, false, false, 1>(G, L, L, BN_, xcd, s);
+    else launch_gemm<T, float, 2, 2, false, false, 1>(G, L, L, BN_, xcd, s);
+  } else if (L >= 512) {
+    launch_gemm<T, float, 4, 4>(G, L, L, BN_, xcd, s);
+  } else {
+    launch_gemm<T, float, 2, 2>(G, L, L, BN_, xcd, s);
+  }
   // dS = scale w (dW - rowsum(w dW)) (attention_kernel.cu:195-203)
-  {
+  if (!fused) {
     const int64_t nrows = BN_ * L;
     const dim3 grid((unsigned)ceil_div(nrows, 4));
     const bool vec = L % 4 == 0 && ((uintptr_t)w % 8) == 0;
@@ -1173,12 +1283,12 @@ size_t attention_mfma_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64
   return bwd_workspace(dtype == MEGA_F32 ? 4 : 2, B, L, Nh, H1, H2).total;
 }
 
-int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, void* dq,
-                           void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
+int attention_mfma_bwd_run(const void* dy, const void* q, const void* k, const void* v, const void* w, const void* y,
+                           void* dq, void* dk, void* dv, int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2,
                            float scale, int causal, void* ws, hipStream_t s) {
   if (dtype == MEGA_BF16)
-    return run_attention_bwd<bf16_t>(dy, q, k, v, w, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
-  return run_attention_bwd<f16_t>(dy, q, k, v, w, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
+    return run_attention_bwd<bf16_t>(dy, q, k, v, w, y, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
+  return run_attention_bwd<f16_t>(dy, q, k, v, w, y, dq, dk, dv, B, L, Nh, H1, H2, scale, causal, (char*)ws, s);
 }
 
 }  // namespace mega

@@ -702,15 +702,15 @@ class AttentionFunc(torch.autograd.Function):
                 training: bool = True, seed=None):
         y, w = ops.attention_fwd(q, k, v, scale, dropout if training else 0.0, use_causal_mask, need_weights=True,
                                  seed=seed)
-        ctx.save_for_backward(q, k, v, w)
+        ctx.save_for_backward(q, k, v, w, y)          # y: lets the backward form the softmax's row sums as y_grad . y
         ctx.scale = scale
         ctx.use_causal_mask = use_causal_mask
         return y
 
     @staticmethod
     def backward(ctx, y_grad):
-        q, k, v, w = ctx.saved_tensors
-        q_grad, k_grad, v_grad = ops.attention_bwd(y_grad, q, k, v, w, ctx.scale, ctx.use_causal_mask)
+        q, k, v, w, y = ctx.saved_tensors
+        q_grad, k_grad, v_grad = ops.attention_bwd(y_grad, q, k, v, w, ctx.scale, ctx.use_causal_mask, y=y)
         return q_grad, k_grad, v_grad, None, None, None, None, None
 
 

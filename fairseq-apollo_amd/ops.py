@@ -510,12 +510,14 @@ def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask
     return dx
 
 
-def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool):
+def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool, y=None):
     """-> (q_grad, k_grad, v_grad).  Reference: attention_bwd, fairseq/csrc/ops/attention_kernel.cu:133-255:
     four batched products around the softmax backward; w [B, Nh, L, L] are the forward's weights.
     16-bit activations with head sizes that are multiples of 8 run through the library's own matrix-core
     products (mega_attention_bwd: head-strided operands read in place, the causal half of every product
-    skipped); fp32 and odd head sizes through four batched library GEMMs around mega_attention_softmax_bwd."""
+    skipped); fp32 and odd head sizes through four batched library GEMMs around mega_attention_softmax_bwd.
+    `y` (not in the reference's signature): the forward's output; with it the softmax backward's row sums are
+    y_grad . y and the L x L weight gradient never reaches memory."""
     dev = _need_gpu(y_grad, q, k, v, w)
     if q.dim() != 4 or w is None or w.dim() != 4:
         raise RuntimeError("attention_bwd: q, k, v must be [B,L,N,H] and w [B,N,L,L]")
@@ -530,10 +532,13 @@ def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool):
     lib = _lib.load()
     nws = lib.mega_attention_bwd_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2) if qd.numel() else 0
     if nws:
+        yd = None
+        if y is not None and y.shape == vd.shape and y.dtype == vd.dtype:
+            yd = y.detach().contiguous()
         q_grad, k_grad, v_grad = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
         ws = _scratch_buffer(dev, nws)
         with _on_device(dev):
-            rc = lib.mega_attention_bwd(_ptr(g), _ptr(qd), _ptr(kd), _ptr(vd), _ptr(wd), _ptr(q_grad), _ptr(k_grad),
+            rc = lib.mega_attention_bwd(_ptr(g), _ptr(qd), _ptr(kd), _ptr(vd), _ptr(wd), _ptr(yd), _ptr(q_grad), _ptr(k_grad),
                                         _ptr(v_grad), _dtype_code(qd), B, L, Nh, H1, H2, float(scale),
                                         1 if use_causal_mask else 0, _ptr(ws), ws.numel(), _stream(dev))
         _lib.check(rc, "attention_bwd")

@@ -433,12 +433,16 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, voi
  * with the causal half of every product skipped when causal != 0.  Weights that DropKey zeroed in
  * the forward give zero gradients by the same formulas.  16-bit activations with H1 % 8 == 0 and
  * H2 % 8 == 0, 16-byte aligned tensors, B * Nh <= 65535, L < 32768 (MEGA_ERR_UNSUPPORTED otherwise;
- * mega_attention_bwd_workspace_bytes returns 0 for such a request).  The workspace holds the fp32
- * weight gradient, s_grad and the transposed copies of w, s_grad, y_grad, q and k.       */
+ * mega_attention_bwd_workspace_bytes returns 0 for such a request).
+ *   y: the forward's output [B,L,Nh,H2], or NULL (the reference's backward does not take it).  With
+ *   y, rowsum(w w_grad) = rowsum(y_grad y) is known before the first product, and when L % 8 == 0
+ *   s_grad leaves that product's epilogue directly: no L x L fp32 weight gradient in memory.
+ * The workspace holds the fp32 weight gradient, s_grad, the row sums and, for rows of w that are
+ * not whole 16-byte pieces (L % 8 != 0), transposed copies of w, s_grad, y_grad, q and k.   */
 size_t mega_attention_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,
                                           int64_t H2);
 int mega_attention_bwd(const void* y_grad, const void* q, const void* k, const void* v,
-                       const void* w, void* q_grad, void* k_grad, void* v_grad, int dtype,
+                       const void* w, const void* y, void* q_grad, void* k_grad, void* v_grad, int dtype,
                        int64_t B, int64_t L, int64_t Nh, int64_t H1, int64_t H2, float scale,
                        int causal, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -409,14 +409,17 @@ def test_attention_bwd_entry_point(dtype, tol, B, L, Nh, H1, H2, causal):
     lib = M._lib.load()
     assert lib.mega_attention_bwd_workspace_bytes(M.ops._dtype_code(q), B, L, Nh, H1, H2) > 0
     y, w = M.ops.attention_fwd(q, k, v, scale, 0.0, causal, need_weights=True)
-    got = M.ops.attention_bwd(dy, q, k, v, w, scale, causal)
     want = O.attention_bwd(dy64, q64, k64, v64, scale, causal)
-    for name, g, ref in zip("qkv", got, want):
-        assert g.shape == ref.shape and g.dtype == dtype
-        e = host(g) - ref
-        rms = np.sqrt((ref ** 2).mean())
-        assert np.isfinite(host(g)).all(), name
-        assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max()), name
+    # without and with the forward's output (the second lets the entry point take the row sums from y_grad . y)
+    for with_y in (False, True):
+        got = M.ops.attention_bwd(dy, q, k, v, w, scale, causal, y=y if with_y else None)
+        for name, g, ref in zip("qkv", got, want):
+            tag = f"{name} with_y={with_y}"
+            assert g.shape == ref.shape and g.dtype == dtype
+            e = host(g) - ref
+            rms = np.sqrt((ref ** 2).mean())
+            assert np.isfinite(host(g)).all(), tag
+            assert np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max()), tag
 
 
 def test_attention_bwd_entry_point_refuses_what_it_does_not_cover():
@@ -433,7 +436,7 @@ def test_attention_bwd_entry_point_refuses_what_it_does_not_cover():
     ref = O.attention_bwd(np.ones((1, 64, 1, 16)), host(q), host(q), host(v), 0.3, True)
     assert rel_err(host(gv), ref[2]) < 2e-2
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=q.device)
-    rc = lib.mega_attention_bwd(M.ops._ptr(v), M.ops._ptr(q), M.ops._ptr(q), M.ops._ptr(v), M.ops._ptr(w),
+    rc = lib.mega_attention_bwd(M.ops._ptr(v), M.ops._ptr(q), M.ops._ptr(q), M.ops._ptr(v), M.ops._ptr(w), None,
                                 M.ops._ptr(gq), M.ops._ptr(gk), M.ops._ptr(gv), 1, 1, 64, 1, 12, 16, 0.3, 1,
                                 M.ops._ptr(ws), ws.numel(), None)
     assert rc == -2                                     # MEGA_ERR_UNSUPPORTED
