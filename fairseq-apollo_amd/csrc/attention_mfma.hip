@@ -139,32 +139,56 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   const int nk = (Kend + BK - 1) / BK;
   const int kt0 = G.causal == 3 ? max(0, m0 - G.kshift) / BK : 0;      // first K step that can hold a non-zero
 
-  // global -> register staging
+  // global -> register staging: a wave-uniform tile pointer plus a 32-bit byte offset per lane and piece
   const int lrow = tid / KP, lcol = (tid % KP) * 8;              // rows 0 .. NT/KP - 1 (+ h * NT/KP)
   uint4 ra[NLA], rb[NLB];
+  uint32_t offa[NLA], offb[NLB];
+  int kra[NLA], krb[NLB];                                        // K-major: the piece's row of the K step
+  bool oka[NLA], okb[NLB];                                       // the piece's row / column lies inside the matrix
+#pragma unroll
+  for (int h = 0; h < NLA; ++h) {
+    if (AT) {
+      const int pi = tid + h * NT;
+      kra[h] = pi / (TM / 8);
+      const int mc = (pi % (TM / 8)) * 8;
+      oka[h] = m0 + mc < G.M;
+      offa[h] = (uint32_t)(((int64_t)kra[h] * G.lda + mc) * 2);
+    } else {
+      const int r = lrow + h * (NT / KP);
+      kra[h] = 0;
+      oka[h] = m0 + r < G.M;
+      offa[h] = (uint32_t)(((int64_t)r * G.lda + lcol) * 2);
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < NLB; ++h) {
+    if (BT) {
+      const int pi = tid + h * NT;
+      krb[h] = pi / (TN / 8);
+      const int nc = (pi % (TN / 8)) * 8;
+      okb[h] = n0 + nc < G.N;
+      offb[h] = (uint32_t)(((int64_t)krb[h] * G.ldb + nc) * 2);
+    } else {
+      const int r = lrow + h * (NT / KP);
+      krb[h] = 0;
+      okb[h] = n0 + r < G.N;
+      offb[h] = (uint32_t)(((int64_t)r * G.ldb + lcol) * 2);
+    }
+  }
   auto gload = [&](int kt) {
     const int k = kt * BK + lcol;
+    // tile origin of this K step: row m0 / n0 at column kt BK, or (K-major) row kt BK at column m0 / n0
+    const char* Au = (const char*)(AT ? A + (int64_t)kt * BK * G.lda + m0 : A + (int64_t)m0 * G.lda + kt * BK);
+    const char* Bu = (const char*)(BT ? Bm + (int64_t)kt * BK * G.ldb + n0 : Bm + (int64_t)n0 * G.ldb + kt * BK);
 #pragma unroll
     for (int h = 0; h < NLA; ++h) {
       ra[h] = make_uint4(0, 0, 0, 0);
-      if (AT) {
-        const int pi = tid + h * NT, kr = kt * BK + pi / (TM / 8), mc = m0 + (pi % (TM / 8)) * 8;
-        if (kr < Kend && mc < G.M) ra[h] = *(const uint4*)(A + (int64_t)kr * G.lda + mc);
-      } else {
-        const int r = lrow + h * (NT / KP);
-        if (m0 + r < G.M && k < Kend) ra[h] = *(const uint4*)(A + (int64_t)(m0 + r) * G.lda + k);
-      }
+      if (oka[h] && (AT ? kt * BK + kra[h] < Kend : k < Kend)) ra[h] = *(const uint4*)(Au + offa[h]);
     }
 #pragma unroll
     for (int h = 0; h < NLB; ++h) {
       rb[h] = make_uint4(0, 0, 0, 0);
-      if (BT) {
-        const int pi = tid + h * NT, kr = kt * BK + pi / (TN / 8), nc = n0 + (pi % (TN / 8)) * 8;
-        if (kr < Kend && nc < G.N) rb[h] = *(const uint4*)(Bm + (int64_t)kr * G.ldb + nc);
-      } else {
-        const int r = lrow + h * (NT / KP);
-        if (n0 + r < G.N && k < Kend) rb[h] = *(const uint4*)(Bm + (int64_t)(n0 + r) * G.ldb + k);
-      }
+      if (okb[h] && (BT ? kt * BK + krb[h] < Kend : k < Kend)) rb[h] = *(const uint4*)(Bu + offb[h]);
     }
   };
   auto lstore = [&](int buf) {
@@ -218,7 +242,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     const char* lb = la + TM * PITCH;
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
-      uint4 fa[4], fb[4];
+      uint4 fa[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (AT)
@@ -226,17 +250,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
         else
           fa[i] = *(const uint4*)(la + (wm + i * 16 + fr) * PITCH + lds_piece(wm + i * 16 + fr, kk * 4 + (lane >> 4)) * 16);
       }
+      // the B fragments one column block at a time (four at once do not fit the 128 registers of a 16-wave
+      // workgroup next to the K-major address arithmetic)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        uint4 fb;
         if (BT)
-          fb[j] = kmajor_frag(lb + kk * 32 * (TN * 2) + klane_b, TN * 2, (wn >> 4) + j, kvsw);
+          fb = kmajor_frag(lb + kk * 32 * (TN * 2) + klane_b, TN * 2, (wn >> 4) + j, kvsw);
         else
-          fb[j] = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+          fb = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i][j] = mfma16<TIn>(fa[i], fb, acc[i][j]);
+        // K-major forms: keep the compiler from fetching all four B fragments ahead (that spills in the loop)
+        if ((AT || BT) && WM * WN == 16 && (j & 1)) __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<TIn>(fa[i], fb[j], acc[i][j]);
     }
     if (kt + 1 < nk) lstore(buf ^ 1);
     __syncthreads();
