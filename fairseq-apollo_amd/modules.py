@@ -11,8 +11,8 @@ shapes (so reference checkpoints load) and the same incremental-state keys.
     SwiGLU                  no counterpart in the reference (its FFN is
                             fairseq/modules/normalized_feedforward_network.py:77-93)
 
-Forward / inference only: the HIP kernels have no backward pass yet, so a forward that
-would need gradients raises instead of silently detaching.
+Every module works under autograd through the library's backward kernels (the autograd functions below);
+what has no backward (incremental state under a graph) raises instead of silently detaching.
 """
 from __future__ import annotations
 
