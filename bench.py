@@ -589,7 +589,8 @@ def bench_layer(args):
     ws = torch.randn(1, L4, D4, device=dev).to(torch.bfloat16)
 
     def step(i):
-        if train:                      # forward + backward of sum(y * w); gradients accumulate in .grad
+        if train:                      # forward + backward of sum(y * w), from cleared gradients as a trainer's
+            blk.zero_grad(set_to_none=True)    # zero_grad leaves them (fairseq/trainer.py:438)
             (blk(xs[i % 4]) * ws).sum().backward()
         else:
             blk(xs[i % 4])
