@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       {
         // all loads of a batch are issued before the first one is looked at
         constexpr int kBatch = 8;
-        const int w0 = p0 * W;                        // first word of this round in the list of all records
+        const int w0 = p0 * W;                        // first word of this pass in the list of all records
         const int nw = np * W;
         auto word = [&](const int i) -> const unsigned long long* {
           const int gw = w0 + i;
