@@ -706,6 +706,19 @@ __device__ __forceinline__ void lds_dma16(const void* addr /* per lane */, uint3
       : [addr] "v"(addr), [lds] "s"(lds_base)
       : "memory");
 }
+// maximum over the four lanes that hold one query column (lanes n, n + 16, n + 32, n + 48), the same value in all
+// four, with the lane-swap instructions of gfx950 instead of two trips through the LDS crossbar:
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second,
+// v_permlane16_swap the odd rows of 16 lanes of the first with the even rows of the second
+__device__ __forceinline__ float quad_max(float t) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, t);
+  const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const float m = fmaxf(__builtin_bit_cast(float, h[0]), __builtin_bit_cast(float, h[1]));
+  const uint32_t v = __builtin_bit_cast(uint32_t, m);
+  const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
@@ -905,8 +918,7 @@ __global__ __launch_bounds__(64 * FNW) void flash_fwd_kernel(const FlashArgs A) 
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int u = 0; u < 4; ++u) tmax = fmaxf(tmax, S[kb][j][u]);
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      tmax = quad_max(tmax);
       tmax *= A.scale_log2;                                        // scale > 0: the maximum commutes with it
       // the running maximum moves only when a tile exceeds it by more than 2^8: probabilities up to 256
       // are as exact as those below 1, and y is rescaled on few tiles
