@@ -121,8 +121,11 @@ __device__ __forceinline__ int plane_off(int i) {
 // multiple of 4.  BOTH (second kernel, L a multiple of 1024, VEC): a wave forms both directions of its 1024 tokens
 // of memory, backward first, and adds them up in LDS, so that y is written once and no partial sums pass
 // through memory.
+#ifndef MEGA_ROWS_MINB
+#define MEGA_ROWS_MINB 3
+#endif
 template <typename T, int NX, bool F16, bool STATE, bool VEC, bool BOTH>
-__global__ __launch_bounds__(64 * kRW, 4) void ema_rows_kernel(const RowsArgs A) {
+__global__ __launch_bounds__(64 * kRW, MEGA_ROWS_MINB) void ema_rows_kernel(const RowsArgs A) {
   constexpr int kWaveLds = (BOTH ? 2 : 1) * kRWaveLds;
   __shared__ __attribute__((aligned(16))) char lds[kRW * kWaveLds];
   const int lane = threadIdx.x & 63;
