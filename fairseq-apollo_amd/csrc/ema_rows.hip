@@ -121,6 +121,9 @@ __device__ __forceinline__ int plane_off(int i) {
 // multiple of 4.  BOTH (second kernel, L a multiple of 1024, VEC): a wave forms both directions of its 1024 tokens
 // of memory, backward first, and adds them up in LDS, so that y is written once and no partial sums pass
 // through memory.
+// Workgroups per CU the register budget is set for.  The apply kernel wants about 150 registers per lane: at four
+// workgroups (128 registers) it spills inside the block loop, and every reload of a spilled register waits
+// (vmcnt(0)) for the row loads in flight as well; at three it keeps everything in registers.
 #ifndef MEGA_ROWS_MINB
 #define MEGA_ROWS_MINB 3
 #endif
