@@ -150,3 +150,15 @@ def test_eval_caches_follow_the_parameters():
     c_b, m_b, v_b = norm._prior_state(3)
     assert torch.equal(g_b, sd["weight"] + 1.0) and torch.equal(b_b, sd["bias"])
     assert torch.equal(m_b, sd["prior_mean"].expand(3, -1)) and torch.allclose(v_b, sd["prior_logv"].exp().expand(3, -1))
+
+
+def test_bench_measures_one_gpu_only():
+    """bench.py --gpus N with N > 1 exits with a message instead of starting ranks."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
