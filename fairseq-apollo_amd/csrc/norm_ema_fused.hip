@@ -599,7 +599,11 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       for (int w = 0; w < kNWC; ++w)
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
-      if (steps > 1) load_c4(img, kSlotRJ, loff, Jr, Ji);      // else (q^64)^j is 1, q^64, then nothing
+      // requested whatever `steps` says (for steps <= 1 the consumer replaces it by 1, q^64, 0): a load under a branch
+      // has to be waited for inside the branch, where its registers are merged with the other path's, and that wait
+      // (vmcnt is in order) would also cover the operand loads above and the previous channel's stores of y
+      (void)steps;
+      load_c4(img, kSlotRJ, loff, Jr, Ji);
     };
     bf16x8 Cn[kNWC][2];
     float Jnr[4] = {0.f, 0.f, 0.f, 0.f}, Jni[4] = {0.f, 0.f, 0.f, 0.f};
