@@ -23,6 +23,8 @@
 // Blocks map to workgroup ids time-major and workgroups are dispatched in id order, so a block only
 // waits for blocks dispatched before it; every wait is bounded and poisons the block's outputs with
 // NaN (and sets the error word of the workspace header) when it gives up.
+#include <type_traits>
+
 #include "ema_mfma.h"
 #include "tsn_common.h"
 
@@ -57,11 +59,6 @@ constexpr size_t kFSmem = (size_t)kFTile + 2 * kFSeg * 4 + 64 + (size_t)kFTabs *
 static_assert(kSEGT == 2, "the fused kernel uses the q^64 segment multipliers of the image");
 static_assert(kFSmem <= 160 * 1024, "LDS of one workgroup");
 
-// the MFMA A operands of one channel
-struct ImgSet {
-  bf16x8 P[kNWP][2], K[kNWK][2], C[kNWC][2];
-};
-
 struct FusedArgs {
   const bf16_t* x;       // [B, L, D]
   bf16_t* xn;            // [B, L, D]
@@ -79,7 +76,7 @@ struct FusedArgs {
   const float* h_in;     // [B, D, N, 2] or null
   float* h_out;          // [B, D, N, 2] or null
   TsnHeader* hdr;
-  unsigned long long* rec;   // [B * G][S][kFRecW]
+  unsigned long long* rec;   // [B * G][S + 1][kFRecW]; slot S: the caller's carried state, put there by block 0
   int B, L, D, G, N, S;
   float eps;
   int is_complex;
@@ -205,7 +202,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   const size_t xblk = ((size_t)b * A.L + t0) * A.D + (size_t)g * kFC;
   const uint32_t toff = (uint32_t)tokl * (uint32_t)A.D + piece * 8;
   const size_t brow = (size_t)b * G + g;
-  unsigned long long* const myrec = A.rec + (brow * A.S + s) * kFRecW;
+  unsigned long long* const myrec = A.rec + (brow * (A.S + 1) + s) * kFRecW;
   bool poison = false;
 
   MEGA_FTR(0);
@@ -231,6 +228,19 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
             *(const uint4*)(ibase + (size_t)c * kImgRowBytes + t * 128 + pc * 16);
       }
     }
+  }
+
+  // ---- the caller's carried state joins the records the later look-ups read: slot S of the row, written by block 0
+  if (s == 0 && A.h_in) {
+    const int c = tid >> 4, n = tid & 15;
+    float2 v = make_float2(0.f, 0.f);
+    if (n < A.N) {
+      v = *(const float2*)(A.h_in + (((size_t)b * A.D + g * kFC + c) * A.N + n) * 2);
+      if (!A.is_complex) v.y = 0.f;
+    }
+    unsigned long long* e = A.rec + (brow * (A.S + 1) + A.S) * kFRecW + 4 + ((size_t)c * kNS + n) * 2;
+    put_rec(e, tagged(__float_as_uint(v.x), tag));
+    put_rec(e + 1, tagged(__float_as_uint(v.y), tag));
   }
 
   // ---- moments of every token's group (64 channels = the 8 lanes of a line)
@@ -301,7 +311,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     // earlier blocks of this (row, group): lane i fetches block i's aggregate
     Moments accp = {0.f, 0.f, 0.f};
     if (s > 0) {
-      const unsigned long long* rp = A.rec + (brow * A.S + (lane < s ? lane : s - 1)) * kFRecW;
+      const unsigned long long* rp = A.rec + (brow * (A.S + 1) + (lane < s ? lane : s - 1)) * kFRecW;
       unsigned long long w0, w1, w2;
       uint32_t spins = 0;
       for (;;) {
@@ -345,20 +355,20 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   }
   __syncthreads();
 
-  // the operands of the wave's first channel travel under the normalisation
+  // operand loaders of the moving-average phases (one register set: a channel's operands are requested as soon
+  // as the previous channel's have been used, and travel under the rest of that channel's work)
   const uint32_t loff0 = (uint32_t)lane * 16;
   const uint32_t koff0 = (uint32_t)(((lane & 15) - 8 * (lane >> 4) + 24) * 16);
-  // the P operand of channel c (requested one channel ahead)
-  auto load_p = [&](const int c, ImgSet& I) {
+  auto load_p = [&](const int c, bf16x8 (&P)[kNWP][2]) {
     const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
 #pragma unroll
     for (int w = 0; w < kNWP; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) I.P[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotP + 2 * w + mb, loff));
+      for (int mb = 0; mb < 2; ++mb) P[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotP + 2 * w + mb, loff));
   };
-  auto load_kc = [&](const int c, ImgSet& I) {
+  auto load_kc = [&](const int c, bf16x8 (&K)[kNWK][2], bf16x8 (&C)[kNWC][2]) {
     const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
@@ -369,15 +379,15 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     for (int w = 0; w < kNWK; ++w)
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
-        I.K[w][mb] = __builtin_bit_cast(bf16x8, *(const uint4*)(img + (kSlotKT + w) * 1024 + mb * 256 + koff));
+        K[w][mb] = __builtin_bit_cast(bf16x8, *(const uint4*)(img + ((kSlotKT + w) * 1024 + mb * 256) + koff));
 #pragma unroll
     for (int w = 0; w < kNWC; ++w)
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) I.C[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
+      for (int mb = 0; mb < 2; ++mb) C[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
   };
-  ImgSet img_set[2];
-  load_p(wave, img_set[0]);
-  load_kc(wave, img_set[0]);
+  // the P operand of the wave's first channel travels under the normalisation
+  bf16x8 Pa[kNWP][2];
+  load_p(wave, Pa);
 
   // ---- normalise from registers and stage xn (bf16, as the layer sees it) transposed: channel rows of 16
   // segments x 128 bytes, 16-byte chunk c of segment j at chunk c ^ (j >> 1) (the 16 lanes of a matrix-core
@@ -390,6 +400,13 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const int tl = tokl & ~1;
     char* wbase = tile + row_base(piece * 8 + odd * 4) + (tl >> 6) * 128 + ((tl & 7) >> 1) * 4;
     const int c8 = (tl & 63) >> 3;
+    // weight + 1 = 1 and bias = 0 for every channel of the group (the module's initial values): the affine step
+    // is skipped, one multiply-add per element less (a wave sees all 64 channels, so the branch is uniform)
+    bool plain = true;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) plain = plain && gam[i] == 1.f && bet[i] == 0.f;
+    const bool ident = __all(plain);
+    auto stage = [&](auto IDENT) {
 #pragma unroll
     for (int k = 0; k < kFNLD; ++k) {
       const int tok = k * 128 + tokl;
@@ -401,7 +418,8 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       for (int i = 0; i < 4; ++i) {
         const float lo = fmaf(__uint_as_float(w[i] << 16), r, -mr);
         const float hi = fmaf(__uint_as_float(w[i] & 0xffff0000u), r, -mr);
-        o[i] = pack_bf16(fmaf(lo, gam[2 * i], bet[2 * i]), fmaf(hi, gam[2 * i + 1], bet[2 * i + 1]));
+        o[i] = decltype(IDENT)::value ? pack_bf16(lo, hi)
+                                      : pack_bf16(fmaf(lo, gam[2 * i], bet[2 * i]), fmaf(hi, gam[2 * i + 1], bet[2 * i + 1]));
       }
       store_stream((uint4*)(A.xn + xblk + (size_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
       const uint32_t s0 = odd ? o[0] : o[2], s1 = odd ? o[1] : o[3];
@@ -412,6 +430,12 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       *(uint32_t*)(wp + kFRow) = __builtin_amdgcn_perm(r0, m0, sel_hi);
       *(uint32_t*)(wp + 2 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_lo);
       *(uint32_t*)(wp + 3 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_hi);
+    }
+    };
+    if (ident) {
+      stage(std::true_type{});
+    } else {
+      stage(std::false_type{});
     }
   }
   __syncthreads();
@@ -451,24 +475,20 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     }
   };
 
-  // pass 1 over channel c, everything that does not need the earlier blocks: end states of the 16 segments
-  // from a zero start (P products), scanned across the row; the block's end state from a zero start is
-  // published; y = K x + C (segment start state from a zero block start) goes back into LDS over x as bf16
-  auto pass1 = [&](const int c, const int cnext, const int steps, ImgSet& cur, ImgSet& nxt) {
-    uint32_t roff = roff0;
-    asm volatile("" : "+v"(roff));
-    float Qr[4], Qi[4];
-    lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
-    char* row = tile + row_base(c) + j * 128;
-    float Er[4], Ei[4], Fr[4], Fi[4];              // F: state after the segment's first tile from a zero segment start
+  // End states of channel c's 16 segments from a zero start (P products; F = the state after a segment's first
+  // tile), scanned across the row by doubling: E becomes the state after segment j with the block started from
+  // zero.  A step over d segments is skipped (uniform branch) when |q|^(64 d) < 2^-24 for every state of the
+  // channel: what it would add is below fp32 resolution.
+  auto segment_scan = [&](const int c, const int steps, const bf16x8 (&P)[kNWP][2], const bf16x8& X0, const bf16x8& X1,
+                          const float (&Qr)[4], const float (&Qi)[4], float (&Er)[4], float (&Ei)[4], float (&Fr)[4],
+                          float (&Fi)[4], const uint32_t roff) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const bf16x8 X = *(const bf16x8*)(row + (((4 * t + r) ^ (j >> 1)) << 4));
       f32x4 S0 = {0.f, 0.f, 0.f, 0.f}, S1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int w = 0; w < kNWP; ++w) {
-        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.P[w][0], X, S0, 0, 0, 0);
-        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.P[w][1], X, S1, 0, 0, 0);
+        S0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(P[w][0], t == 0 ? X0 : X1, S0, 0, 0, 0);
+        S1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(P[w][1], t == 0 ? X0 : X1, S1, 0, 0, 0);
       }
       const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
       const float si[4] = {S0[1], S0[3], S1[1], S1[3]};
@@ -483,13 +503,6 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         }
       }
     }
-    MEGA_FTR2(0);
-    // the next channel's P operand is requested as soon as this one's is used up
-    __builtin_amdgcn_sched_barrier(0);
-    if (cnext >= 0) load_p(cnext, nxt);
-    __builtin_amdgcn_sched_barrier(0);
-    // inclusive scan over the 16 segments by doubling; a step over d segments is skipped (uniform branch) when
-    // |q|^(64 d) < 2^-24 for every state of the channel: what it would add is below fp32 resolution
     if (steps > 0) {
       float Rr[4], Ri[4], R2r[4], R2i[4];
       lds_cmp(s_tab, kCmpRS, c, roff, Rr, Ri);
@@ -507,70 +520,34 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         }
       }
     }
-    MEGA_FTR2(1);
-    // lane 15 of a row holds the block's end state from a zero start: parked in LDS, published for the later
-    // blocks after the wave's last channel (and kept for the carried state the last block returns)
+  };
+
+  // ---- phase A, what the later blocks wait for: the block's end state from a zero start (lane 15 of every row
+  // after the scan), parked in LDS and published
+  MEGA_FTR(5);
+  // it goes before the other waves' phase B
+  __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+  for (int i = 0; i < kFCPW; ++i) {
+    const int c = wave + kFW * i;
+    uint32_t roff = roff0;
+    asm volatile("" : "+v"(roff));
+    float Qr[4], Qi[4];
+    lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
+    const char* row = tile + row_base(c) + j * 128;
+    const bf16x8 X0 = *(const bf16x8*)(row + (((r) ^ (j >> 1)) << 4));
+    const bf16x8 X1 = *(const bf16x8*)(row + (((4 + r) ^ (j >> 1)) << 4));
+    float Er[4], Ei[4], Fr[4], Fi[4];
+    segment_scan(c, nsteps[i], Pa, X0, X1, Qr, Qi, Er, Ei, Fr, Fi, roff);
     if (j == 15) {
       *(float4*)(s_end + (c * kNS + 2 * r) * 2) = make_float4(Er[0], Ei[0], Er[1], Ei[1]);
       *(float4*)(s_end + (c * kNS + 8 + 2 * r) * 2) = make_float4(Er[2], Ei[2], Er[3], Ei[3]);
     }
-    MEGA_FTR2(2);
-    // ... and its K and C operands a whole pass before they are needed
+    // the next channel's P operand (after the last channel: the first one's again, for phase B)
     __builtin_amdgcn_sched_barrier(0);
-    if (cnext >= 0) load_kc(cnext, nxt);
+    load_p(i + 1 < kFCPW ? wave + kFW * (i + 1) : wave, Pa);
     __builtin_amdgcn_sched_barrier(0);
-    MEGA_FTR2(3);
-    // start state of segment j = inclusive value of segment j - 1; of its second tile: q^32 times that + F
-    float hr[4], hi[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      hr[u] = dpp_f<0x111>(Er[u]);
-      hi[u] = dpp_f<0x111>(Ei[u]);
-    }
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const bf16x8 X = *(const bf16x8*)(row + (((4 * t + r) ^ (j >> 1)) << 4));
-      bf16x8 Hop;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        Hop[2 * u] = (__bf16)hr[u];
-        Hop[2 * u + 1] = (__bf16)hi[u];
-      }
-      f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int w = 0; w < kNWC; ++w) {
-        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.C[w][0], Hop, Y0, 0, 0, 0);
-        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.C[w][1], Hop, Y1, 0, 0, 0);
-      }
-#pragma unroll
-      for (int w = 0; w < kNWK; ++w) {
-        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.K[w][0], X, Y0, 0, 0, 0);
-        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.K[w][1], X, Y1, 0, 0, 0);
-      }
-      if (t == 0) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const float nr = fmaf(Qr[u], hr[u], fmaf(-Qi[u], hi[u], Fr[u]));
-          hi[u] = fmaf(Qr[u], hi[u], fmaf(Qi[u], hr[u], Fi[u]));
-          hr[u] = nr;
-        }
-      }
-      // y (bf16) over x: tokens 32 t + 4 r + {0..3} and 32 t + 16 + 4 r + {0..3} of segment j
-      const uint2 o0 = make_uint2(pack_bf16(Y0[0], Y0[1]), pack_bf16(Y0[2], Y0[3]));
-      const uint2 o1 = make_uint2(pack_bf16(Y1[0], Y1[1]), pack_bf16(Y1[2], Y1[3]));
-      *(uint2*)(row + (((4 * t + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) = o0;
-      *(uint2*)(row + (((4 * t + 2 + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) = o1;
-    }
-  };
-
-  MEGA_FTR(5);
-  {
-#pragma unroll
-    for (int i = 0; i < kFCPW; ++i) {
-      pass1(wave + kFW * i, i + 1 < kFCPW ? wave + kFW * (i + 1) : -1, nsteps[i], img_set[i & 1], img_set[(i + 1) & 1]);
-      __builtin_amdgcn_sched_barrier(0);
-      MEGA_FTR(6 + i);
-    }
+    MEGA_FTR(6 + i);
   }
   if (!last_block && !(A.lb.withhold_first && s == 0)) {
     // the wave's four channels x 16 states x (re, im) = 128 words: two per lane
@@ -582,209 +559,204 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     put_rec(e, tagged(__float_as_uint(v.x), tag));
     put_rec(e + 1, tagged(__float_as_uint(v.y), tag));
   }
-  if (LOUT == 0 && nterms == 0) {                    // nothing comes in from earlier blocks: y is final
-#pragma unroll
-    for (int i = 0; i < kFCPW; ++i) store_row(wave + kFW * i);
-  }
+  __builtin_amdgcn_s_setprio(0);
 
+  // the operands of phase B's first channel travel under the wait for the earlier blocks
+  bf16x8 Ka[kNWK][2], Ca[kNWC][2];
+  load_kc(wave, Ka, Ca);
+  float Jr[4] = {0.f, 0.f, 0.f, 0.f}, Ji[4] = {0.f, 0.f, 0.f, 0.f};
+  auto load_j = [&](const int c) {
+    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    uint32_t loff = loff0;
+    asm volatile("" : "+v"(loff));
+    load_c4(img, kSlotRJ, loff, Jr, Ji);             // (q^64)^j
+  };
+  load_j(wave);
+
+  // ---- start state of the block: h_start = sum_{d >= 0} (q^1024)^d E_{s-1-d}, E_{-1} being the caller's carried
+  // state (slot S of the row's records).  Lane (j, r) works for channel wave + 16 (j >> 2) and takes the terms
+  // d = (j & 3) + 4 k; the four lanes of a quad add up.
+  float Cr[4] = {0.f, 0.f, 0.f, 0.f}, Ci[4] = {0.f, 0.f, 0.f, 0.f};
   if (nterms > 0) {
-    // ---- start state of the block: h_start = sum_{d >= 0} (q^1024)^d E_{s-1-d} (+ (q^1024)^s h_in).  Lane (j, r)
-    // works for channel wave + 16 (j >> 2) and takes the terms d = (j & 3) + 4 k; the four lanes of a quad add up.
-    // the operands of pass 2's first channel are requested before the wait for the earlier blocks
-    auto load2 = [&](const int c, const int steps, bf16x8 (&Cw)[kNWC][2], float (&Jr)[4], float (&Ji)[4]) {
-      const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
-      uint32_t loff = loff0;
-      asm volatile("" : "+v"(loff));
+    const int cl = wave + kFW * (j >> 2);
+    const int chl = g * kFC + cl;
+    int look = 0;                                  // blocks back that still reach this lane's channel
 #pragma unroll
-      for (int w = 0; w < kNWC; ++w)
+    for (int i = 0; i < kFCPW; ++i) look = (j >> 2) == i ? nlook[i] : look;
+    const char* wimg = (const char*)A.image + (size_t)chl * kImgRowBytes;
+    int maxlook = 0;
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotC + 2 * w + mb, loff));
-      // requested whatever `steps` says (for steps <= 1 the consumer replaces it by 1, q^64, 0): a load under a branch
-      // has to be waited for inside the branch, where its registers are merged with the other path's, and that wait
-      // (vmcnt is in order) would also cover the operand loads above and the previous channel's stores of y
-      (void)steps;
-      load_c4(img, kSlotRJ, loff, Jr, Ji);
-    };
-    bf16x8 Cn[kNWC][2];
-    float Jnr[4] = {0.f, 0.f, 0.f, 0.f}, Jni[4] = {0.f, 0.f, 0.f, 0.f};
-    load2(wave, nsteps[0], Cn, Jnr, Jni);
-    float Cr[4] = {0.f, 0.f, 0.f, 0.f}, Ci[4] = {0.f, 0.f, 0.f, 0.f};
-    {
-      const int cl = wave + kFW * (j >> 2);
-      const int chl = g * kFC + cl;
-      int look = 0;                                  // blocks back that still reach this lane's channel
+    for (int i = 0; i < kFCPW; ++i) maxlook = nlook[i] > maxlook ? nlook[i] : maxlook;
+    const int nrounds = nterms < maxlook ? nterms : maxlook;
+    for (int d0 = 0; d0 < nrounds; d0 += 4) {
+      const int d = d0 + (j & 3);
+      const bool have = d < nterms && d < look;
+      const int slot = have ? (d < s ? s - 1 - d : A.S) : 0;
+      const unsigned long long* e = A.rec + (brow * (A.S + 1) + slot) * kFRecW + 4 + (size_t)cl * kNS * 2 + 4 * r;
+      float Wr[4], Wi[4];
+      load_c4(wimg, kSlotRWJ, (uint32_t)(((r << 4) | (have ? d : 0)) * 16), Wr, Wi);      // (q^1024)^d
+      unsigned long long w[8];
+      uint32_t spins = 0;
+      for (;;) {
+        bool ok = true;
 #pragma unroll
-      for (int i = 0; i < kFCPW; ++i) look = (j >> 2) == i ? nlook[i] : look;
-      const char* wimg = (const char*)A.image + (size_t)chl * kImgRowBytes;
-      int maxlook = 0;
-#pragma unroll
-      for (int i = 0; i < kFCPW; ++i) maxlook = nlook[i] > maxlook ? nlook[i] : maxlook;
-      const int nrounds = nterms < maxlook ? nterms : maxlook;
-      for (int d0 = 0; d0 < nrounds; d0 += 4) {
-        const int d = d0 + (j & 3);
-        const bool have = d < nterms && d < look;
-        const bool from_state = d == s;              // the caller's carried state enters behind block 0
-        const bool from_rec = have && !from_state;
-        const unsigned long long* e =
-            A.rec + (brow * A.S + (from_rec ? s - 1 - d : 0)) * kFRecW + 4 + (size_t)cl * kNS * 2 + 4 * r;
-        float Wr[4], Wi[4];
-        load_c4(wimg, kSlotRWJ, (uint32_t)(((r << 4) | (have ? d : 0)) * 16), Wr, Wi);      // (q^1024)^d
-        unsigned long long w[8];
-        uint32_t spins = 0;
-        for (;;) {
-          bool ok = true;
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {              // states (2r, 2r+1) and (8+2r, 9+2r): two runs of four words
-            w[u] = from_rec ? get_rec(e + u) : tagged(0u, tag);
-            w[4 + u] = from_rec ? get_rec(e + 16 + u) : tagged(0u, tag);
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) ok &= (uint32_t)(w[u] >> 32) == tag;
-          if (__all(ok)) break;
-          if (++spins > A.lb.spin_limit) {
-            poison = true;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(1);
-        }
-        float er[4], ei[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          er[u] = __uint_as_float((uint32_t)w[2 * u]);
-          ei[u] = __uint_as_float((uint32_t)w[2 * u + 1]);
-        }
-        if (have && from_state) {
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            er[u] = ei[u] = 0.f;
-            if (nn[u] < A.N) {
-              const size_t o = (((size_t)b * A.D + chl) * A.N + nn[u]) * 2;
-              er[u] = A.h_in[o];
-              ei[u] = A.is_complex ? A.h_in[o + 1] : 0.f;
-            }
-          }
+        for (int u = 0; u < 4; ++u) {              // states (2r, 2r+1) and (8+2r, 9+2r): two runs of four words
+          w[u] = have ? get_rec(e + u) : tagged(0u, tag);
+          w[4 + u] = have ? get_rec(e + 16 + u) : tagged(0u, tag);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          Cr[u] = fmaf(Wr[u], er[u], fmaf(-Wi[u], ei[u], Cr[u]));
-          Ci[u] = fmaf(Wr[u], ei[u], fmaf(Wi[u], er[u], Ci[u]));
+        for (int u = 0; u < 8; ++u) ok &= (uint32_t)(w[u] >> 32) == tag;
+        if (__all(ok)) break;
+        if (++spins > A.lb.spin_limit) {
+          poison = true;
+          break;
         }
+        __builtin_amdgcn_s_sleep(1);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        Cr[u] = group_sum<4>(Cr[u]);
-        Ci[u] = group_sum<4>(Ci[u]);
-      }
-      if (poison) {
-        Cr[0] = __builtin_nanf("");
-        if (lane == 0) report_give_up(A.hdr, A.lb.status);
+        const float er = __uint_as_float((uint32_t)w[2 * u]), ei = __uint_as_float((uint32_t)w[2 * u + 1]);
+        Cr[u] = fmaf(Wr[u], er, fmaf(-Wi[u], ei, Cr[u]));
+        Ci[u] = fmaf(Wr[u], ei, fmaf(Wi[u], er, Ci[u]));
       }
     }
-    MEGA_FTR(10);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      Cr[u] = group_sum<4>(Cr[u]);
+      Ci[u] = group_sum<4>(Ci[u]);
+    }
+    if (poison) {
+      Cr[0] = __builtin_nanf("");
+      if (lane == 0) report_give_up(A.hdr, A.lb.status);
+    }
+  }
+  // h_start (zero when nothing comes in) is parked over the wave's own end states, which have left; the last block
+  // first returns the state after its last token: end state from a zero start + (q^1024) h_start
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  if (last_block && A.h_out && (j & 3) == 0) {
+    const int cl = wave + kFW * (j >> 2);
+    const int ch = g * kFC + cl;
+    float Rr[4], Ri[4];
+    load_cmp((const char*)A.image + (size_t)ch * kImgRowBytes, kCmpRW, roff0, Rr, Ri);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (nn[u] < A.N) {
+        const float er = s_end[(cl * kNS + nn[u]) * 2], ei = s_end[(cl * kNS + nn[u]) * 2 + 1];
+        const size_t o = (((size_t)b * A.D + ch) * A.N + nn[u]) * 2;
+        A.h_out[o] = fmaf(Rr[u], Cr[u], fmaf(-Ri[u], Ci[u], er));
+        A.h_out[o + 1] = fmaf(Rr[u], Ci[u], fmaf(Ri[u], Cr[u], ei));
+      }
+    }
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  if ((j & 3) == 0) {
+    const int cl = wave + kFW * (j >> 2);
+    *(float4*)(s_end + (cl * kNS + 2 * r) * 2) = make_float4(Cr[0], Ci[0], Cr[1], Ci[1]);
+    *(float4*)(s_end + (cl * kNS + 8 + 2 * r) * 2) = make_float4(Cr[2], Ci[2], Cr[3], Ci[3]);
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+  MEGA_FTR(10);
 
-    // ---- pass 2: add C ((q^64)^j h_start) (one more factor q^32 for a segment's second tile) to y and send it out;
-    // the operands of the next channel travel under the current one
+  // ---- phase B per channel: the segment scan again (cheaper than keeping four channels' scans in registers across
+  // the wait), start state of segment j = what segment j - 1 left + (q^64)^j h_start, then
+  // y_tile = K x_tile + C h (h: the state at the tile's first token, carried into the product as two bf16 terms where
+  // the channel's poles are slow enough for the states to dwarf y; at a segment's second tile h = q^32 h + F), bf16,
+  // back into LDS over x, and out as whole rows.
 #pragma unroll
-    for (int i = 0; i < kFCPW; ++i) {
-      const int c = wave + kFW * i;
-      const int ch = g * kFC + c;
-      const char* img = (const char*)A.image + (size_t)ch * kImgRowBytes;
-      uint32_t roff = roff0;
-      asm volatile("" : "+v"(roff));
-      bf16x8 Cw[kNWC][2];
-      float Qr[4], Qi[4], Jr[4], Ji[4], ar[4], ai[4], br[4], bi[4];
-#pragma unroll
-      for (int w = 0; w < kNWC; ++w)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = Cn[w][mb];
+  for (int i = 0; i < kFCPW; ++i) {
+    const int c = wave + kFW * i;
+    const bool two_terms = nsteps[i] >= 2;           // |q|^128 >= 2^-24 for some state of the channel
+    uint32_t roff = roff0;
+    asm volatile("" : "+v"(roff));
+    char* row = tile + row_base(c) + j * 128;
+    const bf16x8 X0 = *(const bf16x8*)(row + (((r) ^ (j >> 1)) << 4));
+    const bf16x8 X1 = *(const bf16x8*)(row + (((4 + r) ^ (j >> 1)) << 4));
+    float hr[4], hi[4], Fr[4], Fi[4];
+    {
+      float Qr[4], Qi[4];
+      lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
+      segment_scan(c, nsteps[i], Pa, X0, X1, Qr, Qi, hr, hi, Fr, Fi, roff);
+    }
+    MEGA_FTR2(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 1 < kFCPW) load_p(wave + kFW * (i + 1), Pa);
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const float4 b0 = *(const float4*)(s_end + (c * kNS + 2 * r) * 2);
+      const float4 b1 = *(const float4*)(s_end + (c * kNS + 8 + 2 * r) * 2);
+      const float br[4] = {b0.x, b0.z, b1.x, b1.z}, bi[4] = {b0.y, b0.w, b1.y, b1.w};
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        Jr[u] = Jnr[u];
-        Ji[u] = Jni[u];
+        const float sr = dpp_f<0x111>(hr[u]), si = dpp_f<0x111>(hi[u]);
+        hr[u] = fmaf(Jr[u], br[u], fmaf(-Ji[u], bi[u], sr));
+        hi[u] = fmaf(Jr[u], bi[u], fmaf(Ji[u], br[u], si));
       }
-      __builtin_amdgcn_sched_barrier(0);
-      if (i + 1 < kFCPW) load2(wave + kFW * (i + 1), nsteps[i + 1 < kFCPW ? i + 1 : i], Cn, Jnr, Jni);
-      __builtin_amdgcn_sched_barrier(0);
-      lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
-      if (nsteps[i] <= 1) {                          // |q|^128 < 2^-24: the start state reaches two segments
-        float Sr[4], Si[4];
-        lds_cmp(s_tab, kCmpRS, c, roff, Sr, Si);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 1 < kFCPW) load_j(wave + kFW * (i + 1));
+    __builtin_amdgcn_sched_barrier(0);
+    MEGA_FTR2(1);
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      asm volatile("" ::: "memory");              // x again from LDS: cheaper than eight registers across the scan
+      const bf16x8 X = *(const bf16x8*)(row + (((4 * t + r) ^ (j >> 1)) << 4));
+      f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < kNWK; ++w) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ka[w][0], X, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ka[w][1], X, Y1, 0, 0, 0);
+      }
+      bf16x8 Hop;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        Hop[2 * u] = (__bf16)hr[u];
+        Hop[2 * u + 1] = (__bf16)hi[u];
+      }
+#pragma unroll
+      for (int w = 0; w < kNWC; ++w) {
+        Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ca[w][0], Hop, Y0, 0, 0, 0);
+        Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ca[w][1], Hop, Y1, 0, 0, 0);
+      }
+      if (two_terms) {
+        bf16x8 Hlo;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          Jr[u] = j == 0 ? 1.f : (j == 1 ? Sr[u] : 0.f);
-          Ji[u] = j == 1 ? Si[u] : 0.f;
+          Hlo[2 * u] = (__bf16)(hr[u] - (float)Hop[2 * u]);
+          Hlo[2 * u + 1] = (__bf16)(hi[u] - (float)Hop[2 * u + 1]);
         }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {                  // the quad i of every row holds this channel's start state
-        br[u] = lane_bcast(Cr[u], (lane & 48) | (4 * i));
-        bi[u] = lane_bcast(Ci[u], (lane & 48) | (4 * i));
-        ar[u] = Jr[u] * br[u] - Ji[u] * bi[u];
-        ai[u] = Jr[u] * bi[u] + Ji[u] * br[u];
-      }
-      char* row = tile + row_base(c) + j * 128;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        bf16x8 Hop;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          Hop[2 * u] = (__bf16)ar[u];
-          Hop[2 * u + 1] = (__bf16)ai[u];
-        }
-        f32x4 Y0 = {0.f, 0.f, 0.f, 0.f}, Y1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int w = 0; w < kNWC; ++w) {
-          Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop, Y0, 0, 0, 0);
-          Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop, Y1, 0, 0, 0);
+          Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ca[w][0], Hlo, Y0, 0, 0, 0);
+          Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Ca[w][1], Hlo, Y1, 0, 0, 0);
         }
-        if (t == 0) {
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const float nr = Qr[u] * ar[u] - Qi[u] * ai[u];
-            ai[u] = Qr[u] * ai[u] + Qi[u] * ar[u];
-            ar[u] = nr;
-          }
-        }
-        uint2* p0 = (uint2*)(row + (((4 * t + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8);
-        uint2* p1 = (uint2*)(row + (((4 * t + 2 + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8);
-        const uint2 a0 = *p0, a1 = *p1;
-        *p0 = make_uint2(pack_bf16(Y0[0] + __uint_as_float(a0.x << 16), Y0[1] + __uint_as_float(a0.x & 0xffff0000u)),
-                         pack_bf16(Y0[2] + __uint_as_float(a0.y << 16), Y0[3] + __uint_as_float(a0.y & 0xffff0000u)));
-        *p1 = make_uint2(pack_bf16(Y1[0] + __uint_as_float(a1.x << 16), Y1[1] + __uint_as_float(a1.x & 0xffff0000u)),
-                         pack_bf16(Y1[2] + __uint_as_float(a1.y << 16), Y1[3] + __uint_as_float(a1.y & 0xffff0000u)));
       }
-      if (last_block && A.h_out && j == 15) {
-        // state after the block's last token: end state from a zero start + (q^1024) h_start
-        float Rr[4], Ri[4];
-        load_cmp(img, kCmpRW, roff, Rr, Ri);
+      if (t == 0) {
+        float Qr[4], Qi[4];
+        lds_cmp(s_tab, kCmpQ32, c, roff, Qr, Qi);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          if (nn[u] < A.N) {
-            const float er = s_end[(c * kNS + nn[u]) * 2], ei = s_end[(c * kNS + nn[u]) * 2 + 1];
-            const size_t o = (((size_t)b * A.D + ch) * A.N + nn[u]) * 2;
-            A.h_out[o] = fmaf(Rr[u], br[u], fmaf(-Ri[u], bi[u], er));
-            A.h_out[o + 1] = fmaf(Rr[u], bi[u], fmaf(Ri[u], br[u], ei));
-          }
+          const float nr = fmaf(Qr[u], hr[u], fmaf(-Qi[u], hi[u], Fr[u]));
+          hi[u] = fmaf(Qr[u], hi[u], fmaf(Qi[u], hr[u], Fi[u]));
+          hr[u] = nr;
         }
       }
-      if (LOUT == 0) store_row(c);
-      __builtin_amdgcn_sched_barrier(0);
-      MEGA_FTR(11 + i);
+      // y (bf16) over x: tokens 32 t + 4 r + {0..3} and 32 t + 16 + 4 r + {0..3} of segment j
+      *(uint2*)(row + (((4 * t + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) =
+          make_uint2(pack_bf16(Y0[0], Y0[1]), pack_bf16(Y0[2], Y0[3]));
+      *(uint2*)(row + (((4 * t + 2 + (r >> 1)) ^ (j >> 1)) << 4) + (r & 1) * 8) =
+          make_uint2(pack_bf16(Y1[0], Y1[1]), pack_bf16(Y1[2], Y1[3]));
+      MEGA_FTR2(2 + t);
     }
-  } else if (last_block && A.h_out && j == 15) {
-    // a single block without a carried state: its end state from a zero start is the state to return
-#pragma unroll
-    for (int i = 0; i < kFCPW; ++i) {
-      const int c = wave + kFW * i;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (nn[u] < A.N) {
-          const size_t o = (((size_t)b * A.D + g * kFC + c) * A.N + nn[u]) * 2;
-          A.h_out[o] = s_end[(c * kNS + nn[u]) * 2];
-          A.h_out[o + 1] = s_end[(c * kNS + nn[u]) * 2 + 1];
-        }
-      }
-    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (i + 1 < kFCPW) load_kc(wave + kFW * (i + 1), Ka, Ca);
+    __builtin_amdgcn_sched_barrier(0);
+    MEGA_FTR2(4);
+    if (LOUT == 0) store_row(c);
+    __builtin_amdgcn_sched_barrier(0);
+    MEGA_FTR(11 + i);
   }
   if (LOUT == 1) {
     // [B, L, D]: the inverse of the staging step, whole lines of 64 channels per token
@@ -834,7 +806,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 }
 
 size_t fused_ws_bytes(int64_t B, int64_t G, int64_t S) {
-  return align_up(sizeof(TsnHeader), 256) + align_up((size_t)B * G * S * kFRecW * 8, 256);
+  return align_up(sizeof(TsnHeader), 256) + align_up((size_t)B * G * (S + 1) * kFRecW * 8, 256);
 }
 
 bool fused_covers(int dtype, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N, const void* x, const void* xn,
