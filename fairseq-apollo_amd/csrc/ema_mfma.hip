@@ -36,6 +36,9 @@
 #define MEGA_TR_FLUSH()
 #endif
 
+#ifndef MEGA_TWO_ALWAYS
+#define MEGA_TWO_ALWAYS 0
+#endif
 namespace mega {
 namespace {
 
@@ -361,7 +364,8 @@ struct Geo {
   static constexpr int XBUF = ROWB * kWaves;
   static constexpr int SCANJ = 20;                 // complex slots per segment in the scan buffer (16 + 4 pad)
   static constexpr int SCANB = 16 * SCANJ * 8;     // segment states per channel
-  static constexpr int TOTAL = XBUF + kWaves * SCANB;
+  static constexpr int QTAB = XBUF + kWaves * SCANB;   // q^32 of every wave's channel: [kWaves][4 row blocks][4 states] complex
+  static constexpr int TOTAL = QTAB + kWaves * 128;
   static_assert((ROWB / 4) % 16 == 4, "row stride must spread the four rows of a store over the banks");
   __device__ static __forceinline__ int pos(int t) { return (t / SEG) * SEGB + (t % SEG) * 2; }
 };
@@ -484,10 +488,11 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
 
   // ---- operand images of this channel: registers for the whole kernel
   bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
-  float Qr[4], Qi[4];
+  char* const qtab = smem + G::QTAB + wave * 128;
   // segment scan: lane (n = lane >> 2, c = lane & 3) owns state n over segments 4c .. 4c+3
   float Rr, Ri;                        // q^(32 SEGT) of state n: the scan's multiplier
   float Hcr = 0.f, Hci = 0.f;          // carried state of state n, in the lanes with c == 0 (zero elsewhere)
+  bool two_terms = false;              // the states enter the output product as two bf16 terms (wave-uniform)
   {
     const uint4* img = A.image + (size_t)(A.koff + chc) * kImgSlots * 64 + lane;
     int slot = 0;
@@ -504,12 +509,18 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) Cw[w][mb] = __builtin_bit_cast(bf16x8, img[(slot++) * 64]);
     const uint4 qa = img[(slot++) * 64], qb = img[(slot++) * 64], rr = img[(slot++) * 64];
-    Qr[0] = __uint_as_float(qa.x); Qi[0] = __uint_as_float(qa.y);
-    Qr[1] = __uint_as_float(qa.z); Qi[1] = __uint_as_float(qa.w);
-    Qr[2] = __uint_as_float(qb.x); Qi[2] = __uint_as_float(qb.y);
-    Qr[3] = __uint_as_float(qb.z); Qi[3] = __uint_as_float(qb.w);
+    // q^32 of the lane's four states waits in LDS between uses (eight registers less across the streaming loop);
+    // only the wave itself reads its table
+    if (j == 0) {
+      *(uint4*)(qtab + r * 32) = qa;
+      *(uint4*)(qtab + r * 32 + 16) = qb;
+    }
     Rr = __uint_as_float(rr.x);
     Ri = __uint_as_float(rr.y);
+    // reach word of the image: |q|^128 >= 2^-24 for some state of the channel
+    two_terms = __builtin_amdgcn_readfirstlane(
+                    (int)*(const uint32_t*)((const char*)(A.image + (size_t)(A.koff + chc) * kImgSlots * 64) +
+                                            kSlotCmp * 1024 + kCmpReach * 128)) >= 2;
     if (A.h_in && (lane & 3) == 0 && (lane >> 2) < A.N && ch_ok) {
       const size_t o = (((size_t)b * A.D + ch) * A.N + (lane >> 2)) * 2;
       Hcr = A.h_in[o];
@@ -534,8 +545,6 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     for (int w = 0; w < kNWP; ++w) { pin(Pw[w][0]); pin(Pw[w][1]); }
 #pragma unroll
     for (int w = 0; w < kNWC; ++w) { pin(Cw[w][0]); pin(Cw[w][1]); }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(Qr[u]), "+v"(Qi[u]));
     asm volatile("" : "+v"(Rr), "+v"(Ri), "+v"(Hcr), "+v"(Hci));
   }
 
@@ -574,6 +583,14 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     MEGA_TR(6 + sc * 9);
 
     // ---- sweep 1: segment end states from a zero start
+    float Qr[4], Qi[4];
+    auto load_q = [&]() {
+      asm volatile("" ::: "memory");
+      const float4 qa = *(const float4*)(qtab + r * 32), qb = *(const float4*)(qtab + r * 32 + 16);
+      Qr[0] = qa.x; Qi[0] = qa.y; Qr[1] = qa.z; Qi[1] = qa.w;
+      Qr[2] = qb.x; Qi[2] = qb.y; Qr[3] = qb.z; Qi[3] = qb.w;
+    };
+    load_q();
     float Er[4] = {0.f, 0.f, 0.f, 0.f}, Ei[4] = {0.f, 0.f, 0.f, 0.f};
     const char* xcol = xrow + j * G::SEGB + r * 16;
 #pragma unroll
@@ -678,6 +695,7 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
     MEGA_TR(8 + sc * 9);
     // ---- sweep 2: outputs
+    load_q();
     char* ycol = xrow + j * G::SEGB;
 #pragma unroll
     for (int i = 0; i < kSEGT; ++i) {
@@ -704,6 +722,20 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
       for (int w = 0; w < kNWK; ++w) {
         Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][0], X, Y0, 0, 0, 0);
         Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][1], X, Y1, 0, 0, 0);
+      }
+      if (MEGA_TWO_ALWAYS || two_terms) {
+        // slow poles: the states dwarf y and cancel in the sum over the states, so what bf16 drops of them is carried
+        // into the product as a second term
+        {
+          const float hv[8] = {Hr[0], Hi[0], Hr[1], Hi[1], Hr[2], Hi[2], Hr[3], Hi[3]};
+#pragma unroll
+          for (int t = 0; t < 8; ++t) Hop[t] = (__bf16)(hv[t] - (float)Hop[t]);      // in place: no second register set
+        }
+#pragma unroll
+        for (int w = 0; w < kNWC; ++w) {
+          Y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][0], Hop, Y0, 0, 0, 0);
+          Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Cw[w][1], Hop, Y1, 0, 0, 0);
+        }
       }
       const float sr[4] = {S0[0], S0[2], S1[0], S1[2]};
       const float si[4] = {S0[1], S0[3], S1[1], S1[3]};

@@ -147,15 +147,16 @@ def test_slowly_decaying_poles_across_blocks(mixed):
     layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
     xn, y, _, _, _, h = _run(layer, x, G, np.zeros(D), np.zeros(D), want_state=True)
     yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, incremental=True)
-    # With poles this close to 1 the states are two orders of magnitude above y and enter y through bf16
-    # operands: the worst element of 5e5 sits at 2.1e-2 (2.5e-2 in the mixed case) for this kernel and for the
-    # moving-average kernel alike (same data: 2.07e-2 / 2.2e-2), the rms error at 3e-3 of rms(y).
-    _check_y(y, yo, tol=3e-2)
+    # With poles this close to 1 the states are two orders of magnitude above y and cancel in the sum over the
+    # states; both kernels carry them into the output product as two bf16 terms (one term left the worst element of
+    # 5e5 at 2.1e-2, 2.5e-2 in the mixed case; two terms: 1.3e-2 / 1.7e-2), the rms error is 2.3e-3 of rms(y).
+    _check_y(y, yo, tol=2e-2)
     e = host(y) - yo
-    assert np.sqrt(np.mean(e ** 2)) < 4e-3 * np.sqrt(np.mean(yo ** 2))
+    assert np.sqrt(np.mean(e ** 2)) < 3e-3 * np.sqrt(np.mean(yo ** 2))
     y2, _ = layer(xn.transpose(1, 2))
     torch.cuda.synchronize()
-    assert rel_err(host(y), host(y2)) < 4e-2          # two independent errors of that size
+    assert rel_err(host(y2), yo) < 2e-2
+    assert rel_err(host(y), host(y2)) < 2e-2
     assert rel_err(np.real(host(h)), np.real(ho)) < 2e-3
 
 
