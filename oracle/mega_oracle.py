@@ -18,9 +18,23 @@ place, where that build exists).  Pin status per function:
   ema_forward / ema_one_step             chunk-split invariance, step-vs-parallel equality
   timestep_norm (group / per feature)    numpy.mean/var on prefixes, oracle/_ref
   attention_softmax / attention          explicit masked softmax, rows sum to 1
-  swiglu / silu_ffn / rotary / gated_attention_layer
-                                         closed forms only; SwiGLU and multi-head are not
-                                         in the reference: parity unpinned (spec only)
+  rotary / simple_relative_bias          the reference modules' own outputs
+                                         (tests/golden/position_vectors.npz, written from
+                                         fairseq/modules/relative_positional_bias.py)
+  swiglu / rms_norm                      silu identities and known values, rms of constant
+                                         vectors, scale invariance, torch's F.silu / F.rms_norm
+  swiglu_ffn / silu_ffn                  per-row loops, identity and one-hot weights
+  gated_attention_layer                  MovingAverageGatedAttention.forward restated with the
+                                         library calls the reference makes (torch.split,
+                                         F.normalize, F.softmax, ...) over the pinned primitives,
+                                         all branches (rms / relu2 / laplace / simple bias /
+                                         two-sided / padding), and closed-form special cases
+                                         (gamma = -1: running means of v; W_h = 0; z under the
+                                         normalize clamp; one-hot mx_proj rows)
+                                         (tests/test_oracle_layer.py)
+The SwiGLU feed-forward block and the multi-head split of the gated attention are north-star
+specification, not reference code (the reference FFN is the SiLU block, its layer single-head):
+their formulas are pinned as above, their parity with the reference is unpinned by construction.
 """
 from __future__ import annotations
 
@@ -672,7 +686,7 @@ def attention_bwd(dy, q, k, v, scale: float = 1.0, causal: bool = True, drop=Non
 
 def swiglu(a, b):
     """silu(a) * b -- the gate of the north-star SwiGLU FFN; not present in the
-    reference (its FFN is normalized_feedforward_network.py:77-93): parity unpinned."""
+    reference (its FFN is normalized_feedforward_network.py:77-93): specification only."""
     a = np.asarray(a, np.float64)
     return _silu(a) * np.asarray(b, np.float64)
 
@@ -689,19 +703,33 @@ def silu_ffn(x, w1, b1, w2, b2):
     return x + _silu(x @ np.asarray(w1, np.float64).T + b1) @ np.asarray(w2, np.float64).T + b2
 
 
-def rotary(x, base: float = 10000.0):
-    """modules/relative_positional_bias.py:57-88 (RotaryRelativePositionalBias):
+def rotary(x, base: float = 10000.0, start: int = 0):
+    """modules/relative_positional_bias.py:46-94 (RotaryEmbedding):
     x: [..., L, S]; features (2i, 2i+1) form one complex number that is multiplied by
-    exp(i t base^{-2i/S}) for position t (positions start at 0)."""
+    exp(i t base^{-2i/S}) for position t = start, start + 1, ... (`start`: the reference's `qidx`, the place of
+    a single query behind cached keys, :89-92).  Pinned by the reference module's own outputs
+    (tests/golden/position_vectors.npz)."""
     x = np.asarray(x, np.float64)
     L, S = x.shape[-2], x.shape[-1]
     freq = 1.0 / (base ** (np.arange(0, S, 2) / S))
-    ang = np.arange(L)[:, None] * freq[None, :]
+    ang = (start + np.arange(L))[:, None] * freq[None, :]
     z = (x[..., 0::2] + 1j * x[..., 1::2]) * np.exp(1j * ang)
     out = np.empty_like(x)
     out[..., 0::2] = z.real
     out[..., 1::2] = z.imag
     return out
+
+
+def simple_relative_bias(param, C: int):
+    """modules/relative_positional_bias.py:13-42 (SimpleRelativePositionalBias.forward): the [C, C] matrix added to
+    q k^T, entry (i, j) = param[max_positions - 1 + j - i] for the 2 max_positions - 1 learned offsets.  Pinned by
+    the reference module's own outputs (tests/golden/position_vectors.npz)."""
+    sb = np.asarray(param, np.float64)
+    mp = (sb.shape[0] + 1) // 2
+    if C > mp:
+        raise ValueError(f"sequence length {C} beyond max length {mp}")
+    pos = np.arange(C)
+    return sb[(mp - 1) + pos[None, :] - pos[:, None]]
 
 
 def rms_norm(x, weight=None, eps: float = 1e-5):
@@ -773,10 +801,7 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
         else:
             sc = sc / np.sqrt(C)
         if simple_bias is not None:
-            sb = np.asarray(simple_bias, np.float64)
-            mp = (sb.shape[0] + 1) // 2
-            pos = np.arange(C)
-            sc = sc + sb[(mp - 1) + pos[None, :] - pos[:, None]]
+            sc = sc + simple_relative_bias(simple_bias, C)
         w = np.maximum(sc, 0.0) ** 2 if attention_activation == 'relu2' else _sigmoid((sc - 0.707107) * (1.702 / 0.282095))
         if pad is not None:
             w = w * (~pad)[:, None, None, :]
@@ -789,10 +814,7 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
         # excluded unless the whole chunk is padding, causal for one-sided layers
         sc = np.einsum('blnh,bmnh->bnlm', qr, kr)
         if simple_bias is not None:
-            sb = np.asarray(simple_bias, np.float64)
-            mp = (sb.shape[0] + 1) // 2
-            pos = np.arange(C)
-            sc = sc + sb[(mp - 1) + pos[None, :] - pos[:, None]]
+            sc = sc + simple_relative_bias(simple_bias, C)
         if bidirectional and padding_mask is not None:
             pad = np.asarray(padding_mask, bool).reshape(B * nc, C)
             pad = pad & ~pad.all(-1, keepdims=True)
