@@ -24,6 +24,7 @@ _sz = C.c_size_t
 SIGNATURES = {
     "mega_last_error": (C.c_char_p, []),
     "mega_abi_version": (_int, []),
+    "mega_lookback_init": (_int, []),
     "mega_lookback_status": (_int, [_int]),
     "mega_test_lookback": (None, [C.c_uint, _int, _int]),
     "mega_ema_parameters_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _p, _p]),

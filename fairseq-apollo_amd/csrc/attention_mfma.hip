@@ -385,10 +385,9 @@ void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hi
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr int smem = 2 * (TM + TN) * PITCH;
   auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT, EPI>;
-  static bool attr_set = false;
-  if (!attr_set && smem > 64 * 1024) {
+  static uint64_t attr_seen = 0;
+  if (smem > 64 * 1024 && first_on_device(&attr_seen)) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    attr_set = true;
   }
   G.xcd = xcd ? 1 : 0;
   G.mt = (int)ceil_div(M, TM);
@@ -1067,10 +1066,9 @@ void launch_flash(const void* q, const void* k, const void* v, void* y, int64_t 
 #define MEGA_FLASH(KS_)                                                                                       \
   {                                                                                                           \
     auto kern = flash_fwd_kernel<T, KS_, fqb, fbd>;                                                           \
-    static bool attr_set = false;                                                                             \
-    if (!attr_set) {                                                                                          \
+    static uint64_t attr_seen = 0;                                                                            \
+    if (first_on_device(&attr_seen)) {                                                                        \
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);    \
-      attr_set = true;                                                                                        \
     }                                                                                                         \
     hipLaunchKernelGGL(kern, grid, dim3(64 * FNW), smem, s, F);                                               \
   }

@@ -14,7 +14,7 @@ void set_error(const char* fmt, ...) {
 }  // namespace mega
 
 extern "C" const char* mega_last_error(void) { return mega::g_err; }
-extern "C" int mega_abi_version(void) { return 2; }
+extern "C" int mega_abi_version(void) { return 3; }
 
 // ------------------------------------------------------------------------------------------------
 // Status of the bounded waits.  One word of pinned, device-mapped host memory per device: a kernel that
@@ -89,6 +89,16 @@ int lookback_pending(const char* entry) {
   return MEGA_ERR_LAUNCH;
 }
 }  // namespace mega
+
+extern "C" int mega_lookback_init(void) {
+  auto& s = mega::slot_of(mega::current_slot(), true);
+  if (!s.dev) {
+    mega::set_error("lookback_init: the status word of device %d could not be created (pinned, device-mapped host "
+                    "memory refused)", mega::current_slot());
+    return MEGA_ERR_LAUNCH;
+  }
+  return MEGA_OK;
+}
 
 extern "C" int mega_lookback_status(int clear) {
   auto& s = mega::slot_of(mega::current_slot(), false);

@@ -45,6 +45,18 @@ int lookback_pending(const char* entry);
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Function attributes (the dynamic shared memory limit of a kernel) belong to a device: a call site sets them the
+// first time it launches on each device.  `seen` is the call site's own mask of devices.
+static inline bool first_on_device(uint64_t* seen) {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) {
+    (void)hipGetLastError();
+    d = 0;
+  }
+  const uint64_t bit = 1ull << (d & 63);
+  return !(__atomic_fetch_or(seen, bit, __ATOMIC_RELAXED) & bit);
+}
+
 // Clears `bytes` (a multiple of 4) with a small kernel (elementwise.hip).  Used instead of a memset
 // node so that a caller may record any entry point into a HIP graph.
 void zero_async(void* p, size_t bytes, hipStream_t s);

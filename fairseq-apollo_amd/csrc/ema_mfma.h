@@ -47,10 +47,17 @@ constexpr size_t kImgRowBytes = (size_t)kImgSlots * 64 * 16;
 // bytes of the per-channel operand images for a layer (0: the layer is outside the fast path)
 size_t ema_image_bytes(int64_t D, int64_t N, int bidirectional);
 
-// kernel generation: coefficients -> operand images.  parts: 1 = the bf16 K / P / C operands, 2 = the fp16 ones, 3 =
-// both (an image that is kept and may serve any activation type); a call that generates the image for itself asks
-// for the operands its own kernel reads
-constexpr int kImgBf16 = 1, kImgF16 = 2, kImgAll = 3;
+// kernel generation: coefficients -> operand images.  `parts` says which slots are formed and written (the compact
+// per-state tables and the reach line always are): an image that is kept serves any kernel (kImgAll); a call that
+// generates the image for itself asks for what its own kernel reads
+constexpr int kImgKFull = 1;     // the bf16 K operand, one vector per lane (streaming and row kernels)
+constexpr int kImgF16 = 2;       // K, P, C as two fp16 terms (row kernel on fp32 / fp16 activations)
+constexpr int kImgPC = 4;        // the bf16 P and C operands
+constexpr int kImgStream = 8;    // q^32 and the scan multiplier in the streaming kernel's lane layouts
+constexpr int kImgBlocks = 16;   // (q^64)^j and (q^1024)^j (kernels that work on blocks of 1024 tokens)
+constexpr int kImgKT = 32;       // the bf16 K operand once per distinct vector (one-kernel norm -> moving average)
+constexpr int kImgBf16 = kImgKFull | kImgPC;
+constexpr int kImgAll = 63;
 int ema_image_build(const float* p, const float* q, const float* gamma, int is_complex, const float* omega, int64_t D,
                     int64_t N, int bidirectional, int shift, void* image, hipStream_t s, int parts = kImgAll);
 

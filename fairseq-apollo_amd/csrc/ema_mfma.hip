@@ -149,120 +149,140 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
   __syncthreads();
   uint4* img = A.image + (size_t)kr * kImgSlots * 64;
   const int m = lane & 15, g = lane >> 4;
-  int slot = 0;
-  bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
-  typedef __attribute__((ext_vector_type(8))) _Float16 f16x8v;
-  f16x8v H16[3][2][2];                    // K, P, C as two fp16 terms
+  if (!ok) return;                                 // (no barrier follows)
+  // ---- the K / P / C operands in the matrix-core A layout: bf16 terms (kImgKFull: K, kImgPC: P and C) and fp16 terms
+  // (kImgF16); only what the caller's kernel reads is formed and written
+  const bool want_k = A.parts & kImgKFull, want_pc = A.parts & kImgPC, want_16 = A.parts & kImgF16;
+  if (want_k || want_pc || want_16) {
+    bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
+    typedef __attribute__((ext_vector_type(8))) _Float16 f16x8v;
+    f16x8v H16[3][2][2];                    // K, P, C as two fp16 terms
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) {
-    const int row = 16 * mb + m;
+    for (int mb = 0; mb < 2; ++mb) {
+      const int row = 16 * mb + m;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const int k = 8 * g + t;
-      // K: rows = output time, k = input time (Toeplitz)
-      const float kv = kkt[32 + row - k];
-      // P: rows = (state, part), k = input time i: p q^{31-i}
-      float pv;
-      {
-        const int n = row >> 1, part = row & 1;
-        const float2 w = pw[(31 - k) * kNS + n];
-        pv = pbuf[n] * (part ? w.y : w.x);
-      }
-      // C: rows = output time i; k-slot t of block g <-> state 2g + t/2 (t < 4) or 8 + 2g + (t-4)/2,
-      // part t & 1: Re(gamma q^{i+1-lag}) multiplies Re h, -Im(...) multiplies Im h
-      float cv;
-      {
-        const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
-        const int part = t & 1;
-        const float2 w = pw[(row + 1 - lag) * kNS + n];
-        const float2 gm = gbuf[n];
-        const float re = gm.x * w.x - gm.y * w.y;
-        const float im = gm.x * w.y + gm.y * w.x;
-        cv = part ? -im : re;
-      }
-      __bf16 h;
-      float rem = bf_split(kv, &h);
-      Kw[0][mb][t] = h;
-      if (kNWK > 1) Kw[kNWK - 1][mb][t] = (__bf16)rem;
-      rem = bf_split(pv, &h);
-      Pw[0][mb][t] = h;
-      if (kNWP > 1) Pw[kNWP - 1][mb][t] = (__bf16)rem;
-      rem = bf_split(cv, &h);
-      Cw[0][mb][t] = h;
-      if (kNWC > 1) Cw[kNWC - 1][mb][t] = (__bf16)rem;
-      {
-        const float vals[3] = {kv, pv, cv};
+      for (int t = 0; t < 8; ++t) {
+        const int k = 8 * g + t;
+        // K: rows = output time, k = input time (Toeplitz)
+        const float kv = kkt[32 + row - k];
+        // P: rows = (state, part), k = input time i: p q^{31-i}
+        float pv;
+        {
+          const int n = row >> 1, part = row & 1;
+          const float2 w = pw[(31 - k) * kNS + n];
+          pv = pbuf[n] * (part ? w.y : w.x);
+        }
+        // C: rows = output time i; k-slot t of block g <-> state 2g + t/2 (t < 4) or 8 + 2g + (t-4)/2,
+        // part t & 1: Re(gamma q^{i+1-lag}) multiplies Re h, -Im(...) multiplies Im h
+        float cv;
+        {
+          const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
+          const int part = t & 1;
+          const float2 w = pw[(row + 1 - lag) * kNS + n];
+          const float2 gm = gbuf[n];
+          const float re = gm.x * w.x - gm.y * w.y;
+          const float im = gm.x * w.y + gm.y * w.x;
+          cv = part ? -im : re;
+        }
+        __bf16 h;
+        float rem = bf_split(kv, &h);
+        Kw[0][mb][t] = h;
+        if (kNWK > 1) Kw[kNWK - 1][mb][t] = (__bf16)rem;
+        rem = bf_split(pv, &h);
+        Pw[0][mb][t] = h;
+        if (kNWP > 1) Pw[kNWP - 1][mb][t] = (__bf16)rem;
+        rem = bf_split(cv, &h);
+        Cw[0][mb][t] = h;
+        if (kNWC > 1) Cw[kNWC - 1][mb][t] = (__bf16)rem;
+        {
+          const float vals[3] = {kv, pv, cv};
 #pragma unroll
-        for (int o = 0; o < 3; ++o) {
-          const _Float16 h16 = (_Float16)vals[o];
-          H16[o][0][mb][t] = h16;
-          H16[o][1][mb][t] = (_Float16)(vals[o] - (float)h16);
+          for (int o = 0; o < 3; ++o) {
+            const _Float16 h16 = (_Float16)vals[o];
+            H16[o][0][mb][t] = h16;
+            H16[o][1][mb][t] = (_Float16)(vals[o] - (float)h16);
+          }
         }
       }
     }
-  }
-  if (ok) {
-    if (A.parts & 1) {
+    if (want_k) {
 #pragma unroll
       for (int w = 0; w < kNWK; ++w)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
+        for (int mb = 0; mb < 2; ++mb) img[(kSlotK + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
+    }
+    if (want_pc) {
 #pragma unroll
       for (int w = 0; w < kNWP; ++w)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
+        for (int mb = 0; mb < 2; ++mb) img[(kSlotP + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
 #pragma unroll
       for (int w = 0; w < kNWC; ++w)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(slot++) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
-    } else {
-      slot += 2 * (kNWK + kNWP + kNWC);
+        for (int mb = 0; mb < 2; ++mb) img[(kSlotC + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
     }
+    if (want_16) {
+#pragma unroll
+      for (int o = 0; o < 3; ++o)
+#pragma unroll
+        for (int w = 0; w < 2; ++w)
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+            img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
+    }
+  }
+  if (A.parts & kImgStream) {
     // q^32 of this lane's four states (2r, 2r+1, 8+2r, 9+2r)
     const float2 a = pw[32 * kNS + 2 * r], bq = pw[32 * kNS + 2 * r + 1];
     const float2 c = pw[32 * kNS + 8 + 2 * r], d = pw[32 * kNS + 9 + 2 * r];
-    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(a.x), __float_as_uint(a.y), __float_as_uint(bq.x),
+    img[kSlotQ32 * 64 + lane] = make_uint4(__float_as_uint(a.x), __float_as_uint(a.y), __float_as_uint(bq.x),
                                            __float_as_uint(bq.y));
-    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(c.x), __float_as_uint(c.y), __float_as_uint(d.x),
-                                           __float_as_uint(d.y));
+    img[(kSlotQ32 + 1) * 64 + lane] = make_uint4(__float_as_uint(c.x), __float_as_uint(c.y), __float_as_uint(d.x),
+                                                 __float_as_uint(d.y));
     // scan multiplier q^(32 SEGT) of state `lane >> 2`
     cdouble Rd = {1.0, 0.0};
     const double2 w = q32d[lane >> 2];
     for (int t = 0; t < kSEGT; ++t) Rd = cmuld(Rd, cdouble{w.x, w.y});
     const cfloat R = to_cfloat(Rd);
-    img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
+    img[kSlotScan * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
+  }
+  if (A.parts & kImgBlocks) {
     // multipliers in the matrix-core lane layout (lane = segment j + 16 r, states 2r, 2r+1, 8+2r, 9+2r), for the
-    // kernel that scans 16 segments of 64 tokens across the lanes of a row: per state q^64, (q^64)^j,
-    // (q^64)^16 = q^1024 (the step from one 1024-token block to the next) and (q^1024)^j
+    // kernels that scan 16 segments of 64 tokens across the lanes of a row and look back over blocks of 1024 tokens:
+    // (q^64)^j and (q^1024)^j, each power by squaring and multiplying (at most eight products in a row)
     const int nn[4] = {2 * r, 2 * r + 1, 8 + 2 * r, 9 + 2 * r};
-    cfloat RS[4], RJ[4], RW[4], RWJ[4];
+    cfloat RJ[4], RWJ[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const double2 w32 = q32d[nn[u]];
-      const cdouble rs = cmuld(cdouble{w32.x, w32.y}, cdouble{w32.x, w32.y});
-      RS[u] = to_cfloat(rs);
+      cdouble sq = cmuld(cdouble{w32.x, w32.y}, cdouble{w32.x, w32.y});          // q^64
       cdouble a = {1.0, 0.0};
-      for (int t = 0; t < (lane & 15); ++t) a = cmuld(a, rs);
-      RJ[u] = to_cfloat(a);
-      cdouble w = rs;
-      for (int t = 0; t < 4; ++t) w = cmuld(w, w);
-      RW[u] = to_cfloat(w);
+#pragma unroll
+      for (int bit = 0; bit < 4; ++bit) {
+        if (m & (1 << bit)) a = cmuld(a, sq);
+        sq = cmuld(sq, sq);
+      }
+      RJ[u] = to_cfloat(a);                                                       // sq = q^1024 now
       cdouble c = {1.0, 0.0};
-      for (int t = 0; t < (lane & 15); ++t) c = cmuld(c, w);
+#pragma unroll
+      for (int bit = 0; bit < 4; ++bit) {
+        if (m & (1 << bit)) c = cmuld(c, sq);
+        sq = cmuld(sq, sq);
+      }
       RWJ[u] = to_cfloat(c);
     }
-    auto put2 = [&](const cfloat (&v)[4]) {
-      img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(v[0].re), __float_as_uint(v[0].im),
-                                             __float_as_uint(v[1].re), __float_as_uint(v[1].im));
-      img[(slot++) * 64 + lane] = make_uint4(__float_as_uint(v[2].re), __float_as_uint(v[2].im),
-                                             __float_as_uint(v[3].re), __float_as_uint(v[3].im));
+    auto put2 = [&](const int slot, const cfloat (&v)[4]) {
+      img[slot * 64 + lane] = make_uint4(__float_as_uint(v[0].re), __float_as_uint(v[0].im),
+                                         __float_as_uint(v[1].re), __float_as_uint(v[1].im));
+      img[(slot + 1) * 64 + lane] = make_uint4(__float_as_uint(v[2].re), __float_as_uint(v[2].im),
+                                               __float_as_uint(v[3].re), __float_as_uint(v[3].im));
     };
-    put2(RS);
-    put2(RJ);
-    put2(RW);
-    put2(RWJ);
+    put2(kSlotRJ, RJ);
+    put2(kSlotRWJ, RWJ);
+  }
+  {
     if (lane < kNS) {
-      // the same multipliers once per state (a lane of the streaming kernels reads 16 bytes = two states)
+      // the per-state multipliers once per state (a lane of the streaming kernels reads 16 bytes = two states)
       float2* cmp = (float2*)(img + (size_t)kSlotCmp * 64);
       const double2 w32 = q32d[lane];
       cdouble v = {w32.x, w32.y};
@@ -278,16 +298,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       v = cmuld(v, v);
       cmp[kCmpRW * kNS + lane] = make_float2((float)v.re, (float)v.im);
     }
-    if (A.parts & 2) {
-#pragma unroll
-      for (int o = 0; o < 3; ++o)
-#pragma unroll
-        for (int w = 0; w < 2; ++w)
-#pragma unroll
-          for (int mb = 0; mb < 2; ++mb)
-            img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
-    }
-    if (lane < 56 && (A.parts & 1)) {
+    if (lane < 56 && (A.parts & kImgKT)) {
       // the K operand once per distinct content: lane (m, g) of row block mb holds k[16 mb + m - 8 g - t], t = 0..7,
       // which depends on delta = 16 mb + m - 8 g (-24..31) only; vector delta + 24 of term w sits at byte
       // 16 (delta + 24) of slot kSlotKT + w (7 lines per term instead of 16)
@@ -986,13 +997,12 @@ int ema_mfma_try(const void* x, void* y, int dtype, int64_t sxb, int64_t sxd, in
         ema_mfma_kernel<0, 1, 0>, ema_mfma_kernel<0, 1, 1>, ema_mfma_kernel<0, 1, 2>,
         ema_mfma_kernel<1, 0, 0>, ema_mfma_kernel<1, 0, 1>, ema_mfma_kernel<1, 0, 2>,
         ema_mfma_kernel<1, 1, 0>, ema_mfma_kernel<1, 1, 1>, ema_mfma_kernel<1, 1, 2>};
-    static bool attr_set[12] = {false, false, false, false, false, false, false, false, false, false, false, false};
+    static uint64_t attr_seen[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const int mode = fast ? ((L / G::SC) % 2 == 0 ? 2 : 1) : 0;
     const int ki = (lin * 2 + lout) * 3 + mode;
     const Kern kern = table[ki];
-    if (!attr_set[ki]) {
+    if (first_on_device(&attr_seen[ki])) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::TOTAL);
-      attr_set[ki] = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(kThreadsM), G::TOTAL, s, a);
     MEGA_CHECK_LAUNCH("ema_fwd (matrix-core path)");

@@ -1382,7 +1382,7 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     char* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
     if (!img) {
       rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s,
-                           dtype == MEGA_BF16 ? kImgBf16 : kImgF16);
+                           (dtype == MEGA_BF16 ? kImgBf16 : kImgF16) | kImgBlocks);
       if (rc) return rc;
       img = wimg;
     }
@@ -1394,7 +1394,7 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     if (!img) {
       // no cached image: kernel generation runs with every call
       void* wimg = w + pl.coef_bytes + pl.st_bytes + pl.acc_bytes + pl.tile_bytes;
-      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s, kImgBf16);
+      rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, bidirectional, shift, wimg, s, kImgBf16 | kImgStream);
       if (rc) return rc;
       img = wimg;
     }

@@ -190,10 +190,9 @@ int launch_long_conv_fft(const void* x, void* y, const float* k, int64_t B, int6
                          int bidirectional, int shift, hipStream_t s) {
   auto kern = long_conv_fft_kernel<T>;
   const size_t smem = ((size_t)8) << logm;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static uint64_t attr_seen = 0;
+  if (first_on_device(&attr_seen)) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 8 << kFftMaxLog);
-    attr_set = true;
   }
   // enough workgroups to fill the chip: split the batch when there are few channels
   int64_t nb = 1;

@@ -885,7 +885,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     const void* img = image;
     if (!img) {
       // no cached image: kernel generation runs with every call
-      const int rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, 0, 1, scratch, s, kImgBf16);
+      const int rc = ema_image_build(p, q, gamma, is_complex, omega, D, N, 0, 1, scratch, s, kImgPC | kImgKT | kImgBlocks);
       if (rc) return rc;
       img = scratch;
     }
@@ -902,10 +902,9 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     typedef void (*Kern)(const FusedArgs);
     const int lout = syl == 1 ? 0 : 1;
     const Kern kern = lout == 0 ? norm_ema_fused_kernel<0> : norm_ema_fused_kernel<1>;
-    static bool attr_set[2] = {false, false};
-    if (!attr_set[lout]) {
+    static uint64_t attr_seen[2] = {0, 0};
+    if (first_on_device(&attr_seen[lout])) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFSmem);
-      attr_set[lout] = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(kFT), kFSmem, s, A);
     MEGA_CHECK_LAUNCH("norm_ema_fwd");

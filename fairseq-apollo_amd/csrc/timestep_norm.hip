@@ -645,8 +645,9 @@ __global__ __launch_bounds__(kThreads) void feature_tile_apply(const FeatArgs A)
   }
 }
 
+constexpr int kFeatSerialMax = 2 * kFeatTT;           // rows up to this many tokens take the serial kernel
 size_t feature_tsn_workspace_bytes(int64_t B, int64_t L, int64_t H) {
-  if (L <= 2 * kFeatTT) return 0;                     // short sequences take the serial kernel
+  if (L <= kFeatSerialMax) return 0;
   return (size_t)B * (size_t)ceil_div(L, kFeatTT) * 3 * (size_t)H * 4;
 }
 
@@ -868,6 +869,11 @@ extern "C" int mega_group_timestep_norm_fwd_noalloc(const void* x, void* y, int 
   void* ptr = nullptr;
   const int rc = static_scratch(&ptr);
   if (rc != MEGA_OK) return rc;
+  // a give-up of a bounded wait is reported through the device's status word, which this entry point may not create
+  // (creating it allocates pinned host memory): without it a failure would show only as NaN outputs
+  MEGA_REQUIRE(lookback_launch(false).status != nullptr, MEGA_ERR_UNSUPPORTED,
+               "group_timestep_norm_fwd_noalloc: call mega_lookback_init() once per device first (outside graph "
+               "capture): it creates the status word through which a failed wait is reported");
   return group_tsn_fwd_impl(x, y, dtype, prev_count, prev_mean, prev_var, gamma, beta, mask, B, L, H, G, eps, count,
                             mean, var, group_mean, cummean, cumrstd, ptr, kStaticScratchBytes, true, stream);
 }
@@ -930,6 +936,12 @@ extern "C" int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const i
       return MEGA_OK;
     }
   }
+  // one thread per (row, feature) walking the whole sequence: right for short rows, two orders of magnitude slower
+  // than the tiled kernels for long ones, so a long row without its workspace is refused rather than served slowly
+  MEGA_REQUIRE(L <= kFeatSerialMax, MEGA_ERR_WORKSPACE,
+               "timestep_norm_fwd: L = %ld needs a workspace of %zu bytes (mega_timestep_norm_workspace_bytes with "
+               "G = H); without one only rows of up to %d tokens are served",
+               (long)L, feature_tsn_workspace_bytes(B, L, H), kFeatSerialMax);
   const dim3 grid((unsigned)ceil_div(H, kThreads), (unsigned)B);
 #define LAUNCH_FTSN(T)                                                                            \
   hipLaunchKernelGGL(feature_tsn_kernel<T>, grid, dim3(kThreads), 0, s, (const T*)x, (T*)y,       \

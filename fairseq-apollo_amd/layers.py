@@ -91,7 +91,9 @@ class NormalizedFeedForwardNetwork(nn.Module):
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 
     def forward(self, x: Tensor) -> Tensor:
-        if _training_call(self, x):
+        # hidden dropout acts whenever the module is in training mode, with or without a graph
+        # (normalized_feedforward_network.py:81-83)
+        if _training_call(self, x) or (self.training and self.hidden_dropout_p > 0):
             h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
         else:
             h = ops.silu(self.fc1(self.norm(x)), inplace=True)

@@ -86,7 +86,12 @@ def _tensor_versions(*modules: nn.Module) -> tuple:
     optimiser step or an in-place edit under no_grad bumps the version, `.to()` moves the storage.  (The
     reference recomputes weight + 1, the prior state and the q / k affine on every call,
     timestep_norm.py:118-131, and caches only the moving-average coefficients in eval mode,
-    base_moving_average.py:52-58.)"""
+    base_moving_average.py:52-58.)
+
+    Limit: an edit through `param.data` (`p.data.copy_(...)`, `p.data.mul_(...)`, as some weight-averaging
+    utilities do) changes neither the address nor the version counter of `p`, so it is not seen here; after such an
+    edit call `module.train(); module.eval()` (every mode switch drops the caches) or edit under `torch.no_grad()`
+    through the parameter itself."""
     return tuple((t.data_ptr(), t._version) for m in modules
                  for t in (*m._parameters.values(), *m._buffers.values()) if t is not None)
 

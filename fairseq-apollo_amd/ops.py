@@ -517,7 +517,9 @@ def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool, y=Non
     products (mega_attention_bwd: head-strided operands read in place, the causal half of every product
     skipped); fp32 and odd head sizes through four batched library GEMMs around mega_attention_softmax_bwd.
     `y` (not in the reference's signature): the forward's output; with it the softmax backward's row sums are
-    y_grad . y and the L x L weight gradient never reaches memory."""
+    y_grad . y and the L x L weight gradient never reaches memory.  It must be the output the forward produced
+    from this very `w` (y = w v); a `y` from anywhere else gives a wrong score gradient without any check --
+    pass None when in doubt."""
     dev = _need_gpu(y_grad, q, k, v, w)
     if q.dim() != 4 or w is None or w.dim() != 4:
         raise RuntimeError("attention_bwd: q, k, v must be [B,L,N,H] and w [B,N,L,L]")

@@ -49,7 +49,13 @@ enum {
 /* reason for the last negative return on this thread (never NULL) */
 const char* mega_last_error(void);
 
-/* library version, bumped when a signature changes */
+/* library version, bumped when a signature or a contract changes.
+ *   3: mega_norm_ema_step / mega_norm_ema_steps reject count == prev_count and mega_group_timestep_norm_fwd /
+ *      mega_norm_ema_fwd reject outputs that overlap the prior statistics (version 2 allowed the outputs to alias the
+ *      inputs); MEGA_ERR_LAUNCH may also report an earlier launch's give-up (below); mega_timestep_norm_fwd returns
+ *      MEGA_ERR_WORKSPACE for rows of more than 128 tokens without a workspace (version 2 ran a serial kernel);
+ *      mega_group_timestep_norm_fwd_noalloc requires mega_lookback_init(); the workspace of mega_norm_ema_fwd holds
+ *      one more record per (row, group)                                                                      */
 int mega_abi_version(void);
 
 /* Bounded waits between workgroups.  The group TimestepNorm kernel and the one-kernel TimestepNorm -> moving
@@ -62,8 +68,12 @@ int mega_abi_version(void);
  * sticky launch error does (C10_CUDA_KERNEL_LAUNCH_CHECK(), fairseq/csrc/ops/timestep_norm_kernel.cu:641).
  * mega_lookback_status reads the word of the current device without synchronising (a launch still running
  * may set it later; after a synchronisation it is final); clear != 0 resets it.
- * mega_group_timestep_norm_fwd_noalloc passes the word to its kernel only once another entry point has
- * created it (creating it allocates pinned host memory).                                            */
+ * The word is pinned, device-mapped host memory, created per device by the first regular call that needs it or by
+ * mega_lookback_init (MEGA_OK, or MEGA_ERR_LAUNCH when the runtime refuses the allocation).  Callers that must not
+ * allocate inside a region (HIP graph capture) call mega_lookback_init once per device before it;
+ * mega_group_timestep_norm_fwd_noalloc, which may not create the word itself, returns MEGA_ERR_UNSUPPORTED until
+ * it exists (no counterpart in the reference).                                                        */
+int mega_lookback_init(void);
 int mega_lookback_status(int clear);
 
 /* Test hook for the failure path, so that it can be exercised with every kernel exiting normally:
@@ -287,7 +297,9 @@ int mega_long_conv_fwd(const void* x, void* y, int dtype, const float* k, int64_
  *   the backward pass only)
  * per-feature variant (G == H): stands in for timestep_norm_fwd
  * (timestep_norm.cc:452-510; timestep_norm_kernel.cu:602-654); here prev_mean,
- * prev_var, mean, var, cummean, cumrstd have H in place of G and group_mean is unused. */
+ * prev_var, mean, var, cummean, cumrstd have H in place of G and group_mean is unused.  Rows of more
+ * than 128 tokens need the workspace (mega_timestep_norm_workspace_bytes with G = H); without it the
+ * call returns MEGA_ERR_WORKSPACE (shorter rows run a one-thread-per-feature kernel and need none). */
 size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G);
 int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* prev_count,
                                  const float* prev_mean, const float* prev_var,
@@ -310,6 +322,9 @@ int mega_timestep_norm_fwd(const void* x, void* y, int dtype, const int64_t* pre
  * library (each GPU the library runs on holds its own copy until the process ends); the call
  * itself allocates and frees nothing.  Same arguments, results and errors as
  * mega_group_timestep_norm_fwd, plus:
+ *   - MEGA_ERR_UNSUPPORTED until mega_lookback_init() has created the device's status word (the word
+ *     a failed wait is reported through; creating it allocates pinned host memory, which this entry
+ *     point must not do);
  *   - MEGA_ERR_UNSUPPORTED when the tile records do not fit:
  *     256 + B * (T + ceil(T / 32)) * (2 G + 1) * 8 bytes <= 1 MiB with T = ceil(L / TT) tiles,
  *     TT = tokens per tile (<= 64; one more record per 32 tiles holds their aggregate;
@@ -436,7 +451,9 @@ int mega_attention_fwd(const void* q, const void* k, const void* v, void* y, voi
  * mega_attention_bwd_workspace_bytes returns 0 for such a request).
  *   y: the forward's output [B,L,Nh,H2], or NULL (the reference's backward does not take it).  With
  *   y, rowsum(w w_grad) = rowsum(y_grad y) is known before the first product, and when L % 8 == 0
- *   s_grad leaves that product's epilogue directly: no L x L fp32 weight gradient in memory.
+ *   s_grad leaves that product's epilogue directly: no L x L fp32 weight gradient in memory.  y must
+ *   be what mega_attention_fwd wrote for this very w (y = w v); nothing checks it, and a y from
+ *   elsewhere gives a wrong s_grad.
  * The workspace holds the fp32 weight gradient, s_grad, the row sums and, for rows of w that are
  * not whole 16-byte pieces (L % 8 != 0), transposed copies of w, s_grad, y_grad, q and k.   */
 size_t mega_attention_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t Nh, int64_t H1,

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_argument_checks_need_no_gpu():
     lib = M._lib.load()
-    assert lib.mega_abi_version() == 2
+    assert lib.mega_abi_version() == 3
     # bad dtype is rejected before anything touches a device
     rc = lib.mega_swiglu_fwd(None, None, None, 7, 16, None)
     assert rc == -1 and b"dtype" in lib.mega_last_error()

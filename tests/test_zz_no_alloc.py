@@ -50,6 +50,8 @@ def _case(B, L, H, G, dtype, masked, seed):
 
 def test_noalloc_matches_workspace_entry_twice_then_rejects_oversize():
     lib = M._lib.load()
+    # the status word through which a failed wait is reported: created once per device, outside any capture
+    assert lib.mega_lookback_init() == 0
     ws = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
     # first call: the headline activation shape; second call: a smaller, ragged, masked one
     for (B, L, H, G, dtype, masked, seed) in [(4, 4096, 1024, 16, torch.bfloat16, False, 1),
