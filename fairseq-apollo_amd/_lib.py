@@ -27,6 +27,9 @@ SIGNATURES = {
     "mega_lookback_init": (_int, []),
     "mega_lookback_status": (_int, [_int]),
     "mega_test_lookback": (None, [C.c_uint, _int, _int]),
+    "mega_audit_begin": (None, []),
+    "mega_audit_add": (_int, [_p, _sz]),
+    "mega_audit_end": (_int, [C.POINTER(_int)]),
     "mega_ema_parameters_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _p, _p]),
     "mega_ema_hidden_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "mega_ema_hidden_fwd": (_int, [_p, _int, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _p, _sz, _p]),

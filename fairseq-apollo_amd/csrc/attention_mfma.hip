@@ -389,6 +389,28 @@ void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hi
   if (smem > 64 * 1024 && first_on_device(&attr_seen)) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   }
+  if (audit_on()) {
+    // the last element each operand is addressed at, from the kernel's own indexing: 16-byte pieces whose first
+    // element passes the bounds test, rows below M / N, reduction steps below K; batch bz = bo nin + bi
+    const int64_t bo = (batches - 1) / G.nin, bi = batches - 1 < G.nin ? batches - 1 : G.nin - 1;
+    auto pieces = [](int64_t n) { return (n - 1) / 8 * 8 + 8; };
+    const size_t a_el = AT ? (size_t)((G.K - 1) * G.lda + pieces(G.M)) : (size_t)((G.M - 1) * G.lda + pieces(G.K));
+    const size_t b_el = BT ? (size_t)((G.K - 1) * G.ldb + pieces(G.N)) : (size_t)((G.N - 1) * G.ldb + pieces(G.K));
+    const size_t c_el = (size_t)((G.M - 1) * G.ldc + G.N);
+    audit_use((const TIn*)G.A + bo * G.sa + bi * G.sai, a_el * sizeof(TIn), "gemm operand A");
+    audit_use((const TIn*)G.A, 1, "gemm operand A (first batch)");
+    audit_use((const TIn*)G.Bm + bo * G.sb + bi * G.sbi, b_el * sizeof(TIn), "gemm operand B");
+    audit_use((const TIn*)G.Bm, 1, "gemm operand B (first batch)");
+    if (EPI == 1) {
+      audit_use((TIn*)G.C + bo * G.sc + bi * G.sci, c_el * sizeof(TIn), "gemm result (softmax-backward epilogue)");
+      audit_use((const TIn*)G.E + bo * G.se + bi * G.sei, (size_t)((G.M - 1) * G.lde + G.N) * sizeof(TIn),
+                "gemm epilogue operand E");
+      audit_use(G.rowdot, (size_t)batches * G.M * 4, "gemm epilogue row sums");
+    } else {
+      audit_use((TOut*)G.C + bo * G.sc + bi * G.sci, c_el * sizeof(TOut), "gemm result");
+    }
+    return;
+  }
   G.xcd = xcd ? 1 : 0;
   G.mt = (int)ceil_div(M, TM);
   G.nt = (int)ceil_div(N, TN);
@@ -1168,6 +1190,11 @@ template <typename T>
 void launch_transpose(const T* src, T* dst, int64_t batches, int64_t rows, int64_t nin, int64_t cols, int64_t Lp,
                       hipStream_t s) {
   // src [batches / nin][rows][nin][cols] -> dst [batches][cols][Lp]
+  if (audit_on()) {
+    audit_use(src, (size_t)batches * rows * cols * sizeof(T), "transpose source");
+    audit_use(dst, (size_t)batches * cols * Lp * sizeof(T), "transpose destination");
+    return;
+  }
   const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(cols, 64), (unsigned)batches);
   const int vec = (cols % 8 == 0 && ((uintptr_t)src % 16) == 0) ? 1 : 0;
   hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, src, dst, (int)rows, (int)nin, (int)cols, (int)Lp,
@@ -1210,8 +1237,14 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
   if (fused) {
     float* rd = (float*)(ws + W.rowdot);
     const int64_t nrows = B * L * Nh;
-    hipLaunchKernelGGL(rowdot_kernel<T>, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, s, (const T*)dy, (const T*)y, rd,
-                       (int)L, (int)Nh, (int)H2, nrows);
+    if (audit_on()) {
+      audit_use(dy, (size_t)nrows * H2 * sizeof(T), "row dot: y_grad");
+      audit_use(y, (size_t)nrows * H2 * sizeof(T), "row dot: y");
+      audit_use(rd, (size_t)nrows * 4, "row dot: sums");
+    } else {
+      hipLaunchKernelGGL(rowdot_kernel<T>, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, s, (const T*)dy, (const T*)y,
+                         rd, (int)L, (int)Nh, (int)H2, nrows);
+    }
     G.C = dS; G.E = w; G.rowdot = rd; G.lde = L; G.se = Nh * L * L; G.sei = L * L; G.alpha = scale;
     if (L >= 512) launch_gemm<T, float, 4, 4, false, false, 1>(G, L, L, BN_, xcd, s);
     else launch_gemm<T, float, 2, 2, false, false, 1>(G, L, L, BN_, xcd, s);
@@ -1225,7 +1258,12 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
     const int64_t nrows = BN_ * L;
     const dim3 grid((unsigned)ceil_div(nrows, 4));
     const bool vec = L % 4 == 0 && ((uintptr_t)w % 8) == 0;
-    if (vec)
+    if (audit_on()) {
+      // rows of dW / dS have pitch Lp, rows of w pitch L; L columns each
+      audit_use(dW, (size_t)((nrows - 1) * Lp + L) * 4, "softmax backward: weight gradient");
+      audit_use(w, (size_t)nrows * L * sizeof(T), "softmax backward: weights");
+      audit_use(dS, (size_t)nrows * Lp * sizeof(T), "softmax backward: score gradient (whole rows of the pitch)");
+    } else if (vec)
       hipLaunchKernelGGL((softmax_bwd_f32_kernel<T, 4>), grid, dim3(256), 0, s, dW, (const T*)w, dS, (int)L, (int)L, L, Lp,
                          causal, scale, nrows);
     else
@@ -1250,7 +1288,9 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
     G.Bm = q; G.C = dk;
     G.causal = causal ? 3 : 0;
     launch_gemm<T, T, 2, 2, true, true>(G, L, H1, BN_, xcd, s);
-    MEGA_CHECK_LAUNCH("attention_bwd");
+    if (!audit_on()) {
+      MEGA_CHECK_LAUNCH("attention_bwd");
+    }
     return MEGA_OK;
   }
   // dS [BN][L][Lp] -> dS^T [BN][Lp][Lp]
@@ -1273,7 +1313,9 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
   G.sa = Nh * Lp * Lp; G.sai = Lp * Lp;
   G.causal = causal ? 3 : 0;
   launch_gemm<T, T, 2, 2>(G, L, H1, BN_, xcd, s);
-  MEGA_CHECK_LAUNCH("attention_bwd");
+  if (!audit_on()) {
+    MEGA_CHECK_LAUNCH("attention_bwd");
+  }
   return MEGA_OK;
 }
 

@@ -112,3 +112,53 @@ extern "C" void mega_test_lookback(unsigned spin_limit, int withhold_first, int 
   mega::g_withhold_first.store(withhold_first ? 1 : 0);
   if (raise) *mega::slot_of(mega::current_slot(), false).host = 1u;
 }
+
+// ------------------------------------------------------------------------------------------------
+// Address audit: see common.h.  Thread-local, like the error text.
+namespace mega {
+namespace {
+struct AuditRange {
+  uintptr_t lo, hi;
+};
+struct AuditState {
+  bool on = false;
+  int nranges = 0, nviolations = 0, nchecks = 0;
+  AuditRange ranges[32];
+};
+thread_local AuditState g_audit;
+}  // namespace
+
+bool audit_on() { return g_audit.on; }
+
+bool audit_use(const void* p, size_t bytes, const char* what) {
+  AuditState& a = g_audit;
+  ++a.nchecks;
+  const uintptr_t lo = (uintptr_t)p, hi = lo + bytes;
+  for (int i = 0; i < a.nranges; ++i)
+    if (lo >= a.ranges[i].lo && hi <= a.ranges[i].hi) return true;
+  if (a.nviolations++ == 0)
+    set_error("audit: %s addresses [%p, %p), %zu bytes, outside every registered range", what, p, (const void*)hi,
+              bytes);
+  return false;
+}
+}  // namespace mega
+
+extern "C" void mega_audit_begin(void) {
+  mega::g_audit = mega::AuditState();
+  mega::g_audit.on = true;
+}
+
+extern "C" int mega_audit_add(const void* base, size_t bytes) {
+  mega::AuditState& a = mega::g_audit;
+  if (!a.on || a.nranges >= 32) return MEGA_ERR_ARG;
+  a.ranges[a.nranges++] = {(uintptr_t)base, (uintptr_t)base + bytes};
+  return MEGA_OK;
+}
+
+extern "C" int mega_audit_end(int* checks) {
+  mega::AuditState& a = mega::g_audit;
+  const int v = a.nviolations;
+  if (checks) *checks = a.nchecks;
+  a.on = false;
+  return v;
+}

@@ -57,6 +57,14 @@ static inline bool first_on_device(uint64_t* seen) {
   return !(__atomic_fetch_or(seen, bit, __ATOMIC_RELAXED) & bit);
 }
 
+// ---- address audit (host only).  Between mega_audit_begin() and mega_audit_end() the entry points that take part
+// launch nothing: they compute, for every launch they would make, the last byte each operand is addressed at (from
+// the same sizes and strides the kernel gets) and check that it lies inside one of the byte ranges registered with
+// mega_audit_add (the caller's tensors and workspace, at made-up addresses: no GPU is needed).
+bool audit_on();
+// [p, p + bytes) must lie inside one registered range; records a violation (and returns false) otherwise
+bool audit_use(const void* p, size_t bytes, const char* what);
+
 // Clears `bytes` (a multiple of 4) with a small kernel (elementwise.hip).  Used instead of a memset
 // node so that a caller may record any entry point into a HIP graph.
 void zero_async(void* p, size_t bytes, hipStream_t s);

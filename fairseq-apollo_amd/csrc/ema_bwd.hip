@@ -251,6 +251,21 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
   A.sums = (float*)workspace;
   A.dyx = (float*)((char*)workspace + align_up((size_t)B * D * N * 16, 256));
   A.B = (int)B; A.D = (int)D; A.N = (int)N; A.L = (int)L;
+  if (audit_on()) {
+    // both forms of the kernel leave (b, channel, state) -> 4 floats and (b, channel) -> 1 float; the activations are
+    // addressed from the first token of the walk to the last (the walk may run backwards in memory)
+    const int64_t es = dtype == MEGA_F32 ? 4 : 2;
+    audit_use(A.sums, (size_t)B * D * N * 16, "ema_param_grad: sums");
+    audit_use(A.dyx, (size_t)B * D * 4, "ema_param_grad: dy x");
+    const int64_t hi_g = (B - 1) * sgb + (D - 1) * sgd + (L - 1) * sgl, hi_x = (B - 1) * sxb + (D - 1) * sxd + (L - 1) * sxl;
+    audit_use(dy, (size_t)(hi_g + 1) * es, "ema_param_grad: dy");
+    audit_use(x, (size_t)(hi_x + 1) * es, "ema_param_grad: x");
+    audit_use(dp, (size_t)D * N * 4, "ema_param_grad: dp");
+    audit_use(dq, (size_t)D * N * 8, "ema_param_grad: dq");
+    audit_use(dgamma, (size_t)D * N * 8, "ema_param_grad: dgamma");
+    audit_use(domega, (size_t)D * 4, "ema_param_grad: domega");
+    return MEGA_OK;
+  }
   if (ema_param_grad_tile_covers(dtype, A.dy, A.x, A.sgb, A.sgd, A.sgl, A.sxb, A.sxd, A.sxl, mask, B, D, N, L,
                                  lag_one)) {
     ema_param_grad_tile_launch(A.dy, A.x, A.sgb, A.sgd, A.sgl, A.sxb, A.sxd, A.sxl, q, B, D, N, L, A.sums, A.dyx, s);

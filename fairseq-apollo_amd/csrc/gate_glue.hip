@@ -470,6 +470,17 @@ int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs
                2 * 64 * VEC);
   const unsigned grid = (unsigned)gate_qk_bwd_wgs(T_);
   const size_t lds = (size_t)4 * S * sizeof(float);
+  if (audit_on()) {
+    // every workgroup leaves one row of 4 S sums; rows of T tokens of S (z: pitch zs) elements on the tensors
+    audit_use(part, (size_t)grid * 4 * S * 4, "gate_qk_bwd: rows of parameter sums");
+    audit_use(dq, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: q_grad");
+    audit_use(dk, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: k_grad");
+    audit_use(dz, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: z_grad");
+    audit_use(z, (size_t)((T_ - 1) * zs + S) * sizeof(T), "gate_qk_bwd: z");
+    audit_use(dgamma, (size_t)2 * S * 4, "gate_qk_bwd: gamma_grad");
+    audit_use(dbeta, (size_t)2 * S * 4, "gate_qk_bwd: beta_grad");
+    return MEGA_OK;
+  }
   if (S <= 64 * VEC)
     hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 1>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
                        (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);

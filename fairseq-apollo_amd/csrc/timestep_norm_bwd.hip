@@ -503,18 +503,16 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
   const size_t cells = (size_t)P.TT * P.G;
   const size_t lds0 = (5 * cells + P.G + 2 * (size_t)P.H) * 4 + (P.TT + 1) * 4;
   const size_t lds1 = (5 * cells + P.G) * 4 + (P.TT + 1) * 4;
-  static bool attr0 = false, attr1 = false;
-  if (!attr0) {
+  static uint64_t seen0 = 0, seen1 = 0;
+  if (first_on_device(&seen0)) {
     (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0, false>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 0, true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    attr0 = true;
   }
-  if (!attr1) {
+  if (first_on_device(&seen1)) {
     (void)hipFuncSetAttribute((const void*)tsn_bwd_tile_kernel<T, VEC, 1>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               160 * 1024);
-    attr1 = true;
   }
   const dim3 grid((unsigned)(P.B * P.nt));
   const bool fixed = P.R.PER == 1 && P.R.slots <= kThreads && kThreads % P.R.slots == 0;
@@ -594,6 +592,20 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
   P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.tt; P.nt = g.nt;
   P.R = make_row_tiling(G, H / G, g.vec);
+  if (audit_on()) {
+    // per (row, tile, group): one map of four floats and one pair of state gradients; per (row, tile): the tile's
+    // share of the gamma / beta gradients, 2 H floats
+    const size_t es = dtype == MEGA_F32 ? 4 : 2;
+    audit_use(P.agg, (size_t)B * g.nt * G * 16, "timestep_norm_bwd: tile maps");
+    audit_use(P.state, (size_t)B * g.nt * G * 8, "timestep_norm_bwd: pairs entering the tiles");
+    audit_use(P.part, (size_t)B * g.nt * 2 * H * 4, "timestep_norm_bwd: parameter-gradient shares");
+    audit_use(y_grad, (size_t)B * L * H * es, "timestep_norm_bwd: y_grad");
+    audit_use(x, (size_t)B * L * H * es, "timestep_norm_bwd: x");
+    audit_use(x_grad, (size_t)B * L * H * es, "timestep_norm_bwd: x_grad");
+    audit_use(cummean, (size_t)B * L * G * 4, "timestep_norm_bwd: cummean");
+    audit_use(cumrstd, (size_t)B * L * G * 4, "timestep_norm_bwd: cumrstd");
+    return MEGA_OK;
+  }
   switch (dtype) {
     case MEGA_F32: return launch_bwd<float>(P, g.vec, s);
     case MEGA_BF16: return launch_bwd<bf16_t>(P, g.vec, s);

@@ -82,6 +82,17 @@ int mega_lookback_status(int clear);
  * status word of the current device from the host.  Not for production use.                         */
 void mega_test_lookback(unsigned spin_limit, int withhold_first, int raise);
 
+/* Address audit (host only, nothing is launched, no GPU needed; no counterpart in the reference).  Between
+ * mega_audit_begin() and mega_audit_end() the calling thread's calls to mega_attention_bwd, mega_gate_qk_bwd,
+ * mega_ema_param_grad and mega_(group_)timestep_norm_bwd launch nothing: for every launch they would make they
+ * compute, from the sizes and strides the kernel would get, the last byte every operand is addressed at and check
+ * that it lies inside one of the byte ranges registered with mega_audit_add (the tensors and the workspace of the
+ * call, at any made-up addresses that satisfy the alignment rules).  mega_audit_end returns the number of
+ * violations (the first one in mega_last_error()) and, through `checks`, how many ranges were checked.    */
+void mega_audit_begin(void);
+int mega_audit_add(const void* base, size_t bytes);
+int mega_audit_end(int* checks);
+
 /* ------------------------------------------------------------------------ */
 /* EMA coefficients -> convolution kernel and carried-state bias            */
 /* stands in for ema_parameters_fwd (fairseq/csrc/ops/ema_parameters.cc:211-286,
