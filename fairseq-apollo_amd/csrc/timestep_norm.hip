@@ -734,7 +734,7 @@ extern "C" size_t mega_timestep_norm_workspace_bytes(int dtype, int64_t B, int64
   // G == H names both the per-feature variant (mega_timestep_norm_fwd) and the group variant with one channel per
   // group (mega_group_timestep_norm_fwd): the size covers whichever entry point the workspace is handed to
   size_t need = 256;
-  if (B > 0 && L > 0 && H > 0 && G == H && H > 1) {
+  if (B > 0 && L > 0 && H > 0 && G == H) {
     const size_t f = feature_tsn_workspace_bytes(B, L, H);
     need = f > need ? f : need;
   }

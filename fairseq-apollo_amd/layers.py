@@ -27,25 +27,49 @@ from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOut
 
 
 class RMSNorm(nn.Module):
-    """x / sqrt(mean(x^2) + eps) * weight (fairseq/modules/norm_layer/layer_norm.py:41-59, which
-    wraps apex FusedRMSNorm); one wave per token in the HIP library."""
+    """x / sqrt(mean(x^2) + eps) * (weight + 1): the parameter is stored as the offset from one and starts at zero, as
+    in the reference (fairseq/modules/norm_layer/layer_norm.py:41-59: FusedRMSNorm.reset_parameters zeroes it and
+    forward passes `self.weight + 1.0`), so a reference checkpoint's `*.weight` loads unchanged.  One wave per token
+    in the HIP library."""
 
     def __init__(self, dim: int, elementwise_affine: bool = True, eps: float = 1e-5):
         super().__init__()
         self.eps = eps
         if elementwise_affine:
-            self.weight = Parameter(torch.ones(dim))
+            self.weight = Parameter(torch.zeros(dim))
         else:
             self.register_parameter("weight", None)
 
     def forward(self, x: Tensor) -> Tensor:
+        w = None if self.weight is None else self.weight.float() + 1.0
         if _training_call(self, x):
             y = x.float()
             y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + self.eps)
-            if self.weight is not None:
-                y = y * self.weight.float()
+            if w is not None:
+                y = y * w
             return y.to(x.dtype)
-        return ops.rms_norm_fwd(x, self.weight, self.eps)
+        return ops.rms_norm_fwd(x, w, self.eps)
+
+
+class LayerNorm(nn.Module):
+    """Layer normalisation with the affine weight stored as its offset from one (zero-initialised weight and bias,
+    `weight + 1` in the forward): fairseq/modules/norm_layer/layer_norm.py:85-111 (FairseqLayerNorm; the fused
+    variant at :19-39 does the same).  A torch operation: it is not on the measured path."""
+
+    def __init__(self, dim: int, eps: float = 1e-5, elementwise_affine: bool = True):
+        super().__init__()
+        self.normalized_shape = (dim,)
+        self.eps = eps
+        if elementwise_affine:
+            self.weight = Parameter(torch.zeros(dim))
+            self.bias = Parameter(torch.zeros(dim))
+        else:
+            self.register_parameter("weight", None)
+            self.register_parameter("bias", None)
+
+    def forward(self, x: Tensor) -> Tensor:
+        w = None if self.weight is None else self.weight + 1.0
+        return F.layer_norm(x, self.normalized_shape, w, self.bias, self.eps)
 
 
 class NormalizedFeedForwardNetwork(nn.Module):
@@ -64,7 +88,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
         self.layer_scale = layer_scale
         self.dropout_p, self.hidden_dropout_p = float(dropout), float(hidden_dropout)
         if norm_type == 'layernorm':
-            self.norm = nn.LayerNorm(embed_dim, eps=norm_eps, elementwise_affine=norm_affine)
+            self.norm = LayerNorm(embed_dim, eps=norm_eps, elementwise_affine=norm_affine)
         elif norm_type == 'rmsnorm':
             self.norm = RMSNorm(embed_dim, elementwise_affine=norm_affine, eps=norm_eps)
         else:

@@ -283,7 +283,7 @@ def timestep_norm_fwd(x, prev_count, prev_mean, prev_var, gamma, beta, padding_m
     key = ("tsn_feat", dt, B, L, H)
     nws = _ws_bytes_cache.get(key)
     if nws is None:
-        nws = _ws_bytes_cache[key] = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, H) if H > 1 else 0
+        nws = _ws_bytes_cache[key] = lib.mega_timestep_norm_workspace_bytes(dt, B, L, H, H)
     stream = _stream(dev)
     ws = _scratch_buffer(dev, nws, stream) if nws else None      # tile states of the time-parallel kernels
     with _on_device(dev):

@@ -32,6 +32,12 @@ place, where that build exists).  Pin status per function:
                                          (gamma = -1: running means of v; W_h = 0; z under the
                                          normalize clamp; one-hot mx_proj rows)
                                          (tests/test_oracle_layer.py)
+  normalized_ffn                         torch's F.layer_norm / F.linear / F.silu with the stored
+                                         weight plus one, identity for a zero second projection
+  mega_lm_decoder                        no layers: textbook prefix statistics + library
+                                         projections; two layers: hand composition of the pinned
+                                         pieces, order asymmetry, causality in the tokens, the
+                                         chunk padding cut back, zero logits at padding tokens
 The SwiGLU feed-forward block and the multi-head split of the gated attention are north-star
 specification, not reference code (the reference FFN is the SiLU block, its layer single-head):
 their formulas are pinned as above, their parity with the reference is unpinned by construction.
@@ -748,7 +754,7 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     step.  x: [B, L, D]; P: dict of numpy parameters
       norm_weight, norm_bias [D]; ema p, q, gamma [D, N], omega [D];
       v_w [E, D], v_b [E]; mx_w [D+S+E+D, D], mx_b; h_w [D, E]; gamma, beta [2, S];
-      optional rms_weight [D].
+      optional rms_weight [D] (the stored parameter: the multiplier is rms_weight + 1).
     num_heads > 1 splits q, k (S) and v (E) into heads laid out [B, L, Nh, H] (the layout of the
     fused op, csrc/ops/attention_kernel.cu:46-50); the reference layer itself is single-head."""
     x = np.asarray(x, np.float64)
@@ -767,7 +773,10 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     mx, _ = ema_forward(xn.transpose(0, 2, 1), P['p'], P['q'], P['ema_gamma'], P['omega'], padding_mask,
                         bidirectional=bidirectional)
     mx = mx.transpose(0, 2, 1)
-    mx = _silu(mx) if moving_act == 'silu' else rms_norm(mx, P.get('rms_weight'), eps)
+    # the RMSNorm weight is stored as its offset from one (norm_layer/layer_norm.py:47-56: zero-initialised, the
+    # forward passes `self.weight + 1.0`); P['rms_weight'] is the stored parameter
+    rms_w = None if P.get('rms_weight') is None else np.asarray(P['rms_weight'], np.float64) + 1.0
+    mx = _silu(mx) if moving_act == 'silu' else rms_norm(mx, rms_w, eps)
     base = mx @ np.asarray(P['mx_w'], np.float64).T + P['mx_b']
     u, z, r, hx = np.split(base, [D, D + S, D + S + E], axis=-1)
     u = _sigmoid(u)
@@ -825,3 +834,68 @@ def gated_attention_layer(x, P, chunk: int, num_heads: int = 1, moving_act: str 
     a = a.reshape(B, L, E)
     h = _silu(hx + (a * r) @ np.asarray(P['h_w'], np.float64).T)
     return x + u * (h - x)
+
+
+# --------------------------------------------------------------------------
+# f3/f4: the feed-forward block with its norm, and the decoder-only language model
+# --------------------------------------------------------------------------
+
+
+def normalized_ffn(x, P, norm_type: str = 'layernorm', eps: float = 1e-5):
+    """NormalizedFeedForwardNetwork.forward (modules/normalized_feedforward_network.py:77-93):
+    residual + [layerscale *] fc2(silu(fc1(norm(x)))).  P: norm_weight (stored as the offset from one,
+    norm_layer/layer_norm.py:24-33, 47-56, 105-111) and norm_bias (layernorm only) or None, fc1_w [F, D], fc1_b [F],
+    fc2_w [D, F], optional layerscale [D]."""
+    x = np.asarray(x, np.float64)
+    w = None if P.get('norm_weight') is None else np.asarray(P['norm_weight'], np.float64) + 1.0
+    if norm_type == 'rmsnorm':
+        xn = rms_norm(x, w, eps)
+    else:
+        mu = x.mean(-1, keepdims=True)
+        xn = (x - mu) / np.sqrt(x.var(-1, keepdims=True) + eps)
+        if w is not None:
+            xn = xn * w + np.asarray(P['norm_bias'], np.float64)
+    h = _silu(xn @ np.asarray(P['fc1_w'], np.float64).T + np.asarray(P['fc1_b'], np.float64))
+    h = h @ np.asarray(P['fc2_w'], np.float64).T
+    if P.get('layerscale') is not None:
+        h = h * np.asarray(P['layerscale'], np.float64)
+    return h + x
+
+
+def mega_lm_decoder(tokens, P, chunk: int, padding_idx: int, num_groups: int, embed_scale: Optional[float],
+                    moving_act: str = 'rmsnorm', norm_type: str = 'rmsnorm', eps: float = 1e-5,
+                    simple_bias: bool = False, attention_activation: str = 'softmax'):
+    """MegaDecoderNoCrossAttn.forward (models/mega_lm.py:267-386): tokens [B, T] (int) -> logits [B, T, V].
+    The sequence is padded with padding_idx up to a whole number of chunks (:326-330), embedded and scaled (:333-335),
+    run through the layers (mega_layer then nffn, modules/mega_layer.py:196-200) with the padding mask, normalised by
+    the final TimestepNorm (:356), passed through pre_logits (fc + silu when present, :226-232), zeroed at padded
+    positions (:360-363), cut back to T (:366-367) and projected (:379-385).
+    P: embed [V, D]; layers: list of dicts {attn: gated_attention_layer's P (+ 'simple_bias' when simple_bias),
+    ffn: normalized_ffn's P or None}; final_weight, final_bias [D]; optional pre_w [F, D], pre_b [F]; out_w [V, F]."""
+    tokens = np.asarray(tokens)
+    B, T = tokens.shape
+    pad_to = T
+    if T > chunk > 0 and T % chunk != 0:
+        pad_to = -(-T // chunk) * chunk
+        tokens = np.concatenate([tokens, np.full((B, pad_to - T), padding_idx, tokens.dtype)], 1)
+    x = np.asarray(P['embed'], np.float64)[tokens]
+    if embed_scale is not None:
+        x = x * embed_scale
+    mask = tokens == padding_idx
+    if not mask.any():
+        mask = None
+    for lp in P['layers']:
+        x = gated_attention_layer(x, lp['attn'], chunk if chunk > 0 else pad_to, 1, 'rms' if moving_act == 'rmsnorm' else 'silu',
+                                  eps, num_groups, False, mask, lp['attn'].get('simple_bias') if simple_bias else None,
+                                  attention_activation)
+        if lp.get('ffn') is not None:
+            x = normalized_ffn(x, lp['ffn'], norm_type, eps)
+    G = num_groups
+    x = timestep_norm(x, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)),
+                      np.asarray(P['final_weight'], np.float64) + 1.0, P['final_bias'], mask, G, eps)[0]
+    if P.get('pre_w') is not None:
+        x = _silu(x @ np.asarray(P['pre_w'], np.float64).T + np.asarray(P['pre_b'], np.float64))
+    if mask is not None:
+        x = x * (~mask)[..., None]
+    x = x[:, :T]
+    return x @ np.asarray(P['out_w'], np.float64).T

@@ -44,6 +44,8 @@ def test_gated_attention_layer(dtype, tol, heads, act, moving):
             prm.normal_(0, 0.15)
         layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
         layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+        if act == 'rmsnorm':
+            layer.move_act.weight.normal_(0, 0.2)        # stored as the offset from one
     P = _params(layer)                       # fp32 master copy of the parameters
     if dtype != torch.float32:               # the module rounds its projection weights to the activation type
         for k_ in ('v_w', 'v_b', 'mx_w', 'mx_b', 'h_w', 'gamma', 'beta', 'norm_weight', 'norm_bias', 'rms_weight'):
@@ -108,16 +110,17 @@ def test_normalized_feed_forward(dtype, tol, norm_type, layer_scale):
     ffn = M.NormalizedFeedForwardNetwork(D, Hd, norm_type=norm_type, layer_scale=layer_scale, init_mode='xavier')
     with torch.no_grad():
         ffn.fc1.bias.normal_(0, 0.1)
+        ffn.norm.weight.normal_(0, 0.2)                   # away from the initial zero (= a multiplier of one)
     ffn = ffn.to(DEV).to(dtype).eval()
     x = torch.randn(B, L, D).to(dtype).to(DEV)
     with torch.no_grad():
         y = ffn(x)
     x64 = host(x)
     if norm_type == "rmsnorm":
-        xn = O.rms_norm(x64, host(ffn.norm.weight))
+        xn = O.rms_norm(x64, host(ffn.norm.weight) + 1.0)          # stored as the offset from one (layer_norm.py:47-56)
     else:
         mu = x64.mean(-1, keepdims=True)
-        xn = (x64 - mu) / np.sqrt(x64.var(-1, keepdims=True) + 1e-5) * host(ffn.norm.weight) + host(ffn.norm.bias)
+        xn = (x64 - mu) / np.sqrt(x64.var(-1, keepdims=True) + 1e-5) * (host(ffn.norm.weight) + 1.0) + host(ffn.norm.bias)
     w2 = host(ffn.fc2.weight)
     if layer_scale is not None:
         w2 = w2 * host(ffn.layerscale_weight)[:, None]

@@ -429,6 +429,8 @@ def test_gated_attention_layer_sweep(seed):
                 prm.normal_(0, 0.15)
             layer.gamma.normal_(0, 0.1); layer.beta.normal_(0, 0.1)
             layer.norm.weight.normal_(0, 0.1); layer.norm.bias.normal_(0, 0.1)
+            if isinstance(layer.move_act, M.RMSNorm):
+                layer.move_act.weight.normal_(0, 0.2)
         p, q, g = layer.move.coeffs()
         P = dict(norm_weight=host(layer.norm.weight), norm_bias=host(layer.norm.bias), p=host(p.squeeze(-1)),
                  q=host(q.squeeze(-1)), ema_gamma=host(g), omega=host(layer.move.omega).reshape(-1),

@@ -133,7 +133,7 @@ def _params(rng, D, S, E, N, bidirectional=False):
                 omega=rng.normal(size=D), v_w=rng.normal(size=(E, D)) * 0.3, v_b=rng.normal(size=E) * 0.1,
                 mx_w=rng.normal(size=(2 * D + S + E, D)) * 0.3, mx_b=rng.normal(size=2 * D + S + E) * 0.1,
                 h_w=rng.normal(size=(D, E)) * 0.3, gamma=rng.normal(size=(2, S)) * 0.3, beta=rng.normal(size=(2, S)) * 0.3,
-                rms_weight=rng.normal(size=D) * 0.2 + 1.0)
+                rms_weight=rng.normal(size=D) * 0.2)
 
 
 def _restated_layer(x, P, chunk, num_groups, moving_act="silu", bidirectional=False, padding_mask=None,
@@ -153,7 +153,8 @@ def _restated_layer(x, P, chunk, num_groups, moving_act="silu", bidirectional=Fa
     mx = O.ema_forward(xn.transpose(0, 2, 1), P["p"], P["q"], P["ema_gamma"], P["omega"], padding_mask,
                        bidirectional=bidirectional)[0].transpose(0, 2, 1)   # :312-314
     mx = t(np.ascontiguousarray(mx))
-    mx = F.silu(mx) if moving_act == "silu" else F.rms_norm(mx, (D,), t(P["rms_weight"]), eps)      # :315
+    # :315; RMSNorm = FusedRMSNorm: `weight = self.weight + 1.0`, rms norm with it (norm_layer/layer_norm.py:54-56)
+    mx = F.silu(mx) if moving_act == "silu" else F.rms_norm(mx, (D,), t(P["rms_weight"]) + 1.0, eps)
     base = F.linear(mx, t(P["mx_w"]), t(P["mx_b"]))                         # :318
     u, z, r, hx = torch.split(base, [D, S, E, D], dim=-1)                    # :319
     u = torch.sigmoid(u)                                                     # :321
@@ -344,3 +345,115 @@ def test_layer_heads_split_features_not_tokens():
             a[0, c0:c0 + chunk, n * H2:(n + 1) * H2] = w @ v[0, c0:c0 + chunk, n * H2:(n + 1) * H2]
     want = x + u * (silu(hx + (a * r)[..., :D]) - x)
     assert np.allclose(got, want, atol=1e-12)
+
+
+# --------------------------------------------------------------------------
+# the feed-forward block with its norm, and the whole decoder-only model
+# --------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("norm_type", ["layernorm", "rmsnorm"])
+@pytest.mark.parametrize("affine,scale", [(True, True), (True, False), (False, False)])
+def test_normalized_ffn_against_library_calls(norm_type, affine, scale):
+    """normalized_feedforward_network.py:77-93 typed with torch's own layer_norm / linear / silu, the norm's multiplier
+    being the stored weight plus one (norm_layer/layer_norm.py:24-33, 47-56, 105-111)."""
+    rng = np.random.default_rng(11)
+    D, Fh = 12, 20
+    x = rng.standard_normal((2, 5, D))
+    P = dict(norm_weight=rng.standard_normal(D) * 0.3 if affine else None,
+             norm_bias=rng.standard_normal(D) * 0.3 if affine and norm_type == "layernorm" else None,
+             fc1_w=rng.standard_normal((Fh, D)), fc1_b=rng.standard_normal(Fh), fc2_w=rng.standard_normal((D, Fh)),
+             layerscale=rng.random(D) + 0.1 if scale else None)
+    t = lambda a: None if a is None else torch.from_numpy(np.asarray(a, np.float64))
+    xt = t(x)
+    if norm_type == "layernorm":
+        xn = F.layer_norm(xt, (D,), None if not affine else t(P["norm_weight"]) + 1.0, t(P["norm_bias"]), 1e-5)
+    else:
+        xn = xt * torch.rsqrt(xt.pow(2).mean(-1, keepdim=True) + 1e-5)
+        if affine:
+            xn = xn * (t(P["norm_weight"]) + 1.0)
+    h = F.linear(F.silu(F.linear(xn, t(P["fc1_w"]), t(P["fc1_b"]))), t(P["fc2_w"]))
+    want = (h * t(P["layerscale"]) if scale else h) + xt
+    got = O.normalized_ffn(x, P, norm_type, 1e-5)
+    assert np.abs(got - want.numpy()).max() < 1e-12
+    # zero second projection: the block is the identity, whatever the norm does
+    P0 = dict(P, fc2_w=np.zeros((D, Fh)))
+    assert np.array_equal(O.normalized_ffn(x, P0, norm_type), x)
+
+
+def _model_params(rng, V, D, S, E, N, Fh, n_layers, G, rep=None):
+    layers = []
+    for _ in range(n_layers):
+        A = _params(rng, D, S, E, N)
+        A["rms_weight"] = rng.standard_normal(D) * 0.2
+        ffn = dict(norm_weight=rng.standard_normal(D) * 0.2, norm_bias=None, fc1_w=rng.standard_normal((Fh, D)) * 0.3,
+                   fc1_b=rng.standard_normal(Fh) * 0.1, fc2_w=rng.standard_normal((D, Fh)) * 0.3, layerscale=None)
+        layers.append(dict(attn=A, ffn=ffn))
+    emb = rng.standard_normal((V, D))
+    emb[1] = 0.0                                                     # the padding row of nn.Embedding
+    P = dict(embed=emb, layers=layers, final_weight=rng.standard_normal(D) * 0.2, final_bias=rng.standard_normal(D) * 0.2,
+             out_w=rng.standard_normal((V, rep or D)))
+    if rep:
+        P["pre_w"], P["pre_b"] = rng.standard_normal((rep, D)), rng.standard_normal(rep)
+    return P
+
+
+def test_model_without_layers_is_norm_and_projection():
+    """No layers: logits = W_out silu(W_pre tsn(scale * E[tokens]) + b_pre), the norm in its textbook form (prefix
+    means and variances), the rest through torch's library calls; a dropped scale, a missing `+ 1` on the norm's
+    weight, a transposed projection or a forgotten pre_logits activation each change the result."""
+    rng = np.random.default_rng(12)
+    V, D, G, rep = 17, 8, 2, 6
+    P = _model_params(rng, V, D, 4, 8, 2, 8, 0, G, rep)
+    tok = rng.integers(2, V, (2, 9))
+    got = O.mega_lm_decoder(tok, P, 4, 1, G, 3.0)                     # 9 tokens, chunk 4: padded to 12, cut back to 9
+    pad = np.zeros((2, 12), bool)
+    pad[:, 9:] = True
+    x = np.concatenate([P["embed"][tok] * 3.0, np.zeros((2, 3, D))], 1)
+    y = O.timestep_norm_closed_form(x, pad, G, 1e-5, P["final_weight"] + 1.0, P["final_bias"])[0][:, :9]
+    t = lambda a: torch.from_numpy(np.asarray(a, np.float64))
+    want = F.linear(F.silu(F.linear(t(y), t(P["pre_w"]), t(P["pre_b"]))), t(P["out_w"])).numpy()
+    assert got.shape == (2, 9, V) and np.abs(got - want).max() < 1e-10
+    # without the scale the norm sees other numbers (eps is not scale-free) and without pre_logits other features
+    assert np.abs(O.mega_lm_decoder(tok, P, 4, 1, G, None) - want).max() > 1e-7
+    P2 = {k: v for k, v in P.items() if k not in ("pre_w", "pre_b")}
+    P2["out_w"] = rng.standard_normal((V, D))
+    assert np.abs(O.mega_lm_decoder(tok, P2, 4, 1, G, 3.0) - y @ P2["out_w"].T).max() < 1e-10
+
+
+def test_model_is_layers_then_ffn_in_order_and_pads_like_the_reference():
+    """Two layers: (a) the order is attention layer, feed-forward, attention layer, feed-forward (mega_layer.py:196-200,
+    mega_lm.py:348-354), checked by composing the pinned pieces by hand; (b) every position is causal in the tokens;
+    (c) a length that is not a whole number of chunks gives the first rows of the longer sequence's logits, the padded
+    end being cut off (mega_lm.py:326-330, 366-367); (d) padding tokens inside the input give zero logits there
+    (mega_lm.py:360-363) and do not count in the norms."""
+    rng = np.random.default_rng(13)
+    V, D, S, E, N, Fh, G, C = 19, 8, 4, 8, 2, 12, 2, 4
+    P = _model_params(rng, V, D, S, E, N, Fh, 2, G)
+    tok = rng.integers(2, V, (2, 12))
+    got = O.mega_lm_decoder(tok, P, C, 1, G, 2.0)
+    x = P["embed"][tok] * 2.0
+    for lp in P["layers"]:
+        x = O.gated_attention_layer(x, lp["attn"], C, 1, "rms", 1e-5, G)
+        x = O.normalized_ffn(x, lp["ffn"], "rmsnorm", 1e-5)
+    y = O.timestep_norm_closed_form(x, None, G, 1e-5, P["final_weight"] + 1.0, P["final_bias"])[0]
+    assert np.abs(got - y @ P["out_w"].T).max() < 1e-10
+    # swapping the two layers' parameters changes the result: the order is not symmetric
+    Q = dict(P, layers=P["layers"][::-1])
+    assert np.abs(O.mega_lm_decoder(tok, Q, C, 1, G, 2.0) - got).max() > 1e-6
+    # (b)
+    tok2 = tok.copy()
+    tok2[:, 7] = (tok2[:, 7] - 2 + 1) % (V - 2) + 2
+    alt = O.mega_lm_decoder(tok2, P, C, 1, G, 2.0)
+    assert np.abs(alt[:, :7] - got[:, :7]).max() < 1e-11 and np.abs(alt[:, 7:] - got[:, 7:]).max() > 1e-6
+    # (c)
+    short = O.mega_lm_decoder(tok[:, :10], P, C, 1, G, 2.0)
+    assert short.shape == (2, 10, V) and np.abs(short - got[:, :10]).max() < 1e-11
+    # a single chunk or less is not padded (seq_len > chunk fails, mega_lm.py:326): three tokens stay three
+    assert np.abs(O.mega_lm_decoder(tok[:, :3], P, C, 1, G, 2.0) - got[:, :3]).max() < 1e-11
+    # (d)
+    tok3 = tok.copy()
+    tok3[0, 8:] = 1
+    padded = O.mega_lm_decoder(tok3, P, C, 1, G, 2.0)
+    assert np.array_equal(padded[0, 8:], np.zeros((4, V)))
+    assert np.abs(padded[0, :8] - got[0, :8]).max() < 1e-11 and np.abs(padded[1] - got[1]).max() < 1e-11
