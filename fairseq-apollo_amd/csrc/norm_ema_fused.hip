@@ -54,7 +54,7 @@ constexpr int kFTile = kFC * kFRow + (kFC / 4) * 16;
 constexpr int kFRecW = 4 + kFC * kNS * 2;     // 64-bit words per block record: n, mean, var, pad, end states
 constexpr int kFMaxBlocks = 16;               // terms of the look-back sum (earlier blocks + the carried state): one per lane of a row
 constexpr int kFTabs = 2;                     // per-state multiplier tables kept in LDS: q^32, q^64
-constexpr size_t kFSmem = (size_t)kFTile + 2 * kFSeg * 4 + 64 + (size_t)kFTabs * kFC * 128;
+constexpr size_t kFSmem = (size_t)kFTile + 2 * kFSeg * 4 + 64 + (size_t)kFTabs * kFC * 128 + kFC * 8;
 
 static_assert(kSEGT == 2, "the fused kernel uses the q^64 segment multipliers of the image");
 static_assert(kFSmem <= 160 * 1024, "LDS of one workgroup");
@@ -178,6 +178,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   float* s_wt = s_gv + kFSeg;                 // [4][4] totals of the four scanning waves
   float* s_end = s_gm;                        // [kFC][kNS][2] block end states from a zero start (after step 2)
   char* s_tab = (char*)(s_wt + 16);           // [kFTabs][kFC][kNS] complex: q^32, q^64 of every channel
+  uint2* s_reach = (uint2*)(s_tab + kFTabs * kFC * 128);   // [kFC] reach of every channel's slowest pole
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: channel rows and image addresses stay scalar
@@ -228,6 +229,8 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
             *(const uint4*)(ibase + (size_t)c * kImgRowBytes + t * 128 + pc * 16);
       }
     }
+    // and how far every channel's slowest pole reaches (asked for here, used after the norm: no wave waits for it)
+    if (tid < kFC) s_reach[tid] = *(const uint2*)(ibase + (size_t)tid * kImgRowBytes + kCmpReach * 128);
   }
 
   // ---- the caller's carried state joins the records the later look-ups read: slot S of the row, written by block 0
@@ -452,8 +455,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   int nsteps[kFCPW], nlook[kFCPW];
 #pragma unroll
   for (int i = 0; i < kFCPW; ++i) {
-    const uint2 rw = *(const uint2*)((const char*)A.image + (size_t)(g * kFC + wave + kFW * i) * kImgRowBytes +
-                                     kSlotCmp * 1024 + kCmpReach * 128);
+    const uint2 rw = s_reach[wave + kFW * i];
     nsteps[i] = __builtin_amdgcn_readfirstlane((int)rw.x);
     nlook[i] = __builtin_amdgcn_readfirstlane((int)rw.y);
   }
