@@ -76,7 +76,7 @@ struct FusedArgs {
   const float* h_in;     // [B, D, N, 2] or null
   float* h_out;          // [B, D, N, 2] or null
   TsnHeader* hdr;
-  unsigned long long* rec;   // [B * G][S + 1][kFRecW]; slot S: the caller's carried state, put there by block 0
+  unsigned long long* rec;   // [B * D / 64][S + 1][kFRecW]; slot S: the caller's carried state, put there by block 0
   int B, L, D, G, N, S;
   float eps;
   int is_complex;
@@ -168,9 +168,13 @@ __device__ __forceinline__ void lds_cmp(const char* s_tab, int tab, int c, uint3
   re[2] = b.x; im[2] = b.y; re[3] = b.z; im[3] = b.w;
 }
 
-// LOUT 0: y as [B, D, L] rows; 1: y as [B, L, D]
-template <int LOUT>
+// LOUT 0: y as [B, D, L] rows; 1: y as [B, L, D].  GC: channels per norm group, 64 or 128.  A group of 128 channels
+// is shared by two workgroups: each reads the group's whole lines for the moments (both add in the same order, so
+// both arrive at the same statistics to the last bit) and keeps its own 64 channels.
+template <int LOUT, int GC>
 __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) {
+  constexpr int kParts = GC / kFC;
+  static_assert(kParts == 1 || kParts == 2, "one or two workgroups per norm group");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* tile = smem;
   float* s_gm = (float*)(smem + kFTile);      // [kFSeg] group mean of a token, later the running mean
@@ -183,43 +187,55 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: channel rows and image addresses stay scalar
   const int G = A.G;
-  const int BG = A.B * G;
-  const int s = (int)blockIdx.x / BG, local = (int)blockIdx.x - s * BG;
-  int b, g;
+  const int U = G * kParts;                              // workgroups per (batch row, block)
+  const int BU = A.B * U;
+  const int s = (int)blockIdx.x / BU, local = (int)blockIdx.x - s * BU;
+  int b, unit;
   if (A.xcd_map) {
     // consecutive workgroup ids go to the 8 XCDs in turn: keep a group's blocks (and with them the operand
-    // images of its 64 channels) on one XCD, G / 8 groups per XCD
-    const int gp = G >> 3, xcd = local & 7, slot = local >> 3;
-    g = xcd * gp + slot % gp;
-    b = slot / gp;
+    // images of its channels and the lines its two halves share) on one XCD, U / 8 units per XCD
+    const int up = U >> 3, xcd = local & 7, slot = local >> 3;
+    unit = xcd * up + slot % up;
+    b = slot / up;
   } else {
-    b = local / G;
-    g = local - b * G;
+    b = local / U;
+    unit = local - b * U;
   }
+  const int g = unit / kParts, part = unit - g * kParts;
+  const int cb = g * GC + part * kFC;                    // the workgroup's first channel
   const uint32_t tag = A.hdr->epoch + 1u;
   const int t0 = s * kFSeg;
   const int piece = tid & 7, tokl = tid >> 3;            // 16-byte piece of the 128-byte line, token 0..127
   // addresses of the block's lines: a uniform base per 128-token round plus one 32-bit lane offset
-  const size_t xblk = ((size_t)b * A.L + t0) * A.D + (size_t)g * kFC;
+  const size_t xblk = ((size_t)b * A.L + t0) * A.D + (size_t)cb;
   const uint32_t toff = (uint32_t)tokl * (uint32_t)A.D + piece * 8;
-  const size_t brow = (size_t)b * G + g;
-  unsigned long long* const myrec = A.rec + (brow * (A.S + 1) + s) * kFRecW;
+  const size_t brow = (size_t)b * G + g;                 // statistics of the group
+  const size_t rrow = brow * kParts + part;              // records of the workgroup (its own copy of the statistics too)
+  unsigned long long* const myrec = A.rec + (rrow * (A.S + 1) + s) * kFRecW;
   bool poison = false;
 
   MEGA_FTR(0);
   // ---- everything the norm needs from memory is requested before the block itself
   const Moments prior = {(float)A.prev_count[b], A.prev_mean[brow], A.prev_var[brow]};
   float gam[8], bet[8];
-  load_params<8>(A.gamma + g * kFC + piece * 8, gam);
-  load_params<8>(A.beta + g * kFC + piece * 8, bet);
+  load_params<8>(A.gamma + cb + piece * 8, gam);
+  load_params<8>(A.beta + cb + piece * 8, bet);
   uint4 xv[kFNLD];
 #pragma unroll
   for (int k = 0; k < kFNLD; ++k) xv[k] = *(const uint4*)(A.x + xblk + (size_t)k * 128 * A.D + toff);
+  // the other half of the group's lines, for the moments only (the workgroup of that half reads the same lines on the
+  // same XCD)
+  uint4 xo[kParts == 2 ? kFNLD : 1];
+  if (kParts == 2) {
+    const size_t oblk = ((size_t)b * A.L + t0) * A.D + (size_t)(g * GC + (1 - part) * kFC);
+#pragma unroll
+    for (int k = 0; k < kFNLD; ++k) xo[k] = *(const uint4*)(A.x + oblk + (size_t)k * 128 * A.D + toff);
+  }
 
   // the per-state multipliers of the group's 64 channels (three lines per channel) go to LDS once
   {
     static_assert(kCmpQ32 == 0 && kCmpRS == 1 && kFTabs == 2, "tables 0..1 of the compact slot are staged");
-    const char* ibase = (const char*)A.image + (size_t)g * kFC * kImgRowBytes + kSlotCmp * 1024;
+    const char* ibase = (const char*)A.image + (size_t)cb * kImgRowBytes + kSlotCmp * 1024;
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int idx = it * kFT + tid;               // (table, channel, 16-byte piece)
@@ -238,10 +254,10 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const int c = tid >> 4, n = tid & 15;
     float2 v = make_float2(0.f, 0.f);
     if (n < A.N) {
-      v = *(const float2*)(A.h_in + (((size_t)b * A.D + g * kFC + c) * A.N + n) * 2);
+      v = *(const float2*)(A.h_in + (((size_t)b * A.D + cb + c) * A.N + n) * 2);
       if (!A.is_complex) v.y = 0.f;
     }
-    unsigned long long* e = A.rec + (brow * (A.S + 1) + A.S) * kFRecW + 4 + ((size_t)c * kNS + n) * 2;
+    unsigned long long* e = A.rec + (rrow * (A.S + 1) + A.S) * kFRecW + 4 + ((size_t)c * kNS + n) * 2;
     put_rec(e, tagged(__float_as_uint(v.x), tag));
     put_rec(e + 1, tagged(__float_as_uint(v.y), tag));
   }
@@ -256,8 +272,20 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       sm = dot2_ones<bf16_t>(w[i], sm);
       sq = dot2_self<bf16_t>(w[i], sq);
     }
-    const float m = group_sum<8>(sm) * (1.0f / kFC);
-    const float v = fmaxf(group_sum<8>(sq) * (1.0f / kFC) - m * m, 0.f);
+    if (kParts == 2) {
+      const uint32_t wo[4] = {xo[k].x, xo[k].y, xo[k].z, xo[k].w};
+      float so = 0.f, qo = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        so = dot2_ones<bf16_t>(wo[i], so);
+        qo = dot2_self<bf16_t>(wo[i], qo);
+      }
+      // lower half first in both workgroups
+      sm = part == 0 ? sm + so : so + sm;
+      sq = part == 0 ? sq + qo : qo + sq;
+    }
+    const float m = group_sum<8>(sm) * (1.0f / GC);
+    const float v = fmaxf(group_sum<8>(sq) * (1.0f / GC) - m * m, 0.f);
     if (piece == 0) {
       s_gm[k * 128 + tokl] = m;
       s_gv[k * 128 + tokl] = v;
@@ -314,7 +342,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     // earlier blocks of this (row, group): lane i fetches block i's aggregate
     Moments accp = {0.f, 0.f, 0.f};
     if (s > 0) {
-      const unsigned long long* rp = A.rec + (brow * (A.S + 1) + (lane < s ? lane : s - 1)) * kFRecW;
+      const unsigned long long* rp = A.rec + (rrow * (A.S + 1) + (lane < s ? lane : s - 1)) * kFRecW;
       unsigned long long w0, w1, w2;
       uint32_t spins = 0;
       for (;;) {
@@ -350,7 +378,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       s_gm[wave * 256 + lane * 4 + u] = full.mean;
       s_gv[wave * 256 + lane * 4 + u] = __builtin_amdgcn_rsqf(full.var + A.eps);
     }
-    if (s == A.S - 1 && wave == 3 && lane == 63) {
+    if (s == A.S - 1 && wave == 3 && lane == 63 && part == 0) {
       A.mean[brow] = full.mean;
       A.var[brow] = full.var;
       if (g == 0) A.count[b] = poison ? (int64_t)-1 : A.prev_count[b] + (int64_t)A.L;
@@ -363,7 +391,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   const uint32_t loff0 = (uint32_t)lane * 16;
   const uint32_t koff0 = (uint32_t)(((lane & 15) - 8 * (lane >> 4) + 24) * 16);
   auto load_p = [&](const int c, bf16x8 (&P)[kNWP][2]) {
-    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    const char* img = (const char*)A.image + (size_t)(cb + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
 #pragma unroll
@@ -372,7 +400,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       for (int mb = 0; mb < 2; ++mb) P[w][mb] = __builtin_bit_cast(bf16x8, img_slot(img, kSlotP + 2 * w + mb, loff));
   };
   auto load_kc = [&](const int c, bf16x8 (&K)[kNWK][2], bf16x8 (&C)[kNWC][2]) {
-    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    const char* img = (const char*)A.image + (size_t)(cb + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
     // K from the slot that holds each distinct vector once: 7 lines per term leave the cache instead of 16
@@ -468,7 +496,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     const char* rb = tile + row_base(c);
-    bf16_t* yr = A.y + (size_t)b * A.syb + (size_t)(g * kFC + c) * A.syd + t0;
+    bf16_t* yr = A.y + (size_t)b * A.syb + (size_t)(cb + c) * A.syd + t0;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int q = k * 64 + lane;                 // 16-byte chunk of the row: segment q >> 3, chunk q & 7
@@ -568,7 +596,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   load_kc(wave, Ka, Ca);
   float Jr[4] = {0.f, 0.f, 0.f, 0.f}, Ji[4] = {0.f, 0.f, 0.f, 0.f};
   auto load_j = [&](const int c) {
-    const char* img = (const char*)A.image + (size_t)(g * kFC + c) * kImgRowBytes;
+    const char* img = (const char*)A.image + (size_t)(cb + c) * kImgRowBytes;
     uint32_t loff = loff0;
     asm volatile("" : "+v"(loff));
     load_c4(img, kSlotRJ, loff, Jr, Ji);             // (q^64)^j
@@ -581,7 +609,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   float Cr[4] = {0.f, 0.f, 0.f, 0.f}, Ci[4] = {0.f, 0.f, 0.f, 0.f};
   if (nterms > 0) {
     const int cl = wave + kFW * (j >> 2);
-    const int chl = g * kFC + cl;
+    const int chl = cb + cl;
     int look = 0;                                  // blocks back that still reach this lane's channel
 #pragma unroll
     for (int i = 0; i < kFCPW; ++i) look = (j >> 2) == i ? nlook[i] : look;
@@ -594,7 +622,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       const int d = d0 + (j & 3);
       const bool have = d < nterms && d < look;
       const int slot = have ? (d < s ? s - 1 - d : A.S) : 0;
-      const unsigned long long* e = A.rec + (brow * (A.S + 1) + slot) * kFRecW + 4 + (size_t)cl * kNS * 2 + 4 * r;
+      const unsigned long long* e = A.rec + (rrow * (A.S + 1) + slot) * kFRecW + 4 + (size_t)cl * kNS * 2 + 4 * r;
       float Wr[4], Wi[4];
       load_c4(wimg, kSlotRWJ, (uint32_t)(((r << 4) | (have ? d : 0)) * 16), Wr, Wi);      // (q^1024)^d
       unsigned long long w[8];
@@ -638,7 +666,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   __builtin_amdgcn_wave_barrier();
   if (last_block && A.h_out && (j & 3) == 0) {
     const int cl = wave + kFW * (j >> 2);
-    const int ch = g * kFC + cl;
+    const int ch = cb + cl;
     float Rr[4], Ri[4];
     load_cmp((const char*)A.image + (size_t)ch * kImgRowBytes, kCmpRW, roff0, Rr, Ri);
 #pragma unroll
@@ -769,7 +797,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const int tl = tokl & ~1;
     const char* rbase = tile + row_base(piece * 8 + odd * 4) + (tl >> 6) * 128 + ((tl & 7) >> 1) * 4;
     const int c8 = (tl & 63) >> 3;
-    bf16_t* yb = A.y + (size_t)b * A.syb + (size_t)(g * kFC + piece * 8) * A.syd;
+    bf16_t* yb = A.y + (size_t)b * A.syb + (size_t)(cb + piece * 8) * A.syd;
 #pragma unroll
     for (int k = 0; k < kFNLD; ++k) {
       const int tok = k * 128 + tokl;
@@ -807,19 +835,20 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   }
 }
 
-size_t fused_ws_bytes(int64_t B, int64_t G, int64_t S) {
-  return align_up(sizeof(TsnHeader), 256) + align_up((size_t)B * G * (S + 1) * kFRecW * 8, 256);
+// R: record rows = workgroups per block = B * D / 64
+size_t fused_ws_bytes(int64_t R, int64_t S) {
+  return align_up(sizeof(TsnHeader), 256) + align_up((size_t)R * (S + 1) * kFRecW * 8, 256);
 }
 
 bool fused_covers(int dtype, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N, const void* x, const void* xn,
                   const void* y, int64_t syb, int64_t syd, int64_t syl, const uint8_t* mask, const float* h_in) {
-  if (dtype != MEGA_BF16 || mask || G <= 0 || D != G * kFC || N > kNS || N <= 0) return false;
+  if (dtype != MEGA_BF16 || mask || G <= 0 || (D != G * kFC && D != G * 2 * kFC) || N > kNS || N <= 0) return false;
   if (L <= 0 || L % kFSeg != 0 || L / kFSeg + (h_in ? 1 : 0) > kFMaxBlocks) return false;
   if (((uintptr_t)x % 16) || ((uintptr_t)xn % 16) || ((uintptr_t)y % 16)) return false;
   const bool rows = syl == 1 && syd % 8 == 0 && syb % 8 == 0;
   const bool lines = syd == 1 && syl % 8 == 0 && syb % 8 == 0;
   if (!rows && !lines) return false;
-  if (B * G * (L / kFSeg) >= (int64_t)1 << 31) return false;
+  if (B * (D / kFC) * (L / kFSeg) >= (int64_t)1 << 31) return false;
   return true;
 }
 
@@ -832,7 +861,7 @@ using namespace mega;
 extern "C" size_t mega_norm_ema_fwd_workspace_bytes(int64_t B, int64_t L, int64_t D, int64_t G, int64_t N) {
   (void)N;
   if (B <= 0 || L <= 0 || D <= 0 || G <= 0) return 256;
-  const size_t fused = fused_ws_bytes(B, G, ceil_div(L, kFSeg));
+  const size_t fused = fused_ws_bytes(B * ceil_div(D, kFC), ceil_div(L, kFSeg));
   const size_t tsn = mega_timestep_norm_workspace_bytes(MEGA_BF16, B, L, D, G);
   return fused > tsn ? fused : tsn;
 }
@@ -898,14 +927,17 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     A.hdr = (TsnHeader*)w; A.rec = (unsigned long long*)(w + align_up(sizeof(TsnHeader), 256));
     A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
     A.is_complex = is_complex;
-    A.xcd_map = (G % 8 == 0) ? 1 : 0;
+    const int parts = (int)(D / (G * kFC));              // workgroups per norm group
+    A.xcd_map = ((G * parts) % 8 == 0) ? 1 : 0;
     A.lb = lookback_launch(true);
-    const dim3 grid((unsigned)(B * G * S));
+    const dim3 grid((unsigned)(B * G * parts * S));
     typedef void (*Kern)(const FusedArgs);
     const int lout = syl == 1 ? 0 : 1;
-    const Kern kern = lout == 0 ? norm_ema_fused_kernel<0> : norm_ema_fused_kernel<1>;
-    static uint64_t attr_seen[2] = {0, 0};
-    if (first_on_device(&attr_seen[lout])) {
+    const Kern kerns[2][2] = {{norm_ema_fused_kernel<0, 64>, norm_ema_fused_kernel<1, 64>},
+                              {norm_ema_fused_kernel<0, 128>, norm_ema_fused_kernel<1, 128>}};
+    const Kern kern = kerns[parts - 1][lout];
+    static uint64_t attr_seen[2][2] = {{0, 0}, {0, 0}};
+    if (first_on_device(&attr_seen[parts - 1][lout])) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFSmem);
     }
     hipLaunchKernelGGL(kern, grid, dim3(kFT), kFSmem, s, A);

@@ -48,11 +48,14 @@ def _run(layer, x, G, nw, nb, prior=None, **kw):
 
 
 @pytest.mark.parametrize("out_layout", ["rows", "input"])
-@pytest.mark.parametrize("B,L,G,N,cplx", [(2, 1024, 2, 16, True), (1, 4096, 8, 16, True), (3, 2048, 1, 7, False),
-                                         (1, 3072, 16, 16, True)])
-def test_one_kernel_envelope_against_oracle(out_layout, B, L, G, N, cplx):
-    print(f"case out={out_layout} B={B} L={L} G={G} N={N} cplx={cplx}", flush=True)
-    D = 64 * G
+@pytest.mark.parametrize("B,L,G,N,cplx,cpg", [(2, 1024, 2, 16, True, 64), (1, 4096, 8, 16, True, 64),
+                                             (3, 2048, 1, 7, False, 64), (1, 3072, 16, 16, True, 64),
+                                             (2, 2048, 2, 16, True, 128), (1, 3072, 8, 9, False, 128),
+                                             (3, 1024, 1, 16, True, 128)])
+def test_one_kernel_envelope_against_oracle(out_layout, B, L, G, N, cplx, cpg):
+    """cpg: channels per norm group; groups of 128 channels are shared by two workgroups."""
+    print(f"case out={out_layout} B={B} L={L} G={G} N={N} cplx={cplx} cpg={cpg}", flush=True)
+    D = cpg * G
     rng = np.random.default_rng(51)
     p, q, g, om, nw, nb = _setup(rng, D, N, cplx)
     x, x64 = rounded(rng.normal(size=(B, L, D)) * 1.5 + 0.3, BF)
@@ -106,13 +109,14 @@ def test_config2_headline_shape():
     assert rel_err(np.real(host(h)), np.real(host(h2))) < 2e-3
 
 
+@pytest.mark.parametrize("cpg", [64, 128])
 @pytest.mark.parametrize("L1,L2", [(1024, 2048), (2048, 1024), (1024, 1000)])
-def test_carried_state_and_prior_statistics(L1, L2):
+def test_carried_state_and_prior_statistics(L1, L2, cpg):
     """Two chunks with the norm statistics and the moving-average state carried from the first call to the
     second equal one call on the whole sequence (the second chunk of the last case leaves the one-kernel
     envelope and runs as two operators out of the same workspace)."""
     B, G, N = 2, 4, 16
-    D, L = 64 * G, L1 + L2
+    D, L = cpg * G, L1 + L2
     rng = np.random.default_rng(52)
     p, q, g, om, nw, nb = _setup(rng, D, N)
     x, x64 = rounded(rng.normal(size=(B, L, D)) + 0.5, BF)
