@@ -72,6 +72,7 @@ struct FusedArgs {
   float* var;
   const float* gamma;    // [D] (weight + 1)
   const float* beta;     // [D]
+  const uint8_t* mask;   // [B, L], nonzero = padding: no part in the statistics, xn = 0; or null
   const uint4* image;    // [D][kImgSlots][64]
   const float* h_in;     // [B, D, N, 2] or null
   float* h_out;          // [B, D, N, 2] or null
@@ -232,6 +233,14 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     for (int k = 0; k < kFNLD; ++k) xo[k] = *(const uint4*)(A.x + oblk + (size_t)k * 128 * A.D + toff);
   }
 
+  // padding flags of the thread's eight tokens (bit k: token k * 128 + tokl)
+  uint32_t mbits = 0;
+  if (A.mask) {
+    const uint8_t* mrow = A.mask + (size_t)b * A.L + t0 + tokl;
+#pragma unroll
+    for (int k = 0; k < kFNLD; ++k) mbits |= (mrow[k * 128] != 0 ? 1u : 0u) << k;
+  }
+
   // the per-state multipliers of the group's 64 channels (three lines per channel) go to LDS once
   {
     static_assert(kCmpQ32 == 0 && kCmpRS == 1 && kFTabs == 2, "tables 0..1 of the compact slot are staged");
@@ -288,7 +297,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const float v = fmaxf(group_sum<8>(sq) * (1.0f / GC) - m * m, 0.f);
     if (piece == 0) {
       s_gm[k * 128 + tokl] = m;
-      s_gv[k * 128 + tokl] = v;
+      s_gv[k * 128 + tokl] = ((mbits >> k) & 1u) ? -1.f : v;        // a negative variance marks padding
     }
   }
   __syncthreads();
@@ -300,11 +309,12 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const float4 m4 = *(const float4*)(s_gm + wave * 256 + lane * 4);
     const float4 v4 = *(const float4*)(s_gv + wave * 256 + lane * 4);
     const float mm[4] = {m4.x, m4.y, m4.z, m4.w}, vv[4] = {v4.x, v4.y, v4.z, v4.w};
-    Moments st = {1.f, mm[0], vv[0]};
+    // padding counts for nothing: weight 0 (the merges keep the other side's statistics)
+    Moments st = {vv[0] >= 0.f ? 1.f : 0.f, mm[0], fmaxf(vv[0], 0.f)};
     pref[0] = st;
 #pragma unroll
     for (int u = 1; u < 4; ++u) {
-      st = merge(st, Moments{1.f, mm[u], vv[u]});
+      st = merge(st, Moments{vv[u] >= 0.f ? 1.f : 0.f, mm[u], fmaxf(vv[u], 0.f)});
       pref[u] = st;
     }
     const Moments inc = row_scan(st);
@@ -381,7 +391,8 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     if (s == A.S - 1 && wave == 3 && lane == 63 && part == 0) {
       A.mean[brow] = full.mean;
       A.var[brow] = full.var;
-      if (g == 0) A.count[b] = poison ? (int64_t)-1 : A.prev_count[b] + (int64_t)A.L;
+      // tokens that count: whole numbers below 2^24, exact in the float sums
+      if (g == 0) A.count[b] = poison ? (int64_t)-1 : A.prev_count[b] + (int64_t)(accp.n + tot.n);
     }
   }
   __syncthreads();
@@ -437,7 +448,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 #pragma unroll
     for (int i = 0; i < 8; ++i) plain = plain && gam[i] == 1.f && bet[i] == 0.f;
     const bool ident = __all(plain);
-    auto stage = [&](auto IDENT) {
+    auto stage = [&](auto IDENT, auto MASKED) {
 #pragma unroll
     for (int k = 0; k < kFNLD; ++k) {
       const int tok = k * 128 + tokl;
@@ -452,6 +463,11 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
         o[i] = decltype(IDENT)::value ? pack_bf16(lo, hi)
                                       : pack_bf16(fmaf(lo, gam[2 * i], bet[2 * i]), fmaf(hi, gam[2 * i + 1], bet[2 * i + 1]));
       }
+      if (decltype(MASKED)::value) {
+        const bool pad = (mbits >> k) & 1u;                 // padding leaves as zeros, whatever x holds there
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = pad ? 0u : o[i];
+      }
       store_stream((uint4*)(A.xn + xblk + (size_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
       const uint32_t s0 = odd ? o[0] : o[2], s1 = odd ? o[1] : o[3];
       const uint32_t r0 = dpp_u<0x128>(s0), r1 = dpp_u<0x128>(s1);       // row_ror:8 = the partner token's lane
@@ -463,10 +479,16 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       *(uint32_t*)(wp + 3 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_hi);
     }
     };
-    if (ident) {
-      stage(std::true_type{});
+    if (A.mask) {
+      if (ident) {
+        stage(std::true_type{}, std::true_type{});
+      } else {
+        stage(std::false_type{}, std::true_type{});
+      }
+    } else if (ident) {
+      stage(std::true_type{}, std::false_type{});
     } else {
-      stage(std::false_type{});
+      stage(std::false_type{}, std::false_type{});
     }
   }
   __syncthreads();
@@ -842,7 +864,8 @@ size_t fused_ws_bytes(int64_t R, int64_t S) {
 
 bool fused_covers(int dtype, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N, const void* x, const void* xn,
                   const void* y, int64_t syb, int64_t syd, int64_t syl, const uint8_t* mask, const float* h_in) {
-  if (dtype != MEGA_BF16 || mask || G <= 0 || (D != G * kFC && D != G * 2 * kFC) || N > kNS || N <= 0) return false;
+  (void)mask;
+  if (dtype != MEGA_BF16 || G <= 0 || (D != G * kFC && D != G * 2 * kFC) || N > kNS || N <= 0) return false;
   if (L <= 0 || L % kFSeg != 0 || L / kFSeg + (h_in ? 1 : 0) > kFMaxBlocks) return false;
   if (((uintptr_t)x % 16) || ((uintptr_t)xn % 16) || ((uintptr_t)y % 16)) return false;
   const bool rows = syl == 1 && syd % 8 == 0 && syb % 8 == 0;
@@ -923,7 +946,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     FusedArgs A;
     A.x = (const bf16_t*)x; A.xn = (bf16_t*)xn; A.y = (bf16_t*)y; A.syb = syb; A.syd = syd; A.syl = syl;
     A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var; A.count = count; A.mean = mean;
-    A.var = var; A.gamma = norm_gamma; A.beta = norm_beta; A.image = (const uint4*)img; A.h_in = h_in; A.h_out = h_out;
+    A.var = var; A.gamma = norm_gamma; A.beta = norm_beta; A.mask = mask; A.image = (const uint4*)img; A.h_in = h_in; A.h_out = h_out;
     A.hdr = (TsnHeader*)w; A.rec = (unsigned long long*)(w + align_up(sizeof(TsnHeader), 256));
     A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
     A.is_complex = is_complex;

@@ -164,7 +164,7 @@ def test_slowly_decaying_poles_across_blocks(mixed):
     assert rel_err(np.real(host(h)), np.real(ho)) < 2e-3
 
 
-@pytest.mark.parametrize("dtype,B,L,D,G,masked", [(BF, 2, 700, 128, 2, False), (BF, 2, 1024, 128, 2, True),
+@pytest.mark.parametrize("dtype,B,L,D,G,masked", [(BF, 2, 700, 128, 2, False), (BF, 2, 1000, 128, 2, True),
                                                   (torch.float32, 1, 1024, 64, 1, False), (BF, 1, 2048, 96, 3, False)])
 def test_outside_the_envelope_runs_two_operators(dtype, B, L, D, G, masked):
     rng = np.random.default_rng(54)
@@ -187,6 +187,47 @@ def test_outside_the_envelope_runs_two_operators(dtype, B, L, D, G, masked):
 
 
 M_TOL = {torch.float32: 1e-4, BF: 2e-2}
+
+
+@pytest.mark.parametrize("out_layout", ["rows", "input"])
+@pytest.mark.parametrize("B,L,G,cpg,affine", [(3, 3072, 2, 64, True), (2, 2048, 1, 128, False), (4, 1024, 8, 64, True)])
+def test_one_kernel_with_padding_mask(out_layout, B, L, G, cpg, affine):
+    """Padding inside the one-kernel envelope: masked tokens take no part in the running statistics and leave the norm
+    as zeros (timestep_norm.cc:283-311), the moving average sees those zeros.  The masks: a padded tail, a row that
+    starts padded, a whole block of 1024 padded tokens in the middle of a row, single tokens, and a row without
+    padding."""
+    print(f"case out={out_layout} B={B} L={L} G={G} cpg={cpg} affine={affine}", flush=True)
+    D, N = cpg * G, 16
+    rng = np.random.default_rng(57)
+    p, q, g, om, nw, nb = _setup(rng, D, N)
+    if not affine:
+        nw, nb = np.zeros(D), np.zeros(D)
+    x, x64 = rounded(rng.normal(size=(B, L, D)) * 1.3 - 0.2, BF)
+    mask = np.zeros((B, L), bool)
+    mask[0, L - 300:] = True
+    mask[1, :70] = True
+    mask[1, 500:503] = True
+    if B > 2 and L >= 3072:
+        mask[2, 1024:2048] = True
+    mask[-1, ::97] |= B > 3
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+    xn, y, cnt, mean, var, h = _run(layer, x, G, nw, nb, padding_mask=dev(mask, torch.bool), out_layout=out_layout,
+                                    want_state=True)
+    xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, mask, G)
+    assert rel_err(host(xn), xno) < 2e-2
+    assert np.array_equal(host(xn)[mask], np.zeros_like(host(xn)[mask]))
+    assert cnt.tolist() == c.tolist()
+    assert rel_err(host(mean), mu) < 1e-4 and rel_err(host(var), v) < 1e-4
+    yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, mask, incremental=True)
+    _check_y(y, yo)
+    assert rel_err(np.real(host(h)), np.real(ho)) < 2e-3 and rel_err(np.imag(host(h)), np.imag(ho)) < 2e-3
+    # and the two operators on the same input
+    xn2 = M.ops.group_timestep_norm_fwd(x, torch.zeros(B, dtype=torch.int64, device=DEV), torch.zeros(B, G, device=DEV),
+                                        torch.ones(B, G, device=DEV), dev(nw + 1), dev(nb), dev(mask, torch.bool), G, 1e-5,
+                                        need_stats=False)[0]
+    y2, _ = layer(xn2.transpose(1, 2), dev(mask, torch.bool))
+    torch.cuda.synchronize()
+    assert rel_err(host(xn), host(xn2)) < 1e-2 and rel_err(host(y), host(y2)) < 2e-2
 
 
 def test_kernel_generation_inside_the_call():
