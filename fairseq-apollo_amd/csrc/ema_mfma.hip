@@ -12,9 +12,9 @@
 // fairseq/csrc/ops/ema_parameters.cc:37-77) applied per tile.  K, P, C are 32x32 matrices that
 // depend on the channel only.
 //
-// Kernel generation (ema_image_kernel): one wave per coefficient row builds a q-power table in
-// LDS and from it the MFMA A-operand images of K, P, C (bf16, optionally with a second bf16
-// correction term) plus the per-state multipliers q^32 and q^(32 SEGT).  The image is what the
+// Kernel generation (ema_image_kernel): a workgroup of four waves per coefficient row; every wave builds the
+// q-power table in LDS and the waves share out what is formed from it: the MFMA A-operand images of K, P, C
+// (bf16, optionally with a second bf16 correction term) plus the per-state multipliers q^32 and q^(32 SEGT).  The image is what the
 // reference caches as `_coeffs` / recomputes as the D x L kernel; here it is 9-13 KB per channel
 // whatever L is.
 //
@@ -86,9 +86,7 @@ __device__ __forceinline__ cfloat to_cfloat(cdouble a) { return {(float)a.re, (f
 __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageArgs A) {
   __shared__ __attribute__((aligned(16))) char smem[kPrepWaves * (kPowB + kAuxB)];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int kr_raw = blockIdx.x * kPrepWaves + wave;
-  const bool ok = kr_raw < A.K;
-  const int kr = ok ? kr_raw : A.K - 1;
+  const int kr = blockIdx.x;                        // one coefficient row per workgroup, shared by its four waves
   const int lag = (kr >= A.D && A.lag_back) ? 1 : 0;
   float2* pw = (float2*)(smem + wave * kPowB);
   float* kkt = (float*)(smem + kPrepWaves * kPowB + wave * kAuxB);   // [64]: k[idx] at kkt[32 + idx]
@@ -149,89 +147,60 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
   __syncthreads();
   uint4* img = A.image + (size_t)kr * kImgSlots * 64;
   const int m = lane & 15, g = lane >> 4;
-  if (!ok) return;                                 // (no barrier follows)
   // ---- the K / P / C operands in the matrix-core A layout: bf16 terms (kImgKFull: K, kImgPC: P and C) and fp16 terms
-  // (kImgF16); only what the caller's kernel reads is formed and written
+  // (kImgF16); only what the caller's kernel reads is formed and written.  The four waves of the workgroup hold the
+  // same tables and share the channel's work: wave 0 the P operand and the per-state tables, wave 1 the C operand,
+  // wave 2 the K operand (full and compact), wave 3 the multipliers of the block kernels.
   const bool want_k = A.parts & kImgKFull, want_pc = A.parts & kImgPC, want_16 = A.parts & kImgF16;
-  if (want_k || want_pc || want_16) {
-    bf16x8 Kw[kNWK][2], Pw[kNWP][2], Cw[kNWC][2];
-    typedef __attribute__((ext_vector_type(8))) _Float16 f16x8v;
-    f16x8v H16[3][2][2];                    // K, P, C as two fp16 terms
+  typedef __attribute__((ext_vector_type(8))) _Float16 f16x8v;
+  // value of operand `o` (0: K, 1: P, 2: C) at row `row`, k-slot t of block g
+  auto value = [&](const int o, const int row, const int t) -> float {
+    const int k = 8 * g + t;
+    if (o == 0) return kkt[32 + row - k];                  // K: rows = output time, k = input time (Toeplitz)
+    if (o == 1) {                                          // P: rows = (state, part), k = input time i: p q^{31-i}
+      const int n = row >> 1, part = row & 1;
+      const float2 w = pw[(31 - k) * kNS + n];
+      return pbuf[n] * (part ? w.y : w.x);
+    }
+    // C: rows = output time i; k-slot t of block g <-> state 2g + t/2 (t < 4) or 8 + 2g + (t-4)/2, part t & 1:
+    // Re(gamma q^{i+1-lag}) multiplies Re h, -Im(...) multiplies Im h
+    const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
+    const float2 w = pw[(row + 1 - lag) * kNS + n];
+    const float2 gm = gbuf[n];
+    return (t & 1) ? -(gm.x * w.y + gm.y * w.x) : (gm.x * w.x - gm.y * w.y);
+  };
+  auto build = [&](const int o, const int nw, const int slot, const bool want_bf, const int slot16) {
+    if (!want_bf && !want_16) return;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
-      const int row = 16 * mb + m;
+      bf16x8 hi8, lo8;
+      f16x8v h0, h1;
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const int k = 8 * g + t;
-        // K: rows = output time, k = input time (Toeplitz)
-        const float kv = kkt[32 + row - k];
-        // P: rows = (state, part), k = input time i: p q^{31-i}
-        float pv;
-        {
-          const int n = row >> 1, part = row & 1;
-          const float2 w = pw[(31 - k) * kNS + n];
-          pv = pbuf[n] * (part ? w.y : w.x);
-        }
-        // C: rows = output time i; k-slot t of block g <-> state 2g + t/2 (t < 4) or 8 + 2g + (t-4)/2,
-        // part t & 1: Re(gamma q^{i+1-lag}) multiplies Re h, -Im(...) multiplies Im h
-        float cv;
-        {
-          const int n = (t < 4) ? (2 * g + (t >> 1)) : (8 + 2 * g + ((t - 4) >> 1));
-          const int part = t & 1;
-          const float2 w = pw[(row + 1 - lag) * kNS + n];
-          const float2 gm = gbuf[n];
-          const float re = gm.x * w.x - gm.y * w.y;
-          const float im = gm.x * w.y + gm.y * w.x;
-          cv = part ? -im : re;
-        }
+        const float v = value(o, 16 * mb + m, t);
         __bf16 h;
-        float rem = bf_split(kv, &h);
-        Kw[0][mb][t] = h;
-        if (kNWK > 1) Kw[kNWK - 1][mb][t] = (__bf16)rem;
-        rem = bf_split(pv, &h);
-        Pw[0][mb][t] = h;
-        if (kNWP > 1) Pw[kNWP - 1][mb][t] = (__bf16)rem;
-        rem = bf_split(cv, &h);
-        Cw[0][mb][t] = h;
-        if (kNWC > 1) Cw[kNWC - 1][mb][t] = (__bf16)rem;
-        {
-          const float vals[3] = {kv, pv, cv};
-#pragma unroll
-          for (int o = 0; o < 3; ++o) {
-            const _Float16 h16 = (_Float16)vals[o];
-            H16[o][0][mb][t] = h16;
-            H16[o][1][mb][t] = (_Float16)(vals[o] - (float)h16);
-          }
-        }
+        const float rem = bf_split(v, &h);
+        hi8[t] = h;
+        lo8[t] = (__bf16)rem;
+        const _Float16 h16 = (_Float16)v;
+        h0[t] = h16;
+        h1[t] = (_Float16)(v - (float)h16);
+      }
+      if (want_bf) {
+        img[(slot + mb) * 64 + lane] = __builtin_bit_cast(uint4, hi8);
+        if (nw > 1) img[(slot + 2 * (nw - 1) + mb) * 64 + lane] = __builtin_bit_cast(uint4, lo8);
+      }
+      if (want_16) {
+        img[(size_t)(slot16 + mb) * 64 + lane] = __builtin_bit_cast(uint4, h0);
+        img[(size_t)(slot16 + 2 + mb) * 64 + lane] = __builtin_bit_cast(uint4, h1);
       }
     }
-    if (want_k) {
-#pragma unroll
-      for (int w = 0; w < kNWK; ++w)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(kSlotK + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Kw[w][mb]);
-    }
-    if (want_pc) {
-#pragma unroll
-      for (int w = 0; w < kNWP; ++w)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(kSlotP + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Pw[w][mb]);
-#pragma unroll
-      for (int w = 0; w < kNWC; ++w)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) img[(kSlotC + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, Cw[w][mb]);
-    }
-    if (want_16) {
-#pragma unroll
-      for (int o = 0; o < 3; ++o)
-#pragma unroll
-        for (int w = 0; w < 2; ++w)
-#pragma unroll
-          for (int mb = 0; mb < 2; ++mb)
-            img[(size_t)(kSlotK16 + 4 * o + 2 * w + mb) * 64 + lane] = __builtin_bit_cast(uint4, H16[o][w][mb]);
-    }
-  }
-  if (A.parts & kImgStream) {
+  };
+  static_assert(kNWK <= 2 && kNWP <= 2 && kNWC <= 2, "operands of one or two bf16 terms");
+  if (wave == 0) build(1, kNWP, kSlotP, want_pc, kSlotK16 + 4);
+  if (wave == 1) build(2, kNWC, kSlotC, want_pc, kSlotK16 + 8);
+  if (wave == 2) build(0, kNWK, kSlotK, want_k, kSlotK16);
+  if (wave == 0 && (A.parts & kImgStream)) {
     // q^32 of this lane's four states (2r, 2r+1, 8+2r, 9+2r)
     const float2 a = pw[32 * kNS + 2 * r], bq = pw[32 * kNS + 2 * r + 1];
     const float2 c = pw[32 * kNS + 8 + 2 * r], d = pw[32 * kNS + 9 + 2 * r];
@@ -246,7 +215,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     const cfloat R = to_cfloat(Rd);
     img[kSlotScan * 64 + lane] = make_uint4(__float_as_uint(R.re), __float_as_uint(R.im), 0u, 0u);
   }
-  if (A.parts & kImgBlocks) {
+  if (wave == 3 && (A.parts & kImgBlocks)) {
     // multipliers in the matrix-core lane layout (lane = segment j + 16 r, states 2r, 2r+1, 8+2r, 9+2r), for the
     // kernels that scan 16 segments of 64 tokens across the lanes of a row and look back over blocks of 1024 tokens:
     // (q^64)^j and (q^1024)^j, each power by squaring and multiplying (at most eight products in a row)
@@ -281,7 +250,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
     put2(kSlotRWJ, RWJ);
   }
   {
-    if (lane < kNS) {
+    if (wave == 0 && lane < kNS) {
       // the per-state multipliers once per state (a lane of the streaming kernels reads 16 bytes = two states)
       float2* cmp = (float2*)(img + (size_t)kSlotCmp * 64);
       const double2 w32 = q32d[lane];
@@ -298,7 +267,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
       v = cmuld(v, v);
       cmp[kCmpRW * kNS + lane] = make_float2((float)v.re, (float)v.im);
     }
-    if (lane < 56 && (A.parts & kImgKT)) {
+    if (wave == 2 && lane < 56 && (A.parts & kImgKT)) {
       // the K operand once per distinct content: lane (m, g) of row block mb holds k[16 mb + m - 8 g - t], t = 0..7,
       // which depends on delta = 16 mb + m - 8 g (-24..31) only; vector delta + 24 of term w sits at byte
       // 16 (delta + 24) of slot kSlotKT + w (7 lines per term instead of 16)
@@ -336,7 +305,7 @@ __global__ __launch_bounds__(kPrepWaves * 64) void ema_image_kernel(const ImageA
         w *= md;
         ++nlook;
       }
-      if (lane == 0) {
+      if (wave == 0 && lane == 0) {
         uint32_t* rw = (uint32_t*)(img + (size_t)kSlotCmp * 64) + kCmpReach * kNS * 2;
         rw[0] = (uint32_t)nsteps;
         rw[1] = (uint32_t)nlook;
@@ -964,7 +933,7 @@ int ema_image_build(const float* p, const float* q, const float* gamma, int is_c
   A.p = p; A.q = q; A.gamma = gamma; A.omega = omega; A.image = (uint4*)image;
   A.K = (int)(bidirectional ? 2 * D : D); A.D = (int)D; A.N = (int)N; A.is_complex = is_complex;
   A.lag_back = shift ? 1 : 0;
-  hipLaunchKernelGGL(ema_image_kernel, dim3((unsigned)ceil_div(A.K, kPrepWaves)), dim3(kPrepWaves * 64), 0, s, A);
+  hipLaunchKernelGGL(ema_image_kernel, dim3((unsigned)A.K), dim3(kPrepWaves * 64), 0, s, A);
   MEGA_CHECK_LAUNCH("ema kernel generation");
   return MEGA_OK;
 }
