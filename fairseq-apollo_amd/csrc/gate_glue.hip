@@ -16,8 +16,9 @@ namespace {
 constexpr int kRowThreads = 256;                 // 4 waves, one token each
 constexpr int kRowsPerWg = kRowThreads / 64;
 
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// hardware reciprocal (1 ulp) in the place of a full division
+__device__ __forceinline__ float silu_f(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
