@@ -96,6 +96,49 @@ def test_config3_b64_d2048_2048_steps():
     assert rel_err(host(y_s[sel]), yo.transpose(0, 2, 1)) < 1e-4
 
 
+def test_config3_bf16_full_width():
+    """configs[3] in its own arithmetic: 64 streams, D = 2048, N = 16, bf16 activations, 512 consecutive single-token
+    steps and then the same tokens as launches of 64; a sample of streams against the fp64 oracle (the norm on the
+    bf16 inputs, the moving average on the bf16 xn the step produced, as a layer behind it would see it), every stream
+    against the parallel path in bf16."""
+    B, D, N, G, T = 64, 2048, 16, 16, 512
+    rng, p, q, g, om, nw, nb = _setup(B, D, N, G, 1241)
+    gen = torch.Generator().manual_seed(1241)
+    x = torch.randn(B, T, D, generator=gen).to(torch.bfloat16).to(DEV)
+    step = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    xn_s = torch.empty_like(x)
+    y_s = torch.empty_like(x)
+    for t in range(T):
+        xn_s[:, t], y_s[:, t] = step(x[:, t])
+    torch.cuda.synchronize()
+    sel = [0, 21, 42, 63]
+    x64 = x[sel].double().cpu().numpy()
+    xno, c_o, mu_o, v_o = O.timestep_norm(x64, np.zeros(4, np.int64), np.zeros((4, G)), np.ones((4, G)), nw + 1, nb, None, G)
+    assert rel_err(host(xn_s[sel]), xno) < 2e-2
+    assert step.count[sel].tolist() == c_o.tolist() == [T] * 4
+    assert rel_err(host(step.mean[sel]), mu_o) < 1e-4 and rel_err(host(step.var[sel]), v_o) < 1e-4
+    yo, ho = O.ema_forward(host(xn_s[sel]).transpose(0, 2, 1), p, q, g, om, incremental=True)
+    assert rel_err(host(y_s[sel]), yo.transpose(0, 2, 1)) < 2e-2
+    assert rel_err(np.real(host(step.state[sel])), np.real(ho)) < 2e-3
+    # the parallel path on the whole batch
+    norm = M.TimestepNorm(D, G).to(DEV).eval()
+    with torch.no_grad():
+        norm.weight.copy_(dev(nw)); norm.bias.copy_(dev(nb))
+        xn_p = norm(x, None, {})
+        # the moving average on the xn the steps produced: both paths then see the same bf16 inputs
+        y_p, _ = M.ops.ema_forward(xn_s.transpose(1, 2), dev(p), dev(q), dev(g), dev(om))
+    torch.cuda.synchronize()
+    # two bf16 paths against each other (each is held to 2e-2 of the fp64 result above): 3e-2
+    assert rel_err(host(xn_s), host(xn_p)) < 2e-2 and rel_err(host(y_s), host(y_p.transpose(1, 2))) < 3e-2
+    # the same tokens, 64 per launch
+    step2 = M.ops.DecodeStep(dev(nw), dev(nb), G, 1e-5, dev(p), dev(q), dev(g), dev(om), B)
+    outs = [step2.steps(x[:, a:a + 64]) for a in range(0, T, 64)]
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    assert rel_err(host(torch.cat([o[0] for o in outs], 1)), host(xn_s)) < 2e-2
+    assert rel_err(host(torch.cat([o[1] for o in outs], 1)), host(y_s)) < 2e-2
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
 @pytest.mark.parametrize("B,D,N,G,chunks", [(3, 96, 16, 4, (1, 7, 64, 65, 130)), (2, 256, 8, 2, (16, 16)),
                                             (5, 64, 4, 1, (3, 200))])
