@@ -241,7 +241,9 @@ extern "C" int mega_attention_fwd(const void* q, const void* k, const void* v, v
                (double)dropout);
   MEGA_REQUIRE(B >= 0 && L >= 0 && Nh > 0 && H1 > 0 && H2 > 0, MEGA_ERR_ARG, "attention_fwd: bad shape");
   if (B == 0 || L == 0) return MEGA_OK;
-  MEGA_REQUIRE(q && k && v && y, MEGA_ERR_ARG, "attention_fwd: null pointer argument");
+  MEGA_REQUIRE(q && k && v && (y || w), MEGA_ERR_ARG, "attention_fwd: null pointer argument");
+  MEGA_REQUIRE(y || attention_mfma_covers(dtype, q, k, v, B, L, Nh, H1, H2), MEGA_ERR_UNSUPPORTED,
+               "attention_fwd: the weights alone (y = NULL) are formed on the matrix-core path only");
   MEGA_REQUIRE(B * L * Nh < (int64_t)1 << 31, MEGA_ERR_UNSUPPORTED, "attention_fwd: too many rows");
   if (attention_mfma_covers(dtype, q, k, v, B, L, Nh, H1, H2)) {
     const size_t need = attention_mfma_workspace_bytes(dtype, B, L, Nh, H2);

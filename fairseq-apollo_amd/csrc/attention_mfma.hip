@@ -1119,7 +1119,7 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
   // v enters the second product through its columns: read in place (K-major form of the kernel) when its rows are
   // whole 16-byte pieces, through a transposed, zero-padded copy otherwise
   const bool v_inplace = H2 % 8 == 0 && ((uintptr_t)v % 16) == 0;
-  if (!v_inplace) {
+  if (!v_inplace && y) {
     const dim3 grid((unsigned)ceil_div(Lp, 64), (unsigned)ceil_div(H2, 64), (unsigned)BN_);
     hipLaunchKernelGGL(transpose_v_kernel<T>, grid, dim3(256), 0, s, (const T*)v, Vt, (int)L, (int)Nh, (int)H2, (int)Lp,
                        0);
@@ -1141,6 +1141,10 @@ int run_attention(const void* q, const void* k, const void* v, void* y, void* w,
     // the weights the reference returns: [B, Nh, L, L]
     hipMemcpy2DAsync(w, (size_t)L * sizeof(T), P, (size_t)Lp * sizeof(T), (size_t)L * sizeof(T), (size_t)(BN_ * L),
                      hipMemcpyDeviceToDevice, s);
+  }
+  if (!y) {                                        // the weights alone (a backward that forms them again)
+    MEGA_CHECK_LAUNCH("attention_fwd (weights)");
+    return MEGA_OK;
   }
   // y[b,:,n,:] = P[b,n] v[b,:,n,:]  ==  P (v^T)^T
   G.A = P; G.C = y;

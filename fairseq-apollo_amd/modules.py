@@ -698,23 +698,38 @@ class AttentionSoftmaxFunc(torch.autograd.Function):
 
 
 class AttentionFunc(torch.autograd.Function):
-    """fairseq/modules/efficient_attention.py:11-40: the forward keeps the L x L weights (after
-    DropKey) for the backward pass, as the reference does.  `seed` (not in the reference) pins
-    the mask."""
+    """fairseq/modules/efficient_attention.py:11-40.  The reference's forward keeps the L x L weights (after
+    DropKey) for the backward pass.  Here they are kept only with DropKey or outside the matrix-core envelope;
+    otherwise the forward is the one-kernel attention (no L x L array at all), q, k, v and y are saved, and the backward
+    forms the weights again in scratch memory before its four products: B Nh L^2 elements less to hold per layer
+    between the passes (134 MB at configs[4]), the same gradients.  `KEEP_WEIGHTS = True` restores the reference's
+    behaviour.  `seed` (not in the reference) pins the DropKey mask."""
+
+    KEEP_WEIGHTS = False
 
     @staticmethod
     def forward(ctx, q, k, v, scale: float = 1.0, dropout: float = 0.0, use_causal_mask: bool = True,
                 training: bool = True, seed=None):
-        y, w = ops.attention_fwd(q, k, v, scale, dropout if training else 0.0, use_causal_mask, need_weights=True,
-                                 seed=seed)
-        ctx.save_for_backward(q, k, v, w, y)          # y: lets the backward form the softmax's row sums as y_grad . y
+        drop = dropout if training else 0.0
         ctx.scale = scale
         ctx.use_causal_mask = use_causal_mask
+        if not AttentionFunc.KEEP_WEIGHTS and ops.attention_keeps_no_weights(q, k, v, drop):
+            y, _ = ops.attention_fwd(q, k, v, scale, 0.0, use_causal_mask, need_weights=False)
+            ctx.save_for_backward(q, k, v, y)
+            ctx.has_weights = False
+            return y
+        y, w = ops.attention_fwd(q, k, v, scale, drop, use_causal_mask, need_weights=True, seed=seed)
+        ctx.save_for_backward(q, k, v, w, y)          # y: lets the backward form the softmax's row sums as y_grad . y
+        ctx.has_weights = True
         return y
 
     @staticmethod
     def backward(ctx, y_grad):
-        q, k, v, w, y = ctx.saved_tensors
+        if ctx.has_weights:
+            q, k, v, w, y = ctx.saved_tensors
+        else:
+            q, k, v, y = ctx.saved_tensors
+            _, w = ops.attention_fwd(q, k, v, ctx.scale, 0.0, ctx.use_causal_mask, weights_only=True)
         q_grad, k_grad, v_grad = ops.attention_bwd(y_grad, q, k, v, w, ctx.scale, ctx.use_causal_mask, y=y)
         return q_grad, k_grad, v_grad, None, None, None, None, None
 

@@ -462,11 +462,13 @@ def attention_softmax_fwd(x: torch.Tensor, dropout: float, use_causal_mask: bool
 
 
 def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, need_weights: bool = False,
-                  seed: Optional[int] = None):
+                  seed: Optional[int] = None, weights_only: bool = False):
     """-> (y[B,L,Nh,H2], w[B,Nh,L,L] or None).  Reference: attention_fwd,
     fairseq/csrc/ops/attention_kernel.cu:40-131; the L x L weights are only written on request.
     `dropout` is DropKey on the scaled scores, `seed` names the mask (shared with
-    attention_softmax_fwd on the [B,Nh,L,L] scores)."""
+    attention_softmax_fwd on the [B,Nh,L,L] scores).  `weights_only`: -> (None, w), the second product is not
+    formed (what a backward that did not keep the weights asks for; matrix-core shapes only)."""
+    need_weights = need_weights or weights_only
     seed = _dropkey_seed(dropout, seed)
     dev = _need_gpu(q, k, v)
     lib = _lib.load()
@@ -477,7 +479,7 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
         raise RuntimeError("attention_fwd: q, k, v must share one dtype")
     B, L, Nh, H1 = qd.shape
     H2 = vd.shape[3]
-    y = torch.empty(B, L, Nh, H2, dtype=qd.dtype, device=dev)
+    y = None if weights_only else torch.empty(B, L, Nh, H2, dtype=qd.dtype, device=dev)
     w = torch.empty(B, Nh, L, L, dtype=qd.dtype, device=dev) if need_weights else None
     nws = lib.mega_attention_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2)
     ws = _scratch_buffer(dev, nws) if nws else None
@@ -508,6 +510,19 @@ def attention_softmax_bwd(y_grad: torch.Tensor, y: torch.Tensor, use_causal_mask
                                             1 if use_causal_mask else 0, float(scale), _stream(dev))
     _lib.check(rc, "attention_softmax_bwd")
     return dx
+
+
+def attention_keeps_no_weights(q, k, v, dropout: float) -> bool:
+    """True when a training forward of these operands can leave the L x L weights unsaved: no DropKey, and a shape
+    whose weights the matrix-core path can form again in the backward."""
+    if dropout > 0.0 or q.dim() != 4 or q.dtype == torch.float32 or not q.is_cuda:
+        return False
+    B, L, Nh, H1 = q.shape
+    H2 = v.shape[3]
+    lib = _lib.load()
+    dt = _dtype_code(q)
+    return bool(lib.mega_attention_workspace_bytes(dt, B, L, Nh, H1, H2)) and \
+        bool(lib.mega_attention_bwd_workspace_bytes(dt, B, L, Nh, H1, H2))
 
 
 def attention_bwd(y_grad, q, k, v, w, scale: float, use_causal_mask: bool, y=None):

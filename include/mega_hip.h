@@ -439,7 +439,8 @@ int mega_attention_softmax_bwd(const void* y_grad, const void* y, void* x_grad, 
 /* stands in for attention_fwd (fairseq/csrc/ops/attention_kernel.cu:40-131, 257-276):
  *   q, k [B,L,Nh,H1]; v, y [B,L,Nh,H2] contiguous of `dtype`;
  *   y[b,:,n,:] = softmax_causal(scale q k^T) v per (b, n).  The L x L weights are
- *   not returned unless w != NULL (w [B,Nh,L,L] of `dtype`).
+ *   not returned unless w != NULL (w [B,Nh,L,L] of `dtype`).  y = NULL with w != NULL forms the weights
+ *   alone (matrix-core path only, MEGA_ERR_UNSUPPORTED otherwise): for a backward that did not keep them.
  *   dropout, seed: DropKey on the scaled scores, as in mega_attention_softmax_fwd; element
  *   e is the score's place in the [B,Nh,L,L] weights.
  *   16-bit activations with H1 % 8 == 0 run on the matrix cores and need the workspace

@@ -766,3 +766,42 @@ def test_attention_dropkey_autograd(dtype, tol):
     ref = O.attention_softmax_bwd(g64, host(yy))
     assert rel_err(host(xg.grad), ref) < TOL[dtype]
     assert np.all(host(xg.grad)[O.dropkey_draws(seed, (3, 20, 20)) < p] == 0)
+
+
+@pytest.mark.parametrize("B,L,Nh,H1,H2,causal", [(2, 256, 2, 64, 128, True), (1, 520, 1, 32, 64, True),
+                                                 (2, 128, 4, 16, 24, False)])
+def test_attention_backward_without_kept_weights(B, L, Nh, H1, H2, causal):
+    """Training through the fused attention without keeping the L x L weights between the passes (the forward is
+    the one-kernel attention, the backward forms the weights again): same output and same gradients as with the
+    reference's kept weights, to the rounding of the 16-bit output; and the saved tensors hold no L x L array."""
+    torch.manual_seed(77)
+    q, k = (torch.randn(B, L, Nh, H1, device=DEV).to(torch.bfloat16) for _ in range(2))
+    v = torch.randn(B, L, Nh, H2, device=DEV).to(torch.bfloat16)
+    dy = torch.randn(B, L, Nh, H2, device=DEV).to(torch.bfloat16)
+    outs = {}
+    for keep in (True, False):
+        M.modules.AttentionFunc.KEEP_WEIGHTS = keep
+        try:
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            y = M.modules.attention(qq, kk, vv, 0.125, 0.0, causal, True)
+            saved = [t.shape for t in y.grad_fn.saved_tensors]
+            y.backward(dy)
+            outs[keep] = (y.detach(), qq.grad, kk.grad, vv.grad, saved)
+        finally:
+            M.modules.AttentionFunc.KEEP_WEIGHTS = False
+    torch.cuda.synchronize()
+    assert any(len(s) == 4 and s[-1] == L and s[-2] == L for s in outs[True][4])
+    assert not any(len(s) == 4 and s[-1] == L and s[-2] == L for s in outs[False][4])
+    def close(got, ref, tol=2e-2):           # the bound of test_attention_autograd: rms error and worst element
+        e = host(got) - np.asarray(ref)
+        rms = np.sqrt((np.asarray(ref) ** 2).mean())
+        return np.sqrt((e ** 2).mean()) < tol * rms and np.abs(e).max() < 4 * tol * max(rms, np.abs(ref).max())
+
+    for a, b in zip(outs[True][:4], outs[False][:4]):      # two 16-bit paths against each other
+        assert close(b, host(a))
+    # and against the fp64 oracle
+    yo, _ = O.attention(host(q), host(k), host(v), 0.125, causal)
+    assert rel_err(host(outs[False][0]), yo) < 2e-2
+    dq, dk, dv = O.attention_bwd(host(dy), host(q), host(k), host(v), 0.125, causal)
+    for got, want in zip(outs[False][1:4], (dq, dk, dv)):
+        assert close(got, want)
