@@ -194,8 +194,8 @@ M_TOL = {torch.float32: 1e-4, BF: 2e-2}
 def test_one_kernel_with_padding_mask(out_layout, B, L, G, cpg, affine):
     """Padding inside the one-kernel envelope: masked tokens take no part in the running statistics and leave the norm
     as zeros (timestep_norm.cc:283-311), the moving average sees those zeros.  The masks: a padded tail, a row that
-    starts padded, a whole block of 1024 padded tokens in the middle of a row, single tokens, and a row without
-    padding."""
+    starts padded, a whole block of 1024 padded tokens in the middle of a row, single tokens, a row of nothing but
+    padding, and a row without padding."""
     print(f"case out={out_layout} B={B} L={L} G={G} cpg={cpg} affine={affine}", flush=True)
     D, N = cpg * G, 16
     rng = np.random.default_rng(57)
@@ -210,6 +210,8 @@ def test_one_kernel_with_padding_mask(out_layout, B, L, G, cpg, affine):
     if B > 2 and L >= 3072:
         mask[2, 1024:2048] = True
     mask[-1, ::97] |= B > 3
+    if B > 3:
+        mask[2, :] = True                                  # a row of nothing but padding: the prior statistics come back
     layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
     xn, y, cnt, mean, var, h = _run(layer, x, G, nw, nb, padding_mask=dev(mask, torch.bool), out_layout=out_layout,
                                     want_state=True)
