@@ -135,7 +135,7 @@ def test_norm_then_moving_average_sweep(seed):
     rng = np.random.default_rng(3000 + seed)
     for case in range(6):
         G = int(rng.choice([1, 2, 4]))
-        dg = int(rng.choice([64, 64, 32, 16]))
+        dg = int(rng.choice([64, 64, 128, 32, 16]))           # 64 and 128 per group: the one-kernel block
         D = G * dg
         L = int(rng.choice([64, 300, 1024, 2048, 2050, 3072]))
         B = int(rng.choice([1, 2, 3]))
@@ -155,6 +155,9 @@ def test_norm_then_moving_average_sweep(seed):
         mask = None
         if masked:
             mask = np.zeros((B, L), bool); mask[0, L - L // 4:] = True
+            if rng.integers(0, 2):
+                mask[-1, :int(rng.integers(1, min(L, 1500)))] = True       # a row that starts padded (whole blocks too)
+                mask[B // 2] |= rng.random(L) < 0.05
         h0 = None
         if with_state:
             h0 = (rng.normal(size=(B, D, N)) + (1j * rng.normal(size=(B, D, N)) if cplx else 0))
