@@ -79,6 +79,7 @@ struct FusedArgs {
   TsnHeader* hdr;
   unsigned long long* rec;   // [B * D / 64][S + 1][kFRecW]; slot S: the caller's carried state, put there by block 0
   int B, L, D, G, N, S;
+  int pad;               // S * 1024 - L virtual tokens in front of every row: the block grid ends at the row's last token
   float eps;
   int is_complex;
   int xcd_map;
@@ -205,10 +206,14 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   const int g = unit / kParts, part = unit - g * kParts;
   const int cb = g * GC + part * kFC;                    // the workgroup's first channel
   const uint32_t tag = A.hdr->epoch + 1u;
-  const int t0 = s * kFSeg;
+  // The blocks are aligned to the end of the row: block 0 starts `pad` virtual tokens before the first one (they
+  // count as padding: no statistics, zeros into the moving average, nothing stored), so the last block ends at the
+  // last token and the state handed back is the state after it.
+  const int t0 = s * kFSeg - A.pad;
+  const bool front = s == 0 && A.pad > 0;                // uniform: this block holds virtual tokens
   const int piece = tid & 7, tokl = tid >> 3;            // 16-byte piece of the 128-byte line, token 0..127
   // addresses of the block's lines: a uniform base per 128-token round plus one 32-bit lane offset
-  const size_t xblk = ((size_t)b * A.L + t0) * A.D + (size_t)cb;
+  const int64_t xblk = ((int64_t)b * A.L + t0) * A.D + (int64_t)cb;      // (negative offsets inside a front block are never used)
   const uint32_t toff = (uint32_t)tokl * (uint32_t)A.D + piece * 8;
   const size_t brow = (size_t)b * G + g;                 // statistics of the group
   const size_t rrow = brow * kParts + part;              // records of the workgroup (its own copy of the statistics too)
@@ -222,23 +227,35 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   load_params<8>(A.gamma + cb + piece * 8, gam);
   load_params<8>(A.beta + cb + piece * 8, bet);
   uint4 xv[kFNLD];
-#pragma unroll
-  for (int k = 0; k < kFNLD; ++k) xv[k] = *(const uint4*)(A.x + xblk + (size_t)k * 128 * A.D + toff);
-  // the other half of the group's lines, for the moments only (the workgroup of that half reads the same lines on the
-  // same XCD)
   uint4 xo[kParts == 2 ? kFNLD : 1];
-  if (kParts == 2) {
-    const size_t oblk = ((size_t)b * A.L + t0) * A.D + (size_t)(g * GC + (1 - part) * kFC);
-#pragma unroll
-    for (int k = 0; k < kFNLD; ++k) xo[k] = *(const uint4*)(A.x + oblk + (size_t)k * 128 * A.D + toff);
-  }
-
-  // padding flags of the thread's eight tokens (bit k: token k * 128 + tokl)
+  const int64_t oblk = ((int64_t)b * A.L + t0) * A.D + (int64_t)(g * GC + (1 - part) * kFC);
+  // padding flags of the thread's eight tokens (bit k: token k * 128 + tokl): the caller's mask and the virtual
+  // tokens of a front block
   uint32_t mbits = 0;
-  if (A.mask) {
-    const uint8_t* mrow = A.mask + (size_t)b * A.L + t0 + tokl;
+  if (!front) {
 #pragma unroll
-    for (int k = 0; k < kFNLD; ++k) mbits |= (mrow[k * 128] != 0 ? 1u : 0u) << k;
+    for (int k = 0; k < kFNLD; ++k) xv[k] = *(const uint4*)(A.x + xblk + (int64_t)k * 128 * A.D + toff);
+    // the other half of the group's lines, for the moments only (the workgroup of that half reads the same lines on
+    // the same XCD)
+    if (kParts == 2) {
+#pragma unroll
+      for (int k = 0; k < kFNLD; ++k) xo[k] = *(const uint4*)(A.x + oblk + (int64_t)k * 128 * A.D + toff);
+    }
+    if (A.mask) {
+      const uint8_t* mrow = A.mask + (int64_t)b * A.L + t0 + tokl;
+#pragma unroll
+      for (int k = 0; k < kFNLD; ++k) mbits |= (mrow[k * 128] != 0 ? 1u : 0u) << k;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kFNLD; ++k) {
+      const bool real = k * 128 + tokl >= A.pad;
+      const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+      xv[k] = real ? *(const uint4*)(A.x + xblk + (int64_t)k * 128 * A.D + toff) : zero;
+      if (kParts == 2) xo[k] = real ? *(const uint4*)(A.x + oblk + (int64_t)k * 128 * A.D + toff) : zero;
+      const bool padded = !real || (A.mask && A.mask[(int64_t)b * A.L + t0 + k * 128 + tokl] != 0);
+      mbits |= (padded ? 1u : 0u) << k;
+    }
   }
 
   // the per-state multipliers of the group's 64 channels (three lines per channel) go to LDS once
@@ -448,7 +465,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 #pragma unroll
     for (int i = 0; i < 8; ++i) plain = plain && gam[i] == 1.f && bet[i] == 0.f;
     const bool ident = __all(plain);
-    auto stage = [&](auto IDENT, auto MASKED) {
+    auto stage = [&](auto IDENT, auto MASKED, auto FRONT) {
 #pragma unroll
     for (int k = 0; k < kFNLD; ++k) {
       const int tok = k * 128 + tokl;
@@ -468,7 +485,8 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = pad ? 0u : o[i];
       }
-      store_stream((uint4*)(A.xn + xblk + (size_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
+      if (!decltype(FRONT)::value || k * 128 + tokl >= A.pad)              // virtual tokens have no place in xn
+        store_stream((uint4*)(A.xn + xblk + (int64_t)k * 128 * A.D + toff), make_uint4(o[0], o[1], o[2], o[3]));
       const uint32_t s0 = odd ? o[0] : o[2], s1 = odd ? o[1] : o[3];
       const uint32_t r0 = dpp_u<0x128>(s0), r1 = dpp_u<0x128>(s1);       // row_ror:8 = the partner token's lane
       const uint32_t m0 = odd ? o[2] : o[0], m1 = odd ? o[3] : o[1];
@@ -479,16 +497,22 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       *(uint32_t*)(wp + 3 * kFRow) = __builtin_amdgcn_perm(r1, m1, sel_hi);
     }
     };
-    if (A.mask) {
+    if (front) {
       if (ident) {
-        stage(std::true_type{}, std::true_type{});
+        stage(std::true_type{}, std::true_type{}, std::true_type{});
       } else {
-        stage(std::false_type{}, std::true_type{});
+        stage(std::false_type{}, std::true_type{}, std::true_type{});
+      }
+    } else if (A.mask) {
+      if (ident) {
+        stage(std::true_type{}, std::true_type{}, std::false_type{});
+      } else {
+        stage(std::false_type{}, std::true_type{}, std::false_type{});
       }
     } else if (ident) {
-      stage(std::true_type{}, std::false_type{});
+      stage(std::true_type{}, std::false_type{}, std::false_type{});
     } else {
-      stage(std::false_type{}, std::false_type{});
+      stage(std::false_type{}, std::false_type{}, std::false_type{});
     }
   }
   __syncthreads();
@@ -518,12 +542,12 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     const char* rb = tile + row_base(c);
-    bf16_t* yr = A.y + (size_t)b * A.syb + (size_t)(cb + c) * A.syd + t0;
+    bf16_t* yr = A.y + (int64_t)b * A.syb + (int64_t)(cb + c) * A.syd + t0;
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       const int q = k * 64 + lane;                 // 16-byte chunk of the row: segment q >> 3, chunk q & 7
       const uint4 v = *(const uint4*)(rb + (q >> 3) * 128 + (((q & 7) ^ (q >> 4)) << 4));
-      store_stream((uint4*)(yr + q * 8), v);
+      if (q * 8 >= -t0) store_stream((uint4*)(yr + q * 8), v);      // (a front block: the row begins inside it, at a multiple of 8)
     }
   };
 
@@ -819,7 +843,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
     const int tl = tokl & ~1;
     const char* rbase = tile + row_base(piece * 8 + odd * 4) + (tl >> 6) * 128 + ((tl & 7) >> 1) * 4;
     const int c8 = (tl & 63) >> 3;
-    bf16_t* yb = A.y + (size_t)b * A.syb + (size_t)(cb + piece * 8) * A.syd;
+    bf16_t* yb = A.y + (int64_t)b * A.syb + (int64_t)(cb + piece * 8) * A.syd;
 #pragma unroll
     for (int k = 0; k < kFNLD; ++k) {
       const int tok = k * 128 + tokl;
@@ -836,7 +860,7 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
       o.y = odd ? got1 : keep1;
       o.z = odd ? keep0 : got0;
       o.w = odd ? keep1 : got1;
-      store_stream((uint4*)(yb + (size_t)(t0 + tok) * A.syl), o);
+      if (t0 + tok >= 0) store_stream((uint4*)(yb + (int64_t)(t0 + tok) * A.syl), o);
     }
   }
 
@@ -866,12 +890,15 @@ bool fused_covers(int dtype, int64_t B, int64_t L, int64_t D, int64_t G, int64_t
                   const void* y, int64_t syb, int64_t syd, int64_t syl, const uint8_t* mask, const float* h_in) {
   (void)mask;
   if (dtype != MEGA_BF16 || G <= 0 || (D != G * kFC && D != G * 2 * kFC) || N > kNS || N <= 0) return false;
-  if (L <= 0 || L % kFSeg != 0 || L / kFSeg + (h_in ? 1 : 0) > kFMaxBlocks) return false;
+  if (L <= 0 || ceil_div(L, kFSeg) + (h_in ? 1 : 0) > kFMaxBlocks) return false;
+  // a ragged first block (the block grid is aligned to the end of the row): no carried state in (it would have to
+  // enter in the middle of a block), and rows in time must begin at a multiple of 8 inside it
+  if (L % kFSeg != 0 && (h_in || (syl == 1 && L % 8 != 0))) return false;
   if (((uintptr_t)x % 16) || ((uintptr_t)xn % 16) || ((uintptr_t)y % 16)) return false;
   const bool rows = syl == 1 && syd % 8 == 0 && syb % 8 == 0;
   const bool lines = syd == 1 && syl % 8 == 0 && syb % 8 == 0;
   if (!rows && !lines) return false;
-  if (B * (D / kFC) * (L / kFSeg) >= (int64_t)1 << 31) return false;
+  if (B * (D / kFC) * ceil_div(L, kFSeg) >= (int64_t)1 << 31) return false;
   return true;
 }
 
@@ -949,6 +976,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     A.var = var; A.gamma = norm_gamma; A.beta = norm_beta; A.mask = mask; A.image = (const uint4*)img; A.h_in = h_in; A.h_out = h_out;
     A.hdr = (TsnHeader*)w; A.rec = (unsigned long long*)(w + align_up(sizeof(TsnHeader), 256));
     A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
+    A.pad = (int)(S * kFSeg - L);
     A.is_complex = is_complex;
     const int parts = (int)(D / (G * kFC));              // workgroups per norm group
     A.xcd_map = ((G * parts) % 8 == 0) ? 1 : 0;

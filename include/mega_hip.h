@@ -230,9 +230,11 @@ int mega_norm_ema_steps(const void* x, void* xn, void* y, int dtype, int64_t K,
  *   norm state / parameters / mask as mega_group_timestep_norm_fwd (norm_gamma = weight + 1);
  *   moving-average coefficients, h_in / h_out and `image` as mega_ema_fwd (unidirectional,
  *   no truncation); h_out must not overlap h_in.
- * bf16 activations with 64 channels per norm group (D = 64 G), ndim <= 16, no mask, L a
- * multiple of 1024 with L / 1024 (+ 1 with h_in) <= 16 run as ONE kernel that reads x once and
- * writes xn and y once; everything else runs the two operators one after the other.
+ * bf16 activations with 64 or 128 channels per norm group (D = 64 G or 128 G), ndim <= 16, with or
+ * without a mask, ceil(L / 1024) (+ 1 with h_in) <= 16 run as ONE kernel that reads x once and writes xn
+ * and y once.  L need not be a multiple of 1024 (the blocks are aligned to the end of the row, so h_out is
+ * the state after the last token), but such a row takes no h_in, and [B,D,L] rows then need L % 8 == 0.
+ * Everything else runs the two operators one after the other.
  * `workspace` (launch epoch, block / tile records) must be zero-filled once and then belongs to
  * these calls, exactly like the TimestepNorm workspace (the two may be the same buffer);
  * `scratch` needs no initialisation and is used only when the two operators run one after the

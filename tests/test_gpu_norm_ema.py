@@ -1,6 +1,6 @@
 """TimestepNorm -> moving average in one call (mega_norm_ema_fwd) against the fp64 oracle and against
-the two operators run one after the other: the one-kernel envelope (bf16, 64 channels per group, L a
-multiple of 1024), carried state in and out, both output layouts, slowly decaying poles, prior
+the two operators run one after the other: the one-kernel envelope (bf16, 64 or 128 channels per group, padding
+masks, rows of any length), carried state in and out, both output layouts, slowly decaying poles, prior
 statistics, and shapes outside the envelope (which take the two-operator route inside the call)."""
 import numpy as np
 import pytest
@@ -187,6 +187,56 @@ def test_outside_the_envelope_runs_two_operators(dtype, B, L, D, G, masked):
 
 
 M_TOL = {torch.float32: 1e-4, BF: 2e-2}
+
+
+@pytest.mark.parametrize("L,out_layout,masked", [(1000, "rows", False), (1032, "rows", True), (2056, "input", False),
+                                                 (3001, "input", True), (300, "input", False), (8, "rows", False),
+                                                 (1, "input", False), (5000, "rows", False)])
+@pytest.mark.parametrize("cpg", [64, 128])
+def test_one_kernel_rows_of_any_length(L, out_layout, masked, cpg):
+    """Rows that are not whole blocks of 1024 tokens: the block grid is aligned to the end of the row (the first block
+    starts before the row), so the state handed back is the state after the last token -- what a prompt of any length
+    needs before decoding continues from it.  Statistics carried in, state out, both layouts (rows in time need a length
+    that is a multiple of 8), with and without padding; the continuation of the row by a second call (two operators:
+    it carries a state in) agrees with one call on the whole."""
+    print(f"case L={L} out={out_layout} masked={masked} cpg={cpg}", flush=True)
+    B, G, N = 2, 2, 16
+    D = cpg * G
+    rng = np.random.default_rng(58)
+    p, q, g, om, nw, nb = _setup(rng, D, N)
+    L2 = 64
+    x, x64 = rounded(rng.normal(size=(B, L + L2, D)) * 1.2 + 0.4, BF)
+    mask = None
+    if masked:
+        mask = np.zeros((B, L + L2), bool)
+        mask[0, max(L - 40, 0):L] = True
+        mask[1, :min(10, L)] = True
+        mask[1, L // 2] = True
+    pc = np.array([5, 0])
+    pm = rng.normal(size=(B, G)).astype(np.float32).astype(np.float64)
+    pv = (rng.random((B, G)) + 0.5).astype(np.float32).astype(np.float64)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+    tm = None if mask is None else dev(mask[:, :L], torch.bool)
+    xn, y, cnt, mean, var, h = _run(layer, x[:, :L].contiguous(), G, nw, nb,
+                                    prior=(dev(pc, torch.int64), dev(pm), dev(pv)), padding_mask=tm,
+                                    out_layout=out_layout, want_state=True)
+    assert y.shape == (B, D, L)
+    xno, c, mu, v = O.timestep_norm(x64, pc, pm, pv, nw + 1, nb, mask, G)
+    assert rel_err(host(xn), xno[:, :L]) < 2e-2
+    m1 = None if mask is None else mask[:, :L]
+    _, c1, mu1, v1 = O.timestep_norm(x64[:, :L], pc, pm, pv, nw + 1, nb, m1, G)
+    assert cnt.tolist() == c1.tolist()
+    assert rel_err(host(mean), mu1) < 1e-4 and rel_err(host(var), v1) < 1e-4
+    yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, m1, incremental=True)
+    _check_y(y, yo)
+    assert rel_err(np.real(host(h)), np.real(ho)) < 2e-3 and rel_err(np.imag(host(h)), np.imag(ho)) < 2e-3
+    # the row continues: statistics and state carried into a second call
+    tm2 = None if mask is None else dev(mask[:, L:], torch.bool)
+    xn2, y2, c2, _, _, _ = _run(layer, x[:, L:].contiguous(), G, nw, nb, prior=(cnt, mean, var), h=h, padding_mask=tm2,
+                                out_layout=out_layout)
+    assert rel_err(host(xn2), xno[:, L:]) < 2e-2 and c2.tolist() == c.tolist()
+    yo2, _ = O.ema_forward(host(torch.cat([xn, xn2], 1)).transpose(0, 2, 1), p, q, g, om, mask)
+    _check_y(y2, yo2[:, :, L:])
 
 
 @pytest.mark.parametrize("out_layout", ["rows", "input"])
