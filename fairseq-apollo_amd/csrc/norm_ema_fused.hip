@@ -1,5 +1,5 @@
-// TimestepNorm -> moving-average layer in one kernel (gfx950, bf16 activations, 64 channels per
-// norm group, ndim <= 16): what MovingAverageGatedAttention.forward does at
+// TimestepNorm -> moving-average layer in one kernel (gfx950, bf16 activations, 64 or 128 channels per
+// norm group, ndim <= 16, optional padding mask, rows of any length up to 16 blocks): what MovingAverageGatedAttention.forward does at
 // fairseq/modules/moving_average_gated_attention.py:304-315 (x = norm(x); mx = move(x^T)) with
 // TimestepNorm per fairseq/csrc/ops/timestep_norm.cc:218-316 and the layer per
 // fairseq/modules/base_moving_average.py:120-172.  x is read once, xn (the norm's output, which the
