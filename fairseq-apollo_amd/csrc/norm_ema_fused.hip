@@ -5,20 +5,23 @@
 // fairseq/modules/base_moving_average.py:120-172.  x is read once, xn (the norm's output, which the
 // layer also feeds to v_proj) and y are written once.
 //
-// A workgroup (16 waves) owns one (batch row, norm group, block of 1024 tokens): whole 128-byte
-// lines of x, xn and -- with [B, D, L] rows -- y.
+// A workgroup (16 waves) owns one (batch row, 64 channels of a norm group, block of 1024 tokens): whole 128-byte
+// lines of x, xn and -- with [B, D, L] rows -- y.  A group of 128 channels is shared by two workgroups, each of
+// which reads the group's whole lines for the moments.  The blocks are aligned to the end of the row: a row that is
+// not a whole number of blocks starts inside block 0, behind virtual tokens that count as padding.
 //   1. load the block, per-token moments of the group (packed dot products + DPP), Welford scan over
-//      the block's tokens, publish the block aggregate, fold the earlier blocks' aggregates of the
-//      same (row, group) and the prior state into the carry-in, finish mean / rstd per token;
-//   2. normalise from registers, store xn, and stage xn (bf16, as the layer sees it) into LDS
+//      the block's tokens (padding weighs nothing), publish the block aggregate, fold the earlier blocks'
+//      aggregates of the same (row, group) and the prior state into the carry-in, finish mean / rstd per token;
+//   2. normalise from registers, store xn (zeros at padding), and stage xn (bf16, as the layer sees it) into LDS
 //      transposed to channel rows;
 //   3. per channel (4 per wave), with the operand images of ema_image_kernel:
-//        sweep 1: end states of the 16 segments (64 tokens = 2 tiles each) from a zero start on the
+//        phase A: end states of the 16 segments (64 tokens = 2 tiles each) from a zero start on the
 //                 matrix cores, scanned across the 16 lanes of a DPP row; the block's end state from a
-//                 zero start is published, the segments' start states are parked as bf16;
+//                 zero start is parked in LDS and published;
 //      look-back: the earlier blocks' end states (and the caller's carried state) folded into the
-//                 block's start state, h_start = sum_d (q^1024)^d E_{s-1-d};
-//        sweep 2: y_tile = K x_tile + C (h_seg + (q^64)^j h_start), bf16, back into LDS over x, and
+//                 block's start state, h_start = sum_d (q^1024)^d E_{s-1-d}, parked over the end states;
+//        phase B: the segment scan again, segment start state = what the segment before left + (q^64)^j h_start,
+//                 y_tile = K x_tile + C h (h as one bf16 term, two for slow poles), bf16, back into LDS over x, and
 //                 out as whole rows.
 // Blocks map to workgroup ids time-major and workgroups are dispatched in id order, so a block only
 // waits for blocks dispatched before it; every wait is bounded and poisons the block's outputs with
