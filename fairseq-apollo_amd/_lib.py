@@ -47,6 +47,9 @@ SIGNATURES = {
     "mega_norm_ema_fwd_scratch_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
     "mega_norm_ema_fwd": (_int, [_p, _p, _p, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, C.c_double, _p, _p, _p,
                                  _p, _p, _p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _sz, _p, _sz, _p]),
+    "mega_norm_ema_fwd_train": (_int, [_p, _p, _p, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, C.c_double, _p, _p,
+                                       _p, _p, _p, _p, _p, _p, _int, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p,
+                                       _sz, _p, _sz, _p]),
     "mega_ema_param_grad_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "mega_ema_param_grad": (_int, [_p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64,
                                    _i64, _int, _int, _p, _p, _p, _p, _p, _sz, _p]),

@@ -79,6 +79,8 @@ struct FusedArgs {
   const uint4* image;    // [D][kImgSlots][64]
   const float* h_in;     // [B, D, N, 2] or null
   float* h_out;          // [B, D, N, 2] or null
+  float* cummean;        // [B, L, G] running mean / rstd of every token, kept for the norm's backward pass; or null
+  float* cumrstd;
   TsnHeader* hdr;
   unsigned long long* rec;   // [B * D / 64][S + 1][kFRecW]; slot S: the caller's carried state, put there by block 0
   int B, L, D, G, N, S;
@@ -405,8 +407,18 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       full = merge(base, pref[u]);
+      const float rstd = __builtin_amdgcn_rsqf(full.var + A.eps);
       s_gm[wave * 256 + lane * 4 + u] = full.mean;
-      s_gv[wave * 256 + lane * 4 + u] = __builtin_amdgcn_rsqf(full.var + A.eps);
+      s_gv[wave * 256 + lane * 4 + u] = rstd;
+      // training: the statistics the norm's backward pass reads (a padded token holds the carried ones)
+      if (A.cummean && part == 0) {
+        const int64_t tok = (int64_t)t0 + wave * 256 + lane * 4 + u;
+        if (tok >= 0) {
+          const int64_t o = ((int64_t)b * A.L + tok) * A.G + g;
+          A.cummean[o] = full.mean;
+          A.cumrstd[o] = rstd;
+        }
+      }
     }
     if (s == A.S - 1 && wave == 3 && lane == 63 && part == 0) {
       A.mean[brow] = full.mean;
@@ -929,15 +941,18 @@ extern "C" size_t mega_norm_ema_fwd_scratch_bytes(int64_t B, int64_t L, int64_t 
   return align_up(ema > img ? ema : img, 256);
 }
 
-extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd, int64_t syl,
-                                 const int64_t* prev_count, const float* prev_mean, const float* prev_var,
-                                 const float* norm_gamma, const float* norm_beta, const uint8_t* mask, double eps,
-                                 int64_t* count, float* mean, float* var, const float* p, const float* q,
-                                 const float* gamma, int is_complex, const float* omega, const float* h_in,
-                                 float* h_out, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N,
-                                 const void* image, void* workspace, size_t workspace_bytes, void* scratch,
-                                 size_t scratch_bytes, void* stream) {
+extern "C" int mega_norm_ema_fwd_train(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd,
+                                       int64_t syl, const int64_t* prev_count, const float* prev_mean,
+                                       const float* prev_var, const float* norm_gamma, const float* norm_beta,
+                                       const uint8_t* mask, double eps, int64_t* count, float* mean, float* var,
+                                       float* cummean, float* cumrstd, const float* p, const float* q,
+                                       const float* gamma, int is_complex, const float* omega, const float* h_in,
+                                       float* h_out, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N,
+                                       const void* image, void* workspace, size_t workspace_bytes, void* scratch,
+                                       size_t scratch_bytes, void* stream) {
   if (const int rc = lookback_pending("norm_ema_fwd")) return rc;
+  MEGA_REQUIRE((cummean == nullptr) == (cumrstd == nullptr), MEGA_ERR_ARG,
+               "norm_ema_fwd: cummean and cumrstd go together");
   MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
                "norm_ema_fwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(B >= 0 && L >= 0 && D > 0 && G > 0 && N > 0 && D % G == 0, MEGA_ERR_ARG,
@@ -977,6 +992,7 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
     A.x = (const bf16_t*)x; A.xn = (bf16_t*)xn; A.y = (bf16_t*)y; A.syb = syb; A.syd = syd; A.syl = syl;
     A.prev_count = prev_count; A.prev_mean = prev_mean; A.prev_var = prev_var; A.count = count; A.mean = mean;
     A.var = var; A.gamma = norm_gamma; A.beta = norm_beta; A.mask = mask; A.image = (const uint4*)img; A.h_in = h_in; A.h_out = h_out;
+    A.cummean = cummean; A.cumrstd = cumrstd;
     A.hdr = (TsnHeader*)w; A.rec = (unsigned long long*)(w + align_up(sizeof(TsnHeader), 256));
     A.B = (int)B; A.L = (int)L; A.D = (int)D; A.G = (int)G; A.N = (int)N; A.S = (int)S; A.eps = (float)eps;
     A.pad = (int)(S * kFSeg - L);
@@ -1002,9 +1018,22 @@ extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, in
   // (x -> xn by the norm, xn read through its transposed view by the moving average); the norm keeps its
   // launch header and tile records in the same workspace (same header, same protocol)
   int rc = mega_group_timestep_norm_fwd(x, xn, dtype, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, mask, B, L,
-                                        D, G, eps, count, mean, var, nullptr, nullptr, nullptr, workspace,
+                                        D, G, eps, count, mean, var, nullptr, cummean, cumrstd, workspace,
                                         workspace_bytes, stream);
   if (rc) return rc;
   return mega_ema_fwd(xn, y, dtype, L * D, 1, D, syb, syd, syl, p, q, gamma, is_complex, omega, mask, h_in, h_out, B, D,
                       N, L, 0, 0, 1, image, scratch, scratch_bytes, stream);
+}
+
+extern "C" int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd, int64_t syl,
+                                 const int64_t* prev_count, const float* prev_mean, const float* prev_var,
+                                 const float* norm_gamma, const float* norm_beta, const uint8_t* mask, double eps,
+                                 int64_t* count, float* mean, float* var, const float* p, const float* q,
+                                 const float* gamma, int is_complex, const float* omega, const float* h_in,
+                                 float* h_out, int64_t B, int64_t L, int64_t D, int64_t G, int64_t N,
+                                 const void* image, void* workspace, size_t workspace_bytes, void* scratch,
+                                 size_t scratch_bytes, void* stream) {
+  return mega_norm_ema_fwd_train(x, xn, y, dtype, syb, syd, syl, prev_count, prev_mean, prev_var, norm_gamma, norm_beta,
+                                 mask, eps, count, mean, var, nullptr, nullptr, p, q, gamma, is_complex, omega, h_in,
+                                 h_out, B, L, D, G, N, image, workspace, workspace_bytes, scratch, scratch_bytes, stream);
 }

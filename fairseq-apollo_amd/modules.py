@@ -528,6 +528,46 @@ class TimestepNorm(nn.Module, IncrementalState):
             **self.__dict__)
 
 
+class NormThenMoveFunc(torch.autograd.Function):
+    """x = norm(x); mx = move(x^T) as one differentiable operator whose forward is one library call
+    (moving_average_gated_attention.py:304-315; the reference chains GroupTimestepNormFunc,
+    norm_layer/timestep_norm.py:14-66, EMAParametersFunc and FFTConvFunc).  The forward keeps x, xn and the
+    norm's running statistics; the backward runs the moving average backwards in time on mx's gradient, adds
+    the result to xn's own gradient and hands the sum to the norm's backward pass."""
+
+    ENABLED = True          # False: training runs the two modules' own operators one after the other
+
+    @staticmethod
+    def forward(ctx, x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, p, q, gamma, omega, padding_mask,
+                num_groups, eps, out_layout, shift):
+        layer = ops.PreparedEMA(p.squeeze(-1), q.squeeze(-1), gamma, omega.reshape(-1), False, None, shift)
+        xn, y, count, _, _, _, cummean, cumrstd = layer.norm_forward(
+            x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, num_groups, eps, padding_mask, None,
+            want_state=False, out_layout=out_layout, want_stats=True)
+        ctx.layer = layer
+        ctx.num_groups = num_groups
+        ctx.save_for_backward(x, xn, prev_mean, count, cummean, cumrstd, norm_gamma, p, q, gamma, omega, padding_mask)
+        return xn, y
+
+    @staticmethod
+    def backward(ctx, xn_grad, y_grad):
+        x, xn, prev_mean, count, cummean, cumrstd, norm_gamma, p, q, gamma, omega, padding_mask = ctx.saved_tensors
+        total = xn_grad
+        dp = dq = dg = dom = None
+        if y_grad is not None:
+            dxe, dp, dq, dg, dom = ops.ema_backward(y_grad, xn.transpose(1, 2), p.squeeze(-1), q.squeeze(-1), gamma,
+                                                    omega.reshape(-1), padding_mask, layer=ctx.layer)
+            dxe = dxe.transpose(1, 2)
+            total = dxe if total is None else total + dxe
+            dp, dq = dp.to(p.dtype).view_as(p), dq.to(q.dtype).view_as(q)
+            dg, dom = dg.to(gamma.dtype).view_as(gamma), dom.to(omega.dtype).view_as(omega)
+        x_grad, pm_grad, pv_grad, ng_grad, nb_grad = ops.group_timestep_norm_bwd(
+            total.contiguous(), None, None, x, prev_mean, count, None, cummean, cumrstd, norm_gamma, padding_mask,
+            ctx.num_groups)
+        return (x_grad, None, pm_grad.to(prev_mean.dtype).view_as(prev_mean), pv_grad.view_as(prev_mean),
+                ng_grad.to(norm_gamma.dtype), nb_grad, dp, dq, dg, dom, None, None, None, None, None)
+
+
 def norm_then_move(norm: nn.Module, move: nn.Module, x: Tensor, padding_mask: Optional[Tensor] = None,
                    incremental_state: Optional[Dict[str, Dict[str, Optional[Tensor]]]] = None,
                    out_layout: str = "rows") -> Tuple[Tensor, Tensor]:
@@ -535,12 +575,19 @@ def norm_then_move(norm: nn.Module, move: nn.Module, x: Tensor, padding_mask: Op
     x: [B, L, D] -> (xn [B, L, D], mx [B, D, L] in `out_layout`).  A group TimestepNorm in front of a
     one-sided layer without kernel truncation, called without autograd, goes to the library as one call
     (x is read once, xn and mx are written once); both modules' incremental state is kept exactly as the
-    two calls keep it.  Every other combination runs the two modules one after the other."""
+    two calls keep it.  Under autograd the same call is one differentiable operator (NormThenMoveFunc) when no
+    state is carried.  Every other combination runs the two modules one after the other."""
     one_call = (isinstance(norm, TimestepNorm) and norm.num_groups is not None and isinstance(move, BaseMovingLayer)
                 and not move.bidirectional and (move.truncation is None or move.truncation < 1)
-                and x.is_cuda and x.dim() == 3 and x.size(0) > 0 and x.size(1) > 0
-                and not _training_call(norm, x) and not _training_call(move, x))
-    if not one_call:
+                and x.is_cuda and x.dim() == 3 and x.size(0) > 0 and x.size(1) > 0)
+    training = one_call and (_training_call(norm, x) or _training_call(move, x))
+    if training and incremental_state is None and NormThenMoveFunc.ENABLED:
+        prev_count, prev_mean, prev_var = norm._prior_state(x.size(0), differentiable=True)
+        p, q, gamma = move._calc_coeffs()               # stay in the graph
+        return NormThenMoveFunc.apply(x, prev_count, prev_mean, prev_var, norm.weight.float() + 1.0,
+                                      norm.bias.float(), p, q, gamma, move.omega, padding_mask, norm.num_groups,
+                                      norm.eps, out_layout, move.shift)
+    if not one_call or training:
         xn = norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
         return xn, move(xn.transpose(1, 2), padding_mask, incremental_state, out_layout=out_layout)
     batch_size = x.size(0)

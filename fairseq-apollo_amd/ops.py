@@ -660,12 +660,15 @@ class PreparedEMA:
 
     def norm_forward(self, x: torch.Tensor, prev_count, prev_mean, prev_var, norm_gamma, norm_beta,
                      num_groups: int, eps: float, padding_mask: Optional[torch.Tensor] = None,
-                     h: Optional[torch.Tensor] = None, want_state: bool = False, out_layout: str = "rows"):
+                     h: Optional[torch.Tensor] = None, want_state: bool = False, out_layout: str = "rows",
+                     want_stats: bool = False):
         """TimestepNorm followed by this layer in one call (moving_average_gated_attention.py:304-315:
         x = norm(x); mx = move(x^T)).  x: [B, L, D].  -> (xn [B, L, D], y, count, mean, var, h_out); y is a
         contiguous [B, D, L] tensor (out_layout "rows", what the reference's convolution returns) or a
         [B, D, L] view of [B, L, D] memory (out_layout "input").  Covered shapes run as one kernel, the
-        rest as the two operators one after the other (mega_norm_ema_fwd)."""
+        rest as the two operators one after the other (mega_norm_ema_fwd).  want_stats (a training
+        forward): two more results, cummean and cumrstd [B, L, G], what the norm's backward pass reads
+        (timestep_norm.py:35-43)."""
         dev = self.dev
         _need_gpu(x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, padding_mask, h)
         if self.bidirectional or self.trunc:
@@ -703,16 +706,23 @@ class PreparedEMA:
         sc = _scratch_buffer(dev, sizes[1], stream)
         m8 = _mask_u8(padding_mask, B, L)
         gf, bf = _f32c(norm_gamma), _f32c(norm_beta)
+        cm = cr = None
+        if want_stats:
+            cm = torch.empty(B, L, G, dtype=torch.float32, device=dev)
+            cr = torch.empty(B, L, G, dtype=torch.float32, device=dev)
         with _on_device(dev):
-            rc = lib.mega_norm_ema_fwd(_ptr(xd), _ptr(xn), _ptr(y), dt, y.stride(0), y.stride(1), y.stride(2),
-                                       _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf), _ptr(m8), float(eps),
-                                       _ptr(count), _ptr(mean), _ptr(var), _ptr(self.p), _ptr(self.q), _ptr(self.gamma),
-                                       1 if self.is_complex else 0, _ptr(self.omega), _ptr(hin), _ptr(hout), B, L, D, G,
-                                       N, _ptr(self.image), _ptr(ws), ws.numel(), _ptr(sc), sc.numel(), stream)
+            rc = lib.mega_norm_ema_fwd_train(_ptr(xd), _ptr(xn), _ptr(y), dt, y.stride(0), y.stride(1), y.stride(2),
+                                             _ptr(pc), _ptr(pm), _ptr(pv), _ptr(gf), _ptr(bf), _ptr(m8), float(eps),
+                                             _ptr(count), _ptr(mean), _ptr(var), _ptr(cm), _ptr(cr), _ptr(self.p),
+                                             _ptr(self.q), _ptr(self.gamma), 1 if self.is_complex else 0,
+                                             _ptr(self.omega), _ptr(hin), _ptr(hout), B, L, D, G, N, _ptr(self.image),
+                                             _ptr(ws), ws.numel(), _ptr(sc), sc.numel(), stream)
         _lib.check(rc, "norm_ema_fwd")
         hc = None
         if hout is not None:
             hc = torch.view_as_complex(hout) if self.is_complex else hout[..., 0]
+        if want_stats:
+            return xn, y, count, mean, var, hc, cm, cr
         return xn, y, count, mean, var, hc
 
     def adjoint(self, y_grad: torch.Tensor, padding_mask: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -249,6 +249,21 @@ int mega_norm_ema_fwd(const void* x, void* xn, void* y, int dtype, int64_t syb, 
                       const float* omega, const float* h_in, float* h_out, int64_t B, int64_t L,
                       int64_t D, int64_t G, int64_t N, const void* image, void* workspace,
                       size_t workspace_bytes, void* scratch, size_t scratch_bytes, void* stream);
+/* The same call for a training forward: additionally writes cummean, cumrstd [B,L,G] fp32, the
+ * running statistics of every token that group_timestep_norm_fwd hands to its backward pass
+ * (fairseq/modules/norm_layer/timestep_norm.py:35-43; at a padded token the carried statistics), so
+ * that mega_group_timestep_norm_bwd (group_mean = NULL) and the moving-average backward can follow
+ * a forward that ran as one kernel.  Both pointers NULL: exactly mega_norm_ema_fwd.            */
+int mega_norm_ema_fwd_train(const void* x, void* xn, void* y, int dtype, int64_t syb, int64_t syd,
+                            int64_t syl, const int64_t* prev_count, const float* prev_mean,
+                            const float* prev_var, const float* norm_gamma, const float* norm_beta,
+                            const uint8_t* mask, double eps, int64_t* count, float* mean, float* var,
+                            float* cummean, float* cumrstd, const float* p, const float* q,
+                            const float* gamma, int is_complex, const float* omega,
+                            const float* h_in, float* h_out, int64_t B, int64_t L, int64_t D,
+                            int64_t G, int64_t N, const void* image, void* workspace,
+                            size_t workspace_bytes, void* scratch, size_t scratch_bytes,
+                            void* stream);
 
 /* ------------------------------------------------------------------------ */
 /* Moving-average backward (unidirectional, no carried state)                  */

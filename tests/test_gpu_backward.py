@@ -103,6 +103,68 @@ def test_timestep_norm_module_autograd(groups, prior_count):
         assert rel_err(host(mod.prior_logv.grad), (dpv * pv).sum(0)) < 2e-4
 
 
+@pytest.mark.parametrize("dtype,B,L,D,G,N,masked,layout", [
+    (torch.bfloat16, 2, 1024, 128, 2, 16, False, "rows"),      # one kernel, one block
+    (torch.bfloat16, 1, 2048, 256, 2, 16, False, "input"),     # groups of 128 channels, two blocks
+    (torch.bfloat16, 2, 1000, 64, 1, 8, True, "input"),        # ragged row with padding
+    (torch.float32, 2, 70, 32, 4, 4, True, "rows"),            # outside the one-kernel envelope
+])
+def test_norm_then_move_trains_as_one_operator(dtype, B, L, D, G, N, masked, layout):
+    """norm_then_move under autograd is one operator whose forward is the one-kernel block (with the norm's
+    running statistics kept); gradients of x and of every parameter of both modules against the two modules'
+    own operators one after the other, and the kept statistics against the fp64 oracle."""
+    rng = np.random.default_rng(71)
+    torch.manual_seed(17)
+    norm = M.TimestepNorm(D, G, prior_count=2).to(DEV).train()
+    move = M.MultiHeadComplexEMA(D, ndim=N).to(DEV).train()
+    with torch.no_grad():
+        norm.weight.normal_(0, 0.2); norm.bias.normal_(0, 0.2)
+        norm.prior_mean.normal_(0, 0.2); norm.prior_logv.normal_(0, 0.2)
+    x0 = torch.randn(B, L, D, device=DEV).mul_(1.3).add_(0.2).to(dtype)
+    w1 = torch.randn(B, L, D, device=DEV).to(dtype)
+    w2 = torch.randn(B, D, L, device=DEV).to(dtype)
+    mask = None
+    if masked:
+        mask = torch.from_numpy(rng.random((B, L)) < 0.2).to(DEV)
+    params = list(norm.parameters()) + list(move.parameters())
+
+    def run(enabled):
+        for q in params:
+            q.grad = None
+        x = x0.clone().requires_grad_(True)
+        M.modules.NormThenMoveFunc.ENABLED = enabled
+        try:
+            xn, y = M.norm_then_move(norm, move, x, mask, None, out_layout=layout)
+        finally:
+            M.modules.NormThenMoveFunc.ENABLED = True
+        assert y.shape == (B, D, L) and (layout == "rows") == y.is_contiguous()
+        ((xn * w1).sum() + (y * w2).sum()).backward()
+        torch.cuda.synchronize()
+        return xn.detach(), y.detach(), x.grad, [None if q.grad is None else q.grad.clone() for q in params]
+
+    xn_a, y_a, dx_a, g_a = run(True)
+    xn_b, y_b, dx_b, g_b = run(False)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    assert rel_err(host(xn_a), host(xn_b)) < tol and rel_err(host(y_a), host(y_b)) < tol
+    assert rel_err(host(dx_a), host(dx_b)) < tol
+    for (name, _), ga, gb in zip(list(norm.named_parameters()) + list(move.named_parameters()), g_a, g_b):
+        assert (ga is None) == (gb is None), name
+        if ga is not None:
+            assert rel_err(host(ga), host(gb)) < tol, name
+
+    # the statistics the one call keeps for the backward pass
+    layer = move._prepared_layer()
+    pc, pm, pv = norm._prior_state(B)
+    with torch.no_grad():
+        out = layer.norm_forward(x0, pc, pm, pv, norm.weight.float() + 1.0, norm.bias.float(), G, norm.eps, mask,
+                                 None, want_stats=True)
+    x64 = host(x0)
+    m64 = None if mask is None else host(mask).astype(bool)
+    ocnt, _, ocm, ocr = O.timestep_norm_saved(x64, host(pc).astype(np.int64), host(pm), host(pv), m64, G, norm.eps)
+    assert host(out[2]).tolist() == ocnt.tolist()
+    assert rel_err(host(out[6]), ocm) < 1e-4 and rel_err(host(out[7]), ocr) < 1e-4
+
+
 # ----------------------------------------------------------------------------------------------
 # moving-average layer
 # ----------------------------------------------------------------------------------------------

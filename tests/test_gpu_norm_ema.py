@@ -326,7 +326,7 @@ def test_module_pair_keeps_both_incremental_states():
     assert rel_err(host(sa['prev_var']), host(sb['prev_var'])) < 1e-5
     ha, hb = move._get_input_buffer(inc_a)['prev_state'], move._get_input_buffer(inc_b)['prev_state']
     assert rel_err(np.real(host(ha)), np.real(host(hb))) < 2e-3
-    # with autograd the pair runs as the two modules
+    # with autograd the pair is one differentiable operator
     xg = x[:, :64].float().requires_grad_(True)
     xn_g, y_g = M.norm_then_move(norm, move, xg)
     assert y_g.requires_grad and xn_g.requires_grad
