@@ -29,6 +29,7 @@ SOURCES = [
     "attention.hip",
     "attention_mfma.hip",
     "long_conv.hip",
+    "param_prep.hip",
 ]
 
 FLAGS = [

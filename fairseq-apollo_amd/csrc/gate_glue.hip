@@ -122,8 +122,8 @@ __global__ __launch_bounds__(kRowThreads) void gate_qk_kernel(const T* __restric
 template <typename T, int VEC, int NV>
 __global__ __launch_bounds__(kRowThreads) void gate_qk_bwd_kernel(
     const T* __restrict__ dq, const T* __restrict__ dk, const T* __restrict__ z, int64_t zs,
-    const float* __restrict__ gamma, const float* __restrict__ freqs, T* __restrict__ dz, float* __restrict__ part,
-    int64_t T_, int S, int Hd, int64_t chunk, int64_t pos0, float eps) {
+    const float* __restrict__ gamma, const float* __restrict__ freqs, T* __restrict__ dz, int64_t dzs,
+    float* __restrict__ part, int64_t T_, int S, int Hd, int64_t chunk, int64_t pos0, float eps) {
   using V = Vec<T, VEC>;
   static_assert(VEC % 2 == 0, "pairs of features stay inside one vector");
   extern __shared__ float s_acc[];                     // [4][S]
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kRowThreads) void gate_qk_bwd_kernel(
         V o;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) o.v[i] = from_float<T>((dzn[u][i] - zf[u][i] * dot) * inv);
-        *(V*)(dz + t * (int64_t)S + j) = o;
+        *(V*)(dz + t * dzs + j) = o;
       }
     }
   }
@@ -325,7 +325,8 @@ __device__ __forceinline__ float dsilu_f(float a) {
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void gate_mul_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ a,
                                                            int64_t as, const T* __restrict__ r, int64_t rs,
-                                                           T* __restrict__ da, T* __restrict__ dr, int64_t T_, int E) {
+                                                           T* __restrict__ da, T* __restrict__ dr, int64_t drs,
+                                                           int64_t T_, int E) {
   using V = Vec<T, VEC>;
   for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
     for (int j = threadIdx.x * VEC; j < E; j += 256 * VEC) {
@@ -340,7 +341,7 @@ __global__ __launch_bounds__(256) void gate_mul_bwd_kernel(const T* __restrict__
         orr.v[i] = from_float<T>(g * to_float(av.v[i]) * dsilu_f(rr));
       }
       *(V*)(da + t * (int64_t)E + j) = oa;
-      *(V*)(dr + t * (int64_t)E + j) = orr;
+      *(V*)(dr + t * drs + j) = orr;
     }
   }
 }
@@ -352,7 +353,8 @@ __global__ __launch_bounds__(256) void gate_out_bwd_kernel(const T* __restrict__
                                                            int64_t ress, const T* __restrict__ u, int64_t us,
                                                            const T* __restrict__ hx, int64_t hxs,
                                                            const T* __restrict__ hp, int64_t hps, T* __restrict__ dres,
-                                                           T* __restrict__ du, T* __restrict__ da, int64_t T_, int D) {
+                                                           T* __restrict__ du, int64_t dus, T* __restrict__ da,
+                                                           int64_t das, int64_t T_, int D) {
   using V = Vec<T, VEC>;
   for (int64_t t = blockIdx.x; t < T_; t += gridDim.x) {
     for (int j = threadIdx.x * VEC; j < D; j += 256 * VEC) {
@@ -372,8 +374,8 @@ __global__ __launch_bounds__(256) void gate_out_bwd_kernel(const T* __restrict__
         o2.v[i] = from_float<T>(g * sg * dsilu_f(a));
       }
       *(V*)(dres + t * (int64_t)D + j) = o0;
-      *(V*)(du + t * (int64_t)D + j) = o1;
-      *(V*)(da + t * (int64_t)D + j) = o2;
+      *(V*)(du + t * dus + j) = o1;
+      *(V*)(da + t * das + j) = o2;
     }
   }
 }
@@ -461,11 +463,11 @@ inline int64_t gate_qk_bwd_wgs(int64_t T_) {
 
 template <typename T>
 int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs, const float* gamma,
-                       const float* freqs, void* dz, float* dgamma, float* dbeta, float* part, int64_t T_, int64_t S,
-                       int64_t Hd, int64_t chunk, int64_t pos0, float eps, hipStream_t s) {
+                       const float* freqs, void* dz, int64_t dzs, float* dgamma, float* dbeta, float* part, int64_t T_,
+                       int64_t S, int64_t Hd, int64_t chunk, int64_t pos0, float eps, hipStream_t s) {
   constexpr int VEC = 16 / (int)sizeof(T);
   MEGA_REQUIRE(S % VEC == 0 && S <= 2 * 64 * VEC && vec_ok(z, zs, sizeof(T), VEC) && vec_ok(dq, S, sizeof(T), VEC) &&
-                   vec_ok(dk, S, sizeof(T), VEC) && vec_ok(dz, S, sizeof(T), VEC),
+                   vec_ok(dk, S, sizeof(T), VEC) && vec_ok(dz, dzs, sizeof(T), VEC),
                MEGA_ERR_UNSUPPORTED,
                "gate_qk_bwd: S=%lld must be a multiple of %d, at most %d, with 16-byte aligned rows", (long long)S, VEC,
                2 * 64 * VEC);
@@ -476,7 +478,7 @@ int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs
     audit_use(part, (size_t)grid * 4 * S * 4, "gate_qk_bwd: rows of parameter sums");
     audit_use(dq, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: q_grad");
     audit_use(dk, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: k_grad");
-    audit_use(dz, (size_t)T_ * S * sizeof(T), "gate_qk_bwd: z_grad");
+    audit_use(dz, (size_t)((T_ - 1) * dzs + S) * sizeof(T), "gate_qk_bwd: z_grad");
     audit_use(z, (size_t)((T_ - 1) * zs + S) * sizeof(T), "gate_qk_bwd: z");
     audit_use(dgamma, (size_t)2 * S * 4, "gate_qk_bwd: gamma_grad");
     audit_use(dbeta, (size_t)2 * S * 4, "gate_qk_bwd: beta_grad");
@@ -484,10 +486,10 @@ int launch_gate_qk_bwd(const void* dq, const void* dk, const void* z, int64_t zs
   }
   if (S <= 64 * VEC)
     hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 1>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
-                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
+                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, dzs, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
   else
     hipLaunchKernelGGL((gate_qk_bwd_kernel<T, VEC, 2>), dim3(grid), dim3(kRowThreads), lds, s, (const T*)dq,
-                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
+                       (const T*)dk, (const T*)z, zs, gamma, freqs, (T*)dz, dzs, part, T_, (int)S, (int)Hd, chunk, pos0, eps);
   MEGA_CHECK_LAUNCH("gate_qk_bwd");
   hipLaunchKernelGGL(gate_qk_param_kernel, dim3((unsigned)ceil_div(4 * S, 64)), dim3(64 * kParamSlices), 0, s, part,
                      (int)grid,
@@ -527,36 +529,36 @@ int launch_gate_out(const void* res, int64_t ress, const void* u, int64_t us, co
 
 template <typename T>
 int launch_gate_mul_bwd(const void* dy, const void* a, int64_t as, const void* r, int64_t rs, void* da, void* dr,
-                        int64_t T_, int64_t E, hipStream_t s) {
+                        int64_t drs, int64_t T_, int64_t E, hipStream_t s) {
   constexpr int VEC = 16 / (int)sizeof(T);
   const bool v = E % VEC == 0 && vec_ok(dy, E, sizeof(T), VEC) && vec_ok(a, as, sizeof(T), VEC) &&
-                 vec_ok(r, rs, sizeof(T), VEC) && vec_ok(da, E, sizeof(T), VEC) && vec_ok(dr, E, sizeof(T), VEC);
+                 vec_ok(r, rs, sizeof(T), VEC) && vec_ok(da, E, sizeof(T), VEC) && vec_ok(dr, drs, sizeof(T), VEC);
   if (v)
     hipLaunchKernelGGL((gate_mul_bwd_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)a,
-                       as, (const T*)r, rs, (T*)da, (T*)dr, T_, (int)E);
+                       as, (const T*)r, rs, (T*)da, (T*)dr, drs, T_, (int)E);
   else
     hipLaunchKernelGGL((gate_mul_bwd_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)a, as,
-                       (const T*)r, rs, (T*)da, (T*)dr, T_, (int)E);
+                       (const T*)r, rs, (T*)da, (T*)dr, drs, T_, (int)E);
   MEGA_CHECK_LAUNCH("gate_mul_bwd");
   return MEGA_OK;
 }
 
 template <typename T>
 int launch_gate_out_bwd(const void* dy, const void* res, int64_t ress, const void* u, int64_t us, const void* hx,
-                        int64_t hxs, const void* hp, int64_t hps, void* dres, void* du, void* da, int64_t T_,
-                        int64_t D, hipStream_t s) {
+                        int64_t hxs, const void* hp, int64_t hps, void* dres, void* du, int64_t dus, void* da,
+                        int64_t das, int64_t T_, int64_t D, hipStream_t s) {
   constexpr int VEC = 16 / (int)sizeof(T);
   const bool v = D % VEC == 0 && vec_ok(dy, D, sizeof(T), VEC) && vec_ok(res, ress, sizeof(T), VEC) &&
                  vec_ok(u, us, sizeof(T), VEC) && vec_ok(hx, hxs, sizeof(T), VEC) && vec_ok(hp, hps, sizeof(T), VEC) &&
-                 vec_ok(dres, D, sizeof(T), VEC) && vec_ok(du, D, sizeof(T), VEC) && vec_ok(da, D, sizeof(T), VEC);
+                 vec_ok(dres, D, sizeof(T), VEC) && vec_ok(du, dus, sizeof(T), VEC) && vec_ok(da, das, sizeof(T), VEC);
   if (v)
     hipLaunchKernelGGL((gate_out_bwd_kernel<T, VEC>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)res,
-                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, (T*)da, T_,
-                       (int)D);
+                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, dus, (T*)da, das,
+                       T_, (int)D);
   else
     hipLaunchKernelGGL((gate_out_bwd_kernel<T, 1>), dim3(row_grid(T_)), dim3(256), 0, s, (const T*)dy, (const T*)res,
-                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, (T*)da, T_,
-                       (int)D);
+                       ress, (const T*)u, us, (const T*)hx, hxs, (const T*)hp, hps, (T*)dres, (T*)du, dus, (T*)da, das,
+                       T_, (int)D);
   MEGA_CHECK_LAUNCH("gate_out_bwd");
   return MEGA_OK;
 }
@@ -630,10 +632,11 @@ extern "C" size_t mega_gate_qk_bwd_workspace_bytes(int64_t T_, int64_t S) {
   return align_up((size_t)gate_qk_bwd_wgs(T_) * 4 * (size_t)S * sizeof(float), 256);
 }
 
-extern "C" int mega_gate_qk_bwd(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
-                                const float* gamma, const float* freqs, void* z_grad, float* gamma_grad,
-                                float* beta_grad, int dtype, int64_t T_, int64_t S, int64_t heads, int64_t chunk,
-                                int64_t pos0, double eps, void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int mega_gate_qk_bwd_strided(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
+                                        const float* gamma, const float* freqs, void* z_grad, int64_t z_grad_stride,
+                                        float* gamma_grad, float* beta_grad, int dtype, int64_t T_, int64_t S,
+                                        int64_t heads, int64_t chunk, int64_t pos0, double eps, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_qk_bwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(T_ >= 0 && S >= 2 && S < (1ll << 30) && heads >= 1 && chunk >= 1 && pos0 >= 0, MEGA_ERR_ARG,
                "gate_qk_bwd: bad sizes T=%lld S=%lld heads=%lld chunk=%lld pos0=%lld", (long long)T_, (long long)S,
@@ -648,13 +651,22 @@ extern "C" int mega_gate_qk_bwd(const void* q_grad, const void* k_grad, const vo
     return MEGA_OK;
   }
   MEGA_REQUIRE(q_grad && k_grad && z && gamma && freqs && z_grad, MEGA_ERR_ARG, "gate_qk_bwd: null pointer argument");
-  MEGA_REQUIRE(z_stride >= S, MEGA_ERR_ARG, "gate_qk_bwd: row stride %lld below the row length %lld",
-               (long long)z_stride, (long long)S);
+  MEGA_REQUIRE(z_stride >= S && z_grad_stride >= S, MEGA_ERR_ARG,
+               "gate_qk_bwd: row stride %lld / %lld below the row length %lld", (long long)z_stride,
+               (long long)z_grad_stride, (long long)S);
   const size_t need = mega_gate_qk_bwd_workspace_bytes(T_, S);
   MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
                "gate_qk_bwd: workspace of %zu bytes (16-byte aligned) needed", need);
-  MEGA_GLUE_DISPATCH(launch_gate_qk_bwd, q_grad, k_grad, z, z_stride, gamma, freqs, z_grad, gamma_grad, beta_grad,
-                     (float*)workspace, T_, S, S / heads, chunk, pos0, (float)eps, s);
+  MEGA_GLUE_DISPATCH(launch_gate_qk_bwd, q_grad, k_grad, z, z_stride, gamma, freqs, z_grad, z_grad_stride, gamma_grad,
+                     beta_grad, (float*)workspace, T_, S, S / heads, chunk, pos0, (float)eps, s);
+}
+
+extern "C" int mega_gate_qk_bwd(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
+                                const float* gamma, const float* freqs, void* z_grad, float* gamma_grad,
+                                float* beta_grad, int dtype, int64_t T_, int64_t S, int64_t heads, int64_t chunk,
+                                int64_t pos0, double eps, void* workspace, size_t workspace_bytes, void* stream) {
+  return mega_gate_qk_bwd_strided(q_grad, k_grad, z, z_stride, gamma, freqs, z_grad, S, gamma_grad, beta_grad, dtype,
+                                  T_, S, heads, chunk, pos0, eps, workspace, workspace_bytes, stream);
 }
 
 extern "C" int mega_gate_mul_fwd(const void* a, int64_t a_stride, const void* r, int64_t r_stride, void* y, int dtype,
@@ -684,33 +696,50 @@ extern "C" int mega_gate_out_fwd(const void* residual, int64_t residual_stride, 
                      s);
 }
 
-extern "C" int mega_gate_mul_bwd(const void* y_grad, const void* a, int64_t a_stride, const void* r, int64_t r_stride,
-                                 void* a_grad, void* r_grad, int dtype, int64_t T_, int64_t E, void* stream) {
+extern "C" int mega_gate_mul_bwd_strided(const void* y_grad, const void* a, int64_t a_stride, const void* r,
+                                         int64_t r_stride, void* a_grad, void* r_grad, int64_t r_grad_stride,
+                                         int dtype, int64_t T_, int64_t E, void* stream) {
   MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_mul_bwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(T_ >= 0 && E >= 1 && E < (1ll << 30), MEGA_ERR_ARG, "gate_mul_bwd: bad sizes T=%lld E=%lld",
                (long long)T_, (long long)E);
   if (T_ == 0) return MEGA_OK;
   MEGA_REQUIRE(y_grad && a && r && a_grad && r_grad, MEGA_ERR_ARG, "gate_mul_bwd: null pointer argument");
-  MEGA_REQUIRE(a_stride >= E && r_stride >= E, MEGA_ERR_ARG, "gate_mul_bwd: a row stride is below the row length");
+  MEGA_REQUIRE(a_stride >= E && r_stride >= E && r_grad_stride >= E, MEGA_ERR_ARG,
+               "gate_mul_bwd: a row stride is below the row length");
   hipStream_t s = (hipStream_t)stream;
-  MEGA_GLUE_DISPATCH(launch_gate_mul_bwd, y_grad, a, a_stride, r, r_stride, a_grad, r_grad, T_, E, s);
+  MEGA_GLUE_DISPATCH(launch_gate_mul_bwd, y_grad, a, a_stride, r, r_stride, a_grad, r_grad, r_grad_stride, T_, E, s);
 }
 
-extern "C" int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual_stride, const void* u,
-                                 int64_t u_stride, const void* hx, int64_t hx_stride, const void* hp,
-                                 int64_t hp_stride, void* residual_grad, void* u_grad, void* h_grad, int dtype,
-                                 int64_t T_, int64_t D, void* stream) {
+extern "C" int mega_gate_mul_bwd(const void* y_grad, const void* a, int64_t a_stride, const void* r, int64_t r_stride,
+                                 void* a_grad, void* r_grad, int dtype, int64_t T_, int64_t E, void* stream) {
+  return mega_gate_mul_bwd_strided(y_grad, a, a_stride, r, r_stride, a_grad, r_grad, E, dtype, T_, E, stream);
+}
+
+extern "C" int mega_gate_out_bwd_strided(const void* y_grad, const void* residual, int64_t residual_stride,
+                                         const void* u, int64_t u_stride, const void* hx, int64_t hx_stride,
+                                         const void* hp, int64_t hp_stride, void* residual_grad, void* u_grad,
+                                         int64_t u_grad_stride, void* h_grad, int64_t h_grad_stride, int dtype,
+                                         int64_t T_, int64_t D, void* stream) {
   MEGA_REQUIRE(known_dtype(dtype), MEGA_ERR_ARG, "gate_out_bwd: unknown dtype %d", dtype);
   MEGA_REQUIRE(T_ >= 0 && D >= 1 && D < (1ll << 30), MEGA_ERR_ARG, "gate_out_bwd: bad sizes T=%lld D=%lld",
                (long long)T_, (long long)D);
   if (T_ == 0) return MEGA_OK;
   MEGA_REQUIRE(y_grad && residual && u && hx && hp && residual_grad && u_grad && h_grad, MEGA_ERR_ARG,
                "gate_out_bwd: null pointer argument");
-  MEGA_REQUIRE(residual_stride >= D && u_stride >= D && hx_stride >= D && hp_stride >= D, MEGA_ERR_ARG,
-               "gate_out_bwd: a row stride is below the row length");
+  MEGA_REQUIRE(residual_stride >= D && u_stride >= D && hx_stride >= D && hp_stride >= D && u_grad_stride >= D &&
+                   h_grad_stride >= D,
+               MEGA_ERR_ARG, "gate_out_bwd: a row stride is below the row length");
   hipStream_t s = (hipStream_t)stream;
   MEGA_GLUE_DISPATCH(launch_gate_out_bwd, y_grad, residual, residual_stride, u, u_stride, hx, hx_stride, hp, hp_stride,
-                     residual_grad, u_grad, h_grad, T_, D, s);
+                     residual_grad, u_grad, u_grad_stride, h_grad, h_grad_stride, T_, D, s);
+}
+
+extern "C" int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual_stride, const void* u,
+                                 int64_t u_stride, const void* hx, int64_t hx_stride, const void* hp,
+                                 int64_t hp_stride, void* residual_grad, void* u_grad, void* h_grad, int dtype,
+                                 int64_t T_, int64_t D, void* stream) {
+  return mega_gate_out_bwd_strided(y_grad, residual, residual_stride, u, u_stride, hx, hx_stride, hp, hp_stride,
+                                   residual_grad, u_grad, D, h_grad, D, dtype, T_, D, stream);
 }
 
 extern "C" int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_grad, void* b_grad, int dtype,

@@ -22,8 +22,9 @@ from torch import Tensor, nn
 from torch.nn import Parameter
 
 from . import ops
-from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState, MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SwiGLU, linear_residual, norm_then_move,
-                      TimestepNorm, _tensor_versions, _training_call)
+from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState,
+                      MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SplitFunc, SplitGrads, SwiGLU, TimestepNorm,
+                      _tensor_versions, _training_call, linear_residual, norm_then_move)
 
 
 class RMSNorm(nn.Module):
@@ -414,12 +415,15 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         residual = x
         if self.bidirectional:
             x = self.norm(x, padding_mask, length_last=False)
+            mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
         else:
-            x = self.norm(x, padding_mask=padding_mask)
+            x, mx = norm_then_move(self.norm, self.move, x, padding_mask, None, out_layout="input")
+            mx = mx.transpose(1, 2)
         v = F.silu(self.v_proj(x))
-        mx = self.move(x.transpose(1, 2), padding_mask, None, out_layout="input").transpose(1, 2)
         base = self.mx_proj(F.dropout(self.move_act(mx), self.hidden_dropout_p, self.training))
-        u, z, r, hx = torch.split(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim], dim=-1)
+        # the four slices' gradients are written into one buffer by the backward kernels of their consumers
+        arena = SplitGrads(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim])
+        u, z, r, hx = SplitFunc.apply(base, arena)
         Nh = self.num_heads
         C = self.chunk_size if 1 < self.chunk_size < seq_len else seq_len
         nc = seq_len // C
@@ -429,7 +433,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         if self.zdim % vec == 0 and self.zdim <= 128 * vec:
             # one kernel forward, one backward (rows of whole 16-byte vectors, at most two per lane)
             freqs = self._no_rotation if simple else self.rel_pos_bias.freqs
-            q, k = GateQKFunc.apply(z, self.gamma, self.beta, freqs.detach().float().contiguous(), Nh, C)
+            q, k = GateQKFunc.apply(z, self.gamma, self.beta, freqs.detach().float().contiguous(), Nh, C, (arena, 1))
             q4 = q.view(bsz * nc, C, Nh, -1)
             k4 = k.view(bsz * nc, C, Nh, -1)
         else:
@@ -461,14 +465,14 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             attn = torch.einsum('bnqk,bknh->bqnh', w, v4)
         else:
             attn = self.efficient_attn(q4, k4, v4)
-        gated = GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r)
+        gated = GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r, (arena, 2))
         hp = self.h_proj(F.dropout(gated, self.hidden_dropout_p, self.training))
         if self.training and self.dropout_p > 0:
             # the output dropout sits between the activation and the residual mix
             # (moving_average_gated_attention.py:409-412), so the fused gate is taken apart
             h = F.dropout(F.silu(hx + hp), self.dropout_p, True)
             return torch.addcmul(residual, torch.sigmoid(u), h - residual)
-        return GateOutFunc.apply(residual, u, hx, hp)
+        return GateOutFunc.apply(residual, u, hx, hp, (arena, 0, 3))
 
     def _cached_attention(self, z: Tensor, v: Tensor, saved_state, incremental_state) -> Tensor:
         """Attention with the partial-chunk key / value cache

@@ -96,6 +96,60 @@ def _tensor_versions(*modules: nn.Module) -> tuple:
                  for t in (*m._parameters.values(), *m._buffers.values()) if t is not None)
 
 
+class EMACoeffsFunc(torch.autograd.Function):
+    """(p, q, gamma, omega) of a moving-average layer from its stored parameters, one launch forwards and one
+    backwards (the chain of torch operations of complex_exponential_moving_average.py:79-96 and
+    exponential_moving_average.py:71-80, which `_calc_coeffs_torch` of the two classes keeps): parameters are read
+    in their storage type, results are fp32 in the library's layout, parameter gradients come back in the
+    storage type."""
+
+    @staticmethod
+    def forward(ctx, alpha, delta, third, gamma, omega, is_complex):
+        p, q2, g2, om = ops.ema_coeffs_fwd(alpha, delta, third, gamma, omega, is_complex)
+        ctx.save_for_backward(alpha, delta, third)
+        ctx.is_complex = is_complex
+        ctx.like = (gamma.shape, omega.shape)
+        if is_complex:
+            return p.unsqueeze(-1), torch.view_as_complex(q2).unsqueeze(-1), torch.view_as_complex(g2), om.view(omega.shape)
+        return p.unsqueeze(-1), q2[..., 0].unsqueeze(-1), g2[..., 0], om.view(omega.shape)
+
+    @staticmethod
+    def backward(ctx, p_grad, q_grad, g_grad, om_grad):
+        alpha, delta, third = ctx.saved_tensors
+        if ctx.is_complex:
+            q_grad = torch.view_as_real(q_grad.resolve_conj().contiguous())
+            g_grad = torch.view_as_real(g_grad.resolve_conj().contiguous())
+        gl = torch.empty(ctx.like[0], dtype=alpha.dtype, device="meta")
+        ol = torch.empty(ctx.like[1], dtype=alpha.dtype, device="meta")
+        da, dd, dt, dg, dom = ops.ema_coeffs_bwd(p_grad, q_grad, g_grad, om_grad, alpha, delta, third, gl, ol,
+                                                 ctx.is_complex)
+        return da, dd, dt, dg, dom, None
+
+
+def _one_cuda_dtype(*ts) -> bool:
+    return all(t.is_cuda for t in ts) and len({t.dtype for t in ts}) == 1 and \
+        ts[0].dtype in (torch.float32, torch.bfloat16, torch.float16)
+
+
+class NormParamsFunc(torch.autograd.Function):
+    """(weight + 1, bias, prior mean and exp(prior log-variance) over the batch) in fp32 from TimestepNorm's
+    parameters, one launch each way (timestep_norm.py:118-131)."""
+
+    @staticmethod
+    def forward(ctx, weight, bias, prior_mean, prior_logv, batch_size):
+        ctx.save_for_backward(weight, prior_mean, prior_logv)
+        ctx.batch_size = batch_size
+        ctx.prior_needs_grad = prior_mean.requires_grad or prior_logv.requires_grad
+        return ops.norm_params_fwd(weight, bias, prior_mean, prior_logv, batch_size)
+
+    @staticmethod
+    def backward(ctx, gamma_grad, beta_grad, mean_grad, var_grad):
+        weight, prior_mean, prior_logv = ctx.saved_tensors
+        dw, db, dpm, dpl = ops.norm_params_bwd(gamma_grad, beta_grad, mean_grad, var_grad, weight, prior_mean,
+                                               prior_logv, ctx.batch_size, ctx.prior_needs_grad)
+        return dw, db, dpm, dpl, None
+
+
 class BaseMovingLayer(nn.Module, IncrementalState):
     """fairseq/modules/base_moving_average.py:18-197."""
 
@@ -182,8 +236,8 @@ class BaseMovingLayer(nn.Module, IncrementalState):
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
             if incremental_state is not None or (self.truncation is not None and self.truncation >= 1):
                 return self._chained_forward(x, padding_mask, incremental_state, out_layout)
-            p, q, gamma = self._calc_coeffs()           # stays in the graph
-            return MovingAverageFunc.apply(x, p, q, gamma, self.omega, padding_mask, out_layout, self.bidirectional,
+            p, q, gamma, omega = self._calc_all()       # stays in the graph
+            return MovingAverageFunc.apply(x, p, q, gamma, omega, padding_mask, out_layout, self.bidirectional,
                                            self.shift)
         layer = self._prepared_layer()
         if incremental_state is not None:
@@ -296,8 +350,17 @@ class MultiHeadEMA(BaseMovingLayer):
 
     def _calc_coeffs(self):
         """p = sigmoid(alpha) beta, q = 1 - sigmoid(alpha) sigmoid(delta), gamma scaled by sqrt(1 / N)
-        (exponential_moving_average.py:71-80)."""
+        (exponential_moving_average.py:71-80); on the GPU one launch."""
         self._coeffs = None
+        return self._calc_all()[:3]
+
+    def _calc_all(self):
+        """(p, q, gamma, omega): the coefficients and the residual weight as the kernels take them."""
+        if _one_cuda_dtype(self.alpha, self.delta, self.beta, self.gamma, self.omega):
+            return EMACoeffsFunc.apply(self.alpha, self.delta, self.beta, self.gamma, self.omega, False)
+        return self._calc_coeffs_torch() + (self.omega,)
+
+    def _calc_coeffs_torch(self):
         a = torch.sigmoid(self.alpha.float())
         return a * self.beta.float(), 1.0 - a * torch.sigmoid(self.delta.float()), self.gamma.float() * self.scale
 
@@ -340,8 +403,17 @@ class MultiHeadComplexEMA(BaseMovingLayer):
     def _calc_coeffs(self):
         """p = sigmoid(alpha); q: state n of a channel shrinks by 1 - sigmoid(alpha) sigmoid(delta) and turns by
         (n + 1) sigmoid(theta) 2 pi / N per token; gamma complex, scaled by sqrt(1 / N)
-        (complex_exponential_moving_average.py:79-96)."""
+        (complex_exponential_moving_average.py:79-96); on the GPU one launch."""
         self._coeffs = None
+        return self._calc_all()[:3]
+
+    def _calc_all(self):
+        """(p, q, gamma, omega): the coefficients and the residual weight as the kernels take them."""
+        if _one_cuda_dtype(self.alpha, self.delta, self.theta, self.gamma, self.omega):
+            return EMACoeffsFunc.apply(self.alpha, self.delta, self.theta, self.gamma, self.omega, True)
+        return self._calc_coeffs_torch() + (self.omega,)
+
+    def _calc_coeffs_torch(self):
         a = torch.sigmoid(self.alpha.float())
         d = torch.sigmoid(self.delta.float())
         turn = torch.sigmoid(self.theta.float()) * (2.0 * math.pi / self.ndim)                      # [K, 1, 1]
@@ -430,6 +502,9 @@ class TimestepNorm(nn.Module, IncrementalState):
                 assert 'prev_var' in saved_state and 'prev_count' in saved_state
                 prev_var = saved_state['prev_var']
                 prev_count = saved_state['prev_count']
+        norm_gamma = norm_beta = None
+        if train and prev_count is None and prev_mean is None and prev_var is None:
+            prev_count, norm_gamma, norm_beta, prev_mean, prev_var = self._training_operands(batch_size)
         if prev_count is None or prev_mean is None or prev_var is None:
             d_count, d_mean, d_var = self._prior_state(batch_size, train)
             prev_count = d_count if prev_count is None else prev_count
@@ -438,8 +513,10 @@ class TimestepNorm(nn.Module, IncrementalState):
         if train:
             # the autograd path of the reference (timestep_norm.py:129-136): prior, weight + 1 and
             # bias stay in the graph; statistics for the backward pass are kept
-            out, count, mean, var = timestep_norm(x, prev_count, prev_mean, prev_var, self.weight.float() + 1.0,
-                                                  self.bias.float(), padding_mask, self.num_groups, self.eps)
+            if norm_gamma is None:
+                norm_gamma, norm_beta = self.weight.float() + 1.0, self.bias.float()
+            out, count, mean, var = timestep_norm(x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta,
+                                                  padding_mask, self.num_groups, self.eps)
             if incremental_state is not None:
                 saved_state['prev_mean'], saved_state['prev_var'], saved_state['prev_count'] = mean, var, count
                 self._set_input_buffer(incremental_state, saved_state)
@@ -458,6 +535,16 @@ class TimestepNorm(nn.Module, IncrementalState):
             saved_state['prev_count'] = count
             self._set_input_buffer(incremental_state, saved_state)
         return out
+
+    def _training_operands(self, batch_size: int):
+        """(count [B], weight + 1 [H], bias [H], prior mean [B, G], prior variance [B, G]) with the last four in the
+        autograd graph (timestep_norm.py:118-131): one launch on the GPU, torch operations elsewhere."""
+        count = self.prior_count.expand(batch_size).contiguous()
+        if _one_cuda_dtype(self.weight, self.bias) and _one_cuda_dtype(self.prior_mean, self.prior_logv):
+            return (count,) + tuple(NormParamsFunc.apply(self.weight, self.bias, self.prior_mean, self.prior_logv,
+                                                         batch_size))
+        _, mean, var = self._prior_state(batch_size, differentiable=True)
+        return count, self.weight.float() + 1.0, self.bias.float(), mean, var
 
     def _prior_state(self, batch_size: int, differentiable: bool = False):
         """(count[B], mean[B,G], var[B,G]) of the prior (timestep_norm.py:122-127); cached in eval mode."""
@@ -582,11 +669,10 @@ def norm_then_move(norm: nn.Module, move: nn.Module, x: Tensor, padding_mask: Op
                 and x.is_cuda and x.dim() == 3 and x.size(0) > 0 and x.size(1) > 0)
     training = one_call and (_training_call(norm, x) or _training_call(move, x))
     if training and incremental_state is None and NormThenMoveFunc.ENABLED:
-        prev_count, prev_mean, prev_var = norm._prior_state(x.size(0), differentiable=True)
-        p, q, gamma = move._calc_coeffs()               # stay in the graph
-        return NormThenMoveFunc.apply(x, prev_count, prev_mean, prev_var, norm.weight.float() + 1.0,
-                                      norm.bias.float(), p, q, gamma, move.omega, padding_mask, norm.num_groups,
-                                      norm.eps, out_layout, move.shift)
+        prev_count, norm_gamma, norm_beta, prev_mean, prev_var = norm._training_operands(x.size(0))
+        p, q, gamma, omega = move._calc_all()           # stay in the graph
+        return NormThenMoveFunc.apply(x, prev_count, prev_mean, prev_var, norm_gamma, norm_beta, p, q, gamma, omega,
+                                      padding_mask, norm.num_groups, norm.eps, out_layout, move.shift)
     if not one_call or training:
         xn = norm(x, padding_mask=padding_mask, incremental_state=incremental_state)
         return xn, move(xn.transpose(1, 2), padding_mask, incremental_state, out_layout=out_layout)
@@ -666,37 +752,95 @@ class SequenceNorm(nn.Module):
         return 'num_features={num_features}, num_groups={num_groups}, eps={eps}'.format(**self.__dict__)
 
 
+class SplitGrads(object):
+    """The gradients of the slices of one split tensor, written in place.  `torch.split` hands every slice's
+    gradient to a concatenation in its backward pass (the mx_proj output of
+    moving_average_gated_attention.py:319 is split four ways: a 142 MB copy per step at the Mega2 layer's size).
+    The backward kernels of the slices' consumers instead write into the slices of one buffer that this
+    object hands out (`slot(i)`), and SplitFunc's backward returns that buffer when every gradient it receives
+    is the slot it handed out, and concatenates otherwise.  A new buffer per backward pass."""
+
+    taken = 0        # backward passes that needed no concatenation (all objects; read by the tests)
+
+    def __init__(self, like: Tensor, widths):
+        self.shape, self.dtype, self.device = like.shape, like.dtype, like.device
+        self.widths = list(widths)
+        self.offsets = [sum(self.widths[:i]) for i in range(len(self.widths))]
+        self.buf = None
+
+    def slot(self, i: int) -> Tensor:
+        if self.buf is None:
+            self.buf = torch.empty(self.shape, dtype=self.dtype, device=self.device)
+        return self.buf.narrow(-1, self.offsets[i], self.widths[i])
+
+    def take(self, grads) -> Optional[Tensor]:
+        """The buffer, if `grads` are exactly its slots; the buffer is released either way."""
+        buf, self.buf = self.buf, None
+        if buf is None or len(grads) != len(self.widths):
+            return None
+        for i, g in enumerate(grads):
+            if g is None or g.dtype != buf.dtype or g.shape[:-1] != buf.shape[:-1] or g.shape[-1] != self.widths[i] \
+                    or g.stride() != buf.stride() \
+                    or g.data_ptr() != buf.data_ptr() + self.offsets[i] * buf.element_size():
+                return None
+        SplitGrads.taken += 1
+        return buf
+
+
+class SplitFunc(torch.autograd.Function):
+    """torch.split(base, widths, -1) whose backward takes the slices' gradients from a SplitGrads buffer."""
+
+    @staticmethod
+    def forward(ctx, base, arena):
+        ctx.arena = arena
+        return tuple(base.narrow(-1, o, w) for o, w in zip(arena.offsets, arena.widths))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        arena = ctx.arena
+        buf = arena.take(grads)
+        if buf is not None:
+            return buf, None
+        parts = [g if g is not None else torch.zeros(arena.shape[:-1] + (w,), dtype=arena.dtype, device=arena.device)
+                 for g, w in zip(grads, arena.widths)]
+        return torch.cat(parts, dim=-1), None
+
+
 class GateQKFunc(torch.autograd.Function):
     """q, k = rotary(normalize(z) * (gamma + 1) + beta) in one pass over z, with one backward pass
     (moving_average_gated_attention.py:324-328, relative_positional_bias.py:86-97).  gamma, beta are
     the layer's [2, S] parameters; freqs holds zeros when the layer does not rotate."""
 
     @staticmethod
-    def forward(ctx, z, gamma, beta, freqs, num_heads, chunk):
+    def forward(ctx, z, gamma, beta, freqs, num_heads, chunk, slot=None):
         g1 = gamma.detach().float() + 1.0
         ctx.save_for_backward(z, g1, freqs)
-        ctx.num_heads, ctx.chunk = num_heads, chunk
+        ctx.num_heads, ctx.chunk, ctx.slot = num_heads, chunk, slot
         ctx.param_dtypes = (gamma.dtype, beta.dtype)
         return ops.gate_qk_fwd(z, g1, beta.detach().float(), freqs, num_heads, chunk)
 
     @staticmethod
     def backward(ctx, q_grad, k_grad):
         z, g1, freqs = ctx.saved_tensors
-        dz, dgamma, dbeta = ops.gate_qk_bwd(q_grad, k_grad, z, g1, freqs, ctx.num_heads, ctx.chunk)
-        return dz, dgamma.to(ctx.param_dtypes[0]), dbeta.to(ctx.param_dtypes[1]), None, None, None
+        out = None if ctx.slot is None else ctx.slot[0].slot(ctx.slot[1])
+        dz, dgamma, dbeta = ops.gate_qk_bwd(q_grad, k_grad, z, g1, freqs, ctx.num_heads, ctx.chunk, z_grad_out=out)
+        return dz, dgamma.to(ctx.param_dtypes[0]), dbeta.to(ctx.param_dtypes[1]), None, None, None, None
 
 
 class GateMulFunc(torch.autograd.Function):
     """a * silu(r) with its own backward (moving_average_gated_attention.py:330, 407)."""
 
     @staticmethod
-    def forward(ctx, a, r):
+    def forward(ctx, a, r, slot=None):
         ctx.save_for_backward(a, r)
+        ctx.slot = slot
         return ops.gate_mul_fwd(a, r)
 
     @staticmethod
     def backward(ctx, y_grad):
-        return ops.gate_mul_bwd(y_grad, *ctx.saved_tensors)
+        out = None if ctx.slot is None else ctx.slot[0].slot(ctx.slot[1])
+        da, dr = ops.gate_mul_bwd(y_grad, *ctx.saved_tensors, r_grad_out=out)
+        return da, dr, None
 
 
 class GateOutFunc(torch.autograd.Function):
@@ -704,14 +848,19 @@ class GateOutFunc(torch.autograd.Function):
     (moving_average_gated_attention.py:322, 409, 412)."""
 
     @staticmethod
-    def forward(ctx, residual, u, hx, hp):
+    def forward(ctx, residual, u, hx, hp, slots=None):
         ctx.save_for_backward(residual, u, hx, hp)
+        ctx.slots = slots
         return ops.gate_out_fwd(residual, u, hx, hp)
 
     @staticmethod
     def backward(ctx, y_grad):
-        dres, du, dh = ops.gate_out_bwd(y_grad, *ctx.saved_tensors)
-        return dres, du, dh, dh
+        uo = ho = None
+        if ctx.slots is not None:
+            arena, iu, ih = ctx.slots
+            uo, ho = arena.slot(iu), arena.slot(ih)
+        dres, du, dh = ops.gate_out_bwd(y_grad, *ctx.saved_tensors, u_grad_out=uo, h_grad_out=ho)
+        return dres, du, dh, dh, None
 
 
 class SwiGLUFunc(torch.autograd.Function):

@@ -147,6 +147,103 @@ def check_lookback(where: str = "") -> None:
 # --------------------------------------------------------------------------------------
 
 
+def ema_coeffs_fwd(alpha: torch.Tensor, delta: torch.Tensor, third: torch.Tensor, gamma: torch.Tensor,
+                   omega: torch.Tensor, is_complex: bool):
+    """The layer's coefficients from its stored parameters in one launch
+    (complex_exponential_moving_average.py:79-96 / exponential_moving_average.py:71-80): alpha, delta [K, N, 1];
+    third = theta [K, 1, 1] (complex) or beta [K, N, 1] (real); gamma [K, N, 2] or [K, N]; omega [D(, 1)], all of one
+    dtype.  -> (p [K, N], q [K, N, 2], gamma [K, N, 2], omega [D]) in fp32, the library's own layout."""
+    dev = _need_gpu(alpha, delta, third, gamma, omega)
+    lib = _lib.load()
+    K, N = alpha.shape[0], alpha.shape[1]
+    D = omega.numel()
+    ts = [t.detach().contiguous() for t in (alpha, delta, third, gamma, omega)]
+    if len({t.dtype for t in ts}) != 1:
+        raise RuntimeError("ema_coeffs_fwd: the parameters must share one dtype")
+    if ts[1].numel() != K * N or ts[2].numel() != (K if is_complex else K * N) or \
+            ts[3].numel() != (2 * K * N if is_complex else K * N):
+        raise RuntimeError("ema_coeffs_fwd: parameter shapes do not belong to one layer")
+    p = torch.empty(K, N, dtype=torch.float32, device=dev)
+    q = torch.empty(K, N, 2, dtype=torch.float32, device=dev)
+    g = torch.empty(K, N, 2, dtype=torch.float32, device=dev)
+    om = torch.empty(D, dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_ema_coeffs_fwd(_ptr(ts[0]), _ptr(ts[1]), _ptr(ts[2]), _ptr(ts[3]), _ptr(ts[4]), _dtype_code(ts[0]),
+                                     1 if is_complex else 0, K, N, D, _ptr(p), _ptr(q), _ptr(g), _ptr(om), _stream(dev))
+    _lib.check(rc, "ema_coeffs_fwd")
+    return p, q, g, om
+
+
+def ema_coeffs_bwd(p_grad: torch.Tensor, q_grad: torch.Tensor, g_grad: torch.Tensor, om_grad: torch.Tensor,
+                   alpha: torch.Tensor, delta: torch.Tensor, third: torch.Tensor, gamma_like: torch.Tensor,
+                   omega_like: torch.Tensor, is_complex: bool):
+    """Backward of ema_coeffs_fwd: gradients of (p [K, N], q, gamma [K, N, 2] as (re, im) pairs -- [K, N] for the real
+    layer --, omega [D]) in fp32 -> gradients of (alpha, delta, third, gamma, omega) in the parameters' dtype and
+    shapes."""
+    dev = _need_gpu(p_grad, q_grad, g_grad, om_grad, alpha, delta, third)
+    lib = _lib.load()
+    K, N = alpha.shape[0], alpha.shape[1]
+    D = omega_like.numel()
+    a, d, t = (x.detach().contiguous() for x in (alpha, delta, third))
+    gs = [_f32c(x) for x in (p_grad, q_grad, g_grad, om_grad)]
+    pair = 2 if is_complex else 1
+    if gs[0].numel() != K * N or gs[1].numel() != pair * K * N or gs[2].numel() != pair * K * N or gs[3].numel() != D:
+        raise RuntimeError("ema_coeffs_bwd: gradient shapes do not belong to this layer")
+    outs = [torch.empty(x.shape, dtype=a.dtype, device=dev) for x in (alpha, delta, third, gamma_like, omega_like)]
+    with _on_device(dev):
+        rc = lib.mega_ema_coeffs_bwd(_ptr(gs[0]), _ptr(gs[1]), _ptr(gs[2]), _ptr(gs[3]), _ptr(a), _ptr(d), _ptr(t),
+                                     _dtype_code(a), 1 if is_complex else 0, K, N, D, _ptr(outs[0]), _ptr(outs[1]),
+                                     _ptr(outs[2]), _ptr(outs[3]), _ptr(outs[4]), _stream(dev))
+    _lib.check(rc, "ema_coeffs_bwd")
+    return tuple(outs)
+
+
+def norm_params_fwd(weight: torch.Tensor, bias: torch.Tensor, prior_mean: torch.Tensor, prior_logv: torch.Tensor,
+                    batch_size: int):
+    """What TimestepNorm.forward derives from its parameters on every call (timestep_norm.py:118-131), in one
+    launch: -> (weight + 1 [H], bias [H], prior mean [B, G], exp(prior log-variance) [B, G]) in fp32."""
+    dev = _need_gpu(weight, bias, prior_mean, prior_logv)
+    lib = _lib.load()
+    H, G, B = weight.numel(), prior_mean.numel(), int(batch_size)
+    w, b, pm, pl = (x.detach().contiguous() for x in (weight, bias, prior_mean, prior_logv))
+    if w.dtype != b.dtype or pm.dtype != pl.dtype or b.numel() != H or pl.numel() != G:
+        raise RuntimeError("norm_params_fwd: weight / bias and prior_mean / prior_logv must pair up")
+    gamma = torch.empty(H, dtype=torch.float32, device=dev)
+    beta = torch.empty(H, dtype=torch.float32, device=dev)
+    mean = torch.empty(B, G, dtype=torch.float32, device=dev)
+    var = torch.empty(B, G, dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_norm_params_fwd(_ptr(w), _ptr(b), _dtype_code(w), _ptr(pm), _ptr(pl), _dtype_code(pm), H, G, B,
+                                      _ptr(gamma), _ptr(beta), _ptr(mean), _ptr(var), _stream(dev))
+    _lib.check(rc, "norm_params_fwd")
+    return gamma, beta, mean, var
+
+
+def norm_params_bwd(gamma_grad: torch.Tensor, beta_grad: torch.Tensor, mean_grad: Optional[torch.Tensor],
+                    var_grad: Optional[torch.Tensor], weight: torch.Tensor, prior_mean: torch.Tensor,
+                    prior_logv: torch.Tensor, batch_size: int, prior_needs_grad: bool):
+    """Backward of norm_params_fwd -> (weight_grad, bias_grad, prior_mean_grad, prior_logv_grad) in the
+    parameters' dtypes; the prior's are None unless prior_needs_grad."""
+    dev = _need_gpu(gamma_grad, beta_grad, weight, prior_logv)
+    lib = _lib.load()
+    H, G, B = weight.numel(), prior_mean.numel(), int(batch_size)
+    gg, gb = _f32c(gamma_grad), _f32c(beta_grad)
+    dw = torch.empty(weight.shape, dtype=weight.dtype, device=dev)
+    db = torch.empty(weight.shape, dtype=weight.dtype, device=dev)
+    dpm = dpl = gm = gv = None
+    pl = prior_logv.detach().contiguous()
+    if prior_needs_grad:
+        gm = torch.zeros(B, G, dtype=torch.float32, device=dev) if mean_grad is None else _f32c(mean_grad)
+        gv = torch.zeros(B, G, dtype=torch.float32, device=dev) if var_grad is None else _f32c(var_grad)
+        dpm = torch.empty(prior_mean.shape, dtype=prior_mean.dtype, device=dev)
+        dpl = torch.empty(prior_mean.shape, dtype=prior_mean.dtype, device=dev)
+    with _on_device(dev):
+        rc = lib.mega_norm_params_bwd(_ptr(gg), _ptr(gb), _ptr(gm), _ptr(gv), _ptr(pl), _dtype_code(weight),
+                                      _dtype_code(pl), H, G, B, _ptr(dw), _ptr(db), _ptr(dpm), _ptr(dpl), _stream(dev))
+    _lib.check(rc, "norm_params_bwd")
+    return dw, db, dpm, dpl
+
+
 def ema_parameters_fwd(p: torch.Tensor, log_q: torch.Tensor, gamma: torch.Tensor,
                        h: Optional[torch.Tensor], L: int):
     """-> (w[K,L], b[B,K,L] or None, None).  Reference: ema_parameters_fwd,
@@ -1128,6 +1225,21 @@ def _rows(t: torch.Tensor):
     return t, t.stride(-2) if t.shape[-2] > 1 else max(t.stride(-2), t.shape[-1])
 
 
+def _grad_slot(out: Optional[torch.Tensor], like: torch.Tensor):
+    """(tensor to write a gradient of `like`'s shape into, its row stride): `out` when the caller hands over a
+    row-strided slice of a wider buffer (last axis contiguous, rows uniformly spaced, 16-byte aligned rows),
+    else a new contiguous tensor."""
+    if out is not None:
+        ok = out.shape == like.shape and out.dtype == like.dtype and out.device == like.device and out.dim() >= 2
+        ok = ok and (out.stride(-1) == 1) and (out.stride(-2) * out.element_size()) % 16 == 0 and out.data_ptr() % 16 == 0
+        for i in range(out.dim() - 2):
+            ok = ok and (out.shape[i] == 1 or out.stride(i) == out.stride(i + 1) * out.shape[i + 1])
+        if ok:
+            return out, out.stride(-2)
+    t = torch.empty(like.shape, dtype=like.dtype, device=like.device)
+    return t, like.shape[-1]
+
+
 def _ntok(t: torch.Tensor) -> int:
     return t.numel() // t.shape[-1] if t.shape[-1] else 0
 
@@ -1173,8 +1285,10 @@ def gate_qk_fwd(z: torch.Tensor, gamma: torch.Tensor, beta: torch.Tensor, freqs:
 
 
 def gate_qk_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tensor, gamma: torch.Tensor, freqs: torch.Tensor,
-                num_heads: int, chunk: int, pos0: int = 0, eps: float = 1e-5):
+                num_heads: int, chunk: int, pos0: int = 0, eps: float = 1e-5,
+                z_grad_out: Optional[torch.Tensor] = None):
     """Backward of gate_qk_fwd: -> (z_grad [..., S] in z's dtype, gamma_grad [2, S] fp32, beta_grad [2, S] fp32).
+    z_grad_out: a row-strided slice of a wider gradient buffer to write z_grad into (returned as z_grad).
     The autograd graph it replaces is normalize -> affine -> rotary
     (moving_average_gated_attention.py:324-328, relative_positional_bias.py:86-97)."""
     dev = _need_gpu(q_grad, k_grad, z)
@@ -1190,7 +1304,7 @@ def gate_qk_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tensor, gam
         raise RuntimeError("gate_qk_bwd: q_grad, k_grad must have z's shape")
     dq = q_grad.detach().to(z.dtype).contiguous()
     dk = k_grad.detach().to(z.dtype).contiguous()
-    dz = torch.empty(z.shape, dtype=z.dtype, device=dev)
+    dz, dzs = _grad_slot(z_grad_out, z)
     dgamma = torch.empty(2, S, dtype=torch.float32, device=dev)
     dbeta = torch.empty(2, S, dtype=torch.float32, device=dev)
     T = _ntok(z)
@@ -1198,9 +1312,9 @@ def gate_qk_bwd(q_grad: torch.Tensor, k_grad: torch.Tensor, z: torch.Tensor, gam
     with _on_device(dev):
         stream = _stream(dev)
         ws = _scratch_buffer(dev, nws, stream)
-        rc = lib.mega_gate_qk_bwd(_ptr(dq), _ptr(dk), _ptr(zr), zs, _ptr(g), _ptr(f), _ptr(dz), _ptr(dgamma),
-                                  _ptr(dbeta), _dtype_code(zr), T, S, num_heads, int(chunk), int(pos0), float(eps),
-                                  _ptr(ws), ws.numel(), stream)
+        rc = lib.mega_gate_qk_bwd_strided(_ptr(dq), _ptr(dk), _ptr(zr), zs, _ptr(g), _ptr(f), _ptr(dz), dzs,
+                                          _ptr(dgamma), _ptr(dbeta), _dtype_code(zr), T, S, num_heads, int(chunk),
+                                          int(pos0), float(eps), _ptr(ws), ws.numel(), stream)
     _lib.check(rc, "gate_qk_bwd")
     return dz, dgamma, dbeta
 
@@ -1305,24 +1419,26 @@ def ema_backward(y_grad: torch.Tensor, x: torch.Tensor, p: torch.Tensor, q: torc
     return dx, dp, dq[..., 0], dg[..., 0], dom
 
 
-def gate_mul_bwd(y_grad: torch.Tensor, a: torch.Tensor, r: torch.Tensor):
-    """Backward of gate_mul_fwd: -> (a_grad, r_grad)."""
+def gate_mul_bwd(y_grad: torch.Tensor, a: torch.Tensor, r: torch.Tensor, r_grad_out: Optional[torch.Tensor] = None):
+    """Backward of gate_mul_fwd: -> (a_grad, r_grad); r_grad_out: a row-strided slice to write r_grad into."""
     dev = _need_gpu(y_grad, a, r)
     lib = _lib.load()
     ar, as_ = _rows(a)
     rr, rs = _rows(r)
     g = y_grad.detach().to(a.dtype).contiguous()
     da = torch.empty(a.shape, dtype=a.dtype, device=dev)
-    dr = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    dr, drs = _grad_slot(r_grad_out, a)
     with _on_device(dev):
-        rc = lib.mega_gate_mul_bwd(_ptr(g), _ptr(ar), as_, _ptr(rr), rs, _ptr(da), _ptr(dr), _dtype_code(ar),
-                                   _ntok(a), a.shape[-1], _stream(dev))
+        rc = lib.mega_gate_mul_bwd_strided(_ptr(g), _ptr(ar), as_, _ptr(rr), rs, _ptr(da), _ptr(dr), drs,
+                                           _dtype_code(ar), _ntok(a), a.shape[-1], _stream(dev))
     _lib.check(rc, "gate_mul_bwd")
     return da, dr
 
 
-def gate_out_bwd(y_grad: torch.Tensor, residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: torch.Tensor):
-    """Backward of gate_out_fwd: -> (residual_grad, u_grad, h_grad); h_grad is the gradient of hx and of hp."""
+def gate_out_bwd(y_grad: torch.Tensor, residual: torch.Tensor, u: torch.Tensor, hx: torch.Tensor, hp: torch.Tensor,
+                 u_grad_out: Optional[torch.Tensor] = None, h_grad_out: Optional[torch.Tensor] = None):
+    """Backward of gate_out_fwd: -> (residual_grad, u_grad, h_grad); h_grad is the gradient of hx and of hp.
+    u_grad_out, h_grad_out: row-strided slices to write those two into."""
     dev = _need_gpu(y_grad, residual, u, hx, hp)
     lib = _lib.load()
     r0, rs = _rows(residual)
@@ -1330,13 +1446,15 @@ def gate_out_bwd(y_grad: torch.Tensor, residual: torch.Tensor, u: torch.Tensor, 
     x0, xs = _rows(hx)
     p0, ps = _rows(hp)
     g = y_grad.detach().to(residual.dtype).contiguous()
-    outs = [torch.empty(residual.shape, dtype=residual.dtype, device=dev) for _ in range(3)]
+    dres = torch.empty(residual.shape, dtype=residual.dtype, device=dev)
+    du, dus = _grad_slot(u_grad_out, residual)
+    dh, dhs = _grad_slot(h_grad_out, residual)
     with _on_device(dev):
-        rc = lib.mega_gate_out_bwd(_ptr(g), _ptr(r0), rs, _ptr(u0), us, _ptr(x0), xs, _ptr(p0), ps, _ptr(outs[0]),
-                                   _ptr(outs[1]), _ptr(outs[2]), _dtype_code(r0), _ntok(residual), residual.shape[-1],
-                                   _stream(dev))
+        rc = lib.mega_gate_out_bwd_strided(_ptr(g), _ptr(r0), rs, _ptr(u0), us, _ptr(x0), xs, _ptr(p0), ps, _ptr(dres),
+                                           _ptr(du), dus, _ptr(dh), dhs, _dtype_code(r0), _ntok(residual),
+                                           residual.shape[-1], _stream(dev))
     _lib.check(rc, "gate_out_bwd")
-    return tuple(outs)
+    return dres, du, dh
 
 
 def swiglu_bwd(y_grad: torch.Tensor, a: torch.Tensor, b: torch.Tensor):

@@ -295,6 +295,41 @@ int mega_ema_param_grad(const void* dy, const void* x, int dtype, int64_t sgb, i
                         size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------ */
+/* Parameter formulas in front of the kernels, one launch each way                            */
+/* mega_ema_coeffs_fwd / _bwd: the coefficients of the moving average from the stored parameters, in the
+ * reference a chain of torch operations per call (complex layer:
+ * fairseq/modules/complex_exponential_moving_average.py:79-96, p = sigmoid(alpha),
+ * q = (1 - sigmoid(alpha) sigmoid(delta)) exp(i (n + 1) sigmoid(theta) 2 pi / N), gamma complex times sqrt(1 / N);
+ * real layer: exponential_moving_average.py:71-80, p = sigmoid(alpha) beta, q = 1 - sigmoid(alpha) sigmoid(delta),
+ * gamma times sqrt(1 / N)).  alpha, delta [K, N]; theta [K] (complex) or beta [K, N] (real); gamma [K, N, 2]
+ * (complex) or [K, N] (real); omega [D]; all of `dtype` (the parameters' storage type), K = D or 2 D.
+ * Results in the layout every other entry point takes: p [K, N], q, gamma_out [K, N, 2], omega_out [D], fp32.
+ * The backward takes the gradients of those four (fp32; for the complex layer q_grad, gamma_out_grad [K, N, 2] as
+ * (d/dRe, d/dIm) pairs, which is torch's convention for a real loss; for the real layer [K, N]) and writes the
+ * parameters' gradients in `dtype`.                                                                       */
+int mega_ema_coeffs_fwd(const void* alpha, const void* delta, const void* theta_or_beta,
+                        const void* gamma, const void* omega, int dtype, int is_complex, int64_t K,
+                        int64_t N, int64_t D, float* p, float* q, float* gamma_out, float* omega_out,
+                        void* stream);
+int mega_ema_coeffs_bwd(const float* p_grad, const float* q_grad, const float* gamma_out_grad,
+                        const float* omega_out_grad, const void* alpha, const void* delta,
+                        const void* theta_or_beta, int dtype, int is_complex, int64_t K, int64_t N,
+                        int64_t D, void* alpha_grad, void* delta_grad, void* theta_or_beta_grad,
+                        void* gamma_grad, void* omega_grad, void* stream);
+/* mega_norm_params_fwd / _bwd: the operands TimestepNorm.forward derives from its parameters on every call
+ * (fairseq/modules/norm_layer/timestep_norm.py:118-131): gamma = weight + 1, beta = bias [H] fp32, and the
+ * prior expanded over the batch, prev_mean = prior_mean, prev_var = exp(prior_logv) [B, G] fp32.  weight, bias
+ * of `dtype`, prior_mean, prior_logv [G] of `prior_dtype`.  The backward writes the four parameter gradients in
+ * their storage types (the prior's are sums over the batch; both NULL when the prior is a buffer).       */
+int mega_norm_params_fwd(const void* weight, const void* bias, int dtype, const void* prior_mean,
+                         const void* prior_logv, int prior_dtype, int64_t H, int64_t G, int64_t B,
+                         float* gamma, float* beta, float* prev_mean, float* prev_var, void* stream);
+int mega_norm_params_bwd(const float* gamma_grad, const float* beta_grad, const float* prev_mean_grad,
+                         const float* prev_var_grad, const void* prior_logv, int dtype,
+                         int prior_dtype, int64_t H, int64_t G, int64_t B, void* weight_grad,
+                         void* bias_grad, void* prior_mean_grad, void* prior_logv_grad, void* stream);
+
+/* ------------------------------------------------------------------------ */
 /* Long convolution with an explicit time-domain kernel                      */
 /* stands in for fftconv(x, k) (fairseq/modules/fused_ops/fftconv.py:11-27, 45-61;
  * fused CUDA op fftconv_fwd, ops/fftconv_kernel.cu:431-470) and
@@ -560,6 +595,24 @@ int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual
                       void* h_grad, int dtype, int64_t T, int64_t D, void* stream);
 int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_grad, void* b_grad,
                     int dtype, int64_t n, void* stream);
+/* The same three with row strides (in elements) on the gradients of u, z, r, hx: these four are slices of
+ * the mx_proj output (torch.split, moving_average_gated_attention.py:319), whose backward in the reference is
+ * a concatenation of the four gradients; a caller that owns one [T, D + S + E + D] gradient buffer lets each
+ * kernel write its slice in place (row stride = the buffer's width) and skips that copy.  h_grad is read by
+ * the output projection's backward as well: a row-strided matrix operand.                               */
+int mega_gate_qk_bwd_strided(const void* q_grad, const void* k_grad, const void* z, int64_t z_stride,
+                             const float* gamma, const float* freqs, void* z_grad,
+                             int64_t z_grad_stride, float* gamma_grad, float* beta_grad, int dtype,
+                             int64_t T, int64_t S, int64_t heads, int64_t chunk, int64_t pos0,
+                             double eps, void* workspace, size_t workspace_bytes, void* stream);
+int mega_gate_mul_bwd_strided(const void* y_grad, const void* a, int64_t a_stride, const void* r,
+                              int64_t r_stride, void* a_grad, void* r_grad, int64_t r_grad_stride,
+                              int dtype, int64_t T, int64_t E, void* stream);
+int mega_gate_out_bwd_strided(const void* y_grad, const void* residual, int64_t residual_stride,
+                              const void* u, int64_t u_stride, const void* hx, int64_t hx_stride,
+                              const void* hp, int64_t hp_stride, void* residual_grad, void* u_grad,
+                              int64_t u_grad_stride, void* h_grad, int64_t h_grad_stride, int dtype,
+                              int64_t T, int64_t D, void* stream);
 
 #ifdef __cplusplus
 }

@@ -165,6 +165,82 @@ def test_norm_then_move_trains_as_one_operator(dtype, B, L, D, G, N, masked, lay
     assert rel_err(host(out[6]), ocm) < 1e-4 and rel_err(host(out[7]), ocr) < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("cplx,K,N,D", [(True, 24, 16, 24), (True, 10, 3, 5), (False, 12, 4, 12), (False, 8, 2, 4)])
+def test_coefficient_kernels(dtype, cplx, K, N, D):
+    """The layer's coefficients from its parameters in one launch, forwards against the fp64 oracle's formulas and
+    backwards against torch's autograd of the same formulas in fp64 on the CPU (random upstream gradients)."""
+    rng = np.random.default_rng(77)
+    alpha, a64 = rounded(rng.normal(0, 0.4, (K, N, 1)), dtype)
+    delta, d64 = rounded(rng.normal(0, 0.4, (K, N, 1)), dtype)
+    omega, o64 = rounded(rng.normal(size=(D, 1) if cplx else (D,)), dtype)
+    if cplx:
+        third, t64 = rounded(rng.normal(0, 1.5, (K, 1, 1)), dtype)
+        gamma, g64 = rounded(rng.normal(size=(K, N, 2)), dtype)
+        po, qo, go = O.ema_coeffs_complex(a64, d64, t64, g64)
+    else:
+        third, t64 = rounded(rng.normal(0, 1.0, (K, N, 1)), dtype)
+        gamma, g64 = rounded(rng.normal(size=(K, N)), dtype)
+        po, qo, go = O.ema_coeffs_real(a64, d64, t64, g64)
+    p, q2, g2, om = M.ops.ema_coeffs_fwd(alpha, delta, third, gamma, omega, cplx)
+    assert p.dtype == q2.dtype == g2.dtype == om.dtype == torch.float32
+    assert rel_err(host(p), po.reshape(K, N)) < 2e-6
+    qo, go = np.asarray(qo, np.complex128).reshape(K, N), np.asarray(go, np.complex128).reshape(K, N)
+    assert rel_err(host(q2), np.stack([qo.real, qo.imag], -1)) < 2e-6
+    assert rel_err(host(g2), np.stack([go.real, go.imag], -1)) < 2e-6
+    assert np.array_equal(host(om), o64.reshape(-1))
+    # backward: arbiter = autograd of the formulas in fp64
+    ta, td, tt, tg = (torch.from_numpy(v).requires_grad_(True) for v in (a64, d64, t64, g64))
+    sa, sd = torch.sigmoid(ta), torch.sigmoid(td)
+    up = [rng.normal(size=(K, N)), rng.normal(size=(K, N, 2)), rng.normal(size=(K, N, 2)), rng.normal(size=D)]
+    up = [u.astype(np.float32).astype(np.float64) for u in up]
+    if cplx:
+        ang = torch.arange(1, N + 1, dtype=torch.float64).view(1, N, 1) * torch.sigmoid(tt) * (2 * np.pi / N)
+        r = 1 - sa * sd
+        qre, qim = (r * torch.cos(ang)).squeeze(-1), (r * torch.sin(ang)).squeeze(-1)
+        gs = tg / np.sqrt(N)
+        loss = (sa.squeeze(-1) * torch.from_numpy(up[0])).sum() + (qre * torch.from_numpy(up[1][..., 0])).sum() + \
+            (qim * torch.from_numpy(up[1][..., 1])).sum() + (gs * torch.from_numpy(up[2])).sum()
+        gq, gg = dev(up[1]), dev(up[2])
+    else:
+        loss = ((sa * tt).squeeze(-1) * torch.from_numpy(up[0])).sum() + \
+            ((1 - sa * sd).squeeze(-1) * torch.from_numpy(up[1][..., 0])).sum() + \
+            (tg / np.sqrt(N) * torch.from_numpy(up[2][..., 0])).sum()
+        gq, gg = dev(up[1][..., 0].copy()), dev(up[2][..., 0].copy())
+    loss.backward()
+    da, dd, dt, dg, dom = M.ops.ema_coeffs_bwd(dev(up[0]), gq, gg, dev(up[3]), alpha, delta, third, gamma, omega, cplx)
+    assert da.dtype == dd.dtype == dt.dtype == dg.dtype == dom.dtype == dtype
+    assert da.shape == alpha.shape and dt.shape == third.shape and dg.shape == gamma.shape and dom.shape == omega.shape
+    tol = TOL[dtype] if dtype != torch.float32 else 1e-5
+    for got, ref in ((da, ta.grad), (dd, td.grad), (dt, tt.grad), (dg, tg.grad)):
+        assert rel_err(host(got), ref.numpy()) < tol
+    assert rel_err(host(dom).reshape(-1), up[3]) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,B,learned", [(64, 4, 3, True), (40, 40, 2, True), (32, 8, 1, False)])
+def test_norm_parameter_kernels(dtype, H, G, B, learned):
+    """weight + 1, bias, the prior over the batch: values, and parameter gradients with the sums over the batch."""
+    rng = np.random.default_rng(78)
+    w, w64 = rounded(rng.normal(0, 0.3, H), dtype)
+    b, b64 = rounded(rng.normal(0, 0.3, H), dtype)
+    pm, pm64 = rounded(rng.normal(0, 0.3, G), dtype)
+    pl, pl64 = rounded(rng.normal(0, 0.3, G), dtype)
+    gamma, beta, mean, var = M.ops.norm_params_fwd(w, b, pm, pl, B)
+    assert np.allclose(host(gamma), w64 + 1, rtol=1e-6, atol=0) and np.array_equal(host(beta), b64)
+    assert np.array_equal(host(mean), np.broadcast_to(pm64, (B, G)))
+    assert rel_err(host(var), np.broadcast_to(np.exp(pl64), (B, G))) < 1e-6
+    up = [rng.normal(size=s).astype(np.float32).astype(np.float64) for s in ((H,), (H,), (B, G), (B, G))]
+    dw, db, dpm, dpl = M.ops.norm_params_bwd(dev(up[0]), dev(up[1]), dev(up[2]), dev(up[3]), w, pm, pl, B, learned)
+    tol = 1e-6 if dtype == torch.float32 else TOL[dtype]
+    assert dw.dtype == dtype and rel_err(host(dw), up[0]) < tol and rel_err(host(db), up[1]) < tol
+    if learned:
+        assert rel_err(host(dpm), up[2].sum(0)) < tol
+        assert rel_err(host(dpl), up[3].sum(0) * np.exp(pl64)) < tol
+    else:
+        assert dpm is None and dpl is None
+
+
 # ----------------------------------------------------------------------------------------------
 # moving-average layer
 # ----------------------------------------------------------------------------------------------
@@ -531,7 +607,10 @@ def test_gated_attention_layer_trains(heads, act, moving, bidir):
         w64 = w64 * (~mask)[..., None]         # padded positions carry no loss
     x = dev(x64).requires_grad_(True)
     out, _ = layer(x, None if mask is None else torch.from_numpy(mask).to(DEV))
+    in_place = M.modules.SplitGrads.taken
     (out * dev(w64)).sum().backward()
+    # the gradients of the four slices of the mx_proj output were written into one buffer (no concatenation)
+    assert M.modules.SplitGrads.taken == in_place + 1
     P = _params(layer)
     okw = dict(chunk=C, num_heads=heads, moving_act=act, num_groups=4, bidirectional=bool(bidir), padding_mask=mask)
     loss = lambda Pd, xx: (O.gated_attention_layer(xx, Pd, **okw) * w64).sum()
@@ -669,6 +748,18 @@ def test_gate_backwards(dtype, shape, width, off):
     assert rel_err(host(dres), dy64 * (1 - s)) < TOL[dtype]
     assert rel_err(host(du), dy64 * (O._silu(aa) - res64) * s * (1 - s)) < TOL[dtype]
     assert rel_err(host(dh), dy64 * s * dsilu(aa)) < TOL[dtype]
+    # the same gradients written into slices of one wider buffer (row stride = its width): the values next to
+    # the slices stay as they were
+    W = 3 * shape[-1] + 8
+    buf = torch.full(shape[:-1] + (W,), 7.0, dtype=dtype, device=DEV)
+    s0, s1, s2 = buf.narrow(-1, 0, shape[-1]), buf.narrow(-1, shape[-1] + 8, shape[-1]), buf.narrow(-1, 2 * shape[-1] + 8, shape[-1])
+    _, dr2 = M.ops.gate_mul_bwd(dy, a, r, r_grad_out=s0)
+    _, du2, dh2 = M.ops.gate_out_bwd(dy, res, u, hx, hp, u_grad_out=s1, h_grad_out=s2)
+    torch.cuda.synchronize()
+    if (shape[-1] * dy.element_size()) % 16 == 0:
+        assert dr2.data_ptr() == s0.data_ptr() and du2.data_ptr() == s1.data_ptr() and dh2.data_ptr() == s2.data_ptr()
+        assert bool((buf.narrow(-1, shape[-1], 8) == 7.0).all())
+    assert torch.equal(dr2, dr) and torch.equal(du2, du) and torch.equal(dh2, dh)
     b, b64 = rounded(rng.normal(size=shape), dtype)
     ga, gb = M.ops.swiglu_bwd(dy, a, b)
     assert rel_err(host(ga), dy64 * b64 * dsilu(a64)) < TOL[dtype]
@@ -697,6 +788,13 @@ def test_gate_qk_bwd(dtype, B, L, S, heads, chunk, width, off):
     dq, dq64 = rounded(up[0], dtype)
     dk, dk64 = rounded(up[1], dtype)
     dz, dg, db = M.ops.gate_qk_bwd(dq, dk, z, dev(g), dev(freqs), heads, chunk)
+    # the same gradient written into a slice of a wider buffer
+    wide = torch.full((B, L, S + 24), 3.0, dtype=dtype, device=DEV)
+    dz2, dg2, db2 = M.ops.gate_qk_bwd(dq, dk, z, dev(g), dev(freqs), heads, chunk, z_grad_out=wide.narrow(-1, 16, S))
+    torch.cuda.synchronize()
+    assert dz2.data_ptr() == wide.narrow(-1, 16, S).data_ptr() and torch.equal(dz2, dz)
+    assert torch.equal(dg2, dg) and torch.equal(db2, db)
+    assert bool((wide[..., :16] == 3.0).all()) and bool((wide[..., 16 + S:] == 3.0).all())
     # arbiter
     tz = torch.from_numpy(z64).requires_grad_(True)
     tg = torch.from_numpy(g).requires_grad_(True)
