@@ -103,10 +103,12 @@ __device__ __forceinline__ uint4 kmajor_frag(const char* base, int rowbytes, int
 // AT / BT: the operand is stored K-major, [K][M] with pitch lda / [K][N] with pitch ldb (C = A^T-stored ... : the
 // product reduces over the operand's rows), and is read in place: its tile goes to LDS as it lies in memory and the
 // fragments come out of transposing LDS reads.  M (N) must be a multiple of 8 then.
-template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0>
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0, int FM = 4,
+          int FN = FM>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G) {
   static_assert(EPI == 0 || sizeof(TOut) == 4, "the softmax-backward epilogue stages fp32");
-  constexpr int TM = 64 * WM, TN = 64 * WN, NT = 64 * WM * WN;
+  constexpr int WTM = 16 * FM, WTN = 16 * FN;                     // a wave's block of the output tile
+  constexpr int TM = WTM * WM, TN = WTN * WN, NT = 64 * WM * WN;
   constexpr int NLA = TM * KP / NT, NLB = TN * KP / NT;          // 16-byte pieces per thread and K step
   static_assert(TM * KP % NT == 0 && TN * KP % NT == 0, "tile rows must divide over the threads");
   extern __shared__ __attribute__((aligned(16))) char lds[];     // 2 x (TM + TN) x PITCH
@@ -215,12 +217,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
       }
     }
   };
-  f32x4 acc[4][4];
+  f32x4 acc[FM][FN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int wm = (wave / WN) * 64, wn = (wave % WN) * 64;
+    for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int wm = (wave / WN) * WTM, wn = (wave % WN) * WTN;
   const int fr = lane & 15;                                       // fragment row; lane >> 4 is its 16-byte k block
   // the lane's part of a K-major fragment address: row 8 g + (n >> 2) of the 32-row block, 8-byte column n & 3
   const int ksr = fr >> 2, kvsw = ksr + 4 * ((lane >> 4) & 1);
@@ -242,9 +244,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     const char* lb = la + TM * PITCH;
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
-      uint4 fa[4];
+      uint4 fa[FM];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < FM; ++i) {
         if (AT)
           fa[i] = kmajor_frag(la + kk * 32 * (TM * 2) + klane_a, TM * 2, (wm >> 4) + i, kvsw);
         else
@@ -253,14 +255,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
       // the B fragments one column block at a time (four at once do not fit the 128 registers of a 16-wave
       // workgroup next to the K-major address arithmetic)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < FN; ++j) {
         uint4 fb;
         if (BT)
           fb = kmajor_frag(lb + kk * 32 * (TN * 2) + klane_b, TN * 2, (wn >> 4) + j, kvsw);
         else
           fb = *(const uint4*)(lb + (wn + j * 16 + fr) * PITCH + lds_piece(wn + j * 16 + fr, kk * 4 + (lane >> 4)) * 16);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i][j] = mfma16<TIn>(fa[i], fb, acc[i][j]);
+        for (int i = 0; i < FM; ++i) acc[i][j] = mfma16<TIn>(fa[i], fb, acc[i][j]);
         // K-major forms: keep the compiler from fetching all four B fragments ahead (that spills in the loop)
         if ((AT || BT) && WM * WN == 16 && (j & 1)) __builtin_amdgcn_sched_barrier(0);
       }
@@ -292,13 +294,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
 #pragma unroll
       for (int h = 0; h < NH; ++h) {
         if (h > 0) __syncthreads();
-        if (wm / HR == h) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < FM; ++i) {
+          if ((wm + i * 16) / HR != h) continue;                 // this block of rows belongs to another slice
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+          for (int j = 0; j < FN; ++j)
 #pragma unroll
-              for (int u = 0; u < 4; ++u) Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = acc[i][j][u];
+            for (int u = 0; u < 4; ++u) Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = acc[i][j][u];
         }
         __syncthreads();
         constexpr int PPR = TN / 4;
@@ -323,9 +325,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
       return;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < FN; ++j) {
         const int n = n0 + wn + j * 16 + cn;
         if (n >= G.N) continue;
 #pragma unroll
@@ -340,19 +342,19 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
   }
   const bool wide = NH > 0 && (G.ldc % VW) == 0 && (((uintptr_t)C) % 16) == 0 && n0 + TN <= G.N;
   if (NH > 0 && wide) {
-    constexpr int HR = TM / (NH > 0 ? NH : 1);                   // rows per slice (a multiple of a wave's 64)
+    constexpr int HR = TM / (NH > 0 ? NH : 1);                   // rows per slice (a multiple of 16)
     TOut* Cs = (TOut*)lds;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
       if (h > 0) __syncthreads();                                // the previous slice has left
-      if (wm / HR == h) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < FM; ++i) {
+        if ((wm + i * 16) / HR != h) continue;                   // this block of rows belongs to another slice
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-              Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
+          for (int u = 0; u < 4; ++u)
+            Cs[(wm - h * HR + i * 16 + cr + u) * CP + wn + j * 16 + cn] = from_float<TOut>(acc[i][j][u] * G.alpha);
       }
       __syncthreads();
       constexpr int PPR = TN / VW;                               // pieces per row
@@ -367,9 +369,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < FN; ++j) {
       const int n = n0 + wn + j * 16 + cn;
       if (n >= G.N) continue;
 #pragma unroll
@@ -380,11 +382,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_nt_kernel(const GemmArgs G)
     }
 }
 
-template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0>
+template <typename TIn, typename TOut, int WM, int WN, bool AT = false, bool BT = false, int EPI = 0, int FM = 4,
+          int FN = FM>
 void launch_gemm(GemmArgs G, int64_t M, int64_t N, int64_t batches, bool xcd, hipStream_t s) {
-  constexpr int TM = 64 * WM, TN = 64 * WN;
+  constexpr int TM = 16 * FM * WM, TN = 16 * FN * WN;
   constexpr int smem = 2 * (TM + TN) * PITCH;
-  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT, EPI>;
+  auto kern = gemm_nt_kernel<TIn, TOut, WM, WN, AT, BT, EPI, FM, FN>;
   static uint64_t attr_seen = 0;
   if (smem > 64 * 1024 && first_on_device(&attr_seen)) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -1280,14 +1283,14 @@ int run_attention_bwd(const void* dy, const void* q, const void* k, const void* 
     G.lda = L; G.ldb = Nh * H2; G.ldc = Nh * H2;
     G.sa = Nh * L * L; G.sai = L * L; G.sb = L * Nh * H2; G.sbi = H2; G.sc = L * Nh * H2; G.sci = H2;
     G.M = (int)L; G.N = (int)H2; G.K = (int)L; G.alpha = 1.0f; G.causal = causal ? 3 : 0;
-    if (L >= 256 && H2 >= 256) launch_gemm<T, T, 4, 4, true, true>(G, L, H2, BN_, xcd, s);
+    if (L >= 256 && H2 >= 256) launch_gemm<T, T, 2, 4, true, true, 0, 8, 4>(G, L, H2, BN_, xcd, s);
     else launch_gemm<T, T, 2, 2, true, true>(G, L, H2, BN_, xcd, s);
     // dq[b,:,n,:] = dS[b,n] k[b,:,n,:] (attention_kernel.cu:205-222): k K-major
     G.A = dS; G.Bm = k; G.C = dq;
     G.lda = Lp; G.ldb = Nh * H1; G.ldc = Nh * H1;
     G.sa = Nh * L * Lp; G.sai = L * Lp; G.sb = L * Nh * H1; G.sbi = H1; G.sc = L * Nh * H1; G.sci = H1;
     G.N = (int)H1; G.causal = causal ? 2 : 0;
-    launch_gemm<T, T, 2, 2, false, true>(G, L, H1, BN_, xcd, s);
+    launch_gemm<T, T, 2, 2, false, true, 0, 2, 4>(G, L, H1, BN_, xcd, s);
     // dk[b,:,n,:] = dS[b,n]^T q[b,:,n,:] (attention_kernel.cu:224-241): both operands K-major
     G.Bm = q; G.C = dk;
     G.causal = causal ? 3 : 0;
