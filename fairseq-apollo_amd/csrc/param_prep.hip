@@ -74,40 +74,66 @@ __global__ __launch_bounds__(256) void ema_coeffs_fwd_kernel(const CoeffArgs A) 
   }
 }
 
-// one thread per row: the gradient of theta is a sum over the row's states
-__global__ __launch_bounds__(256) void ema_coeffs_bwd_kernel(const CoeffArgs A) {
-  const int k = (int)blockIdx.x * 256 + (int)threadIdx.x;
-  if (k < A.D) st(A.domega, A.dtype, k, A.dom[k]);
-  if (k >= A.K) return;
-  float tsum = 0.f, st0 = 0.f;
-  if (A.is_complex) st0 = sigm(ld(A.third, A.dtype, k));
-  for (int n = 0; n < A.N; ++n) {
-    const int64_t i = (int64_t)k * A.N + n;
-    const float a = sigm(ld(A.alpha, A.dtype, i)), d = sigm(ld(A.delta, A.dtype, i));
-    float da, dr;
-    if (A.is_complex) {
-      const float r = 1.0f - a * d;
-      const float ang = (float)(n + 1) * (st0 * A.turn);
-      float sn, cs;
-      sincosf(ang, &sn, &cs);
-      const float gr = A.dq[2 * i], gi = A.dq[2 * i + 1];      // dL/dRe q, dL/dIm q
-      dr = gr * cs + gi * sn;
-      tsum = fmaf((float)(n + 1), r * (gi * cs - gr * sn), tsum);
-      da = A.dp[i];
-      st(A.dgamma, A.dtype, 2 * i, A.dg[2 * i] * A.scale);
-      st(A.dgamma, A.dtype, 2 * i + 1, A.dg[2 * i + 1] * A.scale);
-    } else {
-      const float b = ld(A.third, A.dtype, i);
-      dr = A.dq[i];                                            // real layer: [K, N] gradients, no pairs
-      da = A.dp[i] * b;
-      st(A.dthird, A.dtype, i, A.dp[i] * a);
-      st(A.dgamma, A.dtype, i, A.dg[i] * A.scale);
-    }
-    // r = 1 - a d
-    st(A.dalpha, A.dtype, i, (da - dr * d) * a * (1.0f - a));
-    st(A.ddelta, A.dtype, i, -dr * a * d * (1.0f - d));
+// one lane per (row, state), 64 / N rows per wave (N <= 64): the gradient of theta, a sum over the row's states, is
+// collected from the row's lanes.  Rows of more than 64 states: one lane per row walking its states (rpw = 0).
+__global__ __launch_bounds__(256) void ema_coeffs_bwd_kernel(const CoeffArgs A, const int rpw) {
+  const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
+  const int gid = (int)blockIdx.x * 256 + (int)threadIdx.x;
+  if (gid < A.D) st(A.domega, A.dtype, gid, A.dom[gid]);
+  int k, n0, n1;
+  bool live;
+  if (rpw > 0) {
+    const int r = lane / A.N;
+    k = ((int)blockIdx.x * 4 + wave) * rpw + r;
+    n0 = lane - r * A.N;
+    n1 = n0 + 1;
+    live = r < rpw && k < A.K;
+  } else {
+    k = gid;
+    n0 = 0;
+    n1 = A.N;
+    live = k < A.K;
   }
-  if (A.is_complex) st(A.dthird, A.dtype, k, tsum * A.turn * st0 * (1.0f - st0));
+  float tsum = 0.f, st0 = 0.f;
+  if (live) {
+    if (A.is_complex) st0 = sigm(ld(A.third, A.dtype, k));
+    for (int n = n0; n < n1; ++n) {
+      const int64_t i = (int64_t)k * A.N + n;
+      const float a = sigm(ld(A.alpha, A.dtype, i)), d = sigm(ld(A.delta, A.dtype, i));
+      float da, dr;
+      if (A.is_complex) {
+        const float r = 1.0f - a * d;
+        const float ang = (float)(n + 1) * (st0 * A.turn);
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        const float gr = A.dq[2 * i], gi = A.dq[2 * i + 1];      // dL/dRe q, dL/dIm q
+        dr = gr * cs + gi * sn;
+        tsum = fmaf((float)(n + 1), r * (gi * cs - gr * sn), tsum);
+        da = A.dp[i];
+        st(A.dgamma, A.dtype, 2 * i, A.dg[2 * i] * A.scale);
+        st(A.dgamma, A.dtype, 2 * i + 1, A.dg[2 * i + 1] * A.scale);
+      } else {
+        const float b = ld(A.third, A.dtype, i);
+        dr = A.dq[i];                                            // real layer: [K, N] gradients, no pairs
+        da = A.dp[i] * b;
+        st(A.dthird, A.dtype, i, A.dp[i] * a);
+        st(A.dgamma, A.dtype, i, A.dg[i] * A.scale);
+      }
+      // r = 1 - a d
+      st(A.dalpha, A.dtype, i, (da - dr * d) * a * (1.0f - a));
+      st(A.ddelta, A.dtype, i, -dr * a * d * (1.0f - d));
+    }
+  }
+  if (!A.is_complex) return;
+  if (rpw > 0) {
+    // the row's states in order, the same sum every run: lane n0 = 0 of the row adds the others' terms
+    const int base = lane - n0;
+    float total = 0.f;
+    for (int j = 0; j < A.N; ++j) total += __shfl(tsum, base + j, 64);
+    tsum = total;
+    live = live && n0 == 0;
+  }
+  if (live) st(A.dthird, A.dtype, k, tsum * A.turn * st0 * (1.0f - st0));
 }
 
 struct NormParamArgs {
@@ -204,7 +230,10 @@ extern "C" int mega_ema_coeffs_bwd(const float* p_grad, const float* q_grad, con
   A.dp = p_grad; A.dq = q_grad; A.dg = gamma_out_grad; A.dom = omega_out_grad;
   A.dalpha = alpha_grad; A.ddelta = delta_grad; A.dthird = theta_or_beta_grad; A.dgamma = gamma_grad;
   A.domega = omega_grad;
-  hipLaunchKernelGGL(ema_coeffs_bwd_kernel, dim3((unsigned)ceil_div(K, 256)), dim3(256), 0, (hipStream_t)stream, A);
+  const int rpw = N <= 64 ? (int)(64 / N) : 0;                   // rows per wave, one lane per (row, state)
+  int64_t blocks = rpw > 0 ? ceil_div(K, 4 * rpw) : ceil_div(K, 256);
+  if (blocks * 256 < D) blocks = ceil_div(D, 256);               // the first D threads also copy omega's gradient
+  hipLaunchKernelGGL(ema_coeffs_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, A, rpw);
   MEGA_CHECK_LAUNCH("ema_coeffs_bwd");
   return MEGA_OK;
 }

@@ -166,7 +166,8 @@ def test_norm_then_move_trains_as_one_operator(dtype, B, L, D, G, N, masked, lay
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("cplx,K,N,D", [(True, 24, 16, 24), (True, 10, 3, 5), (False, 12, 4, 12), (False, 8, 2, 4)])
+@pytest.mark.parametrize("cplx,K,N,D", [(True, 24, 16, 24), (True, 10, 3, 5), (True, 6, 80, 6), (True, 2048, 16, 2048),
+                                         (False, 12, 4, 12), (False, 8, 2, 4)])
 def test_coefficient_kernels(dtype, cplx, K, N, D):
     """The layer's coefficients from its parameters in one launch, forwards against the fp64 oracle's formulas and
     backwards against torch's autograd of the same formulas in fp64 on the CPU (random upstream gradients)."""
