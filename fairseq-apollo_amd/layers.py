@@ -115,7 +115,8 @@ class NormalizedFeedForwardNetwork(nn.Module):
         if self.layerscale_weight is not None:
             nn.init.constant_(self.layerscale_weight, self.layer_scale)
 
-    def forward(self, x: Tensor) -> Tensor:
+    def forward(self, x: Tensor, consume_input: bool = False) -> Tensor:
+        """consume_input: the caller owns x and does not use it again (the residual sum may be formed in it)."""
         # hidden dropout acts whenever the module is in training mode, with or without a graph
         # (normalized_feedforward_network.py:81-83)
         if _training_call(self, x) or (self.training and self.hidden_dropout_p > 0):
@@ -123,7 +124,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
         else:
             h = ops.silu(self.fc1(self.norm(x)), inplace=True)
         if self.layerscale_weight is None and not (self.training and self.dropout_p > 0):
-            return linear_residual(self.fc2, h, x)      # the residual rides in the product
+            return linear_residual(self.fc2, h, x, consume_input)      # the residual rides in the product
         h = F.dropout(self.fc2(h), self.dropout_p, self.training)
         if self.layerscale_weight is not None:
             h = h * self.layerscale_weight
@@ -567,7 +568,8 @@ class Mega2Layer(nn.Module):
 
     def forward(self, x: Tensor, padding_mask: Optional[Tensor] = None, incremental_state=None) -> Tensor:
         x, _ = self.attn(x, padding_mask, incremental_state)
-        return self.ffn(self.ffn_norm(x, padding_mask, incremental_state), residual=x)
+        # x is this layer's own intermediate: the feed-forward block may accumulate into it
+        return self.ffn(self.ffn_norm(x, padding_mask, incremental_state), residual=x, consume_residual=True)
 
 
 def _arg(args, name, default):
@@ -613,7 +615,7 @@ class MegaDecoderLayer(nn.Module):
         """x: [B, L, D] -> (x, None, None), the reference's return triple."""
         x, attn = self.mega_layer(x, decoder_padding_mask, incremental_state, need_weights=need_attn)
         if self.nffn is not None:
-            x = self.nffn(x)
+            x = self.nffn(x, consume_input=True)      # x is this layer's own intermediate
         return x, attn, None
 
 
@@ -647,7 +649,7 @@ class MegaEncoderLayer(nn.Module):
     def forward(self, x: Tensor, encoder_padding_mask: Optional[Tensor] = None) -> Tensor:
         x, _ = self.mega_layer(x, encoder_padding_mask)
         if self.nffn is not None:
-            x = self.nffn(x)
+            x = self.nffn(x, consume_input=True)      # x is this layer's own intermediate
         return x
 
 

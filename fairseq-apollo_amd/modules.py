@@ -439,10 +439,13 @@ class TimestepNormFunc(torch.autograd.Function):
             ctx.save_for_backward(x, prev_mean, count, group_mean, cummean, cumrstd, gamma, padding_mask)
         ctx.num_groups = num_groups
         ctx.mark_non_differentiable(count)
+        ctx.set_materialize_grads(False)        # unused final statistics: no zero tensors made for their gradients
         return y, count, mean, var
 
     @staticmethod
     def backward(ctx, y_grad, _, mean_grad, var_grad):
+        if y_grad is None:
+            y_grad = torch.zeros_like(ctx.saved_tensors[0])
         if ctx.num_groups is None:
             x, prev_mean, count, cummean, cumrstd, gamma, padding_mask = ctx.saved_tensors
             grads = ops.timestep_norm_bwd(y_grad, mean_grad, var_grad, x, prev_mean, count, cummean, cumrstd, gamma,
@@ -979,15 +982,20 @@ class EfficientAttention(nn.Module):
         return 'causal={}, dropout={}'.format(self._causal, self._dropout)
 
 
-def linear_residual(lin: nn.Linear, h: Tensor, residual: Optional[Tensor]) -> Tensor:
+def linear_residual(lin: nn.Linear, h: Tensor, residual: Optional[Tensor], consume: bool = False) -> Tensor:
     """lin(h) + residual as one library GEMM (the residual is the accumulator's start, rounded once with the
-    product); lin(h) when there is no residual."""
+    product); lin(h) when there is no residual.  consume: the caller owns `residual` and has no further use for
+    it, so outside autograd the product is accumulated into it in place (the out-of-place form first copies the
+    residual into its result: one more pass over the activations)."""
     if residual is None:
         return lin(h)
     if lin.bias is not None or residual.dtype != h.dtype or not residual.is_contiguous():
         return lin(h) + residual
-    out = torch.addmm(residual.reshape(-1, residual.shape[-1]), h.reshape(-1, h.shape[-1]), lin.weight.t())
-    return out.view(residual.shape)
+    r2, h2 = residual.reshape(-1, residual.shape[-1]), h.reshape(-1, h.shape[-1])
+    if consume and not torch.is_grad_enabled() and not residual.requires_grad:
+        r2.addmm_(h2, lin.weight.t())
+        return residual
+    return torch.addmm(r2, h2, lin.weight.t()).view(residual.shape)
 
 
 class SwiGLU(nn.Module):
@@ -1000,8 +1008,8 @@ class SwiGLU(nn.Module):
         self.w3 = nn.Linear(embed_dim, hidden_dim, bias=bias)
         self.w2 = nn.Linear(hidden_dim, embed_dim, bias=bias)
 
-    def forward(self, x: Tensor, residual: Optional[Tensor] = None) -> Tensor:
+    def forward(self, x: Tensor, residual: Optional[Tensor] = None, consume_residual: bool = False) -> Tensor:
         """W2 (silu(W1 x) * W3 x) (+ residual, which then enters the last product as its accumulator start: no
-        separate addition pass over the activations)."""
+        separate addition pass over the activations; consume_residual: see linear_residual)."""
         gate = SwiGLUFunc.apply(self.w1(x), self.w3(x)) if _training_call(self, x) else ops.swiglu(self.w1(x), self.w3(x))
-        return linear_residual(self.w2, gate, residual)
+        return linear_residual(self.w2, gate, residual, consume_residual)

@@ -504,3 +504,21 @@ def test_weights_loaded_after_an_eval_forward_take_effect():
         ya3, _ = a(x)
         yb3, _ = b(x)
         assert torch.equal(ya3, yb3) and not torch.equal(ya3, ya2)
+
+
+def test_residual_product_in_place():
+    """linear_residual: outside autograd a residual the caller gives up takes the product in place (no copy of the
+    residual first); under autograd, or without `consume`, the residual is left as it was."""
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(96, 64, bias=False).to(DEV).to(torch.bfloat16)
+    h = torch.randn(2, 40, 96, device=DEV).to(torch.bfloat16)
+    res = torch.randn(2, 40, 64, device=DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        ref = M.modules.linear_residual(lin, h, res)
+        assert ref.data_ptr() != res.data_ptr()
+        mine = res.clone()
+        out = M.modules.linear_residual(lin, h, mine, consume=True)
+        assert out.data_ptr() == mine.data_ptr() and torch.equal(out, ref)
+    keep = res.clone()
+    out = M.modules.linear_residual(lin, h, res, consume=True)          # autograd on: lin.weight requires grad
+    assert out.data_ptr() != res.data_ptr() and torch.equal(res, keep) and torch.equal(out, ref)
