@@ -88,6 +88,134 @@ int launch_silu(const void* a, void* y, int64_t n, hipStream_t s) {
   return MEGA_OK;
 }
 
+// dx = dy silu'(x),  silu'(x) = s (1 + x (1 - s)), s = sigmoid(x)
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void silu_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ a,
+                                                       T* __restrict__ dx, int64_t n) {
+  using V = Vec<T, VEC>;
+  const int64_t nv = n / VEC;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  auto f = [](float g, float x) {
+    const float sg = __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+    return g * sg * fmaf(x, 1.0f - sg, 1.0f);
+  };
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nv; i += stride) {
+    const V gv = ((const V*)dy)[i];
+    const V av = ((const V*)a)[i];
+    V o;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) o.v[k] = from_float<T>(f(to_float(gv.v[k]), to_float(av.v[k])));
+    ((V*)dx)[i] = o;
+  }
+  const int64_t t = nv * VEC + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) dx[t] = from_float<T>(f(to_float(dy[t]), to_float(a[t])));
+}
+
+template <typename T>
+int launch_silu_bwd(const void* dy, const void* a, void* dx, int64_t n, hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const bool aligned = (((uintptr_t)dy | (uintptr_t)a | (uintptr_t)dx) % 16) == 0;
+  int64_t blocks = ceil_div(ceil_div(n, VEC), 256);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  if (aligned)
+    hipLaunchKernelGGL((silu_bwd_kernel<T, VEC>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)dy, (const T*)a,
+                       (T*)dx, n);
+  else
+    hipLaunchKernelGGL((silu_bwd_kernel<T, 1>), dim3((unsigned)blocks), dim3(256), 0, s, (const T*)dy, (const T*)a,
+                       (T*)dx, n);
+  MEGA_CHECK_LAUNCH("silu_bwd");
+  return MEGA_OK;
+}
+
+// Column sums of a [T, W] matrix (the bias gradient of a projection: the sum of its output's gradient over the
+// tokens).  A workgroup owns kColBlock columns (a lane VEC adjacent ones) and one slab of rows; its four waves take
+// every fourth row of the slab, four rows in flight per wave, and add up through LDS in wave order; one row of
+// partial sums per slab of 256 rows goes to the workspace, and colsum_finish_kernel adds the slabs in order: the
+// same bits on every run.
+constexpr int kColSlabRows = 256;
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ x, int64_t rs, int64_t T_, int W,
+                                                             float* __restrict__ part) {
+  using V = Vec<T, VEC>;
+  __shared__ float s_acc[3][64 * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c0 = ((int)blockIdx.x * 64 + lane) * VEC;
+  const int64_t r0 = (int64_t)blockIdx.y * kColSlabRows;
+  const int64_t r1 = r0 + kColSlabRows < T_ ? r0 + kColSlabRows : T_;
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+  if (c0 < W) {
+    for (int64_t r = r0 + wave; r < r1; r += 16) {
+      V v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t rr = r + 4 * u;
+        if (rr < r1) {
+          v[u] = *(const V*)(x + rr * rs + c0);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) v[u].v[e] = from_float<T>(0.f);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += to_float(v[u].v[e]);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s_acc[wave - 1][lane * VEC + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && c0 < W) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float t = acc[e];
+      for (int w = 0; w < 3; ++w) t += s_acc[w][lane * VEC + e];
+      part[(int64_t)blockIdx.y * W + c0 + e] = t;
+    }
+  }
+}
+
+template <typename TOut>
+__global__ __launch_bounds__(64) void colsum_finish_kernel(const float* __restrict__ part, int nslab, int W,
+                                                            TOut* __restrict__ out) {
+  const int c = (int)blockIdx.x * 64 + (int)threadIdx.x;
+  if (c >= W) return;
+  float t = 0.f;
+  for (int s0 = 0; s0 < nslab; s0 += 8) {          // eight slabs requested together, added in slab order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = s0 + u < nslab ? part[(int64_t)(s0 + u) * W + c] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t += v[u];
+  }
+  out[c] = from_float<TOut>(t);
+}
+
+template <typename T>
+int launch_colsum(const void* x, int64_t rs, int64_t T_, int64_t W, void* out, int out_dtype, float* part,
+                  hipStream_t s) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  const int nslab = (int)ceil_div(T_, kColSlabRows);
+  const dim3 grid((unsigned)ceil_div(W, 64 * VEC), (unsigned)nslab);
+  hipLaunchKernelGGL((colsum_partial_kernel<T, VEC>), grid, dim3(256), 0, s, (const T*)x, rs, T_, (int)W, part);
+  MEGA_CHECK_LAUNCH("colsum");
+  const dim3 g2((unsigned)ceil_div(W, 64));
+  if (out_dtype == MEGA_F32)
+    hipLaunchKernelGGL(colsum_finish_kernel<float>, g2, dim3(64), 0, s, part, nslab, (int)W, (float*)out);
+  else if (out_dtype == MEGA_BF16)
+    hipLaunchKernelGGL(colsum_finish_kernel<bf16_t>, g2, dim3(64), 0, s, part, nslab, (int)W, (bf16_t*)out);
+  else
+    hipLaunchKernelGGL(colsum_finish_kernel<f16_t>, g2, dim3(64), 0, s, part, nslab, (int)W, (f16_t*)out);
+  MEGA_CHECK_LAUNCH("colsum (slabs)");
+  return MEGA_OK;
+}
+
 // zeros for small outputs of degenerate calls
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* __restrict__ p, size_t n) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -131,5 +259,53 @@ extern "C" int mega_silu_fwd(const void* a, void* y, int dtype, int64_t n, void*
     case MEGA_F32: return launch_silu<float>(a, y, n, s);
     case MEGA_BF16: return launch_silu<bf16_t>(a, y, n, s);
     default: return launch_silu<f16_t>(a, y, n, s);
+  }
+}
+
+extern "C" int mega_silu_bwd(const void* y_grad, const void* a, void* a_grad, int dtype, int64_t n, void* stream) {
+  MEGA_REQUIRE(dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16, MEGA_ERR_ARG,
+               "silu_bwd: unknown dtype %d", dtype);
+  MEGA_REQUIRE(n >= 0, MEGA_ERR_ARG, "silu_bwd: negative size");
+  if (n == 0) return MEGA_OK;
+  MEGA_REQUIRE(y_grad && a && a_grad, MEGA_ERR_ARG, "silu_bwd: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case MEGA_F32: return launch_silu_bwd<float>(y_grad, a, a_grad, n, s);
+    case MEGA_BF16: return launch_silu_bwd<bf16_t>(y_grad, a, a_grad, n, s);
+    default: return launch_silu_bwd<f16_t>(y_grad, a, a_grad, n, s);
+  }
+}
+
+extern "C" size_t mega_colsum_workspace_bytes(int64_t T_, int64_t W) {
+  if (T_ <= 0 || W <= 0) return 256;
+  return (size_t)ceil_div(T_, kColSlabRows) * (size_t)W * 4;
+}
+
+extern "C" int mega_colsum(const void* x, int64_t row_stride, int dtype, int64_t T_, int64_t W, void* out,
+                           int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  MEGA_REQUIRE((dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16) &&
+                   (out_dtype == MEGA_F32 || out_dtype == MEGA_BF16 || out_dtype == MEGA_F16),
+               MEGA_ERR_ARG, "colsum: unknown dtype %d / %d", dtype, out_dtype);
+  MEGA_REQUIRE(T_ >= 0 && W >= 1 && W < (1ll << 30) && row_stride >= W, MEGA_ERR_ARG,
+               "colsum: bad sizes T=%lld W=%lld row stride %lld", (long long)T_, (long long)W, (long long)row_stride);
+  MEGA_REQUIRE(out, MEGA_ERR_ARG, "colsum: null pointer argument");
+  hipStream_t s = (hipStream_t)stream;
+  const size_t esz = dtype == MEGA_F32 ? 4 : 2;
+  if (T_ == 0) {
+    MEGA_REQUIRE(out_dtype == MEGA_F32 ? true : (W % 2 == 0), MEGA_ERR_UNSUPPORTED,
+                 "colsum: an empty matrix with an odd number of 16-bit columns");
+    zero_async(out, (size_t)W * (out_dtype == MEGA_F32 ? 4 : 2), s);
+    return MEGA_OK;
+  }
+  MEGA_REQUIRE(x, MEGA_ERR_ARG, "colsum: null pointer argument");
+  // whole 16-byte pieces per lane: the width, the row pitch and the base address in pieces
+  MEGA_REQUIRE((W * esz) % 16 == 0 && (row_stride * esz) % 16 == 0 && ((uintptr_t)x % 16) == 0, MEGA_ERR_UNSUPPORTED,
+               "colsum: rows of whole 16-byte pieces only (W=%lld, row stride %lld)", (long long)W, (long long)row_stride);
+  const size_t need = mega_colsum_workspace_bytes(T_, W);
+  MEGA_REQUIRE(workspace && workspace_bytes >= need, MEGA_ERR_WORKSPACE, "colsum: workspace of %zu bytes needed", need);
+  switch (dtype) {
+    case MEGA_F32: return launch_colsum<float>(x, row_stride, T_, W, out, out_dtype, (float*)workspace, s);
+    case MEGA_BF16: return launch_colsum<bf16_t>(x, row_stride, T_, W, out, out_dtype, (float*)workspace, s);
+    default: return launch_colsum<f16_t>(x, row_stride, T_, W, out, out_dtype, (float*)workspace, s);
   }
 }

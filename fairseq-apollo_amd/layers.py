@@ -24,7 +24,7 @@ from torch.nn import Parameter
 from . import ops
 from .modules import (AttentionSoftmax, EfficientAttention, GateMulFunc, GateOutFunc, GateQKFunc, IncrementalState,
                       MultiHeadComplexEMA, MultiHeadEMA, SequenceNorm, SplitFunc, SplitGrads, SwiGLU, TimestepNorm,
-                      _tensor_versions, _training_call, linear_residual, norm_then_move)
+                      _tensor_versions, _training_call, linear, linear_residual, norm_then_move, silu)
 
 
 class RMSNorm(nn.Module):
@@ -120,7 +120,7 @@ class NormalizedFeedForwardNetwork(nn.Module):
         # hidden dropout acts whenever the module is in training mode, with or without a graph
         # (normalized_feedforward_network.py:81-83)
         if _training_call(self, x) or (self.training and self.hidden_dropout_p > 0):
-            h = F.dropout(F.silu(self.fc1(self.norm(x))), self.hidden_dropout_p, self.training)
+            h = F.dropout(silu(linear(self.fc1, self.norm(x))), self.hidden_dropout_p, self.training)
         else:
             h = ops.silu(self.fc1(self.norm(x)), inplace=True)
         if self.layerscale_weight is None and not (self.training and self.dropout_p > 0):
@@ -420,8 +420,9 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         else:
             x, mx = norm_then_move(self.norm, self.move, x, padding_mask, None, out_layout="input")
             mx = mx.transpose(1, 2)
-        v = F.silu(self.v_proj(x))
-        base = self.mx_proj(F.dropout(self.move_act(mx), self.hidden_dropout_p, self.training))
+        v = silu(linear(self.v_proj, x))
+        mx = self.move_act(mx) if isinstance(self.move_act, RMSNorm) else silu(mx)
+        base = linear(self.mx_proj, F.dropout(mx, self.hidden_dropout_p, self.training))
         # the four slices' gradients are written into one buffer by the backward kernels of their consumers
         arena = SplitGrads(base, [self.embed_dim, self.zdim, self.hdim, self.embed_dim])
         u, z, r, hx = SplitFunc.apply(base, arena)
@@ -467,7 +468,7 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
         else:
             attn = self.efficient_attn(q4, k4, v4)
         gated = GateMulFunc.apply(attn.reshape(bsz, seq_len, self.hdim), r, (arena, 2))
-        hp = self.h_proj(F.dropout(gated, self.hidden_dropout_p, self.training))
+        hp = linear(self.h_proj, F.dropout(gated, self.hidden_dropout_p, self.training))
         if self.training and self.dropout_p > 0:
             # the output dropout sits between the activation and the residual mix
             # (moving_average_gated_attention.py:409-412), so the fused gate is taken apart

@@ -866,6 +866,62 @@ class GateOutFunc(torch.autograd.Function):
         return dres, du, dh, dh, None
 
 
+class SiluFunc(torch.autograd.Function):
+    """F.silu with the library's kernels both ways."""
+
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return ops.silu(x)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        return ops.silu_bwd(y_grad, ctx.saved_tensors[0])
+
+
+def silu(x: Tensor) -> Tensor:
+    """silu(x): the library's kernels on the GPU (with their own backward under autograd), F.silu elsewhere."""
+    if not x.is_cuda:
+        return F.silu(x)
+    if torch.is_grad_enabled() and x.requires_grad:
+        return SiluFunc.apply(x)
+    return ops.silu(x)
+
+
+class LinearFunc(torch.autograd.Function):
+    """F.linear whose backward takes the bias gradient from the library's column sums (torch's sum over the tokens
+    runs at a third of the memory rate on matrices this wide); the three products stay library GEMMs, and a
+    row-strided output gradient (a slice of a wider gradient buffer) is read in place."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return F.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, y_grad):
+        x, weight = ctx.saved_tensors
+        g2 = y_grad.reshape(-1, y_grad.shape[-1])
+        x2 = x.reshape(-1, x.shape[-1])
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.mm(g2, weight).view(x.shape)
+        if ctx.needs_input_grad[1]:
+            dw = torch.mm(g2.t(), x2)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = ops.colsum(y_grad, weight.dtype)
+        return dx, dw, db
+
+
+def linear(lin: nn.Linear, x: Tensor) -> Tensor:
+    """lin(x); under autograd on the GPU with the bias gradient as the library's column sums."""
+    if lin.bias is not None and x.is_cuda and x.dtype == lin.weight.dtype and torch.is_grad_enabled() and \
+            (x.requires_grad or lin.weight.requires_grad):
+        return LinearFunc.apply(x, lin.weight, lin.bias)
+    return lin(x)
+
+
 class SwiGLUFunc(torch.autograd.Function):
     """silu(a) * b with its own backward."""
 

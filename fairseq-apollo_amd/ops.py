@@ -1207,6 +1207,39 @@ def silu(x: torch.Tensor, inplace: bool = False) -> torch.Tensor:
     return y
 
 
+def silu_bwd(y_grad: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """Backward of silu: y_grad * silu'(x)."""
+    dev = _need_gpu(y_grad, x)
+    lib = _lib.load()
+    xd = x.detach().contiguous()
+    g = y_grad.detach().to(xd.dtype).contiguous()
+    dx = torch.empty_like(xd)
+    with _on_device(dev):
+        rc = lib.mega_silu_bwd(_ptr(g), _ptr(xd), _ptr(dx), _dtype_code(xd), xd.numel(), _stream(dev))
+    _lib.check(rc, "silu_bwd")
+    return dx
+
+
+def colsum(x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Sum of a [..., W] tensor over everything but its last axis (a projection's bias gradient), slabs of rows
+    added in a fixed order; rows that are not whole 16-byte pieces go through torch."""
+    dev = _need_gpu(x)
+    lib = _lib.load()
+    W = x.shape[-1]
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    xr, rs = _rows(x)
+    T = _ntok(x)
+    if T == 0 or (W * xr.element_size()) % 16 or (rs * xr.element_size()) % 16 or xr.data_ptr() % 16:
+        return x.detach().reshape(-1, W).sum(0, dtype=torch.float32).to(out_dtype)
+    out = torch.empty(W, dtype=out_dtype, device=dev)
+    stream = _stream(dev)
+    ws = _scratch_buffer(dev, lib.mega_colsum_workspace_bytes(T, W), stream)
+    with _on_device(dev):
+        rc = lib.mega_colsum(_ptr(xr), rs, _dtype_code(xr), T, W, _ptr(out), _DT[out_dtype], _ptr(ws), ws.numel(), stream)
+    _lib.check(rc, "colsum")
+    return out
+
+
 # ------------------------------------------------------------------------------------------------
 # per-token glue of the gated-attention layer (rows of a wider projection output are passed in
 # place: every input carries its own row stride)

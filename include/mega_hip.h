@@ -595,6 +595,15 @@ int mega_gate_out_bwd(const void* y_grad, const void* residual, int64_t residual
                       void* h_grad, int dtype, int64_t T, int64_t D, void* stream);
 int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_grad, void* b_grad,
                     int dtype, int64_t n, void* stream);
+/* Backward of mega_silu_fwd (F.silu under autograd): a_grad = y_grad silu'(a), contiguous, n elements.   */
+int mega_silu_bwd(const void* y_grad, const void* a, void* a_grad, int dtype, int64_t n, void* stream);
+/* Column sums of x [T, W] (row stride in elements) into out [W] of `out_dtype`: the bias gradient of a projection
+ * (in the reference torch's sum over the tokens inside the backward of F.linear).  Rows of whole 16-byte pieces;
+ * slabs of 256 rows are added in a fixed order (the same bits on every run); workspace of
+ * mega_colsum_workspace_bytes(T, W), no initialisation.                                              */
+size_t mega_colsum_workspace_bytes(int64_t T, int64_t W);
+int mega_colsum(const void* x, int64_t row_stride, int dtype, int64_t T, int64_t W, void* out,
+                int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 /* The same three with row strides (in elements) on the gradients of u, z, r, hx: these four are slices of
  * the mx_proj output (torch.split, moving_average_gated_attention.py:319), whose backward in the reference is
  * a concatenation of the four gradients; a caller that owns one [T, D + S + E + D] gradient buffer lets each

@@ -768,6 +768,37 @@ def test_gate_backwards(dtype, shape, width, off):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_silu_backward_and_column_sums(dtype):
+    """silu backward against the closed form; column sums (bias gradients) of contiguous and row-strided matrices
+    against fp64 sums, the same bits on a second run; LinearFunc against torch's own backward of F.linear."""
+    rng = np.random.default_rng(97)
+    sg = O._sigmoid
+    x, x64 = rounded(rng.normal(size=(3, 37, 24)) * 2, dtype)
+    dy, dy64 = rounded(rng.normal(size=(3, 37, 24)), dtype)
+    assert rel_err(host(M.ops.silu_bwd(dy, x)), dy64 * sg(x64) * (1 + x64 * (1 - sg(x64)))) < TOL[dtype]
+    for T, W, width, off in ((200, 48, 48, 0), (1000, 64, 160, 32), (63, 8, 8, 0), (8192, 520, 1048, 8)):
+        wide, w64 = rounded(rng.normal(size=(T, width)), dtype)
+        sl = wide.narrow(-1, off, W)
+        got = M.ops.colsum(sl, torch.float32)
+        ref = w64[:, off:off + W].sum(0)
+        assert rel_err(host(got), ref) < 1e-5 and torch.equal(got, M.ops.colsum(sl, torch.float32))
+        assert M.ops.colsum(sl).dtype == dtype
+    assert rel_err(host(M.ops.colsum(x, torch.float32)), x64.reshape(-1, 24).sum(0)) < 1e-5      # leading axes fold
+    odd, o64 = rounded(rng.normal(size=(50, 7)), dtype)                                          # torch's route
+    assert rel_err(host(M.ops.colsum(odd, torch.float32)), o64.sum(0)) < 1e-5
+    lin = torch.nn.Linear(24, 40).to(DEV).to(dtype)
+    up = torch.randn(3, 37, 40, device=DEV).to(dtype)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    (M.modules.linear(lin, xa) * up).sum().backward()
+    ga = [xa.grad, lin.weight.grad.clone(), lin.bias.grad.clone()]
+    lin.zero_grad()
+    (lin(xb) * up).sum().backward()
+    tol = 1e-5 if dtype == torch.float32 else TOL[dtype]
+    for a, b in zip(ga, [xb.grad, lin.weight.grad, lin.bias.grad]):
+        assert a.dtype == b.dtype and a.shape == b.shape and rel_err(host(a), host(b)) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,L,S,heads,chunk,width,off", [(2, 64, 128, 1, 64, 128, 0), (1, 96, 64, 4, 32, 200, 72),
                                                          (3, 40, 40, 2, 40, 56, 8), (1, 4096, 512, 4, 2048, 512, 0),
                                                          (2, 300, 512, 2, 100, 1024, 512)])
