@@ -26,6 +26,7 @@ SIGNATURES = {
     "mega_abi_version": (_int, []),
     "mega_lookback_init": (_int, []),
     "mega_lookback_status": (_int, [_int]),
+    "mega_lookback_checked": (None, [_int]),
     "mega_test_lookback": (None, [C.c_uint, _int, _int]),
     "mega_audit_begin": (None, []),
     "mega_audit_add": (_int, [_p, _sz]),

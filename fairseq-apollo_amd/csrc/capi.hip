@@ -21,6 +21,8 @@ extern "C" int mega_abi_version(void) { return 3; }
 // gives up stores 1 into it (system scope); the entry points that launch such kernels look at it first and
 // refuse the call once, the way a sticky launch error surfaces on the next call
 // (C10_CUDA_KERNEL_LAUNCH_CHECK(), fairseq/csrc/ops/timestep_norm_kernel.cu:641).
+#include <stdlib.h>
+
 #include <atomic>
 #include <mutex>
 
@@ -38,6 +40,7 @@ volatile uint32_t g_plain[kMaxDevices];   // stands in where no pinned word exis
 std::mutex g_status_mu;
 std::atomic<uint32_t> g_spin_limit{kDefaultSpinLimit};
 std::atomic<int> g_withhold_first{0};
+std::atomic<int> g_checked{-1};             // -1: not decided yet (the environment decides at the first question)
 
 int current_slot() {
   int d = 0;
@@ -78,6 +81,34 @@ LookbackLaunch lookback_launch(bool may_allocate) {
   return l;
 }
 
+bool lookback_checked() {
+  int v = g_checked.load();
+  if (v < 0) {
+    const char* e = getenv("MEGA_LOOKBACK_CHECKED");
+    v = (e && e[0] && e[0] != '0') ? 1 : 0;
+    g_checked.store(v);
+  }
+  return v != 0;
+}
+
+int lookback_verify(const char* entry, hipStream_t stream) {
+  if (!lookback_checked()) return MEGA_OK;
+  const hipError_t e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    set_error("%s: checked mode could not wait for the launch (%s); it cannot be used under stream capture", entry,
+              hipGetErrorString(e));
+    return MEGA_ERR_LAUNCH;
+  }
+  StatusSlot& s = slot_of(current_slot(), false);
+  if (*s.host == 0u) return MEGA_OK;
+  *s.host = 0u;
+  set_error("%s: this launch gave up waiting for the words of an earlier tile (workgroups not dispatched in id "
+            "order, or a workspace shared by launches that overlap); it has written NaN into the outputs and "
+            "statistics that depended on them.  The status is now clear", entry);
+  return MEGA_ERR_LAUNCH;
+}
+
 int lookback_pending(const char* entry) {
   StatusSlot& s = slot_of(current_slot(), false);
   if (*s.host == 0u) return MEGA_OK;
@@ -99,6 +130,8 @@ extern "C" int mega_lookback_init(void) {
   }
   return MEGA_OK;
 }
+
+extern "C" void mega_lookback_checked(int on) { mega::g_checked.store(on ? 1 : 0); }
 
 extern "C" int mega_lookback_status(int clear) {
   auto& s = mega::slot_of(mega::current_slot(), false);

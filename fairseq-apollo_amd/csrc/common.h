@@ -25,6 +25,9 @@ struct LookbackLaunch {
 LookbackLaunch lookback_launch(bool may_allocate);
 // MEGA_ERR_LAUNCH (message set, word cleared) when a launch on the current device has given up since the last check
 int lookback_pending(const char* entry);
+// checked mode (mega_lookback_checked / MEGA_LOOKBACK_CHECKED=1): waits for the stream and reports a give-up of the
+// launch just made; MEGA_OK at once when the mode is off
+int lookback_verify(const char* entry, hipStream_t stream);
 
 #define MEGA_REQUIRE(cond, code, ...)  \
   do {                                 \

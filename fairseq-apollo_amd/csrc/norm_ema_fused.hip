@@ -1012,7 +1012,7 @@ extern "C" int mega_norm_ema_fwd_train(const void* x, void* xn, void* y, int dty
     }
     hipLaunchKernelGGL(kern, grid, dim3(kFT), kFSmem, s, A);
     MEGA_CHECK_LAUNCH("norm_ema_fwd");
-    return MEGA_OK;
+    return lookback_verify("norm_ema_fwd", s);
   }
   // outside the one-kernel envelope: the two operators one after the other
   // (x -> xn by the norm, xn read through its transposed view by the moving average); the norm keeps its

@@ -805,11 +805,14 @@ static int group_tsn_fwd_impl(const void* x, void* y, int dtype, const int64_t* 
   P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G;
   P.TT = g.tt; P.ntiles = g.ntiles; P.nblk = (int)ceil_div(g.ntiles, kLbBlock); P.TPT = g.tpt; P.LPG = g.lpg; P.eps = (float)eps;
   P.lb = lookback_launch(!fixed_scratch);
+  int rc;
   switch (dtype) {
-    case MEGA_F32: return dispatch_vec<float>(P, g, s);
-    case MEGA_BF16: return dispatch_vec<bf16_t>(P, g, s);
-    default: return dispatch_vec<f16_t>(P, g, s);
+    case MEGA_F32: rc = dispatch_vec<float>(P, g, s); break;
+    case MEGA_BF16: rc = dispatch_vec<bf16_t>(P, g, s); break;
+    default: rc = dispatch_vec<f16_t>(P, g, s); break;
   }
+  // the entry point that may not allocate may not wait either (it serves callers under stream capture)
+  return rc != MEGA_OK || fixed_scratch ? rc : lookback_verify("group_timestep_norm_fwd", s);
 }
 
 extern "C" int mega_group_timestep_norm_fwd(const void* x, void* y, int dtype,

@@ -132,6 +132,12 @@ def lookback_status(clear: bool = False) -> int:
     return int(_lib.load().mega_lookback_status(1 if clear else 0))
 
 
+def lookback_checked(on: bool) -> None:
+    """Checked mode of the bounded waits (mega_lookback_checked): the calls that launch such kernels wait for
+    their stream and raise for a give-up of that very call.  Off by default."""
+    _lib.load().mega_lookback_checked(1 if on else 0)
+
+
 def check_lookback(where: str = "") -> None:
     """Raise (and clear the status) if a launch has given up since the last check.  The library does the same
     at the start of the calls that launch such kernels; streaming helpers call this once more when they are

@@ -75,6 +75,11 @@ int mega_abi_version(void);
  * it exists (no counterpart in the reference).                                                        */
 int mega_lookback_init(void);
 int mega_lookback_status(int clear);
+/* Checked mode, off by default (on: mega_lookback_checked(1), or MEGA_LOOKBACK_CHECKED=1 in the environment when the
+ * library is first asked): mega_group_timestep_norm_fwd and mega_norm_ema_fwd(_train) wait for their stream after
+ * the launch and return MEGA_ERR_LAUNCH for a give-up of that very call instead of leaving it to the next one.  For
+ * debugging and for callers that prefer a synchronous error to throughput; not usable under stream capture.   */
+void mega_lookback_checked(int on);
 
 /* Test hook for the failure path, so that it can be exercised with every kernel exiting normally:
  * spin_limit = polls before a wait gives up (0 = the default, 2^22); withhold_first != 0 makes the first

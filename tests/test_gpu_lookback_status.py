@@ -93,3 +93,34 @@ def test_one_kernel_block_that_gives_up(hooks):
     torch.cuda.synchronize()
     assert torch.equal(again[0], good[0]) and torch.equal(again[1], good[1]) and torch.equal(again[3], good[3])
     assert M.ops.lookback_status() == 0
+
+
+def test_checked_mode_reports_the_give_up_of_the_same_call(hooks):
+    """With checked mode on, the call whose launch gave up raises itself (after waiting for its stream); nothing is
+    left over for the next call."""
+    lib = hooks
+    B, L, G, N = 2, 4096, 2, 16
+    D = 64 * G
+    rng = np.random.default_rng(63)
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, D, N))
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(rng.normal(size=D)))
+    x = torch.randn(B, L, D, device=DEV).to(BF)
+    gamma, beta = torch.ones(D, device=DEV), torch.zeros(D, device=DEV)
+    block = lambda: layer.norm_forward(x, *_state(B, G), gamma, beta, G, 1e-5)
+    norm = lambda: M.ops.group_timestep_norm_fwd(x, *_state(B, G), gamma, beta, None, G, 1e-5, need_stats=False)
+    good_b, good_n = block(), norm()
+    torch.cuda.synchronize()
+    M.ops.lookback_checked(True)
+    try:
+        for run, good in ((block, good_b), (norm, good_n)):
+            print("forced give-up in checked mode", flush=True)
+            lib.mega_test_lookback(64, 1, 0)
+            with pytest.raises(RuntimeError, match="this launch gave up"):
+                run()
+            lib.mega_test_lookback(0, 0, 0)
+            assert M.ops.lookback_status() == 0
+            again = run()                                    # nothing pending: the next call runs, and is right
+            torch.cuda.synchronize()
+            assert torch.equal(again[0], good[0]) and torch.equal(again[1], good[1])
+    finally:
+        M.ops.lookback_checked(False)
