@@ -162,3 +162,63 @@ def test_bench_measures_one_gpu_only():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=120)
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_split_keeps_its_gradient_buffer_or_concatenates():
+    """SplitFunc / SplitGrads (the backward of the split of the mx_proj output): when every slice's gradient is the
+    slot the buffer handed out, the buffer itself comes back (no copy); any other mix -- a slice nobody used, a
+    gradient made elsewhere -- is concatenated, and the result equals torch.split's in both cases."""
+    import torch
+
+    from fairseq_apollo_amd.modules import SplitFunc, SplitGrads
+
+    class IntoSlot(torch.autograd.Function):
+        """y = 2 x whose backward writes into the slot it is given."""
+
+        @staticmethod
+        def forward(ctx, x, slot):
+            ctx.slot = slot
+            return 2 * x
+
+        @staticmethod
+        def backward(ctx, g):
+            out = ctx.slot[0].slot(ctx.slot[1])
+            out.copy_(2 * g)
+            return out, None
+
+    torch.manual_seed(0)
+    widths = [3, 5, 4]
+    base0 = torch.randn(2, 6, sum(widths))
+    w = [torch.randn(2, 6, k) for k in widths]
+
+    def reference(used):
+        b = base0.clone().requires_grad_(True)
+        parts = torch.split(b, widths, dim=-1)
+        sum((2 * parts[i] * w[i]).sum() for i in used).backward()
+        return b.grad
+
+    # every slice through a consumer that writes its slot: the buffer comes back as it is
+    b = base0.clone().requires_grad_(True)
+    arena = SplitGrads(b, widths)
+    parts = SplitFunc.apply(b, arena)
+    before = SplitGrads.taken
+    sum((IntoSlot.apply(parts[i], (arena, i)) * w[i]).sum() for i in range(3)).backward()
+    assert SplitGrads.taken == before + 1 and arena.buf is None
+    assert torch.equal(b.grad, reference(range(3)))
+    # one slice unused, one gradient made by torch: concatenation, same values
+    b = base0.clone().requires_grad_(True)
+    arena = SplitGrads(b, widths)
+    parts = SplitFunc.apply(b, arena)
+    before = SplitGrads.taken
+    ((IntoSlot.apply(parts[0], (arena, 0)) * w[0]).sum() + (2 * parts[2] * w[2]).sum()).backward()
+    assert SplitGrads.taken == before and arena.buf is None
+    assert torch.equal(b.grad, reference([0, 2]))
+    # a second backward pass through a retained graph gets a buffer of its own
+    b = base0.clone().requires_grad_(True)
+    arena = SplitGrads(b, widths)
+    parts = SplitFunc.apply(b, arena)
+    loss = sum((IntoSlot.apply(parts[i], (arena, i)) * w[i]).sum() for i in range(3))
+    loss.backward(retain_graph=True)
+    first = b.grad.clone()
+    loss.backward()
+    assert torch.equal(b.grad, 2 * first)
