@@ -36,6 +36,8 @@
 #define MEGA_TR_FLUSH()
 #endif
 
+// 1: the states enter the output product as two bf16 terms for every channel (one term leaves an error of 2^-9 of
+// sum |gamma q h| at the first tokens of every tile); 0: only for slow poles and layers of few states
 #ifndef MEGA_TWO_ALWAYS
 #define MEGA_TWO_ALWAYS 0
 #endif
@@ -497,8 +499,11 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
     }
     Rr = __uint_as_float(rr.x);
     Ri = __uint_as_float(rr.y);
-    // reach word of the image: |q|^128 >= 2^-24 for some state of the channel
-    two_terms = __builtin_amdgcn_readfirstlane(
+    // the second term where the reach word of the image says |q|^128 >= 2^-24 for some state of the channel, in
+    // layers of few states (their rounding errors do not average out in the sum over the states) and in real-valued
+    // layers (input weights of alternating sign: the states cancel by construction)
+    two_terms = A.N <= 8 || !A.is_complex ||
+                __builtin_amdgcn_readfirstlane(
                     (int)*(const uint32_t*)((const char*)(A.image + (size_t)(A.koff + chc) * kImgSlots * 64) +
                                             kSlotCmp * 1024 + kCmpReach * 128)) >= 2;
     if (A.h_in && (lane & 3) == 0 && (lane >> 2) < A.N && ch_ok) {
@@ -704,8 +709,8 @@ __global__ __launch_bounds__(kThreadsM) void ema_mfma_kernel(const MfmaArgs A) {
         Y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Kw[w][1], X, Y1, 0, 0, 0);
       }
       if (MEGA_TWO_ALWAYS || two_terms) {
-        // slow poles: the states dwarf y and cancel in the sum over the states, so what bf16 drops of them is carried
-        // into the product as a second term
+        // the states can dwarf y and cancel in the sum over the states, so what bf16 drops of them is carried into
+        // the product as a second term
         {
           const float hv[8] = {Hr[0], Hi[0], Hr[1], Hi[1], Hr[2], Hi[2], Hr[3], Hi[3]};
 #pragma unroll

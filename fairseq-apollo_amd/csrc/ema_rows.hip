@@ -403,11 +403,15 @@ __global__ __launch_bounds__(64 * kRW, MEGA_ROWS_MINB) void ema_rows_kernel(cons
     Y1 = mfma<F16>(Kw[0][1], Xh, Y1);
     Y0 = mfma<F16>(Kw[1][0], Xh, Y0);
     Y1 = mfma<F16>(Kw[1][1], Xh, Y1);
-    if (NC > 1) {
+    {
+      // the states as two terms in either operand type (one bf16 term leaves 2^-9 of sum |gamma q h| at the first
+      // tokens of every tile, which shows where the states cancel in the sum over the states)
       const uint4 Hl = make_uint4(hl[0] | ((uint32_t)hl[1] << 16), hl[2] | ((uint32_t)hl[3] << 16),
                                   hl[4] | ((uint32_t)hl[5] << 16), hl[6] | ((uint32_t)hl[7] << 16));
-      Y0 = mfma<F16>(Cw[NC - 1][0], Hh, Y0);
-      Y1 = mfma<F16>(Cw[NC - 1][1], Hh, Y1);
+      if (NC > 1) {
+        Y0 = mfma<F16>(Cw[NC - 1][0], Hh, Y0);
+        Y1 = mfma<F16>(Cw[NC - 1][1], Hh, Y1);
+      }
       Y0 = mfma<F16>(Cw[0][0], Hl, Y0);
       Y1 = mfma<F16>(Cw[0][1], Hl, Y1);
     }

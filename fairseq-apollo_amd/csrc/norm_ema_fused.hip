@@ -21,7 +21,7 @@
 //      look-back: the earlier blocks' end states (and the caller's carried state) folded into the
 //                 block's start state, h_start = sum_d (q^1024)^d E_{s-1-d}, parked over the end states;
 //        phase B: the segment scan again, segment start state = what the segment before left + (q^64)^j h_start,
-//                 y_tile = K x_tile + C h (h as one bf16 term, two for slow poles), bf16, back into LDS over x, and
+//                 y_tile = K x_tile + C h (h as one bf16 term, two for slow poles and few states), bf16, back into LDS over x, and
 //                 out as whole rows.
 // Blocks map to workgroup ids time-major and workgroups are dispatched in id order, so a block only
 // waits for blocks dispatched before it; every wait is bounded and poisons the block's outputs with
@@ -38,6 +38,10 @@
 #endif
 #ifndef MEGA_FTR2
 #define MEGA_FTR2(k)
+#endif
+
+#ifndef MEGA_FUSED_TWO_TERMS
+#define MEGA_FUSED_TWO_TERMS 0
 #endif
 
 namespace mega {
@@ -754,12 +758,18 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   // ---- phase B per channel: the segment scan again (cheaper than keeping four channels' scans in registers across
   // the wait), start state of segment j = what segment j - 1 left + (q^64)^j h_start, then
   // y_tile = K x_tile + C h (h: the state at the tile's first token, carried into the product as two bf16 terms where
-  // the channel's poles are slow enough for the states to dwarf y; at a segment's second tile h = q^32 h + F), bf16,
+  // one would show; at a segment's second tile h = q^32 h + F), bf16,
   // back into LDS over x, and out as whole rows.
 #pragma unroll
   for (int i = 0; i < kFCPW; ++i) {
     const int c = wave + kFW * i;
-    const bool two_terms = nsteps[i] >= 2;           // |q|^128 >= 2^-24 for some state of the channel
+    // One bf16 term for the states leaves an error of 2^-9 of sum |gamma q h| at the first tokens of every tile.  It
+    // shows where the states dwarf y (slow poles: |q|^128 >= 2^-24 for some state of the channel), in layers of few
+    // states, whose rounding errors do not average out in the sum over the states, and in real-valued layers, whose
+    // input weights alternate in sign along the states so that the states cancel by construction: those take a
+    // second term (hi + lo).  MEGA_FUSED_TWO_TERMS=1 gives every channel the second term (+ 0.7 us at the headline
+    // shape).
+    const bool two_terms = MEGA_FUSED_TWO_TERMS || nsteps[i] >= 2 || A.N <= 8 || !A.is_complex;
     uint32_t roff = roff0;
     asm volatile("" : "+v"(roff));
     char* row = tile + row_base(c) + j * 128;

@@ -439,14 +439,17 @@ class MovingAverageGatedAttention(nn.Module, IncrementalState):
             q4 = q.view(bsz * nc, C, Nh, -1)
             k4 = k.view(bsz * nc, C, Nh, -1)
         else:
-            z = F.normalize(z, p=2, dim=-1, eps=1e-5)
-            z = z.unsqueeze(2) * (self.gamma + 1.0) + self.beta
-            q, k = torch.unbind(z, dim=2)
+            # rows the q / k kernel does not take: torch operations, in fp32 like the kernel (in fp16 the backward of
+            # the division by a norm clamped at 1e-5 squares a subnormal and returns NaN), results back in z's type
+            zt = F.normalize(z.float(), p=2, dim=-1, eps=1e-5)
+            zt = zt.unsqueeze(2) * (self.gamma.float() + 1.0) + self.beta.float()
+            q, k = torch.unbind(zt, dim=2)
             q4 = q.reshape(bsz * nc, C, Nh, -1)
             k4 = k.reshape(bsz * nc, C, Nh, -1)
             if not simple:
                 q4 = self.rel_pos_bias.rotary(q4.transpose(1, 2), 0).transpose(1, 2)
                 k4 = self.rel_pos_bias.rotary(k4.transpose(1, 2), 0).transpose(1, 2)
+            q4, k4 = q4.to(z.dtype), k4.to(z.dtype)
         if self.attention_activation != 'softmax':
             attn = self._element_attention(q4, k4, v4, None if padding_mask is None
                                            else padding_mask.reshape(bsz * nc, C))
