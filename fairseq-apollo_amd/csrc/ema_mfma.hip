@@ -37,7 +37,8 @@
 #endif
 
 // 1: the states enter the output product as two bf16 terms for every channel (one term leaves an error of 2^-9 of
-// sum |gamma q h| at the first tokens of every tile); 0: only for slow poles and layers of few states
+// sum |gamma q h| at the first tokens of every tile); 0: only for slow poles, layers of few states and real-valued
+// layers, the rule of the one-kernel block.  The C operand is one bf16 term either way (2^-9 of the same sum)
 #ifndef MEGA_TWO_ALWAYS
 #define MEGA_TWO_ALWAYS 0
 #endif

@@ -41,6 +41,15 @@ def _out_err(y, yo, eps=1.0):
     return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
 
 
+def _worst(y, yo):
+    """Where rel_err takes its maximum, for the messages of failing cases."""
+    a, b = np.asarray(y, np.float64), np.asarray(yo, np.float64)
+    rms = float(np.sqrt(np.mean(b * b)))
+    ratio = np.abs(a - b) / np.maximum(np.abs(b), rms + 1e-300)
+    idx = np.unravel_index(int(np.argmax(ratio)), ratio.shape)
+    return f"worst at {tuple(int(i) for i in idx)}: got {a[idx]:.6g} ref {b[idx]:.6g} rms {rms:.4g} max |ref| {np.abs(b).max():.4g}"
+
+
 def _coeffs(rng, K, N, cplx):
     if cplx:
         return O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
@@ -92,7 +101,7 @@ def test_moving_average_sweep(seed):
         yo, ho = O.ema_forward(x64, p, q, g, om, mask, h=h0, bidirectional=bidir, truncation=trunc if trunc else None,
                                shift=shift, incremental=with_state)
         assert y.shape == (B, D, L), tag
-        assert rel_err(host(y), yo) < TOL[dtype], tag
+        assert rel_err(host(y), yo) < TOL[dtype], (tag, _worst(host(y), yo))
         if with_state:
             tol = 1e-4 if dtype is torch.float32 else 2e-3
             assert _state_err(np.real(host(h)), np.real(ho)) < tol, tag
