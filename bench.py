@@ -623,6 +623,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--settle", type=float, default=0.3, metavar="SECONDS",
+                    help="block workload: seconds of untimed load before the warm-up steps (device clocks settle)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device copies of one [B, L, D] bf16 buffer (32 MiB read + 32 MiB "
                          "written each): the known-size kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -718,7 +720,19 @@ def main():
             regions_log[name] = [max(r[0], r[1]) for r in runs]
         return sorted(runs, key=lambda r: max(r[0], r[1]))[len(runs) // 2]
 
+    def settle(fn, seconds):
+        """Set-up, not measurement: the device enters the run from idle and its clocks need some tens of
+        milliseconds of load to settle (the first of three timed regions read 10 % slower than the third without
+        this).  Runs the step for `seconds` of wall time before the W warm-up steps; neither is timed."""
+        t0, i = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(50):
+                fn(i)
+                i += 1
+            torch.cuda.synchronize()
+
     with torch.no_grad():
+        settle(step, args.settle)
         gpu_ms, wall_ms, host_step = timed(step, args.steps, args.warmup, name="one_call")
         ms_per_step = max(wall_ms, gpu_ms)
         reps = max(20, min(args.steps, 200))
@@ -781,7 +795,7 @@ def main():
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
-        "warmup": args.warmup,
+        "warmup": args.warmup, "settle_s": args.settle,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
