@@ -60,6 +60,22 @@ static inline bool first_on_device(uint64_t* seen) {
   return !(__atomic_fetch_or(seen, bit, __ATOMIC_RELAXED) & bit);
 }
 
+// Compute units of the current device, queried once per device (256 when the query fails).
+static inline int device_cu_count() {
+  static int cu_count[64] = {0};
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= 64) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  int n = __atomic_load_n(&cu_count[d], __ATOMIC_RELAXED);
+  if (n == 0) {
+    n = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) == hipSuccess && n > 0) ? n : 256;
+    __atomic_store_n(&cu_count[d], n, __ATOMIC_RELAXED);
+  }
+  return n;
+}
+
 // ---- address audit (host only).  Between mega_audit_begin() and mega_audit_end() the entry points that take part
 // launch nothing: they compute, for every launch they would make, the last byte each operand is addressed at (from
 // the same sizes and strides the kernel gets) and check that it lies inside one of the byte ranges registered with

@@ -276,18 +276,7 @@ extern "C" int mega_ema_param_grad(const void* dy, const void* x, int dtype, int
     return MEGA_OK;
   }
   // 16 channels per workgroup, 8 when that would leave compute units idle
-  static int cu_count[64] = {0};     // per device, queried once
-  int cus = 256;
-  {
-    int dev_id = 0;
-    if (hipGetDevice(&dev_id) == hipSuccess && dev_id >= 0 && dev_id < 64) {
-      if (cu_count[dev_id] == 0) {
-        int n = 0;
-        cu_count[dev_id] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev_id) == hipSuccess && n > 0) ? n : 256;
-      }
-      cus = cu_count[dev_id];
-    }
-  }
+  const int cus = device_cu_count();
   // one role set per workgroup only when the grid fills every SIMD with several waves anyway
   const bool narrow = B * ceil_div(D, 16) < cus;
   const int ch = narrow ? 8 : 16;

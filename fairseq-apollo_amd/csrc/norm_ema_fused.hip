@@ -40,6 +40,17 @@
 #define MEGA_FTR2(k)
 #endif
 
+// Held-back block starts of a one-round launch: ticks of 10 ns per block index (mod 4), and the least share of the
+// compute units the launch has to fill (1 / MEGA_FUSED_STAGGER_FILL) for them to be used.
+#ifndef MEGA_FUSED_STAGGER
+#define MEGA_FUSED_STAGGER 60
+#endif
+#ifndef MEGA_FUSED_STAGGER_FILL
+#define MEGA_FUSED_STAGGER_FILL 4
+#endif
+#ifndef MEGA_FUSED_STAGGER_BLOCKS
+#define MEGA_FUSED_STAGGER_BLOCKS 4
+#endif
 #ifndef MEGA_FUSED_TWO_TERMS
 #define MEGA_FUSED_TWO_TERMS 0
 #endif
@@ -92,6 +103,7 @@ struct FusedArgs {
   float eps;
   int is_complex;
   int xcd_map;
+  int stagger;           // start of block s held back by (s & 3) * stagger ticks of 10 ns (0: all start at once)
   LookbackLaunch lb;     // status word, poll limit, test hook
 };
 
@@ -182,7 +194,9 @@ __device__ __forceinline__ void lds_cmp(const char* s_tab, int tab, int c, uint3
 // LOUT 0: y as [B, D, L] rows; 1: y as [B, L, D].  GC: channels per norm group, 64 or 128.  A group of 128 channels
 // is shared by two workgroups: each reads the group's whole lines for the moments (both add in the same order, so
 // both arrive at the same statistics to the last bit) and keeps its own 64 channels.
-template <int LOUT, int GC>
+// STAG: the start of block s is held back by s * A.stagger ticks (an instance of its own: the launches that do not
+// hold anything back run the code without the wait).
+template <int LOUT, int GC, bool STAG>
 __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) {
   constexpr int kParts = GC / kFC;
   static_assert(kParts == 1 || kParts == 2, "one or two workgroups per norm group");
@@ -230,6 +244,14 @@ __global__ __launch_bounds__(kFT) void norm_ema_fused_kernel(const FusedArgs A) 
   bool poison = false;
 
   MEGA_FTR(0);
+  // A launch of a single round has every workgroup of the chip asking for its block at the same moment, and every
+  // block after a row's first then waits for the records of the blocks before it.  Blocks 1..3 of every four ask a
+  // little later each (constant 100 MHz clock, a bounded wait): the requests spread out, and the later start is time
+  // the block would have spent waiting for those records.
+  if (STAG && s != 0) {
+    const uint64_t t_end = wall_clock64() + (uint64_t)(s * A.stagger);
+    while (wall_clock64() < t_end) __builtin_amdgcn_s_sleep(4);
+  }
   // ---- everything the norm needs from memory is requested before the block itself
   const Moments prior = {(float)A.prev_count[b], A.prev_mean[brow], A.prev_var[brow]};
   float gam[8], bet[8];
@@ -1011,13 +1033,23 @@ extern "C" int mega_norm_ema_fwd_train(const void* x, void* xn, void* y, int dty
     A.xcd_map = ((G * parts) % 8 == 0) ? 1 : 0;
     A.lb = lookback_launch(true);
     const dim3 grid((unsigned)(B * G * parts * S));
+    // held-back starts only where the launch is one round of workgroups (one per compute unit) and fills most of it
+    const int cus = device_cu_count();
+    A.stagger = (S > 1 && S <= MEGA_FUSED_STAGGER_BLOCKS && (int64_t)grid.x <= cus &&
+                 (int64_t)grid.x * MEGA_FUSED_STAGGER_FILL >= cus * (MEGA_FUSED_STAGGER_FILL - 1))
+                    ? MEGA_FUSED_STAGGER
+                    : 0;
     typedef void (*Kern)(const FusedArgs);
     const int lout = syl == 1 ? 0 : 1;
-    const Kern kerns[2][2] = {{norm_ema_fused_kernel<0, 64>, norm_ema_fused_kernel<1, 64>},
-                              {norm_ema_fused_kernel<0, 128>, norm_ema_fused_kernel<1, 128>}};
-    const Kern kern = kerns[parts - 1][lout];
-    static uint64_t attr_seen[2][2] = {{0, 0}, {0, 0}};
-    if (first_on_device(&attr_seen[parts - 1][lout])) {
+    const Kern kerns[2][2][2] = {
+        {{norm_ema_fused_kernel<0, 64, false>, norm_ema_fused_kernel<0, 64, true>},
+         {norm_ema_fused_kernel<1, 64, false>, norm_ema_fused_kernel<1, 64, true>}},
+        {{norm_ema_fused_kernel<0, 128, false>, norm_ema_fused_kernel<0, 128, true>},
+         {norm_ema_fused_kernel<1, 128, false>, norm_ema_fused_kernel<1, 128, true>}}};
+    const int stag = A.stagger > 0 ? 1 : 0;
+    const Kern kern = kerns[parts - 1][lout][stag];
+    static uint64_t attr_seen[2][2][2] = {{{0, 0}, {0, 0}}, {{0, 0}, {0, 0}}};
+    if (first_on_device(&attr_seen[parts - 1][lout][stag])) {
       (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kFSmem);
     }
     hipLaunchKernelGGL(kern, grid, dim3(kFT), kFSmem, s, A);
