@@ -28,6 +28,7 @@ SIGNATURES = {
     "mega_lookback_status": (_int, [_int]),
     "mega_lookback_checked": (None, [_int]),
     "mega_test_lookback": (None, [C.c_uint, _int, _int]),
+    "mega_test_timestep_norm_bwd_onepass": (None, [_int]),
     "mega_audit_begin": (None, []),
     "mega_audit_add": (_int, [_p, _sz]),
     "mega_audit_end": (_int, [C.POINTER(_int)]),

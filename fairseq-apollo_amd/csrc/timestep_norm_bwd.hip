@@ -20,10 +20,17 @@
 //   3. tsn_bwd_tile_kernel<.., 1>: per tile, the same ds / db again, the walk inside the tile from
 //      its entering pair, then dx;
 //   4. tsn_bwd_param_kernel: sums the per-tile gamma / beta shares.
+// One launch instead of 1 - 3 (tsn_bwd_onepass_kernel: 16-bit activations in 16-byte vectors, at most 16 groups, a
+// tile's dy and x held in registers): every tile publishes its map as tagged words, composes the maps of the tiles
+// behind it in walk order (block records of 32 tiles for rows of more than 128 tiles, bounded waits) and goes on to dx with the dy and
+// x it already holds, so both are read once.
 // Masked tokens are skipped by the walk (identity map, dx = 0).  "Previous cumulative mean" is
 // cummean[t-1]; the forward kernels of this library store the carried mean at masked tokens, so
 // this is the state before token t also behind a masked token.
+#include <atomic>
+
 #include "common.h"
+#include "tsn_common.h"
 
 namespace mega {
 namespace {
@@ -53,6 +60,11 @@ struct TsnBwdParams {
   float* beta_grad;
   int B, L, H, G, Dg, TT, nt;
   RowTiling R;
+  // one-launch form: [B * nt][G][4] tagged words, a tile's map, and [B * nblk][G][4], the map of kOpBlock tiles
+  unsigned long long* rec;
+  unsigned long long* brec;
+  int nblk;
+  LookbackLaunch lb;
 };
 
 struct TileMap { float a, m, bu, bv; };
@@ -399,6 +411,306 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   }
 }
 
+// ---- one launch: tile maps, look-back over the tiles behind, dx
+constexpr int kOpThreads = 512;  // 8 waves; two workgroups share a compute unit (128 registers a lane)
+constexpr int kOpNV = 8;        // 16-byte vectors of dy (and of x) a thread holds
+constexpr int kOpBlock = 32;    // tiles per block record
+constexpr int kOpDirect = 128;  // rows of up to this many tiles look back over the tiles themselves: one stage of
+                                // waiting instead of two
+constexpr uint32_t kOpTag = 1u; // the records are cleared before every launch
+
+__device__ __forceinline__ TileMap shfl32(const TileMap v, int l) {
+  return TileMap{__shfl(v.a, l, 32), __shfl(v.m, l, 32), __shfl(v.bu, l, 32), __shfl(v.bv, l, 32)};
+}
+
+// Workgroups are handed out in the order of their ids, so tile = nt - 1 - id / B: whatever a tile waits for was
+// started before it.  512 threads: for the loads thread = (token of a round, slot of 8 channels), always the same
+// channels; for the walk thread = (group, position in walk order).
+template <typename T>
+__global__ __launch_bounds__(kOpThreads, 4) void tsn_bwd_onepass_kernel(const TsnBwdParams P) {
+  constexpr int VEC = 8;
+  using V = Vec<T, VEC>;
+  extern __shared__ float smem[];
+  const int G = P.G, H = P.H, TT = P.TT, Dg = P.Dg;
+  const int cells = TT * G;
+  float* s_r = smem;
+  float* s_u = s_r + cells;
+  float* s_ux = s_u + cells;
+  float* s_ds = s_ux + cells;    // dux after the walk
+  float* s_db = s_ds + cells;    // dvx after the walk
+  float* s_up0 = s_db + cells;   // [G] cumulative mean before the tile's first token
+  float* s_wg = s_up0 + G;       // [H]
+  float* s_bg = s_wg + H;
+  int* s_mask = (int*)(s_bg + H);   // [TT] + counter of later unmasked tokens + give-up flag
+  const int tid = threadIdx.x;
+  const int ticket = (int)blockIdx.x;
+  const int tile = P.nt - 1 - ticket / P.B;
+  const int b = ticket % P.B;
+  const int t0 = tile * TT;
+  const int ntok = min(TT, P.L - t0);
+  const T* dy = (const T*)P.dy + ((size_t)b * P.L + t0) * H;
+  const T* x = (const T*)P.x + ((size_t)b * P.L + t0) * H;
+
+  // ---- the tile's dy and x are requested first: thread = (token tokb + j * tps, slot)
+  const int slots = P.R.slots, tps = kOpThreads / slots;
+  const int slot = tid % slots, tokb = tid / slots;
+  const int gs = slot >> P.R.lpg_shift;
+  const int cc = gs * Dg + (slot - (gs << P.R.lpg_shift)) * VEC;
+  static_assert(sizeof(V) == 16, "a vector is 16 bytes");
+  uint4 dq[kOpNV], xq[kOpNV];             // kept packed: the values are unpacked where they are used, twice
+#pragma unroll
+  for (int j = 0; j < kOpNV; ++j) {
+    // rounds beyond the tile's last token read that token again: whatever they compute is dropped (no branch here,
+    // so that the sixteen words of a round stay sixteen registers)
+    const int tok = min(tokb + j * tps, ntok - 1);
+    dq[j] = *(const uint4*)(dy + (size_t)tok * H + cc);
+    xq[j] = *(const uint4*)(x + (size_t)tok * H + cc);
+  }
+  float gw[VEC];
+  load_params<VEC>(P.gamma + cc, gw);
+
+  // ---- statistics of the tile, mask, tokens that count after the tile
+  for (int i = tid; i < cells; i += kOpThreads) {
+    const int tok = i / G;
+    if (tok < ntok) {
+      const size_t o = ((size_t)b * P.L + t0) * G + i;
+      s_r[i] = P.cumrstd[o];
+      s_u[i] = P.cummean[o];
+      s_ux[i] = P.group_mean ? P.group_mean[o] : 0.f;
+    }
+  }
+  for (int g = tid; g < G; g += kOpThreads)
+    s_up0[g] = t0 == 0 ? P.prev_mean[(size_t)b * G + g] : P.cummean[((size_t)b * P.L + t0 - 1) * G + g];
+  for (int c = tid; c < H; c += kOpThreads) { s_wg[c] = 0.f; s_bg[c] = 0.f; }
+  if (tid == 0) { s_mask[TT] = 0; s_mask[TT + 1] = 0; }
+  for (int tok = tid; tok < TT; tok += kOpThreads)
+    s_mask[tok] = (tok >= ntok) || (P.mask && P.mask[(size_t)b * P.L + t0 + tok]);
+  __syncthreads();
+  if (P.mask) {
+    int later = 0;   // unmasked tokens behind this tile
+    for (int t = t0 + TT + tid; t < P.L; t += kOpThreads) later += P.mask[(size_t)b * P.L + t] ? 0 : 1;
+    if (later) atomicAdd(&s_mask[TT], later);
+  }
+
+  // ---- ds, db (and the group mean when it was not handed in) per (token, group)
+#pragma unroll
+  for (int j = 0; j < kOpNV; ++j) {
+    int tok = tokb + j * tps;
+    asm volatile("" : "+v"(tok));
+    const bool live = tok < ntok;
+    const int cell = live ? tok * G + gs : gs;
+    const float u_ = s_u[cell];
+    float ds = 0.f, db = 0.f, sx = 0.f;
+    asm volatile("" : "+v"(dq[j].x), "+v"(dq[j].y), "+v"(dq[j].z), "+v"(dq[j].w));
+    asm volatile("" : "+v"(xq[j].x), "+v"(xq[j].y), "+v"(xq[j].z), "+v"(xq[j].w));
+    const V dvj = __builtin_bit_cast(V, dq[j]), xvj = __builtin_bit_cast(V, xq[j]);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float d = to_float(dvj.v[e]), xe = to_float(xvj.v[e]), w = gw[e];
+      ds = fmaf(d * (xe - u_), w, ds);
+      db = fmaf(d, w, db);
+      sx += xe;
+    }
+    for (int o = 1; o < P.R.LPG; o <<= 1) {
+      ds += __shfl_xor(ds, o);
+      db += __shfl_xor(db, o);
+      sx += __shfl_xor(sx, o);
+    }
+    if (live && slot == (gs << P.R.lpg_shift)) {
+      s_ds[cell] = ds;
+      s_db[cell] = db;
+      if (!P.group_mean) s_ux[cell] = sx / (float)Dg;
+    }
+    __builtin_amdgcn_sched_barrier(0);      // one token's temporaries at a time: the tile itself fills half the registers
+  }
+  __syncthreads();
+
+  // ---- every token's map and the scan over the positions: 32 lanes per group, lane = position in walk order
+  {
+  const int64_t n_end = P.count[b] - (P.mask ? s_mask[TT] : max(0, P.L - t0 - TT));
+  const int pos = tid & 31, grp = tid >> 5;
+  const bool valid = grp < G;
+  const int g = valid ? grp : 0;
+  const int tok = ntok - 1 - pos;
+  const bool has = valid && tok >= 0 && !s_mask[max(tok, 0)];
+  const unsigned long long bal = __ballot(has);
+  const unsigned half = (unsigned)(bal >> (tid & 32));
+  const int64_t n = n_end - __popc(half & ((1u << pos) - 1u));
+  const int cell = max(tok, 0) * G + g;
+  float c2 = 0.f, e = 0.f, rdb = 0.f, mj = 0.f;
+  TileMap own{1.f, 0.f, 0.f, 0.f};
+  if (has) {
+    c2 = 1.0f / (float)n;
+    const float c1 = (float)(n - 1) * c2;
+    const float r = s_r[cell];
+    const float up = tok == 0 ? s_up0[g] : s_u[cell - G];
+    const float delta = s_ux[cell] - up;
+    e = 0.5f * r * r * r * s_ds[cell];
+    rdb = r * s_db[cell];
+    mj = -2.0f * c1 * c2 * delta;
+    own = TileMap{c1, mj, -c1 * rdb - mj * e, -c1 * e};
+  }
+  TileMap inc = own;
+#pragma unroll
+  for (int o = 1; o < 32; o <<= 1) {
+    const TileMap prev = shfl_up32(inc, o);
+    if (pos >= o) inc = then(prev, inc);
+  }
+  TileMap exc = shfl_up32(inc, 1);
+  if (pos == 0) exc = TileMap{1.f, 0.f, 0.f, 0.f};
+  const TileMap tmap = shfl32(inc, 31);           // the tile's map, in every lane of the group
+
+  // ---- publish it (lanes 0..3 of the group: one word each)
+  auto word_of = [&](const TileMap& m_) -> uint32_t {
+    return __float_as_uint(pos == 0 ? m_.a : pos == 1 ? m_.m : pos == 2 ? m_.bu : m_.bv);
+  };
+  if (valid && pos < 4 && !(P.lb.withhold_first && tile == P.nt - 1))
+    put_rec(P.rec + (((size_t)b * P.nt + tile) * G + g) * 4 + pos, tagged(word_of(tmap), kOpTag));
+
+  // ---- the maps of everything behind the tile, in walk order: the later blocks from the row's last one down, then
+  // the later tiles of the tile's own block.  Lane i of a group fetches record i of a round of 32; the round is
+  // composed in order by a scan over the lanes.
+  const bool blocks = P.nt > kOpDirect;
+  const int lbb = blocks ? kOpBlock : P.nt;
+  const int kb = tile / lbb;
+  const int bend = min(P.nt, (kb + 1) * lbb);     // one past the block's last tile
+  const int nb = blocks ? P.nblk - 1 - kb : 0;    // later blocks
+  const int nown = bend - 1 - tile;               // later tiles of the own block
+  bool gave = false;
+  auto fetch = [&](const int i0, const int i1) -> TileMap {
+    TileMap acc{1.f, 0.f, 0.f, 0.f};
+    for (int r0 = i0; r0 < i1; r0 += 32) {
+      const int i = r0 + pos;
+      TileMap v{1.f, 0.f, 0.f, 0.f};
+      if (valid && i < i1) {
+        const unsigned long long* src =
+            i < nb ? P.brec + (((size_t)b * P.nblk + (P.nblk - 1 - i)) * G + g) * 4
+                   : P.rec + (((size_t)b * P.nt + (bend - 1 - (i - nb))) * G + g) * 4;
+        // the four words are asked for together; those that are not there yet are asked for again together
+        unsigned long long w[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) w[u] = get_rec(src + u);
+        uint32_t spins = 0;
+        for (;;) {
+          bool pending = false;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) pending |= (uint32_t)(w[u] >> 32) != kOpTag;
+          if (!pending) break;
+          if (++spins > P.lb.spin_limit) {
+            gave = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if ((uint32_t)(w[u] >> 32) != kOpTag) w[u] = get_rec(src + u);
+        }
+        v = TileMap{__uint_as_float((uint32_t)w[0]), __uint_as_float((uint32_t)w[1]), __uint_as_float((uint32_t)w[2]),
+                    __uint_as_float((uint32_t)w[3])};
+      }
+      TileMap sc = v;
+#pragma unroll
+      for (int o = 1; o < 32; o <<= 1) {
+        const TileMap prev = shfl_up32(sc, o);
+        if (pos >= o) sc = then(prev, sc);
+      }
+      acc = then(acc, shfl32(sc, 31));
+    }
+    return acc;
+  };
+  // a group whose wait gave up: every lane of the group knows (and nothing is built on the missing words)
+  auto group_gave = [&]() -> bool {
+    const unsigned long long gb = __ballot(gave);
+    return ((unsigned)(gb >> (tid & 32))) != 0u;
+  };
+  const TileMap own_blk = fetch(nb, nb + nown);
+  bool lost = group_gave();
+  if (blocks && tile == kb * lbb && valid && pos < 4 && !lost)
+    put_rec(P.brec + (((size_t)b * P.nblk + kb) * G + g) * 4 + pos, tagged(word_of(then(own_blk, tmap)), kOpTag));
+  const TileMap ent = then(fetch(0, nb), own_blk);
+  lost = group_gave();
+  if (lost && pos == 0) {
+    s_mask[TT + 1] = 1;
+    if (P.lb.status) __hip_atomic_store(P.lb.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+
+  // ---- the pair that enters the tile, the pairs at its tokens, dux / dvx
+  const float u0 = P.mean_grad ? P.mean_grad[(size_t)b * G + g] : 0.f;
+  const float v0 = P.var_grad ? P.var_grad[(size_t)b * G + g] : 0.f;
+  float ug0 = fmaf(ent.a, u0, fmaf(ent.m, v0, ent.bu));
+  const float vg0 = fmaf(ent.a, v0, ent.bv);
+  if (lost) ug0 = __builtin_nanf("");
+  if (valid && tok >= 0) {
+    const float ug = fmaf(exc.a, ug0, fmaf(exc.m, vg0, exc.bu));
+    const float vg = fmaf(exc.a, vg0, exc.bv);
+    const float du = ug - rdb, dv = vg - e;
+    s_ds[cell] = has ? c2 * du - mj * dv : 0.f;      // dux
+    s_db[cell] = has ? c2 * dv : 0.f;                // dvx
+  }
+  if (tile == 0 && valid && pos == 31) {
+    const TileMap full = then(ent, tmap);
+    const size_t i = (size_t)b * G + g;
+    P.prev_mean_grad[i] = lost ? __builtin_nanf("") : fmaf(full.a, u0, fmaf(full.m, v0, full.bu));
+    P.prev_var_grad[i] = lost ? __builtin_nanf("") : fmaf(full.a, v0, full.bv);
+  }
+  }
+  __syncthreads();
+
+  // ---- dx from the dy and x the thread holds, and the thread's gamma / beta shares (always the same channels)
+  float rw[VEC], rb[VEC];
+#pragma unroll
+  for (int q = 0; q < VEC; ++q) { rw[q] = 0.f; rb[q] = 0.f; }
+  {
+    // the channels' weights again (out of the cache) rather than eight registers held across the look-back
+    const float* gp = P.gamma + cc;
+    asm volatile("" : "+v"(gp));
+    load_params<VEC>(gp, gw);
+    T* dx = (T*)P.dx + ((size_t)b * P.L + t0) * H;
+    const float cg = 1.0f / (float)Dg;
+    const bool poison = s_mask[TT + 1] != 0;
+#pragma unroll
+    for (int j = 0; j < kOpNV; ++j) {
+      int tk = tokb + j * tps;
+      asm volatile("" : "+v"(tk));      // addresses and cells are formed again here, not kept from the loads
+      // the packed words are taken as they are (no unpacked copy is carried over from the first use)
+      asm volatile("" : "+v"(dq[j].x), "+v"(dq[j].y), "+v"(dq[j].z), "+v"(dq[j].w));
+      asm volatile("" : "+v"(xq[j].x), "+v"(xq[j].y), "+v"(xq[j].z), "+v"(xq[j].w));
+      const V dvj = __builtin_bit_cast(V, dq[j]), xvj = __builtin_bit_cast(V, xq[j]);
+      if (tk < ntok) {
+        const int cl = tk * G + gs;
+        const float r = s_r[cl], ux = s_ux[cl], um = s_u[cl];
+        const float a0 = s_ds[cl] * cg, a1 = 2.0f * s_db[cl] * cg;
+        const bool keep = !s_mask[tk];
+        V o;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) {
+          const float d = to_float(dvj.v[q]), xe = to_float(xvj.v[q]);
+          float v = fmaf(d * r, gw[q], fmaf(a1, xe - ux, a0));
+          if (poison) v = __builtin_nanf("");
+          o.v[q] = from_float<T>(keep ? v : 0.f);
+          if (keep) {
+            rw[q] = fmaf(d * (xe - um), r, rw[q]);
+            rb[q] += d;
+          }
+        }
+        *(V*)(dx + (size_t)tk * H + cc) = o;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- the tile's share of the gamma / beta gradients: the threads of one slot add up in a fixed order
+  for (int turn = 0; turn < tps; ++turn) {
+    if (tokb == turn) {
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) { s_wg[cc + q] += rw[q]; s_bg[cc + q] += rb[q]; }
+    }
+    __syncthreads();
+  }
+  float* dst = P.part + ((size_t)b * P.nt + tile) * 2 * H;
+  for (int c = tid; c < H; c += kOpThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
+}
+
 // One wave per (row, group).  The tiles are walked from the last to the first; lane l owns the
 // l-th run of `per` tiles in that order, composes its run, the runs are combined by a scan over
 // the lanes, and every lane then replays its run from the pair that enters it.
@@ -479,7 +791,13 @@ __global__ __launch_bounds__(256) void tsn_bwd_param_kernel(const TsnBwdParams P
 struct BwdGeom {
   int tt, nt, vec;
   size_t agg_bytes, state_bytes, part_bytes;
+  // the one-launch form (onepass): its own tile length and records
+  bool onepass;
+  int op_tt, op_nt, op_nblk;
+  size_t op_rec_bytes, op_brec_bytes, op_part_bytes;
 };
+
+std::atomic<int> g_onepass{1};     // test hook: 0 keeps every call on the three-pass form
 
 bool bwd_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, BwdGeom* g) {
   if (G > kMaxTileCells || H > 8192 || B * L >= (int64_t)1 << 31) return false;
@@ -495,7 +813,34 @@ bool bwd_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, BwdGeom
   g->agg_bytes = align_up((size_t)B * g->nt * G * 16, 256);
   g->state_bytes = align_up((size_t)B * g->nt * G * 8, 256);
   g->part_bytes = align_up((size_t)B * g->nt * 2 * H * 4, 256);
+  // one launch: 16-bit activations as 16-byte vectors, one vector per lane and token, at most 16 groups, and a tile
+  // of at most kOpNV rounds of the workgroup's threads
+  g->onepass = false;
+  g->op_rec_bytes = g->op_brec_bytes = g->op_part_bytes = 0;
+  if (dtype != MEGA_F32 && g->vec == 8 && G <= 16) {
+    const RowTiling R = make_row_tiling(G, Dg, 8);
+    if (R.PER == 1 && R.slots <= kOpThreads && kOpThreads % R.slots == 0) {
+      const int per_round = kOpThreads / R.slots;
+      const int ott = per_round * kOpNV < 32 ? per_round * kOpNV : 32;
+      const int64_t ont = ceil_div(L, ott);
+      if (ott >= 8 && B * ont < (int64_t)1 << 31) {
+        g->onepass = true;
+        g->op_tt = ott;
+        g->op_nt = (int)ont;
+        g->op_nblk = ont > kOpDirect ? (int)ceil_div(ont, kOpBlock) : 0;
+        g->op_rec_bytes = align_up((size_t)B * ont * G * 32, 256);
+        g->op_brec_bytes = align_up((size_t)B * g->op_nblk * G * 32, 256);
+        g->op_part_bytes = align_up((size_t)B * ont * 2 * H * 4, 256);
+      }
+    }
+  }
   return true;
+}
+
+size_t bwd_workspace_need(const BwdGeom& g) {
+  const size_t three = g.agg_bytes + g.state_bytes + g.part_bytes;
+  const size_t one = g.op_rec_bytes + g.op_brec_bytes + g.op_part_bytes;
+  return three > one ? three : one;
 }
 
 template <typename T, int VEC>
@@ -529,6 +874,26 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
 }
 
 template <typename T>
+int launch_onepass(const TsnBwdParams& P, size_t rec_bytes, hipStream_t s) {
+  if constexpr (sizeof(T) != 2) {
+    return MEGA_ERR_UNSUPPORTED;
+  } else {
+    const size_t cells = (size_t)P.TT * P.G;
+    const size_t lds = (5 * cells + P.G + 2 * (size_t)P.H) * 4 + (P.TT + 2) * 4;
+    static uint64_t seen = 0;
+    if (first_on_device(&seen))
+      (void)hipFuncSetAttribute((const void*)tsn_bwd_onepass_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024);
+    zero_async(P.rec, rec_bytes, s);       // tile and block records (one range): no word carries the tag
+    hipLaunchKernelGGL((tsn_bwd_onepass_kernel<T>), dim3((unsigned)(P.B * P.nt)), dim3(kOpThreads), lds, s, P);
+    MEGA_CHECK_LAUNCH("timestep_norm_bwd (one launch)");
+    hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 32)), dim3(256), 0, s, P);
+    MEGA_CHECK_LAUNCH("timestep_norm_bwd (parameters)");
+    return MEGA_OK;
+  }
+}
+
+template <typename T>
 int launch_bwd(const TsnBwdParams& P, int vec, hipStream_t s) {
   constexpr int FULL = 16 / (int)sizeof(T);
   return vec == FULL ? launch_tiles<T, FULL>(P, s) : launch_tiles<T, 1>(P, s);
@@ -542,8 +907,10 @@ using namespace mega;
 extern "C" size_t mega_timestep_norm_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G) {
   BwdGeom g;
   if (B <= 0 || L <= 0 || H <= 0 || G <= 0 || H % G != 0 || !bwd_geometry(dtype, B, L, H, G, &g)) return 256;
-  return g.agg_bytes + g.state_bytes + g.part_bytes;
+  return bwd_workspace_need(g);
 }
+
+extern "C" void mega_test_timestep_norm_bwd_onepass(int on) { g_onepass.store(on ? 1 : 0); }
 
 extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,
                                             const void* x, int dtype, const float* prev_mean, const int64_t* count,
@@ -579,11 +946,45 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
                kMaxTileCells);
   if (g.vec > 1 && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad | (uintptr_t)gamma) % 16) != 0))
     g.vec = 1;                             // element-wise tiling when a buffer is not 16-byte aligned
-  const size_t need = g.agg_bytes + g.state_bytes + g.part_bytes;
+  const size_t need = bwd_workspace_need(g);
   MEGA_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, MEGA_ERR_WORKSPACE,
                "timestep_norm_bwd: workspace of %zu bytes (16-byte aligned) needed", need);
   char* w = (char*)workspace;
   TsnBwdParams P;
+  const bool onepass = g.onepass && g.vec == 8 && g_onepass.load() != 0;
+  if (onepass) {
+    if (!audit_on())
+      if (const int rc = lookback_pending("timestep_norm_bwd")) return rc;
+    P.dy = y_grad; P.x = x; P.dx = x_grad; P.mean_grad = mean_grad; P.var_grad = var_grad; P.prev_mean = prev_mean;
+    P.count = count; P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd; P.gamma = gamma; P.mask = mask;
+    P.agg = nullptr; P.state = nullptr;
+    P.rec = (unsigned long long*)w; w += g.op_rec_bytes;
+    P.brec = (unsigned long long*)w; w += g.op_brec_bytes;
+    P.part = (float*)w;
+    P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
+    P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = (int)(H / G); P.TT = g.op_tt; P.nt = g.op_nt;
+    P.nblk = g.op_nblk;
+    P.R = make_row_tiling(G, H / G, 8);
+    if (audit_on()) {
+      // per (row, tile, group) and per (row, block of tiles, group): one map of four tagged words; per (row, tile): the
+      // tile's share of the gamma / beta gradients, 2 H floats
+      audit_use(P.rec, (size_t)B * g.op_nt * G * 32, "timestep_norm_bwd: tile records");
+      if (g.op_nblk) audit_use(P.brec, (size_t)B * g.op_nblk * G * 32, "timestep_norm_bwd: block records");
+      else audit_use(P.rec, 32, "timestep_norm_bwd: block records (none)");
+      audit_use(P.part, (size_t)B * g.op_nt * 2 * H * 4, "timestep_norm_bwd: parameter-gradient shares");
+      audit_use(y_grad, (size_t)B * L * H * 2, "timestep_norm_bwd: y_grad");
+      audit_use(x, (size_t)B * L * H * 2, "timestep_norm_bwd: x");
+      audit_use(x_grad, (size_t)B * L * H * 2, "timestep_norm_bwd: x_grad");
+      audit_use(cummean, (size_t)B * L * G * 4, "timestep_norm_bwd: cummean");
+      audit_use(cumrstd, (size_t)B * L * G * 4, "timestep_norm_bwd: cumrstd");
+      return MEGA_OK;
+    }
+    P.lb = lookback_launch(true);
+    const int rc = dtype == MEGA_BF16 ? launch_onepass<bf16_t>(P, g.op_rec_bytes + g.op_brec_bytes, s)
+                                      : launch_onepass<f16_t>(P, g.op_rec_bytes + g.op_brec_bytes, s);
+    return rc != MEGA_OK ? rc : lookback_verify("timestep_norm_bwd", s);
+  }
+  P.rec = nullptr; P.brec = nullptr; P.nblk = 0; P.lb = LookbackLaunch{nullptr, 0u, 0};
   P.dy = y_grad; P.x = x; P.dx = x_grad; P.mean_grad = mean_grad; P.var_grad = var_grad; P.prev_mean = prev_mean;
   P.count = count; P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd; P.gamma = gamma; P.mask = mask;
   P.agg = (float*)w; w += g.agg_bytes;

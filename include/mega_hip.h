@@ -87,6 +87,12 @@ void mega_lookback_checked(int on);
  * status word of the current device from the host.  Not for production use.                         */
 void mega_test_lookback(unsigned spin_limit, int withhold_first, int raise);
 
+/* Test hook: on == 0 keeps mega_(group_)timestep_norm_bwd on its three-pass form (tile maps, carry, dx) also where
+ * the one-launch form with its look-back over the later tiles would run (16-bit activations in 16-byte vectors, at
+ * most 16 groups); on != 0 (the default) restores the choice.  For tests that compare the two forms; no counterpart
+ * in the reference.                                                                                   */
+void mega_test_timestep_norm_bwd_onepass(int on);
+
 /* Address audit (host only, nothing is launched, no GPU needed; no counterpart in the reference).  Between
  * mega_audit_begin() and mega_audit_end() the calling thread's calls to mega_attention_bwd, mega_gate_qk_bwd,
  * mega_ema_param_grad and mega_(group_)timestep_norm_bwd launch nothing: for every launch they would make they
@@ -419,7 +425,15 @@ int mega_group_timestep_norm_fwd_noalloc(const void* x, void* y, int dtype,
  *   recomputed from x), cummean, cumrstd [B,L,G] fp32 as the forward wrote them (at a masked
  *   token cummean must hold the carried mean, which is what this library's forward stores);
  *   gamma [H] fp32 (weight + 1).  Outputs: x_grad, prev_mean_grad, prev_var_grad [B,G],
- *   gamma_grad, beta_grad [H] fp32.  The per-feature form has H in place of G.           */
+ *   gamma_grad, beta_grad [H] fp32.  The per-feature form has H in place of G.
+ *   bf16 / fp16 activations whose groups are whole 16-byte vectors (one vector per lane), with at
+ *   most 16 groups, run as ONE launch that reads y_grad and x once: every tile of 32 (or 16)
+ *   tokens publishes its map of the carried pair (u_grad, v_grad) and composes the maps of the
+ *   tiles behind it with bounded waits, like the forward's look-back.  A wait that gives up leaves
+ *   NaN in x_grad / prev_mean_grad / prev_var_grad and is reported like the forward's: the next
+ *   call returns MEGA_ERR_LAUNCH (mega_lookback_status, checked mode: the same call).  Everything
+ *   else takes three passes (tile maps, carry, x_grad) without waits.  The workspace needs no
+ *   initialisation and nothing in it survives the call (the records are cleared by the call). */
 size_t mega_timestep_norm_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G);
 int mega_group_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,
                                  const void* x, int dtype, const float* prev_mean,

@@ -61,6 +61,50 @@ def test_timestep_norm_bwd(dtype, B, L, H, G, masked, prior):
         assert rel_err(host(a), b) < 2e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,L,H,G,masked,prior,saved_gm", [
+    (4, 4096, 1024, 16, False, False, True),    # the headline geometry: 128 tiles a row, block records of 16 tiles
+    (2, 2000, 1024, 16, True, True, False),     # ragged last tile, padding, carried statistics, group means formed again
+    (1, 8192, 2048, 16, False, True, True),     # 128 channels per group: tiles of 16 tokens, 512 tiles a row
+    (3, 700, 128, 16, True, False, True),       # one vector per group, 22 tiles: look-back over the tiles themselves
+    (2, 1030, 256, 2, True, True, False),       # two groups of 128 channels
+    (5, 31, 64, 1, False, True, True),          # a single partial tile
+])
+def test_timestep_norm_bwd_one_launch(dtype, B, L, H, G, masked, prior, saved_gm):
+    """The one-launch form (every tile composes the maps of the tiles behind it) against the three-pass form on the
+    same inputs, and against the oracle where that is quick."""
+    print(f"case {dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior} saved_gm={saved_gm}", flush=True)
+    rng = np.random.default_rng(53)
+    x, x64, dy, dy64, mask, pc, pm, pv, gamma, beta, dm, dv = _tsn_case(rng, B, L, H, G, masked, prior, dtype)
+    tm = None if mask is None else torch.from_numpy(mask).to(DEV)
+    y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma),
+                                                                dev(beta), tm, G, 1e-5)
+    run = lambda: M.ops.group_timestep_norm_bwd(dy, dev(dm), dev(dv), x, dev(pm), cnt, gm if saved_gm else None, cm, cr,
+                                                dev(gamma), tm, G)
+    lib = M._lib.load()
+    one = run()
+    torch.cuda.synchronize()
+    assert M.ops.lookback_status() == 0
+    lib.mega_test_timestep_norm_bwd_onepass(0)
+    try:
+        three = run()
+        torch.cuda.synchronize()
+    finally:
+        lib.mega_test_timestep_norm_bwd_onepass(1)
+    assert not torch.isnan(one[0].float()).any()
+    # fp32 walks composed in another order, dx rounded once to the activation type: the odd last-bit difference
+    assert rel_err(host(one[0]), host(three[0])) < 1e-2
+    assert (one[0] != three[0]).float().mean().item() < 0.02
+    for a, b_ in zip(one[1:], three[1:]):
+        assert rel_err(host(a), host(b_)) < 1e-4
+    if B * L * H <= 2 * 2000 * 1024:
+        ocnt, ogm, ocm, ocr = O.timestep_norm_saved(x64, pc, pm, pv, mask, G, 1e-5)
+        ref = O.timestep_norm_bwd(dy64, dm, dv, x64, pm, ocnt, ogm, ocm, ocr, gamma, mask, G)
+        assert rel_err(host(one[0]), ref[0]) < TOL[dtype]
+        for a, b_ in zip(one[1:], ref[1:]):
+            assert rel_err(host(a), b_) < 3e-4
+
+
 def test_timestep_norm_bwd_zero_upstream_state_grads():
     rng = np.random.default_rng(52)
     x, x64, dy, dy64, mask, pc, pm, pv, gamma, beta, _, _ = _tsn_case(rng, 2, 40, 32, 4, False, True, torch.float32)

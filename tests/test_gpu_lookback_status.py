@@ -95,6 +95,42 @@ def test_one_kernel_block_that_gives_up(hooks):
     assert M.ops.lookback_status() == 0
 
 
+@pytest.mark.parametrize("L", [4096, 8192])
+def test_norm_backward_tile_that_gives_up(hooks, L):
+    """The one-launch TimestepNorm backward walks a row from its last tile to its first: with the row's last tile
+    publishing nothing, every other tile gives up (4096 tokens: 128 tiles that look back over the tiles themselves;
+    8192: block records, which a block's first tile withholds when it gave up itself)."""
+    lib = hooks
+    B, D, G = 2, 1024, 16
+    torch.manual_seed(64)
+    x = torch.randn(B, L, D, device=DEV).to(BF)
+    dy = torch.randn(B, L, D, device=DEV).to(BF)
+    gamma, beta = torch.ones(D, device=DEV), torch.zeros(D, device=DEV)
+    y, cnt, mu, var, gm, cm, cr = M.ops.group_timestep_norm_fwd(x, *_state(B, G), gamma, beta, None, G, 1e-5)
+    pm = torch.zeros(B, G, device=DEV)
+    run = lambda: M.ops.group_timestep_norm_bwd(dy, None, None, x, pm, cnt, gm, cm, cr, gamma, None, G)
+    good = run()
+    torch.cuda.synchronize()
+    print("forced give-up: group_timestep_norm_bwd", flush=True)
+    lib.mega_test_lookback(64, 1, 0)
+    bad = run()
+    torch.cuda.synchronize()
+    lib.mega_test_lookback(0, 0, 0)
+    nan_tok = torch.isnan(bad[0].float()).any(-1)                # [B, L]
+    assert nan_tok[:, :L - 32].all() and not nan_tok[:, L - 32:].any()
+    assert torch.equal(bad[0][:, L - 32:], good[0][:, L - 32:])   # the last tile waits for nobody
+    assert torch.isnan(bad[1]).all() and torch.isnan(bad[2]).all()
+    assert M.ops.lookback_status() == 1
+    with pytest.raises(RuntimeError, match="gave up"):
+        run()
+    assert M.ops.lookback_status() == 0
+    again = run()
+    torch.cuda.synchronize()
+    for a, b_ in zip(again, good):
+        assert torch.equal(a, b_)
+    assert M.ops.lookback_status() == 0
+
+
 def test_checked_mode_reports_the_give_up_of_the_same_call(hooks):
     """With checked mode on, the call whose launch gave up raises itself (after waiting for its stream); nothing is
     left over for the next call."""
