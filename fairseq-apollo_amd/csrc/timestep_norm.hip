@@ -126,13 +126,10 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   V xv[kNV];
 #pragma unroll
   for (int j = 0; j < kNV; ++j) {
-    const int v = j * kThreads + tid;
-    if (v < nvec) {
-      xv[j] = xin[v];
-    } else {
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) xv[j].v[i] = from_float<T>(0.f);
-    }
+    // vectors beyond the tile read its last one again and whatever is computed from them is dropped: a branch here
+    // makes the compiler carry a vector of 16-bit values as separate registers from the load on
+    const int v = min(j * kThreads + tid, nvec - 1);
+    xv[j] = xin[v];
   }
   for (int t = tid; t < nt; t += kThreads)
     s_mask[t] = P.mask ? (P.mask[(size_t)b * P.L + t0 + t] != 0) : 0;
@@ -233,12 +230,8 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
   const size_t trow = (size_t)b * P.ntiles;
   const bool last_tile = tile == P.ntiles - 1;
   const int W = 2 * G + 1;                          // words per tile record
-  const int RT = kLbWords / W;                      // earlier tiles per look-back round
-  for (int gbase = 0; gbase < G; gbase += 16) {
-    const int g = gbase + row16;
-    const bool active = g < G;
-    const int gc = active ? g : G - 1;
-    Moments pref[4];
+  // the tile's own statistics of a set of 16 groups: every lane's prefixes over its tokens, the row's scan
+  auto own_scan = [&](const int gc, const bool active, const int g, const bool first_pass, Moments (&pref)[4]) -> Moments {
     Moments st = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -246,14 +239,41 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       if (u < TPL && tok < nt) {
         const float gm = s_mean[tok * G + gc];
         const float gv = s_var[tok * G + gc];
-        if (P.group_mean && active) P.group_mean[((size_t)b * P.L + t0 + tok) * G + g] = gm;
+        if (first_pass && P.group_mean && active) P.group_mean[((size_t)b * P.L + t0 + tok) * G + g] = gm;
         if (!s_mask[tok]) st = merge(st, Moments{1.f, gm, gv});
       }
       pref[u] = st;
     }
-    const Moments inc = row_scan(st);
+    return row_scan(st);
+  };
+  // With more than 16 groups the aggregates of all of them are published before the first look-back: a tile that
+  // waited for the earlier tiles' first 16 groups before publishing its own next 16 would make the row a chain.
+  if (G > 16) {
+    for (int gbase = 0; gbase < G; gbase += 16) {
+      const int g = gbase + row16;
+      const bool active = g < G;
+      Moments pref[4];
+      const Moments inc = own_scan(active ? g : G - 1, active, g, true, pref);
+      if (l16 == 15 && active && !(P.lb.withhold_first && tile == 0)) {
+        unsigned long long* mine = P.rec + (trow + tile) * W;
+        put_rec(mine + 1 + 2 * g, tagged(__float_as_uint(inc.mean), tag));
+        put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(inc.var), tag));
+        if (g == 0) put_rec(mine, tagged((uint32_t)inc.n, tag));
+      }
+    }
+  }
+  for (int gbase = 0; gbase < G; gbase += 16) {
+    const int g = gbase + row16;
+    const bool active = g < G;
+    const int gc = active ? g : G - 1;
+    // a look-back fetches the count word and the words of this set of groups only
+    const int wlo = 1 + 2 * gbase;                    // first group word of the set
+    const int WS = min(32, W - wlo) + 1;              // words per record staged: count + the set's
+    const int RT = kLbWords / WS;                     // earlier tiles per look-back round
+    Moments pref[4];
+    const Moments inc = own_scan(gc, active, g, G <= 16, pref);
     const Moments exc = dpp_m<0x111>(inc);          // exclusive: what the lanes before this one hold
-    if (l16 == 15 && active && !(P.lb.withhold_first && tile == 0)) {
+    if (G <= 16 && l16 == 15 && active && !(P.lb.withhold_first && tile == 0)) {
       unsigned long long* mine = P.rec + (trow + tile) * W;
       put_rec(mine + 1 + 2 * g, tagged(__float_as_uint(inc.mean), tag));
       put_rec(mine + 2 + 2 * g, tagged(__float_as_uint(inc.var), tag));
@@ -267,7 +287,7 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
     const int nprev = kblk + itile;
     const unsigned long long* bsrc = P.brec + (size_t)b * P.nblk * W;
     const unsigned long long* tsrc = P.rec + (trow + (size_t)kblk * lbb) * W;
-    const int nwb = kblk * W;                         // words of the block records
+    const int nrb = kblk;                             // block records come first in the list
     Moments accB = {0.f, 0.f, 0.f}, accT = {0.f, 0.f, 0.f};
     uint32_t prevcnt = 0;
     auto fetch = [&](const int r0, const int r1) {      // records r0 .. r1 - 1 of the list
@@ -277,11 +297,12 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       {
         // all loads of a batch are issued before the first one is looked at
         constexpr int kBatch = 8;
-        const int w0 = p0 * W;                        // first word of this pass in the list of all records
-        const int nw = np * W;
+        const int nw = np * WS;                       // staged words of this pass
         auto word = [&](const int i) -> const unsigned long long* {
-          const int gw = w0 + i;
-          return gw < nwb ? bsrc + gw : tsrc + (gw - nwb);
+          const int r = i / WS, k = i - r * WS;       // record of the pass, word of the staged record
+          const int rec = p0 + r;                     // record in the list of all records
+          const int wsrc = k == 0 ? 0 : wlo + k - 1;
+          return (rec < nrb ? bsrc + (size_t)rec * W : tsrc + (size_t)(rec - nrb) * W) + wsrc;
         };
         for (int i0 = tid; i0 < nw; i0 += kThreads * kBatch) {
           unsigned long long w[kBatch];
@@ -318,12 +339,12 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       }
       __syncthreads();
       for (int i = l16; i < np; i += 16) {
-        const unsigned long long* rw = s_lbw + i * W;
+        const unsigned long long* rw = s_lbw + i * WS;
         const uint32_t c = (uint32_t)rw[0];
         Moments a;
         a.n = (float)c;
-        a.mean = __uint_as_float((uint32_t)rw[1 + 2 * gc]);
-        a.var = __uint_as_float((uint32_t)rw[2 + 2 * gc]);
+        a.mean = __uint_as_float((uint32_t)rw[1 + 2 * (gc - gbase)]);
+        a.var = __uint_as_float((uint32_t)rw[2 + 2 * (gc - gbase)]);
         if (p0 + i < kblk) accB = merge(accB, a);
         else accT = merge(accT, a);
         prevcnt += c;

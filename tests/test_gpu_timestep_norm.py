@@ -52,6 +52,38 @@ def test_group_matches_oracle(dtype, B, L, H, G, masked, prior):
         assert rel_err(host(out[4]), x64.reshape(B, L, G, -1).mean(-1)) < 1e-4
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,H,G,masked,prior", [(2, 3000, 256, 32, True, True), (1, 2100, 384, 48, False, False),
+                                                  (2, 1500, 512, 256, True, False), (1, 9000, 128, 64, False, True)])
+def test_more_than_sixteen_groups_over_many_tiles(dtype, B, L, H, G, masked, prior):
+    """Groups are handled 16 at a time.  Every set's aggregates are published before the first look-back (a tile does
+    not wait for the earlier tiles with its later sets still unpublished), and a look-back reads only its set's words
+    of the records; 9000 tokens: block records as well.  Also a bound on the time, which a row that turned into a
+    chain of tiles misses by two orders of magnitude."""
+    print(f"case dtype={dtype} B={B} L={L} H={H} G={G} masked={masked} prior={prior}", flush=True)
+    x, x64, mask, pc, pm, pv, gamma, beta = _case(11, B, L, H, G, dtype, masked, prior)
+    run = lambda: M.ops.group_timestep_norm_fwd(x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gamma), dev(beta),
+                                                None if mask is None else dev(mask, torch.bool), G, 1e-5)
+    out = run()
+    torch.cuda.synchronize()
+    assert M.ops.timestep_norm_status() == 0
+    y, c, mu, v = O.timestep_norm(x64, pc, pm, pv, gamma, beta, mask, G, 1e-5)
+    assert rel_err(host(out[0]), y) < TOL[dtype]
+    assert np.array_equal(host(out[1]), c)
+    assert rel_err(host(out[2]), mu) < 1e-4 and rel_err(host(out[3]), v) < 1e-4
+    if not prior and mask is None:
+        _, muc, varc = O.timestep_norm_closed_form(x64, mask, G)
+        assert rel_err(host(out[5]), muc) < 1e-4
+        assert rel_err(host(out[6]), 1 / np.sqrt(varc + 1e-5)) < 1e-4
+    a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(5):
+        run()
+    b_.record()
+    torch.cuda.synchronize()
+    assert a.elapsed_time(b_) / 5 < 2.0, "milliseconds per call"
+
+
 def test_chunked_streaming_equals_one_shot():
     rng = np.random.default_rng(5)
     B, L, H, G = 2, 256, 128, 8
