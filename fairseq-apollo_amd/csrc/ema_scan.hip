@@ -1389,7 +1389,11 @@ extern "C" int mega_ema_fwd(const void* x, void* y, int dtype, int64_t sxb, int6
     return ema_rows_run(x, y, dtype, sxb, sxd, syb, syd, img, is_complex, omega, mask, h_in, h_out, B, D, N, L,
                         bidirectional, acc, (float*)(wimg + pl.image_bytes), s);
   }
-  if (stream_ok) {
+  // rows too long for the rows kernel (more than 16 blocks of 1024 tokens) with fewer than 16 channel blocks: the
+  // streaming kernel would run on that many workgroups, the time-parallel vector-ALU passes below are quicker
+  // (B1 x D64 x L65536 in bf16: 155 -> 77 us one-sided, 427 -> 102 us two-sided; from 16 channel blocks on they lose)
+  const bool few_rows = sxl == 1 && syl == 1 && B * ceil_div(D, 16) < 16;
+  if (stream_ok && !few_rows) {
     const void* img = image;
     if (!img) {
       // no cached image: kernel generation runs with every call

@@ -24,6 +24,8 @@
 // tile's dy and x held in registers): every tile publishes its map as tagged words, composes the maps of the tiles
 // behind it in walk order (block records of 32 tiles for rows of more than 128 tiles, bounded waits) and goes on to dx with the dy and
 // x it already holds, so both are read once.
+// The per-feature norm with an even number of channels takes the same three steps with the channels across the
+// lanes (tsn_bwd_feature_kernel: a thread owns two channels and walks its tile's 64 tokens itself).
 // Masked tokens are skipped by the walk (identity map, dx = 0).  "Previous cumulative mean" is
 // cummean[t-1]; the forward kernels of this library store the carried mean at masked tokens, so
 // this is the state before token t also behind a masked token.
@@ -411,6 +413,190 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
   }
 }
 
+// ---- per-feature statistics (one channel per group, group_mean = x): a thread owns two neighbouring channels and
+// walks the tokens of its tile itself, from the last to the first; the tiles' maps are carried per channel.
+// The same three steps as above (maps, carry, dx) with the channels, not the groups, across the lanes: every load is
+// a row of neighbouring channels.  kFbT tokens per tile, kFbThreads x 2 channels per workgroup.
+constexpr int kFbT = 64;
+constexpr int kFbThreads = 256;
+constexpr int kFbU = 8;            // tokens whose loads are in flight together
+
+template <typename T>
+__device__ __forceinline__ float2 load2(const T* p) {
+  if constexpr (sizeof(T) == 4) {
+    return *(const float2*)p;
+  } else {
+    const uint32_t w = *(const uint32_t*)p;
+    T lo, hi;
+    const uint16_t l16 = (uint16_t)(w & 0xffffu), h16 = (uint16_t)(w >> 16);
+    __builtin_memcpy(&lo, &l16, 2);
+    __builtin_memcpy(&hi, &h16, 2);
+    return make_float2(to_float(lo), to_float(hi));
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store2(T* p, float a, float b) {
+  if constexpr (sizeof(T) == 4) {
+    *(float2*)p = make_float2(a, b);
+  } else {
+    const T lo = from_float<T>(a), hi = from_float<T>(b);
+    uint16_t l16, h16;
+    __builtin_memcpy(&l16, &lo, 2);
+    __builtin_memcpy(&h16, &hi, 2);
+    *(uint32_t*)p = (uint32_t)l16 | ((uint32_t)h16 << 16);
+  }
+}
+
+// PHASE 0: the tile's map of every channel and its gamma / beta shares; PHASE 1: dx from the pair entering the tile
+template <typename T, int PHASE>
+__global__ __launch_bounds__(kFbThreads) void tsn_bwd_feature_kernel(const TsnBwdParams P) {
+  __shared__ float s_c1[kFbT], s_c2[kFbT];
+  __shared__ int s_keep[kFbT];
+  __shared__ int s_later;
+  const int H = P.H, tid = threadIdx.x;
+  const int cblocks = (H + 2 * kFbThreads - 1) / (2 * kFbThreads);
+  const int cblk = (int)blockIdx.x % cblocks;
+  const int rest = (int)blockIdx.x / cblocks;
+  const int tile = rest % P.nt, b = rest / P.nt;
+  const int t0 = tile * kFbT;
+  const int ntok = min(kFbT, P.L - t0);
+  const int c = cblk * 2 * kFbThreads + 2 * tid;      // H is even: a thread's two channels are both inside or outside
+  const bool live = c < H;
+
+  // ---- the running count at every token of the tile (the same for all channels)
+  if (tid == 0) s_later = 0;
+  __syncthreads();
+  if (P.mask) {
+    int later = 0;
+    for (int t = t0 + kFbT + tid; t < P.L; t += kFbThreads) later += P.mask[(size_t)b * P.L + t] ? 0 : 1;
+    if (later) atomicAdd(&s_later, later);
+  }
+  __syncthreads();
+  if (tid < kFbT) {
+    const bool has = tid < ntok && !(P.mask && P.mask[(size_t)b * P.L + t0 + tid]);
+    const unsigned long long bal = __ballot(has);
+    const int after = tid >= 63 ? 0 : __popcll(bal >> (tid + 1));     // unmasked tokens of the tile behind this one
+    const int64_t n_end = P.count[b] - (P.mask ? (int64_t)s_later : (int64_t)max(0, P.L - t0 - kFbT));
+    const float n = (float)(n_end - after);
+    const float c2 = has ? 1.0f / n : 0.f;
+    s_c2[tid] = c2;
+    s_c1[tid] = has ? (n - 1.0f) * c2 : 1.f;
+    s_keep[tid] = has ? 1 : 0;
+  }
+  __syncthreads();
+  if (!live) return;
+
+  const size_t row = ((size_t)b * P.L + t0) * H + c;
+  const T* dy = (const T*)P.dy + row;
+  const T* x = (const T*)P.x + row;
+  const float* cm = P.cummean + row;
+  const float* cr = P.cumrstd + row;
+  const float2 w = *(const float2*)(P.gamma + c);
+  // cumulative mean before the tile's first token
+  const float2 up0 = t0 == 0 ? *(const float2*)(P.prev_mean + (size_t)b * H + c) : *(const float2*)(cm - H);
+
+  float2 ug = make_float2(0.f, 0.f), vg = make_float2(0.f, 0.f);     // PHASE 1: the carried pair
+  float2 ma = make_float2(1.f, 1.f), mm = make_float2(0.f, 0.f);     // PHASE 0: the composed map
+  float2 mbu = make_float2(0.f, 0.f), mbv = make_float2(0.f, 0.f);
+  float2 gwv = make_float2(0.f, 0.f), gbv = make_float2(0.f, 0.f);
+  if (PHASE == 1) {
+    const float4 st = *(const float4*)(P.state + (((size_t)b * P.nt + tile) * H + c) * 2);   // (u, v) of both channels
+    ug = make_float2(st.x, st.z);
+    vg = make_float2(st.y, st.w);
+  }
+  T* dx = PHASE == 1 ? (T*)P.dx + row : nullptr;
+  for (int hi = ntok; hi > 0; hi -= kFbU) {
+    // tokens hi - 1 down to hi - kFbU (those below 0 repeat token 0 and are dropped)
+    float2 d[kFbU], xv[kFbU], m_[kFbU + 1], r_[kFbU];
+#pragma unroll
+    for (int k = 0; k < kFbU; ++k) {
+      const int t = max(hi - 1 - k, 0);
+      d[k] = load2<T>(dy + (size_t)t * H);
+      xv[k] = load2<T>(x + (size_t)t * H);
+      m_[k] = *(const float2*)(cm + (size_t)t * H);
+      r_[k] = *(const float2*)(cr + (size_t)t * H);
+    }
+    {
+      const int t = hi - 1 - kFbU;                    // the token before the batch: its cumulative mean
+      m_[kFbU] = t >= 0 ? *(const float2*)(cm + (size_t)t * H) : up0;
+    }
+#pragma unroll
+    for (int k = 0; k < kFbU; ++k) {
+      const int t = hi - 1 - k;
+      if (t < 0) break;
+      const bool keep = s_keep[t] != 0;
+      const float c1 = s_c1[t], c2 = s_c2[t];
+      const float2 up = t == 0 ? up0 : m_[k + 1];
+      float dxv[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const float dq = q ? d[k].y : d[k].x, xq = q ? xv[k].y : xv[k].x, mq = q ? m_[k].y : m_[k].x;
+        const float rq = q ? r_[k].y : r_[k].x, wq = q ? w.y : w.x, upq = q ? up.y : up.x;
+        const float ds = dq * (xq - mq) * wq, db = dq * wq;
+        const float e = 0.5f * rq * rq * rq * ds, rdb = rq * db;
+        const float mj = -2.0f * c1 * c2 * (xq - upq);
+        float& a_ = q ? ma.y : ma.x; float& m2 = q ? mm.y : mm.x; float& bu = q ? mbu.y : mbu.x; float& bv = q ? mbv.y : mbv.x;
+        float& u_ = q ? ug.y : ug.x; float& v_ = q ? vg.y : vg.x;
+        float& gw_ = q ? gwv.y : gwv.x; float& gb_ = q ? gbv.y : gbv.x;
+        dxv[q] = 0.f;
+        if (keep) {
+          if (PHASE == 0) {
+            // this token's map after the maps of the tokens behind it
+            const float buj = -c1 * rdb - mj * e, bvj = -c1 * e;
+            const float na = c1 * a_, nm = fmaf(c1, m2, mj * a_);
+            const float nbu = fmaf(c1, bu, fmaf(mj, bv, buj)), nbv = fmaf(c1, bv, bvj);
+            a_ = na; m2 = nm; bu = nbu; bv = nbv;
+            gw_ = fmaf(dq * (xq - mq), rq, gw_);
+            gb_ += dq;
+          } else {
+            const float du = u_ - rdb, dv = v_ - e;
+            dxv[q] = fmaf(dq * rq, wq, c2 * du - mj * dv);      // group_mean = x: the dvx term vanishes
+            u_ = fmaf(c1, du, mj * dv);
+            v_ = c1 * dv;
+          }
+        }
+      }
+      if (PHASE == 1) store2<T>(dx + (size_t)t * H, dxv[0], dxv[1]);
+    }
+  }
+  if (PHASE == 0) {
+    float4* dst = (float4*)P.agg + ((size_t)b * P.nt + tile) * H + c;
+    dst[0] = make_float4(ma.x, mm.x, mbu.x, mbv.x);
+    dst[1] = make_float4(ma.y, mm.y, mbu.y, mbv.y);
+    float* pt = P.part + ((size_t)b * P.nt + tile) * 2 * H;
+    *(float2*)(pt + c) = gwv;
+    *(float2*)(pt + H + c) = gbv;
+  }
+}
+
+// one thread per (row, channel): the tiles' maps from the last tile to the first, eight maps in flight
+__global__ __launch_bounds__(kFbThreads) void tsn_bwd_feature_carry_kernel(const TsnBwdParams P) {
+  const int H = P.H;
+  const int i = (int)blockIdx.x * kFbThreads + (int)threadIdx.x;      // (row, channel)
+  if (i >= P.B * H) return;
+  const int b = i / H, c = i - b * H;
+  float ug = P.mean_grad ? P.mean_grad[i] : 0.f;
+  float vg = P.var_grad ? P.var_grad[i] : 0.f;
+  const float4* agg = (const float4*)P.agg + (size_t)b * P.nt * H + c;
+  float2* st = (float2*)P.state + (size_t)b * P.nt * H + c;
+  for (int hi = P.nt; hi > 0; hi -= 8) {
+    float4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = agg[(size_t)max(hi - 1 - k, 0) * H];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int tile = hi - 1 - k;
+      if (tile < 0) break;
+      st[(size_t)tile * H] = make_float2(ug, vg);
+      const float nu = fmaf(v[k].x, ug, fmaf(v[k].y, vg, v[k].z));
+      vg = fmaf(v[k].x, vg, v[k].w);
+      ug = nu;
+    }
+  }
+  P.prev_mean_grad[i] = ug;
+  P.prev_var_grad[i] = vg;
+}
+
 // ---- one launch: tile maps, look-back over the tiles behind, dx
 constexpr int kOpThreads = 512;  // 8 waves; two workgroups share a compute unit (128 registers a lane)
 constexpr int kOpNV = 8;        // 16-byte vectors of dy (and of x) a thread holds
@@ -795,6 +981,10 @@ struct BwdGeom {
   bool onepass;
   int op_tt, op_nt, op_nblk;
   size_t op_rec_bytes, op_brec_bytes, op_part_bytes;
+  // per-feature statistics with an even number of channels: the channel-parallel form
+  bool feature;
+  int fb_nt;
+  size_t fb_agg_bytes, fb_state_bytes, fb_part_bytes;
 };
 
 std::atomic<int> g_onepass{1};     // test hook: 0 keeps every call on the three-pass form
@@ -834,13 +1024,23 @@ bool bwd_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, BwdGeom
       }
     }
   }
+  g->feature = G == H && H % 2 == 0 && B * H < (int64_t)1 << 31;
+  g->fb_nt = (int)ceil_div(L, kFbT);
+  g->fb_agg_bytes = g->fb_state_bytes = g->fb_part_bytes = 0;
+  if (g->feature) {
+    g->fb_agg_bytes = align_up((size_t)B * g->fb_nt * H * 16, 256);
+    g->fb_state_bytes = align_up((size_t)B * g->fb_nt * H * 8, 256);
+    g->fb_part_bytes = align_up((size_t)B * g->fb_nt * 2 * H * 4, 256);
+  }
   return true;
 }
 
 size_t bwd_workspace_need(const BwdGeom& g) {
   const size_t three = g.agg_bytes + g.state_bytes + g.part_bytes;
   const size_t one = g.op_rec_bytes + g.op_brec_bytes + g.op_part_bytes;
-  return three > one ? three : one;
+  const size_t feat = g.fb_agg_bytes + g.fb_state_bytes + g.fb_part_bytes;
+  size_t need = three > one ? three : one;
+  return need > feat ? need : feat;
 }
 
 template <typename T, int VEC>
@@ -868,6 +1068,22 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (carry)");
   hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 1>), grid, dim3(kThreads), lds1, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (dx)");
+  hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 32)), dim3(256), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (parameters)");
+  return MEGA_OK;
+}
+
+template <typename T>
+int launch_feature(const TsnBwdParams& P, hipStream_t s) {
+  const int cblocks = (P.H + 2 * kFbThreads - 1) / (2 * kFbThreads);
+  const dim3 grid((unsigned)((int64_t)P.B * P.nt * cblocks));
+  hipLaunchKernelGGL((tsn_bwd_feature_kernel<T, 0>), grid, dim3(kFbThreads), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (per-feature maps)");
+  hipLaunchKernelGGL(tsn_bwd_feature_carry_kernel, dim3((unsigned)ceil_div((int64_t)P.B * P.H, kFbThreads)),
+                     dim3(kFbThreads), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (per-feature carry)");
+  hipLaunchKernelGGL((tsn_bwd_feature_kernel<T, 1>), grid, dim3(kFbThreads), 0, s, P);
+  MEGA_CHECK_LAUNCH("timestep_norm_bwd (per-feature dx)");
   hipLaunchKernelGGL(tsn_bwd_param_kernel, dim3((unsigned)ceil_div(2 * (int64_t)P.H, 32)), dim3(256), 0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (parameters)");
   return MEGA_OK;
@@ -985,6 +1201,36 @@ extern "C" int mega_group_timestep_norm_bwd(const void* y_grad, const float* mea
     return rc != MEGA_OK ? rc : lookback_verify("timestep_norm_bwd", s);
   }
   P.rec = nullptr; P.brec = nullptr; P.nblk = 0; P.lb = LookbackLaunch{nullptr, 0u, 0};
+  const size_t es_ = dtype == MEGA_F32 ? 4 : 2;
+  if (g.feature && ((((uintptr_t)y_grad | (uintptr_t)x | (uintptr_t)x_grad) % (2 * es_)) == 0) &&
+      ((((uintptr_t)cummean | (uintptr_t)cumrstd | (uintptr_t)gamma | (uintptr_t)prev_mean) % 8) == 0)) {
+    P.dy = y_grad; P.x = x; P.dx = x_grad; P.mean_grad = mean_grad; P.var_grad = var_grad; P.prev_mean = prev_mean;
+    P.count = count; P.group_mean = nullptr; P.cummean = cummean; P.cumrstd = cumrstd; P.gamma = gamma; P.mask = mask;
+    P.agg = (float*)w; w += g.fb_agg_bytes;
+    P.state = (float*)w; w += g.fb_state_bytes;
+    P.part = (float*)w;
+    P.prev_mean_grad = prev_mean_grad; P.prev_var_grad = prev_var_grad; P.gamma_grad = gamma_grad; P.beta_grad = beta_grad;
+    P.B = (int)B; P.L = (int)L; P.H = (int)H; P.G = (int)G; P.Dg = 1; P.TT = kFbT; P.nt = g.fb_nt;
+    P.R = make_row_tiling(G, 1, 1);
+    if (audit_on()) {
+      // per (row, tile, channel): one map of four floats and one pair of state gradients; per (row, tile): the tile's
+      // share of the gamma / beta gradients, 2 H floats
+      audit_use(P.agg, (size_t)B * g.fb_nt * H * 16, "timestep_norm_bwd: per-feature tile maps");
+      audit_use(P.state, (size_t)B * g.fb_nt * H * 8, "timestep_norm_bwd: per-feature pairs entering the tiles");
+      audit_use(P.part, (size_t)B * g.fb_nt * 2 * H * 4, "timestep_norm_bwd: parameter-gradient shares");
+      audit_use(y_grad, (size_t)B * L * H * es_, "timestep_norm_bwd: y_grad");
+      audit_use(x, (size_t)B * L * H * es_, "timestep_norm_bwd: x");
+      audit_use(x_grad, (size_t)B * L * H * es_, "timestep_norm_bwd: x_grad");
+      audit_use(cummean, (size_t)B * L * G * 4, "timestep_norm_bwd: cummean");
+      audit_use(cumrstd, (size_t)B * L * G * 4, "timestep_norm_bwd: cumrstd");
+      return MEGA_OK;
+    }
+    switch (dtype) {
+      case MEGA_F32: return launch_feature<float>(P, s);
+      case MEGA_BF16: return launch_feature<bf16_t>(P, s);
+      default: return launch_feature<f16_t>(P, s);
+    }
+  }
   P.dy = y_grad; P.x = x; P.dx = x_grad; P.mean_grad = mean_grad; P.var_grad = var_grad; P.prev_mean = prev_mean;
   P.count = count; P.group_mean = group_mean; P.cummean = cummean; P.cumrstd = cumrstd; P.gamma = gamma; P.mask = mask;
   P.agg = (float*)w; w += g.agg_bytes;

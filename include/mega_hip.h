@@ -432,7 +432,8 @@ int mega_group_timestep_norm_fwd_noalloc(const void* x, void* y, int dtype,
  *   tiles behind it with bounded waits, like the forward's look-back.  A wait that gives up leaves
  *   NaN in x_grad / prev_mean_grad / prev_var_grad and is reported like the forward's: the next
  *   call returns MEGA_ERR_LAUNCH (mega_lookback_status, checked mode: the same call).  Everything
- *   else takes three passes (tile maps, carry, x_grad) without waits.  The workspace needs no
+ *   else takes three passes (tile maps, carry, x_grad) without waits; the per-feature form with an even
+ *   number of channels runs them with the channels across the lanes (a thread walks its tile's tokens).  The workspace needs no
  *   initialisation and nothing in it survives the call (the records are cleared by the call). */
 size_t mega_timestep_norm_bwd_workspace_bytes(int dtype, int64_t B, int64_t L, int64_t H, int64_t G);
 int mega_group_timestep_norm_bwd(const void* y_grad, const float* mean_grad, const float* var_grad,

@@ -36,6 +36,8 @@ def _tsn_case(rng, B, L, H, G, masked, prior, dtype):
     (2, 50, 48, 2, True, False),       # 24 channels per group: three vectors per lane
     (2, 33, 30, 5, True, True),        # 6 channels per group: element-wise path
     (2, 45, 24, None, True, True),     # per-feature statistics
+    (2, 300, 1100, None, True, True),  # per-feature, three blocks of 512 channels (the last partial), five tiles of 64 tokens
+    (1, 130, 25, None, False, False),  # per-feature with an odd number of channels: the group form with one channel a group
 ])
 def test_timestep_norm_bwd(dtype, B, L, H, G, masked, prior):
     rng = np.random.default_rng(51)
