@@ -82,7 +82,7 @@ __device__ __forceinline__ TileMap shfl_up32(const TileMap v, int o) {
 // PHASE 0: tile maps + parameter shares; PHASE 1: dx.
 // FIXED (PHASE 0 only): slots divides the workgroup size and every lane moves one vector, so a
 // thread meets the same VEC channels at every token it visits and keeps their gamma / beta shares
-// in registers; otherwise the shares are added into LDS element by element.
+// in registers; otherwise tsn_bwd_shares_kernel forms the shares (a thread per vector of channels).
 template <typename T, int VEC, int PHASE, bool FIXED = false>
 __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdParams P) {
   using V = Vec<T, VEC>;
@@ -174,9 +174,6 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
             if (FIXED) {
               rw[e] = fmaf(d * (xe - u_), r, rw[e]);
               rb[e] += d;
-            } else {
-              atomicAdd(&s_wg[cc[u] + e], d * (xe - u_) * r);
-              atomicAdd(&s_bg[cc[u] + e], d);
             }
           }
         }
@@ -215,10 +212,6 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
           ds = fmaf(d * (xe - u), w, ds);
           db = fmaf(d, w, db);
           sx += xe;
-          if (PHASE == 0 && keep) {
-            atomicAdd(&s_wg[c + e], d * (xe - u) * r);
-            atomicAdd(&s_bg[c + e], d);
-          }
         }
       }
     }
@@ -345,8 +338,10 @@ __global__ __launch_bounds__(kThreads) void tsn_bwd_tile_kernel(const TsnBwdPara
         __syncthreads();
       }
     }
-    float* dst = P.part + ((size_t)b * P.nt + tile) * 2 * H;
-    for (int c = tid; c < H; c += kThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
+    if (FIXED) {
+      float* dst = P.part + ((size_t)b * P.nt + tile) * 2 * H;
+      for (int c = tid; c < H; c += kThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
+    }
   } else {
     T* dx = (T*)P.dx + ((size_t)b * P.L + t0) * H;
     const float cg = 1.0f / (float)Dg;
@@ -897,6 +892,60 @@ __global__ __launch_bounds__(kOpThreads, 4) void tsn_bwd_onepass_kernel(const Ts
   for (int c = tid; c < H; c += kOpThreads) { dst[c] = s_wg[c]; dst[H + c] = s_bg[c]; }
 }
 
+// The gamma / beta shares of a tile where the tile kernel's threads do not keep to the same channels (group sizes
+// that are not a power of two of vectors, more vectors per token than threads): a thread owns one vector of
+// channels and walks the tile's tokens, four tokens' loads in flight.  Same output as the tile kernel's:
+// part[row, tile][2][H].
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void tsn_bwd_shares_kernel(const TsnBwdParams P) {
+  using V = Vec<T, VEC>;
+  const int H = P.H, G = P.G, TT = P.TT;
+  const int nvec = H / VEC;
+  const int cblocks = (nvec + 255) / 256;
+  const int cblk = (int)blockIdx.x % cblocks, rt = (int)blockIdx.x / cblocks;    // rt = row * nt + tile
+  const int tile = rt % P.nt, b = rt / P.nt;
+  const int v = cblk * 256 + (int)threadIdx.x;
+  if (v >= nvec) return;
+  const int c = v * VEC, g = c / P.Dg;
+  const int t0 = tile * TT, ntok = min(TT, P.L - t0);
+  const T* dy = (const T*)P.dy + ((size_t)b * P.L + t0) * H + c;
+  const T* x = (const T*)P.x + ((size_t)b * P.L + t0) * H + c;
+  const float* cm = P.cummean + ((size_t)b * P.L + t0) * G + g;
+  const float* cr = P.cumrstd + ((size_t)b * P.L + t0) * G + g;
+  const uint8_t* mk = P.mask ? P.mask + (size_t)b * P.L + t0 : nullptr;
+  float rw[VEC], rb[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) { rw[e] = 0.f; rb[e] = 0.f; }
+  for (int tb = 0; tb < ntok; tb += 4) {
+    V dv[4], xv[4];
+    float u[4], r[4];
+    bool keep[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = min(tb + k, ntok - 1);
+      dv[k] = *(const V*)(dy + (size_t)t * H);
+      xv[k] = *(const V*)(x + (size_t)t * H);
+      u[k] = cm[(size_t)t * G];
+      r[k] = cr[(size_t)t * G];
+      keep[k] = tb + k < ntok && !(mk && mk[t]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (keep[k]) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float d = to_float(dv[k].v[e]);
+          rw[e] = fmaf(d * (to_float(xv[k].v[e]) - u[k]), r[k], rw[e]);
+          rb[e] += d;
+        }
+      }
+    }
+  }
+  float* dst = P.part + (size_t)rt * 2 * H + c;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) { dst[e] = rw[e]; dst[H + e] = rb[e]; }
+}
+
 // One wave per (row, group).  The tiles are walked from the last to the first; lane l owns the
 // l-th run of `per` tiles in that order, composes its run, the runs are combined by a scan over
 // the lanes, and every lane then replays its run from the pair that enters it.
@@ -1061,8 +1110,14 @@ int launch_tiles(const TsnBwdParams& P, hipStream_t s) {
   }
   const dim3 grid((unsigned)(P.B * P.nt));
   const bool fixed = P.R.PER == 1 && P.R.slots <= kThreads && kThreads % P.R.slots == 0;
-  if (fixed) hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, true>), grid, dim3(kThreads), lds0, s, P);
-  else hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, false>), grid, dim3(kThreads), lds0, s, P);
+  if (fixed) {
+    hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, true>), grid, dim3(kThreads), lds0, s, P);
+  } else {
+    hipLaunchKernelGGL((tsn_bwd_tile_kernel<T, VEC, 0, false>), grid, dim3(kThreads), lds0, s, P);
+    MEGA_CHECK_LAUNCH("timestep_norm_bwd (tile maps)");
+    const int64_t cblocks = ceil_div((int64_t)P.H / VEC, 256);
+    hipLaunchKernelGGL((tsn_bwd_shares_kernel<T, VEC>), dim3((unsigned)(P.B * P.nt * cblocks)), dim3(256), 0, s, P);
+  }
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (tile maps)");
   hipLaunchKernelGGL(tsn_bwd_carry_kernel, dim3((unsigned)(P.B * P.G)), dim3(64), 0, s, P);
   MEGA_CHECK_LAUNCH("timestep_norm_bwd (carry)");
