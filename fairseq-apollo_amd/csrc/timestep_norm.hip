@@ -174,6 +174,38 @@ __global__ __launch_bounds__(kThreads) void group_tsn_kernel(const TsnParams P) 
       }
     }
     __syncthreads();
+  } else if constexpr (sizeof(T) == 2 && VEC >= 2) {
+    // groups of any number of vectors, 16-bit activations: every vector's sum and sum of squares (packed dot
+    // products, as above) go through LDS once, and a thread per (token, group) adds the group's up
+    float2* part2 = (float2*)part;
+#pragma unroll
+    for (int j = 0; j < kNV; ++j) {
+      const int v = j * kThreads + tid;
+      if (v < nvec) {
+        float s = 0.f, q = 0.f;
+        const uint32_t* w = (const uint32_t*)&xv[j];
+#pragma unroll
+        for (int i = 0; i < VEC / 2; ++i) {
+          s = dot2_ones<T>(w[i], s);
+          q = dot2_self<T>(w[i], q);
+        }
+        part2[v] = make_float2(s, q);
+      }
+    }
+    __syncthreads();
+    for (int item = tid; item < nt * G; item += kThreads) {
+      const int tok = item / G, g = item - tok * G;
+      const float2* pp = part2 + tok * TPT + g * LPG;
+      float s = 0.f, q = 0.f;
+      for (int i = 0; i < LPG; ++i) {
+        s += pp[i].x;
+        q += pp[i].y;
+      }
+      const float m = s * inv_dg;
+      s_mean[item] = m;
+      s_var[item] = fmaxf(q * inv_dg - m * m, 0.f);
+    }
+    __syncthreads();
   } else {
 #pragma unroll
     for (int j = 0; j < kNV; ++j) {
@@ -697,7 +729,7 @@ bool tsn_geometry(int dtype, int64_t B, int64_t L, int64_t H, int64_t G, TsnGeom
   const int lpg = g->lpg;
   g->lpgt = (lpg <= 64 && (lpg & (lpg - 1)) == 0) ? lpg : 0;
   size_t bytes = 2 * (size_t)tt * G * 4 + align_up((size_t)tt, 16) + (size_t)kLbWords * 8;
-  if (g->lpgt == 0) bytes += (size_t)kPartCap * 4;
+  if (g->lpgt == 0) bytes += (size_t)kPartCap * (esize == 2 && vec >= 2 ? 8 : 4);   // 16-bit: (sum, sum of squares)
   g->smem = bytes;
   return g->smem <= 150 * 1024;
 }
