@@ -585,6 +585,18 @@ def attention_fwd(q, k, v, scale: float, dropout: float, use_causal_mask: bool, 
     y = None if weights_only else torch.empty(B, L, Nh, H2, dtype=qd.dtype, device=dev)
     w = torch.empty(B, Nh, L, L, dtype=qd.dtype, device=dev) if need_weights else None
     nws = lib.mega_attention_workspace_bytes(_dtype_code(qd), B, L, Nh, H1, H2)
+    if not nws and L >= 64 and qd.numel():
+        # outside the matrix-core kernels (fp32, head sizes that are not multiples of 8): the two products as batched
+        # library GEMMs around this library's softmax, which is what the reference does for every shape
+        # (attention_kernel.cu:40-131); the library's own fallback is a kernel of one thread per score.  The scores
+        # are rounded to the activation type before the softmax, as the reference's are.
+        s = torch.einsum('bqnh,bknh->bnqk', qd, kd)
+        if float(scale) != 1.0:
+            s.mul_(float(scale))
+        wts = attention_softmax_fwd(s, dropout, use_causal_mask, seed)
+        del s
+        y = None if weights_only else torch.einsum('bnqk,bknh->bqnh', wts, vd).contiguous()
+        return y, (wts if need_weights else None)
     ws = _scratch_buffer(dev, nws) if nws else None
     with _on_device(dev):
         rc = lib.mega_attention_fwd(_ptr(qd), _ptr(kd), _ptr(vd), _ptr(y), _ptr(w), _dtype_code(qd), B, L, Nh, H1, H2,
