@@ -326,6 +326,12 @@ def bench_tsn_feature(args):
 
     par = timed(lambda i: M.ops.timestep_norm_fwd(xs[i % NBUF], pc, pm, pv, gamma, beta, None, 1e-5, need_stats=False),
                 args.steps)
+    # a training step of the same norm: the forward that also writes the running statistics, then the backward
+    dys = [torch.randn(B, L, D, device=dev).to(torch.bfloat16) for _ in range(2)]
+    saved = M.ops.timestep_norm_fwd(xs[0], pc, pm, pv, gamma, beta, None, 1e-5)
+    fwd_stats = timed(lambda i: M.ops.timestep_norm_fwd(xs[i % NBUF], pc, pm, pv, gamma, beta, None, 1e-5), args.steps)
+    bwd = timed(lambda i: M.ops.timestep_norm_bwd(dys[i % 2], None, None, xs[0], pm, saved[1], saved[4], saved[5], gamma,
+                                                  None), args.steps)
     lib = M._lib.load()
     y = torch.empty_like(xs[0])
     cnt = torch.empty(B, dtype=torch.int64, device=dev)
@@ -343,7 +349,8 @@ def bench_tsn_feature(args):
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": par,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "TimestepNorm without groups (every feature its own statistics) at configs[2]'s activation shape"},
-        "kernels": {"time_tiles_ms": par},
+        "kernels": {"time_tiles_ms": par, "forward_with_saved_statistics_ms": fwd_stats, "backward_ms": bwd,
+                    "backward_algorithmic_bytes": 3 * B * L * D * 2 + 2 * B * L * D * 4},
         "roofline": {"bound": "hbm", "kernel": "feature_tile_moments + feature_tile_scan + feature_tile_apply",
                      "achieved": alg / (par * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg / (par * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_step": alg},
