@@ -99,6 +99,7 @@ SIGNATURES = {
     "mega_silu_bwd": (_int, [_p, _p, _p, _int, _i64, _p]),
     "mega_colsum_workspace_bytes": (_sz, [_i64, _i64]),
     "mega_colsum": (_int, [_p, _i64, _int, _i64, _i64, _p, _int, _p, _sz, _p]),
+    "mega_transpose_2d": (_int, [_p, _p, _int, _i64, _i64, _i64, _int, _int, _p]),
     "mega_ema_coeffs_fwd": (_int, [_p, _p, _p, _p, _p, _int, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p]),
     "mega_ema_coeffs_bwd": (_int, [_p, _p, _p, _p, _p, _p, _p, _int, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p]),
     "mega_norm_params_fwd": (_int, [_p, _p, _int, _p, _p, _int, _i64, _i64, _i64, _p, _p, _p, _p, _p]),

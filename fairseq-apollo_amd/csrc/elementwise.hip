@@ -281,6 +281,62 @@ extern "C" size_t mega_colsum_workspace_bytes(int64_t T_, int64_t W) {
   return (size_t)ceil_div(T_, kColSlabRows) * (size_t)W * 4;
 }
 
+namespace mega {
+namespace {
+
+// out[b][c][r] = in[b][r'][c'] with r' = r or rows - 1 - r, c' = c or cols - 1 - c: tiles of 64 x 64 elements
+// through LDS, rows of the tile read and written as whole runs of 64 neighbouring elements.  E: the element as an
+// unsigned integer of its size.
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_tile_kernel(const E* __restrict__ in, E* __restrict__ out, int64_t rows,
+                                                             int64_t cols, int tiles_r, int tiles_c, int rev_r, int rev_c) {
+  __shared__ E tile[64][64 + (sizeof(E) == 4 ? 1 : 2)];
+  const int t = (int)blockIdx.x;
+  const int tc = t % tiles_c, rest = t / tiles_c;
+  const int tr = rest % tiles_r;
+  const int64_t b = rest / tiles_r;
+  const int64_t r0 = (int64_t)tr * 64, c0 = (int64_t)tc * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const E* src = in + b * rows * cols;
+  E* dst = out + b * rows * cols;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t r = r0 + ty + 4 * i, c = c0 + tx;
+    if (r < rows && c < cols) tile[ty + 4 * i][tx] = src[(rev_r ? rows - 1 - r : r) * cols + (rev_c ? cols - 1 - c : c)];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t c = c0 + ty + 4 * i, r = r0 + tx;
+    if (c < cols && r < rows) dst[c * rows + r] = tile[tx][ty + 4 * i];
+  }
+}
+
+}  // namespace
+}  // namespace mega
+
+extern "C" int mega_transpose_2d(const void* in, void* out, int elem_bytes, int64_t batch, int64_t rows, int64_t cols,
+                                 int reverse_rows, int reverse_cols, void* stream) {
+  MEGA_REQUIRE(elem_bytes == 2 || elem_bytes == 4, MEGA_ERR_ARG, "transpose_2d: elements of 2 or 4 bytes, got %d",
+               elem_bytes);
+  MEGA_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, MEGA_ERR_ARG, "transpose_2d: bad sizes %lld x %lld x %lld",
+               (long long)batch, (long long)rows, (long long)cols);
+  if (batch == 0 || rows == 0 || cols == 0) return MEGA_OK;
+  MEGA_REQUIRE(in && out && in != out, MEGA_ERR_ARG, "transpose_2d: null or aliased pointer argument");
+  const int64_t tr = (rows + 63) / 64, tc = (cols + 63) / 64;
+  MEGA_REQUIRE(batch * tr * tc < ((int64_t)1 << 31), MEGA_ERR_UNSUPPORTED, "transpose_2d: too many tiles");
+  const dim3 grid((unsigned)(batch * tr * tc));
+  hipStream_t s = (hipStream_t)stream;
+  if (elem_bytes == 4)
+    hipLaunchKernelGGL((mega::transpose_tile_kernel<uint32_t>), grid, dim3(256), 0, s, (const uint32_t*)in, (uint32_t*)out,
+                       rows, cols, (int)tr, (int)tc, reverse_rows ? 1 : 0, reverse_cols ? 1 : 0);
+  else
+    hipLaunchKernelGGL((mega::transpose_tile_kernel<uint16_t>), grid, dim3(256), 0, s, (const uint16_t*)in, (uint16_t*)out,
+                       rows, cols, (int)tr, (int)tc, reverse_rows ? 1 : 0, reverse_cols ? 1 : 0);
+  MEGA_CHECK_LAUNCH("transpose_2d");
+  return MEGA_OK;
+}
+
 extern "C" int mega_colsum(const void* x, int64_t row_stride, int dtype, int64_t T_, int64_t W, void* out,
                            int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   MEGA_REQUIRE((dtype == MEGA_F32 || dtype == MEGA_BF16 || dtype == MEGA_F16) &&

@@ -617,6 +617,15 @@ int mega_swiglu_bwd(const void* y_grad, const void* a, const void* b, void* a_gr
                     int dtype, int64_t n, void* stream);
 /* Backward of mega_silu_fwd (F.silu under autograd): a_grad = y_grad silu'(a), contiguous, n elements.   */
 int mega_silu_bwd(const void* y_grad, const void* a, void* a_grad, int dtype, int64_t n, void* stream);
+/* out[b][c][r] = in[b][r'][c'] for `batch` matrices of rows x cols elements of 2 or 4 bytes (any values: the
+ * elements are moved, not interpreted), with r' = rows - 1 - r when reverse_rows and c' = cols - 1 - c when
+ * reverse_cols; in and out are contiguous and must not overlap.  No counterpart in the reference, which calls
+ * Tensor::transpose(...).contiguous() and flip(): the Python host uses it to hand fp32 / fp16 activations that lie
+ * time-major in memory ([B, L, D]) to the moving average's rows kernels ([B, D, L]) and back, reversed in time for
+ * the input gradient.                                                                                         */
+int mega_transpose_2d(const void* in, void* out, int elem_bytes, int64_t batch, int64_t rows, int64_t cols,
+                      int reverse_rows, int reverse_cols, void* stream);
+
 /* Column sums of x [T, W] (row stride in elements) into out [W] of `out_dtype`: the bias gradient of a projection
  * (in the reference torch's sum over the tokens inside the backward of F.linear).  Rows of whole 16-byte pieces;
  * slabs of 256 rows are added in a fixed order (the same bits on every run); workspace of

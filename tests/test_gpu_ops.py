@@ -398,3 +398,52 @@ def test_spectral_convolution_operators(dtype, L):
     assert rel_err(host(xt), host(x_grad)) < TOL[dtype] and rel_err(host(kt), host(k_grad)) < 1e-4
     with pytest.raises(RuntimeError):
         M.ops.fftconv_fwd(x, k_f[:, :-1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,R,C", [(2, 64, 64), (3, 100, 37), (1, 1, 300), (2, 257, 1), (1, 4096, 1024), (0, 5, 5)])
+def test_transpose_2d(dtype, B, R, C):
+    """The tiled transposition the host uses between time-major memory and rows in time: elements are moved as they
+    are, whole and partial tiles of 64 x 64."""
+    x = torch.randn(B, R, C, device=DEV).to(dtype)
+    y = M.ops.transpose_2d(x)
+    assert y.shape == (B, C, R) and y.is_contiguous()
+    assert torch.equal(y, x.transpose(1, 2).contiguous())
+    assert torch.equal(M.ops.transpose_2d(x, reverse_rows=True), x.flip(1).transpose(1, 2).contiguous())
+    assert torch.equal(M.ops.transpose_2d(x, reverse_cols=True), x.flip(2).transpose(1, 2).contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("bidirectional", [False, True])
+@pytest.mark.parametrize("B,D,L,masked", [(2, 96, 1500, True), (1, 40, 4096, False), (3, 16, 64, False)])
+def test_time_major_rows_route(dtype, bidirectional, B, D, L, masked):
+    """fp32 / fp16 activations that lie time-major in memory run on the rows kernels between two transpositions: the
+    same result as from rows in time, in both output layouts, and the oracle's."""
+    print(f"case {dtype} bidirectional={bidirectional} B={B} D={D} L={L} masked={masked}", flush=True)
+    rng = np.random.default_rng(71)
+    N = 16
+    K = 2 * D if bidirectional else D
+    p, q, g = O.ema_coeffs_complex(*mega_init_complex(rng, K, N))
+    om = rng.normal(size=D)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om), bidirectional=bidirectional)
+    xt, x64 = rounded(rng.normal(size=(B, L, D)), dtype)          # [B, L, D] memory
+    mask = None
+    if masked:
+        mask = np.zeros((B, L), bool)
+        for b in range(B):
+            mask[b, L - 17 * (b + 1):] = True
+    tm = None if mask is None else dev(mask, torch.bool)
+    y_rows, _ = layer(xt.transpose(1, 2), tm)
+    y_in, _ = layer(xt.transpose(1, 2), tm, out_layout="input")
+    y_ref, _ = layer(xt.transpose(1, 2).contiguous(), tm)
+    torch.cuda.synchronize()
+    assert y_rows.is_contiguous() and y_in.stride() == (L * D, 1, D)
+    assert torch.equal(y_rows, y_ref) and torch.equal(y_in, y_ref)
+    yo, _ = O.ema_forward(x64.transpose(0, 2, 1), p, q, g, om, padding_mask=mask, bidirectional=bidirectional)
+    assert rel_err(host(y_rows), yo) < TOL[dtype]
+    # the input gradient through the same route (time reversed inside the transpositions) against the rows form
+    gt = torch.randn(B, L, D, device=DEV).to(dtype)
+    dx = layer.adjoint(gt.transpose(1, 2), tm)
+    dx_ref = layer.adjoint(gt.transpose(1, 2).contiguous(), tm)
+    assert dx.stride() == (L * D, 1, D)
+    assert rel_err(host(dx), host(dx_ref)) < 1e-5
