@@ -823,6 +823,21 @@ class PreparedEMA:
             raise RuntimeError(f"num_features={D} is not divisible by num_groups={G}")
         xd = x if (x.is_contiguous() and not x.requires_grad) else x.detach().contiguous()
         dt = _dtype_code(xd)
+        if out_layout not in ("rows", "input"):
+            raise RuntimeError(f"out_layout must be 'rows' or 'input', got {out_layout!r}")
+        if xd.dtype is not torch.bfloat16 and 64 <= L <= 16384 and self.N <= 16 and B > 0 \
+                and not ((want_state or h is not None) and L % 1024):
+            # fp32 / fp16: the two operators, the second through PreparedEMA.__call__, which takes the normalised
+            # activations (time-major in memory) onto the rows kernels; inside the library's own two-operator
+            # route the moving average would read them in place on its vector-ALU path
+            if want_stats:
+                xn, count, mean, var, _, cm, cr = group_timestep_norm_fwd(xd, prev_count, prev_mean, prev_var, norm_gamma,
+                                                                          norm_beta, padding_mask, G, eps)
+            else:
+                xn, count, mean, var = group_timestep_norm_fwd(xd, prev_count, prev_mean, prev_var, norm_gamma,
+                                                               norm_beta, padding_mask, G, eps, need_stats=False)[:4]
+            y, hc = self(xn.transpose(1, 2), padding_mask, h, want_state, out_layout=out_layout)
+            return (xn, y, count, mean, var, hc, cm, cr) if want_stats else (xn, y, count, mean, var, hc)
         xn = torch.empty_like(xd)
         if out_layout == "rows":
             y = torch.empty(B, D, L, dtype=xd.dtype, device=dev)

@@ -368,3 +368,58 @@ def test_module_pair_keeps_both_incremental_states():
     xg = x[:, :64].float().requires_grad_(True)
     xn_g, y_g = M.norm_then_move(norm, move, xg)
     assert y_g.requires_grad and xn_g.requires_grad
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.float16, 4e-3)])
+@pytest.mark.parametrize("out_layout,masked", [("rows", False), ("input", True)])
+def test_fp32_fp16_two_slices_with_state(dtype, tol, out_layout, masked):
+    """fp32 / fp16 activations: the norm, then the moving average on rows in time through a transposition each way.
+    Two slices of a row (1024 + 2048 tokens, the state of both operators carried across) against the oracle on the
+    whole row, in both output layouts, with padded tails."""
+    print(f"case dtype={dtype} out={out_layout} masked={masked}", flush=True)
+    B, G, N, D, L1, L2 = 2, 4, 16, 256, 1024, 2048
+    L = L1 + L2
+    rng = np.random.default_rng(57)
+    p, q, g, om, nw, nb = _setup(rng, D, N)
+    x, x64 = rounded(rng.normal(size=(B, L, D)) + 0.5, dtype)
+    mask = tm = None
+    if masked:
+        mask = np.zeros((B, L), bool)
+        mask[1, L - 300:] = True
+        tm = dev(mask, torch.bool)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+    m1 = None if tm is None else tm[:, :L1].contiguous()
+    m2 = None if tm is None else tm[:, L1:].contiguous()
+    xn1, y1, c1, mu1, v1, h1 = _run(layer, x[:, :L1].contiguous(), G, nw, nb, want_state=True, out_layout=out_layout,
+                                    padding_mask=m1)
+    xn2, y2, c2, mu2, v2, h2 = _run(layer, x[:, L1:].contiguous(), G, nw, nb, prior=(c1, mu1, v1), h=h1,
+                                    out_layout=out_layout, padding_mask=m2)
+    assert y2.shape == (B, D, L2)
+    assert y2.stride() == ((D * L2, L2, 1) if out_layout == "rows" else (L2 * D, 1, D))
+    xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, mask, G)
+    xn = torch.cat([xn1, xn2], 1)
+    assert rel_err(host(xn), xno) < tol
+    assert c2.tolist() == c.tolist()
+    assert rel_err(host(mu2), mu) < 1e-4 and rel_err(host(v2), v) < 1e-4
+    yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, mask, incremental=True)
+    assert rel_err(host(torch.cat([y1, y2], -1)), yo) < tol
+    assert rel_err(np.real(host(h2)), np.real(ho)) < 1e-3 and rel_err(np.imag(host(h2)), np.imag(ho)) < 1e-3
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.float16, 4e-3)])
+def test_fp32_fp16_ragged_row_and_training_statistics(dtype, tol):
+    """A row that is no whole number of blocks (no state asked for) with the statistics a training forward keeps."""
+    B, G, N, D, L = 2, 2, 16, 128, 1500
+    rng = np.random.default_rng(58)
+    p, q, g, om, nw, nb = _setup(rng, D, N)
+    x, x64 = rounded(rng.normal(size=(B, L, D)) * 1.2 - 0.2, dtype)
+    layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+    xn, y, cnt, mean, var, h, cm, cr = _run(layer, x, G, nw, nb, want_stats=True)
+    assert h is None and cm.shape == (B, L, G) and cr.shape == (B, L, G)
+    xno, c, mu, v = O.timestep_norm(x64, np.zeros(B, np.int64), np.zeros((B, G)), np.ones((B, G)), nw + 1, nb, None, G)
+    assert rel_err(host(xn), xno) < tol
+    assert cnt.tolist() == c.tolist()
+    assert rel_err(host(cm)[:, -1], mu) < 1e-4
+    assert rel_err(host(cr)[:, -1], 1.0 / np.sqrt(v + 1e-5)) < 1e-4
+    yo, _ = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om)
+    assert rel_err(host(y), yo) < tol
