@@ -210,6 +210,62 @@ def test_norm_then_moving_average_sweep(seed):
     assert M.ops.timestep_norm_status() == 0
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_norm_then_moving_average_sweep_fp32_fp16(seed):
+    """The same call in fp32 / fp16: rows of 64 to 16 384 tokens go through the norm and the moving average on rows in
+    time, shorter rows, more than 16 states and carried states into ragged rows through the library's own pair."""
+    rng = np.random.default_rng(3500 + seed + SEED_SHIFT)
+    for case in range(6):
+        dtype = torch.float32 if rng.integers(0, 2) else torch.float16
+        tol = 2e-4 if dtype is torch.float32 else 4e-3
+        G = int(rng.choice([1, 2, 4]))
+        D = G * int(rng.choice([64, 24, 128, 8]))
+        L = int(rng.choice([40, 64, 300, 1024, 2048, 2050, 3072]))
+        B = int(rng.choice([1, 2, 3]))
+        N = int(rng.choice([2, 7, 16, 20]))
+        cplx = bool(rng.integers(0, 2))
+        masked = rng.integers(0, 3) == 0
+        with_state = bool(rng.integers(0, 2))
+        out_layout = "input" if rng.integers(0, 2) else "rows"
+        tag = (f"seed {seed} case {case}: {dtype} B={B} L={L} D={D} G={G} N={N} cplx={cplx} masked={masked} "
+               f"state={with_state} out={out_layout}")
+        print(tag, flush=True)
+        p, q, g = _coeffs(rng, D, N, cplx)
+        om = rng.normal(size=D)
+        gam = (rng.normal(size=D) * 0.1 + 1.0).astype(np.float32).astype(np.float64)
+        bet = (rng.normal(size=D) * 0.1).astype(np.float32).astype(np.float64)
+        x, x64 = rounded(rng.normal(size=(B, L, D)) * 1.5 + 0.3, dtype)
+        mask = None
+        if masked:
+            mask = np.zeros((B, L), bool); mask[0, L - L // 4:] = True
+            if rng.integers(0, 2):
+                mask[-1, :int(rng.integers(1, min(L, 1500)))] = True
+                mask[B // 2] |= rng.random(L) < 0.05
+        h0 = None
+        if with_state:
+            h0 = (rng.normal(size=(B, D, N)) + (1j * rng.normal(size=(B, D, N)) if cplx else 0))
+            h0 = h0.astype(np.complex64) if cplx else h0.astype(np.float32)
+        pc = rng.integers(0, 30, size=B)
+        pm = rng.normal(size=(B, G)).astype(np.float32).astype(np.float64)
+        pv = (rng.random((B, G)) + 0.5).astype(np.float32).astype(np.float64)
+        layer = M.ops.PreparedEMA(dev(p), dev(q), dev(g), dev(om))
+        xn, y, cnt, mean, var, h = layer.norm_forward(
+            x, dev(pc, torch.int64), dev(pm), dev(pv), dev(gam), dev(bet), G, 1e-5,
+            padding_mask=None if mask is None else dev(mask, torch.bool), h=None if h0 is None else dev(h0),
+            want_state=with_state, out_layout=out_layout)
+        torch.cuda.synchronize()
+        assert y.shape == (B, D, L), tag
+        xno, co, mo, vo = O.timestep_norm(x64, pc, pm, pv, gam, bet, mask, G)
+        assert cnt.tolist() == co.tolist(), tag
+        assert rel_err(host(xn), xno) < tol, tag
+        assert rel_err(host(mean), mo) < 1e-4 and rel_err(host(var), vo) < 1e-4, tag
+        yo, ho = O.ema_forward(host(xn).transpose(0, 2, 1), p, q, g, om, mask, h=h0, incremental=with_state)
+        assert _out_err(host(y), yo) < tol, tag
+        if with_state:
+            assert _state_err(np.real(host(h)), np.real(ho)) < 2e-3, tag
+    assert M.ops.timestep_norm_status() == 0
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_attention_sweep(seed):
     """EfficientAttention's forward with and without the weights: head sizes on both sides of what the one-kernel
